@@ -1,0 +1,237 @@
+"""Pins the CPU oracle (oracle/) before anything is compared with it.
+
+The reference (cocoalex00/Mamba2D) ships no tests, golden vectors or CPU path, so each
+function of the oracle is pinned by what the mathematics fixes: an independent brute
+force, closed forms, invariants, finite differences and torch.autograd through an
+independently written forward.  Each check is chosen so that a plausible slip (a dropped
+term, a wrong mask, a transposed operand, T/L swapped) fails at least one of them.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import scan_oracle as so
+
+F64 = torch.float64
+
+
+def tiny(B=1, H=3, W=4, E=2, N=2, seed=0):
+    return so.make_inputs(B, H, W, E, N, seed=seed, dtype=F64)
+
+
+def args(inp):
+    return [inp[k] for k in so.INPUT_NAMES]
+
+
+# ------------------------------------------------------------------ forward (F)
+@pytest.mark.parametrize("H,W", [(2, 2), (2, 3), (3, 2), (3, 5), (5, 3), (4, 4)])
+def test_c_forward_matches_python_loops(cscan, H, W):
+    inp = tiny(B=2, H=H, W=W, E=2, N=3, seed=H * 10 + W)
+    y_c, hs_c = cscan.forward(*args(inp), want_hs=True)
+    y_l, hs_l = so.scan_forward_loops(*[t.numpy() for t in args(inp)])
+    np.testing.assert_allclose(hs_c, hs_l, rtol=1e-13, atol=1e-14)
+    np.testing.assert_allclose(y_c, y_l, rtol=1e-13, atol=1e-14)
+
+
+def test_torch_forward_matches_c(cscan):
+    inp = so.make_inputs(2, 6, 5, 3, 4, seed=3, dtype=F64)
+    y_c, hs_c = cscan.forward(*args(inp), want_hs=True)
+    y_t, hs_t = so.scan_forward_torch(*args(inp), return_hs=True)
+    np.testing.assert_allclose(hs_t.numpy(), hs_c, rtol=1e-12, atol=1e-14)
+    np.testing.assert_allclose(y_t.numpy(), y_c, rtol=1e-12, atol=1e-13)
+
+
+def test_first_row_and_column_are_1d_scans(cscan):
+    """Row 0 is a 1-D selective scan along W with the L parameters; column 0 is one along H
+    with the T parameters seeded by h[0,0] = uL[0,0] (wf_cuda.cu:58-63)."""
+    inp = so.make_inputs(2, 7, 6, 3, 4, seed=5, dtype=F64)
+    _, hs = cscan.forward(*args(inp), want_hs=True)
+    x, dT, dL, AT, AL, BT, BL = [inp[k].numpy() for k in ("x", "deltaT", "deltaL", "AT", "AL", "BT", "BL")]
+    B, H, W, E = x.shape
+    aL = np.exp(dL[..., None] * AL)
+    aT = np.exp(dT[..., None] * AT)
+    uL = dL[..., None] * BL[:, :, :, None, :] * x[..., None]
+    uT = dT[..., None] * BT[:, :, :, None, :] * x[..., None]
+    # closed form  h_j = sum_k (prod_{k<m<=j} a_m) u_k  through cumulative log-products
+    cum = np.cumsum(np.log(aL[:, 0]), axis=1)                      # (B,W,E,N)
+    want = np.stack([sum(np.exp(cum[:, j] - cum[:, k]) * uL[:, 0, k] for k in range(j + 1))
+                     for j in range(W)], axis=1)
+    np.testing.assert_allclose(hs[:, 0], want, rtol=1e-11, atol=1e-13)
+    cumT = np.cumsum(np.log(aT[:, :, 0]), axis=1)                  # (B,H,E,N)
+    col = []
+    for i in range(H):
+        acc = np.exp(cumT[:, i] - cumT[:, 0]) * uL[:, 0, 0]        # seed is the L term at the origin
+        for k in range(1, i + 1):
+            acc = acc + np.exp(cumT[:, i] - cumT[:, k]) * uT[:, k, 0]
+        col.append(acc)
+    np.testing.assert_allclose(hs[:, :, 0], np.stack(col, axis=1), rtol=1e-11, atol=1e-13)
+
+
+def test_closed_form_zero_A_constant_inputs(cscan):
+    """A=0 (gates 1), constant delta, B, x: h[i,j] = (i+j+1)*delta*beta*xi."""
+    B, H, W, E, N = 1, 6, 9, 2, 3
+    dl, be, xi, c, dskip = 0.3, -0.7, 1.9, 0.25, 0.5
+    one = lambda *s: torch.ones(*s, dtype=F64)
+    y, hs = cscan.forward(xi * one(B, H, W, E), dl * one(B, H, W, E), dl * one(B, H, W, E),
+                          0 * one(E, N), 0 * one(E, N), be * one(B, H, W, N), be * one(B, H, W, N),
+                          c * one(B, H, W, N), dskip * one(E), want_hs=True)
+    ij = np.add.outer(np.arange(H), np.arange(W)) + 1.0
+    np.testing.assert_allclose(hs, np.broadcast_to((ij * dl * be * xi)[None, :, :, None, None], hs.shape),
+                               rtol=1e-13)
+    np.testing.assert_allclose(y, np.broadcast_to((ij * dl * be * xi * c * N + xi * dskip)[None, :, :, None], y.shape),
+                               rtol=1e-13)
+
+
+def test_impulse_at_origin(cscan):
+    """x nonzero only at (0,0): with gates 1 the averaging keeps every state equal to the
+    impulse; with equal constant gates a the edges decay as a^j / a^i and the interior is the
+    path-weighted mean a^(i+j) (every monotone path has i+j steps, weights sum to one)."""
+    B, H, W, E, N = 1, 5, 6, 1, 2
+    x = torch.zeros(B, H, W, E, dtype=F64)
+    x[:, 0, 0] = 2.0
+    one = lambda *s: torch.ones(*s, dtype=F64)
+    for A, dl in ((0.0, 0.5), (-0.8, 0.5)):
+        a = np.exp(A * dl)
+        _, hs = cscan.forward(x, dl * one(B, H, W, E), dl * one(B, H, W, E), A * one(E, N), A * one(E, N),
+                              one(B, H, W, N), 3 * one(B, H, W, N), one(B, H, W, N), one(E), want_hs=True)
+        u0 = dl * 3.0 * 2.0                                         # the L term at the origin
+        ij = np.add.outer(np.arange(H), np.arange(W))
+        np.testing.assert_allclose(hs[0, :, :, 0, 0], u0 * a ** ij, rtol=1e-12)
+
+
+def test_origin_uses_L_direction_only(cscan):
+    inp = tiny(H=3, W=3, seed=11)
+    _, hs = cscan.forward(*args(inp), want_hs=True)
+    want = (inp["deltaL"][:, 0, 0, :, None] * inp["BL"][:, 0, 0, None, :] * inp["x"][:, 0, 0, :, None]).numpy()
+    np.testing.assert_allclose(hs[:, 0, 0], want, rtol=1e-14)
+    other = (inp["deltaT"][:, 0, 0, :, None] * inp["BT"][:, 0, 0, None, :] * inp["x"][:, 0, 0, :, None]).numpy()
+    assert np.abs(hs[:, 0, 0] - other).max() > 1e-3
+
+
+def test_linearity_in_x(cscan):
+    inp = so.make_inputs(1, 5, 4, 3, 4, seed=7, dtype=F64)
+    x2 = torch.randn(inp["x"].shape, generator=torch.Generator().manual_seed(1), dtype=F64)
+    a = args(inp)
+    f = lambda xx: cscan.forward(xx, *a[1:]) - (xx * inp["D"]).numpy()
+    lhs = f(1.5 * inp["x"] - 0.25 * x2)
+    np.testing.assert_allclose(lhs, 1.5 * f(inp["x"]) - 0.25 * f(x2), rtol=1e-11, atol=1e-12)
+
+
+def test_transpose_symmetry(cscan):
+    """Swapping the axes H<->W together with the roles T<->L transposes the states, provided
+    the two input terms agree at the origin (where only the L term is used)."""
+    inp = so.make_inputs(2, 4, 6, 3, 4, seed=9, dtype=F64)
+    inp["x"][:, 0, 0] = 0.0
+    _, hs = cscan.forward(*args(inp), want_hs=True)
+    tr = lambda t: t.transpose(1, 2).contiguous()
+    _, hs_t = cscan.forward(tr(inp["x"]), tr(inp["deltaL"]), tr(inp["deltaT"]), inp["AL"], inp["AT"],
+                            tr(inp["BL"]), tr(inp["BT"]), tr(inp["C"]), inp["D"], want_hs=True)
+    np.testing.assert_allclose(hs_t.transpose(0, 2, 1, 3, 4), hs, rtol=1e-12, atol=1e-14)
+
+
+def test_small_spatial_dims_raise(cscan):
+    for H, W in ((1, 4), (4, 1), (1, 1)):
+        inp = so.make_inputs(1, H, W, 2, 2, dtype=F64)
+        with pytest.raises(ValueError, match="spatial dims > 1"):
+            cscan.forward(*args(inp))
+        with pytest.raises(ValueError, match="spatial dims > 1"):
+            cscan.backward(*args(inp), inp["dy"])
+
+
+def test_fp32_instance_tracks_fp64(cscan):
+    inp = so.make_inputs(2, 14, 14, 8, 16, seed=2, dtype=torch.float32)
+    y64 = cscan.forward(*args(inp))
+    y32 = cscan.forward(*args(inp), dtype=np.float32)
+    assert so.rel_err(y32, y64) < 1e-5
+
+
+# ------------------------------------------------------------------ backward (B + M)
+@pytest.mark.parametrize("shape", [(1, 2, 2, 1, 1), (2, 2, 5, 2, 3), (2, 5, 2, 2, 3), (2, 4, 6, 3, 4),
+                                   (1, 7, 7, 2, 16)])
+def test_c_backward_matches_autograd(cscan, shape):
+    B, H, W, E, N = shape
+    inp = so.make_inputs(B, H, W, E, N, seed=sum(shape), dtype=F64)
+    got = cscan.backward(*args(inp), inp["dy"])
+    y_ag, want = so.scan_grads_autograd(inp)
+    np.testing.assert_allclose(cscan.forward(*args(inp)), y_ag.numpy(), rtol=1e-12, atol=1e-13)
+    for k in so.CScan.GRADS:
+        assert so.rel_err(got[k], want[k]) < 1e-12, k
+
+
+def test_adjoint_intermediates_match_autograd(cscan):
+    """dDAT / dDAL are dL/d(gate); dBX masked by (i>0) resp. (j>0 or i==0) is dL/d(input term)
+    (wf_cuda.cu:149-160, wavefront_cuda.py:122-123)."""
+    inp = so.make_inputs(2, 5, 4, 2, 3, seed=21, dtype=F64)
+    res = cscan.backward(*args(inp), inp["dy"], want_intermediates=True)
+    x, dT, dL, AT, AL, BT, BL, C, D = args(inp)
+    leaves = [t.clone().requires_grad_(True) for t in (
+        torch.exp(dT.unsqueeze(-1) * AT), torch.exp(dL.unsqueeze(-1) * AL),
+        (dT.unsqueeze(-1) * BT.unsqueeze(-2)) * x.unsqueeze(-1),
+        (dL.unsqueeze(-1) * BL.unsqueeze(-2)) * x.unsqueeze(-1))]
+    hs = so.scan_core_torch(*leaves)
+    y = (hs * C.unsqueeze(-2)).sum(-1) + x * D
+    g_gT, g_gL, g_uT, g_uL = torch.autograd.grad(y, leaves, inp["dy"])
+    H, W = x.shape[1:3]
+    ii = np.arange(H)[None, :, None, None, None]
+    jj = np.arange(W)[None, None, :, None, None]
+    np.testing.assert_allclose(res["hs"], hs.detach().numpy(), rtol=1e-12, atol=1e-14)
+    np.testing.assert_allclose(res["dDAT"], g_gT.numpy(), rtol=1e-11, atol=1e-13)
+    np.testing.assert_allclose(res["dDAL"], g_gL.numpy(), rtol=1e-11, atol=1e-13)
+    np.testing.assert_allclose(res["dBX"] * (ii > 0), g_uT.numpy(), rtol=1e-11, atol=1e-13)
+    np.testing.assert_allclose(res["dBX"] * ((jj > 0) | (ii == 0)), g_uL.numpy(), rtol=1e-11, atol=1e-13)
+
+
+def test_c_backward_matches_finite_differences(cscan):
+    """Central differences of L = <y, dy> in every input, independent of autograd."""
+    inp = so.make_inputs(1, 3, 4, 2, 2, seed=31, dtype=F64)
+    got = cscan.backward(*args(inp), inp["dy"])
+    dy = inp["dy"].numpy()
+    loss = lambda d: float((cscan.forward(*[d[k] for k in so.INPUT_NAMES]) * dy).sum())
+    eps = 1e-6
+    rng = np.random.default_rng(0)
+    for name, gname in zip(so.INPUT_NAMES, so.CScan.GRADS):
+        flat_n = inp[name].numel()
+        for idx in rng.choice(flat_n, size=min(flat_n, 6), replace=False):
+            p = {k: v.clone() for k, v in inp.items()}
+            m = {k: v.clone() for k, v in inp.items()}
+            p[name].view(-1)[idx] += eps
+            m[name].view(-1)[idx] -= eps
+            fd = (loss(p) - loss(m)) / (2 * eps)
+            an = got[gname].reshape(-1)[idx]
+            assert abs(fd - an) <= 1e-6 * max(1.0, abs(an)), (name, idx, fd, an)
+
+
+# ------------------------------------------------------------------ projections / entry point
+def test_proj_params_split_order_and_casts():
+    torch.manual_seed(0)
+    E, N, R = 8, 4, 2
+    x = torch.randn(1, 3, 3, E)
+    w = torch.randn(2 * R + 3 * N, E)
+    wT, bT, wL, bL = torch.randn(E, R), torch.randn(E), torch.randn(E, R), torch.randn(E)
+    Alog = torch.log(torch.arange(1, N + 1, dtype=torch.float32)).repeat(E, 1)
+    dT, dL, AT, AL, BT, BL, C = so.proj_params_ref(x, Alog, Alog, w, wT, bT, wL, bL)
+    z = x @ w.t()
+    assert torch.allclose(dT, torch.nn.functional.softplus(z[..., :R] @ wT.t() + bT), atol=1e-6)
+    assert torch.allclose(dL, torch.nn.functional.softplus(z[..., R:2 * R] @ wL.t() + bL), atol=1e-6)
+    assert torch.allclose(BT, z[..., 2 * R:2 * R + N]) and torch.allclose(BL, z[..., 2 * R + N:2 * R + 2 * N])
+    assert torch.allclose(C, z[..., 2 * R + 2 * N:])
+    assert torch.allclose(AT, -torch.arange(1, N + 1, dtype=torch.float32).repeat(E, 1))
+    outs = so.proj_params_ref(x.bfloat16(), Alog, Alog, w.bfloat16(), wT.bfloat16(), bT.bfloat16(),
+                              wL.bfloat16(), bL.bfloat16())
+    assert all(t.dtype == torch.bfloat16 for t in outs)
+
+
+# ------------------------------------------------------------------ golden fixtures
+@pytest.mark.parametrize("name", ["cfg0_B2_E32_14x14_N16", "ragged_B3_E4_5x9_N16"])
+def test_oracle_reproduces_golden(cscan, name):
+    import os
+    blob = np.load(os.path.join(os.path.dirname(__file__), "golden", name + ".npz"))
+    a = [blob["in_" + k] for k in so.INPUT_NAMES]
+    B, H, W, E, N, seed = [int(v) for v in blob["meta"]]
+    fresh = so.make_inputs(B, H, W, E, N, seed=seed)
+    for k in so.INPUT_NAMES + ("dy",):
+        np.testing.assert_array_equal(fresh[k].numpy(), blob["in_" + k])
+    np.testing.assert_allclose(cscan.forward(*a), blob["y"], rtol=1e-12, atol=1e-13)
+    g = cscan.backward(*a, blob["in_dy"])
+    for k in so.CScan.GRADS:
+        np.testing.assert_allclose(g[k], blob[k], rtol=1e-11, atol=1e-12)
