@@ -1,0 +1,119 @@
+/*
+ * m2dscan -- C ABI of the MI355X (gfx950) wavefront 2-D selective scan.
+ *
+ * A torch-free HIP shared library (libm2dscan.so) exports exactly these symbols.  They
+ * are what a binding for the reference's native module would call in place of its two
+ * pybind entry points
+ *     wf_fwd(hs, x, deltaT, deltaL, BT, BL, AT, AL)                     wf_cuda_bind.cpp:24-33
+ *     wf_bwd(hs, x, deltaT, deltaL, AT, AL, grad_output, dDAT, dDAL, omega)   wf_cuda_bind.cpp:35-46
+ * together with the tensor algebra the reference performs around them in Python
+ * (output projection wavefront_cuda.py:156, its backward :176-178, parameter gradients
+ * :97-139, d_x assembly :193-194): one fused forward producing y and one fused backward
+ * producing the nine gradients, neither of which materialises the (B,H,W,E,N) state.
+ *
+ * Conventions
+ *   - All tensor arguments are DEVICE pointers to contiguous, channel-last arrays in
+ *     the reference's layout:  x, deltaT, deltaL, y, dy, dx, d_deltaT, d_deltaL : (B,H,W,E)
+ *                              BT, BL, C, d_BT, d_BL, d_C : (B,H,W,N)
+ *                              AT, AL, d_AT, d_AL : (E,N)        D, d_D : (E)
+ *     every one of them in the element type named by m2d_desc.dtype (the reference
+ *     requires one common dtype too, wf_cuda.cu:182).  State and accumulation are fp32.
+ *   - The caller owns every buffer, including workspace and checkpoints; the library
+ *     allocates nothing and keeps no mutable global state, so calls are re-entrant.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream).  Calls only
+ *     enqueue work; they do not synchronise.
+ *   - Every function returns an m2d_status; nothing is launched unless it is M2D_OK.
+ */
+#ifndef M2DSCAN_H
+#define M2DSCAN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum m2d_status {
+  M2D_OK = 0,
+  M2D_ERR_NULL_POINTER = 1,   /* a required pointer argument is NULL */
+  M2D_ERR_BAD_SHAPE = 2,      /* a dimension is < 1, or H < 2 or W < 2 (reference: wavefront_cuda.py:323-324) */
+  M2D_ERR_UNSUPPORTED = 3,    /* dtype / N outside what the kernels are built for */
+  M2D_ERR_WORKSPACE = 4,      /* workspace or checkpoint buffer smaller than required */
+  M2D_ERR_MISALIGNED = 5,     /* a tensor pointer is not 16-byte aligned / workspace not 256-byte aligned */
+  M2D_ERR_HIP = 6             /* a HIP runtime call or kernel launch failed */
+} m2d_status;
+
+typedef enum m2d_dtype {
+  M2D_F32 = 0,                /* fp32 in, fp32 out */
+  M2D_BF16 = 1                /* bf16 in, bf16 out, fp32 state and accumulation */
+} m2d_dtype;
+
+/* Problem descriptor.  N must be 16 in this build (the reference's d_state default,
+ * models/mamba2d.py:23).  flags: bit 0 = M2D_FLAG_FLIP, scan from the bottom-right
+ * corner (equivalent to torch.flip(x,(1,2)) of every spatial tensor before and of the
+ * outputs after, models/mamba2d.py:163-173). */
+typedef struct m2d_desc {
+  int32_t B, H, W, E, N;
+  int32_t dtype;              /* m2d_dtype */
+  int32_t flags;
+  int32_t reserved;           /* must be 0 */
+} m2d_desc;
+
+#define M2D_FLAG_FLIP 1
+
+#define M2D_PASS_FWD 0
+#define M2D_PASS_BWD 1
+
+/* Library version (major*10000 + minor*100 + patch). */
+int m2d_version(void);
+
+/* Human-readable text for a status code (static storage). */
+const char* m2d_status_str(int status);
+
+/* Validates a descriptor without touching the GPU. */
+int m2d_desc_check(const m2d_desc* desc);
+
+/* Bytes of scratch the forward (M2D_PASS_FWD) or backward (M2D_PASS_BWD) pass needs.
+ * `have_ckpt` != 0 means the caller passes a checkpoint buffer to that pass (forward:
+ * to be filled; backward: filled by the forward), which reduces the scratch.
+ * Returns 0 for an invalid descriptor. */
+size_t m2d_scan_workspace_bytes(const m2d_desc* desc, int pass, int have_ckpt);
+
+/* Bytes of the checkpoint buffer (anti-diagonal state snapshots every few steps plus
+ * band-boundary rows; linear in H*W, about 1/4 of the full state tensor in fp32). */
+size_t m2d_scan_ckpt_bytes(const m2d_desc* desc);
+
+/* Fused forward:  y = sum_n h*C + x*D  with h from the recurrence of wf_cuda.cu:40-69.
+ * Replaces wf_fwd (wf_cuda_bind.cpp:24) + wavefront_cuda.py:152-156.
+ * ckpt may be NULL (inference); if given it is filled for a later m2d_scan_bwd. */
+int m2d_scan_fwd(const m2d_desc* desc,
+                 const void* x, const void* deltaT, const void* deltaL,
+                 const void* AT, const void* AL,
+                 const void* BT, const void* BL, const void* C, const void* D,
+                 void* y,
+                 void* ckpt, size_t ckpt_bytes,
+                 void* workspace, size_t workspace_bytes,
+                 void* stream);
+
+/* Fused backward: the nine gradients of the forward above for upstream gradient dy.
+ * Replaces wavefront_cuda.py:169-196 (state recompute, wf_bwd of wf_cuda_bind.cpp:35,
+ * fused_backward_math, output-projection backward).  ckpt may be NULL, in which case
+ * the checkpoints are rebuilt inside the call (one extra forward sweep).
+ * d_AT, d_AL, d_D are written (not accumulated). */
+int m2d_scan_bwd(const m2d_desc* desc,
+                 const void* x, const void* deltaT, const void* deltaL,
+                 const void* AT, const void* AL,
+                 const void* BT, const void* BL, const void* C, const void* D,
+                 const void* dy,
+                 const void* ckpt, size_t ckpt_bytes,
+                 void* dx, void* d_deltaT, void* d_deltaL,
+                 void* d_AT, void* d_AL,
+                 void* d_BT, void* d_BL, void* d_C, void* d_D,
+                 void* workspace, size_t workspace_bytes,
+                 void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* M2DSCAN_H */

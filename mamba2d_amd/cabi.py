@@ -1,0 +1,144 @@
+"""ctypes view of libm2dscan.so -- the C ABI declared in include/m2dscan.h.
+
+PyTorch appears here only as the owner of device memory and of the current HIP stream.
+There is no fallback: if the library has not been built, importing this module raises.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libm2dscan.so")
+
+M2D_F32, M2D_BF16 = 0, 1
+M2D_FLAG_FLIP = 1
+M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
+
+EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
+           "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_bwd")
+
+
+class Desc(ctypes.Structure):
+    _fields_ = [(k, ctypes.c_int32) for k in ("B", "H", "W", "E", "N", "dtype", "flags", "reserved")]
+
+
+class M2DError(RuntimeError):
+    def __init__(self, status: int, text: str):
+        super().__init__(f"m2dscan: {text} (status {status})")
+        self.status = status
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python -m mamba2d_amd.build` "
+            "(there is no CPU or eager fallback for the scan)")
+    lib = ctypes.CDLL(LIB_PATH)
+    vp, sz, i32 = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
+    dp = ctypes.POINTER(Desc)
+    lib.m2d_version.restype = i32
+    lib.m2d_status_str.restype = ctypes.c_char_p
+    lib.m2d_status_str.argtypes = [i32]
+    lib.m2d_desc_check.restype = i32
+    lib.m2d_desc_check.argtypes = [dp]
+    lib.m2d_scan_workspace_bytes.restype = sz
+    lib.m2d_scan_workspace_bytes.argtypes = [dp, i32, i32]
+    lib.m2d_scan_ckpt_bytes.restype = sz
+    lib.m2d_scan_ckpt_bytes.argtypes = [dp]
+    lib.m2d_scan_fwd.restype = i32
+    lib.m2d_scan_fwd.argtypes = [dp] + [vp] * 9 + [vp, vp, sz, vp, sz, vp]
+    lib.m2d_scan_bwd.restype = i32
+    lib.m2d_scan_bwd.argtypes = [dp] + [vp] * 10 + [vp, sz] + [vp] * 9 + [vp, sz, vp]
+    return lib
+
+
+lib = _load()
+
+
+def status_str(code: int) -> str:
+    return lib.m2d_status_str(int(code)).decode()
+
+
+def check(code: int) -> None:
+    if code != 0:
+        raise M2DError(code, status_str(code))
+
+
+def make_desc(x: torch.Tensor, N: int, flip: bool = False) -> Desc:
+    B, H, W, E = x.shape
+    if x.dtype == torch.float32:
+        dt = M2D_F32
+    elif x.dtype == torch.bfloat16:
+        dt = M2D_BF16
+    else:
+        raise TypeError(f"m2dscan supports float32 and bfloat16, got {x.dtype}")
+    return Desc(B, H, W, E, N, dt, M2D_FLAG_FLIP if flip else 0, 0)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def _stream(dev):
+    return ctypes.c_void_p(torch.cuda.current_stream(dev).cuda_stream)
+
+
+def _same(x, *ts):
+    for t in ts:
+        if t.dtype != x.dtype or t.device != x.device or not t.is_contiguous():
+            raise ValueError("m2dscan: all tensors must be contiguous, on one device and of one dtype")
+
+
+def _shapes(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy=None):
+    """The library only sees pointers, so every extent it will index is checked here."""
+    if x.dim() != 4 or AT.dim() != 2:
+        raise ValueError("m2dscan: x must be (B,H,W,E) and AT (E,N)")
+    B, H, W, E = x.shape
+    N = AT.shape[1]
+    want = {"deltaT": (deltaT, (B, H, W, E)), "deltaL": (deltaL, (B, H, W, E)), "AT": (AT, (E, N)),
+            "AL": (AL, (E, N)), "BT": (BT, (B, H, W, N)), "BL": (BL, (B, H, W, N)), "C": (C, (B, H, W, N)),
+            "D": (D, (E,))}
+    if dy is not None:
+        want["dy"] = (dy, (B, H, W, E))
+    for k, (t, shp) in want.items():
+        if tuple(t.shape) != shp:
+            raise ValueError(f"m2dscan: {k} has shape {tuple(t.shape)}, expected {shp}")
+    if not x.is_cuda:
+        raise ValueError("m2dscan: tensors must live on the GPU")
+
+
+def _bytes(n, dev):
+    # torch's caching allocator returns 512-byte aligned blocks
+    return torch.empty(max(int(n), 1), dtype=torch.uint8, device=dev)
+
+
+def scan_fwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, save_ckpt=False, flip=False):
+    """y (and the checkpoint buffer when ``save_ckpt``) through m2d_scan_fwd."""
+    _same(x, deltaT, deltaL, AT, AL, BT, BL, C, D)
+    _shapes(x, deltaT, deltaL, AT, AL, BT, BL, C, D)
+    d = make_desc(x, AT.shape[1], flip)
+    check(lib.m2d_desc_check(ctypes.byref(d)))
+    y = torch.empty_like(x)
+    ck = _bytes(lib.m2d_scan_ckpt_bytes(ctypes.byref(d)), x.device) if save_ckpt else None
+    ws = _bytes(lib.m2d_scan_workspace_bytes(ctypes.byref(d), M2D_PASS_FWD, int(save_ckpt)), x.device)
+    check(lib.m2d_scan_fwd(ctypes.byref(d), *[_ptr(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D)],
+                           _ptr(y), _ptr(ck), ck.numel() if ck is not None else 0, _ptr(ws), ws.numel(),
+                           _stream(x.device)))
+    return (y, ck) if save_ckpt else y
+
+
+def scan_bwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt=None, flip=False):
+    """The nine gradients (order of the inputs) through m2d_scan_bwd."""
+    _same(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy)
+    _shapes(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy)
+    d = make_desc(x, AT.shape[1], flip)
+    check(lib.m2d_desc_check(ctypes.byref(d)))
+    outs = [torch.empty_like(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D)]
+    ws = _bytes(lib.m2d_scan_workspace_bytes(ctypes.byref(d), M2D_PASS_BWD, int(ckpt is not None)), x.device)
+    check(lib.m2d_scan_bwd(ctypes.byref(d), *[_ptr(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy)],
+                           _ptr(ckpt), ckpt.numel() if ckpt is not None else 0, *[_ptr(t) for t in outs],
+                           _ptr(ws), ws.numel(), _stream(x.device)))
+    return tuple(outs)

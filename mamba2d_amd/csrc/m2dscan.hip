@@ -1,0 +1,728 @@
+// m2dscan: wavefront 2-D selective scan for gfx950 (MI355X), forward and backward.
+//
+// Mapping (both passes).  The recurrence  h[i,j] = cL*(aL*h[i,j-1] + uL) + cT*(aT*h[i-1,j] + uT)
+// (reference: models/kernels/wf_cuda/wf_cuda.cu:40-69) is independent across (batch, channel,
+// state).  One 64-lane wavefront owns a few channels of one problem and sweeps it
+// anti-diagonal by anti-diagonal: lane r holds grid row r and at step t works on the cell
+// (r, t-r), so one step of the wave IS one anti-diagonal.  The 16 states of a cell stay in
+// VGPRs; h[i,j-1] is the lane's own previous value and h[i-1,j] is the previous value of lane
+// r-1, fetched with a DPP wave shift.  y = C.h is a 16-term in-register sum.  Grids with
+// fewer than 33 rows are packed several problems per wave (power-of-two lane slots); grids
+// with more than 64 rows are cut in bands of 64 rows whose boundary rows travel through
+// memory.
+//
+// The interior factor 1/2 and the first-row/column special cases are folded into the gate
+// exponent (exp2(delta*A*log2e + log2 c)) and into the input coefficient, so the inner loop
+// has no branches.
+//
+// Backward (adjoint of the above; reference wf_cuda.cu:108-160 and
+// models/kernels/wavefront_cuda.py:97-139,176-178,193-194).  The forward stores the wave's
+// register state every CK steps (a checkpoint is one anti-diagonal).  The backward walks the
+// blocks of CK steps in reverse: it restores the checkpoint, recomputes the CK states of the
+// block into registers, then runs the adjoint over the block backwards, with
+//     lambda = dy*C + muL(own, previous step) + muT(lane r+1, previous step)
+//     muT = cT*aT*lambda,  muL = cL*aL*lambda
+// and emits all gradients on the fly.  Sums over channels (d_BT, d_BL, d_C) go through
+// per-wave LDS slots that are added in a fixed order; sums over positions (d_AT, d_AL, d_D)
+// are register accumulators reduced at the end.  Everything is deterministic.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/m2dscan.h"
+
+namespace {
+
+constexpr int kN = 16;            // states per channel
+#ifndef M2D_CK
+#define M2D_CK 4
+#endif
+constexpr int kCK = M2D_CK;       // checkpoint interval (steps)
+constexpr int kFwdWaves = 4;      // waves per forward workgroup
+constexpr int kBwdWaves = 8;      // waves per backward workgroup
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+struct bf16_t { uint16_t v; };
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t lo16) { return __uint_as_float(lo16 << 16); }
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);  // NaN
+  u += 0x7fffu + ((u >> 16) & 1u);                                            // round to nearest even
+  return (uint16_t)(u >> 16);
+}
+
+template <typename T> struct IO;
+template <> struct IO<float> {
+  static __device__ __forceinline__ float ld(const float* p) { return *p; }
+  static __device__ __forceinline__ void st(float* p, float v) { *p = v; }
+  template <int EC> static __device__ __forceinline__ void ldv(const float* p, float (&v)[EC]) {
+    if constexpr (EC == 2) { float2 t = *reinterpret_cast<const float2*>(p); v[0] = t.x; v[1] = t.y; }
+    else { for (int c = 0; c < EC; ++c) v[c] = p[c]; }
+  }
+  template <int EC> static __device__ __forceinline__ void stv(float* p, const float (&v)[EC]) {
+    if constexpr (EC == 2) { *reinterpret_cast<float2*>(p) = make_float2(v[0], v[1]); }
+    else { for (int c = 0; c < EC; ++c) p[c] = v[c]; }
+  }
+  static __device__ __forceinline__ void ld16(const float* p, float (&v)[kN]) {
+    const float4* q = reinterpret_cast<const float4*>(p);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) { float4 t = q[k]; v[4*k] = t.x; v[4*k+1] = t.y; v[4*k+2] = t.z; v[4*k+3] = t.w; }
+  }
+  static __device__ __forceinline__ void st4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+};
+template <> struct IO<bf16_t> {
+  static __device__ __forceinline__ float ld(const bf16_t* p) { return bf16_bits_to_f32(p->v); }
+  static __device__ __forceinline__ void st(bf16_t* p, float v) { p->v = f32_to_bf16_bits(v); }
+  template <int EC> static __device__ __forceinline__ void ldv(const bf16_t* p, float (&v)[EC]) {
+    if constexpr (EC == 2) {
+      uint32_t t = *reinterpret_cast<const uint32_t*>(p);
+      v[0] = __uint_as_float(t << 16); v[1] = __uint_as_float(t & 0xffff0000u);
+    } else { for (int c = 0; c < EC; ++c) v[c] = bf16_bits_to_f32(p[c].v); }
+  }
+  template <int EC> static __device__ __forceinline__ void stv(bf16_t* p, const float (&v)[EC]) {
+    if constexpr (EC == 2) {
+      *reinterpret_cast<uint32_t*>(p) = (uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16);
+    } else { for (int c = 0; c < EC; ++c) p[c].v = f32_to_bf16_bits(v[c]); }
+  }
+  static __device__ __forceinline__ void ld16(const bf16_t* p, float (&v)[kN]) {
+    const uint4* q = reinterpret_cast<const uint4*>(p);
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      uint4 t = q[k];
+      uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        v[8*k + 2*m] = __uint_as_float(w[m] << 16);
+        v[8*k + 2*m + 1] = __uint_as_float(w[m] & 0xffff0000u);
+      }
+    }
+  }
+  static __device__ __forceinline__ void st4(bf16_t* p, float4 v) {
+    uint2 t;
+    t.x = (uint32_t)f32_to_bf16_bits(v.x) | ((uint32_t)f32_to_bf16_bits(v.y) << 16);
+    t.y = (uint32_t)f32_to_bf16_bits(v.z) | ((uint32_t)f32_to_bf16_bits(v.w) << 16);
+    *reinterpret_cast<uint2*>(p) = t;
+  }
+};
+
+// lane l receives the value of lane l-1 (lane 0 receives 0)
+__device__ __forceinline__ float from_lane_below(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x138 /*wave_shr:1*/, 0xf, 0xf, true));
+}
+// lane l receives the value of lane l+1 (lane 63 receives 0)
+__device__ __forceinline__ float from_lane_above(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x130 /*wave_shl:1*/, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float fexp2(float v) { return __builtin_amdgcn_exp2f(v); }
+
+struct ScanParams {
+  const void *x, *dT, *dL, *BT, *BL, *C, *dy;
+  const float *A2T, *A2L, *Df;      // A*log2(e) and D in fp32, (E,16) / (E)
+  void *y, *dx, *ddT, *ddL;
+  float* ckpt;                      // [NG][nbands][nblk][E][16][64]
+  float* top;                       // [nbands-1][B][W][E][16]  last row of each band (forward states)
+  float* bot;                       // [B][W][E][16]            first-row muT of the band below (adjoint)
+  float* part;                      // [EG][3][P][16]           per-workgroup channel sums
+  float* pA;                        // [NG][E][2][16]
+  float* pD;                        // [NG][E]
+  int B, H, W, E;
+  int HP, hp_shift, S, NG, nbands, nblk, blocks_per_group, NET, flip;
+};
+
+struct Cell {          // what a lane needs to know about its cell at one step
+  bool act;
+  int64_t idx;         // flat (b,i,j) index, clamped to a valid cell when !act
+  float cT, cL, offT, offL;
+  int j;
+};
+
+__device__ __forceinline__ Cell locate(const ScanParams& p, int b, int i, int t, int r, bool row_ok) {
+  Cell c;
+  const int j = t - r;
+  c.j = j;
+  c.act = row_ok && j >= 0 && j < p.W;
+  const int bc = b < p.B ? b : p.B - 1;
+  const int ic = i < p.H ? i : p.H - 1;
+  const int jc = j < 0 ? 0 : (j < p.W ? j : p.W - 1);
+  const int im = p.flip ? p.H - 1 - ic : ic;
+  const int jm = p.flip ? p.W - 1 - jc : jc;
+  c.idx = ((int64_t)bc * p.H + im) * p.W + jm;
+  const float ninf = -__builtin_huge_valf();
+  if (!c.act)      { c.cT = 0.f;  c.cL = 0.f;  c.offT = ninf; c.offL = ninf; }
+  else if (i == 0) { c.cT = 0.f;  c.cL = 1.f;  c.offT = ninf; c.offL = 0.f; }
+  else if (j == 0) { c.cT = 1.f;  c.cL = 0.f;  c.offT = 0.f;  c.offL = ninf; }
+  else             { c.cT = 0.5f; c.cL = 0.5f; c.offT = -1.f; c.offL = -1.f; }
+  return c;
+}
+
+// ------------------------------------------------------------------------------------ forward
+template <typename T, int EC, bool CKPT, bool WRITE_Y>
+__global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParams p) {
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int g = blockIdx.x / p.blocks_per_group;
+  const int et = (blockIdx.x % p.blocks_per_group) * kFwdWaves + wave;
+  if (et >= p.NET) return;
+  const int e0 = et * EC;
+
+  float a2t[EC][kN], a2l[EC][kN], dsk[EC];
+#pragma unroll
+  for (int c = 0; c < EC; ++c) {
+#pragma unroll
+    for (int n = 0; n < kN; ++n) { a2t[c][n] = p.A2T[(e0 + c) * kN + n]; a2l[c][n] = p.A2L[(e0 + c) * kN + n]; }
+    dsk[c] = p.Df[e0 + c];
+  }
+
+  const int slot = lane >> p.hp_shift, r = lane & (p.HP - 1);
+  const int b = g * p.S + slot;
+  const T* X = static_cast<const T*>(p.x);
+  const T* DT = static_cast<const T*>(p.dT);
+  const T* DL = static_cast<const T*>(p.dL);
+  const T* BTp = static_cast<const T*>(p.BT);
+  const T* BLp = static_cast<const T*>(p.BL);
+  const T* Cp = static_cast<const T*>(p.C);
+  T* Y = static_cast<T*>(p.y);
+
+  for (int band = 0; band < p.nbands; ++band) {
+    const int i = band * 64 + r;
+    const int HB = p.nbands == 1 ? p.H : (p.H - band * 64 < 64 ? p.H - band * 64 : 64);
+    const bool row_ok = b < p.B && i < p.H;
+    const int T_steps = p.W + HB - 1;
+    float h[EC][kN];
+#pragma unroll
+    for (int c = 0; c < EC; ++c)
+#pragma unroll
+      for (int n = 0; n < kN; ++n) h[c][n] = 0.f;
+
+    for (int t = 0; t < T_steps; ++t) {
+      // snapshot of the state after step t-1; lanes that have not started or are past the last
+      // column hold nothing the backward needs
+      if (CKPT && t > 0 && (t % kCK) == 0 && row_ok && t - 1 - r >= 0 && t - 1 - r < p.W) {
+        float* ck = p.ckpt + ((((int64_t)g * p.nbands + band) * p.nblk + t / kCK) * p.E + e0) * (kN * 64) + lane;
+#pragma unroll
+        for (int c = 0; c < EC; ++c)
+#pragma unroll
+          for (int n = 0; n < kN; ++n) ck[(c * kN + n) * 64] = h[c][n];
+      }
+      const Cell cl = locate(p, b, i, t, r, row_ok);
+      float xv[EC], dtv[EC], dlv[EC], bt[kN], bl[kN], cc[kN];
+      IO<T>::template ldv<EC>(X + cl.idx * p.E + e0, xv);
+      IO<T>::template ldv<EC>(DT + cl.idx * p.E + e0, dtv);
+      IO<T>::template ldv<EC>(DL + cl.idx * p.E + e0, dlv);
+      IO<T>::ld16(BTp + cl.idx * kN, bt);
+      IO<T>::ld16(BLp + cl.idx * kN, bl);
+      if (WRITE_Y) IO<T>::ld16(Cp + cl.idx * kN, cc);
+      const bool from_top = band > 0 && r == 0;
+      float yv[EC];
+#pragma unroll
+      for (int c = 0; c < EC; ++c) {
+        const float sT = cl.cT * dtv[c] * xv[c];
+        const float sL = cl.cL * dlv[c] * xv[c];
+        float tp[kN];
+        if (from_top) {   // only lanes on the first row of a lower band (wave-divergent, rare)
+          const float* tb = p.top + ((((int64_t)(band - 1) * p.B + (b < p.B ? b : p.B - 1)) * p.W +
+                                      (cl.act ? cl.j : 0)) * p.E + e0 + c) * kN;
+#pragma unroll
+          for (int n = 0; n < kN; ++n) tp[n] = __builtin_nontemporal_load(tb + n);
+        }
+        float acc = 0.f;
+#pragma unroll
+        for (int n = 0; n < kN; ++n) {
+          const float aT = fexp2(__builtin_fmaf(dtv[c], a2t[c][n], cl.offT));
+          const float aL = fexp2(__builtin_fmaf(dlv[c], a2l[c][n], cl.offL));
+          float hT = from_lane_below(h[c][n]);
+          if (from_top) hT = tp[n];
+          float u = sL * bl[n];
+          u = __builtin_fmaf(sT, bt[n], u);
+          u = __builtin_fmaf(aT, hT, u);
+          const float hn = __builtin_fmaf(aL, h[c][n], u);
+          h[c][n] = hn;
+          if (WRITE_Y) acc = __builtin_fmaf(hn, cc[n], acc);
+        }
+        yv[c] = __builtin_fmaf(xv[c], dsk[c], acc);
+        if (p.nbands > 1 && band + 1 < p.nbands && r == 63 && cl.act) {
+          float* tb = p.top + ((((int64_t)band * p.B + b) * p.W + cl.j) * p.E + e0 + c) * kN;
+#pragma unroll
+          for (int n = 0; n < kN; ++n) tb[n] = h[c][n];
+        }
+      }
+      if (WRITE_Y && cl.act) IO<T>::template stv<EC>(Y + cl.idx * p.E + e0, yv);
+    }
+    if (p.nbands > 1) __threadfence();   // boundary row of this band is read back by the next one
+  }
+}
+
+// ----------------------------------------------------------------------------------- backward
+template <typename T>
+__global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParams p) {
+  extern __shared__ float4 slots[];   // [wave][3][4][64] float4: per-wave d_C, d_BT, d_BL of the step
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int g = blockIdx.x / p.blocks_per_group;
+  const int eg = blockIdx.x % p.blocks_per_group;
+  const int e_raw = eg * kBwdWaves + wave;
+  const bool wave_ok = e_raw < p.E;           // padding waves still take part in the barriers
+  const int e = wave_ok ? e_raw : p.E - 1;
+
+  float a2t[kN], a2l[kN];
+#pragma unroll
+  for (int n = 0; n < kN; ++n) { a2t[n] = p.A2T[e * kN + n]; a2l[n] = p.A2L[e * kN + n]; }
+  const float dsk = p.Df[e];
+
+  const int slot = lane >> p.hp_shift, r = lane & (p.HP - 1);
+  const int b = g * p.S + slot;
+  const T* X = static_cast<const T*>(p.x);
+  const T* DT = static_cast<const T*>(p.dT);
+  const T* DL = static_cast<const T*>(p.dL);
+  const T* BTp = static_cast<const T*>(p.BT);
+  const T* BLp = static_cast<const T*>(p.BL);
+  const T* Cp = static_cast<const T*>(p.C);
+  const T* DY = static_cast<const T*>(p.dy);
+  T* DX = static_cast<T*>(p.dx);
+  T* DDT = static_cast<T*>(p.ddT);
+  T* DDL = static_cast<T*>(p.ddL);
+  const int64_t P = (int64_t)p.B * p.H * p.W;
+
+  float accAT[kN], accAL[kN], accD = 0.f;
+  float muT[kN], muL[kN];
+#pragma unroll
+  for (int n = 0; n < kN; ++n) { accAT[n] = 0.f; accAL[n] = 0.f; }
+
+  for (int band = p.nbands - 1; band >= 0; --band) {
+    const int i = band * 64 + r;
+    const int HB = p.nbands == 1 ? p.H : (p.H - band * 64 < 64 ? p.H - band * 64 : 64);
+    const bool row_ok = wave_ok && b < p.B && i < p.H;
+    const int T_steps = p.W + HB - 1;
+    const bool from_top = band > 0 && r == 0;
+    const bool from_bot = band + 1 < p.nbands && r == 63;
+    const int bcl = b < p.B ? b : p.B - 1;
+#pragma unroll
+    for (int n = 0; n < kN; ++n) { muT[n] = 0.f; muL[n] = 0.f; }
+
+    for (int m = (T_steps - 1) / kCK; m >= 0; --m) {
+      const int t0 = m * kCK;
+      float hb[kCK + 1][kN];
+      if (m == 0 || !(row_ok && t0 - 1 - r >= 0 && t0 - 1 - r < p.W)) {
+#pragma unroll
+        for (int n = 0; n < kN; ++n) hb[0][n] = 0.f;
+      } else {
+        const float* ck = p.ckpt + ((((int64_t)g * p.nbands + band) * p.nblk + m) * p.E + e) * (kN * 64) + lane;
+#pragma unroll
+        for (int n = 0; n < kN; ++n) hb[0][n] = ck[n * 64];
+      }
+      // ---- recompute the states of the block
+#pragma unroll
+      for (int k = 0; k < kCK; ++k) {
+        const int t = t0 + k;
+        if (t < T_steps) {
+          const Cell cl = locate(p, b, i, t, r, row_ok);
+          float bt[kN], bl[kN];
+          const float xv = IO<T>::ld(X + cl.idx * p.E + e);
+          const float dtv = IO<T>::ld(DT + cl.idx * p.E + e);
+          const float dlv = IO<T>::ld(DL + cl.idx * p.E + e);
+          IO<T>::ld16(BTp + cl.idx * kN, bt);
+          IO<T>::ld16(BLp + cl.idx * kN, bl);
+          const float* tb = p.top + ((((int64_t)(band > 0 ? band - 1 : 0) * p.B + bcl) * p.W + (cl.act ? cl.j : 0)) * p.E + e) * kN;
+          const float sT = cl.cT * dtv * xv, sL = cl.cL * dlv * xv;
+#pragma unroll
+          for (int n = 0; n < kN; ++n) {
+            const float aT = fexp2(__builtin_fmaf(dtv, a2t[n], cl.offT));
+            const float aL = fexp2(__builtin_fmaf(dlv, a2l[n], cl.offL));
+            float hT = from_lane_below(hb[k][n]);
+            if (from_top) hT = tb[n];
+            float u = sL * bl[n];
+            u = __builtin_fmaf(sT, bt[n], u);
+            u = __builtin_fmaf(aT, hT, u);
+            hb[k + 1][n] = __builtin_fmaf(aL, hb[k][n], u);
+          }
+        }
+      }
+      // ---- adjoint over the block, last step first
+#pragma unroll
+      for (int k = kCK - 1; k >= 0; --k) {
+        const int t = t0 + k;
+        if (t < T_steps) {
+          const Cell cl = locate(p, b, i, t, r, row_ok);
+          float bt[kN], bl[kN], cc[kN];
+          const float xv = IO<T>::ld(X + cl.idx * p.E + e);
+          const float dtv = IO<T>::ld(DT + cl.idx * p.E + e);
+          const float dlv = IO<T>::ld(DL + cl.idx * p.E + e);
+          const float dyv = IO<T>::ld(DY + cl.idx * p.E + e);
+          IO<T>::ld16(BTp + cl.idx * kN, bt);
+          IO<T>::ld16(BLp + cl.idx * kN, bl);
+          IO<T>::ld16(Cp + cl.idx * kN, cc);
+          const float* tb = p.top + ((((int64_t)(band > 0 ? band - 1 : 0) * p.B + bcl) * p.W + (cl.act ? cl.j : 0)) * p.E + e) * kN;
+          float* bb = p.bot + (((int64_t)bcl * p.W + (cl.act ? cl.j : 0)) * p.E + e) * kN;
+          const float qT = cl.cT * dtv * xv, qL = cl.cL * dlv * xv;
+          const float keep = cl.act ? 1.f : 0.f;
+          const float qC = keep * dyv;
+          float sT = 0.f, sL = 0.f, zT = 0.f, zL = 0.f;
+          float4* sw = slots + (size_t)wave * (3 * 4 * 64) + lane;
+          __syncthreads();   // the flush of the previous step has finished reading the slots
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            float vC[4], vBT[4], vBL[4];
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+              const int n = 4 * q + m;
+              const float aT = fexp2(__builtin_fmaf(dtv, a2t[n], cl.offT));
+              const float aL = fexp2(__builtin_fmaf(dlv, a2l[n], cl.offL));
+              float mb = from_lane_above(muT[n]);
+              if (from_bot) mb = __builtin_nontemporal_load(bb + n);
+              const float lam = __builtin_fmaf(dyv, cc[n], muL[n] + mb);
+              float hT = from_lane_below(hb[k][n]);
+              if (from_top) hT = tb[n];
+              const float mT = aT * lam, mL = aL * lam;
+              muT[n] = mT;
+              muL[n] = mL;
+              const float ZT = mT * hT, ZL = mL * hb[k][n];
+              accAT[n] = __builtin_fmaf(ZT, dtv, accAT[n]);
+              accAL[n] = __builtin_fmaf(ZL, dlv, accAL[n]);
+              zT = __builtin_fmaf(ZT, a2t[n], zT);
+              zL = __builtin_fmaf(ZL, a2l[n], zL);
+              sT = __builtin_fmaf(lam, bt[n], sT);
+              sL = __builtin_fmaf(lam, bl[n], sL);
+              vBT[m] = qT * lam;       // qT, qL are zero on inactive lanes
+              vBL[m] = qL * lam;
+              vC[m] = qC * hb[k + 1][n];
+            }
+            // channel sums of the step: per-wave slots, added in wave order by the flush
+            sw[(0 * 4 + q) * 64] = make_float4(vC[0], vC[1], vC[2], vC[3]);
+            sw[(1 * 4 + q) * 64] = make_float4(vBT[0], vBT[1], vBT[2], vBT[3]);
+            sw[(2 * 4 + q) * 64] = make_float4(vBL[0], vBL[1], vBL[2], vBL[3]);
+          }
+          if (from_top && cl.act) {   // hand muT of this band's first row to the band above
+#pragma unroll
+            for (int n = 0; n < kN; ++n) bb[n] = muT[n];
+          }
+          if (cl.act) {
+            accD = __builtin_fmaf(dyv, xv, accD);
+            IO<T>::st(DDT + cl.idx * p.E + e, __builtin_fmaf(cl.cT * xv, sT, kLn2 * zT));
+            IO<T>::st(DDL + cl.idx * p.E + e, __builtin_fmaf(cl.cL * xv, sL, kLn2 * zL));
+            IO<T>::st(DX + cl.idx * p.E + e, __builtin_fmaf(cl.cT * dtv, sT, __builtin_fmaf(cl.cL * dlv, sL, dyv * dsk)));
+          }
+          __syncthreads();
+          for (int it = threadIdx.x; it < 3 * 4 * 64; it += kBwdWaves * 64) {
+            const int fl = it & 63, q = (it >> 6) & 3, v = it >> 8;
+            const int fr = fl & (p.HP - 1), fb = g * p.S + (fl >> p.hp_shift);
+            const int fi = band * 64 + fr, fj = t - fr;
+            if (fb < p.B && fi < p.H && fj >= 0 && fj < p.W) {
+              float4 s = slots[(size_t)(0 * 3 + v) * (4 * 64) + q * 64 + fl];
+#pragma unroll
+              for (int w = 1; w < kBwdWaves; ++w) {
+                const float4 o = slots[(size_t)(w * 3 + v) * (4 * 64) + q * 64 + fl];
+                s.x += o.x; s.y += o.y; s.z += o.z; s.w += o.w;
+              }
+              const int im = p.flip ? p.H - 1 - fi : fi, jm = p.flip ? p.W - 1 - fj : fj;
+              const int64_t cell = ((int64_t)fb * p.H + im) * p.W + jm;
+              *reinterpret_cast<float4*>(p.part + (((int64_t)eg * 3 + v) * P + cell) * kN + 4 * q) = s;
+            }
+          }
+        }
+      }
+    }
+    if (p.nbands > 1) __threadfence();
+  }
+
+  // ---- sums over positions: reduce the 64 lanes, one partial per (group, channel)
+  float red[2 * kN + 1];
+#pragma unroll
+  for (int n = 0; n < kN; ++n) { red[n] = accAT[n]; red[kN + n] = accAL[n]; }
+  red[2 * kN] = accD;
+#pragma unroll
+  for (int k = 0; k < 2 * kN + 1; ++k) {
+    float v = red[k];
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    red[k] = v;
+  }
+  if (wave_ok && lane == 0) {
+    float* pa = p.pA + ((int64_t)g * p.E + e) * (2 * kN);
+#pragma unroll
+    for (int n = 0; n < 2 * kN; ++n) pa[n] = red[n];
+    p.pD[(int64_t)g * p.E + e] = red[2 * kN];
+  }
+}
+
+// -------------------------------------------------------------------------- small helper kernels
+template <typename T>
+__global__ void m2d_prep_kernel(const T* AT, const T* AL, const T* D, float* A2T, float* A2L, float* Df, int E) {
+  const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx < E * kN) {
+    A2T[idx] = IO<T>::ld(AT + idx) * kLog2e;
+    A2L[idx] = IO<T>::ld(AL + idx) * kLog2e;
+  }
+  if (idx < E) Df[idx] = IO<T>::ld(D + idx);
+}
+
+// d_C, d_BT, d_BL: add the per-workgroup channel sums in workgroup order and round to T.
+// d_AT, d_AL, d_D: add the per-group partials in group order.
+template <typename T>
+__global__ void m2d_finalize_kernel(const ScanParams p, T* dC, T* dBT, T* dBL, T* dAT, T* dAL, T* dD) {
+  const int64_t P = (int64_t)p.B * p.H * p.W;
+  const int64_t nquad = 3 * P * (kN / 4);
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid < nquad) {
+    const int64_t v = gid / (P * 4), rem = gid % (P * 4);
+    float4 s = *reinterpret_cast<const float4*>(p.part + (v * P * kN) + rem * 4);
+    for (int egi = 1; egi < p.blocks_per_group; ++egi) {
+      const float4 o = *reinterpret_cast<const float4*>(p.part + (((int64_t)egi * 3 + v) * P * kN) + rem * 4);
+      s.x += o.x; s.y += o.y; s.z += o.z; s.w += o.w;
+    }
+    T* out = v == 0 ? dC : (v == 1 ? dBT : dBL);
+    IO<T>::st4(out + rem * 4, s);
+  }
+  const int64_t k = gid;
+  if (k < (int64_t)p.E * 2 * kN) {
+    const int e = (int)(k / (2 * kN)), w = (int)(k % (2 * kN));
+    float s = 0.f;
+    for (int g = 0; g < p.NG; ++g) s += p.pA[((int64_t)g * p.E + e) * (2 * kN) + w];
+    if (w < kN) IO<T>::st(dAT + e * kN + w, s); else IO<T>::st(dAL + e * kN + (w - kN), s);
+  }
+  if (k < p.E) {
+    float s = 0.f;
+    for (int g = 0; g < p.NG; ++g) s += p.pD[(int64_t)g * p.E + k];
+    IO<T>::st(dD + k, s);
+  }
+}
+
+// ------------------------------------------------------------------------------------ host side
+inline size_t align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
+
+struct Geometry {
+  int HP, hp_shift, S, NG, nbands, nblk;
+  int fwd_ec, fwd_net, fwd_bpg;      // forward: channels per wave, waves per group, workgroups per group
+  int bwd_bpg;                       // backward: workgroups per group (= channel groups EG)
+  size_t prep_bytes, ckpt_diag_bytes, top_bytes, bot_bytes, part_bytes, pa_bytes, pd_bytes;
+};
+
+int check_desc(const m2d_desc* d) {
+  if (!d) return M2D_ERR_NULL_POINTER;
+  if (d->B < 1 || d->E < 1 || d->N < 1 || d->H < 2 || d->W < 2) return M2D_ERR_BAD_SHAPE;
+  if (d->N != kN) return M2D_ERR_UNSUPPORTED;
+  if (d->dtype != M2D_F32 && d->dtype != M2D_BF16) return M2D_ERR_UNSUPPORTED;
+  if (d->reserved != 0 || (d->flags & ~M2D_FLAG_FLIP)) return M2D_ERR_UNSUPPORTED;
+  if ((int64_t)d->B * d->H * d->W >= ((int64_t)1 << 40)) return M2D_ERR_BAD_SHAPE;
+  return M2D_OK;
+}
+
+Geometry make_geometry(const m2d_desc* d) {
+  Geometry g;
+  if (d->H > 32) { g.HP = 64; }
+  else { g.HP = 2; while (g.HP < d->H) g.HP *= 2; }
+  g.hp_shift = 0;
+  while ((1 << g.hp_shift) < g.HP) ++g.hp_shift;
+  g.S = 64 / g.HP;
+  g.NG = (d->B + g.S - 1) / g.S;
+  g.nbands = g.HP == 64 ? (d->H + 63) / 64 : 1;
+  const int hb = d->H < 64 ? d->H : 64;
+  g.nblk = (d->W + hb - 1 + kCK - 1) / kCK;
+  g.fwd_ec = (d->E % 2 == 0) ? 2 : 1;
+  g.fwd_net = d->E / g.fwd_ec;
+  g.fwd_bpg = (g.fwd_net + kFwdWaves - 1) / kFwdWaves;
+  g.bwd_bpg = (d->E + kBwdWaves - 1) / kBwdWaves;
+  const size_t P = (size_t)d->B * d->H * d->W;
+  g.prep_bytes = align_up(sizeof(float) * ((size_t)2 * d->E * kN + d->E));
+  g.ckpt_diag_bytes = align_up(sizeof(float) * (size_t)g.NG * g.nbands * g.nblk * d->E * kN * 64);
+  g.top_bytes = g.nbands > 1 ? align_up(sizeof(float) * (size_t)(g.nbands - 1) * d->B * d->W * d->E * kN) : 0;
+  g.bot_bytes = g.nbands > 1 ? align_up(sizeof(float) * (size_t)d->B * d->W * d->E * kN) : 0;
+  g.part_bytes = align_up(sizeof(float) * (size_t)g.bwd_bpg * 3 * P * kN);
+  g.pa_bytes = align_up(sizeof(float) * (size_t)g.NG * d->E * 2 * kN);
+  g.pd_bytes = align_up(sizeof(float) * (size_t)g.NG * d->E);
+  return g;
+}
+
+size_t ckpt_bytes_of(const Geometry& g) { return g.ckpt_diag_bytes + g.top_bytes; }
+
+size_t workspace_bytes_of(const Geometry& g, int pass, int have_ckpt) {
+  size_t n = g.prep_bytes;
+  if (pass == M2D_PASS_FWD) {
+    if (!have_ckpt) n += g.top_bytes;
+  } else {
+    n += g.part_bytes + g.pa_bytes + g.pd_bytes + g.bot_bytes;
+    if (!have_ckpt) n += ckpt_bytes_of(g);
+  }
+  return n;
+}
+
+bool misaligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
+
+void fill_common(ScanParams& sp, const m2d_desc* d, const Geometry& g) {
+  sp.B = d->B; sp.H = d->H; sp.W = d->W; sp.E = d->E;
+  sp.HP = g.HP; sp.hp_shift = g.hp_shift; sp.S = g.S; sp.NG = g.NG; sp.nbands = g.nbands; sp.nblk = g.nblk;
+  sp.flip = (d->flags & M2D_FLAG_FLIP) ? 1 : 0;
+}
+
+template <typename T>
+int launch_prep(const m2d_desc* d, const void* AT, const void* AL, const void* D, float* base, hipStream_t st) {
+  float* A2T = base;
+  float* A2L = base + (size_t)d->E * kN;
+  float* Df = base + (size_t)2 * d->E * kN;
+  const int n = d->E * kN;
+  hipLaunchKernelGGL(m2d_prep_kernel<T>, dim3((n + 255) / 256), dim3(256), 0, st, static_cast<const T*>(AT),
+                     static_cast<const T*>(AL), static_cast<const T*>(D), A2T, A2L, Df, d->E);
+  return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+}
+
+template <typename T>
+int launch_fwd(const ScanParams& sp0, const Geometry& g, bool ckpt, bool write_y, hipStream_t st) {
+  ScanParams sp = sp0;
+  sp.NET = g.fwd_net;
+  sp.blocks_per_group = g.fwd_bpg;
+  const dim3 grid((unsigned)((size_t)g.NG * g.fwd_bpg)), block(kFwdWaves * 64);
+#define M2D_FWD(EC, CK, WY) hipLaunchKernelGGL((m2d_fwd_kernel<T, EC, CK, WY>), grid, block, 0, st, sp)
+  if (g.fwd_ec == 2) {
+    if (ckpt && write_y) M2D_FWD(2, true, true);
+    else if (ckpt) M2D_FWD(2, true, false);
+    else M2D_FWD(2, false, true);
+  } else {
+    if (ckpt && write_y) M2D_FWD(1, true, true);
+    else if (ckpt) M2D_FWD(1, true, false);
+    else M2D_FWD(1, false, true);
+  }
+#undef M2D_FWD
+  return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+}
+
+template <typename T>
+int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT, const void* AL, const void* D,
+            void* ckpt, void* ws, hipStream_t st) {
+  char* w = static_cast<char*>(ws);
+  float* prep = reinterpret_cast<float*>(w);
+  w += g.prep_bytes;
+  sp.A2T = prep; sp.A2L = prep + (size_t)d->E * kN; sp.Df = prep + (size_t)2 * d->E * kN;
+  if (ckpt) {
+    sp.ckpt = static_cast<float*>(ckpt);
+    sp.top = reinterpret_cast<float*>(static_cast<char*>(ckpt) + g.ckpt_diag_bytes);
+  } else {
+    sp.ckpt = nullptr;
+    sp.top = reinterpret_cast<float*>(w);
+  }
+  int rc = launch_prep<T>(d, AT, AL, D, prep, st);
+  if (rc) return rc;
+  return launch_fwd<T>(sp, g, ckpt != nullptr, true, st);
+}
+
+template <typename T>
+int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT, const void* AL, const void* D,
+            const void* ckpt, void* dAT, void* dAL, void* dBT, void* dBL, void* dC, void* dD, void* ws,
+            hipStream_t st) {
+  char* w = static_cast<char*>(ws);
+  float* prep = reinterpret_cast<float*>(w); w += g.prep_bytes;
+  sp.A2T = prep; sp.A2L = prep + (size_t)d->E * kN; sp.Df = prep + (size_t)2 * d->E * kN;
+  sp.part = reinterpret_cast<float*>(w); w += g.part_bytes;
+  sp.pA = reinterpret_cast<float*>(w); w += g.pa_bytes;
+  sp.pD = reinterpret_cast<float*>(w); w += g.pd_bytes;
+  sp.bot = reinterpret_cast<float*>(w); w += g.bot_bytes;
+  int rc = launch_prep<T>(d, AT, AL, D, prep, st);
+  if (rc) return rc;
+  if (ckpt) {
+    sp.ckpt = const_cast<float*>(static_cast<const float*>(ckpt));
+    sp.top = reinterpret_cast<float*>(const_cast<char*>(static_cast<const char*>(ckpt)) + g.ckpt_diag_bytes);
+  } else {   // rebuild the checkpoints with one forward sweep that writes no y
+    sp.ckpt = reinterpret_cast<float*>(w);
+    sp.top = reinterpret_cast<float*>(w + g.ckpt_diag_bytes);
+    rc = launch_fwd<T>(sp, g, true, false, st);
+    if (rc) return rc;
+  }
+  sp.NET = d->E;
+  sp.blocks_per_group = g.bwd_bpg;
+  const size_t lds = sizeof(float4) * kBwdWaves * 3 * 4 * 64;
+  static bool attr_f32 = false, attr_bf16 = false;   // idempotent, value never changes
+  bool& attr = sizeof(T) == 4 ? attr_f32 : attr_bf16;
+  if (!attr) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_bwd_kernel<T>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return M2D_ERR_HIP;
+    attr = true;
+  }
+  hipLaunchKernelGGL(m2d_bwd_kernel<T>, dim3((unsigned)((size_t)g.NG * g.bwd_bpg)), dim3(kBwdWaves * 64), lds, st, sp);
+  if (hipGetLastError() != hipSuccess) return M2D_ERR_HIP;
+  const int64_t P = (int64_t)d->B * d->H * d->W;
+  int64_t work = 3 * P * (kN / 4);
+  if (work < (int64_t)d->E * 2 * kN) work = (int64_t)d->E * 2 * kN;
+  hipLaunchKernelGGL(m2d_finalize_kernel<T>, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, st, sp,
+                     static_cast<T*>(dC), static_cast<T*>(dBT), static_cast<T*>(dBL), static_cast<T*>(dAT),
+                     static_cast<T*>(dAL), static_cast<T*>(dD));
+  return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------------------- C ABI
+extern "C" {
+
+int m2d_version(void) { return 100; }
+
+const char* m2d_status_str(int status) {
+  switch (status) {
+    case M2D_OK: return "ok";
+    case M2D_ERR_NULL_POINTER: return "null pointer argument";
+    case M2D_ERR_BAD_SHAPE: return "bad shape (all dims >= 1, H >= 2, W >= 2 required)";
+    case M2D_ERR_UNSUPPORTED: return "unsupported dtype, d_state or flags (this build: f32/bf16, N=16)";
+    case M2D_ERR_WORKSPACE: return "workspace or checkpoint buffer too small";
+    case M2D_ERR_MISALIGNED: return "misaligned pointer (tensors 16 B, workspace/checkpoints 256 B)";
+    case M2D_ERR_HIP: return "HIP runtime error";
+    default: return "unknown status";
+  }
+}
+
+int m2d_desc_check(const m2d_desc* desc) { return check_desc(desc); }
+
+size_t m2d_scan_workspace_bytes(const m2d_desc* desc, int pass, int have_ckpt) {
+  if (check_desc(desc) != M2D_OK || (pass != M2D_PASS_FWD && pass != M2D_PASS_BWD)) return 0;
+  return workspace_bytes_of(make_geometry(desc), pass, have_ckpt);
+}
+
+size_t m2d_scan_ckpt_bytes(const m2d_desc* desc) {
+  if (check_desc(desc) != M2D_OK) return 0;
+  return ckpt_bytes_of(make_geometry(desc));
+}
+
+int m2d_scan_fwd(const m2d_desc* desc, const void* x, const void* deltaT, const void* deltaL, const void* AT,
+                 const void* AL, const void* BT, const void* BL, const void* C, const void* D, void* y, void* ckpt,
+                 size_t ckpt_bytes, void* workspace, size_t workspace_bytes, void* stream) {
+  int rc = check_desc(desc);
+  if (rc) return rc;
+  const void* req[] = {x, deltaT, deltaL, AT, AL, BT, BL, C, D, y, workspace};
+  for (const void* q : req) if (!q) return M2D_ERR_NULL_POINTER;
+  for (const void* q : req) if (misaligned(q, 16)) return M2D_ERR_MISALIGNED;
+  if (misaligned(workspace, 256) || (ckpt && misaligned(ckpt, 256))) return M2D_ERR_MISALIGNED;
+  const Geometry g = make_geometry(desc);
+  if (workspace_bytes < workspace_bytes_of(g, M2D_PASS_FWD, ckpt != nullptr)) return M2D_ERR_WORKSPACE;
+  if (ckpt && ckpt_bytes < ckpt_bytes_of(g)) return M2D_ERR_WORKSPACE;
+  ScanParams sp = {};
+  fill_common(sp, desc, g);
+  sp.x = x; sp.dT = deltaT; sp.dL = deltaL; sp.BT = BT; sp.BL = BL; sp.C = C; sp.y = y;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return desc->dtype == M2D_F32 ? run_fwd<float>(desc, g, sp, AT, AL, D, ckpt, workspace, st)
+                                : run_fwd<bf16_t>(desc, g, sp, AT, AL, D, ckpt, workspace, st);
+}
+
+int m2d_scan_bwd(const m2d_desc* desc, const void* x, const void* deltaT, const void* deltaL, const void* AT,
+                 const void* AL, const void* BT, const void* BL, const void* C, const void* D, const void* dy,
+                 const void* ckpt, size_t ckpt_bytes, void* dx, void* d_deltaT, void* d_deltaL, void* d_AT,
+                 void* d_AL, void* d_BT, void* d_BL, void* d_C, void* d_D, void* workspace,
+                 size_t workspace_bytes, void* stream) {
+  int rc = check_desc(desc);
+  if (rc) return rc;
+  const void* req[] = {x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, dx, d_deltaT, d_deltaL,
+                       d_AT, d_AL, d_BT, d_BL, d_C, d_D, workspace};
+  for (const void* q : req) if (!q) return M2D_ERR_NULL_POINTER;
+  for (const void* q : req) if (misaligned(q, 16)) return M2D_ERR_MISALIGNED;
+  if (misaligned(workspace, 256) || (ckpt && misaligned(ckpt, 256))) return M2D_ERR_MISALIGNED;
+  const Geometry g = make_geometry(desc);
+  if (workspace_bytes < workspace_bytes_of(g, M2D_PASS_BWD, ckpt != nullptr)) return M2D_ERR_WORKSPACE;
+  if (ckpt && ckpt_bytes < ckpt_bytes_of(g)) return M2D_ERR_WORKSPACE;
+  ScanParams sp = {};
+  fill_common(sp, desc, g);
+  sp.x = x; sp.dT = deltaT; sp.dL = deltaL; sp.BT = BT; sp.BL = BL; sp.C = C; sp.dy = dy;
+  sp.dx = dx; sp.ddT = d_deltaT; sp.ddL = d_deltaL;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return desc->dtype == M2D_F32
+             ? run_bwd<float>(desc, g, sp, AT, AL, D, ckpt, d_AT, d_AL, d_BT, d_BL, d_C, d_D, workspace, st)
+             : run_bwd<bf16_t>(desc, g, sp, AT, AL, D, ckpt, d_AT, d_AL, d_BT, d_BL, d_C, d_D, workspace, st);
+}
+
+}  // extern "C"
