@@ -113,6 +113,14 @@ int m2d_scan_bwd(const m2d_desc* desc,
                  void* workspace, size_t workspace_bytes,
                  void* stream);
 
+/* Measurement aid; no counterpart in the reference.  While enabled, every m2d_scan_fwd /
+ * m2d_scan_bwd call records a pair of HIP events on its stream around the main scan kernel of
+ * the pass (not around the small set-up and reduction kernels).  m2d_profile_last_ms waits for
+ * the most recent such pair and returns the elapsed milliseconds.  The events are process-wide:
+ * enable it only from a single-threaded benchmark. */
+int m2d_profile_enable(int on);
+int m2d_profile_last_ms(int pass, float* ms);
+
 #ifdef __cplusplus
 }
 #endif

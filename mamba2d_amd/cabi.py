@@ -18,7 +18,7 @@ M2D_FLAG_FLIP = 1
 M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
-           "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_bwd")
+           "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_bwd", "m2d_profile_enable", "m2d_profile_last_ms")
 
 
 class Desc(ctypes.Structure):
@@ -52,10 +52,24 @@ def _load():
     lib.m2d_scan_fwd.argtypes = [dp] + [vp] * 9 + [vp, vp, sz, vp, sz, vp]
     lib.m2d_scan_bwd.restype = i32
     lib.m2d_scan_bwd.argtypes = [dp] + [vp] * 10 + [vp, sz] + [vp] * 9 + [vp, sz, vp]
+    lib.m2d_profile_enable.restype = i32
+    lib.m2d_profile_enable.argtypes = [i32]
+    lib.m2d_profile_last_ms.restype = i32
+    lib.m2d_profile_last_ms.argtypes = [i32, ctypes.POINTER(ctypes.c_float)]
     return lib
 
 
 lib = _load()
+
+
+def profile_enable(on: bool) -> None:
+    check(lib.m2d_profile_enable(int(on)))
+
+
+def profile_last_ms(which: int) -> float:
+    ms = ctypes.c_float(0.0)
+    check(lib.m2d_profile_last_ms(which, ctypes.byref(ms)))
+    return float(ms.value)
 
 
 def status_str(code: int) -> str:

@@ -488,6 +488,10 @@ __global__ void m2d_finalize_kernel(const ScanParams p, T* dC, T* dBT, T* dBL, T
 }
 
 // ------------------------------------------------------------------------------------ host side
+// Optional timing of the main kernel of each pass (off by default; see m2d_profile_enable).
+bool g_profile = false;
+hipEvent_t g_ev[2][2] = {{nullptr, nullptr}, {nullptr, nullptr}};
+
 inline size_t align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
 
 struct Geometry {
@@ -601,7 +605,10 @@ int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   }
   int rc = launch_prep<T>(d, AT, AL, D, prep, st);
   if (rc) return rc;
-  return launch_fwd<T>(sp, g, ckpt != nullptr, true, st);
+  if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_FWD][0], st);
+  rc = launch_fwd<T>(sp, g, ckpt != nullptr, true, st);
+  if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_FWD][1], st);
+  return rc;
 }
 
 template <typename T>
@@ -637,7 +644,9 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
       return M2D_ERR_HIP;
     attr = true;
   }
+  if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][0], st);
   hipLaunchKernelGGL(m2d_bwd_kernel<T>, dim3((unsigned)((size_t)g.NG * g.bwd_bpg)), dim3(kBwdWaves * 64), lds, st, sp);
+  if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][1], st);
   if (hipGetLastError() != hipSuccess) return M2D_ERR_HIP;
   const int64_t P = (int64_t)d->B * d->H * d->W;
   int64_t work = 3 * P * (kN / 4);
@@ -669,6 +678,23 @@ const char* m2d_status_str(int status) {
 }
 
 int m2d_desc_check(const m2d_desc* desc) { return check_desc(desc); }
+
+int m2d_profile_enable(int on) {
+  if (on && !g_ev[0][0]) {
+    for (auto& pr : g_ev)
+      for (auto& ev : pr)
+        if (hipEventCreate(&ev) != hipSuccess) return M2D_ERR_HIP;
+  }
+  g_profile = on != 0;
+  return M2D_OK;
+}
+
+int m2d_profile_last_ms(int pass, float* ms) {
+  if (!ms) return M2D_ERR_NULL_POINTER;
+  if ((pass != M2D_PASS_FWD && pass != M2D_PASS_BWD) || !g_ev[0][0]) return M2D_ERR_UNSUPPORTED;
+  if (hipEventSynchronize(g_ev[pass][1]) != hipSuccess) return M2D_ERR_HIP;
+  return hipEventElapsedTime(ms, g_ev[pass][0], g_ev[pass][1]) == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+}
 
 size_t m2d_scan_workspace_bytes(const m2d_desc* desc, int pass, int have_ckpt) {
   if (check_desc(desc) != M2D_OK || (pass != M2D_PASS_FWD && pass != M2D_PASS_BWD)) return 0;

@@ -1,0 +1,125 @@
+"""GPU tests of the Python operator surface (mamba2d_amd.wavefront) through the PyTorch shim:
+autograd Functions with the reference's signatures, entry point, both recompute modes."""
+import math
+
+import pytest
+import torch
+
+from oracle import scan_oracle as so
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def wf():
+    from mamba2d_amd import wavefront
+    return wavefront
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 2e-2)], ids=["f32", "bf16"])
+@pytest.mark.parametrize("save", [True, False], ids=["ckpt_saved", "ckpt_rebuilt"])
+def test_fn_pr_forward_backward(wf, cscan, dtype, tol, save):
+    say(f"\ncase fn_pr {dtype} save={save}")
+    inp = so.make_inputs(4, 14, 14, 16, 16, seed=11, dtype=dtype)
+    leaves = [inp[k].cuda().requires_grad_(True) for k in so.INPUT_NAMES]
+    old = wf.SAVE_CHECKPOINTS
+    wf.SAVE_CHECKPOINTS = save
+    try:
+        y = wf.wf_cuda_fn_pr.apply(*leaves)
+        grads = torch.autograd.grad(y, leaves, inp["dy"].cuda())
+    finally:
+        wf.SAVE_CHECKPOINTS = old
+    ref_in = [inp[k].double() for k in so.INPUT_NAMES]
+    assert y.dtype == dtype and so.rel_err(y.float().cpu(), cscan.forward(*ref_in)) < tol
+    g_ref = cscan.backward(*ref_in, inp["dy"].double())
+    for k, g, leaf in zip(so.CScan.GRADS, grads, leaves):
+        assert g.dtype == leaf.dtype and g.shape == leaf.shape
+        assert so.rel_err(g.float().cpu(), g_ref[k]) < tol, k
+
+
+def make_block_params(E, N, R, seed, device):
+    """Parameters shaped and initialised like M2DBlock's (models/mamba2d.py:57-111)."""
+    g = torch.Generator().manual_seed(seed)
+    dt = torch.exp(torch.rand(E, generator=g) * (math.log(0.1) - math.log(0.001)) + math.log(0.001)).clamp(min=1e-4)
+    inv_dt = dt + torch.log(-torch.expm1(-dt))
+    std = R ** -0.5
+    p = dict(
+        AT_log=torch.log(torch.arange(1, N + 1, dtype=torch.float32).repeat(E, 1)),
+        AL_log=torch.log(torch.arange(1, N + 1, dtype=torch.float32).repeat(E, 1)),
+        x_proj_w=(torch.rand(2 * R + 3 * N, E, generator=g) * 2 - 1) / math.sqrt(E),
+        dt_projT_w=(torch.rand(E, R, generator=g) * 2 - 1) * std, dt_projT_b=inv_dt.clone(),
+        dt_projL_w=(torch.rand(E, R, generator=g) * 2 - 1) * std, dt_projL_b=inv_dt.clone(),
+        D=torch.ones(E))
+    return {k: v.to(device) for k, v in p.items()}
+
+
+ORDER = ("AT_log", "AL_log", "x_proj_w", "dt_projT_w", "dt_projT_b", "dt_projL_w", "dt_projL_b", "D")
+
+
+@pytest.mark.parametrize("recomp", ["partial", "full"])
+def test_entry_point_matches_oracle_fp32(wf, recomp):
+    say(f"\ncase entry_point {recomp}")
+    B, H, W, E, N = 2, 9, 12, 32, 16
+    R = math.ceil(E / 16)
+    p = make_block_params(E, N, R, 0, "cuda")
+    x = torch.randn(B, H, W, E, generator=torch.Generator().manual_seed(1)).cuda()
+    dy = torch.randn(B, H, W, E, generator=torch.Generator().manual_seed(2)).cuda()
+    leaves = [x.clone().requires_grad_(True)] + [p[k].clone().requires_grad_(True) for k in ORDER]
+    y = wf.wavefront_scan_cuda(*leaves, recomp=recomp)
+    grads = torch.autograd.grad(y, leaves, dy)
+    # oracle: same projections in fp64 on the CPU, scan by the differentiable restatement
+    ref_leaves = [t.detach().double().cpu().requires_grad_(True) for t in leaves]
+    y_ref = so.wavefront_scan_ref(*ref_leaves)
+    g_ref = torch.autograd.grad(y_ref, ref_leaves, dy.double().cpu())
+    assert so.rel_err(y.cpu(), y_ref.detach()) < 1e-4
+    for name, g, gr in zip(("x",) + ORDER, grads, g_ref):
+        assert so.rel_err(g.cpu(), gr) < 2e-4, name
+
+
+def test_partial_and_full_agree_bf16(wf):
+    """The two recompute modes are the same function of the nine raw inputs."""
+    say("\ncase partial_vs_full bf16")
+    B, H, W, E, N = 3, 14, 14, 64, 16
+    R = math.ceil(E / 16)
+    p = make_block_params(E, N, R, 3, "cuda")
+    x = torch.randn(B, H, W, E, generator=torch.Generator().manual_seed(4)).cuda().bfloat16()
+    dy = torch.randn(B, H, W, E, generator=torch.Generator().manual_seed(5)).cuda().bfloat16()
+    outs = {}
+    for mode in ("partial", "full"):
+        leaves = [x.clone().requires_grad_(True)] + [p[k].clone().requires_grad_(True) for k in ORDER]
+        y = wf.wavefront_scan_cuda(*leaves, recomp=mode)
+        outs[mode] = (y, torch.autograd.grad(y, leaves, dy))
+    assert y.dtype == torch.bfloat16
+    assert torch.equal(outs["partial"][0], outs["full"][0])
+    for a, b in zip(outs["partial"][1], outs["full"][1]):
+        assert a.dtype == b.dtype and so.rel_err(a.float().cpu(), b.float().cpu()) < 2e-2
+
+
+def test_small_spatial_dims_raise_on_gpu(wf):
+    p = make_block_params(4, 16, 1, 0, "cuda")
+    with pytest.raises(ValueError, match="spatial dims > 1"):
+        wf.wavefront_scan_cuda(torch.zeros(1, 1, 8, 4, device="cuda"), *[p[k] for k in ORDER])
+
+
+def test_wrong_shapes_and_dtypes_are_rejected(wf):
+    inp = so.make_inputs(1, 4, 4, 4, 16, seed=0)
+    a = [inp[k].cuda() for k in so.INPUT_NAMES]
+    bad = list(a)
+    bad[5] = bad[5][:, :, :3].contiguous()          # BT with the wrong width
+    with pytest.raises(RuntimeError, match="BT has shape"):
+        wf.scan_fwd_op(*bad, False, False)
+    bad = list(a)
+    bad[1] = bad[1].bfloat16()
+    with pytest.raises(RuntimeError, match="share one dtype"):
+        wf.scan_fwd_op(*bad, False, False)
+    bad = [t.double() for t in a]
+    with pytest.raises(RuntimeError, match="float32 and bfloat16"):
+        wf.scan_fwd_op(*bad, False, False)
+    a8 = [inp[k][..., :8].contiguous().cuda() if k in ("AT", "AL", "BT", "BL", "C") else inp[k].cuda()
+          for k in so.INPUT_NAMES]
+    with pytest.raises(RuntimeError, match="unsupported"):
+        wf.scan_fwd_op(*a8, False, False)
