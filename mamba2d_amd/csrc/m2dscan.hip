@@ -1,30 +1,36 @@
 // m2dscan: wavefront 2-D selective scan for gfx950 (MI355X), forward and backward.
 //
-// Mapping (both passes).  The recurrence  h[i,j] = cL*(aL*h[i,j-1] + uL) + cT*(aT*h[i-1,j] + uT)
-// (reference: models/kernels/wf_cuda/wf_cuda.cu:40-69) is independent across (batch, channel,
-// state).  One 64-lane wavefront owns a few channels of one problem and sweeps it
-// anti-diagonal by anti-diagonal: lane r holds grid row r and at step t works on the cell
-// (r, t-r), so one step of the wave IS one anti-diagonal.  The 16 states of a cell stay in
-// VGPRs; h[i,j-1] is the lane's own previous value and h[i-1,j] is the previous value of lane
-// r-1, fetched with a DPP wave shift.  y = C.h is a 16-term in-register sum.  Grids with
-// fewer than 33 rows are packed several problems per wave (power-of-two lane slots); grids
-// with more than 64 rows are cut in bands of 64 rows whose boundary rows travel through
-// memory.
+// The recurrence (reference: models/kernels/wf_cuda/wf_cuda.cu:40-69)
+//     h[i,j] = cL*(aL*h[i,j-1] + uL) + cT*(aT*h[i-1,j] + uT),   a = exp(delta*A),  u = delta*B*x
+// with (cT,cL) = (0,1) on the first row, (1,0) on the first column and (1/2,1/2) inside, is
+// independent across (batch, channel, state).
 //
-// The interior factor 1/2 and the first-row/column special cases are folded into the gate
-// exponent (exp2(delta*A*log2e + log2 c)) and into the input coefficient, so the inner loop
-// has no branches.
+// Mapping.  The grid rows are cut in bands of HB rows (HB = 16 for most shapes).  A 64-lane
+// wavefront owns CS = 64/HB channel slots of one image: lane = slot*HB + r holds band row r of
+// its channel(s).  At step t the lane works on the cell (row r, column t-r): one step of the
+// wave is one anti-diagonal of the band for CS channels at once.  The 16 states of the cell
+// stay in VGPRs; h[i,j-1] is the lane's own previous value, h[i-1,j] is the previous value of
+// the lane below, fetched with a DPP wave shift; the first row of a band takes it from the
+// last row of the band above, which travels through a small buffer in memory.  y = C.h is a
+// 16-term sum in registers.  Short bands keep the skew waste low (W/(W+HB-1) of the steps do
+// useful work) and put several channels of the same cell in one wave, which the backward
+// needs for its channel sums.
 //
-// Backward (adjoint of the above; reference wf_cuda.cu:108-160 and
-// models/kernels/wavefront_cuda.py:97-139,176-178,193-194).  The forward stores the wave's
-// register state every CK steps (a checkpoint is one anti-diagonal).  The backward walks the
-// blocks of CK steps in reverse: it restores the checkpoint, recomputes the CK states of the
-// block into registers, then runs the adjoint over the block backwards, with
-//     lambda = dy*C + muL(own, previous step) + muT(lane r+1, previous step)
+// The factor 1/2 and the first-row/column cases are folded into the gate exponent
+// (exp2(delta*A*log2e + log2 c)) and into the input coefficient: the inner loop is branch-free.
+//
+// Backward (adjoint; reference wf_cuda.cu:108-160 and models/kernels/wavefront_cuda.py:97-139,
+// 176-178, 193-194).  The forward stores the register state every CK steps (one anti-diagonal
+// of the band per checkpoint).  The backward walks bands bottom-up and, inside a band, the
+// blocks of CK steps in reverse: restore the checkpoint, recompute the CK states into
+// registers, then run the adjoint over the block backwards,
+//     lambda = dy*C + muL(own, previous step) + muT(lane above, previous step)
 //     muT = cT*aT*lambda,  muL = cL*aL*lambda
-// and emits all gradients on the fly.  Sums over channels (d_BT, d_BL, d_C) go through
-// per-wave LDS slots that are added in a fixed order; sums over positions (d_AT, d_AL, d_D)
-// are register accumulators reduced at the end.  Everything is deterministic.
+// emitting every gradient on the fly.  Channel sums (d_BT, d_BL, d_C) are reduced inside the
+// wave with lane-swap butterflies over the channel slots, then across the 8 waves of the
+// workgroup through LDS in a fixed order, then across workgroups by a small kernel.  Sums over
+// positions (d_AT, d_AL, d_D) are register accumulators reduced at the end.  No atomics:
+// results are bit-reproducible.
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -37,6 +43,8 @@ constexpr int kN = 16;            // states per channel
 #define M2D_CK 4
 #endif
 constexpr int kCK = M2D_CK;       // checkpoint interval (steps)
+constexpr int kHB = 16;           // rows per band = lanes per DPP row
+constexpr int kHBShift = 4;
 constexpr int kFwdWaves = 4;      // waves per forward workgroup
 constexpr int kBwdWaves = 8;      // waves per backward workgroup
 constexpr float kLog2e = 1.4426950408889634f;
@@ -64,11 +72,6 @@ template <> struct IO<float> {
     if constexpr (EC == 2) { *reinterpret_cast<float2*>(p) = make_float2(v[0], v[1]); }
     else { for (int c = 0; c < EC; ++c) p[c] = v[c]; }
   }
-  static __device__ __forceinline__ void ld16(const float* p, float (&v)[kN]) {
-    const float4* q = reinterpret_cast<const float4*>(p);
-#pragma unroll
-    for (int k = 0; k < 4; ++k) { float4 t = q[k]; v[4*k] = t.x; v[4*k+1] = t.y; v[4*k+2] = t.z; v[4*k+3] = t.w; }
-  }
   static __device__ __forceinline__ void st4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
 };
 template <> struct IO<bf16_t> {
@@ -85,19 +88,6 @@ template <> struct IO<bf16_t> {
       *reinterpret_cast<uint32_t*>(p) = (uint32_t)f32_to_bf16_bits(v[0]) | ((uint32_t)f32_to_bf16_bits(v[1]) << 16);
     } else { for (int c = 0; c < EC; ++c) p[c].v = f32_to_bf16_bits(v[c]); }
   }
-  static __device__ __forceinline__ void ld16(const bf16_t* p, float (&v)[kN]) {
-    const uint4* q = reinterpret_cast<const uint4*>(p);
-#pragma unroll
-    for (int k = 0; k < 2; ++k) {
-      uint4 t = q[k];
-      uint32_t w[4] = {t.x, t.y, t.z, t.w};
-#pragma unroll
-      for (int m = 0; m < 4; ++m) {
-        v[8*k + 2*m] = __uint_as_float(w[m] << 16);
-        v[8*k + 2*m + 1] = __uint_as_float(w[m] & 0xffff0000u);
-      }
-    }
-  }
   static __device__ __forceinline__ void st4(bf16_t* p, float4 v) {
     uint2 t;
     t.x = (uint32_t)f32_to_bf16_bits(v.x) | ((uint32_t)f32_to_bf16_bits(v.y) << 16);
@@ -106,29 +96,64 @@ template <> struct IO<bf16_t> {
   }
 };
 
-// lane l receives the value of lane l-1 (lane 0 receives 0)
-__device__ __forceinline__ float from_lane_below(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x138 /*wave_shr:1*/, 0xf, 0xf, true));
+__device__ __forceinline__ void ld16f(const float* p, float (&v)[kN]) {
+  const float4* q = reinterpret_cast<const float4*>(p);
+#pragma unroll
+  for (int k = 0; k < 4; ++k) { float4 t = q[k]; v[4*k] = t.x; v[4*k+1] = t.y; v[4*k+2] = t.z; v[4*k+3] = t.w; }
 }
-// lane l receives the value of lane l+1 (lane 63 receives 0)
-__device__ __forceinline__ float from_lane_above(float v) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x130 /*wave_shl:1*/, 0xf, 0xf, true));
+
+// Rows of 16 lanes (one band of one channel slot).  Lane r receives the value of lane r-1 of its
+// row; lane 0 of each row, which has no lane below, keeps `edge` (the state of the last row of
+// the band above, or 0).
+__device__ __forceinline__ float from_row_below(float v, float edge) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(edge), __float_as_int(v), 0x111 /*row_shr:1*/, 0xf, 0xf, false));
+}
+// Lane r receives the value of lane r+1 of its row; lane 15 keeps `edge`.
+__device__ __forceinline__ float from_row_above(float v, float edge) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(edge), __float_as_int(v), 0x101 /*row_shl:1*/, 0xf, 0xf, false));
 }
 __device__ __forceinline__ float fexp2(float v) { return __builtin_amdgcn_exp2f(v); }
 
+// a[lanes 32..63] <-> b[lanes 0..31]; returns a+b: lanes 0..31 hold the two-half sum of a,
+// lanes 32..63 that of b.
+__device__ __forceinline__ float fold32(float a, float b) {
+  auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+// rows of 16 lanes: a.row1 <-> b.row0, a.row3 <-> b.row2; returns a+b: even rows hold the
+// (row, row+1) sum of a, odd rows that of b.
+__device__ __forceinline__ float fold16(float a, float b) {
+  auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+  return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 struct ScanParams {
-  const void *x, *dT, *dL, *BT, *BL, *C, *dy;
+  const void *x, *dT, *dL, *dy;
+  const float *bt, *bl, *cc;        // B_T, B_L, C in fp32, element (cell, n) at [cell*bc_stride + n]
   const float *A2T, *A2L, *Df;      // A*log2(e) and D in fp32, (E,16) / (E)
   void *y, *dx, *ddT, *ddL;
-  float* ckpt;                      // [NG][nbands][nblk][E][16][64]
-  float* top;                       // [nbands-1][B][W][E][16]  last row of each band (forward states)
-  float* bot;                       // [B][W][E][16]            first-row muT of the band below (adjoint)
-  float* part;                      // [EG][3][P][16]           per-workgroup channel sums
-  float* pA;                        // [NG][E][2][16]
-  float* pD;                        // [NG][E]
+  float* ckpt;                      // [B][nbands][nblk][E][16][HB]  state snapshots
+  float* top;                       // [nbands-1][B][W][E][16]       last row of each band (forward states)
+  float* bot;                       // [B][W][E][16]                 first-row muT of the band below (adjoint)
+  float* part;                      // [G][3][P][16]                 per-workgroup channel sums
+  float* pA;                        // [B][E][2][16]
+  float* pD;                        // [B][E]
   int B, H, W, E;
-  int HP, hp_shift, S, NG, nbands, nblk, blocks_per_group, NET, flip;
+  int nbands, nblk, bc_stride, flip;
+  int wpb;                          // waves per image (channel groups of CS*EC channels)
+  int bpb;                          // workgroups per image
+  int nwg;                          // total workgroups
 };
+
+// Workgroups are dealt round-robin to the 8 XCDs; renumber so that consecutive logical ids
+// (the channel groups of one image, which share B, C and cache lines of x) sit on one XCD and
+// therefore share its L2.
+__device__ __forceinline__ int logical_block(int nwg) {
+  const int id = blockIdx.x;
+  const int per = nwg >> 3;
+  if (per == 0 || id >= (per << 3)) return id;
+  return (id & 7) * per + (id >> 3);
+}
 
 struct Cell {          // what a lane needs to know about its cell at one step
   bool act;
@@ -142,109 +167,122 @@ __device__ __forceinline__ Cell locate(const ScanParams& p, int b, int i, int t,
   const int j = t - r;
   c.j = j;
   c.act = row_ok && j >= 0 && j < p.W;
-  const int bc = b < p.B ? b : p.B - 1;
   const int ic = i < p.H ? i : p.H - 1;
   const int jc = j < 0 ? 0 : (j < p.W ? j : p.W - 1);
   const int im = p.flip ? p.H - 1 - ic : ic;
   const int jm = p.flip ? p.W - 1 - jc : jc;
-  c.idx = ((int64_t)bc * p.H + im) * p.W + jm;
+  c.idx = ((int64_t)b * p.H + im) * p.W + jm;
   const float ninf = -__builtin_huge_valf();
   if (!c.act)      { c.cT = 0.f;  c.cL = 0.f;  c.offT = ninf; c.offL = ninf; }
-  else if (i == 0) { c.cT = 0.f;  c.cL = 1.f;  c.offT = ninf; c.offL = 0.f; }
+  else if (i == 0) { c.cT = 0.f;  c.cL = 1.f;  c.offT = ninf; c.offL = j == 0 ? ninf : 0.f; }
   else if (j == 0) { c.cT = 1.f;  c.cL = 0.f;  c.offT = 0.f;  c.offL = ninf; }
   else             { c.cT = 0.5f; c.cL = 0.5f; c.offT = -1.f; c.offL = -1.f; }
   return c;
 }
 
 // ------------------------------------------------------------------------------------ forward
+template <int EC>
+struct FwdLoad {           // operands of one step, as loaded
+  float x[EC], dt[EC], dl[EC];
+  float bt[kN], bl[kN], cc[kN];
+};
+
 template <typename T, int EC, bool CKPT, bool WRITE_Y>
 __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParams p) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int g = blockIdx.x / p.blocks_per_group;
-  const int et = (blockIdx.x % p.blocks_per_group) * kFwdWaves + wave;
-  if (et >= p.NET) return;
-  const int e0 = et * EC;
+  const int lb = logical_block(p.nwg);
+  const int b = lb / p.bpb;
+  const int wv = (lb % p.bpb) * kFwdWaves + wave;
+  if (wv >= p.wpb) return;
+  const int slot = lane >> kHBShift, r = lane & (kHB - 1);
+  constexpr int CS = 64 >> kHBShift;
+  const int e_raw = (wv * CS + slot) * EC;
+  const bool ch_ok = e_raw < p.E;
+  const int e0 = ch_ok ? e_raw : p.E - EC;
 
   float a2t[EC][kN], a2l[EC][kN], dsk[EC];
 #pragma unroll
   for (int c = 0; c < EC; ++c) {
-#pragma unroll
-    for (int n = 0; n < kN; ++n) { a2t[c][n] = p.A2T[(e0 + c) * kN + n]; a2l[c][n] = p.A2L[(e0 + c) * kN + n]; }
+    ld16f(p.A2T + (e0 + c) * kN, a2t[c]);
+    ld16f(p.A2L + (e0 + c) * kN, a2l[c]);
     dsk[c] = p.Df[e0 + c];
   }
 
-  const int slot = lane >> p.hp_shift, r = lane & (p.HP - 1);
-  const int b = g * p.S + slot;
   const T* X = static_cast<const T*>(p.x);
   const T* DT = static_cast<const T*>(p.dT);
   const T* DL = static_cast<const T*>(p.dL);
-  const T* BTp = static_cast<const T*>(p.BT);
-  const T* BLp = static_cast<const T*>(p.BL);
-  const T* Cp = static_cast<const T*>(p.C);
   T* Y = static_cast<T*>(p.y);
 
   for (int band = 0; band < p.nbands; ++band) {
-    const int i = band * 64 + r;
-    const int HB = p.nbands == 1 ? p.H : (p.H - band * 64 < 64 ? p.H - band * 64 : 64);
-    const bool row_ok = b < p.B && i < p.H;
-    const int T_steps = p.W + HB - 1;
+    const int i = band * kHB + r;
+    const int HBk = p.H - band * kHB < kHB ? p.H - band * kHB : kHB;
+    const bool row_ok = ch_ok && r < HBk;
+    const int T_steps = p.W + HBk - 1;
+    const bool from_top = band > 0 && r == 0;
+    const bool to_top = band + 1 < p.nbands && r == kHB - 1;
     float h[EC][kN];
 #pragma unroll
     for (int c = 0; c < EC; ++c)
 #pragma unroll
       for (int n = 0; n < kN; ++n) h[c][n] = 0.f;
 
+    auto load = [&](int t, FwdLoad<EC>& o) {
+      const Cell cl = locate(p, b, i, t, r, row_ok);
+      IO<T>::template ldv<EC>(X + cl.idx * p.E + e0, o.x);
+      IO<T>::template ldv<EC>(DT + cl.idx * p.E + e0, o.dt);
+      IO<T>::template ldv<EC>(DL + cl.idx * p.E + e0, o.dl);
+      ld16f(p.bt + cl.idx * p.bc_stride, o.bt);
+      ld16f(p.bl + cl.idx * p.bc_stride, o.bl);
+      if (WRITE_Y) ld16f(p.cc + cl.idx * p.bc_stride, o.cc);
+    };
+
+    FwdLoad<EC> nxt;
+    load(0, nxt);
     for (int t = 0; t < T_steps; ++t) {
       // snapshot of the state after step t-1; lanes that have not started or are past the last
       // column hold nothing the backward needs
       if (CKPT && t > 0 && (t % kCK) == 0 && row_ok && t - 1 - r >= 0 && t - 1 - r < p.W) {
-        float* ck = p.ckpt + ((((int64_t)g * p.nbands + band) * p.nblk + t / kCK) * p.E + e0) * (kN * 64) + lane;
+        float* ck = p.ckpt + (((((int64_t)b * p.nbands + band) * p.nblk + t / kCK) * p.E + e0) * kN) * kHB + r;
 #pragma unroll
         for (int c = 0; c < EC; ++c)
 #pragma unroll
-          for (int n = 0; n < kN; ++n) ck[(c * kN + n) * 64] = h[c][n];
+          for (int n = 0; n < kN; ++n) ck[(c * kN + n) * kHB] = h[c][n];
       }
+      const FwdLoad<EC> cur = nxt;
+      if (t + 1 < T_steps) load(t + 1, nxt);   // operands of the next step fly during this one
       const Cell cl = locate(p, b, i, t, r, row_ok);
-      float xv[EC], dtv[EC], dlv[EC], bt[kN], bl[kN], cc[kN];
-      IO<T>::template ldv<EC>(X + cl.idx * p.E + e0, xv);
-      IO<T>::template ldv<EC>(DT + cl.idx * p.E + e0, dtv);
-      IO<T>::template ldv<EC>(DL + cl.idx * p.E + e0, dlv);
-      IO<T>::ld16(BTp + cl.idx * kN, bt);
-      IO<T>::ld16(BLp + cl.idx * kN, bl);
-      if (WRITE_Y) IO<T>::ld16(Cp + cl.idx * kN, cc);
-      const bool from_top = band > 0 && r == 0;
       float yv[EC];
 #pragma unroll
       for (int c = 0; c < EC; ++c) {
-        const float sT = cl.cT * dtv[c] * xv[c];
-        const float sL = cl.cL * dlv[c] * xv[c];
+        const float sT = cl.cT * cur.dt[c] * cur.x[c];
+        const float sL = cl.cL * cur.dl[c] * cur.x[c];
         float tp[kN];
-        if (from_top) {   // only lanes on the first row of a lower band (wave-divergent, rare)
-          const float* tb = p.top + ((((int64_t)(band - 1) * p.B + (b < p.B ? b : p.B - 1)) * p.W +
-                                      (cl.act ? cl.j : 0)) * p.E + e0 + c) * kN;
+#pragma unroll
+        for (int n = 0; n < kN; ++n) tp[n] = 0.f;
+        if (from_top) {   // first row of a lower band: the row above lives in memory
+          const float* tb = p.top + ((((int64_t)(band - 1) * p.B + b) * p.W + (cl.act ? cl.j : 0)) * p.E + e0 + c) * kN;
 #pragma unroll
           for (int n = 0; n < kN; ++n) tp[n] = __builtin_nontemporal_load(tb + n);
         }
         float acc = 0.f;
 #pragma unroll
         for (int n = 0; n < kN; ++n) {
-          const float aT = fexp2(__builtin_fmaf(dtv[c], a2t[c][n], cl.offT));
-          const float aL = fexp2(__builtin_fmaf(dlv[c], a2l[c][n], cl.offL));
-          float hT = from_lane_below(h[c][n]);
-          if (from_top) hT = tp[n];
-          float u = sL * bl[n];
-          u = __builtin_fmaf(sT, bt[n], u);
+          const float aT = fexp2(__builtin_fmaf(cur.dt[c], a2t[c][n], cl.offT));
+          const float aL = fexp2(__builtin_fmaf(cur.dl[c], a2l[c][n], cl.offL));
+          const float hT = from_row_below(h[c][n], tp[n]);
+          float u = sL * cur.bl[n];
+          u = __builtin_fmaf(sT, cur.bt[n], u);
           u = __builtin_fmaf(aT, hT, u);
           const float hn = __builtin_fmaf(aL, h[c][n], u);
           h[c][n] = hn;
-          if (WRITE_Y) acc = __builtin_fmaf(hn, cc[n], acc);
+          if (WRITE_Y) acc = __builtin_fmaf(hn, cur.cc[n], acc);
         }
-        yv[c] = __builtin_fmaf(xv[c], dsk[c], acc);
-        if (p.nbands > 1 && band + 1 < p.nbands && r == 63 && cl.act) {
-          float* tb = p.top + ((((int64_t)band * p.B + b) * p.W + cl.j) * p.E + e0 + c) * kN;
+        yv[c] = __builtin_fmaf(cur.x[c], dsk[c], acc);
+        if (to_top && cl.act) {
+          float* tw = p.top + ((((int64_t)band * p.B + b) * p.W + cl.j) * p.E + e0 + c) * kN;
 #pragma unroll
-          for (int n = 0; n < kN; ++n) tb[n] = h[c][n];
+          for (int n = 0; n < kN; ++n) tw[n] = h[c][n];
         }
       }
       if (WRITE_Y && cl.act) IO<T>::template stv<EC>(Y + cl.idx * p.E + e0, yv);
@@ -254,30 +292,49 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
 }
 
 // ----------------------------------------------------------------------------------- backward
-template <typename T>
+// Channel sums by lane-swap butterflies.  The wave holds CS channel slots; for a group of CS
+// states every lane lists its values v[0..CS-1] and the folds leave, in the lane of slot q, the
+// sum over all slots of the value that was listed for state fold_state(m, .) with result slot q.
+// fold_state(m, qi) is the state a lane must list at position qi of group m so that afterwards
+// slot q holds state q*NV + m (NV = 16/CS groups per lane).
+//   CS=4: fold16(fold32(v0,v1), fold32(v2,v3)) leaves position 0,1,2,3 in slot 0,2,1,3.
+//   CS=2: fold32(v0,v1) leaves position 0,1 in slot 0,1.
+template <int CS> __device__ __forceinline__ constexpr int fold_state(int m, int qi) {
+  constexpr int NV = kN / CS;
+  if (CS == 4) { const int q = (qi == 1) ? 2 : (qi == 2) ? 1 : qi; return q * NV + m; }
+  if (CS == 2) return qi * NV + m;
+  return m;
+}
+
+template <typename T, int CS>
 __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParams p) {
-  extern __shared__ float4 slots[];   // [wave][3][4][64] float4: per-wave d_C, d_BT, d_BL of the step
+  constexpr int NV = kN / CS;            // channel-summed states a lane holds after the butterflies
+  constexpr int NQ = NV / 4;             // ... as float4s
+  constexpr int SLOT = 3 * NQ * 64;      // float4s per wave in the exchange buffer
+  extern __shared__ float4 smem[];
+  float4* slots = smem;                                                  // [wave][3][NQ][64]
+  float* a_lds = reinterpret_cast<float*>(smem + kBwdWaves * SLOT);      // [wave][CS][2][16]
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int g = blockIdx.x / p.blocks_per_group;
-  const int eg = blockIdx.x % p.blocks_per_group;
-  const int e_raw = eg * kBwdWaves + wave;
-  const bool wave_ok = e_raw < p.E;           // padding waves still take part in the barriers
-  const int e = wave_ok ? e_raw : p.E - 1;
+  const int lb = logical_block(p.nwg);
+  const int b = lb / p.bpb;
+  const int eg = lb % p.bpb;
+  const int slot = lane >> kHBShift, r = lane & (kHB - 1);
+  const int e_raw = (eg * kBwdWaves + wave) * CS + slot;
+  const bool ch_ok = e_raw < p.E;           // padding lanes/waves still take part in the barriers
+  const int e = ch_ok ? e_raw : p.E - 1;
 
-  float a2t[kN], a2l[kN];
-#pragma unroll
-  for (int n = 0; n < kN; ++n) { a2t[n] = p.A2T[e * kN + n]; a2l[n] = p.A2L[e * kN + n]; }
+  {  // A of the wave's channels into LDS (read back state by state; keeps them out of VGPRs)
+    float* mine = a_lds + (wave * CS + slot) * (2 * kN);
+    for (int n = r; n < kN; n += kHB) { mine[n] = p.A2T[e * kN + n]; mine[kN + n] = p.A2L[e * kN + n]; }
+  }
+  const float* a_mine = a_lds + (wave * CS + slot) * (2 * kN);
   const float dsk = p.Df[e];
+  __syncthreads();
 
-  const int slot = lane >> p.hp_shift, r = lane & (p.HP - 1);
-  const int b = g * p.S + slot;
   const T* X = static_cast<const T*>(p.x);
   const T* DT = static_cast<const T*>(p.dT);
   const T* DL = static_cast<const T*>(p.dL);
-  const T* BTp = static_cast<const T*>(p.BT);
-  const T* BLp = static_cast<const T*>(p.BL);
-  const T* Cp = static_cast<const T*>(p.C);
   const T* DY = static_cast<const T*>(p.dy);
   T* DX = static_cast<T*>(p.dx);
   T* DDT = static_cast<T*>(p.ddT);
@@ -290,13 +347,12 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   for (int n = 0; n < kN; ++n) { accAT[n] = 0.f; accAL[n] = 0.f; }
 
   for (int band = p.nbands - 1; band >= 0; --band) {
-    const int i = band * 64 + r;
-    const int HB = p.nbands == 1 ? p.H : (p.H - band * 64 < 64 ? p.H - band * 64 : 64);
-    const bool row_ok = wave_ok && b < p.B && i < p.H;
-    const int T_steps = p.W + HB - 1;
+    const int i = band * kHB + r;
+    const int HBk = p.H - band * kHB < kHB ? p.H - band * kHB : kHB;
+    const bool row_ok = ch_ok && r < HBk;
+    const int T_steps = p.W + HBk - 1;
     const bool from_top = band > 0 && r == 0;
-    const bool from_bot = band + 1 < p.nbands && r == 63;
-    const int bcl = b < p.B ? b : p.B - 1;
+    const bool from_bot = band + 1 < p.nbands && r == kHB - 1;
 #pragma unroll
     for (int n = 0; n < kN; ++n) { muT[n] = 0.f; muL[n] = 0.f; }
 
@@ -307,9 +363,9 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
 #pragma unroll
         for (int n = 0; n < kN; ++n) hb[0][n] = 0.f;
       } else {
-        const float* ck = p.ckpt + ((((int64_t)g * p.nbands + band) * p.nblk + m) * p.E + e) * (kN * 64) + lane;
+        const float* ck = p.ckpt + (((((int64_t)b * p.nbands + band) * p.nblk + m) * p.E + e) * kN) * kHB + r;
 #pragma unroll
-        for (int n = 0; n < kN; ++n) hb[0][n] = ck[n * 64];
+        for (int n = 0; n < kN; ++n) hb[0][n] = ck[n * kHB];
       }
       // ---- recompute the states of the block
 #pragma unroll
@@ -321,16 +377,21 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
           const float xv = IO<T>::ld(X + cl.idx * p.E + e);
           const float dtv = IO<T>::ld(DT + cl.idx * p.E + e);
           const float dlv = IO<T>::ld(DL + cl.idx * p.E + e);
-          IO<T>::ld16(BTp + cl.idx * kN, bt);
-          IO<T>::ld16(BLp + cl.idx * kN, bl);
-          const float* tb = p.top + ((((int64_t)(band > 0 ? band - 1 : 0) * p.B + bcl) * p.W + (cl.act ? cl.j : 0)) * p.E + e) * kN;
+          ld16f(p.bt + cl.idx * p.bc_stride, bt);
+          ld16f(p.bl + cl.idx * p.bc_stride, bl);
+          float tp[kN];
+#pragma unroll
+          for (int n = 0; n < kN; ++n) tp[n] = 0.f;
+          if (from_top) {
+            const float* tb = p.top + ((((int64_t)(band - 1) * p.B + b) * p.W + (cl.act ? cl.j : 0)) * p.E + e) * kN;
+            ld16f(tb, tp);
+          }
           const float sT = cl.cT * dtv * xv, sL = cl.cL * dlv * xv;
 #pragma unroll
           for (int n = 0; n < kN; ++n) {
-            const float aT = fexp2(__builtin_fmaf(dtv, a2t[n], cl.offT));
-            const float aL = fexp2(__builtin_fmaf(dlv, a2l[n], cl.offL));
-            float hT = from_lane_below(hb[k][n]);
-            if (from_top) hT = tb[n];
+            const float aT = fexp2(__builtin_fmaf(dtv, a_mine[n], cl.offT));
+            const float aL = fexp2(__builtin_fmaf(dlv, a_mine[kN + n], cl.offL));
+            const float hT = from_row_below(hb[k][n], tp[n]);
             float u = sL * bl[n];
             u = __builtin_fmaf(sT, bt[n], u);
             u = __builtin_fmaf(aT, hT, u);
@@ -349,48 +410,65 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
           const float dtv = IO<T>::ld(DT + cl.idx * p.E + e);
           const float dlv = IO<T>::ld(DL + cl.idx * p.E + e);
           const float dyv = IO<T>::ld(DY + cl.idx * p.E + e);
-          IO<T>::ld16(BTp + cl.idx * kN, bt);
-          IO<T>::ld16(BLp + cl.idx * kN, bl);
-          IO<T>::ld16(Cp + cl.idx * kN, cc);
-          const float* tb = p.top + ((((int64_t)(band > 0 ? band - 1 : 0) * p.B + bcl) * p.W + (cl.act ? cl.j : 0)) * p.E + e) * kN;
-          float* bb = p.bot + (((int64_t)bcl * p.W + (cl.act ? cl.j : 0)) * p.E + e) * kN;
-          const float qT = cl.cT * dtv * xv, qL = cl.cL * dlv * xv;
-          const float keep = cl.act ? 1.f : 0.f;
-          const float qC = keep * dyv;
+          ld16f(p.bt + cl.idx * p.bc_stride, bt);
+          ld16f(p.bl + cl.idx * p.bc_stride, bl);
+          ld16f(p.cc + cl.idx * p.bc_stride, cc);
+          float* bb = p.bot + (((int64_t)b * p.W + (cl.act ? cl.j : 0)) * p.E + e) * kN;
+          float tp[kN], bo[kN];
+#pragma unroll
+          for (int n = 0; n < kN; ++n) { tp[n] = 0.f; bo[n] = 0.f; }
+          if (from_top) {
+            const float* tb = p.top + ((((int64_t)(band - 1) * p.B + b) * p.W + (cl.act ? cl.j : 0)) * p.E + e) * kN;
+            ld16f(tb, tp);
+          }
+          if (from_bot) {   // muT of the first row of the band below, left there by this wave
+#pragma unroll
+            for (int n = 0; n < kN; ++n) bo[n] = __builtin_nontemporal_load(bb + n);
+          }
+          const float qT = cl.cT * dtv * xv, qL = cl.cL * dlv * xv;   // zero on inactive lanes
+          const float qC = cl.act ? dyv : 0.f;
           float sT = 0.f, sL = 0.f, zT = 0.f, zL = 0.f;
-          float4* sw = slots + (size_t)wave * (3 * 4 * 64) + lane;
-          __syncthreads();   // the flush of the previous step has finished reading the slots
+          // States are visited in groups of CS so that the channel sums of a group (values of
+          // the CS channel slots of the wave) can be folded as soon as the group is done; after
+          // the folds the lane of slot q holds the states q*NV .. q*NV+NV-1 of its cell.
+          float rC[NV], rBT[NV], rBL[NV];
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            float vC[4], vBT[4], vBL[4];
+          for (int m = 0; m < NV; ++m) {
+            float vC[CS], vBT[CS], vBL[CS];
 #pragma unroll
-            for (int m = 0; m < 4; ++m) {
-              const int n = 4 * q + m;
-              const float aT = fexp2(__builtin_fmaf(dtv, a2t[n], cl.offT));
-              const float aL = fexp2(__builtin_fmaf(dlv, a2l[n], cl.offL));
-              float mb = from_lane_above(muT[n]);
-              if (from_bot) mb = __builtin_nontemporal_load(bb + n);
+            for (int qi = 0; qi < CS; ++qi) {
+              const int n = fold_state<CS>(m, qi);
+              const float a2t = a_mine[n], a2l = a_mine[kN + n];
+              const float aT = fexp2(__builtin_fmaf(dtv, a2t, cl.offT));
+              const float aL = fexp2(__builtin_fmaf(dlv, a2l, cl.offL));
+              const float mb = from_row_above(muT[n], bo[n]);
               const float lam = __builtin_fmaf(dyv, cc[n], muL[n] + mb);
-              float hT = from_lane_below(hb[k][n]);
-              if (from_top) hT = tb[n];
+              const float hT = from_row_below(hb[k][n], tp[n]);
               const float mT = aT * lam, mL = aL * lam;
               muT[n] = mT;
               muL[n] = mL;
               const float ZT = mT * hT, ZL = mL * hb[k][n];
               accAT[n] = __builtin_fmaf(ZT, dtv, accAT[n]);
               accAL[n] = __builtin_fmaf(ZL, dlv, accAL[n]);
-              zT = __builtin_fmaf(ZT, a2t[n], zT);
-              zL = __builtin_fmaf(ZL, a2l[n], zL);
+              zT = __builtin_fmaf(ZT, a2t, zT);
+              zL = __builtin_fmaf(ZL, a2l, zL);
               sT = __builtin_fmaf(lam, bt[n], sT);
               sL = __builtin_fmaf(lam, bl[n], sL);
-              vBT[m] = qT * lam;       // qT, qL are zero on inactive lanes
-              vBL[m] = qL * lam;
-              vC[m] = qC * hb[k + 1][n];
+              vBT[qi] = qT * lam;
+              vBL[qi] = qL * lam;
+              vC[qi] = qC * hb[k + 1][n];
             }
-            // channel sums of the step: per-wave slots, added in wave order by the flush
-            sw[(0 * 4 + q) * 64] = make_float4(vC[0], vC[1], vC[2], vC[3]);
-            sw[(1 * 4 + q) * 64] = make_float4(vBT[0], vBT[1], vBT[2], vBT[3]);
-            sw[(2 * 4 + q) * 64] = make_float4(vBL[0], vBL[1], vBL[2], vBL[3]);
+            if constexpr (CS == 4) {
+              rC[m] = fold16(fold32(vC[0], vC[1]), fold32(vC[2], vC[3]));
+              rBT[m] = fold16(fold32(vBT[0], vBT[1]), fold32(vBT[2], vBT[3]));
+              rBL[m] = fold16(fold32(vBL[0], vBL[1]), fold32(vBL[2], vBL[3]));
+            } else if constexpr (CS == 2) {
+              rC[m] = fold32(vC[0], vC[1]);
+              rBT[m] = fold32(vBT[0], vBT[1]);
+              rBL[m] = fold32(vBL[0], vBL[1]);
+            } else {
+              rC[m] = vC[0]; rBT[m] = vBT[0]; rBL[m] = vBL[0];
+            }
           }
           if (from_top && cl.act) {   // hand muT of this band's first row to the band above
 #pragma unroll
@@ -402,21 +480,32 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
             IO<T>::st(DDL + cl.idx * p.E + e, __builtin_fmaf(cl.cL * xv, sL, kLn2 * zL));
             IO<T>::st(DX + cl.idx * p.E + e, __builtin_fmaf(cl.cT * dtv, sT, __builtin_fmaf(cl.cL * dlv, sL, dyv * dsk)));
           }
+          // ... then per-wave slots, added in wave order by the flush
+          __syncthreads();   // the flush of the previous step has finished reading the slots
+          {
+            float4* sw = slots + wave * SLOT + lane;
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+              sw[(0 * NQ + q) * 64] = make_float4(rC[4*q], rC[4*q+1], rC[4*q+2], rC[4*q+3]);
+              sw[(1 * NQ + q) * 64] = make_float4(rBT[4*q], rBT[4*q+1], rBT[4*q+2], rBT[4*q+3]);
+              sw[(2 * NQ + q) * 64] = make_float4(rBL[4*q], rBL[4*q+1], rBL[4*q+2], rBL[4*q+3]);
+            }
+          }
           __syncthreads();
-          for (int it = threadIdx.x; it < 3 * 4 * 64; it += kBwdWaves * 64) {
-            const int fl = it & 63, q = (it >> 6) & 3, v = it >> 8;
-            const int fr = fl & (p.HP - 1), fb = g * p.S + (fl >> p.hp_shift);
-            const int fi = band * 64 + fr, fj = t - fr;
-            if (fb < p.B && fi < p.H && fj >= 0 && fj < p.W) {
-              float4 s = slots[(size_t)(0 * 3 + v) * (4 * 64) + q * 64 + fl];
+          for (int it = threadIdx.x; it < SLOT; it += kBwdWaves * 64) {
+            const int fl = it & 63, q = (it >> 6) % NQ, v = (it >> 6) / NQ;
+            const int fr = fl & (kHB - 1), fs = fl >> kHBShift;
+            const int fi = band * kHB + fr, fj = t - fr;
+            if (fi < p.H && fj >= 0 && fj < p.W) {
+              float4 s = slots[it];
 #pragma unroll
               for (int w = 1; w < kBwdWaves; ++w) {
-                const float4 o = slots[(size_t)(w * 3 + v) * (4 * 64) + q * 64 + fl];
+                const float4 o = slots[w * SLOT + it];
                 s.x += o.x; s.y += o.y; s.z += o.z; s.w += o.w;
               }
               const int im = p.flip ? p.H - 1 - fi : fi, jm = p.flip ? p.W - 1 - fj : fj;
-              const int64_t cell = ((int64_t)fb * p.H + im) * p.W + jm;
-              *reinterpret_cast<float4*>(p.part + (((int64_t)eg * 3 + v) * P + cell) * kN + 4 * q) = s;
+              const int64_t cell = ((int64_t)b * p.H + im) * p.W + jm;
+              *reinterpret_cast<float4*>(p.part + (((int64_t)eg * 3 + v) * P + cell) * kN + fs * NV + 4 * q) = s;
             }
           }
         }
@@ -425,7 +514,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
     if (p.nbands > 1) __threadfence();
   }
 
-  // ---- sums over positions: reduce the 64 lanes, one partial per (group, channel)
+  // ---- sums over positions: reduce over the rows of the band (lanes of one channel slot)
   float red[2 * kN + 1];
 #pragma unroll
   for (int n = 0; n < kN; ++n) { red[n] = accAT[n]; red[kN + n] = accAL[n]; }
@@ -433,15 +522,14 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
 #pragma unroll
   for (int k = 0; k < 2 * kN + 1; ++k) {
     float v = red[k];
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    for (int off = kHB >> 1; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
     red[k] = v;
   }
-  if (wave_ok && lane == 0) {
-    float* pa = p.pA + ((int64_t)g * p.E + e) * (2 * kN);
+  if (ch_ok && r == 0) {
+    float* pa = p.pA + ((int64_t)b * p.E + e) * (2 * kN);
 #pragma unroll
     for (int n = 0; n < 2 * kN; ++n) pa[n] = red[n];
-    p.pD[(int64_t)g * p.E + e] = red[2 * kN];
+    p.pD[(int64_t)b * p.E + e] = red[2 * kN];
   }
 }
 
@@ -456,8 +544,28 @@ __global__ void m2d_prep_kernel(const T* AT, const T* AL, const T* D, float* A2T
   if (idx < E) Df[idx] = IO<T>::ld(D + idx);
 }
 
+// bf16 B_T, B_L, C -> one fp32 record of 48 values per cell (three runs of 16), so the scan
+// kernels load fp32 operands without unpacking them state by state.
+__global__ void m2d_widen_bc_kernel(const bf16_t* BT, const bf16_t* BL, const bf16_t* C, float* out, int64_t P) {
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // one thread per (cell, tensor, half)
+  if (gid >= P * 6) return;
+  const int64_t cell = gid / 6;
+  const int w = (int)(gid % 6), tsr = w >> 1, half = w & 1;
+  const bf16_t* src = (tsr == 0 ? BT : (tsr == 1 ? BL : C)) + cell * kN + half * 8;
+  const uint4 t = *reinterpret_cast<const uint4*>(src);
+  const uint32_t wds[4] = {t.x, t.y, t.z, t.w};
+  float4 lo, hi;
+  lo.x = __uint_as_float(wds[0] << 16); lo.y = __uint_as_float(wds[0] & 0xffff0000u);
+  lo.z = __uint_as_float(wds[1] << 16); lo.w = __uint_as_float(wds[1] & 0xffff0000u);
+  hi.x = __uint_as_float(wds[2] << 16); hi.y = __uint_as_float(wds[2] & 0xffff0000u);
+  hi.z = __uint_as_float(wds[3] << 16); hi.w = __uint_as_float(wds[3] & 0xffff0000u);
+  float4* dst = reinterpret_cast<float4*>(out + cell * 48 + tsr * kN + half * 8);
+  dst[0] = lo;
+  dst[1] = hi;
+}
+
 // d_C, d_BT, d_BL: add the per-workgroup channel sums in workgroup order and round to T.
-// d_AT, d_AL, d_D: add the per-group partials in group order.
+// d_AT, d_AL, d_D: add the per-image partials in image order.
 template <typename T>
 __global__ void m2d_finalize_kernel(const ScanParams p, T* dC, T* dBT, T* dBL, T* dAT, T* dAL, T* dD) {
   const int64_t P = (int64_t)p.B * p.H * p.W;
@@ -466,7 +574,7 @@ __global__ void m2d_finalize_kernel(const ScanParams p, T* dC, T* dBT, T* dBL, T
   if (gid < nquad) {
     const int64_t v = gid / (P * 4), rem = gid % (P * 4);
     float4 s = *reinterpret_cast<const float4*>(p.part + (v * P * kN) + rem * 4);
-    for (int egi = 1; egi < p.blocks_per_group; ++egi) {
+    for (int egi = 1; egi < p.bpb; ++egi) {
       const float4 o = *reinterpret_cast<const float4*>(p.part + (((int64_t)egi * 3 + v) * P * kN) + rem * 4);
       s.x += o.x; s.y += o.y; s.z += o.z; s.w += o.w;
     }
@@ -477,12 +585,12 @@ __global__ void m2d_finalize_kernel(const ScanParams p, T* dC, T* dBT, T* dBL, T
   if (k < (int64_t)p.E * 2 * kN) {
     const int e = (int)(k / (2 * kN)), w = (int)(k % (2 * kN));
     float s = 0.f;
-    for (int g = 0; g < p.NG; ++g) s += p.pA[((int64_t)g * p.E + e) * (2 * kN) + w];
+    for (int g = 0; g < p.B; ++g) s += p.pA[((int64_t)g * p.E + e) * (2 * kN) + w];
     if (w < kN) IO<T>::st(dAT + e * kN + w, s); else IO<T>::st(dAL + e * kN + (w - kN), s);
   }
   if (k < p.E) {
     float s = 0.f;
-    for (int g = 0; g < p.NG; ++g) s += p.pD[(int64_t)g * p.E + k];
+    for (int g = 0; g < p.B; ++g) s += p.pD[(int64_t)g * p.E + k];
     IO<T>::st(dD + k, s);
   }
 }
@@ -495,10 +603,10 @@ hipEvent_t g_ev[2][2] = {{nullptr, nullptr}, {nullptr, nullptr}};
 inline size_t align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
 
 struct Geometry {
-  int HP, hp_shift, S, NG, nbands, nblk;
-  int fwd_ec, fwd_net, fwd_bpg;      // forward: channels per wave, waves per group, workgroups per group
-  int bwd_bpg;                       // backward: workgroups per group (= channel groups EG)
-  size_t prep_bytes, ckpt_diag_bytes, top_bytes, bot_bytes, part_bytes, pa_bytes, pd_bytes;
+  int HB, hb_shift, CS, nbands, nblk;
+  int fwd_ec, fwd_wpb, fwd_bpb;      // forward: channels per lane, waves and workgroups per image
+  int bwd_wpb, bwd_bpb;              // backward: waves and workgroups (channel groups) per image
+  size_t prep_bytes, bc_bytes, ckpt_diag_bytes, top_bytes, bot_bytes, part_bytes, pa_bytes, pd_bytes;
 };
 
 int check_desc(const m2d_desc* d) {
@@ -513,36 +621,39 @@ int check_desc(const m2d_desc* d) {
 
 Geometry make_geometry(const m2d_desc* d) {
   Geometry g;
-  if (d->H > 32) { g.HP = 64; }
-  else { g.HP = 2; while (g.HP < d->H) g.HP *= 2; }
-  g.hp_shift = 0;
-  while ((1 << g.hp_shift) < g.HP) ++g.hp_shift;
-  g.S = 64 / g.HP;
-  g.NG = (d->B + g.S - 1) / g.S;
-  g.nbands = g.HP == 64 ? (d->H + 63) / 64 : 1;
-  const int hb = d->H < 64 ? d->H : 64;
+  // band height: 16 rows keeps W/(W+HB-1) of the steps busy and gives 4 channel slots per wave
+  g.HB = kHB;
+  g.hb_shift = kHBShift;
+  g.CS = 64 / g.HB;
+  g.nbands = (d->H + g.HB - 1) / g.HB;
+  const int hb = d->H < g.HB ? d->H : g.HB;
   g.nblk = (d->W + hb - 1 + kCK - 1) / kCK;
-  g.fwd_ec = (d->E % 2 == 0) ? 2 : 1;
-  g.fwd_net = d->E / g.fwd_ec;
-  g.fwd_bpg = (g.fwd_net + kFwdWaves - 1) / kFwdWaves;
-  g.bwd_bpg = (d->E + kBwdWaves - 1) / kBwdWaves;
+  // forward: two channels per lane when that still yields enough waves to fill the device
+  const bool ec2 = (d->E % 2 == 0) && ((int64_t)d->B * ((d->E / 2 + g.CS - 1) / g.CS) >= 2048);
+  g.fwd_ec = ec2 ? 2 : 1;
+  g.fwd_wpb = (d->E / g.fwd_ec + g.CS - 1) / g.CS;
+  g.fwd_bpb = (g.fwd_wpb + kFwdWaves - 1) / kFwdWaves;
+  g.bwd_wpb = (d->E + g.CS - 1) / g.CS;
+  g.bwd_bpb = (g.bwd_wpb + kBwdWaves - 1) / kBwdWaves;
   const size_t P = (size_t)d->B * d->H * d->W;
   g.prep_bytes = align_up(sizeof(float) * ((size_t)2 * d->E * kN + d->E));
-  g.ckpt_diag_bytes = align_up(sizeof(float) * (size_t)g.NG * g.nbands * g.nblk * d->E * kN * 64);
+  g.bc_bytes = d->dtype == M2D_BF16 ? align_up(sizeof(float) * P * 48) : 0;
+  g.ckpt_diag_bytes = align_up(sizeof(float) * (size_t)d->B * g.nbands * g.nblk * d->E * kN * g.HB);
   g.top_bytes = g.nbands > 1 ? align_up(sizeof(float) * (size_t)(g.nbands - 1) * d->B * d->W * d->E * kN) : 0;
   g.bot_bytes = g.nbands > 1 ? align_up(sizeof(float) * (size_t)d->B * d->W * d->E * kN) : 0;
-  g.part_bytes = align_up(sizeof(float) * (size_t)g.bwd_bpg * 3 * P * kN);
-  g.pa_bytes = align_up(sizeof(float) * (size_t)g.NG * d->E * 2 * kN);
-  g.pd_bytes = align_up(sizeof(float) * (size_t)g.NG * d->E);
+  g.part_bytes = align_up(sizeof(float) * (size_t)g.bwd_bpb * 3 * P * kN);
+  g.pa_bytes = align_up(sizeof(float) * (size_t)d->B * d->E * 2 * kN);
+  g.pd_bytes = align_up(sizeof(float) * (size_t)d->B * d->E);
   return g;
 }
 
-size_t ckpt_bytes_of(const Geometry& g) { return g.ckpt_diag_bytes + g.top_bytes; }
+// checkpoint buffer: [state snapshots][band boundary rows][widened B,C (bf16 input only)]
+size_t ckpt_bytes_of(const Geometry& g) { return g.ckpt_diag_bytes + g.top_bytes + g.bc_bytes; }
 
 size_t workspace_bytes_of(const Geometry& g, int pass, int have_ckpt) {
   size_t n = g.prep_bytes;
   if (pass == M2D_PASS_FWD) {
-    if (!have_ckpt) n += g.top_bytes;
+    if (!have_ckpt) n += g.top_bytes + g.bc_bytes;
   } else {
     n += g.part_bytes + g.pa_bytes + g.pd_bytes + g.bot_bytes;
     if (!have_ckpt) n += ckpt_bytes_of(g);
@@ -554,7 +665,7 @@ bool misaligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p
 
 void fill_common(ScanParams& sp, const m2d_desc* d, const Geometry& g) {
   sp.B = d->B; sp.H = d->H; sp.W = d->W; sp.E = d->E;
-  sp.HP = g.HP; sp.hp_shift = g.hp_shift; sp.S = g.S; sp.NG = g.NG; sp.nbands = g.nbands; sp.nblk = g.nblk;
+  sp.nbands = g.nbands; sp.nblk = g.nblk;
   sp.flip = (d->flags & M2D_FLAG_FLIP) ? 1 : 0;
 }
 
@@ -569,12 +680,33 @@ int launch_prep(const m2d_desc* d, const void* AT, const void* AL, const void* D
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
+// Points sp.bt/bl/cc at fp32 B_T, B_L, C: the caller's tensors for fp32 input, a widened copy
+// (made here unless `ready`) for bf16 input.
 template <typename T>
-int launch_fwd(const ScanParams& sp0, const Geometry& g, bool ckpt, bool write_y, hipStream_t st) {
+int stage_bc(ScanParams& sp, const m2d_desc* d, const void* BT, const void* BL, const void* C, float* wide,
+             bool ready, hipStream_t st) {
+  if (sizeof(T) == 4) {
+    sp.bt = static_cast<const float*>(BT); sp.bl = static_cast<const float*>(BL); sp.cc = static_cast<const float*>(C);
+    sp.bc_stride = kN;
+    return M2D_OK;
+  }
+  sp.bt = wide; sp.bl = wide + kN; sp.cc = wide + 2 * kN;
+  sp.bc_stride = 48;
+  if (ready) return M2D_OK;
+  const int64_t P = (int64_t)d->B * d->H * d->W;
+  hipLaunchKernelGGL(m2d_widen_bc_kernel, dim3((unsigned)((P * 6 + 255) / 256)), dim3(256), 0, st,
+                     static_cast<const bf16_t*>(BT), static_cast<const bf16_t*>(BL), static_cast<const bf16_t*>(C),
+                     wide, P);
+  return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+}
+
+template <typename T>
+int launch_fwd(const ScanParams& sp0, const m2d_desc* d, const Geometry& g, bool ckpt, bool write_y, hipStream_t st) {
   ScanParams sp = sp0;
-  sp.NET = g.fwd_net;
-  sp.blocks_per_group = g.fwd_bpg;
-  const dim3 grid((unsigned)((size_t)g.NG * g.fwd_bpg)), block(kFwdWaves * 64);
+  sp.wpb = g.fwd_wpb;
+  sp.bpb = g.fwd_bpb;
+  sp.nwg = d->B * g.fwd_bpb;
+  const dim3 grid((unsigned)sp.nwg), block(kFwdWaves * 64);
 #define M2D_FWD(EC, CK, WY) hipLaunchKernelGGL((m2d_fwd_kernel<T, EC, CK, WY>), grid, block, 0, st, sp)
   if (g.fwd_ec == 2) {
     if (ckpt && write_y) M2D_FWD(2, true, true);
@@ -590,31 +722,44 @@ int launch_fwd(const ScanParams& sp0, const Geometry& g, bool ckpt, bool write_y
 }
 
 template <typename T>
-int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT, const void* AL, const void* D,
-            void* ckpt, void* ws, hipStream_t st) {
+int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT, const void* AL, const void* BT,
+            const void* BL, const void* C, const void* D, void* ckpt, void* ws, hipStream_t st) {
   char* w = static_cast<char*>(ws);
   float* prep = reinterpret_cast<float*>(w);
   w += g.prep_bytes;
   sp.A2T = prep; sp.A2L = prep + (size_t)d->E * kN; sp.Df = prep + (size_t)2 * d->E * kN;
-  if (ckpt) {
-    sp.ckpt = static_cast<float*>(ckpt);
-    sp.top = reinterpret_cast<float*>(static_cast<char*>(ckpt) + g.ckpt_diag_bytes);
-  } else {
-    sp.ckpt = nullptr;
-    sp.top = reinterpret_cast<float*>(w);
-  }
+  char* keep = ckpt ? static_cast<char*>(ckpt) + g.ckpt_diag_bytes : w;   // [top][widened B,C]
+  sp.ckpt = ckpt ? static_cast<float*>(ckpt) : nullptr;
+  sp.top = reinterpret_cast<float*>(keep);
   int rc = launch_prep<T>(d, AT, AL, D, prep, st);
   if (rc) return rc;
+  rc = stage_bc<T>(sp, d, BT, BL, C, reinterpret_cast<float*>(keep + g.top_bytes), false, st);
+  if (rc) return rc;
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_FWD][0], st);
-  rc = launch_fwd<T>(sp, g, ckpt != nullptr, true, st);
+  rc = launch_fwd<T>(sp, d, g, ckpt != nullptr, true, st);
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_FWD][1], st);
   return rc;
 }
 
+template <typename T, int CS>
+int launch_bwd(const ScanParams& sp, hipStream_t st) {
+  constexpr int NQ = kN / CS / 4;
+  const size_t lds = sizeof(float4) * kBwdWaves * 3 * NQ * 64 + sizeof(float) * kBwdWaves * CS * 2 * kN;
+  static bool attr = false;   // idempotent, the value never changes
+  if (!attr) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_bwd_kernel<T, CS>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return M2D_ERR_HIP;
+    attr = true;
+  }
+  hipLaunchKernelGGL((m2d_bwd_kernel<T, CS>), dim3((unsigned)sp.nwg), dim3(kBwdWaves * 64), lds, st, sp);
+  return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+}
+
 template <typename T>
-int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT, const void* AL, const void* D,
-            const void* ckpt, void* dAT, void* dAL, void* dBT, void* dBL, void* dC, void* dD, void* ws,
-            hipStream_t st) {
+int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT, const void* AL, const void* BT,
+            const void* BL, const void* C, const void* D, const void* ckpt, void* dAT, void* dAL, void* dBT,
+            void* dBL, void* dC, void* dD, void* ws, hipStream_t st) {
   char* w = static_cast<char*>(ws);
   float* prep = reinterpret_cast<float*>(w); w += g.prep_bytes;
   sp.A2T = prep; sp.A2L = prep + (size_t)d->E * kN; sp.Df = prep + (size_t)2 * d->E * kN;
@@ -624,30 +769,22 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   sp.bot = reinterpret_cast<float*>(w); w += g.bot_bytes;
   int rc = launch_prep<T>(d, AT, AL, D, prep, st);
   if (rc) return rc;
-  if (ckpt) {
-    sp.ckpt = const_cast<float*>(static_cast<const float*>(ckpt));
-    sp.top = reinterpret_cast<float*>(const_cast<char*>(static_cast<const char*>(ckpt)) + g.ckpt_diag_bytes);
-  } else {   // rebuild the checkpoints with one forward sweep that writes no y
-    sp.ckpt = reinterpret_cast<float*>(w);
-    sp.top = reinterpret_cast<float*>(w + g.ckpt_diag_bytes);
-    rc = launch_fwd<T>(sp, g, true, false, st);
+  char* ck = ckpt ? const_cast<char*>(static_cast<const char*>(ckpt)) : w;
+  sp.ckpt = reinterpret_cast<float*>(ck);
+  sp.top = reinterpret_cast<float*>(ck + g.ckpt_diag_bytes);
+  rc = stage_bc<T>(sp, d, BT, BL, C, reinterpret_cast<float*>(ck + g.ckpt_diag_bytes + g.top_bytes), ckpt != nullptr, st);
+  if (rc) return rc;
+  if (!ckpt) {   // rebuild the checkpoints with one forward sweep that writes no y
+    rc = launch_fwd<T>(sp, d, g, true, false, st);
     if (rc) return rc;
   }
-  sp.NET = d->E;
-  sp.blocks_per_group = g.bwd_bpg;
-  const size_t lds = sizeof(float4) * kBwdWaves * 3 * 4 * 64;
-  static bool attr_f32 = false, attr_bf16 = false;   // idempotent, value never changes
-  bool& attr = sizeof(T) == 4 ? attr_f32 : attr_bf16;
-  if (!attr) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_bwd_kernel<T>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return M2D_ERR_HIP;
-    attr = true;
-  }
+  sp.wpb = g.bwd_wpb;
+  sp.bpb = g.bwd_bpb;
+  sp.nwg = d->B * g.bwd_bpb;
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][0], st);
-  hipLaunchKernelGGL(m2d_bwd_kernel<T>, dim3((unsigned)((size_t)g.NG * g.bwd_bpg)), dim3(kBwdWaves * 64), lds, st, sp);
+  rc = launch_bwd<T, 4>(sp, st);
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][1], st);
-  if (hipGetLastError() != hipSuccess) return M2D_ERR_HIP;
+  if (rc) return rc;
   const int64_t P = (int64_t)d->B * d->H * d->W;
   int64_t work = 3 * P * (kN / 4);
   if (work < (int64_t)d->E * 2 * kN) work = (int64_t)d->E * 2 * kN;
@@ -662,7 +799,7 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
 // ---------------------------------------------------------------------------------------- C ABI
 extern "C" {
 
-int m2d_version(void) { return 100; }
+int m2d_version(void) { return 200; }
 
 const char* m2d_status_str(int status) {
   switch (status) {
@@ -720,10 +857,10 @@ int m2d_scan_fwd(const m2d_desc* desc, const void* x, const void* deltaT, const 
   if (ckpt && ckpt_bytes < ckpt_bytes_of(g)) return M2D_ERR_WORKSPACE;
   ScanParams sp = {};
   fill_common(sp, desc, g);
-  sp.x = x; sp.dT = deltaT; sp.dL = deltaL; sp.BT = BT; sp.BL = BL; sp.C = C; sp.y = y;
+  sp.x = x; sp.dT = deltaT; sp.dL = deltaL; sp.y = y;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  return desc->dtype == M2D_F32 ? run_fwd<float>(desc, g, sp, AT, AL, D, ckpt, workspace, st)
-                                : run_fwd<bf16_t>(desc, g, sp, AT, AL, D, ckpt, workspace, st);
+  return desc->dtype == M2D_F32 ? run_fwd<float>(desc, g, sp, AT, AL, BT, BL, C, D, ckpt, workspace, st)
+                                : run_fwd<bf16_t>(desc, g, sp, AT, AL, BT, BL, C, D, ckpt, workspace, st);
 }
 
 int m2d_scan_bwd(const m2d_desc* desc, const void* x, const void* deltaT, const void* deltaL, const void* AT,
@@ -743,12 +880,12 @@ int m2d_scan_bwd(const m2d_desc* desc, const void* x, const void* deltaT, const 
   if (ckpt && ckpt_bytes < ckpt_bytes_of(g)) return M2D_ERR_WORKSPACE;
   ScanParams sp = {};
   fill_common(sp, desc, g);
-  sp.x = x; sp.dT = deltaT; sp.dL = deltaL; sp.BT = BT; sp.BL = BL; sp.C = C; sp.dy = dy;
+  sp.x = x; sp.dT = deltaT; sp.dL = deltaL; sp.dy = dy;
   sp.dx = dx; sp.ddT = d_deltaT; sp.ddL = d_deltaL;
   hipStream_t st = static_cast<hipStream_t>(stream);
   return desc->dtype == M2D_F32
-             ? run_bwd<float>(desc, g, sp, AT, AL, D, ckpt, d_AT, d_AL, d_BT, d_BL, d_C, d_D, workspace, st)
-             : run_bwd<bf16_t>(desc, g, sp, AT, AL, D, ckpt, d_AT, d_AL, d_BT, d_BL, d_C, d_D, workspace, st);
+             ? run_bwd<float>(desc, g, sp, AT, AL, BT, BL, C, D, ckpt, d_AT, d_AL, d_BT, d_BL, d_C, d_D, workspace, st)
+             : run_bwd<bf16_t>(desc, g, sp, AT, AL, BT, BL, C, D, ckpt, d_AT, d_AL, d_BT, d_BL, d_C, d_D, workspace, st);
 }
 
 }  // extern "C"
