@@ -45,8 +45,9 @@ constexpr int kN = 16;            // states per channel
 constexpr int kCK = M2D_CK;       // checkpoint interval (steps)
 constexpr int kHB = 16;           // rows per band = lanes per DPP row
 constexpr int kHBShift = 4;
-constexpr int kFwdWaves = 4;      // waves per forward workgroup
+constexpr int kFwdWaves = 8;      // waves per forward workgroup
 constexpr int kBwdWaves = 8;      // waves per backward workgroup
+constexpr int kZeroFloats = 64;     // page of zeros at the head of the set-up area
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -131,6 +132,7 @@ struct ScanParams {
   const void *x, *dT, *dL, *dy;
   const float *bt, *bl, *cc;        // B_T, B_L, C in fp32, element (cell, n) at [cell*bc_stride + n]
   const float *A2T, *A2L, *Df;      // A*log2(e) and D in fp32, (E,16) / (E)
+  const float* zeros;               // 256 bytes of zeros (source for out-of-grid staging chunks)
   void *y, *dx, *ddT, *ddL;
   float* ckpt;                      // [B][nbands][nblk][E][16][HB]  state snapshots
   float* top;                       // [nbands-1][B][W][E][16]       last row of each band (forward states)
@@ -155,6 +157,12 @@ __device__ __forceinline__ int logical_block(int nwg) {
   return (id & 7) * per + (id >> 3);
 }
 
+__device__ __forceinline__ int64_t cell_index(const ScanParams& p, int b, int i, int j) {
+  const int im = p.flip ? p.H - 1 - i : i;
+  const int jm = p.flip ? p.W - 1 - j : j;
+  return ((int64_t)b * p.H + im) * p.W + jm;
+}
+
 struct Cell {          // what a lane needs to know about its cell at one step
   bool act;
   int64_t idx;         // flat (b,i,j) index, clamped to a valid cell when !act
@@ -169,9 +177,7 @@ __device__ __forceinline__ Cell locate(const ScanParams& p, int b, int i, int t,
   c.act = row_ok && j >= 0 && j < p.W;
   const int ic = i < p.H ? i : p.H - 1;
   const int jc = j < 0 ? 0 : (j < p.W ? j : p.W - 1);
-  const int im = p.flip ? p.H - 1 - ic : ic;
-  const int jm = p.flip ? p.W - 1 - jc : jc;
-  c.idx = ((int64_t)b * p.H + im) * p.W + jm;
+  c.idx = cell_index(p, b, ic, jc);
   const float ninf = -__builtin_huge_valf();
   if (!c.act)      { c.cT = 0.f;  c.cL = 0.f;  c.offT = ninf; c.offL = ninf; }
   else if (i == 0) { c.cT = 0.f;  c.cL = 1.f;  c.offT = ninf; c.offL = j == 0 ? ninf : 0.f; }
@@ -180,25 +186,93 @@ __device__ __forceinline__ Cell locate(const ScanParams& p, int b, int i, int t,
   return c;
 }
 
-// ------------------------------------------------------------------------------------ forward
-template <int EC>
-struct FwdLoad {           // operands of one step, as loaded
-  float x[EC], dt[EC], dl[EC];
-  float bt[kN], bl[kN], cc[kN];
+// ------------------------------------------------------------------------------ operand staging
+// The operands of a block of kCK steps of a band are copied to LDS one block ahead of their use
+// with direct global->LDS loads (no registers, asynchronous): lane i of a wave-wide load fills
+// the 16-byte chunk i of a 1 KB LDS window.  Two regions per buffer:
+//   BC: per (step k, band row r) a record of 13 chunks: B_T, B_L, C of the cell (r, t0+k-r) as
+//       3 x 16 fp32, plus one pad chunk so that the 16 rows fall in distinct banks;
+//   XD: per (k, r) a record of NT tensors x CW channels of the workgroup in the tensor dtype
+//       (x, deltaT, deltaL[, dy]), plus one pad chunk.  Needs E to be a multiple of the chunk.
+// Cells outside the grid read from a page of zeros.
+template <typename T, int NT, int CW>
+struct Stage {
+  static constexpr int kElem = 16 / sizeof(T);           // elements per chunk
+  static constexpr int kCpt = CW / kElem;                // chunks per tensor per cell
+  static constexpr int kXRec = NT * kCpt + 1;            // chunks per XD record (with pad)
+  static constexpr int kXStride = kXRec * kElem;         // XD record stride in elements
+  static constexpr int kBRec = 13;                       // chunks per BC record (with pad)
+  static constexpr int kBStride = kBRec * 4;             // BC record stride in floats
+  static constexpr int kBChunks = kCK * kHB * kBRec;
+  static constexpr int kXChunks = kCK * kHB * kXRec;
+  static constexpr int kBBytes = kBChunks * 16;
+  static constexpr int kBytes = (kBChunks + kXChunks) * 16;   // one buffer
+  static_assert(CW % kElem == 0, "workgroup channel count must fill whole chunks");
 };
 
-template <typename T, int EC, bool CKPT, bool WRITE_Y>
+__device__ __forceinline__ void lds_fill16(const void* src, char* lds_window) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
+                                   (__attribute__((address_space(3))) void*)lds_window, 16, 0, 0);
+}
+
+template <typename T, int NT, int CW, bool STAGE_X, int NWAVES>
+__device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int b, int band, int t0, int e_wg0,
+                                            int wave, int lane, const T* const (&xs)[NT]) {
+  using SG = Stage<T, NT, CW>;
+  for (int c0 = wave * 64; c0 < SG::kBChunks; c0 += NWAVES * 64) {
+    const int c = c0 + lane;
+    const int rec = c / SG::kBRec, part = c - rec * SG::kBRec;
+    if (c < SG::kBChunks && part < 12) {
+      const int k = rec >> kHBShift, r = rec & (kHB - 1);
+      const int i = band * kHB + r, j = t0 + k - r;
+      const float* src = p.zeros;
+      if (i < p.H && j >= 0 && j < p.W) {
+        const int tau = part >> 2;
+        src = (tau == 0 ? p.bt : (tau == 1 ? p.bl : p.cc)) + cell_index(p, b, i, j) * p.bc_stride + (part & 3) * 4;
+      }
+      lds_fill16(src, buf + c0 * 16);
+    }
+  }
+  if constexpr (STAGE_X) {
+    char* xbuf = buf + SG::kBBytes;
+    for (int c0 = wave * 64; c0 < SG::kXChunks; c0 += NWAVES * 64) {
+      const int c = c0 + lane;
+      const int rec = c / SG::kXRec, part = c - rec * SG::kXRec;
+      if (c < SG::kXChunks && part < NT * SG::kCpt) {
+        const int k = rec >> kHBShift, r = rec & (kHB - 1);
+        const int i = band * kHB + r, j = t0 + k - r;
+        const int tau = part / SG::kCpt, ch = e_wg0 + (part - tau * SG::kCpt) * SG::kElem;
+        const void* src = p.zeros;
+        if (i < p.H && j >= 0 && j < p.W && ch < p.E) src = xs[tau] + cell_index(p, b, i, j) * p.E + ch;
+        lds_fill16(src, xbuf + c0 * 16);
+      }
+    }
+  }
+}
+
+// all direct-to-LDS loads of this wave have landed; then meet the other waves
+__device__ __forceinline__ void staging_fence() {
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+}
+
+// ------------------------------------------------------------------------------------ forward
+template <typename T, int EC, bool CKPT, bool WRITE_Y, bool STAGE_X>
 __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParams p) {
+  constexpr int CS = 64 >> kHBShift;
+  constexpr int CW = kFwdWaves * CS * EC;
+  using SG = Stage<T, 3, CW>;
+  extern __shared__ float4 smem[];
+  char* lds = reinterpret_cast<char*>(smem);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lb = logical_block(p.nwg);
   const int b = lb / p.bpb;
-  const int wv = (lb % p.bpb) * kFwdWaves + wave;
-  if (wv >= p.wpb) return;
+  const int e_wg0 = (lb % p.bpb) * CW;
   const int slot = lane >> kHBShift, r = lane & (kHB - 1);
-  constexpr int CS = 64 >> kHBShift;
-  const int e_raw = (wv * CS + slot) * EC;
-  const bool ch_ok = e_raw < p.E;
+  const int ch_loc = (wave * CS + slot) * EC;      // first channel of the lane inside the workgroup
+  const int e_raw = e_wg0 + ch_loc;
+  const bool ch_ok = e_raw < p.E;                  // idle lanes still take part in staging and barriers
   const int e0 = ch_ok ? e_raw : p.E - EC;
 
   float a2t[EC][kN], a2l[EC][kN], dsk[EC];
@@ -212,93 +286,112 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   const T* X = static_cast<const T*>(p.x);
   const T* DT = static_cast<const T*>(p.dT);
   const T* DL = static_cast<const T*>(p.dL);
+  const T* const xs[3] = {X, DT, DL};
   T* Y = static_cast<T*>(p.y);
 
-  for (int band = 0; band < p.nbands; ++band) {
+  int band = 0, m = 0, cur = 0;
+  stage_block<T, 3, CW, STAGE_X, kFwdWaves>(p, lds, b, 0, 0, e_wg0, wave, lane, xs);
+  staging_fence();
+
+  float h[EC][kN];
+  while (band < p.nbands) {
     const int i = band * kHB + r;
     const int HBk = p.H - band * kHB < kHB ? p.H - band * kHB : kHB;
     const bool row_ok = ch_ok && r < HBk;
     const int T_steps = p.W + HBk - 1;
     const bool from_top = band > 0 && r == 0;
     const bool to_top = band + 1 < p.nbands && r == kHB - 1;
-    float h[EC][kN];
-#pragma unroll
-    for (int c = 0; c < EC; ++c)
-#pragma unroll
-      for (int n = 0; n < kN; ++n) h[c][n] = 0.f;
+    const int t0 = m * kCK;
+    int nband = band, nm = m + 1;
+    if (nm * kCK >= T_steps) { nband = band + 1; nm = 0; }
+    if (nband < p.nbands)
+      stage_block<T, 3, CW, STAGE_X, kFwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, nband, nm * kCK, e_wg0, wave, lane, xs);
 
-    auto load = [&](int t, FwdLoad<EC>& o) {
-      const Cell cl = locate(p, b, i, t, r, row_ok);
-      IO<T>::template ldv<EC>(X + cl.idx * p.E + e0, o.x);
-      IO<T>::template ldv<EC>(DT + cl.idx * p.E + e0, o.dt);
-      IO<T>::template ldv<EC>(DL + cl.idx * p.E + e0, o.dl);
-      ld16f(p.bt + cl.idx * p.bc_stride, o.bt);
-      ld16f(p.bl + cl.idx * p.bc_stride, o.bl);
-      if (WRITE_Y) ld16f(p.cc + cl.idx * p.bc_stride, o.cc);
-    };
-
-    FwdLoad<EC> nxt;
-    load(0, nxt);
-    for (int t = 0; t < T_steps; ++t) {
-      // snapshot of the state after step t-1; lanes that have not started or are past the last
-      // column hold nothing the backward needs
-      if (CKPT && t > 0 && (t % kCK) == 0 && row_ok && t - 1 - r >= 0 && t - 1 - r < p.W) {
-        float* ck = p.ckpt + (((((int64_t)b * p.nbands + band) * p.nblk + t / kCK) * p.E + e0) * kN) * kHB + r;
+    if (m == 0) {
 #pragma unroll
-        for (int c = 0; c < EC; ++c)
+      for (int c = 0; c < EC; ++c)
 #pragma unroll
-          for (int n = 0; n < kN; ++n) ck[(c * kN + n) * kHB] = h[c][n];
-      }
-      const FwdLoad<EC> cur = nxt;
-      if (t + 1 < T_steps) load(t + 1, nxt);   // operands of the next step fly during this one
-      const Cell cl = locate(p, b, i, t, r, row_ok);
-      float yv[EC];
-#pragma unroll
-      for (int c = 0; c < EC; ++c) {
-        const float sT = cl.cT * cur.dt[c] * cur.x[c];
-        const float sL = cl.cL * cur.dl[c] * cur.x[c];
-        float tp[kN];
-#pragma unroll
-        for (int n = 0; n < kN; ++n) tp[n] = 0.f;
-        if (from_top) {   // first row of a lower band: the row above lives in memory
-          const float* tb = p.top + ((((int64_t)(band - 1) * p.B + b) * p.W + (cl.act ? cl.j : 0)) * p.E + e0 + c) * kN;
-#pragma unroll
-          for (int n = 0; n < kN; ++n) tp[n] = __builtin_nontemporal_load(tb + n);
-        }
-        float acc = 0.f;
-#pragma unroll
-        for (int n = 0; n < kN; ++n) {
-          const float aT = fexp2(__builtin_fmaf(cur.dt[c], a2t[c][n], cl.offT));
-          const float aL = fexp2(__builtin_fmaf(cur.dl[c], a2l[c][n], cl.offL));
-          const float hT = from_row_below(h[c][n], tp[n]);
-          float u = sL * cur.bl[n];
-          u = __builtin_fmaf(sT, cur.bt[n], u);
-          u = __builtin_fmaf(aT, hT, u);
-          const float hn = __builtin_fmaf(aL, h[c][n], u);
-          h[c][n] = hn;
-          if (WRITE_Y) acc = __builtin_fmaf(hn, cur.cc[n], acc);
-        }
-        yv[c] = __builtin_fmaf(cur.x[c], dsk[c], acc);
-        if (to_top && cl.act) {
-          float* tw = p.top + ((((int64_t)band * p.B + b) * p.W + cl.j) * p.E + e0 + c) * kN;
-#pragma unroll
-          for (int n = 0; n < kN; ++n) tw[n] = h[c][n];
-        }
-      }
-      if (WRITE_Y && cl.act) IO<T>::template stv<EC>(Y + cl.idx * p.E + e0, yv);
+        for (int n = 0; n < kN; ++n) h[c][n] = 0.f;
     }
-    if (p.nbands > 1) __threadfence();   // boundary row of this band is read back by the next one
+    // snapshot of the state before the block (after step t0-1); lanes that have not started or
+    // are past the last column hold nothing the backward needs
+    if (CKPT && m > 0 && row_ok && t0 - 1 - r >= 0 && t0 - 1 - r < p.W) {
+      float* ck = p.ckpt + (((((int64_t)b * p.nbands + band) * p.nblk + m) * p.E + e0) * kN) * kHB + r;
+#pragma unroll
+      for (int c = 0; c < EC; ++c)
+#pragma unroll
+        for (int n = 0; n < kN; ++n) ck[(c * kN + n) * kHB] = h[c][n];
+    }
+    const float* bcb = reinterpret_cast<const float*>(lds + cur * SG::kBytes);
+    const T* xdb = reinterpret_cast<const T*>(lds + cur * SG::kBytes + SG::kBBytes);
+#pragma unroll
+    for (int k = 0; k < kCK; ++k) {
+      const int t = t0 + k;
+      if (t < T_steps) {
+        const Cell cl = locate(p, b, i, t, r, row_ok);
+        const float* rec = bcb + (k * kHB + r) * SG::kBStride;
+        float xv[EC], dtv[EC], dlv[EC];
+        if constexpr (STAGE_X) {
+          const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
+          IO<T>::template ldv<EC>(xr, xv);
+          IO<T>::template ldv<EC>(xr + CW, dtv);
+          IO<T>::template ldv<EC>(xr + 2 * CW, dlv);
+        } else {
+          IO<T>::template ldv<EC>(X + cl.idx * p.E + e0, xv);
+          IO<T>::template ldv<EC>(DT + cl.idx * p.E + e0, dtv);
+          IO<T>::template ldv<EC>(DL + cl.idx * p.E + e0, dlv);
+        }
+        float yv[EC];
+#pragma unroll
+        for (int c = 0; c < EC; ++c) {
+          const float sT = cl.cT * dtv[c] * xv[c];
+          const float sL = cl.cL * dlv[c] * xv[c];
+          float tp[kN];
+#pragma unroll
+          for (int n = 0; n < kN; ++n) tp[n] = 0.f;
+          if (from_top) {   // first row of a lower band: the row above lives in memory
+            const float* tb = p.top + ((((int64_t)(band - 1) * p.B + b) * p.W + (cl.act ? cl.j : 0)) * p.E + e0 + c) * kN;
+#pragma unroll
+            for (int n = 0; n < kN; ++n) tp[n] = __builtin_nontemporal_load(tb + n);
+          }
+          float acc = 0.f;
+#pragma unroll
+          for (int n = 0; n < kN; ++n) {
+            const float aT = fexp2(__builtin_fmaf(dtv[c], a2t[c][n], cl.offT));
+            const float aL = fexp2(__builtin_fmaf(dlv[c], a2l[c][n], cl.offL));
+            const float hT = from_row_below(h[c][n], tp[n]);
+            float u = sL * rec[kN + n];
+            u = __builtin_fmaf(sT, rec[n], u);
+            u = __builtin_fmaf(aT, hT, u);
+            const float hn = __builtin_fmaf(aL, h[c][n], u);
+            h[c][n] = hn;
+            if (WRITE_Y) acc = __builtin_fmaf(hn, rec[2 * kN + n], acc);
+          }
+          yv[c] = __builtin_fmaf(xv[c], dsk[c], acc);
+          if (to_top && cl.act) {
+            float* tw = p.top + ((((int64_t)band * p.B + b) * p.W + cl.j) * p.E + e0 + c) * kN;
+#pragma unroll
+            for (int n = 0; n < kN; ++n) tw[n] = h[c][n];
+          }
+        }
+        if (WRITE_Y && cl.act) IO<T>::template stv<EC>(Y + cl.idx * p.E + e0, yv);
+      }
+    }
+    if (nm == 0 && p.nbands > 1) __threadfence();   // boundary row of this band is read back by the next one
+    staging_fence();
+    cur ^= 1;
+    band = nband;
+    m = nm;
   }
 }
 
 // ----------------------------------------------------------------------------------- backward
 // Channel sums by lane-swap butterflies.  The wave holds CS channel slots; for a group of CS
 // states every lane lists its values v[0..CS-1] and the folds leave, in the lane of slot q, the
-// sum over all slots of the value that was listed for state fold_state(m, .) with result slot q.
+// sum over all slots of the value listed for the state fold_state(m, .) whose result slot is q.
 // fold_state(m, qi) is the state a lane must list at position qi of group m so that afterwards
 // slot q holds state q*NV + m (NV = 16/CS groups per lane).
 //   CS=4: fold16(fold32(v0,v1), fold32(v2,v3)) leaves position 0,1,2,3 in slot 0,2,1,3.
-//   CS=2: fold32(v0,v1) leaves position 0,1 in slot 0,1.
 template <int CS> __device__ __forceinline__ constexpr int fold_state(int m, int qi) {
   constexpr int NV = kN / CS;
   if (CS == 4) { const int q = (qi == 1) ? 2 : (qi == 2) ? 1 : qi; return q * NV + m; }
@@ -306,212 +399,226 @@ template <int CS> __device__ __forceinline__ constexpr int fold_state(int m, int
   return m;
 }
 
-template <typename T, int CS>
+template <typename T, bool STAGE_X>
 __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParams p) {
+  constexpr int CS = 64 >> kHBShift;     // 4 channel slots
   constexpr int NV = kN / CS;            // channel-summed states a lane holds after the butterflies
-  constexpr int NQ = NV / 4;             // ... as float4s
-  constexpr int SLOT = 3 * NQ * 64;      // float4s per wave in the exchange buffer
+  constexpr int SLOT = 3 * 64;           // float4s per wave in the exchange buffer
+  constexpr int CW = kBwdWaves * CS;
+  using SG = Stage<T, 4, CW>;
+  static_assert(NV == 4, "one float4 of channel sums per lane and tensor");
   extern __shared__ float4 smem[];
-  float4* slots = smem;                                                  // [wave][3][NQ][64]
+  float4* slots = smem;                                                  // [wave][3][64]
   float* a_lds = reinterpret_cast<float*>(smem + kBwdWaves * SLOT);      // [wave][CS][2][16]
+  char* lds = reinterpret_cast<char*>(a_lds + kBwdWaves * CS * 2 * kN);  // 2 staging buffers
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lb = logical_block(p.nwg);
   const int b = lb / p.bpb;
   const int eg = lb % p.bpb;
+  const int e_wg0 = eg * CW;
   const int slot = lane >> kHBShift, r = lane & (kHB - 1);
-  const int e_raw = (eg * kBwdWaves + wave) * CS + slot;
+  const int ch_loc = wave * CS + slot;
+  const int e_raw = e_wg0 + ch_loc;
   const bool ch_ok = e_raw < p.E;           // padding lanes/waves still take part in the barriers
   const int e = ch_ok ? e_raw : p.E - 1;
-
-  {  // A of the wave's channels into LDS (read back state by state; keeps them out of VGPRs)
-    float* mine = a_lds + (wave * CS + slot) * (2 * kN);
-    for (int n = r; n < kN; n += kHB) { mine[n] = p.A2T[e * kN + n]; mine[kN + n] = p.A2L[e * kN + n]; }
-  }
-  const float* a_mine = a_lds + (wave * CS + slot) * (2 * kN);
-  const float dsk = p.Df[e];
-  __syncthreads();
 
   const T* X = static_cast<const T*>(p.x);
   const T* DT = static_cast<const T*>(p.dT);
   const T* DL = static_cast<const T*>(p.dL);
   const T* DY = static_cast<const T*>(p.dy);
+  const T* const xs[4] = {X, DT, DL, DY};
   T* DX = static_cast<T*>(p.dx);
   T* DDT = static_cast<T*>(p.ddT);
   T* DDL = static_cast<T*>(p.ddL);
   const int64_t P = (int64_t)p.B * p.H * p.W;
 
+  int band = p.nbands - 1;
+  int HBk = p.H - band * kHB < kHB ? p.H - band * kHB : kHB;
+  int m = (p.W + HBk - 2) / kCK;     // last block of the last band
+  int cur = 0;
+  stage_block<T, 4, CW, STAGE_X, kBwdWaves>(p, lds, b, band, m * kCK, e_wg0, wave, lane, xs);
+  {  // A of the wave's channels into LDS (read back state by state; keeps them out of VGPRs)
+    float* mine = a_lds + ch_loc * (2 * kN);
+    if (r < kN) { mine[r] = p.A2T[e * kN + r]; mine[kN + r] = p.A2L[e * kN + r]; }
+  }
+  const float* a_mine = a_lds + ch_loc * (2 * kN);
+  const float dsk = p.Df[e];
+  staging_fence();
+
   float accAT[kN], accAL[kN], accD = 0.f;
   float muT[kN], muL[kN];
 #pragma unroll
-  for (int n = 0; n < kN; ++n) { accAT[n] = 0.f; accAL[n] = 0.f; }
+  for (int n = 0; n < kN; ++n) { accAT[n] = 0.f; accAL[n] = 0.f; muT[n] = 0.f; muL[n] = 0.f; }
 
-  for (int band = p.nbands - 1; band >= 0; --band) {
+  while (band >= 0) {
     const int i = band * kHB + r;
-    const int HBk = p.H - band * kHB < kHB ? p.H - band * kHB : kHB;
+    HBk = p.H - band * kHB < kHB ? p.H - band * kHB : kHB;
     const bool row_ok = ch_ok && r < HBk;
     const int T_steps = p.W + HBk - 1;
     const bool from_top = band > 0 && r == 0;
     const bool from_bot = band + 1 < p.nbands && r == kHB - 1;
-#pragma unroll
-    for (int n = 0; n < kN; ++n) { muT[n] = 0.f; muL[n] = 0.f; }
+    const int t0 = m * kCK;
+    int nband = band, nm = m - 1;
+    if (nm < 0) { nband = band - 1; nm = (p.W + kHB - 2) / kCK; }   // bands above are full bands
+    if (nband >= 0)
+      stage_block<T, 4, CW, STAGE_X, kBwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, nband, nm * kCK, e_wg0, wave, lane, xs);
+    const float* bcb = reinterpret_cast<const float*>(lds + cur * SG::kBytes);
+    const T* xdb = reinterpret_cast<const T*>(lds + cur * SG::kBytes + SG::kBBytes);
 
-    for (int m = (T_steps - 1) / kCK; m >= 0; --m) {
-      const int t0 = m * kCK;
-      float hb[kCK + 1][kN];
-      if (m == 0 || !(row_ok && t0 - 1 - r >= 0 && t0 - 1 - r < p.W)) {
+    float hb[kCK + 1][kN];
+    if (m == 0 || !(row_ok && t0 - 1 - r >= 0 && t0 - 1 - r < p.W)) {
 #pragma unroll
-        for (int n = 0; n < kN; ++n) hb[0][n] = 0.f;
-      } else {
-        const float* ck = p.ckpt + (((((int64_t)b * p.nbands + band) * p.nblk + m) * p.E + e) * kN) * kHB + r;
+      for (int n = 0; n < kN; ++n) hb[0][n] = 0.f;
+    } else {
+      const float* ck = p.ckpt + (((((int64_t)b * p.nbands + band) * p.nblk + m) * p.E + e) * kN) * kHB + r;
 #pragma unroll
-        for (int n = 0; n < kN; ++n) hb[0][n] = ck[n * kHB];
-      }
-      // ---- recompute the states of the block
+      for (int n = 0; n < kN; ++n) hb[0][n] = ck[n * kHB];
+    }
+    // ---- recompute the states of the block
 #pragma unroll
-      for (int k = 0; k < kCK; ++k) {
-        const int t = t0 + k;
-        if (t < T_steps) {
-          const Cell cl = locate(p, b, i, t, r, row_ok);
-          float bt[kN], bl[kN];
-          const float xv = IO<T>::ld(X + cl.idx * p.E + e);
-          const float dtv = IO<T>::ld(DT + cl.idx * p.E + e);
-          const float dlv = IO<T>::ld(DL + cl.idx * p.E + e);
-          ld16f(p.bt + cl.idx * p.bc_stride, bt);
-          ld16f(p.bl + cl.idx * p.bc_stride, bl);
-          float tp[kN];
+    for (int k = 0; k < kCK; ++k) {
+      const int t = t0 + k;
+      if (t < T_steps) {
+        const Cell cl = locate(p, b, i, t, r, row_ok);
+        const float* rec = bcb + (k * kHB + r) * SG::kBStride;
+        float xv, dtv, dlv;
+        if constexpr (STAGE_X) {
+          const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
+          xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW);
+        } else {
+          xv = IO<T>::ld(X + cl.idx * p.E + e); dtv = IO<T>::ld(DT + cl.idx * p.E + e); dlv = IO<T>::ld(DL + cl.idx * p.E + e);
+        }
+        float tp[kN];
 #pragma unroll
-          for (int n = 0; n < kN; ++n) tp[n] = 0.f;
-          if (from_top) {
-            const float* tb = p.top + ((((int64_t)(band - 1) * p.B + b) * p.W + (cl.act ? cl.j : 0)) * p.E + e) * kN;
-            ld16f(tb, tp);
-          }
-          const float sT = cl.cT * dtv * xv, sL = cl.cL * dlv * xv;
+        for (int n = 0; n < kN; ++n) tp[n] = 0.f;
+        if (from_top) {
+          const float* tb = p.top + ((((int64_t)(band - 1) * p.B + b) * p.W + (cl.act ? cl.j : 0)) * p.E + e) * kN;
+          ld16f(tb, tp);
+        }
+        const float sT = cl.cT * dtv * xv, sL = cl.cL * dlv * xv;
 #pragma unroll
-          for (int n = 0; n < kN; ++n) {
-            const float aT = fexp2(__builtin_fmaf(dtv, a_mine[n], cl.offT));
-            const float aL = fexp2(__builtin_fmaf(dlv, a_mine[kN + n], cl.offL));
-            const float hT = from_row_below(hb[k][n], tp[n]);
-            float u = sL * bl[n];
-            u = __builtin_fmaf(sT, bt[n], u);
-            u = __builtin_fmaf(aT, hT, u);
-            hb[k + 1][n] = __builtin_fmaf(aL, hb[k][n], u);
-          }
+        for (int n = 0; n < kN; ++n) {
+          const float aT = fexp2(__builtin_fmaf(dtv, a_mine[n], cl.offT));
+          const float aL = fexp2(__builtin_fmaf(dlv, a_mine[kN + n], cl.offL));
+          const float hT = from_row_below(hb[k][n], tp[n]);
+          float u = sL * rec[kN + n];
+          u = __builtin_fmaf(sT, rec[n], u);
+          u = __builtin_fmaf(aT, hT, u);
+          hb[k + 1][n] = __builtin_fmaf(aL, hb[k][n], u);
         }
       }
-      // ---- adjoint over the block, last step first
+    }
+    // ---- adjoint over the block, last step first
 #pragma unroll
-      for (int k = kCK - 1; k >= 0; --k) {
-        const int t = t0 + k;
-        if (t < T_steps) {
-          const Cell cl = locate(p, b, i, t, r, row_ok);
-          float bt[kN], bl[kN], cc[kN];
-          const float xv = IO<T>::ld(X + cl.idx * p.E + e);
-          const float dtv = IO<T>::ld(DT + cl.idx * p.E + e);
-          const float dlv = IO<T>::ld(DL + cl.idx * p.E + e);
-          const float dyv = IO<T>::ld(DY + cl.idx * p.E + e);
-          ld16f(p.bt + cl.idx * p.bc_stride, bt);
-          ld16f(p.bl + cl.idx * p.bc_stride, bl);
-          ld16f(p.cc + cl.idx * p.bc_stride, cc);
-          float* bb = p.bot + (((int64_t)b * p.W + (cl.act ? cl.j : 0)) * p.E + e) * kN;
-          float tp[kN], bo[kN];
+    for (int k = kCK - 1; k >= 0; --k) {
+      const int t = t0 + k;
+      if (t < T_steps) {
+        const Cell cl = locate(p, b, i, t, r, row_ok);
+        const float* rec = bcb + (k * kHB + r) * SG::kBStride;
+        float xv, dtv, dlv, dyv;
+        if constexpr (STAGE_X) {
+          const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
+          xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW); dyv = IO<T>::ld(xr + 3 * CW);
+        } else {
+          xv = IO<T>::ld(X + cl.idx * p.E + e); dtv = IO<T>::ld(DT + cl.idx * p.E + e);
+          dlv = IO<T>::ld(DL + cl.idx * p.E + e); dyv = IO<T>::ld(DY + cl.idx * p.E + e);
+        }
+        float* bb = p.bot + (((int64_t)b * p.W + (cl.act ? cl.j : 0)) * p.E + e) * kN;
+        float tp[kN], bo[kN];
 #pragma unroll
-          for (int n = 0; n < kN; ++n) { tp[n] = 0.f; bo[n] = 0.f; }
-          if (from_top) {
-            const float* tb = p.top + ((((int64_t)(band - 1) * p.B + b) * p.W + (cl.act ? cl.j : 0)) * p.E + e) * kN;
-            ld16f(tb, tp);
+        for (int n = 0; n < kN; ++n) { tp[n] = 0.f; bo[n] = 0.f; }
+        if (from_top) {
+          const float* tb = p.top + ((((int64_t)(band - 1) * p.B + b) * p.W + (cl.act ? cl.j : 0)) * p.E + e) * kN;
+          ld16f(tb, tp);
+        }
+        if (from_bot) {   // muT of the first row of the band below, left there by this wave
+#pragma unroll
+          for (int n = 0; n < kN; ++n) bo[n] = __builtin_nontemporal_load(bb + n);
+        }
+        const float qT = cl.cT * dtv * xv, qL = cl.cL * dlv * xv;   // zero on inactive lanes
+        const float qC = cl.act ? dyv : 0.f;
+        float sT = 0.f, sL = 0.f, zT = 0.f, zL = 0.f;
+        // States are visited in groups of CS so that the channel sums of a group can be folded
+        // as soon as the group is done; afterwards the lane of slot q holds the states
+        // q*NV .. q*NV+NV-1 of its cell.
+        float rC[NV], rBT[NV], rBL[NV];
+#pragma unroll
+        for (int mg = 0; mg < NV; ++mg) {
+          float vC[CS], vBT[CS], vBL[CS];
+#pragma unroll
+          for (int qi = 0; qi < CS; ++qi) {
+            const int n = fold_state<CS>(mg, qi);
+            const float a2t = a_mine[n], a2l = a_mine[kN + n];
+            const float aT = fexp2(__builtin_fmaf(dtv, a2t, cl.offT));
+            const float aL = fexp2(__builtin_fmaf(dlv, a2l, cl.offL));
+            const float mb = from_row_above(muT[n], bo[n]);
+            const float lam = __builtin_fmaf(dyv, rec[2 * kN + n], muL[n] + mb);
+            const float hT = from_row_below(hb[k][n], tp[n]);
+            const float mT = aT * lam, mL = aL * lam;
+            muT[n] = mT;
+            muL[n] = mL;
+            const float ZT = mT * hT, ZL = mL * hb[k][n];
+            accAT[n] = __builtin_fmaf(ZT, dtv, accAT[n]);
+            accAL[n] = __builtin_fmaf(ZL, dlv, accAL[n]);
+            zT = __builtin_fmaf(ZT, a2t, zT);
+            zL = __builtin_fmaf(ZL, a2l, zL);
+            sT = __builtin_fmaf(lam, rec[n], sT);
+            sL = __builtin_fmaf(lam, rec[kN + n], sL);
+            vBT[qi] = qT * lam;
+            vBL[qi] = qL * lam;
+            vC[qi] = qC * hb[k + 1][n];
           }
-          if (from_bot) {   // muT of the first row of the band below, left there by this wave
+          rC[mg] = fold16(fold32(vC[0], vC[1]), fold32(vC[2], vC[3]));
+          rBT[mg] = fold16(fold32(vBT[0], vBT[1]), fold32(vBT[2], vBT[3]));
+          rBL[mg] = fold16(fold32(vBL[0], vBL[1]), fold32(vBL[2], vBL[3]));
+        }
+        if (from_top && cl.act) {   // hand muT of this band's first row to the band above
 #pragma unroll
-            for (int n = 0; n < kN; ++n) bo[n] = __builtin_nontemporal_load(bb + n);
-          }
-          const float qT = cl.cT * dtv * xv, qL = cl.cL * dlv * xv;   // zero on inactive lanes
-          const float qC = cl.act ? dyv : 0.f;
-          float sT = 0.f, sL = 0.f, zT = 0.f, zL = 0.f;
-          // States are visited in groups of CS so that the channel sums of a group (values of
-          // the CS channel slots of the wave) can be folded as soon as the group is done; after
-          // the folds the lane of slot q holds the states q*NV .. q*NV+NV-1 of its cell.
-          float rC[NV], rBT[NV], rBL[NV];
+          for (int n = 0; n < kN; ++n) bb[n] = muT[n];
+        }
+        if (cl.act) {
+          accD = __builtin_fmaf(dyv, xv, accD);
+          IO<T>::st(DDT + cl.idx * p.E + e, __builtin_fmaf(cl.cT * xv, sT, kLn2 * zT));
+          IO<T>::st(DDL + cl.idx * p.E + e, __builtin_fmaf(cl.cL * xv, sL, kLn2 * zL));
+          IO<T>::st(DX + cl.idx * p.E + e, __builtin_fmaf(cl.cT * dtv, sT, __builtin_fmaf(cl.cL * dlv, sL, dyv * dsk)));
+        }
+        // ---- across the waves of the workgroup: per-wave slots, added in wave order
+        __syncthreads();   // the flush of the previous step has finished reading the slots
+        {
+          float4* sw = slots + wave * SLOT + lane;
+          sw[0] = make_float4(rC[0], rC[1], rC[2], rC[3]);
+          sw[64] = make_float4(rBT[0], rBT[1], rBT[2], rBT[3]);
+          sw[128] = make_float4(rBL[0], rBL[1], rBL[2], rBL[3]);
+        }
+        __syncthreads();
+        if (threadIdx.x < SLOT) {
+          const int it = threadIdx.x;
+          const int fl = it & 63, v = it >> 6;
+          const int fr = fl & (kHB - 1), fs = fl >> kHBShift;
+          const int fi = band * kHB + fr, fj = t - fr;
+          if (fi < p.H && fj >= 0 && fj < p.W) {
+            float4 s = slots[it];
 #pragma unroll
-          for (int m = 0; m < NV; ++m) {
-            float vC[CS], vBT[CS], vBL[CS];
-#pragma unroll
-            for (int qi = 0; qi < CS; ++qi) {
-              const int n = fold_state<CS>(m, qi);
-              const float a2t = a_mine[n], a2l = a_mine[kN + n];
-              const float aT = fexp2(__builtin_fmaf(dtv, a2t, cl.offT));
-              const float aL = fexp2(__builtin_fmaf(dlv, a2l, cl.offL));
-              const float mb = from_row_above(muT[n], bo[n]);
-              const float lam = __builtin_fmaf(dyv, cc[n], muL[n] + mb);
-              const float hT = from_row_below(hb[k][n], tp[n]);
-              const float mT = aT * lam, mL = aL * lam;
-              muT[n] = mT;
-              muL[n] = mL;
-              const float ZT = mT * hT, ZL = mL * hb[k][n];
-              accAT[n] = __builtin_fmaf(ZT, dtv, accAT[n]);
-              accAL[n] = __builtin_fmaf(ZL, dlv, accAL[n]);
-              zT = __builtin_fmaf(ZT, a2t, zT);
-              zL = __builtin_fmaf(ZL, a2l, zL);
-              sT = __builtin_fmaf(lam, bt[n], sT);
-              sL = __builtin_fmaf(lam, bl[n], sL);
-              vBT[qi] = qT * lam;
-              vBL[qi] = qL * lam;
-              vC[qi] = qC * hb[k + 1][n];
+            for (int w = 1; w < kBwdWaves; ++w) {
+              const float4 o = slots[w * SLOT + it];
+              s.x += o.x; s.y += o.y; s.z += o.z; s.w += o.w;
             }
-            if constexpr (CS == 4) {
-              rC[m] = fold16(fold32(vC[0], vC[1]), fold32(vC[2], vC[3]));
-              rBT[m] = fold16(fold32(vBT[0], vBT[1]), fold32(vBT[2], vBT[3]));
-              rBL[m] = fold16(fold32(vBL[0], vBL[1]), fold32(vBL[2], vBL[3]));
-            } else if constexpr (CS == 2) {
-              rC[m] = fold32(vC[0], vC[1]);
-              rBT[m] = fold32(vBT[0], vBT[1]);
-              rBL[m] = fold32(vBL[0], vBL[1]);
-            } else {
-              rC[m] = vC[0]; rBT[m] = vBT[0]; rBL[m] = vBL[0];
-            }
-          }
-          if (from_top && cl.act) {   // hand muT of this band's first row to the band above
-#pragma unroll
-            for (int n = 0; n < kN; ++n) bb[n] = muT[n];
-          }
-          if (cl.act) {
-            accD = __builtin_fmaf(dyv, xv, accD);
-            IO<T>::st(DDT + cl.idx * p.E + e, __builtin_fmaf(cl.cT * xv, sT, kLn2 * zT));
-            IO<T>::st(DDL + cl.idx * p.E + e, __builtin_fmaf(cl.cL * xv, sL, kLn2 * zL));
-            IO<T>::st(DX + cl.idx * p.E + e, __builtin_fmaf(cl.cT * dtv, sT, __builtin_fmaf(cl.cL * dlv, sL, dyv * dsk)));
-          }
-          // ... then per-wave slots, added in wave order by the flush
-          __syncthreads();   // the flush of the previous step has finished reading the slots
-          {
-            float4* sw = slots + wave * SLOT + lane;
-#pragma unroll
-            for (int q = 0; q < NQ; ++q) {
-              sw[(0 * NQ + q) * 64] = make_float4(rC[4*q], rC[4*q+1], rC[4*q+2], rC[4*q+3]);
-              sw[(1 * NQ + q) * 64] = make_float4(rBT[4*q], rBT[4*q+1], rBT[4*q+2], rBT[4*q+3]);
-              sw[(2 * NQ + q) * 64] = make_float4(rBL[4*q], rBL[4*q+1], rBL[4*q+2], rBL[4*q+3]);
-            }
-          }
-          __syncthreads();
-          for (int it = threadIdx.x; it < SLOT; it += kBwdWaves * 64) {
-            const int fl = it & 63, q = (it >> 6) % NQ, v = (it >> 6) / NQ;
-            const int fr = fl & (kHB - 1), fs = fl >> kHBShift;
-            const int fi = band * kHB + fr, fj = t - fr;
-            if (fi < p.H && fj >= 0 && fj < p.W) {
-              float4 s = slots[it];
-#pragma unroll
-              for (int w = 1; w < kBwdWaves; ++w) {
-                const float4 o = slots[w * SLOT + it];
-                s.x += o.x; s.y += o.y; s.z += o.z; s.w += o.w;
-              }
-              const int im = p.flip ? p.H - 1 - fi : fi, jm = p.flip ? p.W - 1 - fj : fj;
-              const int64_t cell = ((int64_t)b * p.H + im) * p.W + jm;
-              *reinterpret_cast<float4*>(p.part + (((int64_t)eg * 3 + v) * P + cell) * kN + fs * NV + 4 * q) = s;
-            }
+            const int64_t cell = cell_index(p, b, fi, fj);
+            *reinterpret_cast<float4*>(p.part + (((int64_t)eg * 3 + v) * P + cell) * kN + fs * NV) = s;
           }
         }
       }
     }
-    if (p.nbands > 1) __threadfence();
+    if (m == 0 && p.nbands > 1) {   // band finished: its first-row muT is read back by the band above
+      __threadfence();
+#pragma unroll
+      for (int n = 0; n < kN; ++n) { muT[n] = 0.f; muL[n] = 0.f; }
+    }
+    staging_fence();
+    cur ^= 1;
+    band = nband;
+    m = nm;
   }
 
   // ---- sums over positions: reduce over the rows of the band (lanes of one channel slot)
@@ -522,6 +629,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
 #pragma unroll
   for (int k = 0; k < 2 * kN + 1; ++k) {
     float v = red[k];
+#pragma unroll
     for (int off = kHB >> 1; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
     red[k] = v;
   }
@@ -535,8 +643,9 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
 
 // -------------------------------------------------------------------------- small helper kernels
 template <typename T>
-__global__ void m2d_prep_kernel(const T* AT, const T* AL, const T* D, float* A2T, float* A2L, float* Df, int E) {
+__global__ void m2d_prep_kernel(const T* AT, const T* AL, const T* D, float* zeros, float* A2T, float* A2L, float* Df, int E) {
   const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx < kZeroFloats) zeros[idx] = 0.f;
   if (idx < E * kN) {
     A2T[idx] = IO<T>::ld(AT + idx) * kLog2e;
     A2L[idx] = IO<T>::ld(AL + idx) * kLog2e;
@@ -606,6 +715,7 @@ struct Geometry {
   int HB, hb_shift, CS, nbands, nblk;
   int fwd_ec, fwd_wpb, fwd_bpb;      // forward: channels per lane, waves and workgroups per image
   int bwd_wpb, bwd_bpb;              // backward: waves and workgroups (channel groups) per image
+  bool stage_x;                      // x, delta, dy rows are whole 16-byte chunks: stage them through LDS
   size_t prep_bytes, bc_bytes, ckpt_diag_bytes, top_bytes, bot_bytes, part_bytes, pa_bytes, pd_bytes;
 };
 
@@ -629,14 +739,15 @@ Geometry make_geometry(const m2d_desc* d) {
   const int hb = d->H < g.HB ? d->H : g.HB;
   g.nblk = (d->W + hb - 1 + kCK - 1) / kCK;
   // forward: two channels per lane when that still yields enough waves to fill the device
-  const bool ec2 = (d->E % 2 == 0) && ((int64_t)d->B * ((d->E / 2 + g.CS - 1) / g.CS) >= 2048);
+  const bool ec2 = (d->E % 2 == 0) && ((int64_t)d->B * ((d->E + kFwdWaves * g.CS * 2 - 1) / (kFwdWaves * g.CS * 2)) >= 256);
   g.fwd_ec = ec2 ? 2 : 1;
-  g.fwd_wpb = (d->E / g.fwd_ec + g.CS - 1) / g.CS;
-  g.fwd_bpb = (g.fwd_wpb + kFwdWaves - 1) / kFwdWaves;
-  g.bwd_wpb = (d->E + g.CS - 1) / g.CS;
-  g.bwd_bpb = (g.bwd_wpb + kBwdWaves - 1) / kBwdWaves;
+  g.fwd_bpb = (d->E + kFwdWaves * g.CS * g.fwd_ec - 1) / (kFwdWaves * g.CS * g.fwd_ec);
+  g.fwd_wpb = g.fwd_bpb * kFwdWaves;
+  g.bwd_bpb = (d->E + kBwdWaves * g.CS - 1) / (kBwdWaves * g.CS);
+  g.bwd_wpb = g.bwd_bpb * kBwdWaves;
+  g.stage_x = (d->E % (d->dtype == M2D_BF16 ? 8 : 4)) == 0;
   const size_t P = (size_t)d->B * d->H * d->W;
-  g.prep_bytes = align_up(sizeof(float) * ((size_t)2 * d->E * kN + d->E));
+  g.prep_bytes = align_up(sizeof(float) * (kZeroFloats + (size_t)2 * d->E * kN + d->E));
   g.bc_bytes = d->dtype == M2D_BF16 ? align_up(sizeof(float) * P * 48) : 0;
   g.ckpt_diag_bytes = align_up(sizeof(float) * (size_t)d->B * g.nbands * g.nblk * d->E * kN * g.HB);
   g.top_bytes = g.nbands > 1 ? align_up(sizeof(float) * (size_t)(g.nbands - 1) * d->B * d->W * d->E * kN) : 0;
@@ -669,14 +780,17 @@ void fill_common(ScanParams& sp, const m2d_desc* d, const Geometry& g) {
   sp.flip = (d->flags & M2D_FLAG_FLIP) ? 1 : 0;
 }
 
+// Set-up area: [page of zeros][A_T*log2e][A_L*log2e][D], all fp32.
 template <typename T>
-int launch_prep(const m2d_desc* d, const void* AT, const void* AL, const void* D, float* base, hipStream_t st) {
-  float* A2T = base;
-  float* A2L = base + (size_t)d->E * kN;
-  float* Df = base + (size_t)2 * d->E * kN;
-  const int n = d->E * kN;
+int launch_prep(ScanParams& sp, const m2d_desc* d, const void* AT, const void* AL, const void* D, float* base, hipStream_t st) {
+  float* zeros = base;
+  float* A2T = base + kZeroFloats;
+  float* A2L = A2T + (size_t)d->E * kN;
+  float* Df = A2L + (size_t)d->E * kN;
+  sp.zeros = zeros; sp.A2T = A2T; sp.A2L = A2L; sp.Df = Df;
+  const int n = d->E * kN > kZeroFloats ? d->E * kN : kZeroFloats;
   hipLaunchKernelGGL(m2d_prep_kernel<T>, dim3((n + 255) / 256), dim3(256), 0, st, static_cast<const T*>(AT),
-                     static_cast<const T*>(AL), static_cast<const T*>(D), A2T, A2L, Df, d->E);
+                     static_cast<const T*>(AL), static_cast<const T*>(D), zeros, A2T, A2L, Df, d->E);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
@@ -700,25 +814,37 @@ int stage_bc(ScanParams& sp, const m2d_desc* d, const void* BT, const void* BL, 
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
+template <typename T, int EC, bool CK, bool WY, bool SX>
+int launch_fwd_as(const ScanParams& sp, hipStream_t st) {
+  using SG = Stage<T, 3, kFwdWaves * 4 * EC>;
+  const size_t lds = 2 * (size_t)SG::kBytes;
+  static bool attr = false;   // idempotent, the value never changes
+  if (!attr) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_fwd_kernel<T, EC, CK, WY, SX>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return M2D_ERR_HIP;
+    attr = true;
+  }
+  hipLaunchKernelGGL((m2d_fwd_kernel<T, EC, CK, WY, SX>), dim3((unsigned)sp.nwg), dim3(kFwdWaves * 64), lds, st, sp);
+  return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+}
+
+template <typename T, int EC, bool SX>
+int launch_fwd_mode(const ScanParams& sp, bool ckpt, bool write_y, hipStream_t st) {
+  if (ckpt && write_y) return launch_fwd_as<T, EC, true, true, SX>(sp, st);
+  if (ckpt) return launch_fwd_as<T, EC, true, false, SX>(sp, st);
+  return launch_fwd_as<T, EC, false, true, SX>(sp, st);
+}
+
 template <typename T>
 int launch_fwd(const ScanParams& sp0, const m2d_desc* d, const Geometry& g, bool ckpt, bool write_y, hipStream_t st) {
   ScanParams sp = sp0;
   sp.wpb = g.fwd_wpb;
   sp.bpb = g.fwd_bpb;
   sp.nwg = d->B * g.fwd_bpb;
-  const dim3 grid((unsigned)sp.nwg), block(kFwdWaves * 64);
-#define M2D_FWD(EC, CK, WY) hipLaunchKernelGGL((m2d_fwd_kernel<T, EC, CK, WY>), grid, block, 0, st, sp)
-  if (g.fwd_ec == 2) {
-    if (ckpt && write_y) M2D_FWD(2, true, true);
-    else if (ckpt) M2D_FWD(2, true, false);
-    else M2D_FWD(2, false, true);
-  } else {
-    if (ckpt && write_y) M2D_FWD(1, true, true);
-    else if (ckpt) M2D_FWD(1, true, false);
-    else M2D_FWD(1, false, true);
-  }
-#undef M2D_FWD
-  return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+  if (g.fwd_ec == 2)
+    return g.stage_x ? launch_fwd_mode<T, 2, true>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 2, false>(sp, ckpt, write_y, st);
+  return g.stage_x ? launch_fwd_mode<T, 1, true>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 1, false>(sp, ckpt, write_y, st);
 }
 
 template <typename T>
@@ -727,11 +853,10 @@ int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   char* w = static_cast<char*>(ws);
   float* prep = reinterpret_cast<float*>(w);
   w += g.prep_bytes;
-  sp.A2T = prep; sp.A2L = prep + (size_t)d->E * kN; sp.Df = prep + (size_t)2 * d->E * kN;
   char* keep = ckpt ? static_cast<char*>(ckpt) + g.ckpt_diag_bytes : w;   // [top][widened B,C]
   sp.ckpt = ckpt ? static_cast<float*>(ckpt) : nullptr;
   sp.top = reinterpret_cast<float*>(keep);
-  int rc = launch_prep<T>(d, AT, AL, D, prep, st);
+  int rc = launch_prep<T>(sp, d, AT, AL, D, prep, st);
   if (rc) return rc;
   rc = stage_bc<T>(sp, d, BT, BL, C, reinterpret_cast<float*>(keep + g.top_bytes), false, st);
   if (rc) return rc;
@@ -741,18 +866,18 @@ int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   return rc;
 }
 
-template <typename T, int CS>
+template <typename T, bool SX>
 int launch_bwd(const ScanParams& sp, hipStream_t st) {
-  constexpr int NQ = kN / CS / 4;
-  const size_t lds = sizeof(float4) * kBwdWaves * 3 * NQ * 64 + sizeof(float) * kBwdWaves * CS * 2 * kN;
+  using SG = Stage<T, 4, kBwdWaves * 4>;
+  const size_t lds = sizeof(float4) * kBwdWaves * 3 * 64 + sizeof(float) * kBwdWaves * 4 * 2 * kN + 2 * (size_t)SG::kBytes;
   static bool attr = false;   // idempotent, the value never changes
   if (!attr) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_bwd_kernel<T, CS>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_bwd_kernel<T, SX>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return M2D_ERR_HIP;
     attr = true;
   }
-  hipLaunchKernelGGL((m2d_bwd_kernel<T, CS>), dim3((unsigned)sp.nwg), dim3(kBwdWaves * 64), lds, st, sp);
+  hipLaunchKernelGGL((m2d_bwd_kernel<T, SX>), dim3((unsigned)sp.nwg), dim3(kBwdWaves * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
@@ -762,12 +887,11 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
             void* dBL, void* dC, void* dD, void* ws, hipStream_t st) {
   char* w = static_cast<char*>(ws);
   float* prep = reinterpret_cast<float*>(w); w += g.prep_bytes;
-  sp.A2T = prep; sp.A2L = prep + (size_t)d->E * kN; sp.Df = prep + (size_t)2 * d->E * kN;
   sp.part = reinterpret_cast<float*>(w); w += g.part_bytes;
   sp.pA = reinterpret_cast<float*>(w); w += g.pa_bytes;
   sp.pD = reinterpret_cast<float*>(w); w += g.pd_bytes;
   sp.bot = reinterpret_cast<float*>(w); w += g.bot_bytes;
-  int rc = launch_prep<T>(d, AT, AL, D, prep, st);
+  int rc = launch_prep<T>(sp, d, AT, AL, D, prep, st);
   if (rc) return rc;
   char* ck = ckpt ? const_cast<char*>(static_cast<const char*>(ckpt)) : w;
   sp.ckpt = reinterpret_cast<float*>(ck);
@@ -782,7 +906,7 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   sp.bpb = g.bwd_bpb;
   sp.nwg = d->B * g.bwd_bpb;
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][0], st);
-  rc = launch_bwd<T, 4>(sp, st);
+  rc = g.stage_x ? launch_bwd<T, true>(sp, st) : launch_bwd<T, false>(sp, st);
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][1], st);
   if (rc) return rc;
   const int64_t P = (int64_t)d->B * d->H * d->W;
