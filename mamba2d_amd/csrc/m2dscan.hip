@@ -45,6 +45,7 @@ constexpr int kN = 16;            // states per channel
 constexpr int kCK = M2D_CK;       // checkpoint interval (steps)
 constexpr int kHB = 16;           // rows per band = lanes per DPP row
 constexpr int kHBShift = 4;
+constexpr int kRB = 14;           // grid rows per band; lanes 0 and 15 of a row are boundary ghosts
 constexpr int kFwdWaves = 8;      // waves per forward workgroup
 constexpr int kBwdWaves = 8;      // waves per backward workgroup
 constexpr int kZeroFloats = 64;     // page of zeros at the head of the set-up area
@@ -103,15 +104,14 @@ __device__ __forceinline__ void ld16f(const float* p, float (&v)[kN]) {
   for (int k = 0; k < 4; ++k) { float4 t = q[k]; v[4*k] = t.x; v[4*k+1] = t.y; v[4*k+2] = t.z; v[4*k+3] = t.w; }
 }
 
-// Rows of 16 lanes (one band of one channel slot).  Lane r receives the value of lane r-1 of its
-// row; lane 0 of each row, which has no lane below, keeps `edge` (the state of the last row of
-// the band above, or 0).
-__device__ __forceinline__ float from_row_below(float v, float edge) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(edge), __float_as_int(v), 0x111 /*row_shr:1*/, 0xf, 0xf, false));
+// Rows of 16 lanes (one band of one channel slot).  Lane r receives the value of lane r-1 of
+// its row (lane 0, which has no lane below, receives 0) ...
+__device__ __forceinline__ float from_row_below(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x111 /*row_shr:1*/, 0xf, 0xf, true));
 }
-// Lane r receives the value of lane r+1 of its row; lane 15 keeps `edge`.
-__device__ __forceinline__ float from_row_above(float v, float edge) {
-  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(edge), __float_as_int(v), 0x101 /*row_shl:1*/, 0xf, 0xf, false));
+// ... or the value of lane r+1 (lane 15 receives 0).
+__device__ __forceinline__ float from_row_above(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x101 /*row_shl:1*/, 0xf, 0xf, true));
 }
 __device__ __forceinline__ float fexp2(float v) { return __builtin_amdgcn_exp2f(v); }
 
@@ -130,11 +130,11 @@ __device__ __forceinline__ float fold16(float a, float b) {
 
 struct ScanParams {
   const void *x, *dT, *dL, *dy;
-  const float *bt, *bl, *cc;        // B_T, B_L, C in fp32, element (cell, n) at [cell*bc_stride + n]
+  const float *bt, *bl, *cc;        // B_T, B_L, C in fp32, state n of a cell at [cell*bc_stride + spos(n)]
   const float *A2T, *A2L, *Df;      // A*log2(e) and D in fp32, (E,16) / (E)
   const float* zeros;               // 256 bytes of zeros (source for out-of-grid staging chunks)
   void *y, *dx, *ddT, *ddL;
-  float* ckpt;                      // [B][nbands][nblk][E][16][HB]  state snapshots
+  float* ckpt;                      // [B][nbands][nblk][E][16][16]  state snapshots
   float* top;                       // [nbands-1][B][W][E][16]       last row of each band (forward states)
   float* bot;                       // [B][W][E][16]                 first-row muT of the band below (adjoint)
   float* part;                      // [G][3][P][16]                 per-workgroup channel sums
@@ -142,7 +142,6 @@ struct ScanParams {
   float* pD;                        // [B][E]
   int B, H, W, E;
   int nbands, nblk, bc_stride, flip;
-  int wpb;                          // waves per image (channel groups of CS*EC channels)
   int bpb;                          // workgroups per image
   int nwg;                          // total workgroups
 };
@@ -157,45 +156,40 @@ __device__ __forceinline__ int logical_block(int nwg) {
   return (id & 7) * per + (id >> 3);
 }
 
-__device__ __forceinline__ int64_t cell_index(const ScanParams& p, int b, int i, int j) {
+// offset of cell (i,j) inside its image, in cells
+__device__ __forceinline__ int cell_in_image(const ScanParams& p, int i, int j) {
   const int im = p.flip ? p.H - 1 - i : i;
   const int jm = p.flip ? p.W - 1 - j : j;
-  return ((int64_t)b * p.H + im) * p.W + jm;
+  return im * p.W + jm;
 }
 
-struct Cell {          // what a lane needs to know about its cell at one step
-  bool act;
-  int64_t idx;         // flat (b,i,j) index, clamped to a valid cell when !act
-  float cT, cL, offT, offL;
-  int j;
-};
+// Position of state n inside a 16-float record.  With PERM the four states that the backward
+// folds together (n = q*4 + m for q = 0..3) sit in one float4, in fold order.
+template <bool PERM> __device__ __forceinline__ constexpr int spos(int n) {
+  if (!PERM) return n;
+  const int q = n >> 2, m = n & 3;
+  return 4 * m + ((q == 1) ? 2 : (q == 2) ? 1 : q);
+}
 
-__device__ __forceinline__ Cell locate(const ScanParams& p, int b, int i, int t, int r, bool row_ok) {
-  Cell c;
-  const int j = t - r;
-  c.j = j;
-  c.act = row_ok && j >= 0 && j < p.W;
-  const int ic = i < p.H ? i : p.H - 1;
-  const int jc = j < 0 ? 0 : (j < p.W ? j : p.W - 1);
-  c.idx = cell_index(p, b, ic, jc);
-  const float ninf = -__builtin_huge_valf();
-  if (!c.act)      { c.cT = 0.f;  c.cL = 0.f;  c.offT = ninf; c.offL = ninf; }
-  else if (i == 0) { c.cT = 0.f;  c.cL = 1.f;  c.offT = ninf; c.offL = j == 0 ? ninf : 0.f; }
-  else if (j == 0) { c.cT = 1.f;  c.cL = 0.f;  c.offT = 0.f;  c.offL = ninf; }
-  else             { c.cT = 0.5f; c.cL = 0.5f; c.offT = -1.f; c.offL = -1.f; }
-  return c;
+// state stored at position pos of a record (inverse of spos)
+template <bool PERM> __device__ __forceinline__ constexpr int sinv(int pos) {
+  if (!PERM) return pos;
+  const int m = pos >> 2, qi = pos & 3;
+  return ((qi == 1) ? 2 : (qi == 2) ? 1 : qi) * 4 + m;
 }
 
 // ------------------------------------------------------------------------------ operand staging
 // The operands of a block of kCK steps of a band are copied to LDS one block ahead of their use
 // with direct global->LDS loads (no registers, asynchronous): lane i of a wave-wide load fills
-// the 16-byte chunk i of a 1 KB LDS window.  Two regions per buffer:
-//   BC: per (step k, band row r) a record of 13 chunks: B_T, B_L, C of the cell (r, t0+k-r) as
-//       3 x 16 fp32, plus one pad chunk so that the 16 rows fall in distinct banks;
-//   XD: per (k, r) a record of NT tensors x CW channels of the workgroup in the tensor dtype
-//       (x, deltaT, deltaL[, dy]), plus one pad chunk.  Needs E to be a multiple of the chunk.
+// the 16-byte chunk i of a 1 KB LDS window.  Regions of one buffer:
+//   BC : per (step k, lane row r) a record of 13 chunks: B_T, B_L, C of the cell (row r, column
+//        t0+k-r) as 3 x 16 fp32, plus one pad chunk so that the 16 rows fall in distinct banks;
+//   XD : per (k, r) a record of NT tensors x CW channels of the workgroup in the tensor dtype
+//        (x, deltaT, deltaL[, dy]), plus one pad chunk (needs E to be a multiple of a chunk);
+//   TOP: per (k, channel) the 16 states of the last row of the band above at column t0+k;
+//   BOT: per (k, channel) the 16 muT of the first row of the band below at column t0+k-15.
 // Cells outside the grid read from a page of zeros.
-template <typename T, int NT, int CW>
+template <typename T, int NT, int CW, bool WITH_BOT>
 struct Stage {
   static constexpr int kElem = 16 / sizeof(T);           // elements per chunk
   static constexpr int kCpt = CW / kElem;                // chunks per tensor per cell
@@ -205,46 +199,81 @@ struct Stage {
   static constexpr int kBStride = kBRec * 4;             // BC record stride in floats
   static constexpr int kBChunks = kCK * kHB * kBRec;
   static constexpr int kXChunks = kCK * kHB * kXRec;
-  static constexpr int kBBytes = kBChunks * 16;
-  static constexpr int kBytes = (kBChunks + kXChunks) * 16;   // one buffer
+  static constexpr int kTChunks = kCK * CW * 4;
+  static constexpr int kXOff = kBChunks * 16;
+  static constexpr int kTOff = kXOff + kXChunks * 16;
+  static constexpr int kOOff = kTOff + kTChunks * 16;
+  static constexpr int kBytes = kOOff + (WITH_BOT ? kTChunks * 16 : 0);   // one buffer
   static_assert(CW % kElem == 0, "workgroup channel count must fill whole chunks");
 };
 
+template <int AUX>
 __device__ __forceinline__ void lds_fill16(const void* src, char* lds_window) {
   __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                   (__attribute__((address_space(3))) void*)lds_window, 16, 0, 0);
+                                   (__attribute__((address_space(3))) void*)lds_window, 16, 0, AUX);
 }
 
-template <typename T, int NT, int CW, bool STAGE_X, int NWAVES>
-__device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int b, int band, int t0, int e_wg0,
+struct BandGeom {   // wave-uniform description of the band being swept
+  int band, i0, rows;          // first grid row, number of grid rows (<= kRB)
+  bool has_above, has_below;
+};
+
+template <typename T, int NT, int CW, bool WITH_BOT, bool STAGE_X, int NWAVES>
+__device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int b, const BandGeom& g, int t0, int e_wg0,
                                             int wave, int lane, const T* const (&xs)[NT]) {
-  using SG = Stage<T, NT, CW>;
+  using SG = Stage<T, NT, CW, WITH_BOT>;
+  const int64_t img = (int64_t)b * p.H * p.W;
   for (int c0 = wave * 64; c0 < SG::kBChunks; c0 += NWAVES * 64) {
     const int c = c0 + lane;
     const int rec = c / SG::kBRec, part = c - rec * SG::kBRec;
-    if (c < SG::kBChunks && part < 12) {
-      const int k = rec >> kHBShift, r = rec & (kHB - 1);
-      const int i = band * kHB + r, j = t0 + k - r;
+    const int k = rec >> kHBShift, r = rec & (kHB - 1);
+    if (c < SG::kBChunks && part < 12 && r >= 1 && r <= g.rows) {
+      const int j = t0 + k - r;
       const float* src = p.zeros;
-      if (i < p.H && j >= 0 && j < p.W) {
+      if (j >= 0 && j < p.W) {
         const int tau = part >> 2;
-        src = (tau == 0 ? p.bt : (tau == 1 ? p.bl : p.cc)) + cell_index(p, b, i, j) * p.bc_stride + (part & 3) * 4;
+        src = (tau == 0 ? p.bt : (tau == 1 ? p.bl : p.cc)) + (img + cell_in_image(p, g.i0 + r - 1, j)) * p.bc_stride + (part & 3) * 4;
       }
-      lds_fill16(src, buf + c0 * 16);
+      lds_fill16<0>(src, buf + c0 * 16);
     }
   }
   if constexpr (STAGE_X) {
-    char* xbuf = buf + SG::kBBytes;
     for (int c0 = wave * 64; c0 < SG::kXChunks; c0 += NWAVES * 64) {
       const int c = c0 + lane;
       const int rec = c / SG::kXRec, part = c - rec * SG::kXRec;
-      if (c < SG::kXChunks && part < NT * SG::kCpt) {
-        const int k = rec >> kHBShift, r = rec & (kHB - 1);
-        const int i = band * kHB + r, j = t0 + k - r;
+      const int k = rec >> kHBShift, r = rec & (kHB - 1);
+      if (c < SG::kXChunks && part < NT * SG::kCpt && r >= 1 && r <= g.rows) {
+        const int j = t0 + k - r;
         const int tau = part / SG::kCpt, ch = e_wg0 + (part - tau * SG::kCpt) * SG::kElem;
         const void* src = p.zeros;
-        if (i < p.H && j >= 0 && j < p.W && ch < p.E) src = xs[tau] + cell_index(p, b, i, j) * p.E + ch;
-        lds_fill16(src, xbuf + c0 * 16);
+        if (j >= 0 && j < p.W && ch < p.E) src = xs[tau] + (img + cell_in_image(p, g.i0 + r - 1, j)) * p.E + ch;
+        lds_fill16<0>(src, buf + SG::kXOff + c0 * 16);
+      }
+    }
+  }
+  // boundary rows were written earlier in this launch (or by the forward launch): read them at
+  // device scope, past the L1
+  for (int c0 = wave * 64; c0 < SG::kTChunks; c0 += NWAVES * 64) {
+    const int c = c0 + lane;
+    const int rec = c >> 2, k = rec / CW, ch = e_wg0 + rec - k * CW;
+    if (c < SG::kTChunks) {
+      const int j = t0 + k;
+      const float* src = p.zeros;
+      if (g.has_above && j >= 0 && j < p.W && ch < p.E)
+        src = p.top + ((((int64_t)(g.band - 1) * p.B + b) * p.W + j) * p.E + ch) * kN + (c & 3) * 4;
+      lds_fill16<16>(src, buf + SG::kTOff + c0 * 16);
+    }
+  }
+  if constexpr (WITH_BOT) {
+    for (int c0 = wave * 64; c0 < SG::kTChunks; c0 += NWAVES * 64) {
+      const int c = c0 + lane;
+      const int rec = c >> 2, k = rec / CW, ch = e_wg0 + rec - k * CW;
+      if (c < SG::kTChunks) {
+        const int j = t0 + k - (kHB - 1);
+        const float* src = p.zeros;
+        if (g.has_below && j >= 0 && j < p.W && ch < p.E)
+          src = p.bot + (((int64_t)b * p.W + j) * p.E + ch) * kN + (c & 3) * 4;
+        lds_fill16<16>(src, buf + SG::kOOff + c0 * 16);
       }
     }
   }
@@ -256,14 +285,28 @@ __device__ __forceinline__ void staging_fence() {
   __syncthreads();
 }
 
+// Per-lane, per-step roles.  Lanes 1..14 of every 16-lane row are grid rows of the band; lane 0
+// is a ghost that replays the last row of the band above (it reads its "B_T" from the TOP record
+// with input coefficient 1 and closed gates, so its state IS that row), lane 15 is the ghost of
+// the first row of the band below for the adjoint.  All of this is operand selection: the inner
+// loops have no boundary cases.
+struct LaneRole {
+  bool real;       // a grid row of this band (and a valid channel)
+  bool gtop;       // ghost of the row above
+  bool gbot;       // ghost of the row below (adjoint only)
+  bool first_row;  // grid row 0
+};
+
 // ------------------------------------------------------------------------------------ forward
 template <typename T, int EC, bool CKPT, bool WRITE_Y, bool STAGE_X>
 __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParams p) {
   constexpr int CS = 64 >> kHBShift;
   constexpr int CW = kFwdWaves * CS * EC;
-  using SG = Stage<T, 3, CW>;
+  constexpr bool PERM = sizeof(T) == 2;
+  using SG = Stage<T, 3, CW, false>;
   extern __shared__ float4 smem[];
-  char* lds = reinterpret_cast<char*>(smem);
+  float* zrec = reinterpret_cast<float*>(smem);            // 64 zero floats
+  char* lds = reinterpret_cast<char*>(smem + 16);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lb = logical_block(p.nwg);
@@ -274,6 +317,7 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   const int e_raw = e_wg0 + ch_loc;
   const bool ch_ok = e_raw < p.E;                  // idle lanes still take part in staging and barriers
   const int e0 = ch_ok ? e_raw : p.E - EC;
+  if (threadIdx.x < 64) zrec[threadIdx.x] = 0.f;
 
   float a2t[EC][kN], a2l[EC][kN], dsk[EC];
 #pragma unroll
@@ -288,129 +332,147 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   const T* DL = static_cast<const T*>(p.dL);
   const T* const xs[3] = {X, DT, DL};
   T* Y = static_cast<T*>(p.y);
+  const float ninf = -__builtin_huge_valf();
 
-  int band = 0, m = 0, cur = 0;
-  stage_block<T, 3, CW, STAGE_X, kFwdWaves>(p, lds, b, 0, 0, e_wg0, wave, lane, xs);
-  staging_fence();
+  for (int band = 0; band < p.nbands; ++band) {
+    BandGeom g;
+    g.band = band; g.i0 = band * kRB;
+    g.rows = p.H - g.i0 < kRB ? p.H - g.i0 : kRB;
+    g.has_above = band > 0; g.has_below = band + 1 < p.nbands;
+    const int T_steps = g.has_below ? p.W + kHB - 1 : p.W + g.rows;   // same step count as the backward
+    const int nb = (T_steps + kCK - 1) / kCK;
+    LaneRole ro;
+    ro.real = ch_ok && r >= 1 && r <= g.rows;
+    ro.gtop = ch_ok && r == 0 && g.has_above;
+    ro.gbot = false;
+    ro.first_row = g.i0 + r - 1 == 0;
+    const bool to_top = ro.real && g.has_below && r == kRB;
+    const float oT_in = ro.first_row ? ninf : -1.f, oT_j0 = ro.first_row ? ninf : 0.f, oL_in = ro.first_row ? 0.f : -1.f;
+    const int64_t cell0 = (int64_t)b * p.H * p.W;
+    const int irow = g.i0 + (ro.real ? r - 1 : 0);
 
-  float h[EC][kN];
-  while (band < p.nbands) {
-    const int i = band * kHB + r;
-    const int HBk = p.H - band * kHB < kHB ? p.H - band * kHB : kHB;
-    const bool row_ok = ch_ok && r < HBk;
-    const int T_steps = p.W + HBk - 1;
-    const bool from_top = band > 0 && r == 0;
-    const bool to_top = band + 1 < p.nbands && r == kHB - 1;
-    const int t0 = m * kCK;
-    int nband = band, nm = m + 1;
-    if (nm * kCK >= T_steps) { nband = band + 1; nm = 0; }
-    if (nband < p.nbands)
-      stage_block<T, 3, CW, STAGE_X, kFwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, nband, nm * kCK, e_wg0, wave, lane, xs);
-
-    if (m == 0) {
-#pragma unroll
-      for (int c = 0; c < EC; ++c)
-#pragma unroll
-        for (int n = 0; n < kN; ++n) h[c][n] = 0.f;
-    }
-    // snapshot of the state before the block (after step t0-1); lanes that have not started or
-    // are past the last column hold nothing the backward needs
-    if (CKPT && m > 0 && row_ok && t0 - 1 - r >= 0 && t0 - 1 - r < p.W) {
-      float* ck = p.ckpt + (((((int64_t)b * p.nbands + band) * p.nblk + m) * p.E + e0) * kN) * kHB + r;
-#pragma unroll
-      for (int c = 0; c < EC; ++c)
-#pragma unroll
-        for (int n = 0; n < kN; ++n) ck[(c * kN + n) * kHB] = h[c][n];
-    }
-    const float* bcb = reinterpret_cast<const float*>(lds + cur * SG::kBytes);
-    const T* xdb = reinterpret_cast<const T*>(lds + cur * SG::kBytes + SG::kBBytes);
-#pragma unroll
-    for (int k = 0; k < kCK; ++k) {
-      const int t = t0 + k;
-      if (t < T_steps) {
-        const Cell cl = locate(p, b, i, t, r, row_ok);
-        const float* rec = bcb + (k * kHB + r) * SG::kBStride;
-        float xv[EC], dtv[EC], dlv[EC];
-        if constexpr (STAGE_X) {
-          const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
-          IO<T>::template ldv<EC>(xr, xv);
-          IO<T>::template ldv<EC>(xr + CW, dtv);
-          IO<T>::template ldv<EC>(xr + 2 * CW, dlv);
-        } else {
-          IO<T>::template ldv<EC>(X + cl.idx * p.E + e0, xv);
-          IO<T>::template ldv<EC>(DT + cl.idx * p.E + e0, dtv);
-          IO<T>::template ldv<EC>(DL + cl.idx * p.E + e0, dlv);
-        }
-        float yv[EC];
-#pragma unroll
-        for (int c = 0; c < EC; ++c) {
-          const float sT = cl.cT * dtv[c] * xv[c];
-          const float sL = cl.cL * dlv[c] * xv[c];
-          float tp[kN];
-#pragma unroll
-          for (int n = 0; n < kN; ++n) tp[n] = 0.f;
-          if (from_top) {   // first row of a lower band: the row above lives in memory
-            const float* tb = p.top + ((((int64_t)(band - 1) * p.B + b) * p.W + (cl.act ? cl.j : 0)) * p.E + e0 + c) * kN;
-#pragma unroll
-            for (int n = 0; n < kN; ++n) tp[n] = __builtin_nontemporal_load(tb + n);
-          }
-          float acc = 0.f;
-#pragma unroll
-          for (int n = 0; n < kN; ++n) {
-            const float aT = fexp2(__builtin_fmaf(dtv[c], a2t[c][n], cl.offT));
-            const float aL = fexp2(__builtin_fmaf(dlv[c], a2l[c][n], cl.offL));
-            const float hT = from_row_below(h[c][n], tp[n]);
-            float u = sL * rec[kN + n];
-            u = __builtin_fmaf(sT, rec[n], u);
-            u = __builtin_fmaf(aT, hT, u);
-            const float hn = __builtin_fmaf(aL, h[c][n], u);
-            h[c][n] = hn;
-            if (WRITE_Y) acc = __builtin_fmaf(hn, rec[2 * kN + n], acc);
-          }
-          yv[c] = __builtin_fmaf(xv[c], dsk[c], acc);
-          if (to_top && cl.act) {
-            float* tw = p.top + ((((int64_t)band * p.B + b) * p.W + cl.j) * p.E + e0 + c) * kN;
-#pragma unroll
-            for (int n = 0; n < kN; ++n) tw[n] = h[c][n];
-          }
-        }
-        if (WRITE_Y && cl.act) IO<T>::template stv<EC>(Y + cl.idx * p.E + e0, yv);
-      }
-    }
-    if (nm == 0 && p.nbands > 1) __threadfence();   // boundary row of this band is read back by the next one
+    stage_block<T, 3, CW, false, STAGE_X, kFwdWaves>(p, lds, b, g, 0, e_wg0, wave, lane, xs);
     staging_fence();
-    cur ^= 1;
-    band = nband;
-    m = nm;
+    int cur = 0;
+    float h[EC][kN];
+#pragma unroll
+    for (int c = 0; c < EC; ++c)
+#pragma unroll
+      for (int n = 0; n < kN; ++n) h[c][n] = 0.f;
+
+    for (int m = 0; m < nb; ++m) {
+      const int t0 = m * kCK;
+      if (m + 1 < nb)
+        stage_block<T, 3, CW, false, STAGE_X, kFwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, g, t0 + kCK, e_wg0, wave, lane, xs);
+      // snapshot of the state before the block (after step t0-1); lanes that have not started or
+      // are past the last column hold nothing the backward needs
+      if (CKPT && m > 0 && (ro.real || ro.gtop) && t0 - 1 - r >= 0 && t0 - 1 - r < p.W) {
+        float* ck = p.ckpt + (((((int64_t)b * p.nbands + band) * p.nblk + m) * p.E + e0) * kN) * kHB + r;
+#pragma unroll
+        for (int c = 0; c < EC; ++c)
+#pragma unroll
+          for (int n = 0; n < kN; ++n) ck[(c * kN + n) * kHB] = h[c][n];
+      }
+      const char* bufc = lds + cur * SG::kBytes;
+      const float* bcb = reinterpret_cast<const float*>(bufc);
+      const T* xdb = reinterpret_cast<const T*>(bufc + SG::kXOff);
+      const float* tpb = reinterpret_cast<const float*>(bufc + SG::kTOff);
+#pragma unroll
+      for (int k = 0; k < kCK; ++k) {
+        const int t = t0 + k;
+        if (t < T_steps) {
+          const int j = t - r;
+          const bool inw = j >= 0 && j < p.W;
+          const bool act = ro.real && inw;
+          const bool gact = ro.gtop && inw;
+          float offT = act ? (j == 0 ? oT_j0 : oT_in) : ninf;
+          float offL = (act && j != 0) ? oL_in : ninf;
+          const float cT = act ? (ro.first_row ? 0.f : (j == 0 ? 1.f : 0.5f)) : 0.f;
+          const float cL = act ? (ro.first_row ? 1.f : (j == 0 ? 0.f : 0.5f)) : 0.f;
+          float xv[EC], dtv[EC], dlv[EC];
+          if constexpr (STAGE_X) {
+            const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
+            IO<T>::template ldv<EC>(xr, xv);
+            IO<T>::template ldv<EC>(xr + CW, dtv);
+            IO<T>::template ldv<EC>(xr + 2 * CW, dlv);
+          } else {
+            const int64_t idx = cell0 + cell_in_image(p, irow, inw ? j : 0);
+            IO<T>::template ldv<EC>(X + idx * p.E + e0, xv);
+            IO<T>::template ldv<EC>(DT + idx * p.E + e0, dtv);
+            IO<T>::template ldv<EC>(DL + idx * p.E + e0, dlv);
+          }
+          if (!act) {
+#pragma unroll
+            for (int c = 0; c < EC; ++c) { xv[c] = 0.f; dtv[c] = 0.f; dlv[c] = 0.f; }
+          }
+          float yv[EC];
+#pragma unroll
+          for (int c = 0; c < EC; ++c) {
+            // operand records: a grid row reads B_T, B_L, C of its cell; the ghost reads the row
+            // above as its B_T (and as harmless finite stand-ins for the other two)
+            const float* pbt = act ? bcb + (k * kHB + r) * SG::kBStride : (gact ? tpb + (k * CW + ch_loc + c) * kN : zrec);
+            const float* pbl = act ? pbt + kN : pbt;
+            const float* pcc = act ? pbt + 2 * kN : pbt;
+            const float sT = gact ? 1.f : cT * dtv[c] * xv[c];
+            const float sL = cL * dlv[c] * xv[c];
+            float acc = 0.f;
+#pragma unroll
+            for (int n = 0; n < kN; ++n) {
+              const float aT = fexp2(__builtin_fmaf(dtv[c], a2t[c][n], offT));
+              const float aL = fexp2(__builtin_fmaf(dlv[c], a2l[c][n], offL));
+              const float hT = from_row_below(h[c][n]);
+              float u = sL * pbl[spos<PERM>(n)];
+              u = __builtin_fmaf(sT, pbt[spos<PERM>(n)], u);
+              u = __builtin_fmaf(aT, hT, u);
+              const float hn = __builtin_fmaf(aL, h[c][n], u);
+              h[c][n] = hn;
+              if (WRITE_Y) acc = __builtin_fmaf(hn, pcc[spos<PERM>(n)], acc);
+            }
+            yv[c] = __builtin_fmaf(xv[c], dsk[c], acc);
+            if (to_top && act) {   // last row of the band: the next band's ghost will replay it
+              float* tw = p.top + ((((int64_t)band * p.B + b) * p.W + j) * p.E + e0 + c) * kN;
+#pragma unroll
+              for (int q = 0; q < 4; ++q)
+                reinterpret_cast<float4*>(tw)[q] = make_float4(h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)],
+                                                               h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
+            }
+          }
+          if (WRITE_Y && act) {
+            const int64_t idx = cell0 + cell_in_image(p, irow, j);
+            IO<T>::template stv<EC>(Y + idx * p.E + e0, yv);
+          }
+        }
+      }
+      if (m + 1 == nb && p.nbands > 1) __threadfence();   // the band's last row is read back by the next band
+      staging_fence();
+      cur ^= 1;
+    }
   }
 }
 
 // ----------------------------------------------------------------------------------- backward
-// Channel sums by lane-swap butterflies.  The wave holds CS channel slots; for a group of CS
-// states every lane lists its values v[0..CS-1] and the folds leave, in the lane of slot q, the
-// sum over all slots of the value listed for the state fold_state(m, .) whose result slot is q.
-// fold_state(m, qi) is the state a lane must list at position qi of group m so that afterwards
-// slot q holds state q*NV + m (NV = 16/CS groups per lane).
-//   CS=4: fold16(fold32(v0,v1), fold32(v2,v3)) leaves position 0,1,2,3 in slot 0,2,1,3.
-template <int CS> __device__ __forceinline__ constexpr int fold_state(int m, int qi) {
-  constexpr int NV = kN / CS;
-  if (CS == 4) { const int q = (qi == 1) ? 2 : (qi == 2) ? 1 : qi; return q * NV + m; }
-  if (CS == 2) return qi * NV + m;
-  return m;
+// Channel sums by lane-swap butterflies.  The wave holds 4 channel slots; for a group of 4 states
+// every lane lists its values v[0..3] and fold16(fold32(v0,v1), fold32(v2,v3)) leaves, in the
+// lane of slot 0,2,1,3, the sum over all slots of the value at position 0,1,2,3.
+// fold_state(m, qi) is the state to list at position qi of group m so that afterwards slot q
+// holds state q*4 + m.
+__device__ __forceinline__ constexpr int fold_state(int m, int qi) {
+  const int q = (qi == 1) ? 2 : (qi == 2) ? 1 : qi;
+  return q * 4 + m;
 }
 
 template <typename T, bool STAGE_X>
 __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParams p) {
   constexpr int CS = 64 >> kHBShift;     // 4 channel slots
-  constexpr int NV = kN / CS;            // channel-summed states a lane holds after the butterflies
   constexpr int SLOT = 3 * 64;           // float4s per wave in the exchange buffer
   constexpr int CW = kBwdWaves * CS;
-  using SG = Stage<T, 4, CW>;
-  static_assert(NV == 4, "one float4 of channel sums per lane and tensor");
+  constexpr bool PERM = sizeof(T) == 2;
+  using SG = Stage<T, 4, CW, true>;
   extern __shared__ float4 smem[];
   float4* slots = smem;                                                  // [wave][3][64]
-  float* a_lds = reinterpret_cast<float*>(smem + kBwdWaves * SLOT);      // [wave][CS][2][16]
-  char* lds = reinterpret_cast<char*>(a_lds + kBwdWaves * CS * 2 * kN);  // 2 staging buffers
+  float* a_lds = reinterpret_cast<float*>(smem + kBwdWaves * SLOT);      // [wave][CS][2][16], fold order
+  float* zrec = a_lds + kBwdWaves * CS * 2 * kN;                         // 64 zero floats
+  char* lds = reinterpret_cast<char*>(zrec + 64);                        // 2 staging buffers
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lb = logical_block(p.nwg);
@@ -422,6 +484,14 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   const int e_raw = e_wg0 + ch_loc;
   const bool ch_ok = e_raw < p.E;           // padding lanes/waves still take part in the barriers
   const int e = ch_ok ? e_raw : p.E - 1;
+  {  // A of the wave's channels into LDS in fold order (read back group by group)
+    float* mine = a_lds + ch_loc * (2 * kN);
+    mine[spos<true>(r)] = p.A2T[e * kN + r];
+    mine[kN + spos<true>(r)] = p.A2L[e * kN + r];
+    if (threadIdx.x < 64) zrec[threadIdx.x] = 0.f;
+  }
+  const float* a_mine = a_lds + ch_loc * (2 * kN);
+  const float dsk = p.Df[e];
 
   const T* X = static_cast<const T*>(p.x);
   const T* DT = static_cast<const T*>(p.dT);
@@ -432,193 +502,205 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   T* DDT = static_cast<T*>(p.ddT);
   T* DDL = static_cast<T*>(p.ddL);
   const int64_t P = (int64_t)p.B * p.H * p.W;
-
-  int band = p.nbands - 1;
-  int HBk = p.H - band * kHB < kHB ? p.H - band * kHB : kHB;
-  int m = (p.W + HBk - 2) / kCK;     // last block of the last band
-  int cur = 0;
-  stage_block<T, 4, CW, STAGE_X, kBwdWaves>(p, lds, b, band, m * kCK, e_wg0, wave, lane, xs);
-  {  // A of the wave's channels into LDS (read back state by state; keeps them out of VGPRs)
-    float* mine = a_lds + ch_loc * (2 * kN);
-    if (r < kN) { mine[r] = p.A2T[e * kN + r]; mine[kN + r] = p.A2L[e * kN + r]; }
-  }
-  const float* a_mine = a_lds + ch_loc * (2 * kN);
-  const float dsk = p.Df[e];
-  staging_fence();
+  const float ninf = -__builtin_huge_valf();
 
   float accAT[kN], accAL[kN], accD = 0.f;
   float muT[kN], muL[kN];
 #pragma unroll
-  for (int n = 0; n < kN; ++n) { accAT[n] = 0.f; accAL[n] = 0.f; muT[n] = 0.f; muL[n] = 0.f; }
+  for (int n = 0; n < kN; ++n) { accAT[n] = 0.f; accAL[n] = 0.f; }
 
-  while (band >= 0) {
-    const int i = band * kHB + r;
-    HBk = p.H - band * kHB < kHB ? p.H - band * kHB : kHB;
-    const bool row_ok = ch_ok && r < HBk;
-    const int T_steps = p.W + HBk - 1;
-    const bool from_top = band > 0 && r == 0;
-    const bool from_bot = band + 1 < p.nbands && r == kHB - 1;
-    const int t0 = m * kCK;
-    int nband = band, nm = m - 1;
-    if (nm < 0) { nband = band - 1; nm = (p.W + kHB - 2) / kCK; }   // bands above are full bands
-    if (nband >= 0)
-      stage_block<T, 4, CW, STAGE_X, kBwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, nband, nm * kCK, e_wg0, wave, lane, xs);
-    const float* bcb = reinterpret_cast<const float*>(lds + cur * SG::kBytes);
-    const T* xdb = reinterpret_cast<const T*>(lds + cur * SG::kBytes + SG::kBBytes);
+  for (int band = p.nbands - 1; band >= 0; --band) {
+    BandGeom g;
+    g.band = band; g.i0 = band * kRB;
+    g.rows = p.H - g.i0 < kRB ? p.H - g.i0 : kRB;
+    g.has_above = band > 0; g.has_below = band + 1 < p.nbands;
+    const int T_steps = g.has_below ? p.W + kHB - 1 : p.W + g.rows;   // the lower ghost trails by 15 steps
+    const int nb = (T_steps + kCK - 1) / kCK;
+    LaneRole ro;
+    ro.real = ch_ok && r >= 1 && r <= g.rows;
+    ro.gtop = ch_ok && r == 0 && g.has_above;
+    ro.gbot = ch_ok && r == kHB - 1 && g.has_below;
+    ro.first_row = g.i0 + r - 1 == 0;
+    const bool to_bot = ro.real && g.has_above && r == 1;
+    const float oT_in = ro.first_row ? ninf : -1.f, oT_j0 = ro.first_row ? ninf : 0.f, oL_in = ro.first_row ? 0.f : -1.f;
+    const int64_t cell0 = (int64_t)b * p.H * p.W;
+    const int irow = g.i0 + (ro.real ? r - 1 : 0);
 
-    float hb[kCK + 1][kN];
-    if (m == 0 || !(row_ok && t0 - 1 - r >= 0 && t0 - 1 - r < p.W)) {
-#pragma unroll
-      for (int n = 0; n < kN; ++n) hb[0][n] = 0.f;
-    } else {
-      const float* ck = p.ckpt + (((((int64_t)b * p.nbands + band) * p.nblk + m) * p.E + e) * kN) * kHB + r;
-#pragma unroll
-      for (int n = 0; n < kN; ++n) hb[0][n] = ck[n * kHB];
-    }
-    // ---- recompute the states of the block
-#pragma unroll
-    for (int k = 0; k < kCK; ++k) {
-      const int t = t0 + k;
-      if (t < T_steps) {
-        const Cell cl = locate(p, b, i, t, r, row_ok);
-        const float* rec = bcb + (k * kHB + r) * SG::kBStride;
-        float xv, dtv, dlv;
-        if constexpr (STAGE_X) {
-          const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
-          xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW);
-        } else {
-          xv = IO<T>::ld(X + cl.idx * p.E + e); dtv = IO<T>::ld(DT + cl.idx * p.E + e); dlv = IO<T>::ld(DL + cl.idx * p.E + e);
-        }
-        float tp[kN];
-#pragma unroll
-        for (int n = 0; n < kN; ++n) tp[n] = 0.f;
-        if (from_top) {
-          const float* tb = p.top + ((((int64_t)(band - 1) * p.B + b) * p.W + (cl.act ? cl.j : 0)) * p.E + e) * kN;
-          ld16f(tb, tp);
-        }
-        const float sT = cl.cT * dtv * xv, sL = cl.cL * dlv * xv;
-#pragma unroll
-        for (int n = 0; n < kN; ++n) {
-          const float aT = fexp2(__builtin_fmaf(dtv, a_mine[n], cl.offT));
-          const float aL = fexp2(__builtin_fmaf(dlv, a_mine[kN + n], cl.offL));
-          const float hT = from_row_below(hb[k][n], tp[n]);
-          float u = sL * rec[kN + n];
-          u = __builtin_fmaf(sT, rec[n], u);
-          u = __builtin_fmaf(aT, hT, u);
-          hb[k + 1][n] = __builtin_fmaf(aL, hb[k][n], u);
-        }
-      }
-    }
-    // ---- adjoint over the block, last step first
-#pragma unroll
-    for (int k = kCK - 1; k >= 0; --k) {
-      const int t = t0 + k;
-      if (t < T_steps) {
-        const Cell cl = locate(p, b, i, t, r, row_ok);
-        const float* rec = bcb + (k * kHB + r) * SG::kBStride;
-        float xv, dtv, dlv, dyv;
-        if constexpr (STAGE_X) {
-          const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
-          xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW); dyv = IO<T>::ld(xr + 3 * CW);
-        } else {
-          xv = IO<T>::ld(X + cl.idx * p.E + e); dtv = IO<T>::ld(DT + cl.idx * p.E + e);
-          dlv = IO<T>::ld(DL + cl.idx * p.E + e); dyv = IO<T>::ld(DY + cl.idx * p.E + e);
-        }
-        float* bb = p.bot + (((int64_t)b * p.W + (cl.act ? cl.j : 0)) * p.E + e) * kN;
-        float tp[kN], bo[kN];
-#pragma unroll
-        for (int n = 0; n < kN; ++n) { tp[n] = 0.f; bo[n] = 0.f; }
-        if (from_top) {
-          const float* tb = p.top + ((((int64_t)(band - 1) * p.B + b) * p.W + (cl.act ? cl.j : 0)) * p.E + e) * kN;
-          ld16f(tb, tp);
-        }
-        if (from_bot) {   // muT of the first row of the band below, left there by this wave
-#pragma unroll
-          for (int n = 0; n < kN; ++n) bo[n] = __builtin_nontemporal_load(bb + n);
-        }
-        const float qT = cl.cT * dtv * xv, qL = cl.cL * dlv * xv;   // zero on inactive lanes
-        const float qC = cl.act ? dyv : 0.f;
-        float sT = 0.f, sL = 0.f, zT = 0.f, zL = 0.f;
-        // States are visited in groups of CS so that the channel sums of a group can be folded
-        // as soon as the group is done; afterwards the lane of slot q holds the states
-        // q*NV .. q*NV+NV-1 of its cell.
-        float rC[NV], rBT[NV], rBL[NV];
-#pragma unroll
-        for (int mg = 0; mg < NV; ++mg) {
-          float vC[CS], vBT[CS], vBL[CS];
-#pragma unroll
-          for (int qi = 0; qi < CS; ++qi) {
-            const int n = fold_state<CS>(mg, qi);
-            const float a2t = a_mine[n], a2l = a_mine[kN + n];
-            const float aT = fexp2(__builtin_fmaf(dtv, a2t, cl.offT));
-            const float aL = fexp2(__builtin_fmaf(dlv, a2l, cl.offL));
-            const float mb = from_row_above(muT[n], bo[n]);
-            const float lam = __builtin_fmaf(dyv, rec[2 * kN + n], muL[n] + mb);
-            const float hT = from_row_below(hb[k][n], tp[n]);
-            const float mT = aT * lam, mL = aL * lam;
-            muT[n] = mT;
-            muL[n] = mL;
-            const float ZT = mT * hT, ZL = mL * hb[k][n];
-            accAT[n] = __builtin_fmaf(ZT, dtv, accAT[n]);
-            accAL[n] = __builtin_fmaf(ZL, dlv, accAL[n]);
-            zT = __builtin_fmaf(ZT, a2t, zT);
-            zL = __builtin_fmaf(ZL, a2l, zL);
-            sT = __builtin_fmaf(lam, rec[n], sT);
-            sL = __builtin_fmaf(lam, rec[kN + n], sL);
-            vBT[qi] = qT * lam;
-            vBL[qi] = qL * lam;
-            vC[qi] = qC * hb[k + 1][n];
-          }
-          rC[mg] = fold16(fold32(vC[0], vC[1]), fold32(vC[2], vC[3]));
-          rBT[mg] = fold16(fold32(vBT[0], vBT[1]), fold32(vBT[2], vBT[3]));
-          rBL[mg] = fold16(fold32(vBL[0], vBL[1]), fold32(vBL[2], vBL[3]));
-        }
-        if (from_top && cl.act) {   // hand muT of this band's first row to the band above
-#pragma unroll
-          for (int n = 0; n < kN; ++n) bb[n] = muT[n];
-        }
-        if (cl.act) {
-          accD = __builtin_fmaf(dyv, xv, accD);
-          IO<T>::st(DDT + cl.idx * p.E + e, __builtin_fmaf(cl.cT * xv, sT, kLn2 * zT));
-          IO<T>::st(DDL + cl.idx * p.E + e, __builtin_fmaf(cl.cL * xv, sL, kLn2 * zL));
-          IO<T>::st(DX + cl.idx * p.E + e, __builtin_fmaf(cl.cT * dtv, sT, __builtin_fmaf(cl.cL * dlv, sL, dyv * dsk)));
-        }
-        // ---- across the waves of the workgroup: per-wave slots, added in wave order
-        __syncthreads();   // the flush of the previous step has finished reading the slots
-        {
-          float4* sw = slots + wave * SLOT + lane;
-          sw[0] = make_float4(rC[0], rC[1], rC[2], rC[3]);
-          sw[64] = make_float4(rBT[0], rBT[1], rBT[2], rBT[3]);
-          sw[128] = make_float4(rBL[0], rBL[1], rBL[2], rBL[3]);
-        }
-        __syncthreads();
-        if (threadIdx.x < SLOT) {
-          const int it = threadIdx.x;
-          const int fl = it & 63, v = it >> 6;
-          const int fr = fl & (kHB - 1), fs = fl >> kHBShift;
-          const int fi = band * kHB + fr, fj = t - fr;
-          if (fi < p.H && fj >= 0 && fj < p.W) {
-            float4 s = slots[it];
-#pragma unroll
-            for (int w = 1; w < kBwdWaves; ++w) {
-              const float4 o = slots[w * SLOT + it];
-              s.x += o.x; s.y += o.y; s.z += o.z; s.w += o.w;
-            }
-            const int64_t cell = cell_index(p, b, fi, fj);
-            *reinterpret_cast<float4*>(p.part + (((int64_t)eg * 3 + v) * P + cell) * kN + fs * NV) = s;
-          }
-        }
-      }
-    }
-    if (m == 0 && p.nbands > 1) {   // band finished: its first-row muT is read back by the band above
-      __threadfence();
-#pragma unroll
-      for (int n = 0; n < kN; ++n) { muT[n] = 0.f; muL[n] = 0.f; }
-    }
+    stage_block<T, 4, CW, true, STAGE_X, kBwdWaves>(p, lds, b, g, (nb - 1) * kCK, e_wg0, wave, lane, xs);
     staging_fence();
-    cur ^= 1;
-    band = nband;
-    m = nm;
+    int cur = 0;
+#pragma unroll
+    for (int n = 0; n < kN; ++n) { muT[n] = 0.f; muL[n] = 0.f; }
+
+    for (int m = nb - 1; m >= 0; --m) {
+      const int t0 = m * kCK;
+      if (m > 0)
+        stage_block<T, 4, CW, true, STAGE_X, kBwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, g, t0 - kCK, e_wg0, wave, lane, xs);
+      const char* bufc = lds + cur * SG::kBytes;
+      const float* bcb = reinterpret_cast<const float*>(bufc);
+      const T* xdb = reinterpret_cast<const T*>(bufc + SG::kXOff);
+      const float* tpb = reinterpret_cast<const float*>(bufc + SG::kTOff);
+      const float* bob = reinterpret_cast<const float*>(bufc + SG::kOOff);
+
+      float hb[kCK + 1][kN];
+      if (m == 0 || !((ro.real || ro.gtop) && t0 - 1 - r >= 0 && t0 - 1 - r < p.W)) {
+#pragma unroll
+        for (int n = 0; n < kN; ++n) hb[0][n] = 0.f;
+      } else {
+        const float* ck = p.ckpt + (((((int64_t)b * p.nbands + band) * p.nblk + m) * p.E + e) * kN) * kHB + r;
+#pragma unroll
+        for (int n = 0; n < kN; ++n) hb[0][n] = ck[n * kHB];
+      }
+      // ---- recompute the states of the block
+#pragma unroll
+      for (int k = 0; k < kCK; ++k) {
+        const int t = t0 + k;
+        if (t < T_steps) {
+          const int j = t - r;
+          const bool inw = j >= 0 && j < p.W;
+          const bool act = ro.real && inw;
+          const bool gact = ro.gtop && inw;
+          const float offT = act ? (j == 0 ? oT_j0 : oT_in) : ninf;
+          const float offL = (act && j != 0) ? oL_in : ninf;
+          const float cT = act ? (ro.first_row ? 0.f : (j == 0 ? 1.f : 0.5f)) : 0.f;
+          const float cL = act ? (ro.first_row ? 1.f : (j == 0 ? 0.f : 0.5f)) : 0.f;
+          float xv, dtv, dlv;
+          if constexpr (STAGE_X) {
+            const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
+            xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW);
+          } else {
+            const int64_t idx = cell0 + cell_in_image(p, irow, inw ? j : 0);
+            xv = IO<T>::ld(X + idx * p.E + e); dtv = IO<T>::ld(DT + idx * p.E + e); dlv = IO<T>::ld(DL + idx * p.E + e);
+          }
+          if (!act) { xv = 0.f; dtv = 0.f; dlv = 0.f; }
+          const float* pbt = act ? bcb + (k * kHB + r) * SG::kBStride : (gact ? tpb + (k * CW + ch_loc) * kN : zrec);
+          const float* pbl = act ? pbt + kN : pbt;
+          const float sT = gact ? 1.f : cT * dtv * xv;
+          const float sL = cL * dlv * xv;
+#pragma unroll
+          for (int mg = 0; mg < 4; ++mg) {
+#pragma unroll
+            for (int qi = 0; qi < 4; ++qi) {
+              const int n = fold_state(mg, qi);
+              const float aT = fexp2(__builtin_fmaf(dtv, a_mine[4 * mg + qi], offT));
+              const float aL = fexp2(__builtin_fmaf(dlv, a_mine[kN + 4 * mg + qi], offL));
+              const float hT = from_row_below(hb[k][n]);
+              float u = sL * pbl[spos<PERM>(n)];
+              u = __builtin_fmaf(sT, pbt[spos<PERM>(n)], u);
+              u = __builtin_fmaf(aT, hT, u);
+              hb[k + 1][n] = __builtin_fmaf(aL, hb[k][n], u);
+            }
+          }
+        }
+      }
+      // ---- adjoint over the block, last step first
+#pragma unroll
+      for (int k = kCK - 1; k >= 0; --k) {
+        const int t = t0 + k;
+        if (t < T_steps) {
+          const int j = t - r;
+          const bool inw = j >= 0 && j < p.W;
+          const bool act = ro.real && inw;
+          const bool gact = ro.gbot && inw;     // ghost of the row below: muT := staged row
+          float offT = act ? (j == 0 ? oT_j0 : oT_in) : ninf;
+          const float offL = (act && j != 0) ? oL_in : ninf;
+          const float cT = act ? (ro.first_row ? 0.f : (j == 0 ? 1.f : 0.5f)) : 0.f;
+          const float cL = act ? (ro.first_row ? 1.f : (j == 0 ? 0.f : 0.5f)) : 0.f;
+          if (gact) offT = 0.f;                 // open T gate with delta 0: muT = lambda = staged value
+          float xv, dtv, dlv, dyv;
+          if constexpr (STAGE_X) {
+            const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
+            xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW); dyv = IO<T>::ld(xr + 3 * CW);
+          } else {
+            const int64_t idx = cell0 + cell_in_image(p, irow, inw ? j : 0);
+            xv = IO<T>::ld(X + idx * p.E + e); dtv = IO<T>::ld(DT + idx * p.E + e);
+            dlv = IO<T>::ld(DL + idx * p.E + e); dyv = IO<T>::ld(DY + idx * p.E + e);
+          }
+          if (!act) { dtv = 0.f; dlv = 0.f; dyv = gact ? 1.f : 0.f; xv = 0.f; }
+          const float* pbt = act ? bcb + (k * kHB + r) * SG::kBStride : (gact ? bob + (k * CW + ch_loc) * kN : zrec);
+          const float* pbl = act ? pbt + kN : pbt;
+          const float* pcc = act ? pbt + 2 * kN : pbt;
+          const float qT = cT * dtv * xv, qL = cL * dlv * xv;   // zero on lanes that are not grid cells
+          const float qC = act ? dyv : 0.f;
+          float sT = 0.f, sL = 0.f, zT = 0.f, zL = 0.f;
+          // States are visited in groups of 4 so that the channel sums of a group can be folded as
+          // soon as the group is done; afterwards the lane of slot q holds the states 4q..4q+3.
+          float rC[4], rBT[4], rBL[4];
+#pragma unroll
+          for (int mg = 0; mg < 4; ++mg) {
+            float vC[4], vBT[4], vBL[4];
+#pragma unroll
+            for (int qi = 0; qi < 4; ++qi) {
+              const int n = fold_state(mg, qi);
+              const float a2t = a_mine[4 * mg + qi], a2l = a_mine[kN + 4 * mg + qi];
+              const float aT = fexp2(__builtin_fmaf(dtv, a2t, offT));
+              const float aL = fexp2(__builtin_fmaf(dlv, a2l, offL));
+              const float mb = from_row_above(muT[n]);
+              const float lam = __builtin_fmaf(dyv, pcc[spos<PERM>(n)], muL[n] + mb);
+              const float hT = from_row_below(hb[k][n]);
+              const float mT = aT * lam, mL = aL * lam;
+              muT[n] = mT;
+              muL[n] = mL;
+              const float ZT = mT * hT, ZL = mL * hb[k][n];
+              accAT[n] = __builtin_fmaf(ZT, dtv, accAT[n]);
+              accAL[n] = __builtin_fmaf(ZL, dlv, accAL[n]);
+              zT = __builtin_fmaf(ZT, a2t, zT);
+              zL = __builtin_fmaf(ZL, a2l, zL);
+              sT = __builtin_fmaf(lam, pbt[spos<PERM>(n)], sT);
+              sL = __builtin_fmaf(lam, pbl[spos<PERM>(n)], sL);
+              vBT[qi] = qT * lam;
+              vBL[qi] = qL * lam;
+              vC[qi] = qC * hb[k + 1][n];
+            }
+            rC[mg] = fold16(fold32(vC[0], vC[1]), fold32(vC[2], vC[3]));
+            rBT[mg] = fold16(fold32(vBT[0], vBT[1]), fold32(vBT[2], vBT[3]));
+            rBL[mg] = fold16(fold32(vBL[0], vBL[1]), fold32(vBL[2], vBL[3]));
+          }
+          if (to_bot && act) {   // first row of the band: the band above's lower ghost will replay its muT
+            float* bb = p.bot + (((int64_t)b * p.W + j) * p.E + e) * kN;
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+              reinterpret_cast<float4*>(bb)[q] = make_float4(muT[sinv<PERM>(4 * q)], muT[sinv<PERM>(4 * q + 1)],
+                                                             muT[sinv<PERM>(4 * q + 2)], muT[sinv<PERM>(4 * q + 3)]);
+          }
+          if (act) {
+            const int64_t idx = cell0 + cell_in_image(p, irow, j);
+            accD = __builtin_fmaf(dyv, xv, accD);
+            IO<T>::st(DDT + idx * p.E + e, __builtin_fmaf(cT * xv, sT, kLn2 * zT));
+            IO<T>::st(DDL + idx * p.E + e, __builtin_fmaf(cL * xv, sL, kLn2 * zL));
+            IO<T>::st(DX + idx * p.E + e, __builtin_fmaf(cT * dtv, sT, __builtin_fmaf(cL * dlv, sL, dyv * dsk)));
+          }
+          // ---- across the waves of the workgroup: per-wave slots, added in wave order
+          __syncthreads();   // the flush of the previous step has finished reading the slots
+          {
+            float4* sw = slots + wave * SLOT + lane;
+            sw[0] = make_float4(rC[0], rC[1], rC[2], rC[3]);
+            sw[64] = make_float4(rBT[0], rBT[1], rBT[2], rBT[3]);
+            sw[128] = make_float4(rBL[0], rBL[1], rBL[2], rBL[3]);
+          }
+          __syncthreads();
+          if (threadIdx.x < SLOT) {
+            const int it = threadIdx.x;
+            const int fl = it & 63, v = it >> 6;
+            const int fr = fl & (kHB - 1), fs = fl >> kHBShift;
+            const int fj = t - fr;
+            if (fr >= 1 && fr <= g.rows && fj >= 0 && fj < p.W) {
+              float4 s = slots[it];
+#pragma unroll
+              for (int w = 1; w < kBwdWaves; ++w) {
+                const float4 o = slots[w * SLOT + it];
+                s.x += o.x; s.y += o.y; s.z += o.z; s.w += o.w;
+              }
+              const int64_t cell = cell0 + cell_in_image(p, g.i0 + fr - 1, fj);
+              *reinterpret_cast<float4*>(p.part + (((int64_t)eg * 3 + v) * P + cell) * kN + fs * 4) = s;
+            }
+          }
+        }
+      }
+      if (m == 0 && p.nbands > 1) __threadfence();   // the band's first-row muT is read back by the band above
+      staging_fence();
+      cur ^= 1;
+    }
   }
 
   // ---- sums over positions: reduce over the rows of the band (lanes of one channel slot)
@@ -653,24 +735,23 @@ __global__ void m2d_prep_kernel(const T* AT, const T* AL, const T* D, float* zer
   if (idx < E) Df[idx] = IO<T>::ld(D + idx);
 }
 
-// bf16 B_T, B_L, C -> one fp32 record of 48 values per cell (three runs of 16), so the scan
-// kernels load fp32 operands without unpacking them state by state.
+// bf16 B_T, B_L, C -> one fp32 record of 48 values per cell (three runs of 16, each in fold
+// order, see spos), so the scan kernels read fp32 operands a float4 per state group.
 __global__ void m2d_widen_bc_kernel(const bf16_t* BT, const bf16_t* BL, const bf16_t* C, float* out, int64_t P) {
-  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // one thread per (cell, tensor, half)
-  if (gid >= P * 6) return;
-  const int64_t cell = gid / 6;
-  const int w = (int)(gid % 6), tsr = w >> 1, half = w & 1;
-  const bf16_t* src = (tsr == 0 ? BT : (tsr == 1 ? BL : C)) + cell * kN + half * 8;
-  const uint4 t = *reinterpret_cast<const uint4*>(src);
-  const uint32_t wds[4] = {t.x, t.y, t.z, t.w};
-  float4 lo, hi;
-  lo.x = __uint_as_float(wds[0] << 16); lo.y = __uint_as_float(wds[0] & 0xffff0000u);
-  lo.z = __uint_as_float(wds[1] << 16); lo.w = __uint_as_float(wds[1] & 0xffff0000u);
-  hi.x = __uint_as_float(wds[2] << 16); hi.y = __uint_as_float(wds[2] & 0xffff0000u);
-  hi.z = __uint_as_float(wds[3] << 16); hi.w = __uint_as_float(wds[3] & 0xffff0000u);
-  float4* dst = reinterpret_cast<float4*>(out + cell * 48 + tsr * kN + half * 8);
-  dst[0] = lo;
-  dst[1] = hi;
+  const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // one thread per (cell, tensor)
+  if (gid >= P * 3) return;
+  const int64_t cell = gid / 3;
+  const int tsr = (int)(gid % 3);
+  const bf16_t* src = (tsr == 0 ? BT : (tsr == 1 ? BL : C)) + cell * kN;
+  const uint4 t0 = reinterpret_cast<const uint4*>(src)[0], t1 = reinterpret_cast<const uint4*>(src)[1];
+  const uint32_t wds[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
+  float v[kN];
+#pragma unroll
+  for (int k = 0; k < 8; ++k) { v[2 * k] = __uint_as_float(wds[k] << 16); v[2 * k + 1] = __uint_as_float(wds[k] & 0xffff0000u); }
+  float4* dst = reinterpret_cast<float4*>(out + cell * 48 + tsr * kN);
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+    dst[q] = make_float4(v[sinv<true>(4 * q)], v[sinv<true>(4 * q + 1)], v[sinv<true>(4 * q + 2)], v[sinv<true>(4 * q + 3)]);
 }
 
 // d_C, d_BT, d_BL: add the per-workgroup channel sums in workgroup order and round to T.
@@ -735,9 +816,8 @@ Geometry make_geometry(const m2d_desc* d) {
   g.HB = kHB;
   g.hb_shift = kHBShift;
   g.CS = 64 / g.HB;
-  g.nbands = (d->H + g.HB - 1) / g.HB;
-  const int hb = d->H < g.HB ? d->H : g.HB;
-  g.nblk = (d->W + hb - 1 + kCK - 1) / kCK;
+  g.nbands = (d->H + kRB - 1) / kRB;
+  g.nblk = (d->W + kHB - 1 + kCK - 1) / kCK;
   // forward: two channels per lane when that still yields enough waves to fill the device
   const bool ec2 = (d->E % 2 == 0) && ((int64_t)d->B * ((d->E + kFwdWaves * g.CS * 2 - 1) / (kFwdWaves * g.CS * 2)) >= 256);
   g.fwd_ec = ec2 ? 2 : 1;
@@ -808,7 +888,7 @@ int stage_bc(ScanParams& sp, const m2d_desc* d, const void* BT, const void* BL, 
   sp.bc_stride = 48;
   if (ready) return M2D_OK;
   const int64_t P = (int64_t)d->B * d->H * d->W;
-  hipLaunchKernelGGL(m2d_widen_bc_kernel, dim3((unsigned)((P * 6 + 255) / 256)), dim3(256), 0, st,
+  hipLaunchKernelGGL(m2d_widen_bc_kernel, dim3((unsigned)((P * 3 + 255) / 256)), dim3(256), 0, st,
                      static_cast<const bf16_t*>(BT), static_cast<const bf16_t*>(BL), static_cast<const bf16_t*>(C),
                      wide, P);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
@@ -816,8 +896,8 @@ int stage_bc(ScanParams& sp, const m2d_desc* d, const void* BT, const void* BL, 
 
 template <typename T, int EC, bool CK, bool WY, bool SX>
 int launch_fwd_as(const ScanParams& sp, hipStream_t st) {
-  using SG = Stage<T, 3, kFwdWaves * 4 * EC>;
-  const size_t lds = 2 * (size_t)SG::kBytes;
+  using SG = Stage<T, 3, kFwdWaves * 4 * EC, false>;
+  const size_t lds = 256 + 2 * (size_t)SG::kBytes;
   static bool attr = false;   // idempotent, the value never changes
   if (!attr) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_fwd_kernel<T, EC, CK, WY, SX>),
@@ -839,7 +919,6 @@ int launch_fwd_mode(const ScanParams& sp, bool ckpt, bool write_y, hipStream_t s
 template <typename T>
 int launch_fwd(const ScanParams& sp0, const m2d_desc* d, const Geometry& g, bool ckpt, bool write_y, hipStream_t st) {
   ScanParams sp = sp0;
-  sp.wpb = g.fwd_wpb;
   sp.bpb = g.fwd_bpb;
   sp.nwg = d->B * g.fwd_bpb;
   if (g.fwd_ec == 2)
@@ -868,8 +947,8 @@ int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
 
 template <typename T, bool SX>
 int launch_bwd(const ScanParams& sp, hipStream_t st) {
-  using SG = Stage<T, 4, kBwdWaves * 4>;
-  const size_t lds = sizeof(float4) * kBwdWaves * 3 * 64 + sizeof(float) * kBwdWaves * 4 * 2 * kN + 2 * (size_t)SG::kBytes;
+  using SG = Stage<T, 4, kBwdWaves * 4, true>;
+  const size_t lds = sizeof(float4) * kBwdWaves * 3 * 64 + sizeof(float) * kBwdWaves * 4 * 2 * kN + 256 + 2 * (size_t)SG::kBytes;
   static bool attr = false;   // idempotent, the value never changes
   if (!attr) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_bwd_kernel<T, SX>),
@@ -902,7 +981,6 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
     rc = launch_fwd<T>(sp, d, g, true, false, st);
     if (rc) return rc;
   }
-  sp.wpb = g.bwd_wpb;
   sp.bpb = g.bwd_bpb;
   sp.nwg = d->B * g.bwd_bpb;
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][0], st);
