@@ -21,7 +21,7 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
     # packed fp32 VALU ops are kept out of the generated code on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-    "-Wno-unused-result",
+    "-Wno-unused-result", "-Wno-inline-asm",
 ]
 
 

@@ -11,7 +11,7 @@ import os
 import torch
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libm2dscan.so")
+LIB_PATH = os.environ.get("M2D_LIB") or os.path.join(_HERE, "libm2dscan.so")
 
 M2D_F32, M2D_BF16 = 0, 1
 M2D_FLAG_FLIP = 1

@@ -113,7 +113,11 @@ __device__ __forceinline__ float from_row_below(float v) {
 __device__ __forceinline__ float from_row_above(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x101 /*row_shl:1*/, 0xf, 0xf, true));
 }
+#ifdef M2D_X_NOEXP
+__device__ __forceinline__ float fexp2(float v) { return v * 0.001f; }
+#else
 __device__ __forceinline__ float fexp2(float v) { return __builtin_amdgcn_exp2f(v); }
+#endif
 
 // a[lanes 32..63] <-> b[lanes 0..31]; returns a+b: lanes 0..31 hold the two-half sum of a,
 // lanes 32..63 that of b.
@@ -207,10 +211,18 @@ struct Stage {
   static_assert(CW % kElem == 0, "workgroup channel count must fill whole chunks");
 };
 
-template <int AUX>
+// One wave-wide direct load: lane i copies 16 bytes from its own global address to
+// lds_window + 16*i.  Written as inline assembly on purpose: the copy is asynchronous, and its
+// completion is awaited once per block by staging_landed() (counter vmcnt), not before every LDS
+// read that follows it, which is what the compiler does for the builtin.
+// DEVICE_SCOPE: read past the L1 (data written earlier in the same launch by this workgroup).
+template <bool DEVICE_SCOPE>
 __device__ __forceinline__ void lds_fill16(const void* src, char* lds_window) {
-  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void*)src,
-                                   (__attribute__((address_space(3))) void*)lds_window, 16, 0, AUX);
+  const uint32_t base = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) char*)lds_window);
+  if constexpr (DEVICE_SCOPE)
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off sc1" ::"v"(src), "s"(base) : "memory", "m0");
+  else
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(base) : "memory", "m0");
 }
 
 struct BandGeom {   // wave-uniform description of the band being swept
@@ -220,7 +232,7 @@ struct BandGeom {   // wave-uniform description of the band being swept
 
 template <typename T, int NT, int CW, bool WITH_BOT, bool STAGE_X, int NWAVES>
 __device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int b, const BandGeom& g, int t0, int e_wg0,
-                                            int wave, int lane, const T* const (&xs)[NT]) {
+                                            int wave, int lane, const T* x0, const T* x1, const T* x2, const T* x3) {
   using SG = Stage<T, NT, CW, WITH_BOT>;
   const int64_t img = (int64_t)b * p.H * p.W;
   for (int c0 = wave * 64; c0 < SG::kBChunks; c0 += NWAVES * 64) {
@@ -230,11 +242,9 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int 
     if (c < SG::kBChunks && part < 12 && r >= 1 && r <= g.rows) {
       const int j = t0 + k - r;
       const float* src = p.zeros;
-      if (j >= 0 && j < p.W) {
-        const int tau = part >> 2;
-        src = (tau == 0 ? p.bt : (tau == 1 ? p.bl : p.cc)) + (img + cell_in_image(p, g.i0 + r - 1, j)) * p.bc_stride + (part & 3) * 4;
-      }
-      lds_fill16<0>(src, buf + c0 * 16);
+      if (j >= 0 && j < p.W)   // the packed record holds B_T, B_L, C back to back: chunk `part` of 12
+        src = p.bt + (img + cell_in_image(p, g.i0 + r - 1, j)) * p.bc_stride + part * 4;
+      lds_fill16<false>(src, buf + c0 * 16);
     }
   }
   if constexpr (STAGE_X) {
@@ -246,8 +256,12 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int 
         const int j = t0 + k - r;
         const int tau = part / SG::kCpt, ch = e_wg0 + (part - tau * SG::kCpt) * SG::kElem;
         const void* src = p.zeros;
-        if (j >= 0 && j < p.W && ch < p.E) src = xs[tau] + (img + cell_in_image(p, g.i0 + r - 1, j)) * p.E + ch;
-        lds_fill16<0>(src, buf + SG::kXOff + c0 * 16);
+        if (j >= 0 && j < p.W && ch < p.E) {
+          // selected with compares: an indexed pointer table would live in (scratch) memory
+          const T* base = tau == 0 ? x0 : (tau == 1 ? x1 : (tau == 2 ? x2 : x3));
+          src = base + (img + cell_in_image(p, g.i0 + r - 1, j)) * p.E + ch;
+        }
+        lds_fill16<false>(src, buf + SG::kXOff + c0 * 16);
       }
     }
   }
@@ -261,7 +275,7 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int 
       const float* src = p.zeros;
       if (g.has_above && j >= 0 && j < p.W && ch < p.E)
         src = p.top + ((((int64_t)(g.band - 1) * p.B + b) * p.W + j) * p.E + ch) * kN + (c & 3) * 4;
-      lds_fill16<16>(src, buf + SG::kTOff + c0 * 16);
+      lds_fill16<true>(src, buf + SG::kTOff + c0 * 16);
     }
   }
   if constexpr (WITH_BOT) {
@@ -273,15 +287,22 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int 
         const float* src = p.zeros;
         if (g.has_below && j >= 0 && j < p.W && ch < p.E)
           src = p.bot + (((int64_t)b * p.W + j) * p.E + ch) * kN + (c & 3) * 4;
-        lds_fill16<16>(src, buf + SG::kOOff + c0 * 16);
+        lds_fill16<true>(src, buf + SG::kOOff + c0 * 16);
       }
     }
   }
 }
 
-// all direct-to-LDS loads of this wave have landed; then meet the other waves
+// Every load the compiler knows about has returned (vmcnt 0, other counters untouched).  Placed
+// after the start-up loads so that no conservative wait for them is emitted inside the main
+// loop, where it would also wait for the asynchronous staging copies.
+__device__ __forceinline__ void settle_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
+
+// all direct-to-LDS loads of this wave have landed ...
+__device__ __forceinline__ void staging_landed() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+// ... and those of the other waves too
 __device__ __forceinline__ void staging_fence() {
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  staging_landed();
   __syncthreads();
 }
 
@@ -302,7 +323,7 @@ template <typename T, int EC, bool CKPT, bool WRITE_Y, bool STAGE_X>
 __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParams p) {
   constexpr int CS = 64 >> kHBShift;
   constexpr int CW = kFwdWaves * CS * EC;
-  constexpr bool PERM = sizeof(T) == 2;
+  constexpr bool PERM = true;
   using SG = Stage<T, 3, CW, false>;
   extern __shared__ float4 smem[];
   float* zrec = reinterpret_cast<float*>(smem);            // 64 zero floats
@@ -327,10 +348,11 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
     dsk[c] = p.Df[e0 + c];
   }
 
+  settle_loads();
   const T* X = static_cast<const T*>(p.x);
   const T* DT = static_cast<const T*>(p.dT);
   const T* DL = static_cast<const T*>(p.dL);
-  const T* const xs[3] = {X, DT, DL};
+  const T* DY = DL;   // not staged by the forward (NT = 3)
   T* Y = static_cast<T*>(p.y);
   const float ninf = -__builtin_huge_valf();
 
@@ -351,7 +373,7 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
     const int64_t cell0 = (int64_t)b * p.H * p.W;
     const int irow = g.i0 + (ro.real ? r - 1 : 0);
 
-    stage_block<T, 3, CW, false, STAGE_X, kFwdWaves>(p, lds, b, g, 0, e_wg0, wave, lane, xs);
+    stage_block<T, 3, CW, false, STAGE_X, kFwdWaves>(p, lds, b, g, 0, e_wg0, wave, lane, X, DT, DL, DY);
     staging_fence();
     int cur = 0;
     float h[EC][kN];
@@ -363,7 +385,7 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
     for (int m = 0; m < nb; ++m) {
       const int t0 = m * kCK;
       if (m + 1 < nb)
-        stage_block<T, 3, CW, false, STAGE_X, kFwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, g, t0 + kCK, e_wg0, wave, lane, xs);
+        stage_block<T, 3, CW, false, STAGE_X, kFwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, g, t0 + kCK, e_wg0, wave, lane, X, DT, DL, DY);
       // snapshot of the state before the block (after step t0-1); lanes that have not started or
       // are past the last column hold nothing the backward needs
       if (CKPT && m > 0 && (ro.real || ro.gtop) && t0 - 1 - r >= 0 && t0 - 1 - r < p.W) {
@@ -380,6 +402,10 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
 #pragma unroll
       for (int k = 0; k < kCK; ++k) {
         const int t = t0 + k;
+        // The operands of the next block must have landed before the barrier that ends this block.
+        // Waiting here, before the stores of the last step are issued, keeps the latency of those
+        // stores off the critical path (the counter covers loads and stores alike).
+        if (k == kCK - 1) staging_landed();
         if (t < T_steps) {
           const int j = t - r;
           const bool inw = j >= 0 && j < p.W;
@@ -417,16 +443,23 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
             const float sL = cL * dlv[c] * xv[c];
             float acc = 0.f;
 #pragma unroll
-            for (int n = 0; n < kN; ++n) {
-              const float aT = fexp2(__builtin_fmaf(dtv[c], a2t[c][n], offT));
-              const float aL = fexp2(__builtin_fmaf(dlv[c], a2l[c][n], offL));
-              const float hT = from_row_below(h[c][n]);
-              float u = sL * pbl[spos<PERM>(n)];
-              u = __builtin_fmaf(sT, pbt[spos<PERM>(n)], u);
-              u = __builtin_fmaf(aT, hT, u);
-              const float hn = __builtin_fmaf(aL, h[c][n], u);
-              h[c][n] = hn;
-              if (WRITE_Y) acc = __builtin_fmaf(hn, pcc[spos<PERM>(n)], acc);
+            for (int q = 0; q < 4; ++q) {
+              const float4 b4 = reinterpret_cast<const float4*>(pbt)[q], l4 = reinterpret_cast<const float4*>(pbl)[q];
+              const float4 c4 = WRITE_Y ? reinterpret_cast<const float4*>(pcc)[q] : make_float4(0, 0, 0, 0);
+              const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w}, cq[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+              for (int w = 0; w < 4; ++w) {
+                const int n = sinv<PERM>(4 * q + w);
+                const float aT = fexp2(__builtin_fmaf(dtv[c], a2t[c][n], offT));
+                const float aL = fexp2(__builtin_fmaf(dlv[c], a2l[c][n], offL));
+                const float hT = from_row_below(h[c][n]);
+                float u = sL * lq[w];
+                u = __builtin_fmaf(sT, bq[w], u);
+                u = __builtin_fmaf(aT, hT, u);
+                const float hn = __builtin_fmaf(aL, h[c][n], u);
+                h[c][n] = hn;
+                if (WRITE_Y) acc = __builtin_fmaf(hn, cq[w], acc);
+              }
             }
             yv[c] = __builtin_fmaf(xv[c], dsk[c], acc);
             if (to_top && act) {   // last row of the band: the next band's ghost will replay it
@@ -444,7 +477,9 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
         }
       }
       if (m + 1 == nb && p.nbands > 1) __threadfence();   // the band's last row is read back by the next band
-      staging_fence();
+#ifndef M2D_X_NOBLOCKBAR
+      __syncthreads();
+#endif
       cur ^= 1;
     }
   }
@@ -466,7 +501,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   constexpr int CS = 64 >> kHBShift;     // 4 channel slots
   constexpr int SLOT = 3 * 64;           // float4s per wave in the exchange buffer
   constexpr int CW = kBwdWaves * CS;
-  constexpr bool PERM = sizeof(T) == 2;
+  constexpr bool PERM = true;
   using SG = Stage<T, 4, CW, true>;
   extern __shared__ float4 smem[];
   float4* slots = smem;                                                  // [wave][3][64]
@@ -490,14 +525,14 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
     mine[kN + spos<true>(r)] = p.A2L[e * kN + r];
     if (threadIdx.x < 64) zrec[threadIdx.x] = 0.f;
   }
-  const float* a_mine = a_lds + ch_loc * (2 * kN);
+  const float* a_base = a_lds + ch_loc * (2 * kN);
   const float dsk = p.Df[e];
+  settle_loads();
 
   const T* X = static_cast<const T*>(p.x);
   const T* DT = static_cast<const T*>(p.dT);
   const T* DL = static_cast<const T*>(p.dL);
   const T* DY = static_cast<const T*>(p.dy);
-  const T* const xs[4] = {X, DT, DL, DY};
   T* DX = static_cast<T*>(p.dx);
   T* DDT = static_cast<T*>(p.ddT);
   T* DDL = static_cast<T*>(p.ddL);
@@ -526,7 +561,21 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
     const int64_t cell0 = (int64_t)b * p.H * p.W;
     const int irow = g.i0 + (ro.real ? r - 1 : 0);
 
-    stage_block<T, 4, CW, true, STAGE_X, kBwdWaves>(p, lds, b, g, (nb - 1) * kCK, e_wg0, wave, lane, xs);
+    // state snapshot at the start of block mm (zero for lanes that were not under way)
+    float cknext[kN];
+    auto load_ckpt = [&](int mm) {
+      const int tt = mm * kCK;
+      if (mm == 0 || !((ro.real || ro.gtop) && tt - 1 - r >= 0 && tt - 1 - r < p.W)) {
+#pragma unroll
+        for (int n = 0; n < kN; ++n) cknext[n] = 0.f;
+      } else {
+        const float* ck = p.ckpt + (((((int64_t)b * p.nbands + band) * p.nblk + mm) * p.E + e) * kN) * kHB + r;
+#pragma unroll
+        for (int n = 0; n < kN; ++n) cknext[n] = ck[n * kHB];
+      }
+    };
+    load_ckpt(nb - 1);
+    stage_block<T, 4, CW, true, STAGE_X, kBwdWaves>(p, lds, b, g, (nb - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
     staging_fence();
     int cur = 0;
 #pragma unroll
@@ -534,8 +583,6 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
 
     for (int m = nb - 1; m >= 0; --m) {
       const int t0 = m * kCK;
-      if (m > 0)
-        stage_block<T, 4, CW, true, STAGE_X, kBwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, g, t0 - kCK, e_wg0, wave, lane, xs);
       const char* bufc = lds + cur * SG::kBytes;
       const float* bcb = reinterpret_cast<const float*>(bufc);
       const T* xdb = reinterpret_cast<const T*>(bufc + SG::kXOff);
@@ -543,14 +590,10 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
       const float* bob = reinterpret_cast<const float*>(bufc + SG::kOOff);
 
       float hb[kCK + 1][kN];
-      if (m == 0 || !((ro.real || ro.gtop) && t0 - 1 - r >= 0 && t0 - 1 - r < p.W)) {
 #pragma unroll
-        for (int n = 0; n < kN; ++n) hb[0][n] = 0.f;
-      } else {
-        const float* ck = p.ckpt + (((((int64_t)b * p.nbands + band) * p.nblk + m) * p.E + e) * kN) * kHB + r;
-#pragma unroll
-        for (int n = 0; n < kN; ++n) hb[0][n] = ck[n * kHB];
-      }
+      for (int n = 0; n < kN; ++n) hb[0][n] = cknext[n];
+      if (m > 0)
+        stage_block<T, 4, CW, true, STAGE_X, kBwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, g, t0 - kCK, e_wg0, wave, lane, X, DT, DL, DY);
       // ---- recompute the states of the block
 #pragma unroll
       for (int k = 0; k < kCK; ++k) {
@@ -573,23 +616,30 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
             xv = IO<T>::ld(X + idx * p.E + e); dtv = IO<T>::ld(DT + idx * p.E + e); dlv = IO<T>::ld(DL + idx * p.E + e);
           }
           if (!act) { xv = 0.f; dtv = 0.f; dlv = 0.f; }
+          const float* a_mine = a_base;
+          asm volatile("" : "+v"(a_mine));   // keep the per-step reads of A in LDS, not in 32 live registers
           const float* pbt = act ? bcb + (k * kHB + r) * SG::kBStride : (gact ? tpb + (k * CW + ch_loc) * kN : zrec);
           const float* pbl = act ? pbt + kN : pbt;
           const float sT = gact ? 1.f : cT * dtv * xv;
           const float sL = cL * dlv * xv;
 #pragma unroll
           for (int mg = 0; mg < 4; ++mg) {
+            const float4 at4 = reinterpret_cast<const float4*>(a_mine)[mg], al4 = reinterpret_cast<const float4*>(a_mine + kN)[mg];
+            const float4 b4 = reinterpret_cast<const float4*>(pbt)[mg], l4 = reinterpret_cast<const float4*>(pbl)[mg];
+            const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
+            const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w};
 #pragma unroll
             for (int qi = 0; qi < 4; ++qi) {
               const int n = fold_state(mg, qi);
-              const float aT = fexp2(__builtin_fmaf(dtv, a_mine[4 * mg + qi], offT));
-              const float aL = fexp2(__builtin_fmaf(dlv, a_mine[kN + 4 * mg + qi], offL));
+              const float aT = fexp2(__builtin_fmaf(dtv, atq[qi], offT));
+              const float aL = fexp2(__builtin_fmaf(dlv, alq[qi], offL));
               const float hT = from_row_below(hb[k][n]);
-              float u = sL * pbl[spos<PERM>(n)];
-              u = __builtin_fmaf(sT, pbt[spos<PERM>(n)], u);
+              float u = sL * lq[qi];
+              u = __builtin_fmaf(sT, bq[qi], u);
               u = __builtin_fmaf(aT, hT, u);
               hb[k + 1][n] = __builtin_fmaf(aL, hb[k][n], u);
             }
+            __builtin_amdgcn_sched_barrier(0);
           }
         }
       }
@@ -597,6 +647,9 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
 #pragma unroll
       for (int k = kCK - 1; k >= 0; --k) {
         const int t = t0 + k;
+        if (k == 0) staging_landed();   // before the last stores of the block, see the forward kernel
+        // the states of the later steps are dead by now: their registers take the next snapshot
+        if (k == (kCK > 1 ? 1 : 0) && m > 0) load_ckpt(m - 1);
         if (t < T_steps) {
           const int j = t - r;
           const bool inw = j >= 0 && j < p.W;
@@ -617,26 +670,37 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
             dlv = IO<T>::ld(DL + idx * p.E + e); dyv = IO<T>::ld(DY + idx * p.E + e);
           }
           if (!act) { dtv = 0.f; dlv = 0.f; dyv = gact ? 1.f : 0.f; xv = 0.f; }
+          const float* a_mine = a_base;
+          asm volatile("" : "+v"(a_mine));
           const float* pbt = act ? bcb + (k * kHB + r) * SG::kBStride : (gact ? bob + (k * CW + ch_loc) * kN : zrec);
           const float* pbl = act ? pbt + kN : pbt;
           const float* pcc = act ? pbt + 2 * kN : pbt;
           const float qT = cT * dtv * xv, qL = cL * dlv * xv;   // zero on lanes that are not grid cells
           const float qC = act ? dyv : 0.f;
           float sT = 0.f, sL = 0.f, zT = 0.f, zL = 0.f;
+#ifndef M2D_X_NOSLOTBAR
+          __syncthreads();   // the flush of the previous step has finished reading the slots
+#endif
+          float* sw = reinterpret_cast<float*>(slots + wave * SLOT + lane);
           // States are visited in groups of 4 so that the channel sums of a group can be folded as
-          // soon as the group is done; afterwards the lane of slot q holds the states 4q..4q+3.
-          float rC[4], rBT[4], rBL[4];
+          // soon as the group is done; afterwards the lane of slot q holds the states 4q..4q+3
+          // (component mg of its float4 after group mg).
 #pragma unroll
           for (int mg = 0; mg < 4; ++mg) {
+            const float4 at4 = reinterpret_cast<const float4*>(a_mine)[mg], al4 = reinterpret_cast<const float4*>(a_mine + kN)[mg];
+            const float4 b4 = reinterpret_cast<const float4*>(pbt)[mg], l4 = reinterpret_cast<const float4*>(pbl)[mg];
+            const float4 c4 = reinterpret_cast<const float4*>(pcc)[mg];
+            const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
+            const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w}, cq[4] = {c4.x, c4.y, c4.z, c4.w};
             float vC[4], vBT[4], vBL[4];
 #pragma unroll
             for (int qi = 0; qi < 4; ++qi) {
               const int n = fold_state(mg, qi);
-              const float a2t = a_mine[4 * mg + qi], a2l = a_mine[kN + 4 * mg + qi];
+              const float a2t = atq[qi], a2l = alq[qi];
               const float aT = fexp2(__builtin_fmaf(dtv, a2t, offT));
               const float aL = fexp2(__builtin_fmaf(dlv, a2l, offL));
               const float mb = from_row_above(muT[n]);
-              const float lam = __builtin_fmaf(dyv, pcc[spos<PERM>(n)], muL[n] + mb);
+              const float lam = __builtin_fmaf(dyv, cq[qi], muL[n] + mb);
               const float hT = from_row_below(hb[k][n]);
               const float mT = aT * lam, mL = aL * lam;
               muT[n] = mT;
@@ -646,15 +710,16 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
               accAL[n] = __builtin_fmaf(ZL, dlv, accAL[n]);
               zT = __builtin_fmaf(ZT, a2t, zT);
               zL = __builtin_fmaf(ZL, a2l, zL);
-              sT = __builtin_fmaf(lam, pbt[spos<PERM>(n)], sT);
-              sL = __builtin_fmaf(lam, pbl[spos<PERM>(n)], sL);
+              sT = __builtin_fmaf(lam, bq[qi], sT);
+              sL = __builtin_fmaf(lam, lq[qi], sL);
               vBT[qi] = qT * lam;
               vBL[qi] = qL * lam;
               vC[qi] = qC * hb[k + 1][n];
             }
-            rC[mg] = fold16(fold32(vC[0], vC[1]), fold32(vC[2], vC[3]));
-            rBT[mg] = fold16(fold32(vBT[0], vBT[1]), fold32(vBT[2], vBT[3]));
-            rBL[mg] = fold16(fold32(vBL[0], vBL[1]), fold32(vBL[2], vBL[3]));
+            sw[mg] = fold16(fold32(vC[0], vC[1]), fold32(vC[2], vC[3]));
+            sw[64 * 4 + mg] = fold16(fold32(vBT[0], vBT[1]), fold32(vBT[2], vBT[3]));
+            sw[128 * 4 + mg] = fold16(fold32(vBL[0], vBL[1]), fold32(vBL[2], vBL[3]));
+            __builtin_amdgcn_sched_barrier(0);
           }
           if (to_bot && act) {   // first row of the band: the band above's lower ghost will replay its muT
             float* bb = p.bot + (((int64_t)b * p.W + j) * p.E + e) * kN;
@@ -670,15 +735,10 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
             IO<T>::st(DDL + idx * p.E + e, __builtin_fmaf(cL * xv, sL, kLn2 * zL));
             IO<T>::st(DX + idx * p.E + e, __builtin_fmaf(cT * dtv, sT, __builtin_fmaf(cL * dlv, sL, dyv * dsk)));
           }
-          // ---- across the waves of the workgroup: per-wave slots, added in wave order
-          __syncthreads();   // the flush of the previous step has finished reading the slots
-          {
-            float4* sw = slots + wave * SLOT + lane;
-            sw[0] = make_float4(rC[0], rC[1], rC[2], rC[3]);
-            sw[64] = make_float4(rBT[0], rBT[1], rBT[2], rBT[3]);
-            sw[128] = make_float4(rBL[0], rBL[1], rBL[2], rBL[3]);
-          }
+          // ---- across the waves of the workgroup: the per-wave slots are added in wave order
+#ifndef M2D_X_NOSLOTBAR
           __syncthreads();
+#endif
           if (threadIdx.x < SLOT) {
             const int it = threadIdx.x;
             const int fl = it & 63, v = it >> 6;
@@ -698,7 +758,9 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
         }
       }
       if (m == 0 && p.nbands > 1) __threadfence();   // the band's first-row muT is read back by the band above
-      staging_fence();
+#ifndef M2D_X_NOBLOCKBAR
+      __syncthreads();
+#endif
       cur ^= 1;
     }
   }
@@ -735,19 +797,24 @@ __global__ void m2d_prep_kernel(const T* AT, const T* AL, const T* D, float* zer
   if (idx < E) Df[idx] = IO<T>::ld(D + idx);
 }
 
-// bf16 B_T, B_L, C -> one fp32 record of 48 values per cell (three runs of 16, each in fold
-// order, see spos), so the scan kernels read fp32 operands a float4 per state group.
-__global__ void m2d_widen_bc_kernel(const bf16_t* BT, const bf16_t* BL, const bf16_t* C, float* out, int64_t P) {
+// B_T, B_L, C -> one fp32 record of 48 values per cell (three runs of 16, each in fold order,
+// see spos), so the scan kernels read their operands a float4 per state group.
+template <typename T>
+__global__ void m2d_pack_bc_kernel(const T* BT, const T* BL, const T* C, float* out, int64_t P) {
   const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;   // one thread per (cell, tensor)
   if (gid >= P * 3) return;
   const int64_t cell = gid / 3;
   const int tsr = (int)(gid % 3);
-  const bf16_t* src = (tsr == 0 ? BT : (tsr == 1 ? BL : C)) + cell * kN;
-  const uint4 t0 = reinterpret_cast<const uint4*>(src)[0], t1 = reinterpret_cast<const uint4*>(src)[1];
-  const uint32_t wds[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
+  const T* src = (tsr == 0 ? BT : (tsr == 1 ? BL : C)) + cell * kN;
   float v[kN];
+  if constexpr (sizeof(T) == 2) {
+    const uint4 t0 = reinterpret_cast<const uint4*>(src)[0], t1 = reinterpret_cast<const uint4*>(src)[1];
+    const uint32_t wds[8] = {t0.x, t0.y, t0.z, t0.w, t1.x, t1.y, t1.z, t1.w};
 #pragma unroll
-  for (int k = 0; k < 8; ++k) { v[2 * k] = __uint_as_float(wds[k] << 16); v[2 * k + 1] = __uint_as_float(wds[k] & 0xffff0000u); }
+    for (int k = 0; k < 8; ++k) { v[2 * k] = __uint_as_float(wds[k] << 16); v[2 * k + 1] = __uint_as_float(wds[k] & 0xffff0000u); }
+  } else {
+    ld16f(reinterpret_cast<const float*>(src), v);
+  }
   float4* dst = reinterpret_cast<float4*>(out + cell * 48 + tsr * kN);
 #pragma unroll
   for (int q = 0; q < 4; ++q)
@@ -828,7 +895,7 @@ Geometry make_geometry(const m2d_desc* d) {
   g.stage_x = (d->E % (d->dtype == M2D_BF16 ? 8 : 4)) == 0;
   const size_t P = (size_t)d->B * d->H * d->W;
   g.prep_bytes = align_up(sizeof(float) * (kZeroFloats + (size_t)2 * d->E * kN + d->E));
-  g.bc_bytes = d->dtype == M2D_BF16 ? align_up(sizeof(float) * P * 48) : 0;
+  g.bc_bytes = align_up(sizeof(float) * P * 48);
   g.ckpt_diag_bytes = align_up(sizeof(float) * (size_t)d->B * g.nbands * g.nblk * d->E * kN * g.HB);
   g.top_bytes = g.nbands > 1 ? align_up(sizeof(float) * (size_t)(g.nbands - 1) * d->B * d->W * d->E * kN) : 0;
   g.bot_bytes = g.nbands > 1 ? align_up(sizeof(float) * (size_t)d->B * d->W * d->E * kN) : 0;
@@ -874,23 +941,16 @@ int launch_prep(ScanParams& sp, const m2d_desc* d, const void* AT, const void* A
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
-// Points sp.bt/bl/cc at fp32 B_T, B_L, C: the caller's tensors for fp32 input, a widened copy
-// (made here unless `ready`) for bf16 input.
+// Points sp.bt/bl/cc at the packed fp32 copy of B_T, B_L, C (made here unless `ready`).
 template <typename T>
 int stage_bc(ScanParams& sp, const m2d_desc* d, const void* BT, const void* BL, const void* C, float* wide,
              bool ready, hipStream_t st) {
-  if (sizeof(T) == 4) {
-    sp.bt = static_cast<const float*>(BT); sp.bl = static_cast<const float*>(BL); sp.cc = static_cast<const float*>(C);
-    sp.bc_stride = kN;
-    return M2D_OK;
-  }
   sp.bt = wide; sp.bl = wide + kN; sp.cc = wide + 2 * kN;
   sp.bc_stride = 48;
   if (ready) return M2D_OK;
   const int64_t P = (int64_t)d->B * d->H * d->W;
-  hipLaunchKernelGGL(m2d_widen_bc_kernel, dim3((unsigned)((P * 3 + 255) / 256)), dim3(256), 0, st,
-                     static_cast<const bf16_t*>(BT), static_cast<const bf16_t*>(BL), static_cast<const bf16_t*>(C),
-                     wide, P);
+  hipLaunchKernelGGL(m2d_pack_bc_kernel<T>, dim3((unsigned)((P * 3 + 255) / 256)), dim3(256), 0, st,
+                     static_cast<const T*>(BT), static_cast<const T*>(BL), static_cast<const T*>(C), wide, P);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
