@@ -234,6 +234,13 @@ template <typename T, int NT, int CW, bool WITH_BOT, bool STAGE_X, int NWAVES>
 __device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int b, const BandGeom& g, int t0, int e_wg0,
                                             int wave, int lane, const T* x0, const T* x1, const T* x2, const T* x3) {
   using SG = Stage<T, NT, CW, WITH_BOT>;
+  // The chunk -> (step, row, part) decomposition depends only on the lane; hiding the lane from
+  // the optimiser here keeps it from precomputing all of it once and holding (and spilling)
+  // dozens of registers for the whole kernel.
+  asm volatile("" : "+v"(lane));
+#ifdef M2D_X_NOSTAGE
+  return;
+#endif
   const int64_t img = (int64_t)b * p.H * p.W;
   for (int c0 = wave * 64; c0 < SG::kBChunks; c0 += NWAVES * 64) {
     const int c = c0 + lane;
@@ -470,10 +477,14 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
                                                                h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
             }
           }
+#ifndef M2D_X_NOSTORE
           if (WRITE_Y && act) {
             const int64_t idx = cell0 + cell_in_image(p, irow, j);
             IO<T>::template stv<EC>(Y + idx * p.E + e0, yv);
           }
+#else
+          if (WRITE_Y && act && yv[0] == 123.456f) Y[0] = T{};
+#endif
         }
       }
       if (m + 1 == nb && p.nbands > 1) __threadfence();   // the band's last row is read back by the next band
@@ -588,171 +599,186 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
       const T* xdb = reinterpret_cast<const T*>(bufc + SG::kXOff);
       const float* tpb = reinterpret_cast<const float*>(bufc + SG::kTOff);
       const float* bob = reinterpret_cast<const float*>(bufc + SG::kOOff);
-
-      float hb[kCK + 1][kN];
+      float ck0[kN];
 #pragma unroll
-      for (int n = 0; n < kN; ++n) hb[0][n] = cknext[n];
+      for (int n = 0; n < kN; ++n) ck0[n] = cknext[n];
       if (m > 0)
         stage_block<T, 4, CW, true, STAGE_X, kBwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, g, t0 - kCK, e_wg0, wave, lane, X, DT, DL, DY);
-      // ---- recompute the states of the block
+
+      // The 16 states are swept in two halves of 8 (state groups 0,1 then 2,3), each half
+      // recomputing and then back-propagating the whole block: only 5 x 8 recomputed states are
+      // live at a time.  The state sums of the first half wait in `part4` for the second.
+      float part4[kCK][4];
 #pragma unroll
-      for (int k = 0; k < kCK; ++k) {
-        const int t = t0 + k;
-        if (t < T_steps) {
-          const int j = t - r;
-          const bool inw = j >= 0 && j < p.W;
-          const bool act = ro.real && inw;
-          const bool gact = ro.gtop && inw;
-          const float offT = act ? (j == 0 ? oT_j0 : oT_in) : ninf;
-          const float offL = (act && j != 0) ? oL_in : ninf;
-          const float cT = act ? (ro.first_row ? 0.f : (j == 0 ? 1.f : 0.5f)) : 0.f;
-          const float cL = act ? (ro.first_row ? 1.f : (j == 0 ? 0.f : 0.5f)) : 0.f;
-          float xv, dtv, dlv;
-          if constexpr (STAGE_X) {
-            const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
-            xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW);
-          } else {
-            const int64_t idx = cell0 + cell_in_image(p, irow, inw ? j : 0);
-            xv = IO<T>::ld(X + idx * p.E + e); dtv = IO<T>::ld(DT + idx * p.E + e); dlv = IO<T>::ld(DL + idx * p.E + e);
-          }
-          if (!act) { xv = 0.f; dtv = 0.f; dlv = 0.f; }
-          const float* a_mine = a_base;
-          asm volatile("" : "+v"(a_mine));   // keep the per-step reads of A in LDS, not in 32 live registers
-          const float* pbt = act ? bcb + (k * kHB + r) * SG::kBStride : (gact ? tpb + (k * CW + ch_loc) * kN : zrec);
-          const float* pbl = act ? pbt + kN : pbt;
-          const float sT = gact ? 1.f : cT * dtv * xv;
-          const float sL = cL * dlv * xv;
+      for (int half = 0; half < 2; ++half) {
+        float hb[kCK + 1][8];
 #pragma unroll
-          for (int mg = 0; mg < 4; ++mg) {
-            const float4 at4 = reinterpret_cast<const float4*>(a_mine)[mg], al4 = reinterpret_cast<const float4*>(a_mine + kN)[mg];
-            const float4 b4 = reinterpret_cast<const float4*>(pbt)[mg], l4 = reinterpret_cast<const float4*>(pbl)[mg];
-            const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
-            const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w};
+        for (int mgl = 0; mgl < 2; ++mgl)
 #pragma unroll
-            for (int qi = 0; qi < 4; ++qi) {
-              const int n = fold_state(mg, qi);
-              const float aT = fexp2(__builtin_fmaf(dtv, atq[qi], offT));
-              const float aL = fexp2(__builtin_fmaf(dlv, alq[qi], offL));
-              const float hT = from_row_below(hb[k][n]);
-              float u = sL * lq[qi];
-              u = __builtin_fmaf(sT, bq[qi], u);
-              u = __builtin_fmaf(aT, hT, u);
-              hb[k + 1][n] = __builtin_fmaf(aL, hb[k][n], u);
+          for (int qi = 0; qi < 4; ++qi) hb[0][4 * mgl + qi] = ck0[fold_state(2 * half + mgl, qi)];
+        // ---- recompute the states of the block
+#pragma unroll
+        for (int k = 0; k < kCK; ++k) {
+          const int t = t0 + k;
+          if (t < T_steps) {
+            const int j = t - r;
+            const bool inw = j >= 0 && j < p.W;
+            const bool act = ro.real && inw;
+            const bool gact = ro.gtop && inw;
+            const float offT = act ? (j == 0 ? oT_j0 : oT_in) : ninf;
+            const float offL = (act && j != 0) ? oL_in : ninf;
+            const float cT = act ? (ro.first_row ? 0.f : (j == 0 ? 1.f : 0.5f)) : 0.f;
+            const float cL = act ? (ro.first_row ? 1.f : (j == 0 ? 0.f : 0.5f)) : 0.f;
+            float xv, dtv, dlv;
+            if constexpr (STAGE_X) {
+              const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
+              xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW);
+            } else {
+              const int64_t idx = cell0 + cell_in_image(p, irow, inw ? j : 0);
+              xv = IO<T>::ld(X + idx * p.E + e); dtv = IO<T>::ld(DT + idx * p.E + e); dlv = IO<T>::ld(DL + idx * p.E + e);
             }
-            __builtin_amdgcn_sched_barrier(0);
+            if (!act) { xv = 0.f; dtv = 0.f; dlv = 0.f; }
+            const float* a_mine = a_base;
+            asm volatile("" : "+v"(a_mine));   // keep the per-step reads of A in LDS, not in live registers
+            const float* pbt = act ? bcb + (k * kHB + r) * SG::kBStride : (gact ? tpb + (k * CW + ch_loc) * kN : zrec);
+            const float* pbl = act ? pbt + kN : pbt;
+            const float sT = gact ? 1.f : cT * dtv * xv;
+            const float sL = cL * dlv * xv;
+#pragma unroll
+            for (int mgl = 0; mgl < 2; ++mgl) {
+              const int mg = 2 * half + mgl;
+              const float4 at4 = reinterpret_cast<const float4*>(a_mine)[mg], al4 = reinterpret_cast<const float4*>(a_mine + kN)[mg];
+              const float4 b4 = reinterpret_cast<const float4*>(pbt)[mg], l4 = reinterpret_cast<const float4*>(pbl)[mg];
+              const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
+              const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w};
+#pragma unroll
+              for (int qi = 0; qi < 4; ++qi) {
+                const int s8 = 4 * mgl + qi;
+                const float aT = fexp2(__builtin_fmaf(dtv, atq[qi], offT));
+                const float aL = fexp2(__builtin_fmaf(dlv, alq[qi], offL));
+                const float hT = from_row_below(hb[k][s8]);
+                float u = sL * lq[qi];
+                u = __builtin_fmaf(sT, bq[qi], u);
+                u = __builtin_fmaf(aT, hT, u);
+                hb[k + 1][s8] = __builtin_fmaf(aL, hb[k][s8], u);
+              }
+            }
           }
         }
-      }
-      // ---- adjoint over the block, last step first
+        // ---- adjoint over the block, last step first
 #pragma unroll
-      for (int k = kCK - 1; k >= 0; --k) {
-        const int t = t0 + k;
-        if (k == 0) staging_landed();   // before the last stores of the block, see the forward kernel
-        // the states of the later steps are dead by now: their registers take the next snapshot
-        if (k == (kCK > 1 ? 1 : 0) && m > 0) load_ckpt(m - 1);
-        if (t < T_steps) {
-          const int j = t - r;
-          const bool inw = j >= 0 && j < p.W;
-          const bool act = ro.real && inw;
-          const bool gact = ro.gbot && inw;     // ghost of the row below: muT := staged row
-          float offT = act ? (j == 0 ? oT_j0 : oT_in) : ninf;
-          const float offL = (act && j != 0) ? oL_in : ninf;
-          const float cT = act ? (ro.first_row ? 0.f : (j == 0 ? 1.f : 0.5f)) : 0.f;
-          const float cL = act ? (ro.first_row ? 1.f : (j == 0 ? 0.f : 0.5f)) : 0.f;
-          if (gact) offT = 0.f;                 // open T gate with delta 0: muT = lambda = staged value
-          float xv, dtv, dlv, dyv;
-          if constexpr (STAGE_X) {
-            const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
-            xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW); dyv = IO<T>::ld(xr + 3 * CW);
-          } else {
-            const int64_t idx = cell0 + cell_in_image(p, irow, inw ? j : 0);
-            xv = IO<T>::ld(X + idx * p.E + e); dtv = IO<T>::ld(DT + idx * p.E + e);
-            dlv = IO<T>::ld(DL + idx * p.E + e); dyv = IO<T>::ld(DY + idx * p.E + e);
-          }
-          if (!act) { dtv = 0.f; dlv = 0.f; dyv = gact ? 1.f : 0.f; xv = 0.f; }
-          const float* a_mine = a_base;
-          asm volatile("" : "+v"(a_mine));
-          const float* pbt = act ? bcb + (k * kHB + r) * SG::kBStride : (gact ? bob + (k * CW + ch_loc) * kN : zrec);
-          const float* pbl = act ? pbt + kN : pbt;
-          const float* pcc = act ? pbt + 2 * kN : pbt;
-          const float qT = cT * dtv * xv, qL = cL * dlv * xv;   // zero on lanes that are not grid cells
-          const float qC = act ? dyv : 0.f;
-          float sT = 0.f, sL = 0.f, zT = 0.f, zL = 0.f;
-#ifndef M2D_X_NOSLOTBAR
-          __syncthreads();   // the flush of the previous step has finished reading the slots
-#endif
-          float* sw = reinterpret_cast<float*>(slots + wave * SLOT + lane);
-          // States are visited in groups of 4 so that the channel sums of a group can be folded as
-          // soon as the group is done; afterwards the lane of slot q holds the states 4q..4q+3
-          // (component mg of its float4 after group mg).
-#pragma unroll
-          for (int mg = 0; mg < 4; ++mg) {
-            const float4 at4 = reinterpret_cast<const float4*>(a_mine)[mg], al4 = reinterpret_cast<const float4*>(a_mine + kN)[mg];
-            const float4 b4 = reinterpret_cast<const float4*>(pbt)[mg], l4 = reinterpret_cast<const float4*>(pbl)[mg];
-            const float4 c4 = reinterpret_cast<const float4*>(pcc)[mg];
-            const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
-            const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w}, cq[4] = {c4.x, c4.y, c4.z, c4.w};
-            float vC[4], vBT[4], vBL[4];
-#pragma unroll
-            for (int qi = 0; qi < 4; ++qi) {
-              const int n = fold_state(mg, qi);
-              const float a2t = atq[qi], a2l = alq[qi];
-              const float aT = fexp2(__builtin_fmaf(dtv, a2t, offT));
-              const float aL = fexp2(__builtin_fmaf(dlv, a2l, offL));
-              const float mb = from_row_above(muT[n]);
-              const float lam = __builtin_fmaf(dyv, cq[qi], muL[n] + mb);
-              const float hT = from_row_below(hb[k][n]);
-              const float mT = aT * lam, mL = aL * lam;
-              muT[n] = mT;
-              muL[n] = mL;
-              const float ZT = mT * hT, ZL = mL * hb[k][n];
-              accAT[n] = __builtin_fmaf(ZT, dtv, accAT[n]);
-              accAL[n] = __builtin_fmaf(ZL, dlv, accAL[n]);
-              zT = __builtin_fmaf(ZT, a2t, zT);
-              zL = __builtin_fmaf(ZL, a2l, zL);
-              sT = __builtin_fmaf(lam, bq[qi], sT);
-              sL = __builtin_fmaf(lam, lq[qi], sL);
-              vBT[qi] = qT * lam;
-              vBL[qi] = qL * lam;
-              vC[qi] = qC * hb[k + 1][n];
+        for (int k = kCK - 1; k >= 0; --k) {
+          const int t = t0 + k;
+          if (half == 1 && k == 0) staging_landed();   // before the last stores of the block, see the forward kernel
+          // the states of the later steps are dead by now: their registers take the next snapshot
+          if (half == 1 && k == (kCK > 1 ? 1 : 0) && m > 0) load_ckpt(m - 1);
+          if (t < T_steps) {
+            const int j = t - r;
+            const bool inw = j >= 0 && j < p.W;
+            const bool act = ro.real && inw;
+            const bool gact = ro.gbot && inw;     // ghost of the row below: muT := staged row
+            float offT = act ? (j == 0 ? oT_j0 : oT_in) : ninf;
+            const float offL = (act && j != 0) ? oL_in : ninf;
+            const float cT = act ? (ro.first_row ? 0.f : (j == 0 ? 1.f : 0.5f)) : 0.f;
+            const float cL = act ? (ro.first_row ? 1.f : (j == 0 ? 0.f : 0.5f)) : 0.f;
+            if (gact) offT = 0.f;                 // open T gate with delta 0: muT = lambda = staged value
+            float xv, dtv, dlv, dyv;
+            if constexpr (STAGE_X) {
+              const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
+              xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW); dyv = IO<T>::ld(xr + 3 * CW);
+            } else {
+              const int64_t idx = cell0 + cell_in_image(p, irow, inw ? j : 0);
+              xv = IO<T>::ld(X + idx * p.E + e); dtv = IO<T>::ld(DT + idx * p.E + e);
+              dlv = IO<T>::ld(DL + idx * p.E + e); dyv = IO<T>::ld(DY + idx * p.E + e);
             }
-            sw[mg] = fold16(fold32(vC[0], vC[1]), fold32(vC[2], vC[3]));
-            sw[64 * 4 + mg] = fold16(fold32(vBT[0], vBT[1]), fold32(vBT[2], vBT[3]));
-            sw[128 * 4 + mg] = fold16(fold32(vBL[0], vBL[1]), fold32(vBL[2], vBL[3]));
-            __builtin_amdgcn_sched_barrier(0);
-          }
-          if (to_bot && act) {   // first row of the band: the band above's lower ghost will replay its muT
-            float* bb = p.bot + (((int64_t)b * p.W + j) * p.E + e) * kN;
+            if (!act) { dtv = 0.f; dlv = 0.f; dyv = gact ? 1.f : 0.f; xv = 0.f; }
+            const float* a_mine = a_base;
+            asm volatile("" : "+v"(a_mine));
+            const float* pbt = act ? bcb + (k * kHB + r) * SG::kBStride : (gact ? bob + (k * CW + ch_loc) * kN : zrec);
+            const float* pbl = act ? pbt + kN : pbt;
+            const float* pcc = act ? pbt + 2 * kN : pbt;
+            const float qT = cT * dtv * xv, qL = cL * dlv * xv;   // zero on lanes that are not grid cells
+            const float qC = act ? dyv : 0.f;
+            float sT = 0.f, sL = 0.f, zT = 0.f, zL = 0.f;
+            if (half == 1) { sT = part4[k][0]; sL = part4[k][1]; zT = part4[k][2]; zL = part4[k][3]; }
+            __syncthreads();   // the flush of the previous exchange has finished reading the slots
+            float* sw = reinterpret_cast<float*>(slots + wave * SLOT + lane);
+            // A group of 4 states is folded over the 4 channel slots of the wave as soon as it is
+            // done; afterwards the lane of slot q holds the channel sums of the states 4q..4q+3
+            // (component mg of its float4 after group mg).
 #pragma unroll
-            for (int q = 0; q < 4; ++q)
-              reinterpret_cast<float4*>(bb)[q] = make_float4(muT[sinv<PERM>(4 * q)], muT[sinv<PERM>(4 * q + 1)],
-                                                             muT[sinv<PERM>(4 * q + 2)], muT[sinv<PERM>(4 * q + 3)]);
-          }
-          if (act) {
-            const int64_t idx = cell0 + cell_in_image(p, irow, j);
-            accD = __builtin_fmaf(dyv, xv, accD);
-            IO<T>::st(DDT + idx * p.E + e, __builtin_fmaf(cT * xv, sT, kLn2 * zT));
-            IO<T>::st(DDL + idx * p.E + e, __builtin_fmaf(cL * xv, sL, kLn2 * zL));
-            IO<T>::st(DX + idx * p.E + e, __builtin_fmaf(cT * dtv, sT, __builtin_fmaf(cL * dlv, sL, dyv * dsk)));
-          }
-          // ---- across the waves of the workgroup: the per-wave slots are added in wave order
-#ifndef M2D_X_NOSLOTBAR
-          __syncthreads();
-#endif
-          if (threadIdx.x < SLOT) {
-            const int it = threadIdx.x;
-            const int fl = it & 63, v = it >> 6;
-            const int fr = fl & (kHB - 1), fs = fl >> kHBShift;
-            const int fj = t - fr;
-            if (fr >= 1 && fr <= g.rows && fj >= 0 && fj < p.W) {
-              float4 s = slots[it];
+            for (int mgl = 0; mgl < 2; ++mgl) {
+              const int mg = 2 * half + mgl;
+              const float4 at4 = reinterpret_cast<const float4*>(a_mine)[mg], al4 = reinterpret_cast<const float4*>(a_mine + kN)[mg];
+              const float4 b4 = reinterpret_cast<const float4*>(pbt)[mg], l4 = reinterpret_cast<const float4*>(pbl)[mg];
+              const float4 c4 = reinterpret_cast<const float4*>(pcc)[mg];
+              const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
+              const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w}, cq[4] = {c4.x, c4.y, c4.z, c4.w};
+              float vC[4], vBT[4], vBL[4];
 #pragma unroll
-              for (int w = 1; w < kBwdWaves; ++w) {
-                const float4 o = slots[w * SLOT + it];
-                s.x += o.x; s.y += o.y; s.z += o.z; s.w += o.w;
+              for (int qi = 0; qi < 4; ++qi) {
+                const int n = fold_state(mg, qi), s8 = 4 * mgl + qi;
+                const float a2t = atq[qi], a2l = alq[qi];
+                const float aT = fexp2(__builtin_fmaf(dtv, a2t, offT));
+                const float aL = fexp2(__builtin_fmaf(dlv, a2l, offL));
+                const float mb = from_row_above(muT[n]);
+                const float lam = __builtin_fmaf(dyv, cq[qi], muL[n] + mb);
+                const float hT = from_row_below(hb[k][s8]);
+                const float mT = aT * lam, mL = aL * lam;
+                muT[n] = mT;
+                muL[n] = mL;
+                const float ZT = mT * hT, ZL = mL * hb[k][s8];
+                accAT[n] = __builtin_fmaf(ZT, dtv, accAT[n]);
+                accAL[n] = __builtin_fmaf(ZL, dlv, accAL[n]);
+                zT = __builtin_fmaf(ZT, a2t, zT);
+                zL = __builtin_fmaf(ZL, a2l, zL);
+                sT = __builtin_fmaf(lam, bq[qi], sT);
+                sL = __builtin_fmaf(lam, lq[qi], sL);
+                vBT[qi] = qT * lam;
+                vBL[qi] = qL * lam;
+                vC[qi] = qC * hb[k + 1][s8];
               }
-              const int64_t cell = cell0 + cell_in_image(p, g.i0 + fr - 1, fj);
-              *reinterpret_cast<float4*>(p.part + (((int64_t)eg * 3 + v) * P + cell) * kN + fs * 4) = s;
+              sw[mg] = fold16(fold32(vC[0], vC[1]), fold32(vC[2], vC[3]));
+              sw[64 * 4 + mg] = fold16(fold32(vBT[0], vBT[1]), fold32(vBT[2], vBT[3]));
+              sw[128 * 4 + mg] = fold16(fold32(vBL[0], vBL[1]), fold32(vBL[2], vBL[3]));
+            }
+            if (to_bot && act) {   // first row of the band: the band above's lower ghost will replay its muT
+              float* bb = p.bot + (((int64_t)b * p.W + j) * p.E + e) * kN;
+#pragma unroll
+              for (int q = 2 * half; q < 2 * half + 2; ++q)   // the two state groups of this half, as of this step
+                reinterpret_cast<float4*>(bb)[q] = make_float4(muT[sinv<PERM>(4 * q)], muT[sinv<PERM>(4 * q + 1)],
+                                                               muT[sinv<PERM>(4 * q + 2)], muT[sinv<PERM>(4 * q + 3)]);
+            }
+            if (half == 0) {
+              part4[k][0] = sT; part4[k][1] = sL; part4[k][2] = zT; part4[k][3] = zL;
+            } else {
+              if (act) {
+                const int64_t idx = cell0 + cell_in_image(p, irow, j);
+                accD = __builtin_fmaf(dyv, xv, accD);
+                IO<T>::st(DDT + idx * p.E + e, __builtin_fmaf(cT * xv, sT, kLn2 * zT));
+                IO<T>::st(DDL + idx * p.E + e, __builtin_fmaf(cL * xv, sL, kLn2 * zL));
+                IO<T>::st(DX + idx * p.E + e, __builtin_fmaf(cT * dtv, sT, __builtin_fmaf(cL * dlv, sL, dyv * dsk)));
+              }
+            }
+            // ---- across the waves of the workgroup: the per-wave slots (this half's two state
+            // groups) are added in wave order
+            __syncthreads();
+            if (threadIdx.x < SLOT) {
+              const int it = threadIdx.x;
+              const int fl = it & 63, v = it >> 6;
+              const int fr = fl & (kHB - 1), fs = fl >> kHBShift;
+              const int fj = t - fr;
+              if (fr >= 1 && fr <= g.rows && fj >= 0 && fj < p.W) {
+                const float2* sl2 = reinterpret_cast<const float2*>(slots) + half;
+                float2 s = sl2[2 * it];
+#pragma unroll
+                for (int w = 1; w < kBwdWaves; ++w) {
+                  const float2 o = sl2[2 * (w * SLOT + it)];
+                  s.x += o.x; s.y += o.y;
+                }
+                const int64_t cell = cell0 + cell_in_image(p, g.i0 + fr - 1, fj);
+                *reinterpret_cast<float2*>(p.part + (((int64_t)eg * 3 + v) * P + cell) * kN + fs * 4 + 2 * half) = s;
+              }
             }
           }
         }
