@@ -87,6 +87,9 @@ def main():
     ap.add_argument("--workload", default="cfg1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-ckpt", action="store_true", help="rebuild checkpoints inside the backward")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run one plain 256 MiB device copy (a known-size kernel to scale rocprofv3's "
+                         "FETCH_SIZE / WRITE_SIZE readings by)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the scan shards over the batch with no "
@@ -113,10 +116,18 @@ def main():
     dy = r(B, H, W, E).to(dtype).to(dev)
 
     cabi.profile_enable(True)
+    if args.calib_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
+    frozen = [t.detach() for t in leaves]   # inference: nothing requires grad, no checkpoints are kept
 
     def fwd_only():
         with torch.no_grad():
-            return wavefront.wf_cuda_fn_pr.apply(*leaves)
+            return wavefront.wf_cuda_fn_pr.apply(*frozen)
 
     def fwd_bwd():
         y = wavefront.wf_cuda_fn_pr.apply(*leaves)

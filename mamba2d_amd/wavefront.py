@@ -82,7 +82,8 @@ class wf_cuda_fn_pr(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, deltaT, deltaL, AT, AL, BT, BL, C, D):
         args = [_c(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D)]
-        keep = SAVE_CHECKPOINTS and torch.is_grad_enabled() and any(ctx.needs_input_grad)
+        # (grad mode is always off inside forward(); needs_input_grad is what tells training from inference)
+        keep = SAVE_CHECKPOINTS and any(ctx.needs_input_grad)
         y, ck = scan_fwd_op(*args, keep, False)
         ctx.save_for_backward(*args, ck)
         return y

@@ -30,6 +30,8 @@ def test_fn_pr_forward_backward(wf, cscan, dtype, tol, save):
     wf.SAVE_CHECKPOINTS = save
     try:
         y = wf.wf_cuda_fn_pr.apply(*leaves)
+        # the forward keeps its checkpoints exactly when asked to (a 1-byte tensor stands for none)
+        assert (y.grad_fn.saved_tensors[-1].numel() > 1) == save
         grads = torch.autograd.grad(y, leaves, inp["dy"].cuda())
     finally:
         wf.SAVE_CHECKPOINTS = old
