@@ -38,6 +38,10 @@ WORKLOADS = {
 }
 N = 16
 HBM_PEAK_GBS = 8000.0
+# HBM bytes per launch of the backward scan kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
+# (profiles/scan_cfg1_kernel_trace_and_traffic.txt: 503082 KiB x 2.0 + 422921 KiB x 1.0); counters
+# cannot be read from inside this script, so the figure is carried here per workload.
+MEASURED_TRAFFIC = {"cfg1": 1.4634e9}
 
 
 def algorithmic_bytes(B, E, H, W, s):
@@ -197,7 +201,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": None,
+            "traffic": MEASURED_TRAFFIC.get(args.workload),
             "kernel_ms": round(bwd_kernel, 4),
             "algorithmic_bytes": bb,
             "fwd_kernel_ms": round(fwd_kernel_ms, 4),
