@@ -52,6 +52,15 @@ constexpr int kZeroFloats = 64;     // page of zeros at the head of the set-up a
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
+#ifdef M2D_X_TIMING
+__device__ long long g_dbg[4096 * 8];
+#define TICK(var) const long long var = clock64()
+#define TACC(slot, a, b) dbg_acc[slot] += (b) - (a)
+#else
+#define TICK(var)
+#define TACC(slot, a, b)
+#endif
+
 struct bf16_t { uint16_t v; };
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t lo16) { return __uint_as_float(lo16 << 16); }
@@ -331,6 +340,7 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   constexpr int CS = 64 >> kHBShift;
   constexpr int CW = kFwdWaves * CS * EC;
   constexpr bool PERM = true;
+  constexpr bool AHEAD = EC == 1;   // operands of step t+1 are fetched from LDS during step t
   using SG = Stage<T, 3, CW, false>;
   extern __shared__ float4 smem[];
   float* zrec = reinterpret_cast<float*>(smem);            // 64 zero floats
@@ -356,6 +366,10 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   }
 
   settle_loads();
+#ifdef M2D_X_TIMING
+  long long dbg_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  const long long dbg_t0 = clock64();
+#endif
   const T* X = static_cast<const T*>(p.x);
   const T* DT = static_cast<const T*>(p.dT);
   const T* DL = static_cast<const T*>(p.dL);
@@ -363,39 +377,166 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   T* Y = static_cast<T*>(p.y);
   const float ninf = -__builtin_huge_valf();
 
-  for (int band = 0; band < p.nbands; ++band) {
+  // Everything about a band that the inner loops need (wave-uniform geometry, per-lane roles).
+  struct BandCtx {
     BandGeom g;
-    g.band = band; g.i0 = band * kRB;
-    g.rows = p.H - g.i0 < kRB ? p.H - g.i0 : kRB;
-    g.has_above = band > 0; g.has_below = band + 1 < p.nbands;
-    const int T_steps = g.has_below ? p.W + kHB - 1 : p.W + g.rows;   // same step count as the backward
-    const int nb = (T_steps + kCK - 1) / kCK;
     LaneRole ro;
-    ro.real = ch_ok && r >= 1 && r <= g.rows;
-    ro.gtop = ch_ok && r == 0 && g.has_above;
-    ro.gbot = false;
-    ro.first_row = g.i0 + r - 1 == 0;
-    const bool to_top = ro.real && g.has_below && r == kRB;
-    const float oT_in = ro.first_row ? ninf : -1.f, oT_j0 = ro.first_row ? ninf : 0.f, oL_in = ro.first_row ? 0.f : -1.f;
-    const int64_t cell0 = (int64_t)b * p.H * p.W;
-    const int irow = g.i0 + (ro.real ? r - 1 : 0);
+    int T_steps, nb, irow;
+    bool to_top;
+    float oT_in, oT_j0, oL_in;
+  };
+  auto band_ctx = [&](int band) {
+    BandCtx c;
+    c.g.band = band; c.g.i0 = band * kRB;
+    c.g.rows = p.H - c.g.i0 < kRB ? p.H - c.g.i0 : kRB;
+    c.g.has_above = band > 0; c.g.has_below = band + 1 < p.nbands;
+    c.T_steps = c.g.has_below ? p.W + kHB - 1 : p.W + c.g.rows;   // same step count as the backward
+    c.nb = (c.T_steps + kCK - 1) / kCK;
+    c.ro.real = ch_ok && r >= 1 && r <= c.g.rows;
+    c.ro.gtop = ch_ok && r == 0 && c.g.has_above;
+    c.ro.gbot = false;
+    c.ro.first_row = c.g.i0 + r - 1 == 0;
+    c.to_top = c.ro.real && c.g.has_below && r == kRB;
+    c.oT_in = c.ro.first_row ? ninf : -1.f; c.oT_j0 = c.ro.first_row ? ninf : 0.f; c.oL_in = c.ro.first_row ? 0.f : -1.f;
+    c.irow = c.g.i0 + (c.ro.real ? r - 1 : 0);
+    return c;
+  };
+  const int64_t cell0 = (int64_t)b * p.H * p.W;
 
-    stage_block<T, 3, CW, false, STAGE_X, kFwdWaves>(p, lds, b, g, 0, e_wg0, wave, lane, X, DT, DL, DY);
-    staging_fence();
-    int cur = 0;
-    float h[EC][kN];
+  // Operands of one step, read from the staging buffer one step ahead of their use so that the
+  // LDS latency hides behind the arithmetic of the step before.
+  struct Ops {
+    float xv[EC], dtv[EC], dlv[EC];
+    float4 bt[EC][4], bl[4], cc[4];
+  };
+  auto fetch = [&](const BandCtx& cx, const char* bufc, int k, int t, Ops& o) {
+    const float* bcb = reinterpret_cast<const float*>(bufc);
+    const T* xdb = reinterpret_cast<const T*>(bufc + SG::kXOff);
+    const float* tpb = reinterpret_cast<const float*>(bufc + SG::kTOff);
+    const int j = t - r;
+    const bool inw = j >= 0 && j < p.W;
+    const bool act = cx.ro.real && inw;
+    const bool gact = cx.ro.gtop && inw;
+    if constexpr (STAGE_X) {
+      const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
+      IO<T>::template ldv<EC>(xr, o.xv);
+      IO<T>::template ldv<EC>(xr + CW, o.dtv);
+      IO<T>::template ldv<EC>(xr + 2 * CW, o.dlv);
+    } else {
+      const int64_t idx = cell0 + cell_in_image(p, cx.irow, inw ? j : 0);
+      IO<T>::template ldv<EC>(X + idx * p.E + e0, o.xv);
+      IO<T>::template ldv<EC>(DT + idx * p.E + e0, o.dtv);
+      IO<T>::template ldv<EC>(DL + idx * p.E + e0, o.dlv);
+    }
+    // operand records: a grid row reads B_T, B_L, C of its cell; the ghost reads the row above
+    // as its B_T (and harmless finite stand-ins for the other two)
+    const float* rec = bcb + (k * kHB + r) * SG::kBStride;
+#pragma unroll
+    for (int c = 0; c < EC; ++c) {
+      const float* pbt = act ? rec : (gact ? tpb + (k * CW + ch_loc + c) * kN : zrec);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) o.bt[c][q] = reinterpret_cast<const float4*>(pbt)[q];
+    }
+    const float* pbl = act ? rec + kN : zrec;
+    const float* pcc = act ? rec + 2 * kN : zrec;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      o.bl[q] = reinterpret_cast<const float4*>(pbl)[q];
+      o.cc[q] = WRITE_Y ? reinterpret_cast<const float4*>(pcc)[q] : make_float4(0, 0, 0, 0);
+    }
+  };
+
+  float h[EC][kN];
+  auto step = [&](const BandCtx& cx, int t, Ops& o) {
+    const int j = t - r;
+    const bool inw = j >= 0 && j < p.W;
+    const bool act = cx.ro.real && inw;
+    const bool gact = cx.ro.gtop && inw;
+    const float offT = act ? (j == 0 ? cx.oT_j0 : cx.oT_in) : ninf;
+    const float offL = (act && j != 0) ? cx.oL_in : ninf;
+    const float cT = act ? (cx.ro.first_row ? 0.f : (j == 0 ? 1.f : 0.5f)) : 0.f;
+    const float cL = act ? (cx.ro.first_row ? 1.f : (j == 0 ? 0.f : 0.5f)) : 0.f;
+    if (!act) {   // records of cells outside the grid are not staged
+#pragma unroll
+      for (int c = 0; c < EC; ++c) { o.xv[c] = 0.f; o.dtv[c] = 0.f; o.dlv[c] = 0.f; }
+    }
+    float yv[EC];
+#pragma unroll
+    for (int c = 0; c < EC; ++c) {
+      const float sT = gact ? 1.f : cT * o.dtv[c] * o.xv[c];
+      const float sL = cL * o.dlv[c] * o.xv[c];
+      float acc = 0.f;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const float4 b4 = o.bt[c][q], l4 = o.bl[q], c4 = o.cc[q];
+        const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w}, cq[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const int n = sinv<PERM>(4 * q + w);
+          const float aT = fexp2(__builtin_fmaf(o.dtv[c], a2t[c][n], offT));
+          const float aL = fexp2(__builtin_fmaf(o.dlv[c], a2l[c][n], offL));
+          const float hT = from_row_below(h[c][n]);
+          float u = sL * lq[w];
+          u = __builtin_fmaf(sT, bq[w], u);
+          u = __builtin_fmaf(aT, hT, u);
+          const float hn = __builtin_fmaf(aL, h[c][n], u);
+          h[c][n] = hn;
+          if (WRITE_Y) acc = __builtin_fmaf(hn, cq[w], acc);
+        }
+      }
+      yv[c] = __builtin_fmaf(o.xv[c], dsk[c], acc);
+      if (cx.to_top && act) {   // last row of the band: the next band's ghost will replay it
+        float* tw = p.top + ((((int64_t)cx.g.band * p.B + b) * p.W + j) * p.E + e0 + c) * kN;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          reinterpret_cast<float4*>(tw)[q] = make_float4(h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)],
+                                                         h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
+      }
+    }
+    if (WRITE_Y && act) {
+      const int64_t idx = cell0 + cell_in_image(p, cx.irow, j);
+      IO<T>::template stv<EC>(Y + idx * p.E + e0, yv);
+    }
+  };
+
+  // The bands of the image are swept one after the other without draining the pipeline: while
+  // the last block of a band runs, the first block of the next band is staged.  The rows of
+  // the band above that this needs (columns 0..kCK-1) were stored at steps 14..14+kCK-1 of the
+  // band and completed (vmcnt 0) before a block-end barrier, long before; they are read back
+  // past the L1.  Grids narrower than 8 columns, where that does not hold, restart per band.
+  const bool streamed = p.W >= 8;
+  BandCtx cx = band_ctx(0);
+  Ops ahead;
+  int cur = 0;
+  for (int band = 0; band < p.nbands; ++band) {
+    const bool more = band + 1 < p.nbands;
+    const BandCtx nx = band_ctx(more ? band + 1 : band);
+    if (band == 0 || !streamed) {
+      TICK(tb0);
+      stage_block<T, 3, CW, false, STAGE_X, kFwdWaves>(p, lds + cur * SG::kBytes, b, cx.g, 0, e_wg0, wave, lane, X, DT, DL, DY);
+      staging_fence();
+      TICK(tb1); TACC(0, tb0, tb1);
+      if constexpr (AHEAD) fetch(cx, lds + cur * SG::kBytes, 0, 0, ahead);
+    }
 #pragma unroll
     for (int c = 0; c < EC; ++c)
 #pragma unroll
       for (int n = 0; n < kN; ++n) h[c][n] = 0.f;
+    const int nb = cx.nb, T_steps = cx.T_steps;
 
     for (int m = 0; m < nb; ++m) {
       const int t0 = m * kCK;
-      if (m + 1 < nb)
-        stage_block<T, 3, CW, false, STAGE_X, kFwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, g, t0 + kCK, e_wg0, wave, lane, X, DT, DL, DY);
+      const bool last = m + 1 == nb;
+      const bool into_next = last && more && streamed;
+      TICK(ts0);
+      if (!last)
+        stage_block<T, 3, CW, false, STAGE_X, kFwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, cx.g, t0 + kCK, e_wg0, wave, lane, X, DT, DL, DY);
+      else if (into_next)
+        stage_block<T, 3, CW, false, STAGE_X, kFwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, nx.g, 0, e_wg0, wave, lane, X, DT, DL, DY);
+      TICK(ts1); TACC(1, ts0, ts1);
       // snapshot of the state before the block (after step t0-1); lanes that have not started or
       // are past the last column hold nothing the backward needs
-      if (CKPT && m > 0 && (ro.real || ro.gtop) && t0 - 1 - r >= 0 && t0 - 1 - r < p.W) {
+      if (CKPT && m > 0 && (cx.ro.real || cx.ro.gtop) && t0 - 1 - r >= 0 && t0 - 1 - r < p.W) {
         float* ck = p.ckpt + (((((int64_t)b * p.nbands + band) * p.nblk + m) * p.E + e0) * kN) * kHB + r;
 #pragma unroll
         for (int c = 0; c < EC; ++c)
@@ -403,97 +544,60 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
           for (int n = 0; n < kN; ++n) ck[(c * kN + n) * kHB] = h[c][n];
       }
       const char* bufc = lds + cur * SG::kBytes;
-      const float* bcb = reinterpret_cast<const float*>(bufc);
-      const T* xdb = reinterpret_cast<const T*>(bufc + SG::kXOff);
-      const float* tpb = reinterpret_cast<const float*>(bufc + SG::kTOff);
+      const char* bufn = lds + (cur ^ 1) * SG::kBytes;
 #pragma unroll
       for (int k = 0; k < kCK; ++k) {
         const int t = t0 + k;
-        // The operands of the next block must have landed before the barrier that ends this block.
-        // Waiting here, before the stores of the last step are issued, keeps the latency of those
-        // stores off the critical path (the counter covers loads and stores alike).
-        if (k == kCK - 1) staging_landed();
-        if (t < T_steps) {
-          const int j = t - r;
-          const bool inw = j >= 0 && j < p.W;
-          const bool act = ro.real && inw;
-          const bool gact = ro.gtop && inw;
-          float offT = act ? (j == 0 ? oT_j0 : oT_in) : ninf;
-          float offL = (act && j != 0) ? oL_in : ninf;
-          const float cT = act ? (ro.first_row ? 0.f : (j == 0 ? 1.f : 0.5f)) : 0.f;
-          const float cL = act ? (ro.first_row ? 1.f : (j == 0 ? 0.f : 0.5f)) : 0.f;
-          float xv[EC], dtv[EC], dlv[EC];
-          if constexpr (STAGE_X) {
-            const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
-            IO<T>::template ldv<EC>(xr, xv);
-            IO<T>::template ldv<EC>(xr + CW, dtv);
-            IO<T>::template ldv<EC>(xr + 2 * CW, dlv);
+        if constexpr (AHEAD) {
+          Ops now = ahead;
+          if (k + 1 < kCK) {
+            fetch(cx, bufc, k + 1, t + 1, ahead);
           } else {
-            const int64_t idx = cell0 + cell_in_image(p, irow, inw ? j : 0);
-            IO<T>::template ldv<EC>(X + idx * p.E + e0, xv);
-            IO<T>::template ldv<EC>(DT + idx * p.E + e0, dtv);
-            IO<T>::template ldv<EC>(DL + idx * p.E + e0, dlv);
+            // Last step of the block: its operands are in registers already, so the buffer can be
+            // handed over now.  The copies of the next block have landed in every wave after this
+            // barrier, and no wave reads the current buffer any more.
+            TICK(tw0);
+            staging_landed();
+            TICK(tw1); TACC(2, tw0, tw1);
+            __syncthreads();
+            TICK(tw2); TACC(3, tw1, tw2);
+            if (!last) fetch(cx, bufn, 0, t + 1, ahead);
+            else if (into_next) fetch(nx, bufn, 0, 0, ahead);
           }
-          if (!act) {
-#pragma unroll
-            for (int c = 0; c < EC; ++c) { xv[c] = 0.f; dtv[c] = 0.f; dlv[c] = 0.f; }
+          TICK(tc0);
+          if (t < T_steps) step(cx, t, now);
+          TICK(tc1); TACC(4, tc0, tc1);
+        } else {
+          // The operands of the next block must have landed before the barrier that ends this
+          // block.  Waiting here, before the stores of the last step are issued, keeps the latency
+          // of those stores off the critical path (the counter covers loads and stores alike).
+          if (k == kCK - 1) staging_landed();
+          if (t < T_steps) {
+            Ops now;
+            fetch(cx, bufc, k, t, now);
+            step(cx, t, now);
           }
-          float yv[EC];
-#pragma unroll
-          for (int c = 0; c < EC; ++c) {
-            // operand records: a grid row reads B_T, B_L, C of its cell; the ghost reads the row
-            // above as its B_T (and as harmless finite stand-ins for the other two)
-            const float* pbt = act ? bcb + (k * kHB + r) * SG::kBStride : (gact ? tpb + (k * CW + ch_loc + c) * kN : zrec);
-            const float* pbl = act ? pbt + kN : pbt;
-            const float* pcc = act ? pbt + 2 * kN : pbt;
-            const float sT = gact ? 1.f : cT * dtv[c] * xv[c];
-            const float sL = cL * dlv[c] * xv[c];
-            float acc = 0.f;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-              const float4 b4 = reinterpret_cast<const float4*>(pbt)[q], l4 = reinterpret_cast<const float4*>(pbl)[q];
-              const float4 c4 = WRITE_Y ? reinterpret_cast<const float4*>(pcc)[q] : make_float4(0, 0, 0, 0);
-              const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w}, cq[4] = {c4.x, c4.y, c4.z, c4.w};
-#pragma unroll
-              for (int w = 0; w < 4; ++w) {
-                const int n = sinv<PERM>(4 * q + w);
-                const float aT = fexp2(__builtin_fmaf(dtv[c], a2t[c][n], offT));
-                const float aL = fexp2(__builtin_fmaf(dlv[c], a2l[c][n], offL));
-                const float hT = from_row_below(h[c][n]);
-                float u = sL * lq[w];
-                u = __builtin_fmaf(sT, bq[w], u);
-                u = __builtin_fmaf(aT, hT, u);
-                const float hn = __builtin_fmaf(aL, h[c][n], u);
-                h[c][n] = hn;
-                if (WRITE_Y) acc = __builtin_fmaf(hn, cq[w], acc);
-              }
-            }
-            yv[c] = __builtin_fmaf(xv[c], dsk[c], acc);
-            if (to_top && act) {   // last row of the band: the next band's ghost will replay it
-              float* tw = p.top + ((((int64_t)band * p.B + b) * p.W + j) * p.E + e0 + c) * kN;
-#pragma unroll
-              for (int q = 0; q < 4; ++q)
-                reinterpret_cast<float4*>(tw)[q] = make_float4(h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)],
-                                                               h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
-            }
-          }
-#ifndef M2D_X_NOSTORE
-          if (WRITE_Y && act) {
-            const int64_t idx = cell0 + cell_in_image(p, irow, j);
-            IO<T>::template stv<EC>(Y + idx * p.E + e0, yv);
-          }
-#else
-          if (WRITE_Y && act && yv[0] == 123.456f) Y[0] = T{};
-#endif
         }
       }
-      if (m + 1 == nb && p.nbands > 1) __threadfence();   // the band's last row is read back by the next band
-#ifndef M2D_X_NOBLOCKBAR
-      __syncthreads();
-#endif
+      // restart per band: the band's last row is read back by the next band's first staging
+      if (last && more && !streamed) {
+        __threadfence();
+        __syncthreads();
+      } else if constexpr (!AHEAD) {
+        __syncthreads();
+      }
       cur ^= 1;
     }
+    cx = nx;
   }
+#ifdef M2D_X_TIMING
+  if (lane == 0 && blockIdx.x < 512) {
+    long long* d = g_dbg + (blockIdx.x * 8 + wave) * 8;
+    for (int i = 0; i < 5; ++i) d[i] = dbg_acc[i];
+    d[5] = clock64() - dbg_t0;
+    d[6] = wall_clock64();
+  }
+#endif
 }
 
 // ----------------------------------------------------------------------------------- backward
@@ -1086,6 +1190,13 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
 
 // ---------------------------------------------------------------------------------------- C ABI
 extern "C" {
+
+#ifdef M2D_X_TIMING
+int m2d_dbg_read(long long* host, size_t n) {
+  (void)hipDeviceSynchronize();
+  return hipMemcpyFromSymbol(host, HIP_SYMBOL(g_dbg), n * sizeof(long long)) == hipSuccess ? 0 : 1;
+}
+#endif
 
 int m2d_version(void) { return 200; }
 
