@@ -659,40 +659,59 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
 #pragma unroll
   for (int n = 0; n < kN; ++n) { accAT[n] = 0.f; accAL[n] = 0.f; }
 
-  for (int band = p.nbands - 1; band >= 0; --band) {
+  struct BandCtx {
     BandGeom g;
-    g.band = band; g.i0 = band * kRB;
-    g.rows = p.H - g.i0 < kRB ? p.H - g.i0 : kRB;
-    g.has_above = band > 0; g.has_below = band + 1 < p.nbands;
-    const int T_steps = g.has_below ? p.W + kHB - 1 : p.W + g.rows;   // the lower ghost trails by 15 steps
-    const int nb = (T_steps + kCK - 1) / kCK;
     LaneRole ro;
-    ro.real = ch_ok && r >= 1 && r <= g.rows;
-    ro.gtop = ch_ok && r == 0 && g.has_above;
-    ro.gbot = ch_ok && r == kHB - 1 && g.has_below;
-    ro.first_row = g.i0 + r - 1 == 0;
-    const bool to_bot = ro.real && g.has_above && r == 1;
-    const float oT_in = ro.first_row ? ninf : -1.f, oT_j0 = ro.first_row ? ninf : 0.f, oL_in = ro.first_row ? 0.f : -1.f;
-    const int64_t cell0 = (int64_t)b * p.H * p.W;
-    const int irow = g.i0 + (ro.real ? r - 1 : 0);
+    int T_steps, nb, irow;
+    bool to_bot;
+    float oT_in, oT_j0, oL_in;
+  };
+  auto band_ctx = [&](int band) {
+    BandCtx c;
+    c.g.band = band; c.g.i0 = band * kRB;
+    c.g.rows = p.H - c.g.i0 < kRB ? p.H - c.g.i0 : kRB;
+    c.g.has_above = band > 0; c.g.has_below = band + 1 < p.nbands;
+    c.T_steps = c.g.has_below ? p.W + kHB - 1 : p.W + c.g.rows;   // the lower ghost trails by 15 steps
+    c.nb = (c.T_steps + kCK - 1) / kCK;
+    c.ro.real = ch_ok && r >= 1 && r <= c.g.rows;
+    c.ro.gtop = ch_ok && r == 0 && c.g.has_above;
+    c.ro.gbot = ch_ok && r == kHB - 1 && c.g.has_below;
+    c.ro.first_row = c.g.i0 + r - 1 == 0;
+    c.to_bot = c.ro.real && c.g.has_above && r == 1;
+    c.oT_in = c.ro.first_row ? ninf : -1.f; c.oT_j0 = c.ro.first_row ? ninf : 0.f; c.oL_in = c.ro.first_row ? 0.f : -1.f;
+    c.irow = c.g.i0 + (c.ro.real ? r - 1 : 0);
+    return c;
+  };
+  const int64_t cell0 = (int64_t)b * p.H * p.W;
+  // state snapshot at the start of block mm of a band (zero for lanes that were not under way)
+  float cknext[kN];
+  auto load_ckpt = [&](const BandCtx& c, int mm) {
+    const int tt = mm * kCK;
+    if (mm == 0 || !((c.ro.real || c.ro.gtop) && tt - 1 - r >= 0 && tt - 1 - r < p.W)) {
+#pragma unroll
+      for (int n = 0; n < kN; ++n) cknext[n] = 0.f;
+    } else {
+      const float* ck = p.ckpt + (((((int64_t)b * p.nbands + c.g.band) * p.nblk + mm) * p.E + e) * kN) * kHB + r;
+#pragma unroll
+      for (int n = 0; n < kN; ++n) cknext[n] = ck[n * kHB];
+    }
+  };
 
-    // state snapshot at the start of block mm (zero for lanes that were not under way)
-    float cknext[kN];
-    auto load_ckpt = [&](int mm) {
-      const int tt = mm * kCK;
-      if (mm == 0 || !((ro.real || ro.gtop) && tt - 1 - r >= 0 && tt - 1 - r < p.W)) {
-#pragma unroll
-        for (int n = 0; n < kN; ++n) cknext[n] = 0.f;
-      } else {
-        const float* ck = p.ckpt + (((((int64_t)b * p.nbands + band) * p.nblk + mm) * p.E + e) * kN) * kHB + r;
-#pragma unroll
-        for (int n = 0; n < kN; ++n) cknext[n] = ck[n * kHB];
-      }
-    };
-    load_ckpt(nb - 1);
-    stage_block<T, 4, CW, true, STAGE_X, kBwdWaves>(p, lds, b, g, (nb - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
-    staging_fence();
-    int cur = 0;
+  // Bands are swept bottom-up without draining the pipeline: while block 0 of a band runs, the
+  // last block of the band above is staged (its lower-ghost row was stored at the start of this
+  // band's sweep) and its snapshot fetched.  Grids narrower than 8 columns restart per band.
+  const bool streamed = p.W >= 8;
+  BandCtx cx = band_ctx(p.nbands - 1);
+  int cur = 0;
+  for (int band = p.nbands - 1; band >= 0; --band) {
+    const bool more = band > 0;
+    const BandCtx nx = band_ctx(more ? band - 1 : band);
+    const int nb = cx.nb, T_steps = cx.T_steps;
+    if (band == p.nbands - 1 || !streamed) {
+      load_ckpt(cx, nb - 1);
+      stage_block<T, 4, CW, true, STAGE_X, kBwdWaves>(p, lds + cur * SG::kBytes, b, cx.g, (nb - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
+      staging_fence();
+    }
 #pragma unroll
     for (int n = 0; n < kN; ++n) { muT[n] = 0.f; muL[n] = 0.f; }
 
@@ -706,8 +725,11 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
       float ck0[kN];
 #pragma unroll
       for (int n = 0; n < kN; ++n) ck0[n] = cknext[n];
+      const bool into_next = m == 0 && more && streamed;
       if (m > 0)
-        stage_block<T, 4, CW, true, STAGE_X, kBwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, g, t0 - kCK, e_wg0, wave, lane, X, DT, DL, DY);
+        stage_block<T, 4, CW, true, STAGE_X, kBwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, cx.g, t0 - kCK, e_wg0, wave, lane, X, DT, DL, DY);
+      else if (into_next)
+        stage_block<T, 4, CW, true, STAGE_X, kBwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, nx.g, (nx.nb - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
 
       // The 16 states are swept in two halves of 8 (state groups 0,1 then 2,3), each half
       // recomputing and then back-propagating the whole block: only 5 x 8 recomputed states are
@@ -727,18 +749,18 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
           if (t < T_steps) {
             const int j = t - r;
             const bool inw = j >= 0 && j < p.W;
-            const bool act = ro.real && inw;
-            const bool gact = ro.gtop && inw;
-            const float offT = act ? (j == 0 ? oT_j0 : oT_in) : ninf;
-            const float offL = (act && j != 0) ? oL_in : ninf;
-            const float cT = act ? (ro.first_row ? 0.f : (j == 0 ? 1.f : 0.5f)) : 0.f;
-            const float cL = act ? (ro.first_row ? 1.f : (j == 0 ? 0.f : 0.5f)) : 0.f;
+            const bool act = cx.ro.real && inw;
+            const bool gact = cx.ro.gtop && inw;
+            const float offT = act ? (j == 0 ? cx.oT_j0 : cx.oT_in) : ninf;
+            const float offL = (act && j != 0) ? cx.oL_in : ninf;
+            const float cT = act ? (cx.ro.first_row ? 0.f : (j == 0 ? 1.f : 0.5f)) : 0.f;
+            const float cL = act ? (cx.ro.first_row ? 1.f : (j == 0 ? 0.f : 0.5f)) : 0.f;
             float xv, dtv, dlv;
             if constexpr (STAGE_X) {
               const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
               xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW);
             } else {
-              const int64_t idx = cell0 + cell_in_image(p, irow, inw ? j : 0);
+              const int64_t idx = cell0 + cell_in_image(p, cx.irow, inw ? j : 0);
               xv = IO<T>::ld(X + idx * p.E + e); dtv = IO<T>::ld(DT + idx * p.E + e); dlv = IO<T>::ld(DL + idx * p.E + e);
             }
             if (!act) { xv = 0.f; dtv = 0.f; dlv = 0.f; }
@@ -775,23 +797,26 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
           const int t = t0 + k;
           if (half == 1 && k == 0) staging_landed();   // before the last stores of the block, see the forward kernel
           // the states of the later steps are dead by now: their registers take the next snapshot
-          if (half == 1 && k == (kCK > 1 ? 1 : 0) && m > 0) load_ckpt(m - 1);
+          if (half == 1 && k == (kCK > 1 ? 1 : 0)) {
+            if (m > 0) load_ckpt(cx, m - 1);
+            else if (into_next) load_ckpt(nx, nx.nb - 1);
+          }
           if (t < T_steps) {
             const int j = t - r;
             const bool inw = j >= 0 && j < p.W;
-            const bool act = ro.real && inw;
-            const bool gact = ro.gbot && inw;     // ghost of the row below: muT := staged row
-            float offT = act ? (j == 0 ? oT_j0 : oT_in) : ninf;
-            const float offL = (act && j != 0) ? oL_in : ninf;
-            const float cT = act ? (ro.first_row ? 0.f : (j == 0 ? 1.f : 0.5f)) : 0.f;
-            const float cL = act ? (ro.first_row ? 1.f : (j == 0 ? 0.f : 0.5f)) : 0.f;
+            const bool act = cx.ro.real && inw;
+            const bool gact = cx.ro.gbot && inw;     // ghost of the row below: muT := staged row
+            float offT = act ? (j == 0 ? cx.oT_j0 : cx.oT_in) : ninf;
+            const float offL = (act && j != 0) ? cx.oL_in : ninf;
+            const float cT = act ? (cx.ro.first_row ? 0.f : (j == 0 ? 1.f : 0.5f)) : 0.f;
+            const float cL = act ? (cx.ro.first_row ? 1.f : (j == 0 ? 0.f : 0.5f)) : 0.f;
             if (gact) offT = 0.f;                 // open T gate with delta 0: muT = lambda = staged value
             float xv, dtv, dlv, dyv;
             if constexpr (STAGE_X) {
               const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
               xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW); dyv = IO<T>::ld(xr + 3 * CW);
             } else {
-              const int64_t idx = cell0 + cell_in_image(p, irow, inw ? j : 0);
+              const int64_t idx = cell0 + cell_in_image(p, cx.irow, inw ? j : 0);
               xv = IO<T>::ld(X + idx * p.E + e); dtv = IO<T>::ld(DT + idx * p.E + e);
               dlv = IO<T>::ld(DL + idx * p.E + e); dyv = IO<T>::ld(DY + idx * p.E + e);
             }
@@ -846,7 +871,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
               sw[64 * 4 + mg] = fold16(fold32(vBT[0], vBT[1]), fold32(vBT[2], vBT[3]));
               sw[128 * 4 + mg] = fold16(fold32(vBL[0], vBL[1]), fold32(vBL[2], vBL[3]));
             }
-            if (to_bot && act) {   // first row of the band: the band above's lower ghost will replay its muT
+            if (cx.to_bot && act) {   // first row of the band: the band above's lower ghost will replay its muT
               float* bb = p.bot + (((int64_t)b * p.W + j) * p.E + e) * kN;
 #pragma unroll
               for (int q = 2 * half; q < 2 * half + 2; ++q)   // the two state groups of this half, as of this step
@@ -857,7 +882,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
               part4[k][0] = sT; part4[k][1] = sL; part4[k][2] = zT; part4[k][3] = zL;
             } else {
               if (act) {
-                const int64_t idx = cell0 + cell_in_image(p, irow, j);
+                const int64_t idx = cell0 + cell_in_image(p, cx.irow, j);
                 accD = __builtin_fmaf(dyv, xv, accD);
                 IO<T>::st(DDT + idx * p.E + e, __builtin_fmaf(cT * xv, sT, kLn2 * zT));
                 IO<T>::st(DDL + idx * p.E + e, __builtin_fmaf(cL * xv, sL, kLn2 * zL));
@@ -872,7 +897,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
               const int fl = it & 63, v = it >> 6;
               const int fr = fl & (kHB - 1), fs = fl >> kHBShift;
               const int fj = t - fr;
-              if (fr >= 1 && fr <= g.rows && fj >= 0 && fj < p.W) {
+              if (fr >= 1 && fr <= cx.g.rows && fj >= 0 && fj < p.W) {
                 const float2* sl2 = reinterpret_cast<const float2*>(slots) + half;
                 float2 s = sl2[2 * it];
 #pragma unroll
@@ -880,19 +905,21 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
                   const float2 o = sl2[2 * (w * SLOT + it)];
                   s.x += o.x; s.y += o.y;
                 }
-                const int64_t cell = cell0 + cell_in_image(p, g.i0 + fr - 1, fj);
+                const int64_t cell = cell0 + cell_in_image(p, cx.g.i0 + fr - 1, fj);
                 *reinterpret_cast<float2*>(p.part + (((int64_t)eg * 3 + v) * P + cell) * kN + fs * 4 + 2 * half) = s;
               }
             }
           }
         }
       }
-      if (m == 0 && p.nbands > 1) __threadfence();   // the band's first-row muT is read back by the band above
+      // restart per band: the band's first-row muT is read back by the first staging of the band above
+      if (m == 0 && more && !streamed) __threadfence();
 #ifndef M2D_X_NOBLOCKBAR
       __syncthreads();
 #endif
       cur ^= 1;
     }
+    cx = nx;
   }
 
   // ---- sums over positions: reduce over the rows of the band (lanes of one channel slot)
