@@ -239,53 +239,97 @@ struct BandGeom {   // wave-uniform description of the band being swept
   bool has_above, has_below;
 };
 
-template <typename T, int NT, int CW, bool WITH_BOT, bool STAGE_X, int NWAVES>
-__device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int b, const BandGeom& g, int t0, int e_wg0,
-                                            int wave, int lane, const T* x0, const T* x1, const T* x2, const T* x3) {
+// The chunk -> (step, row, part of record) decomposition of the BC and XD regions depends only on
+// the thread.  It is worked out once (divisions by the odd record sizes) and kept as one packed
+// word per wave-wide copy: bits 0-3 row, 4-8 part, 9-10 step, bit 31 set if the chunk carries data.
+template <typename T, int NT, int CW, bool WITH_BOT, int NWAVES, bool KEEP>
+struct StagePlan {
   using SG = Stage<T, NT, CW, WITH_BOT>;
-  // The chunk -> (step, row, part) decomposition depends only on the lane; hiding the lane from
-  // the optimiser here keeps it from precomputing all of it once and holding (and spilling)
-  // dozens of registers for the whole kernel.
-  asm volatile("" : "+v"(lane));
+  static constexpr int kPer = NWAVES * 64;
+  static constexpr int kItB = (SG::kBChunks + kPer - 1) / kPer;
+  static constexpr int kItX = (SG::kXChunks + kPer - 1) / kPer;
+  uint32_t bc[KEEP ? kItB : 1], xd[KEEP ? kItX : 1];
+  static __device__ __forceinline__ uint32_t word(int c, int nchunks, int reclen, int nparts) {
+    const int rec = c / reclen, part = c - rec * reclen;
+    const int k = rec >> kHBShift, r = rec & (kHB - 1);
+    return (c < nchunks && part < nparts && r >= 1 && r <= kRB) ? (0x80000000u | (k << 9) | (part << 4) | r) : 0u;
+  }
+  __device__ __forceinline__ void init(int wave, int lane) {
+    if constexpr (KEEP) {
+#pragma unroll
+      for (int i = 0; i < kItB; ++i) bc[i] = word(i * kPer + wave * 64 + lane, SG::kBChunks, SG::kBRec, 12);
+#pragma unroll
+      for (int i = 0; i < kItX; ++i) xd[i] = word(i * kPer + wave * 64 + lane, SG::kXChunks, SG::kXRec, NT * SG::kCpt);
+    }
+  }
+  // Kernels short of registers work the word out again at every use instead of keeping it.
+  __device__ __forceinline__ uint32_t get_bc(int i, int wave, int lane) const {
+    uint32_t w;
+    if constexpr (KEEP) { w = bc[i]; } else { asm volatile("" : "+v"(lane)); w = word(i * kPer + wave * 64 + lane, SG::kBChunks, SG::kBRec, 12); }
+    asm volatile("" : "+v"(w));   // unpack per use: the fields must not be hoisted into live registers
+    return w;
+  }
+  __device__ __forceinline__ uint32_t get_xd(int i, int wave, int lane) const {
+    uint32_t w;
+    if constexpr (KEEP) { w = xd[i]; } else { asm volatile("" : "+v"(lane)); w = word(i * kPer + wave * 64 + lane, SG::kXChunks, SG::kXRec, NT * SG::kCpt); }
+    asm volatile("" : "+v"(w));
+    return w;
+  }
+};
+
+template <typename T, int NT, int CW, bool WITH_BOT, bool STAGE_X, int NWAVES, bool KEEP>
+__device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan<T, NT, CW, WITH_BOT, NWAVES, KEEP>& plan, char* buf,
+                                            int b, const BandGeom& g, int t0, int e_wg0, int wave, int lane,
+                                            const T* x0, const T* x1, const T* x2, const T* x3) {
+  using SG = Stage<T, NT, CW, WITH_BOT>;
+  using PL = StagePlan<T, NT, CW, WITH_BOT, NWAVES, KEEP>;
+  static_assert((SG::kCpt & (SG::kCpt - 1)) == 0, "chunks per tensor row must be a power of two");
 #ifdef M2D_X_NOSTAGE
   return;
 #endif
   const int64_t img = (int64_t)b * p.H * p.W;
-  for (int c0 = wave * 64; c0 < SG::kBChunks; c0 += NWAVES * 64) {
-    const int c = c0 + lane;
-    const int rec = c / SG::kBRec, part = c - rec * SG::kBRec;
-    const int k = rec >> kHBShift, r = rec & (kHB - 1);
-    if (c < SG::kBChunks && part < 12 && r >= 1 && r <= g.rows) {
+  const int hw1 = p.H * p.W - 1;
+#pragma unroll
+  for (int i = 0; i < PL::kItB; ++i) {
+    const uint32_t w = plan.get_bc(i, wave, lane);
+    const int r = w & 15, part = (w >> 4) & 31, k = (w >> 9) & 3;
+    if ((int)w < 0 && r <= g.rows) {
       const int j = t0 + k - r;
       const float* src = p.zeros;
-      if (j >= 0 && j < p.W)   // the packed record holds B_T, B_L, C back to back: chunk `part` of 12
-        src = p.bt + (img + cell_in_image(p, g.i0 + r - 1, j)) * p.bc_stride + part * 4;
-      lds_fill16<false>(src, buf + c0 * 16);
+      if ((unsigned)j < (unsigned)p.W) {   // the packed record holds B_T, B_L, C back to back: chunk `part` of 12
+        int cell = (g.i0 + r - 1) * p.W + j;
+        cell = p.flip ? hw1 - cell : cell;
+        src = p.bt + (img + cell) * p.bc_stride + part * 4;
+      }
+      lds_fill16<false>(src, buf + (i * PL::kPer + wave * 64) * 16);
     }
   }
   if constexpr (STAGE_X) {
-    for (int c0 = wave * 64; c0 < SG::kXChunks; c0 += NWAVES * 64) {
-      const int c = c0 + lane;
-      const int rec = c / SG::kXRec, part = c - rec * SG::kXRec;
-      const int k = rec >> kHBShift, r = rec & (kHB - 1);
-      if (c < SG::kXChunks && part < NT * SG::kCpt && r >= 1 && r <= g.rows) {
+#pragma unroll
+    for (int i = 0; i < PL::kItX; ++i) {
+      const uint32_t w = plan.get_xd(i, wave, lane);
+      const int r = w & 15, part = (w >> 4) & 31, k = (w >> 9) & 3;
+      if ((int)w < 0 && r <= g.rows) {
         const int j = t0 + k - r;
-        const int tau = part / SG::kCpt, ch = e_wg0 + (part - tau * SG::kCpt) * SG::kElem;
+        const int tau = part / SG::kCpt, ch = e_wg0 + (part & (SG::kCpt - 1)) * SG::kElem;
         const void* src = p.zeros;
-        if (j >= 0 && j < p.W && ch < p.E) {
+        if ((unsigned)j < (unsigned)p.W && ch < p.E) {
+          int cell = (g.i0 + r - 1) * p.W + j;
+          cell = p.flip ? hw1 - cell : cell;
           // selected with compares: an indexed pointer table would live in (scratch) memory
           const T* base = tau == 0 ? x0 : (tau == 1 ? x1 : (tau == 2 ? x2 : x3));
-          src = base + (img + cell_in_image(p, g.i0 + r - 1, j)) * p.E + ch;
+          src = base + (img + cell) * p.E + ch;
         }
-        lds_fill16<false>(src, buf + SG::kXOff + c0 * 16);
+        lds_fill16<false>(src, buf + SG::kXOff + (i * PL::kPer + wave * 64) * 16);
       }
     }
   }
-  // boundary rows were written earlier in this launch (or by the forward launch): read them at
-  // device scope, past the L1
+  // boundary rows were written earlier in this launch (or by the forward launch): read them
+  // past the L1
+  static_assert((CW & (CW - 1)) == 0, "channels per workgroup must be a power of two");
   for (int c0 = wave * 64; c0 < SG::kTChunks; c0 += NWAVES * 64) {
     const int c = c0 + lane;
-    const int rec = c >> 2, k = rec / CW, ch = e_wg0 + rec - k * CW;
+    const int rec = c >> 2, k = rec / CW, ch = e_wg0 + (rec & (CW - 1));
     if (c < SG::kTChunks) {
       const int j = t0 + k;
       const float* src = p.zeros;
@@ -297,7 +341,7 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int 
   if constexpr (WITH_BOT) {
     for (int c0 = wave * 64; c0 < SG::kTChunks; c0 += NWAVES * 64) {
       const int c = c0 + lane;
-      const int rec = c >> 2, k = rec / CW, ch = e_wg0 + rec - k * CW;
+      const int rec = c >> 2, k = rec / CW, ch = e_wg0 + (rec & (CW - 1));
       if (c < SG::kTChunks) {
         const int j = t0 + k - (kHB - 1);
         const float* src = p.zeros;
@@ -356,6 +400,8 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   const bool ch_ok = e_raw < p.E;                  // idle lanes still take part in staging and barriers
   const int e0 = ch_ok ? e_raw : p.E - EC;
   if (threadIdx.x < 64) zrec[threadIdx.x] = 0.f;
+  StagePlan<T, 3, CW, false, kFwdWaves, true> plan;
+  plan.init(wave, lane);
 
   float a2t[EC][kN], a2l[EC][kN], dsk[EC];
 #pragma unroll
@@ -513,7 +559,7 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
     const BandCtx nx = band_ctx(more ? band + 1 : band);
     if (band == 0 || !streamed) {
       TICK(tb0);
-      stage_block<T, 3, CW, false, STAGE_X, kFwdWaves>(p, lds + cur * SG::kBytes, b, cx.g, 0, e_wg0, wave, lane, X, DT, DL, DY);
+      stage_block<T, 3, CW, false, STAGE_X, kFwdWaves, true>(p, plan, lds + cur * SG::kBytes, b, cx.g, 0, e_wg0, wave, lane, X, DT, DL, DY);
       staging_fence();
       TICK(tb1); TACC(0, tb0, tb1);
       if constexpr (AHEAD) fetch(cx, lds + cur * SG::kBytes, 0, 0, ahead);
@@ -530,9 +576,9 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
       const bool into_next = last && more && streamed;
       TICK(ts0);
       if (!last)
-        stage_block<T, 3, CW, false, STAGE_X, kFwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, cx.g, t0 + kCK, e_wg0, wave, lane, X, DT, DL, DY);
+        stage_block<T, 3, CW, false, STAGE_X, kFwdWaves, true>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, cx.g, t0 + kCK, e_wg0, wave, lane, X, DT, DL, DY);
       else if (into_next)
-        stage_block<T, 3, CW, false, STAGE_X, kFwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, nx.g, 0, e_wg0, wave, lane, X, DT, DL, DY);
+        stage_block<T, 3, CW, false, STAGE_X, kFwdWaves, true>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, nx.g, 0, e_wg0, wave, lane, X, DT, DL, DY);
       TICK(ts1); TACC(1, ts0, ts1);
       // snapshot of the state before the block (after step t0-1); lanes that have not started or
       // are past the last column hold nothing the backward needs
@@ -642,6 +688,8 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   }
   const float* a_base = a_lds + ch_loc * (2 * kN);
   const float dsk = p.Df[e];
+  StagePlan<T, 4, CW, true, kBwdWaves, false> plan;
+  plan.init(wave, lane);
   settle_loads();
 
   const T* X = static_cast<const T*>(p.x);
@@ -709,7 +757,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
     const int nb = cx.nb, T_steps = cx.T_steps;
     if (band == p.nbands - 1 || !streamed) {
       load_ckpt(cx, nb - 1);
-      stage_block<T, 4, CW, true, STAGE_X, kBwdWaves>(p, lds + cur * SG::kBytes, b, cx.g, (nb - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
+      stage_block<T, 4, CW, true, STAGE_X, kBwdWaves, false>(p, plan, lds + cur * SG::kBytes, b, cx.g, (nb - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
       staging_fence();
     }
 #pragma unroll
@@ -727,9 +775,9 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
       for (int n = 0; n < kN; ++n) ck0[n] = cknext[n];
       const bool into_next = m == 0 && more && streamed;
       if (m > 0)
-        stage_block<T, 4, CW, true, STAGE_X, kBwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, cx.g, t0 - kCK, e_wg0, wave, lane, X, DT, DL, DY);
+        stage_block<T, 4, CW, true, STAGE_X, kBwdWaves, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, cx.g, t0 - kCK, e_wg0, wave, lane, X, DT, DL, DY);
       else if (into_next)
-        stage_block<T, 4, CW, true, STAGE_X, kBwdWaves>(p, lds + (cur ^ 1) * SG::kBytes, b, nx.g, (nx.nb - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
+        stage_block<T, 4, CW, true, STAGE_X, kBwdWaves, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, nx.g, (nx.nb - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
 
       // The 16 states are swept in two halves of 8 (state groups 0,1 then 2,3), each half
       // recomputing and then back-propagating the whole block: only 5 x 8 recomputed states are

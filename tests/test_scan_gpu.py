@@ -82,7 +82,9 @@ SHAPES = [
     (1, 60, 10, 3),   # tall, odd channel count (one channel per wave)
     (1, 70, 50, 2),   # two bands of rows
     (2, 130, 20, 2),  # three bands, last one 2 rows
-    (1, 64, 17, 10),  # exactly one full band, channels not a multiple of the workgroup
+    (1, 64, 17, 10),  # channels not a multiple of the workgroup
+    (1, 40, 4, 3),    # three bands narrower than 8 columns: every band restarts the pipeline
+    (2, 31, 8, 2),    # narrowest grid whose bands are streamed back to back
 ]
 
 
