@@ -62,6 +62,8 @@ __device__ long long g_dbg[4096 * 8];
 #endif
 
 struct bf16_t { uint16_t v; };
+typedef float v4f_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) v4f_t lds_float4;   // a float4 known to live in LDS
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t lo16) { return __uint_as_float(lo16 << 16); }
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
@@ -359,7 +361,11 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan
 __device__ __forceinline__ void settle_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
 // all direct-to-LDS loads of this wave have landed ...
-__device__ __forceinline__ void staging_landed() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void staging_landed() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0); known to the compiler, so loads it tracks need no further wait
+  asm volatile("" ::: "memory");
+}
 // ... and those of the other waves too
 __device__ __forceinline__ void staging_fence() {
   staging_landed();
@@ -660,12 +666,15 @@ __device__ __forceinline__ constexpr int fold_state(int m, int qi) {
 template <typename T, bool STAGE_X>
 __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParams p) {
   constexpr int CS = 64 >> kHBShift;     // 4 channel slots
-  constexpr int SLOT = 3 * 64;           // float4s per wave in the exchange buffer
+  constexpr int SLOT = 3 * 64;           // float2s per wave in one exchange buffer
   constexpr int CW = kBwdWaves * CS;
   constexpr bool PERM = true;
   using SG = Stage<T, 4, CW, true>;
   extern __shared__ float4 smem[];
-  float4* slots = smem;                                                  // [wave][3][64]
+  // Exchange buffers for the channel sums of one (step, half of the states): two of them, used
+  // alternately, so that one barrier per exchange is enough (a buffer is rewritten two exchanges
+  // later, after a barrier that every wave reaches only once it has finished reading it).
+  float2* slots = reinterpret_cast<float2*>(smem);                       // [2][wave][3][64]
   float* a_lds = reinterpret_cast<float*>(smem + kBwdWaves * SLOT);      // [wave][CS][2][16], fold order
   float* zrec = a_lds + kBwdWaves * CS * 2 * kN;                         // 64 zero floats
   char* lds = reinterpret_cast<char*>(zrec + 64);                        // 2 staging buffers
@@ -686,10 +695,14 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
     mine[kN + spos<true>(r)] = p.A2L[e * kN + r];
     if (threadIdx.x < 64) zrec[threadIdx.x] = 0.f;
   }
-  const float* a_base = a_lds + ch_loc * (2 * kN);
+  const uint32_t a_base_off = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) float*)(a_lds + ch_loc * (2 * kN)));
   const float dsk = p.Df[e];
   StagePlan<T, 4, CW, true, kBwdWaves, false> plan;
   plan.init(wave, lane);
+#ifdef M2D_X_TIMING
+  long long dbg_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+  const long long dbg_t0 = clock64();
+#endif
   settle_loads();
 
   const T* X = static_cast<const T*>(p.x);
@@ -710,9 +723,8 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   struct BandCtx {
     BandGeom g;
     LaneRole ro;
-    int T_steps, nb, irow;
+    int T_steps, nb;
     bool to_bot;
-    float oT_in, oT_j0, oL_in;
   };
   auto band_ctx = [&](int band) {
     BandCtx c;
@@ -726,20 +738,18 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
     c.ro.gbot = ch_ok && r == kHB - 1 && c.g.has_below;
     c.ro.first_row = c.g.i0 + r - 1 == 0;
     c.to_bot = c.ro.real && c.g.has_above && r == 1;
-    c.oT_in = c.ro.first_row ? ninf : -1.f; c.oT_j0 = c.ro.first_row ? ninf : 0.f; c.oL_in = c.ro.first_row ? 0.f : -1.f;
-    c.irow = c.g.i0 + (c.ro.real ? r - 1 : 0);
     return c;
   };
   const int64_t cell0 = (int64_t)b * p.H * p.W;
   // state snapshot at the start of block mm of a band (zero for lanes that were not under way)
   float cknext[kN];
-  auto load_ckpt = [&](const BandCtx& c, int mm) {
+  auto load_ckpt = [&](int bandi, bool under_way, int mm) {
     const int tt = mm * kCK;
-    if (mm == 0 || !((c.ro.real || c.ro.gtop) && tt - 1 - r >= 0 && tt - 1 - r < p.W)) {
+    if (mm == 0 || !(under_way && tt - 1 - r >= 0 && tt - 1 - r < p.W)) {
 #pragma unroll
       for (int n = 0; n < kN; ++n) cknext[n] = 0.f;
     } else {
-      const float* ck = p.ckpt + (((((int64_t)b * p.nbands + c.g.band) * p.nblk + mm) * p.E + e) * kN) * kHB + r;
+      const float* ck = p.ckpt + (((((int64_t)b * p.nbands + bandi) * p.nblk + mm) * p.E + e) * kN) * kHB + r;
 #pragma unroll
       for (int n = 0; n < kN; ++n) cknext[n] = ck[n * kHB];
     }
@@ -751,12 +761,13 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   const bool streamed = p.W >= 8;
   BandCtx cx = band_ctx(p.nbands - 1);
   int cur = 0;
+  int xpar = 0;   // exchange buffer in use
   for (int band = p.nbands - 1; band >= 0; --band) {
     const bool more = band > 0;
     const BandCtx nx = band_ctx(more ? band - 1 : band);
     const int nb = cx.nb, T_steps = cx.T_steps;
     if (band == p.nbands - 1 || !streamed) {
-      load_ckpt(cx, nb - 1);
+      load_ckpt(cx.g.band, cx.ro.real || cx.ro.gtop, nb - 1);
       stage_block<T, 4, CW, true, STAGE_X, kBwdWaves, false>(p, plan, lds + cur * SG::kBytes, b, cx.g, (nb - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
       staging_fence();
     }
@@ -774,10 +785,12 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
 #pragma unroll
       for (int n = 0; n < kN; ++n) ck0[n] = cknext[n];
       const bool into_next = m == 0 && more && streamed;
+      TICK(ts0);
       if (m > 0)
         stage_block<T, 4, CW, true, STAGE_X, kBwdWaves, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, cx.g, t0 - kCK, e_wg0, wave, lane, X, DT, DL, DY);
       else if (into_next)
         stage_block<T, 4, CW, true, STAGE_X, kBwdWaves, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, nx.g, (nx.nb - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
+      TICK(ts1); TACC(0, ts0, ts1);
 
       // The 16 states are swept in two halves of 8 (state groups 0,1 then 2,3), each half
       // recomputing and then back-propagating the whole block: only 5 x 8 recomputed states are
@@ -791,6 +804,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
 #pragma unroll
           for (int qi = 0; qi < 4; ++qi) hb[0][4 * mgl + qi] = ck0[fold_state(2 * half + mgl, qi)];
         // ---- recompute the states of the block
+        TICK(tr0);
 #pragma unroll
         for (int k = 0; k < kCK; ++k) {
           const int t = t0 + k;
@@ -799,8 +813,8 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
             const bool inw = j >= 0 && j < p.W;
             const bool act = cx.ro.real && inw;
             const bool gact = cx.ro.gtop && inw;
-            const float offT = act ? (j == 0 ? cx.oT_j0 : cx.oT_in) : ninf;
-            const float offL = (act && j != 0) ? cx.oL_in : ninf;
+            const float offT = (act && !cx.ro.first_row) ? (j == 0 ? 0.f : -1.f) : ninf;
+            const float offL = (act && j != 0) ? (cx.ro.first_row ? 0.f : -1.f) : ninf;
             const float cT = act ? (cx.ro.first_row ? 0.f : (j == 0 ? 1.f : 0.5f)) : 0.f;
             const float cL = act ? (cx.ro.first_row ? 1.f : (j == 0 ? 0.f : 0.5f)) : 0.f;
             float xv, dtv, dlv;
@@ -808,12 +822,15 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
               const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
               xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW);
             } else {
-              const int64_t idx = cell0 + cell_in_image(p, cx.irow, inw ? j : 0);
+              const int64_t idx = cell0 + cell_in_image(p, cx.g.i0 + (cx.ro.real ? r - 1 : 0), inw ? j : 0);
               xv = IO<T>::ld(X + idx * p.E + e); dtv = IO<T>::ld(DT + idx * p.E + e); dlv = IO<T>::ld(DL + idx * p.E + e);
             }
             if (!act) { xv = 0.f; dtv = 0.f; dlv = 0.f; }
-            const float* a_mine = a_base;
-            asm volatile("" : "+v"(a_mine));   // keep the per-step reads of A in LDS, not in live registers
+            // keep the per-step reads of A in LDS, not in live registers (the offset is hidden from
+            // the optimiser; the pointer stays an LDS pointer so that the reads are ds_read)
+            uint32_t a_off = a_base_off;
+            asm volatile("" : "+v"(a_off));
+            const lds_float4* a_mine = (const lds_float4*)(uintptr_t)a_off;
             const float* pbt = act ? bcb + (k * kHB + r) * SG::kBStride : (gact ? tpb + (k * CW + ch_loc) * kN : zrec);
             const float* pbl = act ? pbt + kN : pbt;
             const float sT = gact ? 1.f : cT * dtv * xv;
@@ -821,7 +838,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
 #pragma unroll
             for (int mgl = 0; mgl < 2; ++mgl) {
               const int mg = 2 * half + mgl;
-              const float4 at4 = reinterpret_cast<const float4*>(a_mine)[mg], al4 = reinterpret_cast<const float4*>(a_mine + kN)[mg];
+              const v4f_t at4 = a_mine[mg], al4 = a_mine[kN / 4 + mg];
               const float4 b4 = reinterpret_cast<const float4*>(pbt)[mg], l4 = reinterpret_cast<const float4*>(pbl)[mg];
               const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
               const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w};
@@ -839,6 +856,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
             }
           }
         }
+        TICK(tr1); TACC(1, tr0, tr1);
         // ---- adjoint over the block, last step first
 #pragma unroll
         for (int k = kCK - 1; k >= 0; --k) {
@@ -846,16 +864,19 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
           if (half == 1 && k == 0) staging_landed();   // before the last stores of the block, see the forward kernel
           // the states of the later steps are dead by now: their registers take the next snapshot
           if (half == 1 && k == (kCK > 1 ? 1 : 0)) {
-            if (m > 0) load_ckpt(cx, m - 1);
-            else if (into_next) load_ckpt(nx, nx.nb - 1);
+            // one load site for both cases, so that the wait at the start of the next step covers it
+            const bool same = m > 0;
+            if (same || into_next)
+              load_ckpt(same ? cx.g.band : nx.g.band, same ? (cx.ro.real || cx.ro.gtop) : (nx.ro.real || nx.ro.gtop),
+                        same ? m - 1 : nx.nb - 1);
           }
           if (t < T_steps) {
             const int j = t - r;
             const bool inw = j >= 0 && j < p.W;
             const bool act = cx.ro.real && inw;
             const bool gact = cx.ro.gbot && inw;     // ghost of the row below: muT := staged row
-            float offT = act ? (j == 0 ? cx.oT_j0 : cx.oT_in) : ninf;
-            const float offL = (act && j != 0) ? cx.oL_in : ninf;
+            float offT = (act && !cx.ro.first_row) ? (j == 0 ? 0.f : -1.f) : ninf;
+            const float offL = (act && j != 0) ? (cx.ro.first_row ? 0.f : -1.f) : ninf;
             const float cT = act ? (cx.ro.first_row ? 0.f : (j == 0 ? 1.f : 0.5f)) : 0.f;
             const float cL = act ? (cx.ro.first_row ? 1.f : (j == 0 ? 0.f : 0.5f)) : 0.f;
             if (gact) offT = 0.f;                 // open T gate with delta 0: muT = lambda = staged value
@@ -864,13 +885,14 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
               const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
               xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW); dyv = IO<T>::ld(xr + 3 * CW);
             } else {
-              const int64_t idx = cell0 + cell_in_image(p, cx.irow, inw ? j : 0);
+              const int64_t idx = cell0 + cell_in_image(p, cx.g.i0 + (cx.ro.real ? r - 1 : 0), inw ? j : 0);
               xv = IO<T>::ld(X + idx * p.E + e); dtv = IO<T>::ld(DT + idx * p.E + e);
               dlv = IO<T>::ld(DL + idx * p.E + e); dyv = IO<T>::ld(DY + idx * p.E + e);
             }
             if (!act) { dtv = 0.f; dlv = 0.f; dyv = gact ? 1.f : 0.f; xv = 0.f; }
-            const float* a_mine = a_base;
-            asm volatile("" : "+v"(a_mine));
+            uint32_t a_off = a_base_off;
+            asm volatile("" : "+v"(a_off));
+            const lds_float4* a_mine = (const lds_float4*)(uintptr_t)a_off;
             const float* pbt = act ? bcb + (k * kHB + r) * SG::kBStride : (gact ? bob + (k * CW + ch_loc) * kN : zrec);
             const float* pbl = act ? pbt + kN : pbt;
             const float* pcc = act ? pbt + 2 * kN : pbt;
@@ -878,15 +900,15 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
             const float qC = act ? dyv : 0.f;
             float sT = 0.f, sL = 0.f, zT = 0.f, zL = 0.f;
             if (half == 1) { sT = part4[k][0]; sL = part4[k][1]; zT = part4[k][2]; zL = part4[k][3]; }
-            __syncthreads();   // the flush of the previous exchange has finished reading the slots
-            float* sw = reinterpret_cast<float*>(slots + wave * SLOT + lane);
+            TICK(ta1);
+            float* sw = reinterpret_cast<float*>(slots + (xpar * kBwdWaves + wave) * SLOT + lane);
             // A group of 4 states is folded over the 4 channel slots of the wave as soon as it is
             // done; afterwards the lane of slot q holds the channel sums of the states 4q..4q+3
-            // (component mg of its float4 after group mg).
+            // (component mgl of its float2 after group mgl of this half).
 #pragma unroll
             for (int mgl = 0; mgl < 2; ++mgl) {
               const int mg = 2 * half + mgl;
-              const float4 at4 = reinterpret_cast<const float4*>(a_mine)[mg], al4 = reinterpret_cast<const float4*>(a_mine + kN)[mg];
+              const v4f_t at4 = a_mine[mg], al4 = a_mine[kN / 4 + mg];
               const float4 b4 = reinterpret_cast<const float4*>(pbt)[mg], l4 = reinterpret_cast<const float4*>(pbl)[mg];
               const float4 c4 = reinterpret_cast<const float4*>(pcc)[mg];
               const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
@@ -915,9 +937,9 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
                 vBL[qi] = qL * lam;
                 vC[qi] = qC * hb[k + 1][s8];
               }
-              sw[mg] = fold16(fold32(vC[0], vC[1]), fold32(vC[2], vC[3]));
-              sw[64 * 4 + mg] = fold16(fold32(vBT[0], vBT[1]), fold32(vBT[2], vBT[3]));
-              sw[128 * 4 + mg] = fold16(fold32(vBL[0], vBL[1]), fold32(vBL[2], vBL[3]));
+              sw[mgl] = fold16(fold32(vC[0], vC[1]), fold32(vC[2], vC[3]));
+              sw[64 * 2 + mgl] = fold16(fold32(vBT[0], vBT[1]), fold32(vBT[2], vBT[3]));
+              sw[128 * 2 + mgl] = fold16(fold32(vBL[0], vBL[1]), fold32(vBL[2], vBL[3]));
             }
             if (cx.to_bot && act) {   // first row of the band: the band above's lower ghost will replay its muT
               float* bb = p.bot + (((int64_t)b * p.W + j) * p.E + e) * kN;
@@ -930,7 +952,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
               part4[k][0] = sT; part4[k][1] = sL; part4[k][2] = zT; part4[k][3] = zL;
             } else {
               if (act) {
-                const int64_t idx = cell0 + cell_in_image(p, cx.irow, j);
+                const int64_t idx = cell0 + cell_in_image(p, cx.g.i0 + r - 1, j);
                 accD = __builtin_fmaf(dyv, xv, accD);
                 IO<T>::st(DDT + idx * p.E + e, __builtin_fmaf(cT * xv, sT, kLn2 * zT));
                 IO<T>::st(DDL + idx * p.E + e, __builtin_fmaf(cL * xv, sL, kLn2 * zL));
@@ -939,37 +961,44 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
             }
             // ---- across the waves of the workgroup: the per-wave slots (this half's two state
             // groups) are added in wave order
+            TICK(ta2); TACC(3, ta1, ta2); TACC(2, ta2, ta2);
             __syncthreads();
-            if (threadIdx.x < SLOT) {
-              const int it = threadIdx.x;
+            TICK(ta3); TACC(4, ta2, ta3);
+            if (threadIdx.x < 2 * SLOT) {   // one sum per thread, 6 of the 8 waves
+              const int it = threadIdx.x >> 1, comp = threadIdx.x & 1;
               const int fl = it & 63, v = it >> 6;
               const int fr = fl & (kHB - 1), fs = fl >> kHBShift;
               const int fj = t - fr;
               if (fr >= 1 && fr <= cx.g.rows && fj >= 0 && fj < p.W) {
-                const float2* sl2 = reinterpret_cast<const float2*>(slots) + half;
-                float2 s = sl2[2 * it];
+                const float* sl = reinterpret_cast<const float*>(slots + xpar * kBwdWaves * SLOT + it) + comp;
+                float s = sl[0];
 #pragma unroll
-                for (int w = 1; w < kBwdWaves; ++w) {
-                  const float2 o = sl2[2 * (w * SLOT + it)];
-                  s.x += o.x; s.y += o.y;
-                }
+                for (int w = 1; w < kBwdWaves; ++w) s += sl[2 * w * SLOT];
                 const int64_t cell = cell0 + cell_in_image(p, cx.g.i0 + fr - 1, fj);
-                *reinterpret_cast<float2*>(p.part + (((int64_t)eg * 3 + v) * P + cell) * kN + fs * 4 + 2 * half) = s;
+                p.part[(((int64_t)eg * 3 + v) * P + cell) * kN + fs * 4 + 2 * half + comp] = s;
               }
             }
+            xpar ^= 1;
           }
         }
       }
       // restart per band: the band's first-row muT is read back by the first staging of the band above
       if (m == 0 && more && !streamed) __threadfence();
-#ifndef M2D_X_NOBLOCKBAR
+      TICK(tz0);
       __syncthreads();
-#endif
+      TICK(tz1); TACC(5, tz0, tz1);
       cur ^= 1;
     }
     cx = nx;
   }
 
+#ifdef M2D_X_TIMING
+  if (lane == 0 && blockIdx.x < 512) {
+    long long* d = g_dbg + (blockIdx.x * 8 + wave) * 8;
+    for (int i = 0; i < 6; ++i) d[i] = dbg_acc[i];
+    d[6] = clock64() - dbg_t0;
+  }
+#endif
   // ---- sums over positions: reduce over the rows of the band (lanes of one channel slot)
   float red[2 * kN + 1];
 #pragma unroll
