@@ -203,8 +203,12 @@ template <bool PERM> __device__ __forceinline__ constexpr int sinv(int pos) {
 //        (x, deltaT, deltaL[, dy]), plus one pad chunk (needs E to be a multiple of a chunk);
 //   TOP: per (k, channel) the 16 states of the last row of the band above at column t0+k;
 //   BOT: per (k, channel) the 16 muT of the first row of the band below at column t0+k-15.
-// Cells outside the grid read from a page of zeros.
-template <typename T, int NT, int CW, bool WITH_BOT>
+// With UNI, BC, TOP and BOT advance by the same number of bytes (kKStr) from one step to the
+// next, so a lane that reads "its record" finds it at one per-lane offset plus a constant per
+// step, whether it is a grid row (BC record) or a boundary ghost (TOP/BOT record).  Records of lanes and cells
+// outside the grid are filled from a page of zeros: such lanes compute on finite operands and
+// never need to be masked.
+template <typename T, int NT, int CW, bool WITH_BOT, bool UNI>
 struct Stage {
   static constexpr int kElem = 16 / sizeof(T);           // elements per chunk
   static constexpr int kCpt = CW / kElem;                // chunks per tensor per cell
@@ -212,14 +216,18 @@ struct Stage {
   static constexpr int kXStride = kXRec * kElem;         // XD record stride in elements
   static constexpr int kBRec = 13;                       // chunks per BC record (with pad)
   static constexpr int kBStride = kBRec * 4;             // BC record stride in floats
-  static constexpr int kBChunks = kCK * kHB * kBRec;
+  static constexpr int kKChunks = kHB * kBRec > CW * 4 ? kHB * kBRec : CW * 4;   // chunks per step in BC / TOP / BOT
+  static constexpr int kKStr = kKChunks * 16;            // the same in bytes
+  static constexpr int kBChunks = kCK * kKChunks;
   static constexpr int kXChunks = kCK * kHB * kXRec;
-  static constexpr int kTChunks = kCK * CW * 4;
+  static constexpr int kTInstr = kCK * CW / 16;          // wave-wide copies that fill TOP (or BOT): 16 channels each
   static constexpr int kXOff = kBChunks * 16;
   static constexpr int kTOff = kXOff + kXChunks * 16;
-  static constexpr int kOOff = kTOff + kTChunks * 16;
-  static constexpr int kBytes = kOOff + (WITH_BOT ? kTChunks * 16 : 0);   // one buffer
+  static constexpr int kTKStr = UNI ? kKStr : CW * 64;   // bytes per step in TOP / BOT (UNI: the same as in BC)
+  static constexpr int kOOff = kTOff + kCK * kTKStr;
+  static constexpr int kBytes = kOOff + (WITH_BOT ? kCK * kTKStr : 0);   // one buffer
   static_assert(CW % kElem == 0, "workgroup channel count must fill whole chunks");
+  static_assert(CW % 16 == 0, "boundary rows are copied 16 channels at a time");
 };
 
 // One wave-wide direct load: lane i copies 16 bytes from its own global address to
@@ -244,47 +252,48 @@ struct BandGeom {   // wave-uniform description of the band being swept
 // The chunk -> (step, row, part of record) decomposition of the BC and XD regions depends only on
 // the thread.  It is worked out once (divisions by the odd record sizes) and kept as one packed
 // word per wave-wide copy: bits 0-3 row, 4-8 part, 9-10 step, bit 31 set if the chunk carries data.
-template <typename T, int NT, int CW, bool WITH_BOT, int NWAVES, bool KEEP>
+template <typename T, int NT, int CW, bool WITH_BOT, bool UNI, int NWAVES, bool KEEP>
 struct StagePlan {
-  using SG = Stage<T, NT, CW, WITH_BOT>;
+  using SG = Stage<T, NT, CW, WITH_BOT, UNI>;
   static constexpr int kPer = NWAVES * 64;
   static constexpr int kItB = (SG::kBChunks + kPer - 1) / kPer;
   static constexpr int kItX = (SG::kXChunks + kPer - 1) / kPer;
   uint32_t bc[KEEP ? kItB : 1], xd[KEEP ? kItX : 1];
-  static __device__ __forceinline__ uint32_t word(int c, int nchunks, int reclen, int nparts) {
-    const int rec = c / reclen, part = c - rec * reclen;
-    const int k = rec >> kHBShift, r = rec & (kHB - 1);
-    return (c < nchunks && part < nparts && r >= 1 && r <= kRB) ? (0x80000000u | (k << 9) | (part << 4) | r) : 0u;
+  // `perk` chunks per step, of which the first kHB*reclen hold the records of the 16 lane rows
+  static __device__ __forceinline__ uint32_t word(int c, int nchunks, int perk, int reclen, int nparts) {
+    const int k = c / perk, rem = c - k * perk;
+    const int r = rem / reclen, part = rem - r * reclen;
+    return (c < nchunks && r < kHB && part < nparts) ? (0x80000000u | (k << 9) | (part << 4) | r) : 0u;
   }
   __device__ __forceinline__ void init(int wave, int lane) {
     if constexpr (KEEP) {
 #pragma unroll
-      for (int i = 0; i < kItB; ++i) bc[i] = word(i * kPer + wave * 64 + lane, SG::kBChunks, SG::kBRec, 12);
+      for (int i = 0; i < kItB; ++i) bc[i] = word(i * kPer + wave * 64 + lane, SG::kBChunks, SG::kKChunks, SG::kBRec, 12);
 #pragma unroll
-      for (int i = 0; i < kItX; ++i) xd[i] = word(i * kPer + wave * 64 + lane, SG::kXChunks, SG::kXRec, NT * SG::kCpt);
+      for (int i = 0; i < kItX; ++i) xd[i] = word(i * kPer + wave * 64 + lane, SG::kXChunks, kHB * SG::kXRec, SG::kXRec, NT * SG::kCpt);
     }
   }
   // Kernels short of registers work the word out again at every use instead of keeping it.
   __device__ __forceinline__ uint32_t get_bc(int i, int wave, int lane) const {
     uint32_t w;
-    if constexpr (KEEP) { w = bc[i]; } else { asm volatile("" : "+v"(lane)); w = word(i * kPer + wave * 64 + lane, SG::kBChunks, SG::kBRec, 12); }
+    if constexpr (KEEP) { w = bc[i]; } else { asm volatile("" : "+v"(lane)); w = word(i * kPer + wave * 64 + lane, SG::kBChunks, SG::kKChunks, SG::kBRec, 12); }
     asm volatile("" : "+v"(w));   // unpack per use: the fields must not be hoisted into live registers
     return w;
   }
   __device__ __forceinline__ uint32_t get_xd(int i, int wave, int lane) const {
     uint32_t w;
-    if constexpr (KEEP) { w = xd[i]; } else { asm volatile("" : "+v"(lane)); w = word(i * kPer + wave * 64 + lane, SG::kXChunks, SG::kXRec, NT * SG::kCpt); }
+    if constexpr (KEEP) { w = xd[i]; } else { asm volatile("" : "+v"(lane)); w = word(i * kPer + wave * 64 + lane, SG::kXChunks, kHB * SG::kXRec, SG::kXRec, NT * SG::kCpt); }
     asm volatile("" : "+v"(w));
     return w;
   }
 };
 
-template <typename T, int NT, int CW, bool WITH_BOT, bool STAGE_X, int NWAVES, bool KEEP>
-__device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan<T, NT, CW, WITH_BOT, NWAVES, KEEP>& plan, char* buf,
+template <typename T, int NT, int CW, bool WITH_BOT, bool UNI, bool STAGE_X, int NWAVES, bool KEEP>
+__device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan<T, NT, CW, WITH_BOT, UNI, NWAVES, KEEP>& plan, char* buf,
                                             int b, const BandGeom& g, int t0, int e_wg0, int wave, int lane,
                                             const T* x0, const T* x1, const T* x2, const T* x3) {
-  using SG = Stage<T, NT, CW, WITH_BOT>;
-  using PL = StagePlan<T, NT, CW, WITH_BOT, NWAVES, KEEP>;
+  using SG = Stage<T, NT, CW, WITH_BOT, UNI>;
+  using PL = StagePlan<T, NT, CW, WITH_BOT, UNI, NWAVES, KEEP>;
   static_assert((SG::kCpt & (SG::kCpt - 1)) == 0, "chunks per tensor row must be a power of two");
 #ifdef M2D_X_NOSTAGE
   return;
@@ -295,10 +304,10 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan
   for (int i = 0; i < PL::kItB; ++i) {
     const uint32_t w = plan.get_bc(i, wave, lane);
     const int r = w & 15, part = (w >> 4) & 31, k = (w >> 9) & 3;
-    if ((int)w < 0 && r <= g.rows) {
+    if ((int)w < 0) {
       const int j = t0 + k - r;
       const float* src = p.zeros;
-      if ((unsigned)j < (unsigned)p.W) {   // the packed record holds B_T, B_L, C back to back: chunk `part` of 12
+      if ((unsigned)j < (unsigned)p.W && r >= 1 && r <= g.rows) {   // the packed record holds B_T, B_L, C back to back
         int cell = (g.i0 + r - 1) * p.W + j;
         cell = p.flip ? hw1 - cell : cell;
         src = p.bt + (img + cell) * p.bc_stride + part * 4;
@@ -311,11 +320,11 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan
     for (int i = 0; i < PL::kItX; ++i) {
       const uint32_t w = plan.get_xd(i, wave, lane);
       const int r = w & 15, part = (w >> 4) & 31, k = (w >> 9) & 3;
-      if ((int)w < 0 && r <= g.rows) {
+      if ((int)w < 0) {
         const int j = t0 + k - r;
         const int tau = part / SG::kCpt, ch = e_wg0 + (part & (SG::kCpt - 1)) * SG::kElem;
         const void* src = p.zeros;
-        if ((unsigned)j < (unsigned)p.W && ch < p.E) {
+        if ((unsigned)j < (unsigned)p.W && r >= 1 && r <= g.rows && ch < p.E) {
           int cell = (g.i0 + r - 1) * p.W + j;
           cell = p.flip ? hw1 - cell : cell;
           // selected with compares: an indexed pointer table would live in (scratch) memory
@@ -327,30 +336,25 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan
     }
   }
   // boundary rows were written earlier in this launch (or by the forward launch): read them
-  // past the L1
-  static_assert((CW & (CW - 1)) == 0, "channels per workgroup must be a power of two");
-  for (int c0 = wave * 64; c0 < SG::kTChunks; c0 += NWAVES * 64) {
-    const int c = c0 + lane;
-    const int rec = c >> 2, k = rec / CW, ch = e_wg0 + (rec & (CW - 1));
-    if (c < SG::kTChunks) {
-      const int j = t0 + k;
-      const float* src = p.zeros;
-      if (g.has_above && j >= 0 && j < p.W && ch < p.E)
-        src = p.top + ((((int64_t)(g.band - 1) * p.B + b) * p.W + j) * p.E + ch) * kN + (c & 3) * 4;
-      lds_fill16<true>(src, buf + SG::kTOff + c0 * 16);
-    }
+  // past the L1.  One wave-wide copy moves the records of 16 channels at one step.
+  for (int q = wave; q < SG::kTInstr; q += NWAVES) {
+    const int k = q / (CW / 16), sub = q - k * (CW / 16);
+    const int ch = e_wg0 + sub * 16 + (lane >> 2);
+    const int j = t0 + k;
+    const float* src = p.zeros;
+    if (g.has_above && j >= 0 && j < p.W && ch < p.E)
+      src = p.top + ((((int64_t)(g.band - 1) * p.B + b) * p.W + j) * p.E + ch) * kN + (lane & 3) * 4;
+    lds_fill16<true>(src, buf + SG::kTOff + k * SG::kTKStr + sub * 1024);
   }
   if constexpr (WITH_BOT) {
-    for (int c0 = wave * 64; c0 < SG::kTChunks; c0 += NWAVES * 64) {
-      const int c = c0 + lane;
-      const int rec = c >> 2, k = rec / CW, ch = e_wg0 + (rec & (CW - 1));
-      if (c < SG::kTChunks) {
-        const int j = t0 + k - (kHB - 1);
-        const float* src = p.zeros;
-        if (g.has_below && j >= 0 && j < p.W && ch < p.E)
-          src = p.bot + (((int64_t)b * p.W + j) * p.E + ch) * kN + (c & 3) * 4;
-        lds_fill16<true>(src, buf + SG::kOOff + c0 * 16);
-      }
+    for (int q = wave; q < SG::kTInstr; q += NWAVES) {
+      const int k = q / (CW / 16), sub = q - k * (CW / 16);
+      const int ch = e_wg0 + sub * 16 + (lane >> 2);
+      const int j = t0 + k - (kHB - 1);
+      const float* src = p.zeros;
+      if (g.has_below && j >= 0 && j < p.W && ch < p.E)
+        src = p.bot + (((int64_t)b * p.W + j) * p.E + ch) * kN + (lane & 3) * 4;
+      lds_fill16<true>(src, buf + SG::kOOff + k * SG::kTKStr + sub * 1024);
     }
   }
 }
@@ -385,16 +389,19 @@ struct LaneRole {
 };
 
 // ------------------------------------------------------------------------------------ forward
+// Lanes are never masked in the forward: a grid row that has not reached column 0 yet, or is past
+// the last column, works on zero operands (its records come from the page of zeros), which keeps
+// its state finite and never reaches a cell of the grid: at column 0 the left gate is closed, and
+// a row past the end only feeds rows that are past the end too.  Only the stores are predicated.
 template <typename T, int EC, bool CKPT, bool WRITE_Y, bool STAGE_X>
 __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParams p) {
   constexpr int CS = 64 >> kHBShift;
   constexpr int CW = kFwdWaves * CS * EC;
   constexpr bool PERM = true;
   constexpr bool AHEAD = EC == 1;   // operands of step t+1 are fetched from LDS during step t
-  using SG = Stage<T, 3, CW, false>;
+  using SG = Stage<T, 3, CW, false, true>;
   extern __shared__ float4 smem[];
-  float* zrec = reinterpret_cast<float*>(smem);            // 64 zero floats
-  char* lds = reinterpret_cast<char*>(smem + 16);
+  char* lds = reinterpret_cast<char*>(smem);       // two staging buffers and 256 bytes of slack
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lb = logical_block(p.nwg);
@@ -405,8 +412,9 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   const int e_raw = e_wg0 + ch_loc;
   const bool ch_ok = e_raw < p.E;                  // idle lanes still take part in staging and barriers
   const int e0 = ch_ok ? e_raw : p.E - EC;
-  if (threadIdx.x < 64) zrec[threadIdx.x] = 0.f;
-  StagePlan<T, 3, CW, false, kFwdWaves, true> plan;
+  // every byte a lane may read is finite from the start (pads are never written again)
+  for (int i = threadIdx.x; i < (2 * SG::kBytes + 256) / 16; i += kFwdWaves * 64) smem[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+  StagePlan<T, 3, CW, false, true, kFwdWaves, true> plan;
   plan.init(wave, lane);
 
   float a2t[EC][kN], a2l[EC][kN], dsk[EC];
@@ -418,6 +426,7 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   }
 
   settle_loads();
+  __syncthreads();
 #ifdef M2D_X_TIMING
   long long dbg_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   const long long dbg_t0 = clock64();
@@ -426,16 +435,26 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   const T* DT = static_cast<const T*>(p.dT);
   const T* DL = static_cast<const T*>(p.dL);
   const T* DY = DL;   // not staged by the forward (NT = 3)
-  T* Y = static_cast<T*>(p.y);
   const float ninf = -__builtin_huge_valf();
+  const int64_t cell0 = (int64_t)b * p.H * p.W;
+  // (B,H,W,E) tensors are addressed as image base (uniform) + 32-bit byte offset (per lane)
+  const int64_t img_bytes = cell0 * p.E * (int64_t)sizeof(T);
+  char* Yimg = static_cast<char*>(p.y) + img_bytes;
+  const char* Ximg = reinterpret_cast<const char*>(X) + img_bytes;
+  const char* DTimg = reinterpret_cast<const char*>(DT) + img_bytes;
+  const char* DLimg = reinterpret_cast<const char*>(DL) + img_bytes;
+  const uint32_t estep = (uint32_t)(p.flip ? -p.E : p.E) * (uint32_t)sizeof(T);   // one column further
 
-  // Everything about a band that the inner loops need (wave-uniform geometry, per-lane roles).
+  // Everything about a band that the inner loops need: wave-uniform geometry and per-lane constants.
   struct BandCtx {
     BandGeom g;
-    LaneRole ro;
-    int T_steps, nb, irow;
-    bool to_top;
-    float oT_in, oT_j0, oL_in;
+    int T_steps, nb;
+    bool real, ckpt_lane, to_top;
+    float oT, oL, cT, cL;        // gate offsets (log2 of the coefficient) and input coefficients inside the grid
+    float oT0, cT0, cL0;         // the same at column 0 (the left gate is closed there)
+    float g1;                    // 1 on the ghost lane: its T input coefficient
+    uint32_t cell_off;           // byte offset of (lane row, column -r) in a (H,W,E) image: + t*estep = this step's cell
+    uint32_t top_off;            // byte offset of column -r in the row buffer this band writes for the next one
   };
   auto band_ctx = [&](int band) {
     BandCtx c;
@@ -444,16 +463,31 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
     c.g.has_above = band > 0; c.g.has_below = band + 1 < p.nbands;
     c.T_steps = c.g.has_below ? p.W + kHB - 1 : p.W + c.g.rows;   // same step count as the backward
     c.nb = (c.T_steps + kCK - 1) / kCK;
-    c.ro.real = ch_ok && r >= 1 && r <= c.g.rows;
-    c.ro.gtop = ch_ok && r == 0 && c.g.has_above;
-    c.ro.gbot = false;
-    c.ro.first_row = c.g.i0 + r - 1 == 0;
-    c.to_top = c.ro.real && c.g.has_below && r == kRB;
-    c.oT_in = c.ro.first_row ? ninf : -1.f; c.oT_j0 = c.ro.first_row ? ninf : 0.f; c.oL_in = c.ro.first_row ? 0.f : -1.f;
-    c.irow = c.g.i0 + (c.ro.real ? r - 1 : 0);
+    c.real = ch_ok && r >= 1 && r <= c.g.rows;
+    const bool ghost = r == 0;
+    const bool first_row = c.g.i0 + r - 1 == 0;
+    c.ckpt_lane = c.real || (ch_ok && ghost && c.g.has_above);
+    c.to_top = c.real && c.g.has_below && r == kRB;
+    c.oT = !c.real || first_row ? ninf : -1.f;
+    c.oL = !c.real ? ninf : (first_row ? 0.f : -1.f);
+    c.cT = !c.real || first_row ? 0.f : 0.5f;
+    c.cL = !c.real ? 0.f : (first_row ? 1.f : 0.5f);
+    c.oT0 = !c.real || first_row ? ninf : 0.f;
+    c.cT0 = !c.real || first_row ? 0.f : 1.f;
+    c.cL0 = c.real && first_row ? 1.f : 0.f;
+    c.g1 = ghost ? 1.f : 0.f;
+    const int row = c.g.i0 + r - 1;
+    const int cellm = row * p.W - r;                                   // cell index at t = 0
+    c.cell_off = (uint32_t)((p.flip ? p.H * p.W - 1 - cellm : cellm) * p.E + e0) * (uint32_t)sizeof(T);
+    c.top_off = (uint32_t)(-r * p.E + e0) * (uint32_t)(kN * sizeof(float));
     return c;
   };
-  const int64_t cell0 = (int64_t)b * p.H * p.W;
+
+  // byte offsets of the lane's records inside a staging buffer (step 0)
+  const uint32_t rec_off = r == 0 ? SG::kTOff + ch_loc * kN * 4 : r * SG::kBStride * 4;
+  const uint32_t rec_cstep = r == 0 ? kN * 4 : 0;   // the ghost reads a record per channel, grid rows share theirs
+  const uint32_t xd_off = SG::kXOff + (r * SG::kXStride + ch_loc) * (uint32_t)sizeof(T);
+  constexpr uint32_t kXK = kHB * SG::kXStride * sizeof(T);   // XD bytes per step
 
   // Operands of one step, read from the staging buffer one step ahead of their use so that the
   // LDS latency hides behind the arithmetic of the step before.
@@ -462,60 +496,48 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
     float4 bt[EC][4], bl[4], cc[4];
   };
   auto fetch = [&](const BandCtx& cx, const char* bufc, int k, int t, Ops& o) {
-    const float* bcb = reinterpret_cast<const float*>(bufc);
-    const T* xdb = reinterpret_cast<const T*>(bufc + SG::kXOff);
-    const float* tpb = reinterpret_cast<const float*>(bufc + SG::kTOff);
-    const int j = t - r;
-    const bool inw = j >= 0 && j < p.W;
-    const bool act = cx.ro.real && inw;
-    const bool gact = cx.ro.gtop && inw;
     if constexpr (STAGE_X) {
-      const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
+      const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
       IO<T>::template ldv<EC>(xr, o.xv);
       IO<T>::template ldv<EC>(xr + CW, o.dtv);
       IO<T>::template ldv<EC>(xr + 2 * CW, o.dlv);
     } else {
-      const int64_t idx = cell0 + cell_in_image(p, cx.irow, inw ? j : 0);
-      IO<T>::template ldv<EC>(X + idx * p.E + e0, o.xv);
-      IO<T>::template ldv<EC>(DT + idx * p.E + e0, o.dtv);
-      IO<T>::template ldv<EC>(DL + idx * p.E + e0, o.dlv);
-    }
-    // operand records: a grid row reads B_T, B_L, C of its cell; the ghost reads the row above
-    // as its B_T (and harmless finite stand-ins for the other two)
-    const float* rec = bcb + (k * kHB + r) * SG::kBStride;
+      const bool inr = cx.real && (unsigned)(t - r) < (unsigned)p.W;
 #pragma unroll
-    for (int c = 0; c < EC; ++c) {
-      const float* pbt = act ? rec : (gact ? tpb + (k * CW + ch_loc + c) * kN : zrec);
-#pragma unroll
-      for (int q = 0; q < 4; ++q) o.bt[c][q] = reinterpret_cast<const float4*>(pbt)[q];
+      for (int c = 0; c < EC; ++c) { o.xv[c] = 0.f; o.dtv[c] = 0.f; o.dlv[c] = 0.f; }
+      if (inr) {
+        const uint32_t off = cx.cell_off + (uint32_t)t * estep;
+        IO<T>::template ldv<EC>(reinterpret_cast<const T*>(Ximg + off), o.xv);
+        IO<T>::template ldv<EC>(reinterpret_cast<const T*>(DTimg + off), o.dtv);
+        IO<T>::template ldv<EC>(reinterpret_cast<const T*>(DLimg + off), o.dlv);
+      }
     }
-    const float* pbl = act ? rec + kN : zrec;
-    const float* pcc = act ? rec + 2 * kN : zrec;
+    // a grid row reads B_T, B_L, C of its cell; the ghost reads the row above as its B_T (and
+    // the finite records next to it as stand-ins for the other two, which it multiplies by 0)
+    const char* rec = bufc + rec_off + k * SG::kKStr;
+#pragma unroll
+    for (int c = 0; c < EC; ++c)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) o.bt[c][q] = reinterpret_cast<const float4*>(rec + c * rec_cstep)[q];
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      o.bl[q] = reinterpret_cast<const float4*>(pbl)[q];
-      o.cc[q] = WRITE_Y ? reinterpret_cast<const float4*>(pcc)[q] : make_float4(0, 0, 0, 0);
+      o.bl[q] = reinterpret_cast<const float4*>(rec + kN * 4)[q];
+      o.cc[q] = WRITE_Y ? reinterpret_cast<const float4*>(rec + 2 * kN * 4)[q] : make_float4(0, 0, 0, 0);
     }
   };
 
   float h[EC][kN];
-  auto step = [&](const BandCtx& cx, int t, Ops& o) {
-    const int j = t - r;
-    const bool inw = j >= 0 && j < p.W;
-    const bool act = cx.ro.real && inw;
-    const bool gact = cx.ro.gtop && inw;
-    const float offT = act ? (j == 0 ? cx.oT_j0 : cx.oT_in) : ninf;
-    const float offL = (act && j != 0) ? cx.oL_in : ninf;
-    const float cT = act ? (cx.ro.first_row ? 0.f : (j == 0 ? 1.f : 0.5f)) : 0.f;
-    const float cL = act ? (cx.ro.first_row ? 1.f : (j == 0 ? 0.f : 0.5f)) : 0.f;
-    if (!act) {   // records of cells outside the grid are not staged
-#pragma unroll
-      for (int c = 0; c < EC; ++c) { o.xv[c] = 0.f; o.dtv[c] = 0.f; o.dlv[c] = 0.f; }
-    }
+  auto step = [&](const BandCtx& cx, int t, const Ops& o) {
+    const bool col0 = t == r;
+    const float offT = col0 ? cx.oT0 : cx.oT;
+    const float offL = col0 ? ninf : cx.oL;
+    const float cT = col0 ? cx.cT0 : cx.cT;
+    const float cL = col0 ? cx.cL0 : cx.cL;
+    const bool inr = cx.real && (unsigned)(t - r) < (unsigned)p.W;
     float yv[EC];
 #pragma unroll
     for (int c = 0; c < EC; ++c) {
-      const float sT = gact ? 1.f : cT * o.dtv[c] * o.xv[c];
+      const float sT = __builtin_fmaf(cT * o.dtv[c], o.xv[c], cx.g1);
       const float sL = cL * o.dlv[c] * o.xv[c];
       float acc = 0.f;
 #pragma unroll
@@ -537,18 +559,21 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
         }
       }
       yv[c] = __builtin_fmaf(o.xv[c], dsk[c], acc);
-      if (cx.to_top && act) {   // last row of the band: the next band's ghost will replay it
-        float* tw = p.top + ((((int64_t)cx.g.band * p.B + b) * p.W + j) * p.E + e0 + c) * kN;
+    }
+    if (cx.g.has_below) {   // last row of the band: the next band's ghost will replay it
+      if (cx.to_top && inr) {
+        char* tw = reinterpret_cast<char*>(p.top + ((int64_t)cx.g.band * p.B + b) * p.W * p.E * kN) +
+                   (cx.top_off + (uint32_t)t * (uint32_t)(p.E * kN * sizeof(float)));
 #pragma unroll
-        for (int q = 0; q < 4; ++q)
-          reinterpret_cast<float4*>(tw)[q] = make_float4(h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)],
-                                                         h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
+        for (int c = 0; c < EC; ++c)
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            reinterpret_cast<float4*>(tw)[c * 4 + q] = make_float4(h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)],
+                                                                   h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
       }
     }
-    if (WRITE_Y && act) {
-      const int64_t idx = cell0 + cell_in_image(p, cx.irow, j);
-      IO<T>::template stv<EC>(Y + idx * p.E + e0, yv);
-    }
+    if (WRITE_Y && inr)
+      IO<T>::template stv<EC>(reinterpret_cast<T*>(Yimg + (cx.cell_off + (uint32_t)t * estep)), yv);
   };
 
   // The bands of the image are swept one after the other without draining the pipeline: while
@@ -558,17 +583,17 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   // past the L1.  Grids narrower than 8 columns, where that does not hold, restart per band.
   const bool streamed = p.W >= 8;
   BandCtx cx = band_ctx(0);
-  Ops ahead;
+  Ops opsA, opsB;
   int cur = 0;
   for (int band = 0; band < p.nbands; ++band) {
     const bool more = band + 1 < p.nbands;
     const BandCtx nx = band_ctx(more ? band + 1 : band);
     if (band == 0 || !streamed) {
       TICK(tb0);
-      stage_block<T, 3, CW, false, STAGE_X, kFwdWaves, true>(p, plan, lds + cur * SG::kBytes, b, cx.g, 0, e_wg0, wave, lane, X, DT, DL, DY);
+      stage_block<T, 3, CW, false, true, STAGE_X, kFwdWaves, true>(p, plan, lds + cur * SG::kBytes, b, cx.g, 0, e_wg0, wave, lane, X, DT, DL, DY);
       staging_fence();
       TICK(tb1); TACC(0, tb0, tb1);
-      if constexpr (AHEAD) fetch(cx, lds + cur * SG::kBytes, 0, 0, ahead);
+      if constexpr (AHEAD) fetch(cx, lds + cur * SG::kBytes, 0, 0, opsA);
     }
 #pragma unroll
     for (int c = 0; c < EC; ++c)
@@ -582,13 +607,13 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
       const bool into_next = last && more && streamed;
       TICK(ts0);
       if (!last)
-        stage_block<T, 3, CW, false, STAGE_X, kFwdWaves, true>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, cx.g, t0 + kCK, e_wg0, wave, lane, X, DT, DL, DY);
+        stage_block<T, 3, CW, false, true, STAGE_X, kFwdWaves, true>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, cx.g, t0 + kCK, e_wg0, wave, lane, X, DT, DL, DY);
       else if (into_next)
-        stage_block<T, 3, CW, false, STAGE_X, kFwdWaves, true>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, nx.g, 0, e_wg0, wave, lane, X, DT, DL, DY);
+        stage_block<T, 3, CW, false, true, STAGE_X, kFwdWaves, true>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, nx.g, 0, e_wg0, wave, lane, X, DT, DL, DY);
       TICK(ts1); TACC(1, ts0, ts1);
       // snapshot of the state before the block (after step t0-1); lanes that have not started or
       // are past the last column hold nothing the backward needs
-      if (CKPT && m > 0 && (cx.ro.real || cx.ro.gtop) && t0 - 1 - r >= 0 && t0 - 1 - r < p.W) {
+      if (CKPT && m > 0 && cx.ckpt_lane && t0 - 1 - r >= 0 && t0 - 1 - r < p.W) {
         float* ck = p.ckpt + (((((int64_t)b * p.nbands + band) * p.nblk + m) * p.E + e0) * kN) * kHB + r;
 #pragma unroll
         for (int c = 0; c < EC; ++c)
@@ -597,11 +622,13 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
       }
       const char* bufc = lds + cur * SG::kBytes;
       const char* bufn = lds + (cur ^ 1) * SG::kBytes;
+      if constexpr (AHEAD) {
+        static_assert(kCK % 2 == 0, "the two operand sets alternate and must close over a block");
 #pragma unroll
-      for (int k = 0; k < kCK; ++k) {
-        const int t = t0 + k;
-        if constexpr (AHEAD) {
-          Ops now = ahead;
+        for (int k = 0; k < kCK; ++k) {
+          const int t = t0 + k;
+          Ops& now = (k & 1) ? opsB : opsA;
+          Ops& ahead = (k & 1) ? opsA : opsB;
           if (k + 1 < kCK) {
             fetch(cx, bufc, k + 1, t + 1, ahead);
           } else {
@@ -619,15 +646,18 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
           TICK(tc0);
           if (t < T_steps) step(cx, t, now);
           TICK(tc1); TACC(4, tc0, tc1);
-        } else {
+        }
+      } else {
+#pragma unroll
+        for (int k = 0; k < kCK; ++k) {
+          const int t = t0 + k;
           // The operands of the next block must have landed before the barrier that ends this
           // block.  Waiting here, before the stores of the last step are issued, keeps the latency
           // of those stores off the critical path (the counter covers loads and stores alike).
           if (k == kCK - 1) staging_landed();
           if (t < T_steps) {
-            Ops now;
-            fetch(cx, bufc, k, t, now);
-            step(cx, t, now);
+            fetch(cx, bufc, k, t, opsA);
+            step(cx, t, opsA);
           }
         }
       }
@@ -669,7 +699,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   constexpr int SLOT = 3 * 64;           // float2s per wave in one exchange buffer
   constexpr int CW = kBwdWaves * CS;
   constexpr bool PERM = true;
-  using SG = Stage<T, 4, CW, true>;
+  using SG = Stage<T, 4, CW, true, false>;
   extern __shared__ float4 smem[];
   // Exchange buffers for the channel sums of one (step, half of the states): two of them, used
   // alternately, so that one barrier per exchange is enough (a buffer is rewritten two exchanges
@@ -697,7 +727,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   }
   const uint32_t a_base_off = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) float*)(a_lds + ch_loc * (2 * kN)));
   const float dsk = p.Df[e];
-  StagePlan<T, 4, CW, true, kBwdWaves, false> plan;
+  StagePlan<T, 4, CW, true, false, kBwdWaves, false> plan;
   plan.init(wave, lane);
 #ifdef M2D_X_TIMING
   long long dbg_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -768,7 +798,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
     const int nb = cx.nb, T_steps = cx.T_steps;
     if (band == p.nbands - 1 || !streamed) {
       load_ckpt(cx.g.band, cx.ro.real || cx.ro.gtop, nb - 1);
-      stage_block<T, 4, CW, true, STAGE_X, kBwdWaves, false>(p, plan, lds + cur * SG::kBytes, b, cx.g, (nb - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
+      stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds + cur * SG::kBytes, b, cx.g, (nb - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
       staging_fence();
     }
 #pragma unroll
@@ -787,9 +817,9 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
       const bool into_next = m == 0 && more && streamed;
       TICK(ts0);
       if (m > 0)
-        stage_block<T, 4, CW, true, STAGE_X, kBwdWaves, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, cx.g, t0 - kCK, e_wg0, wave, lane, X, DT, DL, DY);
+        stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, cx.g, t0 - kCK, e_wg0, wave, lane, X, DT, DL, DY);
       else if (into_next)
-        stage_block<T, 4, CW, true, STAGE_X, kBwdWaves, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, nx.g, (nx.nb - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
+        stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, nx.g, (nx.nb - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
       TICK(ts1); TACC(0, ts0, ts1);
 
       // The 16 states are swept in two halves of 8 (state groups 0,1 then 2,3), each half
@@ -831,7 +861,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
             uint32_t a_off = a_base_off;
             asm volatile("" : "+v"(a_off));
             const lds_float4* a_mine = (const lds_float4*)(uintptr_t)a_off;
-            const float* pbt = act ? bcb + (k * kHB + r) * SG::kBStride : (gact ? tpb + (k * CW + ch_loc) * kN : zrec);
+            const float* pbt = act ? bcb + k * (SG::kKStr / 4) + r * SG::kBStride : (gact ? tpb + k * (SG::kTKStr / 4) + ch_loc * kN : zrec);
             const float* pbl = act ? pbt + kN : pbt;
             const float sT = gact ? 1.f : cT * dtv * xv;
             const float sL = cL * dlv * xv;
@@ -893,7 +923,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
             uint32_t a_off = a_base_off;
             asm volatile("" : "+v"(a_off));
             const lds_float4* a_mine = (const lds_float4*)(uintptr_t)a_off;
-            const float* pbt = act ? bcb + (k * kHB + r) * SG::kBStride : (gact ? bob + (k * CW + ch_loc) * kN : zrec);
+            const float* pbt = act ? bcb + k * (SG::kKStr / 4) + r * SG::kBStride : (gact ? bob + k * (SG::kTKStr / 4) + ch_loc * kN : zrec);
             const float* pbl = act ? pbt + kN : pbt;
             const float* pcc = act ? pbt + 2 * kN : pbt;
             const float qT = cT * dtv * xv, qL = cL * dlv * xv;   // zero on lanes that are not grid cells
@@ -964,8 +994,9 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
             TICK(ta2); TACC(3, ta1, ta2); TACC(2, ta2, ta2);
             __syncthreads();
             TICK(ta3); TACC(4, ta2, ta3);
-            if (threadIdx.x < 2 * SLOT) {   // one sum per thread, 6 of the 8 waves
-              const int it = threadIdx.x >> 1, comp = threadIdx.x & 1;
+            if (lane < 2 * SLOT / kBwdWaves) {   // one sum per thread, the same share for every wave
+              const int fid = wave * (2 * SLOT / kBwdWaves) + lane;
+              const int it = fid >> 1, comp = fid & 1;
               const int fl = it & 63, v = it >> 6;
               const int fr = fl & (kHB - 1), fs = fl >> kHBShift;
               const int fj = t - fr;
@@ -1190,7 +1221,7 @@ int stage_bc(ScanParams& sp, const m2d_desc* d, const void* BT, const void* BL, 
 
 template <typename T, int EC, bool CK, bool WY, bool SX>
 int launch_fwd_as(const ScanParams& sp, hipStream_t st) {
-  using SG = Stage<T, 3, kFwdWaves * 4 * EC, false>;
+  using SG = Stage<T, 3, kFwdWaves * 4 * EC, false, true>;
   const size_t lds = 256 + 2 * (size_t)SG::kBytes;
   static bool attr = false;   // idempotent, the value never changes
   if (!attr) {
@@ -1241,7 +1272,7 @@ int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
 
 template <typename T, bool SX>
 int launch_bwd(const ScanParams& sp, hipStream_t st) {
-  using SG = Stage<T, 4, kBwdWaves * 4, true>;
+  using SG = Stage<T, 4, kBwdWaves * 4, true, false>;
   const size_t lds = sizeof(float4) * kBwdWaves * 3 * 64 + sizeof(float) * kBwdWaves * 4 * 2 * kN + 256 + 2 * (size_t)SG::kBytes;
   static bool attr = false;   // idempotent, the value never changes
   if (!attr) {
