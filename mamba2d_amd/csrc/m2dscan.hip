@@ -152,7 +152,7 @@ struct ScanParams {
   float* ckpt;                      // [B][nbands][nblk][E][16][16]  state snapshots
   float* top;                       // [nbands-1][B][W][E][16]       last row of each band (forward states)
   float* bot;                       // [B][W][E][16]                 first-row muT of the band below (adjoint)
-  float* part;                      // [G][3][P][16]                 per-workgroup channel sums
+  float* part;                      // [G][P][3][16]                 per-workgroup channel sums of d_C, d_BT, d_BL
   float* pA;                        // [B][E][2][16]
   float* pD;                        // [B][E]
   int B, H, W, E;
@@ -638,7 +638,9 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
             TICK(tw0);
             staging_landed();
             TICK(tw1); TACC(2, tw0, tw1);
+#ifndef M2D_X_NOBLOCKBAR
             __syncthreads();
+#endif
             TICK(tw2); TACC(3, tw1, tw2);
             if (!last) fetch(cx, bufn, 0, t + 1, ahead);
             else if (into_next) fetch(nx, bufn, 0, 0, ahead);
@@ -693,6 +695,10 @@ __device__ __forceinline__ constexpr int fold_state(int m, int qi) {
   return q * 4 + m;
 }
 
+// As in the forward, lanes are never masked: rows outside the grid and cells outside the row work
+// on zero operands.  For the adjoint this means that a row which has not reached its last column
+// yet keeps lambda = mu = 0 exactly, and that a row past column 0 carries finite values that are
+// multiplied by zero coefficients (delta, dy, x are zero there) wherever they meet a sum.
 template <typename T, bool STAGE_X>
 __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParams p) {
   constexpr int CS = 64 >> kHBShift;     // 4 channel slots
@@ -706,8 +712,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   // later, after a barrier that every wave reaches only once it has finished reading it).
   float2* slots = reinterpret_cast<float2*>(smem);                       // [2][wave][3][64]
   float* a_lds = reinterpret_cast<float*>(smem + kBwdWaves * SLOT);      // [wave][CS][2][16], fold order
-  float* zrec = a_lds + kBwdWaves * CS * 2 * kN;                         // 64 zero floats
-  char* lds = reinterpret_cast<char*>(zrec + 64);                        // 2 staging buffers
+  char* lds = reinterpret_cast<char*>(a_lds + kBwdWaves * CS * 2 * kN);  // 2 staging buffers
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lb = logical_block(p.nwg);
@@ -723,7 +728,6 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
     float* mine = a_lds + ch_loc * (2 * kN);
     mine[spos<true>(r)] = p.A2T[e * kN + r];
     mine[kN + spos<true>(r)] = p.A2L[e * kN + r];
-    if (threadIdx.x < 64) zrec[threadIdx.x] = 0.f;
   }
   const uint32_t a_base_off = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) float*)(a_lds + ch_loc * (2 * kN)));
   const float dsk = p.Df[e];
@@ -739,22 +743,52 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   const T* DT = static_cast<const T*>(p.dT);
   const T* DL = static_cast<const T*>(p.dL);
   const T* DY = static_cast<const T*>(p.dy);
-  T* DX = static_cast<T*>(p.dx);
-  T* DDT = static_cast<T*>(p.ddT);
-  T* DDL = static_cast<T*>(p.ddL);
-  const int64_t P = (int64_t)p.B * p.H * p.W;
   const float ninf = -__builtin_huge_valf();
+  const int64_t cell0 = (int64_t)b * p.H * p.W;
+  // (B,H,W,E) tensors: image base (uniform) + 32-bit byte offset (per lane)
+  const int64_t img_bytes = cell0 * p.E * (int64_t)sizeof(T);
+  const char* Ximg = reinterpret_cast<const char*>(X) + img_bytes;
+  const char* DTimg = reinterpret_cast<const char*>(DT) + img_bytes;
+  const char* DLimg = reinterpret_cast<const char*>(DL) + img_bytes;
+  const char* DYimg = reinterpret_cast<const char*>(DY) + img_bytes;
+  char* DXimg = static_cast<char*>(p.dx) + img_bytes;
+  char* DDTimg = static_cast<char*>(p.ddT) + img_bytes;
+  char* DDLimg = static_cast<char*>(p.ddL) + img_bytes;
+  const uint32_t estep = (uint32_t)(p.flip ? -p.E : p.E) * (uint32_t)sizeof(T);   // one column further
+  char* BOTimg = reinterpret_cast<char*>(p.bot + (int64_t)b * p.W * p.E * kN);
+  // per-workgroup channel sums: [channel group][cell][C, B_T, B_L][16]
+  char* PARTimg = reinterpret_cast<char*>(p.part + ((int64_t)eg * p.B * p.H * p.W + cell0) * (3 * kN));
+  const uint32_t pstep = (uint32_t)(p.flip ? -1 : 1) * (uint32_t)(3 * kN * sizeof(float));
 
   float accAT[kN], accAL[kN], accD = 0.f;
   float muT[kN], muL[kN];
 #pragma unroll
   for (int n = 0; n < kN; ++n) { accAT[n] = 0.f; accAL[n] = 0.f; }
 
+  // byte offsets of the lane's operand record inside a staging buffer at step 0 of a block, and
+  // its advance per step: a grid row reads (B_T, B_L, C) of its cell; the upper ghost (lane 0)
+  // reads the row above as its B_T; the lower ghost (lane 15) reads the row of mu_T below as its C.
+  // The neighbouring records that a ghost reads in the other two places are finite and meet zeros.
+  const uint32_t rec_off = r == 0 ? SG::kTOff + ch_loc * kN * 4
+                                  : (r == kHB - 1 ? SG::kOOff + ch_loc * kN * 4 - 2 * kN * 4 : r * SG::kBStride * 4);
+  const uint32_t rec_kstr = (r == 0 || r == kHB - 1) ? SG::kTKStr : SG::kKStr;
+  const uint32_t xd_off = SG::kXOff + (r * SG::kXStride + ch_loc) * (uint32_t)sizeof(T);
+  constexpr uint32_t kXK = kHB * SG::kXStride * sizeof(T);   // XD bytes per step
+  // the sum that this thread adds up in the exchange (one float of one lane's float2, one tensor)
+  const int fid = wave * (2 * SLOT / kBwdWaves) + lane;
+  const bool f_on = lane < 2 * SLOT / kBwdWaves;
+  const int f_it = fid >> 1, f_comp = fid & 1;
+  const int f_r = f_it & (kHB - 1), f_s = (f_it & 63) >> kHBShift, f_v = f_it >> 6;
+
   struct BandCtx {
     BandGeom g;
-    LaneRole ro;
     int T_steps, nb;
-    bool to_bot;
+    bool real, under_way, to_bot, f_real;
+    float oT, oL, cT, cL;        // gate offsets and input coefficients inside the grid
+    float oT0, cT0, cL0;         // the same at column 0
+    float g1, gb1;               // 1 on the upper / lower ghost lane
+    uint32_t cell_off;           // byte offset of (lane row, column -r) in a (H,W,E) image
+    uint32_t f_off;              // byte offset of (exchange row, column -f_r) in the channel-sum image
   };
   auto band_ctx = [&](int band) {
     BandCtx c;
@@ -763,14 +797,29 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
     c.g.has_above = band > 0; c.g.has_below = band + 1 < p.nbands;
     c.T_steps = c.g.has_below ? p.W + kHB - 1 : p.W + c.g.rows;   // the lower ghost trails by 15 steps
     c.nb = (c.T_steps + kCK - 1) / kCK;
-    c.ro.real = ch_ok && r >= 1 && r <= c.g.rows;
-    c.ro.gtop = ch_ok && r == 0 && c.g.has_above;
-    c.ro.gbot = ch_ok && r == kHB - 1 && c.g.has_below;
-    c.ro.first_row = c.g.i0 + r - 1 == 0;
-    c.to_bot = c.ro.real && c.g.has_above && r == 1;
+    c.real = ch_ok && r >= 1 && r <= c.g.rows;
+    const bool first_row = c.g.i0 + r - 1 == 0;
+    const bool gbot = r == kHB - 1 && c.g.has_below;
+    c.under_way = c.real || (ch_ok && r == 0 && c.g.has_above);
+    c.to_bot = c.real && c.g.has_above && r == 1;
+    c.oT = gbot ? 0.f : (!c.real || first_row ? ninf : -1.f);   // lower ghost: open T gate with delta 0, mu_T = lambda
+    c.oL = !c.real ? ninf : (first_row ? 0.f : -1.f);
+    c.cT = !c.real || first_row ? 0.f : 0.5f;
+    c.cL = !c.real ? 0.f : (first_row ? 1.f : 0.5f);
+    c.oT0 = gbot ? 0.f : (!c.real || first_row ? ninf : 0.f);
+    c.cT0 = !c.real || first_row ? 0.f : 1.f;
+    c.cL0 = c.real && first_row ? 1.f : 0.f;
+    c.g1 = r == 0 ? 1.f : 0.f;
+    c.gb1 = gbot ? 1.f : 0.f;
+    const int cellm = (c.g.i0 + r - 1) * p.W - r;   // cell index at t = 0
+    c.cell_off = (uint32_t)((p.flip ? p.H * p.W - 1 - cellm : cellm) * p.E + e) * (uint32_t)sizeof(T);
+    c.f_real = f_on && f_r >= 1 && f_r <= c.g.rows;
+    const int fcell = (c.g.i0 + f_r - 1) * p.W - f_r;
+    c.f_off = (uint32_t)((p.flip ? p.H * p.W - 1 - fcell : fcell) * 3 + f_v) * (uint32_t)(kN * sizeof(float)) +
+              (uint32_t)(f_s * 4 + f_comp) * (uint32_t)sizeof(float);
     return c;
   };
-  const int64_t cell0 = (int64_t)b * p.H * p.W;
+  const uint32_t bot_off = (uint32_t)(-r * p.E + e) * (uint32_t)(kN * sizeof(float));   // column -r of the mu_T row
   // state snapshot at the start of block mm of a band (zero for lanes that were not under way)
   float cknext[kN];
   auto load_ckpt = [&](int bandi, bool under_way, int mm) {
@@ -784,6 +833,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
       for (int n = 0; n < kN; ++n) cknext[n] = ck[n * kHB];
     }
   };
+  auto band_rows = [&](int band) { return p.H - band * kRB < kRB ? p.H - band * kRB : kRB; };
 
   // Bands are swept bottom-up without draining the pipeline: while block 0 of a band runs, the
   // last block of the band above is staged (its lower-ghost row was stored at the start of this
@@ -794,10 +844,14 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   int xpar = 0;   // exchange buffer in use
   for (int band = p.nbands - 1; band >= 0; --band) {
     const bool more = band > 0;
-    const BandCtx nx = band_ctx(more ? band - 1 : band);
+    // what the sweep needs to know of the band above before it gets there
+    BandGeom ng;
+    ng.band = more ? band - 1 : band; ng.i0 = ng.band * kRB; ng.rows = band_rows(ng.band);
+    ng.has_above = ng.band > 0; ng.has_below = ng.band + 1 < p.nbands;
+    const int n_nb = ((ng.has_below ? p.W + kHB - 1 : p.W + ng.rows) + kCK - 1) / kCK;
     const int nb = cx.nb, T_steps = cx.T_steps;
     if (band == p.nbands - 1 || !streamed) {
-      load_ckpt(cx.g.band, cx.ro.real || cx.ro.gtop, nb - 1);
+      load_ckpt(cx.g.band, cx.under_way, nb - 1);
       stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds + cur * SG::kBytes, b, cx.g, (nb - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
       staging_fence();
     }
@@ -807,10 +861,6 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
     for (int m = nb - 1; m >= 0; --m) {
       const int t0 = m * kCK;
       const char* bufc = lds + cur * SG::kBytes;
-      const float* bcb = reinterpret_cast<const float*>(bufc);
-      const T* xdb = reinterpret_cast<const T*>(bufc + SG::kXOff);
-      const float* tpb = reinterpret_cast<const float*>(bufc + SG::kTOff);
-      const float* bob = reinterpret_cast<const float*>(bufc + SG::kOOff);
       float ck0[kN];
 #pragma unroll
       for (int n = 0; n < kN; ++n) ck0[n] = cknext[n];
@@ -819,7 +869,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
       if (m > 0)
         stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, cx.g, t0 - kCK, e_wg0, wave, lane, X, DT, DL, DY);
       else if (into_next)
-        stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, nx.g, (nx.nb - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
+        stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, ng, (n_nb - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
       TICK(ts1); TACC(0, ts0, ts1);
 
       // The 16 states are swept in two halves of 8 (state groups 0,1 then 2,3), each half
@@ -839,37 +889,34 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
         for (int k = 0; k < kCK; ++k) {
           const int t = t0 + k;
           if (t < T_steps) {
-            const int j = t - r;
-            const bool inw = j >= 0 && j < p.W;
-            const bool act = cx.ro.real && inw;
-            const bool gact = cx.ro.gtop && inw;
-            const float offT = (act && !cx.ro.first_row) ? (j == 0 ? 0.f : -1.f) : ninf;
-            const float offL = (act && j != 0) ? (cx.ro.first_row ? 0.f : -1.f) : ninf;
-            const float cT = act ? (cx.ro.first_row ? 0.f : (j == 0 ? 1.f : 0.5f)) : 0.f;
-            const float cL = act ? (cx.ro.first_row ? 1.f : (j == 0 ? 0.f : 0.5f)) : 0.f;
-            float xv, dtv, dlv;
+            const bool col0 = t == r;
+            const float offT = col0 ? cx.oT0 : cx.oT;
+            const float offL = col0 ? ninf : cx.oL;
+            const float cT = col0 ? cx.cT0 : cx.cT;
+            const float cL = col0 ? cx.cL0 : cx.cL;
+            float xv = 0.f, dtv = 0.f, dlv = 0.f;
             if constexpr (STAGE_X) {
-              const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
+              const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
               xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW);
-            } else {
-              const int64_t idx = cell0 + cell_in_image(p, cx.g.i0 + (cx.ro.real ? r - 1 : 0), inw ? j : 0);
-              xv = IO<T>::ld(X + idx * p.E + e); dtv = IO<T>::ld(DT + idx * p.E + e); dlv = IO<T>::ld(DL + idx * p.E + e);
+            } else if (cx.real && (unsigned)(t - r) < (unsigned)p.W) {
+              const uint32_t off = cx.cell_off + (uint32_t)t * estep;
+              xv = IO<T>::ld(reinterpret_cast<const T*>(Ximg + off));
+              dtv = IO<T>::ld(reinterpret_cast<const T*>(DTimg + off));
+              dlv = IO<T>::ld(reinterpret_cast<const T*>(DLimg + off));
             }
-            if (!act) { xv = 0.f; dtv = 0.f; dlv = 0.f; }
             // keep the per-step reads of A in LDS, not in live registers (the offset is hidden from
             // the optimiser; the pointer stays an LDS pointer so that the reads are ds_read)
             uint32_t a_off = a_base_off;
             asm volatile("" : "+v"(a_off));
             const lds_float4* a_mine = (const lds_float4*)(uintptr_t)a_off;
-            const float* pbt = act ? bcb + k * (SG::kKStr / 4) + r * SG::kBStride : (gact ? tpb + k * (SG::kTKStr / 4) + ch_loc * kN : zrec);
-            const float* pbl = act ? pbt + kN : pbt;
-            const float sT = gact ? 1.f : cT * dtv * xv;
+            const char* rec = bufc + (rec_off + k * rec_kstr);
+            const float sT = __builtin_fmaf(cT * dtv, xv, cx.g1);
             const float sL = cL * dlv * xv;
 #pragma unroll
             for (int mgl = 0; mgl < 2; ++mgl) {
               const int mg = 2 * half + mgl;
               const v4f_t at4 = a_mine[mg], al4 = a_mine[kN / 4 + mg];
-              const float4 b4 = reinterpret_cast<const float4*>(pbt)[mg], l4 = reinterpret_cast<const float4*>(pbl)[mg];
+              const float4 b4 = reinterpret_cast<const float4*>(rec)[mg], l4 = reinterpret_cast<const float4*>(rec + kN * 4)[mg];
               const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
               const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w};
 #pragma unroll
@@ -896,38 +943,34 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
           if (half == 1 && k == (kCK > 1 ? 1 : 0)) {
             // one load site for both cases, so that the wait at the start of the next step covers it
             const bool same = m > 0;
+            const bool n_under_way = ch_ok && ((r >= 1 && r <= ng.rows) || (r == 0 && ng.has_above));
             if (same || into_next)
-              load_ckpt(same ? cx.g.band : nx.g.band, same ? (cx.ro.real || cx.ro.gtop) : (nx.ro.real || nx.ro.gtop),
-                        same ? m - 1 : nx.nb - 1);
+              load_ckpt(same ? cx.g.band : ng.band, same ? cx.under_way : n_under_way, same ? m - 1 : n_nb - 1);
           }
           if (t < T_steps) {
-            const int j = t - r;
-            const bool inw = j >= 0 && j < p.W;
-            const bool act = cx.ro.real && inw;
-            const bool gact = cx.ro.gbot && inw;     // ghost of the row below: muT := staged row
-            float offT = (act && !cx.ro.first_row) ? (j == 0 ? 0.f : -1.f) : ninf;
-            const float offL = (act && j != 0) ? (cx.ro.first_row ? 0.f : -1.f) : ninf;
-            const float cT = act ? (cx.ro.first_row ? 0.f : (j == 0 ? 1.f : 0.5f)) : 0.f;
-            const float cL = act ? (cx.ro.first_row ? 1.f : (j == 0 ? 0.f : 0.5f)) : 0.f;
-            if (gact) offT = 0.f;                 // open T gate with delta 0: muT = lambda = staged value
-            float xv, dtv, dlv, dyv;
+            const bool col0 = t == r;
+            const float offT = col0 ? cx.oT0 : cx.oT;
+            const float offL = col0 ? ninf : cx.oL;
+            const float cT = col0 ? cx.cT0 : cx.cT;
+            const float cL = col0 ? cx.cL0 : cx.cL;
+            const bool inr = cx.real && (unsigned)(t - r) < (unsigned)p.W;
+            const uint32_t goff = cx.cell_off + (uint32_t)t * estep;
+            float xv = 0.f, dtv = 0.f, dlv = 0.f, dyv = 0.f;
             if constexpr (STAGE_X) {
-              const T* xr = xdb + (k * kHB + r) * SG::kXStride + ch_loc;
+              const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
               xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW); dyv = IO<T>::ld(xr + 3 * CW);
-            } else {
-              const int64_t idx = cell0 + cell_in_image(p, cx.g.i0 + (cx.ro.real ? r - 1 : 0), inw ? j : 0);
-              xv = IO<T>::ld(X + idx * p.E + e); dtv = IO<T>::ld(DT + idx * p.E + e);
-              dlv = IO<T>::ld(DL + idx * p.E + e); dyv = IO<T>::ld(DY + idx * p.E + e);
+            } else if (inr) {
+              xv = IO<T>::ld(reinterpret_cast<const T*>(Ximg + goff));
+              dtv = IO<T>::ld(reinterpret_cast<const T*>(DTimg + goff));
+              dlv = IO<T>::ld(reinterpret_cast<const T*>(DLimg + goff));
+              dyv = IO<T>::ld(reinterpret_cast<const T*>(DYimg + goff));
             }
-            if (!act) { dtv = 0.f; dlv = 0.f; dyv = gact ? 1.f : 0.f; xv = 0.f; }
             uint32_t a_off = a_base_off;
             asm volatile("" : "+v"(a_off));
             const lds_float4* a_mine = (const lds_float4*)(uintptr_t)a_off;
-            const float* pbt = act ? bcb + k * (SG::kKStr / 4) + r * SG::kBStride : (gact ? bob + k * (SG::kTKStr / 4) + ch_loc * kN : zrec);
-            const float* pbl = act ? pbt + kN : pbt;
-            const float* pcc = act ? pbt + 2 * kN : pbt;
+            const char* rec = bufc + (rec_off + k * rec_kstr);
             const float qT = cT * dtv * xv, qL = cL * dlv * xv;   // zero on lanes that are not grid cells
-            const float qC = act ? dyv : 0.f;
+            const float dyl = dyv + cx.gb1;                        // the lower ghost: lambda = 1 * (row of mu_T below)
             float sT = 0.f, sL = 0.f, zT = 0.f, zL = 0.f;
             if (half == 1) { sT = part4[k][0]; sL = part4[k][1]; zT = part4[k][2]; zL = part4[k][3]; }
             TICK(ta1);
@@ -939,8 +982,8 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
             for (int mgl = 0; mgl < 2; ++mgl) {
               const int mg = 2 * half + mgl;
               const v4f_t at4 = a_mine[mg], al4 = a_mine[kN / 4 + mg];
-              const float4 b4 = reinterpret_cast<const float4*>(pbt)[mg], l4 = reinterpret_cast<const float4*>(pbl)[mg];
-              const float4 c4 = reinterpret_cast<const float4*>(pcc)[mg];
+              const float4 b4 = reinterpret_cast<const float4*>(rec)[mg], l4 = reinterpret_cast<const float4*>(rec + kN * 4)[mg];
+              const float4 c4 = reinterpret_cast<const float4*>(rec + 2 * kN * 4)[mg];
               const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
               const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w}, cq[4] = {c4.x, c4.y, c4.z, c4.w};
               float vC[4], vBT[4], vBL[4];
@@ -951,7 +994,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
                 const float aT = fexp2(__builtin_fmaf(dtv, a2t, offT));
                 const float aL = fexp2(__builtin_fmaf(dlv, a2l, offL));
                 const float mb = from_row_above(muT[n]);
-                const float lam = __builtin_fmaf(dyv, cq[qi], muL[n] + mb);
+                const float lam = __builtin_fmaf(dyl, cq[qi], muL[n] + mb);
                 const float hT = from_row_below(hb[k][s8]);
                 const float mT = aT * lam, mL = aL * lam;
                 muT[n] = mT;
@@ -965,49 +1008,42 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
                 sL = __builtin_fmaf(lam, lq[qi], sL);
                 vBT[qi] = qT * lam;
                 vBL[qi] = qL * lam;
-                vC[qi] = qC * hb[k + 1][s8];
+                vC[qi] = dyv * hb[k + 1][s8];
               }
               sw[mgl] = fold16(fold32(vC[0], vC[1]), fold32(vC[2], vC[3]));
               sw[64 * 2 + mgl] = fold16(fold32(vBT[0], vBT[1]), fold32(vBT[2], vBT[3]));
               sw[128 * 2 + mgl] = fold16(fold32(vBL[0], vBL[1]), fold32(vBL[2], vBL[3]));
             }
-            if (cx.to_bot && act) {   // first row of the band: the band above's lower ghost will replay its muT
-              float* bb = p.bot + (((int64_t)b * p.W + j) * p.E + e) * kN;
+            if (cx.g.has_above) {   // first row of the band: the band above's lower ghost will replay its muT
+              if (cx.to_bot && inr) {
+                char* bb = BOTimg + (bot_off + (uint32_t)t * (uint32_t)(p.E * kN * sizeof(float)));
 #pragma unroll
-              for (int q = 2 * half; q < 2 * half + 2; ++q)   // the two state groups of this half, as of this step
-                reinterpret_cast<float4*>(bb)[q] = make_float4(muT[sinv<PERM>(4 * q)], muT[sinv<PERM>(4 * q + 1)],
-                                                               muT[sinv<PERM>(4 * q + 2)], muT[sinv<PERM>(4 * q + 3)]);
+                for (int q = 2 * half; q < 2 * half + 2; ++q)   // the two state groups of this half, as of this step
+                  reinterpret_cast<float4*>(bb)[q] = make_float4(muT[sinv<PERM>(4 * q)], muT[sinv<PERM>(4 * q + 1)],
+                                                                 muT[sinv<PERM>(4 * q + 2)], muT[sinv<PERM>(4 * q + 3)]);
+              }
             }
             if (half == 0) {
               part4[k][0] = sT; part4[k][1] = sL; part4[k][2] = zT; part4[k][3] = zL;
             } else {
-              if (act) {
-                const int64_t idx = cell0 + cell_in_image(p, cx.g.i0 + r - 1, j);
-                accD = __builtin_fmaf(dyv, xv, accD);
-                IO<T>::st(DDT + idx * p.E + e, __builtin_fmaf(cT * xv, sT, kLn2 * zT));
-                IO<T>::st(DDL + idx * p.E + e, __builtin_fmaf(cL * xv, sL, kLn2 * zL));
-                IO<T>::st(DX + idx * p.E + e, __builtin_fmaf(cT * dtv, sT, __builtin_fmaf(cL * dlv, sL, dyv * dsk)));
+              accD = __builtin_fmaf(dyv, xv, accD);
+              if (inr) {
+                IO<T>::st(reinterpret_cast<T*>(DDTimg + goff), __builtin_fmaf(cT * xv, sT, kLn2 * zT));
+                IO<T>::st(reinterpret_cast<T*>(DDLimg + goff), __builtin_fmaf(cL * xv, sL, kLn2 * zL));
+                IO<T>::st(reinterpret_cast<T*>(DXimg + goff), __builtin_fmaf(cT * dtv, sT, __builtin_fmaf(cL * dlv, sL, dyv * dsk)));
               }
             }
             // ---- across the waves of the workgroup: the per-wave slots (this half's two state
-            // groups) are added in wave order
+            // groups) are added in wave order, one sum per thread, the same share for every wave
             TICK(ta2); TACC(3, ta1, ta2); TACC(2, ta2, ta2);
             __syncthreads();
             TICK(ta3); TACC(4, ta2, ta3);
-            if (lane < 2 * SLOT / kBwdWaves) {   // one sum per thread, the same share for every wave
-              const int fid = wave * (2 * SLOT / kBwdWaves) + lane;
-              const int it = fid >> 1, comp = fid & 1;
-              const int fl = it & 63, v = it >> 6;
-              const int fr = fl & (kHB - 1), fs = fl >> kHBShift;
-              const int fj = t - fr;
-              if (fr >= 1 && fr <= cx.g.rows && fj >= 0 && fj < p.W) {
-                const float* sl = reinterpret_cast<const float*>(slots + xpar * kBwdWaves * SLOT + it) + comp;
-                float s = sl[0];
+            if (cx.f_real && (unsigned)(t - f_r) < (unsigned)p.W) {
+              const float* sl = reinterpret_cast<const float*>(slots + xpar * kBwdWaves * SLOT + f_it) + f_comp;
+              float s = sl[0];
 #pragma unroll
-                for (int w = 1; w < kBwdWaves; ++w) s += sl[2 * w * SLOT];
-                const int64_t cell = cell0 + cell_in_image(p, cx.g.i0 + fr - 1, fj);
-                p.part[(((int64_t)eg * 3 + v) * P + cell) * kN + fs * 4 + 2 * half + comp] = s;
-              }
+              for (int w = 1; w < kBwdWaves; ++w) s += sl[2 * w * SLOT];
+              *reinterpret_cast<float*>(PARTimg + (cx.f_off + (uint32_t)t * pstep + (uint32_t)(2 * half * sizeof(float)))) = s;
             }
             xpar ^= 1;
           }
@@ -1020,7 +1056,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
       TICK(tz1); TACC(5, tz0, tz1);
       cur ^= 1;
     }
-    cx = nx;
+    if (more) cx = band_ctx(band - 1);
   }
 
 #ifdef M2D_X_TIMING
@@ -1094,10 +1130,14 @@ __global__ void m2d_finalize_kernel(const ScanParams p, T* dC, T* dBT, T* dBL, T
   const int64_t nquad = 3 * P * (kN / 4);
   const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (gid < nquad) {
+    // per-workgroup sums are laid out [channel group][cell][C, B_T, B_L][16]
     const int64_t v = gid / (P * 4), rem = gid % (P * 4);
-    float4 s = *reinterpret_cast<const float4*>(p.part + (v * P * kN) + rem * 4);
+    const int64_t cell = rem >> 2;
+    const int q = (int)(rem & 3);
+    const float* src = p.part + (cell * 3 + v) * kN + q * 4;
+    float4 s = *reinterpret_cast<const float4*>(src);
     for (int egi = 1; egi < p.bpb; ++egi) {
-      const float4 o = *reinterpret_cast<const float4*>(p.part + (((int64_t)egi * 3 + v) * P * kN) + rem * 4);
+      const float4 o = *reinterpret_cast<const float4*>(src + (int64_t)egi * P * 3 * kN);
       s.x += o.x; s.y += o.y; s.z += o.z; s.w += o.w;
     }
     T* out = v == 0 ? dC : (v == 1 ? dBT : dBL);
