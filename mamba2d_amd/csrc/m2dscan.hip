@@ -5,25 +5,27 @@
 // with (cT,cL) = (0,1) on the first row, (1,0) on the first column and (1/2,1/2) inside, is
 // independent across (batch, channel, state).
 //
-// Mapping.  The grid rows are cut in bands of HB rows (HB = 16 for most shapes).  A 64-lane
-// wavefront owns CS = 64/HB channel slots of one image: lane = slot*HB + r holds band row r of
-// its channel(s).  At step t the lane works on the cell (row r, column t-r): one step of the
-// wave is one anti-diagonal of the band for CS channels at once.  The 16 states of the cell
-// stay in VGPRs; h[i,j-1] is the lane's own previous value, h[i-1,j] is the previous value of
-// the lane below, fetched with a DPP wave shift; the first row of a band takes it from the
-// last row of the band above, which travels through a small buffer in memory.  y = C.h is a
-// 16-term sum in registers.  Short bands keep the skew waste low (W/(W+HB-1) of the steps do
-// useful work) and put several channels of the same cell in one wave, which the backward
-// needs for its channel sums.
+// Mapping.  The grid rows are cut in bands of 14 rows.  A 64-lane wavefront owns 4 channel slots
+// of one image: lane = slot*16 + r, where lanes r = 1..14 hold band rows, lane 0 a ghost of the
+// row above the band and lane 15 (backward only) a ghost of the row below it.  Every lane walks a
+// "stream" of positions: position s = (band, column) = (s / S, s % S) with a stride S >= W, and at
+// global step t lane r is at position t - r, so one step of the wave is an anti-diagonal of a
+// band for 4 channels at once, and when S = W a lane enters column 0 of the next band on the step
+// after it left the last column of the current one: the pipeline never drains between bands.
+// The 16 states of the cell stay in VGPRs; h[i,j-1] is the lane's own previous value, h[i-1,j] is
+// the previous value of the lane below, fetched with a DPP row shift; the first row of a band
+// takes it from the ghost lane, which replays the last row of the band above out of a small
+// buffer in memory.  y = C.h is a 16-term sum in registers.
 //
 // The factor 1/2 and the first-row/column cases are folded into the gate exponent
-// (exp2(delta*A*log2e + log2 c)) and into the input coefficient: the inner loop is branch-free.
+// (exp2(delta*A*log2e + log2 c)) and into the input coefficient: the inner loop is branch-free,
+// and lanes are never masked (rows and cells outside the grid work on zero operands).
 //
 // Backward (adjoint; reference wf_cuda.cu:108-160 and models/kernels/wavefront_cuda.py:97-139,
 // 176-178, 193-194).  The forward stores the register state every CK steps (one anti-diagonal
-// of the band per checkpoint).  The backward walks bands bottom-up and, inside a band, the
-// blocks of CK steps in reverse: restore the checkpoint, recompute the CK states into
-// registers, then run the adjoint over the block backwards,
+// per checkpoint).  The backward walks the steps in reverse, a block of CK at a time: restore the
+// checkpoint, recompute the CK states into registers, then run the adjoint over the block
+// backwards,
 //     lambda = dy*C + muL(own, previous step) + muT(lane above, previous step)
 //     muT = cT*aT*lambda,  muL = cL*aL*lambda
 // emitting every gradient on the fly.  Channel sums (d_BT, d_BL, d_C) are reduced inside the
@@ -149,7 +151,7 @@ struct ScanParams {
   const float *A2T, *A2L, *Df;      // A*log2(e) and D in fp32, (E,16) / (E)
   const float* zeros;               // 256 bytes of zeros (source for out-of-grid staging chunks)
   void *y, *dx, *ddT, *ddL;
-  float* ckpt;                      // [B][nbands][nblk][E][16][16]  state snapshots
+  float* ckpt;                      // [B][nblk][E][16][16]          state snapshots, one per block of steps
   float* top;                       // [nbands-1][B][W][E][16]       last row of each band (forward states)
   float* bot;                       // [B][W][E][16]                 first-row muT of the band below (adjoint)
   float* part;                      // [G][P][3][16]                 per-workgroup channel sums of d_C, d_BT, d_BL
@@ -157,6 +159,10 @@ struct ScanParams {
   float* pD;                        // [B][E]
   int B, H, W, E;
   int nbands, nblk, bc_stride, flip;
+  int S;                            // stream stride: positions per band (>= W)
+  int T_total;                      // steps of the whole sweep
+  int rows_last;                    // grid rows of the last band
+  uint32_t magicS;                  // floor(2^32 / S)
   int bpb;                          // workgroups per image
   int nwg;                          // total workgroups
 };
@@ -176,6 +182,24 @@ __device__ __forceinline__ int cell_in_image(const ScanParams& p, int i, int j) 
   const int im = p.flip ? p.H - 1 - i : i;
   const int jm = p.flip ? p.W - 1 - j : j;
   return im * p.W + jm;
+}
+
+// Stream position -> (band, column).  s >= -S.  Bands outside [0, nbands) and columns >= W are
+// not on the grid.
+struct Pos { int bnd, col; };
+__device__ __forceinline__ Pos pos_of(const ScanParams& p, int s) {
+  const uint32_t sp = (uint32_t)(s + p.S);
+  uint32_t q = __umulhi(sp, p.magicS);          // q or q-1 of the true quotient for sp < 2^32
+  uint32_t rem = sp - q * (uint32_t)p.S;
+  if (rem >= (uint32_t)p.S) { q += 1; rem -= (uint32_t)p.S; }
+  Pos o; o.bnd = (int)q - 1; o.col = (int)rem;
+  return o;
+}
+__device__ __forceinline__ int band_rows(const ScanParams& p, int bnd) { return bnd == p.nbands - 1 ? p.rows_last : kRB; }
+// cell index inside its image of lane row r of band bnd at column col
+__device__ __forceinline__ int cell_of(const ScanParams& p, int bnd, int r, int col) {
+  const int cell = (bnd * kRB + r - 1) * p.W + col;
+  return p.flip ? p.H * p.W - 1 - cell : cell;
 }
 
 // Position of state n inside a 16-float record.  With PERM the four states that the backward
@@ -244,11 +268,6 @@ __device__ __forceinline__ void lds_fill16(const void* src, char* lds_window) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(base) : "memory", "m0");
 }
 
-struct BandGeom {   // wave-uniform description of the band being swept
-  int band, i0, rows;          // first grid row, number of grid rows (<= kRB)
-  bool has_above, has_below;
-};
-
 // The chunk -> (step, row, part of record) decomposition of the BC and XD regions depends only on
 // the thread.  It is worked out once (divisions by the odd record sizes) and kept as one packed
 // word per wave-wide copy: bits 0-3 row, 4-8 part, 9-10 step, bit 31 set if the chunk carries data.
@@ -288,9 +307,10 @@ struct StagePlan {
   }
 };
 
+// Stages the operands of the block of steps t0 .. t0+kCK-1.
 template <typename T, int NT, int CW, bool WITH_BOT, bool UNI, bool STAGE_X, int NWAVES, bool KEEP>
 __device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan<T, NT, CW, WITH_BOT, UNI, NWAVES, KEEP>& plan, char* buf,
-                                            int b, const BandGeom& g, int t0, int e_wg0, int wave, int lane,
+                                            int b, int t0, int e_wg0, int wave, int lane,
                                             const T* x0, const T* x1, const T* x2, const T* x3) {
   using SG = Stage<T, NT, CW, WITH_BOT, UNI>;
   using PL = StagePlan<T, NT, CW, WITH_BOT, UNI, NWAVES, KEEP>;
@@ -299,19 +319,15 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan
   return;
 #endif
   const int64_t img = (int64_t)b * p.H * p.W;
-  const int hw1 = p.H * p.W - 1;
 #pragma unroll
   for (int i = 0; i < PL::kItB; ++i) {
     const uint32_t w = plan.get_bc(i, wave, lane);
     const int r = w & 15, part = (w >> 4) & 31, k = (w >> 9) & 3;
     if ((int)w < 0) {
-      const int j = t0 + k - r;
+      const Pos q = pos_of(p, t0 + k - r);
       const float* src = p.zeros;
-      if ((unsigned)j < (unsigned)p.W && r >= 1 && r <= g.rows) {   // the packed record holds B_T, B_L, C back to back
-        int cell = (g.i0 + r - 1) * p.W + j;
-        cell = p.flip ? hw1 - cell : cell;
-        src = p.bt + (img + cell) * p.bc_stride + part * 4;
-      }
+      if ((unsigned)q.bnd < (unsigned)p.nbands && q.col < p.W && r >= 1 && r <= band_rows(p, q.bnd))
+        src = p.bt + (img + cell_of(p, q.bnd, r, q.col)) * p.bc_stride + part * 4;   // B_T, B_L, C back to back
       lds_fill16<false>(src, buf + (i * PL::kPer + wave * 64) * 16);
     }
   }
@@ -321,15 +337,13 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan
       const uint32_t w = plan.get_xd(i, wave, lane);
       const int r = w & 15, part = (w >> 4) & 31, k = (w >> 9) & 3;
       if ((int)w < 0) {
-        const int j = t0 + k - r;
+        const Pos q = pos_of(p, t0 + k - r);
         const int tau = part / SG::kCpt, ch = e_wg0 + (part & (SG::kCpt - 1)) * SG::kElem;
         const void* src = p.zeros;
-        if ((unsigned)j < (unsigned)p.W && r >= 1 && r <= g.rows && ch < p.E) {
-          int cell = (g.i0 + r - 1) * p.W + j;
-          cell = p.flip ? hw1 - cell : cell;
+        if ((unsigned)q.bnd < (unsigned)p.nbands && q.col < p.W && r >= 1 && r <= band_rows(p, q.bnd) && ch < p.E) {
           // selected with compares: an indexed pointer table would live in (scratch) memory
           const T* base = tau == 0 ? x0 : (tau == 1 ? x1 : (tau == 2 ? x2 : x3));
-          src = base + (img + cell) * p.E + ch;
+          src = base + (img + cell_of(p, q.bnd, r, q.col)) * p.E + ch;
         }
         lds_fill16<false>(src, buf + SG::kXOff + (i * PL::kPer + wave * 64) * 16);
       }
@@ -337,23 +351,23 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan
   }
   // boundary rows were written earlier in this launch (or by the forward launch): read them
   // past the L1.  One wave-wide copy moves the records of 16 channels at one step.
-  for (int q = wave; q < SG::kTInstr; q += NWAVES) {
-    const int k = q / (CW / 16), sub = q - k * (CW / 16);
+  for (int qi = wave; qi < SG::kTInstr; qi += NWAVES) {
+    const int k = qi / (CW / 16), sub = qi - k * (CW / 16);
     const int ch = e_wg0 + sub * 16 + (lane >> 2);
-    const int j = t0 + k;
+    const Pos q = pos_of(p, t0 + k);                 // the upper ghost is lane 0
     const float* src = p.zeros;
-    if (g.has_above && j >= 0 && j < p.W && ch < p.E)
-      src = p.top + ((((int64_t)(g.band - 1) * p.B + b) * p.W + j) * p.E + ch) * kN + (lane & 3) * 4;
+    if (q.bnd >= 1 && q.bnd < p.nbands && q.col < p.W && ch < p.E)
+      src = p.top + ((((int64_t)(q.bnd - 1) * p.B + b) * p.W + q.col) * p.E + ch) * kN + (lane & 3) * 4;
     lds_fill16<true>(src, buf + SG::kTOff + k * SG::kTKStr + sub * 1024);
   }
   if constexpr (WITH_BOT) {
-    for (int q = wave; q < SG::kTInstr; q += NWAVES) {
-      const int k = q / (CW / 16), sub = q - k * (CW / 16);
+    for (int qi = wave; qi < SG::kTInstr; qi += NWAVES) {
+      const int k = qi / (CW / 16), sub = qi - k * (CW / 16);
       const int ch = e_wg0 + sub * 16 + (lane >> 2);
-      const int j = t0 + k - (kHB - 1);
+      const Pos q = pos_of(p, t0 + k - (kHB - 1));   // the lower ghost is lane 15
       const float* src = p.zeros;
-      if (g.has_below && j >= 0 && j < p.W && ch < p.E)
-        src = p.bot + (((int64_t)b * p.W + j) * p.E + ch) * kN + (lane & 3) * 4;
+      if (q.bnd >= 0 && q.bnd + 1 < p.nbands && q.col < p.W && ch < p.E)
+        src = p.bot + (((int64_t)b * p.W + q.col) * p.E + ch) * kN + (lane & 3) * 4;
       lds_fill16<true>(src, buf + SG::kOOff + k * SG::kTKStr + sub * 1024);
     }
   }
@@ -376,29 +390,55 @@ __device__ __forceinline__ void staging_fence() {
   __syncthreads();
 }
 
-// Per-lane, per-step roles.  Lanes 1..14 of every 16-lane row are grid rows of the band; lane 0
-// is a ghost that replays the last row of the band above (it reads its "B_T" from the TOP record
-// with input coefficient 1 and closed gates, so its state IS that row), lane 15 is the ghost of
-// the first row of the band below for the adjoint.  All of this is operand selection: the inner
-// loops have no boundary cases.
-struct LaneRole {
-  bool real;       // a grid row of this band (and a valid channel)
-  bool gtop;       // ghost of the row above
-  bool gbot;       // ghost of the row below (adjoint only)
-  bool first_row;  // grid row 0
+// Per-lane constants of the band a lane is in.  Lanes 1..14 of every 16-lane row are grid rows;
+// lane 0 is a ghost that replays the last row of the band above (it reads its "B_T" from the TOP
+// record with input coefficient 1 and closed gates, so its state IS that row), lane 15 is the
+// ghost of the first row of the band below for the adjoint (open T gate with delta 0 and dy = 1 on
+// the staged row of mu_T).  All of this is operand selection: the inner loops have no boundary cases.
+struct LaneK {
+  bool real;                   // a grid row of its band (and a valid channel)
+  float oT, oL, cT, cL;        // gate offsets (log2 of the coefficient) and input coefficients inside the grid
+  float oT0, cT0, cL0;         // the same at column 0 (the left gate is closed there)
 };
+template <bool BWD>
+__device__ __forceinline__ LaneK lane_consts(const ScanParams& p, int bnd, int r, bool ch_ok) {
+  const float ninf = -__builtin_huge_valf();
+  const bool in_b = (unsigned)bnd < (unsigned)p.nbands;
+  LaneK c;
+  c.real = ch_ok && in_b && r >= 1 && r <= band_rows(p, bnd);
+  const bool first_row = bnd == 0 && r == 1;
+  const bool gbot = BWD && r == kHB - 1 && in_b && bnd + 1 < p.nbands;
+  c.oT = gbot ? 0.f : (!c.real || first_row ? ninf : -1.f);
+  c.oL = !c.real ? ninf : (first_row ? 0.f : -1.f);
+  c.cT = !c.real || first_row ? 0.f : 0.5f;
+  c.cL = !c.real ? 0.f : (first_row ? 1.f : 0.5f);
+  c.oT0 = gbot ? 0.f : (!c.real || first_row ? ninf : 0.f);
+  c.cT0 = !c.real || first_row ? 0.f : 1.f;
+  c.cL0 = c.real && first_row ? 1.f : 0.f;
+  return c;
+}
+
+// The forward keeps, and the backward restores, the state of a lane at the start of a block only
+// if the lane's previous position was a cell of the grid (the ghost: a cell of the row above).
+__device__ __forceinline__ bool snapshot_lane(const ScanParams& p, Pos at, int r, bool ch_ok) {
+  Pos pv;
+  pv.bnd = at.col >= 1 ? at.bnd : at.bnd - 1;
+  pv.col = at.col >= 1 ? at.col - 1 : p.S - 1;
+  const bool row_ok = r == 0 ? pv.bnd >= 1 : (r <= kRB && r <= band_rows(p, pv.bnd));
+  return ch_ok && (unsigned)pv.bnd < (unsigned)p.nbands && pv.col < p.W && row_ok;
+}
 
 // ------------------------------------------------------------------------------------ forward
-// Lanes are never masked in the forward: a grid row that has not reached column 0 yet, or is past
-// the last column, works on zero operands (its records come from the page of zeros), which keeps
-// its state finite and never reaches a cell of the grid: at column 0 the left gate is closed, and
-// a row past the end only feeds rows that are past the end too.  Only the stores are predicated.
+// Lanes are never masked in the forward: a grid row that is between bands, or a lane that is no
+// grid row, works on zero operands (its records come from the page of zeros), which keeps its
+// state finite and never reaches a cell of the grid: at column 0 the left gate is closed, and
+// what the lane below hands to a cell comes from the cell above it.  Only stores are predicated.
 template <typename T, int EC, bool CKPT, bool WRITE_Y, bool STAGE_X>
 __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParams p) {
   constexpr int CS = 64 >> kHBShift;
   constexpr int CW = kFwdWaves * CS * EC;
   constexpr bool PERM = true;
-  constexpr bool AHEAD = EC == 1;   // operands of step t+1 are fetched from LDS during step t
+  constexpr bool AHEAD = EC == 1 && STAGE_X;   // operands of step t+1 are fetched from LDS during step t
   using SG = Stage<T, 3, CW, false, true>;
   extern __shared__ float4 smem[];
   char* lds = reinterpret_cast<char*>(smem);       // two staging buffers and 256 bytes of slack
@@ -445,43 +485,20 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   const char* DLimg = reinterpret_cast<const char*>(DL) + img_bytes;
   const uint32_t estep = (uint32_t)(p.flip ? -p.E : p.E) * (uint32_t)sizeof(T);   // one column further
 
-  // Everything about a band that the inner loops need: wave-uniform geometry and per-lane constants.
-  struct BandCtx {
-    BandGeom g;
-    int T_steps, nb;
-    bool real, ckpt_lane, to_top;
-    float oT, oL, cT, cL;        // gate offsets (log2 of the coefficient) and input coefficients inside the grid
-    float oT0, cT0, cL0;         // the same at column 0 (the left gate is closed there)
-    float g1;                    // 1 on the ghost lane: its T input coefficient
-    uint32_t cell_off;           // byte offset of (lane row, column -r) in a (H,W,E) image: + t*estep = this step's cell
-    uint32_t top_off;            // byte offset of column -r in the row buffer this band writes for the next one
+  // where the lane is in its stream, and what depends on it
+  Pos at = pos_of(p, -r);
+  LaneK K = lane_consts<false>(p, at.bnd, r, ch_ok);
+  const float g1 = r == 0 ? 1.f : 0.f;             // the ghost's T input coefficient
+  uint32_t cell_off = 0;                           // byte offset of the lane's cell in a (H,W,E) image
+  float* top_ptr = p.top;                          // where lane 14 stores its states for the next band's ghost
+  bool to_top = false;
+  auto enter_band = [&]() {                        // the lane is at (at.bnd, at.col): refresh what depends on the band
+    K = lane_consts<false>(p, at.bnd, r, ch_ok);
+    cell_off = (uint32_t)(cell_of(p, at.bnd, r, at.col) * p.E + e0) * (uint32_t)sizeof(T);
+    to_top = K.real && r == kRB && at.bnd + 1 < p.nbands;
+    if (to_top) top_ptr = p.top + ((((int64_t)at.bnd * p.B + b) * p.W + at.col) * p.E + e0) * kN;
   };
-  auto band_ctx = [&](int band) {
-    BandCtx c;
-    c.g.band = band; c.g.i0 = band * kRB;
-    c.g.rows = p.H - c.g.i0 < kRB ? p.H - c.g.i0 : kRB;
-    c.g.has_above = band > 0; c.g.has_below = band + 1 < p.nbands;
-    c.T_steps = c.g.has_below ? p.W + kHB - 1 : p.W + c.g.rows;   // same step count as the backward
-    c.nb = (c.T_steps + kCK - 1) / kCK;
-    c.real = ch_ok && r >= 1 && r <= c.g.rows;
-    const bool ghost = r == 0;
-    const bool first_row = c.g.i0 + r - 1 == 0;
-    c.ckpt_lane = c.real || (ch_ok && ghost && c.g.has_above);
-    c.to_top = c.real && c.g.has_below && r == kRB;
-    c.oT = !c.real || first_row ? ninf : -1.f;
-    c.oL = !c.real ? ninf : (first_row ? 0.f : -1.f);
-    c.cT = !c.real || first_row ? 0.f : 0.5f;
-    c.cL = !c.real ? 0.f : (first_row ? 1.f : 0.5f);
-    c.oT0 = !c.real || first_row ? ninf : 0.f;
-    c.cT0 = !c.real || first_row ? 0.f : 1.f;
-    c.cL0 = c.real && first_row ? 1.f : 0.f;
-    c.g1 = ghost ? 1.f : 0.f;
-    const int row = c.g.i0 + r - 1;
-    const int cellm = row * p.W - r;                                   // cell index at t = 0
-    c.cell_off = (uint32_t)((p.flip ? p.H * p.W - 1 - cellm : cellm) * p.E + e0) * (uint32_t)sizeof(T);
-    c.top_off = (uint32_t)(-r * p.E + e0) * (uint32_t)(kN * sizeof(float));
-    return c;
-  };
+  enter_band();
 
   // byte offsets of the lane's records inside a staging buffer (step 0)
   const uint32_t rec_off = r == 0 ? SG::kTOff + ch_loc * kN * 4 : r * SG::kBStride * 4;
@@ -495,21 +512,19 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
     float xv[EC], dtv[EC], dlv[EC];
     float4 bt[EC][4], bl[4], cc[4];
   };
-  auto fetch = [&](const BandCtx& cx, const char* bufc, int k, int t, Ops& o) {
+  auto fetch = [&](const char* bufc, int k, Ops& o) {
     if constexpr (STAGE_X) {
       const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
       IO<T>::template ldv<EC>(xr, o.xv);
       IO<T>::template ldv<EC>(xr + CW, o.dtv);
       IO<T>::template ldv<EC>(xr + 2 * CW, o.dlv);
-    } else {
-      const bool inr = cx.real && (unsigned)(t - r) < (unsigned)p.W;
+    } else {   // straight from memory, for the lane's current position
 #pragma unroll
       for (int c = 0; c < EC; ++c) { o.xv[c] = 0.f; o.dtv[c] = 0.f; o.dlv[c] = 0.f; }
-      if (inr) {
-        const uint32_t off = cx.cell_off + (uint32_t)t * estep;
-        IO<T>::template ldv<EC>(reinterpret_cast<const T*>(Ximg + off), o.xv);
-        IO<T>::template ldv<EC>(reinterpret_cast<const T*>(DTimg + off), o.dtv);
-        IO<T>::template ldv<EC>(reinterpret_cast<const T*>(DLimg + off), o.dlv);
+      if (K.real && at.col < p.W) {
+        IO<T>::template ldv<EC>(reinterpret_cast<const T*>(Ximg + cell_off), o.xv);
+        IO<T>::template ldv<EC>(reinterpret_cast<const T*>(DTimg + cell_off), o.dtv);
+        IO<T>::template ldv<EC>(reinterpret_cast<const T*>(DLimg + cell_off), o.dlv);
       }
     }
     // a grid row reads B_T, B_L, C of its cell; the ghost reads the row above as its B_T (and
@@ -527,17 +542,22 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   };
 
   float h[EC][kN];
-  auto step = [&](const BandCtx& cx, int t, const Ops& o) {
-    const bool col0 = t == r;
-    const float offT = col0 ? cx.oT0 : cx.oT;
-    const float offL = col0 ? ninf : cx.oL;
-    const float cT = col0 ? cx.cT0 : cx.cT;
-    const float cL = col0 ? cx.cL0 : cx.cL;
-    const bool inr = cx.real && (unsigned)(t - r) < (unsigned)p.W;
+#pragma unroll
+  for (int c = 0; c < EC; ++c)
+#pragma unroll
+    for (int n = 0; n < kN; ++n) h[c][n] = 0.f;
+
+  auto step = [&](const Ops& o) {
+    const bool col0 = at.col == 0;
+    const float offT = col0 ? K.oT0 : K.oT;
+    const float offL = col0 ? ninf : K.oL;
+    const float cT = col0 ? K.cT0 : K.cT;
+    const float cL = col0 ? K.cL0 : K.cL;
+    const bool inr = K.real && at.col < p.W;   // K.real is false outside the bands of the grid
     float yv[EC];
 #pragma unroll
     for (int c = 0; c < EC; ++c) {
-      const float sT = __builtin_fmaf(cT * o.dtv[c], o.xv[c], cx.g1);
+      const float sT = __builtin_fmaf(cT * o.dtv[c], o.xv[c], g1);
       const float sL = cL * o.dlv[c] * o.xv[c];
       float acc = 0.f;
 #pragma unroll
@@ -560,119 +580,95 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
       }
       yv[c] = __builtin_fmaf(o.xv[c], dsk[c], acc);
     }
-    if (cx.g.has_below) {   // last row of the band: the next band's ghost will replay it
-      if (cx.to_top && inr) {
-        char* tw = reinterpret_cast<char*>(p.top + ((int64_t)cx.g.band * p.B + b) * p.W * p.E * kN) +
-                   (cx.top_off + (uint32_t)t * (uint32_t)(p.E * kN * sizeof(float)));
+    if (p.nbands > 1) {   // last row of a band: the next band's ghost will replay it
+      if (to_top && inr) {
 #pragma unroll
         for (int c = 0; c < EC; ++c)
 #pragma unroll
           for (int q = 0; q < 4; ++q)
-            reinterpret_cast<float4*>(tw)[c * 4 + q] = make_float4(h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)],
-                                                                   h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
+            reinterpret_cast<float4*>(top_ptr)[c * 4 + q] = make_float4(h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)],
+                                                                        h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
+      }
+      top_ptr += p.E * kN;
+    }
+    if (WRITE_Y && inr) IO<T>::template stv<EC>(reinterpret_cast<T*>(Yimg + cell_off), yv);
+    // one position further; a lane that leaves its band enters column 0 of the next one
+    at.col += 1;
+    cell_off += estep;
+    if (__any(at.col == p.S)) {
+      if (at.col == p.S) {
+        at.col = 0;
+        at.bnd += 1;
+        enter_band();
       }
     }
-    if (WRITE_Y && inr)
-      IO<T>::template stv<EC>(reinterpret_cast<T*>(Yimg + (cx.cell_off + (uint32_t)t * estep)), yv);
   };
 
-  // The bands of the image are swept one after the other without draining the pipeline: while
-  // the last block of a band runs, the first block of the next band is staged.  The rows of
-  // the band above that this needs (columns 0..kCK-1) were stored at steps 14..14+kCK-1 of the
-  // band and completed (vmcnt 0) before a block-end barrier, long before; they are read back
-  // past the L1.  Grids narrower than 8 columns, where that does not hold, restart per band.
-  const bool streamed = p.W >= 8;
-  BandCtx cx = band_ctx(0);
+  stage_block<T, 3, CW, false, true, STAGE_X, kFwdWaves, true>(p, plan, lds, b, 0, e_wg0, wave, lane, X, DT, DL, DY);
+  staging_fence();
   Ops opsA, opsB;
+  if constexpr (AHEAD) fetch(lds, 0, opsA);
   int cur = 0;
-  for (int band = 0; band < p.nbands; ++band) {
-    const bool more = band + 1 < p.nbands;
-    const BandCtx nx = band_ctx(more ? band + 1 : band);
-    if (band == 0 || !streamed) {
-      TICK(tb0);
-      stage_block<T, 3, CW, false, true, STAGE_X, kFwdWaves, true>(p, plan, lds + cur * SG::kBytes, b, cx.g, 0, e_wg0, wave, lane, X, DT, DL, DY);
-      staging_fence();
-      TICK(tb1); TACC(0, tb0, tb1);
-      if constexpr (AHEAD) fetch(cx, lds + cur * SG::kBytes, 0, 0, opsA);
+  for (int m = 0; m < p.nblk; ++m) {
+    const int t0 = m * kCK;
+    const bool last = m + 1 == p.nblk;
+    TICK(ts0);
+    if (!last)
+      stage_block<T, 3, CW, false, true, STAGE_X, kFwdWaves, true>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, t0 + kCK, e_wg0, wave, lane, X, DT, DL, DY);
+    TICK(ts1); TACC(1, ts0, ts1);
+    // snapshot of the state before the block (after step t0-1) for the lanes whose previous
+    // position was a cell of the grid; the others hold nothing the backward needs
+    if (CKPT && m > 0 && snapshot_lane(p, at, r, ch_ok)) {
+      float* ck = p.ckpt + ((((int64_t)b * p.nblk + m) * p.E + e0) * kN) * kHB + r;
+#pragma unroll
+      for (int c = 0; c < EC; ++c)
+#pragma unroll
+        for (int n = 0; n < kN; ++n) ck[(c * kN + n) * kHB] = h[c][n];
     }
+    const char* bufc = lds + cur * SG::kBytes;
+    const char* bufn = lds + (cur ^ 1) * SG::kBytes;
+    if constexpr (AHEAD) {
+      static_assert(kCK % 2 == 0, "the two operand sets alternate and must close over a block");
 #pragma unroll
-    for (int c = 0; c < EC; ++c)
-#pragma unroll
-      for (int n = 0; n < kN; ++n) h[c][n] = 0.f;
-    const int nb = cx.nb, T_steps = cx.T_steps;
-
-    for (int m = 0; m < nb; ++m) {
-      const int t0 = m * kCK;
-      const bool last = m + 1 == nb;
-      const bool into_next = last && more && streamed;
-      TICK(ts0);
-      if (!last)
-        stage_block<T, 3, CW, false, true, STAGE_X, kFwdWaves, true>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, cx.g, t0 + kCK, e_wg0, wave, lane, X, DT, DL, DY);
-      else if (into_next)
-        stage_block<T, 3, CW, false, true, STAGE_X, kFwdWaves, true>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, nx.g, 0, e_wg0, wave, lane, X, DT, DL, DY);
-      TICK(ts1); TACC(1, ts0, ts1);
-      // snapshot of the state before the block (after step t0-1); lanes that have not started or
-      // are past the last column hold nothing the backward needs
-      if (CKPT && m > 0 && cx.ckpt_lane && t0 - 1 - r >= 0 && t0 - 1 - r < p.W) {
-        float* ck = p.ckpt + (((((int64_t)b * p.nbands + band) * p.nblk + m) * p.E + e0) * kN) * kHB + r;
-#pragma unroll
-        for (int c = 0; c < EC; ++c)
-#pragma unroll
-          for (int n = 0; n < kN; ++n) ck[(c * kN + n) * kHB] = h[c][n];
-      }
-      const char* bufc = lds + cur * SG::kBytes;
-      const char* bufn = lds + (cur ^ 1) * SG::kBytes;
-      if constexpr (AHEAD) {
-        static_assert(kCK % 2 == 0, "the two operand sets alternate and must close over a block");
-#pragma unroll
-        for (int k = 0; k < kCK; ++k) {
-          const int t = t0 + k;
-          Ops& now = (k & 1) ? opsB : opsA;
-          Ops& ahead = (k & 1) ? opsA : opsB;
-          if (k + 1 < kCK) {
-            fetch(cx, bufc, k + 1, t + 1, ahead);
-          } else {
-            // Last step of the block: its operands are in registers already, so the buffer can be
-            // handed over now.  The copies of the next block have landed in every wave after this
-            // barrier, and no wave reads the current buffer any more.
-            TICK(tw0);
-            staging_landed();
-            TICK(tw1); TACC(2, tw0, tw1);
+      for (int k = 0; k < kCK; ++k) {
+        const int t = t0 + k;
+        Ops& now = (k & 1) ? opsB : opsA;
+        Ops& ahead = (k & 1) ? opsA : opsB;
+        if (k + 1 < kCK) {
+          fetch(bufc, k + 1, ahead);
+        } else {
+          // Last step of the block: its operands are in registers already, so the buffer can be
+          // handed over now.  The copies of the next block have landed in every wave after this
+          // barrier, and no wave reads the current buffer any more.
+          TICK(tw0);
+          staging_landed();
+          TICK(tw1); TACC(2, tw0, tw1);
 #ifndef M2D_X_NOBLOCKBAR
-            __syncthreads();
+          __syncthreads();
 #endif
-            TICK(tw2); TACC(3, tw1, tw2);
-            if (!last) fetch(cx, bufn, 0, t + 1, ahead);
-            else if (into_next) fetch(nx, bufn, 0, 0, ahead);
-          }
-          TICK(tc0);
-          if (t < T_steps) step(cx, t, now);
-          TICK(tc1); TACC(4, tc0, tc1);
+          TICK(tw2); TACC(3, tw1, tw2);
+          if (!last) fetch(bufn, 0, ahead);
         }
-      } else {
+        TICK(tc0);
+        if (t < p.T_total) step(now);
+        TICK(tc1); TACC(4, tc0, tc1);
+      }
+    } else {
 #pragma unroll
-        for (int k = 0; k < kCK; ++k) {
-          const int t = t0 + k;
-          // The operands of the next block must have landed before the barrier that ends this
-          // block.  Waiting here, before the stores of the last step are issued, keeps the latency
-          // of those stores off the critical path (the counter covers loads and stores alike).
-          if (k == kCK - 1) staging_landed();
-          if (t < T_steps) {
-            fetch(cx, bufc, k, t, opsA);
-            step(cx, t, opsA);
-          }
+      for (int k = 0; k < kCK; ++k) {
+        const int t = t0 + k;
+        // The operands of the next block must have landed before the barrier that ends this
+        // block.  Waiting here, before the stores of the last step are issued, keeps the latency
+        // of those stores off the critical path (the counter covers loads and stores alike).
+        if (k == kCK - 1) staging_landed();
+        if (t < p.T_total) {
+          fetch(bufc, k, opsA);
+          step(opsA);
         }
       }
-      // restart per band: the band's last row is read back by the next band's first staging
-      if (last && more && !streamed) {
-        __threadfence();
-        __syncthreads();
-      } else if constexpr (!AHEAD) {
-        __syncthreads();
-      }
-      cur ^= 1;
+      __syncthreads();
     }
-    cx = nx;
+    cur ^= 1;
   }
 #ifdef M2D_X_TIMING
   if (lane == 0 && blockIdx.x < 512) {
@@ -754,16 +750,14 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   char* DXimg = static_cast<char*>(p.dx) + img_bytes;
   char* DDTimg = static_cast<char*>(p.ddT) + img_bytes;
   char* DDLimg = static_cast<char*>(p.ddL) + img_bytes;
-  const uint32_t estep = (uint32_t)(p.flip ? -p.E : p.E) * (uint32_t)sizeof(T);   // one column further
   char* BOTimg = reinterpret_cast<char*>(p.bot + (int64_t)b * p.W * p.E * kN);
   // per-workgroup channel sums: [channel group][cell][C, B_T, B_L][16]
   char* PARTimg = reinterpret_cast<char*>(p.part + ((int64_t)eg * p.B * p.H * p.W + cell0) * (3 * kN));
-  const uint32_t pstep = (uint32_t)(p.flip ? -1 : 1) * (uint32_t)(3 * kN * sizeof(float));
 
   float accAT[kN], accAL[kN], accD = 0.f;
   float muT[kN], muL[kN];
 #pragma unroll
-  for (int n = 0; n < kN; ++n) { accAT[n] = 0.f; accAL[n] = 0.f; }
+  for (int n = 0; n < kN; ++n) { accAT[n] = 0.f; accAL[n] = 0.f; muT[n] = 0.f; muL[n] = 0.f; }
 
   // byte offsets of the lane's operand record inside a staging buffer at step 0 of a block, and
   // its advance per step: a grid row reads (B_T, B_L, C) of its cell; the upper ghost (lane 0)
@@ -774,289 +768,260 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   const uint32_t rec_kstr = (r == 0 || r == kHB - 1) ? SG::kTKStr : SG::kKStr;
   const uint32_t xd_off = SG::kXOff + (r * SG::kXStride + ch_loc) * (uint32_t)sizeof(T);
   constexpr uint32_t kXK = kHB * SG::kXStride * sizeof(T);   // XD bytes per step
-  // the sum that this thread adds up in the exchange (one float of one lane's float2, one tensor)
+  // the sum that this thread adds up in the exchange (one float of one lane's float2, one tensor):
+  // it belongs to lane row f_r, which is f_d positions ahead of this thread's own row
   const int fid = wave * (2 * SLOT / kBwdWaves) + lane;
   const bool f_on = lane < 2 * SLOT / kBwdWaves;
   const int f_it = fid >> 1, f_comp = fid & 1;
   const int f_r = f_it & (kHB - 1), f_s = (f_it & 63) >> kHBShift, f_v = f_it >> 6;
+  const int f_d = r - f_r;
+  const uint32_t f_sub = (uint32_t)(f_v * kN + f_s * 4 + f_comp) * (uint32_t)sizeof(float);
+  const float g1 = r == 0 ? 1.f : 0.f;
 
-  struct BandCtx {
-    BandGeom g;
-    int T_steps, nb;
-    bool real, under_way, to_bot, f_real;
-    float oT, oL, cT, cL;        // gate offsets and input coefficients inside the grid
-    float oT0, cT0, cL0;         // the same at column 0
-    float g1, gb1;               // 1 on the upper / lower ghost lane
-    uint32_t cell_off;           // byte offset of (lane row, column -r) in a (H,W,E) image
-    uint32_t f_off;              // byte offset of (exchange row, column -f_r) in the channel-sum image
+  // Where the lane is in its stream and the constants of its band; both follow the lane as it
+  // walks forward through a block (recompute) and back (adjoint).
+  Pos at = pos_of(p, (p.nblk - 1) * kCK - r);
+  LaneK K = lane_consts<true>(p, at.bnd, r, ch_ok);
+  float gb1 = 0.f;                        // 1 on an active lower ghost: lambda = 1 * (row of mu_T below)
+  auto enter_band = [&]() {
+    K = lane_consts<true>(p, at.bnd, r, ch_ok);
+    gb1 = (r == kHB - 1 && at.bnd >= 0 && at.bnd + 1 < p.nbands) ? 1.f : 0.f;
   };
-  auto band_ctx = [&](int band) {
-    BandCtx c;
-    c.g.band = band; c.g.i0 = band * kRB;
-    c.g.rows = p.H - c.g.i0 < kRB ? p.H - c.g.i0 : kRB;
-    c.g.has_above = band > 0; c.g.has_below = band + 1 < p.nbands;
-    c.T_steps = c.g.has_below ? p.W + kHB - 1 : p.W + c.g.rows;   // the lower ghost trails by 15 steps
-    c.nb = (c.T_steps + kCK - 1) / kCK;
-    c.real = ch_ok && r >= 1 && r <= c.g.rows;
-    const bool first_row = c.g.i0 + r - 1 == 0;
-    const bool gbot = r == kHB - 1 && c.g.has_below;
-    c.under_way = c.real || (ch_ok && r == 0 && c.g.has_above);
-    c.to_bot = c.real && c.g.has_above && r == 1;
-    c.oT = gbot ? 0.f : (!c.real || first_row ? ninf : -1.f);   // lower ghost: open T gate with delta 0, mu_T = lambda
-    c.oL = !c.real ? ninf : (first_row ? 0.f : -1.f);
-    c.cT = !c.real || first_row ? 0.f : 0.5f;
-    c.cL = !c.real ? 0.f : (first_row ? 1.f : 0.5f);
-    c.oT0 = gbot ? 0.f : (!c.real || first_row ? ninf : 0.f);
-    c.cT0 = !c.real || first_row ? 0.f : 1.f;
-    c.cL0 = c.real && first_row ? 1.f : 0.f;
-    c.g1 = r == 0 ? 1.f : 0.f;
-    c.gb1 = gbot ? 1.f : 0.f;
-    const int cellm = (c.g.i0 + r - 1) * p.W - r;   // cell index at t = 0
-    c.cell_off = (uint32_t)((p.flip ? p.H * p.W - 1 - cellm : cellm) * p.E + e) * (uint32_t)sizeof(T);
-    c.f_real = f_on && f_r >= 1 && f_r <= c.g.rows;
-    const int fcell = (c.g.i0 + f_r - 1) * p.W - f_r;
-    c.f_off = (uint32_t)((p.flip ? p.H * p.W - 1 - fcell : fcell) * 3 + f_v) * (uint32_t)(kN * sizeof(float)) +
-              (uint32_t)(f_s * 4 + f_comp) * (uint32_t)sizeof(float);
-    return c;
+  enter_band();
+  auto advance = [&]() {
+    at.col += 1;
+    if (__any(at.col == p.S)) {
+      if (at.col == p.S) { at.col = 0; at.bnd += 1; enter_band(); }
+    }
   };
-  const uint32_t bot_off = (uint32_t)(-r * p.E + e) * (uint32_t)(kN * sizeof(float));   // column -r of the mu_T row
-  // state snapshot at the start of block mm of a band (zero for lanes that were not under way)
+  auto retreat = [&](int n) {
+    at.col -= n;
+    if (__any(at.col < 0)) {
+      if (at.col < 0) { at.col += p.S; at.bnd -= 1; enter_band(); }
+    }
+  };
+  auto cell_bytes = [&]() {   // byte offset of the lane's cell in a (H,W,E) image
+    return (uint32_t)(cell_of(p, at.bnd, r, at.col) * p.E + e) * (uint32_t)sizeof(T);
+  };
+
+  // state snapshot at the start of block mm (zero for lanes that were not under way)
   float cknext[kN];
-  auto load_ckpt = [&](int bandi, bool under_way, int mm) {
-    const int tt = mm * kCK;
-    if (mm == 0 || !(under_way && tt - 1 - r >= 0 && tt - 1 - r < p.W)) {
+  auto load_ckpt = [&](int mm) {
+    const Pos q = pos_of(p, mm * kCK - r);
+    if (mm == 0 || !snapshot_lane(p, q, r, ch_ok)) {
 #pragma unroll
       for (int n = 0; n < kN; ++n) cknext[n] = 0.f;
     } else {
-      const float* ck = p.ckpt + (((((int64_t)b * p.nbands + bandi) * p.nblk + mm) * p.E + e) * kN) * kHB + r;
+      const float* ck = p.ckpt + ((((int64_t)b * p.nblk + mm) * p.E + e) * kN) * kHB + r;
 #pragma unroll
       for (int n = 0; n < kN; ++n) cknext[n] = ck[n * kHB];
     }
   };
-  auto band_rows = [&](int band) { return p.H - band * kRB < kRB ? p.H - band * kRB : kRB; };
 
-  // Bands are swept bottom-up without draining the pipeline: while block 0 of a band runs, the
-  // last block of the band above is staged (its lower-ghost row was stored at the start of this
-  // band's sweep) and its snapshot fetched.  Grids narrower than 8 columns restart per band.
-  const bool streamed = p.W >= 8;
-  BandCtx cx = band_ctx(p.nbands - 1);
+  load_ckpt(p.nblk - 1);
+  stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds, b, (p.nblk - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
+  staging_fence();
   int cur = 0;
   int xpar = 0;   // exchange buffer in use
-  for (int band = p.nbands - 1; band >= 0; --band) {
-    const bool more = band > 0;
-    // what the sweep needs to know of the band above before it gets there
-    BandGeom ng;
-    ng.band = more ? band - 1 : band; ng.i0 = ng.band * kRB; ng.rows = band_rows(ng.band);
-    ng.has_above = ng.band > 0; ng.has_below = ng.band + 1 < p.nbands;
-    const int n_nb = ((ng.has_below ? p.W + kHB - 1 : p.W + ng.rows) + kCK - 1) / kCK;
-    const int nb = cx.nb, T_steps = cx.T_steps;
-    if (band == p.nbands - 1 || !streamed) {
-      load_ckpt(cx.g.band, cx.under_way, nb - 1);
-      stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds + cur * SG::kBytes, b, cx.g, (nb - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
-      staging_fence();
-    }
-#pragma unroll
-    for (int n = 0; n < kN; ++n) { muT[n] = 0.f; muL[n] = 0.f; }
 
-    for (int m = nb - 1; m >= 0; --m) {
-      const int t0 = m * kCK;
-      const char* bufc = lds + cur * SG::kBytes;
-      float ck0[kN];
+  for (int m = p.nblk - 1; m >= 0; --m) {
+    const int t0 = m * kCK;
+    const char* bufc = lds + cur * SG::kBytes;
+    float ck0[kN];
 #pragma unroll
-      for (int n = 0; n < kN; ++n) ck0[n] = cknext[n];
-      const bool into_next = m == 0 && more && streamed;
-      TICK(ts0);
-      if (m > 0)
-        stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, cx.g, t0 - kCK, e_wg0, wave, lane, X, DT, DL, DY);
-      else if (into_next)
-        stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, ng, (n_nb - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
-      TICK(ts1); TACC(0, ts0, ts1);
+    for (int n = 0; n < kN; ++n) ck0[n] = cknext[n];
+    TICK(ts0);
+    if (m > 0)
+      stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, t0 - kCK, e_wg0, wave, lane, X, DT, DL, DY);
+    TICK(ts1); TACC(0, ts0, ts1);
 
-      // The 16 states are swept in two halves of 8 (state groups 0,1 then 2,3), each half
-      // recomputing and then back-propagating the whole block: only 5 x 8 recomputed states are
-      // live at a time.  The state sums of the first half wait in `part4` for the second.
-      float part4[kCK][4];
+    // The 16 states are swept in two halves of 8 (state groups 0,1 then 2,3), each half
+    // recomputing and then back-propagating the whole block: only 5 x 8 recomputed states are
+    // live at a time.  The state sums of the first half wait in `part4` for the second.
+    float part4[kCK][4];
 #pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        float hb[kCK + 1][8];
+    for (int half = 0; half < 2; ++half) {
+      float hb[kCK + 1][8];
 #pragma unroll
-        for (int mgl = 0; mgl < 2; ++mgl)
+      for (int mgl = 0; mgl < 2; ++mgl)
 #pragma unroll
-          for (int qi = 0; qi < 4; ++qi) hb[0][4 * mgl + qi] = ck0[fold_state(2 * half + mgl, qi)];
-        // ---- recompute the states of the block
-        TICK(tr0);
+        for (int qi = 0; qi < 4; ++qi) hb[0][4 * mgl + qi] = ck0[fold_state(2 * half + mgl, qi)];
+      // ---- recompute the states of the block (the lane is at its position of step t0)
+      TICK(tr0);
 #pragma unroll
-        for (int k = 0; k < kCK; ++k) {
-          const int t = t0 + k;
-          if (t < T_steps) {
-            const bool col0 = t == r;
-            const float offT = col0 ? cx.oT0 : cx.oT;
-            const float offL = col0 ? ninf : cx.oL;
-            const float cT = col0 ? cx.cT0 : cx.cT;
-            const float cL = col0 ? cx.cL0 : cx.cL;
-            float xv = 0.f, dtv = 0.f, dlv = 0.f;
-            if constexpr (STAGE_X) {
-              const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
-              xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW);
-            } else if (cx.real && (unsigned)(t - r) < (unsigned)p.W) {
-              const uint32_t off = cx.cell_off + (uint32_t)t * estep;
-              xv = IO<T>::ld(reinterpret_cast<const T*>(Ximg + off));
-              dtv = IO<T>::ld(reinterpret_cast<const T*>(DTimg + off));
-              dlv = IO<T>::ld(reinterpret_cast<const T*>(DLimg + off));
-            }
-            // keep the per-step reads of A in LDS, not in live registers (the offset is hidden from
-            // the optimiser; the pointer stays an LDS pointer so that the reads are ds_read)
-            uint32_t a_off = a_base_off;
-            asm volatile("" : "+v"(a_off));
-            const lds_float4* a_mine = (const lds_float4*)(uintptr_t)a_off;
-            const char* rec = bufc + (rec_off + k * rec_kstr);
-            const float sT = __builtin_fmaf(cT * dtv, xv, cx.g1);
-            const float sL = cL * dlv * xv;
+      for (int k = 0; k < kCK; ++k) {
+        const int t = t0 + k;
+        if (t < p.T_total) {
+          const bool col0 = at.col == 0;
+          const float offT = col0 ? K.oT0 : K.oT;
+          const float offL = col0 ? ninf : K.oL;
+          const float cT = col0 ? K.cT0 : K.cT;
+          const float cL = col0 ? K.cL0 : K.cL;
+          float xv = 0.f, dtv = 0.f, dlv = 0.f;
+          if constexpr (STAGE_X) {
+            const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
+            xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW);
+          } else if (K.real && at.col < p.W) {
+            const uint32_t off = cell_bytes();
+            xv = IO<T>::ld(reinterpret_cast<const T*>(Ximg + off));
+            dtv = IO<T>::ld(reinterpret_cast<const T*>(DTimg + off));
+            dlv = IO<T>::ld(reinterpret_cast<const T*>(DLimg + off));
+          }
+          // keep the per-step reads of A in LDS, not in live registers (the offset is hidden from
+          // the optimiser; the pointer stays an LDS pointer so that the reads are ds_read)
+          uint32_t a_off = a_base_off;
+          asm volatile("" : "+v"(a_off));
+          const lds_float4* a_mine = (const lds_float4*)(uintptr_t)a_off;
+          const char* rec = bufc + (rec_off + k * rec_kstr);
+          const float sT = __builtin_fmaf(cT * dtv, xv, g1);
+          const float sL = cL * dlv * xv;
 #pragma unroll
-            for (int mgl = 0; mgl < 2; ++mgl) {
-              const int mg = 2 * half + mgl;
-              const v4f_t at4 = a_mine[mg], al4 = a_mine[kN / 4 + mg];
-              const float4 b4 = reinterpret_cast<const float4*>(rec)[mg], l4 = reinterpret_cast<const float4*>(rec + kN * 4)[mg];
-              const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
-              const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w};
+          for (int mgl = 0; mgl < 2; ++mgl) {
+            const int mg = 2 * half + mgl;
+            const v4f_t at4 = a_mine[mg], al4 = a_mine[kN / 4 + mg];
+            const float4 b4 = reinterpret_cast<const float4*>(rec)[mg], l4 = reinterpret_cast<const float4*>(rec + kN * 4)[mg];
+            const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
+            const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w};
 #pragma unroll
-              for (int qi = 0; qi < 4; ++qi) {
-                const int s8 = 4 * mgl + qi;
-                const float aT = fexp2(__builtin_fmaf(dtv, atq[qi], offT));
-                const float aL = fexp2(__builtin_fmaf(dlv, alq[qi], offL));
-                const float hT = from_row_below(hb[k][s8]);
-                float u = sL * lq[qi];
-                u = __builtin_fmaf(sT, bq[qi], u);
-                u = __builtin_fmaf(aT, hT, u);
-                hb[k + 1][s8] = __builtin_fmaf(aL, hb[k][s8], u);
-              }
+            for (int qi = 0; qi < 4; ++qi) {
+              const int s8 = 4 * mgl + qi;
+              const float aT = fexp2(__builtin_fmaf(dtv, atq[qi], offT));
+              const float aL = fexp2(__builtin_fmaf(dlv, alq[qi], offL));
+              const float hT = from_row_below(hb[k][s8]);
+              float u = sL * lq[qi];
+              u = __builtin_fmaf(sT, bq[qi], u);
+              u = __builtin_fmaf(aT, hT, u);
+              hb[k + 1][s8] = __builtin_fmaf(aL, hb[k][s8], u);
             }
           }
         }
-        TICK(tr1); TACC(1, tr0, tr1);
-        // ---- adjoint over the block, last step first
+        advance();
+      }
+      TICK(tr1); TACC(1, tr0, tr1);
+      // ---- adjoint over the block, last step first (the lane is one position past the block)
 #pragma unroll
-        for (int k = kCK - 1; k >= 0; --k) {
-          const int t = t0 + k;
-          if (half == 1 && k == 0) staging_landed();   // before the last stores of the block, see the forward kernel
-          // the states of the later steps are dead by now: their registers take the next snapshot
-          if (half == 1 && k == (kCK > 1 ? 1 : 0)) {
-            // one load site for both cases, so that the wait at the start of the next step covers it
-            const bool same = m > 0;
-            const bool n_under_way = ch_ok && ((r >= 1 && r <= ng.rows) || (r == 0 && ng.has_above));
-            if (same || into_next)
-              load_ckpt(same ? cx.g.band : ng.band, same ? cx.under_way : n_under_way, same ? m - 1 : n_nb - 1);
+      for (int k = kCK - 1; k >= 0; --k) {
+        const int t = t0 + k;
+        retreat(1);
+        if (half == 1 && k == 0) staging_landed();   // before the last stores of the block, see the forward kernel
+        // the states of the later steps are dead by now: their registers take the next snapshot
+        if (half == 1 && k == (kCK > 1 ? 1 : 0) && m > 0) load_ckpt(m - 1);
+        if (t < p.T_total) {
+          const bool col0 = at.col == 0;
+          const float offT = col0 ? K.oT0 : K.oT;
+          const float offL = col0 ? ninf : K.oL;
+          const float cT = col0 ? K.cT0 : K.cT;
+          const float cL = col0 ? K.cL0 : K.cL;
+          const bool inr = K.real && at.col < p.W;   // K.real is false outside the bands of the grid
+          float xv = 0.f, dtv = 0.f, dlv = 0.f, dyv = 0.f;
+          if constexpr (STAGE_X) {
+            const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
+            xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW); dyv = IO<T>::ld(xr + 3 * CW);
+          } else if (inr) {
+            const uint32_t off = cell_bytes();
+            xv = IO<T>::ld(reinterpret_cast<const T*>(Ximg + off));
+            dtv = IO<T>::ld(reinterpret_cast<const T*>(DTimg + off));
+            dlv = IO<T>::ld(reinterpret_cast<const T*>(DLimg + off));
+            dyv = IO<T>::ld(reinterpret_cast<const T*>(DYimg + off));
           }
-          if (t < T_steps) {
-            const bool col0 = t == r;
-            const float offT = col0 ? cx.oT0 : cx.oT;
-            const float offL = col0 ? ninf : cx.oL;
-            const float cT = col0 ? cx.cT0 : cx.cT;
-            const float cL = col0 ? cx.cL0 : cx.cL;
-            const bool inr = cx.real && (unsigned)(t - r) < (unsigned)p.W;
-            const uint32_t goff = cx.cell_off + (uint32_t)t * estep;
-            float xv = 0.f, dtv = 0.f, dlv = 0.f, dyv = 0.f;
-            if constexpr (STAGE_X) {
-              const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
-              xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW); dyv = IO<T>::ld(xr + 3 * CW);
-            } else if (inr) {
-              xv = IO<T>::ld(reinterpret_cast<const T*>(Ximg + goff));
-              dtv = IO<T>::ld(reinterpret_cast<const T*>(DTimg + goff));
-              dlv = IO<T>::ld(reinterpret_cast<const T*>(DLimg + goff));
-              dyv = IO<T>::ld(reinterpret_cast<const T*>(DYimg + goff));
-            }
-            uint32_t a_off = a_base_off;
-            asm volatile("" : "+v"(a_off));
-            const lds_float4* a_mine = (const lds_float4*)(uintptr_t)a_off;
-            const char* rec = bufc + (rec_off + k * rec_kstr);
-            const float qT = cT * dtv * xv, qL = cL * dlv * xv;   // zero on lanes that are not grid cells
-            const float dyl = dyv + cx.gb1;                        // the lower ghost: lambda = 1 * (row of mu_T below)
-            float sT = 0.f, sL = 0.f, zT = 0.f, zL = 0.f;
-            if (half == 1) { sT = part4[k][0]; sL = part4[k][1]; zT = part4[k][2]; zL = part4[k][3]; }
-            TICK(ta1);
-            float* sw = reinterpret_cast<float*>(slots + (xpar * kBwdWaves + wave) * SLOT + lane);
-            // A group of 4 states is folded over the 4 channel slots of the wave as soon as it is
-            // done; afterwards the lane of slot q holds the channel sums of the states 4q..4q+3
-            // (component mgl of its float2 after group mgl of this half).
+          uint32_t a_off = a_base_off;
+          asm volatile("" : "+v"(a_off));
+          const lds_float4* a_mine = (const lds_float4*)(uintptr_t)a_off;
+          const char* rec = bufc + (rec_off + k * rec_kstr);
+          const float qT = cT * dtv * xv, qL = cL * dlv * xv;   // zero on lanes that are not grid cells
+          const float dyl = dyv + gb1;
+          float sT = 0.f, sL = 0.f, zT = 0.f, zL = 0.f;
+          if (half == 1) { sT = part4[k][0]; sL = part4[k][1]; zT = part4[k][2]; zL = part4[k][3]; }
+          TICK(ta1);
+          float* sw = reinterpret_cast<float*>(slots + (xpar * kBwdWaves + wave) * SLOT + lane);
+          // A group of 4 states is folded over the 4 channel slots of the wave as soon as it is
+          // done; afterwards the lane of slot q holds the channel sums of the states 4q..4q+3
+          // (component mgl of its float2 after group mgl of this half).
 #pragma unroll
-            for (int mgl = 0; mgl < 2; ++mgl) {
-              const int mg = 2 * half + mgl;
-              const v4f_t at4 = a_mine[mg], al4 = a_mine[kN / 4 + mg];
-              const float4 b4 = reinterpret_cast<const float4*>(rec)[mg], l4 = reinterpret_cast<const float4*>(rec + kN * 4)[mg];
-              const float4 c4 = reinterpret_cast<const float4*>(rec + 2 * kN * 4)[mg];
-              const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
-              const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w}, cq[4] = {c4.x, c4.y, c4.z, c4.w};
-              float vC[4], vBT[4], vBL[4];
+          for (int mgl = 0; mgl < 2; ++mgl) {
+            const int mg = 2 * half + mgl;
+            const v4f_t at4 = a_mine[mg], al4 = a_mine[kN / 4 + mg];
+            const float4 b4 = reinterpret_cast<const float4*>(rec)[mg], l4 = reinterpret_cast<const float4*>(rec + kN * 4)[mg];
+            const float4 c4 = reinterpret_cast<const float4*>(rec + 2 * kN * 4)[mg];
+            const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
+            const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w}, cq[4] = {c4.x, c4.y, c4.z, c4.w};
+            float vC[4], vBT[4], vBL[4];
 #pragma unroll
-              for (int qi = 0; qi < 4; ++qi) {
-                const int n = fold_state(mg, qi), s8 = 4 * mgl + qi;
-                const float a2t = atq[qi], a2l = alq[qi];
-                const float aT = fexp2(__builtin_fmaf(dtv, a2t, offT));
-                const float aL = fexp2(__builtin_fmaf(dlv, a2l, offL));
-                const float mb = from_row_above(muT[n]);
-                const float lam = __builtin_fmaf(dyl, cq[qi], muL[n] + mb);
-                const float hT = from_row_below(hb[k][s8]);
-                const float mT = aT * lam, mL = aL * lam;
-                muT[n] = mT;
-                muL[n] = mL;
-                const float ZT = mT * hT, ZL = mL * hb[k][s8];
-                accAT[n] = __builtin_fmaf(ZT, dtv, accAT[n]);
-                accAL[n] = __builtin_fmaf(ZL, dlv, accAL[n]);
-                zT = __builtin_fmaf(ZT, a2t, zT);
-                zL = __builtin_fmaf(ZL, a2l, zL);
-                sT = __builtin_fmaf(lam, bq[qi], sT);
-                sL = __builtin_fmaf(lam, lq[qi], sL);
-                vBT[qi] = qT * lam;
-                vBL[qi] = qL * lam;
-                vC[qi] = dyv * hb[k + 1][s8];
-              }
-              sw[mgl] = fold16(fold32(vC[0], vC[1]), fold32(vC[2], vC[3]));
-              sw[64 * 2 + mgl] = fold16(fold32(vBT[0], vBT[1]), fold32(vBT[2], vBT[3]));
-              sw[128 * 2 + mgl] = fold16(fold32(vBL[0], vBL[1]), fold32(vBL[2], vBL[3]));
+            for (int qi = 0; qi < 4; ++qi) {
+              const int n = fold_state(mg, qi), s8 = 4 * mgl + qi;
+              const float a2t = atq[qi], a2l = alq[qi];
+              const float aT = fexp2(__builtin_fmaf(dtv, a2t, offT));
+              const float aL = fexp2(__builtin_fmaf(dlv, a2l, offL));
+              const float mb = from_row_above(muT[n]);
+              const float lam = __builtin_fmaf(dyl, cq[qi], muL[n] + mb);
+              const float hT = from_row_below(hb[k][s8]);
+              const float mT = aT * lam, mL = aL * lam;
+              muT[n] = mT;
+              muL[n] = mL;
+              const float ZT = mT * hT, ZL = mL * hb[k][s8];
+              accAT[n] = __builtin_fmaf(ZT, dtv, accAT[n]);
+              accAL[n] = __builtin_fmaf(ZL, dlv, accAL[n]);
+              zT = __builtin_fmaf(ZT, a2t, zT);
+              zL = __builtin_fmaf(ZL, a2l, zL);
+              sT = __builtin_fmaf(lam, bq[qi], sT);
+              sL = __builtin_fmaf(lam, lq[qi], sL);
+              vBT[qi] = qT * lam;
+              vBL[qi] = qL * lam;
+              vC[qi] = dyv * hb[k + 1][s8];
             }
-            if (cx.g.has_above) {   // first row of the band: the band above's lower ghost will replay its muT
-              if (cx.to_bot && inr) {
-                char* bb = BOTimg + (bot_off + (uint32_t)t * (uint32_t)(p.E * kN * sizeof(float)));
+            sw[mgl] = fold16(fold32(vC[0], vC[1]), fold32(vC[2], vC[3]));
+            sw[64 * 2 + mgl] = fold16(fold32(vBT[0], vBT[1]), fold32(vBT[2], vBT[3]));
+            sw[128 * 2 + mgl] = fold16(fold32(vBL[0], vBL[1]), fold32(vBL[2], vBL[3]));
+          }
+          if (p.nbands > 1) {   // first row of a band: the lower ghost of the band above will replay its muT
+            if (inr && r == 1 && at.bnd >= 1) {
+              char* bb = BOTimg + (uint32_t)(at.col * p.E + e) * (uint32_t)(kN * sizeof(float));
 #pragma unroll
-                for (int q = 2 * half; q < 2 * half + 2; ++q)   // the two state groups of this half, as of this step
-                  reinterpret_cast<float4*>(bb)[q] = make_float4(muT[sinv<PERM>(4 * q)], muT[sinv<PERM>(4 * q + 1)],
-                                                                 muT[sinv<PERM>(4 * q + 2)], muT[sinv<PERM>(4 * q + 3)]);
-              }
+              for (int q = 2 * half; q < 2 * half + 2; ++q)   // the two state groups of this half, as of this step
+                reinterpret_cast<float4*>(bb)[q] = make_float4(muT[sinv<PERM>(4 * q)], muT[sinv<PERM>(4 * q + 1)],
+                                                               muT[sinv<PERM>(4 * q + 2)], muT[sinv<PERM>(4 * q + 3)]);
             }
-            if (half == 0) {
-              part4[k][0] = sT; part4[k][1] = sL; part4[k][2] = zT; part4[k][3] = zL;
-            } else {
-              accD = __builtin_fmaf(dyv, xv, accD);
-              if (inr) {
-                IO<T>::st(reinterpret_cast<T*>(DDTimg + goff), __builtin_fmaf(cT * xv, sT, kLn2 * zT));
-                IO<T>::st(reinterpret_cast<T*>(DDLimg + goff), __builtin_fmaf(cL * xv, sL, kLn2 * zL));
-                IO<T>::st(reinterpret_cast<T*>(DXimg + goff), __builtin_fmaf(cT * dtv, sT, __builtin_fmaf(cL * dlv, sL, dyv * dsk)));
-              }
+          }
+          if (half == 0) {
+            part4[k][0] = sT; part4[k][1] = sL; part4[k][2] = zT; part4[k][3] = zL;
+          } else {
+            accD = __builtin_fmaf(dyv, xv, accD);
+            if (inr) {
+              const uint32_t goff = cell_bytes();
+              IO<T>::st(reinterpret_cast<T*>(DDTimg + goff), __builtin_fmaf(cT * xv, sT, kLn2 * zT));
+              IO<T>::st(reinterpret_cast<T*>(DDLimg + goff), __builtin_fmaf(cL * xv, sL, kLn2 * zL));
+              IO<T>::st(reinterpret_cast<T*>(DXimg + goff), __builtin_fmaf(cT * dtv, sT, __builtin_fmaf(cL * dlv, sL, dyv * dsk)));
             }
-            // ---- across the waves of the workgroup: the per-wave slots (this half's two state
-            // groups) are added in wave order, one sum per thread, the same share for every wave
-            TICK(ta2); TACC(3, ta1, ta2); TACC(2, ta2, ta2);
-            __syncthreads();
-            TICK(ta3); TACC(4, ta2, ta3);
-            if (cx.f_real && (unsigned)(t - f_r) < (unsigned)p.W) {
+          }
+          // ---- across the waves of the workgroup: the per-wave slots (this half's two state
+          // groups) are added in wave order, one sum per thread, the same share for every wave
+          TICK(ta2); TACC(3, ta1, ta2); TACC(2, ta2, ta2);
+          __syncthreads();
+          TICK(ta3); TACC(4, ta2, ta3);
+          {
+            // position of lane row f_r at this step, from the thread's own
+            Pos fq;
+            fq.col = at.col + f_d; fq.bnd = at.bnd;
+            if (fq.col < 0) { fq.col += p.S; fq.bnd -= 1; }
+            if (fq.col >= p.S) { fq.col -= p.S; fq.bnd += 1; }
+            if (f_on && (unsigned)fq.bnd < (unsigned)p.nbands && fq.col < p.W && f_r >= 1 && f_r <= kRB && f_r <= band_rows(p, fq.bnd)) {
               const float* sl = reinterpret_cast<const float*>(slots + xpar * kBwdWaves * SLOT + f_it) + f_comp;
               float s = sl[0];
 #pragma unroll
               for (int w = 1; w < kBwdWaves; ++w) s += sl[2 * w * SLOT];
-              *reinterpret_cast<float*>(PARTimg + (cx.f_off + (uint32_t)t * pstep + (uint32_t)(2 * half * sizeof(float)))) = s;
+              const uint32_t off = (uint32_t)cell_of(p, fq.bnd, f_r, fq.col) * (uint32_t)(3 * kN * sizeof(float)) + f_sub;
+              *reinterpret_cast<float*>(PARTimg + (off + (uint32_t)(2 * half * sizeof(float)))) = s;
             }
-            xpar ^= 1;
           }
+          xpar ^= 1;
         }
       }
-      // restart per band: the band's first-row muT is read back by the first staging of the band above
-      if (m == 0 && more && !streamed) __threadfence();
-      TICK(tz0);
-      __syncthreads();
-      TICK(tz1); TACC(5, tz0, tz1);
-      cur ^= 1;
     }
-    if (more) cx = band_ctx(band - 1);
+    TICK(tz0);
+    __syncthreads();
+    TICK(tz1); TACC(5, tz0, tz1);
+    retreat(kCK);   // to the position of the first step of the next block
+    cur ^= 1;
   }
 
 #ifdef M2D_X_TIMING
@@ -1166,6 +1131,7 @@ inline size_t align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
 
 struct Geometry {
   int HB, hb_shift, CS, nbands, nblk;
+  int S, T_total, rows_last;         // stream stride, total steps, rows of the last band
   int fwd_ec, fwd_wpb, fwd_bpb;      // forward: channels per lane, waves and workgroups per image
   int bwd_wpb, bwd_bpb;              // backward: waves and workgroups (channel groups) per image
   bool stage_x;                      // x, delta, dy rows are whole 16-byte chunks: stage them through LDS
@@ -1189,7 +1155,13 @@ Geometry make_geometry(const m2d_desc* d) {
   g.hb_shift = kHBShift;
   g.CS = 64 / g.HB;
   g.nbands = (d->H + kRB - 1) / kRB;
-  g.nblk = (d->W + kHB - 1 + kCK - 1) / kCK;
+  g.rows_last = d->H - (g.nbands - 1) * kRB;
+  // A band's ghost reads the row that the band before stored S - 14 steps earlier, one block
+  // ahead of its use: S - 14 >= 12 steps cover the store, the block-end barrier and the staging.
+  // Wide grids run the bands back to back (S = W); narrow ones are padded.
+  g.S = (g.nbands > 1 && d->W >= 26) ? d->W : (d->W + kHB - 1 > 26 ? d->W + kHB - 1 : 26);
+  g.T_total = (g.nbands - 1) * g.S + d->W + g.rows_last;
+  g.nblk = (g.T_total + kCK - 1) / kCK;
   // forward: two channels per lane when that still yields enough waves to fill the device
   const bool ec2 = (d->E % 2 == 0) && ((int64_t)d->B * ((d->E + kFwdWaves * g.CS * 2 - 1) / (kFwdWaves * g.CS * 2)) >= 256);
   g.fwd_ec = ec2 ? 2 : 1;
@@ -1201,7 +1173,7 @@ Geometry make_geometry(const m2d_desc* d) {
   const size_t P = (size_t)d->B * d->H * d->W;
   g.prep_bytes = align_up(sizeof(float) * (kZeroFloats + (size_t)2 * d->E * kN + d->E));
   g.bc_bytes = align_up(sizeof(float) * P * 48);
-  g.ckpt_diag_bytes = align_up(sizeof(float) * (size_t)d->B * g.nbands * g.nblk * d->E * kN * g.HB);
+  g.ckpt_diag_bytes = align_up(sizeof(float) * (size_t)d->B * g.nblk * d->E * kN * g.HB);
   g.top_bytes = g.nbands > 1 ? align_up(sizeof(float) * (size_t)(g.nbands - 1) * d->B * d->W * d->E * kN) : 0;
   g.bot_bytes = g.nbands > 1 ? align_up(sizeof(float) * (size_t)d->B * d->W * d->E * kN) : 0;
   g.part_bytes = align_up(sizeof(float) * (size_t)g.bwd_bpb * 3 * P * kN);
@@ -1229,6 +1201,8 @@ bool misaligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p
 void fill_common(ScanParams& sp, const m2d_desc* d, const Geometry& g) {
   sp.B = d->B; sp.H = d->H; sp.W = d->W; sp.E = d->E;
   sp.nbands = g.nbands; sp.nblk = g.nblk;
+  sp.S = g.S; sp.T_total = g.T_total; sp.rows_last = g.rows_last;
+  sp.magicS = (uint32_t)(((uint64_t)1 << 32) / (uint64_t)g.S);
   sp.flip = (d->flags & M2D_FLAG_FLIP) ? 1 : 0;
 }
 
