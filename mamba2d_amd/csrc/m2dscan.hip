@@ -198,7 +198,7 @@ __device__ __forceinline__ Pos pos_of(const ScanParams& p, int s) {
 __device__ __forceinline__ int band_rows(const ScanParams& p, int bnd) { return bnd == p.nbands - 1 ? p.rows_last : kRB; }
 // cell index inside its image of lane row r of band bnd at column col
 __device__ __forceinline__ int cell_of(const ScanParams& p, int bnd, int r, int col) {
-  const int cell = (bnd * kRB + r - 1) * p.W + col;
+  const int cell = __mul24(bnd * kRB + r - 1, p.W) + col;   // rows and columns are far below 2^24
   return p.flip ? p.H * p.W - 1 - cell : cell;
 }
 
@@ -307,10 +307,21 @@ struct StagePlan {
   }
 };
 
-// Stages the operands of the block of steps t0 .. t0+kCK-1.
+// Position of the stream index (index of A) + d, for 0 <= d < S.
+__device__ __forceinline__ Pos pos_after(const ScanParams& p, Pos A, int d) {
+  Pos q;
+  q.col = A.col + d;
+  const bool w = q.col >= p.S;
+  q.col = w ? q.col - p.S : q.col;
+  q.bnd = w ? A.bnd + 1 : A.bnd;
+  return q;
+}
+
+// Stages the operands of a block of kCK steps; A is the position of the stream index
+// (first step of the block) - 15, from which every row's position in the block follows.
 template <typename T, int NT, int CW, bool WITH_BOT, bool UNI, bool STAGE_X, int NWAVES, bool KEEP>
 __device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan<T, NT, CW, WITH_BOT, UNI, NWAVES, KEEP>& plan, char* buf,
-                                            int b, int t0, int e_wg0, int wave, int lane,
+                                            int b, Pos A, int e_wg0, int wave, int lane,
                                             const T* x0, const T* x1, const T* x2, const T* x3) {
   using SG = Stage<T, NT, CW, WITH_BOT, UNI>;
   using PL = StagePlan<T, NT, CW, WITH_BOT, UNI, NWAVES, KEEP>;
@@ -324,7 +335,7 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan
     const uint32_t w = plan.get_bc(i, wave, lane);
     const int r = w & 15, part = (w >> 4) & 31, k = (w >> 9) & 3;
     if ((int)w < 0) {
-      const Pos q = pos_of(p, t0 + k - r);
+      const Pos q = pos_after(p, A, k - r + (kHB - 1));
       const float* src = p.zeros;
       if ((unsigned)q.bnd < (unsigned)p.nbands && q.col < p.W && r >= 1 && r <= band_rows(p, q.bnd))
         src = p.bt + (img + cell_of(p, q.bnd, r, q.col)) * p.bc_stride + part * 4;   // B_T, B_L, C back to back
@@ -337,7 +348,7 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan
       const uint32_t w = plan.get_xd(i, wave, lane);
       const int r = w & 15, part = (w >> 4) & 31, k = (w >> 9) & 3;
       if ((int)w < 0) {
-        const Pos q = pos_of(p, t0 + k - r);
+        const Pos q = pos_after(p, A, k - r + (kHB - 1));
         const int tau = part / SG::kCpt, ch = e_wg0 + (part & (SG::kCpt - 1)) * SG::kElem;
         const void* src = p.zeros;
         if ((unsigned)q.bnd < (unsigned)p.nbands && q.col < p.W && r >= 1 && r <= band_rows(p, q.bnd) && ch < p.E) {
@@ -354,7 +365,7 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan
   for (int qi = wave; qi < SG::kTInstr; qi += NWAVES) {
     const int k = qi / (CW / 16), sub = qi - k * (CW / 16);
     const int ch = e_wg0 + sub * 16 + (lane >> 2);
-    const Pos q = pos_of(p, t0 + k);                 // the upper ghost is lane 0
+    const Pos q = pos_after(p, A, k + (kHB - 1));    // the upper ghost is lane 0
     const float* src = p.zeros;
     if (q.bnd >= 1 && q.bnd < p.nbands && q.col < p.W && ch < p.E)
       src = p.top + ((((int64_t)(q.bnd - 1) * p.B + b) * p.W + q.col) * p.E + ch) * kN + (lane & 3) * 4;
@@ -364,7 +375,7 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan
     for (int qi = wave; qi < SG::kTInstr; qi += NWAVES) {
       const int k = qi / (CW / 16), sub = qi - k * (CW / 16);
       const int ch = e_wg0 + sub * 16 + (lane >> 2);
-      const Pos q = pos_of(p, t0 + k - (kHB - 1));   // the lower ghost is lane 15
+      const Pos q = pos_after(p, A, k);              // the lower ghost is lane 15
       const float* src = p.zeros;
       if (q.bnd >= 0 && q.bnd + 1 < p.nbands && q.col < p.W && ch < p.E)
         src = p.bot + (((int64_t)b * p.W + q.col) * p.E + ch) * kN + (lane & 3) * 4;
@@ -403,11 +414,12 @@ struct LaneK {
 template <bool BWD>
 __device__ __forceinline__ LaneK lane_consts(const ScanParams& p, int bnd, int r, bool ch_ok) {
   const float ninf = -__builtin_huge_valf();
-  const bool in_b = (unsigned)bnd < (unsigned)p.nbands;
+  // `bnd` is a band of the grid (callers clamp): a row that is before the first band or past the
+  // last one works on zero operands with the constants of that band
   LaneK c;
-  c.real = ch_ok && in_b && r >= 1 && r <= band_rows(p, bnd);
+  c.real = ch_ok && r >= 1 && r <= kRB && r <= band_rows(p, bnd);
   const bool first_row = bnd == 0 && r == 1;
-  const bool gbot = BWD && r == kHB - 1 && in_b && bnd + 1 < p.nbands;
+  const bool gbot = BWD && r == kHB - 1 && bnd + 1 < p.nbands;
   c.oT = gbot ? 0.f : (!c.real || first_row ? ninf : -1.f);
   c.oL = !c.real ? ninf : (first_row ? 0.f : -1.f);
   c.cT = !c.real || first_row ? 0.f : 0.5f;
@@ -426,6 +438,42 @@ __device__ __forceinline__ bool snapshot_lane(const ScanParams& p, Pos at, int r
   pv.col = at.col >= 1 ? at.col - 1 : p.S - 1;
   const bool row_ok = r == 0 ? pv.bnd >= 1 : (r <= kRB && r <= band_rows(p, pv.bnd));
   return ch_ok && (unsigned)pv.bnd < (unsigned)p.nbands && pv.col < p.W && row_ok;
+}
+
+// Positions of one lane row over a block of kCK steps.  All rows of the wave sit within 19
+// consecutive stream positions, which touch at most two bands, so everything derives from the
+// (wave-uniform) position A of the stream index t0 - 15 with adds and compares.
+struct BlockPos {
+  int bnd0, col0;      // position at the first step of the block
+  int kw;              // first step of the block at which the row is in the next band (>= kCK: never)
+  int kz;              // step of the block at which the row is at column 0 (>= kCK: never)
+  uint32_t in_grid;    // bit k: the row is at a cell of the grid at step k
+};
+__device__ __forceinline__ BlockPos block_pos(const ScanParams& p, Pos A, int r, bool lane_ok) {
+  BlockPos q;
+  q.col0 = A.col + (kHB - 1 - r);
+  const bool w = q.col0 >= p.S;
+  q.col0 = w ? q.col0 - p.S : q.col0;
+  q.bnd0 = w ? A.bnd + 1 : A.bnd;
+  q.kw = p.S - q.col0;
+  q.kz = q.col0 == 0 ? 0 : q.kw;
+  q.in_grid = 0;
+  const bool row = lane_ok && r >= 1 && r <= kRB;
+#pragma unroll
+  for (int k = 0; k < kCK; ++k) {
+    const bool wk = k >= q.kw;
+    const int bk = wk ? q.bnd0 + 1 : q.bnd0;
+    const int ck = wk ? q.col0 + k - p.S : q.col0 + k;
+    const bool in = row && (unsigned)bk < (unsigned)p.nbands && ck < p.W && r <= band_rows(p, bk);
+    q.in_grid |= in ? (1u << k) : 0u;
+  }
+  return q;
+}
+__device__ __forceinline__ int clamp_band(const ScanParams& p, int bnd) { return bnd < 0 ? 0 : (bnd >= p.nbands ? p.nbands - 1 : bnd); }
+// A row changes its constants only when it moves between the first band and the second (grid row
+// 0 has no row above) or into / out of the last band (fewer rows, no band below).
+__device__ __forceinline__ bool special_boundary(const ScanParams& p, int bnd_lo, int r) {
+  return (bnd_lo == 0 && r == 1) || (bnd_lo + 1 == p.nbands - 1 && (r > p.rows_last || r == kHB - 1));
 }
 
 // ------------------------------------------------------------------------------------ forward
@@ -485,26 +533,20 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   const char* DLimg = reinterpret_cast<const char*>(DL) + img_bytes;
   const uint32_t estep = (uint32_t)(p.flip ? -p.E : p.E) * (uint32_t)sizeof(T);   // one column further
 
-  // where the lane is in its stream, and what depends on it
-  Pos at = pos_of(p, -r);
-  LaneK K = lane_consts<false>(p, at.bnd, r, ch_ok);
   const float g1 = r == 0 ? 1.f : 0.f;             // the ghost's T input coefficient
-  uint32_t cell_off = 0;                           // byte offset of the lane's cell in a (H,W,E) image
-  float* top_ptr = p.top;                          // where lane 14 stores its states for the next band's ghost
-  bool to_top = false;
-  auto enter_band = [&]() {                        // the lane is at (at.bnd, at.col): refresh what depends on the band
-    K = lane_consts<false>(p, at.bnd, r, ch_ok);
-    cell_off = (uint32_t)(cell_of(p, at.bnd, r, at.col) * p.E + e0) * (uint32_t)sizeof(T);
-    to_top = K.real && r == kRB && at.bnd + 1 < p.nbands;
-    if (to_top) top_ptr = p.top + ((((int64_t)at.bnd * p.B + b) * p.W + at.col) * p.E + e0) * kN;
-  };
-  enter_band();
+  const uint32_t wrap_adj = (uint32_t)(kRB * p.W - p.S) * estep;   // extra offset of a cell reached through a band change
 
   // byte offsets of the lane's records inside a staging buffer (step 0)
   const uint32_t rec_off = r == 0 ? SG::kTOff + ch_loc * kN * 4 : r * SG::kBStride * 4;
   const uint32_t rec_cstep = r == 0 ? kN * 4 : 0;   // the ghost reads a record per channel, grid rows share theirs
   const uint32_t xd_off = SG::kXOff + (r * SG::kXStride + ch_loc) * (uint32_t)sizeof(T);
   constexpr uint32_t kXK = kHB * SG::kXStride * sizeof(T);   // XD bytes per step
+
+  // per block: where the lane is and what depends on it
+  BlockPos bp;
+  LaneK K;
+  uint32_t cell_off0 = 0;       // byte offset in a (H,W,E) image of the lane's cell at the first step of the block
+  bool per_step_K = false;      // (uniform) a row crosses a band boundary that changes its constants inside the block
 
   // Operands of one step, read from the staging buffer one step ahead of their use so that the
   // LDS latency hides behind the arithmetic of the step before.
@@ -518,13 +560,14 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
       IO<T>::template ldv<EC>(xr, o.xv);
       IO<T>::template ldv<EC>(xr + CW, o.dtv);
       IO<T>::template ldv<EC>(xr + 2 * CW, o.dlv);
-    } else {   // straight from memory, for the lane's current position
+    } else {   // straight from memory, for the lane's position at step k of the current block
 #pragma unroll
       for (int c = 0; c < EC; ++c) { o.xv[c] = 0.f; o.dtv[c] = 0.f; o.dlv[c] = 0.f; }
-      if (K.real && at.col < p.W) {
-        IO<T>::template ldv<EC>(reinterpret_cast<const T*>(Ximg + cell_off), o.xv);
-        IO<T>::template ldv<EC>(reinterpret_cast<const T*>(DTimg + cell_off), o.dtv);
-        IO<T>::template ldv<EC>(reinterpret_cast<const T*>(DLimg + cell_off), o.dlv);
+      if ((bp.in_grid >> k) & 1u) {
+        const uint32_t off = cell_off0 + (uint32_t)k * estep + (k >= bp.kw ? wrap_adj : 0u);
+        IO<T>::template ldv<EC>(reinterpret_cast<const T*>(Ximg + off), o.xv);
+        IO<T>::template ldv<EC>(reinterpret_cast<const T*>(DTimg + off), o.dtv);
+        IO<T>::template ldv<EC>(reinterpret_cast<const T*>(DLimg + off), o.dlv);
       }
     }
     // a grid row reads B_T, B_L, C of its cell; the ghost reads the row above as its B_T (and
@@ -547,13 +590,14 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
 #pragma unroll
     for (int n = 0; n < kN; ++n) h[c][n] = 0.f;
 
-  auto step = [&](const Ops& o) {
-    const bool col0 = at.col == 0;
+  auto step = [&](int k, const Ops& o) {
+    if (per_step_K) K = lane_consts<false>(p, clamp_band(p, k >= bp.kw ? bp.bnd0 + 1 : bp.bnd0), r, ch_ok);
+    const bool col0 = bp.kz == k;
     const float offT = col0 ? K.oT0 : K.oT;
     const float offL = col0 ? ninf : K.oL;
     const float cT = col0 ? K.cT0 : K.cT;
     const float cL = col0 ? K.cL0 : K.cL;
-    const bool inr = K.real && at.col < p.W;   // K.real is false outside the bands of the grid
+    const bool inr = (bp.in_grid >> k) & 1u;
     float yv[EC];
 #pragma unroll
     for (int c = 0; c < EC; ++c) {
@@ -581,30 +625,25 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
       yv[c] = __builtin_fmaf(o.xv[c], dsk[c], acc);
     }
     if (p.nbands > 1) {   // last row of a band: the next band's ghost will replay it
-      if (to_top && inr) {
+      const bool wk = k >= bp.kw;
+      const int bk = wk ? bp.bnd0 + 1 : bp.bnd0;
+      if (inr && r == kRB && bk + 1 < p.nbands) {
+        const int ck = wk ? bp.col0 + k - p.S : bp.col0 + k;
+        float4* tw = reinterpret_cast<float4*>(p.top + ((((int64_t)bk * p.B + b) * p.W + ck) * p.E + e0) * kN);
 #pragma unroll
         for (int c = 0; c < EC; ++c)
 #pragma unroll
           for (int q = 0; q < 4; ++q)
-            reinterpret_cast<float4*>(top_ptr)[c * 4 + q] = make_float4(h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)],
-                                                                        h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
-      }
-      top_ptr += p.E * kN;
-    }
-    if (WRITE_Y && inr) IO<T>::template stv<EC>(reinterpret_cast<T*>(Yimg + cell_off), yv);
-    // one position further; a lane that leaves its band enters column 0 of the next one
-    at.col += 1;
-    cell_off += estep;
-    if (__any(at.col == p.S)) {
-      if (at.col == p.S) {
-        at.col = 0;
-        at.bnd += 1;
-        enter_band();
+            tw[c * 4 + q] = make_float4(h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)],
+                                        h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
       }
     }
+    if (WRITE_Y && inr)
+      IO<T>::template stv<EC>(reinterpret_cast<T*>(Yimg + (cell_off0 + (uint32_t)k * estep + (k >= bp.kw ? wrap_adj : 0u))), yv);
   };
 
-  stage_block<T, 3, CW, false, true, STAGE_X, kFwdWaves, true>(p, plan, lds, b, 0, e_wg0, wave, lane, X, DT, DL, DY);
+  Pos A = pos_of(p, -(kHB - 1));     // position of the stream index t0 - 15 (wave-uniform)
+  stage_block<T, 3, CW, false, true, STAGE_X, kFwdWaves, true>(p, plan, lds, b, A, e_wg0, wave, lane, X, DT, DL, DY);
   staging_fence();
   Ops opsA, opsB;
   if constexpr (AHEAD) fetch(lds, 0, opsA);
@@ -614,16 +653,23 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
     const bool last = m + 1 == p.nblk;
     TICK(ts0);
     if (!last)
-      stage_block<T, 3, CW, false, true, STAGE_X, kFwdWaves, true>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, t0 + kCK, e_wg0, wave, lane, X, DT, DL, DY);
+      stage_block<T, 3, CW, false, true, STAGE_X, kFwdWaves, true>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, pos_after(p, A, kCK), e_wg0, wave, lane, X, DT, DL, DY);
     TICK(ts1); TACC(1, ts0, ts1);
+    bp = block_pos(p, A, r, ch_ok);
+    K = lane_consts<false>(p, clamp_band(p, bp.bnd0), r, ch_ok);
+    per_step_K = __any(bp.kw < kCK && special_boundary(p, bp.bnd0, r));
+    cell_off0 = (uint32_t)(cell_of(p, bp.bnd0, r, bp.col0) * p.E + e0) * (uint32_t)sizeof(T);
     // snapshot of the state before the block (after step t0-1) for the lanes whose previous
     // position was a cell of the grid; the others hold nothing the backward needs
-    if (CKPT && m > 0 && snapshot_lane(p, at, r, ch_ok)) {
-      float* ck = p.ckpt + ((((int64_t)b * p.nblk + m) * p.E + e0) * kN) * kHB + r;
+    if (CKPT && m > 0) {
+      Pos at; at.bnd = bp.bnd0; at.col = bp.col0;
+      if (snapshot_lane(p, at, r, ch_ok)) {
+        float* ck = p.ckpt + ((((int64_t)b * p.nblk + m) * p.E + e0) * kN) * kHB + r;
 #pragma unroll
-      for (int c = 0; c < EC; ++c)
+        for (int c = 0; c < EC; ++c)
 #pragma unroll
-        for (int n = 0; n < kN; ++n) ck[(c * kN + n) * kHB] = h[c][n];
+          for (int n = 0; n < kN; ++n) ck[(c * kN + n) * kHB] = h[c][n];
+      }
     }
     const char* bufc = lds + cur * SG::kBytes;
     const char* bufn = lds + (cur ^ 1) * SG::kBytes;
@@ -650,7 +696,7 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
           if (!last) fetch(bufn, 0, ahead);
         }
         TICK(tc0);
-        if (t < p.T_total) step(now);
+        if (t < p.T_total) step(k, now);
         TICK(tc1); TACC(4, tc0, tc1);
       }
     } else {
@@ -663,12 +709,14 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
         if (k == kCK - 1) staging_landed();
         if (t < p.T_total) {
           fetch(bufc, k, opsA);
-          step(opsA);
+          step(k, opsA);
         }
       }
       __syncthreads();
     }
     cur ^= 1;
+    A.col += kCK;
+    if (A.col >= p.S) { A.col -= p.S; A.bnd += 1; }
   }
 #ifdef M2D_X_TIMING
   if (lane == 0 && blockIdx.x < 512) {
@@ -778,37 +826,29 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   const uint32_t f_sub = (uint32_t)(f_v * kN + f_s * 4 + f_comp) * (uint32_t)sizeof(float);
   const float g1 = r == 0 ? 1.f : 0.f;
 
-  // Where the lane is in its stream and the constants of its band; both follow the lane as it
-  // walks forward through a block (recompute) and back (adjoint).
-  Pos at = pos_of(p, (p.nblk - 1) * kCK - r);
-  LaneK K = lane_consts<true>(p, at.bnd, r, ch_ok);
-  float gb1 = 0.f;                        // 1 on an active lower ghost: lambda = 1 * (row of mu_T below)
-  auto enter_band = [&]() {
-    K = lane_consts<true>(p, at.bnd, r, ch_ok);
-    gb1 = (r == kHB - 1 && at.bnd >= 0 && at.bnd + 1 < p.nbands) ? 1.f : 0.f;
-  };
-  enter_band();
-  auto advance = [&]() {
-    at.col += 1;
-    if (__any(at.col == p.S)) {
-      if (at.col == p.S) { at.col = 0; at.bnd += 1; enter_band(); }
-    }
-  };
-  auto retreat = [&](int n) {
-    at.col -= n;
-    if (__any(at.col < 0)) {
-      if (at.col < 0) { at.col += p.S; at.bnd -= 1; enter_band(); }
-    }
-  };
-  auto cell_bytes = [&]() {   // byte offset of the lane's cell in a (H,W,E) image
-    return (uint32_t)(cell_of(p, at.bnd, r, at.col) * p.E + e) * (uint32_t)sizeof(T);
+  const uint32_t estep = (uint32_t)(p.flip ? -p.E : p.E) * (uint32_t)sizeof(T);   // one column further
+  const uint32_t wrap_adj = (uint32_t)(kRB * p.W - p.S) * estep;   // extra offset of a cell reached through a band change
+  const uint32_t pstep = (uint32_t)(p.flip ? -1 : 1) * (uint32_t)(3 * kN * sizeof(float));
+  const uint32_t pwrap_adj = (uint32_t)(kRB * p.W - p.S) * pstep;
+
+  // per block: where the lane (and the lane row whose sums this thread adds up) is, and what
+  // depends on it
+  BlockPos bp, fp;
+  LaneK K;
+  float gb1 = 0.f;              // 1 on an active lower ghost: lambda = 1 * (row of mu_T below)
+  uint32_t cell_off0 = 0;       // byte offset in a (H,W,E) image of the lane's cell at the first step of the block
+  uint32_t f_off0 = 0;          // byte offset in the channel-sum image of this thread's sum at the first step
+  bool per_step_K = false;      // (uniform) a row crosses a band boundary that changes its constants inside the block
+  auto band_consts = [&](int bnd) {
+    const int bc = clamp_band(p, bnd);
+    K = lane_consts<true>(p, bc, r, ch_ok);
+    gb1 = (r == kHB - 1 && bc + 1 < p.nbands) ? 1.f : 0.f;
   };
 
-  // state snapshot at the start of block mm (zero for lanes that were not under way)
+  // state snapshot at the start of the block whose position A is given (zero for lanes that were not under way)
   float cknext[kN];
-  auto load_ckpt = [&](int mm) {
-    const Pos q = pos_of(p, mm * kCK - r);
-    if (mm == 0 || !snapshot_lane(p, q, r, ch_ok)) {
+  auto load_ckpt = [&](int mm, Pos Am) {
+    if (mm == 0 || !snapshot_lane(p, pos_after(p, Am, kHB - 1 - r), r, ch_ok)) {
 #pragma unroll
       for (int n = 0; n < kN; ++n) cknext[n] = 0.f;
     } else {
@@ -817,9 +857,15 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
       for (int n = 0; n < kN; ++n) cknext[n] = ck[n * kHB];
     }
   };
+  auto pos_before = [&](Pos Q) {   // kCK positions earlier
+    Q.col -= kCK;
+    if (Q.col < 0) { Q.col += p.S; Q.bnd -= 1; }
+    return Q;
+  };
 
-  load_ckpt(p.nblk - 1);
-  stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds, b, (p.nblk - 1) * kCK, e_wg0, wave, lane, X, DT, DL, DY);
+  Pos A = pos_of(p, (p.nblk - 1) * kCK - (kHB - 1));   // position of the stream index t0 - 15 (wave-uniform)
+  load_ckpt(p.nblk - 1, A);
+  stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds, b, A, e_wg0, wave, lane, X, DT, DL, DY);
   staging_fence();
   int cur = 0;
   int xpar = 0;   // exchange buffer in use
@@ -830,10 +876,17 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
     float ck0[kN];
 #pragma unroll
     for (int n = 0; n < kN; ++n) ck0[n] = cknext[n];
+    const Pos Aprev = pos_before(A);
     TICK(ts0);
     if (m > 0)
-      stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, t0 - kCK, e_wg0, wave, lane, X, DT, DL, DY);
+      stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, Aprev, e_wg0, wave, lane, X, DT, DL, DY);
     TICK(ts1); TACC(0, ts0, ts1);
+    bp = block_pos(p, A, r, ch_ok);
+    fp = block_pos(p, A, f_r, f_on);
+    band_consts(bp.bnd0);
+    per_step_K = __any(bp.kw < kCK && special_boundary(p, bp.bnd0, r));
+    cell_off0 = (uint32_t)(cell_of(p, bp.bnd0, r, bp.col0) * p.E + e) * (uint32_t)sizeof(T);
+    f_off0 = (uint32_t)cell_of(p, fp.bnd0, f_r, fp.col0) * (uint32_t)(3 * kN * sizeof(float)) + f_sub;
 
     // The 16 states are swept in two halves of 8 (state groups 0,1 then 2,3), each half
     // recomputing and then back-propagating the whole block: only 5 x 8 recomputed states are
@@ -846,13 +899,14 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
       for (int mgl = 0; mgl < 2; ++mgl)
 #pragma unroll
         for (int qi = 0; qi < 4; ++qi) hb[0][4 * mgl + qi] = ck0[fold_state(2 * half + mgl, qi)];
-      // ---- recompute the states of the block (the lane is at its position of step t0)
+      // ---- recompute the states of the block
       TICK(tr0);
 #pragma unroll
       for (int k = 0; k < kCK; ++k) {
         const int t = t0 + k;
         if (t < p.T_total) {
-          const bool col0 = at.col == 0;
+          if (per_step_K) band_consts(k >= bp.kw ? bp.bnd0 + 1 : bp.bnd0);
+          const bool col0 = bp.kz == k;
           const float offT = col0 ? K.oT0 : K.oT;
           const float offL = col0 ? ninf : K.oL;
           const float cT = col0 ? K.cT0 : K.cT;
@@ -861,8 +915,8 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
           if constexpr (STAGE_X) {
             const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
             xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW);
-          } else if (K.real && at.col < p.W) {
-            const uint32_t off = cell_bytes();
+          } else if ((bp.in_grid >> k) & 1u) {
+            const uint32_t off = cell_off0 + (uint32_t)k * estep + (k >= bp.kw ? wrap_adj : 0u);
             xv = IO<T>::ld(reinterpret_cast<const T*>(Ximg + off));
             dtv = IO<T>::ld(reinterpret_cast<const T*>(DTimg + off));
             dlv = IO<T>::ld(reinterpret_cast<const T*>(DLimg + off));
@@ -895,34 +949,33 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
             }
           }
         }
-        advance();
       }
       TICK(tr1); TACC(1, tr0, tr1);
-      // ---- adjoint over the block, last step first (the lane is one position past the block)
+      // ---- adjoint over the block, last step first
 #pragma unroll
       for (int k = kCK - 1; k >= 0; --k) {
         const int t = t0 + k;
-        retreat(1);
         if (half == 1 && k == 0) staging_landed();   // before the last stores of the block, see the forward kernel
         // the states of the later steps are dead by now: their registers take the next snapshot
-        if (half == 1 && k == (kCK > 1 ? 1 : 0) && m > 0) load_ckpt(m - 1);
+        if (half == 1 && k == (kCK > 1 ? 1 : 0) && m > 0) load_ckpt(m - 1, Aprev);
         if (t < p.T_total) {
-          const bool col0 = at.col == 0;
+          if (per_step_K) band_consts(k >= bp.kw ? bp.bnd0 + 1 : bp.bnd0);
+          const bool col0 = bp.kz == k;
           const float offT = col0 ? K.oT0 : K.oT;
           const float offL = col0 ? ninf : K.oL;
           const float cT = col0 ? K.cT0 : K.cT;
           const float cL = col0 ? K.cL0 : K.cL;
-          const bool inr = K.real && at.col < p.W;   // K.real is false outside the bands of the grid
+          const bool inr = (bp.in_grid >> k) & 1u;
+          const uint32_t goff = cell_off0 + (uint32_t)k * estep + (k >= bp.kw ? wrap_adj : 0u);
           float xv = 0.f, dtv = 0.f, dlv = 0.f, dyv = 0.f;
           if constexpr (STAGE_X) {
             const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
             xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW); dyv = IO<T>::ld(xr + 3 * CW);
           } else if (inr) {
-            const uint32_t off = cell_bytes();
-            xv = IO<T>::ld(reinterpret_cast<const T*>(Ximg + off));
-            dtv = IO<T>::ld(reinterpret_cast<const T*>(DTimg + off));
-            dlv = IO<T>::ld(reinterpret_cast<const T*>(DLimg + off));
-            dyv = IO<T>::ld(reinterpret_cast<const T*>(DYimg + off));
+            xv = IO<T>::ld(reinterpret_cast<const T*>(Ximg + goff));
+            dtv = IO<T>::ld(reinterpret_cast<const T*>(DTimg + goff));
+            dlv = IO<T>::ld(reinterpret_cast<const T*>(DLimg + goff));
+            dyv = IO<T>::ld(reinterpret_cast<const T*>(DYimg + goff));
           }
           uint32_t a_off = a_base_off;
           asm volatile("" : "+v"(a_off));
@@ -974,8 +1027,10 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
             sw[128 * 2 + mgl] = fold16(fold32(vBL[0], vBL[1]), fold32(vBL[2], vBL[3]));
           }
           if (p.nbands > 1) {   // first row of a band: the lower ghost of the band above will replay its muT
-            if (inr && r == 1 && at.bnd >= 1) {
-              char* bb = BOTimg + (uint32_t)(at.col * p.E + e) * (uint32_t)(kN * sizeof(float));
+            const bool wk = k >= bp.kw;
+            if (inr && r == 1 && (wk ? bp.bnd0 + 1 : bp.bnd0) >= 1) {
+              const int ck = wk ? bp.col0 + k - p.S : bp.col0 + k;
+              char* bb = BOTimg + (uint32_t)(ck * p.E + e) * (uint32_t)(kN * sizeof(float));
 #pragma unroll
               for (int q = 2 * half; q < 2 * half + 2; ++q)   // the two state groups of this half, as of this step
                 reinterpret_cast<float4*>(bb)[q] = make_float4(muT[sinv<PERM>(4 * q)], muT[sinv<PERM>(4 * q + 1)],
@@ -987,7 +1042,6 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
           } else {
             accD = __builtin_fmaf(dyv, xv, accD);
             if (inr) {
-              const uint32_t goff = cell_bytes();
               IO<T>::st(reinterpret_cast<T*>(DDTimg + goff), __builtin_fmaf(cT * xv, sT, kLn2 * zT));
               IO<T>::st(reinterpret_cast<T*>(DDLimg + goff), __builtin_fmaf(cL * xv, sL, kLn2 * zL));
               IO<T>::st(reinterpret_cast<T*>(DXimg + goff), __builtin_fmaf(cT * dtv, sT, __builtin_fmaf(cL * dlv, sL, dyv * dsk)));
@@ -998,20 +1052,13 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
           TICK(ta2); TACC(3, ta1, ta2); TACC(2, ta2, ta2);
           __syncthreads();
           TICK(ta3); TACC(4, ta2, ta3);
-          {
-            // position of lane row f_r at this step, from the thread's own
-            Pos fq;
-            fq.col = at.col + f_d; fq.bnd = at.bnd;
-            if (fq.col < 0) { fq.col += p.S; fq.bnd -= 1; }
-            if (fq.col >= p.S) { fq.col -= p.S; fq.bnd += 1; }
-            if (f_on && (unsigned)fq.bnd < (unsigned)p.nbands && fq.col < p.W && f_r >= 1 && f_r <= kRB && f_r <= band_rows(p, fq.bnd)) {
-              const float* sl = reinterpret_cast<const float*>(slots + xpar * kBwdWaves * SLOT + f_it) + f_comp;
-              float s = sl[0];
+          if ((fp.in_grid >> k) & 1u) {
+            const float* sl = reinterpret_cast<const float*>(slots + xpar * kBwdWaves * SLOT + f_it) + f_comp;
+            float s = sl[0];
 #pragma unroll
-              for (int w = 1; w < kBwdWaves; ++w) s += sl[2 * w * SLOT];
-              const uint32_t off = (uint32_t)cell_of(p, fq.bnd, f_r, fq.col) * (uint32_t)(3 * kN * sizeof(float)) + f_sub;
-              *reinterpret_cast<float*>(PARTimg + (off + (uint32_t)(2 * half * sizeof(float)))) = s;
-            }
+            for (int w = 1; w < kBwdWaves; ++w) s += sl[2 * w * SLOT];
+            const uint32_t off = f_off0 + (uint32_t)k * pstep + (k >= fp.kw ? pwrap_adj : 0u) + (uint32_t)(2 * half * sizeof(float));
+            *reinterpret_cast<float*>(PARTimg + off) = s;
           }
           xpar ^= 1;
         }
@@ -1020,7 +1067,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
     TICK(tz0);
     __syncthreads();
     TICK(tz1); TACC(5, tz0, tz1);
-    retreat(kCK);   // to the position of the first step of the next block
+    A = Aprev;
     cur ^= 1;
   }
 
