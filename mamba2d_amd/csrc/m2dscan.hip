@@ -1142,18 +1142,18 @@ __global__ void m2d_finalize_kernel(const ScanParams p, T* dC, T* dBT, T* dBL, T
   const int64_t nquad = 3 * P * (kN / 4);
   const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (gid < nquad) {
-    // per-workgroup sums are laid out [channel group][cell][C, B_T, B_L][16]
-    const int64_t v = gid / (P * 4), rem = gid % (P * 4);
-    const int64_t cell = rem >> 2;
-    const int q = (int)(rem & 3);
-    const float* src = p.part + (cell * 3 + v) * kN + q * 4;
+    // per-workgroup sums are laid out [channel group][cell][C, B_T, B_L][16]: consecutive threads
+    // read consecutive float4s
+    const int64_t cell = gid / 12;
+    const int rem = (int)(gid - cell * 12), v = rem >> 2, q = rem & 3;
+    const float* src = p.part + cell * (3 * kN) + rem * 4;
     float4 s = *reinterpret_cast<const float4*>(src);
     for (int egi = 1; egi < p.bpb; ++egi) {
       const float4 o = *reinterpret_cast<const float4*>(src + (int64_t)egi * P * 3 * kN);
       s.x += o.x; s.y += o.y; s.z += o.z; s.w += o.w;
     }
     T* out = v == 0 ? dC : (v == 1 ? dBT : dBL);
-    IO<T>::st4(out + rem * 4, s);
+    IO<T>::st4(out + cell * kN + q * 4, s);
   }
   const int64_t k = gid;
   if (k < (int64_t)p.E * 2 * kN) {
