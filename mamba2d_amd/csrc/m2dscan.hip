@@ -51,6 +51,8 @@ constexpr int kRB = 14;           // grid rows per band; lanes 0 and 15 of a row
 constexpr int kFwdWaves = 8;      // waves per forward workgroup
 constexpr int kBwdWaves = 8;      // waves per backward workgroup
 constexpr int kZeroFloats = 64;     // page of zeros at the head of the set-up area
+constexpr int kSliceQ = 4;         // sliced sweep: blocks of steps per band and launch
+constexpr int kSliceLag = 2;       // sliced sweep: launches by which a band trails the band it depends on
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -153,16 +155,24 @@ struct ScanParams {
   void *y, *dx, *ddT, *ddL;
   float* ckpt;                      // [B][nblk][E][16][16]          state snapshots, one per block of steps
   float* top;                       // [nbands-1][B][W][E][16]       last row of each band (forward states)
-  float* bot;                       // [B][W][E][16]                 first-row muT of the band below (adjoint)
+  float* bot;                       // [nbands or 1][B][W][E][16]    first-row muT of a band, for the band above (adjoint)
   float* part;                      // [G][P][3][16]                 per-workgroup channel sums of d_C, d_BT, d_BL
-  float* pA;                        // [B][E][2][16]
-  float* pD;                        // [B][E]
+  float* pA;                        // [B*pa_slots][E][2][16]
+  float* pD;                        // [B*pa_slots][E]
   int B, H, W, E;
   int nbands, nblk, bc_stride, flip;
   int S;                            // stream stride: positions per band (>= W)
   int T_total;                      // steps of the whole sweep
   int rows_last;                    // grid rows of the last band
   uint32_t magicS;                  // floor(2^32 / S)
+  // Sliced sweep (few images, many bands): every band has its own workgroups, a launch advances
+  // each active band by kSliceQ blocks, and a band trails the one it depends on by kSliceLag
+  // launches, so that what it reads was stored by an earlier launch.
+  int sliced, sl_ell, sl_band0;     // on/off, launch index, first active band of the launch
+  int sl_nbb;                       // blocks per band (S / kCK)
+  float* carry;                     // state handed from launch to launch: fwd [B][nbands][E][16][16], bwd [B][nbands][E][65][16]
+  int64_t bot_stride;               // floats between the mu_T rows of consecutive bands (0: one row buffer, bands in sequence)
+  int pa_slots;                     // partial sums over positions per image (1, or one per band when sliced)
   int bpb;                          // workgroups per image
   int nwg;                          // total workgroups
 };
@@ -378,7 +388,7 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan
       const Pos q = pos_after(p, A, k);              // the lower ghost is lane 15
       const float* src = p.zeros;
       if (q.bnd >= 0 && q.bnd + 1 < p.nbands && q.col < p.W && ch < p.E)
-        src = p.bot + (((int64_t)b * p.W + q.col) * p.E + ch) * kN + (lane & 3) * 4;
+        src = p.bot + (q.bnd + 1) * p.bot_stride + (((int64_t)b * p.W + q.col) * p.E + ch) * kN + (lane & 3) * 4;
       lds_fill16<true>(src, buf + SG::kOOff + k * SG::kTKStr + sub * 1024);
     }
   }
@@ -492,7 +502,18 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   char* lds = reinterpret_cast<char*>(smem);       // two staging buffers and 256 bytes of slack
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int lb = logical_block(p.nwg);
+  int lb = logical_block(p.nwg);
+  int m_lo = 0, m_hi = p.nblk;                     // blocks of steps this launch sweeps
+  int my_band = 0, band_q0 = 0;
+  if (p.sliced) {
+    const int per = p.B * p.bpb;
+    const int kk = lb / per;
+    lb -= kk * per;
+    my_band = p.sl_band0 + kk;
+    band_q0 = (p.sl_ell - kSliceLag * my_band) * kSliceQ;
+    m_lo = my_band * p.sl_nbb + band_q0;
+    m_hi = my_band * p.sl_nbb + (band_q0 + kSliceQ < p.sl_nbb ? band_q0 + kSliceQ : p.sl_nbb);
+  }
   const int b = lb / p.bpb;
   const int e_wg0 = (lb % p.bpb) * CW;
   const int slot = lane >> kHBShift, r = lane & (kHB - 1);
@@ -589,6 +610,16 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   for (int c = 0; c < EC; ++c)
 #pragma unroll
     for (int n = 0; n < kN; ++n) h[c][n] = 0.f;
+  float* carry = p.sliced ? p.carry + ((((int64_t)b * p.nbands + my_band) * p.E + e0) * kN) * kHB + r : nullptr;
+  if (p.sliced && band_q0 > 0) {   // the band is under way: take over the state of the previous launch
+    if (ch_ok) {
+#pragma unroll
+      for (int c = 0; c < EC; ++c)
+#pragma unroll
+        for (int n = 0; n < kN; ++n) h[c][n] = carry[(c * kN + n) * kHB];
+    }
+    settle_loads();
+  }
 
   auto step = [&](int k, const Ops& o) {
     if (per_step_K) K = lane_consts<false>(p, clamp_band(p, k >= bp.kw ? bp.bnd0 + 1 : bp.bnd0), r, ch_ok);
@@ -642,15 +673,15 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
       IO<T>::template stv<EC>(reinterpret_cast<T*>(Yimg + (cell_off0 + (uint32_t)k * estep + (k >= bp.kw ? wrap_adj : 0u))), yv);
   };
 
-  Pos A = pos_of(p, -(kHB - 1));     // position of the stream index t0 - 15 (wave-uniform)
+  Pos A = pos_of(p, m_lo * kCK - (kHB - 1));     // position of the stream index t0 - 15 (wave-uniform)
   stage_block<T, 3, CW, false, true, STAGE_X, kFwdWaves, true>(p, plan, lds, b, A, e_wg0, wave, lane, X, DT, DL, DY);
   staging_fence();
   Ops opsA, opsB;
   if constexpr (AHEAD) fetch(lds, 0, opsA);
   int cur = 0;
-  for (int m = 0; m < p.nblk; ++m) {
+  for (int m = m_lo; m < m_hi; ++m) {
     const int t0 = m * kCK;
-    const bool last = m + 1 == p.nblk;
+    const bool last = m + 1 == m_hi;
     TICK(ts0);
     if (!last)
       stage_block<T, 3, CW, false, true, STAGE_X, kFwdWaves, true>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, pos_after(p, A, kCK), e_wg0, wave, lane, X, DT, DL, DY);
@@ -718,6 +749,12 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
     A.col += kCK;
     if (A.col >= p.S) { A.col -= p.S; A.bnd += 1; }
   }
+  if (p.sliced && ch_ok && m_hi < (my_band + 1) * p.sl_nbb) {   // more of the band to come: hand the state to the next launch
+#pragma unroll
+    for (int c = 0; c < EC; ++c)
+#pragma unroll
+      for (int n = 0; n < kN; ++n) carry[(c * kN + n) * kHB] = h[c][n];
+  }
 #ifdef M2D_X_TIMING
   if (lane == 0 && blockIdx.x < 512) {
     long long* d = g_dbg + (blockIdx.x * 8 + wave) * 8;
@@ -759,7 +796,18 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   char* lds = reinterpret_cast<char*>(a_lds + kBwdWaves * CS * 2 * kN);  // 2 staging buffers
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const int lb = logical_block(p.nwg);
+  int lb = logical_block(p.nwg);
+  int m_lo = 0, m_hi = p.nblk;              // blocks of steps this launch sweeps (from m_hi - 1 down to m_lo)
+  int my_band = 0, band_q0 = 0;
+  if (p.sliced) {
+    const int per = p.B * p.bpb;
+    const int kk = lb / per;
+    lb -= kk * per;
+    my_band = p.sl_band0 + kk;
+    band_q0 = (p.sl_ell - kSliceLag * (p.nbands - 1 - my_band)) * kSliceQ;   // blocks of the band already swept
+    m_hi = (my_band + 1) * p.sl_nbb - band_q0;
+    m_lo = m_hi - kSliceQ > my_band * p.sl_nbb ? m_hi - kSliceQ : my_band * p.sl_nbb;
+  }
   const int b = lb / p.bpb;
   const int eg = lb % p.bpb;
   const int e_wg0 = eg * CW;
@@ -798,7 +846,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   char* DXimg = static_cast<char*>(p.dx) + img_bytes;
   char* DDTimg = static_cast<char*>(p.ddT) + img_bytes;
   char* DDLimg = static_cast<char*>(p.ddL) + img_bytes;
-  char* BOTimg = reinterpret_cast<char*>(p.bot + (int64_t)b * p.W * p.E * kN);
+  char* BOTimg = reinterpret_cast<char*>(p.bot + (int64_t)b * p.W * p.E * kN);   // + band * bot_stride
   // per-workgroup channel sums: [channel group][cell][C, B_T, B_L][16]
   char* PARTimg = reinterpret_cast<char*>(p.part + ((int64_t)eg * p.B * p.H * p.W + cell0) * (3 * kN));
 
@@ -806,6 +854,19 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   float muT[kN], muL[kN];
 #pragma unroll
   for (int n = 0; n < kN; ++n) { accAT[n] = 0.f; accAL[n] = 0.f; muT[n] = 0.f; muL[n] = 0.f; }
+  // sliced sweep: adjoint state and position sums travel from launch to launch
+  float* carry = p.sliced ? p.carry + ((((int64_t)b * p.nbands + my_band) * p.E + e) * (4 * kN + 1)) * kHB + r : nullptr;
+  if (p.sliced && band_q0 > 0) {
+    if (ch_ok) {
+#pragma unroll
+      for (int n = 0; n < kN; ++n) {
+        muT[n] = carry[n * kHB]; muL[n] = carry[(kN + n) * kHB];
+        accAT[n] = carry[(2 * kN + n) * kHB]; accAL[n] = carry[(3 * kN + n) * kHB];
+      }
+      accD = carry[4 * kN * kHB];
+    }
+    settle_loads();
+  }
 
   // byte offsets of the lane's operand record inside a staging buffer at step 0 of a block, and
   // its advance per step: a grid row reads (B_T, B_L, C) of its cell; the upper ghost (lane 0)
@@ -863,14 +924,14 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
     return Q;
   };
 
-  Pos A = pos_of(p, (p.nblk - 1) * kCK - (kHB - 1));   // position of the stream index t0 - 15 (wave-uniform)
-  load_ckpt(p.nblk - 1, A);
+  Pos A = pos_of(p, (m_hi - 1) * kCK - (kHB - 1));   // position of the stream index t0 - 15 (wave-uniform)
+  load_ckpt(m_hi - 1, A);
   stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds, b, A, e_wg0, wave, lane, X, DT, DL, DY);
   staging_fence();
   int cur = 0;
   int xpar = 0;   // exchange buffer in use
 
-  for (int m = p.nblk - 1; m >= 0; --m) {
+  for (int m = m_hi - 1; m >= m_lo; --m) {
     const int t0 = m * kCK;
     const char* bufc = lds + cur * SG::kBytes;
     float ck0[kN];
@@ -878,7 +939,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
     for (int n = 0; n < kN; ++n) ck0[n] = cknext[n];
     const Pos Aprev = pos_before(A);
     TICK(ts0);
-    if (m > 0)
+    if (m > m_lo)
       stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, Aprev, e_wg0, wave, lane, X, DT, DL, DY);
     TICK(ts1); TACC(0, ts0, ts1);
     bp = block_pos(p, A, r, ch_ok);
@@ -957,7 +1018,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
         const int t = t0 + k;
         if (half == 1 && k == 0) staging_landed();   // before the last stores of the block, see the forward kernel
         // the states of the later steps are dead by now: their registers take the next snapshot
-        if (half == 1 && k == (kCK > 1 ? 1 : 0) && m > 0) load_ckpt(m - 1, Aprev);
+        if (half == 1 && k == (kCK > 1 ? 1 : 0) && m > m_lo) load_ckpt(m - 1, Aprev);
         if (t < p.T_total) {
           if (per_step_K) band_consts(k >= bp.kw ? bp.bnd0 + 1 : bp.bnd0);
           const bool col0 = bp.kz == k;
@@ -1030,7 +1091,8 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
             const bool wk = k >= bp.kw;
             if (inr && r == 1 && (wk ? bp.bnd0 + 1 : bp.bnd0) >= 1) {
               const int ck = wk ? bp.col0 + k - p.S : bp.col0 + k;
-              char* bb = BOTimg + (uint32_t)(ck * p.E + e) * (uint32_t)(kN * sizeof(float));
+              char* bb = BOTimg + (wk ? bp.bnd0 + 1 : bp.bnd0) * p.bot_stride * (int64_t)sizeof(float) +
+                         (uint32_t)(ck * p.E + e) * (uint32_t)(kN * sizeof(float));
 #pragma unroll
               for (int q = 2 * half; q < 2 * half + 2; ++q)   // the two state groups of this half, as of this step
                 reinterpret_cast<float4*>(bb)[q] = make_float4(muT[sinv<PERM>(4 * q)], muT[sinv<PERM>(4 * q + 1)],
@@ -1078,6 +1140,17 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
     d[6] = clock64() - dbg_t0;
   }
 #endif
+  if (p.sliced && m_lo > my_band * p.sl_nbb) {   // more of the band to come: hand over to the next launch
+    if (ch_ok) {
+#pragma unroll
+      for (int n = 0; n < kN; ++n) {
+        carry[n * kHB] = muT[n]; carry[(kN + n) * kHB] = muL[n];
+        carry[(2 * kN + n) * kHB] = accAT[n]; carry[(3 * kN + n) * kHB] = accAL[n];
+      }
+      carry[4 * kN * kHB] = accD;
+    }
+    return;
+  }
   // ---- sums over positions: reduce over the rows of the band (lanes of one channel slot)
   float red[2 * kN + 1];
 #pragma unroll
@@ -1091,10 +1164,11 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
     red[k] = v;
   }
   if (ch_ok && r == 0) {
-    float* pa = p.pA + ((int64_t)b * p.E + e) * (2 * kN);
+    const int64_t slot_e = ((int64_t)b * p.pa_slots + (p.sliced ? my_band : 0)) * p.E + e;
+    float* pa = p.pA + slot_e * (2 * kN);
 #pragma unroll
     for (int n = 0; n < 2 * kN; ++n) pa[n] = red[n];
-    p.pD[(int64_t)b * p.E + e] = red[2 * kN];
+    p.pD[slot_e] = red[2 * kN];
   }
 }
 
@@ -1159,12 +1233,12 @@ __global__ void m2d_finalize_kernel(const ScanParams p, T* dC, T* dBT, T* dBL, T
   if (k < (int64_t)p.E * 2 * kN) {
     const int e = (int)(k / (2 * kN)), w = (int)(k % (2 * kN));
     float s = 0.f;
-    for (int g = 0; g < p.B; ++g) s += p.pA[((int64_t)g * p.E + e) * (2 * kN) + w];
+    for (int g = 0; g < p.B * p.pa_slots; ++g) s += p.pA[((int64_t)g * p.E + e) * (2 * kN) + w];
     if (w < kN) IO<T>::st(dAT + e * kN + w, s); else IO<T>::st(dAL + e * kN + (w - kN), s);
   }
   if (k < p.E) {
     float s = 0.f;
-    for (int g = 0; g < p.B; ++g) s += p.pD[(int64_t)g * p.E + k];
+    for (int g = 0; g < p.B * p.pa_slots; ++g) s += p.pD[(int64_t)g * p.E + k];
     IO<T>::st(dD + k, s);
   }
 }
@@ -1182,6 +1256,9 @@ struct Geometry {
   int fwd_ec, fwd_wpb, fwd_bpb;      // forward: channels per lane, waves and workgroups per image
   int bwd_wpb, bwd_bpb;              // backward: waves and workgroups (channel groups) per image
   bool stage_x;                      // x, delta, dy rows are whole 16-byte chunks: stage them through LDS
+  bool sliced;                       // bands on workgroups of their own, swept by a sequence of launches
+  int nbb, nlaunch;                  // sliced: blocks per band, launches per sweep
+  size_t carry_fwd_bytes, carry_bwd_bytes;
   size_t prep_bytes, bc_bytes, ckpt_diag_bytes, top_bytes, bot_bytes, part_bytes, pa_bytes, pd_bytes;
 };
 
@@ -1209,6 +1286,20 @@ Geometry make_geometry(const m2d_desc* d) {
   g.S = (g.nbands > 1 && d->W >= 26) ? d->W : (d->W + kHB - 1 > 26 ? d->W + kHB - 1 : 26);
   g.T_total = (g.nbands - 1) * g.S + d->W + g.rows_last;
   g.nblk = (g.T_total + kCK - 1) / kCK;
+  // Few images with many bands leave most of the device idle when each image is one sequential
+  // stream.  Then every band gets workgroups of its own (a padded stream, one window of S steps
+  // per band) and the sweep becomes a sequence of launches in which band k trails band k-1.
+  const int groups = (d->E + kBwdWaves * (64 / kHB) - 1) / (kBwdWaves * (64 / kHB));
+  g.sliced = g.nbands >= 4 && (int64_t)d->B * groups <= 64;
+  g.nbb = 0; g.nlaunch = 1;
+  if (g.sliced) {
+    g.S = (d->W + kHB - 1 + kCK - 1) / kCK * kCK;
+    if (g.S < 28) g.S = 28;
+    g.nbb = g.S / kCK;
+    g.T_total = g.nbands * g.S;
+    g.nblk = g.nbands * g.nbb;
+    g.nlaunch = kSliceLag * (g.nbands - 1) + (g.nbb + kSliceQ - 1) / kSliceQ;
+  }
   // forward: two channels per lane when that still yields enough waves to fill the device
   const bool ec2 = (d->E % 2 == 0) && ((int64_t)d->B * ((d->E + kFwdWaves * g.CS * 2 - 1) / (kFwdWaves * g.CS * 2)) >= 256);
   g.fwd_ec = ec2 ? 2 : 1;
@@ -1222,10 +1313,13 @@ Geometry make_geometry(const m2d_desc* d) {
   g.bc_bytes = align_up(sizeof(float) * P * 48);
   g.ckpt_diag_bytes = align_up(sizeof(float) * (size_t)d->B * g.nblk * d->E * kN * g.HB);
   g.top_bytes = g.nbands > 1 ? align_up(sizeof(float) * (size_t)(g.nbands - 1) * d->B * d->W * d->E * kN) : 0;
-  g.bot_bytes = g.nbands > 1 ? align_up(sizeof(float) * (size_t)d->B * d->W * d->E * kN) : 0;
+  g.bot_bytes = g.nbands > 1 ? align_up(sizeof(float) * (size_t)(g.sliced ? g.nbands : 1) * d->B * d->W * d->E * kN) : 0;
+  g.carry_fwd_bytes = g.sliced ? align_up(sizeof(float) * (size_t)d->B * g.nbands * d->E * kN * kHB) : 0;
+  g.carry_bwd_bytes = g.sliced ? align_up(sizeof(float) * (size_t)d->B * g.nbands * d->E * (4 * kN + 1) * kHB) : 0;
   g.part_bytes = align_up(sizeof(float) * (size_t)g.bwd_bpb * 3 * P * kN);
-  g.pa_bytes = align_up(sizeof(float) * (size_t)d->B * d->E * 2 * kN);
-  g.pd_bytes = align_up(sizeof(float) * (size_t)d->B * d->E);
+  const size_t slots = g.sliced ? g.nbands : 1;
+  g.pa_bytes = align_up(sizeof(float) * (size_t)d->B * slots * d->E * 2 * kN);
+  g.pd_bytes = align_up(sizeof(float) * (size_t)d->B * slots * d->E);
   return g;
 }
 
@@ -1233,11 +1327,11 @@ Geometry make_geometry(const m2d_desc* d) {
 size_t ckpt_bytes_of(const Geometry& g) { return g.ckpt_diag_bytes + g.top_bytes + g.bc_bytes; }
 
 size_t workspace_bytes_of(const Geometry& g, int pass, int have_ckpt) {
-  size_t n = g.prep_bytes;
+  size_t n = g.prep_bytes + g.carry_fwd_bytes;   // (a backward without checkpoints runs a forward sweep first)
   if (pass == M2D_PASS_FWD) {
     if (!have_ckpt) n += g.top_bytes + g.bc_bytes;
   } else {
-    n += g.part_bytes + g.pa_bytes + g.pd_bytes + g.bot_bytes;
+    n += g.part_bytes + g.pa_bytes + g.pd_bytes + g.bot_bytes + g.carry_bwd_bytes;
     if (!have_ckpt) n += ckpt_bytes_of(g);
   }
   return n;
@@ -1250,6 +1344,9 @@ void fill_common(ScanParams& sp, const m2d_desc* d, const Geometry& g) {
   sp.nbands = g.nbands; sp.nblk = g.nblk;
   sp.S = g.S; sp.T_total = g.T_total; sp.rows_last = g.rows_last;
   sp.magicS = (uint32_t)(((uint64_t)1 << 32) / (uint64_t)g.S);
+  sp.sliced = g.sliced ? 1 : 0; sp.sl_nbb = g.nbb; sp.sl_ell = 0; sp.sl_band0 = 0;
+  sp.pa_slots = g.sliced ? g.nbands : 1;
+  sp.bot_stride = g.sliced ? (int64_t)d->B * d->W * d->E * kN : 0;
   sp.flip = (d->flags & M2D_FLAG_FLIP) ? 1 : 0;
 }
 
@@ -1307,9 +1404,25 @@ int launch_fwd(const ScanParams& sp0, const m2d_desc* d, const Geometry& g, bool
   ScanParams sp = sp0;
   sp.bpb = g.fwd_bpb;
   sp.nwg = d->B * g.fwd_bpb;
-  if (g.fwd_ec == 2)
-    return g.stage_x ? launch_fwd_mode<T, 2, true>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 2, false>(sp, ckpt, write_y, st);
-  return g.stage_x ? launch_fwd_mode<T, 1, true>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 1, false>(sp, ckpt, write_y, st);
+  auto once = [&]() {
+    if (g.fwd_ec == 2)
+      return g.stage_x ? launch_fwd_mode<T, 2, true>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 2, false>(sp, ckpt, write_y, st);
+    return g.stage_x ? launch_fwd_mode<T, 1, true>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 1, false>(sp, ckpt, write_y, st);
+  };
+  if (!g.sliced) return once();
+  // launch l advances band k by blocks [(l - lag*k)*Q, +Q) of its window, for the bands under way
+  const int nlb = (g.nbb + kSliceQ - 1) / kSliceQ;
+  for (int l = 0; l < g.nlaunch; ++l) {
+    int k_hi = l / kSliceLag, k_lo = (l - nlb + 1 + kSliceLag - 1) / kSliceLag;
+    if (l - nlb + 1 < 0) k_lo = 0;
+    if (k_hi > g.nbands - 1) k_hi = g.nbands - 1;
+    if (k_lo > k_hi) continue;
+    sp.sl_ell = l; sp.sl_band0 = k_lo;
+    sp.nwg = (k_hi - k_lo + 1) * d->B * g.fwd_bpb;
+    const int rc = once();
+    if (rc) return rc;
+  }
+  return M2D_OK;
 }
 
 template <typename T>
@@ -1318,6 +1431,7 @@ int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   char* w = static_cast<char*>(ws);
   float* prep = reinterpret_cast<float*>(w);
   w += g.prep_bytes;
+  sp.carry = reinterpret_cast<float*>(w); w += g.carry_fwd_bytes;
   char* keep = ckpt ? static_cast<char*>(ckpt) + g.ckpt_diag_bytes : w;   // [top][widened B,C]
   sp.ckpt = ckpt ? static_cast<float*>(ckpt) : nullptr;
   sp.top = reinterpret_cast<float*>(keep);
@@ -1352,6 +1466,8 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
             void* dBL, void* dC, void* dD, void* ws, hipStream_t st) {
   char* w = static_cast<char*>(ws);
   float* prep = reinterpret_cast<float*>(w); w += g.prep_bytes;
+  float* carry_fwd = reinterpret_cast<float*>(w); w += g.carry_fwd_bytes;
+  float* carry_bwd = reinterpret_cast<float*>(w); w += g.carry_bwd_bytes;
   sp.part = reinterpret_cast<float*>(w); w += g.part_bytes;
   sp.pA = reinterpret_cast<float*>(w); w += g.pa_bytes;
   sp.pD = reinterpret_cast<float*>(w); w += g.pd_bytes;
@@ -1364,13 +1480,29 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   rc = stage_bc<T>(sp, d, BT, BL, C, reinterpret_cast<float*>(ck + g.ckpt_diag_bytes + g.top_bytes), ckpt != nullptr, st);
   if (rc) return rc;
   if (!ckpt) {   // rebuild the checkpoints with one forward sweep that writes no y
+    sp.carry = carry_fwd;
     rc = launch_fwd<T>(sp, d, g, true, false, st);
     if (rc) return rc;
   }
+  sp.carry = carry_bwd;
   sp.bpb = g.bwd_bpb;
   sp.nwg = d->B * g.bwd_bpb;
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][0], st);
-  rc = g.stage_x ? launch_bwd<T, true>(sp, st) : launch_bwd<T, false>(sp, st);
+  if (!g.sliced) {
+    rc = g.stage_x ? launch_bwd<T, true>(sp, st) : launch_bwd<T, false>(sp, st);
+  } else {
+    // as the forward, bottom-up: launch l advances the band k' from the bottom by Q blocks of its window
+    const int nlb = (g.nbb + kSliceQ - 1) / kSliceQ;
+    for (int l = 0; l < g.nlaunch && !rc; ++l) {
+      int k_hi = l / kSliceLag, k_lo = (l - nlb + 1 + kSliceLag - 1) / kSliceLag;
+      if (l - nlb + 1 < 0) k_lo = 0;
+      if (k_hi > g.nbands - 1) k_hi = g.nbands - 1;
+      if (k_lo > k_hi) continue;
+      sp.sl_ell = l; sp.sl_band0 = g.nbands - 1 - k_hi;
+      sp.nwg = (k_hi - k_lo + 1) * d->B * g.bwd_bpb;
+      rc = g.stage_x ? launch_bwd<T, true>(sp, st) : launch_bwd<T, false>(sp, st);
+    }
+  }
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][1], st);
   if (rc) return rc;
   const int64_t P = (int64_t)d->B * d->H * d->W;
