@@ -169,6 +169,8 @@ def main():
         ks.append(cabi.profile_last_ms(cabi.M2D_PASS_BWD))
     bwd_kernel = sum(ks) / len(ks)
 
+    peak_mem = torch.cuda.max_memory_allocated()
+    input_bytes = sum(t.numel() * t.element_size() for t in leaves) + dy.numel() * dy.element_size()
     s = 2 if dts == "bf16" else 4
     fb, bb = algorithmic_bytes(B, E, H, W, s)
     achieved = bb / (bwd_kernel * 1e-3) / 1e9
@@ -190,6 +192,8 @@ def main():
         "fwd_ms": round(fwd_ms, 4),
         "fwd_bwd_ms": round(step_ms, 4),
         "wall_ms_per_step": round(t_wall, 4),
+        "peak_hbm_bytes": int(peak_mem),          # torch allocator peak: inputs, outputs, gradients, checkpoints, scratch
+        "input_bytes": int(input_bytes),
         "pct_hbm_roofline": {
             "fwd": round(100 * fb / (fwd_ms * 1e-3) / (HBM_PEAK_GBS * 1e9), 2),
             "fwd_bwd": round(100 * (fb + bb) / (step_ms * 1e-3) / (HBM_PEAK_GBS * 1e9), 2),

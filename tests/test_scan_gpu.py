@@ -70,21 +70,23 @@ def run_case(cabi, cscan, B, H, W, E, dtype, seed=0, flip=False, with_ckpt=True,
 
 
 SHAPES = [
-    # B, H, W, E      what it exercises
-    (2, 14, 14, 32),  # benchmark config 0
-    (3, 5, 9, 4),     # ragged: 8-lane slots, batch not filling the wave
-    (9, 7, 7, 6),     # 7x7 stage shape, two problem groups
-    (5, 2, 2, 2),     # smallest legal grid, 2-lane slots
-    (2, 28, 28, 8),   # 32-lane slots
-    (1, 56, 56, 4),   # stage-1 spatial size, one 64-lane slot
-    (2, 33, 40, 2),   # 64-lane slot partly filled
-    (1, 10, 60, 2),   # wide
-    (1, 60, 10, 3),   # tall, odd channel count (one channel per wave)
-    (1, 70, 50, 2),   # two bands of rows
-    (2, 130, 20, 2),  # three bands, last one 2 rows
+    # B, H, W, E      what it exercises (bands are 14 rows; a wave holds 4 channels of one image)
+    (2, 14, 14, 32),  # benchmark config 0: one full band
+    (3, 5, 9, 4),     # ragged: short band, one wave partly filled
+    (9, 7, 7, 6),     # 7x7 stage shape, channels not filling the second wave
+    (5, 2, 2, 2),     # smallest legal grid
+    (2, 28, 28, 8),   # two bands run back to back in one stream (W >= 26)
+    (1, 56, 56, 4),   # stage-1 spatial size: four bands, one image -> sequence of launches
+    (2, 33, 40, 2),   # three bands back to back, last one 5 rows
+    (1, 10, 60, 2),   # wide single band
+    (1, 60, 10, 3),   # tall and narrow: five padded bands, odd channel count
+    (1, 70, 50, 2),   # five bands of one image
+    (2, 130, 20, 2),  # ten bands, last one 4 rows, padded windows
     (1, 64, 17, 10),  # channels not a multiple of the workgroup
-    (1, 40, 4, 3),    # three bands narrower than 8 columns: every band restarts the pipeline
-    (2, 31, 8, 2),    # narrowest grid whose bands are streamed back to back
+    (1, 40, 4, 3),    # three bands narrower than the pipeline is deep
+    (2, 31, 8, 2),    # three bands in one padded stream
+    (1, 150, 90, 8),  # 11 bands, one image: every band on workgroups of its own, swept by a sequence of launches
+    (70, 56, 30, 4),  # four bands back to back, more images than the sliced sweep takes
 ]
 
 
