@@ -35,6 +35,7 @@ WORKLOADS = {
     "hires1024": (1, 64, 1024, 1024, "f32"),
     "hires2048": (1, 64, 2048, 2048, "f32"),
     "cfg0": (2, 32, 14, 14, "f32"),
+    "cfg3": None,   # M2D-T backbone inference, handled by backbone_inference()
 }
 N = 16
 HBM_PEAK_GBS = 8000.0
@@ -83,6 +84,58 @@ def cpu_baseline(B, E, H, W, budget_s=20.0):
     }
 
 
+def backbone_inference(args):
+    """M2D-T backbone (blocks [3,3,9,3], channels [64,128,320,512], scan mixers with local path at
+    stages 1-2, rotary attention at stages 3-4, odd blocks scanning from the bottom-right corner),
+    random weights, B=128 images of 3x224x224, inference.  One step = one batch."""
+    import torch
+    from mamba2d_amd import cabi
+    from mamba2d_amd.backbone import Mamba2DBackbone, M2D_T
+    dev = torch.device("cuda:0")
+    torch.manual_seed(0)
+    B = 128
+    net = Mamba2DBackbone(**M2D_T).to(dev).eval()
+    x = torch.randn(B, 3, 224, 224, device=dev)
+    cabi.profile_enable(True)
+
+    def run(model, inp, autocast):
+        with torch.no_grad(), torch.autocast("cuda", dtype=torch.bfloat16, enabled=autocast):
+            return model(inp)
+
+    def timed(model, inp, autocast):
+        for _ in range(args.warmup):
+            run(model, inp, autocast)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            run(model, inp, autocast)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps
+
+    ms_autocast = timed(net, x, True)                  # fp32 weights, bf16 autocast (the reference's bf16-mixed)
+    scan_ms = cabi.profile_last_ms(cabi.M2D_PASS_FWD)  # last scan of the batch: stage 2, 28x28x128
+    net16 = net.to(torch.bfloat16)
+    ms_bf16 = timed(net16, x.to(torch.bfloat16), False)
+    out = {
+        "metric": "M2D-T backbone inference images/sec at 224x224, B=128",
+        "value": round(B / (ms_bf16 * 1e-3), 1),
+        "unit": "images/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_bf16, 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": "cfg3: M2D-T backbone, blocks [3,3,9,3], channels [64,128,320,512], B=128 x 3x224x224, "
+                               "random init, 6 scans (3 at 56x56x64, 3 at 28x28x128, odd blocks bottom-right)"},
+        "images_per_s_bf16_weights": round(B / (ms_bf16 * 1e-3), 1),
+        "images_per_s_autocast_fp32_weights": round(B / (ms_autocast * 1e-3), 1),
+        "last_scan_kernel_ms": round(scan_ms, 4),
+        "roofline": None, "cpu_baseline": None,
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -106,6 +159,9 @@ def main():
         sys.exit(1)
     from mamba2d_amd import cabi, wavefront
 
+    if args.workload == "cfg3":
+        backbone_inference(args)
+        return
     B, E, H, W, dts = WORKLOADS[args.workload]
     dtype = torch.bfloat16 if dts == "bf16" else torch.float32
     if args.no_ckpt:

@@ -1,0 +1,279 @@
+"""M2D backbone around the MI355X scan, for measuring the scan inside a whole model.
+
+The module tree and parameter names follow the reference backbone (``models/mamba2d.py:16-386``,
+``models/utils.py:7-233``) so that a reference state dict maps onto it key by key:
+``ds.{stem,ds1,ds2,ds3}.conv.*``, ``ds.stem.post_norm.norm.*``, ``stages.{s}.{k}.{norm1,norm2}.*``,
+``stages.{s}.{k}.token_mixer.{in_proj,out_proj,x_proj,dt_projT,dt_projL,AT_log,AL_log,D,
+local_norm,local_path.*}`` or ``.token_mixer.{qkv,proj,q_norm,k_norm}.*``,
+``stages.{s}.{k}.res_scale{1,2}.scale``, ``stages.{s}.{k}.MLP.{fc1,fc2}.*`` and the stage
+post-norm ``stages.{s}.{n_blocks}.*``.
+
+Differences in how it runs (not in what it computes):
+  * activations stay channel-last from stem to head; convolutions see them as NCHW views in
+    ``torch.channels_last`` memory format, so there are no layout copies between stages;
+  * a block that scans from the bottom-right corner passes ``flip=True`` to the scan instead of
+    flipping its input and output (``models/mamba2d.py:163-173``): every other operator of the block
+    acts per cell and commutes with the flip;
+  * the rotary tables of the attention stages are built once per grid size.
+"""
+import math
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from .wavefront import wavefront_scan_cuda
+
+M2D_T = dict(n_blocks=(3, 3, 9, 3), embed_dim=(64, 128, 320, 512),
+             token_mixer=("2D_local", "2D_local", "RopeAttention", "RopeAttention"),
+             res_scale_init_values=(1.0, 1.0, 1.0, 1.0), inter_flip=True, drop_path_rate=0.175)
+
+
+class LayerNorm2D(nn.Module):
+    """LayerNorm over channels of a channel-last tensor (kept as a module with a ``norm`` child for
+    the parameter names, ``models/utils.py:7-18``)."""
+
+    def __init__(self, dim):
+        super().__init__()
+        self.norm = nn.LayerNorm(dim)
+
+    def forward(self, x):           # (B, H, W, C)
+        return self.norm(x)
+
+
+class StarReLU(nn.Module):
+    """scale * relu(x)^2 + bias with scalar parameters (``models/utils.py:22-37``)."""
+
+    def __init__(self):
+        super().__init__()
+        self.scale = nn.Parameter(torch.ones(1))
+        self.bias = nn.Parameter(torch.zeros(1))
+
+    def forward(self, x):
+        return torch.addcmul(self.bias, self.scale, F.relu(x).square())
+
+
+class Scale(nn.Module):
+    def __init__(self, dim, init_value=1.0):
+        super().__init__()
+        self.scale = nn.Parameter(init_value * torch.ones(dim))
+
+    def forward(self, x):
+        return x * self.scale
+
+
+class MLP(nn.Module):
+    def __init__(self, dim, expand=4):
+        super().__init__()
+        self.fc1 = nn.Linear(dim, dim * expand)
+        self.fc2 = nn.Linear(dim * expand, dim)
+
+    def forward(self, x):
+        return self.fc2(F.gelu(self.fc1(x)))
+
+
+def _conv_channel_last(conv, x):
+    """conv on a (B, H, W, C) tensor without a layout copy: the NCHW view of a channel-last tensor
+    is already in channels_last memory format; the result is handed back as (B, H', W', C')."""
+    y = conv(x.permute(0, 3, 1, 2))
+    return y.permute(0, 2, 3, 1)
+
+
+class SepConv(nn.Module):
+    """pointwise -> StarReLU -> depthwise 3x3 -> StarReLU -> pointwise, no bias
+    (``models/utils.py:83-113`` as configured at ``models/mamba2d.py:57-60``)."""
+
+    def __init__(self, dim, expansion=2, kernel_size=3, padding=1):
+        super().__init__()
+        med = int(expansion * dim)
+        self.pwconv1 = nn.Linear(dim, med, bias=False)
+        self.act1 = StarReLU()
+        self.dwconv = nn.Conv2d(med, med, kernel_size, padding=padding, groups=med, bias=False)
+        self.act2 = StarReLU()
+        self.pwconv2 = nn.Linear(med, dim, bias=False)
+
+    def forward(self, x):
+        x = self.act1(self.pwconv1(x))
+        x = _conv_channel_last(self.dwconv, x)
+        return self.pwconv2(self.act2(x))
+
+
+class Downsampling(nn.Module):
+    """Strided convolution with an optional norm after it (``models/utils.py:116-136``)."""
+
+    def __init__(self, cin, cout, kernel_size, stride, padding, post_norm=False):
+        super().__init__()
+        self.conv = nn.Conv2d(cin, cout, kernel_size, stride=stride, padding=padding)
+        self.post_norm = LayerNorm2D(cout) if post_norm else nn.Identity()
+
+    def forward(self, x):           # channel-last in, channel-last out
+        return self.post_norm(_conv_channel_last(self.conv, x))
+
+
+class M2DBlock(nn.Module):
+    """Token mixer: in_proj -> GELU -> 2-D selective scan -> GELU -> out_proj, plus an optional local
+    convolution path on the normalised input (``models/mamba2d.py:16-188``).  Parameter
+    initialisation follows ``models/mamba2d.py:66-111``: dt log-uniform in [dt_min, dt_max] through
+    the inverse softplus into the dt biases, A = 1..N (S4D-real), D = 1."""
+
+    def __init__(self, d_model, d_state=16, dt_min=1e-3, dt_max=1e-1, dt_init_floor=1e-4,
+                 local_path=False, scan_start="TL", recomp="partial"):
+        super().__init__()
+        if scan_start not in ("TL", "BR"):
+            raise ValueError(f"Invalid Scan Direction, expected TL or BR and got {scan_start}")
+        self.flip = scan_start == "BR"
+        self.recomp = recomp
+        self.dt_rank = math.ceil(d_model / 16)
+        self.local_norm = nn.LayerNorm(d_model) if local_path else None
+        self.local_path = SepConv(d_model) if local_path else None
+        self.in_proj = nn.Linear(d_model, d_model)
+        self.x_proj = nn.Linear(d_model, 2 * self.dt_rank + 3 * d_state, bias=False)
+        self.dt_projT = nn.Linear(self.dt_rank, d_model)
+        self.dt_projL = nn.Linear(self.dt_rank, d_model)
+        std = self.dt_rank ** -0.5
+        nn.init.uniform_(self.dt_projT.weight, -std, std)
+        nn.init.uniform_(self.dt_projL.weight, -std, std)
+        dt = torch.exp(torch.rand(d_model) * (math.log(dt_max) - math.log(dt_min)) + math.log(dt_min)).clamp(min=dt_init_floor)
+        inv_softplus = dt + torch.log(-torch.expm1(-dt))
+        with torch.no_grad():
+            self.dt_projT.bias.copy_(inv_softplus)
+            self.dt_projL.bias.copy_(inv_softplus)
+        a = torch.log(torch.arange(1, d_state + 1, dtype=torch.float32)).repeat(d_model, 1)
+        self.AT_log = nn.Parameter(a.clone())
+        self.AL_log = nn.Parameter(a.clone())
+        self.D = nn.Parameter(torch.ones(d_model))
+        for prm in (self.AT_log, self.AL_log, self.D):
+            prm._no_weight_decay = True
+        self.out_proj = nn.Linear(d_model, d_model)
+
+    def forward(self, x):           # (B, H, W, C)
+        local = self.local_path(self.local_norm(x)) if self.local_path is not None else None
+        u = F.gelu(self.in_proj(x))
+        y = wavefront_scan_cuda(u, self.AT_log, self.AL_log, self.x_proj.weight,
+                                self.dt_projT.weight, self.dt_projT.bias,
+                                self.dt_projL.weight, self.dt_projL.bias, self.D, self.recomp, flip=self.flip)
+        y = self.out_proj(F.gelu(y))
+        return y if local is None else y + local
+
+
+class RoPEAttention2D(nn.Module):
+    """Multi-head self-attention over the H*W cells with rotary embeddings on the two grid axes
+    (``models/utils.py:165-316``): the first quarter of every head rotates with the row index, the
+    second with the column index, the rest is left alone; q and k are layer-normed per head."""
+
+    def __init__(self, dim, head_dim=32, rope_base=10000.0):
+        super().__init__()
+        self.head_dim = head_dim
+        self.num_heads = max(dim // head_dim, 1)
+        inner = self.num_heads * head_dim
+        self.qkv = nn.Linear(dim, 3 * inner, bias=False)
+        self.proj = nn.Linear(inner, dim, bias=False)
+        self.q_norm = nn.LayerNorm(head_dim)
+        self.k_norm = nn.LayerNorm(head_dim)
+        self.axis_dim = (head_dim // 2 // 2) * 2        # rotated dims per axis
+        self.rope_base = rope_base
+        self._tables = {}
+
+    def _rope_tables(self, H, W, device, dtype):
+        key = (H, W, str(device), dtype)
+        if key not in self._tables:
+            d = self.axis_dim
+            inv_freq = 1.0 / (self.rope_base ** (torch.arange(0, d // 2, device=device, dtype=torch.float32) / (d // 2)))
+            rows = torch.arange(H, device=device, dtype=torch.float32).repeat_interleave(W)
+            cols = torch.arange(W, device=device, dtype=torch.float32).repeat(H)
+            ang = torch.cat([rows[:, None] * inv_freq, cols[:, None] * inv_freq], dim=-1)   # (HW, d)
+            ang = ang.repeat_interleave(2, dim=-1)                                           # pairs share an angle
+            # layout per head: [row-rotated d | column-rotated d | untouched]
+            cos = torch.ones(H * W, self.head_dim, device=device)
+            sin = torch.zeros(H * W, self.head_dim, device=device)
+            cos[:, :2 * d] = torch.cat([ang[:, 0:d].cos(), ang[:, d:2 * d].cos()], dim=-1)
+            sin[:, :2 * d] = torch.cat([ang[:, 0:d].sin(), ang[:, d:2 * d].sin()], dim=-1)
+            self._tables[key] = (cos.to(dtype), sin.to(dtype))
+        return self._tables[key]
+
+    @staticmethod
+    def _rotate_pairs(t):
+        a, b = t.unflatten(-1, (-1, 2)).unbind(-1)
+        return torch.stack((-b, a), dim=-1).flatten(-2)
+
+    def forward(self, x):           # (B, H, W, C)
+        B, H, W, _ = x.shape
+        qkv = self.qkv(x).view(B, H * W, 3, self.num_heads, self.head_dim).permute(2, 0, 3, 1, 4)
+        q, k, v = qkv.unbind(0)     # (B, heads, HW, head_dim)
+        cos, sin = self._rope_tables(H, W, x.device, q.dtype)
+        q = q * cos + self._rotate_pairs(q) * sin      # sin is zero on the untouched dims
+        k = k * cos + self._rotate_pairs(k) * sin
+        q, k = self.q_norm(q), self.k_norm(k)
+        o = F.scaled_dot_product_attention(q, k, v, scale=self.head_dim ** -0.5)
+        return self.proj(o.transpose(1, 2).reshape(B, H, W, self.num_heads * self.head_dim))
+
+
+def _drop_path(x, p, training):
+    if p == 0.0 or not training:
+        return x
+    keep = torch.rand(x.shape[0], *([1] * (x.ndim - 1)), device=x.device) >= p
+    return x * keep.to(x.dtype) / (1.0 - p)
+
+
+class ResBlock(nn.Module):
+    """x <- s1*x + mixer(norm1 x);  x <- s2*x + MLP(norm2 x)  (``models/mamba2d.py:191-254``)."""
+
+    def __init__(self, dim, token_mixer="2D", mlp_expand_factor=4, drop_path=0.0, res_scale_init_value=None,
+                 scan_start="TL", recomp="partial"):
+        super().__init__()
+        self.norm1 = nn.LayerNorm(dim)
+        if token_mixer == "2D":
+            self.token_mixer = M2DBlock(dim, scan_start=scan_start, recomp=recomp)
+        elif token_mixer == "2D_local":
+            self.token_mixer = M2DBlock(dim, scan_start=scan_start, recomp=recomp, local_path=True)
+        elif token_mixer == "RopeAttention":
+            self.token_mixer = RoPEAttention2D(dim)
+        else:
+            raise ValueError(f"Invalid token mixer type: {token_mixer}")
+        self.res_scale1 = Scale(dim, res_scale_init_value) if res_scale_init_value else nn.Identity()
+        self.norm2 = nn.LayerNorm(dim)
+        self.MLP = MLP(dim, mlp_expand_factor)
+        self.res_scale2 = Scale(dim, res_scale_init_value) if res_scale_init_value else nn.Identity()
+        self.drop_path = float(drop_path)
+
+    def forward(self, x):
+        x = self.res_scale1(x) + _drop_path(self.token_mixer(self.norm1(x)), self.drop_path, self.training)
+        return self.res_scale2(x) + _drop_path(self.MLP(self.norm2(x)), self.drop_path, self.training)
+
+
+class Mamba2DBackbone(nn.Module):
+    """Stem (k7 s4 p2 + norm), then per stage a k3 s2 p1 downsampling (from the second stage on),
+    ``n_blocks`` residual blocks and a LayerNorm (``models/mamba2d.py:256-386``).  Takes
+    (B, 3, H, W) images, returns the last stage's features as (B, C, H/32, W/32)."""
+
+    def __init__(self, in_channels=3, n_blocks=(3, 3, 9, 3), embed_dim=(64, 128, 320, 512),
+                 token_mixer=("2D_local", "2D_local", "RopeAttention", "RopeAttention"),
+                 drop_path_rate=0.1, res_scale_init_values=(None, None, 1.0, 1.0), inter_flip=False,
+                 recomp="partial"):
+        super().__init__()
+        if not (len(n_blocks) == len(embed_dim) == len(token_mixer) == len(res_scale_init_values)):
+            raise ValueError("Check backbone init_args are defined for each stage!")
+        self.ds = nn.ModuleDict()
+        for i, dim in enumerate(embed_dim):
+            if i == 0:
+                self.ds["stem"] = Downsampling(in_channels, dim, 7, 4, 2, post_norm=True)
+            else:
+                self.ds[f"ds{i}"] = Downsampling(embed_dim[i - 1], dim, 3, 2, 1)
+        total = sum(n_blocks)
+        rates = [drop_path_rate * k / max(total - 1, 1) for k in range(total)]
+        self.stages = nn.ModuleDict()
+        done = 0
+        for i, (n, dim) in enumerate(zip(n_blocks, embed_dim)):
+            blocks = [ResBlock(dim, token_mixer[i], drop_path=rates[done + k],
+                               res_scale_init_value=res_scale_init_values[i],
+                               scan_start="BR" if inter_flip and k % 2 == 1 else "TL", recomp=recomp)
+                      for k in range(n)]
+            blocks.append(nn.LayerNorm(dim))
+            self.stages[str(i)] = nn.Sequential(*blocks)
+            done += n
+
+    def forward(self, x):
+        x = x.permute(0, 2, 3, 1)                      # channel-last view; the stem makes it real
+        for ds, stage in zip(self.ds.values(), self.stages.values()):
+            x = stage(ds(x).contiguous())
+        return x.permute(0, 3, 1, 2)

@@ -76,23 +76,26 @@ def _c(t):
 class wf_cuda_fn_pr(torch.autograd.Function):
     """Scan + output projection on precomputed parameters (reference ``wavefront_cuda.py:146-196``).
 
-    ``apply(x, deltaT, deltaL, AT, AL, BT, BL, C, D) -> y``; backward returns the nine
-    gradients in input order."""
+    ``apply(x, deltaT, deltaL, AT, AL, BT, BL, C, D[, flip]) -> y``; backward returns the nine
+    gradients in input order.  ``flip=True`` (not in the reference) scans from the bottom-right
+    corner, which equals flipping every spatial tensor before and y after
+    (``models/mamba2d.py:163-173``) without the copies."""
 
     @staticmethod
-    def forward(ctx, x, deltaT, deltaL, AT, AL, BT, BL, C, D):
+    def forward(ctx, x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip=False):
         args = [_c(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D)]
         # (grad mode is always off inside forward(); needs_input_grad is what tells training from inference)
         keep = SAVE_CHECKPOINTS and any(ctx.needs_input_grad)
-        y, ck = scan_fwd_op(*args, keep, False)
+        y, ck = scan_fwd_op(*args, keep, bool(flip))
         ctx.save_for_backward(*args, ck)
+        ctx.flip = bool(flip)
         return y
 
     @staticmethod
     def backward(ctx, grad_output):
         *args, ck = ctx.saved_tensors
         dy = _c(grad_output.to(args[0].dtype))
-        return tuple(scan_bwd_op(*args, dy, ck, False))
+        return (*scan_bwd_op(*args, dy, ck, ctx.flip), None)
 
 
 class wf_cuda_fn_fr(torch.autograd.Function):
@@ -100,13 +103,14 @@ class wf_cuda_fn_fr(torch.autograd.Function):
     are saved; projections, checkpoints and states are rebuilt in the backward."""
 
     @staticmethod
-    def forward(ctx, x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D):
+    def forward(ctx, x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D, flip=False):
         with torch.no_grad():
             deltaT, deltaL, AT, AL, BT, BL, C = proj_params(
                 x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b)
             y, _ = scan_fwd_op(_c(x), _c(deltaT), _c(deltaL), _c(AT), _c(AL), _c(BT), _c(BL), _c(C), _c(D),
-                               False, False)
+                               False, bool(flip))
         ctx.save_for_backward(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D)
+        ctx.flip = bool(flip)
         return y
 
     @staticmethod
@@ -120,19 +124,20 @@ class wf_cuda_fn_fr(torch.autograd.Function):
         det = [_c(t.detach()) for t in (deltaT, deltaL, AT, AL, BT, BL, C)]
         none = x.new_empty((1,), dtype=torch.uint8)
         d_x_scan, d_dT, d_dL, d_AT, d_AL, d_BT, d_BL, d_C, d_D = scan_bwd_op(
-            _c(x), det[0], det[1], det[2], det[3], det[4], det[5], det[6], _c(D), dy, none, False)
+            _c(x), det[0], det[1], det[2], det[3], det[4], det[5], det[6], _c(D), dy, none, ctx.flip)
         grads = torch.autograd.grad([deltaT, deltaL, BT, BL, C, AT, AL], leaves,
                                     [d_dT, d_dL, d_BT, d_BL, d_C, d_AT, d_AL])
         d_x = d_x_scan + grads[0]   # d_x_scan already contains dy*D
-        return (d_x, *grads[1:], d_D)
+        return (d_x, *grads[1:], d_D, None)
 
 
 def wavefront_scan_cuda(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D,
-                        recomp="partial"):
+                        recomp="partial", flip=False):
     """Entry point with the reference's signature (``wavefront_cuda.py:315-347``).
 
     recomp: 'partial' computes the projections once (autograd-tracked) and runs the scan on them;
             'full' recomputes the projections in the backward (minimal saved memory).
+    flip:   (not in the reference) scan from the bottom-right corner by index arithmetic.
     """
     _, H, W, _ = x.shape
     if H < 2 or W < 2:
@@ -148,8 +153,8 @@ def wavefront_scan_cuda(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_
     if recomp == "partial":
         deltaT, deltaL, AT, AL, BT, BL, C = proj_params(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b,
                                                         dt_projL_w, dt_projL_b)
-        return wf_cuda_fn_pr.apply(x, deltaT, deltaL, AT, AL, BT, BL, C, D)
+        return wf_cuda_fn_pr.apply(x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip)
     if recomp == "full":
         return wf_cuda_fn_fr.apply(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w,
-                                   dt_projL_b, D)
+                                   dt_projL_b, D, flip)
     raise ValueError(f"Unknown recomputation mode, got {recomp}...")
