@@ -38,7 +38,8 @@ typedef enum m2d_status {
   M2D_OK = 0,
   M2D_ERR_NULL_POINTER = 1,   /* a required pointer argument is NULL */
   M2D_ERR_BAD_SHAPE = 2,      /* a dimension is < 1, or H < 2 or W < 2 (reference: wavefront_cuda.py:323-324) */
-  M2D_ERR_UNSUPPORTED = 3,    /* dtype / N outside what the kernels are built for */
+  M2D_ERR_UNSUPPORTED = 3,    /* dtype / N outside what the kernels are built for, or one image too large
+                                 for 32-bit offsets (H*W >= 2^24 cells or H*W*E >= 2^30 elements) */
   M2D_ERR_WORKSPACE = 4,      /* workspace or checkpoint buffer smaller than required */
   M2D_ERR_MISALIGNED = 5,     /* a tensor pointer is not 16-byte aligned / workspace not 256-byte aligned */
   M2D_ERR_HIP = 6             /* a HIP runtime call or kernel launch failed */

@@ -1269,6 +1269,9 @@ int check_desc(const m2d_desc* d) {
   if (d->dtype != M2D_F32 && d->dtype != M2D_BF16) return M2D_ERR_UNSUPPORTED;
   if (d->reserved != 0 || (d->flags & ~M2D_FLAG_FLIP)) return M2D_ERR_UNSUPPORTED;
   if ((int64_t)d->B * d->H * d->W >= ((int64_t)1 << 40)) return M2D_ERR_BAD_SHAPE;
+  // one image is addressed with 32-bit byte offsets from its base (fp32: 4 bytes per element;
+  // the widest per-cell record, the channel sums, is 192 bytes)
+  if ((int64_t)d->H * d->W * d->E >= ((int64_t)1 << 30) || (int64_t)d->H * d->W >= ((int64_t)1 << 24)) return M2D_ERR_UNSUPPORTED;
   return M2D_OK;
 }
 
@@ -1533,7 +1536,7 @@ const char* m2d_status_str(int status) {
     case M2D_OK: return "ok";
     case M2D_ERR_NULL_POINTER: return "null pointer argument";
     case M2D_ERR_BAD_SHAPE: return "bad shape (all dims >= 1, H >= 2, W >= 2 required)";
-    case M2D_ERR_UNSUPPORTED: return "unsupported dtype, d_state or flags (this build: f32/bf16, N=16)";
+    case M2D_ERR_UNSUPPORTED: return "unsupported dtype, d_state, flags or image size (this build: f32/bf16, N=16, H*W < 2^24, H*W*E < 2^30)";
     case M2D_ERR_WORKSPACE: return "workspace or checkpoint buffer too small";
     case M2D_ERR_MISALIGNED: return "misaligned pointer (tensors 16 B, workspace/checkpoints 256 B)";
     case M2D_ERR_HIP: return "HIP runtime error";

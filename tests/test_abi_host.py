@@ -52,6 +52,9 @@ def test_descriptor_validation(cabi):
     assert chk(D(cabi, H=1)) == 2 and chk(D(cabi, W=1)) == 2 and chk(D(cabi, B=0)) == 2
     assert chk(D(cabi, N=8)) == 3 and chk(D(cabi, dtype=7)) == 3 and chk(D(cabi, flags=4)) == 3
     assert chk(D(cabi, reserved=1)) == 3
+    # one image must fit 32-bit offsets: H*W < 2^24 cells, H*W*E < 2^30 elements
+    assert chk(D(cabi, B=1, H=4096, W=4096, E=8)) == 3 and chk(D(cabi, B=1, H=2048, W=2048, E=256)) == 3
+    assert chk(D(cabi, B=1, H=2048, W=2048, E=64)) == 0 and chk(D(cabi, B=4, H=4000, W=4000, E=32)) == 0
 
 
 def test_argument_validation_happens_before_any_launch(cabi):
