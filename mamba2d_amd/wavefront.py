@@ -132,7 +132,7 @@ class wf_cuda_fn_fr(torch.autograd.Function):
 
 
 def wavefront_scan_cuda(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D,
-                        recomp="partial", flip=False):
+                        recomp="partial", *, flip=False):
     """Entry point with the reference's signature (``wavefront_cuda.py:315-347``).
 
     recomp: 'partial' computes the projections once (autograd-tracked) and runs the scan on them;

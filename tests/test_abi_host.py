@@ -106,9 +106,13 @@ def test_python_surface_matches_reference_names():
         assert hasattr(w, name)
     import inspect
     sig = inspect.signature(w.wavefront_scan_cuda)
-    assert list(sig.parameters) == ["x", "AT_log", "AL_log", "x_proj_w", "dt_projT_w", "dt_projT_b",
-                                    "dt_projL_w", "dt_projL_b", "D", "recomp"]
+    positional = [n for n, q in sig.parameters.items() if q.kind is not inspect.Parameter.KEYWORD_ONLY]
+    assert positional == ["x", "AT_log", "AL_log", "x_proj_w", "dt_projT_w", "dt_projT_b",
+                          "dt_projL_w", "dt_projL_b", "D", "recomp"]
     assert sig.parameters["recomp"].default == "partial"
+    # anything beyond the reference's signature is keyword-only and off by default
+    extras = {n: q.default for n, q in sig.parameters.items() if q.kind is inspect.Parameter.KEYWORD_ONLY}
+    assert extras == {"flip": False}
 
 
 def test_entry_point_errors_match_reference():
