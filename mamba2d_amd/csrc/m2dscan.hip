@@ -56,15 +56,6 @@ constexpr int kSliceLag = 2;       // sliced sweep: launches by which a band tra
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
-#ifdef M2D_X_TIMING
-__device__ long long g_dbg[4096 * 8];
-#define TICK(var) const long long var = clock64()
-#define TACC(slot, a, b) dbg_acc[slot] += (b) - (a)
-#else
-#define TICK(var)
-#define TACC(slot, a, b)
-#endif
-
 struct bf16_t { uint16_t v; };
 typedef float v4f_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) v4f_t lds_float4;   // a float4 known to live in LDS
@@ -128,11 +119,7 @@ __device__ __forceinline__ float from_row_below(float v) {
 __device__ __forceinline__ float from_row_above(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x101 /*row_shl:1*/, 0xf, 0xf, true));
 }
-#ifdef M2D_X_NOEXP
-__device__ __forceinline__ float fexp2(float v) { return v * 0.001f; }
-#else
 __device__ __forceinline__ float fexp2(float v) { return __builtin_amdgcn_exp2f(v); }
-#endif
 
 // a[lanes 32..63] <-> b[lanes 0..31]; returns a+b: lanes 0..31 hold the two-half sum of a,
 // lanes 32..63 that of b.
@@ -336,9 +323,6 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan
   using SG = Stage<T, NT, CW, WITH_BOT, UNI>;
   using PL = StagePlan<T, NT, CW, WITH_BOT, UNI, NWAVES, KEEP>;
   static_assert((SG::kCpt & (SG::kCpt - 1)) == 0, "chunks per tensor row must be a power of two");
-#ifdef M2D_X_NOSTAGE
-  return;
-#endif
   const int64_t img = (int64_t)b * p.H * p.W;
 #pragma unroll
   for (int i = 0; i < PL::kItB; ++i) {
@@ -536,10 +520,6 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
 
   settle_loads();
   __syncthreads();
-#ifdef M2D_X_TIMING
-  long long dbg_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  const long long dbg_t0 = clock64();
-#endif
   const T* X = static_cast<const T*>(p.x);
   const T* DT = static_cast<const T*>(p.dT);
   const T* DL = static_cast<const T*>(p.dL);
@@ -682,10 +662,8 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   for (int m = m_lo; m < m_hi; ++m) {
     const int t0 = m * kCK;
     const bool last = m + 1 == m_hi;
-    TICK(ts0);
     if (!last)
       stage_block<T, 3, CW, false, true, STAGE_X, kFwdWaves, true>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, pos_after(p, A, kCK), e_wg0, wave, lane, X, DT, DL, DY);
-    TICK(ts1); TACC(1, ts0, ts1);
     bp = block_pos(p, A, r, ch_ok);
     K = lane_consts<false>(p, clamp_band(p, bp.bnd0), r, ch_ok);
     per_step_K = __any(bp.kw < kCK && special_boundary(p, bp.bnd0, r));
@@ -717,18 +695,11 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
           // Last step of the block: its operands are in registers already, so the buffer can be
           // handed over now.  The copies of the next block have landed in every wave after this
           // barrier, and no wave reads the current buffer any more.
-          TICK(tw0);
           staging_landed();
-          TICK(tw1); TACC(2, tw0, tw1);
-#ifndef M2D_X_NOBLOCKBAR
           __syncthreads();
-#endif
-          TICK(tw2); TACC(3, tw1, tw2);
           if (!last) fetch(bufn, 0, ahead);
         }
-        TICK(tc0);
         if (t < p.T_total) step(k, now);
-        TICK(tc1); TACC(4, tc0, tc1);
       }
     } else {
 #pragma unroll
@@ -755,14 +726,6 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
 #pragma unroll
       for (int n = 0; n < kN; ++n) carry[(c * kN + n) * kHB] = h[c][n];
   }
-#ifdef M2D_X_TIMING
-  if (lane == 0 && blockIdx.x < 512) {
-    long long* d = g_dbg + (blockIdx.x * 8 + wave) * 8;
-    for (int i = 0; i < 5; ++i) d[i] = dbg_acc[i];
-    d[5] = clock64() - dbg_t0;
-    d[6] = wall_clock64();
-  }
-#endif
 }
 
 // ----------------------------------------------------------------------------------- backward
@@ -825,10 +788,6 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   const float dsk = p.Df[e];
   StagePlan<T, 4, CW, true, false, kBwdWaves, false> plan;
   plan.init(wave, lane);
-#ifdef M2D_X_TIMING
-  long long dbg_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  const long long dbg_t0 = clock64();
-#endif
   settle_loads();
 
   const T* X = static_cast<const T*>(p.x);
@@ -938,10 +897,8 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
 #pragma unroll
     for (int n = 0; n < kN; ++n) ck0[n] = cknext[n];
     const Pos Aprev = pos_before(A);
-    TICK(ts0);
     if (m > m_lo)
       stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, Aprev, e_wg0, wave, lane, X, DT, DL, DY);
-    TICK(ts1); TACC(0, ts0, ts1);
     bp = block_pos(p, A, r, ch_ok);
     fp = block_pos(p, A, f_r, f_on);
     band_consts(bp.bnd0);
@@ -961,7 +918,6 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
 #pragma unroll
         for (int qi = 0; qi < 4; ++qi) hb[0][4 * mgl + qi] = ck0[fold_state(2 * half + mgl, qi)];
       // ---- recompute the states of the block
-      TICK(tr0);
 #pragma unroll
       for (int k = 0; k < kCK; ++k) {
         const int t = t0 + k;
@@ -1011,7 +967,6 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
           }
         }
       }
-      TICK(tr1); TACC(1, tr0, tr1);
       // ---- adjoint over the block, last step first
 #pragma unroll
       for (int k = kCK - 1; k >= 0; --k) {
@@ -1046,7 +1001,6 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
           const float dyl = dyv + gb1;
           float sT = 0.f, sL = 0.f, zT = 0.f, zL = 0.f;
           if (half == 1) { sT = part4[k][0]; sL = part4[k][1]; zT = part4[k][2]; zL = part4[k][3]; }
-          TICK(ta1);
           float* sw = reinterpret_cast<float*>(slots + (xpar * kBwdWaves + wave) * SLOT + lane);
           // A group of 4 states is folded over the 4 channel slots of the wave as soon as it is
           // done; afterwards the lane of slot q holds the channel sums of the states 4q..4q+3
@@ -1111,9 +1065,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
           }
           // ---- across the waves of the workgroup: the per-wave slots (this half's two state
           // groups) are added in wave order, one sum per thread, the same share for every wave
-          TICK(ta2); TACC(3, ta1, ta2); TACC(2, ta2, ta2);
           __syncthreads();
-          TICK(ta3); TACC(4, ta2, ta3);
           if ((fp.in_grid >> k) & 1u) {
             const float* sl = reinterpret_cast<const float*>(slots + xpar * kBwdWaves * SLOT + f_it) + f_comp;
             float s = sl[0];
@@ -1126,20 +1078,11 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
         }
       }
     }
-    TICK(tz0);
     __syncthreads();
-    TICK(tz1); TACC(5, tz0, tz1);
     A = Aprev;
     cur ^= 1;
   }
 
-#ifdef M2D_X_TIMING
-  if (lane == 0 && blockIdx.x < 512) {
-    long long* d = g_dbg + (blockIdx.x * 8 + wave) * 8;
-    for (int i = 0; i < 6; ++i) d[i] = dbg_acc[i];
-    d[6] = clock64() - dbg_t0;
-  }
-#endif
   if (p.sliced && m_lo > my_band * p.sl_nbb) {   // more of the band to come: hand over to the next launch
     if (ch_ok) {
 #pragma unroll
@@ -1522,12 +1465,6 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
 // ---------------------------------------------------------------------------------------- C ABI
 extern "C" {
 
-#ifdef M2D_X_TIMING
-int m2d_dbg_read(long long* host, size_t n) {
-  (void)hipDeviceSynchronize();
-  return hipMemcpyFromSymbol(host, HIP_SYMBOL(g_dbg), n * sizeof(long long)) == hipSuccess ? 0 : 1;
-}
-#endif
 
 int m2d_version(void) { return 200; }
 
