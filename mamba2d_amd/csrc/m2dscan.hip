@@ -475,7 +475,7 @@ __device__ __forceinline__ bool special_boundary(const ScanParams& p, int bnd_lo
 // grid row, works on zero operands (its records come from the page of zeros), which keeps its
 // state finite and never reaches a cell of the grid: at column 0 the left gate is closed, and
 // what the lane below hands to a cell comes from the cell above it.  Only stores are predicated.
-template <typename T, int EC, bool CKPT, bool WRITE_Y, bool STAGE_X>
+template <typename T, int EC, bool CKPT, bool WRITE_Y, bool STAGE_X, bool SLICED>
 __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParams p) {
   constexpr int CS = 64 >> kHBShift;
   constexpr int CW = kFwdWaves * CS * EC;
@@ -489,7 +489,7 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   int lb = logical_block(p.nwg);
   int m_lo = 0, m_hi = p.nblk;                     // blocks of steps this launch sweeps
   int my_band = 0, band_q0 = 0;
-  if (p.sliced) {
+  if constexpr (SLICED) {
     const int per = p.B * p.bpb;
     const int kk = lb / per;
     lb -= kk * per;
@@ -590,8 +590,8 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   for (int c = 0; c < EC; ++c)
 #pragma unroll
     for (int n = 0; n < kN; ++n) h[c][n] = 0.f;
-  float* carry = p.sliced ? p.carry + ((((int64_t)b * p.nbands + my_band) * p.E + e0) * kN) * kHB + r : nullptr;
-  if (p.sliced && band_q0 > 0) {   // the band is under way: take over the state of the previous launch
+  float* carry = SLICED ? p.carry + ((((int64_t)b * p.nbands + my_band) * p.E + e0) * kN) * kHB + r : nullptr;
+  if (SLICED && band_q0 > 0) {   // the band is under way: take over the state of the previous launch
     if (ch_ok) {
 #pragma unroll
       for (int c = 0; c < EC; ++c)
@@ -720,7 +720,7 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
     A.col += kCK;
     if (A.col >= p.S) { A.col -= p.S; A.bnd += 1; }
   }
-  if (p.sliced && ch_ok && m_hi < (my_band + 1) * p.sl_nbb) {   // more of the band to come: hand the state to the next launch
+  if (SLICED && ch_ok && m_hi < (my_band + 1) * p.sl_nbb) {   // more of the band to come: hand the state to the next launch
 #pragma unroll
     for (int c = 0; c < EC; ++c)
 #pragma unroll
@@ -743,7 +743,7 @@ __device__ __forceinline__ constexpr int fold_state(int m, int qi) {
 // on zero operands.  For the adjoint this means that a row which has not reached its last column
 // yet keeps lambda = mu = 0 exactly, and that a row past column 0 carries finite values that are
 // multiplied by zero coefficients (delta, dy, x are zero there) wherever they meet a sum.
-template <typename T, bool STAGE_X>
+template <typename T, bool STAGE_X, bool SLICED>
 __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParams p) {
   constexpr int CS = 64 >> kHBShift;     // 4 channel slots
   constexpr int SLOT = 3 * 64;           // float2s per wave in one exchange buffer
@@ -762,7 +762,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   int lb = logical_block(p.nwg);
   int m_lo = 0, m_hi = p.nblk;              // blocks of steps this launch sweeps (from m_hi - 1 down to m_lo)
   int my_band = 0, band_q0 = 0;
-  if (p.sliced) {
+  if constexpr (SLICED) {
     const int per = p.B * p.bpb;
     const int kk = lb / per;
     lb -= kk * per;
@@ -814,8 +814,8 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
 #pragma unroll
   for (int n = 0; n < kN; ++n) { accAT[n] = 0.f; accAL[n] = 0.f; muT[n] = 0.f; muL[n] = 0.f; }
   // sliced sweep: adjoint state and position sums travel from launch to launch
-  float* carry = p.sliced ? p.carry + ((((int64_t)b * p.nbands + my_band) * p.E + e) * (4 * kN + 1)) * kHB + r : nullptr;
-  if (p.sliced && band_q0 > 0) {
+  float* carry = SLICED ? p.carry + ((((int64_t)b * p.nbands + my_band) * p.E + e) * (4 * kN + 1)) * kHB + r : nullptr;
+  if (SLICED && band_q0 > 0) {
     if (ch_ok) {
 #pragma unroll
       for (int n = 0; n < kN; ++n) {
@@ -1083,7 +1083,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
     cur ^= 1;
   }
 
-  if (p.sliced && m_lo > my_band * p.sl_nbb) {   // more of the band to come: hand over to the next launch
+  if (SLICED && m_lo > my_band * p.sl_nbb) {   // more of the band to come: hand over to the next launch
     if (ch_ok) {
 #pragma unroll
       for (int n = 0; n < kN; ++n) {
@@ -1107,7 +1107,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
     red[k] = v;
   }
   if (ch_ok && r == 0) {
-    const int64_t slot_e = ((int64_t)b * p.pa_slots + (p.sliced ? my_band : 0)) * p.E + e;
+    const int64_t slot_e = ((int64_t)b * p.pa_slots + (SLICED ? my_band : 0)) * p.E + e;
     float* pa = p.pA + slot_e * (2 * kN);
 #pragma unroll
     for (int n = 0; n < 2 * kN; ++n) pa[n] = red[n];
@@ -1323,26 +1323,26 @@ int stage_bc(ScanParams& sp, const m2d_desc* d, const void* BT, const void* BL, 
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
-template <typename T, int EC, bool CK, bool WY, bool SX>
+template <typename T, int EC, bool CK, bool WY, bool SX, bool SL>
 int launch_fwd_as(const ScanParams& sp, hipStream_t st) {
   using SG = Stage<T, 3, kFwdWaves * 4 * EC, false, true>;
   const size_t lds = 256 + 2 * (size_t)SG::kBytes;
   static bool attr = false;   // idempotent, the value never changes
   if (!attr) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_fwd_kernel<T, EC, CK, WY, SX>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_fwd_kernel<T, EC, CK, WY, SX, SL>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return M2D_ERR_HIP;
     attr = true;
   }
-  hipLaunchKernelGGL((m2d_fwd_kernel<T, EC, CK, WY, SX>), dim3((unsigned)sp.nwg), dim3(kFwdWaves * 64), lds, st, sp);
+  hipLaunchKernelGGL((m2d_fwd_kernel<T, EC, CK, WY, SX, SL>), dim3((unsigned)sp.nwg), dim3(kFwdWaves * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
-template <typename T, int EC, bool SX>
+template <typename T, int EC, bool SX, bool SL>
 int launch_fwd_mode(const ScanParams& sp, bool ckpt, bool write_y, hipStream_t st) {
-  if (ckpt && write_y) return launch_fwd_as<T, EC, true, true, SX>(sp, st);
-  if (ckpt) return launch_fwd_as<T, EC, true, false, SX>(sp, st);
-  return launch_fwd_as<T, EC, false, true, SX>(sp, st);
+  if (ckpt && write_y) return launch_fwd_as<T, EC, true, true, SX, SL>(sp, st);
+  if (ckpt) return launch_fwd_as<T, EC, true, false, SX, SL>(sp, st);
+  return launch_fwd_as<T, EC, false, true, SX, SL>(sp, st);
 }
 
 template <typename T>
@@ -1351,9 +1351,11 @@ int launch_fwd(const ScanParams& sp0, const m2d_desc* d, const Geometry& g, bool
   sp.bpb = g.fwd_bpb;
   sp.nwg = d->B * g.fwd_bpb;
   auto once = [&]() {
+    if (g.sliced)   // (the sliced sweep is only chosen where one channel per lane is)
+      return g.stage_x ? launch_fwd_mode<T, 1, true, true>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 1, false, true>(sp, ckpt, write_y, st);
     if (g.fwd_ec == 2)
-      return g.stage_x ? launch_fwd_mode<T, 2, true>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 2, false>(sp, ckpt, write_y, st);
-    return g.stage_x ? launch_fwd_mode<T, 1, true>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 1, false>(sp, ckpt, write_y, st);
+      return g.stage_x ? launch_fwd_mode<T, 2, true, false>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 2, false, false>(sp, ckpt, write_y, st);
+    return g.stage_x ? launch_fwd_mode<T, 1, true, false>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 1, false, false>(sp, ckpt, write_y, st);
   };
   if (!g.sliced) return once();
   // launch l advances band k by blocks [(l - lag*k)*Q, +Q) of its window, for the bands under way
@@ -1391,18 +1393,18 @@ int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   return rc;
 }
 
-template <typename T, bool SX>
+template <typename T, bool SX, bool SL>
 int launch_bwd(const ScanParams& sp, hipStream_t st) {
   using SG = Stage<T, 4, kBwdWaves * 4, true, false>;
   const size_t lds = sizeof(float4) * kBwdWaves * 3 * 64 + sizeof(float) * kBwdWaves * 4 * 2 * kN + 256 + 2 * (size_t)SG::kBytes;
   static bool attr = false;   // idempotent, the value never changes
   if (!attr) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_bwd_kernel<T, SX>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_bwd_kernel<T, SX, SL>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return M2D_ERR_HIP;
     attr = true;
   }
-  hipLaunchKernelGGL((m2d_bwd_kernel<T, SX>), dim3((unsigned)sp.nwg), dim3(kBwdWaves * 64), lds, st, sp);
+  hipLaunchKernelGGL((m2d_bwd_kernel<T, SX, SL>), dim3((unsigned)sp.nwg), dim3(kBwdWaves * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
@@ -1435,7 +1437,7 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   sp.nwg = d->B * g.bwd_bpb;
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][0], st);
   if (!g.sliced) {
-    rc = g.stage_x ? launch_bwd<T, true>(sp, st) : launch_bwd<T, false>(sp, st);
+    rc = g.stage_x ? launch_bwd<T, true, false>(sp, st) : launch_bwd<T, false, false>(sp, st);
   } else {
     // as the forward, bottom-up: launch l advances the band k' from the bottom by Q blocks of its window
     const int nlb = (g.nbb + kSliceQ - 1) / kSliceQ;
@@ -1446,7 +1448,7 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
       if (k_lo > k_hi) continue;
       sp.sl_ell = l; sp.sl_band0 = g.nbands - 1 - k_hi;
       sp.nwg = (k_hi - k_lo + 1) * d->B * g.bwd_bpb;
-      rc = g.stage_x ? launch_bwd<T, true>(sp, st) : launch_bwd<T, false>(sp, st);
+      rc = g.stage_x ? launch_bwd<T, true, true>(sp, st) : launch_bwd<T, false, true>(sp, st);
     }
   }
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][1], st);
