@@ -220,8 +220,10 @@ template <bool PERM> __device__ __forceinline__ constexpr int sinv(int pos) {
 // the 16-byte chunk i of a 1 KB LDS window.  Regions of one buffer:
 //   BC : per (step k, lane row r) a record of 13 chunks: B_T, B_L, C of the cell (row r, column
 //        t0+k-r) as 3 x 16 fp32, plus one pad chunk so that the 16 rows fall in distinct banks;
-//   XD : per (k, r) a record of NT tensors x CW channels of the workgroup in the tensor dtype
-//        (x, deltaT, deltaL[, dy]), plus one pad chunk (needs E to be a multiple of a chunk);
+//   XD : per tensor (x, deltaT, deltaL[, dy]), step k and chunk of channels, the 16 lane rows side by
+//        side (chunk index = ((tensor*kCK + k)*kCpt + channel chunk)*16 + r, no padding: the rows of
+//        a wave-wide read fall in distinct banks); needs E to be a multiple of a chunk.  A wave-wide
+//        copy stays inside one tensor, so its base address is a scalar;
 //   TOP: per (k, channel) the 16 states of the last row of the band above at column t0+k;
 //   BOT: per (k, channel) the 16 muT of the first row of the band below at column t0+k-15.
 // With UNI, BC, TOP and BOT advance by the same number of bytes (kKStr) from one step to the
@@ -233,14 +235,21 @@ template <typename T, int NT, int CW, bool WITH_BOT, bool UNI>
 struct Stage {
   static constexpr int kElem = 16 / sizeof(T);           // elements per chunk
   static constexpr int kCpt = CW / kElem;                // chunks per tensor per cell
-  static constexpr int kXRec = NT * kCpt + 1;            // chunks per XD record (with pad)
-  static constexpr int kXStride = kXRec * kElem;         // XD record stride in elements
+  static constexpr int kXStepBytes = kCpt * kHB * 16;    // XD bytes per tensor and step
+  static constexpr int kXTauBytes = kCK * kXStepBytes;   // XD bytes per tensor
+  static constexpr int kXTauInstr = kXTauBytes / 1024;   // wave-wide copies per tensor
   static constexpr int kBRec = 13;                       // chunks per BC record (with pad)
   static constexpr int kBStride = kBRec * 4;             // BC record stride in floats
   static constexpr int kKChunks = kHB * kBRec > CW * 4 ? kHB * kBRec : CW * 4;   // chunks per step in BC / TOP / BOT
   static constexpr int kKStr = kKChunks * 16;            // the same in bytes
   static constexpr int kBChunks = kCK * kKChunks;
-  static constexpr int kXChunks = kCK * kHB * kXRec;
+  static constexpr int kXChunks = NT * kXTauBytes / 16;
+  static_assert(kXTauBytes % 1024 == 0, "a wave-wide copy must not straddle two tensors of XD");
+  static_assert((kCpt & (kCpt - 1)) == 0, "chunks per tensor row must be a power of two");
+  // byte offset inside a tensor's part of XD of channel `ch` (of the workgroup) for lane row r at step 0
+  static __host__ __device__ constexpr uint32_t x_off(int r, int ch) {
+    return (uint32_t)(((ch / kElem) * kHB + r) * 16 + (ch % kElem) * (int)sizeof(T));
+  }
   static constexpr int kTInstr = kCK * CW / 16;          // wave-wide copies that fill TOP (or BOT): 16 channels each
   static constexpr int kXOff = kBChunks * 16;
   static constexpr int kTOff = kXOff + kXChunks * 16;
@@ -265,16 +274,15 @@ __device__ __forceinline__ void lds_fill16(const void* src, char* lds_window) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(base) : "memory", "m0");
 }
 
-// The chunk -> (step, row, part of record) decomposition of the BC and XD regions depends only on
-// the thread.  It is worked out once (divisions by the odd record sizes) and kept as one packed
-// word per wave-wide copy: bits 0-3 row, 4-8 part, 9-10 step, bit 31 set if the chunk carries data.
+// The chunk -> (step, row, part of record) decomposition of the BC region depends only on the
+// thread.  It is worked out once (division by the odd record size) and kept as one packed word per
+// wave-wide copy: bits 0-3 row, 4-8 part, 9-10 step, bit 31 set if the chunk carries data.
 template <typename T, int NT, int CW, bool WITH_BOT, bool UNI, int NWAVES, bool KEEP>
 struct StagePlan {
   using SG = Stage<T, NT, CW, WITH_BOT, UNI>;
   static constexpr int kPer = NWAVES * 64;
   static constexpr int kItB = (SG::kBChunks + kPer - 1) / kPer;
-  static constexpr int kItX = (SG::kXChunks + kPer - 1) / kPer;
-  uint32_t bc[KEEP ? kItB : 1], xd[KEEP ? kItX : 1];
+  uint32_t bc[KEEP ? kItB : 1];
   // `perk` chunks per step, of which the first kHB*reclen hold the records of the 16 lane rows
   static __device__ __forceinline__ uint32_t word(int c, int nchunks, int perk, int reclen, int nparts) {
     const int k = c / perk, rem = c - k * perk;
@@ -285,8 +293,6 @@ struct StagePlan {
     if constexpr (KEEP) {
 #pragma unroll
       for (int i = 0; i < kItB; ++i) bc[i] = word(i * kPer + wave * 64 + lane, SG::kBChunks, SG::kKChunks, SG::kBRec, 12);
-#pragma unroll
-      for (int i = 0; i < kItX; ++i) xd[i] = word(i * kPer + wave * 64 + lane, SG::kXChunks, kHB * SG::kXRec, SG::kXRec, NT * SG::kCpt);
     }
   }
   // Kernels short of registers work the word out again at every use instead of keeping it.
@@ -294,12 +300,6 @@ struct StagePlan {
     uint32_t w;
     if constexpr (KEEP) { w = bc[i]; } else { asm volatile("" : "+v"(lane)); w = word(i * kPer + wave * 64 + lane, SG::kBChunks, SG::kKChunks, SG::kBRec, 12); }
     asm volatile("" : "+v"(w));   // unpack per use: the fields must not be hoisted into live registers
-    return w;
-  }
-  __device__ __forceinline__ uint32_t get_xd(int i, int wave, int lane) const {
-    uint32_t w;
-    if constexpr (KEEP) { w = xd[i]; } else { asm volatile("" : "+v"(lane)); w = word(i * kPer + wave * 64 + lane, SG::kXChunks, kHB * SG::kXRec, SG::kXRec, NT * SG::kCpt); }
-    asm volatile("" : "+v"(w));
     return w;
   }
 };
@@ -322,36 +322,36 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan
                                             const T* x0, const T* x1, const T* x2, const T* x3) {
   using SG = Stage<T, NT, CW, WITH_BOT, UNI>;
   using PL = StagePlan<T, NT, CW, WITH_BOT, UNI, NWAVES, KEEP>;
-  static_assert((SG::kCpt & (SG::kCpt - 1)) == 0, "chunks per tensor row must be a power of two");
+  // Source addresses are computed for every chunk and replaced by the page of zeros where the
+  // chunk is not a cell of the grid (selects, no divergent branches).  Cells of one image are
+  // addressed by 32-bit byte offsets from the image's base.
   const int64_t img = (int64_t)b * p.H * p.W;
+  const char* zeros = reinterpret_cast<const char*>(p.zeros);
+  const char* bc_img = reinterpret_cast<const char*>(p.bt + img * p.bc_stride);
 #pragma unroll
   for (int i = 0; i < PL::kItB; ++i) {
     const uint32_t w = plan.get_bc(i, wave, lane);
     const int r = w & 15, part = (w >> 4) & 31, k = (w >> 9) & 3;
-    if ((int)w < 0) {
-      const Pos q = pos_after(p, A, k - r + (kHB - 1));
-      const float* src = p.zeros;
-      if ((unsigned)q.bnd < (unsigned)p.nbands && q.col < p.W && r >= 1 && r <= band_rows(p, q.bnd))
-        src = p.bt + (img + cell_of(p, q.bnd, r, q.col)) * p.bc_stride + part * 4;   // B_T, B_L, C back to back
-      lds_fill16<false>(src, buf + (i * PL::kPer + wave * 64) * 16);
-    }
+    const Pos q = pos_after(p, A, k - r + (kHB - 1));
+    const bool ok = (unsigned)q.bnd < (unsigned)p.nbands && q.col < p.W && r >= 1 && r <= band_rows(p, q.bnd);
+    const uint32_t off = (uint32_t)cell_of(p, q.bnd, r, q.col) * (uint32_t)(p.bc_stride * 4) + (uint32_t)(part * 16);
+    const char* src = ok ? bc_img + off : zeros;          // the packed record holds B_T, B_L, C back to back
+    if ((int)w < 0) lds_fill16<false>(src, buf + (i * PL::kPer + wave * 64) * 16);
   }
   if constexpr (STAGE_X) {
-#pragma unroll
-    for (int i = 0; i < PL::kItX; ++i) {
-      const uint32_t w = plan.get_xd(i, wave, lane);
-      const int r = w & 15, part = (w >> 4) & 31, k = (w >> 9) & 3;
-      if ((int)w < 0) {
-        const Pos q = pos_after(p, A, k - r + (kHB - 1));
-        const int tau = part / SG::kCpt, ch = e_wg0 + (part & (SG::kCpt - 1)) * SG::kElem;
-        const void* src = p.zeros;
-        if ((unsigned)q.bnd < (unsigned)p.nbands && q.col < p.W && r >= 1 && r <= band_rows(p, q.bnd) && ch < p.E) {
-          // selected with compares: an indexed pointer table would live in (scratch) memory
-          const T* base = tau == 0 ? x0 : (tau == 1 ? x1 : (tau == 2 ? x2 : x3));
-          src = base + (img + cell_of(p, q.bnd, r, q.col)) * p.E + ch;
-        }
-        lds_fill16<false>(src, buf + SG::kXOff + (i * PL::kPer + wave * 64) * 16);
-      }
+    const int64_t img_bytes = img * p.E * (int64_t)sizeof(T);
+    for (int qi = wave; qi < NT * SG::kXTauInstr; qi += NWAVES) {
+      const int tau = qi / SG::kXTauInstr;                       // wave-uniform: one tensor per copy
+      const T* base = tau == 0 ? x0 : (tau == 1 ? x1 : (tau == 2 ? x2 : x3));
+      const char* t_img = reinterpret_cast<const char*>(base) + img_bytes;
+      const int c = (qi - tau * SG::kXTauInstr) * 64 + lane;      // chunk inside the tensor's part of XD
+      const int r = c & (kHB - 1), cc = (c >> kHBShift) & (SG::kCpt - 1), k = c / (kHB * SG::kCpt);
+      const Pos q = pos_after(p, A, k - r + (kHB - 1));
+      const int ch = e_wg0 + cc * SG::kElem;
+      const bool ok = (unsigned)q.bnd < (unsigned)p.nbands && q.col < p.W && r >= 1 && r <= band_rows(p, q.bnd) && ch < p.E;
+      const uint32_t off = (uint32_t)(cell_of(p, q.bnd, r, q.col) * p.E + ch) * (uint32_t)sizeof(T);
+      const char* src = ok ? t_img + off : zeros;
+      lds_fill16<false>(src, buf + SG::kXOff + qi * 1024);
     }
   }
   // boundary rows were written earlier in this launch (or by the forward launch): read them
@@ -540,8 +540,8 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   // byte offsets of the lane's records inside a staging buffer (step 0)
   const uint32_t rec_off = r == 0 ? SG::kTOff + ch_loc * kN * 4 : r * SG::kBStride * 4;
   const uint32_t rec_cstep = r == 0 ? kN * 4 : 0;   // the ghost reads a record per channel, grid rows share theirs
-  const uint32_t xd_off = SG::kXOff + (r * SG::kXStride + ch_loc) * (uint32_t)sizeof(T);
-  constexpr uint32_t kXK = kHB * SG::kXStride * sizeof(T);   // XD bytes per step
+  const uint32_t xd_off = SG::kXOff + SG::x_off(r, ch_loc);
+  constexpr uint32_t kXK = SG::kXStepBytes;   // XD bytes per step
 
   // per block: where the lane is and what depends on it
   BlockPos bp;
@@ -559,8 +559,8 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
     if constexpr (STAGE_X) {
       const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
       IO<T>::template ldv<EC>(xr, o.xv);
-      IO<T>::template ldv<EC>(xr + CW, o.dtv);
-      IO<T>::template ldv<EC>(xr + 2 * CW, o.dlv);
+      IO<T>::template ldv<EC>(xr + SG::kXTauBytes / sizeof(T), o.dtv);
+      IO<T>::template ldv<EC>(xr + 2 * SG::kXTauBytes / sizeof(T), o.dlv);
     } else {   // straight from memory, for the lane's position at step k of the current block
 #pragma unroll
       for (int c = 0; c < EC; ++c) { o.xv[c] = 0.f; o.dtv[c] = 0.f; o.dlv[c] = 0.f; }
@@ -834,8 +834,8 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   const uint32_t rec_off = r == 0 ? SG::kTOff + ch_loc * kN * 4
                                   : (r == kHB - 1 ? SG::kOOff + ch_loc * kN * 4 - 2 * kN * 4 : r * SG::kBStride * 4);
   const uint32_t rec_kstr = (r == 0 || r == kHB - 1) ? SG::kTKStr : SG::kKStr;
-  const uint32_t xd_off = SG::kXOff + (r * SG::kXStride + ch_loc) * (uint32_t)sizeof(T);
-  constexpr uint32_t kXK = kHB * SG::kXStride * sizeof(T);   // XD bytes per step
+  const uint32_t xd_off = SG::kXOff + SG::x_off(r, ch_loc);
+  constexpr uint32_t kXK = SG::kXStepBytes;   // XD bytes per step
   // the sum that this thread adds up in the exchange (one float of one lane's float2, one tensor):
   // it belongs to lane row f_r, which is f_d positions ahead of this thread's own row
   const int fid = wave * (2 * SLOT / kBwdWaves) + lane;
@@ -931,7 +931,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
           float xv = 0.f, dtv = 0.f, dlv = 0.f;
           if constexpr (STAGE_X) {
             const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
-            xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW);
+            xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + SG::kXTauBytes / sizeof(T)); dlv = IO<T>::ld(xr + 2 * SG::kXTauBytes / sizeof(T));
           } else if ((bp.in_grid >> k) & 1u) {
             const uint32_t off = cell_off0 + (uint32_t)k * estep + (k >= bp.kw ? wrap_adj : 0u);
             xv = IO<T>::ld(reinterpret_cast<const T*>(Ximg + off));
@@ -986,7 +986,8 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
           float xv = 0.f, dtv = 0.f, dlv = 0.f, dyv = 0.f;
           if constexpr (STAGE_X) {
             const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
-            xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + CW); dlv = IO<T>::ld(xr + 2 * CW); dyv = IO<T>::ld(xr + 3 * CW);
+            xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + SG::kXTauBytes / sizeof(T)); dlv = IO<T>::ld(xr + 2 * SG::kXTauBytes / sizeof(T));
+            dyv = IO<T>::ld(xr + 3 * SG::kXTauBytes / sizeof(T));
           } else if (inr) {
             xv = IO<T>::ld(reinterpret_cast<const T*>(Ximg + goff));
             dtv = IO<T>::ld(reinterpret_cast<const T*>(DTimg + goff));
