@@ -51,6 +51,7 @@ constexpr int kRB = 14;           // grid rows per band; lanes 0 and 15 of a row
 constexpr int kFwdWaves = 8;      // waves per forward workgroup
 constexpr int kBwdWaves = 8;      // waves per backward workgroup
 constexpr int kZeroFloats = 64;     // page of zeros at the head of the set-up area
+constexpr int kModeSweep = 0, kModeSliced = 1, kModeStacked = 2;   // how the bands of the batch are scheduled
 constexpr int kSliceQ = 4;         // sliced sweep: blocks of steps per band and launch
 constexpr int kSliceLag = 2;       // sliced sweep: launches by which a band trails the band it depends on
 constexpr float kLog2e = 1.4426950408889634f;
@@ -160,6 +161,12 @@ struct ScanParams {
   float* carry;                     // state handed from launch to launch: fwd [B][nbands][E][16][16], bwd [B][nbands][E][65][16]
   int64_t bot_stride;               // floats between the mu_T rows of consecutive bands (0: one row buffer, bands in sequence)
   int pa_slots;                     // partial sums over positions per image (1, or one per band when sliced)
+  // Stacked images (grids of one band whose height divides 14): `ips` images in a row of the batch
+  // are swept as one tall image whose bands do not depend on each other: B, H above are then the
+  // number and height of the stacks, and a workgroup shortens H for a last, shorter stack.
+  int stacked, ips, Himg, Breal;    // on/off, images per stack, rows per image, images in the batch
+  int Hs;                           // rows between the bases of consecutive (stacked) images
+  int64_t Ptot;                     // cells of the whole batch
   int bpb;                          // workgroups per image
   int nwg;                          // total workgroups
 };
@@ -174,22 +181,15 @@ __device__ __forceinline__ int logical_block(int nwg) {
   return (id & 7) * per + (id >> 3);
 }
 
-// offset of cell (i,j) inside its image, in cells
-__device__ __forceinline__ int cell_in_image(const ScanParams& p, int i, int j) {
-  const int im = p.flip ? p.H - 1 - i : i;
-  const int jm = p.flip ? p.W - 1 - j : j;
-  return im * p.W + jm;
-}
-
-// Stream position -> (band, column).  s >= -S.  Bands outside [0, nbands) and columns >= W are
-// not on the grid.
+// Stream position -> (band, column).  s >= -21 (S >= 7, so 3 strides below zero are in range).
+// Bands outside [0, nbands) and columns >= W are not on the grid.
 struct Pos { int bnd, col; };
 __device__ __forceinline__ Pos pos_of(const ScanParams& p, int s) {
-  const uint32_t sp = (uint32_t)(s + p.S);
+  const uint32_t sp = (uint32_t)(s + 3 * p.S);
   uint32_t q = __umulhi(sp, p.magicS);          // q or q-1 of the true quotient for sp < 2^32
   uint32_t rem = sp - q * (uint32_t)p.S;
   if (rem >= (uint32_t)p.S) { q += 1; rem -= (uint32_t)p.S; }
-  Pos o; o.bnd = (int)q - 1; o.col = (int)rem;
+  Pos o; o.bnd = (int)q - 3; o.col = (int)rem;
   return o;
 }
 __device__ __forceinline__ int band_rows(const ScanParams& p, int bnd) { return bnd == p.nbands - 1 ? p.rows_last : kRB; }
@@ -304,13 +304,17 @@ struct StagePlan {
   }
 };
 
-// Position of the stream index (index of A) + d, for 0 <= d < S.
+// Position of the stream index (index of A) + d, for 0 <= d < 19.  Strides below 19 (stacked
+// images) can wrap more than once.
 __device__ __forceinline__ Pos pos_after(const ScanParams& p, Pos A, int d) {
   Pos q;
   q.col = A.col + d;
-  const bool w = q.col >= p.S;
-  q.col = w ? q.col - p.S : q.col;
-  q.bnd = w ? A.bnd + 1 : A.bnd;
+  q.bnd = A.bnd;
+  if (q.col >= p.S) { q.col -= p.S; q.bnd += 1; }
+  if (p.S < kHB + kCK - 1) {   // uniform
+    if (q.col >= p.S) { q.col -= p.S; q.bnd += 1; }
+    if (q.col >= p.S) { q.col -= p.S; q.bnd += 1; }
+  }
   return q;
 }
 
@@ -325,7 +329,7 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan
   // Source addresses are computed for every chunk and replaced by the page of zeros where the
   // chunk is not a cell of the grid (selects, no divergent branches).  Cells of one image are
   // addressed by 32-bit byte offsets from the image's base.
-  const int64_t img = (int64_t)b * p.H * p.W;
+  const int64_t img = (int64_t)b * p.Hs * p.W;
   const char* zeros = reinterpret_cast<const char*>(p.zeros);
   const char* bc_img = reinterpret_cast<const char*>(p.bt + img * p.bc_stride);
 #pragma unroll
@@ -361,7 +365,7 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan
     const int ch = e_wg0 + sub * 16 + (lane >> 2);
     const Pos q = pos_after(p, A, k + (kHB - 1));    // the upper ghost is lane 0
     const float* src = p.zeros;
-    if (q.bnd >= 1 && q.bnd < p.nbands && q.col < p.W && ch < p.E)
+    if (!p.stacked && q.bnd >= 1 && q.bnd < p.nbands && q.col < p.W && ch < p.E)
       src = p.top + ((((int64_t)(q.bnd - 1) * p.B + b) * p.W + q.col) * p.E + ch) * kN + (lane & 3) * 4;
     lds_fill16<true>(src, buf + SG::kTOff + k * SG::kTKStr + sub * 1024);
   }
@@ -371,7 +375,7 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan
       const int ch = e_wg0 + sub * 16 + (lane >> 2);
       const Pos q = pos_after(p, A, k);              // the lower ghost is lane 15
       const float* src = p.zeros;
-      if (q.bnd >= 0 && q.bnd + 1 < p.nbands && q.col < p.W && ch < p.E)
+      if (!p.stacked && q.bnd >= 0 && q.bnd + 1 < p.nbands && q.col < p.W && ch < p.E)
         src = p.bot + (q.bnd + 1) * p.bot_stride + (((int64_t)b * p.W + q.col) * p.E + ch) * kN + (lane & 3) * 4;
       lds_fill16<true>(src, buf + SG::kOOff + k * SG::kTKStr + sub * 1024);
     }
@@ -412,8 +416,9 @@ __device__ __forceinline__ LaneK lane_consts(const ScanParams& p, int bnd, int r
   // last one works on zero operands with the constants of that band
   LaneK c;
   c.real = ch_ok && r >= 1 && r <= kRB && r <= band_rows(p, bnd);
-  const bool first_row = bnd == 0 && r == 1;
-  const bool gbot = BWD && r == kHB - 1 && bnd + 1 < p.nbands;
+  // grid row 0 of an image: no row above (stacked images: 14 is a multiple of the image height)
+  const bool first_row = p.stacked ? (r - 1) % p.Himg == 0 : (bnd == 0 && r == 1);
+  const bool gbot = BWD && !p.stacked && r == kHB - 1 && bnd + 1 < p.nbands;
   c.oT = gbot ? 0.f : (!c.real || first_row ? ninf : -1.f);
   c.oL = !c.real ? ninf : (first_row ? 0.f : -1.f);
   c.cT = !c.real || first_row ? 0.f : 0.5f;
@@ -445,10 +450,8 @@ struct BlockPos {
 };
 __device__ __forceinline__ BlockPos block_pos(const ScanParams& p, Pos A, int r, bool lane_ok) {
   BlockPos q;
-  q.col0 = A.col + (kHB - 1 - r);
-  const bool w = q.col0 >= p.S;
-  q.col0 = w ? q.col0 - p.S : q.col0;
-  q.bnd0 = w ? A.bnd + 1 : A.bnd;
+  const Pos at = pos_after(p, A, kHB - 1 - r);
+  q.col0 = at.col; q.bnd0 = at.bnd;
   q.kw = p.S - q.col0;
   q.kz = q.col0 == 0 ? 0 : q.kw;
   q.in_grid = 0;
@@ -467,7 +470,7 @@ __device__ __forceinline__ int clamp_band(const ScanParams& p, int bnd) { return
 // A row changes its constants only when it moves between the first band and the second (grid row
 // 0 has no row above) or into / out of the last band (fewer rows, no band below).
 __device__ __forceinline__ bool special_boundary(const ScanParams& p, int bnd_lo, int r) {
-  return (bnd_lo == 0 && r == 1) || (bnd_lo + 1 == p.nbands - 1 && (r > p.rows_last || r == kHB - 1));
+  return (!p.stacked && bnd_lo == 0 && r == 1) || (bnd_lo + 1 == p.nbands - 1 && (r > p.rows_last || r == kHB - 1));
 }
 
 // ------------------------------------------------------------------------------------ forward
@@ -475,8 +478,14 @@ __device__ __forceinline__ bool special_boundary(const ScanParams& p, int bnd_lo
 // grid row, works on zero operands (its records come from the page of zeros), which keeps its
 // state finite and never reaches a cell of the grid: at column 0 the left gate is closed, and
 // what the lane below hands to a cell comes from the cell above it.  Only stores are predicated.
-template <typename T, int EC, bool CKPT, bool WRITE_Y, bool STAGE_X, bool SLICED>
-__global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParams p) {
+template <typename T, int EC, bool CKPT, bool WRITE_Y, bool STAGE_X, int MODE>
+__global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParams pin) {
+  constexpr bool SLICED = MODE == kModeSliced, STACKED = MODE == kModeStacked;
+  ScanParams p = pin;   // (stacked images: the height is shortened below for a last, shorter stack)
+  if constexpr (!STACKED) {   // lets the compiler drop what only stacked images need
+    __builtin_assume(p.stacked == 0);
+    __builtin_assume(p.S >= kHB + kCK - 1);
+  }
   constexpr int CS = 64 >> kHBShift;
   constexpr int CW = kFwdWaves * CS * EC;
   constexpr bool PERM = true;
@@ -500,6 +509,12 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   }
   const int b = lb / p.bpb;
   const int e_wg0 = (lb % p.bpb) * CW;
+  if constexpr (STACKED) {   // the last stack of the batch may hold fewer images
+    const int nimg = p.Breal - b * p.ips < p.ips ? p.Breal - b * p.ips : p.ips;
+    p.H = nimg * p.Himg;
+    p.nbands = (p.H + kRB - 1) / kRB;
+    p.rows_last = p.H - (p.nbands - 1) * kRB;
+  }
   const int slot = lane >> kHBShift, r = lane & (kHB - 1);
   const int ch_loc = (wave * CS + slot) * EC;      // first channel of the lane inside the workgroup
   const int e_raw = e_wg0 + ch_loc;
@@ -525,7 +540,7 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   const T* DL = static_cast<const T*>(p.dL);
   const T* DY = DL;   // not staged by the forward (NT = 3)
   const float ninf = -__builtin_huge_valf();
-  const int64_t cell0 = (int64_t)b * p.H * p.W;
+  const int64_t cell0 = (int64_t)b * p.Hs * p.W;
   // (B,H,W,E) tensors are addressed as image base (uniform) + 32-bit byte offset (per lane)
   const int64_t img_bytes = cell0 * p.E * (int64_t)sizeof(T);
   char* Yimg = static_cast<char*>(p.y) + img_bytes;
@@ -635,7 +650,7 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
       }
       yv[c] = __builtin_fmaf(o.xv[c], dsk[c], acc);
     }
-    if (p.nbands > 1) {   // last row of a band: the next band's ghost will replay it
+    if (p.nbands > 1 && !p.stacked) {   // last row of a band: the next band's ghost will replay it
       const bool wk = k >= bp.kw;
       const int bk = wk ? bp.bnd0 + 1 : bp.bnd0;
       if (inr && r == kRB && bk + 1 < p.nbands) {
@@ -743,8 +758,14 @@ __device__ __forceinline__ constexpr int fold_state(int m, int qi) {
 // on zero operands.  For the adjoint this means that a row which has not reached its last column
 // yet keeps lambda = mu = 0 exactly, and that a row past column 0 carries finite values that are
 // multiplied by zero coefficients (delta, dy, x are zero there) wherever they meet a sum.
-template <typename T, bool STAGE_X, bool SLICED>
-__global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParams p) {
+template <typename T, bool STAGE_X, int MODE>
+__global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParams pin) {
+  constexpr bool SLICED = MODE == kModeSliced, STACKED = MODE == kModeStacked;
+  ScanParams p = pin;   // (stacked images: the height is shortened below for a last, shorter stack)
+  if constexpr (!STACKED) {   // lets the compiler drop what only stacked images need
+    __builtin_assume(p.stacked == 0);
+    __builtin_assume(p.S >= kHB + kCK - 1);
+  }
   constexpr int CS = 64 >> kHBShift;     // 4 channel slots
   constexpr int SLOT = 3 * 64;           // float2s per wave in one exchange buffer
   constexpr int CW = kBwdWaves * CS;
@@ -773,6 +794,12 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   }
   const int b = lb / p.bpb;
   const int eg = lb % p.bpb;
+  if constexpr (STACKED) {   // the last stack of the batch may hold fewer images
+    const int nimg = p.Breal - b * p.ips < p.ips ? p.Breal - b * p.ips : p.ips;
+    p.H = nimg * p.Himg;
+    p.nbands = (p.H + kRB - 1) / kRB;
+    p.rows_last = p.H - (p.nbands - 1) * kRB;
+  }
   const int e_wg0 = eg * CW;
   const int slot = lane >> kHBShift, r = lane & (kHB - 1);
   const int ch_loc = wave * CS + slot;
@@ -795,7 +822,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   const T* DL = static_cast<const T*>(p.dL);
   const T* DY = static_cast<const T*>(p.dy);
   const float ninf = -__builtin_huge_valf();
-  const int64_t cell0 = (int64_t)b * p.H * p.W;
+  const int64_t cell0 = (int64_t)b * p.Hs * p.W;
   // (B,H,W,E) tensors: image base (uniform) + 32-bit byte offset (per lane)
   const int64_t img_bytes = cell0 * p.E * (int64_t)sizeof(T);
   const char* Ximg = reinterpret_cast<const char*>(X) + img_bytes;
@@ -807,7 +834,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   char* DDLimg = static_cast<char*>(p.ddL) + img_bytes;
   char* BOTimg = reinterpret_cast<char*>(p.bot + (int64_t)b * p.W * p.E * kN);   // + band * bot_stride
   // per-workgroup channel sums: [channel group][cell][C, B_T, B_L][16]
-  char* PARTimg = reinterpret_cast<char*>(p.part + ((int64_t)eg * p.B * p.H * p.W + cell0) * (3 * kN));
+  char* PARTimg = reinterpret_cast<char*>(p.part + ((int64_t)eg * p.Ptot + cell0) * (3 * kN));
 
   float accAT[kN], accAL[kN], accD = 0.f;
   float muT[kN], muL[kN];
@@ -1042,7 +1069,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
             sw[64 * 2 + mgl] = fold16(fold32(vBT[0], vBT[1]), fold32(vBT[2], vBT[3]));
             sw[128 * 2 + mgl] = fold16(fold32(vBL[0], vBL[1]), fold32(vBL[2], vBL[3]));
           }
-          if (p.nbands > 1) {   // first row of a band: the lower ghost of the band above will replay its muT
+          if (p.nbands > 1 && !p.stacked) {   // first row of a band: the lower ghost of the band above will replay its muT
             const bool wk = k >= bp.kw;
             if (inr && r == 1 && (wk ? bp.bnd0 + 1 : bp.bnd0) >= 1) {
               const int ck = wk ? bp.col0 + k - p.S : bp.col0 + k;
@@ -1156,7 +1183,7 @@ __global__ void m2d_pack_bc_kernel(const T* BT, const T* BL, const T* C, float* 
 // d_AT, d_AL, d_D: add the per-image partials in image order.
 template <typename T>
 __global__ void m2d_finalize_kernel(const ScanParams p, T* dC, T* dBT, T* dBL, T* dAT, T* dAL, T* dD) {
-  const int64_t P = (int64_t)p.B * p.H * p.W;
+  const int64_t P = p.Ptot;
   const int64_t nquad = 3 * P * (kN / 4);
   const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (gid < nquad) {
@@ -1201,6 +1228,8 @@ struct Geometry {
   int bwd_wpb, bwd_bpb;              // backward: waves and workgroups (channel groups) per image
   bool stage_x;                      // x, delta, dy rows are whole 16-byte chunks: stage them through LDS
   bool sliced;                       // bands on workgroups of their own, swept by a sequence of launches
+  bool stacked;                      // images of one band stacked into tall images of independent bands
+  int ips, vB, vH;                   // images per stack; number and height of what the kernels sweep
   int nbb, nlaunch;                  // sliced: blocks per band, launches per sweep
   size_t carry_fwd_bytes, carry_bwd_bytes;
   size_t prep_bytes, bc_bytes, ckpt_diag_bytes, top_bytes, bot_bytes, part_bytes, pa_bytes, pd_bytes;
@@ -1221,23 +1250,52 @@ int check_desc(const m2d_desc* d) {
 
 Geometry make_geometry(const m2d_desc* d) {
   Geometry g;
-  // band height: 16 rows keeps W/(W+HB-1) of the steps busy and gives 4 channel slots per wave
   g.HB = kHB;
   g.hb_shift = kHBShift;
   g.CS = 64 / g.HB;
-  g.nbands = (d->H + kRB - 1) / kRB;
-  g.rows_last = d->H - (g.nbands - 1) * kRB;
+  const int groups = (d->E + kBwdWaves * g.CS - 1) / (kBwdWaves * g.CS);   // workgroups per image
+  // Grids of a single band whose height divides 14 (14x14, 7x7): a sweep spends as many steps
+  // filling and draining the 16-lane pipeline as working.  `ips` consecutive images of the batch
+  // are then stacked into one tall image whose bands do not depend on each other and swept back to
+  // back with stride S = W.  ips is chosen for the fewest steps over all rounds of workgroups
+  // (one workgroup per CU at a time).
+  g.stacked = false; g.ips = 1; g.vB = d->B; g.vH = d->H;
+  if (d->H <= kRB && kRB % d->H == 0 && d->B >= 2) {
+    const int S = d->W > 7 ? d->W : 7;
+    int64_t best = -1;
+    for (int ips = 1; ips <= 64 && ips <= d->B; ++ips) {
+      if ((int64_t)ips * d->H * d->W * d->E >= ((int64_t)1 << 30)) break;   // a stack is addressed like one image
+      const int vB = (d->B + ips - 1) / ips;
+      const int nb = (ips * d->H + kRB - 1) / kRB;
+      const int64_t rounds = ((int64_t)vB * groups + 255) / 256;
+      const int64_t cost = rounds * ((nb - 1) * S + d->W + kRB + 8);
+      if (best < 0 || cost < best) { best = cost; g.ips = ips; }
+    }
+    if (g.ips > 1) {
+      g.stacked = true;
+      g.vB = (d->B + g.ips - 1) / g.ips;
+      g.vH = g.ips * d->H;
+    }
+  }
+  const int B = g.vB, H = g.vH;   // what the kernels sweep
+  g.nbands = (H + kRB - 1) / kRB;
+  g.rows_last = H - (g.nbands - 1) * kRB;
   // A band's ghost reads the row that the band before stored S - 14 steps earlier, one block
   // ahead of its use: S - 14 >= 12 steps cover the store, the block-end barrier and the staging.
-  // Wide grids run the bands back to back (S = W); narrow ones are padded.
-  g.S = (g.nbands > 1 && d->W >= 26) ? d->W : (d->W + kHB - 1 > 26 ? d->W + kHB - 1 : 26);
-  g.T_total = (g.nbands - 1) * g.S + d->W + g.rows_last;
+  // Wide grids run the bands back to back (S = W); narrow ones are padded.  Stacked images have no
+  // such dependence.
+  if (g.stacked) {
+    g.S = d->W > 7 ? d->W : 7;
+    g.T_total = (g.nbands - 1) * g.S + d->W + kRB;
+  } else {
+    g.S = (g.nbands > 1 && d->W >= 26) ? d->W : (d->W + kHB - 1 > 26 ? d->W + kHB - 1 : 26);
+    g.T_total = (g.nbands - 1) * g.S + d->W + g.rows_last;
+  }
   g.nblk = (g.T_total + kCK - 1) / kCK;
   // Few images with many bands leave most of the device idle when each image is one sequential
   // stream.  Then every band gets workgroups of its own (a padded stream, one window of S steps
   // per band) and the sweep becomes a sequence of launches in which band k trails band k-1.
-  const int groups = (d->E + kBwdWaves * (64 / kHB) - 1) / (kBwdWaves * (64 / kHB));
-  g.sliced = g.nbands >= 4 && (int64_t)d->B * groups <= 64;
+  g.sliced = !g.stacked && g.nbands >= 4 && (int64_t)B * groups <= 64;
   g.nbb = 0; g.nlaunch = 1;
   if (g.sliced) {
     g.S = (d->W + kHB - 1 + kCK - 1) / kCK * kCK;
@@ -1248,25 +1306,26 @@ Geometry make_geometry(const m2d_desc* d) {
     g.nlaunch = kSliceLag * (g.nbands - 1) + (g.nbb + kSliceQ - 1) / kSliceQ;
   }
   // forward: two channels per lane when that still yields enough waves to fill the device
-  const bool ec2 = (d->E % 2 == 0) && ((int64_t)d->B * ((d->E + kFwdWaves * g.CS * 2 - 1) / (kFwdWaves * g.CS * 2)) >= 256);
+  const bool ec2 = (d->E % 2 == 0) && ((int64_t)B * ((d->E + kFwdWaves * g.CS * 2 - 1) / (kFwdWaves * g.CS * 2)) >= 256);
   g.fwd_ec = ec2 ? 2 : 1;
   g.fwd_bpb = (d->E + kFwdWaves * g.CS * g.fwd_ec - 1) / (kFwdWaves * g.CS * g.fwd_ec);
   g.fwd_wpb = g.fwd_bpb * kFwdWaves;
-  g.bwd_bpb = (d->E + kBwdWaves * g.CS - 1) / (kBwdWaves * g.CS);
+  g.bwd_bpb = groups;
   g.bwd_wpb = g.bwd_bpb * kBwdWaves;
   g.stage_x = (d->E % (d->dtype == M2D_BF16 ? 8 : 4)) == 0;
   const size_t P = (size_t)d->B * d->H * d->W;
   g.prep_bytes = align_up(sizeof(float) * (kZeroFloats + (size_t)2 * d->E * kN + d->E));
   g.bc_bytes = align_up(sizeof(float) * P * 48);
-  g.ckpt_diag_bytes = align_up(sizeof(float) * (size_t)d->B * g.nblk * d->E * kN * g.HB);
-  g.top_bytes = g.nbands > 1 ? align_up(sizeof(float) * (size_t)(g.nbands - 1) * d->B * d->W * d->E * kN) : 0;
-  g.bot_bytes = g.nbands > 1 ? align_up(sizeof(float) * (size_t)(g.sliced ? g.nbands : 1) * d->B * d->W * d->E * kN) : 0;
-  g.carry_fwd_bytes = g.sliced ? align_up(sizeof(float) * (size_t)d->B * g.nbands * d->E * kN * kHB) : 0;
-  g.carry_bwd_bytes = g.sliced ? align_up(sizeof(float) * (size_t)d->B * g.nbands * d->E * (4 * kN + 1) * kHB) : 0;
+  g.ckpt_diag_bytes = align_up(sizeof(float) * (size_t)B * g.nblk * d->E * kN * g.HB);
+  const bool rows = g.nbands > 1 && !g.stacked;   // boundary rows travel between bands
+  g.top_bytes = rows ? align_up(sizeof(float) * (size_t)(g.nbands - 1) * B * d->W * d->E * kN) : 0;
+  g.bot_bytes = rows ? align_up(sizeof(float) * (size_t)(g.sliced ? g.nbands : 1) * B * d->W * d->E * kN) : 0;
+  g.carry_fwd_bytes = g.sliced ? align_up(sizeof(float) * (size_t)B * g.nbands * d->E * kN * kHB) : 0;
+  g.carry_bwd_bytes = g.sliced ? align_up(sizeof(float) * (size_t)B * g.nbands * d->E * (4 * kN + 1) * kHB) : 0;
   g.part_bytes = align_up(sizeof(float) * (size_t)g.bwd_bpb * 3 * P * kN);
   const size_t slots = g.sliced ? g.nbands : 1;
-  g.pa_bytes = align_up(sizeof(float) * (size_t)d->B * slots * d->E * 2 * kN);
-  g.pd_bytes = align_up(sizeof(float) * (size_t)d->B * slots * d->E);
+  g.pa_bytes = align_up(sizeof(float) * (size_t)B * slots * d->E * 2 * kN);
+  g.pd_bytes = align_up(sizeof(float) * (size_t)B * slots * d->E);
   return g;
 }
 
@@ -1287,13 +1346,15 @@ size_t workspace_bytes_of(const Geometry& g, int pass, int have_ckpt) {
 bool misaligned(const void* p, size_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
 
 void fill_common(ScanParams& sp, const m2d_desc* d, const Geometry& g) {
-  sp.B = d->B; sp.H = d->H; sp.W = d->W; sp.E = d->E;
+  sp.B = g.vB; sp.H = g.vH; sp.W = d->W; sp.E = d->E;
+  sp.stacked = g.stacked ? 1 : 0; sp.ips = g.ips; sp.Himg = d->H; sp.Breal = d->B; sp.Hs = g.vH;
+  sp.Ptot = (int64_t)d->B * d->H * d->W;
   sp.nbands = g.nbands; sp.nblk = g.nblk;
   sp.S = g.S; sp.T_total = g.T_total; sp.rows_last = g.rows_last;
   sp.magicS = (uint32_t)(((uint64_t)1 << 32) / (uint64_t)g.S);
   sp.sliced = g.sliced ? 1 : 0; sp.sl_nbb = g.nbb; sp.sl_ell = 0; sp.sl_band0 = 0;
   sp.pa_slots = g.sliced ? g.nbands : 1;
-  sp.bot_stride = g.sliced ? (int64_t)d->B * d->W * d->E * kN : 0;
+  sp.bot_stride = g.sliced ? (int64_t)g.vB * d->W * d->E * kN : 0;
   sp.flip = (d->flags & M2D_FLAG_FLIP) ? 1 : 0;
 }
 
@@ -1324,39 +1385,44 @@ int stage_bc(ScanParams& sp, const m2d_desc* d, const void* BT, const void* BL, 
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
-template <typename T, int EC, bool CK, bool WY, bool SX, bool SL>
+template <typename T, int EC, bool CK, bool WY, bool SX, int MODE>
 int launch_fwd_as(const ScanParams& sp, hipStream_t st) {
   using SG = Stage<T, 3, kFwdWaves * 4 * EC, false, true>;
   const size_t lds = 256 + 2 * (size_t)SG::kBytes;
   static bool attr = false;   // idempotent, the value never changes
   if (!attr) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_fwd_kernel<T, EC, CK, WY, SX, SL>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_fwd_kernel<T, EC, CK, WY, SX, MODE>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return M2D_ERR_HIP;
     attr = true;
   }
-  hipLaunchKernelGGL((m2d_fwd_kernel<T, EC, CK, WY, SX, SL>), dim3((unsigned)sp.nwg), dim3(kFwdWaves * 64), lds, st, sp);
+  hipLaunchKernelGGL((m2d_fwd_kernel<T, EC, CK, WY, SX, MODE>), dim3((unsigned)sp.nwg), dim3(kFwdWaves * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
-template <typename T, int EC, bool SX, bool SL>
+template <typename T, int EC, bool SX, int MODE>
 int launch_fwd_mode(const ScanParams& sp, bool ckpt, bool write_y, hipStream_t st) {
-  if (ckpt && write_y) return launch_fwd_as<T, EC, true, true, SX, SL>(sp, st);
-  if (ckpt) return launch_fwd_as<T, EC, true, false, SX, SL>(sp, st);
-  return launch_fwd_as<T, EC, false, true, SX, SL>(sp, st);
+  if (ckpt && write_y) return launch_fwd_as<T, EC, true, true, SX, MODE>(sp, st);
+  if (ckpt) return launch_fwd_as<T, EC, true, false, SX, MODE>(sp, st);
+  return launch_fwd_as<T, EC, false, true, SX, MODE>(sp, st);
 }
 
 template <typename T>
 int launch_fwd(const ScanParams& sp0, const m2d_desc* d, const Geometry& g, bool ckpt, bool write_y, hipStream_t st) {
   ScanParams sp = sp0;
   sp.bpb = g.fwd_bpb;
-  sp.nwg = d->B * g.fwd_bpb;
+  sp.nwg = g.vB * g.fwd_bpb;
   auto once = [&]() {
     if (g.sliced)   // (the sliced sweep is only chosen where one channel per lane is)
-      return g.stage_x ? launch_fwd_mode<T, 1, true, true>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 1, false, true>(sp, ckpt, write_y, st);
+      return g.stage_x ? launch_fwd_mode<T, 1, true, kModeSliced>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 1, false, kModeSliced>(sp, ckpt, write_y, st);
+    if (g.stacked) {
+      if (g.fwd_ec == 2)
+        return g.stage_x ? launch_fwd_mode<T, 2, true, kModeStacked>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 2, false, kModeStacked>(sp, ckpt, write_y, st);
+      return g.stage_x ? launch_fwd_mode<T, 1, true, kModeStacked>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 1, false, kModeStacked>(sp, ckpt, write_y, st);
+    }
     if (g.fwd_ec == 2)
-      return g.stage_x ? launch_fwd_mode<T, 2, true, false>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 2, false, false>(sp, ckpt, write_y, st);
-    return g.stage_x ? launch_fwd_mode<T, 1, true, false>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 1, false, false>(sp, ckpt, write_y, st);
+      return g.stage_x ? launch_fwd_mode<T, 2, true, kModeSweep>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 2, false, kModeSweep>(sp, ckpt, write_y, st);
+    return g.stage_x ? launch_fwd_mode<T, 1, true, kModeSweep>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 1, false, kModeSweep>(sp, ckpt, write_y, st);
   };
   if (!g.sliced) return once();
   // launch l advances band k by blocks [(l - lag*k)*Q, +Q) of its window, for the bands under way
@@ -1367,7 +1433,7 @@ int launch_fwd(const ScanParams& sp0, const m2d_desc* d, const Geometry& g, bool
     if (k_hi > g.nbands - 1) k_hi = g.nbands - 1;
     if (k_lo > k_hi) continue;
     sp.sl_ell = l; sp.sl_band0 = k_lo;
-    sp.nwg = (k_hi - k_lo + 1) * d->B * g.fwd_bpb;
+    sp.nwg = (k_hi - k_lo + 1) * g.vB * g.fwd_bpb;
     const int rc = once();
     if (rc) return rc;
   }
@@ -1394,18 +1460,18 @@ int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   return rc;
 }
 
-template <typename T, bool SX, bool SL>
+template <typename T, bool SX, int MODE>
 int launch_bwd(const ScanParams& sp, hipStream_t st) {
   using SG = Stage<T, 4, kBwdWaves * 4, true, false>;
   const size_t lds = sizeof(float4) * kBwdWaves * 3 * 64 + sizeof(float) * kBwdWaves * 4 * 2 * kN + 256 + 2 * (size_t)SG::kBytes;
   static bool attr = false;   // idempotent, the value never changes
   if (!attr) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_bwd_kernel<T, SX, SL>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_bwd_kernel<T, SX, MODE>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
       return M2D_ERR_HIP;
     attr = true;
   }
-  hipLaunchKernelGGL((m2d_bwd_kernel<T, SX, SL>), dim3((unsigned)sp.nwg), dim3(kBwdWaves * 64), lds, st, sp);
+  hipLaunchKernelGGL((m2d_bwd_kernel<T, SX, MODE>), dim3((unsigned)sp.nwg), dim3(kBwdWaves * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
@@ -1435,10 +1501,11 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   }
   sp.carry = carry_bwd;
   sp.bpb = g.bwd_bpb;
-  sp.nwg = d->B * g.bwd_bpb;
+  sp.nwg = g.vB * g.bwd_bpb;
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][0], st);
   if (!g.sliced) {
-    rc = g.stage_x ? launch_bwd<T, true, false>(sp, st) : launch_bwd<T, false, false>(sp, st);
+    if (g.stacked) rc = g.stage_x ? launch_bwd<T, true, kModeStacked>(sp, st) : launch_bwd<T, false, kModeStacked>(sp, st);
+    else rc = g.stage_x ? launch_bwd<T, true, kModeSweep>(sp, st) : launch_bwd<T, false, kModeSweep>(sp, st);
   } else {
     // as the forward, bottom-up: launch l advances the band k' from the bottom by Q blocks of its window
     const int nlb = (g.nbb + kSliceQ - 1) / kSliceQ;
@@ -1448,8 +1515,8 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
       if (k_hi > g.nbands - 1) k_hi = g.nbands - 1;
       if (k_lo > k_hi) continue;
       sp.sl_ell = l; sp.sl_band0 = g.nbands - 1 - k_hi;
-      sp.nwg = (k_hi - k_lo + 1) * d->B * g.bwd_bpb;
-      rc = g.stage_x ? launch_bwd<T, true, true>(sp, st) : launch_bwd<T, false, true>(sp, st);
+      sp.nwg = (k_hi - k_lo + 1) * g.vB * g.bwd_bpb;
+      rc = g.stage_x ? launch_bwd<T, true, kModeSliced>(sp, st) : launch_bwd<T, false, kModeSliced>(sp, st);
     }
   }
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][1], st);

@@ -87,6 +87,9 @@ SHAPES = [
     (2, 31, 8, 2),    # three bands in one padded stream
     (1, 150, 90, 8),  # 11 bands, one image: every band on workgroups of its own, swept by a sequence of launches
     (70, 56, 30, 4),  # four bands back to back, more images than the sliced sweep takes
+    (301, 7, 7, 4),   # 7x7 images stacked two to a band, last stack of one image
+    (600, 14, 14, 4), # 14x14 images stacked three to a sweep, bands back to back with stride 14
+    (900, 2, 5, 2),   # 2-row images, several to a band
 ]
 
 
@@ -103,7 +106,7 @@ def test_parity_backward_rebuilds_checkpoints(cabi, cscan, shape):
     run_case(cabi, cscan, *shape, dtype=torch.float32, seed=5, with_ckpt=False)
 
 
-@pytest.mark.parametrize("shape", [(2, 14, 14, 4), (1, 70, 9, 2), (3, 5, 9, 4)], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("shape", [(2, 14, 14, 4), (1, 70, 9, 2), (3, 5, 9, 4), (301, 7, 7, 4)], ids=lambda s: "x".join(map(str, s)))
 def test_parity_flipped_scan(cabi, cscan, shape):
     say(f"\ncase flipped_scan shape={shape}")
     run_case(cabi, cscan, *shape, dtype=torch.float32, seed=6, flip=True)
