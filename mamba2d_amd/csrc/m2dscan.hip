@@ -1200,17 +1200,32 @@ __global__ void m2d_finalize_kernel(const ScanParams p, T* dC, T* dBT, T* dBL, T
     T* out = v == 0 ? dC : (v == 1 ? dBT : dBL);
     IO<T>::st4(out + cell * kN + q * 4, s);
   }
-  const int64_t k = gid;
-  if (k < (int64_t)p.E * 2 * kN) {
-    const int e = (int)(k / (2 * kN)), w = (int)(k % (2 * kN));
+  // d_AT, d_AL, d_D: the blocks after the last block of quads add up the per-image partials, 16
+  // lanes to a sum (lane l takes images l, l+16, ...; the 16 partial sums are folded in a fixed
+  // order), so that the loads of one sum are in flight together.
+  const int64_t tail = gid - (nquad + blockDim.x - 1) / blockDim.x * blockDim.x;
+  if (tail >= 0) {
+    const int64_t out = tail >> 4;
+    const int l = (int)(tail & 15);
+    const int nA = p.B * p.pa_slots;
+    const int64_t n_at = (int64_t)p.E * 2 * kN;
     float s = 0.f;
-    for (int g = 0; g < p.B * p.pa_slots; ++g) s += p.pA[((int64_t)g * p.E + e) * (2 * kN) + w];
-    if (w < kN) IO<T>::st(dAT + e * kN + w, s); else IO<T>::st(dAL + e * kN + (w - kN), s);
-  }
-  if (k < p.E) {
-    float s = 0.f;
-    for (int g = 0; g < p.B * p.pa_slots; ++g) s += p.pD[(int64_t)g * p.E + k];
-    IO<T>::st(dD + k, s);
+    if (out < n_at) {
+      const int e = (int)(out / (2 * kN)), w = (int)(out % (2 * kN));
+      for (int g = l; g < nA; g += 16) s += p.pA[((int64_t)g * p.E + e) * (2 * kN) + w];
+    } else if (out < n_at + p.E) {
+      for (int g = l; g < nA; g += 16) s += p.pD[(int64_t)g * p.E + (out - n_at)];
+    }
+#pragma unroll
+    for (int off = 8; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    if (l == 0) {
+      if (out < n_at) {
+        const int e = (int)(out / (2 * kN)), w = (int)(out % (2 * kN));
+        if (w < kN) IO<T>::st(dAT + e * kN + w, s); else IO<T>::st(dAL + e * kN + (w - kN), s);
+      } else if (out < n_at + p.E) {
+        IO<T>::st(dD + (out - n_at), s);
+      }
+    }
   }
 }
 
@@ -1522,9 +1537,9 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][1], st);
   if (rc) return rc;
   const int64_t P = (int64_t)d->B * d->H * d->W;
-  int64_t work = 3 * P * (kN / 4);
-  if (work < (int64_t)d->E * 2 * kN) work = (int64_t)d->E * 2 * kN;
-  hipLaunchKernelGGL(m2d_finalize_kernel<T>, dim3((unsigned)((work + 255) / 256)), dim3(256), 0, st, sp,
+  const int64_t quad_blocks = (3 * P * (kN / 4) + 255) / 256;
+  const int64_t tail_blocks = (((int64_t)d->E * 2 * kN + d->E) * 16 + 255) / 256;   // 16 lanes per position sum
+  hipLaunchKernelGGL(m2d_finalize_kernel<T>, dim3((unsigned)(quad_blocks + tail_blocks)), dim3(256), 0, st, sp,
                      static_cast<T*>(dC), static_cast<T*>(dBT), static_cast<T*>(dBL), static_cast<T*>(dAT),
                      static_cast<T*>(dAL), static_cast<T*>(dD));
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
