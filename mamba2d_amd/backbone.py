@@ -158,8 +158,9 @@ class M2DBlock(nn.Module):
 
 class RoPEAttention2D(nn.Module):
     """Multi-head self-attention over the H*W cells with rotary embeddings on the two grid axes
-    (``models/utils.py:165-316``): the first quarter of every head rotates with the row index, the
-    second with the column index, the rest is left alone; q and k are layer-normed per head."""
+    (``models/utils.py:165-316``): of every head, the first 2*floor(head_dim/4) dims
+    rotate with the row index, the next as many with the column index (16 + 16 of a 32-wide head) and
+    any remainder is left alone; q and k are layer-normed per head."""
 
     def __init__(self, dim, head_dim=32, rope_base=10000.0):
         super().__init__()
@@ -277,3 +278,26 @@ class Mamba2DBackbone(nn.Module):
         for ds, stage in zip(self.ds.values(), self.stages.values()):
             x = stage(ds(x).contiguous())
         return x.permute(0, 3, 1, 2)
+
+
+def load_backbone_checkpoint(model: Mamba2DBackbone, path: str, layers=("ds", "stages")) -> None:
+    """Loads the backbone weights of a training checkpoint of the reference: a file whose
+    ``["state_dict"]`` holds the backbone under the prefix ``backbone.`` next to the classifier head
+    (the convention of ``downstream/Mamba2D/mamba2d.py:397-415``).  Only tensors are read
+    (``weights_only=True``); keys outside ``layers`` are ignored; any key of ``layers`` that is missing
+    on either side raises."""
+    try:
+        ckpt = torch.load(path, weights_only=True, mmap=True)
+    except FileNotFoundError:
+        raise FileNotFoundError(f"Pretrained checkpoint not found: {path}")
+    wanted = lambda name: any(name.startswith(l + ".") for l in layers)
+    sd = {}
+    for name, tensor in ckpt["state_dict"].items():
+        name = name[len("backbone."):] if name.startswith("backbone.") else name
+        if wanted(name):
+            sd[name] = tensor
+    missing, unexpected = model.load_state_dict(sd, strict=False)
+    missing = [k for k in missing if wanted(k)]
+    unexpected = [k for k in unexpected if wanted(k)]
+    if missing or unexpected:
+        raise RuntimeError(f"Backbone/checkpoint key mismatch.\nmissing: {missing}\nunexpected: {unexpected}")

@@ -91,6 +91,30 @@ def test_rotary_tables_match_a_direct_evaluation():
     assert torch.equal(att._rotate_pairs(t), torch.tensor([[-1., 0., -3., 2., -5., 4., -7., 6.]]))
 
 
+def test_training_checkpoint_of_the_reference_layout_loads(tmp_path):
+    """A file shaped like the reference's Lightning checkpoints (state_dict with the backbone under
+    'backbone.' next to head weights, downstream/Mamba2D/mamba2d.py:397-415) loads key by key."""
+    from mamba2d_amd.backbone import load_backbone_checkpoint
+    torch.manual_seed(3)
+    src = build(n_blocks=(1, 1, 1, 1))
+    sd = {"backbone." + k: v.clone() for k, v in src.state_dict().items()}
+    sd["head.fc1.weight"] = torch.zeros(4, 4)          # classifier parts are ignored
+    sd["norm.weight"] = torch.ones(512)
+    path = tmp_path / "m2d.ckpt"
+    torch.save({"state_dict": sd, "epoch": 3}, path)
+    dst = build(n_blocks=(1, 1, 1, 1))
+    assert not torch.equal(dst.state_dict()["stages.0.0.token_mixer.in_proj.weight"], src.state_dict()["stages.0.0.token_mixer.in_proj.weight"])
+    load_backbone_checkpoint(dst, str(path))
+    for k, v in src.state_dict().items():
+        assert torch.equal(dst.state_dict()[k], v), k
+    # a checkpoint of another depth does not load silently
+    other = build(n_blocks=(2, 1, 1, 1))
+    with pytest.raises(RuntimeError):
+        load_backbone_checkpoint(other, str(path))
+    with pytest.raises(FileNotFoundError):
+        load_backbone_checkpoint(dst, str(tmp_path / "nope.ckpt"))
+
+
 @pytest.mark.gpu
 def test_bottom_right_block_equals_flipped_top_left_block():
     from mamba2d_amd.backbone import M2DBlock
