@@ -116,6 +116,25 @@ __device__ __forceinline__ void ld16f(const float* p, float (&v)[kN]) {
 __device__ __forceinline__ float from_row_below(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x111 /*row_shr:1*/, 0xf, 0xf, true));
 }
+// The same move folded into the instruction that uses the value (the compiler does this for adds
+// but not for multiply-adds): acc + a * (v of the lane below), a * (v of the lane below),
+// a + (v of the lane above).  The operand v is always a value of the step before, produced many
+// instructions earlier, so the two wait states a DPP read needs after a VALU write of the same
+// register have long passed.
+__device__ __forceinline__ float fma_row_below(float a, float v, float acc) {
+  asm("v_fmac_f32_dpp %0, %1, %2 row_shr:1 row_mask:0xf bank_mask:0xf bound_ctrl:1" : "+v"(acc) : "v"(v), "v"(a));
+  return acc;
+}
+__device__ __forceinline__ float mul_row_below(float a, float v) {
+  float d;
+  asm("v_mul_f32_dpp %0, %1, %2 row_shr:1 row_mask:0xf bank_mask:0xf bound_ctrl:1" : "=v"(d) : "v"(v), "v"(a));
+  return d;
+}
+__device__ __forceinline__ float add_row_above(float a, float v) {
+  float d;
+  asm("v_add_f32_dpp %0, %1, %2 row_shl:1 row_mask:0xf bank_mask:0xf bound_ctrl:1" : "=v"(d) : "v"(v), "v"(a));
+  return d;
+}
 // ... or the value of lane r+1 (lane 15 receives 0).
 __device__ __forceinline__ float from_row_above(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x101 /*row_shl:1*/, 0xf, 0xf, true));
@@ -634,16 +653,24 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
       for (int q = 0; q < 4; ++q) {
         const float4 b4 = o.bt[c][q], l4 = o.bl[q], c4 = o.cc[q];
         const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w}, cq[4] = {c4.x, c4.y, c4.z, c4.w};
+        // The T gates first, then the L gates, then the four state chains: the multiply-add that
+        // takes the state of the row above through DPP is inline assembly, which the compiler's
+        // hazard recogniser does not see, and it must not issue right behind the v_exp that
+        // produces its gate (a transcendental result needs one wait state before a VALU reads it).
+        float aT[4], aL[4];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) aT[w] = fexp2(__builtin_fmaf(o.dtv[c], a2t[c][sinv<PERM>(4 * q + w)], offT));
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) aL[w] = fexp2(__builtin_fmaf(o.dlv[c], a2l[c][sinv<PERM>(4 * q + w)], offL));
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
           const int n = sinv<PERM>(4 * q + w);
-          const float aT = fexp2(__builtin_fmaf(o.dtv[c], a2t[c][n], offT));
-          const float aL = fexp2(__builtin_fmaf(o.dlv[c], a2l[c][n], offL));
-          const float hT = from_row_below(h[c][n]);
           float u = sL * lq[w];
           u = __builtin_fmaf(sT, bq[w], u);
-          u = __builtin_fmaf(aT, hT, u);
-          const float hn = __builtin_fmaf(aL, h[c][n], u);
+          u = fma_row_below(aT[w], h[c][n], u);       // + aT * h of the row above (the lane below)
+          const float hn = __builtin_fmaf(aL[w], h[c][n], u);
           h[c][n] = hn;
           if (WRITE_Y) acc = __builtin_fmaf(hn, cq[w], acc);
         }
@@ -980,16 +1007,20 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
             const float4 b4 = reinterpret_cast<const float4*>(rec)[mg], l4 = reinterpret_cast<const float4*>(rec + kN * 4)[mg];
             const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
             const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w};
+            float aT[4], aL[4];   // gates before chains, see the forward kernel
+#pragma unroll
+            for (int qi = 0; qi < 4; ++qi) aT[qi] = fexp2(__builtin_fmaf(dtv, atq[qi], offT));
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int qi = 0; qi < 4; ++qi) aL[qi] = fexp2(__builtin_fmaf(dlv, alq[qi], offL));
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int qi = 0; qi < 4; ++qi) {
               const int s8 = 4 * mgl + qi;
-              const float aT = fexp2(__builtin_fmaf(dtv, atq[qi], offT));
-              const float aL = fexp2(__builtin_fmaf(dlv, alq[qi], offL));
-              const float hT = from_row_below(hb[k][s8]);
               float u = sL * lq[qi];
               u = __builtin_fmaf(sT, bq[qi], u);
-              u = __builtin_fmaf(aT, hT, u);
-              hb[k + 1][s8] = __builtin_fmaf(aL, hb[k][s8], u);
+              u = fma_row_below(aT[qi], hb[k][s8], u);
+              hb[k + 1][s8] = __builtin_fmaf(aL[qi], hb[k][s8], u);
             }
           }
         }
@@ -1048,13 +1079,11 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
               const float a2t = atq[qi], a2l = alq[qi];
               const float aT = fexp2(__builtin_fmaf(dtv, a2t, offT));
               const float aL = fexp2(__builtin_fmaf(dlv, a2l, offL));
-              const float mb = from_row_above(muT[n]);
-              const float lam = __builtin_fmaf(dyl, cq[qi], muL[n] + mb);
-              const float hT = from_row_below(hb[k][s8]);
+              const float lam = __builtin_fmaf(dyl, cq[qi], add_row_above(muL[n], muT[n]));
               const float mT = aT * lam, mL = aL * lam;
               muT[n] = mT;
               muL[n] = mL;
-              const float ZT = mT * hT, ZL = mL * hb[k][s8];
+              const float ZT = mul_row_below(mT, hb[k][s8]), ZL = mL * hb[k][s8];
               accAT[n] = __builtin_fmaf(ZT, dtv, accAT[n]);
               accAL[n] = __builtin_fmaf(ZL, dlv, accAL[n]);
               zT = __builtin_fmaf(ZT, a2t, zT);
