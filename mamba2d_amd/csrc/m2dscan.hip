@@ -412,6 +412,16 @@ __device__ __forceinline__ void staging_landed() {
   __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0); known to the compiler, so loads it tracks need no further wait
   asm volatile("" ::: "memory");
 }
+// The same with the N youngest vector-memory operations of the wave left in flight.  The counter
+// retires loads and stores in issue order, so everything older than those N has completed; the
+// caller must know that at least N operations were issued after the loads it waits for.
+template <int N>
+__device__ __forceinline__ void staging_landed_behind() {
+  static_assert(N >= 0 && N < 16, "low bits of the counter field only");
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt(0x0F70 | N);
+  asm volatile("" ::: "memory");
+}
 // ... and those of the other waves too
 __device__ __forceinline__ void staging_fence() {
   staging_landed();
@@ -724,6 +734,13 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
     }
     const char* bufc = lds + cur * SG::kBytes;
     const char* bufn = lds + (cur ^ 1) * SG::kBytes;
+    // (uniform) some lane writes y at each of the first three steps: the wave issues at least
+    // three stores between the copies for the next block and the barrier that ends this one
+    const bool y_thrice = WRITE_Y && __any((bp.in_grid & 7u) == 7u);
+    auto next_block_landed = [&] {
+      // the stores just issued need not have completed, only the copies before them
+      if (y_thrice) staging_landed_behind<3>(); else staging_landed();
+    };
     if constexpr (AHEAD) {
       static_assert(kCK % 2 == 0, "the two operand sets alternate and must close over a block");
 #pragma unroll
@@ -737,7 +754,7 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
           // Last step of the block: its operands are in registers already, so the buffer can be
           // handed over now.  The copies of the next block have landed in every wave after this
           // barrier, and no wave reads the current buffer any more.
-          staging_landed();
+          next_block_landed();
           __syncthreads();
           if (!last) fetch(bufn, 0, ahead);
         }
@@ -750,7 +767,7 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
         // The operands of the next block must have landed before the barrier that ends this
         // block.  Waiting here, before the stores of the last step are issued, keeps the latency
         // of those stores off the critical path (the counter covers loads and stores alike).
-        if (k == kCK - 1) staging_landed();
+        if (k == kCK - 1) next_block_landed();
         if (t < p.T_total) {
           fetch(bufc, k, opsA);
           step(k, opsA);
