@@ -114,6 +114,45 @@ int m2d_scan_bwd(const m2d_desc* desc,
                  void* workspace, size_t workspace_bytes,
                  void* stream);
 
+/* ---- Projections either side of the scan -------------------------------------------------
+ * The reference computes the scan's parameters from x with stock operators (proj_params,
+ * models/kernels/wavefront_cuda.py:63-95) and differentiates them with autograd
+ * (wavefront_cuda.py:262-296).  The two calls below do the same work in hand-written kernels.
+ * desc->H and desc->W only enter through the number of positions P = B*H*W; flags are ignored.
+ * Activations have the element type of desc->dtype; weights, biases and their gradients are
+ * fp32 (pass the values the reference would use, i.e. already rounded to the activation dtype
+ * if the caller casts its weights, wavefront_cuda.py:327-332).  dt_rank <= 32, E <= 4096.
+ *
+ *   x_proj_w  (2*dt_rank + 3*N, E)     dt_proj{T,L}_w (E, dt_rank)     dt_proj{T,L}_b (E)
+ *   lowrank   (B,H,W, 2*dt_rank)       the inputs of the two dt projections, T then L
+ */
+size_t m2d_proj_workspace_bytes(const m2d_desc* desc, int dt_rank, int pass);
+
+/* lowrank | BT | BL | C = split(x @ x_proj_w^T);  delta{T,L} = softplus(lowrank{T,L} @ dt_proj{T,L}_w^T + b)
+ * (wavefront_cuda.py:75-86).  All six outputs are written. */
+int m2d_proj_fwd(const m2d_desc* desc, int dt_rank,
+                 const void* x,
+                 const float* x_proj_w, const float* dt_projT_w, const float* dt_projT_b,
+                 const float* dt_projL_w, const float* dt_projL_b,
+                 void* lowrank, void* deltaT, void* deltaL, void* BT, void* BL, void* C,
+                 void* workspace, size_t workspace_bytes,
+                 void* stream);
+
+/* Backward of m2d_proj_fwd for the gradients d_deltaT ... d_C that m2d_scan_bwd produced.
+ * dx is read and written: on entry the scan's own gradient for x, on return that plus the
+ * gradient through the projections (wavefront_cuda.py:303-311).  The five weight gradients are
+ * written (not accumulated). */
+int m2d_proj_bwd(const m2d_desc* desc, int dt_rank,
+                 const void* x, const void* lowrank, const void* deltaT, const void* deltaL,
+                 const float* x_proj_w, const float* dt_projT_w, const float* dt_projL_w,
+                 const void* d_deltaT, const void* d_deltaL,
+                 const void* d_BT, const void* d_BL, const void* d_C,
+                 void* dx,
+                 float* d_x_proj_w, float* d_dt_projT_w, float* d_dt_projT_b,
+                 float* d_dt_projL_w, float* d_dt_projL_b,
+                 void* workspace, size_t workspace_bytes,
+                 void* stream);
+
 /* Measurement aid; no counterpart in the reference.  While enabled, every m2d_scan_fwd /
  * m2d_scan_bwd call records a pair of HIP events on its stream around the main scan kernel of
  * the pass (not around the small set-up and reduction kernels).  m2d_profile_last_ms waits for

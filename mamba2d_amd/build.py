@@ -26,8 +26,8 @@ HIPCC_FLAGS = [
 
 
 def build_lib(verbose: bool = True) -> str:
-    src = os.path.join(HERE, "csrc", "m2dscan.hip")
-    cmd = ["hipcc", *HIPCC_FLAGS, "-I", os.path.join(ROOT, "include"), "-o", LIB, src]
+    srcs = [os.path.join(HERE, "csrc", n) for n in ("m2dscan.hip", "m2dproj.hip")]
+    cmd = ["hipcc", *HIPCC_FLAGS, "-I", os.path.join(ROOT, "include"), "-o", LIB, *srcs]
     if verbose:
         print(" ".join(cmd), flush=True)
     subprocess.check_call(cmd)

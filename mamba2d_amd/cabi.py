@@ -18,7 +18,8 @@ M2D_FLAG_FLIP = 1
 M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
-           "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_bwd", "m2d_profile_enable", "m2d_profile_last_ms")
+           "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_bwd", "m2d_proj_workspace_bytes", "m2d_proj_fwd",
+           "m2d_proj_bwd", "m2d_profile_enable", "m2d_profile_last_ms")
 
 
 class Desc(ctypes.Structure):
@@ -52,6 +53,12 @@ def _load():
     lib.m2d_scan_fwd.argtypes = [dp] + [vp] * 9 + [vp, vp, sz, vp, sz, vp]
     lib.m2d_scan_bwd.restype = i32
     lib.m2d_scan_bwd.argtypes = [dp] + [vp] * 10 + [vp, sz] + [vp] * 9 + [vp, sz, vp]
+    lib.m2d_proj_workspace_bytes.restype = sz
+    lib.m2d_proj_workspace_bytes.argtypes = [dp, i32, i32]
+    lib.m2d_proj_fwd.restype = i32
+    lib.m2d_proj_fwd.argtypes = [dp, i32] + [vp] * 12 + [vp, sz, vp]
+    lib.m2d_proj_bwd.restype = i32
+    lib.m2d_proj_bwd.argtypes = [dp, i32] + [vp] * 18 + [vp, sz, vp]
     lib.m2d_profile_enable.restype = i32
     lib.m2d_profile_enable.argtypes = [i32]
     lib.m2d_profile_last_ms.restype = i32
@@ -155,4 +162,55 @@ def scan_bwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt=None, flip=False)
     check(lib.m2d_scan_bwd(ctypes.byref(d), *[_ptr(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy)],
                            _ptr(ckpt), ckpt.numel() if ckpt is not None else 0, *[_ptr(t) for t in outs],
                            _ptr(ws), ws.numel(), _stream(x.device)))
+    return tuple(outs)
+
+
+def _proj_check(x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, N):
+    if x.dim() != 4 or not x.is_cuda or not x.is_contiguous():
+        raise ValueError("m2dscan: x must be a contiguous (B,H,W,E) tensor on the GPU")
+    E = x.shape[-1]
+    R = dt_projT_w.shape[1]
+    want = {"x_proj_w": (x_proj_w, (2 * R + 3 * N, E)), "dt_projT_w": (dt_projT_w, (E, R)), "dt_projT_b": (dt_projT_b, (E,)),
+            "dt_projL_w": (dt_projL_w, (E, R)), "dt_projL_b": (dt_projL_b, (E,))}
+    for k, (t, shp) in want.items():
+        if tuple(t.shape) != shp or t.dtype != torch.float32 or t.device != x.device or not t.is_contiguous():
+            raise ValueError(f"m2dscan: {k} must be a contiguous float32 tensor of shape {shp} on {x.device}")
+    return R
+
+
+def proj_fwd(x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, N=16):
+    """(lowrank, deltaT, deltaL, BT, BL, C) through m2d_proj_fwd; weights are float32 tensors."""
+    R = _proj_check(x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, N)
+    B, H, W, E = x.shape
+    d = make_desc(x, N)
+    low = x.new_empty((B, H, W, 2 * R))
+    dT, dL = torch.empty_like(x), torch.empty_like(x)
+    BT, BL, C = (x.new_empty((B, H, W, N)) for _ in range(3))
+    ws = _bytes(lib.m2d_proj_workspace_bytes(ctypes.byref(d), R, M2D_PASS_FWD), x.device)
+    check(lib.m2d_proj_fwd(ctypes.byref(d), R, *[_ptr(t) for t in (x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w,
+                                                                  dt_projL_b, low, dT, dL, BT, BL, C)],
+                           _ptr(ws), ws.numel(), _stream(x.device)))
+    return low, dT, dL, BT, BL, C
+
+
+def proj_bwd(x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w, dt_projL_w, d_deltaT, d_deltaL, d_BT, d_BL, d_C, dx):
+    """Adds the gradient through the projections to ``dx`` in place and returns the five weight
+    gradients (x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b; float32) through m2d_proj_bwd."""
+    N = d_BT.shape[-1]
+    zb = torch.zeros(x.shape[-1], device=x.device)
+    R = _proj_check(x, x_proj_w, dt_projT_w, zb, dt_projL_w, zb, N)
+    B, H, W, E = x.shape
+    _same(x, lowrank, deltaT, deltaL, d_deltaT, d_deltaL, d_BT, d_BL, d_C, dx)
+    want = {"lowrank": (lowrank, (B, H, W, 2 * R)), "deltaT": (deltaT, (B, H, W, E)), "deltaL": (deltaL, (B, H, W, E)),
+            "d_deltaT": (d_deltaT, (B, H, W, E)), "d_deltaL": (d_deltaL, (B, H, W, E)), "d_BT": (d_BT, (B, H, W, N)),
+            "d_BL": (d_BL, (B, H, W, N)), "d_C": (d_C, (B, H, W, N)), "dx": (dx, (B, H, W, E))}
+    for k, (t, shp) in want.items():
+        if tuple(t.shape) != shp:
+            raise ValueError(f"m2dscan: {k} has shape {tuple(t.shape)}, expected {shp}")
+    d = make_desc(x, N)
+    outs = [torch.empty_like(t) for t in (x_proj_w, dt_projT_w, zb, dt_projL_w, zb)]
+    ws = _bytes(lib.m2d_proj_workspace_bytes(ctypes.byref(d), R, M2D_PASS_BWD), x.device)
+    check(lib.m2d_proj_bwd(ctypes.byref(d), R, *[_ptr(t) for t in (x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w,
+                                                                  dt_projL_w, d_deltaT, d_deltaL, d_BT, d_BL, d_C, dx)],
+                           *[_ptr(t) for t in outs], _ptr(ws), ws.numel(), _stream(x.device)))
     return tuple(outs)

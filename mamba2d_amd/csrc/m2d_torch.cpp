@@ -2,7 +2,9 @@
 //
 // Registers two functional operators, m2dscan::scan_fwd and m2dscan::scan_bwd, which take the
 // place of the reference's pair of in-place custom ops mamba2d::wf_fwd / mamba2d::wf_bwd
-// (models/kernels/wavefront_cuda.py:25-57) plus the tensor algebra around them.  The shim only
+// (models/kernels/wavefront_cuda.py:25-57) plus the tensor algebra around them, and
+// m2dscan::proj_fwd / m2dscan::proj_bwd for the projections that feed the scan
+// (wavefront_cuda.py:63-95 and their autograd backward).  The shim only
 // validates tensors, allocates outputs / scratch through the caching allocator, picks the
 // current HIP stream and forwards raw pointers; all arithmetic lives behind the C ABI.
 #include <ATen/ATen.h>
@@ -107,6 +109,86 @@ std::vector<Tensor> scan_bwd(const Tensor& x, const Tensor& dT, const Tensor& dL
   return g;
 }
 
+// ---- projections either side of the scan (reference: proj_params, wavefront_cuda.py:63-95)
+void expect_weight(const Tensor& t, const char* name, const Tensor& x, at::IntArrayRef shape) {
+  TORCH_CHECK(t.device() == x.device(), "m2dscan: ", name, " is on ", t.device(), ", x on ", x.device());
+  TORCH_CHECK(t.scalar_type() == at::kFloat, "m2dscan: ", name, " must be float32, got ", t.scalar_type());
+  TORCH_CHECK(t.sizes() == shape, "m2dscan: ", name, " has shape ", t.sizes(), ", expected ", shape);
+  TORCH_CHECK(t.is_contiguous(), "m2dscan: ", name, " must be contiguous");
+}
+
+m2d_desc describe_proj(const Tensor& x, int64_t N) {
+  TORCH_CHECK(x.dim() == 4 && x.is_cuda() && x.is_contiguous(), "m2dscan: x must be a contiguous (B,H,W,E) tensor on the GPU");
+  m2d_desc d{};
+  d.B = static_cast<int32_t>(x.size(0));
+  d.H = static_cast<int32_t>(x.size(1));
+  d.W = static_cast<int32_t>(x.size(2));
+  d.E = static_cast<int32_t>(x.size(3));
+  d.N = static_cast<int32_t>(N);
+  if (x.scalar_type() == at::kFloat) d.dtype = M2D_F32;
+  else if (x.scalar_type() == at::kBFloat16) d.dtype = M2D_BF16;
+  else TORCH_CHECK(false, "m2dscan: float32 and bfloat16 are supported, got ", x.scalar_type());
+  return d;
+}
+
+std::vector<Tensor> proj_fwd(const Tensor& x, const Tensor& Wx, const Tensor& wT, const Tensor& bT, const Tensor& wL,
+                             const Tensor& bL, int64_t N) {
+  const m2d_desc d = describe_proj(x, N);
+  TORCH_CHECK(wT.dim() == 2, "m2dscan: dt_projT_w must be (E, dt_rank)");
+  const int64_t B = d.B, H = d.H, W = d.W, E = d.E, R = wT.size(1);
+  expect_weight(Wx, "x_proj_w", x, {2 * R + 3 * N, E});
+  expect_weight(wT, "dt_projT_w", x, {E, R});
+  expect_weight(bT, "dt_projT_b", x, {E});
+  expect_weight(wL, "dt_projL_w", x, {E, R});
+  expect_weight(bL, "dt_projL_b", x, {E});
+  c10::DeviceGuard guard(x.device());
+  std::vector<Tensor> o = {at::empty({B, H, W, 2 * R}, x.options()), at::empty_like(x), at::empty_like(x),
+                           at::empty({B, H, W, N}, x.options()), at::empty({B, H, W, N}, x.options()),
+                           at::empty({B, H, W, N}, x.options())};
+  const size_t need = m2d_proj_workspace_bytes(&d, static_cast<int>(R), M2D_PASS_FWD);
+  TORCH_CHECK(need > 0, "m2dscan: projection shapes outside what the kernels are built for (N = 16, dt_rank <= 32, E <= 4096)");
+  Tensor ws = bytes(need, x);
+  hipStream_t st = c10::hip::getCurrentHIPStream(x.device().index()).stream();
+  check(m2d_proj_fwd(&d, static_cast<int>(R), x.data_ptr(), Wx.data_ptr<float>(), wT.data_ptr<float>(), bT.data_ptr<float>(),
+                     wL.data_ptr<float>(), bL.data_ptr<float>(), o[0].data_ptr(), o[1].data_ptr(), o[2].data_ptr(),
+                     o[3].data_ptr(), o[4].data_ptr(), o[5].data_ptr(), ws.data_ptr(), static_cast<size_t>(ws.numel()), st));
+  return o;
+}
+
+std::vector<Tensor> proj_bwd(const Tensor& x, const Tensor& low, const Tensor& dT, const Tensor& dL, const Tensor& Wx,
+                             const Tensor& wT, const Tensor& wL, const Tensor& ddT, const Tensor& ddL, const Tensor& dBT,
+                             const Tensor& dBL, const Tensor& dC, Tensor dx) {
+  TORCH_CHECK(dBT.dim() == 4 && wT.dim() == 2, "m2dscan: d_BT must be (B,H,W,N) and dt_projT_w (E, dt_rank)");
+  const int64_t N = dBT.size(3);
+  const m2d_desc d = describe_proj(x, N);
+  const int64_t B = d.B, H = d.H, W = d.W, E = d.E, R = wT.size(1);
+  expect_weight(Wx, "x_proj_w", x, {2 * R + 3 * N, E});
+  expect_weight(wT, "dt_projT_w", x, {E, R});
+  expect_weight(wL, "dt_projL_w", x, {E, R});
+  expect(low, "lowrank", x, {B, H, W, 2 * R});
+  expect(dT, "deltaT", x, {B, H, W, E});
+  expect(dL, "deltaL", x, {B, H, W, E});
+  expect(ddT, "d_deltaT", x, {B, H, W, E});
+  expect(ddL, "d_deltaL", x, {B, H, W, E});
+  expect(dBT, "d_BT", x, {B, H, W, N});
+  expect(dBL, "d_BL", x, {B, H, W, N});
+  expect(dC, "d_C", x, {B, H, W, N});
+  expect(dx, "dx", x, {B, H, W, E});
+  c10::DeviceGuard guard(x.device());
+  std::vector<Tensor> g = {at::empty_like(Wx), at::empty_like(wT), at::empty({E}, wT.options()), at::empty_like(wL),
+                           at::empty({E}, wT.options())};
+  const size_t need = m2d_proj_workspace_bytes(&d, static_cast<int>(R), M2D_PASS_BWD);
+  TORCH_CHECK(need > 0, "m2dscan: projection shapes outside what the kernels are built for (N = 16, dt_rank <= 32, E <= 4096)");
+  Tensor ws = bytes(need, x);
+  hipStream_t st = c10::hip::getCurrentHIPStream(x.device().index()).stream();
+  check(m2d_proj_bwd(&d, static_cast<int>(R), x.data_ptr(), low.data_ptr(), dT.data_ptr(), dL.data_ptr(),
+                     Wx.data_ptr<float>(), wT.data_ptr<float>(), wL.data_ptr<float>(), ddT.data_ptr(), ddL.data_ptr(),
+                     dBT.data_ptr(), dBL.data_ptr(), dC.data_ptr(), dx.data_ptr(), g[0].data_ptr<float>(),
+                     g[1].data_ptr<float>(), g[2].data_ptr<float>(), g[3].data_ptr<float>(), g[4].data_ptr<float>(),
+                     ws.data_ptr(), static_cast<size_t>(ws.numel()), st));
+  return g;
+}
+
 int64_t abi_version() { return m2d_version(); }
 
 }  // namespace
@@ -116,10 +198,16 @@ TORCH_LIBRARY(m2dscan, m) {
         "Tensor D, bool save_ckpt, bool flip) -> (Tensor, Tensor)");
   m.def("scan_bwd(Tensor x, Tensor deltaT, Tensor deltaL, Tensor AT, Tensor AL, Tensor BT, Tensor BL, Tensor C, "
         "Tensor D, Tensor dy, Tensor ckpt, bool flip) -> Tensor[]");
+  m.def("proj_fwd(Tensor x, Tensor x_proj_w, Tensor dt_projT_w, Tensor dt_projT_b, Tensor dt_projL_w, Tensor dt_projL_b, "
+        "int d_state) -> Tensor[]");
+  m.def("proj_bwd(Tensor x, Tensor lowrank, Tensor deltaT, Tensor deltaL, Tensor x_proj_w, Tensor dt_projT_w, "
+        "Tensor dt_projL_w, Tensor d_deltaT, Tensor d_deltaL, Tensor d_BT, Tensor d_BL, Tensor d_C, Tensor(a!) dx) -> Tensor[]");
   m.def("abi_version() -> int", &abi_version);
 }
 
 TORCH_LIBRARY_IMPL(m2dscan, CUDA, m) {   // ROCm devices dispatch under the CUDA key
   m.impl("scan_fwd", &scan_fwd);
   m.impl("scan_bwd", &scan_bwd);
+  m.impl("proj_fwd", &proj_fwd);
+  m.impl("proj_bwd", &proj_bwd);
 }

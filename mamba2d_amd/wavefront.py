@@ -10,6 +10,9 @@ argument order and the same error behaviour, so that ``M2DBlock.ssm``
   ``m2dscan::scan_fwd`` and ``m2dscan::scan_bwd`` (csrc/m2d_torch.cpp -> include/m2dscan.h);
   the (B,H,W,E,N) state tensor never exists in memory.
 * state and accumulation are fp32 also for bf16 tensors.
+* the entry point runs the projections (``proj_params``, ``wavefront_cuda.py:63-95``) and their
+  backward in the library's own kernels (``wf_cuda_fn_proj``); ``proj_params``, ``wf_cuda_fn_pr``
+  and ``wf_cuda_fn_fr`` keep the reference's form for callers that use them directly.
 
 There is no fallback path: importing this module raises if the native parts are not built.
 """
@@ -31,11 +34,17 @@ torch.ops.load_library(_SHIM)
 
 scan_fwd_op = torch.ops.m2dscan.scan_fwd
 scan_bwd_op = torch.ops.m2dscan.scan_bwd
+proj_fwd_op = torch.ops.m2dscan.proj_fwd
+proj_bwd_op = torch.ops.m2dscan.proj_bwd
 
 # Keep the forward's anti-diagonal checkpoints for the backward (faster backward, more saved
 # memory) or rebuild them inside the backward (nothing saved beyond the inputs, like the
 # reference's partial recomputation).  Module-level switch, read at forward time.
 SAVE_CHECKPOINTS = os.environ.get("M2D_SAVE_CHECKPOINTS", "1") != "0"
+
+# The entry point computes the projections with the library's own kernels (wf_cuda_fn_proj) or
+# with stock torch operators followed by wf_cuda_fn_pr / wf_cuda_fn_fr.  Read at call time.
+FUSED_PROJECTIONS = os.environ.get("M2D_FUSED_PROJECTIONS", "1") != "0"
 
 
 def _ckpt_bytes(x, N, flip=False) -> int:
@@ -52,6 +61,20 @@ def _scan_fwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, save_ckpt, flip):
 @torch.library.register_fake("m2dscan::scan_bwd")
 def _scan_bwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt, flip):
     return [torch.empty_like(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D)]
+
+
+@torch.library.register_fake("m2dscan::proj_fwd")
+def _proj_fwd_fake(x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, d_state):
+    B, H, W, _ = x.shape
+    R = dt_projT_w.shape[1]
+    bc = [x.new_empty((B, H, W, d_state)) for _ in range(3)]
+    return [x.new_empty((B, H, W, 2 * R)), torch.empty_like(x), torch.empty_like(x), *bc]
+
+
+@torch.library.register_fake("m2dscan::proj_bwd")
+def _proj_bwd_fake(x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w, dt_projL_w, d_deltaT, d_deltaL, d_BT, d_BL, d_C, dx):
+    b = dt_projT_w.new_empty((x.shape[-1],))
+    return [torch.empty_like(x_proj_w), torch.empty_like(dt_projT_w), b, torch.empty_like(dt_projL_w), torch.empty_like(b)]
 
 
 def proj_params(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b):
@@ -131,6 +154,64 @@ class wf_cuda_fn_fr(torch.autograd.Function):
         return (d_x, *grads[1:], d_D, None)
 
 
+def _proj_kernels_cover(x, AT_log, dt_projT_w) -> bool:
+    """Shapes the projection kernels are built for; anything else takes the stock operators."""
+    return AT_log.shape[1] == 16 and dt_projT_w.shape[1] <= 32 and x.shape[-1] <= 4096
+
+
+class wf_cuda_fn_proj(torch.autograd.Function):
+    """Projections and scan behind one Function, all in the library's own kernels.
+
+    Same function of the nine raw inputs as ``proj_params`` followed by ``wf_cuda_fn_pr``
+    (reference ``wavefront_cuda.py:63-95``, ``:146-196``) or as ``wf_cuda_fn_fr`` (``:199-313``).
+    ``full=False`` keeps the projection outputs and the scan's checkpoints for the backward;
+    ``full=True`` keeps only x and the weights and rebuilds the rest in the backward."""
+
+    @staticmethod
+    def _project(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b):
+        w32 = [_c(t.float()) for t in (x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b)]
+        AT = (-torch.exp(AT_log.float())).to(x.dtype)
+        AL = (-torch.exp(AL_log.float())).to(x.dtype)
+        return w32, AT, AL, proj_fwd_op(x, *w32, AT_log.shape[1])
+
+    @staticmethod
+    def forward(ctx, x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D,
+                full=False, flip=False):
+        x, D = _c(x), _c(D)
+        weights = (AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b)
+        _, AT, AL, (low, dT, dL, BT, BL, C) = wf_cuda_fn_proj._project(x, *weights)
+        keep = SAVE_CHECKPOINTS and not full and any(ctx.needs_input_grad)
+        y, ck = scan_fwd_op(x, dT, dL, AT, AL, BT, BL, C, D, keep, bool(flip))
+        if full:
+            ctx.save_for_backward(x, *weights, D)
+        else:
+            ctx.save_for_backward(x, *weights, D, low, dT, dL, BT, BL, C, ck)
+        ctx.full, ctx.flip = bool(full), bool(flip)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        x, *weights, D = ctx.saved_tensors[:9]
+        AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b = weights
+        dy = _c(grad_output.to(x.dtype))
+        if ctx.full:
+            w32, AT, AL, (low, dT, dL, BT, BL, C) = wf_cuda_fn_proj._project(x, *weights)
+            ck = x.new_empty((1,), dtype=torch.uint8)
+        else:
+            low, dT, dL, BT, BL, C, ck = ctx.saved_tensors[9:]
+            w32 = [_c(t.float()) for t in (x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b)]
+            AT = (-torch.exp(AT_log.float())).to(x.dtype)
+            AL = (-torch.exp(AL_log.float())).to(x.dtype)
+        d_x, d_dT, d_dL, d_AT, d_AL, d_BT, d_BL, d_C, d_D = scan_bwd_op(x, dT, dL, AT, AL, BT, BL, C, D, dy, ck, ctx.flip)
+        # d_x holds the scan's own gradient (dy*D included); the projections add theirs in place
+        g_xw, g_wT, g_bT, g_wL, g_bL = proj_bwd_op(x, low, dT, dL, w32[0], w32[1], w32[3], d_dT, d_dL, d_BT, d_BL, d_C, d_x)
+        # A = -exp(A_log): dA/dA_log = A
+        d_AT_log = (d_AT.float() * -torch.exp(AT_log.float())).to(AT_log.dtype)
+        d_AL_log = (d_AL.float() * -torch.exp(AL_log.float())).to(AL_log.dtype)
+        return (d_x, d_AT_log, d_AL_log, g_xw.to(x_proj_w.dtype), g_wT.to(dt_projT_w.dtype), g_bT.to(dt_projT_b.dtype),
+                g_wL.to(dt_projL_w.dtype), g_bL.to(dt_projL_b.dtype), d_D, None, None)
+
+
 def wavefront_scan_cuda(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D,
                         recomp="partial", *, flip=False):
     """Entry point with the reference's signature (``wavefront_cuda.py:315-347``).
@@ -150,11 +231,14 @@ def wavefront_scan_cuda(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_
     dt_projL_b = dt_projL_b.to(x.dtype)
     D = D.to(x.dtype)
 
+    if recomp not in ("partial", "full"):
+        raise ValueError(f"Unknown recomputation mode, got {recomp}...")
+    if FUSED_PROJECTIONS and _proj_kernels_cover(x, AT_log, dt_projT_w):
+        return wf_cuda_fn_proj.apply(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D,
+                                     recomp == "full", flip)
     if recomp == "partial":
         deltaT, deltaL, AT, AL, BT, BL, C = proj_params(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b,
                                                         dt_projL_w, dt_projL_b)
         return wf_cuda_fn_pr.apply(x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip)
-    if recomp == "full":
-        return wf_cuda_fn_fr.apply(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w,
-                                   dt_projL_b, D, flip)
-    raise ValueError(f"Unknown recomputation mode, got {recomp}...")
+    return wf_cuda_fn_fr.apply(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w,
+                               dt_projL_b, D, flip)

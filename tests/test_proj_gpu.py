@@ -1,0 +1,107 @@
+"""GPU parity tests of the projection kernels (m2d_proj_fwd / m2d_proj_bwd) through the C ABI.
+
+The checker is the restatement of the reference's proj_params with stock torch operators in
+fp64 on the CPU (oracle.scan_oracle.proj_params_ref, models/kernels/wavefront_cuda.py:63-95)
+and torch.autograd through it, which is how the reference itself differentiates the projections
+(wavefront_cuda.py:262-296).  Tolerances: fp32 1e-4, bf16 tensors 2e-2 (max error over max value).
+"""
+import math
+
+import pytest
+import torch
+
+from oracle import scan_oracle as so
+
+pytestmark = pytest.mark.gpu
+
+N = 16
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+@pytest.fixture(scope="module")
+def cabi():
+    from mamba2d_amd import cabi
+    return cabi
+
+
+def make_case(B, H, W, E, seed, dtype):
+    """x and weights with the magnitudes of an M2D block (models/mamba2d.py:57-111); the weights are
+    rounded to `dtype` as the reference's entry point does (wavefront_cuda.py:327-332)."""
+    R = math.ceil(E / 16)
+    g = torch.Generator().manual_seed(seed)
+    dt = torch.exp(torch.rand(E, generator=g) * (math.log(0.1) - math.log(0.001)) + math.log(0.001)).clamp(min=1e-4)
+    w = dict(
+        x_proj_w=(torch.rand(2 * R + 3 * N, E, generator=g) * 2 - 1) / math.sqrt(E),
+        dt_projT_w=(torch.rand(E, R, generator=g) * 2 - 1) * R ** -0.5,
+        dt_projT_b=dt + torch.log(-torch.expm1(-dt)),
+        dt_projL_w=(torch.rand(E, R, generator=g) * 2 - 1) * R ** -0.5,
+        dt_projL_b=(dt + torch.log(-torch.expm1(-dt))).flip(0).contiguous())
+    w = {k: v.to(dtype).float() for k, v in w.items()}
+    x = torch.randn(B, H, W, E, generator=g).to(dtype)
+    up = {k: torch.randn(B, H, W, n, generator=g).to(dtype)
+          for k, n in (("d_deltaT", E), ("d_deltaL", E), ("d_BT", N), ("d_BL", N), ("d_C", N), ("dx", E))}
+    return R, x, w, up
+
+
+WNAMES = ("x_proj_w", "dt_projT_w", "dt_projT_b", "dt_projL_w", "dt_projL_b")
+
+# (B, H, W, E): tiles that end inside the batch, channel counts that are no multiple of the
+# 64-channel chunk, one to seven 16-wide chunks of outputs, the largest rank
+SHAPES = [(2, 9, 12, 32), (1, 5, 7, 3), (2, 14, 14, 64), (1, 8, 8, 128), (1, 40, 4, 100), (1, 7, 9, 320),
+          (3, 7, 7, 512), (5, 31, 30, 64)]
+
+
+def reference(x, w, up, R):
+    """fp64 outputs and gradients of the projections for the upstream gradients `up`."""
+    x64 = x.double().requires_grad_(True)
+    w64 = {k: v.double().requires_grad_(True) for k, v in w.items()}
+    z = torch.nn.functional.linear(x64, w64["x_proj_w"])
+    low = z[..., :2 * R]
+    A = torch.zeros(x.shape[-1], N, dtype=torch.float64)
+    dT, dL, _, _, BT, BL, C = so.proj_params_ref(x64, A, A, *[w64[k] for k in WNAMES])
+    outs = dict(lowrank=low, deltaT=dT, deltaL=dL, BT=BT, BL=BL, C=C)
+    loss = sum((outs[k] * up["d_" + k].double()).sum() for k in ("deltaT", "deltaL", "BT", "BL", "C"))
+    grads = torch.autograd.grad(loss, [x64] + [w64[k] for k in WNAMES])
+    g = dict(zip(("x",) + WNAMES, grads))
+    g["x"] = g["x"] + up["dx"].double()
+    return {k: v.detach() for k, v in outs.items()}, g
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 2e-2)], ids=["f32", "bf16"])
+@pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_projections_match_reference(cabi, shape, dtype, tol):
+    say(f"\ncase proj {shape} {dtype}")
+    B, H, W, E = shape
+    R, x, w, up = make_case(B, H, W, E, seed=sum(shape), dtype=dtype)
+    ref_out, ref_g = reference(x, w, up, R)
+    xd = x.cuda()
+    wd = {k: v.cuda() for k, v in w.items()}
+    low, dT, dL, BT, BL, C = cabi.proj_fwd(xd, *[wd[k] for k in WNAMES], N)
+    got = dict(lowrank=low, deltaT=dT, deltaL=dL, BT=BT, BL=BL, C=C)
+    for k, v in got.items():
+        assert v.dtype == dtype and v.shape == ref_out[k].shape
+        assert so.rel_err(v.float().cpu(), ref_out[k]) < tol, k
+    # the step sizes span two decades: also hold every element to the tolerance
+    assert so.elem_rel_err(dT.float().cpu(), ref_out["deltaT"]) < 2 * tol
+
+    upd = {k: v.cuda() for k, v in up.items()}
+    dx = upd["dx"].clone()
+    gw = cabi.proj_bwd(xd, low, dT, dL, wd["x_proj_w"], wd["dt_projT_w"], wd["dt_projL_w"],
+                       upd["d_deltaT"], upd["d_deltaL"], upd["d_BT"], upd["d_BL"], upd["d_C"], dx)
+    torch.cuda.synchronize()
+    assert dx.dtype == dtype and so.rel_err(dx.float().cpu(), ref_g["x"]) < tol, "dx"
+    for k, g in zip(WNAMES, gw):
+        assert g.dtype == torch.float32 and g.shape == ref_g[k].shape
+        assert so.rel_err(g.cpu(), ref_g[k]) < tol, k
+
+
+def test_projection_limits_are_reported(cabi):
+    import ctypes
+    d = cabi.Desc(1, 4, 4, 64, 16, cabi.M2D_F32, 0, 0)
+    assert cabi.lib.m2d_proj_workspace_bytes(ctypes.byref(d), 4, cabi.M2D_PASS_FWD) > 0
+    assert cabi.lib.m2d_proj_workspace_bytes(ctypes.byref(d), 33, cabi.M2D_PASS_FWD) == 0     # dt_rank > 32
+    d8 = cabi.Desc(1, 4, 4, 64, 8, cabi.M2D_F32, 0, 0)
+    assert cabi.lib.m2d_proj_workspace_bytes(ctypes.byref(d8), 4, cabi.M2D_PASS_BWD) == 0    # d_state != 16

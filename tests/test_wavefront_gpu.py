@@ -62,9 +62,18 @@ def make_block_params(E, N, R, seed, device):
 ORDER = ("AT_log", "AL_log", "x_proj_w", "dt_projT_w", "dt_projT_b", "dt_projL_w", "dt_projL_b", "D")
 
 
+@pytest.fixture(params=[True, False], ids=["own_projections", "torch_projections"])
+def projections(wf, request):
+    """The entry point with the library's projection kernels and with stock torch operators."""
+    old = wf.FUSED_PROJECTIONS
+    wf.FUSED_PROJECTIONS = request.param
+    yield request.param
+    wf.FUSED_PROJECTIONS = old
+
+
 @pytest.mark.parametrize("recomp", ["partial", "full"])
-def test_entry_point_matches_oracle_fp32(wf, recomp):
-    say(f"\ncase entry_point {recomp}")
+def test_entry_point_matches_oracle_fp32(wf, recomp, projections):
+    say(f"\ncase entry_point {recomp} own_projections={projections}")
     B, H, W, E, N = 2, 9, 12, 32, 16
     R = math.ceil(E / 16)
     p = make_block_params(E, N, R, 0, "cuda")
@@ -82,9 +91,9 @@ def test_entry_point_matches_oracle_fp32(wf, recomp):
         assert so.rel_err(g.cpu(), gr) < 2e-4, name
 
 
-def test_partial_and_full_agree_bf16(wf):
+def test_partial_and_full_agree_bf16(wf, projections):
     """The two recompute modes are the same function of the nine raw inputs."""
-    say("\ncase partial_vs_full bf16")
+    say(f"\ncase partial_vs_full bf16 own_projections={projections}")
     B, H, W, E, N = 3, 14, 14, 64, 16
     R = math.ceil(E / 16)
     p = make_block_params(E, N, R, 3, "cuda")
