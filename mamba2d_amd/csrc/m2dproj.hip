@@ -49,27 +49,43 @@ __device__ __forceinline__ void st(bf16_t* p, float v) { p->v = f32_to_bf16_bits
 __device__ __forceinline__ float as_stored(float v, const float*) { return v; }
 __device__ __forceinline__ float as_stored(float v, const bf16_t*) { return __uint_as_float((uint32_t)f32_to_bf16_bits(v) << 16); }
 
-// softplus with torch's defaults (beta 1, threshold 20)
-__device__ __forceinline__ float softplus(float v) { return v > 20.f ? v : log1pf(expf(v)); }
-// d softplus / d pre, from the softplus value: sigmoid(pre) = 1 - exp(-softplus(pre))
-__device__ __forceinline__ float softplus_slope(float delta) { return -expm1f(-delta); }
+// exp, log and 1/x as the bare hardware instructions: the arguments below stay in ranges that
+// need none of the library's scaling (results that underflow may flush to zero).
+__device__ __forceinline__ float exp_neg(float v) { return __builtin_amdgcn_exp2f(v * 1.44269504088896341f); }   // v <= 0
+__device__ __forceinline__ float log_1to2(float u) { return __builtin_amdgcn_logf(u) * 0.693147180559945309f; }  // 1 <= u <= 2
+__device__ __forceinline__ float rcp_1to2(float u) { return __builtin_amdgcn_rcpf(u); }
+
+// softplus with torch's defaults (beta 1; above the threshold of 20 the two agree in fp32):
+// max(v,0) + log1p(t), t = exp(-|v|), with log1p(t) = log(u) + (t - (u-1))/u for u = fl(1+t),
+// which makes up for the rounding of 1+t when t is small.
+__device__ __forceinline__ float softplus(float v) {
+  const float t = exp_neg(-fabsf(v));
+  const float u = 1.f + t;
+  return fmaxf(v, 0.f) + __builtin_fmaf(t - (u - 1.f), rcp_1to2(u), log_1to2(u));
+}
+// d softplus / d pre, from the softplus value: sigmoid(pre) = 1 - exp(-softplus(pre)).  Small
+// arguments take the series, where 1 - exp(-d) would cancel.
+__device__ __forceinline__ float softplus_slope(float d) {
+  const float series = d * __builtin_fmaf(d, __builtin_fmaf(d, __builtin_fmaf(d, -1.f / 24.f, 1.f / 6.f), -0.5f), 1.f);
+  return d < 0.0625f ? series : 1.f - exp_neg(-d);
+}
 
 struct ProjArgs {
   // activations, (P, .) row-major, element type T
   const void *x, *r, *dT, *dL;           // x (P,E); r (P,2R) = low-rank inputs of the two dt projections; delta (P,E)
   const void *ddT, *ddL, *dBT, *dBL, *dC;
   void *r_out, *dT_out, *dL_out, *BT_out, *BL_out, *C_out, *dx;
-  // weights, fp32
-  const float *bT, *bL;                  // (E)
-  const float *wT, *wL;                  // (E,R) as given
-  const float *Wt;                       // [Epad][Opad]   Wx transposed, zero padded
-  const float *Wp;                       // [O][Epad]      Wx, rows padded
-  const float *wTp, *wLp;                // [Epad][Rpad]   dt weights, rows padded
-  float* dz;                             // (P,O) fp32
+  // packed weights, fp32, zero where padded
+  const float *Wt;                       // [Epad][Opad]   Wx transposed
+  const float *wTt, *wLt;                // [R][Epad]      dt weights transposed
+  const float *bTp, *bLp;                // [Epad]
+  const float *Wp;                       // [O][Epad]      Wx
+  const float *wTp, *wLp;                // [Epad][Rpad]   dt weights
+  float* dz;                             // (P,O4) fp32, rows padded to a multiple of 4
   float* part;                           // per-workgroup sums of the weight gradients
   float *dWx, *dwT, *dbT, *dwL, *dbL;    // outputs of the reduction
   int64_t P;
-  int E, R, O, Epad, Opad, Rpad;
+  int E, R, O, O4, Epad, Opad, Rpad;
   int ntiles, G, ne;
 };
 
@@ -81,26 +97,119 @@ __device__ __forceinline__ const_floats as_const(const float* p) { return (const
 __device__ __forceinline__ int wave_id() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
 
 // ------------------------------------------------------------------------------- weights
-// Padded copies of the weights (zero where padded).  One thread per element of the largest copy.
-__global__ void m2d_proj_pack_kernel(const float* __restrict__ Wx, const float* __restrict__ wT, const float* __restrict__ wL,
-                                     float* __restrict__ Wt, float* __restrict__ Wp, float* __restrict__ wTp, float* __restrict__ wLp,
-                                     int E, int R, int O, int Epad, int Opad, int Rpad) {
+struct PackArgs {
+  const float *Wx, *wT, *bT, *wL, *bL;
+  float *Wt, *wTt, *wLt, *bTp, *bLp;     // forward set (or null)
+  float *Wp, *wTp, *wLp;                 // backward set (or null)
+  int E, R, O, Epad, Opad, Rpad;
+};
+
+// Padded copies of the weights.  One thread per element of the largest copy.
+__global__ void m2d_proj_pack_kernel(const PackArgs k) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (Wt && i < Epad * Opad) {
-    const int e = i / Opad, o = i - e * Opad;
-    Wt[i] = (e < E && o < O) ? Wx[o * E + e] : 0.f;
+  if (k.Wt) {
+    if (i < k.Epad * k.Opad) {
+      const int e = i / k.Opad, o = i - e * k.Opad;
+      k.Wt[i] = (e < k.E && o < k.O) ? k.Wx[o * k.E + e] : 0.f;
+    }
+    if (i < k.R * k.Epad) {
+      const int q = i / k.Epad, e = i - q * k.Epad;
+      k.wTt[i] = e < k.E ? k.wT[e * k.R + q] : 0.f;
+      k.wLt[i] = e < k.E ? k.wL[e * k.R + q] : 0.f;
+    }
+    if (i < k.Epad) {
+      k.bTp[i] = i < k.E ? k.bT[i] : 0.f;
+      k.bLp[i] = i < k.E ? k.bL[i] : 0.f;
+    }
   }
-  if (Wp && i < O * Epad) {
-    const int o = i / Epad, e = i - o * Epad;
-    Wp[i] = e < E ? Wx[o * E + e] : 0.f;
-  }
-  if (wTp && i < Epad * Rpad) {
-    const int e = i / Rpad, q = i - e * Rpad;
-    const bool ok = e < E && q < R;
-    wTp[i] = ok ? wT[e * R + q] : 0.f;
-    wLp[i] = ok ? wL[e * R + q] : 0.f;
+  if (k.Wp) {
+    if (i < k.O * k.Epad) {
+      const int o = i / k.Epad, e = i - o * k.Epad;
+      k.Wp[i] = e < k.E ? k.Wx[o * k.E + e] : 0.f;
+    }
+    if (i < k.Epad * k.Rpad) {
+      const int e = i / k.Rpad, q = i - e * k.Rpad;
+      const bool ok = e < k.E && q < k.R;
+      k.wTp[i] = ok ? k.wT[e * k.R + q] : 0.f;
+      k.wLp[i] = ok ? k.wL[e * k.R + q] : 0.f;
+    }
   }
 }
+
+// ------------------------------------------------------------------------------- tiles
+// A tile is 64 positions x 64 channels of a (P,E) array, 16 elements per thread.  The loads of a
+// tile are issued back to back into registers and converted when they are consumed, so that a
+// thread waits for memory once per tile and not once per row.
+// VEC (E a multiple of the 16-byte vector): thread t holds, for l < NL, the EPL elements from
+//   column (ci % CPR) * EPL of row ci / CPR, ci = l * 256 + t.  Otherwise element i = l * 256 + t,
+//   row i / 64, column i % 64.
+template <typename T, bool VEC>
+struct Tile {
+  static constexpr int EPL = VEC ? 16 / (int)sizeof(T) : 1;
+  static constexpr int NL = 16 / EPL;
+  static constexpr int CPR = kKC / EPL;
+  struct Regs { uint4 q[VEC ? NL : 1]; float v[VEC ? 1 : 16]; };
+
+  static __device__ __forceinline__ void pos(int t, int l, int& row, int& col) {
+    const int ci = l * kThreads + t;
+    row = ci / CPR;
+    col = (ci % CPR) * EPL;
+  }
+  static __device__ __forceinline__ void load(Regs& r, const T* base, int64_t p0, int64_t P, int E, int e0, int t) {
+#pragma unroll
+    for (int l = 0; l < NL; ++l) {
+      int row, col;
+      pos(t, l, row, col);
+      const int64_t p = p0 + row;
+      const bool ok = p < P && e0 + col < E;
+      if constexpr (VEC) r.q[l] = ok ? *reinterpret_cast<const uint4*>(base + p * E + e0 + col) : make_uint4(0, 0, 0, 0);
+      else r.v[l] = ok ? ld(base + p * E + e0 + col) : 0.f;
+    }
+  }
+  // element j < EPL of load l
+  static __device__ __forceinline__ float get(const Regs& r, int l, int j) {
+    if constexpr (!VEC) return r.v[l];
+    else {
+      const uint32_t w[4] = {r.q[l].x, r.q[l].y, r.q[l].z, r.q[l].w};
+      if constexpr (sizeof(T) == 4) return __uint_as_float(w[j]);
+      else return __uint_as_float((j & 1) ? (w[j >> 1] & 0xffff0000u) : (w[j >> 1] << 16));
+    }
+  }
+  // v(l, j) for every element -> tile[row * stride + col]
+  template <typename F>
+  static __device__ __forceinline__ void to_lds(float* tile, int stride, int t, F value) {
+#pragma unroll
+    for (int l = 0; l < NL; ++l) {
+      int row, col;
+      pos(t, l, row, col);
+#pragma unroll
+      for (int j = 0; j < EPL; ++j) tile[row * stride + col + j] = value(l, j);
+    }
+  }
+  // tile[row * stride + col] (+ what `plus` holds) -> global, rows and channels inside the array only
+  static __device__ __forceinline__ void store(const float* tile, int stride, T* base, int64_t p0, int64_t P, int E, int e0,
+                                               int t, const Regs* plus) {
+#pragma unroll
+    for (int l = 0; l < NL; ++l) {
+      int row, col;
+      pos(t, l, row, col);
+      const int64_t p = p0 + row;
+      if (!(p < P && e0 + col < E)) continue;
+      float v[EPL];
+#pragma unroll
+      for (int j = 0; j < EPL; ++j) v[j] = tile[row * stride + col + j] + (plus ? get(*plus, l, j) : 0.f);
+      T* dst = base + p * E + e0 + col;
+      if constexpr (!VEC) st(dst, v[0]);
+      else if constexpr (sizeof(T) == 4) *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+      else {
+        uint32_t w[4];
+#pragma unroll
+        for (int h = 0; h < 4; ++h) w[h] = (uint32_t)f32_to_bf16_bits(v[2 * h]) | ((uint32_t)f32_to_bf16_bits(v[2 * h + 1]) << 16);
+        *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
+      }
+    }
+  }
+};
 
 // acc[j] += sum_e tile[lane][e] * w[e * stride + j], e < 64, j < 16; w is uniform over the wave
 __device__ __forceinline__ void row_times_weights(const float* tile_row, const_floats w, int stride, float (&acc)[16]) {
@@ -114,17 +223,21 @@ __device__ __forceinline__ void row_times_weights(const float* tile_row, const_f
 }
 
 // ------------------------------------------------------------------------------- forward
-// One workgroup per tile of 64 positions.  LDS: xs[64][65] (a chunk of x), zs[64][O+1] (z).
-template <typename T>
+// One workgroup per tile of 64 positions.  LDS: xs[64][65] (a chunk of x, later the deltaT tile),
+// zs[64][O+1] (z), outL[64][65] (the deltaL tile).
+template <typename T, bool VEC>
 __global__ __launch_bounds__(kThreads) void m2d_proj_fwd_kernel(const ProjArgs a) {
+  using TL = Tile<T, VEC>;
   extern __shared__ float smem[];
   float* xs = smem;
   float* zs = smem + kTP * kXS;
+  float* outL = zs + kTP * (a.O + 1);
+  float* outT = xs;
   const int zst = a.O + 1;
-  const int wave = wave_id(), lane = threadIdx.x & 63;
+  const int wave = wave_id(), lane = threadIdx.x & 63, tid = threadIdx.x;
   const int64_t p0 = (int64_t)blockIdx.x * kTP;
   const T* x = static_cast<const T*>(a.x);
-  const int nOC = a.Opad / 16;
+  const int nOC = a.Opad / 16, nkc = a.Epad / kKC;
 
   float acc[kMaxRounds][16];
 #pragma unroll
@@ -132,13 +245,12 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_fwd_kernel(const ProjArgs a
 #pragma unroll
     for (int j = 0; j < 16; ++j) acc[rd][j] = 0.f;
 
-  for (int kc = 0; kc < a.Epad / kKC; ++kc) {
-    const int e = kc * kKC + lane;
-    for (int c = wave; c < kTP; c += kWaves) {
-      const int64_t p = p0 + c;
-      xs[c * kXS + lane] = (p < a.P && e < a.E) ? ld(x + p * a.E + e) : 0.f;
-    }
+  typename TL::Regs xr;
+  TL::load(xr, x, p0, a.P, a.E, 0, tid);
+  for (int kc = 0; kc < nkc; ++kc) {
+    TL::to_lds(xs, kXS, tid, [&](int l, int j) { return TL::get(xr, l, j); });
     __syncthreads();
+    if (kc + 1 < nkc) TL::load(xr, x, p0, a.P, a.E, (kc + 1) * kKC, tid);   // under way during the products
 #pragma unroll
     for (int rd = 0; rd < kMaxRounds; ++rd) {
       const int oc = wave + kWaves * rd;
@@ -157,11 +269,9 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_fwd_kernel(const ProjArgs a
   }
   __syncthreads();
 
-  // ---- outputs, a row of the tile per wave at a time (rows are contiguous in memory)
+  // ---- low-rank inputs and B_T, B_L, C: a row of the tile per wave at a time
   const int R = a.R, R2 = 2 * a.R;
   T* r_out = static_cast<T*>(a.r_out);
-  T* dT_out = static_cast<T*>(a.dT_out);
-  T* dL_out = static_cast<T*>(a.dL_out);
   for (int c = wave; c < kTP; c += kWaves) {
     const int64_t p = p0 + c;
     if (p >= a.P) break;   // uniform
@@ -171,38 +281,72 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_fwd_kernel(const ProjArgs a
       T* out = static_cast<T*>(lane < kN ? a.BT_out : (lane < 2 * kN ? a.BL_out : a.C_out));
       st(out + p * kN + (lane & (kN - 1)), z[R2 + lane]);
     }
-    for (int e = lane; e < a.E; e += 64) {
-      float preT = a.bT[e], preL = a.bL[e];
-      const float* wt = a.wT + e * R;
-      const float* wl = a.wL + e * R;
-      for (int q = 0; q < R; ++q) {
-        // the dt projections see the low-rank inputs as the tensor holds them
-        preT = __builtin_fmaf(as_stored(z[q], r_out), wt[q], preT);
-        preL = __builtin_fmaf(as_stored(z[R + q], r_out), wl[q], preL);
+  }
+
+  // ---- delta = softplus(r w^T + b), 64 channels at a time: a thread works out 16 channels of
+  // its position with wave-uniform weights, the tile goes out row-wise through LDS
+  const float* zrow = zs + lane * zst;
+  for (int eg = 0; eg < nkc; ++eg) {
+    const int e0 = eg * kKC + wave * 16;
+    float sT[16], sL[16];
+    const_floats bt = as_const(a.bTp) + e0;
+    const_floats bl = as_const(a.bLp) + e0;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) { sT[j] = bt[j]; sL[j] = bl[j]; }
+    for (int q = 0; q < R; ++q) {
+      // the dt projections see the low-rank inputs as the tensor holds them
+      const float zT = as_stored(zrow[q], r_out), zL = as_stored(zrow[R + q], r_out);
+      const_floats wt = as_const(a.wTt) + q * a.Epad + e0;
+      const_floats wl = as_const(a.wLt) + q * a.Epad + e0;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        sT[j] = __builtin_fmaf(zT, wt[j], sT[j]);
+        sL[j] = __builtin_fmaf(zL, wl[j], sL[j]);
       }
-      st(dT_out + p * a.E + e, softplus(preT));
-      st(dL_out + p * a.E + e, softplus(preL));
     }
+    if (eg > 0) __syncthreads();   // the tiles of the previous group have gone out
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      outT[lane * kXS + wave * 16 + j] = softplus(sT[j]);
+      outL[lane * kXS + wave * 16 + j] = softplus(sL[j]);
+    }
+    __syncthreads();
+    TL::store(outT, kXS, static_cast<T*>(a.dT_out), p0, a.P, a.E, eg * kKC, tid, nullptr);
+    TL::store(outL, kXS, static_cast<T*>(a.dL_out), p0, a.P, a.E, eg * kKC, tid, nullptr);
   }
 }
 
 // ------------------------------------------------------------------------------- backward, data
 // One workgroup per tile.  LDS: dps[2][64][65] (chunks of dpreT, dpreL; reused for the dx tile),
-// dzs[64][O+1].  Writes dz (P,O) for the weight-gradient kernel and adds dz Wx to dx.
-template <typename T>
+// dzs[64][O+1].  Writes dz for the weight-gradient kernel and adds dz Wx to dx.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_data_kernel(const ProjArgs a) {
+  using TL = Tile<T, VEC>;
   extern __shared__ float smem[];
   float* dps = smem;
   float* dzs = smem + 2 * kTP * kXS;
   const int zst = a.O + 1;
-  const int wave = wave_id(), lane = threadIdx.x & 63;
+  const int wave = wave_id(), lane = threadIdx.x & 63, tid = threadIdx.x;
   const int64_t p0 = (int64_t)blockIdx.x * kTP;
   const int R = a.R, R2 = 2 * a.R;
   const int nRC = a.Rpad / 16;   // 16-wide chunks of one dt weight; 2*nRC chunks in all (T then L)
+  const int nkc = a.Epad / kKC;
   const T* dT = static_cast<const T*>(a.dT);
   const T* dL = static_cast<const T*>(a.dL);
   const T* ddT = static_cast<const T*>(a.ddT);
   const T* ddL = static_cast<const T*>(a.ddL);
+
+  // dB_T, dB_L, dC of the tile: 64 x 16 contiguous elements each, 4 per thread
+  float bc[3][4];
+#pragma unroll
+  for (int w = 0; w < 3; ++w) {
+    const T* src = static_cast<const T*>(w == 0 ? a.dBT : (w == 1 ? a.dBL : a.dC));
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int i = k * kThreads + tid;
+      bc[w][k] = p0 + (i >> 4) < a.P ? ld(src + p0 * kN + i) : 0.f;
+    }
+  }
 
   float acc[kMaxRounds][16];
 #pragma unroll
@@ -210,19 +354,14 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_data_kernel(const ProjA
 #pragma unroll
     for (int j = 0; j < 16; ++j) acc[rd][j] = 0.f;
 
-  for (int kc = 0; kc < a.Epad / kKC; ++kc) {
-    const int e = kc * kKC + lane;
-    for (int c = wave; c < kTP; c += kWaves) {
-      const int64_t p = p0 + c;
-      float vT = 0.f, vL = 0.f;
-      if (p < a.P && e < a.E) {
-        const int64_t i = p * a.E + e;
-        vT = ld(ddT + i) * softplus_slope(ld(dT + i));
-        vL = ld(ddL + i) * softplus_slope(ld(dL + i));
-      }
-      dps[c * kXS + lane] = vT;
-      dps[kTP * kXS + c * kXS + lane] = vL;
-    }
+  for (int kc = 0; kc < nkc; ++kc) {
+    typename TL::Regs gT, vT, gL, vL;
+    TL::load(gT, ddT, p0, a.P, a.E, kc * kKC, tid);
+    TL::load(vT, dT, p0, a.P, a.E, kc * kKC, tid);
+    TL::load(gL, ddL, p0, a.P, a.E, kc * kKC, tid);
+    TL::load(vL, dL, p0, a.P, a.E, kc * kKC, tid);
+    TL::to_lds(dps, kXS, tid, [&](int l, int j) { return TL::get(gT, l, j) * softplus_slope(TL::get(vT, l, j)); });
+    TL::to_lds(dps + kTP * kXS, kXS, tid, [&](int l, int j) { return TL::get(gL, l, j) * softplus_slope(TL::get(vL, l, j)); });
     __syncthreads();
 #pragma unroll
     for (int rd = 0; rd < kMaxRounds; ++rd) {
@@ -247,25 +386,27 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_data_kernel(const ProjA
         if (qc * 16 + j < R) dzs[lane * zst + (isL ? R : 0) + qc * 16 + j] = acc[rd][j];
     }
   }
-  for (int c = wave; c < kTP; c += kWaves) {
-    const int64_t p = p0 + c;
-    if (lane < 3 * kN) {
-      const T* src = static_cast<const T*>(lane < kN ? a.dBT : (lane < 2 * kN ? a.dBL : a.dC));
-      dzs[c * zst + R2 + lane] = p < a.P ? ld(src + p * kN + (lane & (kN - 1))) : 0.f;
+#pragma unroll
+  for (int w = 0; w < 3; ++w)
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+      const int i = k * kThreads + tid;
+      dzs[(i >> 4) * zst + R2 + w * kN + (i & 15)] = bc[w][k];
     }
-  }
   __syncthreads();
 
   for (int c = wave; c < kTP; c += kWaves) {
     const int64_t p = p0 + c;
     if (p >= a.P) break;   // uniform
-    for (int o = lane; o < a.O; o += 64) a.dz[p * a.O + o] = dzs[c * zst + o];
+    for (int o = lane; o < a.O4; o += 64) a.dz[p * a.O4 + o] = o < a.O ? dzs[c * zst + o] : 0.f;
   }
 
   // ---- dx += dz Wx, 64 channels at a time (16 per wave), through LDS for row-wise stores
   T* dx = static_cast<T*>(a.dx);
   float* outs = dps;
-  for (int eg = 0; eg < a.Epad / kKC; ++eg) {
+  for (int eg = 0; eg < nkc; ++eg) {
+    typename TL::Regs old;
+    TL::load(old, dx, p0, a.P, a.E, eg * kKC, tid);
     float s[16];
 #pragma unroll
     for (int j = 0; j < 16; ++j) s[j] = 0.f;
@@ -278,15 +419,11 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_data_kernel(const ProjA
 #pragma unroll
       for (int j = 0; j < 16; ++j) s[j] = __builtin_fmaf(v, wo[j], s[j]);
     }
+    if (eg > 0) __syncthreads();   // the previous tile has gone out
 #pragma unroll
     for (int j = 0; j < 16; ++j) outs[lane * kXS + wave * 16 + j] = s[j];
     __syncthreads();
-    const int e = eg * kKC + lane;
-    for (int c = wave; c < kTP; c += kWaves) {
-      const int64_t p = p0 + c;
-      if (p < a.P && e < a.E) st(dx + p * a.E + e, ld(dx + p * a.E + e) + outs[c * kXS + lane]);
-    }
-    __syncthreads();
+    TL::store(outs, kXS, dx, p0, a.P, a.E, eg * kKC, tid, &old);
   }
 }
 
@@ -296,12 +433,14 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_data_kernel(const ProjA
 //   rows 0..O-1      dWx[o][.]      = sum_p dz[p][o] x[p][.]
 //   rows O..O+R-1    dwT[.][q]      = sum_p dpreT[p][.] rT[p][q]      rows O+R..O+2R-1 the same for L
 //   rows O+2R, +1    dbT[.], dbL[.] = sum_p dpre[p][.]
-// LDS: xs[64][68], dpT[64][65], dpL[64][65], dzs[64][O4], rs[64][2R+1].
-template <typename T>
+// LDS: xs[64][68], dpT[64][65], dpL[64][65], dzs[64][O4], rs[64][2R].  The loads of the next tile
+// are under way while the sums of the current one are formed.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_weights_kernel(const ProjArgs a) {
+  using TL = Tile<T, VEC>;
   extern __shared__ float smem[];
-  const int O4 = (a.O + 3) & ~3;
-  const int R = a.R, R2 = 2 * a.R, rst = R2 + 1;
+  const int O4 = a.O4;
+  const int R = a.R, R2 = 2 * a.R;
   float* xs = smem;
   float* dpT = xs + kTP * kXS4;
   float* dpL = dpT + kTP * kXS;
@@ -316,6 +455,9 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_weights_kernel(const Pr
   const T* ddT = static_cast<const T*>(a.ddT);
   const T* ddL = static_cast<const T*>(a.ddL);
   const int nmt = (O4 / 4) * 16;   // 4 x 4 blocks of dWx: (o4, e4), e4 fastest
+  constexpr int kZQ = (kTP * ((2 * kMaxR + 3 * kN + 3) / 4) + kThreads - 1) / kThreads;   // float4 of dz per thread, at most
+  constexpr int kRQ = (kTP * 2 * kMaxR + kThreads - 1) / kThreads;                        // elements of r per thread, at most
+  const int nzq = kTP * O4 / 4, nrq = kTP * R2;
 
   float aw[2][16], ar[2][kMaxR / kWaves], ab[2] = {0.f, 0.f};
 #pragma unroll
@@ -326,35 +468,56 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_weights_kernel(const Pr
     for (int i = 0; i < kMaxR / kWaves; ++i) ar[h][i] = 0.f;
   }
 
-  for (int tile = blockIdx.x; tile < a.ntiles; tile += a.G) {
+  typename TL::Regs xr, gT, vT, gL, vL;
+  float4 zq[kZQ];
+  float rq[kRQ];
+  auto fetch = [&](int tile) {
     const int64_t p0 = (int64_t)tile * kTP;
-    const int e = ey * kKC + lane;
-    for (int c = wave; c < kTP; c += kWaves) {
-      const int64_t p = p0 + c;
-      const bool row = p < a.P;
-      float xv = 0.f, vT = 0.f, vL = 0.f;
-      if (row && e < a.E) {
-        const int64_t i = p * a.E + e;
-        xv = ld(x + i);
-        vT = ld(ddT + i) * softplus_slope(ld(dT + i));
-        vL = ld(ddL + i) * softplus_slope(ld(dL + i));
-      }
-      xs[c * kXS4 + lane] = xv;
-      dpT[c * kXS + lane] = vT;
-      dpL[c * kXS + lane] = vL;
-      for (int o = lane; o < O4; o += 64) dzs[c * O4 + o] = (row && o < a.O) ? a.dz[p * a.O + o] : 0.f;
-      for (int q = lane; q < R2; q += 64) rs[c * rst + q] = row ? ld(rr + p * R2 + q) : 0.f;
+    TL::load(xr, x, p0, a.P, a.E, ey * kKC, tid);
+    TL::load(gT, ddT, p0, a.P, a.E, ey * kKC, tid);
+    TL::load(vT, dT, p0, a.P, a.E, ey * kKC, tid);
+    TL::load(gL, ddL, p0, a.P, a.E, ey * kKC, tid);
+    TL::load(vL, dL, p0, a.P, a.E, ey * kKC, tid);
+    const int64_t left = a.P - p0;   // rows of the tile inside the array, if fewer than 64
+    const float4* zsrc = reinterpret_cast<const float4*>(a.dz + p0 * O4);
+#pragma unroll
+    for (int k = 0; k < kZQ; ++k) {
+      const int i = k * kThreads + tid;
+      zq[k] = (i < nzq && (int64_t)(4 * i) < left * O4) ? zsrc[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+#pragma unroll
+    for (int k = 0; k < kRQ; ++k) {
+      const int i = k * kThreads + tid;
+      rq[k] = (i < nrq && (int64_t)i < left * R2) ? ld(rr + p0 * R2 + i) : 0.f;
+    }
+  };
+
+  if ((int)blockIdx.x < a.ntiles) fetch(blockIdx.x);
+  for (int tile = blockIdx.x; tile < a.ntiles; tile += a.G) {
+    TL::to_lds(xs, kXS4, tid, [&](int l, int j) { return TL::get(xr, l, j); });
+    TL::to_lds(dpT, kXS, tid, [&](int l, int j) { return TL::get(gT, l, j) * softplus_slope(TL::get(vT, l, j)); });
+    TL::to_lds(dpL, kXS, tid, [&](int l, int j) { return TL::get(gL, l, j) * softplus_slope(TL::get(vL, l, j)); });
+#pragma unroll
+    for (int k = 0; k < kZQ; ++k) {
+      const int i = k * kThreads + tid;
+      if (i < nzq) reinterpret_cast<float4*>(dzs)[i] = zq[k];
+    }
+#pragma unroll
+    for (int k = 0; k < kRQ; ++k) {
+      const int i = k * kThreads + tid;
+      if (i < nrq) rs[i] = rq[k];
     }
     __syncthreads();
+    if (tile + a.G < a.ntiles) fetch(tile + a.G);
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int mt = tid + kThreads * h;
       if (mt < nmt) {
-        const float4* zq = reinterpret_cast<const float4*>(dzs + 4 * (mt >> 4));
-        const float4* xq = reinterpret_cast<const float4*>(xs + 4 * (mt & 15));
+        const float4* zp = reinterpret_cast<const float4*>(dzs + 4 * (mt >> 4));
+        const float4* xp = reinterpret_cast<const float4*>(xs + 4 * (mt & 15));
 #pragma unroll 4
         for (int c = 0; c < kTP; ++c) {
-          const float4 z4 = zq[c * (O4 / 4)], x4 = xq[c * (kXS4 / 4)];
+          const float4 z4 = zp[c * (O4 / 4)], x4 = xp[c * (kXS4 / 4)];
           const float zz[4] = {z4.x, z4.y, z4.z, z4.w}, xx[4] = {x4.x, x4.y, x4.z, x4.w};
 #pragma unroll
           for (int i = 0; i < 4; ++i)
@@ -366,15 +529,15 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_weights_kernel(const Pr
     // dt weights: this thread's channel is `lane`, its ranks are wave, wave + 4, ...
 #pragma unroll 2
     for (int c = 0; c < kTP; ++c) {
-      const float vT = dpT[c * kXS + lane], vL = dpL[c * kXS + lane];
-      const float* rq = rs + c * rst;
-      if (wave == 0) { ab[0] += vT; ab[1] += vL; }
+      const float tT = dpT[c * kXS + lane], tL = dpL[c * kXS + lane];
+      const float* rc = rs + c * R2;
+      if (wave == 0) { ab[0] += tT; ab[1] += tL; }
 #pragma unroll
       for (int i = 0; i < kMaxR / kWaves; ++i) {
         const int q = wave + kWaves * i;
         if (q < R) {
-          ar[0][i] = __builtin_fmaf(vT, rq[q], ar[0][i]);
-          ar[1][i] = __builtin_fmaf(vL, rq[R + q], ar[1][i]);
+          ar[0][i] = __builtin_fmaf(tT, rc[q], ar[0][i]);
+          ar[1][i] = __builtin_fmaf(tL, rc[R + q], ar[1][i]);
         }
       }
     }
@@ -407,17 +570,26 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_weights_kernel(const Pr
   }
 }
 
-// Sums the per-workgroup parts in workgroup order and scatters them to the five weight gradients.
-__global__ void m2d_proj_reduce_kernel(const ProjArgs a) {
+// Sums the per-workgroup parts in a fixed order and scatters them to the five weight gradients.
+// Grid (rows, ne), 1024 threads: 64 channels x 16 slices of the workgroup index.
+constexpr int kRedSlices = 16;
+__global__ __launch_bounds__(64 * kRedSlices) void m2d_proj_reduce_kernel(const ProjArgs a) {
+  __shared__ float sums[kRedSlices][64];
   const int rows = a.O + 2 * a.R + 2;
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= rows * a.E) return;
-  const int row = i / a.E, e = i - row * a.E;
-  const int ey = e / kKC, el = e - ey * kKC;
+  const int row = blockIdx.x, ey = blockIdx.y;
+  const int el = threadIdx.x & 63, gs = threadIdx.x >> 6;
   const float* src = a.part + ((int64_t)ey * rows + row) * kKC + el;
   const int64_t gstride = (int64_t)a.ne * rows * kKC;
   float s = 0.f;
-  for (int g = 0; g < a.G; ++g) s += src[g * gstride];
+#pragma unroll 8
+  for (int g = gs; g < a.G; g += kRedSlices) s += src[g * gstride];
+  sums[gs][el] = s;
+  __syncthreads();
+  if (gs != 0) return;
+#pragma unroll
+  for (int k = 1; k < kRedSlices; ++k) s += sums[k][el];
+  const int e = ey * kKC + el;
+  if (e >= a.E) return;
   if (row < a.O) a.dWx[row * a.E + e] = s;
   else if (row < a.O + a.R) a.dwT[e * a.R + (row - a.O)] = s;
   else if (row < a.O + 2 * a.R) a.dwL[e * a.R + (row - a.O - a.R)] = s;
@@ -431,8 +603,12 @@ inline bool misaligned(const void* p, size_t a) { return (reinterpret_cast<uintp
 
 struct ProjGeometry {
   int64_t P;
-  int E, R, O, Epad, Opad, Rpad, ntiles, G, ne;
-  size_t off_Wt, off_Wp, off_wTp, off_wLp, off_dz, off_part, bytes_fwd, bytes_bwd;
+  int E, R, O, O4, Epad, Opad, Rpad, ntiles, G, ne;
+  bool vec;   // rows of the (P,E) arrays start on 16-byte boundaries
+  // forward workspace
+  size_t off_Wt, off_wTt, off_wLt, off_bTp, off_bLp, bytes_fwd;
+  // backward workspace
+  size_t off_Wp, off_wTp, off_wLp, off_dz, off_part, bytes_bwd;
 };
 
 int check_proj(const m2d_desc* d, int R) {
@@ -448,45 +624,71 @@ ProjGeometry proj_geometry(const m2d_desc* d, int R) {
   ProjGeometry g;
   g.P = (int64_t)d->B * d->H * d->W;
   g.E = d->E; g.R = R; g.O = 2 * R + 3 * kN;
+  g.O4 = (g.O + 3) & ~3;
   g.Epad = (g.E + kKC - 1) / kKC * kKC;
   g.Opad = (g.O + 15) / 16 * 16;
   g.Rpad = (R + 15) / 16 * 16;
   g.ntiles = (int)((g.P + kTP - 1) / kTP);
   g.ne = g.Epad / kKC;
+  g.vec = d->E % (d->dtype == M2D_F32 ? 4 : 8) == 0;
   const int want = 512 / g.ne > 0 ? 512 / g.ne : 1;   // about two workgroups per compute unit in all
   g.G = g.ntiles < want ? g.ntiles : want;
   size_t o = 0;
   g.off_Wt = o; o += align256((size_t)g.Epad * g.Opad * 4);
+  g.off_wTt = o; o += align256((size_t)R * g.Epad * 4);
+  g.off_wLt = o; o += align256((size_t)R * g.Epad * 4);
+  g.off_bTp = o; o += align256((size_t)g.Epad * 4);
+  g.off_bLp = o; o += align256((size_t)g.Epad * 4);
   g.bytes_fwd = o;
   o = 0;
   g.off_Wp = o; o += align256((size_t)g.O * g.Epad * 4);
   g.off_wTp = o; o += align256((size_t)g.Epad * g.Rpad * 4);
   g.off_wLp = o; o += align256((size_t)g.Epad * g.Rpad * 4);
-  g.off_dz = o; o += align256((size_t)g.P * g.O * 4);
+  g.off_dz = o; o += align256((size_t)g.P * g.O4 * 4);
   g.off_part = o; o += align256((size_t)g.G * g.ne * (g.O + 2 * R + 2) * kKC * 4);
   g.bytes_bwd = o;
   return g;
 }
 
 void fill(ProjArgs& a, const ProjGeometry& g) {
-  a.P = g.P; a.E = g.E; a.R = g.R; a.O = g.O; a.Epad = g.Epad; a.Opad = g.Opad; a.Rpad = g.Rpad;
+  a.P = g.P; a.E = g.E; a.R = g.R; a.O = g.O; a.O4 = g.O4; a.Epad = g.Epad; a.Opad = g.Opad; a.Rpad = g.Rpad;
   a.ntiles = g.ntiles; a.G = g.G; a.ne = g.ne;
 }
 
 inline bool launched() { return hipGetLastError() == hipSuccess; }
 
-constexpr int kMaxLdsWeights = (kTP * kXS4 + 2 * kTP * kXS + kTP * ((2 * kMaxR + 3 * kN + 3) & ~3) + kTP * (2 * kMaxR + 1)) * 4;
+constexpr int kMaxLdsWeights = (kTP * kXS4 + 2 * kTP * kXS + kTP * ((2 * kMaxR + 3 * kN + 3) & ~3) + kTP * 2 * kMaxR) * 4;
 
-template <typename T>
+template <typename T, bool VEC>
 bool allow_lds_weights() {
   static bool done = false;   // idempotent, the value never changes
   if (!done) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_proj_bwd_weights_kernel<T>),
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_proj_bwd_weights_kernel<T, VEC>),
                             hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsWeights) != hipSuccess)
       return false;
     done = true;
   }
   return true;
+}
+
+template <typename T, bool VEC>
+int run_proj_fwd(const ProjGeometry& g, const ProjArgs& a, hipStream_t st) {
+  const size_t lds = (size_t)(2 * kTP * kXS + kTP * (g.O + 1)) * 4;
+  hipLaunchKernelGGL((m2d_proj_fwd_kernel<T, VEC>), dim3(g.ntiles), dim3(kThreads), lds, st, a);
+  return launched() ? M2D_OK : M2D_ERR_HIP;
+}
+
+template <typename T, bool VEC>
+int run_proj_bwd(const ProjGeometry& g, const ProjArgs& a, hipStream_t st) {
+  const size_t lds_data = (size_t)(2 * kTP * kXS + kTP * (g.O + 1)) * 4;
+  hipLaunchKernelGGL((m2d_proj_bwd_data_kernel<T, VEC>), dim3(g.ntiles), dim3(kThreads), lds_data, st, a);
+  if (!launched()) return M2D_ERR_HIP;
+  const size_t lds_w = (size_t)(kTP * kXS4 + 2 * kTP * kXS + kTP * g.O4 + kTP * 2 * g.R) * 4;
+  if (!allow_lds_weights<T, VEC>()) return M2D_ERR_HIP;
+  hipLaunchKernelGGL((m2d_proj_bwd_weights_kernel<T, VEC>), dim3(g.G, g.ne), dim3(kThreads), lds_w, st, a);
+  if (!launched()) return M2D_ERR_HIP;
+  hipLaunchKernelGGL(m2d_proj_reduce_kernel, dim3(g.O + 2 * g.R + 2, g.ne), dim3(64 * kRedSlices), 0, st, a);
+  return launched() ? M2D_OK : M2D_ERR_HIP;
 }
 
 }  // namespace
@@ -513,21 +715,23 @@ int m2d_proj_fwd(const m2d_desc* desc, int dt_rank, const void* x, const float* 
   if (workspace_bytes < g.bytes_fwd) return M2D_ERR_WORKSPACE;
   hipStream_t st = static_cast<hipStream_t>(stream);
   char* ws = static_cast<char*>(workspace);
-  float* Wt = reinterpret_cast<float*>(ws + g.off_Wt);
-  const int n = g.Epad * g.Opad;
-  hipLaunchKernelGGL(m2d_proj_pack_kernel, dim3((n + 255) / 256), dim3(256), 0, st, x_proj_w, dt_projT_w, dt_projL_w, Wt,
-                     (float*)nullptr, (float*)nullptr, (float*)nullptr, g.E, g.R, g.O, g.Epad, g.Opad, g.Rpad);
+  PackArgs k = {};
+  k.Wx = x_proj_w; k.wT = dt_projT_w; k.bT = dt_projT_b; k.wL = dt_projL_w; k.bL = dt_projL_b;
+  k.Wt = reinterpret_cast<float*>(ws + g.off_Wt);
+  k.wTt = reinterpret_cast<float*>(ws + g.off_wTt);
+  k.wLt = reinterpret_cast<float*>(ws + g.off_wLt);
+  k.bTp = reinterpret_cast<float*>(ws + g.off_bTp);
+  k.bLp = reinterpret_cast<float*>(ws + g.off_bLp);
+  k.E = g.E; k.R = g.R; k.O = g.O; k.Epad = g.Epad; k.Opad = g.Opad; k.Rpad = g.Rpad;
+  const int n = g.Epad * g.Opad;   // the largest forward copy (Opad >= R)
+  hipLaunchKernelGGL(m2d_proj_pack_kernel, dim3((n + 255) / 256), dim3(256), 0, st, k);
   if (!launched()) return M2D_ERR_HIP;
   ProjArgs a = {};
   fill(a, g);
-  a.x = x; a.Wt = Wt; a.wT = dt_projT_w; a.wL = dt_projL_w; a.bT = dt_projT_b; a.bL = dt_projL_b;
+  a.x = x; a.Wt = k.Wt; a.wTt = k.wTt; a.wLt = k.wLt; a.bTp = k.bTp; a.bLp = k.bLp;
   a.r_out = lowrank; a.dT_out = deltaT; a.dL_out = deltaL; a.BT_out = BT; a.BL_out = BL; a.C_out = C;
-  const size_t lds = (size_t)(kTP * kXS + kTP * (g.O + 1)) * 4;
-  if (desc->dtype == M2D_F32)
-    hipLaunchKernelGGL(m2d_proj_fwd_kernel<float>, dim3(g.ntiles), dim3(kThreads), lds, st, a);
-  else
-    hipLaunchKernelGGL(m2d_proj_fwd_kernel<bf16_t>, dim3(g.ntiles), dim3(kThreads), lds, st, a);
-  return launched() ? M2D_OK : M2D_ERR_HIP;
+  if (desc->dtype == M2D_F32) return g.vec ? run_proj_fwd<float, true>(g, a, st) : run_proj_fwd<float, false>(g, a, st);
+  return g.vec ? run_proj_fwd<bf16_t, true>(g, a, st) : run_proj_fwd<bf16_t, false>(g, a, st);
 }
 
 int m2d_proj_bwd(const m2d_desc* desc, int dt_rank, const void* x, const void* lowrank, const void* deltaT,
@@ -546,36 +750,26 @@ int m2d_proj_bwd(const m2d_desc* desc, int dt_rank, const void* x, const void* l
   if (workspace_bytes < g.bytes_bwd) return M2D_ERR_WORKSPACE;
   hipStream_t st = static_cast<hipStream_t>(stream);
   char* ws = static_cast<char*>(workspace);
-  float* Wp = reinterpret_cast<float*>(ws + g.off_Wp);
-  float* wTp = reinterpret_cast<float*>(ws + g.off_wTp);
-  float* wLp = reinterpret_cast<float*>(ws + g.off_wLp);
+  PackArgs k = {};
+  k.Wx = x_proj_w; k.wT = dt_projT_w; k.wL = dt_projL_w;
+  k.Wp = reinterpret_cast<float*>(ws + g.off_Wp);
+  k.wTp = reinterpret_cast<float*>(ws + g.off_wTp);
+  k.wLp = reinterpret_cast<float*>(ws + g.off_wLp);
+  k.E = g.E; k.R = g.R; k.O = g.O; k.Epad = g.Epad; k.Opad = g.Opad; k.Rpad = g.Rpad;
   int n = g.O * g.Epad;
   if (g.Epad * g.Rpad > n) n = g.Epad * g.Rpad;
-  hipLaunchKernelGGL(m2d_proj_pack_kernel, dim3((n + 255) / 256), dim3(256), 0, st, x_proj_w, dt_projT_w, dt_projL_w,
-                     (float*)nullptr, Wp, wTp, wLp, g.E, g.R, g.O, g.Epad, g.Opad, g.Rpad);
+  hipLaunchKernelGGL(m2d_proj_pack_kernel, dim3((n + 255) / 256), dim3(256), 0, st, k);
   if (!launched()) return M2D_ERR_HIP;
   ProjArgs a = {};
   fill(a, g);
   a.x = x; a.r = lowrank; a.dT = deltaT; a.dL = deltaL;
   a.ddT = d_deltaT; a.ddL = d_deltaL; a.dBT = d_BT; a.dBL = d_BL; a.dC = d_C; a.dx = dx;
-  a.Wp = Wp; a.wTp = wTp; a.wLp = wLp;
+  a.Wp = k.Wp; a.wTp = k.wTp; a.wLp = k.wLp;
   a.dz = reinterpret_cast<float*>(ws + g.off_dz);
   a.part = reinterpret_cast<float*>(ws + g.off_part);
   a.dWx = d_x_proj_w; a.dwT = d_dt_projT_w; a.dbT = d_dt_projT_b; a.dwL = d_dt_projL_w; a.dbL = d_dt_projL_b;
-  const bool f32 = desc->dtype == M2D_F32;
-  const size_t lds_data = (size_t)(2 * kTP * kXS + kTP * (g.O + 1)) * 4;
-  if (f32) hipLaunchKernelGGL(m2d_proj_bwd_data_kernel<float>, dim3(g.ntiles), dim3(kThreads), lds_data, st, a);
-  else hipLaunchKernelGGL(m2d_proj_bwd_data_kernel<bf16_t>, dim3(g.ntiles), dim3(kThreads), lds_data, st, a);
-  if (!launched()) return M2D_ERR_HIP;
-  const int O4 = (g.O + 3) & ~3;
-  const size_t lds_w = (size_t)(kTP * kXS4 + 2 * kTP * kXS + kTP * O4 + kTP * (2 * g.R + 1)) * 4;
-  if (!(f32 ? allow_lds_weights<float>() : allow_lds_weights<bf16_t>())) return M2D_ERR_HIP;
-  if (f32) hipLaunchKernelGGL(m2d_proj_bwd_weights_kernel<float>, dim3(g.G, g.ne), dim3(kThreads), lds_w, st, a);
-  else hipLaunchKernelGGL(m2d_proj_bwd_weights_kernel<bf16_t>, dim3(g.G, g.ne), dim3(kThreads), lds_w, st, a);
-  if (!launched()) return M2D_ERR_HIP;
-  const int nout = (g.O + 2 * g.R + 2) * g.E;
-  hipLaunchKernelGGL(m2d_proj_reduce_kernel, dim3((nout + 255) / 256), dim3(256), 0, st, a);
-  return launched() ? M2D_OK : M2D_ERR_HIP;
+  if (desc->dtype == M2D_F32) return g.vec ? run_proj_bwd<float, true>(g, a, st) : run_proj_bwd<float, false>(g, a, st);
+  return g.vec ? run_proj_bwd<bf16_t, true>(g, a, st) : run_proj_bwd<bf16_t, false>(g, a, st);
 }
 
 }  // extern "C"
