@@ -37,12 +37,8 @@ struct bf16_t { uint16_t v; };
 
 __device__ __forceinline__ float ld(const float* p) { return *p; }
 __device__ __forceinline__ float ld(const bf16_t* p) { return __uint_as_float((uint32_t)p->v << 16); }
-__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);  // NaN
-  u += 0x7fffu + ((u >> 16) & 1u);                                            // round to nearest even
-  return (uint16_t)(u >> 16);
-}
+// round to nearest even; the conversion is one instruction on gfx950 (v_cvt_pk_bf16_f32)
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
 __device__ __forceinline__ void st(float* p, float v) { *p = v; }
 __device__ __forceinline__ void st(bf16_t* p, float v) { p->v = f32_to_bf16_bits(v); }
 // the value a tensor of type T would hold
@@ -81,11 +77,16 @@ struct ProjArgs {
   const float *bTp, *bLp;                // [Epad]
   const float *Wp;                       // [O][Epad]      Wx
   const float *wTp, *wLp;                // [Epad][Rpad]   dt weights
+  // packed weights for the matrix-core kernels, bf16, zero where padded
+  const uint16_t *Wb;                    // [Opad][Epad]   Wx
+  const uint16_t *wTb, *wLb;             // [Epad][32]     dt weights
+  const uint16_t *wTtb, *wLtb;           // [Rpad][Epad]   dt weights transposed
+  const uint16_t *WxTb;                  // [Epad][Opad32] Wx transposed
   float* dz;                             // (P,O4) fp32, rows padded to a multiple of 4
   float* part;                           // per-workgroup sums of the weight gradients
   float *dWx, *dwT, *dbT, *dwL, *dbL;    // outputs of the reduction
   int64_t P;
-  int E, R, O, O4, Epad, Opad, Rpad;
+  int E, R, O, O4, Epad, Opad, Opad32, Rpad;
   int ntiles, G, ne;
 };
 
@@ -101,7 +102,9 @@ struct PackArgs {
   const float *Wx, *wT, *bT, *wL, *bL;
   float *Wt, *wTt, *wLt, *bTp, *bLp;     // forward set (or null)
   float *Wp, *wTp, *wLp;                 // backward set (or null)
-  int E, R, O, Epad, Opad, Rpad;
+  uint16_t *Wb, *wTb, *wLb;              // forward set of the matrix-core kernels (or null)
+  uint16_t *wTtb, *wLtb, *WxTb;          // backward set of the matrix-core kernels (or null)
+  int E, R, O, Epad, Opad, Opad32, Rpad;
 };
 
 // Padded copies of the weights.  One thread per element of the largest copy.
@@ -117,9 +120,33 @@ __global__ void m2d_proj_pack_kernel(const PackArgs k) {
       k.wTt[i] = e < k.E ? k.wT[e * k.R + q] : 0.f;
       k.wLt[i] = e < k.E ? k.wL[e * k.R + q] : 0.f;
     }
-    if (i < k.Epad) {
-      k.bTp[i] = i < k.E ? k.bT[i] : 0.f;
-      k.bLp[i] = i < k.E ? k.bL[i] : 0.f;
+  }
+  if (k.bTp && i < k.Epad) {
+    k.bTp[i] = i < k.E ? k.bT[i] : 0.f;
+    k.bLp[i] = i < k.E ? k.bL[i] : 0.f;
+  }
+  if (k.Wb) {
+    if (i < k.Opad * k.Epad) {
+      const int o = i / k.Epad, e = i - o * k.Epad;
+      k.Wb[i] = (o < k.O && e < k.E) ? f32_to_bf16_bits(k.Wx[o * k.E + e]) : 0;
+    }
+    if (i < k.Epad * 32) {
+      const int e = i >> 5, q = i & 31;
+      const bool ok = e < k.E && q < k.R;
+      k.wTb[i] = ok ? f32_to_bf16_bits(k.wT[e * k.R + q]) : 0;
+      k.wLb[i] = ok ? f32_to_bf16_bits(k.wL[e * k.R + q]) : 0;
+    }
+  }
+  if (k.WxTb) {
+    if (i < k.Epad * k.Opad32) {
+      const int e = i / k.Opad32, o = i - e * k.Opad32;
+      k.WxTb[i] = (o < k.O && e < k.E) ? f32_to_bf16_bits(k.Wx[o * k.E + e]) : 0;
+    }
+    if (i < k.Rpad * k.Epad) {
+      const int q = i / k.Epad, e = i - q * k.Epad;
+      const bool ok = e < k.E && q < k.R;
+      k.wTtb[i] = ok ? f32_to_bf16_bits(k.wT[e * k.R + q]) : 0;
+      k.wLtb[i] = ok ? f32_to_bf16_bits(k.wL[e * k.R + q]) : 0;
     }
   }
   if (k.Wp) {
@@ -427,6 +454,209 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_data_kernel(const ProjA
   }
 }
 
+// ------------------------------------------------------------------------------- matrix cores
+// bf16 tensors whose rows start on 16-byte boundaries take the products through
+// v_mfma_f32_16x16x32_bf16.  A wave owns 16 positions and needs nothing from the other waves of
+// its workgroup.  Operand layout of the instruction (lane l, m = n = l & 15, kb = l >> 4):
+//   A[m][8 kb + j], B[8 kb + j][n] (j < 8, one 16-byte register set each);  D[4 kb + i][n], i < 4.
+// With positions as rows of A, the 8 values a lane needs are 8 consecutive channels of one
+// position: one 16-byte load straight from the (P,E) array.  The weights are packed so that the
+// same holds for B.
+#ifndef M2D_PROJ_OCC
+#define M2D_PROJ_OCC 5
+#endif
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+constexpr int kMaxNT = (2 * kMaxR + 3 * kN + 15) / 16;   // 16-wide tiles of the 2R+48 outputs
+constexpr int kLowStride = 40;   // bf16 per row of the low-rank scratch: 32 + 8, rows 16-byte aligned and spread over the banks
+
+__device__ __forceinline__ f32x4 mfma16(uint4 a, uint4 b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ uint4 load16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack2(float lo, float hi) {
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){lo, hi}, bf16x2));
+}
+
+// Forward.  LDS: per wave two [16][40] bf16 blocks (low-rank inputs of the T and L projection).
+__global__ __launch_bounds__(kThreads, M2D_PROJ_OCC) void m2d_proj_fwd_mfma_kernel(const ProjArgs a) {
+  extern __shared__ float smem[];
+  const int wave = wave_id(), l = threadIdx.x & 63, mn = l & 15, kb = l >> 4;
+  uint16_t* lowT = reinterpret_cast<uint16_t*>(smem) + wave * 2 * 16 * kLowStride;
+  uint16_t* lowL = lowT + 16 * kLowStride;
+  // columns past the rank meet zero weights; they only have to be finite
+  for (int i = l; i < 16 * kLowStride; i += 64) reinterpret_cast<uint32_t*>(lowT)[i] = 0u;
+  const int64_t p0 = (int64_t)blockIdx.x * kTP + wave * 16;
+  const bf16_t* x = static_cast<const bf16_t*>(a.x);
+  const int64_t pm = p0 + mn;
+  const int NT = a.Opad / 16, R = a.R, R2 = 2 * a.R;
+
+  f32x4 acc[kMaxNT];
+#pragma unroll
+  for (int nt = 0; nt < kMaxNT; ++nt) acc[nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  for (int e = 8 * kb; e < a.Epad; e += 32) {
+    const uint4 A = (pm < a.P && e < a.E) ? load16(x + pm * a.E + e) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int nt = 0; nt < kMaxNT; ++nt)
+      if (nt < NT) acc[nt] = mfma16(A, load16(a.Wb + (16 * nt + mn) * a.Epad + e), acc[nt]);
+  }
+
+  // z[position 4 kb + i][output 16 nt + mn]: low-rank inputs, B_T, B_L, C.  Addresses are a
+  // wave-uniform base (the wave's first position) plus a 32-bit element offset.
+  const int rows = (int)(a.P - p0 < 16 ? a.P - p0 : 16);   // positions of the wave inside the array (may be <= 0)
+  bf16_t* r_out = static_cast<bf16_t*>(a.r_out) + p0 * R2;
+  bf16_t* bt_out = static_cast<bf16_t*>(a.BT_out) + p0 * kN;
+  bf16_t* bl_out = static_cast<bf16_t*>(a.BL_out) + p0 * kN;
+  bf16_t* c_out = static_cast<bf16_t*>(a.C_out) + p0 * kN;
+#pragma unroll
+  for (int nt = 0; nt < kMaxNT; ++nt) {
+    if (nt >= NT) break;
+    const int o = 16 * nt + mn;
+    const int oo = o - R2;
+    bf16_t* bc = (oo < kN ? bt_out : (oo < 2 * kN ? bl_out : c_out)) + (oo & (kN - 1));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = 4 * kb + i;
+      const uint16_t h = f32_to_bf16_bits(acc[nt][i]);
+      if (o < R) lowT[c * kLowStride + o] = h;
+      else if (o < R2) lowL[c * kLowStride + o - R] = h;
+      if (c < rows) {
+        if (o < R2) r_out[(uint32_t)(c * R2 + o)].v = h;
+        else if (o < a.O) bc[(uint32_t)(c * kN)].v = h;
+      }
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+  // delta = softplus(low w^T + b): the rank is the inner dimension (one step of 32)
+  const uint4 AT = load16(lowT + mn * kLowStride + 8 * kb), AL = load16(lowL + mn * kLowStride + 8 * kb);
+  bf16_t* dT_out = static_cast<bf16_t*>(a.dT_out) + p0 * a.E;
+  bf16_t* dL_out = static_cast<bf16_t*>(a.dL_out) + p0 * a.E;
+  for (int e = mn; e < a.Epad; e += 16) {
+    const float bT = a.bTp[e], bL = a.bLp[e];
+    const f32x4 sT = mfma16(AT, load16(a.wTb + e * 32 + 8 * kb), (f32x4){bT, bT, bT, bT});
+    const f32x4 sL = mfma16(AL, load16(a.wLb + e * 32 + 8 * kb), (f32x4){bL, bL, bL, bL});
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = 4 * kb + i;
+      if (c < rows && e < a.E) {
+        st(dT_out + (uint32_t)(c * a.E + e), softplus(sT[i]));
+        st(dL_out + (uint32_t)(c * a.E + e), softplus(sL[i]));
+      }
+    }
+  }
+}
+
+// Backward, data.  LDS: per wave one [16][Opad32 + 8] bf16 block (the rows of dz).
+__global__ __launch_bounds__(kThreads, M2D_PROJ_OCC) void m2d_proj_bwd_data_mfma_kernel(const ProjArgs a) {
+  extern __shared__ float smem[];
+  const int wave = wave_id(), l = threadIdx.x & 63, mn = l & 15, kb = l >> 4;
+  const int zst = a.Opad32 + 8;
+  uint16_t* zs = reinterpret_cast<uint16_t*>(smem) + wave * 16 * zst;
+  for (int i = l; i < 16 * zst / 2; i += 64) reinterpret_cast<uint32_t*>(zs)[i] = 0u;   // padding columns: finite
+  const int64_t p0 = (int64_t)blockIdx.x * kTP + wave * 16;
+  const int rows = (int)(a.P - p0 < 16 ? a.P - p0 : 16);   // positions of the wave inside the array (may be <= 0)
+  const int R = a.R, R2 = 2 * a.R, NQ = a.Rpad / 16;
+  // wave-uniform bases (the wave's first position); lanes add 32-bit element offsets
+  const bf16_t* dT = static_cast<const bf16_t*>(a.dT) + p0 * a.E;
+  const bf16_t* dL = static_cast<const bf16_t*>(a.dL) + p0 * a.E;
+  const bf16_t* ddT = static_cast<const bf16_t*>(a.ddT) + p0 * a.E;
+  const bf16_t* ddL = static_cast<const bf16_t*>(a.ddL) + p0 * a.E;
+  bf16_t* dx = static_cast<bf16_t*>(a.dx) + p0 * a.E;
+  float* dz = a.dz + p0 * a.O4;
+  const uint4 z4 = make_uint4(0, 0, 0, 0);
+
+  // Memory latency is covered by the other waves of the compute unit (registers are kept low
+  // for that), not by fetching ahead.
+  // dB_T, dB_L, dC: lane l holds 4 values of position l >> 2
+  const int cb = l >> 2, n0 = 4 * (l & 3);
+  uint2 bc[3];
+#pragma unroll
+  for (int w = 0; w < 3; ++w) {
+    const bf16_t* src = static_cast<const bf16_t*>(w == 0 ? a.dBT : (w == 1 ? a.dBL : a.dC)) + p0 * kN;
+    bc[w] = cb < rows ? *reinterpret_cast<const uint2*>(src + (uint32_t)(cb * kN + n0)) : make_uint2(0, 0);
+  }
+
+  // dz[., rank] = dpre w, channels as the inner dimension
+  f32x4 accT[2], accL[2];
+#pragma unroll
+  for (int nq = 0; nq < 2; ++nq) { accT[nq] = (f32x4){0.f, 0.f, 0.f, 0.f}; accL[nq] = accT[nq]; }
+  auto dpre = [](uint4 g, uint4 v) {
+    const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, vw[4] = {v.x, v.y, v.z, v.w};
+    uint32_t r[4];
+#pragma unroll
+    for (int h = 0; h < 4; ++h)
+      r[h] = pack2(bf16_lo(gw[h]) * softplus_slope(bf16_lo(vw[h])), bf16_hi(gw[h]) * softplus_slope(bf16_hi(vw[h])));
+    return make_uint4(r[0], r[1], r[2], r[3]);
+  };
+  for (int e = 8 * kb; e < a.Epad; e += 32) {
+    const bool ok = mn < rows && e < a.E;
+    const uint32_t off = (uint32_t)(mn * a.E + e);
+    const uint4 gT = ok ? load16(ddT + off) : z4, vT = ok ? load16(dT + off) : z4;
+    const uint4 gL = ok ? load16(ddL + off) : z4, vL = ok ? load16(dL + off) : z4;
+    const uint4 AT = dpre(gT, vT), AL = dpre(gL, vL);
+#pragma unroll
+    for (int nq = 0; nq < 2; ++nq)
+      if (nq < NQ) {
+        accT[nq] = mfma16(AT, load16(a.wTtb + (16 * nq + mn) * a.Epad + e), accT[nq]);
+        accL[nq] = mfma16(AL, load16(a.wLtb + (16 * nq + mn) * a.Epad + e), accL[nq]);
+      }
+  }
+  // rows of dz: to LDS as bf16 (operand of the next product) and to memory as fp32 (weight gradients)
+#pragma unroll
+  for (int nq = 0; nq < 2; ++nq) {
+    const int q = 16 * nq + mn;
+    if (nq < NQ && q < R) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int c = 4 * kb + i;
+        zs[c * zst + q] = f32_to_bf16_bits(accT[nq][i]);
+        zs[c * zst + R + q] = f32_to_bf16_bits(accL[nq][i]);
+        if (c < rows) {
+          dz[(uint32_t)(c * a.O4 + q)] = accT[nq][i];
+          dz[(uint32_t)(c * a.O4 + R + q)] = accL[nq][i];
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int w = 0; w < 3; ++w) {
+    uint32_t* dst = reinterpret_cast<uint32_t*>(zs + cb * zst + R2 + w * kN + n0);   // even offsets: 4-byte aligned
+    dst[0] = bc[w].x;
+    dst[1] = bc[w].y;
+    if (cb < rows) {
+      float* out = dz + (uint32_t)(cb * a.O4 + R2 + w * kN + n0);
+      out[0] = bf16_lo(bc[w].x); out[1] = bf16_hi(bc[w].x); out[2] = bf16_lo(bc[w].y); out[3] = bf16_hi(bc[w].y);
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+  // dx += dz Wx, outputs as the inner dimension
+  constexpr int kMaxKS = (2 * kMaxR + 3 * kN + 31) / 32;
+  uint4 A2[kMaxKS];
+#pragma unroll
+  for (int ks = 0; ks < kMaxKS; ++ks)
+    A2[ks] = 32 * ks < a.Opad32 ? load16(zs + mn * zst + 32 * ks + 8 * kb) : z4;
+  for (int e = mn; e < a.Epad; e += 16) {
+    float was[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) was[i] = (4 * kb + i < rows && e < a.E) ? ld(dx + (uint32_t)((4 * kb + i) * a.E + e)) : 0.f;
+    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int ks = 0; ks < kMaxKS; ++ks)
+      if (32 * ks < a.Opad32) s = mfma16(A2[ks], load16(a.WxTb + e * a.Opad32 + 32 * ks + 8 * kb), s);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (4 * kb + i < rows && e < a.E) st(dx + (uint32_t)((4 * kb + i) * a.E + e), was[i] + s[i]);
+  }
+}
+
 // ------------------------------------------------------------------------------- backward, weights
 // Grid (G, ne): workgroup (g, ey) adds up, over the tiles g, g+G, ..., the gradients of the weights
 // that touch channels [64 ey, 64 ey + 64) and leaves them in part[g][ey][row][64]:
@@ -603,12 +833,13 @@ inline bool misaligned(const void* p, size_t a) { return (reinterpret_cast<uintp
 
 struct ProjGeometry {
   int64_t P;
-  int E, R, O, O4, Epad, Opad, Rpad, ntiles, G, ne;
-  bool vec;   // rows of the (P,E) arrays start on 16-byte boundaries
+  int E, R, O, O4, Epad, Opad, Opad32, Rpad, ntiles, G, ne;
+  bool vec;    // rows of the (P,E) arrays start on 16-byte boundaries
+  bool mfma;   // bf16 and vec: products on the matrix cores
   // forward workspace
-  size_t off_Wt, off_wTt, off_wLt, off_bTp, off_bLp, bytes_fwd;
+  size_t off_Wt, off_wTt, off_wLt, off_bTp, off_bLp, off_Wb, off_wTb, off_wLb, bytes_fwd;
   // backward workspace
-  size_t off_Wp, off_wTp, off_wLp, off_dz, off_part, bytes_bwd;
+  size_t off_Wp, off_wTp, off_wLp, off_wTtb, off_wLtb, off_WxTb, off_dz, off_part, bytes_bwd;
 };
 
 int check_proj(const m2d_desc* d, int R) {
@@ -627,10 +858,12 @@ ProjGeometry proj_geometry(const m2d_desc* d, int R) {
   g.O4 = (g.O + 3) & ~3;
   g.Epad = (g.E + kKC - 1) / kKC * kKC;
   g.Opad = (g.O + 15) / 16 * 16;
+  g.Opad32 = (g.O + 31) / 32 * 32;
   g.Rpad = (R + 15) / 16 * 16;
   g.ntiles = (int)((g.P + kTP - 1) / kTP);
   g.ne = g.Epad / kKC;
   g.vec = d->E % (d->dtype == M2D_F32 ? 4 : 8) == 0;
+  g.mfma = g.vec && d->dtype == M2D_BF16;
   const int want = 512 / g.ne > 0 ? 512 / g.ne : 1;   // about two workgroups per compute unit in all
   g.G = g.ntiles < want ? g.ntiles : want;
   size_t o = 0;
@@ -639,11 +872,17 @@ ProjGeometry proj_geometry(const m2d_desc* d, int R) {
   g.off_wLt = o; o += align256((size_t)R * g.Epad * 4);
   g.off_bTp = o; o += align256((size_t)g.Epad * 4);
   g.off_bLp = o; o += align256((size_t)g.Epad * 4);
+  g.off_Wb = o; o += align256((size_t)g.Opad * g.Epad * 2);
+  g.off_wTb = o; o += align256((size_t)g.Epad * 32 * 2);
+  g.off_wLb = o; o += align256((size_t)g.Epad * 32 * 2);
   g.bytes_fwd = o;
   o = 0;
   g.off_Wp = o; o += align256((size_t)g.O * g.Epad * 4);
   g.off_wTp = o; o += align256((size_t)g.Epad * g.Rpad * 4);
   g.off_wLp = o; o += align256((size_t)g.Epad * g.Rpad * 4);
+  g.off_wTtb = o; o += align256((size_t)g.Rpad * g.Epad * 2);
+  g.off_wLtb = o; o += align256((size_t)g.Rpad * g.Epad * 2);
+  g.off_WxTb = o; o += align256((size_t)g.Epad * g.Opad32 * 2);
   g.off_dz = o; o += align256((size_t)g.P * g.O4 * 4);
   g.off_part = o; o += align256((size_t)g.G * g.ne * (g.O + 2 * R + 2) * kKC * 4);
   g.bytes_bwd = o;
@@ -651,7 +890,7 @@ ProjGeometry proj_geometry(const m2d_desc* d, int R) {
 }
 
 void fill(ProjArgs& a, const ProjGeometry& g) {
-  a.P = g.P; a.E = g.E; a.R = g.R; a.O = g.O; a.O4 = g.O4; a.Epad = g.Epad; a.Opad = g.Opad; a.Rpad = g.Rpad;
+  a.P = g.P; a.E = g.E; a.R = g.R; a.O = g.O; a.O4 = g.O4; a.Epad = g.Epad; a.Opad = g.Opad; a.Opad32 = g.Opad32; a.Rpad = g.Rpad;
   a.ntiles = g.ntiles; a.G = g.G; a.ne = g.ne;
 }
 
@@ -671,6 +910,12 @@ bool allow_lds_weights() {
   return true;
 }
 
+int run_proj_fwd_mfma(const ProjGeometry& g, const ProjArgs& a, hipStream_t st) {
+  const size_t lds = (size_t)kWaves * 2 * 16 * kLowStride * 2;
+  hipLaunchKernelGGL(m2d_proj_fwd_mfma_kernel, dim3(g.ntiles), dim3(kThreads), lds, st, a);
+  return launched() ? M2D_OK : M2D_ERR_HIP;
+}
+
 template <typename T, bool VEC>
 int run_proj_fwd(const ProjGeometry& g, const ProjArgs& a, hipStream_t st) {
   const size_t lds = (size_t)(2 * kTP * kXS + kTP * (g.O + 1)) * 4;
@@ -680,8 +925,13 @@ int run_proj_fwd(const ProjGeometry& g, const ProjArgs& a, hipStream_t st) {
 
 template <typename T, bool VEC>
 int run_proj_bwd(const ProjGeometry& g, const ProjArgs& a, hipStream_t st) {
-  const size_t lds_data = (size_t)(2 * kTP * kXS + kTP * (g.O + 1)) * 4;
-  hipLaunchKernelGGL((m2d_proj_bwd_data_kernel<T, VEC>), dim3(g.ntiles), dim3(kThreads), lds_data, st, a);
+  if (g.mfma) {
+    const size_t lds_data = (size_t)kWaves * 16 * (g.Opad32 + 8) * 2;
+    hipLaunchKernelGGL(m2d_proj_bwd_data_mfma_kernel, dim3(g.ntiles), dim3(kThreads), lds_data, st, a);
+  } else {
+    const size_t lds_data = (size_t)(2 * kTP * kXS + kTP * (g.O + 1)) * 4;
+    hipLaunchKernelGGL((m2d_proj_bwd_data_kernel<T, VEC>), dim3(g.ntiles), dim3(kThreads), lds_data, st, a);
+  }
   if (!launched()) return M2D_ERR_HIP;
   const size_t lds_w = (size_t)(kTP * kXS4 + 2 * kTP * kXS + kTP * g.O4 + kTP * 2 * g.R) * 4;
   if (!allow_lds_weights<T, VEC>()) return M2D_ERR_HIP;
@@ -722,16 +972,23 @@ int m2d_proj_fwd(const m2d_desc* desc, int dt_rank, const void* x, const float* 
   k.wLt = reinterpret_cast<float*>(ws + g.off_wLt);
   k.bTp = reinterpret_cast<float*>(ws + g.off_bTp);
   k.bLp = reinterpret_cast<float*>(ws + g.off_bLp);
-  k.E = g.E; k.R = g.R; k.O = g.O; k.Epad = g.Epad; k.Opad = g.Opad; k.Rpad = g.Rpad;
-  const int n = g.Epad * g.Opad;   // the largest forward copy (Opad >= R)
+  if (g.mfma) {   // the matrix-core kernel reads the bf16 set
+    k.Wt = nullptr;
+    k.Wb = reinterpret_cast<uint16_t*>(ws + g.off_Wb);
+    k.wTb = reinterpret_cast<uint16_t*>(ws + g.off_wTb);
+    k.wLb = reinterpret_cast<uint16_t*>(ws + g.off_wLb);
+  }
+  k.E = g.E; k.R = g.R; k.O = g.O; k.Epad = g.Epad; k.Opad = g.Opad; k.Opad32 = g.Opad32; k.Rpad = g.Rpad;
+  const int n = g.Epad * (g.Opad > 32 ? g.Opad : 32);   // the largest forward copy
   hipLaunchKernelGGL(m2d_proj_pack_kernel, dim3((n + 255) / 256), dim3(256), 0, st, k);
   if (!launched()) return M2D_ERR_HIP;
   ProjArgs a = {};
   fill(a, g);
   a.x = x; a.Wt = k.Wt; a.wTt = k.wTt; a.wLt = k.wLt; a.bTp = k.bTp; a.bLp = k.bLp;
+  a.Wb = k.Wb; a.wTb = k.wTb; a.wLb = k.wLb;
   a.r_out = lowrank; a.dT_out = deltaT; a.dL_out = deltaL; a.BT_out = BT; a.BL_out = BL; a.C_out = C;
   if (desc->dtype == M2D_F32) return g.vec ? run_proj_fwd<float, true>(g, a, st) : run_proj_fwd<float, false>(g, a, st);
-  return g.vec ? run_proj_fwd<bf16_t, true>(g, a, st) : run_proj_fwd<bf16_t, false>(g, a, st);
+  return g.mfma ? run_proj_fwd_mfma(g, a, st) : run_proj_fwd<bf16_t, false>(g, a, st);
 }
 
 int m2d_proj_bwd(const m2d_desc* desc, int dt_rank, const void* x, const void* lowrank, const void* deltaT,
@@ -755,8 +1012,14 @@ int m2d_proj_bwd(const m2d_desc* desc, int dt_rank, const void* x, const void* l
   k.Wp = reinterpret_cast<float*>(ws + g.off_Wp);
   k.wTp = reinterpret_cast<float*>(ws + g.off_wTp);
   k.wLp = reinterpret_cast<float*>(ws + g.off_wLp);
-  k.E = g.E; k.R = g.R; k.O = g.O; k.Epad = g.Epad; k.Opad = g.Opad; k.Rpad = g.Rpad;
-  int n = g.O * g.Epad;
+  if (g.mfma) {   // the data kernel reads the bf16 set; the weight-gradient kernel needs no weights
+    k.Wp = nullptr;
+    k.wTtb = reinterpret_cast<uint16_t*>(ws + g.off_wTtb);
+    k.wLtb = reinterpret_cast<uint16_t*>(ws + g.off_wLtb);
+    k.WxTb = reinterpret_cast<uint16_t*>(ws + g.off_WxTb);
+  }
+  k.E = g.E; k.R = g.R; k.O = g.O; k.Epad = g.Epad; k.Opad = g.Opad; k.Opad32 = g.Opad32; k.Rpad = g.Rpad;
+  int n = g.Opad32 * g.Epad;
   if (g.Epad * g.Rpad > n) n = g.Epad * g.Rpad;
   hipLaunchKernelGGL(m2d_proj_pack_kernel, dim3((n + 255) / 256), dim3(256), 0, st, k);
   if (!launched()) return M2D_ERR_HIP;
@@ -765,6 +1028,7 @@ int m2d_proj_bwd(const m2d_desc* desc, int dt_rank, const void* x, const void* l
   a.x = x; a.r = lowrank; a.dT = deltaT; a.dL = deltaL;
   a.ddT = d_deltaT; a.ddL = d_deltaL; a.dBT = d_BT; a.dBL = d_BL; a.dC = d_C; a.dx = dx;
   a.Wp = k.Wp; a.wTp = k.wTp; a.wLp = k.wLp;
+  a.wTtb = k.wTtb; a.wLtb = k.wLtb; a.WxTb = k.WxTb;
   a.dz = reinterpret_cast<float*>(ws + g.off_dz);
   a.part = reinterpret_cast<float*>(ws + g.off_part);
   a.dWx = d_x_proj_w; a.dwT = d_dt_projT_w; a.dbT = d_dt_projT_b; a.dwL = d_dt_projL_w; a.dbL = d_dt_projL_b;
