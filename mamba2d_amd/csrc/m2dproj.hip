@@ -83,6 +83,9 @@ struct ProjArgs {
   const uint16_t *wTtb, *wLtb;           // [Rpad][Epad]   dt weights transposed
   const uint16_t *WxTb;                  // [Epad][Opad32] Wx transposed
   float* dz;                             // (P,O4) fp32, rows padded to a multiple of 4
+  // the same for the matrix-core kernels, bf16
+  uint16_t* dzt;                         // (P16, Opad)    dz, P16 = positions rounded up to 16
+  uint16_t* dpt;                         // [2](P16, E)    dpreT, dpreL
   float* part;                           // per-workgroup sums of the weight gradients
   float *dWx, *dwT, *dbT, *dwL, *dbL;    // outputs of the reduction
   int64_t P;
@@ -482,11 +485,40 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
   return __builtin_bit_cast(uint32_t, __builtin_convertvector((f32x2){lo, hi}, bf16x2));
 }
 
-// Forward.  LDS: per wave two [16][40] bf16 blocks (low-rank inputs of the T and L projection).
+// Results leave the accumulators (4 positions x 1 channel per lane and tile) through a per-wave
+// LDS block of 16 positions x 64 channels, so that memory sees 16-byte pieces of rows.
+constexpr int kStageStride = 68;   // floats per row: 64 + 4, rows 16-byte aligned
+__device__ __forceinline__ void wave_sync_lds() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+__device__ __forceinline__ void stage_put(float* stage, int nt, int mn, int kb, f32x4 v) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i) stage[(4 * kb + i) * kStageStride + 16 * nt + mn] = v[i];
+}
+// f(position, first channel, 8 values) for the lane's two pieces of the block
+template <typename F>
+__device__ __forceinline__ void stage_rows(const float* stage, int l, F f) {
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    const int piece = l + 64 * k, c = piece >> 3, c8 = 8 * (piece & 7);
+    const float4 lo = *reinterpret_cast<const float4*>(stage + c * kStageStride + c8);
+    const float4 hi = *reinterpret_cast<const float4*>(stage + c * kStageStride + c8 + 4);
+    const float v[8] = {lo.x, lo.y, lo.z, lo.w, hi.x, hi.y, hi.z, hi.w};
+    f(c, c8, v);
+  }
+}
+__device__ __forceinline__ uint4 pack8(const float (&v)[8]) {
+  return make_uint4(pack2(v[0], v[1]), pack2(v[2], v[3]), pack2(v[4], v[5]), pack2(v[6], v[7]));
+}
+
+// Forward.  LDS: per wave two [16][40] bf16 blocks (low-rank inputs of the T and L projection)
+// and the [16][68] fp32 block the delta tiles leave through.
 __global__ __launch_bounds__(kThreads, M2D_PROJ_OCC) void m2d_proj_fwd_mfma_kernel(const ProjArgs a) {
   extern __shared__ float smem[];
   const int wave = wave_id(), l = threadIdx.x & 63, mn = l & 15, kb = l >> 4;
-  uint16_t* lowT = reinterpret_cast<uint16_t*>(smem) + wave * 2 * 16 * kLowStride;
+  float* stage = smem + wave * (16 * kStageStride + 16 * kLowStride);   // [16][68] floats, then 2 x [16][40] bf16
+  uint16_t* lowT = reinterpret_cast<uint16_t*>(stage + 16 * kStageStride);
   uint16_t* lowL = lowT + 16 * kLowStride;
   // columns past the rank meet zero weights; they only have to be finite
   for (int i = l; i < 16 * kLowStride; i += 64) reinterpret_cast<uint32_t*>(lowT)[i] = 0u;
@@ -537,28 +569,42 @@ __global__ __launch_bounds__(kThreads, M2D_PROJ_OCC) void m2d_proj_fwd_mfma_kern
   const uint4 AT = load16(lowT + mn * kLowStride + 8 * kb), AL = load16(lowL + mn * kLowStride + 8 * kb);
   bf16_t* dT_out = static_cast<bf16_t*>(a.dT_out) + p0 * a.E;
   bf16_t* dL_out = static_cast<bf16_t*>(a.dL_out) + p0 * a.E;
-  for (int e = mn; e < a.Epad; e += 16) {
-    const float bT = a.bTp[e], bL = a.bLp[e];
-    const f32x4 sT = mfma16(AT, load16(a.wTb + e * 32 + 8 * kb), (f32x4){bT, bT, bT, bT});
-    const f32x4 sL = mfma16(AL, load16(a.wLb + e * 32 + 8 * kb), (f32x4){bL, bL, bL, bL});
+  for (int e0 = 0; e0 < a.Epad; e0 += kKC) {
+    f32x4 sT[4], sL[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = 4 * kb + i;
-      if (c < rows && e < a.E) {
-        st(dT_out + (uint32_t)(c * a.E + e), softplus(sT[i]));
-        st(dL_out + (uint32_t)(c * a.E + e), softplus(sL[i]));
+    for (int nt = 0; nt < 4; ++nt) {
+      const int e = e0 + 16 * nt + mn;
+      const float bT = a.bTp[e], bL = a.bLp[e];
+      sT[nt] = mfma16(AT, load16(a.wTb + e * 32 + 8 * kb), (f32x4){bT, bT, bT, bT});
+      sL[nt] = mfma16(AL, load16(a.wLb + e * 32 + 8 * kb), (f32x4){bL, bL, bL, bL});
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        const f32x4 v = h ? sL[nt] : sT[nt];
+        stage_put(stage, nt, mn, kb, (f32x4){softplus(v[0]), softplus(v[1]), softplus(v[2]), softplus(v[3])});
       }
+      wave_sync_lds();
+      bf16_t* out = h ? dL_out : dT_out;
+      stage_rows(stage, l, [&](int c, int c8, const float (&v)[8]) {
+        if (c < rows && e0 + c8 < a.E) *reinterpret_cast<uint4*>(out + (uint32_t)(c * a.E + e0 + c8)) = pack8(v);
+      });
+      wave_sync_lds();
     }
   }
 }
 
-// Backward, data.  LDS: per wave one [16][Opad32 + 8] bf16 block (the rows of dz).
+// Backward, data.  LDS: per wave one [16][Opad32 + 8] bf16 block (the rows of dz) and the [16][68]
+// fp32 block the dx tiles leave through.  dz and dpre are also written out as bf16 arrays for the
+// weight-gradient kernel.
 __global__ __launch_bounds__(kThreads, M2D_PROJ_OCC) void m2d_proj_bwd_data_mfma_kernel(const ProjArgs a) {
   extern __shared__ float smem[];
   const int wave = wave_id(), l = threadIdx.x & 63, mn = l & 15, kb = l >> 4;
   const int zst = a.Opad32 + 8;
-  uint16_t* zs = reinterpret_cast<uint16_t*>(smem) + wave * 16 * zst;
-  for (int i = l; i < 16 * zst / 2; i += 64) reinterpret_cast<uint32_t*>(zs)[i] = 0u;   // padding columns: finite
+  float* stage = smem + wave * (16 * kStageStride + 16 * zst / 2);   // [16][68] floats, then [16][zst] bf16
+  uint16_t* zs = reinterpret_cast<uint16_t*>(stage + 16 * kStageStride);
+  for (int i = l; i < 16 * zst / 2; i += 64) reinterpret_cast<uint32_t*>(zs)[i] = 0u;   // padding columns: zero
   const int64_t p0 = (int64_t)blockIdx.x * kTP + wave * 16;
   const int rows = (int)(a.P - p0 < 16 ? a.P - p0 : 16);   // positions of the wave inside the array (may be <= 0)
   const int R = a.R, R2 = 2 * a.R, NQ = a.Rpad / 16;
@@ -568,7 +614,10 @@ __global__ __launch_bounds__(kThreads, M2D_PROJ_OCC) void m2d_proj_bwd_data_mfma
   const bf16_t* ddT = static_cast<const bf16_t*>(a.ddT) + p0 * a.E;
   const bf16_t* ddL = static_cast<const bf16_t*>(a.ddL) + p0 * a.E;
   bf16_t* dx = static_cast<bf16_t*>(a.dx) + p0 * a.E;
-  float* dz = a.dz + p0 * a.O4;
+  // rows past the end of the arrays (up to the next multiple of 16) are written too, as zeros
+  uint16_t* dzt = a.dzt + p0 * a.Opad;
+  uint16_t* dptT = a.dpt + p0 * a.E;
+  uint16_t* dptL = dptT + (int64_t)a.ntiles * kTP * a.E;
   const uint4 z4 = make_uint4(0, 0, 0, 0);
 
   // Memory latency is covered by the other waves of the compute unit (registers are kept low
@@ -606,8 +655,12 @@ __global__ __launch_bounds__(kThreads, M2D_PROJ_OCC) void m2d_proj_bwd_data_mfma
         accT[nq] = mfma16(AT, load16(a.wTtb + (16 * nq + mn) * a.Epad + e), accT[nq]);
         accL[nq] = mfma16(AL, load16(a.wLtb + (16 * nq + mn) * a.Epad + e), accL[nq]);
       }
+    if (e < a.E) {
+      *reinterpret_cast<uint4*>(dptT + (uint32_t)(mn * a.E + e)) = AT;
+      *reinterpret_cast<uint4*>(dptL + (uint32_t)(mn * a.E + e)) = AL;
+    }
   }
-  // rows of dz: to LDS as bf16 (operand of the next product) and to memory as fp32 (weight gradients)
+  // rows of dz to LDS as bf16: operand of the next product, and source of the copy in memory
 #pragma unroll
   for (int nq = 0; nq < 2; ++nq) {
     const int q = 16 * nq + mn;
@@ -617,10 +670,6 @@ __global__ __launch_bounds__(kThreads, M2D_PROJ_OCC) void m2d_proj_bwd_data_mfma
         const int c = 4 * kb + i;
         zs[c * zst + q] = f32_to_bf16_bits(accT[nq][i]);
         zs[c * zst + R + q] = f32_to_bf16_bits(accL[nq][i]);
-        if (c < rows) {
-          dz[(uint32_t)(c * a.O4 + q)] = accT[nq][i];
-          dz[(uint32_t)(c * a.O4 + R + q)] = accL[nq][i];
-        }
       }
     }
   }
@@ -629,13 +678,16 @@ __global__ __launch_bounds__(kThreads, M2D_PROJ_OCC) void m2d_proj_bwd_data_mfma
     uint32_t* dst = reinterpret_cast<uint32_t*>(zs + cb * zst + R2 + w * kN + n0);   // even offsets: 4-byte aligned
     dst[0] = bc[w].x;
     dst[1] = bc[w].y;
-    if (cb < rows) {
-      float* out = dz + (uint32_t)(cb * a.O4 + R2 + w * kN + n0);
-      out[0] = bf16_lo(bc[w].x); out[1] = bf16_hi(bc[w].x); out[2] = bf16_lo(bc[w].y); out[3] = bf16_hi(bc[w].y);
-    }
   }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  {
+    const int per_row = a.Opad / 8;   // 16-byte pieces of a row
+    for (int i = l; i < 16 * per_row; i += 64) {
+      const int c = i / per_row, o8 = i - c * per_row;
+      *reinterpret_cast<uint4*>(dzt + (uint32_t)(c * a.Opad + 8 * o8)) = load16(zs + c * zst + 8 * o8);
+    }
+  }
 
   // dx += dz Wx, outputs as the inner dimension
   constexpr int kMaxKS = (2 * kMaxR + 3 * kN + 31) / 32;
@@ -643,17 +695,189 @@ __global__ __launch_bounds__(kThreads, M2D_PROJ_OCC) void m2d_proj_bwd_data_mfma
 #pragma unroll
   for (int ks = 0; ks < kMaxKS; ++ks)
     A2[ks] = 32 * ks < a.Opad32 ? load16(zs + mn * zst + 32 * ks + 8 * kb) : z4;
-  for (int e = mn; e < a.Epad; e += 16) {
-    float was[4];
+  for (int e0 = 0; e0 < a.Epad; e0 += kKC) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) was[i] = (4 * kb + i < rows && e < a.E) ? ld(dx + (uint32_t)((4 * kb + i) * a.E + e)) : 0.f;
-    f32x4 s = {0.f, 0.f, 0.f, 0.f};
+    for (int nt = 0; nt < 4; ++nt) {
+      const int e = e0 + 16 * nt + mn;
+      f32x4 s = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int ks = 0; ks < kMaxKS; ++ks)
-      if (32 * ks < a.Opad32) s = mfma16(A2[ks], load16(a.WxTb + e * a.Opad32 + 32 * ks + 8 * kb), s);
+      for (int ks = 0; ks < kMaxKS; ++ks)
+        if (32 * ks < a.Opad32) s = mfma16(A2[ks], load16(a.WxTb + e * a.Opad32 + 32 * ks + 8 * kb), s);
+      stage_put(stage, nt, mn, kb, s);
+    }
+    wave_sync_lds();
+    stage_rows(stage, l, [&](int c, int c8, const float (&v)[8]) {
+      if (c < rows && e0 + c8 < a.E) {
+        bf16_t* at = dx + (uint32_t)(c * a.E + e0 + c8);
+        const uint4 was = load16(at);
+        const uint32_t w[4] = {was.x, was.y, was.z, was.w};
+        float sum[8];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      if (4 * kb + i < rows && e < a.E) st(dx + (uint32_t)((4 * kb + i) * a.E + e), was[i] + s[i]);
+        for (int j = 0; j < 4; ++j) { sum[2 * j] = bf16_lo(w[j]) + v[2 * j]; sum[2 * j + 1] = bf16_hi(w[j]) + v[2 * j + 1]; }
+        *reinterpret_cast<uint4*>(at) = pack8(sum);
+      }
+    });
+    wave_sync_lds();
+  }
+}
+
+// Backward, weights, on the matrix cores.  Positions are the inner dimension of all three sums,
+//   dWx[o][e] = sum_p dz[p][o] x[p][e],  dw[e][q] = sum_p dpre[p][e] r[p][q],  db[e] = sum_p dpre[p][e] * 1,
+// so every operand is wanted position-last while the arrays are position-first.  A tile of 64
+// positions is turned in LDS: a lane loads 16 bytes of one position's row and writes its 8 values
+// into 8 rows of the position-last block (lanes = consecutive positions: no bank conflicts).
+// LDS: xT[64][72], pT[2][64][72], zT[Opad][72], rT[2][16 NQ1][72] with a row of ones after the
+// R rows of r (its column of the product is db).  Grid, parts and the prefetch of the next tile
+// are those of the vector-ALU kernel.
+constexpr int kPosStride = 72;   // bf16 per row of a position-last block: 64 + 8, rows 16-byte aligned
+constexpr int kMaxNQ1 = (kMaxR + 1 + 15) / 16;
+constexpr int kMaxZP = (kMaxNT * 2 + kWaves - 1) / kWaves;   // 16-byte pieces of a dz row per wave
+
+__global__ __launch_bounds__(kThreads) void m2d_proj_bwd_weights_mfma_kernel(const ProjArgs a) {
+  extern __shared__ float smem[];
+  const int wave = wave_id(), l = threadIdx.x & 63, mn = l & 15, kb = l >> 4, tid = threadIdx.x;
+  const int ey = blockIdx.y;
+  const int R = a.R, R2 = 2 * a.R;
+  const int NQ1 = (R + 1 + 15) / 16, MT = a.Opad / 16, ZP = a.Opad / 8;
+  uint16_t* xT = reinterpret_cast<uint16_t*>(smem);
+  uint16_t* pT = xT + kKC * kPosStride;
+  uint16_t* zT = pT + 2 * kKC * kPosStride;
+  uint16_t* rT = zT + a.Opad * kPosStride;
+  const int rblk = 16 * NQ1 * kPosStride;   // one tensor's block of rT
+  for (int i = tid; i < rblk; i += kThreads) reinterpret_cast<uint32_t*>(rT)[i] = 0u;   // both blocks (2 * rblk / 2 words)
+  __syncthreads();
+  if (tid < 2 * kTP) rT[(tid >> 6) * rblk + R * kPosStride + (tid & 63)] = 0x3F80;   // 1.0
+  const bf16_t* x = static_cast<const bf16_t*>(a.x);
+  const bf16_t* rr = static_cast<const bf16_t*>(a.r);
+  const uint16_t* dptL = a.dpt + (int64_t)a.ntiles * kTP * a.E;
+
+  // this thread's part of the r tile (64 x 2R values, contiguous): up to two 16-byte pieces
+  int rp[2], rq[2];
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    const int first = 8 * (k * kThreads + tid);
+    rp[k] = first / R2;
+    rq[k] = first - rp[k] * R2;
+  }
+  const int nr = kTP * R2;   // values in the r tile
+
+  f32x4 aw[2][4], ar[2][kMaxNQ1];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt) aw[h][nt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int nq = 0; nq < kMaxNQ1; ++nq) ar[h][nq] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+
+  const uint4 z4 = make_uint4(0, 0, 0, 0);
+  uint4 xr[2], pr[2][2], zr[kMaxZP], rv[2];
+  auto fetch = [&](int tile) {
+    const int64_t p0 = (int64_t)tile * kTP;
+    const int64_t left = a.P - p0;   // positions of the tile inside the array, if fewer than 64
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int e = ey * kKC + 8 * (2 * wave + k);
+      const bool ok = e < a.E;
+      xr[k] = (l < left && ok) ? load16(x + (p0 + l) * a.E + e) : z4;
+      // dz and dpre are written for whole tiles (zeros past the end of the arrays)
+      pr[0][k] = ok ? load16(a.dpt + (p0 + l) * a.E + e) : z4;
+      pr[1][k] = ok ? load16(dptL + (p0 + l) * a.E + e) : z4;
+      const int first = 8 * (k * kThreads + tid);
+      // a piece of r may straddle the end of the array, by whole values
+      rv[k] = z4;
+      if (first < nr) {
+        if ((int64_t)(first + 8) <= left * R2) rv[k] = load16(rr + p0 * R2 + first);
+        else if ((int64_t)first < left * R2) {
+          uint32_t w[4] = {0, 0, 0, 0};
+          for (int j = 0; j < 8; ++j)
+            if ((int64_t)(first + j) < left * R2) w[j >> 1] |= (uint32_t)rr[p0 * R2 + first + j].v << (16 * (j & 1));
+          rv[k] = make_uint4(w[0], w[1], w[2], w[3]);
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kMaxZP; ++k) {
+      const int o8 = wave + kWaves * k;
+      zr[k] = o8 < ZP ? load16(a.dzt + (p0 + l) * a.Opad + 8 * o8) : z4;
+    }
+  };
+  // lane = position: the 8 values of a 16-byte piece go to 8 consecutive rows of a position-last block
+  auto turn = [&](uint16_t* blk, uint4 v) {
+    const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+    for (int j = 0; j < 8; ++j) blk[j * kPosStride + l] = (uint16_t)(w[j >> 1] >> (16 * (j & 1)));
+  };
+
+  if ((int)blockIdx.x < a.ntiles) fetch(blockIdx.x);
+  for (int tile = blockIdx.x; tile < a.ntiles; tile += a.G) {
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      const int row0 = 8 * (2 * wave + k);
+      turn(xT + row0 * kPosStride, xr[k]);
+      turn(pT + row0 * kPosStride, pr[0][k]);
+      turn(pT + (kKC + row0) * kPosStride, pr[1][k]);
+      const int first = 8 * (k * kThreads + tid);
+      if (first < nr) {
+        const uint32_t v[4] = {rv[k].x, rv[k].y, rv[k].z, rv[k].w};
+        int p = rp[k], q = rq[k];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          if (p < kTP) rT[(q >= R ? rblk + (q - R) * kPosStride : q * kPosStride) + p] = (uint16_t)(v[j >> 1] >> (16 * (j & 1)));
+          if (++q == R2) { q = 0; ++p; }
+        }
+      }
+    }
+#pragma unroll
+    for (int k = 0; k < kMaxZP; ++k) {
+      const int o8 = wave + kWaves * k;
+      if (o8 < ZP) turn(zT + 8 * o8 * kPosStride, zr[k]);
+    }
+    __syncthreads();
+    if (tile + a.G < a.ntiles) fetch(tile + a.G);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const int koff = 32 * ks + 8 * kb;
+      const uint4 A0 = load16(zT + (16 * wave + mn) * kPosStride + koff);
+      const uint4 A1 = wave + kWaves < MT ? load16(zT + (16 * (wave + kWaves) + mn) * kPosStride + koff) : z4;
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        const uint4 B = load16(xT + (16 * nt + mn) * kPosStride + koff);
+        aw[0][nt] = mfma16(A0, B, aw[0][nt]);
+        if (wave + kWaves < MT) aw[1][nt] = mfma16(A1, B, aw[1][nt]);
+      }
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const uint4 Ap = load16(pT + (h * kKC + 16 * wave + mn) * kPosStride + koff);
+#pragma unroll
+        for (int nq = 0; nq < kMaxNQ1; ++nq)
+          if (nq < NQ1) ar[h][nq] = mfma16(Ap, load16(rT + h * rblk + (16 * nq + mn) * kPosStride + koff), ar[h][nq]);
+      }
+    }
+    __syncthreads();
+  }
+
+  // parts: D[4 kb + i][mn] of each accumulator
+  float* out = a.part + ((int64_t)blockIdx.x * a.ne + ey) * (int64_t)(a.O + R2 + 2) * kKC;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int mt = wave + kWaves * h;
+#pragma unroll
+    for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int o = 16 * mt + 4 * kb + i;
+        if (mt < MT && o < a.O) out[o * kKC + 16 * nt + mn] = aw[h][nt][i];
+      }
+#pragma unroll
+    for (int nq = 0; nq < kMaxNQ1; ++nq) {
+      const int q = 16 * nq + mn;
+      const int row = q < R ? a.O + h * R + q : a.O + R2 + h;   // column R of the product is the bias gradient
+      if (nq < NQ1 && q <= R) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) out[row * kKC + 16 * wave + 4 * kb + i] = ar[h][nq][i];
+      }
+    }
   }
 }
 
@@ -839,7 +1063,7 @@ struct ProjGeometry {
   // forward workspace
   size_t off_Wt, off_wTt, off_wLt, off_bTp, off_bLp, off_Wb, off_wTb, off_wLb, bytes_fwd;
   // backward workspace
-  size_t off_Wp, off_wTp, off_wLp, off_wTtb, off_wLtb, off_WxTb, off_dz, off_part, bytes_bwd;
+  size_t off_Wp, off_wTp, off_wLp, off_wTtb, off_wLtb, off_WxTb, off_dz, off_dpt, off_part, bytes_bwd;
 };
 
 int check_proj(const m2d_desc* d, int R) {
@@ -883,7 +1107,13 @@ ProjGeometry proj_geometry(const m2d_desc* d, int R) {
   g.off_wTtb = o; o += align256((size_t)g.Rpad * g.Epad * 2);
   g.off_wLtb = o; o += align256((size_t)g.Rpad * g.Epad * 2);
   g.off_WxTb = o; o += align256((size_t)g.Epad * g.Opad32 * 2);
-  g.off_dz = o; o += align256((size_t)g.P * g.O4 * 4);
+  if (g.mfma) {   // dz and dpre as bf16 blocks per tile
+    g.off_dz = o; o += align256((size_t)g.ntiles * kTP * g.Opad * 2);
+    g.off_dpt = o; o += align256((size_t)2 * g.ntiles * kTP * g.E * 2);
+  } else {
+    g.off_dz = o; o += align256((size_t)g.P * g.O4 * 4);
+    g.off_dpt = o;
+  }
   g.off_part = o; o += align256((size_t)g.G * g.ne * (g.O + 2 * R + 2) * kKC * 4);
   g.bytes_bwd = o;
   return g;
@@ -911,7 +1141,7 @@ bool allow_lds_weights() {
 }
 
 int run_proj_fwd_mfma(const ProjGeometry& g, const ProjArgs& a, hipStream_t st) {
-  const size_t lds = (size_t)kWaves * 2 * 16 * kLowStride * 2;
+  const size_t lds = (size_t)kWaves * (16 * kStageStride * 4 + 2 * 16 * kLowStride * 2);
   hipLaunchKernelGGL(m2d_proj_fwd_mfma_kernel, dim3(g.ntiles), dim3(kThreads), lds, st, a);
   return launched() ? M2D_OK : M2D_ERR_HIP;
 }
@@ -926,8 +1156,14 @@ int run_proj_fwd(const ProjGeometry& g, const ProjArgs& a, hipStream_t st) {
 template <typename T, bool VEC>
 int run_proj_bwd(const ProjGeometry& g, const ProjArgs& a, hipStream_t st) {
   if (g.mfma) {
-    const size_t lds_data = (size_t)kWaves * 16 * (g.Opad32 + 8) * 2;
+    const size_t lds_data = (size_t)kWaves * (16 * kStageStride * 4 + 16 * (g.Opad32 + 8) * 2);
     hipLaunchKernelGGL(m2d_proj_bwd_data_mfma_kernel, dim3(g.ntiles), dim3(kThreads), lds_data, st, a);
+    if (!launched()) return M2D_ERR_HIP;
+    const size_t lds_w = (size_t)(3 * kKC + g.Opad + 2 * 16 * ((g.R + 1 + 15) / 16)) * kPosStride * 2;
+    hipLaunchKernelGGL(m2d_proj_bwd_weights_mfma_kernel, dim3(g.G, g.ne), dim3(kThreads), lds_w, st, a);
+    if (!launched()) return M2D_ERR_HIP;
+    hipLaunchKernelGGL(m2d_proj_reduce_kernel, dim3(g.O + 2 * g.R + 2, g.ne), dim3(64 * kRedSlices), 0, st, a);
+    return launched() ? M2D_OK : M2D_ERR_HIP;
   } else {
     const size_t lds_data = (size_t)(2 * kTP * kXS + kTP * (g.O + 1)) * 4;
     hipLaunchKernelGGL((m2d_proj_bwd_data_kernel<T, VEC>), dim3(g.ntiles), dim3(kThreads), lds_data, st, a);
@@ -1030,6 +1266,8 @@ int m2d_proj_bwd(const m2d_desc* desc, int dt_rank, const void* x, const void* l
   a.Wp = k.Wp; a.wTp = k.wTp; a.wLp = k.wLp;
   a.wTtb = k.wTtb; a.wLtb = k.wLtb; a.WxTb = k.WxTb;
   a.dz = reinterpret_cast<float*>(ws + g.off_dz);
+  a.dzt = reinterpret_cast<uint16_t*>(ws + g.off_dz);
+  a.dpt = reinterpret_cast<uint16_t*>(ws + g.off_dpt);
   a.part = reinterpret_cast<float*>(ws + g.off_part);
   a.dWx = d_x_proj_w; a.dwT = d_dt_projT_w; a.dbT = d_dt_projT_b; a.dwL = d_dt_projL_w; a.dbL = d_dt_projL_b;
   if (desc->dtype == M2D_F32) return g.vec ? run_proj_bwd<float, true>(g, a, st) : run_proj_bwd<float, false>(g, a, st);
