@@ -62,6 +62,9 @@ typedef struct m2d_desc {
 } m2d_desc;
 
 #define M2D_FLAG_FLIP 1
+/* m2d_proj_fwd / m2d_proj_bwd only: round weights and biases to desc->dtype before use, which is
+ * what the reference's cast of its weights to x.dtype does (wavefront_cuda.py:327-332). */
+#define M2D_FLAG_ROUND_WEIGHTS 2
 
 #define M2D_PASS_FWD 0
 #define M2D_PASS_BWD 1
@@ -118,10 +121,9 @@ int m2d_scan_bwd(const m2d_desc* desc,
  * The reference computes the scan's parameters from x with stock operators (proj_params,
  * models/kernels/wavefront_cuda.py:63-95) and differentiates them with autograd
  * (wavefront_cuda.py:262-296).  The two calls below do the same work in hand-written kernels.
- * desc->H and desc->W only enter through the number of positions P = B*H*W; flags are ignored.
- * Activations have the element type of desc->dtype; weights, biases and their gradients are
- * fp32 (pass the values the reference would use, i.e. already rounded to the activation dtype
- * if the caller casts its weights, wavefront_cuda.py:327-332).  dt_rank <= 32, E <= 4096.
+ * desc->H and desc->W only enter through the number of positions P = B*H*W; of the flags only
+ * M2D_FLAG_ROUND_WEIGHTS is read.  Activations have the element type of desc->dtype; weights,
+ * biases and their gradients are fp32.  dt_rank <= 32, E <= 4096.
  *
  *   x_proj_w  (2*dt_rank + 3*N, E)     dt_proj{T,L}_w (E, dt_rank)     dt_proj{T,L}_b (E)
  *   lowrank   (B,H,W, 2*dt_rank)       the inputs of the two dt projections, T then L

@@ -15,6 +15,7 @@ LIB_PATH = os.environ.get("M2D_LIB") or os.path.join(_HERE, "libm2dscan.so")
 
 M2D_F32, M2D_BF16 = 0, 1
 M2D_FLAG_FLIP = 1
+M2D_FLAG_ROUND_WEIGHTS = 2
 M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
@@ -178,11 +179,13 @@ def _proj_check(x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, N):
     return R
 
 
-def proj_fwd(x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, N=16):
-    """(lowrank, deltaT, deltaL, BT, BL, C) through m2d_proj_fwd; weights are float32 tensors."""
+def proj_fwd(x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, N=16, round_weights=False):
+    """(lowrank, deltaT, deltaL, BT, BL, C) through m2d_proj_fwd; weights are float32 tensors
+    (``round_weights``: the library rounds them to x.dtype first)."""
     R = _proj_check(x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, N)
     B, H, W, E = x.shape
     d = make_desc(x, N)
+    d.flags = M2D_FLAG_ROUND_WEIGHTS if round_weights else 0
     low = x.new_empty((B, H, W, 2 * R))
     dT, dL = torch.empty_like(x), torch.empty_like(x)
     BT, BL, C = (x.new_empty((B, H, W, N)) for _ in range(3))
@@ -193,7 +196,8 @@ def proj_fwd(x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, N=16):
     return low, dT, dL, BT, BL, C
 
 
-def proj_bwd(x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w, dt_projL_w, d_deltaT, d_deltaL, d_BT, d_BL, d_C, dx):
+def proj_bwd(x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w, dt_projL_w, d_deltaT, d_deltaL, d_BT, d_BL, d_C, dx,
+             round_weights=False):
     """Adds the gradient through the projections to ``dx`` in place and returns the five weight
     gradients (x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b; float32) through m2d_proj_bwd."""
     N = d_BT.shape[-1]
@@ -208,6 +212,7 @@ def proj_bwd(x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w, dt_projL_w, d_del
         if tuple(t.shape) != shp:
             raise ValueError(f"m2dscan: {k} has shape {tuple(t.shape)}, expected {shp}")
     d = make_desc(x, N)
+    d.flags = M2D_FLAG_ROUND_WEIGHTS if round_weights else 0
     outs = [torch.empty_like(t) for t in (x_proj_w, dt_projT_w, zb, dt_projL_w, zb)]
     ws = _bytes(lib.m2d_proj_workspace_bytes(ctypes.byref(d), R, M2D_PASS_BWD), x.device)
     check(lib.m2d_proj_bwd(ctypes.byref(d), R, *[_ptr(t) for t in (x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w,

@@ -117,7 +117,7 @@ void expect_weight(const Tensor& t, const char* name, const Tensor& x, at::IntAr
   TORCH_CHECK(t.is_contiguous(), "m2dscan: ", name, " must be contiguous");
 }
 
-m2d_desc describe_proj(const Tensor& x, int64_t N) {
+m2d_desc describe_proj(const Tensor& x, int64_t N, bool round_weights) {
   TORCH_CHECK(x.dim() == 4 && x.is_cuda() && x.is_contiguous(), "m2dscan: x must be a contiguous (B,H,W,E) tensor on the GPU");
   m2d_desc d{};
   d.B = static_cast<int32_t>(x.size(0));
@@ -128,12 +128,13 @@ m2d_desc describe_proj(const Tensor& x, int64_t N) {
   if (x.scalar_type() == at::kFloat) d.dtype = M2D_F32;
   else if (x.scalar_type() == at::kBFloat16) d.dtype = M2D_BF16;
   else TORCH_CHECK(false, "m2dscan: float32 and bfloat16 are supported, got ", x.scalar_type());
+  d.flags = round_weights ? M2D_FLAG_ROUND_WEIGHTS : 0;
   return d;
 }
 
 std::vector<Tensor> proj_fwd(const Tensor& x, const Tensor& Wx, const Tensor& wT, const Tensor& bT, const Tensor& wL,
-                             const Tensor& bL, int64_t N) {
-  const m2d_desc d = describe_proj(x, N);
+                             const Tensor& bL, int64_t N, bool round_weights) {
+  const m2d_desc d = describe_proj(x, N, round_weights);
   TORCH_CHECK(wT.dim() == 2, "m2dscan: dt_projT_w must be (E, dt_rank)");
   const int64_t B = d.B, H = d.H, W = d.W, E = d.E, R = wT.size(1);
   expect_weight(Wx, "x_proj_w", x, {2 * R + 3 * N, E});
@@ -157,10 +158,10 @@ std::vector<Tensor> proj_fwd(const Tensor& x, const Tensor& Wx, const Tensor& wT
 
 std::vector<Tensor> proj_bwd(const Tensor& x, const Tensor& low, const Tensor& dT, const Tensor& dL, const Tensor& Wx,
                              const Tensor& wT, const Tensor& wL, const Tensor& ddT, const Tensor& ddL, const Tensor& dBT,
-                             const Tensor& dBL, const Tensor& dC, Tensor dx) {
+                             const Tensor& dBL, const Tensor& dC, Tensor dx, bool round_weights) {
   TORCH_CHECK(dBT.dim() == 4 && wT.dim() == 2, "m2dscan: d_BT must be (B,H,W,N) and dt_projT_w (E, dt_rank)");
   const int64_t N = dBT.size(3);
-  const m2d_desc d = describe_proj(x, N);
+  const m2d_desc d = describe_proj(x, N, round_weights);
   const int64_t B = d.B, H = d.H, W = d.W, E = d.E, R = wT.size(1);
   expect_weight(Wx, "x_proj_w", x, {2 * R + 3 * N, E});
   expect_weight(wT, "dt_projT_w", x, {E, R});
@@ -199,9 +200,10 @@ TORCH_LIBRARY(m2dscan, m) {
   m.def("scan_bwd(Tensor x, Tensor deltaT, Tensor deltaL, Tensor AT, Tensor AL, Tensor BT, Tensor BL, Tensor C, "
         "Tensor D, Tensor dy, Tensor ckpt, bool flip) -> Tensor[]");
   m.def("proj_fwd(Tensor x, Tensor x_proj_w, Tensor dt_projT_w, Tensor dt_projT_b, Tensor dt_projL_w, Tensor dt_projL_b, "
-        "int d_state) -> Tensor[]");
+        "int d_state, bool round_weights) -> Tensor[]");
   m.def("proj_bwd(Tensor x, Tensor lowrank, Tensor deltaT, Tensor deltaL, Tensor x_proj_w, Tensor dt_projT_w, "
-        "Tensor dt_projL_w, Tensor d_deltaT, Tensor d_deltaL, Tensor d_BT, Tensor d_BL, Tensor d_C, Tensor(a!) dx) -> Tensor[]");
+        "Tensor dt_projL_w, Tensor d_deltaT, Tensor d_deltaL, Tensor d_BT, Tensor d_BL, Tensor d_C, Tensor(a!) dx, "
+        "bool round_weights) -> Tensor[]");
   m.def("abi_version() -> int", &abi_version);
 }
 

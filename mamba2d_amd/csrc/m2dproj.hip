@@ -108,10 +108,20 @@ struct PackArgs {
   uint16_t *Wb, *wTb, *wLb;              // forward set of the matrix-core kernels (or null)
   uint16_t *wTtb, *wLtb, *WxTb;          // backward set of the matrix-core kernels (or null)
   int E, R, O, Epad, Opad, Opad32, Rpad;
+  int round;                             // round every weight to bf16 first
 };
 
 // Padded copies of the weights.  One thread per element of the largest copy.
-__global__ void m2d_proj_pack_kernel(const PackArgs k) {
+__global__ void m2d_proj_pack_kernel(const PackArgs k0) {
+  struct Rounded {   // the weight arrays as the kernels are to see them
+    const float* p; bool round;
+    __device__ float operator[](int i) const { return round ? as_stored(p[i], static_cast<const bf16_t*>(nullptr)) : p[i]; }
+  };
+  struct { Rounded Wx, wT, bT, wL, bL; float *Wt, *wTt, *wLt, *bTp, *bLp, *Wp, *wTp, *wLp; uint16_t *Wb, *wTb, *wLb, *wTtb, *wLtb, *WxTb;
+           int E, R, O, Epad, Opad, Opad32, Rpad; } k = {
+      {k0.Wx, k0.round != 0}, {k0.wT, k0.round != 0}, {k0.bT, k0.round != 0}, {k0.wL, k0.round != 0}, {k0.bL, k0.round != 0},
+      k0.Wt, k0.wTt, k0.wLt, k0.bTp, k0.bLp, k0.Wp, k0.wTp, k0.wLp, k0.Wb, k0.wTb, k0.wLb, k0.wTtb, k0.wLtb, k0.WxTb,
+      k0.E, k0.R, k0.O, k0.Epad, k0.Opad, k0.Opad32, k0.Rpad};
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (k.Wt) {
     if (i < k.Epad * k.Opad) {
@@ -1070,6 +1080,7 @@ int check_proj(const m2d_desc* d, int R) {
   if (!d) return M2D_ERR_NULL_POINTER;
   if (d->B < 1 || d->H < 1 || d->W < 1 || d->E < 1 || d->N < 1 || R < 1) return M2D_ERR_BAD_SHAPE;
   if (d->N != kN || (d->dtype != M2D_F32 && d->dtype != M2D_BF16) || d->reserved != 0) return M2D_ERR_UNSUPPORTED;
+  if (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_ROUND_WEIGHTS)) return M2D_ERR_UNSUPPORTED;
   if (R > kMaxR || d->E > 4096) return M2D_ERR_UNSUPPORTED;
   if ((int64_t)d->B * d->H * d->W >= ((int64_t)1 << 31) * kTP) return M2D_ERR_UNSUPPORTED;   // tiles counted in 32 bits
   return M2D_OK;
@@ -1215,6 +1226,7 @@ int m2d_proj_fwd(const m2d_desc* desc, int dt_rank, const void* x, const float* 
     k.wLb = reinterpret_cast<uint16_t*>(ws + g.off_wLb);
   }
   k.E = g.E; k.R = g.R; k.O = g.O; k.Epad = g.Epad; k.Opad = g.Opad; k.Opad32 = g.Opad32; k.Rpad = g.Rpad;
+  k.round = (desc->flags & M2D_FLAG_ROUND_WEIGHTS) && desc->dtype == M2D_BF16;
   const int n = g.Epad * (g.Opad > 32 ? g.Opad : 32);   // the largest forward copy
   hipLaunchKernelGGL(m2d_proj_pack_kernel, dim3((n + 255) / 256), dim3(256), 0, st, k);
   if (!launched()) return M2D_ERR_HIP;
@@ -1255,6 +1267,7 @@ int m2d_proj_bwd(const m2d_desc* desc, int dt_rank, const void* x, const void* l
     k.WxTb = reinterpret_cast<uint16_t*>(ws + g.off_WxTb);
   }
   k.E = g.E; k.R = g.R; k.O = g.O; k.Epad = g.Epad; k.Opad = g.Opad; k.Opad32 = g.Opad32; k.Rpad = g.Rpad;
+  k.round = (desc->flags & M2D_FLAG_ROUND_WEIGHTS) && desc->dtype == M2D_BF16;
   int n = g.Opad32 * g.Epad;
   if (g.Epad * g.Rpad > n) n = g.Epad * g.Rpad;
   hipLaunchKernelGGL(m2d_proj_pack_kernel, dim3((n + 255) / 256), dim3(256), 0, st, k);

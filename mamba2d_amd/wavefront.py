@@ -64,7 +64,7 @@ def _scan_bwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt, flip):
 
 
 @torch.library.register_fake("m2dscan::proj_fwd")
-def _proj_fwd_fake(x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, d_state):
+def _proj_fwd_fake(x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, d_state, round_weights):
     B, H, W, _ = x.shape
     R = dt_projT_w.shape[1]
     bc = [x.new_empty((B, H, W, d_state)) for _ in range(3)]
@@ -72,7 +72,8 @@ def _proj_fwd_fake(x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, 
 
 
 @torch.library.register_fake("m2dscan::proj_bwd")
-def _proj_bwd_fake(x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w, dt_projL_w, d_deltaT, d_deltaL, d_BT, d_BL, d_C, dx):
+def _proj_bwd_fake(x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w, dt_projL_w, d_deltaT, d_deltaL, d_BT, d_BL, d_C, dx,
+                   round_weights):
     b = dt_projT_w.new_empty((x.shape[-1],))
     return [torch.empty_like(x_proj_w), torch.empty_like(dt_projT_w), b, torch.empty_like(dt_projL_w), torch.empty_like(b)]
 
@@ -162,30 +163,32 @@ def _proj_kernels_cover(x, AT_log, dt_projT_w) -> bool:
 class wf_cuda_fn_proj(torch.autograd.Function):
     """Projections and scan behind one Function, all in the library's own kernels.
 
-    Same function of the nine raw inputs as ``proj_params`` followed by ``wf_cuda_fn_pr``
-    (reference ``wavefront_cuda.py:63-95``, ``:146-196``) or as ``wf_cuda_fn_fr`` (``:199-313``).
-    ``full=False`` keeps the projection outputs and the scan's checkpoints for the backward;
-    ``full=True`` keeps only x and the weights and rebuilds the rest in the backward."""
+    Same function of the nine raw inputs as the reference's entry point: the projection weights
+    are rounded to ``x.dtype`` (``wavefront_cuda.py:327-332``; here inside the kernels that pack
+    them), then ``proj_params`` and ``wf_cuda_fn_pr`` (``:63-95``, ``:146-196``) or ``wf_cuda_fn_fr``
+    (``:199-313``).  ``full=False`` keeps the projection outputs and the scan's checkpoints for the
+    backward; ``full=True`` keeps only x and the weights and rebuilds the rest in the backward."""
 
     @staticmethod
     def _project(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b):
         w32 = [_c(t.float()) for t in (x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b)]
-        AT = (-torch.exp(AT_log.float())).to(x.dtype)
-        AL = (-torch.exp(AL_log.float())).to(x.dtype)
-        return w32, AT, AL, proj_fwd_op(x, *w32, AT_log.shape[1])
+        A32 = -torch.exp(torch.stack((AT_log.float(), AL_log.float())))   # both directions at once
+        A = A32.to(x.dtype)
+        return w32, A32, A, proj_fwd_op(x, *w32, AT_log.shape[1], True)
 
     @staticmethod
     def forward(ctx, x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D,
                 full=False, flip=False):
-        x, D = _c(x), _c(D)
+        x = _c(x)
+        Dx = _c(D.to(x.dtype))
         weights = (AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b)
-        _, AT, AL, (low, dT, dL, BT, BL, C) = wf_cuda_fn_proj._project(x, *weights)
+        _, A32, A, (low, dT, dL, BT, BL, C) = wf_cuda_fn_proj._project(x, *weights)
         keep = SAVE_CHECKPOINTS and not full and any(ctx.needs_input_grad)
-        y, ck = scan_fwd_op(x, dT, dL, AT, AL, BT, BL, C, D, keep, bool(flip))
+        y, ck = scan_fwd_op(x, dT, dL, A[0], A[1], BT, BL, C, Dx, keep, bool(flip))
         if full:
             ctx.save_for_backward(x, *weights, D)
         else:
-            ctx.save_for_backward(x, *weights, D, low, dT, dL, BT, BL, C, ck)
+            ctx.save_for_backward(x, *weights, D, A32, A, low, dT, dL, BT, BL, C, ck)
         ctx.full, ctx.flip = bool(full), bool(flip)
         return y
 
@@ -195,21 +198,21 @@ class wf_cuda_fn_proj(torch.autograd.Function):
         AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b = weights
         dy = _c(grad_output.to(x.dtype))
         if ctx.full:
-            w32, AT, AL, (low, dT, dL, BT, BL, C) = wf_cuda_fn_proj._project(x, *weights)
+            w32, A32, A, (low, dT, dL, BT, BL, C) = wf_cuda_fn_proj._project(x, *weights)
             ck = x.new_empty((1,), dtype=torch.uint8)
         else:
-            low, dT, dL, BT, BL, C, ck = ctx.saved_tensors[9:]
+            A32, A, low, dT, dL, BT, BL, C, ck = ctx.saved_tensors[9:]
             w32 = [_c(t.float()) for t in (x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b)]
-            AT = (-torch.exp(AT_log.float())).to(x.dtype)
-            AL = (-torch.exp(AL_log.float())).to(x.dtype)
-        d_x, d_dT, d_dL, d_AT, d_AL, d_BT, d_BL, d_C, d_D = scan_bwd_op(x, dT, dL, AT, AL, BT, BL, C, D, dy, ck, ctx.flip)
+        d_x, d_dT, d_dL, d_AT, d_AL, d_BT, d_BL, d_C, d_D = scan_bwd_op(
+            x, dT, dL, A[0], A[1], BT, BL, C, _c(D.to(x.dtype)), dy, ck, ctx.flip)
         # d_x holds the scan's own gradient (dy*D included); the projections add theirs in place
-        g_xw, g_wT, g_bT, g_wL, g_bL = proj_bwd_op(x, low, dT, dL, w32[0], w32[1], w32[3], d_dT, d_dL, d_BT, d_BL, d_C, d_x)
+        g_xw, g_wT, g_bT, g_wL, g_bL = proj_bwd_op(x, low, dT, dL, w32[0], w32[1], w32[3], d_dT, d_dL, d_BT, d_BL, d_C, d_x,
+                                                   True)
         # A = -exp(A_log): dA/dA_log = A
-        d_AT_log = (d_AT.float() * -torch.exp(AT_log.float())).to(AT_log.dtype)
-        d_AL_log = (d_AL.float() * -torch.exp(AL_log.float())).to(AL_log.dtype)
-        return (d_x, d_AT_log, d_AL_log, g_xw.to(x_proj_w.dtype), g_wT.to(dt_projT_w.dtype), g_bT.to(dt_projT_b.dtype),
-                g_wL.to(dt_projL_w.dtype), g_bL.to(dt_projL_b.dtype), d_D, None, None)
+        d_A_log = torch.stack((d_AT, d_AL)).float() * A32
+        return (d_x, d_A_log[0].to(AT_log.dtype), d_A_log[1].to(AL_log.dtype), g_xw.to(x_proj_w.dtype),
+                g_wT.to(dt_projT_w.dtype), g_bT.to(dt_projT_b.dtype), g_wL.to(dt_projL_w.dtype), g_bL.to(dt_projL_b.dtype),
+                d_D.to(D.dtype), None, None)
 
 
 def wavefront_scan_cuda(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D,
@@ -224,18 +227,19 @@ def wavefront_scan_cuda(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_
     if H < 2 or W < 2:
         raise ValueError(f"Wavefront scan kernel requires spatial dims > 1. Got H={H}, W={W}.")
 
+    if recomp not in ("partial", "full"):
+        raise ValueError(f"Unknown recomputation mode, got {recomp}...")
+    if FUSED_PROJECTIONS and _proj_kernels_cover(x, AT_log, dt_projT_w):
+        # the casts of the weights to x.dtype happen inside (no copies of the parameters)
+        return wf_cuda_fn_proj.apply(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D,
+                                     recomp == "full", flip)
+
     x_proj_w = x_proj_w.to(x.dtype)
     dt_projT_w = dt_projT_w.to(x.dtype)
     dt_projT_b = dt_projT_b.to(x.dtype)
     dt_projL_w = dt_projL_w.to(x.dtype)
     dt_projL_b = dt_projL_b.to(x.dtype)
     D = D.to(x.dtype)
-
-    if recomp not in ("partial", "full"):
-        raise ValueError(f"Unknown recomputation mode, got {recomp}...")
-    if FUSED_PROJECTIONS and _proj_kernels_cover(x, AT_log, dt_projT_w):
-        return wf_cuda_fn_proj.apply(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D,
-                                     recomp == "full", flip)
     if recomp == "partial":
         deltaT, deltaL, AT, AL, BT, BL, C = proj_params(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b,
                                                         dt_projL_w, dt_projL_b)

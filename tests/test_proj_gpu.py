@@ -39,11 +39,12 @@ def make_case(B, H, W, E, seed, dtype):
         dt_projT_b=dt + torch.log(-torch.expm1(-dt)),
         dt_projL_w=(torch.rand(E, R, generator=g) * 2 - 1) * R ** -0.5,
         dt_projL_b=(dt + torch.log(-torch.expm1(-dt))).flip(0).contiguous())
+    raw = dict(w)
     w = {k: v.to(dtype).float() for k, v in w.items()}
     x = torch.randn(B, H, W, E, generator=g).to(dtype)
     up = {k: torch.randn(B, H, W, n, generator=g).to(dtype)
           for k, n in (("d_deltaT", E), ("d_deltaL", E), ("d_BT", N), ("d_BL", N), ("d_C", N), ("dx", E))}
-    return R, x, w, up
+    return R, x, w, up, raw
 
 
 WNAMES = ("x_proj_w", "dt_projT_w", "dt_projT_b", "dt_projL_w", "dt_projL_b")
@@ -75,7 +76,7 @@ def reference(x, w, up, R):
 def test_projections_match_reference(cabi, shape, dtype, tol):
     say(f"\ncase proj {shape} {dtype}")
     B, H, W, E = shape
-    R, x, w, up = make_case(B, H, W, E, seed=sum(shape), dtype=dtype)
+    R, x, w, up, _ = make_case(B, H, W, E, seed=sum(shape), dtype=dtype)
     ref_out, ref_g = reference(x, w, up, R)
     xd = x.cuda()
     wd = {k: v.cuda() for k, v in w.items()}
@@ -96,6 +97,30 @@ def test_projections_match_reference(cabi, shape, dtype, tol):
     for k, g in zip(WNAMES, gw):
         assert g.dtype == torch.float32 and g.shape == ref_g[k].shape
         assert so.rel_err(g.cpu(), ref_g[k]) < tol, k
+
+
+@pytest.mark.parametrize("shape", [(2, 14, 14, 64), (1, 40, 4, 100)], ids=lambda s: "x".join(map(str, s)))
+def test_library_rounds_weights_like_a_cast(cabi, shape):
+    """M2D_FLAG_ROUND_WEIGHTS on fp32 weights gives bit for bit what weights cast to bf16 beforehand give."""
+    say(f"\ncase proj round_weights {shape}")
+    B, H, W, E = shape
+    R, x, w, up, raw = make_case(B, H, W, E, seed=7, dtype=torch.bfloat16)
+    xd = x.cuda()
+    wd = {k: v.cuda() for k, v in w.items()}
+    rd = {k: v.cuda() for k, v in raw.items()}
+    assert any(not torch.equal(wd[k], rd[k]) for k in WNAMES)
+    a = cabi.proj_fwd(xd, *[wd[k] for k in WNAMES], N)
+    b = cabi.proj_fwd(xd, *[rd[k] for k in WNAMES], N, round_weights=True)
+    for u, v in zip(a, b):
+        assert torch.equal(u, v)
+    upd = {k: v.cuda() for k, v in up.items()}
+    dxa, dxb = upd["dx"].clone(), upd["dx"].clone()
+    args = (upd["d_deltaT"], upd["d_deltaL"], upd["d_BT"], upd["d_BL"], upd["d_C"])
+    ga = cabi.proj_bwd(xd, a[0], a[1], a[2], wd["x_proj_w"], wd["dt_projT_w"], wd["dt_projL_w"], *args, dxa)
+    gb = cabi.proj_bwd(xd, a[0], a[1], a[2], rd["x_proj_w"], rd["dt_projT_w"], rd["dt_projL_w"], *args, dxb, round_weights=True)
+    assert torch.equal(dxa, dxb)
+    for u, v in zip(ga, gb):
+        assert torch.equal(u, v)
 
 
 def test_projection_limits_are_reported(cabi):
