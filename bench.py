@@ -36,6 +36,7 @@ WORKLOADS = {
     "hires2048": (1, 64, 2048, 2048, "f32"),
     "cfg0": (2, 32, 14, 14, "f32"),
     "cfg3": None,   # M2D-T backbone inference, handled by backbone_inference()
+    "entry": None,  # wavefront_scan_cuda (projections + scan) at the cfg1 shape, handled by entry_point()
 }
 N = 16
 HBM_PEAK_GBS = 8000.0
@@ -136,6 +137,90 @@ def backbone_inference(args):
     print(json.dumps(out))
 
 
+def entry_point(args):
+    """The reference's entry point, wavefront_scan_cuda(x, A_logs, projection weights, D): projections
+    (x_proj, two dt_proj + softplus), scan, and the backward of both, at the cfg1 shape with fp32
+    parameters initialised like an M2D block and bf16 activations.  One step = forward + backward."""
+    import math
+    import torch
+    from mamba2d_amd import cabi, wavefront as wf
+    dev = torch.device("cuda:0")
+    B, E, H, W = WORKLOADS["cfg1"][:4]
+    R = math.ceil(E / 16)
+    g = torch.Generator().manual_seed(0)
+    dt = torch.exp(torch.rand(E, generator=g) * (math.log(0.1) - math.log(0.001)) + math.log(0.001)).clamp(min=1e-4)
+    inv_dt = dt + torch.log(-torch.expm1(-dt))
+    params = [
+        torch.log(torch.arange(1, N + 1, dtype=torch.float32).repeat(E, 1)),          # AT_log
+        torch.log(torch.arange(1, N + 1, dtype=torch.float32).repeat(E, 1)),          # AL_log
+        (torch.rand(2 * R + 3 * N, E, generator=g) * 2 - 1) / math.sqrt(E),           # x_proj_w
+        (torch.rand(E, R, generator=g) * 2 - 1) * R ** -0.5, inv_dt.clone(),          # dt_projT w, b
+        (torch.rand(E, R, generator=g) * 2 - 1) * R ** -0.5, inv_dt.clone(),          # dt_projL w, b
+        torch.ones(E)]                                                                # D
+    params = [p.to(dev).requires_grad_(True) for p in params]
+    x = torch.randn(B, H, W, E, generator=g).to(torch.bfloat16).to(dev).requires_grad_(True)
+    dy = torch.randn(B, H, W, E, generator=g).to(torch.bfloat16).to(dev)
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps
+
+    def fwd_bwd(recomp):
+        y = wf.wavefront_scan_cuda(x, *params, recomp)
+        torch.autograd.grad(y, [x] + params, dy)
+
+    def fwd_only():
+        with torch.no_grad():
+            wf.wavefront_scan_cuda(x, *params)
+
+    res = {}
+    for own in (True, False):
+        wf.FUSED_PROJECTIONS = own
+        key = "own" if own else "torch"
+        res[key] = {"fwd_ms": round(timed(fwd_only), 4), "fwd_bwd_ms": round(timed(lambda: fwd_bwd("partial")), 4),
+                    "fwd_bwd_full_recompute_ms": round(timed(lambda: fwd_bwd("full")), 4)}
+    wf.FUSED_PROJECTIONS = True
+
+    # the projection passes alone, through the C ABI (they run on torch's current stream)
+    w32 = [p.detach() for p in params[2:7]]
+    xd = x.detach()
+    outs = cabi.proj_fwd(xd, *w32, N, round_weights=True)
+    ups = [torch.randn_like(t) for t in (outs[1], outs[2], outs[3], outs[4], outs[5])]
+    dx = torch.zeros_like(xd)
+    proj_fwd_ms = timed(lambda: cabi.proj_fwd(xd, *w32, N, round_weights=True))
+    proj_bwd_ms = timed(lambda: cabi.proj_bwd(xd, outs[0], outs[1], outs[2], w32[0], w32[1], w32[3], *ups, dx,
+                                              round_weights=True))
+    P, s = B * H * W, 2
+    nw = (2 * R + 3 * N) * E + 2 * E * R + 2 * E
+    proj_fwd_bytes = s * P * (E + 2 * R + 2 * E + 3 * N) + 4 * nw
+    proj_bwd_bytes = s * P * (E + 2 * R + 4 * E + 3 * N + 2 * E) + 8 * nw
+    out = {
+        "metric": "wavefront_scan_cuda (projections + scan) fwd+bwd ms at B=128 D=64 56x56 N=16",
+        "value": res["own"]["fwd_bwd_ms"], "unit": "ms",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": res["own"]["fwd_bwd_ms"],
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16 activations, f32 parameters and state", "data": "synthetic",
+        "config": {"workload": "entry: wavefront_scan_cuda fwd+bwd, B=128 E=64 56x56 N=16 dt_rank=4, recomp=partial"},
+        "own_projection_kernels": res["own"], "stock_torch_projections": res["torch"],
+        "projection_passes": {
+            "fwd_ms": round(proj_fwd_ms, 4), "bwd_ms": round(proj_bwd_ms, 4),
+            "fwd_algorithmic_bytes": proj_fwd_bytes, "bwd_algorithmic_bytes": proj_bwd_bytes,
+            "fwd_frac_of_hbm_peak": round(proj_fwd_bytes / (proj_fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+            "bwd_frac_of_hbm_peak": round(proj_bwd_bytes / (proj_bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
+        "roofline": None, "cpu_baseline": None,
+    }
+    print(json.dumps(out))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -161,6 +246,9 @@ def main():
 
     if args.workload == "cfg3":
         backbone_inference(args)
+        return
+    if args.workload == "entry":
+        entry_point(args)
         return
     B, E, H, W, dts = WORKLOADS[args.workload]
     dtype = torch.bfloat16 if dts == "bf16" else torch.float32

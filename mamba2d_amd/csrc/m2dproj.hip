@@ -497,7 +497,7 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi) {
 
 // Results leave the accumulators (4 positions x 1 channel per lane and tile) through a per-wave
 // LDS block of 16 positions x 64 channels, so that memory sees 16-byte pieces of rows.
-constexpr int kStageStride = 68;   // floats per row: 64 + 4, rows 16-byte aligned
+constexpr int kStageStride = 72;   // floats per row: 64 + 8, rows 16-byte aligned (also holds 2 x [16][72] bf16)
 __device__ __forceinline__ void wave_sync_lds() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -665,9 +665,22 @@ __global__ __launch_bounds__(kThreads, M2D_PROJ_OCC) void m2d_proj_bwd_data_mfma
         accT[nq] = mfma16(AT, load16(a.wTtb + (16 * nq + mn) * a.Epad + e), accT[nq]);
         accL[nq] = mfma16(AL, load16(a.wLtb + (16 * nq + mn) * a.Epad + e), accL[nq]);
       }
-    if (e < a.E) {
-      *reinterpret_cast<uint4*>(dptT + (uint32_t)(mn * a.E + e)) = AT;
-      *reinterpret_cast<uint4*>(dptL + (uint32_t)(mn * a.E + e)) = AL;
+    // dpre leaves through LDS, 64 channels at a time, so that memory sees whole 128-byte rows
+    uint16_t* pst = reinterpret_cast<uint16_t*>(stage);
+    *reinterpret_cast<uint4*>(pst + mn * kStageStride + (e & 63)) = AT;
+    *reinterpret_cast<uint4*>(pst + (16 + mn) * kStageStride + (e & 63)) = AL;
+    if ((e & 32) != 0) {   // uniform: second half of a group of 64
+      const int e0 = e & ~63;
+      wave_sync_lds();
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        const int piece = l + 64 * k, c = piece >> 3, c8 = 8 * (piece & 7);
+        if (e0 + c8 < a.E) {
+          *reinterpret_cast<uint4*>(dptT + (uint32_t)(c * a.E + e0 + c8)) = load16(pst + c * kStageStride + c8);
+          *reinterpret_cast<uint4*>(dptL + (uint32_t)(c * a.E + e0 + c8)) = load16(pst + (16 + c) * kStageStride + c8);
+        }
+      }
+      wave_sync_lds();
     }
   }
   // rows of dz to LDS as bf16: operand of the next product, and source of the copy in memory
