@@ -62,12 +62,8 @@ typedef float v4f_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) v4f_t lds_float4;   // a float4 known to live in LDS
 
 __device__ __forceinline__ float bf16_bits_to_f32(uint32_t lo16) { return __uint_as_float(lo16 << 16); }
-__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x40u);  // NaN
-  u += 0x7fffu + ((u >> 16) & 1u);                                            // round to nearest even
-  return (uint16_t)(u >> 16);
-}
+// round to nearest even; one instruction on gfx950 (v_cvt_pk_bf16_f32)
+__device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
 
 template <typename T> struct IO;
 template <> struct IO<float> {
