@@ -1,0 +1,44 @@
+"""The four operators of the shim trace without a device: their fake implementations (what
+torch.compile sees, like the reference's register_fake no-ops at wavefront_cuda.py:33-57) return
+outputs of the right shapes and dtypes for meta tensors."""
+import math
+
+import pytest
+import torch
+
+
+@pytest.fixture(scope="module")
+def wf():
+    from mamba2d_amd import wavefront
+    return wavefront
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_scan_ops_on_meta_tensors(wf, dtype):
+    B, H, W, E, N = 2, 5, 7, 8, 16
+    m = lambda *s: torch.empty(*s, dtype=dtype, device="meta")
+    args = [m(B, H, W, E), m(B, H, W, E), m(B, H, W, E), m(E, N), m(E, N), m(B, H, W, N), m(B, H, W, N), m(B, H, W, N), m(E)]
+    y, ck = wf.scan_fwd_op(*args, True, False)
+    assert y.shape == (B, H, W, E) and y.dtype == dtype and y.device.type == "meta"
+    assert ck.dtype == torch.uint8 and ck.numel() > 1
+    y2, ck2 = wf.scan_fwd_op(*args, False, True)
+    assert ck2.numel() == 1
+    grads = wf.scan_bwd_op(*args, m(B, H, W, E), ck, False)
+    assert [tuple(g.shape) for g in grads] == [tuple(a.shape) for a in args]
+    assert all(g.dtype == dtype for g in grads)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_projection_ops_on_meta_tensors(wf, dtype):
+    B, H, W, E, N = 2, 5, 7, 40, 16
+    R = math.ceil(E / 16)
+    x = torch.empty(B, H, W, E, dtype=dtype, device="meta")
+    f = lambda *s: torch.empty(*s, dtype=torch.float32, device="meta")
+    w = [f(2 * R + 3 * N, E), f(E, R), f(E), f(E, R), f(E)]
+    low, dT, dL, BT, BL, C = wf.proj_fwd_op(x, *w, N, True)
+    assert low.shape == (B, H, W, 2 * R) and dT.shape == dL.shape == x.shape
+    assert BT.shape == BL.shape == C.shape == (B, H, W, N)
+    assert all(t.dtype == dtype for t in (low, dT, dL, BT, BL, C))
+    g = wf.proj_bwd_op(x, low, dT, dL, w[0], w[1], w[3], dT, dL, BT, BL, C, torch.empty_like(x), True)
+    assert [tuple(t.shape) for t in g] == [tuple(t.shape) for t in w]
+    assert all(t.dtype == torch.float32 for t in g)
