@@ -94,7 +94,10 @@ def proj_params(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w,
 
 
 def _c(t):
-    return t if t.is_contiguous() else t.contiguous()
+    """Contiguous and 16-byte aligned (a contiguous view into a larger buffer may start anywhere)."""
+    if not t.is_contiguous():
+        return t.contiguous()
+    return t if t.data_ptr() % 16 == 0 else t.clone()
 
 
 class wf_cuda_fn_pr(torch.autograd.Function):

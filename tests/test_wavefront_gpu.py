@@ -110,6 +110,20 @@ def test_partial_and_full_agree_bf16(wf, projections):
         assert a.dtype == b.dtype and so.rel_err(a.float().cpu(), b.float().cpu()) < 2e-2
 
 
+def test_views_that_start_off_alignment_are_accepted(wf, cscan):
+    """A contiguous view whose first element is not 16-byte aligned is copied, not rejected."""
+    say("\ncase unaligned views")
+    inp = so.make_inputs(1, 6, 5, 3, 16, seed=2, dtype=torch.float32)
+    a = []
+    for k in so.INPUT_NAMES:
+        big = torch.zeros(inp[k].numel() + 1, device="cuda")
+        big[1:] = inp[k].flatten().cuda()
+        a.append(big[1:].view(inp[k].shape))
+    assert any(t.data_ptr() % 16 for t in a)
+    y = wf.wf_cuda_fn_pr.apply(*a)
+    assert so.rel_err(y.cpu(), cscan.forward(*[inp[k].double() for k in so.INPUT_NAMES])) < 1e-4
+
+
 def test_small_spatial_dims_raise_on_gpu(wf):
     p = make_block_params(4, 16, 1, 0, "cuda")
     with pytest.raises(ValueError, match="spatial dims > 1"):
