@@ -63,7 +63,9 @@ typedef struct m2d_desc {
 
 #define M2D_FLAG_FLIP 1
 /* m2d_proj_fwd / m2d_proj_bwd only: round weights and biases to desc->dtype before use, which is
- * what the reference's cast of its weights to x.dtype does (wavefront_cuda.py:327-332). */
+ * what the reference's cast of its weights to x.dtype does (wavefront_cuda.py:327-332).  Without
+ * the flag bf16 activations still meet bf16-rounded weight matrices (not biases) wherever the
+ * products run on the matrix cores (channel counts that are a multiple of 8). */
 #define M2D_FLAG_ROUND_WEIGHTS 2
 
 #define M2D_PASS_FWD 0

@@ -108,35 +108,28 @@ struct PackArgs {
   uint16_t *Wb, *wTb, *wLb;              // forward set of the matrix-core kernels (or null)
   uint16_t *wTtb, *wLtb, *WxTb;          // backward set of the matrix-core kernels (or null)
   int E, R, O, Epad, Opad, Opad32, Rpad;
-  int round;                             // round every weight to bf16 first
+  int round;                             // round every weight to bf16 first (the bf16 copies are rounded anyway)
 };
 
 // Padded copies of the weights.  One thread per element of the largest copy.
-__global__ void m2d_proj_pack_kernel(const PackArgs k0) {
-  struct Rounded {   // the weight arrays as the kernels are to see them
-    const float* p; bool round;
-    __device__ float operator[](int i) const { return round ? as_stored(p[i], static_cast<const bf16_t*>(nullptr)) : p[i]; }
-  };
-  struct { Rounded Wx, wT, bT, wL, bL; float *Wt, *wTt, *wLt, *bTp, *bLp, *Wp, *wTp, *wLp; uint16_t *Wb, *wTb, *wLb, *wTtb, *wLtb, *WxTb;
-           int E, R, O, Epad, Opad, Opad32, Rpad; } k = {
-      {k0.Wx, k0.round != 0}, {k0.wT, k0.round != 0}, {k0.bT, k0.round != 0}, {k0.wL, k0.round != 0}, {k0.bL, k0.round != 0},
-      k0.Wt, k0.wTt, k0.wLt, k0.bTp, k0.bLp, k0.Wp, k0.wTp, k0.wLp, k0.Wb, k0.wTb, k0.wLb, k0.wTtb, k0.wLtb, k0.WxTb,
-      k0.E, k0.R, k0.O, k0.Epad, k0.Opad, k0.Opad32, k0.Rpad};
+__global__ void m2d_proj_pack_kernel(const PackArgs k) {
+  // a weight as the kernels are to see it
+  auto w = [&](const float* p, int i) { return k.round ? as_stored(p[i], static_cast<const bf16_t*>(nullptr)) : p[i]; };
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (k.Wt) {
     if (i < k.Epad * k.Opad) {
       const int e = i / k.Opad, o = i - e * k.Opad;
-      k.Wt[i] = (e < k.E && o < k.O) ? k.Wx[o * k.E + e] : 0.f;
+      k.Wt[i] = (e < k.E && o < k.O) ? w(k.Wx, o * k.E + e) : 0.f;
     }
     if (i < k.R * k.Epad) {
       const int q = i / k.Epad, e = i - q * k.Epad;
-      k.wTt[i] = e < k.E ? k.wT[e * k.R + q] : 0.f;
-      k.wLt[i] = e < k.E ? k.wL[e * k.R + q] : 0.f;
+      k.wTt[i] = e < k.E ? w(k.wT, e * k.R + q) : 0.f;
+      k.wLt[i] = e < k.E ? w(k.wL, e * k.R + q) : 0.f;
     }
   }
   if (k.bTp && i < k.Epad) {
-    k.bTp[i] = i < k.E ? k.bT[i] : 0.f;
-    k.bLp[i] = i < k.E ? k.bL[i] : 0.f;
+    k.bTp[i] = i < k.E ? w(k.bT, i) : 0.f;
+    k.bLp[i] = i < k.E ? w(k.bL, i) : 0.f;
   }
   if (k.Wb) {
     if (i < k.Opad * k.Epad) {
@@ -165,13 +158,13 @@ __global__ void m2d_proj_pack_kernel(const PackArgs k0) {
   if (k.Wp) {
     if (i < k.O * k.Epad) {
       const int o = i / k.Epad, e = i - o * k.Epad;
-      k.Wp[i] = e < k.E ? k.Wx[o * k.E + e] : 0.f;
+      k.Wp[i] = e < k.E ? w(k.Wx, o * k.E + e) : 0.f;
     }
     if (i < k.Epad * k.Rpad) {
       const int e = i / k.Rpad, q = i - e * k.Rpad;
       const bool ok = e < k.E && q < k.R;
-      k.wTp[i] = ok ? k.wT[e * k.R + q] : 0.f;
-      k.wLp[i] = ok ? k.wL[e * k.R + q] : 0.f;
+      k.wTp[i] = ok ? w(k.wT, e * k.R + q) : 0.f;
+      k.wLp[i] = ok ? w(k.wL, e * k.R + q) : 0.f;
     }
   }
 }
