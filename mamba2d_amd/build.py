@@ -8,9 +8,12 @@ package loads what has been built and fails loudly when it is missing.
 """
 from __future__ import annotations
 
+import glob
 import os
+import shutil
 import subprocess
 import sys
+import tempfile
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
@@ -26,11 +29,33 @@ HIPCC_FLAGS = [
 
 
 def build_lib(verbose: bool = True) -> str:
+    """Compiles the two HIP sources into libm2dscan.so.  The device assembly of the same compile is
+    kept (-save-temps) and checked for the hazards that inline assembly hides from the compiler
+    (asmcheck.py); the library is only put in place if the check passes."""
+    from . import asmcheck
     srcs = [os.path.join(HERE, "csrc", n) for n in ("m2dscan.hip", "m2dproj.hip")]
-    cmd = ["hipcc", *HIPCC_FLAGS, "-I", os.path.join(ROOT, "include"), "-o", LIB, *srcs]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.check_call(cmd)
+    scratch = os.path.join(HERE, "build")   # in-tree, ignored by git
+    os.makedirs(scratch, exist_ok=True)
+    tmp = tempfile.mkdtemp(prefix="lib_", dir=scratch)
+    try:
+        out = os.path.join(tmp, "libm2dscan.so")
+        cmd = ["hipcc", *HIPCC_FLAGS, "-save-temps=obj", "-I", os.path.join(ROOT, "include"), "-o", out, *srcs]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        subprocess.check_call(cmd, cwd=tmp)
+        listings = sorted(glob.glob(os.path.join(tmp, "*-hip-amdgcn-amd-amdhsa-gfx950.s")))
+        if len(listings) != len(srcs):
+            raise RuntimeError(f"expected the device assembly of {len(srcs)} sources, found {listings}")
+        for path in listings:
+            ndpp, bad = asmcheck.check_file(path)
+            if verbose:
+                print(f"asmcheck {os.path.basename(path)}: {ndpp} DPP instructions, {len(bad)} hazards", flush=True)
+            if bad:
+                raise RuntimeError("hazard between inline-assembly DPP instructions and their producers:\n" +
+                                   "\n".join(f"  {k}: {p}  ->  {c}" for k, p, c in bad[:8]))
+        shutil.move(out, LIB)
+    finally:
+        shutil.rmtree(tmp, ignore_errors=True)
     return LIB
 
 

@@ -136,6 +136,10 @@ __device__ __forceinline__ float from_row_above(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x101 /*row_shl:1*/, 0xf, 0xf, true));
 }
 __device__ __forceinline__ float fexp2(float v) { return __builtin_amdgcn_exp2f(v); }
+// All four values exist from here on: nothing may compute one of them later, next to its use.
+// (An empty statement; with the scheduling barrier behind it, it keeps a group of v_exp_f32 in
+// front of the instructions that follow the barrier.)
+__device__ __forceinline__ void pin4(float (&a)[4]) { asm volatile("" : "+v"(a[0]), "+v"(a[1]), "+v"(a[2]), "+v"(a[3])); }
 
 // a[lanes 32..63] <-> b[lanes 0..31]; returns a+b: lanes 0..31 hold the two-half sum of a,
 // lanes 32..63 that of b.
@@ -666,9 +670,11 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
         float aT[4], aL[4];
 #pragma unroll
         for (int w = 0; w < 4; ++w) aT[w] = fexp2(__builtin_fmaf(o.dtv[c], a2t[c][sinv<PERM>(4 * q + w)], offT));
+        pin4(aT);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int w = 0; w < 4; ++w) aL[w] = fexp2(__builtin_fmaf(o.dlv[c], a2l[c][sinv<PERM>(4 * q + w)], offL));
+        pin4(aL);
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
@@ -980,10 +986,14 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
       float hb[kCK + 1][8];
+      float gT_last[8], gL_last[8];   // gates of the last step: the adjoint starts with them
 #pragma unroll
       for (int mgl = 0; mgl < 2; ++mgl)
 #pragma unroll
-        for (int qi = 0; qi < 4; ++qi) hb[0][4 * mgl + qi] = ck0[fold_state(2 * half + mgl, qi)];
+        for (int qi = 0; qi < 4; ++qi) {
+          hb[0][4 * mgl + qi] = ck0[fold_state(2 * half + mgl, qi)];
+          gT_last[4 * mgl + qi] = 0.f; gL_last[4 * mgl + qi] = 0.f;
+        }
       // ---- recompute the states of the block
 #pragma unroll
       for (int k = 0; k < kCK; ++k) {
@@ -1023,9 +1033,11 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
             float aT[4], aL[4];   // gates before chains, see the forward kernel
 #pragma unroll
             for (int qi = 0; qi < 4; ++qi) aT[qi] = fexp2(__builtin_fmaf(dtv, atq[qi], offT));
+            pin4(aT);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int qi = 0; qi < 4; ++qi) aL[qi] = fexp2(__builtin_fmaf(dlv, alq[qi], offL));
+            pin4(aL);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int qi = 0; qi < 4; ++qi) {
@@ -1034,6 +1046,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
               u = __builtin_fmaf(sT, bq[qi], u);
               u = fma_row_below(aT[qi], hb[k][s8], u);
               hb[k + 1][s8] = __builtin_fmaf(aL[qi], hb[k][s8], u);
+              if (k == kCK - 1) { gT_last[s8] = aT[qi]; gL_last[s8] = aL[qi]; }
             }
           }
         }
@@ -1090,8 +1103,8 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
             for (int qi = 0; qi < 4; ++qi) {
               const int n = fold_state(mg, qi), s8 = 4 * mgl + qi;
               const float a2t = atq[qi], a2l = alq[qi];
-              const float aT = fexp2(__builtin_fmaf(dtv, a2t, offT));
-              const float aL = fexp2(__builtin_fmaf(dlv, a2l, offL));
+              const float aT = k == kCK - 1 ? gT_last[s8] : fexp2(__builtin_fmaf(dtv, a2t, offT));
+              const float aL = k == kCK - 1 ? gL_last[s8] : fexp2(__builtin_fmaf(dlv, a2l, offL));
               const float lam = __builtin_fmaf(dyl, cq[qi], add_row_above(muL[n], muT[n]));
               const float mT = aT * lam, mL = aL * lam;
               muT[n] = mT;
