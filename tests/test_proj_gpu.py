@@ -49,10 +49,10 @@ def make_case(B, H, W, E, seed, dtype):
 
 WNAMES = ("x_proj_w", "dt_projT_w", "dt_projT_b", "dt_projL_w", "dt_projL_b")
 
-# (B, H, W, E): tiles that end inside the batch, channel counts that are no multiple of the
-# 64-channel chunk, one to seven 16-wide chunks of outputs, the largest rank
+# (B, H, W, E): tiles that end inside the batch, fewer positions than one wave owns, channel counts
+# that are no multiple of the 64-channel chunk, one to seven 16-wide chunks of outputs, the largest rank
 SHAPES = [(2, 9, 12, 32), (1, 5, 7, 3), (2, 14, 14, 64), (1, 8, 8, 128), (1, 40, 4, 100), (1, 7, 9, 320),
-          (3, 7, 7, 512), (5, 31, 30, 64)]
+          (3, 7, 7, 512), (5, 31, 30, 64), (1, 2, 2, 8), (1, 2, 3, 16), (1, 3, 3, 504), (1, 17, 1, 72)]
 
 
 def reference(x, w, up, R):
