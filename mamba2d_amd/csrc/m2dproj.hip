@@ -19,6 +19,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "m2dscan.h"
 
 namespace {
@@ -1147,13 +1149,16 @@ constexpr int kMaxLdsWeights = (kTP * kXS4 + 2 * kTP * kXS + kTP * ((2 * kMaxR +
 
 template <typename T, bool VEC>
 bool allow_lds_weights() {
-  static bool done = false;   // idempotent, the value never changes
-  if (!done) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_proj_bwd_weights_kernel<T, VEC>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsWeights) != hipSuccess)
-      return false;
-    done = true;
-  }
+  // more than 64 KB of dynamic LDS has to be allowed once per device (one bit per device ordinal)
+  static std::atomic<uint64_t> seen{0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return false;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (seen.load(std::memory_order_relaxed) & bit) return true;
+  if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_proj_bwd_weights_kernel<T, VEC>),
+                          hipFuncAttributeMaxDynamicSharedMemorySize, kMaxLdsWeights) != hipSuccess)
+    return false;
+  seen.fetch_or(bit, std::memory_order_relaxed);
   return true;
 }
 

@@ -34,6 +34,8 @@
 // positions (d_AT, d_AL, d_D) are register accumulators reduced at the end.  No atomics:
 // results are bit-reproducible.
 #include <hip/hip_runtime.h>
+
+#include <atomic>
 #include <stdint.h>
 
 #include "../../include/m2dscan.h"
@@ -1428,6 +1430,18 @@ void fill_common(ScanParams& sp, const m2d_desc* d, const Geometry& g) {
   sp.flip = (d->flags & M2D_FLAG_FLIP) ? 1 : 0;
 }
 
+// A kernel that needs more than 64 KB of dynamic LDS has to be told so once per device (each
+// device loads its own copy of the code object).  `seen` holds one bit per device ordinal.
+inline bool allow_dynamic_lds(const void* kernel, size_t bytes, std::atomic<uint64_t>& seen) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return false;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (seen.load(std::memory_order_relaxed) & bit) return true;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) != hipSuccess) return false;
+  seen.fetch_or(bit, std::memory_order_relaxed);
+  return true;
+}
+
 // Set-up area: [page of zeros][A_T*log2e][A_L*log2e][D], all fp32.
 template <typename T>
 int launch_prep(ScanParams& sp, const m2d_desc* d, const void* AT, const void* AL, const void* D, float* base, hipStream_t st) {
@@ -1459,13 +1473,8 @@ template <typename T, int EC, bool CK, bool WY, bool SX, int MODE>
 int launch_fwd_as(const ScanParams& sp, hipStream_t st) {
   using SG = Stage<T, 3, kFwdWaves * 4 * EC, false, true>;
   const size_t lds = 256 + 2 * (size_t)SG::kBytes;
-  static bool attr = false;   // idempotent, the value never changes
-  if (!attr) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_fwd_kernel<T, EC, CK, WY, SX, MODE>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return M2D_ERR_HIP;
-    attr = true;
-  }
+  static std::atomic<uint64_t> seen{0};
+  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_fwd_kernel<T, EC, CK, WY, SX, MODE>), lds, seen)) return M2D_ERR_HIP;
   hipLaunchKernelGGL((m2d_fwd_kernel<T, EC, CK, WY, SX, MODE>), dim3((unsigned)sp.nwg), dim3(kFwdWaves * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
@@ -1534,13 +1543,8 @@ template <typename T, bool SX, int MODE>
 int launch_bwd(const ScanParams& sp, hipStream_t st) {
   using SG = Stage<T, 4, kBwdWaves * 4, true, false>;
   const size_t lds = sizeof(float4) * kBwdWaves * 3 * 64 + sizeof(float) * kBwdWaves * 4 * 2 * kN + 256 + 2 * (size_t)SG::kBytes;
-  static bool attr = false;   // idempotent, the value never changes
-  if (!attr) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(&m2d_bwd_kernel<T, SX, MODE>),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
-      return M2D_ERR_HIP;
-    attr = true;
-  }
+  static std::atomic<uint64_t> seen{0};
+  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_bwd_kernel<T, SX, MODE>), lds, seen)) return M2D_ERR_HIP;
   hipLaunchKernelGGL((m2d_bwd_kernel<T, SX, MODE>), dim3((unsigned)sp.nwg), dim3(kBwdWaves * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
