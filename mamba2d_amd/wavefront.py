@@ -108,11 +108,16 @@ class wf_cuda_fn_pr(torch.autograd.Function):
     corner, which equals flipping every spatial tensor before and y after
     (``models/mamba2d.py:163-173``) without the copies."""
 
+    @classmethod
+    def apply(cls, x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip=False):
+        # Whether autograd records the call is only known out here: forward() always runs with grad
+        # mode off, and needs_input_grad is also set for parameters under torch.no_grad().
+        return super().apply(x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip, torch.is_grad_enabled())
+
     @staticmethod
-    def forward(ctx, x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip=False):
+    def forward(ctx, x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip=False, recording=True):
         args = [_c(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D)]
-        # (grad mode is always off inside forward(); needs_input_grad is what tells training from inference)
-        keep = SAVE_CHECKPOINTS and any(ctx.needs_input_grad)
+        keep = SAVE_CHECKPOINTS and recording and any(ctx.needs_input_grad)
         y, ck = scan_fwd_op(*args, keep, bool(flip))
         ctx.save_for_backward(*args, ck)
         ctx.flip = bool(flip)
@@ -122,7 +127,7 @@ class wf_cuda_fn_pr(torch.autograd.Function):
     def backward(ctx, grad_output):
         *args, ck = ctx.saved_tensors
         dy = _c(grad_output.to(args[0].dtype))
-        return (*scan_bwd_op(*args, dy, ck, ctx.flip), None)
+        return (*scan_bwd_op(*args, dy, ck, ctx.flip), None, None)
 
 
 class wf_cuda_fn_fr(torch.autograd.Function):
@@ -179,14 +184,20 @@ class wf_cuda_fn_proj(torch.autograd.Function):
         A = A32.to(x.dtype)
         return w32, A32, A, proj_fwd_op(x, *w32, AT_log.shape[1], True)
 
+    @classmethod
+    def apply(cls, x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D, full=False, flip=False):
+        # see wf_cuda_fn_pr.apply
+        return super().apply(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D, full, flip,
+                             torch.is_grad_enabled())
+
     @staticmethod
     def forward(ctx, x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D,
-                full=False, flip=False):
+                full=False, flip=False, recording=True):
         x = _c(x)
         Dx = _c(D.to(x.dtype))
         weights = (AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b)
         _, A32, A, (low, dT, dL, BT, BL, C) = wf_cuda_fn_proj._project(x, *weights)
-        keep = SAVE_CHECKPOINTS and not full and any(ctx.needs_input_grad)
+        keep = SAVE_CHECKPOINTS and not full and recording and any(ctx.needs_input_grad)
         y, ck = scan_fwd_op(x, dT, dL, A[0], A[1], BT, BL, C, Dx, keep, bool(flip))
         if full:
             ctx.save_for_backward(x, *weights, D)
@@ -215,7 +226,7 @@ class wf_cuda_fn_proj(torch.autograd.Function):
         d_A_log = torch.stack((d_AT, d_AL)).float() * A32
         return (d_x, d_A_log[0].to(AT_log.dtype), d_A_log[1].to(AL_log.dtype), g_xw.to(x_proj_w.dtype),
                 g_wT.to(dt_projT_w.dtype), g_bT.to(dt_projT_b.dtype), g_wL.to(dt_projL_w.dtype), g_bL.to(dt_projL_b.dtype),
-                d_D.to(D.dtype), None, None)
+                d_D.to(D.dtype), None, None, None)
 
 
 def wavefront_scan_cuda(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D,

@@ -110,6 +110,32 @@ def test_partial_and_full_agree_bf16(wf, projections):
         assert a.dtype == b.dtype and so.rel_err(a.float().cpu(), b.float().cpu()) < 2e-2
 
 
+def test_no_checkpoints_are_kept_under_no_grad(wf, monkeypatch):
+    """Parameters keep requires_grad=True at inference; torch.no_grad() must still give the
+    inference forward (no checkpoint buffer), for the plain Function and for the entry point."""
+    say("\ncase no_grad keeps nothing")
+    seen = []
+    real = wf.scan_fwd_op
+
+    def spy(*a):
+        seen.append(bool(a[9]))
+        return real(*a)
+
+    monkeypatch.setattr(wf, "scan_fwd_op", spy)
+    inp = so.make_inputs(1, 6, 5, 8, 16, seed=2, dtype=torch.float32)
+    leaves = [inp[k].cuda().requires_grad_(True) for k in so.INPUT_NAMES]
+    E, N, R = 8, 16, 1
+    p = make_block_params(E, N, R, 0, "cuda")
+    params = [p[k].requires_grad_(True) for k in ORDER]
+    with torch.no_grad():
+        wf.wf_cuda_fn_pr.apply(*leaves)
+        wf.wavefront_scan_cuda(leaves[0], *params)
+    assert seen == [False, False]
+    wf.wf_cuda_fn_pr.apply(*leaves)
+    wf.wavefront_scan_cuda(leaves[0], *params)
+    assert seen[2:] == [wf.SAVE_CHECKPOINTS, wf.SAVE_CHECKPOINTS]
+
+
 def test_views_that_start_off_alignment_are_accepted(wf, cscan):
     """A contiguous view whose first element is not 16-byte aligned is copied, not rejected."""
     say("\ncase unaligned views")
