@@ -53,7 +53,7 @@ typedef enum m2d_dtype {
 /* Problem descriptor.  N must be 16 in this build (the reference's d_state default,
  * models/mamba2d.py:23).  flags: bit 0 = M2D_FLAG_FLIP, scan from the bottom-right
  * corner (equivalent to torch.flip(x,(1,2)) of every spatial tensor before and of the
- * outputs after, models/mamba2d.py:163-173). */
+ * outputs after, models/mamba2d.py:163-173); the other flags are described below. */
 typedef struct m2d_desc {
   int32_t B, H, W, E, N;
   int32_t dtype;              /* m2d_dtype */
@@ -67,6 +67,12 @@ typedef struct m2d_desc {
  * the flag bf16 activations still meet bf16-rounded weight matrices (not biases) wherever the
  * products run on the matrix cores (channel counts that are a multiple of 8). */
 #define M2D_FLAG_ROUND_WEIGHTS 2
+/* m2d_scan_fwd / m2d_scan_bwd only: AT, AL and D are the parameters as the reference's module holds
+ * them, fp32: AT and AL point to A_log (E,N) with A = -exp(A_log) (models/mamba2d.py:95-101,
+ * wavefront_cuda.py:72-73), D to (E); the library rounds A and D to desc->dtype as the reference's
+ * casts do (wavefront_cuda.py:90-91, 332).  d_AT, d_AL, d_D are then fp32 gradients with respect to
+ * A_log and D. */
+#define M2D_FLAG_RAW_PARAMS 4
 
 #define M2D_PASS_FWD 0
 #define M2D_PASS_BWD 1

@@ -16,6 +16,7 @@ LIB_PATH = os.environ.get("M2D_LIB") or os.path.join(_HERE, "libm2dscan.so")
 M2D_F32, M2D_BF16 = 0, 1
 M2D_FLAG_FLIP = 1
 M2D_FLAG_ROUND_WEIGHTS = 2
+M2D_FLAG_RAW_PARAMS = 4
 M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",

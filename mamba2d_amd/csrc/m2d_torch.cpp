@@ -21,7 +21,7 @@ namespace {
 
 using at::Tensor;
 
-m2d_desc describe(const Tensor& x, const Tensor& AT, bool flip) {
+m2d_desc describe(const Tensor& x, const Tensor& AT, bool flip, bool raw_params = false) {
   TORCH_CHECK(x.dim() == 4, "m2dscan: x must be (B,H,W,E), got ", x.sizes());
   TORCH_CHECK(AT.dim() == 2, "m2dscan: AT must be (E,N), got ", AT.sizes());
   m2d_desc d{};
@@ -33,7 +33,7 @@ m2d_desc describe(const Tensor& x, const Tensor& AT, bool flip) {
   if (x.scalar_type() == at::kFloat) d.dtype = M2D_F32;
   else if (x.scalar_type() == at::kBFloat16) d.dtype = M2D_BF16;
   else TORCH_CHECK(false, "m2dscan: float32 and bfloat16 are supported, got ", x.scalar_type());
-  d.flags = flip ? M2D_FLAG_FLIP : 0;
+  d.flags = (flip ? M2D_FLAG_FLIP : 0) | (raw_params ? M2D_FLAG_RAW_PARAMS : 0);
   return d;
 }
 
@@ -45,19 +45,28 @@ void expect(const Tensor& t, const char* name, const Tensor& x, at::IntArrayRef 
   TORCH_CHECK(t.is_contiguous(), "m2dscan: ", name, " must be contiguous");
 }
 
+void expect_param(const Tensor& t, const char* name, const Tensor& x, at::IntArrayRef shape, bool raw) {
+  if (!raw) return expect(t, name, x, shape);
+  TORCH_CHECK(t.device() == x.device(), "m2dscan: ", name, " is on ", t.device(), ", x on ", x.device());
+  TORCH_CHECK(t.scalar_type() == at::kFloat, "m2dscan: ", name, " must be float32 when raw parameters are passed, got ", t.scalar_type());
+  TORCH_CHECK(t.sizes() == shape, "m2dscan: ", name, " has shape ", t.sizes(), ", expected ", shape);
+  TORCH_CHECK(t.is_contiguous(), "m2dscan: ", name, " must be contiguous");
+}
+
 void expect_all(const m2d_desc& d, const Tensor& x, const Tensor& dT, const Tensor& dL, const Tensor& AT,
                 const Tensor& AL, const Tensor& BT, const Tensor& BL, const Tensor& C, const Tensor& D) {
+  const bool raw = (d.flags & M2D_FLAG_RAW_PARAMS) != 0;
   TORCH_CHECK(x.is_cuda(), "m2dscan: tensors must live on the GPU");
   TORCH_CHECK(x.is_contiguous(), "m2dscan: x must be contiguous");
   const int64_t B = d.B, H = d.H, W = d.W, E = d.E, N = d.N;
   expect(dT, "deltaT", x, {B, H, W, E});
   expect(dL, "deltaL", x, {B, H, W, E});
-  expect(AT, "AT", x, {E, N});
-  expect(AL, "AL", x, {E, N});
+  expect_param(AT, raw ? "AT_log" : "AT", x, {E, N}, raw);
+  expect_param(AL, raw ? "AL_log" : "AL", x, {E, N}, raw);
   expect(BT, "BT", x, {B, H, W, N});
   expect(BL, "BL", x, {B, H, W, N});
   expect(C, "C", x, {B, H, W, N});
-  expect(D, "D", x, {E});
+  expect_param(D, "D", x, {E}, raw);
 }
 
 void check(int status) { TORCH_CHECK(status == M2D_OK, "m2dscan: ", m2d_status_str(status), " (status ", status, ")"); }
@@ -68,8 +77,8 @@ Tensor bytes(size_t n, const Tensor& like) {
 
 std::tuple<Tensor, Tensor> scan_fwd(const Tensor& x, const Tensor& dT, const Tensor& dL, const Tensor& AT,
                                     const Tensor& AL, const Tensor& BT, const Tensor& BL, const Tensor& C,
-                                    const Tensor& D, bool save_ckpt, bool flip) {
-  const m2d_desc d = describe(x, AT, flip);
+                                    const Tensor& D, bool save_ckpt, bool flip, bool raw_params) {
+  const m2d_desc d = describe(x, AT, flip, raw_params);
   expect_all(d, x, dT, dL, AT, AL, BT, BL, C, D);
   check(m2d_desc_check(&d));
   c10::DeviceGuard guard(x.device());
@@ -86,8 +95,8 @@ std::tuple<Tensor, Tensor> scan_fwd(const Tensor& x, const Tensor& dT, const Ten
 
 std::vector<Tensor> scan_bwd(const Tensor& x, const Tensor& dT, const Tensor& dL, const Tensor& AT, const Tensor& AL,
                              const Tensor& BT, const Tensor& BL, const Tensor& C, const Tensor& D, const Tensor& dy,
-                             const Tensor& ckpt, bool flip) {
-  const m2d_desc d = describe(x, AT, flip);
+                             const Tensor& ckpt, bool flip, bool raw_params) {
+  const m2d_desc d = describe(x, AT, flip, raw_params);
   expect_all(d, x, dT, dL, AT, AL, BT, BL, C, D);
   expect(dy, "dy", x, x.sizes());
   check(m2d_desc_check(&d));
@@ -196,9 +205,9 @@ int64_t abi_version() { return m2d_version(); }
 
 TORCH_LIBRARY(m2dscan, m) {
   m.def("scan_fwd(Tensor x, Tensor deltaT, Tensor deltaL, Tensor AT, Tensor AL, Tensor BT, Tensor BL, Tensor C, "
-        "Tensor D, bool save_ckpt, bool flip) -> (Tensor, Tensor)");
+        "Tensor D, bool save_ckpt, bool flip, bool raw_params=False) -> (Tensor, Tensor)");
   m.def("scan_bwd(Tensor x, Tensor deltaT, Tensor deltaL, Tensor AT, Tensor AL, Tensor BT, Tensor BL, Tensor C, "
-        "Tensor D, Tensor dy, Tensor ckpt, bool flip) -> Tensor[]");
+        "Tensor D, Tensor dy, Tensor ckpt, bool flip, bool raw_params=False) -> Tensor[]");
   m.def("proj_fwd(Tensor x, Tensor x_proj_w, Tensor dt_projT_w, Tensor dt_projT_b, Tensor dt_projL_w, Tensor dt_projL_b, "
         "int d_state, bool round_weights) -> Tensor[]");
   m.def("proj_bwd(Tensor x, Tensor lowrank, Tensor deltaT, Tensor deltaL, Tensor x_proj_w, Tensor dt_projT_w, "

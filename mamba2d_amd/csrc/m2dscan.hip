@@ -1201,15 +1201,32 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
 }
 
 // -------------------------------------------------------------------------- small helper kernels
-template <typename T>
-__global__ void m2d_prep_kernel(const T* AT, const T* AL, const T* D, float* zeros, float* A2T, float* A2L, float* Df, int E) {
+// the value a tensor of type T would hold
+__device__ __forceinline__ float as_stored(float v, const float*) { return v; }
+__device__ __forceinline__ float as_stored(float v, const bf16_t*) { return bf16_bits_to_f32(f32_to_bf16_bits(v)); }
+
+// RAW: the parameters as the module holds them (fp32 A_log, fp32 D): A = -exp(A_log), and both
+// are rounded to T, which is what the reference's casts to x.dtype do (wavefront_cuda.py:72-73,
+// 90-91, 332).
+template <typename T, bool RAW>
+__global__ void m2d_prep_kernel(const void* ATv, const void* ALv, const void* Dv, float* zeros, float* A2T, float* A2L, float* Df, int E) {
   const int idx = blockIdx.x * blockDim.x + threadIdx.x;
   if (idx < kZeroFloats) zeros[idx] = 0.f;
-  if (idx < E * kN) {
-    A2T[idx] = IO<T>::ld(AT + idx) * kLog2e;
-    A2L[idx] = IO<T>::ld(AL + idx) * kLog2e;
+  if constexpr (RAW) {
+    const float *AT = static_cast<const float*>(ATv), *AL = static_cast<const float*>(ALv), *D = static_cast<const float*>(Dv);
+    if (idx < E * kN) {
+      A2T[idx] = as_stored(-expf(AT[idx]), static_cast<const T*>(nullptr)) * kLog2e;
+      A2L[idx] = as_stored(-expf(AL[idx]), static_cast<const T*>(nullptr)) * kLog2e;
+    }
+    if (idx < E) Df[idx] = as_stored(D[idx], static_cast<const T*>(nullptr));
+  } else {
+    const T *AT = static_cast<const T*>(ATv), *AL = static_cast<const T*>(ALv), *D = static_cast<const T*>(Dv);
+    if (idx < E * kN) {
+      A2T[idx] = IO<T>::ld(AT + idx) * kLog2e;
+      A2L[idx] = IO<T>::ld(AL + idx) * kLog2e;
+    }
+    if (idx < E) Df[idx] = IO<T>::ld(D + idx);
   }
-  if (idx < E) Df[idx] = IO<T>::ld(D + idx);
 }
 
 // B_T, B_L, C -> one fp32 record of 48 values per cell (three runs of 16, each in fold order,
@@ -1238,8 +1255,10 @@ __global__ void m2d_pack_bc_kernel(const T* BT, const T* BL, const T* C, float* 
 
 // d_C, d_BT, d_BL: add the per-workgroup channel sums in workgroup order and round to T.
 // d_AT, d_AL, d_D: add the per-image partials in image order.
-template <typename T>
-__global__ void m2d_finalize_kernel(const ScanParams p, T* dC, T* dBT, T* dBL, T* dAT, T* dAL, T* dD) {
+// RAW: d_AT, d_AL, d_D are fp32 and refer to the parameters as the module holds them:
+// A = -exp(A_log), so d_A_log = d_A * A (A is at hand as A2 / log2 e).
+template <typename T, bool RAW>
+__global__ void m2d_finalize_kernel(const ScanParams p, T* dC, T* dBT, T* dBL, void* dATv, void* dALv, void* dDv) {
   const int64_t P = p.Ptot;
   const int64_t nquad = 3 * P * (kN / 4);
   const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -1278,9 +1297,15 @@ __global__ void m2d_finalize_kernel(const ScanParams p, T* dC, T* dBT, T* dBL, T
     if (l == 0) {
       if (out < n_at) {
         const int e = (int)(out / (2 * kN)), w = (int)(out % (2 * kN));
-        if (w < kN) IO<T>::st(dAT + e * kN + w, s); else IO<T>::st(dAL + e * kN + (w - kN), s);
+        if constexpr (RAW) {
+          if (w < kN) static_cast<float*>(dATv)[e * kN + w] = s * p.A2T[e * kN + w] * kLn2;
+          else static_cast<float*>(dALv)[e * kN + (w - kN)] = s * p.A2L[e * kN + (w - kN)] * kLn2;
+        } else {
+          if (w < kN) IO<T>::st(static_cast<T*>(dATv) + e * kN + w, s); else IO<T>::st(static_cast<T*>(dALv) + e * kN + (w - kN), s);
+        }
       } else if (out < n_at + p.E) {
-        IO<T>::st(dD + (out - n_at), s);
+        if constexpr (RAW) static_cast<float*>(dDv)[out - n_at] = s;
+        else IO<T>::st(static_cast<T*>(dDv) + (out - n_at), s);
       }
     }
   }
@@ -1312,7 +1337,7 @@ int check_desc(const m2d_desc* d) {
   if (d->B < 1 || d->E < 1 || d->N < 1 || d->H < 2 || d->W < 2) return M2D_ERR_BAD_SHAPE;
   if (d->N != kN) return M2D_ERR_UNSUPPORTED;
   if (d->dtype != M2D_F32 && d->dtype != M2D_BF16) return M2D_ERR_UNSUPPORTED;
-  if (d->reserved != 0 || (d->flags & ~M2D_FLAG_FLIP)) return M2D_ERR_UNSUPPORTED;
+  if (d->reserved != 0 || (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_RAW_PARAMS))) return M2D_ERR_UNSUPPORTED;
   if ((int64_t)d->B * d->H * d->W >= ((int64_t)1 << 40)) return M2D_ERR_BAD_SHAPE;
   // one image is addressed with 32-bit byte offsets from its base (fp32: 4 bytes per element;
   // the widest per-cell record, the channel sums, is 192 bytes)
@@ -1451,8 +1476,10 @@ int launch_prep(ScanParams& sp, const m2d_desc* d, const void* AT, const void* A
   float* Df = A2L + (size_t)d->E * kN;
   sp.zeros = zeros; sp.A2T = A2T; sp.A2L = A2L; sp.Df = Df;
   const int n = d->E * kN > kZeroFloats ? d->E * kN : kZeroFloats;
-  hipLaunchKernelGGL(m2d_prep_kernel<T>, dim3((n + 255) / 256), dim3(256), 0, st, static_cast<const T*>(AT),
-                     static_cast<const T*>(AL), static_cast<const T*>(D), zeros, A2T, A2L, Df, d->E);
+  if (d->flags & M2D_FLAG_RAW_PARAMS)
+    hipLaunchKernelGGL((m2d_prep_kernel<T, true>), dim3((n + 255) / 256), dim3(256), 0, st, AT, AL, D, zeros, A2T, A2L, Df, d->E);
+  else
+    hipLaunchKernelGGL((m2d_prep_kernel<T, false>), dim3((n + 255) / 256), dim3(256), 0, st, AT, AL, D, zeros, A2T, A2L, Df, d->E);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
@@ -1598,9 +1625,12 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   const int64_t P = (int64_t)d->B * d->H * d->W;
   const int64_t quad_blocks = (3 * P * (kN / 4) + 255) / 256;
   const int64_t tail_blocks = (((int64_t)d->E * 2 * kN + d->E) * 16 + 255) / 256;   // 16 lanes per position sum
-  hipLaunchKernelGGL(m2d_finalize_kernel<T>, dim3((unsigned)(quad_blocks + tail_blocks)), dim3(256), 0, st, sp,
-                     static_cast<T*>(dC), static_cast<T*>(dBT), static_cast<T*>(dBL), static_cast<T*>(dAT),
-                     static_cast<T*>(dAL), static_cast<T*>(dD));
+  if (d->flags & M2D_FLAG_RAW_PARAMS)
+    hipLaunchKernelGGL((m2d_finalize_kernel<T, true>), dim3((unsigned)(quad_blocks + tail_blocks)), dim3(256), 0, st, sp,
+                       static_cast<T*>(dC), static_cast<T*>(dBT), static_cast<T*>(dBL), dAT, dAL, dD);
+  else
+    hipLaunchKernelGGL((m2d_finalize_kernel<T, false>), dim3((unsigned)(quad_blocks + tail_blocks)), dim3(256), 0, st, sp,
+                       static_cast<T*>(dC), static_cast<T*>(dBT), static_cast<T*>(dBL), dAT, dAL, dD);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
@@ -1610,7 +1640,7 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
 extern "C" {
 
 
-int m2d_version(void) { return 300; }
+int m2d_version(void) { return 400; }
 
 const char* m2d_status_str(int status) {
   switch (status) {

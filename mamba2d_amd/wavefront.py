@@ -53,13 +53,13 @@ def _ckpt_bytes(x, N, flip=False) -> int:
 
 
 @torch.library.register_fake("m2dscan::scan_fwd")
-def _scan_fwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, save_ckpt, flip):
+def _scan_fwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, save_ckpt, flip, raw_params=False):
     n = _ckpt_bytes(x, AT.shape[1]) if save_ckpt else 1
     return torch.empty_like(x), x.new_empty((max(n, 1),), dtype=torch.uint8)
 
 
 @torch.library.register_fake("m2dscan::scan_bwd")
-def _scan_bwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt, flip):
+def _scan_bwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt, flip, raw_params=False):
     return [torch.empty_like(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D)]
 
 
@@ -178,11 +178,10 @@ class wf_cuda_fn_proj(torch.autograd.Function):
     backward; ``full=True`` keeps only x and the weights and rebuilds the rest in the backward."""
 
     @staticmethod
-    def _project(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b):
-        w32 = [_c(t.float()) for t in (x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b)]
-        A32 = -torch.exp(torch.stack((AT_log.float(), AL_log.float())))   # both directions at once
-        A = A32.to(x.dtype)
-        return w32, A32, A, proj_fwd_op(x, *w32, AT_log.shape[1], True)
+    def _params(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D):
+        """The parameters as fp32 tensors (no copy if they already are): the library itself forms
+        A = -exp(A_log) and rounds everything to x.dtype as the reference's casts do."""
+        return [_c(t.float()) for t in (AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D)]
 
     @classmethod
     def apply(cls, x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D, full=False, flip=False):
@@ -194,39 +193,34 @@ class wf_cuda_fn_proj(torch.autograd.Function):
     def forward(ctx, x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D,
                 full=False, flip=False, recording=True):
         x = _c(x)
-        Dx = _c(D.to(x.dtype))
-        weights = (AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b)
-        _, A32, A, (low, dT, dL, BT, BL, C) = wf_cuda_fn_proj._project(x, *weights)
+        raw = (AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D)
+        At, Al, *w32, D32 = wf_cuda_fn_proj._params(x, *raw)
+        low, dT, dL, BT, BL, C = proj_fwd_op(x, *w32, AT_log.shape[1], True)
         keep = SAVE_CHECKPOINTS and not full and recording and any(ctx.needs_input_grad)
-        y, ck = scan_fwd_op(x, dT, dL, A[0], A[1], BT, BL, C, Dx, keep, bool(flip))
+        y, ck = scan_fwd_op(x, dT, dL, At, Al, BT, BL, C, D32, keep, bool(flip), True)
         if full:
-            ctx.save_for_backward(x, *weights, D)
+            ctx.save_for_backward(x, *raw)
         else:
-            ctx.save_for_backward(x, *weights, D, A32, A, low, dT, dL, BT, BL, C, ck)
+            ctx.save_for_backward(x, *raw, low, dT, dL, BT, BL, C, ck)
         ctx.full, ctx.flip = bool(full), bool(flip)
         return y
 
     @staticmethod
     def backward(ctx, grad_output):
-        x, *weights, D = ctx.saved_tensors[:9]
-        AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b = weights
+        x, *raw = ctx.saved_tensors[:9]
+        At, Al, *w32, D32 = wf_cuda_fn_proj._params(x, *raw)
         dy = _c(grad_output.to(x.dtype))
         if ctx.full:
-            w32, A32, A, (low, dT, dL, BT, BL, C) = wf_cuda_fn_proj._project(x, *weights)
+            low, dT, dL, BT, BL, C = proj_fwd_op(x, *w32, At.shape[1], True)
             ck = x.new_empty((1,), dtype=torch.uint8)
         else:
-            A32, A, low, dT, dL, BT, BL, C, ck = ctx.saved_tensors[9:]
-            w32 = [_c(t.float()) for t in (x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b)]
-        d_x, d_dT, d_dL, d_AT, d_AL, d_BT, d_BL, d_C, d_D = scan_bwd_op(
-            x, dT, dL, A[0], A[1], BT, BL, C, _c(D.to(x.dtype)), dy, ck, ctx.flip)
+            low, dT, dL, BT, BL, C, ck = ctx.saved_tensors[9:]
+        # with raw parameters the gradients of A_log and D come back in fp32
+        d_x, d_dT, d_dL, d_At, d_Al, d_BT, d_BL, d_C, d_D = scan_bwd_op(x, dT, dL, At, Al, BT, BL, C, D32, dy, ck, ctx.flip, True)
         # d_x holds the scan's own gradient (dy*D included); the projections add theirs in place
-        g_xw, g_wT, g_bT, g_wL, g_bL = proj_bwd_op(x, low, dT, dL, w32[0], w32[1], w32[3], d_dT, d_dL, d_BT, d_BL, d_C, d_x,
-                                                   True)
-        # A = -exp(A_log): dA/dA_log = A
-        d_A_log = torch.stack((d_AT, d_AL)).float() * A32
-        return (d_x, d_A_log[0].to(AT_log.dtype), d_A_log[1].to(AL_log.dtype), g_xw.to(x_proj_w.dtype),
-                g_wT.to(dt_projT_w.dtype), g_bT.to(dt_projT_b.dtype), g_wL.to(dt_projL_w.dtype), g_bL.to(dt_projL_b.dtype),
-                d_D.to(D.dtype), None, None, None)
+        g = proj_bwd_op(x, low, dT, dL, w32[0], w32[1], w32[3], d_dT, d_dL, d_BT, d_BL, d_C, d_x, True)
+        grads = (d_At, d_Al, *g, d_D)
+        return (d_x, *[t.to(r.dtype) for t, r in zip(grads, raw)], None, None, None)
 
 
 def wavefront_scan_cuda(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D,

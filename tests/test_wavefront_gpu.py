@@ -110,6 +110,32 @@ def test_partial_and_full_agree_bf16(wf, projections):
         assert a.dtype == b.dtype and so.rel_err(a.float().cpu(), b.float().cpu()) < 2e-2
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 1e-2)], ids=["f32", "bf16"])
+def test_raw_parameters_match_cast_parameters(wf, dtype, tol):
+    """M2D_FLAG_RAW_PARAMS: fp32 A_log and D in, the library forms A = -exp(A_log) and rounds like
+    the reference's casts; gradients come back for A_log and D in fp32."""
+    say(f"\ncase raw parameters {dtype}")
+    inp = so.make_inputs(2, 9, 30, 8, 16, seed=5, dtype=torch.float32)
+    a = {k: inp[k].cuda() for k in so.INPUT_NAMES}
+    logT, logL = torch.log(-a["AT"]), torch.log(-a["AL"])
+    act = [a[k].to(dtype) for k in ("x", "deltaT", "deltaL")]
+    bc = [a[k].to(dtype) for k in ("BT", "BL", "C")]
+    cast = [(-torch.exp(logT)).to(dtype), (-torch.exp(logL)).to(dtype)]
+    dy = inp["dy"].cuda().to(dtype)
+    y0, ck0 = wf.scan_fwd_op(*act, *cast, *bc, a["D"].to(dtype), True, False)
+    y1, ck1 = wf.scan_fwd_op(*act, logT, logL, *bc, a["D"], True, False, True)
+    assert y1.dtype == dtype and so.rel_err(y1.float().cpu(), y0.float().cpu()) < tol
+    g0 = wf.scan_bwd_op(*act, *cast, *bc, a["D"].to(dtype), dy, ck0, False)
+    g1 = wf.scan_bwd_op(*act, logT, logL, *bc, a["D"], dy, ck1, False, True)
+    for i in (0, 1, 2, 5, 6, 7):
+        assert g1[i].dtype == dtype and so.rel_err(g1[i].float().cpu(), g0[i].float().cpu()) < tol, i
+    for i, lg in ((3, logT), (4, logL)):
+        assert g1[i].dtype == torch.float32
+        want = g0[i].float() * -torch.exp(lg)          # dA/dA_log = A
+        assert so.rel_err(g1[i].cpu(), want.cpu()) < 2 * tol, i
+    assert g1[8].dtype == torch.float32 and so.rel_err(g1[8].cpu(), g0[8].float().cpu()) < tol
+
+
 def test_no_checkpoints_are_kept_under_no_grad(wf, monkeypatch):
     """Parameters keep requires_grad=True at inference; torch.no_grad() must still give the
     inference forward (no checkpoint buffer), for the plain Function and for the entry point."""
