@@ -73,6 +73,13 @@ typedef struct m2d_desc {
  * casts do (wavefront_cuda.py:90-91, 332).  d_AT, d_AL, d_D are then fp32 gradients with respect to
  * A_log and D. */
 #define M2D_FLAG_RAW_PARAMS 4
+/* B_T, B_L and C travel from m2d_proj_fwd to m2d_scan_fwd / m2d_scan_bwd in the form the scan
+ * kernels read, saving the scan its repacking pass: with this flag m2d_proj_fwd writes, to its BT
+ * argument, one fp32 record of 48 values per position (B,H,W,48) -- the values rounded to
+ * desc->dtype, in the library's own order -- and leaves BL and C alone (they may be NULL); the
+ * scan calls read those records through their BT argument and ignore BL and C.  The records are
+ * only meaningful to this library. */
+#define M2D_FLAG_PACKED_BC 8
 
 #define M2D_PASS_FWD 0
 #define M2D_PASS_BWD 1

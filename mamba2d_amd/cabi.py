@@ -17,6 +17,7 @@ M2D_F32, M2D_BF16 = 0, 1
 M2D_FLAG_FLIP = 1
 M2D_FLAG_ROUND_WEIGHTS = 2
 M2D_FLAG_RAW_PARAMS = 4
+M2D_FLAG_PACKED_BC = 8
 M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",

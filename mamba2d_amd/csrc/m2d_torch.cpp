@@ -21,7 +21,7 @@ namespace {
 
 using at::Tensor;
 
-m2d_desc describe(const Tensor& x, const Tensor& AT, bool flip, bool raw_params = false) {
+m2d_desc describe(const Tensor& x, const Tensor& AT, bool flip, bool raw_params = false, bool packed_bc = false) {
   TORCH_CHECK(x.dim() == 4, "m2dscan: x must be (B,H,W,E), got ", x.sizes());
   TORCH_CHECK(AT.dim() == 2, "m2dscan: AT must be (E,N), got ", AT.sizes());
   m2d_desc d{};
@@ -33,7 +33,7 @@ m2d_desc describe(const Tensor& x, const Tensor& AT, bool flip, bool raw_params 
   if (x.scalar_type() == at::kFloat) d.dtype = M2D_F32;
   else if (x.scalar_type() == at::kBFloat16) d.dtype = M2D_BF16;
   else TORCH_CHECK(false, "m2dscan: float32 and bfloat16 are supported, got ", x.scalar_type());
-  d.flags = (flip ? M2D_FLAG_FLIP : 0) | (raw_params ? M2D_FLAG_RAW_PARAMS : 0);
+  d.flags = (flip ? M2D_FLAG_FLIP : 0) | (raw_params ? M2D_FLAG_RAW_PARAMS : 0) | (packed_bc ? M2D_FLAG_PACKED_BC : 0);
   return d;
 }
 
@@ -63,9 +63,15 @@ void expect_all(const m2d_desc& d, const Tensor& x, const Tensor& dT, const Tens
   expect(dL, "deltaL", x, {B, H, W, E});
   expect_param(AT, raw ? "AT_log" : "AT", x, {E, N}, raw);
   expect_param(AL, raw ? "AL_log" : "AL", x, {E, N}, raw);
-  expect(BT, "BT", x, {B, H, W, N});
-  expect(BL, "BL", x, {B, H, W, N});
-  expect(C, "C", x, {B, H, W, N});
+  if (d.flags & M2D_FLAG_PACKED_BC) {   // BT holds the records written by proj_fwd; BL and C are not read
+    TORCH_CHECK(BT.device() == x.device() && BT.scalar_type() == at::kFloat && BT.is_contiguous() &&
+                BT.sizes() == at::IntArrayRef({B, H, W, 3 * N}),
+                "m2dscan: packed B/C must be the contiguous float32 (B,H,W,48) tensor returned by proj_fwd");
+  } else {
+    expect(BT, "BT", x, {B, H, W, N});
+    expect(BL, "BL", x, {B, H, W, N});
+    expect(C, "C", x, {B, H, W, N});
+  }
   expect_param(D, "D", x, {E}, raw);
 }
 
@@ -77,8 +83,8 @@ Tensor bytes(size_t n, const Tensor& like) {
 
 std::tuple<Tensor, Tensor> scan_fwd(const Tensor& x, const Tensor& dT, const Tensor& dL, const Tensor& AT,
                                     const Tensor& AL, const Tensor& BT, const Tensor& BL, const Tensor& C,
-                                    const Tensor& D, bool save_ckpt, bool flip, bool raw_params) {
-  const m2d_desc d = describe(x, AT, flip, raw_params);
+                                    const Tensor& D, bool save_ckpt, bool flip, bool raw_params, bool packed_bc) {
+  const m2d_desc d = describe(x, AT, flip, raw_params, packed_bc);
   expect_all(d, x, dT, dL, AT, AL, BT, BL, C, D);
   check(m2d_desc_check(&d));
   c10::DeviceGuard guard(x.device());
@@ -95,8 +101,8 @@ std::tuple<Tensor, Tensor> scan_fwd(const Tensor& x, const Tensor& dT, const Ten
 
 std::vector<Tensor> scan_bwd(const Tensor& x, const Tensor& dT, const Tensor& dL, const Tensor& AT, const Tensor& AL,
                              const Tensor& BT, const Tensor& BL, const Tensor& C, const Tensor& D, const Tensor& dy,
-                             const Tensor& ckpt, bool flip, bool raw_params) {
-  const m2d_desc d = describe(x, AT, flip, raw_params);
+                             const Tensor& ckpt, bool flip, bool raw_params, bool packed_bc) {
+  const m2d_desc d = describe(x, AT, flip, raw_params, packed_bc);
   expect_all(d, x, dT, dL, AT, AL, BT, BL, C, D);
   expect(dy, "dy", x, x.sizes());
   check(m2d_desc_check(&d));
@@ -106,8 +112,10 @@ std::vector<Tensor> scan_bwd(const Tensor& x, const Tensor& dT, const Tensor& dL
                 "m2dscan: ckpt must be the byte tensor returned by scan_fwd");
   }
   c10::DeviceGuard guard(x.device());
+  const std::vector<int64_t> bc_shape = {d.B, d.H, d.W, d.N};
   std::vector<Tensor> g = {at::empty_like(x),  at::empty_like(dT), at::empty_like(dL), at::empty_like(AT), at::empty_like(AL),
-                           at::empty_like(BT), at::empty_like(BL), at::empty_like(C),  at::empty_like(D)};
+                           at::empty(bc_shape, x.options()), at::empty(bc_shape, x.options()), at::empty(bc_shape, x.options()),
+                           at::empty_like(D)};
   Tensor ws = bytes(m2d_scan_workspace_bytes(&d, M2D_PASS_BWD, have), x);
   hipStream_t st = c10::hip::getCurrentHIPStream(x.device().index()).stream();
   check(m2d_scan_bwd(&d, x.data_ptr(), dT.data_ptr(), dL.data_ptr(), AT.data_ptr(), AL.data_ptr(), BT.data_ptr(),
@@ -126,7 +134,7 @@ void expect_weight(const Tensor& t, const char* name, const Tensor& x, at::IntAr
   TORCH_CHECK(t.is_contiguous(), "m2dscan: ", name, " must be contiguous");
 }
 
-m2d_desc describe_proj(const Tensor& x, int64_t N, bool round_weights) {
+m2d_desc describe_proj(const Tensor& x, int64_t N, bool round_weights, bool packed_bc = false) {
   TORCH_CHECK(x.dim() == 4 && x.is_cuda() && x.is_contiguous(), "m2dscan: x must be a contiguous (B,H,W,E) tensor on the GPU");
   m2d_desc d{};
   d.B = static_cast<int32_t>(x.size(0));
@@ -137,13 +145,13 @@ m2d_desc describe_proj(const Tensor& x, int64_t N, bool round_weights) {
   if (x.scalar_type() == at::kFloat) d.dtype = M2D_F32;
   else if (x.scalar_type() == at::kBFloat16) d.dtype = M2D_BF16;
   else TORCH_CHECK(false, "m2dscan: float32 and bfloat16 are supported, got ", x.scalar_type());
-  d.flags = round_weights ? M2D_FLAG_ROUND_WEIGHTS : 0;
+  d.flags = (round_weights ? M2D_FLAG_ROUND_WEIGHTS : 0) | (packed_bc ? M2D_FLAG_PACKED_BC : 0);
   return d;
 }
 
 std::vector<Tensor> proj_fwd(const Tensor& x, const Tensor& Wx, const Tensor& wT, const Tensor& bT, const Tensor& wL,
-                             const Tensor& bL, int64_t N, bool round_weights) {
-  const m2d_desc d = describe_proj(x, N, round_weights);
+                             const Tensor& bL, int64_t N, bool round_weights, bool packed_bc) {
+  const m2d_desc d = describe_proj(x, N, round_weights, packed_bc);
   TORCH_CHECK(wT.dim() == 2, "m2dscan: dt_projT_w must be (E, dt_rank)");
   const int64_t B = d.B, H = d.H, W = d.W, E = d.E, R = wT.size(1);
   expect_weight(Wx, "x_proj_w", x, {2 * R + 3 * N, E});
@@ -152,9 +160,11 @@ std::vector<Tensor> proj_fwd(const Tensor& x, const Tensor& Wx, const Tensor& wT
   expect_weight(wL, "dt_projL_w", x, {E, R});
   expect_weight(bL, "dt_projL_b", x, {E});
   c10::DeviceGuard guard(x.device());
+  // packed: one float32 (B,H,W,48) tensor of records in the BT place, empty tensors for BL and C
   std::vector<Tensor> o = {at::empty({B, H, W, 2 * R}, x.options()), at::empty_like(x), at::empty_like(x),
-                           at::empty({B, H, W, N}, x.options()), at::empty({B, H, W, N}, x.options()),
-                           at::empty({B, H, W, N}, x.options())};
+                           packed_bc ? at::empty({B, H, W, 3 * N}, x.options().dtype(at::kFloat)) : at::empty({B, H, W, N}, x.options()),
+                           packed_bc ? at::empty({0}, x.options()) : at::empty({B, H, W, N}, x.options()),
+                           packed_bc ? at::empty({0}, x.options()) : at::empty({B, H, W, N}, x.options())};
   const size_t need = m2d_proj_workspace_bytes(&d, static_cast<int>(R), M2D_PASS_FWD);
   TORCH_CHECK(need > 0, "m2dscan: projection shapes outside what the kernels are built for (N = 16, dt_rank <= 32, E <= 4096)");
   Tensor ws = bytes(need, x);
@@ -205,11 +215,11 @@ int64_t abi_version() { return m2d_version(); }
 
 TORCH_LIBRARY(m2dscan, m) {
   m.def("scan_fwd(Tensor x, Tensor deltaT, Tensor deltaL, Tensor AT, Tensor AL, Tensor BT, Tensor BL, Tensor C, "
-        "Tensor D, bool save_ckpt, bool flip, bool raw_params=False) -> (Tensor, Tensor)");
+        "Tensor D, bool save_ckpt, bool flip, bool raw_params=False, bool packed_bc=False) -> (Tensor, Tensor)");
   m.def("scan_bwd(Tensor x, Tensor deltaT, Tensor deltaL, Tensor AT, Tensor AL, Tensor BT, Tensor BL, Tensor C, "
-        "Tensor D, Tensor dy, Tensor ckpt, bool flip, bool raw_params=False) -> Tensor[]");
+        "Tensor D, Tensor dy, Tensor ckpt, bool flip, bool raw_params=False, bool packed_bc=False) -> Tensor[]");
   m.def("proj_fwd(Tensor x, Tensor x_proj_w, Tensor dt_projT_w, Tensor dt_projT_b, Tensor dt_projL_w, Tensor dt_projL_b, "
-        "int d_state, bool round_weights) -> Tensor[]");
+        "int d_state, bool round_weights, bool packed_bc=False) -> Tensor[]");
   m.def("proj_bwd(Tensor x, Tensor lowrank, Tensor deltaT, Tensor deltaL, Tensor x_proj_w, Tensor dt_projT_w, "
         "Tensor dt_projL_w, Tensor d_deltaT, Tensor d_deltaL, Tensor d_BT, Tensor d_BL, Tensor d_C, Tensor(a!) dx, "
         "bool round_weights) -> Tensor[]");

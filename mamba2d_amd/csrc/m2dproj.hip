@@ -68,11 +68,20 @@ __device__ __forceinline__ float softplus_slope(float d) {
   return d < 0.0625f ? series : 1.f - exp_neg(-d);
 }
 
+// Where the scan kernels expect value n (0..47: B_T, B_L, C, 16 states each) inside a position's
+// record of 48 floats: the four states n = 4q + m, q = 0..3, that the scan's backward folds together
+// share a float4, in the order q = 0, 2, 1, 3 (the scan source calls this the fold order).
+__device__ __forceinline__ int record_slot(int n48) {
+  const int n = n48 & 15, q = n >> 2, m = n & 3;
+  return (n48 & ~15) + 4 * m + (q == 1 ? 2 : (q == 2 ? 1 : q));
+}
+
 struct ProjArgs {
   // activations, (P, .) row-major, element type T
   const void *x, *r, *dT, *dL;           // x (P,E); r (P,2R) = low-rank inputs of the two dt projections; delta (P,E)
   const void *ddT, *ddL, *dBT, *dBL, *dC;
   void *r_out, *dT_out, *dL_out, *BT_out, *BL_out, *C_out, *dx;
+  float* bc_packed;                      // (P,48) fp32 records for the scan kernels instead of BT_out, BL_out, C_out (or null)
   // packed weights, fp32, zero where padded
   const float *Wt;                       // [Epad][Opad]   Wx transposed
   const float *wTt, *wLt;                // [R][Epad]      dt weights transposed
@@ -313,8 +322,12 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_fwd_kernel(const ProjArgs a
     const float* z = zs + c * zst;
     for (int q = lane; q < R2; q += 64) st(r_out + p * R2 + q, z[q]);
     if (lane < 3 * kN) {
-      T* out = static_cast<T*>(lane < kN ? a.BT_out : (lane < 2 * kN ? a.BL_out : a.C_out));
-      st(out + p * kN + (lane & (kN - 1)), z[R2 + lane]);
+      if (a.bc_packed) {
+        a.bc_packed[p * (3 * kN) + record_slot(lane)] = as_stored(z[R2 + lane], r_out);
+      } else {
+        T* out = static_cast<T*>(lane < kN ? a.BT_out : (lane < 2 * kN ? a.BL_out : a.C_out));
+        st(out + p * kN + (lane & (kN - 1)), z[R2 + lane]);
+      }
     }
   }
 
@@ -563,7 +576,10 @@ __global__ __launch_bounds__(kThreads, M2D_PROJ_OCC) void m2d_proj_fwd_mfma_kern
       else if (o < R2) lowL[c * kLowStride + o - R] = h;
       if (c < rows) {
         if (o < R2) r_out[(uint32_t)(c * R2 + o)].v = h;
-        else if (o < a.O) bc[(uint32_t)(c * kN)].v = h;
+        else if (o < a.O) {
+          if (a.bc_packed) a.bc_packed[(p0 + c) * (3 * kN) + record_slot(oo)] = bf16_lo(h);
+          else bc[(uint32_t)(c * kN)].v = h;
+        }
       }
     }
   }
@@ -1088,7 +1104,7 @@ int check_proj(const m2d_desc* d, int R) {
   if (!d) return M2D_ERR_NULL_POINTER;
   if (d->B < 1 || d->H < 1 || d->W < 1 || d->E < 1 || d->N < 1 || R < 1) return M2D_ERR_BAD_SHAPE;
   if (d->N != kN || (d->dtype != M2D_F32 && d->dtype != M2D_BF16) || d->reserved != 0) return M2D_ERR_UNSUPPORTED;
-  if (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_ROUND_WEIGHTS | M2D_FLAG_RAW_PARAMS)) return M2D_ERR_UNSUPPORTED;
+  if (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_ROUND_WEIGHTS | M2D_FLAG_RAW_PARAMS | M2D_FLAG_PACKED_BC)) return M2D_ERR_UNSUPPORTED;
   if (R > kMaxR || d->E > 4096) return M2D_ERR_UNSUPPORTED;
   if ((int64_t)d->B * d->H * d->W >= ((int64_t)1 << 31) * kTP) return M2D_ERR_UNSUPPORTED;   // tiles counted in 32 bits
   return M2D_OK;
@@ -1215,7 +1231,9 @@ int m2d_proj_fwd(const m2d_desc* desc, int dt_rank, const void* x, const float* 
                  void* stream) {
   int rc = check_proj(desc, dt_rank);
   if (rc) return rc;
-  const void* req[] = {x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, lowrank, deltaT, deltaL, BT, BL, C, workspace};
+  const bool packed = (desc->flags & M2D_FLAG_PACKED_BC) != 0;   // B_T takes the records, B_L and C are not written
+  const void* req[] = {x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, lowrank, deltaT, deltaL, BT,
+                       packed ? BT : BL, packed ? BT : C, workspace};
   for (const void* q : req) if (!q) return M2D_ERR_NULL_POINTER;
   for (const void* q : req) if (misaligned(q, 16)) return M2D_ERR_MISALIGNED;
   if (misaligned(workspace, 256)) return M2D_ERR_MISALIGNED;
@@ -1246,6 +1264,7 @@ int m2d_proj_fwd(const m2d_desc* desc, int dt_rank, const void* x, const float* 
   a.x = x; a.Wt = k.Wt; a.wTt = k.wTt; a.wLt = k.wLt; a.bTp = k.bTp; a.bLp = k.bLp;
   a.Wb = k.Wb; a.wTb = k.wTb; a.wLb = k.wLb;
   a.r_out = lowrank; a.dT_out = deltaT; a.dL_out = deltaL; a.BT_out = BT; a.BL_out = BL; a.C_out = C;
+  a.bc_packed = packed ? static_cast<float*>(BT) : nullptr;
   if (desc->dtype == M2D_F32) return g.vec ? run_proj_fwd<float, true>(g, a, st) : run_proj_fwd<float, false>(g, a, st);
   return g.mfma ? run_proj_fwd_mfma(g, a, st) : run_proj_fwd<bf16_t, false>(g, a, st);
 }

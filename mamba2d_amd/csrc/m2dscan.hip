@@ -1329,6 +1329,7 @@ struct Geometry {
   int ips, vB, vH;                   // images per stack; number and height of what the kernels sweep
   int nbb, nlaunch;                  // sliced: blocks per band, launches per sweep
   size_t carry_fwd_bytes, carry_bwd_bytes;
+  bool packed_bc;
   size_t prep_bytes, bc_bytes, ckpt_diag_bytes, top_bytes, bot_bytes, part_bytes, pa_bytes, pd_bytes;
 };
 
@@ -1337,7 +1338,7 @@ int check_desc(const m2d_desc* d) {
   if (d->B < 1 || d->E < 1 || d->N < 1 || d->H < 2 || d->W < 2) return M2D_ERR_BAD_SHAPE;
   if (d->N != kN) return M2D_ERR_UNSUPPORTED;
   if (d->dtype != M2D_F32 && d->dtype != M2D_BF16) return M2D_ERR_UNSUPPORTED;
-  if (d->reserved != 0 || (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_RAW_PARAMS))) return M2D_ERR_UNSUPPORTED;
+  if (d->reserved != 0 || (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_RAW_PARAMS | M2D_FLAG_PACKED_BC))) return M2D_ERR_UNSUPPORTED;
   if ((int64_t)d->B * d->H * d->W >= ((int64_t)1 << 40)) return M2D_ERR_BAD_SHAPE;
   // one image is addressed with 32-bit byte offsets from its base (fp32: 4 bytes per element;
   // the widest per-cell record, the channel sums, is 192 bytes)
@@ -1412,7 +1413,8 @@ Geometry make_geometry(const m2d_desc* d) {
   g.stage_x = (d->E % (d->dtype == M2D_BF16 ? 8 : 4)) == 0;
   const size_t P = (size_t)d->B * d->H * d->W;
   g.prep_bytes = align_up(sizeof(float) * (kZeroFloats + (size_t)2 * d->E * kN + d->E));
-  g.bc_bytes = align_up(sizeof(float) * P * 48);
+  g.packed_bc = (d->flags & M2D_FLAG_PACKED_BC) != 0;   // the caller brings the records: nothing to reserve
+  g.bc_bytes = g.packed_bc ? 0 : align_up(sizeof(float) * P * 48);
   g.ckpt_diag_bytes = align_up(sizeof(float) * (size_t)B * g.nblk * d->E * kN * g.HB);
   const bool rows = g.nbands > 1 && !g.stacked;   // boundary rows travel between bands
   g.top_bytes = rows ? align_up(sizeof(float) * (size_t)(g.nbands - 1) * B * d->W * d->E * kN) : 0;
@@ -1483,10 +1485,12 @@ int launch_prep(ScanParams& sp, const m2d_desc* d, const void* AT, const void* A
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
-// Points sp.bt/bl/cc at the packed fp32 copy of B_T, B_L, C (made here unless `ready`).
+// Points sp.bt/bl/cc at the packed fp32 copy of B_T, B_L, C (made here unless `ready`, or brought
+// by the caller in place of B_T).
 template <typename T>
 int stage_bc(ScanParams& sp, const m2d_desc* d, const void* BT, const void* BL, const void* C, float* wide,
              bool ready, hipStream_t st) {
+  if (d->flags & M2D_FLAG_PACKED_BC) { wide = static_cast<float*>(const_cast<void*>(BT)); ready = true; }
   sp.bt = wide; sp.bl = wide + kN; sp.cc = wide + 2 * kN;
   sp.bc_stride = 48;
   if (ready) return M2D_OK;
@@ -1640,7 +1644,7 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
 extern "C" {
 
 
-int m2d_version(void) { return 400; }
+int m2d_version(void) { return 500; }
 
 const char* m2d_status_str(int status) {
   switch (status) {
@@ -1689,7 +1693,8 @@ int m2d_scan_fwd(const m2d_desc* desc, const void* x, const void* deltaT, const 
                  size_t ckpt_bytes, void* workspace, size_t workspace_bytes, void* stream) {
   int rc = check_desc(desc);
   if (rc) return rc;
-  const void* req[] = {x, deltaT, deltaL, AT, AL, BT, BL, C, D, y, workspace};
+  const bool packed = (desc->flags & M2D_FLAG_PACKED_BC) != 0;   // B_T carries the records, B_L and C are not read
+  const void* req[] = {x, deltaT, deltaL, AT, AL, BT, packed ? BT : BL, packed ? BT : C, D, y, workspace};
   for (const void* q : req) if (!q) return M2D_ERR_NULL_POINTER;
   for (const void* q : req) if (misaligned(q, 16)) return M2D_ERR_MISALIGNED;
   if (misaligned(workspace, 256) || (ckpt && misaligned(ckpt, 256))) return M2D_ERR_MISALIGNED;
@@ -1711,7 +1716,8 @@ int m2d_scan_bwd(const m2d_desc* desc, const void* x, const void* deltaT, const 
                  size_t workspace_bytes, void* stream) {
   int rc = check_desc(desc);
   if (rc) return rc;
-  const void* req[] = {x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, dx, d_deltaT, d_deltaL,
+  const bool packed = (desc->flags & M2D_FLAG_PACKED_BC) != 0;   // B_T carries the records, B_L and C are not read
+  const void* req[] = {x, deltaT, deltaL, AT, AL, BT, packed ? BT : BL, packed ? BT : C, D, dy, dx, d_deltaT, d_deltaL,
                        d_AT, d_AL, d_BT, d_BL, d_C, d_D, workspace};
   for (const void* q : req) if (!q) return M2D_ERR_NULL_POINTER;
   for (const void* q : req) if (misaligned(q, 16)) return M2D_ERR_MISALIGNED;

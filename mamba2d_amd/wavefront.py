@@ -53,21 +53,26 @@ def _ckpt_bytes(x, N, flip=False) -> int:
 
 
 @torch.library.register_fake("m2dscan::scan_fwd")
-def _scan_fwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, save_ckpt, flip, raw_params=False):
+def _scan_fwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, save_ckpt, flip, raw_params=False, packed_bc=False):
     n = _ckpt_bytes(x, AT.shape[1]) if save_ckpt else 1
     return torch.empty_like(x), x.new_empty((max(n, 1),), dtype=torch.uint8)
 
 
 @torch.library.register_fake("m2dscan::scan_bwd")
-def _scan_bwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt, flip, raw_params=False):
-    return [torch.empty_like(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D)]
+def _scan_bwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt, flip, raw_params=False, packed_bc=False):
+    bc = [x.new_empty((*x.shape[:3], AT.shape[1])) for _ in range(3)]
+    return [torch.empty_like(x), torch.empty_like(deltaT), torch.empty_like(deltaL), torch.empty_like(AT), torch.empty_like(AL),
+            *bc, torch.empty_like(D)]
 
 
 @torch.library.register_fake("m2dscan::proj_fwd")
-def _proj_fwd_fake(x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, d_state, round_weights):
+def _proj_fwd_fake(x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, d_state, round_weights, packed_bc=False):
     B, H, W, _ = x.shape
     R = dt_projT_w.shape[1]
-    bc = [x.new_empty((B, H, W, d_state)) for _ in range(3)]
+    if packed_bc:
+        bc = [x.new_empty((B, H, W, 3 * d_state), dtype=torch.float32), x.new_empty((0,)), x.new_empty((0,))]
+    else:
+        bc = [x.new_empty((B, H, W, d_state)) for _ in range(3)]
     return [x.new_empty((B, H, W, 2 * R)), torch.empty_like(x), torch.empty_like(x), *bc]
 
 
@@ -195,9 +200,10 @@ class wf_cuda_fn_proj(torch.autograd.Function):
         x = _c(x)
         raw = (AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D)
         At, Al, *w32, D32 = wf_cuda_fn_proj._params(x, *raw)
-        low, dT, dL, BT, BL, C = proj_fwd_op(x, *w32, AT_log.shape[1], True)
+        # B_T, B_L, C go from the projection kernel to the scan as packed records (BT) and two empty tensors
+        low, dT, dL, BT, BL, C = proj_fwd_op(x, *w32, AT_log.shape[1], True, True)
         keep = SAVE_CHECKPOINTS and not full and recording and any(ctx.needs_input_grad)
-        y, ck = scan_fwd_op(x, dT, dL, At, Al, BT, BL, C, D32, keep, bool(flip), True)
+        y, ck = scan_fwd_op(x, dT, dL, At, Al, BT, BL, C, D32, keep, bool(flip), True, True)
         if full:
             ctx.save_for_backward(x, *raw)
         else:
@@ -211,12 +217,13 @@ class wf_cuda_fn_proj(torch.autograd.Function):
         At, Al, *w32, D32 = wf_cuda_fn_proj._params(x, *raw)
         dy = _c(grad_output.to(x.dtype))
         if ctx.full:
-            low, dT, dL, BT, BL, C = proj_fwd_op(x, *w32, At.shape[1], True)
+            low, dT, dL, BT, BL, C = proj_fwd_op(x, *w32, At.shape[1], True, True)
             ck = x.new_empty((1,), dtype=torch.uint8)
         else:
             low, dT, dL, BT, BL, C, ck = ctx.saved_tensors[9:]
         # with raw parameters the gradients of A_log and D come back in fp32
-        d_x, d_dT, d_dL, d_At, d_Al, d_BT, d_BL, d_C, d_D = scan_bwd_op(x, dT, dL, At, Al, BT, BL, C, D32, dy, ck, ctx.flip, True)
+        d_x, d_dT, d_dL, d_At, d_Al, d_BT, d_BL, d_C, d_D = scan_bwd_op(x, dT, dL, At, Al, BT, BL, C, D32, dy, ck, ctx.flip,
+                                                                        True, True)
         # d_x holds the scan's own gradient (dy*D included); the projections add theirs in place
         g = proj_bwd_op(x, low, dT, dL, w32[0], w32[1], w32[3], d_dT, d_dL, d_BT, d_BL, d_C, d_x, True)
         grads = (d_At, d_Al, *g, d_D)

@@ -39,6 +39,8 @@ def test_projection_ops_on_meta_tensors(wf, dtype):
     assert low.shape == (B, H, W, 2 * R) and dT.shape == dL.shape == x.shape
     assert BT.shape == BL.shape == C.shape == (B, H, W, N)
     assert all(t.dtype == dtype for t in (low, dT, dL, BT, BL, C))
+    packed = wf.proj_fwd_op(x, *w, N, True, True)
+    assert packed[3].shape == (B, H, W, 3 * N) and packed[3].dtype == torch.float32 and packed[4].numel() == packed[5].numel() == 0
     g = wf.proj_bwd_op(x, low, dT, dL, w[0], w[1], w[3], dT, dL, BT, BL, C, torch.empty_like(x), True)
     assert [tuple(t.shape) for t in g] == [tuple(t.shape) for t in w]
     assert all(t.dtype == torch.float32 for t in g)

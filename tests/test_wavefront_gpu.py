@@ -136,6 +136,31 @@ def test_raw_parameters_match_cast_parameters(wf, dtype, tol):
     assert g1[8].dtype == torch.float32 and so.rel_err(g1[8].cpu(), g0[8].float().cpu()) < tol
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("E", [24, 12], ids=["matrix_core_shape", "vector_shape"])
+def test_packed_records_equal_separate_tensors(wf, dtype, E):
+    """M2D_FLAG_PACKED_BC: B_T, B_L, C handed from proj_fwd to the scan as records give bit for bit
+    the scan results of the three separate tensors."""
+    say(f"\ncase packed B/C {dtype} E={E}")
+    N, R = 16, math.ceil(E / 16)
+    p = make_block_params(E, N, R, 1, "cuda")
+    x = torch.randn(2, 9, 30, E, generator=torch.Generator().manual_seed(3)).cuda().to(dtype)
+    dy = torch.randn(2, 9, 30, E, generator=torch.Generator().manual_seed(4)).cuda().to(dtype)
+    w = [p[k] for k in ("x_proj_w", "dt_projT_w", "dt_projT_b", "dt_projL_w", "dt_projL_b")]
+    low, dT, dL, BT, BL, C = wf.proj_fwd_op(x, *w, N, True)
+    low2, dT2, dL2, rec, e1, e2 = wf.proj_fwd_op(x, *w, N, True, True)
+    assert torch.equal(dT, dT2) and torch.equal(low, low2) and rec.shape == (2, 9, 30, 48) and e1.numel() == 0
+    logs = [p["AT_log"], p["AL_log"]]
+    y0, ck0 = wf.scan_fwd_op(x, dT, dL, *logs, BT, BL, C, p["D"], True, False, True)
+    y1, ck1 = wf.scan_fwd_op(x, dT, dL, *logs, rec, e1, e2, p["D"], True, False, True, True)
+    assert torch.equal(y0, y1)
+    g0 = wf.scan_bwd_op(x, dT, dL, *logs, BT, BL, C, p["D"], dy, ck0, False, True)
+    g1 = wf.scan_bwd_op(x, dT, dL, *logs, rec, e1, e2, p["D"], dy, ck1, False, True, True)
+    g2 = wf.scan_bwd_op(x, dT, dL, *logs, rec, e1, e2, p["D"], dy, torch.empty(1, dtype=torch.uint8, device="cuda"), False, True, True)
+    for a, b, c in zip(g0, g1, g2):
+        assert a.shape == b.shape and torch.equal(a, b) and torch.equal(a, c)
+
+
 def test_no_checkpoints_are_kept_under_no_grad(wf, monkeypatch):
     """Parameters keep requires_grad=True at inference; torch.no_grad() must still give the
     inference forward (no checkpoint buffer), for the plain Function and for the entry point."""
