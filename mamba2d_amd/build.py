@@ -21,31 +21,46 @@ LIB = os.path.join(HERE, "libm2dscan.so")
 SHIM = os.path.join(HERE, "_m2d_torch.so")
 
 HIPCC_FLAGS = [
-    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     # packed fp32 VALU ops are kept out of the generated code on purpose
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result", "-Wno-inline-asm",
 ]
 
+# Source -> flags of its own.  The scan kernels are long straight-line VALU code at two waves per
+# SIMD: the iterative ILP scheduler orders the backward kernel 4 % faster than the default one
+# (0.92 -> 0.88 ms at B=128, E=64, 56x56, bf16) and costs the forward kernel 2 %.  The projection
+# kernels are memory-bound and do better with the default scheduler.
+SOURCES = {
+    "m2dscan.hip": ["-mllvm", "-amdgpu-sched-strategy=iterative-ilp"],
+    "m2dproj.hip": [],
+}
+
 
 def build_lib(verbose: bool = True) -> str:
-    """Compiles the two HIP sources into libm2dscan.so.  The device assembly of the same compile is
+    """Compiles the HIP sources into libm2dscan.so.  The device assembly of the same compile is
     kept (-save-temps) and checked for the hazards that inline assembly hides from the compiler
     (asmcheck.py); the library is only put in place if the check passes."""
     from . import asmcheck
-    srcs = [os.path.join(HERE, "csrc", n) for n in ("m2dscan.hip", "m2dproj.hip")]
     scratch = os.path.join(HERE, "build")   # in-tree, ignored by git
     os.makedirs(scratch, exist_ok=True)
     tmp = tempfile.mkdtemp(prefix="lib_", dir=scratch)
-    try:
-        out = os.path.join(tmp, "libm2dscan.so")
-        cmd = ["hipcc", *HIPCC_FLAGS, "-save-temps=obj", "-I", os.path.join(ROOT, "include"), "-o", out, *srcs]
+
+    def run(cmd):
         if verbose:
             print(" ".join(cmd), flush=True)
         subprocess.check_call(cmd, cwd=tmp)
+
+    try:
+        objs = []
+        for name, extra in SOURCES.items():
+            obj = os.path.join(tmp, name.replace(".hip", ".o"))
+            run(["hipcc", *HIPCC_FLAGS, *extra, "-save-temps=obj", "-I", os.path.join(ROOT, "include"),
+                 "-c", os.path.join(HERE, "csrc", name), "-o", obj])
+            objs.append(obj)
         listings = sorted(glob.glob(os.path.join(tmp, "*-hip-amdgcn-amd-amdhsa-gfx950.s")))
-        if len(listings) != len(srcs):
-            raise RuntimeError(f"expected the device assembly of {len(srcs)} sources, found {listings}")
+        if len(listings) != len(SOURCES):
+            raise RuntimeError(f"expected the device assembly of {len(SOURCES)} sources, found {listings}")
         for path in listings:
             ndpp, bad = asmcheck.check_file(path)
             if verbose:
@@ -53,6 +68,8 @@ def build_lib(verbose: bool = True) -> str:
             if bad:
                 raise RuntimeError("hazard between inline-assembly DPP instructions and their producers:\n" +
                                    "\n".join(f"  {k}: {p}  ->  {c}" for k, p, c in bad[:8]))
+        out = os.path.join(tmp, "libm2dscan.so")
+        run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out, *objs])
         shutil.move(out, LIB)
     finally:
         shutil.rmtree(tmp, ignore_errors=True)
