@@ -162,7 +162,7 @@ struct ScanParams {
   const float *A2T, *A2L, *Df;      // A*log2(e) and D in fp32, (E,16) / (E)
   const float* zeros;               // 256 bytes of zeros (source for out-of-grid staging chunks)
   void *y, *dx, *ddT, *ddL;
-  float* ckpt;                      // [B][nblk][E][16][16]          state snapshots, one per block of steps
+  float* ckpt;                      // [B][nblk][E][4][16][4]        state snapshots, one per block of steps: [q][row][w] = state sinv(4q+w)
   float* top;                       // [nbands-1][B][W][E][16]       last row of each band (forward states)
   float* bot;                       // [nbands or 1][B][W][E][16]    first-row muT of a band, for the band above (adjoint)
   float* part;                      // [G][P][3][16]                 per-workgroup channel sums of d_C, d_BT, d_BL
@@ -505,6 +505,14 @@ __device__ __forceinline__ bool special_boundary(const ScanParams& p, int bnd_lo
 }
 
 // ------------------------------------------------------------------------------------ forward
+// Store of a snapshot quad with the non-temporal hint: the data is read back once, by the backward
+// pass, long after it has left the caches, and as an ordinary store it costs the forward kernel
+// 0.02 ms at B=128, E=64, 56x56.
+typedef float f4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void store_snapshot(float4* dst, float a, float b, float c, float d) {
+  const f4v v = {a, b, c, d};
+  __builtin_nontemporal_store(v, reinterpret_cast<f4v*>(dst));
+}
 // Lanes are never masked in the forward: a grid row that is between bands, or a lane that is no
 // grid row, works on zero operands (its records come from the page of zeros), which keeps its
 // state finite and never reaches a cell of the grid: at column 0 the left gate is closed, and
@@ -647,6 +655,8 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
     settle_loads();
   }
 
+  bool ck_mine = false;       // the lane stores a snapshot in the first step of the current block
+  float4* ckp = nullptr;      // where to
   auto step = [&](int k, const Ops& o) {
     if (per_step_K) K = lane_consts<false>(p, clamp_band(p, k >= bp.kw ? bp.bnd0 + 1 : bp.bnd0), r, ch_ok);
     const bool col0 = bp.kz == k;
@@ -678,6 +688,9 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
         for (int w = 0; w < 4; ++w) aL[w] = fexp2(__builtin_fmaf(o.dlv[c], a2l[c][sinv<PERM>(4 * q + w)], offL));
         pin4(aL);
         __builtin_amdgcn_sched_barrier(0);
+        if (CKPT && k == 0 && ck_mine)   // the four states as they are before this step
+          store_snapshot(ckp + (c * 4 + q) * kHB, h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)],
+                         h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
           const int n = sinv<PERM>(4 * q + w);
@@ -702,7 +715,7 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
 #pragma unroll
           for (int q = 0; q < 4; ++q)
             tw[c * 4 + q] = make_float4(h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)],
-                                        h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
+                                              h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
       }
     }
     if (WRITE_Y && inr)
@@ -724,17 +737,17 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
     K = lane_consts<false>(p, clamp_band(p, bp.bnd0), r, ch_ok);
     per_step_K = __any(bp.kw < kCK && special_boundary(p, bp.bnd0, r));
     cell_off0 = (uint32_t)(cell_of(p, bp.bnd0, r, bp.col0) * p.E + e0) * (uint32_t)sizeof(T);
-    // snapshot of the state before the block (after step t0-1) for the lanes whose previous
-    // position was a cell of the grid; the others hold nothing the backward needs
+    // Snapshot of the state before the block (after step t0-1) for the lanes whose previous
+    // position was a cell of the grid; the others hold nothing the backward needs.  The stores are
+    // issued inside the first step, each group of four states just before it is overwritten: the
+    // waves of the whole grid run in step, and one burst of all snapshots would stall them.
+    ck_mine = false;
+    bool snapped = false;   // (uniform) the wave issues the 4*EC stores of a snapshot
     if (CKPT && m > 0) {
       Pos at; at.bnd = bp.bnd0; at.col = bp.col0;
-      if (snapshot_lane(p, at, r, ch_ok)) {
-        float* ck = p.ckpt + ((((int64_t)b * p.nblk + m) * p.E + e0) * kN) * kHB + r;
-#pragma unroll
-        for (int c = 0; c < EC; ++c)
-#pragma unroll
-          for (int n = 0; n < kN; ++n) ck[(c * kN + n) * kHB] = h[c][n];
-      }
+      ck_mine = snapshot_lane(p, at, r, ch_ok);
+      snapped = __any(ck_mine);
+      ckp = reinterpret_cast<float4*>(p.ckpt + ((((int64_t)b * p.nblk + m) * p.E + e0) * kN) * kHB) + r;
     }
     const char* bufc = lds + cur * SG::kBytes;
     const char* bufn = lds + (cur ^ 1) * SG::kBytes;
@@ -742,8 +755,12 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
     // three stores between the copies for the next block and the barrier that ends this one
     const bool y_thrice = WRITE_Y && __any((bp.in_grid & 7u) == 7u);
     auto next_block_landed = [&] {
-      // the stores just issued need not have completed, only the copies before them
-      if (y_thrice) staging_landed_behind<3>(); else staging_landed();
+      // the stores issued since (snapshot, y) need not have completed, only the copies before them
+      if (snapped) {
+        if (y_thrice) staging_landed_behind<4 * EC + 3>(); else staging_landed_behind<4 * EC>();
+      } else {
+        if (y_thrice) staging_landed_behind<3>(); else staging_landed();
+      }
     };
     if constexpr (AHEAD) {
       static_assert(kCK % 2 == 0, "the two operand sets alternate and must close over a block");
@@ -947,9 +964,13 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
 #pragma unroll
       for (int n = 0; n < kN; ++n) cknext[n] = 0.f;
     } else {
-      const float* ck = p.ckpt + ((((int64_t)b * p.nblk + mm) * p.E + e) * kN) * kHB + r;
+      const float4* ck = reinterpret_cast<const float4*>(p.ckpt + ((((int64_t)b * p.nblk + mm) * p.E + e) * kN) * kHB) + r;
 #pragma unroll
-      for (int n = 0; n < kN; ++n) cknext[n] = ck[n * kHB];
+      for (int q = 0; q < 4; ++q) {
+        const float4 v = ck[q * kHB];
+        cknext[sinv<PERM>(4 * q)] = v.x; cknext[sinv<PERM>(4 * q + 1)] = v.y;
+        cknext[sinv<PERM>(4 * q + 2)] = v.z; cknext[sinv<PERM>(4 * q + 3)] = v.w;
+      }
     }
   };
   auto pos_before = [&](Pos Q) {   // kCK positions earlier
