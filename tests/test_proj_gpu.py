@@ -130,3 +130,40 @@ def test_projection_limits_are_reported(cabi):
     assert cabi.lib.m2d_proj_workspace_bytes(ctypes.byref(d), 33, cabi.M2D_PASS_FWD) == 0     # dt_rank > 32
     d8 = cabi.Desc(1, 4, 4, 64, 8, cabi.M2D_F32, 0, 0)
     assert cabi.lib.m2d_proj_workspace_bytes(ctypes.byref(d8), 4, cabi.M2D_PASS_BWD) == 0    # d_state != 16
+
+
+def test_positions_beyond_two_giga_elements(cabi):
+    """Maximum sizes: P*E = 2.16e9 elements (more than 2^31).  Positions are independent, so an input that
+    repeats 256 seeded images 42 times must give, bit for bit, the outputs and dx of the 256 images
+    on their own; the weight gradients (sums over positions) must be 42 times theirs."""
+    say("\ncase proj beyond_two_giga_elements")
+    free, _ = torch.cuda.mem_get_info()
+    if free < 100 * 2**30:
+        pytest.skip("needs 100 GB of free device memory")
+    B0, reps, H, W, E = 256, 42, 56, 56, 64
+    R, x, w, up, _ = make_case(B0, H, W, E, seed=11, dtype=torch.bfloat16)
+    wd = {k: v.cuda() for k, v in w.items()}
+    x0 = x.cuda()
+    up0 = {k: v.cuda() for k, v in up.items()}
+    out0 = cabi.proj_fwd(x0, *[wd[k] for k in WNAMES], N)
+    dx0 = up0["dx"].clone()
+    gw0 = cabi.proj_bwd(x0, out0[0], out0[1], out0[2], wd["x_proj_w"], wd["dt_projT_w"], wd["dt_projL_w"],
+                        up0["d_deltaT"], up0["d_deltaL"], up0["d_BT"], up0["d_BL"], up0["d_C"], dx0)
+    xb = x0.repeat(reps, 1, 1, 1)
+    assert xb.numel() > 2**31
+    upb = {k: v.repeat(reps, 1, 1, 1) for k, v in up0.items()}
+    out = cabi.proj_fwd(xb, *[wd[k] for k in WNAMES], N)
+    dx = upb["dx"]   # read and written in place
+    gw = cabi.proj_bwd(xb, out[0], out[1], out[2], wd["x_proj_w"], wd["dt_projT_w"], wd["dt_projL_w"],
+                       upb["d_deltaT"], upb["d_deltaL"], upb["d_BT"], upb["d_BL"], upb["d_C"], dx)
+    torch.cuda.synchronize()
+    for r in range(reps):
+        for u, v in zip(out, out0):
+            assert torch.equal(u[r * B0:(r + 1) * B0], v), r
+        assert torch.equal(dx[r * B0:(r + 1) * B0], dx0), r
+    for k, g, s in zip(WNAMES, gw, gw0):
+        e = so.rel_err(g.cpu(), reps * s.cpu())
+        say(f"  {k} rel_err {e:.3e}")
+        assert e < 5e-4, (k, e)
+    del xb, upb, out, dx
+    torch.cuda.empty_cache()

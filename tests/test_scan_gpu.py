@@ -155,3 +155,40 @@ def test_linearity_at_full_size(cabi):
     err = (y12 - want).abs().max().item() / want.abs().max().item()
     say(f"  linearity err {err:.3e}")
     assert err < 2e-2
+
+
+def test_batch_beyond_two_giga_elements(cabi):
+    """Maximum sizes: B*H*W*E = 2.16e9 elements per (B,H,W,E) tensor (more than 2^31, 4.3 GB in bf16), so
+    element and byte offsets need 64 bits.  Images are independent, so a batch that repeats 256 seeded
+    images 42 times must reproduce, bit for bit, what the 256 images give on their own; the sums over
+    the batch (d_AT, d_AL, d_D) must be 42 times theirs."""
+    say("\ncase batch_beyond_two_giga_elements")
+    free, _ = torch.cuda.mem_get_info()
+    if free < 150 * 2**30:
+        pytest.skip("needs 150 GB of free device memory")
+    B0, reps, H, W, E = 256, 42, 56, 56, 64
+    small = {k: v.cuda() for k, v in so.make_inputs(B0, H, W, E, 16, seed=5, dtype=torch.bfloat16).items()}
+    a0 = [small[k] for k in so.INPUT_NAMES]
+    y0, ck0 = cabi.scan_fwd(*a0, save_ckpt=True)
+    g0 = cabi.scan_bwd(*a0, small["dy"], ckpt=ck0)
+    del ck0
+    per_image = ("x", "deltaT", "deltaL", "BT", "BL", "C", "dy")
+    big = {k: (v.repeat(reps, 1, 1, 1) if k in per_image else v) for k, v in small.items()}
+    assert big["x"].numel() > 2**31
+    a = [big[k] for k in so.INPUT_NAMES]
+    y, ck = cabi.scan_fwd(*a, save_ckpt=True)
+    grads = cabi.scan_bwd(*a, big["dy"], ckpt=ck)
+    torch.cuda.synchronize()
+    del ck
+    for r in range(reps):
+        assert torch.equal(y[r * B0:(r + 1) * B0], y0), ("y", r)
+    for k, g, s in zip(so.CScan.GRADS, grads, g0):
+        if g.ndim == 4:
+            for r in range(reps):
+                assert torch.equal(g[r * B0:(r + 1) * B0], s), (k, r)
+        else:
+            e = so.rel_err(g.float().cpu(), reps * s.float().cpu())
+            say(f"  {k} rel_err {e:.3e}")
+            assert e < 2e-2, (k, e)
+    del y, grads, big, a
+    torch.cuda.empty_cache()
