@@ -90,6 +90,8 @@ SHAPES = [
     (301, 7, 7, 4),   # 7x7 images stacked two to a band, last stack of one image
     (600, 14, 14, 4), # 14x14 images stacked three to a sweep, bands back to back with stride 14
     (900, 2, 5, 2),   # 2-row images, several to a band
+    (1, 512, 512, 2), # 37 bands of one large image (sliced sweep at the size of the latency benchmark's second point)
+    (2, 300, 260, 4), # 22 bands, two images
 ]
 
 
