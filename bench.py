@@ -40,6 +40,7 @@ WORKLOADS = {
 }
 N = 16
 HBM_PEAK_GBS = 8000.0
+VALU_PEAK_SLOTS = 38.3e12   # fp32 lane-operations per second of the whole device (measured)
 # HBM bytes per launch of the backward scan kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/scan_cfg1_kernel_trace_and_traffic.txt: 458158 KiB x 2.0 + 440541 KiB x 1.0); counters
 # cannot be read from inside this script, so the figure is carried here per workload.
@@ -196,12 +197,13 @@ def entry_point(args):
     ups = [torch.randn_like(t) for t in (outs[1], outs[2], outs[3], outs[4], outs[5])]
     dx = torch.zeros_like(xd)
     proj_fwd_ms = timed(lambda: cabi.proj_fwd(xd, *w32, N, round_weights=True))
-    proj_bwd_ms = timed(lambda: cabi.proj_bwd(xd, outs[0], outs[1], outs[2], w32[0], w32[1], w32[3], *ups, dx,
-                                              round_weights=True))
+    # as the entry point calls it: the scan hands over the gradients before the softplus, the deltas are not read
+    proj_bwd_ms = timed(lambda: cabi.proj_bwd(xd, outs[0], None, None, w32[0], w32[1], w32[3], *ups, dx,
+                                              round_weights=True, dpre=True))
     P, s = B * H * W, 2
     nw = (2 * R + 3 * N) * E + 2 * E * R + 2 * E
     proj_fwd_bytes = s * P * (E + 2 * R + 2 * E + 3 * N) + 4 * nw
-    proj_bwd_bytes = s * P * (E + 2 * R + 4 * E + 3 * N + 2 * E) + 8 * nw
+    proj_bwd_bytes = s * P * (E + 2 * R + 2 * E + 3 * N + 2 * E) + 8 * nw   # x, low-rank inputs, 2 dpre, dB_T dB_L dC, dx in and out
     out = {
         "metric": "wavefront_scan_cuda (projections + scan) fwd+bwd ms at B=128 D=64 56x56 N=16",
         "value": res["own"]["fwd_bwd_ms"], "unit": "ms",
@@ -355,6 +357,17 @@ def main():
             "fwd_kernel_ms": round(fwd_kernel_ms, 4),
             "fwd_kernel_frac": round(fb / (fwd_kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
         },
+    }
+    # Informational second ceiling: the scan is bounded by VALU issue, not by HBM.  Per (cell, channel,
+    # state) the forward needs 2 v_exp_f32 (2 issue slots each on gfx950) + 9 FMA-class operations = 13
+    # slots, the backward 11 for the recompute + 24 for the adjoint; the device issues 38.3e12 lane-slots/s
+    # (measured, profiles/microbench_gfx950.txt).
+    units = B * H * W * E * N
+    out["valu_ceiling"] = {
+        "peak_lane_slots_per_s": VALU_PEAK_SLOTS,
+        "fwd_slots_per_unit": 13, "bwd_slots_per_unit": 35, "units": units,
+        "fwd_kernel_frac": round(units * 13 / VALU_PEAK_SLOTS / (fwd_kernel_ms * 1e-3), 4),
+        "bwd_kernel_frac": round(units * 35 / VALU_PEAK_SLOTS / (bwd_kernel * 1e-3), 4),
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(B, E, H, W)

@@ -80,6 +80,12 @@ typedef struct m2d_desc {
  * scan calls read those records through their BT argument and ignore BL and C.  The records are
  * only meaningful to this library. */
 #define M2D_FLAG_PACKED_BC 8
+/* The gradients of the two step sizes travel from m2d_scan_bwd to m2d_proj_bwd as gradients with
+ * respect to what the softplus was applied to (wavefront_cuda.py:85-86): with this flag m2d_scan_bwd
+ * writes d_delta * (1 - exp(-delta)) to d_deltaT and d_deltaL, and m2d_proj_bwd takes its d_deltaT and
+ * d_deltaL arguments as such and does not read deltaT and deltaL (they may be NULL).  This saves
+ * m2d_proj_bwd reading the two step-size tensors and a pass of its own intermediate through memory. */
+#define M2D_FLAG_DPRE 16
 
 #define M2D_PASS_FWD 0
 #define M2D_PASS_BWD 1
@@ -136,8 +142,8 @@ int m2d_scan_bwd(const m2d_desc* desc,
  * The reference computes the scan's parameters from x with stock operators (proj_params,
  * models/kernels/wavefront_cuda.py:63-95) and differentiates them with autograd
  * (wavefront_cuda.py:262-296).  The two calls below do the same work in hand-written kernels.
- * desc->H and desc->W only enter through the number of positions P = B*H*W; of the flags only
- * M2D_FLAG_ROUND_WEIGHTS is read.  Activations have the element type of desc->dtype; weights,
+ * desc->H and desc->W only enter through the number of positions P = B*H*W; of the flags
+ * M2D_FLAG_ROUND_WEIGHTS, M2D_FLAG_PACKED_BC (forward) and M2D_FLAG_DPRE (backward) are read.  Activations have the element type of desc->dtype; weights,
  * biases and their gradients are fp32.  dt_rank <= 32, E <= 4096.
  *
  *   x_proj_w  (2*dt_rank + 3*N, E)     dt_proj{T,L}_w (E, dt_rank)     dt_proj{T,L}_b (E)

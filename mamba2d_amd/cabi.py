@@ -18,6 +18,7 @@ M2D_FLAG_FLIP = 1
 M2D_FLAG_ROUND_WEIGHTS = 2
 M2D_FLAG_RAW_PARAMS = 4
 M2D_FLAG_PACKED_BC = 8
+M2D_FLAG_DPRE = 16
 M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
@@ -154,11 +155,14 @@ def scan_fwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, save_ckpt=False, flip=Fals
     return (y, ck) if save_ckpt else y
 
 
-def scan_bwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt=None, flip=False):
-    """The nine gradients (order of the inputs) through m2d_scan_bwd."""
+def scan_bwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt=None, flip=False, dpre=False):
+    """The nine gradients (order of the inputs) through m2d_scan_bwd.  ``dpre``: d_deltaT and d_deltaL
+    come multiplied by the slope of the softplus that made the deltas (M2D_FLAG_DPRE)."""
     _same(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy)
     _shapes(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy)
     d = make_desc(x, AT.shape[1], flip)
+    if dpre:
+        d.flags |= M2D_FLAG_DPRE
     check(lib.m2d_desc_check(ctypes.byref(d)))
     outs = [torch.empty_like(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D)]
     ws = _bytes(lib.m2d_scan_workspace_bytes(ctypes.byref(d), M2D_PASS_BWD, int(ckpt is not None)), x.device)
@@ -199,22 +203,30 @@ def proj_fwd(x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, N=16, 
 
 
 def proj_bwd(x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w, dt_projL_w, d_deltaT, d_deltaL, d_BT, d_BL, d_C, dx,
-             round_weights=False):
+             round_weights=False, dpre=False):
     """Adds the gradient through the projections to ``dx`` in place and returns the five weight
-    gradients (x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b; float32) through m2d_proj_bwd."""
+    gradients (x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b; float32) through m2d_proj_bwd.
+    ``dpre``: d_deltaT and d_deltaL are gradients before the softplus (M2D_FLAG_DPRE); deltaT and deltaL
+    may then be None."""
     N = d_BT.shape[-1]
     zb = torch.zeros(x.shape[-1], device=x.device)
     R = _proj_check(x, x_proj_w, dt_projT_w, zb, dt_projL_w, zb, N)
     B, H, W, E = x.shape
-    _same(x, lowrank, deltaT, deltaL, d_deltaT, d_deltaL, d_BT, d_BL, d_C, dx)
-    want = {"lowrank": (lowrank, (B, H, W, 2 * R)), "deltaT": (deltaT, (B, H, W, E)), "deltaL": (deltaL, (B, H, W, E)),
+    given = [t for t in (deltaT, deltaL) if t is not None]
+    if not dpre and len(given) < 2:
+        raise ValueError("m2dscan: deltaT and deltaL are needed unless dpre is set")
+    _same(x, lowrank, *given, d_deltaT, d_deltaL, d_BT, d_BL, d_C, dx)
+    want = {"lowrank": (lowrank, (B, H, W, 2 * R)),
             "d_deltaT": (d_deltaT, (B, H, W, E)), "d_deltaL": (d_deltaL, (B, H, W, E)), "d_BT": (d_BT, (B, H, W, N)),
             "d_BL": (d_BL, (B, H, W, N)), "d_C": (d_C, (B, H, W, N)), "dx": (dx, (B, H, W, E))}
+    for k, t in zip(("deltaT", "deltaL"), (deltaT, deltaL)):
+        if t is not None:
+            want[k] = (t, (B, H, W, E))
     for k, (t, shp) in want.items():
         if tuple(t.shape) != shp:
             raise ValueError(f"m2dscan: {k} has shape {tuple(t.shape)}, expected {shp}")
     d = make_desc(x, N)
-    d.flags = M2D_FLAG_ROUND_WEIGHTS if round_weights else 0
+    d.flags = (M2D_FLAG_ROUND_WEIGHTS if round_weights else 0) | (M2D_FLAG_DPRE if dpre else 0)
     outs = [torch.empty_like(t) for t in (x_proj_w, dt_projT_w, zb, dt_projL_w, zb)]
     ws = _bytes(lib.m2d_proj_workspace_bytes(ctypes.byref(d), R, M2D_PASS_BWD), x.device)
     check(lib.m2d_proj_bwd(ctypes.byref(d), R, *[_ptr(t) for t in (x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w,

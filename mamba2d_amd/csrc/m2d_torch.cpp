@@ -21,7 +21,8 @@ namespace {
 
 using at::Tensor;
 
-m2d_desc describe(const Tensor& x, const Tensor& AT, bool flip, bool raw_params = false, bool packed_bc = false) {
+m2d_desc describe(const Tensor& x, const Tensor& AT, bool flip, bool raw_params = false, bool packed_bc = false,
+                  bool dpre = false) {
   TORCH_CHECK(x.dim() == 4, "m2dscan: x must be (B,H,W,E), got ", x.sizes());
   TORCH_CHECK(AT.dim() == 2, "m2dscan: AT must be (E,N), got ", AT.sizes());
   m2d_desc d{};
@@ -33,7 +34,8 @@ m2d_desc describe(const Tensor& x, const Tensor& AT, bool flip, bool raw_params 
   if (x.scalar_type() == at::kFloat) d.dtype = M2D_F32;
   else if (x.scalar_type() == at::kBFloat16) d.dtype = M2D_BF16;
   else TORCH_CHECK(false, "m2dscan: float32 and bfloat16 are supported, got ", x.scalar_type());
-  d.flags = (flip ? M2D_FLAG_FLIP : 0) | (raw_params ? M2D_FLAG_RAW_PARAMS : 0) | (packed_bc ? M2D_FLAG_PACKED_BC : 0);
+  d.flags = (flip ? M2D_FLAG_FLIP : 0) | (raw_params ? M2D_FLAG_RAW_PARAMS : 0) | (packed_bc ? M2D_FLAG_PACKED_BC : 0) |
+            (dpre ? M2D_FLAG_DPRE : 0);
   return d;
 }
 
@@ -101,8 +103,8 @@ std::tuple<Tensor, Tensor> scan_fwd(const Tensor& x, const Tensor& dT, const Ten
 
 std::vector<Tensor> scan_bwd(const Tensor& x, const Tensor& dT, const Tensor& dL, const Tensor& AT, const Tensor& AL,
                              const Tensor& BT, const Tensor& BL, const Tensor& C, const Tensor& D, const Tensor& dy,
-                             const Tensor& ckpt, bool flip, bool raw_params, bool packed_bc) {
-  const m2d_desc d = describe(x, AT, flip, raw_params, packed_bc);
+                             const Tensor& ckpt, bool flip, bool raw_params, bool packed_bc, bool dpre) {
+  const m2d_desc d = describe(x, AT, flip, raw_params, packed_bc, dpre);
   expect_all(d, x, dT, dL, AT, AL, BT, BL, C, D);
   expect(dy, "dy", x, x.sizes());
   check(m2d_desc_check(&d));
@@ -177,10 +179,11 @@ std::vector<Tensor> proj_fwd(const Tensor& x, const Tensor& Wx, const Tensor& wT
 
 std::vector<Tensor> proj_bwd(const Tensor& x, const Tensor& low, const Tensor& dT, const Tensor& dL, const Tensor& Wx,
                              const Tensor& wT, const Tensor& wL, const Tensor& ddT, const Tensor& ddL, const Tensor& dBT,
-                             const Tensor& dBL, const Tensor& dC, Tensor dx, bool round_weights) {
+                             const Tensor& dBL, const Tensor& dC, Tensor dx, bool round_weights, bool dpre) {
   TORCH_CHECK(dBT.dim() == 4 && wT.dim() == 2, "m2dscan: d_BT must be (B,H,W,N) and dt_projT_w (E, dt_rank)");
   const int64_t N = dBT.size(3);
-  const m2d_desc d = describe_proj(x, N, round_weights);
+  m2d_desc d = describe_proj(x, N, round_weights);
+  if (dpre) d.flags |= M2D_FLAG_DPRE;   // d_deltaT, d_deltaL are gradients before the softplus; deltaT, deltaL are not read
   const int64_t B = d.B, H = d.H, W = d.W, E = d.E, R = wT.size(1);
   expect_weight(Wx, "x_proj_w", x, {2 * R + 3 * N, E});
   expect_weight(wT, "dt_projT_w", x, {E, R});
@@ -217,12 +220,12 @@ TORCH_LIBRARY(m2dscan, m) {
   m.def("scan_fwd(Tensor x, Tensor deltaT, Tensor deltaL, Tensor AT, Tensor AL, Tensor BT, Tensor BL, Tensor C, "
         "Tensor D, bool save_ckpt, bool flip, bool raw_params=False, bool packed_bc=False) -> (Tensor, Tensor)");
   m.def("scan_bwd(Tensor x, Tensor deltaT, Tensor deltaL, Tensor AT, Tensor AL, Tensor BT, Tensor BL, Tensor C, "
-        "Tensor D, Tensor dy, Tensor ckpt, bool flip, bool raw_params=False, bool packed_bc=False) -> Tensor[]");
+        "Tensor D, Tensor dy, Tensor ckpt, bool flip, bool raw_params=False, bool packed_bc=False, bool dpre=False) -> Tensor[]");
   m.def("proj_fwd(Tensor x, Tensor x_proj_w, Tensor dt_projT_w, Tensor dt_projT_b, Tensor dt_projL_w, Tensor dt_projL_b, "
         "int d_state, bool round_weights, bool packed_bc=False) -> Tensor[]");
   m.def("proj_bwd(Tensor x, Tensor lowrank, Tensor deltaT, Tensor deltaL, Tensor x_proj_w, Tensor dt_projT_w, "
         "Tensor dt_projL_w, Tensor d_deltaT, Tensor d_deltaL, Tensor d_BT, Tensor d_BL, Tensor d_C, Tensor(a!) dx, "
-        "bool round_weights) -> Tensor[]");
+        "bool round_weights, bool dpre=False) -> Tensor[]");
   m.def("abi_version() -> int", &abi_version);
 }
 

@@ -80,6 +80,7 @@ struct ProjArgs {
   // activations, (P, .) row-major, element type T
   const void *x, *r, *dT, *dL;           // x (P,E); r (P,2R) = low-rank inputs of the two dt projections; delta (P,E)
   const void *ddT, *ddL, *dBT, *dBL, *dC;
+  int dpre_given;                        // ddT, ddL hold the gradients before the softplus already (dT, dL are not read)
   void *r_out, *dT_out, *dL_out, *BT_out, *BL_out, *C_out, *dx;
   float* bc_packed;                      // (P,48) fp32 records for the scan kernels instead of BT_out, BL_out, C_out (or null)
   // packed weights, fp32, zero where padded
@@ -383,6 +384,8 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_data_kernel(const ProjA
   const T* dL = static_cast<const T*>(a.dL);
   const T* ddT = static_cast<const T*>(a.ddT);
   const T* ddL = static_cast<const T*>(a.ddL);
+  const bool given = a.dpre_given != 0;   // (uniform) ddT, ddL are dpre already
+  const int64_t Pv = given ? 0 : a.P;     // rows of deltaT, deltaL to read: none then
 
   // dB_T, dB_L, dC of the tile: 64 x 16 contiguous elements each, 4 per thread
   float bc[3][4];
@@ -405,11 +408,11 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_data_kernel(const ProjA
   for (int kc = 0; kc < nkc; ++kc) {
     typename TL::Regs gT, vT, gL, vL;
     TL::load(gT, ddT, p0, a.P, a.E, kc * kKC, tid);
-    TL::load(vT, dT, p0, a.P, a.E, kc * kKC, tid);
+    TL::load(vT, dT, p0, Pv, a.E, kc * kKC, tid);
     TL::load(gL, ddL, p0, a.P, a.E, kc * kKC, tid);
-    TL::load(vL, dL, p0, a.P, a.E, kc * kKC, tid);
-    TL::to_lds(dps, kXS, tid, [&](int l, int j) { return TL::get(gT, l, j) * softplus_slope(TL::get(vT, l, j)); });
-    TL::to_lds(dps + kTP * kXS, kXS, tid, [&](int l, int j) { return TL::get(gL, l, j) * softplus_slope(TL::get(vL, l, j)); });
+    TL::load(vL, dL, p0, Pv, a.E, kc * kKC, tid);
+    TL::to_lds(dps, kXS, tid, [&](int l, int j) { return TL::get(gT, l, j) * (given ? 1.f : softplus_slope(TL::get(vT, l, j))); });
+    TL::to_lds(dps + kTP * kXS, kXS, tid, [&](int l, int j) { return TL::get(gL, l, j) * (given ? 1.f : softplus_slope(TL::get(vL, l, j))); });
     __syncthreads();
 #pragma unroll
     for (int rd = 0; rd < kMaxRounds; ++rd) {
@@ -640,6 +643,7 @@ __global__ __launch_bounds__(kThreads, M2D_PROJ_OCC) void m2d_proj_bwd_data_mfma
   uint16_t* dptT = a.dpt + p0 * a.E;
   uint16_t* dptL = dptT + (int64_t)a.ntiles * kTP * a.E;
   const uint4 z4 = make_uint4(0, 0, 0, 0);
+  const bool given = a.dpre_given != 0;   // (uniform) ddT, ddL are dpre already: nothing to derive or to write out
 
   // Memory latency is covered by the other waves of the compute unit (registers are kept low
   // for that), not by fetching ahead.
@@ -667,15 +671,18 @@ __global__ __launch_bounds__(kThreads, M2D_PROJ_OCC) void m2d_proj_bwd_data_mfma
   for (int e = 8 * kb; e < a.Epad; e += 32) {
     const bool ok = mn < rows && e < a.E;
     const uint32_t off = (uint32_t)(mn * a.E + e);
-    const uint4 gT = ok ? load16(ddT + off) : z4, vT = ok ? load16(dT + off) : z4;
-    const uint4 gL = ok ? load16(ddL + off) : z4, vL = ok ? load16(dL + off) : z4;
-    const uint4 AT = dpre(gT, vT), AL = dpre(gL, vL);
+    uint4 AT = ok ? load16(ddT + off) : z4, AL = ok ? load16(ddL + off) : z4;
+    if (!given) {
+      AT = dpre(AT, ok ? load16(dT + off) : z4);
+      AL = dpre(AL, ok ? load16(dL + off) : z4);
+    }
 #pragma unroll
     for (int nq = 0; nq < 2; ++nq)
       if (nq < NQ) {
         accT[nq] = mfma16(AT, load16(a.wTtb + (16 * nq + mn) * a.Epad + e), accT[nq]);
         accL[nq] = mfma16(AL, load16(a.wLtb + (16 * nq + mn) * a.Epad + e), accL[nq]);
       }
+    if (given) continue;   // the weight-gradient kernel reads the caller's arrays
     // dpre leaves through LDS, 64 channels at a time, so that memory sees whole 128-byte rows
     uint16_t* pst = reinterpret_cast<uint16_t*>(stage);
     *reinterpret_cast<uint4*>(pst + mn * kStageStride + (e & 63)) = AT;
@@ -783,7 +790,10 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_weights_mfma_kernel(con
   if (tid < 2 * kTP) rT[(tid >> 6) * rblk + R * kPosStride + (tid & 63)] = 0x3F80;   // 1.0
   const bf16_t* x = static_cast<const bf16_t*>(a.x);
   const bf16_t* rr = static_cast<const bf16_t*>(a.r);
-  const uint16_t* dptL = a.dpt + (int64_t)a.ntiles * kTP * a.E;
+  // dpre: the copy the data kernel wrote for whole tiles, or the caller's arrays (P rows)
+  const bool given = a.dpre_given != 0;
+  const uint16_t* dptT = given ? static_cast<const uint16_t*>(a.ddT) : a.dpt;
+  const uint16_t* dptL = given ? static_cast<const uint16_t*>(a.ddL) : a.dpt + (int64_t)a.ntiles * kTP * a.E;
 
   // this thread's part of the r tile (64 x 2R values, contiguous): up to two 16-byte pieces
   int rp[2], rq[2];
@@ -814,9 +824,10 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_weights_mfma_kernel(con
       const int e = ey * kKC + 8 * (2 * wave + k);
       const bool ok = e < a.E;
       xr[k] = (l < left && ok) ? load16(x + (p0 + l) * a.E + e) : z4;
-      // dz and dpre are written for whole tiles (zeros past the end of the arrays)
-      pr[0][k] = ok ? load16(a.dpt + (p0 + l) * a.E + e) : z4;
-      pr[1][k] = ok ? load16(dptL + (p0 + l) * a.E + e) : z4;
+      // dz and the data kernel's dpre are written for whole tiles (zeros past the end of the arrays)
+      const bool pok = ok && (!given || l < left);
+      pr[0][k] = pok ? load16(dptT + (p0 + l) * a.E + e) : z4;
+      pr[1][k] = pok ? load16(dptL + (p0 + l) * a.E + e) : z4;
       const int first = 8 * (k * kThreads + tid);
       // a piece of r may straddle the end of the array, by whole values
       rv[k] = z4;
@@ -942,6 +953,8 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_weights_kernel(const Pr
   const T* dL = static_cast<const T*>(a.dL);
   const T* ddT = static_cast<const T*>(a.ddT);
   const T* ddL = static_cast<const T*>(a.ddL);
+  const bool given = a.dpre_given != 0;   // (uniform) ddT, ddL are dpre already
+  const int64_t Pv = given ? 0 : a.P;     // rows of deltaT, deltaL to read: none then
   const int nmt = (O4 / 4) * 16;   // 4 x 4 blocks of dWx: (o4, e4), e4 fastest
   constexpr int kZQ = (kTP * ((2 * kMaxR + 3 * kN + 3) / 4) + kThreads - 1) / kThreads;   // float4 of dz per thread, at most
   constexpr int kRQ = (kTP * 2 * kMaxR + kThreads - 1) / kThreads;                        // elements of r per thread, at most
@@ -963,9 +976,9 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_weights_kernel(const Pr
     const int64_t p0 = (int64_t)tile * kTP;
     TL::load(xr, x, p0, a.P, a.E, ey * kKC, tid);
     TL::load(gT, ddT, p0, a.P, a.E, ey * kKC, tid);
-    TL::load(vT, dT, p0, a.P, a.E, ey * kKC, tid);
+    TL::load(vT, dT, p0, Pv, a.E, ey * kKC, tid);
     TL::load(gL, ddL, p0, a.P, a.E, ey * kKC, tid);
-    TL::load(vL, dL, p0, a.P, a.E, ey * kKC, tid);
+    TL::load(vL, dL, p0, Pv, a.E, ey * kKC, tid);
     const int64_t left = a.P - p0;   // rows of the tile inside the array, if fewer than 64
     const float4* zsrc = reinterpret_cast<const float4*>(a.dz + p0 * O4);
 #pragma unroll
@@ -983,8 +996,8 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_weights_kernel(const Pr
   if ((int)blockIdx.x < a.ntiles) fetch(blockIdx.x);
   for (int tile = blockIdx.x; tile < a.ntiles; tile += a.G) {
     TL::to_lds(xs, kXS4, tid, [&](int l, int j) { return TL::get(xr, l, j); });
-    TL::to_lds(dpT, kXS, tid, [&](int l, int j) { return TL::get(gT, l, j) * softplus_slope(TL::get(vT, l, j)); });
-    TL::to_lds(dpL, kXS, tid, [&](int l, int j) { return TL::get(gL, l, j) * softplus_slope(TL::get(vL, l, j)); });
+    TL::to_lds(dpT, kXS, tid, [&](int l, int j) { return TL::get(gT, l, j) * (given ? 1.f : softplus_slope(TL::get(vT, l, j))); });
+    TL::to_lds(dpL, kXS, tid, [&](int l, int j) { return TL::get(gL, l, j) * (given ? 1.f : softplus_slope(TL::get(vL, l, j))); });
 #pragma unroll
     for (int k = 0; k < kZQ; ++k) {
       const int i = k * kThreads + tid;
@@ -1104,7 +1117,7 @@ int check_proj(const m2d_desc* d, int R) {
   if (!d) return M2D_ERR_NULL_POINTER;
   if (d->B < 1 || d->H < 1 || d->W < 1 || d->E < 1 || d->N < 1 || R < 1) return M2D_ERR_BAD_SHAPE;
   if (d->N != kN || (d->dtype != M2D_F32 && d->dtype != M2D_BF16) || d->reserved != 0) return M2D_ERR_UNSUPPORTED;
-  if (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_ROUND_WEIGHTS | M2D_FLAG_RAW_PARAMS | M2D_FLAG_PACKED_BC)) return M2D_ERR_UNSUPPORTED;
+  if (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_ROUND_WEIGHTS | M2D_FLAG_RAW_PARAMS | M2D_FLAG_PACKED_BC | M2D_FLAG_DPRE)) return M2D_ERR_UNSUPPORTED;
   if (R > kMaxR || d->E > 4096) return M2D_ERR_UNSUPPORTED;
   if ((int64_t)d->B * d->H * d->W >= ((int64_t)1 << 31) * kTP) return M2D_ERR_UNSUPPORTED;   // tiles counted in 32 bits
   return M2D_OK;
@@ -1276,10 +1289,13 @@ int m2d_proj_bwd(const m2d_desc* desc, int dt_rank, const void* x, const void* l
                  float* d_dt_projL_b, void* workspace, size_t workspace_bytes, void* stream) {
   int rc = check_proj(desc, dt_rank);
   if (rc) return rc;
-  const void* req[] = {x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w, dt_projL_w, d_deltaT, d_deltaL, d_BT, d_BL, d_C,
+  const bool given = (desc->flags & M2D_FLAG_DPRE) != 0;   // d_deltaT, d_deltaL are dpre: deltaT, deltaL are not read
+  const void* req[] = {x, lowrank, x_proj_w, dt_projT_w, dt_projL_w, d_deltaT, d_deltaL, d_BT, d_BL, d_C,
                        dx, d_x_proj_w, d_dt_projT_w, d_dt_projT_b, d_dt_projL_w, d_dt_projL_b, workspace};
   for (const void* q : req) if (!q) return M2D_ERR_NULL_POINTER;
+  if (!given && (!deltaT || !deltaL)) return M2D_ERR_NULL_POINTER;
   for (const void* q : req) if (misaligned(q, 16)) return M2D_ERR_MISALIGNED;
+  if (!given && (misaligned(deltaT, 16) || misaligned(deltaL, 16))) return M2D_ERR_MISALIGNED;
   if (misaligned(workspace, 256)) return M2D_ERR_MISALIGNED;
   const ProjGeometry g = proj_geometry(desc, dt_rank);
   if (workspace_bytes < g.bytes_bwd) return M2D_ERR_WORKSPACE;
@@ -1304,7 +1320,7 @@ int m2d_proj_bwd(const m2d_desc* desc, int dt_rank, const void* x, const void* l
   if (!launched()) return M2D_ERR_HIP;
   ProjArgs a = {};
   fill(a, g);
-  a.x = x; a.r = lowrank; a.dT = deltaT; a.dL = deltaL;
+  a.x = x; a.r = lowrank; a.dT = deltaT; a.dL = deltaL; a.dpre_given = given ? 1 : 0;
   a.ddT = d_deltaT; a.ddL = d_deltaL; a.dBT = d_BT; a.dBL = d_BL; a.dC = d_C; a.dx = dx;
   a.Wp = k.Wp; a.wTp = k.wTp; a.wLp = k.wLp;
   a.wTtb = k.wTtb; a.wLtb = k.wLtb; a.WxTb = k.WxTb;

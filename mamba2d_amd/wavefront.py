@@ -59,7 +59,7 @@ def _scan_fwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, save_ckpt, flip, raw
 
 
 @torch.library.register_fake("m2dscan::scan_bwd")
-def _scan_bwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt, flip, raw_params=False, packed_bc=False):
+def _scan_bwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt, flip, raw_params=False, packed_bc=False, dpre=False):
     bc = [x.new_empty((*x.shape[:3], AT.shape[1])) for _ in range(3)]
     return [torch.empty_like(x), torch.empty_like(deltaT), torch.empty_like(deltaL), torch.empty_like(AT), torch.empty_like(AL),
             *bc, torch.empty_like(D)]
@@ -78,7 +78,7 @@ def _proj_fwd_fake(x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, 
 
 @torch.library.register_fake("m2dscan::proj_bwd")
 def _proj_bwd_fake(x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w, dt_projL_w, d_deltaT, d_deltaL, d_BT, d_BL, d_C, dx,
-                   round_weights):
+                   round_weights, dpre=False):
     b = dt_projT_w.new_empty((x.shape[-1],))
     return [torch.empty_like(x_proj_w), torch.empty_like(dt_projT_w), b, torch.empty_like(dt_projL_w), torch.empty_like(b)]
 
@@ -221,11 +221,12 @@ class wf_cuda_fn_proj(torch.autograd.Function):
             ck = x.new_empty((1,), dtype=torch.uint8)
         else:
             low, dT, dL, BT, BL, C, ck = ctx.saved_tensors[9:]
-        # with raw parameters the gradients of A_log and D come back in fp32
+        # with raw parameters the gradients of A_log and D come back in fp32; the gradients of the two
+        # step sizes come back as gradients before the softplus, which is what the projections' backward wants
         d_x, d_dT, d_dL, d_At, d_Al, d_BT, d_BL, d_C, d_D = scan_bwd_op(x, dT, dL, At, Al, BT, BL, C, D32, dy, ck, ctx.flip,
-                                                                        True, True)
+                                                                        True, True, True)
         # d_x holds the scan's own gradient (dy*D included); the projections add theirs in place
-        g = proj_bwd_op(x, low, dT, dL, w32[0], w32[1], w32[3], d_dT, d_dL, d_BT, d_BL, d_C, d_x, True)
+        g = proj_bwd_op(x, low, dT, dL, w32[0], w32[1], w32[3], d_dT, d_dL, d_BT, d_BL, d_C, d_x, True, True)
         grads = (d_At, d_Al, *g, d_D)
         return (d_x, *[t.to(r.dtype) for t, r in zip(grads, raw)], None, None, None)
 

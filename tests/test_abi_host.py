@@ -50,9 +50,10 @@ def test_descriptor_validation(cabi):
     assert cabi.lib.m2d_desc_check(None) == 1
     # spatial dims must exceed 1, like the reference's ValueError (wavefront_cuda.py:323-324)
     assert chk(D(cabi, H=1)) == 2 and chk(D(cabi, W=1)) == 2 and chk(D(cabi, B=0)) == 2
-    # flags 1 (flip), 4 (raw parameters) and 8 (packed B/C) belong to the scan; 2 is a projection flag, 16 nobody's
-    assert chk(D(cabi, flags=4)) == 0 and chk(D(cabi, flags=13)) == 0 and chk(D(cabi, flags=2)) == 3
-    assert chk(D(cabi, N=8)) == 3 and chk(D(cabi, dtype=7)) == 3 and chk(D(cabi, flags=16)) == 3
+    # flags 1 (flip), 4 (raw parameters), 8 (packed B/C) and 16 (gradients before the softplus) belong to the
+    # scan; 2 is a projection flag, 32 nobody's
+    assert chk(D(cabi, flags=4)) == 0 and chk(D(cabi, flags=29)) == 0 and chk(D(cabi, flags=2)) == 3
+    assert chk(D(cabi, N=8)) == 3 and chk(D(cabi, dtype=7)) == 3 and chk(D(cabi, flags=32)) == 3
     assert chk(D(cabi, reserved=1)) == 3
     # one image must fit 32-bit offsets: H*W < 2^24 cells, H*W*E < 2^30 elements
     assert chk(D(cabi, B=1, H=4096, W=4096, E=8)) == 3 and chk(D(cabi, B=1, H=2048, W=2048, E=256)) == 3

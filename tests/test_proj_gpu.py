@@ -123,6 +123,33 @@ def test_library_rounds_weights_like_a_cast(cabi, shape):
         assert torch.equal(u, v)
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 2e-2)], ids=["f32", "bf16"])
+@pytest.mark.parametrize("shape", [(2, 14, 14, 64), (1, 40, 4, 100), (3, 7, 9, 24)], ids=lambda s: "x".join(map(str, s)))
+def test_gradients_before_the_softplus_are_accepted(cabi, shape, dtype, tol):
+    """M2D_FLAG_DPRE: handed d_delta * (1 - exp(-delta)) in place of d_delta, and no deltas, the backward gives
+    what it gives for d_delta and delta."""
+    say(f"\ncase proj dpre {shape} {dtype}")
+    B, H, W, E = shape
+    R, x, w, up, _ = make_case(B, H, W, E, seed=3, dtype=dtype)
+    xd = x.cuda()
+    wd = {k: v.cuda() for k, v in w.items()}
+    low, dT, dL, BT, BL, C = cabi.proj_fwd(xd, *[wd[k] for k in WNAMES], N)
+    upd = {k: v.cuda() for k, v in up.items()}
+    rest = (upd["d_BT"], upd["d_BL"], upd["d_C"])
+    dxa, dxb = upd["dx"].clone(), upd["dx"].clone()
+    ga = cabi.proj_bwd(xd, low, dT, dL, wd["x_proj_w"], wd["dt_projT_w"], wd["dt_projL_w"], upd["d_deltaT"], upd["d_deltaL"],
+                       *rest, dxa)
+    slope = lambda d: -torch.expm1(-d.double())
+    preT = (upd["d_deltaT"].double() * slope(dT)).to(dtype)
+    preL = (upd["d_deltaL"].double() * slope(dL)).to(dtype)
+    gb = cabi.proj_bwd(xd, low, None, None, wd["x_proj_w"], wd["dt_projT_w"], wd["dt_projL_w"], preT, preL, *rest, dxb,
+                       dpre=True)
+    torch.cuda.synchronize()
+    assert so.rel_err(dxb.float().cpu(), dxa.float().cpu()) < tol
+    for k, u, v in zip(WNAMES, ga, gb):
+        assert so.rel_err(v.cpu(), u.cpu()) < tol, k
+
+
 def test_projection_limits_are_reported(cabi):
     import ctypes
     d = cabi.Desc(1, 4, 4, 64, 16, cabi.M2D_F32, 0, 0)

@@ -141,6 +141,31 @@ def test_repeat_runs_are_bit_identical(cabi):
             assert torch.equal(u, v)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_gradients_before_the_softplus(cabi, dtype):
+    """M2D_FLAG_DPRE: d_deltaT and d_deltaL leave multiplied by 1 - exp(-delta), the slope of the softplus that
+    made the deltas; the other seven gradients are the same bits."""
+    say(f"\ncase dpre {dtype}")
+    inp = {k: v.cuda() for k, v in so.make_inputs(3, 30, 17, 12, 16, seed=9, dtype=dtype).items()}
+    # step sizes down to 1e-4, where 1 - exp(-delta) cancels
+    inp["deltaT"] = (inp["deltaT"].float() * torch.logspace(-4, 0, 12, device="cuda")).to(dtype)
+    a = [inp[k] for k in so.INPUT_NAMES]
+    y, ck = cabi.scan_fwd(*a, save_ckpt=True)
+    g0 = cabi.scan_bwd(*a, inp["dy"], ckpt=ck)
+    g1 = cabi.scan_bwd(*a, inp["dy"], ckpt=ck, dpre=True)
+    torch.cuda.synchronize()
+    for i, (k, u, v) in enumerate(zip(so.CScan.GRADS, g0, g1)):
+        if i in (1, 2):
+            delta = a[i].double()
+            want = (u.double() * -torch.expm1(-delta)).cpu()
+            # u is rounded to dtype before the product here and after it in the kernel
+            tol = 1e-5 if dtype == torch.float32 else 1e-2
+            assert so.rel_err(v.double().cpu(), want) < tol, k
+            assert so.elem_rel_err(v.double().cpu(), want) < (2e-3 if dtype == torch.float32 else 5e-2), k
+        else:
+            assert torch.equal(u, v), k
+
+
 def test_linearity_at_full_size(cabi):
     """Size-independent property at the benchmark shape (B=128, E=64, 56x56, bf16 in):
     y - D*x is linear in x for fixed delta, B, C."""
