@@ -11,6 +11,10 @@ inside inline assembly, so two rules of the ISA are the source's own responsibil
 
 The source arranges its code so that neither can happen; this module verifies it on the assembly
 that was actually produced, and the build fails if it finds a violation.
+
+It also reads the compiler's own per-kernel summary for register spills: the scan kernels are
+written to fit the 256 vector registers of a wave at two waves per SIMD, and a change that pushes
+one of them over the edge spills to scratch memory silently and costs tens of percent.
 """
 from __future__ import annotations
 
@@ -69,3 +73,26 @@ def check_text(text: str):
 def check_file(path: str):
     with open(path) as f:
         return check_text(f.read())
+
+
+_SCRATCH = re.compile(r"^\s*\.amdhsa_private_segment_fixed_size\s+(\d+)")
+_HSA_KERNEL = re.compile(r"^\s*\.amdhsa_kernel\s+(\S+)")
+
+
+def spilling_kernels(text: str):
+    """Kernels whose descriptor asks for scratch memory: list of (kernel, bytes per lane)."""
+    out, kernel = [], None
+    for line in text.splitlines():
+        k = _HSA_KERNEL.match(line)
+        if k:
+            kernel = k.group(1)
+            continue
+        m = _SCRATCH.match(line)
+        if m and int(m.group(1)) > 0:
+            out.append((kernel, int(m.group(1))))
+    return out
+
+
+def spills_in_file(path: str):
+    with open(path) as f:
+        return spilling_kernels(f.read())

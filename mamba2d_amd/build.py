@@ -68,6 +68,10 @@ def build_lib(verbose: bool = True) -> str:
             if bad:
                 raise RuntimeError("hazard between inline-assembly DPP instructions and their producers:\n" +
                                    "\n".join(f"  {k}: {p}  ->  {c}" for k, p, c in bad[:8]))
+            spills = asmcheck.spills_in_file(path)
+            if spills:
+                raise RuntimeError("kernels that spill registers to scratch memory:\n" +
+                                   "\n".join(f"  {k}: {n} bytes per lane" for k, n in spills[:8]))
         out = os.path.join(tmp, "libm2dscan.so")
         run(["hipcc", "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out, *objs])
         shutil.move(out, LIB)

@@ -497,6 +497,8 @@ constexpr int kLowStride = 40;   // bf16 per row of the low-rank scratch: 32 + 8
 __device__ __forceinline__ f32x4 mfma16(uint4 a, uint4 b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
 }
+// written out at every use: as a named constant the register allocator has kept it in scratch memory
+__device__ __forceinline__ uint4 zero16() { return make_uint4(0u, 0u, 0u, 0u); }
 __device__ __forceinline__ uint4 load16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
 __device__ __forceinline__ float bf16_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf16_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
@@ -814,7 +816,6 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_weights_mfma_kernel(con
     for (int nq = 0; nq < kMaxNQ1; ++nq) ar[h][nq] = (f32x4){0.f, 0.f, 0.f, 0.f};
   }
 
-  const uint4 z4 = make_uint4(0, 0, 0, 0);
   uint4 xr[2], pr[2][2], zr[kMaxZP], rv[2];
   auto fetch = [&](int tile) {
     const int64_t p0 = (int64_t)tile * kTP;
@@ -823,19 +824,20 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_weights_mfma_kernel(con
     for (int k = 0; k < 2; ++k) {
       const int e = ey * kKC + 8 * (2 * wave + k);
       const bool ok = e < a.E;
-      xr[k] = (l < left && ok) ? load16(x + (p0 + l) * a.E + e) : z4;
+      xr[k] = (l < left && ok) ? load16(x + (p0 + l) * a.E + e) : zero16();
       // dz and the data kernel's dpre are written for whole tiles (zeros past the end of the arrays)
       const bool pok = ok && (!given || l < left);
-      pr[0][k] = pok ? load16(dptT + (p0 + l) * a.E + e) : z4;
-      pr[1][k] = pok ? load16(dptL + (p0 + l) * a.E + e) : z4;
+      pr[0][k] = pok ? load16(dptT + (p0 + l) * a.E + e) : zero16();
+      pr[1][k] = pok ? load16(dptL + (p0 + l) * a.E + e) : zero16();
       const int first = 8 * (k * kThreads + tid);
       // a piece of r may straddle the end of the array, by whole values
-      rv[k] = z4;
+      rv[k] = zero16();
       if (first < nr) {
         if ((int64_t)(first + 8) <= left * R2) rv[k] = load16(rr + p0 * R2 + first);
         else if ((int64_t)first < left * R2) {
           uint32_t w[4] = {0, 0, 0, 0};
-          for (int j = 0; j < 8; ++j)
+#pragma unroll
+          for (int j = 0; j < 8; ++j)   // (unrolled: w stays in registers)
             if ((int64_t)(first + j) < left * R2) w[j >> 1] |= (uint32_t)rr[p0 * R2 + first + j].v << (16 * (j & 1));
           rv[k] = make_uint4(w[0], w[1], w[2], w[3]);
         }
@@ -844,7 +846,7 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_weights_mfma_kernel(con
 #pragma unroll
     for (int k = 0; k < kMaxZP; ++k) {
       const int o8 = wave + kWaves * k;
-      zr[k] = o8 < ZP ? load16(a.dzt + (p0 + l) * a.Opad + 8 * o8) : z4;
+      zr[k] = o8 < ZP ? load16(a.dzt + (p0 + l) * a.Opad + 8 * o8) : zero16();
     }
   };
   // lane = position: the 8 values of a 16-byte piece go to 8 consecutive rows of a position-last block
@@ -884,7 +886,7 @@ __global__ __launch_bounds__(kThreads) void m2d_proj_bwd_weights_mfma_kernel(con
     for (int ks = 0; ks < 2; ++ks) {
       const int koff = 32 * ks + 8 * kb;
       const uint4 A0 = load16(zT + (16 * wave + mn) * kPosStride + koff);
-      const uint4 A1 = wave + kWaves < MT ? load16(zT + (16 * (wave + kWaves) + mn) * kPosStride + koff) : z4;
+      const uint4 A1 = wave + kWaves < MT ? load16(zT + (16 * (wave + kWaves) + mn) * kPosStride + koff) : zero16();
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt) {
         const uint4 B = load16(xT + (16 * nt + mn) * kPosStride + koff);

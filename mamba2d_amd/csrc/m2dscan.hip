@@ -741,7 +741,6 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   if constexpr (AHEAD) fetch(lds, 0, opsA);
   int cur = 0;
   for (int m = m_lo; m < m_hi; ++m) {
-    const int t0 = m * kCK;
     const bool last = m + 1 == m_hi;
     if (!last)
       stage_block<T, 3, CW, false, true, STAGE_X, kFwdWaves, true>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, pos_after(p, A, kCK), e_wg0, wave, lane, X, DT, DL, DY);
@@ -778,7 +777,6 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
       static_assert(kCK % 2 == 0, "the two operand sets alternate and must close over a block");
 #pragma unroll
       for (int k = 0; k < kCK; ++k) {
-        const int t = t0 + k;
         Ops& now = (k & 1) ? opsB : opsA;
         Ops& ahead = (k & 1) ? opsA : opsB;
         if (k + 1 < kCK) {
@@ -791,20 +789,17 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
           __syncthreads();
           if (!last) fetch(bufn, 0, ahead);
         }
-        if (t < p.T_total) step(k, now);
+        step(k, now);   // also past the end of the sweep (last block): zero operands like any position off the grid, nothing stored
       }
     } else {
 #pragma unroll
       for (int k = 0; k < kCK; ++k) {
-        const int t = t0 + k;
         // The operands of the next block must have landed before the barrier that ends this
         // block.  Waiting here, before the stores of the last step are issued, keeps the latency
         // of those stores off the critical path (the counter covers loads and stores alike).
         if (k == kCK - 1) next_block_landed();
-        if (t < p.T_total) {
-          fetch(bufc, k, opsA);
-          step(k, opsA);
-        }
+        fetch(bufc, k, opsA);
+        step(k, opsA);
       }
       __syncthreads();
     }

@@ -41,3 +41,9 @@ def test_shifted_source_written_within_two_slots_is_reported():
 def test_histories_do_not_cross_kernels():
     text = listing("v_exp_f32_e32 v1, v1") + "_ZN1k3barEv:\n\tv_fmac_f32_dpp v9, v4, v1 row_shr:1\n"
     assert asmcheck.check_text(text)[1] == []
+
+
+def test_kernels_that_ask_for_scratch_memory_are_listed():
+    text = ("\t.amdhsa_kernel _ZN1k3fooEv\n\t\t.amdhsa_private_segment_fixed_size 0\n\t.end_amdhsa_kernel\n"
+            "\t.amdhsa_kernel _ZN1k3barEv\n\t\t.amdhsa_private_segment_fixed_size 932\n\t.end_amdhsa_kernel\n")
+    assert asmcheck.spilling_kernels(text) == [("_ZN1k3barEv", 932)]
