@@ -187,6 +187,49 @@ def test_no_checkpoints_are_kept_under_no_grad(wf, monkeypatch):
     assert seen[2:] == [wf.SAVE_CHECKPOINTS, wf.SAVE_CHECKPOINTS]
 
 
+@pytest.mark.parametrize("shape,dtype", [((1, 150, 90, 8), torch.float32), ((6, 30, 30, 64), torch.bfloat16)],
+                         ids=["sliced_f32", "batch_bf16"])
+def test_entry_point_replays_from_a_graph(wf, shape, dtype):
+    """The library allocates nothing and never synchronises, so a caller can capture forward and backward
+    in a HIP graph (here through torch).  Every replay, with eager work and synchronisations between the
+    replays, must give the bits of an eager run on the same inputs; the first shape is the sliced sweep
+    of one image (a sequence of 40 launches per pass)."""
+    say(f"\ncase graph {shape} {dtype}")
+    B, H, W, E = shape
+    N, R = 16, math.ceil(E / 16)
+    p = make_block_params(E, N, R, 0, "cuda")
+    gen = torch.Generator().manual_seed(1)
+    xs = [torch.randn(B, H, W, E, generator=gen).to(dtype).cuda() for _ in range(4)]
+    dy = torch.randn(B, H, W, E, generator=gen).to(dtype).cuda()
+    x = xs[0].clone().requires_grad_(True)
+    leaves = [x] + [p[k].clone().requires_grad_(True) for k in ORDER]
+
+    def run():
+        y = wf.wavefront_scan_cuda(*leaves)
+        return (y, *torch.autograd.grad(y, leaves, dy))
+
+    side = torch.cuda.Stream()   # default priority
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            run()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        outs = run()
+    for i in range(1, 4):
+        with torch.no_grad():
+            x.copy_(xs[i])
+        g.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in outs]
+        want = run()            # eager work between the replays
+        torch.cuda.synchronize()
+        for a, b in zip(got, want):
+            assert torch.equal(a, b), i
+
+
 def test_views_that_start_off_alignment_are_accepted(wf, cscan):
     """A contiguous view whose first element is not 16-byte aligned is copied, not rejected."""
     say("\ncase unaligned views")
