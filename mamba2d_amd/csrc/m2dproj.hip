@@ -47,19 +47,19 @@ __device__ __forceinline__ void st(bf16_t* p, float v) { p->v = f32_to_bf16_bits
 __device__ __forceinline__ float as_stored(float v, const float*) { return v; }
 __device__ __forceinline__ float as_stored(float v, const bf16_t*) { return __uint_as_float((uint32_t)f32_to_bf16_bits(v) << 16); }
 
-// exp, log and 1/x as the bare hardware instructions: the arguments below stay in ranges that
+// exp and log as the bare hardware instructions: the arguments below stay in ranges that
 // need none of the library's scaling (results that underflow may flush to zero).
 __device__ __forceinline__ float exp_neg(float v) { return __builtin_amdgcn_exp2f(v * 1.44269504088896341f); }   // v <= 0
-__device__ __forceinline__ float log_1to2(float u) { return __builtin_amdgcn_logf(u) * 0.693147180559945309f; }  // 1 <= u <= 2
-__device__ __forceinline__ float rcp_1to2(float u) { return __builtin_amdgcn_rcpf(u); }
 
 // softplus with torch's defaults (beta 1; above the threshold of 20 the two agree in fp32):
-// max(v,0) + log1p(t), t = exp(-|v|), with log1p(t) = log(u) + (t - (u-1))/u for u = fl(1+t),
-// which makes up for the rounding of 1+t when t is small.
+// max(v,0) + log1p(t), t = exp(-|v|), with log1p(t) = log(u) + (t - (u-1)) for u = fl(1+t): the
+// second term makes up for the rounding of 1+t when t is small.  (Exactly it would be divided by u;
+// it is at most half an ulp of u, 6e-8, and u lies in [1, 2], so leaving the division out changes
+// the result by less than 6e-8 t.)
 __device__ __forceinline__ float softplus(float v) {
   const float t = exp_neg(-fabsf(v));
   const float u = 1.f + t;
-  return fmaxf(v, 0.f) + __builtin_fmaf(t - (u - 1.f), rcp_1to2(u), log_1to2(u));
+  return fmaxf(v, 0.f) + __builtin_fmaf(__builtin_amdgcn_logf(u), 0.693147180559945309f, t - (u - 1.f));
 }
 // d softplus / d pre, from the softplus value: sigmoid(pre) = 1 - exp(-softplus(pre)).  Small
 // arguments take the series, where 1 - exp(-d) would cancel.
