@@ -176,6 +176,23 @@ int m2d_proj_bwd(const m2d_desc* desc, int dt_rank,
                  void* workspace, size_t workspace_bytes,
                  void* stream);
 
+/* ---- Two operators of the residual block around the scan (inference forward) -------------------
+ * The reference's blocks normalise channel-last activations with nn.LayerNorm over 64 to 512
+ * channels (models/mamba2d.py:57,220,248,363; models/utils.py:13,232-233) and run a depthwise 3x3
+ * convolution in the local path (models/utils.py:101-114).  Both are bandwidth-bound; these kernels
+ * read the input once and write the output once.  dtype is the element type of x and y, weight_dtype
+ * that of the weights (m2d_dtype each); arithmetic is fp32.  x and y must be 16-byte aligned.
+ *
+ * y[r,:] = (x[r,:] - mean) / sqrt(var + eps) * weight + bias over the C values of each of `rows` rows
+ * (biased variance, as nn.LayerNorm).  C must be a multiple of 8 (bf16) / 4 (fp32), at most 4096 / 2048. */
+int m2d_layernorm_fwd(int64_t rows, int C, int dtype, int weight_dtype,
+                      const void* x, const void* weight, const void* bias, float eps, void* y, void* stream);
+
+/* y = depthwise 3x3 cross-correlation of x (B,H,W,C), stride 1, zero padding 1, no bias; weight is the
+ * (C,1,3,3) tensor of nn.Conv2d(C, C, 3, padding=1, groups=C).  C must be a multiple of 8 (bf16) / 4 (fp32). */
+int m2d_dwconv3x3_fwd(int B, int H, int W, int C, int dtype, int weight_dtype,
+                      const void* x, const void* weight, void* y, void* stream);
+
 /* Measurement aid; no counterpart in the reference.  While enabled, every m2d_scan_fwd /
  * m2d_scan_bwd call records a pair of HIP events on its stream around the main scan kernel of
  * the pass (not around the small set-up and reduction kernels).  m2d_profile_last_ms waits for

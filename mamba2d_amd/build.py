@@ -34,6 +34,7 @@ HIPCC_FLAGS = [
 SOURCES = {
     "m2dscan.hip": ["-mllvm", "-amdgpu-sched-strategy=iterative-ilp"],
     "m2dproj.hip": [],
+    "m2dblock.hip": [],
 }
 
 

@@ -23,7 +23,7 @@ M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
            "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_bwd", "m2d_proj_workspace_bytes", "m2d_proj_fwd",
-           "m2d_proj_bwd", "m2d_profile_enable", "m2d_profile_last_ms")
+           "m2d_proj_bwd", "m2d_layernorm_fwd", "m2d_dwconv3x3_fwd", "m2d_profile_enable", "m2d_profile_last_ms")
 
 
 class Desc(ctypes.Structure):
@@ -63,6 +63,10 @@ def _load():
     lib.m2d_proj_fwd.argtypes = [dp, i32] + [vp] * 12 + [vp, sz, vp]
     lib.m2d_proj_bwd.restype = i32
     lib.m2d_proj_bwd.argtypes = [dp, i32] + [vp] * 18 + [vp, sz, vp]
+    lib.m2d_layernorm_fwd.restype = i32
+    lib.m2d_layernorm_fwd.argtypes = [ctypes.c_int64, i32, i32, i32, vp, vp, vp, ctypes.c_float, vp, vp]
+    lib.m2d_dwconv3x3_fwd.restype = i32
+    lib.m2d_dwconv3x3_fwd.argtypes = [i32, i32, i32, i32, i32, i32, vp, vp, vp, vp]
     lib.m2d_profile_enable.restype = i32
     lib.m2d_profile_enable.argtypes = [i32]
     lib.m2d_profile_last_ms.restype = i32
@@ -233,3 +237,39 @@ def proj_bwd(x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w, dt_projL_w, d_del
                                                                   dt_projL_w, d_deltaT, d_deltaL, d_BT, d_BL, d_C, dx)],
                            *[_ptr(t) for t in outs], _ptr(ws), ws.numel(), _stream(x.device)))
     return tuple(outs)
+
+
+def _dtype_code(t):
+    if t.dtype == torch.float32:
+        return M2D_F32
+    if t.dtype == torch.bfloat16:
+        return M2D_BF16
+    raise TypeError(f"m2dscan supports float32 and bfloat16, got {t.dtype}")
+
+
+def layernorm_fwd(x, weight, bias, eps=1e-5):
+    """LayerNorm over the last axis of a contiguous tensor through m2d_layernorm_fwd (inference forward)."""
+    C = x.shape[-1]
+    if not x.is_cuda or not x.is_contiguous():
+        raise ValueError("m2dscan: x must be a contiguous tensor on the GPU")
+    for k, t in (("weight", weight), ("bias", bias)):
+        if tuple(t.shape) != (C,) or t.device != x.device or not t.is_contiguous() or t.dtype != weight.dtype:
+            raise ValueError(f"m2dscan: {k} must be a contiguous ({C},) tensor on {x.device}, both of one dtype")
+    y = torch.empty_like(x)
+    check(lib.m2d_layernorm_fwd(x.numel() // C, C, _dtype_code(x), _dtype_code(weight), _ptr(x), _ptr(weight), _ptr(bias),
+                                float(eps), _ptr(y), _stream(x.device)))
+    return y
+
+
+def dwconv3x3_fwd(x, weight):
+    """Depthwise 3x3 convolution (padding 1, no bias) of a channel-last (B,H,W,C) tensor with the
+    (C,1,3,3) weight of nn.Conv2d(C, C, 3, padding=1, groups=C), through m2d_dwconv3x3_fwd."""
+    if x.dim() != 4 or not x.is_cuda or not x.is_contiguous():
+        raise ValueError("m2dscan: x must be a contiguous (B,H,W,C) tensor on the GPU")
+    B, H, W, C = x.shape
+    if tuple(weight.shape) != (C, 1, 3, 3) or weight.device != x.device or not weight.is_contiguous():
+        raise ValueError(f"m2dscan: weight must be a contiguous ({C},1,3,3) tensor on {x.device}")
+    y = torch.empty_like(x)
+    check(lib.m2d_dwconv3x3_fwd(B, H, W, C, _dtype_code(x), _dtype_code(weight), _ptr(x), _ptr(weight), _ptr(y),
+                                _stream(x.device)))
+    return y

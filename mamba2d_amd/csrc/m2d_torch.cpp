@@ -4,7 +4,8 @@
 // place of the reference's pair of in-place custom ops mamba2d::wf_fwd / mamba2d::wf_bwd
 // (models/kernels/wavefront_cuda.py:25-57) plus the tensor algebra around them, and
 // m2dscan::proj_fwd / m2dscan::proj_bwd for the projections that feed the scan
-// (wavefront_cuda.py:63-95 and their autograd backward).  The shim only
+// (wavefront_cuda.py:63-95 and their autograd backward), and m2dscan::layernorm_fwd /
+// m2dscan::dwconv3x3_fwd for two operators of the residual block at inference.  The shim only
 // validates tensors, allocates outputs / scratch through the caching allocator, picks the
 // current HIP stream and forwards raw pointers; all arithmetic lives behind the C ABI.
 #include <ATen/ATen.h>
@@ -212,6 +213,45 @@ std::vector<Tensor> proj_bwd(const Tensor& x, const Tensor& low, const Tensor& d
   return g;
 }
 
+// ---- operators of the residual block (inference forward)
+int dtype_code(const Tensor& t, const char* name) {
+  if (t.scalar_type() == at::kFloat) return M2D_F32;
+  if (t.scalar_type() == at::kBFloat16) return M2D_BF16;
+  TORCH_CHECK(false, "m2dscan: ", name, " must be float32 or bfloat16, got ", t.scalar_type());
+  return 0;
+}
+
+Tensor layernorm_fwd(const Tensor& x, const Tensor& weight, const Tensor& bias, double eps) {
+  TORCH_CHECK(x.is_cuda() && x.dim() >= 1 && x.is_contiguous(), "m2dscan: x must be a contiguous tensor on the GPU");
+  const int64_t C = x.size(-1);
+  TORCH_CHECK(weight.sizes() == at::IntArrayRef({C}) && bias.sizes() == at::IntArrayRef({C}) && weight.is_contiguous() &&
+              bias.is_contiguous() && weight.device() == x.device() && bias.device() == x.device() &&
+              weight.scalar_type() == bias.scalar_type(),
+              "m2dscan: weight and bias must be contiguous (", C, ",) tensors of one dtype on x's device");
+  c10::DeviceGuard guard(x.device());
+  Tensor y = at::empty_like(x);
+  if (x.numel() == 0) return y;
+  hipStream_t st = c10::hip::getCurrentHIPStream(x.device().index()).stream();
+  check(m2d_layernorm_fwd(x.numel() / C, static_cast<int>(C), dtype_code(x, "x"), dtype_code(weight, "weight"), x.data_ptr(),
+                          weight.data_ptr(), bias.data_ptr(), static_cast<float>(eps), y.data_ptr(), st));
+  return y;
+}
+
+Tensor dwconv3x3_fwd(const Tensor& x, const Tensor& weight) {
+  TORCH_CHECK(x.is_cuda() && x.dim() == 4 && x.is_contiguous(), "m2dscan: x must be a contiguous (B,H,W,C) tensor on the GPU");
+  const int64_t C = x.size(3);
+  TORCH_CHECK(weight.sizes() == at::IntArrayRef({C, 1, 3, 3}) && weight.is_contiguous() && weight.device() == x.device(),
+              "m2dscan: weight must be a contiguous (", C, ",1,3,3) tensor on x's device");
+  c10::DeviceGuard guard(x.device());
+  Tensor y = at::empty_like(x);
+  if (x.numel() == 0) return y;
+  hipStream_t st = c10::hip::getCurrentHIPStream(x.device().index()).stream();
+  check(m2d_dwconv3x3_fwd(static_cast<int>(x.size(0)), static_cast<int>(x.size(1)), static_cast<int>(x.size(2)),
+                          static_cast<int>(C), dtype_code(x, "x"), dtype_code(weight, "weight"), x.data_ptr(), weight.data_ptr(),
+                          y.data_ptr(), st));
+  return y;
+}
+
 int64_t abi_version() { return m2d_version(); }
 
 }  // namespace
@@ -226,6 +266,8 @@ TORCH_LIBRARY(m2dscan, m) {
   m.def("proj_bwd(Tensor x, Tensor lowrank, Tensor deltaT, Tensor deltaL, Tensor x_proj_w, Tensor dt_projT_w, "
         "Tensor dt_projL_w, Tensor d_deltaT, Tensor d_deltaL, Tensor d_BT, Tensor d_BL, Tensor d_C, Tensor(a!) dx, "
         "bool round_weights, bool dpre=False) -> Tensor[]");
+  m.def("layernorm_fwd(Tensor x, Tensor weight, Tensor bias, float eps) -> Tensor");
+  m.def("dwconv3x3_fwd(Tensor x, Tensor weight) -> Tensor");
   m.def("abi_version() -> int", &abi_version);
 }
 
@@ -234,4 +276,6 @@ TORCH_LIBRARY_IMPL(m2dscan, CUDA, m) {   // ROCm devices dispatch under the CUDA
   m.impl("scan_bwd", &scan_bwd);
   m.impl("proj_fwd", &proj_fwd);
   m.impl("proj_bwd", &proj_bwd);
+  m.impl("layernorm_fwd", &layernorm_fwd);
+  m.impl("dwconv3x3_fwd", &dwconv3x3_fwd);
 }

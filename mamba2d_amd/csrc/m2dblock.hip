@@ -1,0 +1,275 @@
+// m2dblock.hip -- the two memory-bound operators of an M2D residual block that the stock libraries
+// serve badly on gfx950 at this model's shapes: LayerNorm over a short channel axis (64 to 512
+// channels: models/mamba2d.py:57,220,248,363, models/utils.py:13,232-233) and the depthwise 3x3
+// convolution of the local path on channel-last tensors (models/utils.py:101-114).  Inference
+// forward only; both read every input byte once and write every output byte once.
+//
+// Layout: activations are row-major (rows, C) / (B, H, W, C), element type float or bf16; weights
+// are float or bf16, independently of the activations (a bf16 model holds bf16 weights, a fp32
+// model under autocast hands fp32 weights to bf16 activations).  Arithmetic is fp32.
+#include <hip/hip_runtime.h>
+
+#include <stdint.h>
+
+#include "../../include/m2dscan.h"
+
+namespace {
+
+struct bf16_t { uint16_t v; };
+
+__device__ __forceinline__ float bf_lo(uint32_t w) { return __uint_as_float(w << 16); }
+__device__ __forceinline__ float bf_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+  return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)lo) | ((uint32_t)__builtin_bit_cast(uint16_t, (__bf16)hi) << 16);
+}
+
+// A chunk is 16 bytes of a row: kV elements.
+template <typename T> struct Chunk;
+template <> struct Chunk<float> {
+  static constexpr int kV = 4;
+  static __device__ __forceinline__ void load(const float* p, float (&v)[4]) {
+    const float4 q = *reinterpret_cast<const float4*>(p);
+    v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
+    *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+  }
+};
+template <> struct Chunk<bf16_t> {
+  static constexpr int kV = 8;
+  static __device__ __forceinline__ void load(const bf16_t* p, float (&v)[8]) {
+    const uint4 q = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { v[2 * j] = bf_lo(w[j]); v[2 * j + 1] = bf_hi(w[j]); }
+  }
+  static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[8]) {
+    *reinterpret_cast<uint4*>(p) = make_uint4(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7]));
+  }
+};
+
+__device__ __forceinline__ float ldw(const void* w, int wbf16, int i) {
+  return wbf16 ? __uint_as_float((uint32_t)static_cast<const uint16_t*>(w)[i] << 16) : static_cast<const float*>(w)[i];
+}
+
+// ------------------------------------------------------------------------------------ LayerNorm
+// G lanes share a row (G a power of two, 4..64), lane g holds the chunks g, g + G, ... of it: at
+// most kMaxChunks of them, all in registers, so the row is read once.  Mean first, then the sum of
+// squared deviations (the data is at hand, and E[x^2] - mean^2 would cancel for rows far from zero).
+constexpr int kLnThreads = 256;
+constexpr int kMaxChunks = 8;
+
+struct LnArgs {
+  const void* x;
+  const void* w;
+  const void* b;
+  void* y;
+  int64_t rows;
+  int C, wbf16;
+  float eps;
+};
+
+template <typename T, int G, int NC>
+__global__ __launch_bounds__(kLnThreads) void m2d_layernorm_kernel(const LnArgs a) {
+  constexpr int V = Chunk<T>::kV;
+  const int lane_in_row = threadIdx.x & (G - 1);
+  const int row_in_block = threadIdx.x / G;
+  constexpr int kRows = kLnThreads / G;
+  const int nchunks = a.C / V;
+  const float inv_c = 1.f / (float)a.C;
+  // this lane's share of weight and bias, kept for all its rows
+  float wv[NC][V], bv[NC][V];
+#pragma unroll
+  for (int k = 0; k < NC; ++k) {
+    const int c = lane_in_row + k * G;
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      wv[k][j] = c < nchunks ? ldw(a.w, a.wbf16, c * V + j) : 0.f;
+      bv[k][j] = c < nchunks ? ldw(a.b, a.wbf16, c * V + j) : 0.f;
+    }
+  }
+  const T* X = static_cast<const T*>(a.x);
+  T* Y = static_cast<T*>(a.y);
+  for (int64_t row = (int64_t)blockIdx.x * kRows + row_in_block; row < a.rows; row += (int64_t)gridDim.x * kRows) {
+    float v[NC][V];
+    float s = 0.f;
+#pragma unroll
+    for (int k = 0; k < NC; ++k) {
+      const int c = lane_in_row + k * G;
+      if (c < nchunks) {
+        Chunk<T>::load(X + row * a.C + c * V, v[k]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j) v[k][j] = 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < V; ++j) s += v[k][j];
+    }
+#pragma unroll
+    for (int off = G >> 1; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+    const float mean = s * inv_c;
+    float q = 0.f;
+#pragma unroll
+    for (int k = 0; k < NC; ++k) {
+      const int c = lane_in_row + k * G;
+      if (c < nchunks) {
+#pragma unroll
+        for (int j = 0; j < V; ++j) { const float d = v[k][j] - mean; q = __builtin_fmaf(d, d, q); }
+      }
+    }
+#pragma unroll
+    for (int off = G >> 1; off > 0; off >>= 1) q += __shfl_xor(q, off, 64);
+    const float rstd = rsqrtf(q * inv_c + a.eps);
+#pragma unroll
+    for (int k = 0; k < NC; ++k) {
+      const int c = lane_in_row + k * G;
+      if (c < nchunks) {
+        float o[V];
+#pragma unroll
+        for (int j = 0; j < V; ++j) o[j] = __builtin_fmaf((v[k][j] - mean) * rstd, wv[k][j], bv[k][j]);
+        Chunk<T>::store(Y + row * a.C + c * V, o);
+      }
+    }
+  }
+}
+
+template <typename T, int G, int NC>
+int launch_ln(const LnArgs& a, hipStream_t st) {
+  constexpr int kRows = kLnThreads / G;
+  int64_t blocks = (a.rows + kRows - 1) / kRows;
+  if (blocks > 256 * 32) blocks = 256 * 32;   // grid-stride beyond that: the lane's weights are loaded once per block
+  hipLaunchKernelGGL((m2d_layernorm_kernel<T, G, NC>), dim3((unsigned)blocks), dim3(kLnThreads), 0, st, a);
+  return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+}
+
+template <typename T>
+int run_ln(const LnArgs& a, hipStream_t st) {
+  const int nchunks = a.C / Chunk<T>::kV;
+  // the fewest lanes per row that keep a lane's share within kMaxChunks, but at least 4 chunks in
+  // flight per row where the row is long enough
+  if (nchunks <= 4) return launch_ln<T, 4, 1>(a, st);
+  if (nchunks <= 8) return launch_ln<T, 8, 1>(a, st);
+  if (nchunks <= 16) return launch_ln<T, 16, 1>(a, st);
+  if (nchunks <= 32) return launch_ln<T, 16, 2>(a, st);
+  if (nchunks <= 64) return launch_ln<T, 16, 4>(a, st);
+  if (nchunks <= 128) return launch_ln<T, 32, 4>(a, st);
+  if (nchunks <= 256) return launch_ln<T, 64, 4>(a, st);
+  return launch_ln<T, 64, kMaxChunks>(a, st);
+}
+
+// ------------------------------------------------------------------ depthwise 3x3, channel-last
+// y[b,h,w,c] = sum_{i,j} wt[c][i][j] x[b,h+i-1,w+j-1,c], zero padding.  A thread owns one chunk of
+// channels and a strip of kStrip cells along W; the 3x3 window slides along the strip, so every
+// output costs three 16-byte loads, and the 9 x kV weights of the chunk stay in registers.
+constexpr int kDwThreads = 256;
+constexpr int kStrip = 8;
+
+struct DwArgs {
+  const void* x;
+  const void* w;    // (C, 1, 3, 3)
+  void* y;
+  int B, H, W, C, wbf16;
+  int strips;       // strips per image row
+};
+
+template <typename T>
+__global__ __launch_bounds__(kDwThreads) void m2d_dwconv3x3_kernel(const DwArgs a) {
+  constexpr int V = Chunk<T>::kV;
+  const int nchunks = a.C / V;
+  const int64_t total = (int64_t)a.B * a.H * a.strips * nchunks;
+  const int64_t gid = (int64_t)blockIdx.x * kDwThreads + threadIdx.x;
+  if (gid >= total) return;
+  const int c = (int)(gid % nchunks);
+  int64_t rest = gid / nchunks;
+  const int sidx = (int)(rest % a.strips);
+  rest /= a.strips;
+  const int h = (int)(rest % a.H);
+  const int b = (int)(rest / a.H);
+  float wt[9][V];
+#pragma unroll
+  for (int t = 0; t < 9; ++t)
+#pragma unroll
+    for (int j = 0; j < V; ++j) wt[t][j] = ldw(a.w, a.wbf16, (c * V + j) * 9 + t);
+  const T* X = static_cast<const T*>(a.x) + ((int64_t)b * a.H * a.W) * a.C + c * V;
+  T* Y = static_cast<T*>(a.y) + ((int64_t)b * a.H * a.W) * a.C + c * V;
+  const int w0 = sidx * kStrip;
+  // window columns: win[i][0..2] are the cells (h+i-1, w-1), (h+i-1, w), (h+i-1, w+1)
+  float win[3][3][V];
+  auto load_col = [&](int col, int slot) {
+#pragma unroll
+    for (int i = 0; i < 3; ++i) {
+      const int hh = h + i - 1;
+      if (hh >= 0 && hh < a.H && col >= 0 && col < a.W) {
+        Chunk<T>::load(X + ((int64_t)hh * a.W + col) * a.C, win[i][slot]);
+      } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j) win[i][slot][j] = 0.f;
+      }
+    }
+  };
+  load_col(w0 - 1, 0);
+  load_col(w0, 1);
+#pragma unroll
+  for (int s = 0; s < kStrip; ++s) {
+    const int w = w0 + s;
+    if (w >= a.W) break;
+    // slot of column w-1, w, w+1 rotates with s
+    const int sl = s % 3, sm = (s + 1) % 3, sr = (s + 2) % 3;
+    load_col(w + 1, sr);
+    float o[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      float acc = 0.f;
+#pragma unroll
+      for (int i = 0; i < 3; ++i) {
+        acc = __builtin_fmaf(wt[3 * i][j], win[i][sl][j], acc);
+        acc = __builtin_fmaf(wt[3 * i + 1][j], win[i][sm][j], acc);
+        acc = __builtin_fmaf(wt[3 * i + 2][j], win[i][sr][j], acc);
+      }
+      o[j] = acc;
+    }
+    Chunk<T>::store(Y + ((int64_t)h * a.W + w) * a.C, o);
+  }
+}
+
+inline bool misaligned(const void* p, size_t n) { return (reinterpret_cast<uintptr_t>(p) & (n - 1)) != 0; }
+
+}  // namespace
+
+extern "C" {
+
+int m2d_layernorm_fwd(int64_t rows, int C, int dtype, int weight_dtype, const void* x, const void* weight,
+                      const void* bias, float eps, void* y, void* stream) {
+  if (!x || !weight || !bias || !y) return M2D_ERR_NULL_POINTER;
+  if (rows < 1 || C < 1) return M2D_ERR_BAD_SHAPE;
+  if ((dtype != M2D_F32 && dtype != M2D_BF16) || (weight_dtype != M2D_F32 && weight_dtype != M2D_BF16)) return M2D_ERR_UNSUPPORTED;
+  const int V = dtype == M2D_BF16 ? 8 : 4;
+  if (C % V != 0 || C / V > 64 * kMaxChunks) return M2D_ERR_UNSUPPORTED;   // rows of whole 16-byte chunks, at most 4096 (bf16) / 2048 (fp32) channels
+  if (misaligned(x, 16) || misaligned(y, 16) || misaligned(weight, 4) || misaligned(bias, 4)) return M2D_ERR_MISALIGNED;
+  LnArgs a;
+  a.x = x; a.w = weight; a.b = bias; a.y = y; a.rows = rows; a.C = C; a.wbf16 = weight_dtype == M2D_BF16; a.eps = eps;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return dtype == M2D_F32 ? run_ln<float>(a, st) : run_ln<bf16_t>(a, st);
+}
+
+int m2d_dwconv3x3_fwd(int B, int H, int W, int C, int dtype, int weight_dtype, const void* x, const void* weight,
+                      void* y, void* stream) {
+  if (!x || !weight || !y) return M2D_ERR_NULL_POINTER;
+  if (B < 1 || H < 1 || W < 1 || C < 1) return M2D_ERR_BAD_SHAPE;
+  if ((dtype != M2D_F32 && dtype != M2D_BF16) || (weight_dtype != M2D_F32 && weight_dtype != M2D_BF16)) return M2D_ERR_UNSUPPORTED;
+  const int V = dtype == M2D_BF16 ? 8 : 4;
+  if (C % V != 0) return M2D_ERR_UNSUPPORTED;
+  if (misaligned(x, 16) || misaligned(y, 16) || misaligned(weight, 4)) return M2D_ERR_MISALIGNED;
+  DwArgs a;
+  a.x = x; a.w = weight; a.y = y; a.B = B; a.H = H; a.W = W; a.C = C; a.wbf16 = weight_dtype == M2D_BF16;
+  a.strips = (W + kStrip - 1) / kStrip;
+  const int64_t total = (int64_t)B * H * a.strips * (C / V);
+  const int64_t blocks = (total + kDwThreads - 1) / kDwThreads;
+  if (blocks >= ((int64_t)1 << 31)) return M2D_ERR_UNSUPPORTED;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == M2D_F32) hipLaunchKernelGGL(m2d_dwconv3x3_kernel<float>, dim3((unsigned)blocks), dim3(kDwThreads), 0, st, a);
+  else hipLaunchKernelGGL(m2d_dwconv3x3_kernel<bf16_t>, dim3((unsigned)blocks), dim3(kDwThreads), 0, st, a);
+  return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+}
+
+}  // extern "C"

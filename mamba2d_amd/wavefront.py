@@ -36,6 +36,8 @@ scan_fwd_op = torch.ops.m2dscan.scan_fwd
 scan_bwd_op = torch.ops.m2dscan.scan_bwd
 proj_fwd_op = torch.ops.m2dscan.proj_fwd
 proj_bwd_op = torch.ops.m2dscan.proj_bwd
+layernorm_fwd_op = torch.ops.m2dscan.layernorm_fwd
+dwconv3x3_fwd_op = torch.ops.m2dscan.dwconv3x3_fwd
 
 # Keep the forward's anti-diagonal checkpoints for the backward (faster backward, more saved
 # memory) or rebuild them inside the backward (nothing saved beyond the inputs, like the
@@ -81,6 +83,16 @@ def _proj_bwd_fake(x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w, dt_projL_w,
                    round_weights, dpre=False):
     b = dt_projT_w.new_empty((x.shape[-1],))
     return [torch.empty_like(x_proj_w), torch.empty_like(dt_projT_w), b, torch.empty_like(dt_projL_w), torch.empty_like(b)]
+
+
+@torch.library.register_fake("m2dscan::layernorm_fwd")
+def _layernorm_fwd_fake(x, weight, bias, eps):
+    return torch.empty_like(x)
+
+
+@torch.library.register_fake("m2dscan::dwconv3x3_fwd")
+def _dwconv3x3_fwd_fake(x, weight):
+    return torch.empty_like(x)
 
 
 def proj_params(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b):

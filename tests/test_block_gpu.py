@@ -1,0 +1,74 @@
+"""GPU parity of the two residual-block operators (m2d_layernorm_fwd, m2d_dwconv3x3_fwd) through the
+C ABI, against the stock torch operators the reference uses (nn.LayerNorm, models/mamba2d.py:220;
+depthwise nn.Conv2d, models/utils.py:101) evaluated in fp64 on the CPU.  Tolerances: fp32 2e-5,
+bf16 tensors 1e-2 (max error over max value; one bf16 rounding of the result is 4e-3)."""
+import pytest
+import torch
+
+from oracle import scan_oracle as so
+
+pytestmark = pytest.mark.gpu
+
+
+def say(*a):
+    print(*a, flush=True)
+
+
+@pytest.fixture(scope="module")
+def cabi():
+    from mamba2d_amd import cabi
+    return cabi
+
+
+TOL = {torch.float32: 2e-5, torch.bfloat16: 1e-2}
+
+# rows, channels: the block's widths (64 to 512), a head of the attention stages (32), one chunk, the largest row
+LN_SHAPES = [(2 * 9 * 12, 64), (1000, 128), (777, 320), (129, 512), (4 * 6 * 49, 32), (5, 8), (3, 2048), (1, 64), (70, 72)]
+
+
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16], ids=["w_f32", "w_bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("shape", LN_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_layernorm_matches_torch(cabi, shape, dtype, wdtype):
+    say(f"\ncase layernorm {shape} {dtype} {wdtype}")
+    rows, C = shape
+    g = torch.Generator().manual_seed(rows + C)
+    # rows away from zero with different spreads (a variance from E[x^2] - mean^2 would lose digits on them)
+    x = (torch.randn(rows, C, generator=g) * (torch.rand(rows, 1, generator=g) * 3 + 0.5) + torch.randn(rows, 1, generator=g) * 5).to(dtype)
+    w = (torch.rand(C, generator=g) + 0.5).to(wdtype)
+    b = torch.randn(C, generator=g).to(wdtype)
+    want = torch.nn.functional.layer_norm(x.double(), (C,), w.double(), b.double(), 1e-5)
+    got = cabi.layernorm_fwd(x.cuda(), w.cuda(), b.cuda(), 1e-5)
+    torch.cuda.synchronize()
+    assert got.dtype == dtype and got.shape == x.shape
+    assert so.rel_err(got.float().cpu(), want) < TOL[dtype]
+
+
+def test_layernorm_limits_are_reported(cabi):
+    x = torch.zeros(4, 12, device="cuda")
+    w = torch.ones(12, device="cuda")
+    cabi.layernorm_fwd(x, w, w)                                   # 12 = 3 chunks of fp32
+    with pytest.raises(cabi.M2DError):
+        cabi.layernorm_fwd(x.bfloat16(), w, w)                    # 12 is no multiple of 8
+    with pytest.raises(cabi.M2DError):
+        cabi.layernorm_fwd(torch.zeros(2, 4100, device="cuda"), torch.ones(4100, device="cuda"), torch.ones(4100, device="cuda"))
+
+
+# B, H, W, C: the local path's shapes scaled down, a strip that ends inside the row, one-cell images, one chunk
+DW_SHAPES = [(2, 14, 14, 128), (1, 9, 13, 64), (3, 7, 7, 256), (2, 1, 1, 8), (1, 3, 1, 16), (1, 2, 20, 24), (1, 56, 56, 128)]
+
+
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16], ids=["w_f32", "w_bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("shape", DW_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_depthwise_conv_matches_torch(cabi, shape, dtype, wdtype):
+    say(f"\ncase dwconv {shape} {dtype} {wdtype}")
+    B, H, W, C = shape
+    g = torch.Generator().manual_seed(sum(shape))
+    x = torch.randn(B, H, W, C, generator=g).to(dtype)
+    w = (torch.randn(C, 1, 3, 3, generator=g) / 3).to(wdtype)
+    want = torch.nn.functional.conv2d(x.double().permute(0, 3, 1, 2), w.double(), padding=1, groups=C).permute(0, 2, 3, 1)
+    got = cabi.dwconv3x3_fwd(x.cuda(), w.cuda())
+    torch.cuda.synchronize()
+    assert got.dtype == dtype and got.shape == x.shape
+    assert so.rel_err(got.float().cpu(), want) < TOL[dtype]
