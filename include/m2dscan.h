@@ -193,6 +193,16 @@ int m2d_layernorm_fwd(int64_t rows, int C, int dtype, int weight_dtype,
 int m2d_dwconv3x3_fwd(int B, int H, int W, int C, int dtype, int weight_dtype,
                       const void* x, const void* weight, void* y, void* stream);
 
+/* y = scale * relu(x)^2 + bias over n elements with one scale and one bias (StarReLU, models/utils.py:26-44).
+ * n must be a multiple of 8 (bf16) / 4 (fp32). */
+int m2d_starrelu_fwd(int64_t n, int dtype, int weight_dtype, const void* x, const void* scale, const void* bias,
+                     void* y, void* stream);
+
+/* y[r,c] = x[r,c] * scale[c] + residual[r,c]: the residual update of a block with its learned per-channel
+ * scale (models/mamba2d.py:258-259, models/utils.py:46-55).  y may be x or residual. */
+int m2d_scale_residual_fwd(int64_t rows, int C, int dtype, int weight_dtype, const void* x, const void* scale,
+                           const void* residual, void* y, void* stream);
+
 /* Measurement aid; no counterpart in the reference.  While enabled, every m2d_scan_fwd /
  * m2d_scan_bwd call records a pair of HIP events on its stream around the main scan kernel of
  * the pass (not around the small set-up and reduction kernels).  m2d_profile_last_ms waits for

@@ -22,7 +22,8 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .wavefront import dwconv3x3_fwd_op, layernorm_fwd_op, wavefront_scan_cuda
+from .wavefront import (dwconv3x3_fwd_op, layernorm_fwd_op, scale_residual_fwd_op, starrelu_fwd_op,
+                        wavefront_scan_cuda)
 
 M2D_T = dict(n_blocks=(3, 3, 9, 3), embed_dim=(64, 128, 320, 512),
              token_mixer=("2D_local", "2D_local", "RopeAttention", "RopeAttention"),
@@ -70,6 +71,9 @@ class StarReLU(nn.Module):
         self.bias = nn.Parameter(torch.zeros(1))
 
     def forward(self, x):
+        if (x.is_cuda and _inference(x, self.scale, self.bias) and x.is_contiguous() and x.dtype in (torch.float32, torch.bfloat16)
+                and self.scale.dtype in (torch.float32, torch.bfloat16) and x.numel() % 8 == 0 and x.numel() > 0):
+            return starrelu_fwd_op(x, self.scale, self.bias)      # one pass instead of three
         return torch.addcmul(self.bias, self.scale, F.relu(x).square())
 
 
@@ -265,9 +269,19 @@ class ResBlock(nn.Module):
         self.res_scale2 = Scale(dim, res_scale_init_value) if res_scale_init_value else nn.Identity()
         self.drop_path = float(drop_path)
 
+    @staticmethod
+    def _residual(x, scale, branch):
+        """scale(x) + branch; with a learned scale, at inference on the GPU, in one pass."""
+        if (isinstance(scale, Scale) and x.is_cuda and _inference(x, branch, scale.scale) and x.is_contiguous()
+                and branch.is_contiguous() and branch.dtype == x.dtype and branch.shape == x.shape
+                and x.dtype in (torch.float32, torch.bfloat16) and scale.scale.dtype in (torch.float32, torch.bfloat16)
+                and x.shape[-1] % 8 == 0 and x.numel() > 0):
+            return scale_residual_fwd_op(x, scale.scale, branch)
+        return scale(x) + branch
+
     def forward(self, x):
-        x = self.res_scale1(x) + _drop_path(self.token_mixer(self.norm1(x)), self.drop_path, self.training)
-        return self.res_scale2(x) + _drop_path(self.MLP(self.norm2(x)), self.drop_path, self.training)
+        x = self._residual(x, self.res_scale1, _drop_path(self.token_mixer(self.norm1(x)), self.drop_path, self.training))
+        return self._residual(x, self.res_scale2, _drop_path(self.MLP(self.norm2(x)), self.drop_path, self.training))
 
 
 class Mamba2DBackbone(nn.Module):

@@ -23,7 +23,8 @@ M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
            "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_bwd", "m2d_proj_workspace_bytes", "m2d_proj_fwd",
-           "m2d_proj_bwd", "m2d_layernorm_fwd", "m2d_dwconv3x3_fwd", "m2d_profile_enable", "m2d_profile_last_ms")
+           "m2d_proj_bwd", "m2d_layernorm_fwd", "m2d_dwconv3x3_fwd", "m2d_starrelu_fwd",
+           "m2d_scale_residual_fwd", "m2d_profile_enable", "m2d_profile_last_ms")
 
 
 class Desc(ctypes.Structure):
@@ -67,6 +68,10 @@ def _load():
     lib.m2d_layernorm_fwd.argtypes = [ctypes.c_int64, i32, i32, i32, vp, vp, vp, ctypes.c_float, vp, vp]
     lib.m2d_dwconv3x3_fwd.restype = i32
     lib.m2d_dwconv3x3_fwd.argtypes = [i32, i32, i32, i32, i32, i32, vp, vp, vp, vp]
+    lib.m2d_starrelu_fwd.restype = i32
+    lib.m2d_starrelu_fwd.argtypes = [ctypes.c_int64, i32, i32, vp, vp, vp, vp, vp]
+    lib.m2d_scale_residual_fwd.restype = i32
+    lib.m2d_scale_residual_fwd.argtypes = [ctypes.c_int64, i32, i32, i32, vp, vp, vp, vp, vp]
     lib.m2d_profile_enable.restype = i32
     lib.m2d_profile_enable.argtypes = [i32]
     lib.m2d_profile_last_ms.restype = i32
@@ -272,4 +277,30 @@ def dwconv3x3_fwd(x, weight):
     y = torch.empty_like(x)
     check(lib.m2d_dwconv3x3_fwd(B, H, W, C, _dtype_code(x), _dtype_code(weight), _ptr(x), _ptr(weight), _ptr(y),
                                 _stream(x.device)))
+    return y
+
+
+def starrelu_fwd(x, scale, bias):
+    """scale * relu(x)^2 + bias with one-element scale and bias, through m2d_starrelu_fwd."""
+    if not x.is_cuda or not x.is_contiguous():
+        raise ValueError("m2dscan: x must be a contiguous tensor on the GPU")
+    for k, t in (("scale", scale), ("bias", bias)):
+        if t.numel() != 1 or t.device != x.device or t.dtype != scale.dtype:
+            raise ValueError(f"m2dscan: {k} must hold one element on {x.device}, both of one dtype")
+    y = torch.empty_like(x)
+    check(lib.m2d_starrelu_fwd(x.numel(), _dtype_code(x), _dtype_code(scale), _ptr(x), _ptr(scale), _ptr(bias), _ptr(y),
+                               _stream(x.device)))
+    return y
+
+
+def scale_residual_fwd(x, scale, residual):
+    """x * scale + residual with a per-channel scale (last axis), through m2d_scale_residual_fwd."""
+    C = x.shape[-1]
+    if not x.is_cuda or not x.is_contiguous() or not residual.is_contiguous() or residual.shape != x.shape or residual.dtype != x.dtype:
+        raise ValueError("m2dscan: x and residual must be contiguous tensors of one shape and dtype on the GPU")
+    if tuple(scale.shape) != (C,) or scale.device != x.device or not scale.is_contiguous():
+        raise ValueError(f"m2dscan: scale must be a contiguous ({C},) tensor on {x.device}")
+    y = torch.empty_like(x)
+    check(lib.m2d_scale_residual_fwd(x.numel() // C, C, _dtype_code(x), _dtype_code(scale), _ptr(x), _ptr(scale), _ptr(residual),
+                                     _ptr(y), _stream(x.device)))
     return y

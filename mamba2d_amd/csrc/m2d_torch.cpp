@@ -5,7 +5,7 @@
 // (models/kernels/wavefront_cuda.py:25-57) plus the tensor algebra around them, and
 // m2dscan::proj_fwd / m2dscan::proj_bwd for the projections that feed the scan
 // (wavefront_cuda.py:63-95 and their autograd backward), and m2dscan::layernorm_fwd /
-// m2dscan::dwconv3x3_fwd for two operators of the residual block at inference.  The shim only
+// m2dscan::dwconv3x3_fwd / starrelu_fwd / scale_residual_fwd for operators of the residual block at inference.  The shim only
 // validates tensors, allocates outputs / scratch through the caching allocator, picks the
 // current HIP stream and forwards raw pointers; all arithmetic lives behind the C ABI.
 #include <ATen/ATen.h>
@@ -252,6 +252,35 @@ Tensor dwconv3x3_fwd(const Tensor& x, const Tensor& weight) {
   return y;
 }
 
+Tensor starrelu_fwd(const Tensor& x, const Tensor& scale, const Tensor& bias) {
+  TORCH_CHECK(x.is_cuda() && x.is_contiguous(), "m2dscan: x must be a contiguous tensor on the GPU");
+  TORCH_CHECK(scale.numel() == 1 && bias.numel() == 1 && scale.device() == x.device() && bias.device() == x.device() &&
+              scale.scalar_type() == bias.scalar_type(), "m2dscan: scale and bias must hold one element each, of one dtype, on x's device");
+  c10::DeviceGuard guard(x.device());
+  Tensor y = at::empty_like(x);
+  if (x.numel() == 0) return y;
+  hipStream_t st = c10::hip::getCurrentHIPStream(x.device().index()).stream();
+  check(m2d_starrelu_fwd(x.numel(), dtype_code(x, "x"), dtype_code(scale, "scale"), x.data_ptr(), scale.data_ptr(), bias.data_ptr(),
+                         y.data_ptr(), st));
+  return y;
+}
+
+Tensor scale_residual_fwd(const Tensor& x, const Tensor& scale, const Tensor& residual) {
+  TORCH_CHECK(x.is_cuda() && x.dim() >= 1 && x.is_contiguous() && residual.is_contiguous() && residual.sizes() == x.sizes() &&
+              residual.scalar_type() == x.scalar_type() && residual.device() == x.device(),
+              "m2dscan: x and residual must be contiguous tensors of one shape and dtype on the GPU");
+  const int64_t C = x.size(-1);
+  TORCH_CHECK(scale.sizes() == at::IntArrayRef({C}) && scale.is_contiguous() && scale.device() == x.device(),
+              "m2dscan: scale must be a contiguous (", C, ",) tensor on x's device");
+  c10::DeviceGuard guard(x.device());
+  Tensor y = at::empty_like(x);
+  if (x.numel() == 0) return y;
+  hipStream_t st = c10::hip::getCurrentHIPStream(x.device().index()).stream();
+  check(m2d_scale_residual_fwd(x.numel() / C, static_cast<int>(C), dtype_code(x, "x"), dtype_code(scale, "scale"), x.data_ptr(),
+                               scale.data_ptr(), residual.data_ptr(), y.data_ptr(), st));
+  return y;
+}
+
 int64_t abi_version() { return m2d_version(); }
 
 }  // namespace
@@ -268,6 +297,8 @@ TORCH_LIBRARY(m2dscan, m) {
         "bool round_weights, bool dpre=False) -> Tensor[]");
   m.def("layernorm_fwd(Tensor x, Tensor weight, Tensor bias, float eps) -> Tensor");
   m.def("dwconv3x3_fwd(Tensor x, Tensor weight) -> Tensor");
+  m.def("starrelu_fwd(Tensor x, Tensor scale, Tensor bias) -> Tensor");
+  m.def("scale_residual_fwd(Tensor x, Tensor scale, Tensor residual) -> Tensor");
   m.def("abi_version() -> int", &abi_version);
 }
 
@@ -278,4 +309,6 @@ TORCH_LIBRARY_IMPL(m2dscan, CUDA, m) {   // ROCm devices dispatch under the CUDA
   m.impl("proj_bwd", &proj_bwd);
   m.impl("layernorm_fwd", &layernorm_fwd);
   m.impl("dwconv3x3_fwd", &dwconv3x3_fwd);
+  m.impl("starrelu_fwd", &starrelu_fwd);
+  m.impl("scale_residual_fwd", &scale_residual_fwd);
 }

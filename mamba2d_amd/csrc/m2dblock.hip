@@ -1,8 +1,10 @@
-// m2dblock.hip -- the two memory-bound operators of an M2D residual block that the stock libraries
-// serve badly on gfx950 at this model's shapes: LayerNorm over a short channel axis (64 to 512
-// channels: models/mamba2d.py:57,220,248,363, models/utils.py:13,232-233) and the depthwise 3x3
-// convolution of the local path on channel-last tensors (models/utils.py:101-114).  Inference
-// forward only; both read every input byte once and write every output byte once.
+// m2dblock.hip -- memory-bound operators of an M2D residual block that the stock libraries serve
+// badly on gfx950 at this model's shapes, or in several passes where one will do: LayerNorm over
+// a short channel axis (64 to 512 channels: models/mamba2d.py:57,220,248,363, models/utils.py:13,
+// 232-233), the depthwise 3x3 convolution of the local path on channel-last tensors
+// (models/utils.py:101-114), StarReLU (models/utils.py:26-44) and the scaled residual sum
+// (models/mamba2d.py:258-259).  Inference forward only; each reads every input byte once and
+// writes every output byte once.
 //
 // Layout: activations are row-major (rows, C) / (B, H, W, C), element type float or bf16; weights
 // are float or bf16, independently of the activations (a bf16 model holds bf16 weights, a fp32
@@ -232,6 +234,60 @@ __global__ __launch_bounds__(kDwThreads) void m2d_dwconv3x3_kernel(const DwArgs 
   }
 }
 
+// ------------------------------------------------------------------------ fused elementwise
+// StarReLU, y = scale * relu(x)^2 + bias with scalar scale and bias (models/utils.py:22-37), and the
+// residual update of a block, y = x * scale[c] + r (models/mamba2d.py:258-259): one pass each where
+// stock operators take three and two.
+constexpr int kEwThreads = 256;
+
+struct EwArgs {
+  const void* x;
+  const void* r;      // residual branch (scale-residual only)
+  const void* s;      // one scale (StarReLU) or C of them
+  const void* b;      // one bias (StarReLU)
+  void* y;
+  int64_t chunks;     // 16-byte chunks in all
+  int cpr;            // chunks per row (scale-residual)
+  int wbf16;
+};
+
+template <typename T>
+__global__ __launch_bounds__(kEwThreads) void m2d_starrelu_kernel(const EwArgs a) {
+  constexpr int V = Chunk<T>::kV;
+  const float sc = ldw(a.s, a.wbf16, 0), bi = ldw(a.b, a.wbf16, 0);
+  const T* X = static_cast<const T*>(a.x);
+  T* Y = static_cast<T*>(a.y);
+  for (int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x; i < a.chunks; i += (int64_t)gridDim.x * kEwThreads) {
+    float v[V];
+    Chunk<T>::load(X + i * V, v);
+#pragma unroll
+    for (int j = 0; j < V; ++j) { const float t = fmaxf(v[j], 0.f); v[j] = __builtin_fmaf(sc * t, t, bi); }
+    Chunk<T>::store(Y + i * V, v);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kEwThreads) void m2d_scale_residual_kernel(const EwArgs a) {
+  constexpr int V = Chunk<T>::kV;
+  const T* X = static_cast<const T*>(a.x);
+  const T* R = static_cast<const T*>(a.r);
+  T* Y = static_cast<T*>(a.y);
+  for (int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x; i < a.chunks; i += (int64_t)gridDim.x * kEwThreads) {
+    const int c = (int)(i % a.cpr);
+    float v[V], r[V];
+    Chunk<T>::load(X + i * V, v);
+    Chunk<T>::load(R + i * V, r);
+#pragma unroll
+    for (int j = 0; j < V; ++j) v[j] = __builtin_fmaf(v[j], ldw(a.s, a.wbf16, c * V + j), r[j]);
+    Chunk<T>::store(Y + i * V, v);
+  }
+}
+
+inline unsigned ew_blocks(int64_t chunks) {
+  int64_t blocks = (chunks + kEwThreads - 1) / kEwThreads;
+  return (unsigned)(blocks > 256 * 64 ? 256 * 64 : blocks);
+}
+
 inline bool misaligned(const void* p, size_t n) { return (reinterpret_cast<uintptr_t>(p) & (n - 1)) != 0; }
 
 }  // namespace
@@ -269,6 +325,38 @@ int m2d_dwconv3x3_fwd(int B, int H, int W, int C, int dtype, int weight_dtype, c
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == M2D_F32) hipLaunchKernelGGL(m2d_dwconv3x3_kernel<float>, dim3((unsigned)blocks), dim3(kDwThreads), 0, st, a);
   else hipLaunchKernelGGL(m2d_dwconv3x3_kernel<bf16_t>, dim3((unsigned)blocks), dim3(kDwThreads), 0, st, a);
+  return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+}
+
+int m2d_starrelu_fwd(int64_t n, int dtype, int weight_dtype, const void* x, const void* scale, const void* bias, void* y,
+                     void* stream) {
+  if (!x || !scale || !bias || !y) return M2D_ERR_NULL_POINTER;
+  if (n < 1) return M2D_ERR_BAD_SHAPE;
+  if ((dtype != M2D_F32 && dtype != M2D_BF16) || (weight_dtype != M2D_F32 && weight_dtype != M2D_BF16)) return M2D_ERR_UNSUPPORTED;
+  const int V = dtype == M2D_BF16 ? 8 : 4;
+  if (n % V != 0) return M2D_ERR_UNSUPPORTED;
+  if (misaligned(x, 16) || misaligned(y, 16)) return M2D_ERR_MISALIGNED;
+  EwArgs a = {};
+  a.x = x; a.s = scale; a.b = bias; a.y = y; a.chunks = n / V; a.wbf16 = weight_dtype == M2D_BF16;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == M2D_F32) hipLaunchKernelGGL(m2d_starrelu_kernel<float>, dim3(ew_blocks(a.chunks)), dim3(kEwThreads), 0, st, a);
+  else hipLaunchKernelGGL(m2d_starrelu_kernel<bf16_t>, dim3(ew_blocks(a.chunks)), dim3(kEwThreads), 0, st, a);
+  return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+}
+
+int m2d_scale_residual_fwd(int64_t rows, int C, int dtype, int weight_dtype, const void* x, const void* scale,
+                           const void* residual, void* y, void* stream) {
+  if (!x || !scale || !residual || !y) return M2D_ERR_NULL_POINTER;
+  if (rows < 1 || C < 1) return M2D_ERR_BAD_SHAPE;
+  if ((dtype != M2D_F32 && dtype != M2D_BF16) || (weight_dtype != M2D_F32 && weight_dtype != M2D_BF16)) return M2D_ERR_UNSUPPORTED;
+  const int V = dtype == M2D_BF16 ? 8 : 4;
+  if (C % V != 0) return M2D_ERR_UNSUPPORTED;
+  if (misaligned(x, 16) || misaligned(residual, 16) || misaligned(y, 16)) return M2D_ERR_MISALIGNED;
+  EwArgs a = {};
+  a.x = x; a.r = residual; a.s = scale; a.y = y; a.cpr = C / V; a.chunks = rows * a.cpr; a.wbf16 = weight_dtype == M2D_BF16;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (dtype == M2D_F32) hipLaunchKernelGGL(m2d_scale_residual_kernel<float>, dim3(ew_blocks(a.chunks)), dim3(kEwThreads), 0, st, a);
+  else hipLaunchKernelGGL(m2d_scale_residual_kernel<bf16_t>, dim3(ew_blocks(a.chunks)), dim3(kEwThreads), 0, st, a);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 

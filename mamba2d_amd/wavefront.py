@@ -38,6 +38,8 @@ proj_fwd_op = torch.ops.m2dscan.proj_fwd
 proj_bwd_op = torch.ops.m2dscan.proj_bwd
 layernorm_fwd_op = torch.ops.m2dscan.layernorm_fwd
 dwconv3x3_fwd_op = torch.ops.m2dscan.dwconv3x3_fwd
+starrelu_fwd_op = torch.ops.m2dscan.starrelu_fwd
+scale_residual_fwd_op = torch.ops.m2dscan.scale_residual_fwd
 
 # Keep the forward's anti-diagonal checkpoints for the backward (faster backward, more saved
 # memory) or rebuild them inside the backward (nothing saved beyond the inputs, like the
@@ -92,6 +94,16 @@ def _layernorm_fwd_fake(x, weight, bias, eps):
 
 @torch.library.register_fake("m2dscan::dwconv3x3_fwd")
 def _dwconv3x3_fwd_fake(x, weight):
+    return torch.empty_like(x)
+
+
+@torch.library.register_fake("m2dscan::starrelu_fwd")
+def _starrelu_fwd_fake(x, scale, bias):
+    return torch.empty_like(x)
+
+
+@torch.library.register_fake("m2dscan::scale_residual_fwd")
+def _scale_residual_fwd_fake(x, scale, residual):
     return torch.empty_like(x)
 
 

@@ -1,5 +1,5 @@
-"""GPU parity of the two residual-block operators (m2d_layernorm_fwd, m2d_dwconv3x3_fwd) through the
-C ABI, against the stock torch operators the reference uses (nn.LayerNorm, models/mamba2d.py:220;
+"""GPU parity of the residual-block operators (m2d_layernorm_fwd, m2d_dwconv3x3_fwd, m2d_starrelu_fwd,
+m2d_scale_residual_fwd) through the C ABI, against the stock torch operators the reference uses (nn.LayerNorm, models/mamba2d.py:220;
 depthwise nn.Conv2d, models/utils.py:101) evaluated in fp64 on the CPU.  Tolerances: fp32 2e-5,
 bf16 tensors 1e-2 (max error over max value; one bf16 rounding of the result is 4e-3)."""
 import pytest
@@ -72,3 +72,22 @@ def test_depthwise_conv_matches_torch(cabi, shape, dtype, wdtype):
     torch.cuda.synchronize()
     assert got.dtype == dtype and got.shape == x.shape
     assert so.rel_err(got.float().cpu(), want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16], ids=["w_f32", "w_bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("shape", [(2, 9, 12, 64), (1, 5, 8), (3, 1000, 24), (128 * 56, 56, 128)], ids=lambda s: "x".join(map(str, s)))
+def test_fused_elementwise_match_torch(cabi, shape, dtype, wdtype):
+    say(f"\ncase starrelu / scale_residual {shape} {dtype} {wdtype}")
+    g = torch.Generator().manual_seed(len(shape) + shape[-1])
+    x = torch.randn(*shape, generator=g).to(dtype)
+    r = torch.randn(*shape, generator=g).to(dtype)
+    sc, bi = torch.tensor([0.8944]).to(wdtype), torch.tensor([-0.4472]).to(wdtype)
+    chan = (torch.rand(shape[-1], generator=g) + 0.5).to(wdtype)
+    xd, rd = x.cuda(), r.cuda()
+    got = cabi.starrelu_fwd(xd, sc.cuda(), bi.cuda())
+    want = sc.double() * torch.relu(x.double()) ** 2 + bi.double()
+    assert got.dtype == dtype and so.rel_err(got.float().cpu(), want) < TOL[dtype]
+    got = cabi.scale_residual_fwd(xd, chan.cuda(), rd)
+    want = x.double() * chan.double() + r.double()
+    assert got.dtype == dtype and so.rel_err(got.float().cpu(), want) < TOL[dtype]
