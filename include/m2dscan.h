@@ -203,6 +203,17 @@ int m2d_starrelu_fwd(int64_t n, int dtype, int weight_dtype, const void* x, cons
 int m2d_scale_residual_fwd(int64_t rows, int C, int dtype, int weight_dtype, const void* x, const void* scale,
                            const void* residual, void* y, void* stream);
 
+/* Rotary embedding and per-head LayerNorm of q and k in the attention stages (models/utils.py:253-301):
+ * qkv is the output of the qkv projection, (B, L, 3, heads, head_dim); cos and sin are (L, head_dim) tables
+ * of qkv's element type in which the two features of a pair (2i, 2i+1) hold the same angle (cos 1, sin 0 on
+ * features that do not rotate); rotated[2i] = x[2i] cos - x[2i+1] sin, rotated[2i+1] = x[2i+1] cos + x[2i] sin.
+ * q and k receive LayerNorm(rotated) with their own weights, laid out (B, heads, L, head_dim).
+ * head_dim must be 8, 16, ... 256 (bf16) / 4, 8, ... 128 (fp32), a power of two. */
+int m2d_rope_qknorm_fwd(int B, int L, int heads, int head_dim, int dtype, int weight_dtype,
+                        const void* qkv, const void* cos, const void* sin,
+                        const void* q_weight, const void* q_bias, const void* k_weight, const void* k_bias,
+                        float eps, void* q, void* k, void* stream);
+
 /* Measurement aid; no counterpart in the reference.  While enabled, every m2d_scan_fwd /
  * m2d_scan_bwd call records a pair of HIP events on its stream around the main scan kernel of
  * the pass (not around the small set-up and reduction kernels).  m2d_profile_last_ms waits for

@@ -22,8 +22,8 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .wavefront import (dwconv3x3_fwd_op, layernorm_fwd_op, scale_residual_fwd_op, starrelu_fwd_op,
-                        wavefront_scan_cuda)
+from .wavefront import (dwconv3x3_fwd_op, layernorm_fwd_op, rope_qknorm_fwd_op, scale_residual_fwd_op,
+                        starrelu_fwd_op, wavefront_scan_cuda)
 
 M2D_T = dict(n_blocks=(3, 3, 9, 3), embed_dim=(64, 128, 320, 512),
              token_mixer=("2D_local", "2D_local", "RopeAttention", "RopeAttention"),
@@ -231,9 +231,17 @@ class RoPEAttention2D(nn.Module):
 
     def forward(self, x):           # (B, H, W, C)
         B, H, W, _ = x.shape
-        qkv = self.qkv(x).view(B, H * W, 3, self.num_heads, self.head_dim).permute(2, 0, 3, 1, 4)
-        q, k, v = qkv.unbind(0)     # (B, heads, HW, head_dim)
-        cos, sin = self._rope_tables(H, W, x.device, q.dtype)
+        qkv = self.qkv(x).view(B, H * W, 3, self.num_heads, self.head_dim)
+        cos, sin = self._rope_tables(H, W, x.device, qkv.dtype)
+        qn, kn, hd = self.q_norm, self.k_norm, self.head_dim
+        if (qkv.is_cuda and _inference(qkv, qn.weight, qn.bias, kn.weight, kn.bias) and qkv.dtype in (torch.float32, torch.bfloat16)
+                and qn.weight.dtype in (torch.float32, torch.bfloat16) and qn.eps == kn.eps and hd & (hd - 1) == 0
+                and 8 <= hd <= 128 and qkv.numel() > 0):
+            # rotation and the two LayerNorms in one pass, q and k in the attention kernel's layout
+            q, k = rope_qknorm_fwd_op(qkv, cos, sin, qn.weight, qn.bias, kn.weight, kn.bias, qn.eps)
+            o = F.scaled_dot_product_attention(q, k, qkv[:, :, 2].permute(0, 2, 1, 3), scale=hd ** -0.5)
+            return self.proj(o.transpose(1, 2).reshape(B, H, W, self.num_heads * hd))
+        q, k, v = qkv.permute(2, 0, 3, 1, 4).unbind(0)     # (B, heads, HW, head_dim)
         q = q * cos + self._rotate_pairs(q) * sin      # sin is zero on the untouched dims
         k = k * cos + self._rotate_pairs(k) * sin
         q, k = self.q_norm(q), self.k_norm(k)

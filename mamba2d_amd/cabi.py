@@ -24,7 +24,7 @@ M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
            "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_bwd", "m2d_proj_workspace_bytes", "m2d_proj_fwd",
            "m2d_proj_bwd", "m2d_layernorm_fwd", "m2d_dwconv3x3_fwd", "m2d_starrelu_fwd",
-           "m2d_scale_residual_fwd", "m2d_profile_enable", "m2d_profile_last_ms")
+           "m2d_scale_residual_fwd", "m2d_rope_qknorm_fwd", "m2d_profile_enable", "m2d_profile_last_ms")
 
 
 class Desc(ctypes.Structure):
@@ -72,6 +72,8 @@ def _load():
     lib.m2d_starrelu_fwd.argtypes = [ctypes.c_int64, i32, i32, vp, vp, vp, vp, vp]
     lib.m2d_scale_residual_fwd.restype = i32
     lib.m2d_scale_residual_fwd.argtypes = [ctypes.c_int64, i32, i32, i32, vp, vp, vp, vp, vp]
+    lib.m2d_rope_qknorm_fwd.restype = i32
+    lib.m2d_rope_qknorm_fwd.argtypes = [i32] * 6 + [vp] * 7 + [ctypes.c_float, vp, vp, vp]
     lib.m2d_profile_enable.restype = i32
     lib.m2d_profile_enable.argtypes = [i32]
     lib.m2d_profile_last_ms.restype = i32
@@ -304,3 +306,23 @@ def scale_residual_fwd(x, scale, residual):
     check(lib.m2d_scale_residual_fwd(x.numel() // C, C, _dtype_code(x), _dtype_code(scale), _ptr(x), _ptr(scale), _ptr(residual),
                                      _ptr(y), _stream(x.device)))
     return y
+
+
+def rope_qknorm_fwd(qkv, cos, sin, q_weight, q_bias, k_weight, k_bias, eps=1e-5):
+    """(q, k), each (B, heads, L, head_dim): rotary embedding and per-head LayerNorm of the q and k parts of
+    a contiguous (B, L, 3, heads, head_dim) projection, through m2d_rope_qknorm_fwd."""
+    if qkv.dim() != 5 or qkv.shape[2] != 3 or not qkv.is_cuda or not qkv.is_contiguous():
+        raise ValueError("m2dscan: qkv must be a contiguous (B, L, 3, heads, head_dim) tensor on the GPU")
+    B, L, _, nh, hd = qkv.shape
+    for k_, t in (("cos", cos), ("sin", sin)):
+        if tuple(t.shape) != (L, hd) or t.dtype != qkv.dtype or t.device != qkv.device or not t.is_contiguous():
+            raise ValueError(f"m2dscan: {k_} must be a contiguous ({L},{hd}) tensor of qkv's dtype and device")
+    for k_, t in (("q_weight", q_weight), ("q_bias", q_bias), ("k_weight", k_weight), ("k_bias", k_bias)):
+        if tuple(t.shape) != (hd,) or t.dtype != q_weight.dtype or t.device != qkv.device or not t.is_contiguous():
+            raise ValueError(f"m2dscan: {k_} must be a contiguous ({hd},) tensor, all four of one dtype, on qkv's device")
+    q = qkv.new_empty((B, nh, L, hd))
+    k = qkv.new_empty((B, nh, L, hd))
+    check(lib.m2d_rope_qknorm_fwd(B, L, nh, hd, _dtype_code(qkv), _dtype_code(q_weight), _ptr(qkv), _ptr(cos), _ptr(sin),
+                                  _ptr(q_weight), _ptr(q_bias), _ptr(k_weight), _ptr(k_bias), float(eps), _ptr(q), _ptr(k),
+                                  _stream(qkv.device)))
+    return q, k

@@ -281,6 +281,28 @@ Tensor scale_residual_fwd(const Tensor& x, const Tensor& scale, const Tensor& re
   return y;
 }
 
+std::tuple<Tensor, Tensor> rope_qknorm_fwd(const Tensor& qkv, const Tensor& cos, const Tensor& sin, const Tensor& qw,
+                                           const Tensor& qb, const Tensor& kw, const Tensor& kb, double eps) {
+  TORCH_CHECK(qkv.is_cuda() && qkv.dim() == 5 && qkv.size(2) == 3 && qkv.is_contiguous(),
+              "m2dscan: qkv must be a contiguous (B, L, 3, heads, head_dim) tensor on the GPU");
+  const int64_t B = qkv.size(0), L = qkv.size(1), nh = qkv.size(3), hd = qkv.size(4);
+  for (const Tensor* t : {&cos, &sin})
+    TORCH_CHECK(t->sizes() == at::IntArrayRef({L, hd}) && t->scalar_type() == qkv.scalar_type() && t->device() == qkv.device() &&
+                t->is_contiguous(), "m2dscan: cos and sin must be contiguous (", L, ",", hd, ") tensors of qkv's dtype and device");
+  for (const Tensor* t : {&qw, &qb, &kw, &kb})
+    TORCH_CHECK(t->sizes() == at::IntArrayRef({hd}) && t->scalar_type() == qw.scalar_type() && t->device() == qkv.device() &&
+                t->is_contiguous(), "m2dscan: the LayerNorm weights must be contiguous (", hd, ",) tensors of one dtype on qkv's device");
+  c10::DeviceGuard guard(qkv.device());
+  Tensor q = at::empty({B, nh, L, hd}, qkv.options()), k = at::empty({B, nh, L, hd}, qkv.options());
+  if (qkv.numel() == 0) return {q, k};
+  hipStream_t st = c10::hip::getCurrentHIPStream(qkv.device().index()).stream();
+  check(m2d_rope_qknorm_fwd(static_cast<int>(B), static_cast<int>(L), static_cast<int>(nh), static_cast<int>(hd),
+                            dtype_code(qkv, "qkv"), dtype_code(qw, "q_weight"), qkv.data_ptr(), cos.data_ptr(), sin.data_ptr(),
+                            qw.data_ptr(), qb.data_ptr(), kw.data_ptr(), kb.data_ptr(), static_cast<float>(eps), q.data_ptr(),
+                            k.data_ptr(), st));
+  return {q, k};
+}
+
 int64_t abi_version() { return m2d_version(); }
 
 }  // namespace
@@ -299,6 +321,8 @@ TORCH_LIBRARY(m2dscan, m) {
   m.def("dwconv3x3_fwd(Tensor x, Tensor weight) -> Tensor");
   m.def("starrelu_fwd(Tensor x, Tensor scale, Tensor bias) -> Tensor");
   m.def("scale_residual_fwd(Tensor x, Tensor scale, Tensor residual) -> Tensor");
+  m.def("rope_qknorm_fwd(Tensor qkv, Tensor cos, Tensor sin, Tensor q_weight, Tensor q_bias, Tensor k_weight, Tensor k_bias, "
+        "float eps) -> (Tensor, Tensor)");
   m.def("abi_version() -> int", &abi_version);
 }
 
@@ -311,4 +335,5 @@ TORCH_LIBRARY_IMPL(m2dscan, CUDA, m) {   // ROCm devices dispatch under the CUDA
   m.impl("dwconv3x3_fwd", &dwconv3x3_fwd);
   m.impl("starrelu_fwd", &starrelu_fwd);
   m.impl("scale_residual_fwd", &scale_residual_fwd);
+  m.impl("rope_qknorm_fwd", &rope_qknorm_fwd);
 }

@@ -2,8 +2,8 @@
 // badly on gfx950 at this model's shapes, or in several passes where one will do: LayerNorm over
 // a short channel axis (64 to 512 channels: models/mamba2d.py:57,220,248,363, models/utils.py:13,
 // 232-233), the depthwise 3x3 convolution of the local path on channel-last tensors
-// (models/utils.py:101-114), StarReLU (models/utils.py:26-44) and the scaled residual sum
-// (models/mamba2d.py:258-259).  Inference forward only; each reads every input byte once and
+// (models/utils.py:101-114), StarReLU (models/utils.py:26-44), the scaled residual sum
+// (models/mamba2d.py:258-259) and the rotary embedding + LayerNorm of q and k in the attention stages.  Inference forward only; each reads every input byte once and
 // writes every output byte once.
 //
 // Layout: activations are row-major (rows, C) / (B, H, W, C), element type float or bf16; weights
@@ -288,6 +288,85 @@ inline unsigned ew_blocks(int64_t chunks) {
   return (unsigned)(blocks > 256 * 64 ? 256 * 64 : blocks);
 }
 
+// ------------------------------------------------------- rotary embedding + LayerNorm of q and k
+// The attention stages rotate q and k by position (pairs of neighbouring features share an angle,
+// models/utils.py:253-297) and then LayerNorm each head (:299-301).  Input is the output of the
+// qkv projection, (B, L, 3, heads, hd); q and k leave as (B, heads, L, hd), the layout the attention
+// kernel wants.  A head's hd features are G = hd / kV chunks on G neighbouring lanes; the pairs of
+// the rotation never straddle a chunk.  One pass where stock operators take sixteen.
+struct RopeArgs {
+  const void* qkv;
+  const void *cos, *sin;          // (L, hd), element type of qkv
+  const void *qw, *qb, *kw, *kb;  // LayerNorm weights of q and k, (hd)
+  void *q, *k;
+  int64_t total;                  // B * L * 2 * heads * G chunks
+  int L, heads, hd, wbf16;
+  float eps;
+};
+
+template <typename T, int G>
+__global__ __launch_bounds__(kEwThreads) void m2d_rope_qknorm_kernel(const RopeArgs a) {
+  constexpr int V = Chunk<T>::kV;
+  const int64_t gid = (int64_t)blockIdx.x * kEwThreads + threadIdx.x;
+  if (gid >= a.total) return;          // whole groups of G lanes leave together (total is a multiple of G)
+  const int c = (int)(gid % G);
+  int64_t rest = gid / G;
+  const int head = (int)(rest % a.heads);
+  rest /= a.heads;
+  const int which = (int)(rest % 2);   // 0: q, 1: k
+  rest /= 2;
+  const int l = (int)(rest % a.L);
+  const int64_t b = rest / a.L;
+  const T* src = static_cast<const T*>(a.qkv) + (((b * a.L + l) * 3 + which) * a.heads + head) * (int64_t)a.hd + c * V;
+  float x[V], cs[V], sn[V];
+  Chunk<T>::load(src, x);
+  Chunk<T>::load(static_cast<const T*>(a.cos) + (int64_t)l * a.hd + c * V, cs);
+  Chunk<T>::load(static_cast<const T*>(a.sin) + (int64_t)l * a.hd + c * V, sn);
+  float v[V];
+#pragma unroll
+  for (int j = 0; j < V; j += 2) {
+    v[j] = __builtin_fmaf(x[j], cs[j], -x[j + 1] * sn[j]);
+    v[j + 1] = __builtin_fmaf(x[j + 1], cs[j + 1], x[j] * sn[j + 1]);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < V; ++j) s += v[j];
+#pragma unroll
+  for (int off = G >> 1; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+  const float inv = 1.f / (float)a.hd;
+  const float mean = s * inv;
+  float q = 0.f;
+#pragma unroll
+  for (int j = 0; j < V; ++j) { const float d = v[j] - mean; q = __builtin_fmaf(d, d, q); }
+#pragma unroll
+  for (int off = G >> 1; off > 0; off >>= 1) q += __shfl_xor(q, off, 64);
+  const float rstd = rsqrtf(q * inv + a.eps);
+  const void* w = which ? a.kw : a.qw;
+  const void* bi = which ? a.kb : a.qb;
+  float o[V];
+#pragma unroll
+  for (int j = 0; j < V; ++j) o[j] = __builtin_fmaf((v[j] - mean) * rstd, ldw(w, a.wbf16, c * V + j), ldw(bi, a.wbf16, c * V + j));
+  T* dst = static_cast<T*>(which ? a.k : a.q) + ((b * a.heads + head) * a.L + l) * (int64_t)a.hd + c * V;
+  Chunk<T>::store(dst, o);
+}
+
+template <typename T>
+int run_rope(const RopeArgs& a, int G, hipStream_t st) {
+  const int64_t blocks = (a.total + kEwThreads - 1) / kEwThreads;
+  if (blocks >= ((int64_t)1 << 31)) return M2D_ERR_UNSUPPORTED;
+  const dim3 grid((unsigned)blocks), block(kEwThreads);
+  switch (G) {
+    case 1: hipLaunchKernelGGL((m2d_rope_qknorm_kernel<T, 1>), grid, block, 0, st, a); break;
+    case 2: hipLaunchKernelGGL((m2d_rope_qknorm_kernel<T, 2>), grid, block, 0, st, a); break;
+    case 4: hipLaunchKernelGGL((m2d_rope_qknorm_kernel<T, 4>), grid, block, 0, st, a); break;
+    case 8: hipLaunchKernelGGL((m2d_rope_qknorm_kernel<T, 8>), grid, block, 0, st, a); break;
+    case 16: hipLaunchKernelGGL((m2d_rope_qknorm_kernel<T, 16>), grid, block, 0, st, a); break;
+    case 32: hipLaunchKernelGGL((m2d_rope_qknorm_kernel<T, 32>), grid, block, 0, st, a); break;
+    default: return M2D_ERR_UNSUPPORTED;
+  }
+  return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+}
+
 inline bool misaligned(const void* p, size_t n) { return (reinterpret_cast<uintptr_t>(p) & (n - 1)) != 0; }
 
 }  // namespace
@@ -358,6 +437,25 @@ int m2d_scale_residual_fwd(int64_t rows, int C, int dtype, int weight_dtype, con
   if (dtype == M2D_F32) hipLaunchKernelGGL(m2d_scale_residual_kernel<float>, dim3(ew_blocks(a.chunks)), dim3(kEwThreads), 0, st, a);
   else hipLaunchKernelGGL(m2d_scale_residual_kernel<bf16_t>, dim3(ew_blocks(a.chunks)), dim3(kEwThreads), 0, st, a);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+}
+
+int m2d_rope_qknorm_fwd(int B, int L, int heads, int head_dim, int dtype, int weight_dtype, const void* qkv,
+                        const void* cos, const void* sin, const void* q_weight, const void* q_bias, const void* k_weight,
+                        const void* k_bias, float eps, void* q, void* k, void* stream) {
+  const void* req[] = {qkv, cos, sin, q_weight, q_bias, k_weight, k_bias, q, k};
+  for (const void* p : req) if (!p) return M2D_ERR_NULL_POINTER;
+  if (B < 1 || L < 1 || heads < 1 || head_dim < 1) return M2D_ERR_BAD_SHAPE;
+  if ((dtype != M2D_F32 && dtype != M2D_BF16) || (weight_dtype != M2D_F32 && weight_dtype != M2D_BF16)) return M2D_ERR_UNSUPPORTED;
+  const int V = dtype == M2D_BF16 ? 8 : 4;
+  const int G = head_dim / V;
+  if (head_dim % V != 0 || (G & (G - 1)) != 0 || G > 32) return M2D_ERR_UNSUPPORTED;   // a head is 1, 2, 4 ... 32 chunks
+  if (misaligned(qkv, 16) || misaligned(cos, 16) || misaligned(sin, 16) || misaligned(q, 16) || misaligned(k, 16)) return M2D_ERR_MISALIGNED;
+  RopeArgs a = {};
+  a.qkv = qkv; a.cos = cos; a.sin = sin; a.qw = q_weight; a.qb = q_bias; a.kw = k_weight; a.kb = k_bias; a.q = q; a.k = k;
+  a.L = L; a.heads = heads; a.hd = head_dim; a.wbf16 = weight_dtype == M2D_BF16; a.eps = eps;
+  a.total = (int64_t)B * L * 2 * heads * G;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return dtype == M2D_F32 ? run_rope<float>(a, G, st) : run_rope<bf16_t>(a, G, st);
 }
 
 }  // extern "C"

@@ -40,6 +40,7 @@ layernorm_fwd_op = torch.ops.m2dscan.layernorm_fwd
 dwconv3x3_fwd_op = torch.ops.m2dscan.dwconv3x3_fwd
 starrelu_fwd_op = torch.ops.m2dscan.starrelu_fwd
 scale_residual_fwd_op = torch.ops.m2dscan.scale_residual_fwd
+rope_qknorm_fwd_op = torch.ops.m2dscan.rope_qknorm_fwd
 
 # Keep the forward's anti-diagonal checkpoints for the backward (faster backward, more saved
 # memory) or rebuild them inside the backward (nothing saved beyond the inputs, like the
@@ -105,6 +106,12 @@ def _starrelu_fwd_fake(x, scale, bias):
 @torch.library.register_fake("m2dscan::scale_residual_fwd")
 def _scale_residual_fwd_fake(x, scale, residual):
     return torch.empty_like(x)
+
+
+@torch.library.register_fake("m2dscan::rope_qknorm_fwd")
+def _rope_qknorm_fwd_fake(qkv, cos, sin, q_weight, q_bias, k_weight, k_bias, eps):
+    B, L, _, nh, hd = qkv.shape
+    return qkv.new_empty((B, nh, L, hd)), qkv.new_empty((B, nh, L, hd))
 
 
 def proj_params(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b):

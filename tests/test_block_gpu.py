@@ -1,5 +1,5 @@
 """GPU parity of the residual-block operators (m2d_layernorm_fwd, m2d_dwconv3x3_fwd, m2d_starrelu_fwd,
-m2d_scale_residual_fwd) through the C ABI, against the stock torch operators the reference uses (nn.LayerNorm, models/mamba2d.py:220;
+m2d_scale_residual_fwd, m2d_rope_qknorm_fwd) through the C ABI, against the stock torch operators the reference uses (nn.LayerNorm, models/mamba2d.py:220;
 depthwise nn.Conv2d, models/utils.py:101) evaluated in fp64 on the CPU.  Tolerances: fp32 2e-5,
 bf16 tensors 1e-2 (max error over max value; one bf16 rounding of the result is 4e-3)."""
 import pytest
@@ -91,3 +91,35 @@ def test_fused_elementwise_match_torch(cabi, shape, dtype, wdtype):
     got = cabi.scale_residual_fwd(xd, chan.cuda(), rd)
     want = x.double() * chan.double() + r.double()
     assert got.dtype == dtype and so.rel_err(got.float().cpu(), want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16], ids=["w_f32", "w_bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("shape", [(2, 7, 9, 10, 32), (1, 14, 14, 16, 32), (3, 5, 4, 3, 64), (1, 2, 3, 1, 8)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_rope_and_qk_norm_match_the_module(cabi, shape, dtype, wdtype):
+    """Against the attention module's own stock-operator path (mamba2d_amd.backbone.RoPEAttention2D, which
+    restates models/utils.py:253-301) evaluated in fp64 on the CPU."""
+    from mamba2d_amd.backbone import RoPEAttention2D
+    say(f"\ncase rope_qknorm {shape} {dtype} {wdtype}")
+    B, H, W, nh, hd = shape
+    g = torch.Generator().manual_seed(sum(shape))
+    att = RoPEAttention2D(nh * hd, head_dim=hd)
+    with torch.no_grad():
+        for m in (att.q_norm, att.k_norm):
+            m.weight.copy_((torch.rand(hd, generator=g) + 0.5).to(wdtype).float())
+            m.bias.copy_((torch.randn(hd, generator=g) * 0.3).to(wdtype).float())
+    qkv = torch.randn(B, H * W, 3, nh, hd, generator=g).to(dtype)
+    cos, sin = att._rope_tables(H, W, torch.device("cpu"), dtype)
+    q64, k64, _ = qkv.double().permute(2, 0, 3, 1, 4).unbind(0)
+    c64, s64 = cos.double(), sin.double()
+    want = []
+    for t, m in ((q64, att.q_norm), (k64, att.k_norm)):
+        r = t * c64 + att._rotate_pairs(t) * s64
+        want.append(torch.nn.functional.layer_norm(r, (hd,), m.weight.double(), m.bias.double(), m.eps))
+    wts = [t.detach().to(wdtype).cuda() for t in (att.q_norm.weight, att.q_norm.bias, att.k_norm.weight, att.k_norm.bias)]
+    q, k = cabi.rope_qknorm_fwd(qkv.cuda(), cos.cuda(), sin.cuda(), *wts, att.q_norm.eps)
+    torch.cuda.synchronize()
+    assert q.shape == (B, nh, H * W, hd) and q.dtype == dtype and q.is_contiguous()
+    assert so.rel_err(q.float().cpu(), want[0]) < TOL[dtype]
+    assert so.rel_err(k.float().cpu(), want[1]) < TOL[dtype]
