@@ -20,6 +20,7 @@ from __future__ import annotations
 
 import ctypes
 import os
+import weakref
 
 import torch
 import torch.nn.functional as F
@@ -136,6 +137,24 @@ def _c(t):
     return t if t.data_ptr() % 16 == 0 else t.clone()
 
 
+_F32_COPIES = {}   # id(parameter) -> (weak reference, version, data pointer, fp32 copy)
+
+
+def _as_f32(t):
+    """The parameter as a contiguous, aligned fp32 tensor.  fp32 parameters pass through; for others
+    (a model held in bf16) the copy is kept until the parameter changes, so that a forward does not
+    spend eight small kernels per scan on casting weights that did not change."""
+    if t.dtype == torch.float32:
+        return _c(t)
+    key = id(t)
+    hit = _F32_COPIES.get(key)
+    if hit is not None and hit[0]() is t and hit[1] == t._version and hit[2] == t.data_ptr():
+        return hit[3]
+    f = _c(t.detach().float())
+    _F32_COPIES[key] = (weakref.ref(t, lambda _, k=key: _F32_COPIES.pop(k, None)), t._version, t.data_ptr(), f)
+    return f
+
+
 class wf_cuda_fn_pr(torch.autograd.Function):
     """Scan + output projection on precomputed parameters (reference ``wavefront_cuda.py:146-196``).
 
@@ -217,7 +236,7 @@ class wf_cuda_fn_proj(torch.autograd.Function):
     def _params(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D):
         """The parameters as fp32 tensors (no copy if they already are): the library itself forms
         A = -exp(A_log) and rounds everything to x.dtype as the reference's casts do."""
-        return [_c(t.float()) for t in (AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D)]
+        return [_as_f32(t) for t in (AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D)]
 
     @classmethod
     def apply(cls, x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D, full=False, flip=False):

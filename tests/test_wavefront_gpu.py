@@ -230,6 +230,27 @@ def test_entry_point_replays_from_a_graph(wf, shape, dtype):
             assert torch.equal(a, b), i
 
 
+def test_cached_parameter_casts_follow_the_parameters(wf):
+    """Parameters held in bf16 are cast to fp32 once and the copy is reused; an in-place update of a
+    parameter (an optimiser step, a checkpoint load) must show in the next call."""
+    say("\ncase cached parameter casts")
+    B, H, W, E, N = 2, 6, 7, 32, 16
+    R = math.ceil(E / 16)
+    p = {k: v.bfloat16() for k, v in make_block_params(E, N, R, 1, "cuda").items()}
+    x = torch.randn(B, H, W, E, generator=torch.Generator().manual_seed(1)).cuda().bfloat16()
+    args = [p[k] for k in ORDER]
+    with torch.no_grad():
+        y1 = wf.wavefront_scan_cuda(x, *args)
+        y2 = wf.wavefront_scan_cuda(x, *args)
+        assert torch.equal(y1, y2)
+        p["D"].mul_(2.0)                                   # y = scan + x * D
+        y3 = wf.wavefront_scan_cuda(x, *args)
+        want = y1.float() + x.float() * (p["D"].float() / 2)
+        assert so.rel_err(y3.float().cpu(), want.cpu()) < 2e-2 and not torch.equal(y1, y3)
+        fresh = [t.clone() for t in args]                  # same values in new tensors: no stale copy may be used
+        assert torch.equal(wf.wavefront_scan_cuda(x, *fresh), y3)
+
+
 def test_views_that_start_off_alignment_are_accepted(wf, cscan):
     """A contiguous view whose first element is not 16-byte aligned is copied, not rejected."""
     say("\ncase unaligned views")
