@@ -214,6 +214,21 @@ int m2d_rope_qknorm_fwd(int B, int L, int heads, int head_dim, int dtype, int we
                         const void* q_weight, const void* q_bias, const void* k_weight, const void* k_bias,
                         float eps, void* q, void* k, void* stream);
 
+/* y = post(pre(x) weight^T + bias) for the narrow linear layers of a block on bf16 activations: in_proj and
+ * out_proj of the token mixer (models/mamba2d.py:166-176), the pointwise convolutions of the local path
+ * (models/utils.py:87-118) and the MLP (models/utils.py:58-81), together with the activation the block
+ * applies before or after the layer.  x (P,K) and y (P,N) are bf16; weight (N,K), bias (N, may be NULL) and
+ * the activation parameters have weight_dtype.  pre_act / post_act: 0 nothing, 1 GELU (exact form),
+ * 2 StarReLU with the one-element scale and bias given (device pointers, ignored otherwise).
+ * K must be a multiple of 32 up to 512, N a multiple of 16, and N * (K + 8) at most 72000 (the weight
+ * matrix is held in LDS as bf16); M2D_ERR_UNSUPPORTED otherwise. */
+#define M2D_ACT_NONE 0
+#define M2D_ACT_GELU 1
+#define M2D_ACT_STARRELU 2
+int m2d_linear_fwd(int64_t P, int K, int N, int weight_dtype, const void* x, const void* weight, const void* bias,
+                   int pre_act, const void* pre_scale, const void* pre_bias,
+                   int post_act, const void* post_scale, const void* post_bias, void* y, void* stream);
+
 /* Measurement aid; no counterpart in the reference.  While enabled, every m2d_scan_fwd /
  * m2d_scan_bwd call records a pair of HIP events on its stream around the main scan kernel of
  * the pass (not around the small set-up and reduction kernels).  m2d_profile_last_ms waits for

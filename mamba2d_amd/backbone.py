@@ -22,8 +22,8 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .wavefront import (dwconv3x3_fwd_op, layernorm_fwd_op, rope_qknorm_fwd_op, scale_residual_fwd_op,
-                        starrelu_fwd_op, wavefront_scan_cuda)
+from .wavefront import (dwconv3x3_fwd_op, layernorm_fwd_op, linear_act_fwd_op, rope_qknorm_fwd_op,
+                        scale_residual_fwd_op, starrelu_fwd_op, wavefront_scan_cuda)
 
 M2D_T = dict(n_blocks=(3, 3, 9, 3), embed_dim=(64, 128, 320, 512),
              token_mixer=("2D_local", "2D_local", "RopeAttention", "RopeAttention"),
@@ -33,6 +33,32 @@ M2D_T = dict(n_blocks=(3, 3, 9, 3), embed_dim=(64, 128, 320, 512),
 def _inference(*tensors):
     """No gradient will be asked of this call: the library's inference kernels may take it."""
     return not torch.is_grad_enabled() or not any(t.requires_grad for t in tensors)
+
+
+ACT_NONE, ACT_GELU, ACT_STARRELU = 0, 1, 2
+
+
+def _act(kind, star, t):
+    if kind == ACT_GELU:
+        return F.gelu(t)
+    return star(t) if kind == ACT_STARRELU else t
+
+
+def linear_act(lin, x, pre=ACT_NONE, post=ACT_NONE, star=None):
+    """post(lin(pre(x))) for a narrow linear layer: pre / post are nothing, GELU, or the StarReLU module
+    ``star``.  At inference on bf16 activations the product runs in the library's kernel together with its
+    neighbouring activation where the weight matrix fits 46 KB of LDS (64 or 128 channels wide: there the
+    kernel is bound by the activations' bytes; wider layers are faster in the stock library); otherwise
+    stock operators."""
+    w, b = lin.weight, lin.bias
+    N, K = w.shape
+    if (x.is_cuda and x.dtype == torch.bfloat16 and _inference(x, w) and w.dtype in (torch.float32, torch.bfloat16)
+            and K % 32 == 0 and K <= 512 and N % 16 == 0 and N * (K + 8) <= 23000 and x.numel() > 0
+            and (star is None or star.scale.dtype == w.dtype)):
+        ps = (star.scale, star.bias) if pre == ACT_STARRELU else (None, None)
+        qs = (star.scale, star.bias) if post == ACT_STARRELU else (None, None)
+        return linear_act_fwd_op(x.contiguous(), w, b, pre, *ps, post, *qs)
+    return _act(post, star, lin(_act(pre, star, x)))
 
 
 class LayerNorm(nn.LayerNorm):
@@ -93,7 +119,7 @@ class MLP(nn.Module):
         self.fc2 = nn.Linear(dim * expand, dim)
 
     def forward(self, x):
-        return self.fc2(F.gelu(self.fc1(x)))
+        return linear_act(self.fc2, linear_act(self.fc1, x, post=ACT_GELU))
 
 
 def _conv_channel_last(conv, x):
@@ -117,7 +143,7 @@ class SepConv(nn.Module):
         self.pwconv2 = nn.Linear(med, dim, bias=False)
 
     def forward(self, x):
-        x = self.act1(self.pwconv1(x))
+        x = linear_act(self.pwconv1, x, post=ACT_STARRELU, star=self.act1)
         w = self.dwconv.weight
         if (x.is_cuda and _inference(x, w) and self.dwconv.kernel_size == (3, 3) and self.dwconv.padding == (1, 1)
                 and x.dtype in (torch.float32, torch.bfloat16) and w.dtype in (torch.float32, torch.bfloat16)
@@ -127,7 +153,7 @@ class SepConv(nn.Module):
             x = dwconv3x3_fwd_op(x.contiguous(), w)
         else:
             x = _conv_channel_last(self.dwconv, x)
-        return self.pwconv2(self.act2(x))
+        return linear_act(self.pwconv2, x, pre=ACT_STARRELU, star=self.act2)
 
 
 class Downsampling(nn.Module):
@@ -180,11 +206,11 @@ class M2DBlock(nn.Module):
 
     def forward(self, x):           # (B, H, W, C)
         local = self.local_path(self.local_norm(x)) if self.local_path is not None else None
-        u = F.gelu(self.in_proj(x))
+        u = linear_act(self.in_proj, x, post=ACT_GELU)
         y = wavefront_scan_cuda(u, self.AT_log, self.AL_log, self.x_proj.weight,
                                 self.dt_projT.weight, self.dt_projT.bias,
                                 self.dt_projL.weight, self.dt_projL.bias, self.D, self.recomp, flip=self.flip)
-        y = self.out_proj(F.gelu(y))
+        y = linear_act(self.out_proj, y, pre=ACT_GELU)
         return y if local is None else y + local
 
 

@@ -24,7 +24,7 @@ M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
            "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_bwd", "m2d_proj_workspace_bytes", "m2d_proj_fwd",
            "m2d_proj_bwd", "m2d_layernorm_fwd", "m2d_dwconv3x3_fwd", "m2d_starrelu_fwd",
-           "m2d_scale_residual_fwd", "m2d_rope_qknorm_fwd", "m2d_profile_enable", "m2d_profile_last_ms")
+           "m2d_scale_residual_fwd", "m2d_rope_qknorm_fwd", "m2d_linear_fwd", "m2d_profile_enable", "m2d_profile_last_ms")
 
 
 class Desc(ctypes.Structure):
@@ -74,6 +74,8 @@ def _load():
     lib.m2d_scale_residual_fwd.argtypes = [ctypes.c_int64, i32, i32, i32, vp, vp, vp, vp, vp]
     lib.m2d_rope_qknorm_fwd.restype = i32
     lib.m2d_rope_qknorm_fwd.argtypes = [i32] * 6 + [vp] * 7 + [ctypes.c_float, vp, vp, vp]
+    lib.m2d_linear_fwd.restype = i32
+    lib.m2d_linear_fwd.argtypes = [ctypes.c_int64, i32, i32, i32, vp, vp, vp, i32, vp, vp, i32, vp, vp, vp, vp]
     lib.m2d_profile_enable.restype = i32
     lib.m2d_profile_enable.argtypes = [i32]
     lib.m2d_profile_last_ms.restype = i32
@@ -326,3 +328,29 @@ def rope_qknorm_fwd(qkv, cos, sin, q_weight, q_bias, k_weight, k_bias, eps=1e-5)
                                   _ptr(q_weight), _ptr(q_bias), _ptr(k_weight), _ptr(k_bias), float(eps), _ptr(q), _ptr(k),
                                   _stream(qkv.device)))
     return q, k
+
+
+ACT_NONE, ACT_GELU, ACT_STARRELU = 0, 1, 2
+
+
+def linear_fwd(x, weight, bias=None, pre=ACT_NONE, pre_params=None, post=ACT_NONE, post_params=None):
+    """post(pre(x) @ weight.T + bias) on bf16 activations through m2d_linear_fwd; ``*_params`` are the
+    (scale, bias) one-element tensors of a StarReLU."""
+    K = x.shape[-1]
+    N = weight.shape[0]
+    if x.dtype != torch.bfloat16 or not x.is_cuda or not x.is_contiguous():
+        raise ValueError("m2dscan: x must be a contiguous bfloat16 tensor on the GPU")
+    if tuple(weight.shape) != (N, K) or not weight.is_contiguous() or weight.device != x.device:
+        raise ValueError(f"m2dscan: weight must be a contiguous (N,{K}) tensor on {x.device}")
+    small = [t for t in (bias, *(pre_params or ()), *(post_params or ())) if t is not None]
+    for t in small:
+        if t.dtype != weight.dtype or t.device != x.device or not t.is_contiguous():
+            raise ValueError("m2dscan: bias and activation parameters must have the weight's dtype and device")
+    if bias is not None and tuple(bias.shape) != (N,):
+        raise ValueError(f"m2dscan: bias must have shape ({N},)")
+    ps, pb = pre_params if pre == ACT_STARRELU else (None, None)
+    qs, qb = post_params if post == ACT_STARRELU else (None, None)
+    y = x.new_empty((*x.shape[:-1], N))
+    check(lib.m2d_linear_fwd(x.numel() // K, K, N, _dtype_code(weight), _ptr(x), _ptr(weight), _ptr(bias), pre, _ptr(ps), _ptr(pb),
+                             post, _ptr(qs), _ptr(qb), _ptr(y), _stream(x.device)))
+    return y

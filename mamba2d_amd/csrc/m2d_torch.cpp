@@ -303,6 +303,37 @@ std::tuple<Tensor, Tensor> rope_qknorm_fwd(const Tensor& qkv, const Tensor& cos,
   return {q, k};
 }
 
+Tensor linear_act_fwd(const Tensor& x, const Tensor& weight, const c10::optional<Tensor>& bias, int64_t pre,
+                      const c10::optional<Tensor>& pre_scale, const c10::optional<Tensor>& pre_bias, int64_t post,
+                      const c10::optional<Tensor>& post_scale, const c10::optional<Tensor>& post_bias) {
+  TORCH_CHECK(x.is_cuda() && x.dim() >= 1 && x.is_contiguous() && x.scalar_type() == at::kBFloat16,
+              "m2dscan: x must be a contiguous bfloat16 tensor on the GPU");
+  const int64_t K = x.size(-1);
+  TORCH_CHECK(weight.dim() == 2 && weight.size(1) == K && weight.is_contiguous() && weight.device() == x.device(),
+              "m2dscan: weight must be a contiguous (N,", K, ") tensor on x's device");
+  const int64_t N = weight.size(0);
+  auto small = [&](const c10::optional<Tensor>& t, int64_t n, const char* name) -> const void* {
+    if (!t.has_value() || !t->defined()) return nullptr;
+    TORCH_CHECK(t->numel() == n && t->is_contiguous() && t->device() == x.device() && t->scalar_type() == weight.scalar_type(),
+                "m2dscan: ", name, " must hold ", n, " elements of the weight's dtype on x's device");
+    return t->data_ptr();
+  };
+  const void* b = small(bias, N, "bias");
+  const void* ps = small(pre_scale, 1, "pre_scale");
+  const void* pb = small(pre_bias, 1, "pre_bias");
+  const void* qs = small(post_scale, 1, "post_scale");
+  const void* qb = small(post_bias, 1, "post_bias");
+  c10::DeviceGuard guard(x.device());
+  std::vector<int64_t> shape(x.sizes().begin(), x.sizes().end());
+  shape.back() = N;
+  Tensor y = at::empty(shape, x.options());
+  if (x.numel() == 0) return y;
+  hipStream_t st = c10::hip::getCurrentHIPStream(x.device().index()).stream();
+  check(m2d_linear_fwd(x.numel() / K, static_cast<int>(K), static_cast<int>(N), dtype_code(weight, "weight"), x.data_ptr(),
+                       weight.data_ptr(), b, static_cast<int>(pre), ps, pb, static_cast<int>(post), qs, qb, y.data_ptr(), st));
+  return y;
+}
+
 int64_t abi_version() { return m2d_version(); }
 
 }  // namespace
@@ -323,6 +354,8 @@ TORCH_LIBRARY(m2dscan, m) {
   m.def("scale_residual_fwd(Tensor x, Tensor scale, Tensor residual) -> Tensor");
   m.def("rope_qknorm_fwd(Tensor qkv, Tensor cos, Tensor sin, Tensor q_weight, Tensor q_bias, Tensor k_weight, Tensor k_bias, "
         "float eps) -> (Tensor, Tensor)");
+  m.def("linear_act_fwd(Tensor x, Tensor weight, Tensor? bias, int pre, Tensor? pre_scale, Tensor? pre_bias, int post, "
+        "Tensor? post_scale, Tensor? post_bias) -> Tensor");
   m.def("abi_version() -> int", &abi_version);
 }
 
@@ -336,4 +369,5 @@ TORCH_LIBRARY_IMPL(m2dscan, CUDA, m) {   // ROCm devices dispatch under the CUDA
   m.impl("starrelu_fwd", &starrelu_fwd);
   m.impl("scale_residual_fwd", &scale_residual_fwd);
   m.impl("rope_qknorm_fwd", &rope_qknorm_fwd);
+  m.impl("linear_act_fwd", &linear_act_fwd);
 }

@@ -11,6 +11,7 @@
 // model under autocast hands fp32 weights to bf16 activations).  Arithmetic is fp32.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <stdint.h>
 
 #include "../../include/m2dscan.h"
@@ -368,6 +369,165 @@ int run_rope(const RopeArgs& a, int G, hipStream_t st) {
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
+// ---------------------------------------------------------------- small linear layers, bf16
+// y = post(pre(x) W^T + bias) for the narrow layers of a block (K and N up to 512): in_proj, out_proj,
+// the pointwise convolutions of the local path and the MLP at 64 or 128 channels
+// (models/mamba2d.py:166-176, models/utils.py:58-81, 87-118).  These products are bandwidth-bound: a row
+// of x is 128 to 512 bytes and is used once.  The weight matrix lives in LDS as bf16 for the whole
+// (persistent) workgroup; a wave owns 16 rows, whose 16-byte pieces are the A operands of
+// v_mfma_f32_16x16x32_bf16 as they come from memory (lane l: row l & 15, columns 8 (l >> 4) + j of a step
+// of 32), W's rows are the B operands (lane l: output l & 15, the same columns), results leave through a
+// per-wave LDS block so that memory sees 16-byte pieces of rows.  pre and post are nothing, GELU (exact
+// form, through erf) or StarReLU: the activation that the block applies before or after the layer.
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ f32x4_t mfma_bf16(uint4 a, uint4 b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+__device__ __forceinline__ uint4 ld16(const void* p) { return *reinterpret_cast<const uint4*>(p); }
+
+constexpr int kLinThreads = 256;
+constexpr int kLinWaves = 4;
+constexpr int kLinStage = 72;      // floats per row of a wave's result block: 64 + 8
+constexpr int kLinMaxKC = 16;      // steps of 32 along K: K <= 512
+enum { kActNone = 0, kActGelu = 1, kActStarRelu = 2 };
+
+// erf by Abramowitz & Stegun 7.1.26 (absolute error below 1.5e-7), one v_exp_f32 and one v_rcp_f32
+__device__ __forceinline__ float gelu_exact(float v) {
+  const float z = fabsf(v) * 0.70710678118654752f;
+  const float t = __builtin_amdgcn_rcpf(__builtin_fmaf(0.3275911f, z, 1.f));
+  float poly = __builtin_fmaf(t, 1.061405429f, -1.453152027f);
+  poly = __builtin_fmaf(t, poly, 1.421413741f);
+  poly = __builtin_fmaf(t, poly, -0.284496736f);
+  poly = __builtin_fmaf(t, poly, 0.254829592f);
+  const float e = 1.f - poly * t * __builtin_amdgcn_exp2f(-z * z * 1.44269504088896341f);   // erf(|v| / sqrt 2)
+  return 0.5f * v + 0.5f * fabsf(v) * e;                                                   // v erf(v/sqrt 2) = |v| erf(|v|/sqrt 2)
+}
+__device__ __forceinline__ float act(int kind, float v, float s, float b) {
+  if (kind == kActGelu) return gelu_exact(v);
+  if (kind == kActStarRelu) { const float t = fmaxf(v, 0.f); return __builtin_fmaf(s * t, t, b); }
+  return v;
+}
+
+struct LinArgs {
+  const void* x;        // (P, K) bf16
+  const void* w;        // (N, K)
+  const void* bias;     // (N) or null
+  void* y;              // (P, N) bf16
+  int64_t P;
+  int K, N, wbf16, pre, post, ntiles;
+  const void *pre_s, *pre_b, *post_s, *post_b;   // StarReLU scale and bias (one element each, type of w) where pre / post is StarReLU
+};
+
+template <int KCMAX>   // steps of 32 along K that the kernel is built for: 2, 4, 8 or 16
+__global__ __launch_bounds__(kLinThreads) void m2d_linear_kernel(const LinArgs a) {
+  extern __shared__ float smem[];
+  const int tid = threadIdx.x, l = tid & 63, mn = l & 15, kb = l >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int ws = a.K + 8;                                // bf16 per row of W in LDS: rows stay 16-byte aligned and spread over the banks
+  uint16_t* wl = reinterpret_cast<uint16_t*>(smem);
+  float* stage = smem + (a.N * ws / 2 + 3) / 4 * 4 + wave * 16 * kLinStage;
+  for (int i = tid; i < a.N * (a.K / 8); i += kLinThreads) {
+    const int n = i / (a.K / 8), k8 = i - n * (a.K / 8);
+    uint4 q;
+    if (a.wbf16) {
+      q = ld16(static_cast<const uint16_t*>(a.w) + (int64_t)n * a.K + 8 * k8);
+    } else {
+      const float* src = static_cast<const float*>(a.w) + (int64_t)n * a.K + 8 * k8;
+      q = make_uint4(pack_bf16(src[0], src[1]), pack_bf16(src[2], src[3]), pack_bf16(src[4], src[5]), pack_bf16(src[6], src[7]));
+    }
+    *reinterpret_cast<uint4*>(wl + n * ws + 8 * k8) = q;
+  }
+  __syncthreads();
+  const float pre_s = a.pre == kActStarRelu ? ldw(a.pre_s, a.wbf16, 0) : 0.f, pre_b = a.pre == kActStarRelu ? ldw(a.pre_b, a.wbf16, 0) : 0.f;
+  const float post_s = a.post == kActStarRelu ? ldw(a.post_s, a.wbf16, 0) : 0.f, post_b = a.post == kActStarRelu ? ldw(a.post_b, a.wbf16, 0) : 0.f;
+  const int KC = a.K / 32;
+  const uint16_t* X = static_cast<const uint16_t*>(a.x);
+  uint16_t* Y = static_cast<uint16_t*>(a.y);
+  // The rows of the next tile are fetched while the current one is worked on: with the weights in LDS
+  // few waves fit a compute unit, too few to cover the latency of memory by themselves.
+  uint4 Anext[KCMAX];
+  auto fetch = [&](int tile) {
+    const int64_t q0 = (int64_t)tile * 64 + wave * 16;
+#pragma unroll
+    for (int kc = 0; kc < KCMAX; ++kc) {
+      Anext[kc] = make_uint4(0u, 0u, 0u, 0u);
+      if (kc < KC && tile < a.ntiles && q0 + mn < a.P) Anext[kc] = ld16(X + (q0 + mn) * a.K + 32 * kc + 8 * kb);
+    }
+  };
+  fetch(blockIdx.x);
+  for (int tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
+    const int64_t p0 = (int64_t)tile * 64 + wave * 16;
+    const int rows = (int)(a.P - p0 < 16 ? a.P - p0 : 16);     // rows of the wave inside the array (may be <= 0)
+    uint4 A[KCMAX];
+#pragma unroll
+    for (int kc = 0; kc < KCMAX; ++kc) A[kc] = Anext[kc];
+    fetch(tile + gridDim.x);
+    if (a.pre != kActNone) {   // (uniform)
+#pragma unroll
+      for (int kc = 0; kc < KCMAX; ++kc)
+        if (kc < KC) {
+          uint32_t w4[4] = {A[kc].x, A[kc].y, A[kc].z, A[kc].w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            w4[j] = pack_bf16(act(a.pre, bf_lo(w4[j]), pre_s, pre_b), act(a.pre, bf_hi(w4[j]), pre_s, pre_b));
+          A[kc] = make_uint4(w4[0], w4[1], w4[2], w4[3]);
+        }
+    }
+    for (int n0 = 0; n0 < a.N; n0 += 64) {
+#pragma unroll
+      for (int nt = 0; nt < 4; ++nt) {
+        const int n = n0 + 16 * nt + mn;
+        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+        if (n0 + 16 * nt < a.N) {   // (uniform)
+          const uint16_t* wrow = wl + n * ws + 8 * kb;
+#pragma unroll
+          for (int kc = 0; kc < KCMAX; ++kc)
+            if (kc < KC) acc = mfma_bf16(A[kc], ld16(wrow + 32 * kc), acc);
+          const float bn = a.bias ? ldw(a.bias, a.wbf16, n) : 0.f;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[i] = act(a.post, acc[i] + bn, post_s, post_b);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) stage[(4 * kb + i) * kLinStage + 16 * nt + mn] = acc[i];   // position 4 kb + i, output 16 nt + mn
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {   // the block's 16 x 8 pieces of 8 outputs, two per lane
+        const int piece = l + 64 * k, c = piece >> 3, c8 = 8 * (piece & 7);
+        if (c < rows && n0 + c8 < a.N) {
+          const float4 lo = *reinterpret_cast<const float4*>(stage + c * kLinStage + c8);
+          const float4 hi = *reinterpret_cast<const float4*>(stage + c * kLinStage + c8 + 4);
+          *reinterpret_cast<uint4*>(Y + (p0 + c) * a.N + n0 + c8) =
+              make_uint4(pack_bf16(lo.x, lo.y), pack_bf16(lo.z, lo.w), pack_bf16(hi.x, hi.y), pack_bf16(hi.z, hi.w));
+        }
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+  }
+}
+
+constexpr size_t kLinMaxLds = 160 * 1024;   // LDS of a compute unit
+
+// More than 64 KB of dynamic LDS has to be allowed per kernel and device, once.
+inline bool allow_big_lds() {
+  static std::atomic<uint64_t> seen{0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return false;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (seen.load(std::memory_order_acquire) & bit) return true;
+  const void* kernels[] = {reinterpret_cast<const void*>(&m2d_linear_kernel<2>), reinterpret_cast<const void*>(&m2d_linear_kernel<4>),
+                           reinterpret_cast<const void*>(&m2d_linear_kernel<8>), reinterpret_cast<const void*>(&m2d_linear_kernel<16>)};
+  for (const void* k : kernels)
+    if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLinMaxLds) != hipSuccess) return false;
+  seen.fetch_or(bit, std::memory_order_release);
+  return true;
+}
+
+inline size_t linear_lds_bytes(int K, int N) { return ((size_t)N * (K + 8) / 2 + 3) / 4 * 4 * 4 + (size_t)kLinWaves * 16 * kLinStage * 4; }
+
 inline bool misaligned(const void* p, size_t n) { return (reinterpret_cast<uintptr_t>(p) & (n - 1)) != 0; }
 
 }  // namespace
@@ -464,6 +624,38 @@ int m2d_rope_qknorm_fwd(int B, int L, int heads, int head_dim, int dtype, int we
   a.total = (int64_t)B * L * 2 * heads * G;
   hipStream_t st = static_cast<hipStream_t>(stream);
   return dtype == M2D_F32 ? run_rope<float>(a, G, st) : run_rope<bf16_t>(a, G, st);
+}
+
+int m2d_linear_fwd(int64_t P, int K, int N, int weight_dtype, const void* x, const void* weight, const void* bias,
+                   int pre_act, const void* pre_scale, const void* pre_bias, int post_act, const void* post_scale,
+                   const void* post_bias, void* y, void* stream) {
+  if (!x || !weight || !y) return M2D_ERR_NULL_POINTER;
+  if ((pre_act == kActStarRelu && (!pre_scale || !pre_bias)) || (post_act == kActStarRelu && (!post_scale || !post_bias)))
+    return M2D_ERR_NULL_POINTER;
+  if (P < 1 || K < 1 || N < 1) return M2D_ERR_BAD_SHAPE;
+  if (weight_dtype != M2D_F32 && weight_dtype != M2D_BF16) return M2D_ERR_UNSUPPORTED;
+  if (pre_act < kActNone || pre_act > kActStarRelu || post_act < kActNone || post_act > kActStarRelu) return M2D_ERR_UNSUPPORTED;
+  if (K % 32 != 0 || K > 32 * kLinMaxKC || N % 16 != 0 || linear_lds_bytes(K, N) > kLinMaxLds) return M2D_ERR_UNSUPPORTED;
+  if ((P + 63) / 64 >= ((int64_t)1 << 31)) return M2D_ERR_UNSUPPORTED;
+  if (misaligned(x, 16) || misaligned(y, 16) || misaligned(weight, 16) || (bias && misaligned(bias, 4))) return M2D_ERR_MISALIGNED;
+  LinArgs a = {};
+  a.x = x; a.w = weight; a.bias = bias; a.y = y; a.P = P; a.K = K; a.N = N; a.wbf16 = weight_dtype == M2D_BF16;
+  a.pre = pre_act; a.post = post_act; a.pre_s = pre_scale; a.pre_b = pre_bias; a.post_s = post_scale; a.post_b = post_bias;
+  a.ntiles = (int)((P + 63) / 64);
+  const size_t lds = linear_lds_bytes(K, N);
+  if (lds > 64 * 1024 && !allow_big_lds()) return M2D_ERR_HIP;
+  // persistent: the weights are loaded into LDS once per workgroup; as many workgroups as fit the device at once
+  int per_cu = (int)(160 * 1024 / lds);
+  if (per_cu > 8) per_cu = 8;
+  int grid = 256 * per_cu;
+  if (grid > a.ntiles) grid = a.ntiles;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const dim3 g((unsigned)grid), t(kLinThreads);
+  if (K <= 64) hipLaunchKernelGGL(m2d_linear_kernel<2>, g, t, lds, st, a);
+  else if (K <= 128) hipLaunchKernelGGL(m2d_linear_kernel<4>, g, t, lds, st, a);
+  else if (K <= 256) hipLaunchKernelGGL(m2d_linear_kernel<8>, g, t, lds, st, a);
+  else hipLaunchKernelGGL(m2d_linear_kernel<16>, g, t, lds, st, a);
+  return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
 }  // extern "C"

@@ -42,6 +42,7 @@ dwconv3x3_fwd_op = torch.ops.m2dscan.dwconv3x3_fwd
 starrelu_fwd_op = torch.ops.m2dscan.starrelu_fwd
 scale_residual_fwd_op = torch.ops.m2dscan.scale_residual_fwd
 rope_qknorm_fwd_op = torch.ops.m2dscan.rope_qknorm_fwd
+linear_act_fwd_op = torch.ops.m2dscan.linear_act_fwd
 
 # Keep the forward's anti-diagonal checkpoints for the backward (faster backward, more saved
 # memory) or rebuild them inside the backward (nothing saved beyond the inputs, like the
@@ -107,6 +108,11 @@ def _starrelu_fwd_fake(x, scale, bias):
 @torch.library.register_fake("m2dscan::scale_residual_fwd")
 def _scale_residual_fwd_fake(x, scale, residual):
     return torch.empty_like(x)
+
+
+@torch.library.register_fake("m2dscan::linear_act_fwd")
+def _linear_act_fwd_fake(x, weight, bias, pre, pre_scale, pre_bias, post, post_scale, post_bias):
+    return x.new_empty((*x.shape[:-1], weight.shape[0]))
 
 
 @torch.library.register_fake("m2dscan::rope_qknorm_fwd")

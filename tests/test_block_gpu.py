@@ -1,5 +1,5 @@
 """GPU parity of the residual-block operators (m2d_layernorm_fwd, m2d_dwconv3x3_fwd, m2d_starrelu_fwd,
-m2d_scale_residual_fwd, m2d_rope_qknorm_fwd) through the C ABI, against the stock torch operators the reference uses (nn.LayerNorm, models/mamba2d.py:220;
+m2d_scale_residual_fwd, m2d_rope_qknorm_fwd, m2d_linear_fwd) through the C ABI, against the stock torch operators the reference uses (nn.LayerNorm, models/mamba2d.py:220;
 depthwise nn.Conv2d, models/utils.py:101) evaluated in fp64 on the CPU.  Tolerances: fp32 2e-5,
 bf16 tensors 1e-2 (max error over max value; one bf16 rounding of the result is 4e-3)."""
 import pytest
@@ -123,3 +123,52 @@ def test_rope_and_qk_norm_match_the_module(cabi, shape, dtype, wdtype):
     assert q.shape == (B, nh, H * W, hd) and q.dtype == dtype and q.is_contiguous()
     assert so.rel_err(q.float().cpu(), want[0]) < TOL[dtype]
     assert so.rel_err(k.float().cpu(), want[1]) < TOL[dtype]
+
+
+# rows, K, N: the narrow layers of the model at 64 and 128 channels, rows that end inside a tile of 64, one tile
+LIN_SHAPES = [(2 * 9 * 12, 64, 64), (1000, 64, 128), (333, 128, 64), (77, 64, 256), (130, 256, 64), (64, 128, 128), (5, 32, 16),
+              (200, 128, 512), (190, 512, 128), (70, 256, 128)]
+
+
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16], ids=["w_f32", "w_bf16"])
+@pytest.mark.parametrize("acts", [(0, 0), (0, 1), (1, 0), (0, 2), (2, 0), (2, 1)], ids=lambda a: f"pre{a[0]}_post{a[1]}")
+@pytest.mark.parametrize("shape", LIN_SHAPES, ids=lambda s: "x".join(map(str, s)))
+def test_small_linear_matches_torch(cabi, shape, acts, wdtype):
+    """bf16 activations, weights rounded to bf16 (as a bf16 model or autocast would), fp64 reference."""
+    say(f"\ncase linear {shape} pre/post {acts} {wdtype}")
+    rows, K, N = shape
+    pre, post = acts
+    g = torch.Generator().manual_seed(rows + K + N)
+    x = torch.randn(rows, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) / K ** 0.5).to(wdtype)
+    b = (torch.randn(N, generator=g) * 0.3).to(wdtype)
+    sc, bi = torch.tensor([0.8944]).to(wdtype), torch.tensor([-0.4472]).to(wdtype)
+
+    def ref_act(kind, t):
+        if kind == 1:
+            return torch.nn.functional.gelu(t)
+        if kind == 2:
+            return sc.double() * torch.relu(t) ** 2 + bi.double()
+        return t
+
+    a_in = ref_act(pre, x.double())
+    if pre:
+        a_in = a_in.bfloat16().double()       # the activated input is the bf16 operand of the product
+    want = ref_act(post, a_in @ w.bfloat16().double().t() + b.double())
+    params = (sc.cuda(), bi.cuda())
+    got = cabi.linear_fwd(x.cuda(), w.cuda(), b.cuda(), pre, params if pre == 2 else None, post, params if post == 2 else None)
+    torch.cuda.synchronize()
+    assert got.dtype == torch.bfloat16 and got.shape == (rows, N)
+    assert so.rel_err(got.float().cpu(), want) < 1e-2
+    nb = cabi.linear_fwd(x.cuda(), w.cuda(), None, pre, params if pre == 2 else None, post, params if post == 2 else None)
+    want_nb = ref_act(post, a_in @ w.bfloat16().double().t())
+    assert so.rel_err(nb.float().cpu(), want_nb) < 1e-2
+
+
+def test_small_linear_limits_are_reported(cabi):
+    x = torch.zeros(8, 48, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(cabi.M2DError):
+        cabi.linear_fwd(x, torch.zeros(16, 48, device="cuda"))            # K is no multiple of 32
+    x = torch.zeros(8, 512, device="cuda", dtype=torch.bfloat16)
+    with pytest.raises(cabi.M2DError):
+        cabi.linear_fwd(x, torch.zeros(256, 512, device="cuda"))          # the weights do not fit into LDS
