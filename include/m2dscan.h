@@ -220,8 +220,8 @@ int m2d_rope_qknorm_fwd(int B, int L, int heads, int head_dim, int dtype, int we
  * applies before or after the layer.  x (P,K) and y (P,N) are bf16; weight (N,K), bias (N, may be NULL) and
  * the activation parameters have weight_dtype.  pre_act / post_act: 0 nothing, 1 GELU (exact form),
  * 2 StarReLU with the one-element scale and bias given (device pointers, ignored otherwise).
- * K must be a multiple of 32 up to 512, N a multiple of 16, and N * (K + 8) at most 72000 (the weight
- * matrix is held in LDS as bf16); M2D_ERR_UNSUPPORTED otherwise. */
+ * K must be a multiple of 32 up to 512 and N a multiple of 16 (the weight matrix is held in LDS as bf16,
+ * in slices of 64 or more outputs per workgroup); M2D_ERR_UNSUPPORTED otherwise. */
 #define M2D_ACT_NONE 0
 #define M2D_ACT_GELU 1
 #define M2D_ACT_STARRELU 2

@@ -47,13 +47,13 @@ def _act(kind, star, t):
 def linear_act(lin, x, pre=ACT_NONE, post=ACT_NONE, star=None):
     """post(lin(pre(x))) for a narrow linear layer: pre / post are nothing, GELU, or the StarReLU module
     ``star``.  At inference on bf16 activations the product runs in the library's kernel together with its
-    neighbouring activation where the weight matrix fits 46 KB of LDS (64 or 128 channels wide: there the
-    kernel is bound by the activations' bytes; wider layers are faster in the stock library); otherwise
-    stock operators."""
+    neighbouring activation where the layer is narrow (up to 256 inputs and 512 outputs, the layers of the
+    stages with 64 and 128 channels: there the kernel is bound by the activations' bytes; wider layers are
+    faster in the stock library); otherwise stock operators."""
     w, b = lin.weight, lin.bias
     N, K = w.shape
     if (x.is_cuda and x.dtype == torch.bfloat16 and _inference(x, w) and w.dtype in (torch.float32, torch.bfloat16)
-            and K % 32 == 0 and K <= 512 and N % 16 == 0 and N * (K + 8) <= 23000 and x.numel() > 0
+            and K % 32 == 0 and K <= 256 and N % 16 == 0 and N <= 512 and x.numel() > 0
             and (star is None or star.scale.dtype == w.dtype)):
         ps = (star.scale, star.bias) if pre == ACT_STARRELU else (None, None)
         qs = (star.scale, star.bias) if post == ACT_STARRELU else (None, None)

@@ -416,6 +416,7 @@ struct LinArgs {
   void* y;              // (P, N) bf16
   int64_t P;
   int K, N, wbf16, pre, post, ntiles;
+  int nsplit, Ns;       // the workgroups share out the N outputs in nsplit slices of Ns
   const void *pre_s, *pre_b, *post_s, *post_b;   // StarReLU scale and bias (one element each, type of w) where pre / post is StarReLU
 };
 
@@ -426,14 +427,16 @@ __global__ __launch_bounds__(kLinThreads) void m2d_linear_kernel(const LinArgs a
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int ws = a.K + 8;                                // bf16 per row of W in LDS: rows stay 16-byte aligned and spread over the banks
   uint16_t* wl = reinterpret_cast<uint16_t*>(smem);
-  float* stage = smem + (a.N * ws / 2 + 3) / 4 * 4 + wave * 16 * kLinStage;
-  for (int i = tid; i < a.N * (a.K / 8); i += kLinThreads) {
+  float* stage = smem + (a.Ns * ws / 2 + 3) / 4 * 4 + wave * 16 * kLinStage;
+  const int slice = blockIdx.x % a.nsplit, nbase = slice * a.Ns;   // this workgroup's outputs: nbase .. nbase + Ns
+  const int first_tile = blockIdx.x / a.nsplit, tile_step = gridDim.x / a.nsplit;
+  for (int i = tid; i < a.Ns * (a.K / 8); i += kLinThreads) {
     const int n = i / (a.K / 8), k8 = i - n * (a.K / 8);
     uint4 q;
     if (a.wbf16) {
-      q = ld16(static_cast<const uint16_t*>(a.w) + (int64_t)n * a.K + 8 * k8);
+      q = ld16(static_cast<const uint16_t*>(a.w) + (int64_t)(nbase + n) * a.K + 8 * k8);
     } else {
-      const float* src = static_cast<const float*>(a.w) + (int64_t)n * a.K + 8 * k8;
+      const float* src = static_cast<const float*>(a.w) + (int64_t)(nbase + n) * a.K + 8 * k8;
       q = make_uint4(pack_bf16(src[0], src[1]), pack_bf16(src[2], src[3]), pack_bf16(src[4], src[5]), pack_bf16(src[6], src[7]));
     }
     *reinterpret_cast<uint4*>(wl + n * ws + 8 * k8) = q;
@@ -455,14 +458,14 @@ __global__ __launch_bounds__(kLinThreads) void m2d_linear_kernel(const LinArgs a
       if (kc < KC && tile < a.ntiles && q0 + mn < a.P) Anext[kc] = ld16(X + (q0 + mn) * a.K + 32 * kc + 8 * kb);
     }
   };
-  fetch(blockIdx.x);
-  for (int tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
+  fetch(first_tile);
+  for (int tile = first_tile; tile < a.ntiles; tile += tile_step) {
     const int64_t p0 = (int64_t)tile * 64 + wave * 16;
     const int rows = (int)(a.P - p0 < 16 ? a.P - p0 : 16);     // rows of the wave inside the array (may be <= 0)
     uint4 A[KCMAX];
 #pragma unroll
     for (int kc = 0; kc < KCMAX; ++kc) A[kc] = Anext[kc];
-    fetch(tile + gridDim.x);
+    fetch(tile + tile_step);
     if (a.pre != kActNone) {   // (uniform)
 #pragma unroll
       for (int kc = 0; kc < KCMAX; ++kc)
@@ -474,17 +477,17 @@ __global__ __launch_bounds__(kLinThreads) void m2d_linear_kernel(const LinArgs a
           A[kc] = make_uint4(w4[0], w4[1], w4[2], w4[3]);
         }
     }
-    for (int n0 = 0; n0 < a.N; n0 += 64) {
+    for (int n0 = 0; n0 < a.Ns; n0 += 64) {
 #pragma unroll
       for (int nt = 0; nt < 4; ++nt) {
         const int n = n0 + 16 * nt + mn;
         f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-        if (n0 + 16 * nt < a.N) {   // (uniform)
+        if (n0 + 16 * nt < a.Ns) {   // (uniform)
           const uint16_t* wrow = wl + n * ws + 8 * kb;
 #pragma unroll
           for (int kc = 0; kc < KCMAX; ++kc)
             if (kc < KC) acc = mfma_bf16(A[kc], ld16(wrow + 32 * kc), acc);
-          const float bn = a.bias ? ldw(a.bias, a.wbf16, n) : 0.f;
+          const float bn = a.bias ? ldw(a.bias, a.wbf16, nbase + n) : 0.f;
 #pragma unroll
           for (int i = 0; i < 4; ++i) acc[i] = act(a.post, acc[i] + bn, post_s, post_b);
         }
@@ -496,10 +499,10 @@ __global__ __launch_bounds__(kLinThreads) void m2d_linear_kernel(const LinArgs a
 #pragma unroll
       for (int k = 0; k < 2; ++k) {   // the block's 16 x 8 pieces of 8 outputs, two per lane
         const int piece = l + 64 * k, c = piece >> 3, c8 = 8 * (piece & 7);
-        if (c < rows && n0 + c8 < a.N) {
+        if (c < rows && n0 + c8 < a.Ns) {
           const float4 lo = *reinterpret_cast<const float4*>(stage + c * kLinStage + c8);
           const float4 hi = *reinterpret_cast<const float4*>(stage + c * kLinStage + c8 + 4);
-          *reinterpret_cast<uint4*>(Y + (p0 + c) * a.N + n0 + c8) =
+          *reinterpret_cast<uint4*>(Y + (p0 + c) * a.N + nbase + n0 + c8) =
               make_uint4(pack_bf16(lo.x, lo.y), pack_bf16(lo.z, lo.w), pack_bf16(hi.x, hi.y), pack_bf16(hi.z, hi.w));
         }
       }
@@ -635,20 +638,29 @@ int m2d_linear_fwd(int64_t P, int K, int N, int weight_dtype, const void* x, con
   if (P < 1 || K < 1 || N < 1) return M2D_ERR_BAD_SHAPE;
   if (weight_dtype != M2D_F32 && weight_dtype != M2D_BF16) return M2D_ERR_UNSUPPORTED;
   if (pre_act < kActNone || pre_act > kActStarRelu || post_act < kActNone || post_act > kActStarRelu) return M2D_ERR_UNSUPPORTED;
-  if (K % 32 != 0 || K > 32 * kLinMaxKC || N % 16 != 0 || linear_lds_bytes(K, N) > kLinMaxLds) return M2D_ERR_UNSUPPORTED;
+  if (K % 32 != 0 || K > 32 * kLinMaxKC || N % 16 != 0) return M2D_ERR_UNSUPPORTED;
+  // Slices of the outputs, so that a workgroup's share of the weights leaves room for four workgroups on a
+  // compute unit (each slice reads the rows of x again; they are the smaller side where N is large).
+  int nsplit = 1;
+  while (linear_lds_bytes(K, N / nsplit) > 40 * 1024 && (N / nsplit) % 32 == 0 && N / nsplit > 64) nsplit *= 2;
+  const int Ns = N / nsplit;
+  if (linear_lds_bytes(K, Ns) > kLinMaxLds) return M2D_ERR_UNSUPPORTED;
   if ((P + 63) / 64 >= ((int64_t)1 << 31)) return M2D_ERR_UNSUPPORTED;
   if (misaligned(x, 16) || misaligned(y, 16) || misaligned(weight, 16) || (bias && misaligned(bias, 4))) return M2D_ERR_MISALIGNED;
   LinArgs a = {};
   a.x = x; a.w = weight; a.bias = bias; a.y = y; a.P = P; a.K = K; a.N = N; a.wbf16 = weight_dtype == M2D_BF16;
   a.pre = pre_act; a.post = post_act; a.pre_s = pre_scale; a.pre_b = pre_bias; a.post_s = post_scale; a.post_b = post_bias;
   a.ntiles = (int)((P + 63) / 64);
-  const size_t lds = linear_lds_bytes(K, N);
+  a.nsplit = nsplit; a.Ns = Ns;
+  const size_t lds = linear_lds_bytes(K, Ns);
   if (lds > 64 * 1024 && !allow_big_lds()) return M2D_ERR_HIP;
   // persistent: the weights are loaded into LDS once per workgroup; as many workgroups as fit the device at once
   int per_cu = (int)(160 * 1024 / lds);
   if (per_cu > 8) per_cu = 8;
-  int grid = 256 * per_cu;
+  int grid = 256 * per_cu / nsplit;     // workgroups per slice
   if (grid > a.ntiles) grid = a.ntiles;
+  if (grid < 1) grid = 1;
+  grid *= nsplit;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const dim3 g((unsigned)grid), t(kLinThreads);
   if (K <= 64) hipLaunchKernelGGL(m2d_linear_kernel<2>, g, t, lds, st, a);

@@ -169,6 +169,8 @@ def test_small_linear_limits_are_reported(cabi):
     x = torch.zeros(8, 48, device="cuda", dtype=torch.bfloat16)
     with pytest.raises(cabi.M2DError):
         cabi.linear_fwd(x, torch.zeros(16, 48, device="cuda"))            # K is no multiple of 32
-    x = torch.zeros(8, 512, device="cuda", dtype=torch.bfloat16)
+    x = torch.zeros(8, 544, device="cuda", dtype=torch.bfloat16)
     with pytest.raises(cabi.M2DError):
-        cabi.linear_fwd(x, torch.zeros(256, 512, device="cuda"))          # the weights do not fit into LDS
+        cabi.linear_fwd(x, torch.zeros(16, 544, device="cuda"))           # more than 512 inputs
+    with pytest.raises(cabi.M2DError):
+        cabi.linear_fwd(torch.zeros(8, 64, device="cuda", dtype=torch.bfloat16), torch.zeros(24, 64, device="cuda"))   # N is no multiple of 16
