@@ -181,7 +181,7 @@ int m2d_proj_bwd(const m2d_desc* desc, int dt_rank,
  * channels (models/mamba2d.py:57,220,248,363; models/utils.py:13,232-233) and run a depthwise 3x3
  * convolution in the local path (models/utils.py:101-114).  Both are bandwidth-bound; these kernels
  * read the input once and write the output once.  dtype is the element type of x and y, weight_dtype
- * that of the weights (m2d_dtype each); arithmetic is fp32.  x and y must be 16-byte aligned.
+ * that of the weights (m2d_dtype each); arithmetic is fp32.  Every array must be 16-byte aligned.
  *
  * y[r,:] = (x[r,:] - mean) / sqrt(var + eps) * weight + bias over the C values of each of `rows` rows
  * (biased variance, as nn.LayerNorm).  C must be a multiple of 8 (bf16) / 4 (fp32), at most 4096 / 2048. */

@@ -54,6 +54,24 @@ template <> struct Chunk<bf16_t> {
 __device__ __forceinline__ float ldw(const void* w, int wbf16, int i) {
   return wbf16 ? __uint_as_float((uint32_t)static_cast<const uint16_t*>(w)[i] << 16) : static_cast<const float*>(w)[i];
 }
+// V weights from index i0 on (a multiple of V, the array 16-byte aligned), in the fewest loads
+template <int V>
+__device__ __forceinline__ void ldwv(const void* w, int wbf16, int i0, float (&o)[V]) {
+  if (wbf16) {
+    if constexpr (V == 8) {
+      Chunk<bf16_t>::load(static_cast<const bf16_t*>(w) + i0, o);
+    } else {
+      const uint2 q = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(w) + i0);
+      o[0] = bf_lo(q.x); o[1] = bf_hi(q.x); o[2] = bf_lo(q.y); o[3] = bf_hi(q.y);
+    }
+  } else {
+#pragma unroll
+    for (int h = 0; h < V / 4; ++h) {
+      const float4 q = *reinterpret_cast<const float4*>(static_cast<const float*>(w) + i0 + 4 * h);
+      o[4 * h] = q.x; o[4 * h + 1] = q.y; o[4 * h + 2] = q.z; o[4 * h + 3] = q.w;
+    }
+  }
+}
 
 // ------------------------------------------------------------------------------------ LayerNorm
 // G lanes share a row (G a power of two, 4..64), lane g holds the chunks g, g + G, ... of it: at
@@ -86,9 +104,10 @@ __global__ __launch_bounds__(kLnThreads) void m2d_layernorm_kernel(const LnArgs 
   for (int k = 0; k < NC; ++k) {
     const int c = lane_in_row + k * G;
 #pragma unroll
-    for (int j = 0; j < V; ++j) {
-      wv[k][j] = c < nchunks ? ldw(a.w, a.wbf16, c * V + j) : 0.f;
-      bv[k][j] = c < nchunks ? ldw(a.b, a.wbf16, c * V + j) : 0.f;
+    for (int j = 0; j < V; ++j) { wv[k][j] = 0.f; bv[k][j] = 0.f; }
+    if (c < nchunks) {
+      ldwv<V>(a.w, a.wbf16, c * V, wv[k]);
+      ldwv<V>(a.b, a.wbf16, c * V, bv[k]);
     }
   }
   const T* X = static_cast<const T*>(a.x);
@@ -140,7 +159,7 @@ template <typename T, int G, int NC>
 int launch_ln(const LnArgs& a, hipStream_t st) {
   constexpr int kRows = kLnThreads / G;
   int64_t blocks = (a.rows + kRows - 1) / kRows;
-  if (blocks > 256 * 32) blocks = 256 * 32;   // grid-stride beyond that: the lane's weights are loaded once per block
+  if (blocks > 256 * 8) blocks = 256 * 8;   // grid-stride beyond that: the lane's weights are loaded once and serve several rows
   hipLaunchKernelGGL((m2d_layernorm_kernel<T, G, NC>), dim3((unsigned)blocks), dim3(kLnThreads), 0, st, a);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
@@ -279,8 +298,10 @@ __global__ __launch_bounds__(kEwThreads) void m2d_scale_residual_kernel(const Ew
     float v[V], r[V];
     Chunk<T>::load(X + i * V, v);
     Chunk<T>::load(R + i * V, r);
+    float sc[V];
+    ldwv<V>(a.s, a.wbf16, c * V, sc);
 #pragma unroll
-    for (int j = 0; j < V; ++j) v[j] = __builtin_fmaf(v[j], ldw(a.s, a.wbf16, c * V + j), r[j]);
+    for (int j = 0; j < V; ++j) v[j] = __builtin_fmaf(v[j], sc[j], r[j]);
     Chunk<T>::store(Y + i * V, v);
   }
 }
@@ -345,9 +366,11 @@ __global__ __launch_bounds__(kEwThreads) void m2d_rope_qknorm_kernel(const RopeA
   const float rstd = rsqrtf(q * inv + a.eps);
   const void* w = which ? a.kw : a.qw;
   const void* bi = which ? a.kb : a.qb;
-  float o[V];
+  float o[V], wv[V], bv[V];
+  ldwv<V>(w, a.wbf16, c * V, wv);
+  ldwv<V>(bi, a.wbf16, c * V, bv);
 #pragma unroll
-  for (int j = 0; j < V; ++j) o[j] = __builtin_fmaf((v[j] - mean) * rstd, ldw(w, a.wbf16, c * V + j), ldw(bi, a.wbf16, c * V + j));
+  for (int j = 0; j < V; ++j) o[j] = __builtin_fmaf((v[j] - mean) * rstd, wv[j], bv[j]);
   T* dst = static_cast<T*>(which ? a.k : a.q) + ((b * a.heads + head) * a.L + l) * (int64_t)a.hd + c * V;
   Chunk<T>::store(dst, o);
 }
@@ -544,7 +567,7 @@ int m2d_layernorm_fwd(int64_t rows, int C, int dtype, int weight_dtype, const vo
   if ((dtype != M2D_F32 && dtype != M2D_BF16) || (weight_dtype != M2D_F32 && weight_dtype != M2D_BF16)) return M2D_ERR_UNSUPPORTED;
   const int V = dtype == M2D_BF16 ? 8 : 4;
   if (C % V != 0 || C / V > 64 * kMaxChunks) return M2D_ERR_UNSUPPORTED;   // rows of whole 16-byte chunks, at most 4096 (bf16) / 2048 (fp32) channels
-  if (misaligned(x, 16) || misaligned(y, 16) || misaligned(weight, 4) || misaligned(bias, 4)) return M2D_ERR_MISALIGNED;
+  if (misaligned(x, 16) || misaligned(y, 16) || misaligned(weight, 16) || misaligned(bias, 16)) return M2D_ERR_MISALIGNED;
   LnArgs a;
   a.x = x; a.w = weight; a.b = bias; a.y = y; a.rows = rows; a.C = C; a.wbf16 = weight_dtype == M2D_BF16; a.eps = eps;
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -601,7 +624,7 @@ int m2d_scale_residual_fwd(int64_t rows, int C, int dtype, int weight_dtype, con
   if ((dtype != M2D_F32 && dtype != M2D_BF16) || (weight_dtype != M2D_F32 && weight_dtype != M2D_BF16)) return M2D_ERR_UNSUPPORTED;
   const int V = dtype == M2D_BF16 ? 8 : 4;
   if (C % V != 0) return M2D_ERR_UNSUPPORTED;
-  if (misaligned(x, 16) || misaligned(residual, 16) || misaligned(y, 16)) return M2D_ERR_MISALIGNED;
+  if (misaligned(x, 16) || misaligned(residual, 16) || misaligned(y, 16) || misaligned(scale, 16)) return M2D_ERR_MISALIGNED;
   EwArgs a = {};
   a.x = x; a.r = residual; a.s = scale; a.y = y; a.cpr = C / V; a.chunks = rows * a.cpr; a.wbf16 = weight_dtype == M2D_BF16;
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -620,7 +643,7 @@ int m2d_rope_qknorm_fwd(int B, int L, int heads, int head_dim, int dtype, int we
   const int V = dtype == M2D_BF16 ? 8 : 4;
   const int G = head_dim / V;
   if (head_dim % V != 0 || (G & (G - 1)) != 0 || G > 32) return M2D_ERR_UNSUPPORTED;   // a head is 1, 2, 4 ... 32 chunks
-  if (misaligned(qkv, 16) || misaligned(cos, 16) || misaligned(sin, 16) || misaligned(q, 16) || misaligned(k, 16)) return M2D_ERR_MISALIGNED;
+  for (const void* p : req) if (misaligned(p, 16)) return M2D_ERR_MISALIGNED;
   RopeArgs a = {};
   a.qkv = qkv; a.cos = cos; a.sin = sin; a.qw = q_weight; a.qb = q_bias; a.kw = k_weight; a.kb = k_bias; a.q = q; a.k = k;
   a.L = L; a.heads = heads; a.hd = head_dim; a.wbf16 = weight_dtype == M2D_BF16; a.eps = eps;
