@@ -208,11 +208,17 @@ __global__ __launch_bounds__(kDwThreads) void m2d_dwconv3x3_kernel(const DwArgs 
   rest /= a.strips;
   const int h = (int)(rest % a.H);
   const int b = (int)(rest / a.H);
+  // the 9 taps of the chunk's V channels are 9 V consecutive weights: fetched as 9 groups of V
   float wt[9][V];
+  {
+    float flat[9][V];   // flat[g][i] = weight number g V + i of the chunk = channel (g V + i) / 9, tap (g V + i) % 9
 #pragma unroll
-  for (int t = 0; t < 9; ++t)
+    for (int g = 0; g < 9; ++g) ldwv<V>(a.w, a.wbf16, (c * 9 + g) * V, flat[g]);
 #pragma unroll
-    for (int j = 0; j < V; ++j) wt[t][j] = ldw(a.w, a.wbf16, (c * V + j) * 9 + t);
+    for (int t = 0; t < 9; ++t)
+#pragma unroll
+      for (int j = 0; j < V; ++j) wt[t][j] = flat[(j * 9 + t) / V][(j * 9 + t) % V];
+  }
   const T* X = static_cast<const T*>(a.x) + ((int64_t)b * a.H * a.W) * a.C + c * V;
   T* Y = static_cast<T*>(a.y) + ((int64_t)b * a.H * a.W) * a.C + c * V;
   const int w0 = sidx * STRIP;
@@ -581,7 +587,7 @@ int m2d_dwconv3x3_fwd(int B, int H, int W, int C, int dtype, int weight_dtype, c
   if ((dtype != M2D_F32 && dtype != M2D_BF16) || (weight_dtype != M2D_F32 && weight_dtype != M2D_BF16)) return M2D_ERR_UNSUPPORTED;
   const int V = dtype == M2D_BF16 ? 8 : 4;
   if (C % V != 0) return M2D_ERR_UNSUPPORTED;
-  if (misaligned(x, 16) || misaligned(y, 16) || misaligned(weight, 4)) return M2D_ERR_MISALIGNED;
+  if (misaligned(x, 16) || misaligned(y, 16) || misaligned(weight, 16)) return M2D_ERR_MISALIGNED;
   DwArgs a;
   a.x = x; a.w = weight; a.y = y; a.B = B; a.H = H; a.W = W; a.C = C; a.wbf16 = weight_dtype == M2D_BF16;
   const int strip = W % 14 == 0 ? 14 : 8;
