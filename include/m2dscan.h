@@ -207,12 +207,14 @@ int m2d_scale_residual_fwd(int64_t rows, int C, int dtype, int weight_dtype, con
  * qkv is the output of the qkv projection, (B, L, 3, heads, head_dim); cos and sin are (L, head_dim) tables
  * of qkv's element type in which the two features of a pair (2i, 2i+1) hold the same angle (cos 1, sin 0 on
  * features that do not rotate); rotated[2i] = x[2i] cos - x[2i+1] sin, rotated[2i+1] = x[2i+1] cos + x[2i] sin.
- * q and k receive LayerNorm(rotated) with their own weights, laid out (B, heads, L, head_dim).
+ * q and k receive LayerNorm(rotated) with their own weights, laid out (B, heads, L, head_dim), or, with
+ * token_major != 0, (B, L, heads, head_dim): the layout of the projection itself, which an attention
+ * kernel that takes strides reads as it is and answers in, so that its output needs no transposing copy.
  * head_dim must be 8, 16, ... 256 (bf16) / 4, 8, ... 128 (fp32), a power of two. */
 int m2d_rope_qknorm_fwd(int B, int L, int heads, int head_dim, int dtype, int weight_dtype,
                         const void* qkv, const void* cos, const void* sin,
                         const void* q_weight, const void* q_bias, const void* k_weight, const void* k_bias,
-                        float eps, void* q, void* k, void* stream);
+                        float eps, int token_major, void* q, void* k, void* stream);
 
 /* y = post(pre(x) weight^T + bias) for the narrow linear layers of a block on bf16 activations: in_proj and
  * out_proj of the token mixer (models/mamba2d.py:166-176), the pointwise convolutions of the local path

@@ -263,8 +263,9 @@ class RoPEAttention2D(nn.Module):
         if (qkv.is_cuda and _inference(qkv, qn.weight, qn.bias, kn.weight, kn.bias) and qkv.dtype in (torch.float32, torch.bfloat16)
                 and qn.weight.dtype in (torch.float32, torch.bfloat16) and qn.eps == kn.eps and hd & (hd - 1) == 0
                 and 8 <= hd <= 128 and qkv.numel() > 0):
-            # rotation and the two LayerNorms in one pass, q and k in the attention kernel's layout
-            q, k = rope_qknorm_fwd_op(qkv, cos, sin, qn.weight, qn.bias, kn.weight, kn.bias, qn.eps)
+            # rotation and the two LayerNorms in one pass; q and k keep the projection's token-major layout,
+            # like v, so the attention kernel answers in it and its output needs no transposing copy
+            q, k = rope_qknorm_fwd_op(qkv, cos, sin, qn.weight, qn.bias, kn.weight, kn.bias, qn.eps, True)
             o = F.scaled_dot_product_attention(q, k, qkv[:, :, 2].permute(0, 2, 1, 3), scale=hd ** -0.5)
             return self.proj(o.transpose(1, 2).reshape(B, H, W, self.num_heads * hd))
         q, k, v = qkv.permute(2, 0, 3, 1, 4).unbind(0)     # (B, heads, HW, head_dim)

@@ -73,7 +73,7 @@ def _load():
     lib.m2d_scale_residual_fwd.restype = i32
     lib.m2d_scale_residual_fwd.argtypes = [ctypes.c_int64, i32, i32, i32, vp, vp, vp, vp, vp]
     lib.m2d_rope_qknorm_fwd.restype = i32
-    lib.m2d_rope_qknorm_fwd.argtypes = [i32] * 6 + [vp] * 7 + [ctypes.c_float, vp, vp, vp]
+    lib.m2d_rope_qknorm_fwd.argtypes = [i32] * 6 + [vp] * 7 + [ctypes.c_float, i32, vp, vp, vp]
     lib.m2d_linear_fwd.restype = i32
     lib.m2d_linear_fwd.argtypes = [ctypes.c_int64, i32, i32, i32, vp, vp, vp, i32, vp, vp, i32, vp, vp, vp, vp]
     lib.m2d_profile_enable.restype = i32
@@ -310,9 +310,10 @@ def scale_residual_fwd(x, scale, residual):
     return y
 
 
-def rope_qknorm_fwd(qkv, cos, sin, q_weight, q_bias, k_weight, k_bias, eps=1e-5):
+def rope_qknorm_fwd(qkv, cos, sin, q_weight, q_bias, k_weight, k_bias, eps=1e-5, token_major=False):
     """(q, k), each (B, heads, L, head_dim): rotary embedding and per-head LayerNorm of the q and k parts of
-    a contiguous (B, L, 3, heads, head_dim) projection, through m2d_rope_qknorm_fwd."""
+    a contiguous (B, L, 3, heads, head_dim) projection, through m2d_rope_qknorm_fwd.  ``token_major``: the
+    same tensors as views of (B, L, heads, head_dim) memory."""
     if qkv.dim() != 5 or qkv.shape[2] != 3 or not qkv.is_cuda or not qkv.is_contiguous():
         raise ValueError("m2dscan: qkv must be a contiguous (B, L, 3, heads, head_dim) tensor on the GPU")
     B, L, _, nh, hd = qkv.shape
@@ -322,12 +323,12 @@ def rope_qknorm_fwd(qkv, cos, sin, q_weight, q_bias, k_weight, k_bias, eps=1e-5)
     for k_, t in (("q_weight", q_weight), ("q_bias", q_bias), ("k_weight", k_weight), ("k_bias", k_bias)):
         if tuple(t.shape) != (hd,) or t.dtype != q_weight.dtype or t.device != qkv.device or not t.is_contiguous():
             raise ValueError(f"m2dscan: {k_} must be a contiguous ({hd},) tensor, all four of one dtype, on qkv's device")
-    q = qkv.new_empty((B, nh, L, hd))
-    k = qkv.new_empty((B, nh, L, hd))
+    shape = (B, L, nh, hd) if token_major else (B, nh, L, hd)
+    q, k = qkv.new_empty(shape), qkv.new_empty(shape)
     check(lib.m2d_rope_qknorm_fwd(B, L, nh, hd, _dtype_code(qkv), _dtype_code(q_weight), _ptr(qkv), _ptr(cos), _ptr(sin),
-                                  _ptr(q_weight), _ptr(q_bias), _ptr(k_weight), _ptr(k_bias), float(eps), _ptr(q), _ptr(k),
-                                  _stream(qkv.device)))
-    return q, k
+                                  _ptr(q_weight), _ptr(q_bias), _ptr(k_weight), _ptr(k_bias), float(eps), int(token_major),
+                                  _ptr(q), _ptr(k), _stream(qkv.device)))
+    return (q.permute(0, 2, 1, 3), k.permute(0, 2, 1, 3)) if token_major else (q, k)
 
 
 ACT_NONE, ACT_GELU, ACT_STARRELU = 0, 1, 2

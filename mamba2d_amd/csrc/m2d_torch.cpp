@@ -282,7 +282,7 @@ Tensor scale_residual_fwd(const Tensor& x, const Tensor& scale, const Tensor& re
 }
 
 std::tuple<Tensor, Tensor> rope_qknorm_fwd(const Tensor& qkv, const Tensor& cos, const Tensor& sin, const Tensor& qw,
-                                           const Tensor& qb, const Tensor& kw, const Tensor& kb, double eps) {
+                                           const Tensor& qb, const Tensor& kw, const Tensor& kb, double eps, bool token_major) {
   TORCH_CHECK(qkv.is_cuda() && qkv.dim() == 5 && qkv.size(2) == 3 && qkv.is_contiguous(),
               "m2dscan: qkv must be a contiguous (B, L, 3, heads, head_dim) tensor on the GPU");
   const int64_t B = qkv.size(0), L = qkv.size(1), nh = qkv.size(3), hd = qkv.size(4);
@@ -293,13 +293,15 @@ std::tuple<Tensor, Tensor> rope_qknorm_fwd(const Tensor& qkv, const Tensor& cos,
     TORCH_CHECK(t->sizes() == at::IntArrayRef({hd}) && t->scalar_type() == qw.scalar_type() && t->device() == qkv.device() &&
                 t->is_contiguous(), "m2dscan: the LayerNorm weights must be contiguous (", hd, ",) tensors of one dtype on qkv's device");
   c10::DeviceGuard guard(qkv.device());
-  Tensor q = at::empty({B, nh, L, hd}, qkv.options()), k = at::empty({B, nh, L, hd}, qkv.options());
+  // (B, heads, L, hd) tensors either way; token-major they are views of (B, L, heads, hd) memory
+  Tensor q = token_major ? at::empty({B, L, nh, hd}, qkv.options()).permute({0, 2, 1, 3}) : at::empty({B, nh, L, hd}, qkv.options());
+  Tensor k = token_major ? at::empty({B, L, nh, hd}, qkv.options()).permute({0, 2, 1, 3}) : at::empty({B, nh, L, hd}, qkv.options());
   if (qkv.numel() == 0) return {q, k};
   hipStream_t st = c10::hip::getCurrentHIPStream(qkv.device().index()).stream();
   check(m2d_rope_qknorm_fwd(static_cast<int>(B), static_cast<int>(L), static_cast<int>(nh), static_cast<int>(hd),
                             dtype_code(qkv, "qkv"), dtype_code(qw, "q_weight"), qkv.data_ptr(), cos.data_ptr(), sin.data_ptr(),
-                            qw.data_ptr(), qb.data_ptr(), kw.data_ptr(), kb.data_ptr(), static_cast<float>(eps), q.data_ptr(),
-                            k.data_ptr(), st));
+                            qw.data_ptr(), qb.data_ptr(), kw.data_ptr(), kb.data_ptr(), static_cast<float>(eps), token_major ? 1 : 0,
+                            q.data_ptr(), k.data_ptr(), st));
   return {q, k};
 }
 
@@ -353,7 +355,7 @@ TORCH_LIBRARY(m2dscan, m) {
   m.def("starrelu_fwd(Tensor x, Tensor scale, Tensor bias) -> Tensor");
   m.def("scale_residual_fwd(Tensor x, Tensor scale, Tensor residual) -> Tensor");
   m.def("rope_qknorm_fwd(Tensor qkv, Tensor cos, Tensor sin, Tensor q_weight, Tensor q_bias, Tensor k_weight, Tensor k_bias, "
-        "float eps) -> (Tensor, Tensor)");
+        "float eps, bool token_major=False) -> (Tensor, Tensor)");
   m.def("linear_act_fwd(Tensor x, Tensor weight, Tensor? bias, int pre, Tensor? pre_scale, Tensor? pre_bias, int post, "
         "Tensor? post_scale, Tensor? post_bias) -> Tensor");
   m.def("abi_version() -> int", &abi_version);

@@ -330,6 +330,7 @@ struct RopeArgs {
   void *q, *k;
   int64_t total;                  // B * L * 2 * heads * G chunks
   int L, heads, hd, wbf16;
+  int token_major;                // q and k as (B, L, heads, hd) instead of (B, heads, L, hd)
   float eps;
 };
 
@@ -377,7 +378,8 @@ __global__ __launch_bounds__(kEwThreads) void m2d_rope_qknorm_kernel(const RopeA
   ldwv<V>(bi, a.wbf16, c * V, bv);
 #pragma unroll
   for (int j = 0; j < V; ++j) o[j] = __builtin_fmaf((v[j] - mean) * rstd, wv[j], bv[j]);
-  T* dst = static_cast<T*>(which ? a.k : a.q) + ((b * a.heads + head) * a.L + l) * (int64_t)a.hd + c * V;
+  T* dst = static_cast<T*>(which ? a.k : a.q) +
+           (a.token_major ? ((b * a.L + l) * a.heads + head) : ((b * a.heads + head) * a.L + l)) * (int64_t)a.hd + c * V;
   Chunk<T>::store(dst, o);
 }
 
@@ -641,7 +643,7 @@ int m2d_scale_residual_fwd(int64_t rows, int C, int dtype, int weight_dtype, con
 
 int m2d_rope_qknorm_fwd(int B, int L, int heads, int head_dim, int dtype, int weight_dtype, const void* qkv,
                         const void* cos, const void* sin, const void* q_weight, const void* q_bias, const void* k_weight,
-                        const void* k_bias, float eps, void* q, void* k, void* stream) {
+                        const void* k_bias, float eps, int token_major, void* q, void* k, void* stream) {
   const void* req[] = {qkv, cos, sin, q_weight, q_bias, k_weight, k_bias, q, k};
   for (const void* p : req) if (!p) return M2D_ERR_NULL_POINTER;
   if (B < 1 || L < 1 || heads < 1 || head_dim < 1) return M2D_ERR_BAD_SHAPE;
@@ -652,7 +654,7 @@ int m2d_rope_qknorm_fwd(int B, int L, int heads, int head_dim, int dtype, int we
   for (const void* p : req) if (misaligned(p, 16)) return M2D_ERR_MISALIGNED;
   RopeArgs a = {};
   a.qkv = qkv; a.cos = cos; a.sin = sin; a.qw = q_weight; a.qb = q_bias; a.kw = k_weight; a.kb = k_bias; a.q = q; a.k = k;
-  a.L = L; a.heads = heads; a.hd = head_dim; a.wbf16 = weight_dtype == M2D_BF16; a.eps = eps;
+  a.L = L; a.heads = heads; a.hd = head_dim; a.wbf16 = weight_dtype == M2D_BF16; a.eps = eps; a.token_major = token_major != 0;
   a.total = (int64_t)B * L * 2 * heads * G;
   hipStream_t st = static_cast<hipStream_t>(stream);
   return dtype == M2D_F32 ? run_rope<float>(a, G, st) : run_rope<bf16_t>(a, G, st);

@@ -1678,7 +1678,7 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
 extern "C" {
 
 
-int m2d_version(void) { return 600; }
+int m2d_version(void) { return 700; }
 
 const char* m2d_status_str(int status) {
   switch (status) {

@@ -116,8 +116,10 @@ def _linear_act_fwd_fake(x, weight, bias, pre, pre_scale, pre_bias, post, post_s
 
 
 @torch.library.register_fake("m2dscan::rope_qknorm_fwd")
-def _rope_qknorm_fwd_fake(qkv, cos, sin, q_weight, q_bias, k_weight, k_bias, eps):
+def _rope_qknorm_fwd_fake(qkv, cos, sin, q_weight, q_bias, k_weight, k_bias, eps, token_major=False):
     B, L, _, nh, hd = qkv.shape
+    if token_major:
+        return qkv.new_empty((B, L, nh, hd)).permute(0, 2, 1, 3), qkv.new_empty((B, L, nh, hd)).permute(0, 2, 1, 3)
     return qkv.new_empty((B, nh, L, hd)), qkv.new_empty((B, nh, L, hd))
 
 

@@ -123,6 +123,9 @@ def test_rope_and_qk_norm_match_the_module(cabi, shape, dtype, wdtype):
     assert q.shape == (B, nh, H * W, hd) and q.dtype == dtype and q.is_contiguous()
     assert so.rel_err(q.float().cpu(), want[0]) < TOL[dtype]
     assert so.rel_err(k.float().cpu(), want[1]) < TOL[dtype]
+    qt, kt = cabi.rope_qknorm_fwd(qkv.cuda(), cos.cuda(), sin.cuda(), *wts, att.q_norm.eps, token_major=True)
+    assert qt.shape == q.shape and qt.permute(0, 2, 1, 3).is_contiguous()      # the same values in (B, L, heads, hd) memory
+    assert torch.equal(qt, q) and torch.equal(kt, k)
 
 
 # rows, K, N: the narrow layers of the model at 64 and 128 channels, rows that end inside a tile of 64, one tile
