@@ -198,10 +198,12 @@ int m2d_dwconv3x3_fwd(int B, int H, int W, int C, int dtype, int weight_dtype,
 int m2d_starrelu_fwd(int64_t n, int dtype, int weight_dtype, const void* x, const void* scale, const void* bias,
                      void* y, void* stream);
 
-/* y[r,c] = x[r,c] * scale[c] + residual[r,c]: the residual update of a block with its learned per-channel
- * scale (models/mamba2d.py:258-259, models/utils.py:46-55).  y may be x or residual. */
+/* y[r,c] = x[r,c] * scale[c] + residual[r,c] (+ residual2[r,c]): the residual update of a block with its
+ * learned per-channel scale (models/mamba2d.py:258-259, models/utils.py:46-55).  residual2 may be NULL; it
+ * takes the second term of a token mixer whose answer is a sum (scan path + local path,
+ * models/mamba2d.py:176), which then is never written out on its own.  y may be x or a residual. */
 int m2d_scale_residual_fwd(int64_t rows, int C, int dtype, int weight_dtype, const void* x, const void* scale,
-                           const void* residual, void* y, void* stream);
+                           const void* residual, const void* residual2, void* y, void* stream);
 
 /* Rotary embedding and per-head LayerNorm of q and k in the attention stages (models/utils.py:253-301):
  * qkv is the output of the qkv projection, (B, L, 3, heads, head_dim); cos and sin are (L, head_dim) tables

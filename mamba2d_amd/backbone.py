@@ -204,13 +204,17 @@ class M2DBlock(nn.Module):
             prm._no_weight_decay = True
         self.out_proj = nn.Linear(d_model, d_model)
 
-    def forward(self, x):           # (B, H, W, C)
+    def forward(self, x, split=False):           # (B, H, W, C)
+        """The mixed tokens; with ``split`` and a local path, the two terms of the sum, for a caller that
+        adds them in a pass of its own."""
         local = self.local_path(self.local_norm(x)) if self.local_path is not None else None
         u = linear_act(self.in_proj, x, post=ACT_GELU)
         y = wavefront_scan_cuda(u, self.AT_log, self.AL_log, self.x_proj.weight,
                                 self.dt_projT.weight, self.dt_projT.bias,
                                 self.dt_projL.weight, self.dt_projL.bias, self.D, self.recomp, flip=self.flip)
         y = linear_act(self.out_proj, y, pre=ACT_GELU)
+        if split and local is not None:
+            return y, local
         return y if local is None else y + local
 
 
@@ -305,17 +309,22 @@ class ResBlock(nn.Module):
         self.drop_path = float(drop_path)
 
     @staticmethod
-    def _residual(x, scale, branch):
-        """scale(x) + branch; with a learned scale, at inference on the GPU, in one pass."""
-        if (isinstance(scale, Scale) and x.is_cuda and _inference(x, branch, scale.scale) and x.is_contiguous()
-                and branch.is_contiguous() and branch.dtype == x.dtype and branch.shape == x.shape
+    def _residual(x, scale, branch, branch2=None):
+        """scale(x) + branch (+ branch2); with a learned scale, at inference on the GPU, in one pass."""
+        terms = (branch,) if branch2 is None else (branch, branch2)
+        if (isinstance(scale, Scale) and x.is_cuda and _inference(x, scale.scale, *terms) and x.is_contiguous()
+                and all(t.is_contiguous() and t.dtype == x.dtype and t.shape == x.shape for t in terms)
                 and x.dtype in (torch.float32, torch.bfloat16) and scale.scale.dtype in (torch.float32, torch.bfloat16)
                 and x.shape[-1] % 8 == 0 and x.numel() > 0):
-            return scale_residual_fwd_op(x, scale.scale, branch)
-        return scale(x) + branch
+            return scale_residual_fwd_op(x, scale.scale, branch, branch2)
+        return scale(x) + (branch if branch2 is None else branch + branch2)
 
     def forward(self, x):
-        x = self._residual(x, self.res_scale1, _drop_path(self.token_mixer(self.norm1(x)), self.drop_path, self.training))
+        if isinstance(self.token_mixer, M2DBlock) and not self.training:
+            mixed = self.token_mixer(self.norm1(x), split=True)       # scan path and local path, summed below
+            x = self._residual(x, self.res_scale1, *(mixed if isinstance(mixed, tuple) else (mixed,)))
+        else:
+            x = self._residual(x, self.res_scale1, _drop_path(self.token_mixer(self.norm1(x)), self.drop_path, self.training))
         return self._residual(x, self.res_scale2, _drop_path(self.MLP(self.norm2(x)), self.drop_path, self.training))
 
 

@@ -71,7 +71,7 @@ def _load():
     lib.m2d_starrelu_fwd.restype = i32
     lib.m2d_starrelu_fwd.argtypes = [ctypes.c_int64, i32, i32, vp, vp, vp, vp, vp]
     lib.m2d_scale_residual_fwd.restype = i32
-    lib.m2d_scale_residual_fwd.argtypes = [ctypes.c_int64, i32, i32, i32, vp, vp, vp, vp, vp]
+    lib.m2d_scale_residual_fwd.argtypes = [ctypes.c_int64, i32, i32, i32, vp, vp, vp, vp, vp, vp]
     lib.m2d_rope_qknorm_fwd.restype = i32
     lib.m2d_rope_qknorm_fwd.argtypes = [i32] * 6 + [vp] * 7 + [ctypes.c_float, i32, vp, vp, vp]
     lib.m2d_linear_fwd.restype = i32
@@ -297,16 +297,17 @@ def starrelu_fwd(x, scale, bias):
     return y
 
 
-def scale_residual_fwd(x, scale, residual):
-    """x * scale + residual with a per-channel scale (last axis), through m2d_scale_residual_fwd."""
+def scale_residual_fwd(x, scale, residual, residual2=None):
+    """x * scale + residual (+ residual2) with a per-channel scale (last axis), through m2d_scale_residual_fwd."""
     C = x.shape[-1]
-    if not x.is_cuda or not x.is_contiguous() or not residual.is_contiguous() or residual.shape != x.shape or residual.dtype != x.dtype:
-        raise ValueError("m2dscan: x and residual must be contiguous tensors of one shape and dtype on the GPU")
+    for r in (residual,) if residual2 is None else (residual, residual2):
+        if not x.is_cuda or not x.is_contiguous() or not r.is_contiguous() or r.shape != x.shape or r.dtype != x.dtype or r.device != x.device:
+            raise ValueError("m2dscan: x and the residuals must be contiguous tensors of one shape and dtype on the GPU")
     if tuple(scale.shape) != (C,) or scale.device != x.device or not scale.is_contiguous():
         raise ValueError(f"m2dscan: scale must be a contiguous ({C},) tensor on {x.device}")
     y = torch.empty_like(x)
     check(lib.m2d_scale_residual_fwd(x.numel() // C, C, _dtype_code(x), _dtype_code(scale), _ptr(x), _ptr(scale), _ptr(residual),
-                                     _ptr(y), _stream(x.device)))
+                                     None if residual2 is None else _ptr(residual2), _ptr(y), _stream(x.device)))
     return y
 
 

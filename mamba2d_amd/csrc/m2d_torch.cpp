@@ -265,10 +265,11 @@ Tensor starrelu_fwd(const Tensor& x, const Tensor& scale, const Tensor& bias) {
   return y;
 }
 
-Tensor scale_residual_fwd(const Tensor& x, const Tensor& scale, const Tensor& residual) {
-  TORCH_CHECK(x.is_cuda() && x.dim() >= 1 && x.is_contiguous() && residual.is_contiguous() && residual.sizes() == x.sizes() &&
-              residual.scalar_type() == x.scalar_type() && residual.device() == x.device(),
-              "m2dscan: x and residual must be contiguous tensors of one shape and dtype on the GPU");
+Tensor scale_residual_fwd(const Tensor& x, const Tensor& scale, const Tensor& residual, const c10::optional<Tensor>& residual2) {
+  TORCH_CHECK(x.is_cuda() && x.dim() >= 1 && x.is_contiguous(), "m2dscan: x must be a contiguous tensor on the GPU");
+  for (const Tensor* r : {&residual, residual2.has_value() ? &*residual2 : &residual})
+    TORCH_CHECK(r->is_contiguous() && r->sizes() == x.sizes() && r->scalar_type() == x.scalar_type() && r->device() == x.device(),
+                "m2dscan: x and the residuals must be contiguous tensors of one shape and dtype on the GPU");
   const int64_t C = x.size(-1);
   TORCH_CHECK(scale.sizes() == at::IntArrayRef({C}) && scale.is_contiguous() && scale.device() == x.device(),
               "m2dscan: scale must be a contiguous (", C, ",) tensor on x's device");
@@ -277,7 +278,8 @@ Tensor scale_residual_fwd(const Tensor& x, const Tensor& scale, const Tensor& re
   if (x.numel() == 0) return y;
   hipStream_t st = c10::hip::getCurrentHIPStream(x.device().index()).stream();
   check(m2d_scale_residual_fwd(x.numel() / C, static_cast<int>(C), dtype_code(x, "x"), dtype_code(scale, "scale"), x.data_ptr(),
-                               scale.data_ptr(), residual.data_ptr(), y.data_ptr(), st));
+                               scale.data_ptr(), residual.data_ptr(), residual2.has_value() ? residual2->data_ptr() : nullptr,
+                               y.data_ptr(), st));
   return y;
 }
 
@@ -353,7 +355,7 @@ TORCH_LIBRARY(m2dscan, m) {
   m.def("layernorm_fwd(Tensor x, Tensor weight, Tensor bias, float eps) -> Tensor");
   m.def("dwconv3x3_fwd(Tensor x, Tensor weight) -> Tensor");
   m.def("starrelu_fwd(Tensor x, Tensor scale, Tensor bias) -> Tensor");
-  m.def("scale_residual_fwd(Tensor x, Tensor scale, Tensor residual) -> Tensor");
+  m.def("scale_residual_fwd(Tensor x, Tensor scale, Tensor residual, Tensor? residual2=None) -> Tensor");
   m.def("rope_qknorm_fwd(Tensor qkv, Tensor cos, Tensor sin, Tensor q_weight, Tensor q_bias, Tensor k_weight, Tensor k_bias, "
         "float eps, bool token_major=False) -> (Tensor, Tensor)");
   m.def("linear_act_fwd(Tensor x, Tensor weight, Tensor? bias, int pre, Tensor? pre_scale, Tensor? pre_bias, int post, "

@@ -263,13 +263,15 @@ __global__ __launch_bounds__(kDwThreads) void m2d_dwconv3x3_kernel(const DwArgs 
 
 // ------------------------------------------------------------------------ fused elementwise
 // StarReLU, y = scale * relu(x)^2 + bias with scalar scale and bias (models/utils.py:22-37), and the
-// residual update of a block, y = x * scale[c] + r (models/mamba2d.py:258-259): one pass each where
-// stock operators take three and two.
+// residual update of a block, y = x * scale[c] + r (models/mamba2d.py:258-259), with a second branch
+// r2 where the token mixer's answer is itself a sum (models/mamba2d.py:176): one pass each where stock
+// operators take three and two or three.
 constexpr int kEwThreads = 256;
 
 struct EwArgs {
   const void* x;
   const void* r;      // residual branch (scale-residual only)
+  const void* r2;     // second branch, or null (scale-residual only)
   const void* s;      // one scale (StarReLU) or C of them
   const void* b;      // one bias (StarReLU)
   void* y;
@@ -298,12 +300,19 @@ __global__ __launch_bounds__(kEwThreads) void m2d_scale_residual_kernel(const Ew
   constexpr int V = Chunk<T>::kV;
   const T* X = static_cast<const T*>(a.x);
   const T* R = static_cast<const T*>(a.r);
+  const T* R2 = static_cast<const T*>(a.r2);
   T* Y = static_cast<T*>(a.y);
   for (int64_t i = (int64_t)blockIdx.x * kEwThreads + threadIdx.x; i < a.chunks; i += (int64_t)gridDim.x * kEwThreads) {
     const int c = (int)(i % a.cpr);
     float v[V], r[V];
     Chunk<T>::load(X + i * V, v);
     Chunk<T>::load(R + i * V, r);
+    if (R2) {
+      float r2[V];
+      Chunk<T>::load(R2 + i * V, r2);
+#pragma unroll
+      for (int j = 0; j < V; ++j) r[j] += r2[j];
+    }
     float sc[V];
     ldwv<V>(a.s, a.wbf16, c * V, sc);
 #pragma unroll
@@ -626,15 +635,16 @@ int m2d_starrelu_fwd(int64_t n, int dtype, int weight_dtype, const void* x, cons
 }
 
 int m2d_scale_residual_fwd(int64_t rows, int C, int dtype, int weight_dtype, const void* x, const void* scale,
-                           const void* residual, void* y, void* stream) {
+                           const void* residual, const void* residual2, void* y, void* stream) {
   if (!x || !scale || !residual || !y) return M2D_ERR_NULL_POINTER;
   if (rows < 1 || C < 1) return M2D_ERR_BAD_SHAPE;
   if ((dtype != M2D_F32 && dtype != M2D_BF16) || (weight_dtype != M2D_F32 && weight_dtype != M2D_BF16)) return M2D_ERR_UNSUPPORTED;
   const int V = dtype == M2D_BF16 ? 8 : 4;
   if (C % V != 0) return M2D_ERR_UNSUPPORTED;
-  if (misaligned(x, 16) || misaligned(residual, 16) || misaligned(y, 16) || misaligned(scale, 16)) return M2D_ERR_MISALIGNED;
+  if (misaligned(x, 16) || misaligned(residual, 16) || misaligned(residual2, 16) || misaligned(y, 16) || misaligned(scale, 16))
+    return M2D_ERR_MISALIGNED;
   EwArgs a = {};
-  a.x = x; a.r = residual; a.s = scale; a.y = y; a.cpr = C / V; a.chunks = rows * a.cpr; a.wbf16 = weight_dtype == M2D_BF16;
+  a.x = x; a.r = residual; a.r2 = residual2; a.s = scale; a.y = y; a.cpr = C / V; a.chunks = rows * a.cpr; a.wbf16 = weight_dtype == M2D_BF16;
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (dtype == M2D_F32) hipLaunchKernelGGL(m2d_scale_residual_kernel<float>, dim3(ew_blocks(a.chunks)), dim3(kEwThreads), 0, st, a);
   else hipLaunchKernelGGL(m2d_scale_residual_kernel<bf16_t>, dim3(ew_blocks(a.chunks)), dim3(kEwThreads), 0, st, a);

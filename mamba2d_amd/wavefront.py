@@ -106,7 +106,7 @@ def _starrelu_fwd_fake(x, scale, bias):
 
 
 @torch.library.register_fake("m2dscan::scale_residual_fwd")
-def _scale_residual_fwd_fake(x, scale, residual):
+def _scale_residual_fwd_fake(x, scale, residual, residual2=None):
     return torch.empty_like(x)
 
 

@@ -91,6 +91,10 @@ def test_fused_elementwise_match_torch(cabi, shape, dtype, wdtype):
     got = cabi.scale_residual_fwd(xd, chan.cuda(), rd)
     want = x.double() * chan.double() + r.double()
     assert got.dtype == dtype and so.rel_err(got.float().cpu(), want) < TOL[dtype]
+    r2 = torch.randn(*shape, generator=g).to(dtype)
+    got = cabi.scale_residual_fwd(xd, chan.cuda(), rd, r2.cuda())
+    want = x.double() * chan.double() + r.double() + r2.double()
+    assert got.dtype == dtype and so.rel_err(got.float().cpu(), want) < TOL[dtype]
 
 
 @pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16], ids=["w_f32", "w_bf16"])
