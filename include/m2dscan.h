@@ -218,6 +218,17 @@ int m2d_rope_qknorm_fwd(int B, int L, int heads, int head_dim, int dtype, int we
                         const void* q_weight, const void* q_bias, const void* k_weight, const void* k_bias,
                         float eps, int token_major, void* q, void* k, void* stream);
 
+/* The whole attention of a rotary stage (models/utils.py:253-316) for heads of 32 features and up to 256
+ * tokens, bf16: out[b, l, head, :] = softmax_l'(scale * q[l] . k[l']) v[l'] with q and k rotated and
+ * LayerNormed per head as m2d_rope_qknorm_fwd does, v taken as it is; qkv is (B, L, 3, heads, 32), cos and sin
+ * are (L, 32) bf16, out is (B, L, heads, 32), the input of the output projection.  Scores, softmax and the
+ * sums are fp32; the probabilities enter the second product rounded to bf16.
+ * head_dim other than 32 or L > 256: M2D_ERR_UNSUPPORTED. */
+int m2d_rope_attention_fwd(int B, int L, int heads, int head_dim, int weight_dtype,
+                           const void* qkv, const void* cos, const void* sin,
+                           const void* q_weight, const void* q_bias, const void* k_weight, const void* k_bias,
+                           float eps, float scale, void* out, void* stream);
+
 /* y = post(pre(x) weight^T + bias) for the narrow linear layers of a block on bf16 activations: in_proj and
  * out_proj of the token mixer (models/mamba2d.py:166-176), the pointwise convolutions of the local path
  * (models/utils.py:87-118) and the MLP (models/utils.py:58-81), together with the activation the block

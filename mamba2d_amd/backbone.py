@@ -23,7 +23,7 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .wavefront import (dwconv3x3_fwd_op, layernorm_fwd_op, linear_act_fwd_op, rope_qknorm_fwd_op,
-                        scale_residual_fwd_op, starrelu_fwd_op, wavefront_scan_cuda)
+                        rope_attention_fwd_op, scale_residual_fwd_op, starrelu_fwd_op, wavefront_scan_cuda)
 
 M2D_T = dict(n_blocks=(3, 3, 9, 3), embed_dim=(64, 128, 320, 512),
              token_mixer=("2D_local", "2D_local", "RopeAttention", "RopeAttention"),
@@ -267,6 +267,10 @@ class RoPEAttention2D(nn.Module):
         if (qkv.is_cuda and _inference(qkv, qn.weight, qn.bias, kn.weight, kn.bias) and qkv.dtype in (torch.float32, torch.bfloat16)
                 and qn.weight.dtype in (torch.float32, torch.bfloat16) and qn.eps == kn.eps and hd & (hd - 1) == 0
                 and 8 <= hd <= 128 and qkv.numel() > 0):
+            if hd == 32 and H * W <= 256 and qkv.dtype == torch.bfloat16:
+                # the whole attention in one kernel, a head per workgroup, answering in the projection's layout
+                o = rope_attention_fwd_op(qkv, cos, sin, qn.weight, qn.bias, kn.weight, kn.bias, qn.eps, hd ** -0.5)
+                return self.proj(o.view(B, H, W, self.num_heads * hd))
             # rotation and the two LayerNorms in one pass; q and k keep the projection's token-major layout,
             # like v, so the attention kernel answers in it and its output needs no transposing copy
             q, k = rope_qknorm_fwd_op(qkv, cos, sin, qn.weight, qn.bias, kn.weight, kn.bias, qn.eps, True)

@@ -24,7 +24,7 @@ M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
            "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_bwd", "m2d_proj_workspace_bytes", "m2d_proj_fwd",
            "m2d_proj_bwd", "m2d_layernorm_fwd", "m2d_dwconv3x3_fwd", "m2d_starrelu_fwd",
-           "m2d_scale_residual_fwd", "m2d_rope_qknorm_fwd", "m2d_linear_fwd", "m2d_profile_enable", "m2d_profile_last_ms")
+           "m2d_scale_residual_fwd", "m2d_rope_qknorm_fwd", "m2d_rope_attention_fwd", "m2d_linear_fwd", "m2d_profile_enable", "m2d_profile_last_ms")
 
 
 class Desc(ctypes.Structure):
@@ -72,6 +72,8 @@ def _load():
     lib.m2d_starrelu_fwd.argtypes = [ctypes.c_int64, i32, i32, vp, vp, vp, vp, vp]
     lib.m2d_scale_residual_fwd.restype = i32
     lib.m2d_scale_residual_fwd.argtypes = [ctypes.c_int64, i32, i32, i32, vp, vp, vp, vp, vp, vp]
+    lib.m2d_rope_attention_fwd.restype = i32
+    lib.m2d_rope_attention_fwd.argtypes = [i32] * 5 + [vp] * 7 + [ctypes.c_float, ctypes.c_float, vp, vp]
     lib.m2d_rope_qknorm_fwd.restype = i32
     lib.m2d_rope_qknorm_fwd.argtypes = [i32] * 6 + [vp] * 7 + [ctypes.c_float, i32, vp, vp, vp]
     lib.m2d_linear_fwd.restype = i32
@@ -309,6 +311,27 @@ def scale_residual_fwd(x, scale, residual, residual2=None):
     check(lib.m2d_scale_residual_fwd(x.numel() // C, C, _dtype_code(x), _dtype_code(scale), _ptr(x), _ptr(scale), _ptr(residual),
                                      None if residual2 is None else _ptr(residual2), _ptr(y), _stream(x.device)))
     return y
+
+
+def rope_attention_fwd(qkv, cos, sin, q_weight, q_bias, k_weight, k_bias, eps=1e-5, scale=None):
+    """(B, L, heads, head_dim): the attention of a rotary stage (rotation and per-head LayerNorm of q and k, softmax
+    attention) from a contiguous bf16 (B, L, 3, heads, head_dim) projection, through m2d_rope_attention_fwd."""
+    if qkv.dim() != 5 or qkv.shape[2] != 3 or not qkv.is_cuda or not qkv.is_contiguous():
+        raise ValueError("m2dscan: qkv must be a contiguous (B, L, 3, heads, head_dim) tensor on the GPU")
+    B, L, _, nh, hd = qkv.shape
+    for t in (cos, sin):
+        if tuple(t.shape) != (L, hd) or t.dtype != qkv.dtype or t.device != qkv.device or not t.is_contiguous():
+            raise ValueError(f"m2dscan: cos and sin must be contiguous ({L},{hd}) tensors of qkv's dtype and device")
+    for t in (q_weight, q_bias, k_weight, k_bias):
+        if tuple(t.shape) != (hd,) or t.dtype != q_weight.dtype or t.device != qkv.device or not t.is_contiguous():
+            raise ValueError(f"m2dscan: the LayerNorm weights must be contiguous ({hd},) tensors of one dtype on {qkv.device}")
+    if qkv.dtype != torch.bfloat16:
+        raise ValueError("m2dscan: the attention kernel takes bfloat16")
+    out = qkv.new_empty((B, L, nh, hd))
+    check(lib.m2d_rope_attention_fwd(B, L, nh, hd, _dtype_code(q_weight), _ptr(qkv), _ptr(cos), _ptr(sin), _ptr(q_weight),
+                                     _ptr(q_bias), _ptr(k_weight), _ptr(k_bias), float(eps),
+                                     float(hd ** -0.5 if scale is None else scale), _ptr(out), _stream(qkv.device)))
+    return out
 
 
 def rope_qknorm_fwd(qkv, cos, sin, q_weight, q_bias, k_weight, k_bias, eps=1e-5, token_major=False):

@@ -307,6 +307,28 @@ std::tuple<Tensor, Tensor> rope_qknorm_fwd(const Tensor& qkv, const Tensor& cos,
   return {q, k};
 }
 
+Tensor rope_attention_fwd(const Tensor& qkv, const Tensor& cos, const Tensor& sin, const Tensor& qw, const Tensor& qb,
+                          const Tensor& kw, const Tensor& kb, double eps, double scale) {
+  TORCH_CHECK(qkv.is_cuda() && qkv.dim() == 5 && qkv.size(2) == 3 && qkv.is_contiguous() && qkv.scalar_type() == at::kBFloat16,
+              "m2dscan: qkv must be a contiguous bfloat16 (B, L, 3, heads, head_dim) tensor on the GPU");
+  const int64_t B = qkv.size(0), L = qkv.size(1), nh = qkv.size(3), hd = qkv.size(4);
+  for (const Tensor* t : {&cos, &sin})
+    TORCH_CHECK(t->sizes() == at::IntArrayRef({L, hd}) && t->scalar_type() == qkv.scalar_type() && t->device() == qkv.device() &&
+                t->is_contiguous(), "m2dscan: cos and sin must be contiguous (", L, ",", hd, ") tensors of qkv's dtype and device");
+  for (const Tensor* t : {&qw, &qb, &kw, &kb})
+    TORCH_CHECK(t->sizes() == at::IntArrayRef({hd}) && t->scalar_type() == qw.scalar_type() && t->device() == qkv.device() &&
+                t->is_contiguous(), "m2dscan: the LayerNorm weights must be contiguous (", hd, ",) tensors of one dtype on qkv's device");
+  c10::DeviceGuard guard(qkv.device());
+  Tensor out = at::empty({B, L, nh, hd}, qkv.options());
+  if (qkv.numel() == 0) return out;
+  hipStream_t st = c10::hip::getCurrentHIPStream(qkv.device().index()).stream();
+  check(m2d_rope_attention_fwd(static_cast<int>(B), static_cast<int>(L), static_cast<int>(nh), static_cast<int>(hd),
+                               dtype_code(qw, "q_weight"), qkv.data_ptr(), cos.data_ptr(), sin.data_ptr(), qw.data_ptr(),
+                               qb.data_ptr(), kw.data_ptr(), kb.data_ptr(), static_cast<float>(eps), static_cast<float>(scale),
+                               out.data_ptr(), st));
+  return out;
+}
+
 Tensor linear_act_fwd(const Tensor& x, const Tensor& weight, const c10::optional<Tensor>& bias, int64_t pre,
                       const c10::optional<Tensor>& pre_scale, const c10::optional<Tensor>& pre_bias, int64_t post,
                       const c10::optional<Tensor>& post_scale, const c10::optional<Tensor>& post_bias) {
@@ -358,6 +380,8 @@ TORCH_LIBRARY(m2dscan, m) {
   m.def("scale_residual_fwd(Tensor x, Tensor scale, Tensor residual, Tensor? residual2=None) -> Tensor");
   m.def("rope_qknorm_fwd(Tensor qkv, Tensor cos, Tensor sin, Tensor q_weight, Tensor q_bias, Tensor k_weight, Tensor k_bias, "
         "float eps, bool token_major=False) -> (Tensor, Tensor)");
+  m.def("rope_attention_fwd(Tensor qkv, Tensor cos, Tensor sin, Tensor q_weight, Tensor q_bias, Tensor k_weight, Tensor k_bias, "
+        "float eps, float scale) -> Tensor");
   m.def("linear_act_fwd(Tensor x, Tensor weight, Tensor? bias, int pre, Tensor? pre_scale, Tensor? pre_bias, int post, "
         "Tensor? post_scale, Tensor? post_bias) -> Tensor");
   m.def("abi_version() -> int", &abi_version);
@@ -373,5 +397,6 @@ TORCH_LIBRARY_IMPL(m2dscan, CUDA, m) {   // ROCm devices dispatch under the CUDA
   m.impl("starrelu_fwd", &starrelu_fwd);
   m.impl("scale_residual_fwd", &scale_residual_fwd);
   m.impl("rope_qknorm_fwd", &rope_qknorm_fwd);
+  m.impl("rope_attention_fwd", &rope_attention_fwd);
   m.impl("linear_act_fwd", &linear_act_fwd);
 }

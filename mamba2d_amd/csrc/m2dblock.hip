@@ -3,8 +3,9 @@
 // a short channel axis (64 to 512 channels: models/mamba2d.py:57,220,248,363, models/utils.py:13,
 // 232-233), the depthwise 3x3 convolution of the local path on channel-last tensors
 // (models/utils.py:101-114), StarReLU (models/utils.py:26-44), the scaled residual sum
-// (models/mamba2d.py:258-259) and the rotary embedding + LayerNorm of q and k in the attention stages.  Inference forward only; each reads every input byte once and
-// writes every output byte once.
+// (models/mamba2d.py:258-259), the rotary embedding + LayerNorm of q and k in the attention stages,
+// and that attention as a whole where a head is 32 wide and the grid has up to 256 cells.  Inference
+// forward only; each reads every input byte once and writes every output byte once.
 //
 // Layout: activations are row-major (rows, C) / (B, H, W, C), element type float or bf16; weights
 // are float or bf16, independently of the activations (a bf16 model holds bf16 weights, a fp32
@@ -573,6 +574,167 @@ inline size_t linear_lds_bytes(int K, int N) { return ((size_t)N * (K + 8) / 2 +
 
 inline bool misaligned(const void* p, size_t n) { return (reinterpret_cast<uintptr_t>(p) & (n - 1)) != 0; }
 
+// ------------------------------------------ attention of the rotary stages, one head per workgroup
+// softmax(q k^T / sqrt(hd)) v with q and k rotated by position and LayerNormed per head first
+// (models/utils.py:253-316), for heads of 32 features and up to 256 tokens (the 14x14 and 7x7 grids of
+// the attention stages), straight from the output of the qkv projection, (B, L, 3, heads, 32), to
+// (B, L, heads, 32), the input of the output projection: one pass in place of the rotation, the two
+// LayerNorms, the attention kernel and the copies between them.
+//   staging: thread t rotates and normalises q and k of token t (a row of 32 is one thread's work) and
+//     leaves them in LDS as bf16 rows, and v transposed (feature-major), rows and columns past L zero;
+//   a wave takes 16 queries at a time.  S^T = K Q^T, one v_mfma_f32_16x16x32_bf16 per 16 keys (the
+//     contraction is the 32 features): lane (mn, kb) holds the scores of query mn for keys 16 kt + 4 kb + i.
+//     Row maximum and sum are in-lane plus two lane exchanges (kb).  O^T = V^T P^T contracts 32 keys per
+//     instruction; its operands may list the keys in any order as long as both agree, so the lane's
+//     eight slots take the probabilities it already holds (keys 4 kb + i of two neighbouring tiles) and
+//     V^T supplies the same keys: no exchange of the probabilities between lanes.
+constexpr int kAttThreads = 256;
+constexpr int kAttHd = 32;
+constexpr int kAttRow = kAttHd + 8;     // bf16 per row of q and k in LDS
+constexpr int kAttMaxL = 256;
+
+struct AttnArgs {
+  const void* qkv;                 // (B, L, 3, heads, 32) bf16
+  const void *cos, *sin;           // (L, 32) bf16
+  const void *qw, *qb, *kw, *kb;   // LayerNorm weights of q and k, (32)
+  void* out;                       // (B, L, heads, 32) bf16
+  int L, heads, wbf16;
+  float eps, scale_log2e;          // softmax scale times log2(e)
+};
+
+// one token's q or k: rotation, LayerNorm, 32 bf16 to dst
+__device__ __forceinline__ void rope_norm_row(const uint16_t* src, const uint16_t* cs_row, const uint16_t* sn_row, const void* w,
+                                              const void* bi, int wbf16, float eps, uint16_t* dst) {
+  float v[kAttHd];
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    float x[8], cs[8], sn[8];
+    Chunk<bf16_t>::load(reinterpret_cast<const bf16_t*>(src) + 8 * c, x);
+    Chunk<bf16_t>::load(reinterpret_cast<const bf16_t*>(cs_row) + 8 * c, cs);
+    Chunk<bf16_t>::load(reinterpret_cast<const bf16_t*>(sn_row) + 8 * c, sn);
+#pragma unroll
+    for (int j = 0; j < 8; j += 2) {
+      v[8 * c + j] = __builtin_fmaf(x[j], cs[j], -x[j + 1] * sn[j]);
+      v[8 * c + j + 1] = __builtin_fmaf(x[j + 1], cs[j + 1], x[j] * sn[j + 1]);
+    }
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < kAttHd; ++j) sum += v[j];
+  const float mean = sum * (1.f / kAttHd);
+  float sq = 0.f;
+#pragma unroll
+  for (int j = 0; j < kAttHd; ++j) { const float d = v[j] - mean; sq = __builtin_fmaf(d, d, sq); }
+  const float rstd = rsqrtf(sq * (1.f / kAttHd) + eps);
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    float wv[8], bv[8], o[8];
+    ldwv<8>(w, wbf16, 8 * c, wv);
+    ldwv<8>(bi, wbf16, 8 * c, bv);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = __builtin_fmaf((v[8 * c + j] - mean) * rstd, wv[j], bv[j]);
+    *reinterpret_cast<uint4*>(dst + 8 * c) = make_uint4(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]), pack_bf16(o[4], o[5]), pack_bf16(o[6], o[7]));
+  }
+}
+
+template <int NP>   // keys in steps of 32: L <= 32 NP
+__global__ __launch_bounds__(kAttThreads) void m2d_rope_attention_kernel(const AttnArgs a) {
+  constexpr int LP = 32 * NP;
+  constexpr int VS = LP + 8;            // bf16 per row of V^T
+  __shared__ __attribute__((aligned(16))) uint16_t Qs[LP * kAttRow];
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[LP * kAttRow];
+  __shared__ __attribute__((aligned(16))) uint16_t Vt[kAttHd * VS];
+  const int tid = threadIdx.x, l = tid & 63, mn = l & 15, kb = l >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int head = blockIdx.x % a.heads;
+  const int64_t b = blockIdx.x / a.heads;
+  const int part = a.heads * kAttHd;                     // elements from q to k to v of a token
+  const uint16_t* base = static_cast<const uint16_t*>(a.qkv) + (b * a.L * 3 * a.heads + head) * (int64_t)kAttHd;
+  for (int t = tid; t < LP; t += kAttThreads) {
+    if (t < a.L) {
+      const uint16_t* row = base + (int64_t)t * 3 * part;
+      const uint16_t* cs = static_cast<const uint16_t*>(a.cos) + t * kAttHd;
+      const uint16_t* sn = static_cast<const uint16_t*>(a.sin) + t * kAttHd;
+      rope_norm_row(row, cs, sn, a.qw, a.qb, a.wbf16, a.eps, Qs + t * kAttRow);
+      rope_norm_row(row + part, cs, sn, a.kw, a.kb, a.wbf16, a.eps, Ks + t * kAttRow);
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const uint4 q = ld16(row + 2 * part + 8 * c);
+        const uint32_t w4[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          Vt[(8 * c + 2 * j) * VS + t] = (uint16_t)(w4[j] & 0xffffu);
+          Vt[(8 * c + 2 * j + 1) * VS + t] = (uint16_t)(w4[j] >> 16);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        *reinterpret_cast<uint4*>(Qs + t * kAttRow + 8 * c) = make_uint4(0u, 0u, 0u, 0u);
+        *reinterpret_cast<uint4*>(Ks + t * kAttRow + 8 * c) = make_uint4(0u, 0u, 0u, 0u);
+      }
+#pragma unroll
+      for (int d = 0; d < kAttHd; ++d) Vt[d * VS + t] = 0;
+    }
+  }
+  __syncthreads();
+  const float ninf = -__builtin_huge_valf();
+  const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+  uint16_t* out = static_cast<uint16_t*>(a.out);
+  const int nq = (a.L + 15) / 16;
+  for (int qt = wave; qt < nq; qt += kAttThreads / 64) {
+    const uint4 qf = ld16(Qs + (16 * qt + mn) * kAttRow + 8 * kb);
+    f32x4_t s[2 * NP];
+#pragma unroll
+    for (int kt = 0; kt < 2 * NP; ++kt) s[kt] = mfma_bf16(ld16(Ks + (16 * kt + mn) * kAttRow + 8 * kb), qf, zero);
+    float m = ninf;
+#pragma unroll
+    for (int kt = 0; kt < 2 * NP; ++kt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        if (16 * kt + 4 * kb + i >= a.L) s[kt][i] = ninf;      // keys past the end take no part
+        m = fmaxf(m, s[kt][i]);
+      }
+    m = fmaxf(m, __shfl_xor(m, 16, 64));
+    m = fmaxf(m, __shfl_xor(m, 32, 64));
+    const float mc = m * a.scale_log2e;
+    float sum = 0.f;
+#pragma unroll
+    for (int kt = 0; kt < 2 * NP; ++kt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][i], a.scale_log2e, -mc));
+        s[kt][i] = pr;
+        sum += pr;
+      }
+    sum += __shfl_xor(sum, 16, 64);
+    sum += __shfl_xor(sum, 32, 64);
+    f32x4_t o0 = zero, o1 = zero;
+#pragma unroll
+    for (int ks = 0; ks < NP; ++ks) {
+      const uint4 pf = make_uint4(pack_bf16(s[2 * ks][0], s[2 * ks][1]), pack_bf16(s[2 * ks][2], s[2 * ks][3]),
+                                  pack_bf16(s[2 * ks + 1][0], s[2 * ks + 1][1]), pack_bf16(s[2 * ks + 1][2], s[2 * ks + 1][3]));
+      const uint16_t* v0 = Vt + mn * VS + 32 * ks + 4 * kb;      // features mn and 16 + mn, keys 32 ks + 4 kb + {0..3, 16..19}
+      const uint2 a0 = *reinterpret_cast<const uint2*>(v0), a1 = *reinterpret_cast<const uint2*>(v0 + 16);
+      const uint2 c0 = *reinterpret_cast<const uint2*>(v0 + 16 * VS), c1 = *reinterpret_cast<const uint2*>(v0 + 16 * VS + 16);
+      o0 = mfma_bf16(make_uint4(a0.x, a0.y, a1.x, a1.y), pf, o0);
+      o1 = mfma_bf16(make_uint4(c0.x, c0.y, c1.x, c1.y), pf, o1);
+    }
+    const float inv = 1.f / sum;
+    const int q = 16 * qt + mn;
+    if (q < a.L) {      // lane (mn, kb): features 4 kb + i and 16 + 4 kb + i of query mn
+      uint16_t* dst = out + ((b * a.L + q) * a.heads + head) * (int64_t)kAttHd + 4 * kb;
+      *reinterpret_cast<uint2*>(dst) = make_uint2(pack_bf16(o0[0] * inv, o0[1] * inv), pack_bf16(o0[2] * inv, o0[3] * inv));
+      *reinterpret_cast<uint2*>(dst + 16) = make_uint2(pack_bf16(o1[0] * inv, o1[1] * inv), pack_bf16(o1[2] * inv, o1[3] * inv));
+    }
+  }
+}
+
+template <int NP>
+void launch_attention(const AttnArgs& a, unsigned blocks, hipStream_t st) {
+  hipLaunchKernelGGL(m2d_rope_attention_kernel<NP>, dim3(blocks), dim3(kAttThreads), 0, st, a);
+}
+
 }  // namespace
 
 extern "C" {
@@ -668,6 +830,35 @@ int m2d_rope_qknorm_fwd(int B, int L, int heads, int head_dim, int dtype, int we
   a.total = (int64_t)B * L * 2 * heads * G;
   hipStream_t st = static_cast<hipStream_t>(stream);
   return dtype == M2D_F32 ? run_rope<float>(a, G, st) : run_rope<bf16_t>(a, G, st);
+}
+
+int m2d_rope_attention_fwd(int B, int L, int heads, int head_dim, int weight_dtype, const void* qkv, const void* cos,
+                           const void* sin, const void* q_weight, const void* q_bias, const void* k_weight,
+                           const void* k_bias, float eps, float scale, void* out, void* stream) {
+  if (!qkv || !cos || !sin || !q_weight || !q_bias || !k_weight || !k_bias || !out) return M2D_ERR_NULL_POINTER;
+  if (B < 1 || L < 1 || heads < 1) return M2D_ERR_BAD_SHAPE;
+  if (weight_dtype != M2D_F32 && weight_dtype != M2D_BF16) return M2D_ERR_UNSUPPORTED;
+  if (head_dim != kAttHd || L > kAttMaxL) return M2D_ERR_UNSUPPORTED;
+  if ((int64_t)B * heads >= ((int64_t)1 << 31)) return M2D_ERR_UNSUPPORTED;
+  if (misaligned(qkv, 16) || misaligned(cos, 16) || misaligned(sin, 16) || misaligned(out, 16) || misaligned(q_weight, 16) ||
+      misaligned(q_bias, 16) || misaligned(k_weight, 16) || misaligned(k_bias, 16))
+    return M2D_ERR_MISALIGNED;
+  AttnArgs a = {};
+  a.qkv = qkv; a.cos = cos; a.sin = sin; a.qw = q_weight; a.qb = q_bias; a.kw = k_weight; a.kb = k_bias; a.out = out;
+  a.L = L; a.heads = heads; a.wbf16 = weight_dtype == M2D_BF16; a.eps = eps; a.scale_log2e = scale * 1.44269504088896341f;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  const unsigned blocks = (unsigned)((int64_t)B * heads);
+  switch ((L + 31) / 32) {
+    case 1: launch_attention<1>(a, blocks, st); break;
+    case 2: launch_attention<2>(a, blocks, st); break;
+    case 3: launch_attention<3>(a, blocks, st); break;
+    case 4: launch_attention<4>(a, blocks, st); break;
+    case 5: launch_attention<5>(a, blocks, st); break;
+    case 6: launch_attention<6>(a, blocks, st); break;
+    case 7: launch_attention<7>(a, blocks, st); break;
+    default: launch_attention<8>(a, blocks, st); break;
+  }
+  return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
 int m2d_linear_fwd(int64_t P, int K, int N, int weight_dtype, const void* x, const void* weight, const void* bias,

@@ -42,6 +42,7 @@ dwconv3x3_fwd_op = torch.ops.m2dscan.dwconv3x3_fwd
 starrelu_fwd_op = torch.ops.m2dscan.starrelu_fwd
 scale_residual_fwd_op = torch.ops.m2dscan.scale_residual_fwd
 rope_qknorm_fwd_op = torch.ops.m2dscan.rope_qknorm_fwd
+rope_attention_fwd_op = torch.ops.m2dscan.rope_attention_fwd
 linear_act_fwd_op = torch.ops.m2dscan.linear_act_fwd
 
 # Keep the forward's anti-diagonal checkpoints for the backward (faster backward, more saved
@@ -113,6 +114,12 @@ def _scale_residual_fwd_fake(x, scale, residual, residual2=None):
 @torch.library.register_fake("m2dscan::linear_act_fwd")
 def _linear_act_fwd_fake(x, weight, bias, pre, pre_scale, pre_bias, post, post_scale, post_bias):
     return x.new_empty((*x.shape[:-1], weight.shape[0]))
+
+
+@torch.library.register_fake("m2dscan::rope_attention_fwd")
+def _rope_attention_fwd_fake(qkv, cos, sin, q_weight, q_bias, k_weight, k_bias, eps, scale):
+    B, L, _, nh, hd = qkv.shape
+    return qkv.new_empty((B, L, nh, hd))
 
 
 @torch.library.register_fake("m2dscan::rope_qknorm_fwd")

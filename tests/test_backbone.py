@@ -153,8 +153,9 @@ def test_backbone_runs_and_backpropagates_on_gpu():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("shape", [(2, 96, 64), (1, 224, 224), (3, 128, 160)], ids=lambda s: "x".join(map(str, s)))
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 3e-2)], ids=["f32", "bf16"])
-def test_inference_kernels_match_stock_operators(monkeypatch, dtype, tol):
+def test_inference_kernels_match_stock_operators(monkeypatch, dtype, tol, shape):
     """At inference LayerNorm and the local path's depthwise convolution run in the library's kernels; the
     backbone's output must agree with the one the stock operators give (same weights, same input)."""
     from mamba2d_amd import backbone as bb
@@ -166,8 +167,8 @@ def test_inference_kernels_match_stock_operators(monkeypatch, dtype, tol):
             if isinstance(m, torch.nn.LayerNorm):
                 m.weight.uniform_(0.5, 1.5)
                 m.bias.normal_(0, 0.3)
-    x = torch.randn(2, 3, 96, 64, device=dev, dtype=dtype)
-    say(f"\ncase backbone inference kernels vs stock {dtype}")
+    x = torch.randn(shape[0], 3, shape[1], shape[2], device=dev, dtype=dtype)
+    say(f"\ncase backbone inference kernels vs stock {dtype} {shape}")
     calls = {"n": 0}
     real = bb.layernorm_fwd_op
     monkeypatch.setattr(bb, "layernorm_fwd_op", lambda *a: (calls.__setitem__("n", calls["n"] + 1), real(*a))[1])

@@ -1,5 +1,5 @@
 """GPU parity of the residual-block operators (m2d_layernorm_fwd, m2d_dwconv3x3_fwd, m2d_starrelu_fwd,
-m2d_scale_residual_fwd, m2d_rope_qknorm_fwd, m2d_linear_fwd) through the C ABI, against the stock torch operators the reference uses (nn.LayerNorm, models/mamba2d.py:220;
+m2d_scale_residual_fwd, m2d_rope_qknorm_fwd, m2d_rope_attention_fwd, m2d_linear_fwd) through the C ABI, against the stock torch operators the reference uses (nn.LayerNorm, models/mamba2d.py:220;
 depthwise nn.Conv2d, models/utils.py:101) evaluated in fp64 on the CPU.  Tolerances: fp32 2e-5,
 bf16 tensors 1e-2 (max error over max value; one bf16 rounding of the result is 4e-3)."""
 import pytest
@@ -130,6 +130,54 @@ def test_rope_and_qk_norm_match_the_module(cabi, shape, dtype, wdtype):
     qt, kt = cabi.rope_qknorm_fwd(qkv.cuda(), cos.cuda(), sin.cuda(), *wts, att.q_norm.eps, token_major=True)
     assert qt.shape == q.shape and qt.permute(0, 2, 1, 3).is_contiguous()      # the same values in (B, L, heads, hd) memory
     assert torch.equal(qt, q) and torch.equal(kt, k)
+
+
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16], ids=["w_f32", "w_bf16"])
+@pytest.mark.parametrize("shape", [(2, 14, 14, 10), (3, 7, 7, 16), (1, 1, 1, 1), (2, 16, 16, 2), (1, 37, 1, 3), (2, 10, 10, 5), (1, 3, 11, 4),
+                                   (1, 8, 8, 1), (2, 13, 5, 2)], ids=lambda s: "x".join(map(str, s)))
+def test_rotary_attention_matches_the_module(cabi, shape, wdtype):
+    """The one-kernel attention (heads of 32, up to 256 cells) against the module's stock-operator path
+    (mamba2d_amd.backbone.RoPEAttention2D, which restates models/utils.py:253-316) in fp64 on the CPU, from the
+    same bf16 projection output."""
+    from mamba2d_amd.backbone import RoPEAttention2D
+    say(f"\ncase rope_attention {shape} {wdtype}")
+    B, H, W, nh = shape
+    hd, L = 32, H * W
+    g = torch.Generator().manual_seed(sum(shape))
+    att = RoPEAttention2D(nh * hd, head_dim=hd)
+    with torch.no_grad():
+        for m in (att.q_norm, att.k_norm):
+            m.weight.copy_((torch.rand(hd, generator=g) + 0.5).to(wdtype).float())
+            m.bias.copy_((torch.randn(hd, generator=g) * 0.3).to(wdtype).float())
+    qkv = (torch.randn(B, L, 3, nh, hd, generator=g) * 1.5).bfloat16()
+    cos, sin = att._rope_tables(H, W, torch.device("cpu"), torch.bfloat16)
+    q64, k64, v64 = qkv.double().permute(2, 0, 3, 1, 4).unbind(0)
+    c64, s64 = cos.double(), sin.double()
+    qk = []
+    for t, m in ((q64, att.q_norm), (k64, att.k_norm)):
+        r = t * c64 + att._rotate_pairs(t) * s64
+        qk.append(torch.nn.functional.layer_norm(r, (hd,), m.weight.double(), m.bias.double(), m.eps))
+    p = torch.softmax(qk[0] @ qk[1].transpose(-1, -2) * hd ** -0.5, dim=-1)
+    want = (p @ v64).transpose(1, 2)                      # (B, L, heads, hd)
+    wts = [t.detach().to(wdtype).cuda() for t in (att.q_norm.weight, att.q_norm.bias, att.k_norm.weight, att.k_norm.bias)]
+    got = cabi.rope_attention_fwd(qkv.cuda(), cos.cuda(), sin.cuda(), *wts, att.q_norm.eps)
+    torch.cuda.synchronize()
+    assert got.shape == (B, L, nh, hd) and got.dtype == torch.bfloat16 and got.is_contiguous()
+    err = so.rel_err(got.float().cpu(), want)
+    say(f"  rel err {err:.3e}")
+    assert err < TOL[torch.bfloat16]
+
+
+def test_rotary_attention_limits_are_reported(cabi):
+    """Heads that are not 32 wide and grids of more than 256 cells are refused, not computed wrongly."""
+    dev = torch.device("cuda:0")
+    for L, hd in ((257, 32), (16, 64), (16, 16)):
+        qkv = torch.zeros(1, L, 3, 2, hd, device=dev, dtype=torch.bfloat16)
+        t = torch.zeros(L, hd, device=dev, dtype=torch.bfloat16)
+        w = torch.ones(hd, device=dev)
+        with pytest.raises(cabi.M2DError) as e:
+            cabi.rope_attention_fwd(qkv, t, t, w, w, w, w)
+        assert e.value.status == 3      # M2D_ERR_UNSUPPORTED
 
 
 # rows, K, N: the narrow layers of the model at 64 and 128 channels, rows that end inside a tile of 64, one tile
