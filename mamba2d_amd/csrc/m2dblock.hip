@@ -23,8 +23,11 @@ struct bf16_t { uint16_t v; };
 
 __device__ __forceinline__ float bf_lo(uint32_t w) { return __uint_as_float(w << 16); }
 __device__ __forceinline__ float bf_hi(uint32_t w) { return __uint_as_float(w & 0xffff0000u); }
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-  return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)lo) | ((uint32_t)__builtin_bit_cast(uint16_t, (__bf16)hi) << 16);
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {   // one v_cvt_pk_bf16_f32 (round to nearest even)
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
 }
 
 // A chunk is 16 bytes of a row: kV elements.
@@ -580,15 +583,14 @@ inline bool misaligned(const void* p, size_t n) { return (reinterpret_cast<uintp
 // the attention stages), straight from the output of the qkv projection, (B, L, 3, heads, 32), to
 // (B, L, heads, 32), the input of the output projection: one pass in place of the rotation, the two
 // LayerNorms, the attention kernel and the copies between them.
-//   staging: thread t rotates and normalises q and k of token t (a row of 32 is one thread's work) and
-//     leaves them in LDS as bf16 rows, and v transposed (feature-major), rows and columns past L zero;
+//   staging: a quad of lanes rotates and normalises q and k of a token (8 features per lane) and leaves
+//     them in LDS as bf16 rows, and v transposed (feature-major), rows and columns past L zero;
 //   a wave takes 16 queries at a time.  S^T = K Q^T, one v_mfma_f32_16x16x32_bf16 per 16 keys (the
 //     contraction is the 32 features): lane (mn, kb) holds the scores of query mn for keys 16 kt + 4 kb + i.
 //     Row maximum and sum are in-lane plus two lane exchanges (kb).  O^T = V^T P^T contracts 32 keys per
 //     instruction; its operands may list the keys in any order as long as both agree, so the lane's
 //     eight slots take the probabilities it already holds (keys 4 kb + i of two neighbouring tiles) and
 //     V^T supplies the same keys: no exchange of the probabilities between lanes.
-constexpr int kAttThreads = 256;
 constexpr int kAttHd = 32;
 constexpr int kAttRow = kAttHd + 8;     // bf16 per row of q and k in LDS
 constexpr int kAttMaxL = 256;
@@ -602,47 +604,47 @@ struct AttnArgs {
   float eps, scale_log2e;          // softmax scale times log2(e)
 };
 
-// one token's q or k: rotation, LayerNorm, 32 bf16 to dst
-__device__ __forceinline__ void rope_norm_row(const uint16_t* src, const uint16_t* cs_row, const uint16_t* sn_row, const void* w,
-                                              const void* bi, int wbf16, float eps, uint16_t* dst) {
-  float v[kAttHd];
-#pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    float x[8], cs[8], sn[8];
-    Chunk<bf16_t>::load(reinterpret_cast<const bf16_t*>(src) + 8 * c, x);
-    Chunk<bf16_t>::load(reinterpret_cast<const bf16_t*>(cs_row) + 8 * c, cs);
-    Chunk<bf16_t>::load(reinterpret_cast<const bf16_t*>(sn_row) + 8 * c, sn);
-#pragma unroll
-    for (int j = 0; j < 8; j += 2) {
-      v[8 * c + j] = __builtin_fmaf(x[j], cs[j], -x[j + 1] * sn[j]);
-      v[8 * c + j + 1] = __builtin_fmaf(x[j + 1], cs[j + 1], x[j] * sn[j + 1]);
-    }
-  }
-  float sum = 0.f;
-#pragma unroll
-  for (int j = 0; j < kAttHd; ++j) sum += v[j];
-  const float mean = sum * (1.f / kAttHd);
-  float sq = 0.f;
-#pragma unroll
-  for (int j = 0; j < kAttHd; ++j) { const float d = v[j] - mean; sq = __builtin_fmaf(d, d, sq); }
-  const float rstd = rsqrtf(sq * (1.f / kAttHd) + eps);
-#pragma unroll
-  for (int c = 0; c < 4; ++c) {
-    float wv[8], bv[8], o[8];
-    ldwv<8>(w, wbf16, 8 * c, wv);
-    ldwv<8>(bi, wbf16, 8 * c, bv);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) o[j] = __builtin_fmaf((v[8 * c + j] - mean) * rstd, wv[j], bv[j]);
-    *reinterpret_cast<uint4*>(dst + 8 * c) = make_uint4(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]), pack_bf16(o[4], o[5]), pack_bf16(o[6], o[7]));
-  }
+// sum over the four lanes of a quad (lanes 4 g .. 4 g + 3), left in all of them
+__device__ __forceinline__ float quad_sum(float v) {
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1, 0xf, 0xf, true));   // quad_perm [1,0,3,2]
+  v += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E, 0xf, 0xf, true));   // quad_perm [2,3,0,1]
+  return v;
 }
 
-template <int NP>   // keys in steps of 32: L <= 32 NP
-__global__ __launch_bounds__(kAttThreads) void m2d_rope_attention_kernel(const AttnArgs a) {
-  constexpr int LP = 32 * NP;
-  constexpr int VS = LP + 8;            // bf16 per row of V^T
-  __shared__ __attribute__((aligned(16))) uint16_t Qs[LP * kAttRow];
-  __shared__ __attribute__((aligned(16))) uint16_t Ks[LP * kAttRow];
+// A quarter (8 features, one lane of a quad) of one token's q or k: rotation, LayerNorm over the quad, bf16 to dst.
+__device__ __forceinline__ void rope_norm_quarter(const uint16_t* src, const float (&cs)[8], const float (&sn)[8], const float (&wv)[8],
+                                                  const float (&bv)[8], float eps, uint16_t* dst) {
+  float x[8], v[8];
+  Chunk<bf16_t>::load(reinterpret_cast<const bf16_t*>(src), x);
+#pragma unroll
+  for (int j = 0; j < 8; j += 2) {
+    v[j] = __builtin_fmaf(x[j], cs[j], -x[j + 1] * sn[j]);
+    v[j + 1] = __builtin_fmaf(x[j + 1], cs[j + 1], x[j] * sn[j + 1]);
+  }
+  const float mean = quad_sum(((v[0] + v[1]) + (v[2] + v[3])) + ((v[4] + v[5]) + (v[6] + v[7]))) * (1.f / kAttHd);
+  float d[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) d[j] = v[j] - mean;
+  const float sq = quad_sum(((d[0] * d[0] + d[1] * d[1]) + (d[2] * d[2] + d[3] * d[3])) + ((d[4] * d[4] + d[5] * d[5]) + (d[6] * d[6] + d[7] * d[7])));
+  const float rstd = rsqrtf(sq * (1.f / kAttHd) + eps);
+  float o[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) o[j] = __builtin_fmaf(d[j] * rstd, wv[j], bv[j]);
+  *reinterpret_cast<uint4*>(dst) = make_uint4(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]), pack_bf16(o[4], o[5]), pack_bf16(o[6], o[7]));
+}
+
+constexpr int att_waves(int nt) { return nt <= 4 ? nt : (nt + 1) / 2; }   // one or two tiles of 16 queries per wave
+
+template <int NT>   // tiles of 16 tokens: 16 (NT - 1) < L <= 16 NT
+__global__ __launch_bounds__(64 * att_waves(NT)) __attribute__((amdgpu_waves_per_eu(4, 8)))
+void m2d_rope_attention_kernel(const AttnArgs a) {
+  constexpr int NP = (NT + 1) / 2;      // steps of 32 keys in the second product
+  constexpr int LQ = 16 * NT;           // rows of q and k
+  constexpr int LP = 32 * NP;           // columns of V^T
+  constexpr int VS = LP + 4;            // bf16 per row of V^T: rows stay 8-byte aligned and spread over the banks
+  constexpr int kThreads = 64 * att_waves(NT);
+  __shared__ __attribute__((aligned(16))) uint16_t Qs[LQ * kAttRow];
+  __shared__ __attribute__((aligned(16))) uint16_t Ks[LQ * kAttRow];
   __shared__ __attribute__((aligned(16))) uint16_t Vt[kAttHd * VS];
   const int tid = threadIdx.x, l = tid & 63, mn = l & 15, kb = l >> 4;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -650,71 +652,94 @@ __global__ __launch_bounds__(kAttThreads) void m2d_rope_attention_kernel(const A
   const int64_t b = blockIdx.x / a.heads;
   const int part = a.heads * kAttHd;                     // elements from q to k to v of a token
   const uint16_t* base = static_cast<const uint16_t*>(a.qkv) + (b * a.L * 3 * a.heads + head) * (int64_t)kAttHd;
-  for (int t = tid; t < LP; t += kAttThreads) {
-    if (t < a.L) {
-      const uint16_t* row = base + (int64_t)t * 3 * part;
-      const uint16_t* cs = static_cast<const uint16_t*>(a.cos) + t * kAttHd;
-      const uint16_t* sn = static_cast<const uint16_t*>(a.sin) + t * kAttHd;
-      rope_norm_row(row, cs, sn, a.qw, a.qb, a.wbf16, a.eps, Qs + t * kAttRow);
-      rope_norm_row(row + part, cs, sn, a.kw, a.kb, a.wbf16, a.eps, Ks + t * kAttRow);
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        const uint4 q = ld16(row + 2 * part + 8 * c);
-        const uint32_t w4[4] = {q.x, q.y, q.z, q.w};
+  {   // staging: a quad of lanes per token, 8 features each, so that a token's 64 bytes are one piece of a load
+    const int c8 = 8 * (tid & 3);
+    float wq[8], bq[8], wk[8], bk[8];
+    ldwv<8>(a.qw, a.wbf16, c8, wq);
+    ldwv<8>(a.qb, a.wbf16, c8, bq);
+    ldwv<8>(a.kw, a.wbf16, c8, wk);
+    ldwv<8>(a.kb, a.wbf16, c8, bk);
+    for (int t = tid >> 2; t < LP; t += kThreads / 4) {
+      uint16_t* qd = Qs + t * kAttRow + c8;
+      uint16_t* kd = Ks + t * kAttRow + c8;
+      if (t < a.L) {     // (whole quads take the same side)
+        const uint16_t* row = base + (int64_t)t * 3 * part + c8;
+        float cs[8], sn[8];
+        Chunk<bf16_t>::load(static_cast<const bf16_t*>(a.cos) + t * kAttHd + c8, cs);
+        Chunk<bf16_t>::load(static_cast<const bf16_t*>(a.sin) + t * kAttHd + c8, sn);
+        const uint4 vq = ld16(row + 2 * part);
+        rope_norm_quarter(row, cs, sn, wq, bq, a.eps, qd);
+        rope_norm_quarter(row + part, cs, sn, wk, bk, a.eps, kd);
+        const uint32_t w4[4] = {vq.x, vq.y, vq.z, vq.w};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          Vt[(8 * c + 2 * j) * VS + t] = (uint16_t)(w4[j] & 0xffffu);
-          Vt[(8 * c + 2 * j + 1) * VS + t] = (uint16_t)(w4[j] >> 16);
+          Vt[(c8 + 2 * j) * VS + t] = (uint16_t)(w4[j] & 0xffffu);
+          Vt[(c8 + 2 * j + 1) * VS + t] = (uint16_t)(w4[j] >> 16);
         }
-      }
-    } else {
+      } else {
+        if (t < LQ) {
+          *reinterpret_cast<uint4*>(qd) = make_uint4(0u, 0u, 0u, 0u);
+          *reinterpret_cast<uint4*>(kd) = make_uint4(0u, 0u, 0u, 0u);
+        }
 #pragma unroll
-      for (int c = 0; c < 4; ++c) {
-        *reinterpret_cast<uint4*>(Qs + t * kAttRow + 8 * c) = make_uint4(0u, 0u, 0u, 0u);
-        *reinterpret_cast<uint4*>(Ks + t * kAttRow + 8 * c) = make_uint4(0u, 0u, 0u, 0u);
+        for (int j = 0; j < 8; ++j) Vt[(c8 + j) * VS + t] = 0;
       }
-#pragma unroll
-      for (int d = 0; d < kAttHd; ++d) Vt[d * VS + t] = 0;
     }
   }
   __syncthreads();
   const float ninf = -__builtin_huge_valf();
   const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
   uint16_t* out = static_cast<uint16_t*>(a.out);
-  const int nq = (a.L + 15) / 16;
-  for (int qt = wave; qt < nq; qt += kAttThreads / 64) {
+  for (int qt = wave; qt < NT; qt += att_waves(NT)) {
+    // The operands from k and v are the same for both tiles of a wave; read again, they cost LDS cycles that are
+    // free here, kept in registers they would cost a quarter of the waves.  An offset the compiler cannot see
+    // through keeps the loads inside the loop.
+    int again = 0;
+    asm volatile("" : "+v"(again));
+    const uint16_t* Kl = Ks + again;
+    const uint16_t* Vl = Vt + again;
     const uint4 qf = ld16(Qs + (16 * qt + mn) * kAttRow + 8 * kb);
-    f32x4_t s[2 * NP];
+    f32x4_t s[NT];
 #pragma unroll
-    for (int kt = 0; kt < 2 * NP; ++kt) s[kt] = mfma_bf16(ld16(Ks + (16 * kt + mn) * kAttRow + 8 * kb), qf, zero);
-    float m = ninf;
+    for (int kt = 0; kt < NT; ++kt) s[kt] = mfma_bf16(ld16(Kl + (16 * kt + mn) * kAttRow + 8 * kb), qf, zero);
 #pragma unroll
-    for (int kt = 0; kt < 2 * NP; ++kt)
+    for (int i = 0; i < 4; ++i)      // only the last tile can hold keys past the end: they take no part
+      if (16 * (NT - 1) + 4 * kb + i >= a.L) s[NT - 1][i] = ninf;
+    // maximum and sum run as four chains (one per i) and meet at the end
+    float mx[4] = {ninf, ninf, ninf, ninf};
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        if (16 * kt + 4 * kb + i >= a.L) s[kt][i] = ninf;      // keys past the end take no part
-        m = fmaxf(m, s[kt][i]);
-      }
+    for (int kt = 0; kt < NT; ++kt)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) mx[i] = fmaxf(mx[i], s[kt][i]);
+    float m = fmaxf(fmaxf(mx[0], mx[1]), fmaxf(mx[2], mx[3]));
     m = fmaxf(m, __shfl_xor(m, 16, 64));
     m = fmaxf(m, __shfl_xor(m, 32, 64));
     const float mc = m * a.scale_log2e;
-    float sum = 0.f;
+    float sm[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int kt = 0; kt < 2 * NP; ++kt)
+    for (int kt = 0; kt < NT; ++kt)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const float pr = __builtin_amdgcn_exp2f(__builtin_fmaf(s[kt][i], a.scale_log2e, -mc));
         s[kt][i] = pr;
-        sum += pr;
+        sm[i] += pr;
       }
+    float sum = (sm[0] + sm[1]) + (sm[2] + sm[3]);
     sum += __shfl_xor(sum, 16, 64);
     sum += __shfl_xor(sum, 32, 64);
     f32x4_t o0 = zero, o1 = zero;
 #pragma unroll
     for (int ks = 0; ks < NP; ++ks) {
-      const uint4 pf = make_uint4(pack_bf16(s[2 * ks][0], s[2 * ks][1]), pack_bf16(s[2 * ks][2], s[2 * ks][3]),
-                                  pack_bf16(s[2 * ks + 1][0], s[2 * ks + 1][1]), pack_bf16(s[2 * ks + 1][2], s[2 * ks + 1][3]));
-      const uint16_t* v0 = Vt + mn * VS + 32 * ks + 4 * kb;      // features mn and 16 + mn, keys 32 ks + 4 kb + {0..3, 16..19}
+      uint4 pf;
+      pf.x = pack_bf16(s[2 * ks][0], s[2 * ks][1]);
+      pf.y = pack_bf16(s[2 * ks][2], s[2 * ks][3]);
+      if (2 * ks + 1 < NT) {
+        pf.z = pack_bf16(s[2 * ks + 1][0], s[2 * ks + 1][1]);
+        pf.w = pack_bf16(s[2 * ks + 1][2], s[2 * ks + 1][3]);
+      } else {      // an odd number of tiles: the last step holds 16 keys
+        pf.z = 0u; pf.w = 0u;
+      }
+      const uint16_t* v0 = Vl + mn * VS + 32 * ks + 4 * kb;      // features mn and 16 + mn, keys 32 ks + 4 kb + {0..3, 16..19}
       const uint2 a0 = *reinterpret_cast<const uint2*>(v0), a1 = *reinterpret_cast<const uint2*>(v0 + 16);
       const uint2 c0 = *reinterpret_cast<const uint2*>(v0 + 16 * VS), c1 = *reinterpret_cast<const uint2*>(v0 + 16 * VS + 16);
       o0 = mfma_bf16(make_uint4(a0.x, a0.y, a1.x, a1.y), pf, o0);
@@ -730,9 +755,9 @@ __global__ __launch_bounds__(kAttThreads) void m2d_rope_attention_kernel(const A
   }
 }
 
-template <int NP>
+template <int NT>
 void launch_attention(const AttnArgs& a, unsigned blocks, hipStream_t st) {
-  hipLaunchKernelGGL(m2d_rope_attention_kernel<NP>, dim3(blocks), dim3(kAttThreads), 0, st, a);
+  hipLaunchKernelGGL(m2d_rope_attention_kernel<NT>, dim3(blocks), dim3(64 * att_waves(NT)), 0, st, a);
 }
 
 }  // namespace
@@ -848,7 +873,7 @@ int m2d_rope_attention_fwd(int B, int L, int heads, int head_dim, int weight_dty
   a.L = L; a.heads = heads; a.wbf16 = weight_dtype == M2D_BF16; a.eps = eps; a.scale_log2e = scale * 1.44269504088896341f;
   hipStream_t st = static_cast<hipStream_t>(stream);
   const unsigned blocks = (unsigned)((int64_t)B * heads);
-  switch ((L + 31) / 32) {
+  switch ((L + 15) / 16) {
     case 1: launch_attention<1>(a, blocks, st); break;
     case 2: launch_attention<2>(a, blocks, st); break;
     case 3: launch_attention<3>(a, blocks, st); break;
@@ -856,7 +881,15 @@ int m2d_rope_attention_fwd(int B, int L, int heads, int head_dim, int weight_dty
     case 5: launch_attention<5>(a, blocks, st); break;
     case 6: launch_attention<6>(a, blocks, st); break;
     case 7: launch_attention<7>(a, blocks, st); break;
-    default: launch_attention<8>(a, blocks, st); break;
+    case 8: launch_attention<8>(a, blocks, st); break;
+    case 9: launch_attention<9>(a, blocks, st); break;
+    case 10: launch_attention<10>(a, blocks, st); break;
+    case 11: launch_attention<11>(a, blocks, st); break;
+    case 12: launch_attention<12>(a, blocks, st); break;
+    case 13: launch_attention<13>(a, blocks, st); break;
+    case 14: launch_attention<14>(a, blocks, st); break;
+    case 15: launch_attention<15>(a, blocks, st); break;
+    default: launch_attention<16>(a, blocks, st); break;
   }
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }

@@ -41,6 +41,12 @@ __device__ __forceinline__ float ld(const float* p) { return *p; }
 __device__ __forceinline__ float ld(const bf16_t* p) { return __uint_as_float((uint32_t)p->v << 16); }
 // round to nearest even; the conversion is one instruction on gfx950 (v_cvt_pk_bf16_f32)
 __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16_pair(float lo, float hi) {   // one v_cvt_pk_bf16_f32
+  const f32x2_t v = {lo, hi};
+  return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2_t));
+}
 __device__ __forceinline__ void st(float* p, float v) { *p = v; }
 __device__ __forceinline__ void st(bf16_t* p, float v) { p->v = f32_to_bf16_bits(v); }
 // the value a tensor of type T would hold
@@ -249,7 +255,7 @@ struct Tile {
       else {
         uint32_t w[4];
 #pragma unroll
-        for (int h = 0; h < 4; ++h) w[h] = (uint32_t)f32_to_bf16_bits(v[2 * h]) | ((uint32_t)f32_to_bf16_bits(v[2 * h + 1]) << 16);
+        for (int h = 0; h < 4; ++h) w[h] = pack_bf16_pair(v[2 * h], v[2 * h + 1]);
         *reinterpret_cast<uint4*>(dst) = make_uint4(w[0], w[1], w[2], w[3]);
       }
     }
