@@ -205,6 +205,15 @@ int m2d_starrelu_fwd(int64_t n, int dtype, int weight_dtype, const void* x, cons
 int m2d_scale_residual_fwd(int64_t rows, int C, int dtype, int weight_dtype, const void* x, const void* scale,
                            const void* residual, const void* residual2, void* y, void* stream);
 
+/* The residual update with the LayerNorm that follows it (models/mamba2d.py:258-259: the first update feeds
+ * norm2 of the same block, the second norm1 of the next block or the LayerNorm that ends the stage):
+ * x_out = x * scale[c] + residual (+ residual2, may be NULL), y = LayerNorm(x_out) over C with weight, bias, eps,
+ * where the norm sees x_out as stored (rounded to the element type).  Same limits as m2d_layernorm_fwd;
+ * x_out may be x or a residual. */
+int m2d_scale_residual_layernorm_fwd(int64_t rows, int C, int dtype, int weight_dtype, const void* x, const void* scale,
+                                     const void* residual, const void* residual2, const void* weight, const void* bias,
+                                     float eps, void* x_out, void* y, void* stream);
+
 /* Rotary embedding and per-head LayerNorm of q and k in the attention stages (models/utils.py:253-301):
  * qkv is the output of the qkv projection, (B, L, 3, heads, head_dim); cos and sin are (L, head_dim) tables
  * of qkv's element type in which the two features of a pair (2i, 2i+1) hold the same angle (cos 1, sin 0 on

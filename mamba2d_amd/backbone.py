@@ -23,7 +23,8 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 from .wavefront import (dwconv3x3_fwd_op, layernorm_fwd_op, linear_act_fwd_op, rope_qknorm_fwd_op,
-                        rope_attention_fwd_op, scale_residual_fwd_op, starrelu_fwd_op, wavefront_scan_cuda)
+                        rope_attention_fwd_op, scale_residual_fwd_op, scale_residual_layernorm_fwd_op, starrelu_fwd_op,
+                        wavefront_scan_cuda)
 
 M2D_T = dict(n_blocks=(3, 3, 9, 3), embed_dim=(64, 128, 320, 512),
              token_mixer=("2D_local", "2D_local", "RopeAttention", "RopeAttention"),
@@ -323,13 +324,37 @@ class ResBlock(nn.Module):
             return scale_residual_fwd_op(x, scale.scale, branch, branch2)
         return scale(x) + (branch if branch2 is None else branch + branch2)
 
-    def forward(self, x):
+    @staticmethod
+    def _residual_norm(x, scale, terms, norm):
+        """(y, norm(y)) for y = scale(x) + sum(terms); (y, None) without a norm.  At inference on the GPU the update
+        and the LayerNorm behind it are one pass over the rows."""
+        if (norm is not None and isinstance(scale, Scale) and x.is_cuda and x.is_contiguous() and x.numel() > 0
+                and _inference(x, scale.scale, norm.weight, norm.bias, *terms)
+                and all(t.is_contiguous() and t.dtype == x.dtype and t.shape == x.shape for t in terms)
+                and x.dtype in (torch.float32, torch.bfloat16) and scale.scale.dtype in (torch.float32, torch.bfloat16)
+                and norm.weight is not None and norm.bias is not None and norm.weight.dtype == scale.scale.dtype
+                and norm.bias.dtype == scale.scale.dtype and tuple(norm.normalized_shape) == (x.shape[-1],)
+                and x.shape[-1] % 8 == 0 and x.shape[-1] <= 2048):
+            return scale_residual_layernorm_fwd_op(x, scale.scale, terms[0], terms[1] if len(terms) > 1 else None,
+                                                   norm.weight, norm.bias, norm.eps)
+        y = ResBlock._residual(x, scale, *terms)
+        return y, (norm(y) if norm is not None else None)
+
+    def forward_fused(self, x, normed=None, next_norm=None):
+        """The block on x, with ``normed`` = norm1(x) where the caller has it already; returns the block's output
+        and ``next_norm`` of it (None without ``next_norm``): the LayerNorm that follows the block, computed in
+        the pass of the second residual update."""
+        n1 = self.norm1(x) if normed is None else normed
         if isinstance(self.token_mixer, M2DBlock) and not self.training:
-            mixed = self.token_mixer(self.norm1(x), split=True)       # scan path and local path, summed below
-            x = self._residual(x, self.res_scale1, *(mixed if isinstance(mixed, tuple) else (mixed,)))
+            mixed = self.token_mixer(n1, split=True)       # scan path and local path, summed in the update
+            terms = mixed if isinstance(mixed, tuple) else (mixed,)
         else:
-            x = self._residual(x, self.res_scale1, _drop_path(self.token_mixer(self.norm1(x)), self.drop_path, self.training))
-        return self._residual(x, self.res_scale2, _drop_path(self.MLP(self.norm2(x)), self.drop_path, self.training))
+            terms = (_drop_path(self.token_mixer(n1), self.drop_path, self.training),)
+        x, n2 = self._residual_norm(x, self.res_scale1, terms, self.norm2)
+        return self._residual_norm(x, self.res_scale2, (_drop_path(self.MLP(n2), self.drop_path, self.training),), next_norm)
+
+    def forward(self, x):
+        return self.forward_fused(x)[0]
 
 
 class Mamba2DBackbone(nn.Module):
@@ -363,10 +388,27 @@ class Mamba2DBackbone(nn.Module):
             self.stages[str(i)] = nn.Sequential(*blocks)
             done += n
 
+    @staticmethod
+    def _run_stage(stage, x):
+        """The stage's modules in order; a block is handed the LayerNorm that follows it (the next block's norm1 or
+        the norm that ends the stage) so that it can compute it together with its last residual update."""
+        mods = list(stage)
+        normed = None
+        for i, m in enumerate(mods):
+            if isinstance(m, ResBlock):
+                nxt = mods[i + 1] if i + 1 < len(mods) else None
+                follows = nxt.norm1 if isinstance(nxt, ResBlock) else nxt if isinstance(nxt, nn.LayerNorm) else None
+                x, normed = m.forward_fused(x, normed, follows)
+            elif isinstance(m, nn.LayerNorm) and normed is not None:
+                x, normed = normed, None
+            else:
+                x, normed = m(x), None
+        return x
+
     def forward(self, x):
         x = x.permute(0, 2, 3, 1)                      # channel-last view; the stem makes it real
         for ds, stage in zip(self.ds.values(), self.stages.values()):
-            x = stage(ds(x).contiguous())
+            x = self._run_stage(stage, ds(x).contiguous())
         return x.permute(0, 3, 1, 2)
 
 

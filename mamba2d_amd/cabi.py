@@ -24,7 +24,7 @@ M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
            "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_bwd", "m2d_proj_workspace_bytes", "m2d_proj_fwd",
            "m2d_proj_bwd", "m2d_layernorm_fwd", "m2d_dwconv3x3_fwd", "m2d_starrelu_fwd",
-           "m2d_scale_residual_fwd", "m2d_rope_qknorm_fwd", "m2d_rope_attention_fwd", "m2d_linear_fwd", "m2d_profile_enable", "m2d_profile_last_ms")
+           "m2d_scale_residual_fwd", "m2d_scale_residual_layernorm_fwd", "m2d_rope_qknorm_fwd", "m2d_rope_attention_fwd", "m2d_linear_fwd", "m2d_profile_enable", "m2d_profile_last_ms")
 
 
 class Desc(ctypes.Structure):
@@ -70,6 +70,8 @@ def _load():
     lib.m2d_dwconv3x3_fwd.argtypes = [i32, i32, i32, i32, i32, i32, vp, vp, vp, vp]
     lib.m2d_starrelu_fwd.restype = i32
     lib.m2d_starrelu_fwd.argtypes = [ctypes.c_int64, i32, i32, vp, vp, vp, vp, vp]
+    lib.m2d_scale_residual_layernorm_fwd.restype = i32
+    lib.m2d_scale_residual_layernorm_fwd.argtypes = [ctypes.c_int64, i32, i32, i32] + [vp] * 6 + [ctypes.c_float, vp, vp, vp]
     lib.m2d_scale_residual_fwd.restype = i32
     lib.m2d_scale_residual_fwd.argtypes = [ctypes.c_int64, i32, i32, i32, vp, vp, vp, vp, vp, vp]
     lib.m2d_rope_attention_fwd.restype = i32
@@ -311,6 +313,23 @@ def scale_residual_fwd(x, scale, residual, residual2=None):
     check(lib.m2d_scale_residual_fwd(x.numel() // C, C, _dtype_code(x), _dtype_code(scale), _ptr(x), _ptr(scale), _ptr(residual),
                                      None if residual2 is None else _ptr(residual2), _ptr(y), _stream(x.device)))
     return y
+
+
+def scale_residual_layernorm_fwd(x, scale, residual, residual2, weight, bias, eps=1e-5):
+    """(x * scale + residual (+ residual2), LayerNorm of it over the last axis), through
+    m2d_scale_residual_layernorm_fwd."""
+    C = x.shape[-1]
+    for r in (residual,) if residual2 is None else (residual, residual2):
+        if not x.is_cuda or not x.is_contiguous() or not r.is_contiguous() or r.shape != x.shape or r.dtype != x.dtype or r.device != x.device:
+            raise ValueError("m2dscan: x and the residuals must be contiguous tensors of one shape and dtype on the GPU")
+    for t in (scale, weight, bias):
+        if tuple(t.shape) != (C,) or t.device != x.device or not t.is_contiguous() or t.dtype != scale.dtype:
+            raise ValueError(f"m2dscan: scale, weight and bias must be contiguous ({C},) tensors of one dtype on {x.device}")
+    xo, y = torch.empty_like(x), torch.empty_like(x)
+    check(lib.m2d_scale_residual_layernorm_fwd(x.numel() // C, C, _dtype_code(x), _dtype_code(scale), _ptr(x), _ptr(scale),
+                                               _ptr(residual), None if residual2 is None else _ptr(residual2), _ptr(weight),
+                                               _ptr(bias), float(eps), _ptr(xo), _ptr(y), _stream(x.device)))
+    return xo, y
 
 
 def rope_attention_fwd(qkv, cos, sin, q_weight, q_bias, k_weight, k_bias, eps=1e-5, scale=None):

@@ -283,6 +283,29 @@ Tensor scale_residual_fwd(const Tensor& x, const Tensor& scale, const Tensor& re
   return y;
 }
 
+std::tuple<Tensor, Tensor> scale_residual_layernorm_fwd(const Tensor& x, const Tensor& scale, const Tensor& residual,
+                                                        const c10::optional<Tensor>& residual2, const Tensor& weight,
+                                                        const Tensor& bias, double eps) {
+  TORCH_CHECK(x.is_cuda() && x.dim() >= 1 && x.is_contiguous(), "m2dscan: x must be a contiguous tensor on the GPU");
+  for (const Tensor* r : {&residual, residual2.has_value() ? &*residual2 : &residual})
+    TORCH_CHECK(r->is_contiguous() && r->sizes() == x.sizes() && r->scalar_type() == x.scalar_type() && r->device() == x.device(),
+                "m2dscan: x and the residuals must be contiguous tensors of one shape and dtype on the GPU");
+  const int64_t C = x.size(-1);
+  for (const Tensor* t : {&scale, &weight, &bias})
+    TORCH_CHECK(t->sizes() == at::IntArrayRef({C}) && t->is_contiguous() && t->device() == x.device() &&
+                t->scalar_type() == scale.scalar_type(), "m2dscan: scale, weight and bias must be contiguous (", C,
+                ",) tensors of one dtype on x's device");
+  c10::DeviceGuard guard(x.device());
+  Tensor xo = at::empty_like(x), y = at::empty_like(x);
+  if (x.numel() == 0) return {xo, y};
+  hipStream_t st = c10::hip::getCurrentHIPStream(x.device().index()).stream();
+  check(m2d_scale_residual_layernorm_fwd(x.numel() / C, static_cast<int>(C), dtype_code(x, "x"), dtype_code(scale, "scale"),
+                                         x.data_ptr(), scale.data_ptr(), residual.data_ptr(),
+                                         residual2.has_value() ? residual2->data_ptr() : nullptr, weight.data_ptr(),
+                                         bias.data_ptr(), static_cast<float>(eps), xo.data_ptr(), y.data_ptr(), st));
+  return {xo, y};
+}
+
 std::tuple<Tensor, Tensor> rope_qknorm_fwd(const Tensor& qkv, const Tensor& cos, const Tensor& sin, const Tensor& qw,
                                            const Tensor& qb, const Tensor& kw, const Tensor& kb, double eps, bool token_major) {
   TORCH_CHECK(qkv.is_cuda() && qkv.dim() == 5 && qkv.size(2) == 3 && qkv.is_contiguous(),
@@ -378,6 +401,8 @@ TORCH_LIBRARY(m2dscan, m) {
   m.def("dwconv3x3_fwd(Tensor x, Tensor weight) -> Tensor");
   m.def("starrelu_fwd(Tensor x, Tensor scale, Tensor bias) -> Tensor");
   m.def("scale_residual_fwd(Tensor x, Tensor scale, Tensor residual, Tensor? residual2=None) -> Tensor");
+  m.def("scale_residual_layernorm_fwd(Tensor x, Tensor scale, Tensor residual, Tensor? residual2, Tensor weight, Tensor bias, "
+        "float eps) -> (Tensor, Tensor)");
   m.def("rope_qknorm_fwd(Tensor qkv, Tensor cos, Tensor sin, Tensor q_weight, Tensor q_bias, Tensor k_weight, Tensor k_bias, "
         "float eps, bool token_major=False) -> (Tensor, Tensor)");
   m.def("rope_attention_fwd(Tensor qkv, Tensor cos, Tensor sin, Tensor q_weight, Tensor q_bias, Tensor k_weight, Tensor k_bias, "
@@ -397,6 +422,7 @@ TORCH_LIBRARY_IMPL(m2dscan, CUDA, m) {   // ROCm devices dispatch under the CUDA
   m.impl("starrelu_fwd", &starrelu_fwd);
   m.impl("scale_residual_fwd", &scale_residual_fwd);
   m.impl("rope_qknorm_fwd", &rope_qknorm_fwd);
+  m.impl("scale_residual_layernorm_fwd", &scale_residual_layernorm_fwd);
   m.impl("rope_attention_fwd", &rope_attention_fwd);
   m.impl("linear_act_fwd", &linear_act_fwd);
 }

@@ -41,6 +41,7 @@ template <> struct Chunk<float> {
   static __device__ __forceinline__ void store(float* p, const float (&v)[4]) {
     *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
   }
+  static __device__ __forceinline__ void store_rounded(float* p, float (&v)[4]) { store(p, v); }
 };
 template <> struct Chunk<bf16_t> {
   static constexpr int kV = 8;
@@ -52,6 +53,13 @@ template <> struct Chunk<bf16_t> {
   }
   static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[8]) {
     *reinterpret_cast<uint4*>(p) = make_uint4(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7]));
+  }
+  // stores v and leaves in v what a reader of p will find
+  static __device__ __forceinline__ void store_rounded(bf16_t* p, float (&v)[8]) {
+    const uint32_t w[4] = {pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7])};
+    *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { v[2 * j] = bf_lo(w[j]); v[2 * j + 1] = bf_hi(w[j]); }
   }
 };
 
@@ -92,9 +100,12 @@ struct LnArgs {
   int64_t rows;
   int C, wbf16;
   float eps;
+  // with the residual update in front (RES): the rows normalised are xo = x * s[c] + r (+ r2), also written out
+  const void *s, *r, *r2;
+  void* xo;
 };
 
-template <typename T, int G, int NC>
+template <typename T, int G, int NC, bool RES>
 __global__ __launch_bounds__(kLnThreads) void m2d_layernorm_kernel(const LnArgs a) {
   constexpr int V = Chunk<T>::kV;
   const int lane_in_row = threadIdx.x & (G - 1);
@@ -114,7 +125,20 @@ __global__ __launch_bounds__(kLnThreads) void m2d_layernorm_kernel(const LnArgs 
       ldwv<V>(a.b, a.wbf16, c * V, bv[k]);
     }
   }
+  float sv[RES ? NC : 1][V];
+  if constexpr (RES) {
+#pragma unroll
+    for (int k = 0; k < NC; ++k) {
+      const int c = lane_in_row + k * G;
+#pragma unroll
+      for (int j = 0; j < V; ++j) sv[k][j] = 0.f;
+      if (c < nchunks) ldwv<V>(a.s, a.wbf16, c * V, sv[k]);
+    }
+  }
   const T* X = static_cast<const T*>(a.x);
+  const T* R = static_cast<const T*>(a.r);
+  const T* R2 = static_cast<const T*>(a.r2);
+  T* XO = static_cast<T*>(a.xo);
   T* Y = static_cast<T*>(a.y);
   for (int64_t row = (int64_t)blockIdx.x * kRows + row_in_block; row < a.rows; row += (int64_t)gridDim.x * kRows) {
     float v[NC][V];
@@ -124,6 +148,19 @@ __global__ __launch_bounds__(kLnThreads) void m2d_layernorm_kernel(const LnArgs 
       const int c = lane_in_row + k * G;
       if (c < nchunks) {
         Chunk<T>::load(X + row * a.C + c * V, v[k]);
+        if constexpr (RES) {   // the residual update, as m2d_scale_residual_kernel computes it; the norm sees what was stored
+          float r[V];
+          Chunk<T>::load(R + row * a.C + c * V, r);
+          if (R2) {
+            float r2[V];
+            Chunk<T>::load(R2 + row * a.C + c * V, r2);
+#pragma unroll
+            for (int j = 0; j < V; ++j) r[j] += r2[j];
+          }
+#pragma unroll
+          for (int j = 0; j < V; ++j) v[k][j] = __builtin_fmaf(v[k][j], sv[k][j], r[j]);
+          Chunk<T>::store_rounded(XO + row * a.C + c * V, v[k]);
+        }
       } else {
 #pragma unroll
         for (int j = 0; j < V; ++j) v[k][j] = 0.f;
@@ -159,28 +196,28 @@ __global__ __launch_bounds__(kLnThreads) void m2d_layernorm_kernel(const LnArgs 
   }
 }
 
-template <typename T, int G, int NC>
+template <typename T, int G, int NC, bool RES>
 int launch_ln(const LnArgs& a, hipStream_t st) {
   constexpr int kRows = kLnThreads / G;
   int64_t blocks = (a.rows + kRows - 1) / kRows;
   if (blocks > 256 * 8) blocks = 256 * 8;   // grid-stride beyond that: the lane's weights are loaded once and serve several rows
-  hipLaunchKernelGGL((m2d_layernorm_kernel<T, G, NC>), dim3((unsigned)blocks), dim3(kLnThreads), 0, st, a);
+  hipLaunchKernelGGL((m2d_layernorm_kernel<T, G, NC, RES>), dim3((unsigned)blocks), dim3(kLnThreads), 0, st, a);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
-template <typename T>
+template <typename T, bool RES>
 int run_ln(const LnArgs& a, hipStream_t st) {
   const int nchunks = a.C / Chunk<T>::kV;
   // the fewest lanes per row that keep a lane's share within kMaxChunks, but at least 4 chunks in
   // flight per row where the row is long enough
-  if (nchunks <= 4) return launch_ln<T, 4, 1>(a, st);
-  if (nchunks <= 8) return launch_ln<T, 8, 1>(a, st);
-  if (nchunks <= 16) return launch_ln<T, 16, 1>(a, st);
-  if (nchunks <= 32) return launch_ln<T, 16, 2>(a, st);
-  if (nchunks <= 64) return launch_ln<T, 16, 4>(a, st);
-  if (nchunks <= 128) return launch_ln<T, 32, 4>(a, st);
-  if (nchunks <= 256) return launch_ln<T, 64, 4>(a, st);
-  return launch_ln<T, 64, kMaxChunks>(a, st);
+  if (nchunks <= 4) return launch_ln<T, 4, 1, RES>(a, st);
+  if (nchunks <= 8) return launch_ln<T, 8, 1, RES>(a, st);
+  if (nchunks <= 16) return launch_ln<T, 16, 1, RES>(a, st);
+  if (nchunks <= 32) return launch_ln<T, 16, 2, RES>(a, st);
+  if (nchunks <= 64) return launch_ln<T, 16, 4, RES>(a, st);
+  if (nchunks <= 128) return launch_ln<T, 32, 4, RES>(a, st);
+  if (nchunks <= 256) return launch_ln<T, 64, 4, RES>(a, st);
+  return launch_ln<T, 64, kMaxChunks, RES>(a, st);
 }
 
 // ------------------------------------------------------------------ depthwise 3x3, channel-last
@@ -772,10 +809,28 @@ int m2d_layernorm_fwd(int64_t rows, int C, int dtype, int weight_dtype, const vo
   const int V = dtype == M2D_BF16 ? 8 : 4;
   if (C % V != 0 || C / V > 64 * kMaxChunks) return M2D_ERR_UNSUPPORTED;   // rows of whole 16-byte chunks, at most 4096 (bf16) / 2048 (fp32) channels
   if (misaligned(x, 16) || misaligned(y, 16) || misaligned(weight, 16) || misaligned(bias, 16)) return M2D_ERR_MISALIGNED;
-  LnArgs a;
+  LnArgs a = {};
   a.x = x; a.w = weight; a.b = bias; a.y = y; a.rows = rows; a.C = C; a.wbf16 = weight_dtype == M2D_BF16; a.eps = eps;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  return dtype == M2D_F32 ? run_ln<float>(a, st) : run_ln<bf16_t>(a, st);
+  return dtype == M2D_F32 ? run_ln<float, false>(a, st) : run_ln<bf16_t, false>(a, st);
+}
+
+int m2d_scale_residual_layernorm_fwd(int64_t rows, int C, int dtype, int weight_dtype, const void* x, const void* scale,
+                                     const void* residual, const void* residual2, const void* weight, const void* bias,
+                                     float eps, void* x_out, void* y, void* stream) {
+  if (!x || !scale || !residual || !weight || !bias || !x_out || !y) return M2D_ERR_NULL_POINTER;
+  if (rows < 1 || C < 1) return M2D_ERR_BAD_SHAPE;
+  if ((dtype != M2D_F32 && dtype != M2D_BF16) || (weight_dtype != M2D_F32 && weight_dtype != M2D_BF16)) return M2D_ERR_UNSUPPORTED;
+  const int V = dtype == M2D_BF16 ? 8 : 4;
+  if (C % V != 0 || C / V > 64 * kMaxChunks) return M2D_ERR_UNSUPPORTED;
+  if (misaligned(x, 16) || misaligned(residual, 16) || misaligned(residual2, 16) || misaligned(x_out, 16) || misaligned(y, 16) ||
+      misaligned(scale, 16) || misaligned(weight, 16) || misaligned(bias, 16))
+    return M2D_ERR_MISALIGNED;
+  LnArgs a = {};
+  a.x = x; a.w = weight; a.b = bias; a.y = y; a.rows = rows; a.C = C; a.wbf16 = weight_dtype == M2D_BF16; a.eps = eps;
+  a.s = scale; a.r = residual; a.r2 = residual2; a.xo = x_out;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  return dtype == M2D_F32 ? run_ln<float, true>(a, st) : run_ln<bf16_t, true>(a, st);
 }
 
 int m2d_dwconv3x3_fwd(int B, int H, int W, int C, int dtype, int weight_dtype, const void* x, const void* weight,

@@ -41,6 +41,7 @@ layernorm_fwd_op = torch.ops.m2dscan.layernorm_fwd
 dwconv3x3_fwd_op = torch.ops.m2dscan.dwconv3x3_fwd
 starrelu_fwd_op = torch.ops.m2dscan.starrelu_fwd
 scale_residual_fwd_op = torch.ops.m2dscan.scale_residual_fwd
+scale_residual_layernorm_fwd_op = torch.ops.m2dscan.scale_residual_layernorm_fwd
 rope_qknorm_fwd_op = torch.ops.m2dscan.rope_qknorm_fwd
 rope_attention_fwd_op = torch.ops.m2dscan.rope_attention_fwd
 linear_act_fwd_op = torch.ops.m2dscan.linear_act_fwd
@@ -104,6 +105,11 @@ def _dwconv3x3_fwd_fake(x, weight):
 @torch.library.register_fake("m2dscan::starrelu_fwd")
 def _starrelu_fwd_fake(x, scale, bias):
     return torch.empty_like(x)
+
+
+@torch.library.register_fake("m2dscan::scale_residual_layernorm_fwd")
+def _scale_residual_layernorm_fwd_fake(x, scale, residual, residual2, weight, bias, eps):
+    return torch.empty_like(x), torch.empty_like(x)
 
 
 @torch.library.register_fake("m2dscan::scale_residual_fwd")

@@ -170,11 +170,13 @@ def test_inference_kernels_match_stock_operators(monkeypatch, dtype, tol, shape)
     x = torch.randn(shape[0], 3, shape[1], shape[2], device=dev, dtype=dtype)
     say(f"\ncase backbone inference kernels vs stock {dtype} {shape}")
     calls = {"n": 0}
-    real = bb.layernorm_fwd_op
+    real, real_fused = bb.layernorm_fwd_op, bb.scale_residual_layernorm_fwd_op
     monkeypatch.setattr(bb, "layernorm_fwd_op", lambda *a: (calls.__setitem__("n", calls["n"] + 1), real(*a))[1])
+    monkeypatch.setattr(bb, "scale_residual_layernorm_fwd_op",
+                        lambda *a: (calls.__setitem__("n", calls["n"] + 1), real_fused(*a))[1])
     with torch.no_grad():
         got = net(x)
-    assert calls["n"] > 10   # the library's kernel did run
+    assert calls["n"] > 10   # the library's kernels did run (LayerNorm alone or behind a residual update)
     monkeypatch.setattr(bb, "_inference", lambda *t: False)
     with torch.no_grad():
         want = net(x)

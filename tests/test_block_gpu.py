@@ -1,5 +1,5 @@
 """GPU parity of the residual-block operators (m2d_layernorm_fwd, m2d_dwconv3x3_fwd, m2d_starrelu_fwd,
-m2d_scale_residual_fwd, m2d_rope_qknorm_fwd, m2d_rope_attention_fwd, m2d_linear_fwd) through the C ABI, against the stock torch operators the reference uses (nn.LayerNorm, models/mamba2d.py:220;
+m2d_scale_residual_fwd, m2d_scale_residual_layernorm_fwd, m2d_rope_qknorm_fwd, m2d_rope_attention_fwd, m2d_linear_fwd) through the C ABI, against the stock torch operators the reference uses (nn.LayerNorm, models/mamba2d.py:220;
 depthwise nn.Conv2d, models/utils.py:101) evaluated in fp64 on the CPU.  Tolerances: fp32 2e-5,
 bf16 tensors 1e-2 (max error over max value; one bf16 rounding of the result is 4e-3)."""
 import pytest
@@ -95,6 +95,30 @@ def test_fused_elementwise_match_torch(cabi, shape, dtype, wdtype):
     got = cabi.scale_residual_fwd(xd, chan.cuda(), rd, r2.cuda())
     want = x.double() * chan.double() + r.double() + r2.double()
     assert got.dtype == dtype and so.rel_err(got.float().cpu(), want) < TOL[dtype]
+
+
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16], ids=["w_f32", "w_bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("two", [False, True], ids=["one_term", "two_terms"])
+@pytest.mark.parametrize("shape", [(2, 9, 12, 64), (3, 50, 128), (2, 14, 14, 320), (130, 512), (7, 24), (3, 1000, 2048)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_residual_update_with_layernorm_matches_the_two_kernels(cabi, shape, two, dtype, wdtype):
+    """The fused pass writes the same x_out as m2d_scale_residual_fwd, bit for bit, and the LayerNorm of exactly
+    that tensor as m2d_layernorm_fwd gives it; both are checked against torch elsewhere in this file."""
+    say(f"\ncase scale_residual_layernorm {shape} two={two} {dtype} {wdtype}")
+    g = torch.Generator().manual_seed(sum(shape) + two)
+    C = shape[-1]
+    x, r, r2 = (torch.randn(*shape, generator=g).to(dtype).cuda() for _ in range(3))
+    sc = (torch.rand(C, generator=g) + 0.5).to(wdtype).cuda()
+    w = (torch.rand(C, generator=g) + 0.5).to(wdtype).cuda()
+    b = (torch.randn(C, generator=g) * 0.3).to(wdtype).cuda()
+    xo, y = cabi.scale_residual_layernorm_fwd(x, sc, r, r2 if two else None, w, b, 1e-5)
+    want_x = cabi.scale_residual_fwd(x, sc, r, r2 if two else None)
+    want_y = cabi.layernorm_fwd(want_x, w, b, 1e-5)
+    torch.cuda.synchronize()
+    assert xo.dtype == dtype and y.dtype == dtype
+    assert torch.equal(xo, want_x)
+    assert torch.equal(y, want_y)
 
 
 @pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16], ids=["w_f32", "w_bf16"])
