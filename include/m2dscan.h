@@ -253,6 +253,13 @@ int m2d_linear_fwd(int64_t P, int K, int N, int weight_dtype, const void* x, con
                    int pre_act, const void* pre_scale, const void* pre_bias,
                    int post_act, const void* post_scale, const void* post_bias, void* y, void* stream);
 
+/* y = fc2(GELU(fc1 x)) of the MLP (models/utils.py:58-81) where both weight matrices fit LDS together:
+ * C = 32 or 64 channels and hidden = 4 C.  x and y are (P, C) bf16; w1 (hidden, C), b1 (hidden), w2 (C, hidden),
+ * b2 (C) have weight_dtype; b1 and b2 may be NULL.  The hidden activations stay in registers; they enter the
+ * second product rounded to bf16, as the stock path stores them.  Other sizes: M2D_ERR_UNSUPPORTED. */
+int m2d_mlp_fwd(int64_t P, int C, int hidden, int weight_dtype, const void* x, const void* w1, const void* b1,
+                const void* w2, const void* b2, void* y, void* stream);
+
 /* Measurement aid; no counterpart in the reference.  While enabled, every m2d_scan_fwd /
  * m2d_scan_bwd call records a pair of HIP events on its stream around the main scan kernel of
  * the pass (not around the small set-up and reduction kernels).  m2d_profile_last_ms waits for

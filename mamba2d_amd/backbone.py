@@ -22,7 +22,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .wavefront import (dwconv3x3_fwd_op, layernorm_fwd_op, linear_act_fwd_op, rope_qknorm_fwd_op,
+from .wavefront import (dwconv3x3_fwd_op, layernorm_fwd_op, linear_act_fwd_op, mlp_fwd_op, rope_qknorm_fwd_op,
                         rope_attention_fwd_op, scale_residual_fwd_op, scale_residual_layernorm_fwd_op, starrelu_fwd_op,
                         wavefront_scan_cuda)
 
@@ -120,6 +120,11 @@ class MLP(nn.Module):
         self.fc2 = nn.Linear(dim * expand, dim)
 
     def forward(self, x):
+        w1, w2 = self.fc1.weight, self.fc2.weight
+        if (x.is_cuda and x.dtype == torch.bfloat16 and x.numel() > 0 and x.shape[-1] in (32, 64) and w1.shape[0] == 4 * w1.shape[1]
+                and _inference(x, w1, w2) and w1.dtype in (torch.float32, torch.bfloat16) and w2.dtype == w1.dtype):
+            # both layers in one kernel: the hidden activations, four times x, never reach memory
+            return mlp_fwd_op(x.contiguous(), w1, self.fc1.bias, w2, self.fc2.bias)
         return linear_act(self.fc2, linear_act(self.fc1, x, post=ACT_GELU))
 
 

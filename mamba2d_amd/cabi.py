@@ -24,7 +24,7 @@ M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
            "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_bwd", "m2d_proj_workspace_bytes", "m2d_proj_fwd",
            "m2d_proj_bwd", "m2d_layernorm_fwd", "m2d_dwconv3x3_fwd", "m2d_starrelu_fwd",
-           "m2d_scale_residual_fwd", "m2d_scale_residual_layernorm_fwd", "m2d_rope_qknorm_fwd", "m2d_rope_attention_fwd", "m2d_linear_fwd", "m2d_profile_enable", "m2d_profile_last_ms")
+           "m2d_scale_residual_fwd", "m2d_scale_residual_layernorm_fwd", "m2d_rope_qknorm_fwd", "m2d_rope_attention_fwd", "m2d_mlp_fwd", "m2d_linear_fwd", "m2d_profile_enable", "m2d_profile_last_ms")
 
 
 class Desc(ctypes.Structure):
@@ -74,6 +74,8 @@ def _load():
     lib.m2d_scale_residual_layernorm_fwd.argtypes = [ctypes.c_int64, i32, i32, i32] + [vp] * 6 + [ctypes.c_float, vp, vp, vp]
     lib.m2d_scale_residual_fwd.restype = i32
     lib.m2d_scale_residual_fwd.argtypes = [ctypes.c_int64, i32, i32, i32, vp, vp, vp, vp, vp, vp]
+    lib.m2d_mlp_fwd.restype = i32
+    lib.m2d_mlp_fwd.argtypes = [ctypes.c_int64, i32, i32, i32] + [vp] * 7
     lib.m2d_rope_attention_fwd.restype = i32
     lib.m2d_rope_attention_fwd.argtypes = [i32] * 5 + [vp] * 7 + [ctypes.c_float, ctypes.c_float, vp, vp]
     lib.m2d_rope_qknorm_fwd.restype = i32
@@ -330,6 +332,25 @@ def scale_residual_layernorm_fwd(x, scale, residual, residual2, weight, bias, ep
                                                _ptr(residual), None if residual2 is None else _ptr(residual2), _ptr(weight),
                                                _ptr(bias), float(eps), _ptr(xo), _ptr(y), _stream(x.device)))
     return xo, y
+
+
+def mlp_fwd(x, w1, b1, w2, b2):
+    """fc2(GELU(fc1 x)) on a contiguous bf16 (..., C) tensor, through m2d_mlp_fwd (C = 32 or 64, hidden = 4 C)."""
+    C = x.shape[-1]
+    if not x.is_cuda or not x.is_contiguous() or x.dtype != torch.bfloat16:
+        raise ValueError("m2dscan: x must be a contiguous bfloat16 tensor on the GPU")
+    H = w1.shape[0]
+    if w1.dim() != 2 or w1.shape[1] != C or tuple(w2.shape) != (C, H) or w2.dtype != w1.dtype:
+        raise ValueError(f"m2dscan: w1 must be (hidden,{C}) and w2 ({C},hidden), of one dtype")
+    for t, n in ((w1, None), (w2, None), (b1, H), (b2, C)):
+        if t is None:
+            continue
+        if t.device != x.device or not t.is_contiguous() or t.dtype != w1.dtype or (n is not None and t.numel() != n):
+            raise ValueError(f"m2dscan: weights and biases must be contiguous tensors of one dtype on {x.device}")
+    y = torch.empty_like(x)
+    check(lib.m2d_mlp_fwd(x.numel() // C, C, H, _dtype_code(w1), _ptr(x), _ptr(w1), None if b1 is None else _ptr(b1), _ptr(w2),
+                          None if b2 is None else _ptr(b2), _ptr(y), _stream(x.device)))
+    return y
 
 
 def rope_attention_fwd(qkv, cos, sin, q_weight, q_bias, k_weight, k_bias, eps=1e-5, scale=None):

@@ -330,6 +330,33 @@ std::tuple<Tensor, Tensor> rope_qknorm_fwd(const Tensor& qkv, const Tensor& cos,
   return {q, k};
 }
 
+Tensor mlp_fwd(const Tensor& x, const Tensor& w1, const c10::optional<Tensor>& b1, const Tensor& w2,
+               const c10::optional<Tensor>& b2) {
+  TORCH_CHECK(x.is_cuda() && x.dim() >= 1 && x.is_contiguous() && x.scalar_type() == at::kBFloat16,
+              "m2dscan: x must be a contiguous bfloat16 tensor on the GPU");
+  const int64_t C = x.size(-1);
+  TORCH_CHECK(w1.dim() == 2 && w1.size(1) == C && w1.is_contiguous() && w1.device() == x.device(),
+              "m2dscan: w1 must be a contiguous (hidden,", C, ") tensor on x's device");
+  const int64_t H = w1.size(0);
+  TORCH_CHECK(w2.sizes() == at::IntArrayRef({C, H}) && w2.is_contiguous() && w2.device() == x.device() &&
+              w2.scalar_type() == w1.scalar_type(), "m2dscan: w2 must be a contiguous (", C, ",", H, ") tensor of w1's dtype and device");
+  auto small = [&](const c10::optional<Tensor>& t, int64_t n, const char* name) -> const void* {
+    if (!t.has_value() || !t->defined()) return nullptr;
+    TORCH_CHECK(t->numel() == n && t->is_contiguous() && t->device() == x.device() && t->scalar_type() == w1.scalar_type(),
+                "m2dscan: ", name, " must hold ", n, " elements of the weights' dtype on x's device");
+    return t->data_ptr();
+  };
+  const void* b1p = small(b1, H, "b1");
+  const void* b2p = small(b2, C, "b2");
+  c10::DeviceGuard guard(x.device());
+  Tensor y = at::empty_like(x);
+  if (x.numel() == 0) return y;
+  hipStream_t st = c10::hip::getCurrentHIPStream(x.device().index()).stream();
+  check(m2d_mlp_fwd(x.numel() / C, static_cast<int>(C), static_cast<int>(H), dtype_code(w1, "w1"), x.data_ptr(), w1.data_ptr(), b1p,
+                    w2.data_ptr(), b2p, y.data_ptr(), st));
+  return y;
+}
+
 Tensor rope_attention_fwd(const Tensor& qkv, const Tensor& cos, const Tensor& sin, const Tensor& qw, const Tensor& qb,
                           const Tensor& kw, const Tensor& kb, double eps, double scale) {
   TORCH_CHECK(qkv.is_cuda() && qkv.dim() == 5 && qkv.size(2) == 3 && qkv.is_contiguous() && qkv.scalar_type() == at::kBFloat16,
@@ -405,6 +432,7 @@ TORCH_LIBRARY(m2dscan, m) {
         "float eps) -> (Tensor, Tensor)");
   m.def("rope_qknorm_fwd(Tensor qkv, Tensor cos, Tensor sin, Tensor q_weight, Tensor q_bias, Tensor k_weight, Tensor k_bias, "
         "float eps, bool token_major=False) -> (Tensor, Tensor)");
+  m.def("mlp_fwd(Tensor x, Tensor w1, Tensor? b1, Tensor w2, Tensor? b2) -> Tensor");
   m.def("rope_attention_fwd(Tensor qkv, Tensor cos, Tensor sin, Tensor q_weight, Tensor q_bias, Tensor k_weight, Tensor k_bias, "
         "float eps, float scale) -> Tensor");
   m.def("linear_act_fwd(Tensor x, Tensor weight, Tensor? bias, int pre, Tensor? pre_scale, Tensor? pre_bias, int post, "
@@ -424,5 +452,6 @@ TORCH_LIBRARY_IMPL(m2dscan, CUDA, m) {   // ROCm devices dispatch under the CUDA
   m.impl("rope_qknorm_fwd", &rope_qknorm_fwd);
   m.impl("scale_residual_layernorm_fwd", &scale_residual_layernorm_fwd);
   m.impl("rope_attention_fwd", &rope_attention_fwd);
+  m.impl("mlp_fwd", &mlp_fwd);
   m.impl("linear_act_fwd", &linear_act_fwd);
 }

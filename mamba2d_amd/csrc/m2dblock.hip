@@ -593,6 +593,115 @@ __global__ __launch_bounds__(kLinThreads) void m2d_linear_kernel(const LinArgs a
   }
 }
 
+// ------------------------------------------------------------ the MLP of a narrow stage, bf16
+// y = fc2(GELU(fc1 x)) (models/utils.py:58-81) where both weight matrices fit LDS together (C = 32 or 64
+// channels, 4 C hidden units): the hidden activations, four times the size of x and y and the reason why
+// the two layers run at the speed of memory writes when they are separate kernels, never leave the
+// registers.  A wave owns 16 rows.  H^T = W1 X^T puts, in lane (mn, kb), the hidden units 16 nt + 4 kb + i of
+// row mn; Y^T = W2 H^T contracts 32 hidden units per instruction and, as its operands may list them in any
+// order as long as both agree, takes for the lane's eight slots exactly the units the lane holds (4 kb + i of
+// two neighbouring tiles), with W2's rows read to match: no exchange of H between lanes.  Y^T leaves lane
+// (mn, kb) with outputs 16 no + 4 kb + i of row mn: 8-byte stores.
+struct MlpArgs {
+  const void* x;          // (P, C) bf16
+  const void *w1, *b1;    // (H, C), (H) or null
+  const void *w2, *b2;    // (C, H), (C) or null
+  void* y;                // (P, C) bf16
+  int64_t P;
+  int wbf16, ntiles;
+};
+
+template <int KC>   // C = 32 KC channels, 128 KC hidden units
+__global__ __launch_bounds__(kLinThreads) void m2d_mlp_kernel(const MlpArgs a) {
+  constexpr int C = 32 * KC, HD = 4 * C, NH = HD / 16, NO = C / 16, NP = NH / 2;
+  constexpr int W1S = C + 8;      // bf16 per row of W1 in LDS (a row per hidden unit)
+  constexpr int W2S = HD + 4;     // bf16 per row of W2 (a row per output): rows stay 8-byte aligned and spread over the banks
+  extern __shared__ float smem[];
+  uint16_t* w1l = reinterpret_cast<uint16_t*>(smem);
+  uint16_t* w2l = w1l + HD * W1S;
+  float* b1l = reinterpret_cast<float*>(w2l + C * W2S);
+  const int tid = threadIdx.x, l = tid & 63, mn = l & 15, kb = l >> 4;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  auto stage_weights = [&](const void* w, int rows, int cols, uint16_t* dst, int stride) {   // 8 elements at a time
+    for (int i = tid; i < rows * (cols / 8); i += kLinThreads) {
+      const int n = i / (cols / 8), k8 = i - n * (cols / 8);
+      if (a.wbf16) {
+        const uint4 q = ld16(static_cast<const uint16_t*>(w) + (int64_t)n * cols + 8 * k8);
+        uint2* d = reinterpret_cast<uint2*>(dst + n * stride + 8 * k8);      // rows of W2 are 8-byte aligned only
+        d[0] = make_uint2(q.x, q.y);
+        d[1] = make_uint2(q.z, q.w);
+      } else {
+        const float* src = static_cast<const float*>(w) + (int64_t)n * cols + 8 * k8;
+        uint2* d = reinterpret_cast<uint2*>(dst + n * stride + 8 * k8);
+        d[0] = make_uint2(pack_bf16(src[0], src[1]), pack_bf16(src[2], src[3]));
+        d[1] = make_uint2(pack_bf16(src[4], src[5]), pack_bf16(src[6], src[7]));
+      }
+    }
+  };
+  stage_weights(a.w1, HD, C, w1l, W1S);
+  stage_weights(a.w2, C, HD, w2l, W2S);
+  for (int i = tid; i < HD; i += kLinThreads) b1l[i] = a.b1 ? ldw(a.b1, a.wbf16, i) : 0.f;
+  float b2v[NO][4];
+#pragma unroll
+  for (int no = 0; no < NO; ++no)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) b2v[no][i] = a.b2 ? ldw(a.b2, a.wbf16, 16 * no + 4 * kb + i) : 0.f;
+  __syncthreads();
+  const uint16_t* X = static_cast<const uint16_t*>(a.x);
+  uint16_t* Y = static_cast<uint16_t*>(a.y);
+  const f32x4_t zero = {0.f, 0.f, 0.f, 0.f};
+  uint4 Xnext[KC];
+  auto fetch = [&](int tile) {
+    const int64_t q0 = (int64_t)tile * 64 + wave * 16;
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc) {
+      Xnext[kc] = make_uint4(0u, 0u, 0u, 0u);
+      if (tile < a.ntiles && q0 + mn < a.P) Xnext[kc] = ld16(X + (q0 + mn) * C + 32 * kc + 8 * kb);
+    }
+  };
+  fetch(blockIdx.x);
+  for (int tile = blockIdx.x; tile < a.ntiles; tile += gridDim.x) {
+    const int64_t p0 = (int64_t)tile * 64 + wave * 16;
+    uint4 Xf[KC];
+#pragma unroll
+    for (int kc = 0; kc < KC; ++kc) Xf[kc] = Xnext[kc];
+    fetch(tile + gridDim.x);
+    f32x4_t h[NH];
+#pragma unroll
+    for (int nt = 0; nt < NH; ++nt) {
+      f32x4_t acc = zero;
+#pragma unroll
+      for (int kc = 0; kc < KC; ++kc) acc = mfma_bf16(ld16(w1l + (16 * nt + mn) * W1S + 32 * kc + 8 * kb), Xf[kc], acc);
+      const float4 b1 = *reinterpret_cast<const float4*>(b1l + 16 * nt + 4 * kb);
+      h[nt][0] = gelu_exact(acc[0] + b1.x);
+      h[nt][1] = gelu_exact(acc[1] + b1.y);
+      h[nt][2] = gelu_exact(acc[2] + b1.z);
+      h[nt][3] = gelu_exact(acc[3] + b1.w);
+    }
+    uint4 hf[NP];      // the hidden activations as bf16, as fc2 of the stock path would read them
+#pragma unroll
+    for (int ks = 0; ks < NP; ++ks)
+      hf[ks] = make_uint4(pack_bf16(h[2 * ks][0], h[2 * ks][1]), pack_bf16(h[2 * ks][2], h[2 * ks][3]),
+                          pack_bf16(h[2 * ks + 1][0], h[2 * ks + 1][1]), pack_bf16(h[2 * ks + 1][2], h[2 * ks + 1][3]));
+#pragma unroll
+    for (int no = 0; no < NO; ++no) {
+      f32x4_t acc = zero;
+#pragma unroll
+      for (int ks = 0; ks < NP; ++ks) {
+        const uint16_t* w = w2l + (16 * no + mn) * W2S + 32 * ks + 4 * kb;      // output 16 no + mn, units 32 ks + 4 kb + {0..3, 16..19}
+        const uint2 lo = *reinterpret_cast<const uint2*>(w), hi = *reinterpret_cast<const uint2*>(w + 16);
+        acc = mfma_bf16(make_uint4(lo.x, lo.y, hi.x, hi.y), hf[ks], acc);
+      }
+      if (p0 + mn < a.P)
+        *reinterpret_cast<uint2*>(Y + (p0 + mn) * C + 16 * no + 4 * kb) =
+            make_uint2(pack_bf16(acc[0] + b2v[no][0], acc[1] + b2v[no][1]), pack_bf16(acc[2] + b2v[no][2], acc[3] + b2v[no][3]));
+    }
+  }
+}
+
+template <int KC>
+constexpr size_t mlp_lds_bytes() { return (size_t)(128 * KC) * (32 * KC + 8) * 2 + (size_t)(32 * KC) * (128 * KC + 4) * 2 + (size_t)(128 * KC) * 4; }
+
 constexpr size_t kLinMaxLds = 160 * 1024;   // LDS of a compute unit
 
 // More than 64 KB of dynamic LDS has to be allowed per kernel and device, once.
@@ -603,7 +712,8 @@ inline bool allow_big_lds() {
   const uint64_t bit = 1ull << (dev & 63);
   if (seen.load(std::memory_order_acquire) & bit) return true;
   const void* kernels[] = {reinterpret_cast<const void*>(&m2d_linear_kernel<2>), reinterpret_cast<const void*>(&m2d_linear_kernel<4>),
-                           reinterpret_cast<const void*>(&m2d_linear_kernel<8>), reinterpret_cast<const void*>(&m2d_linear_kernel<16>)};
+                           reinterpret_cast<const void*>(&m2d_linear_kernel<8>), reinterpret_cast<const void*>(&m2d_linear_kernel<16>),
+                           reinterpret_cast<const void*>(&m2d_mlp_kernel<1>), reinterpret_cast<const void*>(&m2d_mlp_kernel<2>)};
   for (const void* k : kernels)
     if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLinMaxLds) != hipSuccess) return false;
   seen.fetch_or(bit, std::memory_order_release);
@@ -910,6 +1020,30 @@ int m2d_rope_qknorm_fwd(int B, int L, int heads, int head_dim, int dtype, int we
   a.total = (int64_t)B * L * 2 * heads * G;
   hipStream_t st = static_cast<hipStream_t>(stream);
   return dtype == M2D_F32 ? run_rope<float>(a, G, st) : run_rope<bf16_t>(a, G, st);
+}
+
+int m2d_mlp_fwd(int64_t P, int C, int hidden, int weight_dtype, const void* x, const void* w1, const void* b1, const void* w2,
+                const void* b2, void* y, void* stream) {
+  if (!x || !w1 || !w2 || !y) return M2D_ERR_NULL_POINTER;
+  if (P < 1 || C < 1 || hidden < 1) return M2D_ERR_BAD_SHAPE;
+  if (weight_dtype != M2D_F32 && weight_dtype != M2D_BF16) return M2D_ERR_UNSUPPORTED;
+  if ((C != 32 && C != 64) || hidden != 4 * C) return M2D_ERR_UNSUPPORTED;
+  if ((P + 63) / 64 >= ((int64_t)1 << 31)) return M2D_ERR_UNSUPPORTED;
+  if (misaligned(x, 16) || misaligned(y, 16) || misaligned(w1, 16) || misaligned(w2, 16) || (b1 && misaligned(b1, 4)) || (b2 && misaligned(b2, 4)))
+    return M2D_ERR_MISALIGNED;
+  MlpArgs a = {};
+  a.x = x; a.w1 = w1; a.b1 = b1; a.w2 = w2; a.b2 = b2; a.y = y; a.P = P; a.wbf16 = weight_dtype == M2D_BF16;
+  a.ntiles = (int)((P + 63) / 64);
+  const size_t lds = C == 64 ? mlp_lds_bytes<2>() : mlp_lds_bytes<1>();
+  if (lds > 64 * 1024 && !allow_big_lds()) return M2D_ERR_HIP;
+  int per_cu = (int)(160 * 1024 / lds);      // persistent: the weights go to LDS once per workgroup
+  if (per_cu > 4) per_cu = 4;
+  int grid = 256 * per_cu;
+  if (grid > a.ntiles) grid = a.ntiles;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (C == 64) hipLaunchKernelGGL(m2d_mlp_kernel<2>, dim3((unsigned)grid), dim3(kLinThreads), lds, st, a);
+  else hipLaunchKernelGGL(m2d_mlp_kernel<1>, dim3((unsigned)grid), dim3(kLinThreads), lds, st, a);
+  return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
 int m2d_rope_attention_fwd(int B, int L, int heads, int head_dim, int weight_dtype, const void* qkv, const void* cos,

@@ -44,6 +44,7 @@ scale_residual_fwd_op = torch.ops.m2dscan.scale_residual_fwd
 scale_residual_layernorm_fwd_op = torch.ops.m2dscan.scale_residual_layernorm_fwd
 rope_qknorm_fwd_op = torch.ops.m2dscan.rope_qknorm_fwd
 rope_attention_fwd_op = torch.ops.m2dscan.rope_attention_fwd
+mlp_fwd_op = torch.ops.m2dscan.mlp_fwd
 linear_act_fwd_op = torch.ops.m2dscan.linear_act_fwd
 
 # Keep the forward's anti-diagonal checkpoints for the backward (faster backward, more saved
@@ -120,6 +121,11 @@ def _scale_residual_fwd_fake(x, scale, residual, residual2=None):
 @torch.library.register_fake("m2dscan::linear_act_fwd")
 def _linear_act_fwd_fake(x, weight, bias, pre, pre_scale, pre_bias, post, post_scale, post_bias):
     return x.new_empty((*x.shape[:-1], weight.shape[0]))
+
+
+@torch.library.register_fake("m2dscan::mlp_fwd")
+def _mlp_fwd_fake(x, w1, b1, w2, b2):
+    return torch.empty_like(x)
 
 
 @torch.library.register_fake("m2dscan::rope_attention_fwd")

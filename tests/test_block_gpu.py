@@ -1,5 +1,5 @@
 """GPU parity of the residual-block operators (m2d_layernorm_fwd, m2d_dwconv3x3_fwd, m2d_starrelu_fwd,
-m2d_scale_residual_fwd, m2d_scale_residual_layernorm_fwd, m2d_rope_qknorm_fwd, m2d_rope_attention_fwd, m2d_linear_fwd) through the C ABI, against the stock torch operators the reference uses (nn.LayerNorm, models/mamba2d.py:220;
+m2d_scale_residual_fwd, m2d_scale_residual_layernorm_fwd, m2d_rope_qknorm_fwd, m2d_rope_attention_fwd, m2d_linear_fwd, m2d_mlp_fwd) through the C ABI, against the stock torch operators the reference uses (nn.LayerNorm, models/mamba2d.py:220;
 depthwise nn.Conv2d, models/utils.py:101) evaluated in fp64 on the CPU.  Tolerances: fp32 2e-5,
 bf16 tensors 1e-2 (max error over max value; one bf16 rounding of the result is 4e-3)."""
 import pytest
@@ -242,6 +242,40 @@ def test_small_linear_matches_torch(cabi, shape, acts, wdtype):
     nb = cabi.linear_fwd(x.cuda(), w.cuda(), None, pre, params if pre == 2 else None, post, params if post == 2 else None)
     want_nb = ref_act(post, a_in @ w.bfloat16().double().t())
     assert so.rel_err(nb.float().cpu(), want_nb) < 1e-2
+
+
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16], ids=["w_f32", "w_bf16"])
+@pytest.mark.parametrize("bias", [True, False], ids=["bias", "no_bias"])
+@pytest.mark.parametrize("shape", [(2 * 9 * 12, 64), (1000, 64), (333, 32), (64, 64), (5, 32), (70000, 64)], ids=lambda s: "x".join(map(str, s)))
+def test_fused_mlp_matches_torch(cabi, shape, bias, wdtype):
+    """fc2(GELU(fc1 x)) in one kernel against fp64 on the CPU with the hidden activations rounded to bf16 (as the
+    kernel hands them to fc2 and as the stock path stores them); weights rounded to bf16 as the kernel holds them."""
+    P, C = shape
+    say(f"\ncase mlp {shape} bias={bias} {wdtype}")
+    g = torch.Generator().manual_seed(P + C)
+    x = torch.randn(P, C, generator=g).bfloat16()
+    w1 = (torch.randn(4 * C, C, generator=g) / C ** 0.5).to(wdtype)
+    w2 = (torch.randn(C, 4 * C, generator=g) / (4 * C) ** 0.5).to(wdtype)
+    b1 = (torch.randn(4 * C, generator=g) * 0.5).to(wdtype) if bias else None
+    b2 = (torch.randn(C, generator=g) * 0.5).to(wdtype) if bias else None
+    h = x.double() @ w1.bfloat16().double().T + (b1.double() if bias else 0)
+    h = torch.nn.functional.gelu(h).bfloat16().double()
+    want = h @ w2.bfloat16().double().T + (b2.double() if bias else 0)
+    dev = lambda t: None if t is None else t.cuda()
+    got = cabi.mlp_fwd(x.cuda(), dev(w1), dev(b1), dev(w2), dev(b2))
+    torch.cuda.synchronize()
+    assert got.shape == x.shape and got.dtype == torch.bfloat16
+    err = so.rel_err(got.float().cpu(), want)
+    say(f"  rel err {err:.3e}")
+    assert err < TOL[torch.bfloat16]
+
+
+def test_fused_mlp_limits_are_reported(cabi):
+    for C, H in ((128, 512), (64, 128), (48, 192)):
+        x = torch.zeros(8, C, device="cuda", dtype=torch.bfloat16)
+        with pytest.raises(cabi.M2DError) as e:
+            cabi.mlp_fwd(x, torch.zeros(H, C, device="cuda"), None, torch.zeros(C, H, device="cuda"), None)
+        assert e.value.status == 3      # M2D_ERR_UNSUPPORTED
 
 
 def test_small_linear_limits_are_reported(cabi):
