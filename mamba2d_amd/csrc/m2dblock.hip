@@ -42,6 +42,9 @@ template <> struct Chunk<float> {
     *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
   }
   static __device__ __forceinline__ void store_rounded(float* p, float (&v)[4]) { store(p, v); }
+  static __device__ __forceinline__ void unpack(const uint4& q, float (&v)[4]) {
+    v[0] = __uint_as_float(q.x); v[1] = __uint_as_float(q.y); v[2] = __uint_as_float(q.z); v[3] = __uint_as_float(q.w);
+  }
 };
 template <> struct Chunk<bf16_t> {
   static constexpr int kV = 8;
@@ -53,6 +56,11 @@ template <> struct Chunk<bf16_t> {
   }
   static __device__ __forceinline__ void store(bf16_t* p, const float (&v)[8]) {
     *reinterpret_cast<uint4*>(p) = make_uint4(pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3]), pack_bf16(v[4], v[5]), pack_bf16(v[6], v[7]));
+  }
+  static __device__ __forceinline__ void unpack(const uint4& q, float (&v)[8]) {
+    const uint32_t w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) { v[2 * j] = bf_lo(w[j]); v[2 * j + 1] = bf_hi(w[j]); }
   }
   // stores v and leaves in v what a reader of p will find
   static __device__ __forceinline__ void store_rounded(bf16_t* p, float (&v)[8]) {
@@ -227,6 +235,7 @@ int run_ln(const LnArgs& a, hipStream_t st) {
 // the chunk stay in registers.  The kernel is bound by the number of loads: strips of 14 (which
 // divide the model's widths 56, 28, 14) run 7 % faster than strips of 8, strips of 4 45 % slower.
 constexpr int kDwThreads = 256;
+constexpr int kDwAhead = 4;        // columns between a fetch and its first use (2: 52 us, 3: 50 us, 4: 48 us at 56x56x128, B=128)
 
 struct DwArgs {
   const void* x;
@@ -263,40 +272,44 @@ __global__ __launch_bounds__(kDwThreads) void m2d_dwconv3x3_kernel(const DwArgs 
   const T* X = static_cast<const T*>(a.x) + ((int64_t)b * a.H * a.W) * a.C + c * V;
   T* Y = static_cast<T*>(a.y) + ((int64_t)b * a.H * a.W) * a.C + c * V;
   const int w0 = sidx * STRIP;
-  // window columns: win[i][0..2] are the cells (h+i-1, w-1), (h+i-1, w), (h+i-1, w+1)
-  float win[3][3][V];
+  // Window: the 16-byte chunks of the cells (h+i-1, w-1 .. w+kDwAhead) as they come from memory, columns that
+  // rotate with the step; column w+kDwAhead is fetched kDwAhead steps before its first use, so that a thread has
+  // 3 kDwAhead loads in flight (with one column ahead and three waves per SIMD the kernel waited for memory half of
+  // the time).  Unpacked at every use: the conversions are cheap next to the registers a float window costs.
+  constexpr int NS = kDwAhead + 2;      // columns held
+  uint4 win[3][NS];
   auto load_col = [&](int col, int slot) {
 #pragma unroll
     for (int i = 0; i < 3; ++i) {
       const int hh = h + i - 1;
-      if (hh >= 0 && hh < a.H && col >= 0 && col < a.W) {
-        Chunk<T>::load(X + ((int64_t)hh * a.W + col) * a.C, win[i][slot]);
-      } else {
-#pragma unroll
-        for (int j = 0; j < V; ++j) win[i][slot][j] = 0.f;
-      }
+      win[i][slot] = make_uint4(0u, 0u, 0u, 0u);
+      if (hh >= 0 && hh < a.H && col >= 0 && col < a.W)
+        win[i][slot] = *reinterpret_cast<const uint4*>(X + ((int64_t)hh * a.W + col) * a.C);
     }
   };
-  load_col(w0 - 1, 0);
-  load_col(w0, 1);
+#pragma unroll
+  for (int k = 0; k <= kDwAhead; ++k) load_col(w0 - 1 + k, k);
 #pragma unroll
   for (int s = 0; s < STRIP; ++s) {
     const int w = w0 + s;
     if (w >= a.W) break;
-    // slot of column w-1, w, w+1 rotates with s
-    const int sl = s % 3, sm = (s + 1) % 3, sr = (s + 2) % 3;
-    load_col(w + 1, sr);
+    const int sl = s % NS, sm = (s + 1) % NS, sr = (s + 2) % NS;      // slots of columns w-1, w, w+1
+    if (s + kDwAhead <= STRIP) load_col(w + kDwAhead, (s + kDwAhead + 1) % NS);
     float o[V];
 #pragma unroll
-    for (int j = 0; j < V; ++j) {
-      float acc = 0.f;
+    for (int j = 0; j < V; ++j) o[j] = 0.f;
 #pragma unroll
-      for (int i = 0; i < 3; ++i) {
-        acc = __builtin_fmaf(wt[3 * i][j], win[i][sl][j], acc);
-        acc = __builtin_fmaf(wt[3 * i + 1][j], win[i][sm][j], acc);
-        acc = __builtin_fmaf(wt[3 * i + 2][j], win[i][sr][j], acc);
+    for (int i = 0; i < 3; ++i) {
+      float xl[V], xm[V], xr[V];
+      Chunk<T>::unpack(win[i][sl], xl);
+      Chunk<T>::unpack(win[i][sm], xm);
+      Chunk<T>::unpack(win[i][sr], xr);
+#pragma unroll
+      for (int j = 0; j < V; ++j) {
+        o[j] = __builtin_fmaf(wt[3 * i][j], xl[j], o[j]);
+        o[j] = __builtin_fmaf(wt[3 * i + 1][j], xm[j], o[j]);
+        o[j] = __builtin_fmaf(wt[3 * i + 2][j], xr[j], o[j]);
       }
-      o[j] = acc;
     }
     Chunk<T>::store(Y + ((int64_t)h * a.W + w) * a.C, o);
   }
