@@ -253,12 +253,24 @@ int m2d_linear_fwd(int64_t P, int K, int N, int weight_dtype, const void* x, con
                    int pre_act, const void* pre_scale, const void* pre_bias,
                    int post_act, const void* post_scale, const void* post_bias, void* y, void* stream);
 
+/* m2d_linear_fwd with a LayerNorm over the K inputs in front of the layer (ln_weight, ln_bias: (K), weight_dtype):
+ * y = post(LayerNorm(x) weight^T + bias), for a norm whose only reader is the layer (local_norm before pwconv1,
+ * models/mamba2d.py:57,161; norm2 before fc1, :248).  The normalised rows are rounded to bf16 as a LayerNorm
+ * kernel would store them, and never written.  K up to 128; otherwise as m2d_linear_fwd. */
+int m2d_layernorm_linear_fwd(int64_t P, int K, int N, int weight_dtype, const void* x,
+                             const void* ln_weight, const void* ln_bias, float eps,
+                             const void* weight, const void* bias,
+                             int post_act, const void* post_scale, const void* post_bias, void* y, void* stream);
+
 /* y = fc2(GELU(fc1 x)) of the MLP (models/utils.py:58-81) where both weight matrices fit LDS together:
  * C = 32 or 64 channels and hidden = 4 C.  x and y are (P, C) bf16; w1 (hidden, C), b1 (hidden), w2 (C, hidden),
  * b2 (C) have weight_dtype; b1 and b2 may be NULL.  The hidden activations stay in registers; they enter the
- * second product rounded to bf16, as the stock path stores them.  Other sizes: M2D_ERR_UNSUPPORTED. */
-int m2d_mlp_fwd(int64_t P, int C, int hidden, int weight_dtype, const void* x, const void* w1, const void* b1,
-                const void* w2, const void* b2, void* y, void* stream);
+ * second product rounded to bf16, as the stock path stores them.  With ln_weight and ln_bias (C each, weight_dtype;
+ * both or neither) the rows of x pass through LayerNorm(eps) first (norm2 of the block, models/mamba2d.py:248),
+ * rounded to bf16 as a LayerNorm kernel would store them.  Other sizes: M2D_ERR_UNSUPPORTED. */
+int m2d_mlp_fwd(int64_t P, int C, int hidden, int weight_dtype, const void* x,
+                const void* ln_weight, const void* ln_bias, float eps,
+                const void* w1, const void* b1, const void* w2, const void* b2, void* y, void* stream);
 
 /* Measurement aid; no counterpart in the reference.  While enabled, every m2d_scan_fwd /
  * m2d_scan_bwd call records a pair of HIP events on its stream around the main scan kernel of

@@ -22,7 +22,8 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from .wavefront import (dwconv3x3_fwd_op, layernorm_fwd_op, linear_act_fwd_op, mlp_fwd_op, rope_qknorm_fwd_op,
+from .wavefront import (dwconv3x3_fwd_op, layernorm_fwd_op, layernorm_linear_act_fwd_op, linear_act_fwd_op, mlp_fwd_op,
+                        rope_qknorm_fwd_op,
                         rope_attention_fwd_op, scale_residual_fwd_op, scale_residual_layernorm_fwd_op, starrelu_fwd_op,
                         wavefront_scan_cuda)
 
@@ -45,12 +46,19 @@ def _act(kind, star, t):
     return star(t) if kind == ACT_STARRELU else t
 
 
-def linear_act(lin, x, pre=ACT_NONE, post=ACT_NONE, star=None):
+def _norm_joins(norm, x, w):
+    """The LayerNorm ``norm`` over x's last axis can run inside the kernel of the layer (weights ``w``) that reads it."""
+    return (isinstance(norm, nn.LayerNorm) and norm.weight is not None and norm.bias is not None
+            and tuple(norm.normalized_shape) == (x.shape[-1],) and norm.weight.dtype == w.dtype and norm.bias.dtype == w.dtype
+            and _inference(norm.weight, norm.bias))
+
+
+def linear_act(lin, x, pre=ACT_NONE, post=ACT_NONE, star=None, norm=None):
     """post(lin(pre(x))) for a narrow linear layer: pre / post are nothing, GELU, or the StarReLU module
-    ``star``.  At inference on bf16 activations the product runs in the library's kernel together with its
-    neighbouring activation where the layer is narrow (up to 256 inputs and 512 outputs, the layers of the
-    stages with 64 and 128 channels: there the kernel is bound by the activations' bytes; wider layers are
-    faster in the stock library); otherwise stock operators."""
+    ``star``; with ``norm`` (a LayerNorm, and no ``pre``) the layer reads norm(x).  At inference on bf16 activations
+    the product runs in the library's kernel together with its neighbouring activation, or norm, where the layer is
+    narrow (up to 256 inputs and 512 outputs, the layers of the stages with 64 and 128 channels: there the kernel is
+    bound by the activations' bytes; wider layers are faster in the stock library); otherwise stock operators."""
     w, b = lin.weight, lin.bias
     N, K = w.shape
     if (x.is_cuda and x.dtype == torch.bfloat16 and _inference(x, w) and w.dtype in (torch.float32, torch.bfloat16)
@@ -58,7 +66,14 @@ def linear_act(lin, x, pre=ACT_NONE, post=ACT_NONE, star=None):
             and (star is None or star.scale.dtype == w.dtype)):
         ps = (star.scale, star.bias) if pre == ACT_STARRELU else (None, None)
         qs = (star.scale, star.bias) if post == ACT_STARRELU else (None, None)
+        if norm is not None and pre == ACT_NONE and K <= 128 and _norm_joins(norm, x, w):
+            # the normalised rows go from registers into the product and are never written
+            return layernorm_linear_act_fwd_op(x.contiguous(), norm.weight, norm.bias, norm.eps, w, b, post, *qs)
+        if norm is not None:
+            x = norm(x)
         return linear_act_fwd_op(x.contiguous(), w, b, pre, *ps, post, *qs)
+    if norm is not None:
+        x = norm(x)
     return _act(post, star, lin(_act(pre, star, x)))
 
 
@@ -119,13 +134,23 @@ class MLP(nn.Module):
         self.fc1 = nn.Linear(dim, dim * expand)
         self.fc2 = nn.Linear(dim * expand, dim)
 
-    def forward(self, x):
+    def forward(self, x, norm=None):
+        """fc2(GELU(fc1 x)), of norm(x) with ``norm`` (the block's norm2, which only the MLP reads)."""
         w1, w2 = self.fc1.weight, self.fc2.weight
         if (x.is_cuda and x.dtype == torch.bfloat16 and x.numel() > 0 and x.shape[-1] in (32, 64) and w1.shape[0] == 4 * w1.shape[1]
                 and _inference(x, w1, w2) and w1.dtype in (torch.float32, torch.bfloat16) and w2.dtype == w1.dtype):
             # both layers in one kernel: the hidden activations, four times x, never reach memory
-            return mlp_fwd_op(x.contiguous(), w1, self.fc1.bias, w2, self.fc2.bias)
-        return linear_act(self.fc2, linear_act(self.fc1, x, post=ACT_GELU))
+            if norm is not None and _norm_joins(norm, x, w1):
+                return mlp_fwd_op(x.contiguous(), w1, self.fc1.bias, w2, self.fc2.bias, norm.weight, norm.bias, norm.eps)
+            return mlp_fwd_op((x if norm is None else norm(x)).contiguous(), w1, self.fc1.bias, w2, self.fc2.bias)
+        return linear_act(self.fc2, linear_act(self.fc1, x, post=ACT_GELU, norm=norm))
+
+    def takes_norm(self, x, norm):
+        """norm(x) would not be written: the kernel of the first layer computes it."""
+        w1 = self.fc1.weight
+        return (x.is_cuda and x.dtype == torch.bfloat16 and x.numel() > 0 and _inference(x, w1, self.fc2.weight)
+                and w1.dtype in (torch.float32, torch.bfloat16) and self.fc2.weight.dtype == w1.dtype and _norm_joins(norm, x, w1)
+                and w1.shape[1] % 32 == 0 and w1.shape[1] <= 128 and w1.shape[0] % 16 == 0 and w1.shape[0] <= 512)
 
 
 def _conv_channel_last(conv, x):
@@ -148,8 +173,8 @@ class SepConv(nn.Module):
         self.act2 = StarReLU()
         self.pwconv2 = nn.Linear(med, dim, bias=False)
 
-    def forward(self, x):
-        x = linear_act(self.pwconv1, x, post=ACT_STARRELU, star=self.act1)
+    def forward(self, x, norm=None):
+        x = linear_act(self.pwconv1, x, post=ACT_STARRELU, star=self.act1, norm=norm)
         w = self.dwconv.weight
         if (x.is_cuda and _inference(x, w) and self.dwconv.kernel_size == (3, 3) and self.dwconv.padding == (1, 1)
                 and x.dtype in (torch.float32, torch.bfloat16) and w.dtype in (torch.float32, torch.bfloat16)
@@ -213,7 +238,7 @@ class M2DBlock(nn.Module):
     def forward(self, x, split=False):           # (B, H, W, C)
         """The mixed tokens; with ``split`` and a local path, the two terms of the sum, for a caller that
         adds them in a pass of its own."""
-        local = self.local_path(self.local_norm(x)) if self.local_path is not None else None
+        local = self.local_path(x, norm=self.local_norm) if self.local_path is not None else None
         u = linear_act(self.in_proj, x, post=ACT_GELU)
         y = wavefront_scan_cuda(u, self.AT_log, self.AL_log, self.x_proj.weight,
                                 self.dt_projT.weight, self.dt_projT.bias,
@@ -355,8 +380,13 @@ class ResBlock(nn.Module):
             terms = mixed if isinstance(mixed, tuple) else (mixed,)
         else:
             terms = (_drop_path(self.token_mixer(n1), self.drop_path, self.training),)
-        x, n2 = self._residual_norm(x, self.res_scale1, terms, self.norm2)
-        return self._residual_norm(x, self.res_scale2, (_drop_path(self.MLP(n2), self.drop_path, self.training),), next_norm)
+        if self.MLP.takes_norm(x, self.norm2):      # norm2 inside the MLP's first kernel: nobody else reads it
+            x = self._residual(x, self.res_scale1, *terms)
+            branch = self.MLP(x, norm=self.norm2)
+        else:
+            x, n2 = self._residual_norm(x, self.res_scale1, terms, self.norm2)
+            branch = self.MLP(n2)
+        return self._residual_norm(x, self.res_scale2, (_drop_path(branch, self.drop_path, self.training),), next_norm)
 
     def forward(self, x):
         return self.forward_fused(x)[0]

@@ -24,7 +24,7 @@ M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
            "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_bwd", "m2d_proj_workspace_bytes", "m2d_proj_fwd",
            "m2d_proj_bwd", "m2d_layernorm_fwd", "m2d_dwconv3x3_fwd", "m2d_starrelu_fwd",
-           "m2d_scale_residual_fwd", "m2d_scale_residual_layernorm_fwd", "m2d_rope_qknorm_fwd", "m2d_rope_attention_fwd", "m2d_mlp_fwd", "m2d_linear_fwd", "m2d_profile_enable", "m2d_profile_last_ms")
+           "m2d_scale_residual_fwd", "m2d_scale_residual_layernorm_fwd", "m2d_rope_qknorm_fwd", "m2d_rope_attention_fwd", "m2d_mlp_fwd", "m2d_layernorm_linear_fwd", "m2d_linear_fwd", "m2d_profile_enable", "m2d_profile_last_ms")
 
 
 class Desc(ctypes.Structure):
@@ -75,7 +75,9 @@ def _load():
     lib.m2d_scale_residual_fwd.restype = i32
     lib.m2d_scale_residual_fwd.argtypes = [ctypes.c_int64, i32, i32, i32, vp, vp, vp, vp, vp, vp]
     lib.m2d_mlp_fwd.restype = i32
-    lib.m2d_mlp_fwd.argtypes = [ctypes.c_int64, i32, i32, i32] + [vp] * 7
+    lib.m2d_mlp_fwd.argtypes = [ctypes.c_int64, i32, i32, i32, vp, vp, vp, ctypes.c_float] + [vp] * 6
+    lib.m2d_layernorm_linear_fwd.restype = i32
+    lib.m2d_layernorm_linear_fwd.argtypes = [ctypes.c_int64, i32, i32, i32, vp, vp, vp, ctypes.c_float, vp, vp, i32, vp, vp, vp, vp]
     lib.m2d_rope_attention_fwd.restype = i32
     lib.m2d_rope_attention_fwd.argtypes = [i32] * 5 + [vp] * 7 + [ctypes.c_float, ctypes.c_float, vp, vp]
     lib.m2d_rope_qknorm_fwd.restype = i32
@@ -334,22 +336,23 @@ def scale_residual_layernorm_fwd(x, scale, residual, residual2, weight, bias, ep
     return xo, y
 
 
-def mlp_fwd(x, w1, b1, w2, b2):
-    """fc2(GELU(fc1 x)) on a contiguous bf16 (..., C) tensor, through m2d_mlp_fwd (C = 32 or 64, hidden = 4 C)."""
+def mlp_fwd(x, w1, b1, w2, b2, ln_weight=None, ln_bias=None, eps=1e-5):
+    """fc2(GELU(fc1 x)) on a contiguous bf16 (..., C) tensor, through m2d_mlp_fwd (C = 32 or 64, hidden = 4 C); with
+    ``ln_weight`` and ``ln_bias`` x passes through LayerNorm first."""
     C = x.shape[-1]
     if not x.is_cuda or not x.is_contiguous() or x.dtype != torch.bfloat16:
         raise ValueError("m2dscan: x must be a contiguous bfloat16 tensor on the GPU")
     H = w1.shape[0]
     if w1.dim() != 2 or w1.shape[1] != C or tuple(w2.shape) != (C, H) or w2.dtype != w1.dtype:
         raise ValueError(f"m2dscan: w1 must be (hidden,{C}) and w2 ({C},hidden), of one dtype")
-    for t, n in ((w1, None), (w2, None), (b1, H), (b2, C)):
+    for t, n in ((w1, None), (w2, None), (b1, H), (b2, C), (ln_weight, C), (ln_bias, C)):
         if t is None:
             continue
         if t.device != x.device or not t.is_contiguous() or t.dtype != w1.dtype or (n is not None and t.numel() != n):
             raise ValueError(f"m2dscan: weights and biases must be contiguous tensors of one dtype on {x.device}")
     y = torch.empty_like(x)
-    check(lib.m2d_mlp_fwd(x.numel() // C, C, H, _dtype_code(w1), _ptr(x), _ptr(w1), None if b1 is None else _ptr(b1), _ptr(w2),
-                          None if b2 is None else _ptr(b2), _ptr(y), _stream(x.device)))
+    check(lib.m2d_mlp_fwd(x.numel() // C, C, H, _dtype_code(w1), _ptr(x), _ptr(ln_weight), _ptr(ln_bias), float(eps), _ptr(w1),
+                          _ptr(b1), _ptr(w2), _ptr(b2), _ptr(y), _stream(x.device)))
     return y
 
 
@@ -398,16 +401,17 @@ def rope_qknorm_fwd(qkv, cos, sin, q_weight, q_bias, k_weight, k_bias, eps=1e-5,
 ACT_NONE, ACT_GELU, ACT_STARRELU = 0, 1, 2
 
 
-def linear_fwd(x, weight, bias=None, pre=ACT_NONE, pre_params=None, post=ACT_NONE, post_params=None):
+def linear_fwd(x, weight, bias=None, pre=ACT_NONE, pre_params=None, post=ACT_NONE, post_params=None, ln=None):
     """post(pre(x) @ weight.T + bias) on bf16 activations through m2d_linear_fwd; ``*_params`` are the
-    (scale, bias) one-element tensors of a StarReLU."""
+    (scale, bias) one-element tensors of a StarReLU.  ``ln`` = (weight, bias, eps) of a LayerNorm over x's last
+    axis in front of the layer (then through m2d_layernorm_linear_fwd, and no ``pre``)."""
     K = x.shape[-1]
     N = weight.shape[0]
     if x.dtype != torch.bfloat16 or not x.is_cuda or not x.is_contiguous():
         raise ValueError("m2dscan: x must be a contiguous bfloat16 tensor on the GPU")
     if tuple(weight.shape) != (N, K) or not weight.is_contiguous() or weight.device != x.device:
         raise ValueError(f"m2dscan: weight must be a contiguous (N,{K}) tensor on {x.device}")
-    small = [t for t in (bias, *(pre_params or ()), *(post_params or ())) if t is not None]
+    small = [t for t in (bias, *(pre_params or ()), *(post_params or ()), *((ln or ())[:2])) if t is not None]
     for t in small:
         if t.dtype != weight.dtype or t.device != x.device or not t.is_contiguous():
             raise ValueError("m2dscan: bias and activation parameters must have the weight's dtype and device")
@@ -416,6 +420,12 @@ def linear_fwd(x, weight, bias=None, pre=ACT_NONE, pre_params=None, post=ACT_NON
     ps, pb = pre_params if pre == ACT_STARRELU else (None, None)
     qs, qb = post_params if post == ACT_STARRELU else (None, None)
     y = x.new_empty((*x.shape[:-1], N))
+    if ln is not None:
+        if pre != ACT_NONE or tuple(ln[0].shape) != (K,) or tuple(ln[1].shape) != (K,):
+            raise ValueError(f"m2dscan: a LayerNorm in front of the layer takes ({K},) weights and no other activation before the layer")
+        check(lib.m2d_layernorm_linear_fwd(x.numel() // K, K, N, _dtype_code(weight), _ptr(x), _ptr(ln[0]), _ptr(ln[1]), float(ln[2]),
+                                           _ptr(weight), _ptr(bias), post, _ptr(qs), _ptr(qb), _ptr(y), _stream(x.device)))
+        return y
     check(lib.m2d_linear_fwd(x.numel() // K, K, N, _dtype_code(weight), _ptr(x), _ptr(weight), _ptr(bias), pre, _ptr(ps), _ptr(pb),
                              post, _ptr(qs), _ptr(qb), _ptr(y), _stream(x.device)))
     return y

@@ -331,7 +331,8 @@ std::tuple<Tensor, Tensor> rope_qknorm_fwd(const Tensor& qkv, const Tensor& cos,
 }
 
 Tensor mlp_fwd(const Tensor& x, const Tensor& w1, const c10::optional<Tensor>& b1, const Tensor& w2,
-               const c10::optional<Tensor>& b2) {
+               const c10::optional<Tensor>& b2, const c10::optional<Tensor>& ln_weight, const c10::optional<Tensor>& ln_bias,
+               double eps) {
   TORCH_CHECK(x.is_cuda() && x.dim() >= 1 && x.is_contiguous() && x.scalar_type() == at::kBFloat16,
               "m2dscan: x must be a contiguous bfloat16 tensor on the GPU");
   const int64_t C = x.size(-1);
@@ -348,12 +349,15 @@ Tensor mlp_fwd(const Tensor& x, const Tensor& w1, const c10::optional<Tensor>& b
   };
   const void* b1p = small(b1, H, "b1");
   const void* b2p = small(b2, C, "b2");
+  const void* lw = small(ln_weight, C, "ln_weight");
+  const void* lb = small(ln_bias, C, "ln_bias");
+  TORCH_CHECK((lw != nullptr) == (lb != nullptr), "m2dscan: ln_weight and ln_bias come together");
   c10::DeviceGuard guard(x.device());
   Tensor y = at::empty_like(x);
   if (x.numel() == 0) return y;
   hipStream_t st = c10::hip::getCurrentHIPStream(x.device().index()).stream();
-  check(m2d_mlp_fwd(x.numel() / C, static_cast<int>(C), static_cast<int>(H), dtype_code(w1, "w1"), x.data_ptr(), w1.data_ptr(), b1p,
-                    w2.data_ptr(), b2p, y.data_ptr(), st));
+  check(m2d_mlp_fwd(x.numel() / C, static_cast<int>(C), static_cast<int>(H), dtype_code(w1, "w1"), x.data_ptr(), lw, lb,
+                    static_cast<float>(eps), w1.data_ptr(), b1p, w2.data_ptr(), b2p, y.data_ptr(), st));
   return y;
 }
 
@@ -410,6 +414,37 @@ Tensor linear_act_fwd(const Tensor& x, const Tensor& weight, const c10::optional
   return y;
 }
 
+Tensor layernorm_linear_act_fwd(const Tensor& x, const Tensor& ln_weight, const Tensor& ln_bias, double eps, const Tensor& weight,
+                                const c10::optional<Tensor>& bias, int64_t post, const c10::optional<Tensor>& post_scale,
+                                const c10::optional<Tensor>& post_bias) {
+  TORCH_CHECK(x.is_cuda() && x.dim() >= 1 && x.is_contiguous() && x.scalar_type() == at::kBFloat16,
+              "m2dscan: x must be a contiguous bfloat16 tensor on the GPU");
+  const int64_t K = x.size(-1);
+  TORCH_CHECK(weight.dim() == 2 && weight.size(1) == K && weight.is_contiguous() && weight.device() == x.device(),
+              "m2dscan: weight must be a contiguous (N,", K, ") tensor on x's device");
+  const int64_t N = weight.size(0);
+  auto small = [&](const c10::optional<Tensor>& t, int64_t n, const char* name) -> const void* {
+    if (!t.has_value() || !t->defined()) return nullptr;
+    TORCH_CHECK(t->numel() == n && t->is_contiguous() && t->device() == x.device() && t->scalar_type() == weight.scalar_type(),
+                "m2dscan: ", name, " must hold ", n, " elements of the weight's dtype on x's device");
+    return t->data_ptr();
+  };
+  const void* lw = small(ln_weight, K, "ln_weight");
+  const void* lb = small(ln_bias, K, "ln_bias");
+  const void* b = small(bias, N, "bias");
+  const void* qs = small(post_scale, 1, "post_scale");
+  const void* qb = small(post_bias, 1, "post_bias");
+  c10::DeviceGuard guard(x.device());
+  std::vector<int64_t> shape(x.sizes().begin(), x.sizes().end());
+  shape.back() = N;
+  Tensor y = at::empty(shape, x.options());
+  if (x.numel() == 0) return y;
+  hipStream_t st = c10::hip::getCurrentHIPStream(x.device().index()).stream();
+  check(m2d_layernorm_linear_fwd(x.numel() / K, static_cast<int>(K), static_cast<int>(N), dtype_code(weight, "weight"), x.data_ptr(),
+                                 lw, lb, static_cast<float>(eps), weight.data_ptr(), b, static_cast<int>(post), qs, qb, y.data_ptr(), st));
+  return y;
+}
+
 int64_t abi_version() { return m2d_version(); }
 
 }  // namespace
@@ -432,7 +467,10 @@ TORCH_LIBRARY(m2dscan, m) {
         "float eps) -> (Tensor, Tensor)");
   m.def("rope_qknorm_fwd(Tensor qkv, Tensor cos, Tensor sin, Tensor q_weight, Tensor q_bias, Tensor k_weight, Tensor k_bias, "
         "float eps, bool token_major=False) -> (Tensor, Tensor)");
-  m.def("mlp_fwd(Tensor x, Tensor w1, Tensor? b1, Tensor w2, Tensor? b2) -> Tensor");
+  m.def("mlp_fwd(Tensor x, Tensor w1, Tensor? b1, Tensor w2, Tensor? b2, Tensor? ln_weight=None, Tensor? ln_bias=None, "
+        "float eps=1e-5) -> Tensor");
+  m.def("layernorm_linear_act_fwd(Tensor x, Tensor ln_weight, Tensor ln_bias, float eps, Tensor weight, Tensor? bias, int post, "
+        "Tensor? post_scale, Tensor? post_bias) -> Tensor");
   m.def("rope_attention_fwd(Tensor qkv, Tensor cos, Tensor sin, Tensor q_weight, Tensor q_bias, Tensor k_weight, Tensor k_bias, "
         "float eps, float scale) -> Tensor");
   m.def("linear_act_fwd(Tensor x, Tensor weight, Tensor? bias, int pre, Tensor? pre_scale, Tensor? pre_bias, int post, "
@@ -453,5 +491,6 @@ TORCH_LIBRARY_IMPL(m2dscan, CUDA, m) {   // ROCm devices dispatch under the CUDA
   m.impl("scale_residual_layernorm_fwd", &scale_residual_layernorm_fwd);
   m.impl("rope_attention_fwd", &rope_attention_fwd);
   m.impl("mlp_fwd", &mlp_fwd);
+  m.impl("layernorm_linear_act_fwd", &layernorm_linear_act_fwd);
   m.impl("linear_act_fwd", &linear_act_fwd);
 }

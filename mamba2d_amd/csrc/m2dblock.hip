@@ -484,7 +484,7 @@ constexpr int kLinThreads = 256;
 constexpr int kLinWaves = 4;
 constexpr int kLinStage = 72;      // floats per row of a wave's result block: 64 + 8
 constexpr int kLinMaxKC = 16;      // steps of 32 along K: K <= 512
-enum { kActNone = 0, kActGelu = 1, kActStarRelu = 2 };
+enum { kActNone = 0, kActGelu = 1, kActStarRelu = 2, kActLayerNorm = 3 };   // the last one only before the layer, and only inside this file
 
 // erf by Abramowitz & Stegun 7.1.26 (absolute error below 1.5e-7), one v_exp_f32 and one v_rcp_f32
 __device__ __forceinline__ float gelu_exact(float v) {
@@ -503,6 +503,49 @@ __device__ __forceinline__ float act(int kind, float v, float s, float b) {
   return v;
 }
 
+// LayerNorm of the 16 rows a wave holds as MFMA operands (lane (mn, kb): the 8 values at 32 kc + 8 kb + j of row
+// mn, for kc < KC), in place, rounded to bf16 as a LayerNorm kernel in front of the layer would store them.
+// lnp: weight then bias, K floats each, in LDS.  Two-pass mean / variance; the four lanes of a row meet through
+// two lane exchanges.
+template <int KCMAX>
+__device__ __forceinline__ void norm_rows(uint4 (&A)[KCMAX], int KC, int K, const float* lnp, float eps, int kb) {
+  float v[KCMAX][8];
+  float s = 0.f;
+#pragma unroll
+  for (int kc = 0; kc < KCMAX; ++kc) {
+    Chunk<bf16_t>::unpack(A[kc], v[kc]);
+    if (kc < KC) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) s += v[kc][j];
+    }
+  }
+  s += __shfl_xor(s, 16, 64);
+  s += __shfl_xor(s, 32, 64);
+  const float inv = 1.f / (float)K, mean = s * inv;
+  float q = 0.f;
+#pragma unroll
+  for (int kc = 0; kc < KCMAX; ++kc)
+    if (kc < KC) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) { const float d = v[kc][j] - mean; q = __builtin_fmaf(d, d, q); }
+    }
+  q += __shfl_xor(q, 16, 64);
+  q += __shfl_xor(q, 32, 64);
+  const float rstd = rsqrtf(q * inv + eps);
+#pragma unroll
+  for (int kc = 0; kc < KCMAX; ++kc)
+    if (kc < KC) {
+      const float* w = lnp + 32 * kc + 8 * kb;
+      const float4 w0 = *reinterpret_cast<const float4*>(w), w1 = *reinterpret_cast<const float4*>(w + 4);
+      const float4 b0 = *reinterpret_cast<const float4*>(w + K), b1 = *reinterpret_cast<const float4*>(w + K + 4);
+      const float wv[8] = {w0.x, w0.y, w0.z, w0.w, w1.x, w1.y, w1.z, w1.w}, bv[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
+      float o[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = __builtin_fmaf((v[kc][j] - mean) * rstd, wv[j], bv[j]);
+      A[kc] = make_uint4(pack_bf16(o[0], o[1]), pack_bf16(o[2], o[3]), pack_bf16(o[4], o[5]), pack_bf16(o[6], o[7]));
+    }
+}
+
 struct LinArgs {
   const void* x;        // (P, K) bf16
   const void* w;        // (N, K)
@@ -512,6 +555,8 @@ struct LinArgs {
   int K, N, wbf16, pre, post, ntiles;
   int nsplit, Ns;       // the workgroups share out the N outputs in nsplit slices of Ns
   const void *pre_s, *pre_b, *post_s, *post_b;   // StarReLU scale and bias (one element each, type of w) where pre / post is StarReLU
+  const void *ln_w, *ln_b;                       // LayerNorm over the K inputs in front of the layer (pre == kActLayerNorm): weight and bias, (K), type of w
+  float ln_eps;
 };
 
 template <int KCMAX>   // steps of 32 along K that the kernel is built for: 2, 4, 8 or 16
@@ -535,6 +580,9 @@ __global__ __launch_bounds__(kLinThreads) void m2d_linear_kernel(const LinArgs a
     }
     *reinterpret_cast<uint4*>(wl + n * ws + 8 * k8) = q;
   }
+  float* lnp = smem + (a.Ns * ws / 2 + 3) / 4 * 4 + kLinWaves * 16 * kLinStage;      // behind the waves' result blocks
+  if (a.pre == kActLayerNorm)
+    for (int i = tid; i < a.K; i += kLinThreads) { lnp[i] = ldw(a.ln_w, a.wbf16, i); lnp[a.K + i] = ldw(a.ln_b, a.wbf16, i); }
   __syncthreads();
   const float pre_s = a.pre == kActStarRelu ? ldw(a.pre_s, a.wbf16, 0) : 0.f, pre_b = a.pre == kActStarRelu ? ldw(a.pre_b, a.wbf16, 0) : 0.f;
   const float post_s = a.post == kActStarRelu ? ldw(a.post_s, a.wbf16, 0) : 0.f, post_b = a.post == kActStarRelu ? ldw(a.post_b, a.wbf16, 0) : 0.f;
@@ -560,7 +608,9 @@ __global__ __launch_bounds__(kLinThreads) void m2d_linear_kernel(const LinArgs a
 #pragma unroll
     for (int kc = 0; kc < KCMAX; ++kc) A[kc] = Anext[kc];
     fetch(tile + tile_step);
-    if (a.pre != kActNone) {   // (uniform)
+    if (a.pre == kActLayerNorm) {   // (uniform; the host only asks for it where K <= 128)
+      if constexpr (KCMAX <= 4) norm_rows<KCMAX>(A, KC, a.K, lnp, a.ln_eps, kb);
+    } else if (a.pre != kActNone) {   // (uniform)
 #pragma unroll
       for (int kc = 0; kc < KCMAX; ++kc)
         if (kc < KC) {
@@ -622,6 +672,8 @@ struct MlpArgs {
   void* y;                // (P, C) bf16
   int64_t P;
   int wbf16, ntiles;
+  const void *ln_w, *ln_b;   // LayerNorm over C in front of fc1: weight and bias, (C), or null
+  float ln_eps;
 };
 
 template <int KC>   // C = 32 KC channels, 128 KC hidden units
@@ -654,6 +706,9 @@ __global__ __launch_bounds__(kLinThreads) void m2d_mlp_kernel(const MlpArgs a) {
   stage_weights(a.w1, HD, C, w1l, W1S);
   stage_weights(a.w2, C, HD, w2l, W2S);
   for (int i = tid; i < HD; i += kLinThreads) b1l[i] = a.b1 ? ldw(a.b1, a.wbf16, i) : 0.f;
+  float* lnp = b1l + HD;
+  if (a.ln_w)
+    for (int i = tid; i < C; i += kLinThreads) { lnp[i] = ldw(a.ln_w, a.wbf16, i); lnp[C + i] = ldw(a.ln_b, a.wbf16, i); }
   float b2v[NO][4];
 #pragma unroll
   for (int no = 0; no < NO; ++no)
@@ -679,6 +734,7 @@ __global__ __launch_bounds__(kLinThreads) void m2d_mlp_kernel(const MlpArgs a) {
 #pragma unroll
     for (int kc = 0; kc < KC; ++kc) Xf[kc] = Xnext[kc];
     fetch(tile + gridDim.x);
+    if (a.ln_w) norm_rows<KC>(Xf, KC, C, lnp, a.ln_eps, kb);      // (uniform)
     f32x4_t h[NH];
 #pragma unroll
     for (int nt = 0; nt < NH; ++nt) {
@@ -713,7 +769,7 @@ __global__ __launch_bounds__(kLinThreads) void m2d_mlp_kernel(const MlpArgs a) {
 }
 
 template <int KC>
-constexpr size_t mlp_lds_bytes() { return (size_t)(128 * KC) * (32 * KC + 8) * 2 + (size_t)(32 * KC) * (128 * KC + 4) * 2 + (size_t)(128 * KC) * 4; }
+constexpr size_t mlp_lds_bytes() { return (size_t)(128 * KC) * (32 * KC + 8) * 2 + (size_t)(32 * KC) * (128 * KC + 4) * 2 + (size_t)(128 * KC) * 4 + (size_t)(64 * KC) * 4; }
 
 constexpr size_t kLinMaxLds = 160 * 1024;   // LDS of a compute unit
 
@@ -733,7 +789,9 @@ inline bool allow_big_lds() {
   return true;
 }
 
-inline size_t linear_lds_bytes(int K, int N) { return ((size_t)N * (K + 8) / 2 + 3) / 4 * 4 * 4 + (size_t)kLinWaves * 16 * kLinStage * 4; }
+inline size_t linear_lds_bytes(int K, int N, bool ln = false) {
+  return ((size_t)N * (K + 8) / 2 + 3) / 4 * 4 * 4 + (size_t)kLinWaves * 16 * kLinStage * 4 + (ln ? (size_t)2 * K * 4 : 0);
+}
 
 inline bool misaligned(const void* p, size_t n) { return (reinterpret_cast<uintptr_t>(p) & (n - 1)) != 0; }
 
@@ -1035,16 +1093,18 @@ int m2d_rope_qknorm_fwd(int B, int L, int heads, int head_dim, int dtype, int we
   return dtype == M2D_F32 ? run_rope<float>(a, G, st) : run_rope<bf16_t>(a, G, st);
 }
 
-int m2d_mlp_fwd(int64_t P, int C, int hidden, int weight_dtype, const void* x, const void* w1, const void* b1, const void* w2,
-                const void* b2, void* y, void* stream) {
-  if (!x || !w1 || !w2 || !y) return M2D_ERR_NULL_POINTER;
+int m2d_mlp_fwd(int64_t P, int C, int hidden, int weight_dtype, const void* x, const void* ln_weight, const void* ln_bias, float eps,
+                const void* w1, const void* b1, const void* w2, const void* b2, void* y, void* stream) {
+  if (!x || !w1 || !w2 || !y || (ln_weight != nullptr) != (ln_bias != nullptr)) return M2D_ERR_NULL_POINTER;
   if (P < 1 || C < 1 || hidden < 1) return M2D_ERR_BAD_SHAPE;
   if (weight_dtype != M2D_F32 && weight_dtype != M2D_BF16) return M2D_ERR_UNSUPPORTED;
   if ((C != 32 && C != 64) || hidden != 4 * C) return M2D_ERR_UNSUPPORTED;
   if ((P + 63) / 64 >= ((int64_t)1 << 31)) return M2D_ERR_UNSUPPORTED;
-  if (misaligned(x, 16) || misaligned(y, 16) || misaligned(w1, 16) || misaligned(w2, 16) || (b1 && misaligned(b1, 4)) || (b2 && misaligned(b2, 4)))
+  if (misaligned(x, 16) || misaligned(y, 16) || misaligned(w1, 16) || misaligned(w2, 16) || (b1 && misaligned(b1, 4)) || (b2 && misaligned(b2, 4)) ||
+      (ln_weight && (misaligned(ln_weight, 4) || misaligned(ln_bias, 4))))
     return M2D_ERR_MISALIGNED;
   MlpArgs a = {};
+  a.ln_w = ln_weight; a.ln_b = ln_bias; a.ln_eps = eps;
   a.x = x; a.w1 = w1; a.b1 = b1; a.w2 = w2; a.b2 = b2; a.y = y; a.P = P; a.wbf16 = weight_dtype == M2D_BF16;
   a.ntiles = (int)((P + 63) / 64);
   const size_t lds = C == 64 ? mlp_lds_bytes<2>() : mlp_lds_bytes<1>();
@@ -1096,30 +1156,35 @@ int m2d_rope_attention_fwd(int B, int L, int heads, int head_dim, int weight_dty
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
-int m2d_linear_fwd(int64_t P, int K, int N, int weight_dtype, const void* x, const void* weight, const void* bias,
-                   int pre_act, const void* pre_scale, const void* pre_bias, int post_act, const void* post_scale,
-                   const void* post_bias, void* y, void* stream) {
+static int run_linear(int64_t P, int K, int N, int weight_dtype, const void* x, const void* weight, const void* bias,
+                      int pre_act, const void* pre_scale, const void* pre_bias, int post_act, const void* post_scale,
+                      const void* post_bias, void* y, void* stream, const void* ln_w, const void* ln_b, float ln_eps) {
   if (!x || !weight || !y) return M2D_ERR_NULL_POINTER;
+  const bool ln = pre_act == kActLayerNorm;
+  if (ln && (!ln_w || !ln_b)) return M2D_ERR_NULL_POINTER;
   if ((pre_act == kActStarRelu && (!pre_scale || !pre_bias)) || (post_act == kActStarRelu && (!post_scale || !post_bias)))
     return M2D_ERR_NULL_POINTER;
   if (P < 1 || K < 1 || N < 1) return M2D_ERR_BAD_SHAPE;
   if (weight_dtype != M2D_F32 && weight_dtype != M2D_BF16) return M2D_ERR_UNSUPPORTED;
-  if (pre_act < kActNone || pre_act > kActStarRelu || post_act < kActNone || post_act > kActStarRelu) return M2D_ERR_UNSUPPORTED;
+  if (pre_act < kActNone || pre_act > kActLayerNorm || post_act < kActNone || post_act > kActStarRelu) return M2D_ERR_UNSUPPORTED;
   if (K % 32 != 0 || K > 32 * kLinMaxKC || N % 16 != 0) return M2D_ERR_UNSUPPORTED;
+  if (ln && K > 128) return M2D_ERR_UNSUPPORTED;      // the normalised rows live in registers next to the operands
   // Slices of the outputs, so that a workgroup's share of the weights leaves room for four workgroups on a
   // compute unit (each slice reads the rows of x again; they are the smaller side where N is large).
   int nsplit = 1;
-  while (linear_lds_bytes(K, N / nsplit) > 40 * 1024 && (N / nsplit) % 32 == 0 && N / nsplit > 64) nsplit *= 2;
+  while (linear_lds_bytes(K, N / nsplit, ln) > 40 * 1024 && (N / nsplit) % 32 == 0 && N / nsplit > 64) nsplit *= 2;
   const int Ns = N / nsplit;
-  if (linear_lds_bytes(K, Ns) > kLinMaxLds) return M2D_ERR_UNSUPPORTED;
+  if (linear_lds_bytes(K, Ns, ln) > kLinMaxLds) return M2D_ERR_UNSUPPORTED;
   if ((P + 63) / 64 >= ((int64_t)1 << 31)) return M2D_ERR_UNSUPPORTED;
   if (misaligned(x, 16) || misaligned(y, 16) || misaligned(weight, 16) || (bias && misaligned(bias, 4))) return M2D_ERR_MISALIGNED;
+  if (ln && (misaligned(ln_w, 4) || misaligned(ln_b, 4))) return M2D_ERR_MISALIGNED;
   LinArgs a = {};
+  a.ln_w = ln_w; a.ln_b = ln_b; a.ln_eps = ln_eps;
   a.x = x; a.w = weight; a.bias = bias; a.y = y; a.P = P; a.K = K; a.N = N; a.wbf16 = weight_dtype == M2D_BF16;
   a.pre = pre_act; a.post = post_act; a.pre_s = pre_scale; a.pre_b = pre_bias; a.post_s = post_scale; a.post_b = post_bias;
   a.ntiles = (int)((P + 63) / 64);
   a.nsplit = nsplit; a.Ns = Ns;
-  const size_t lds = linear_lds_bytes(K, Ns);
+  const size_t lds = linear_lds_bytes(K, Ns, ln);
   if (lds > 64 * 1024 && !allow_big_lds()) return M2D_ERR_HIP;
   // persistent: the weights are loaded into LDS once per workgroup; as many workgroups as fit the device at once
   int per_cu = (int)(160 * 1024 / lds);
@@ -1135,6 +1200,21 @@ int m2d_linear_fwd(int64_t P, int K, int N, int weight_dtype, const void* x, con
   else if (K <= 256) hipLaunchKernelGGL(m2d_linear_kernel<8>, g, t, lds, st, a);
   else hipLaunchKernelGGL(m2d_linear_kernel<16>, g, t, lds, st, a);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+}
+
+int m2d_linear_fwd(int64_t P, int K, int N, int weight_dtype, const void* x, const void* weight, const void* bias,
+                   int pre_act, const void* pre_scale, const void* pre_bias, int post_act, const void* post_scale,
+                   const void* post_bias, void* y, void* stream) {
+  if (pre_act == kActLayerNorm) return M2D_ERR_UNSUPPORTED;      // that one has an entry point of its own
+  return run_linear(P, K, N, weight_dtype, x, weight, bias, pre_act, pre_scale, pre_bias, post_act, post_scale, post_bias, y, stream,
+                    nullptr, nullptr, 0.f);
+}
+
+int m2d_layernorm_linear_fwd(int64_t P, int K, int N, int weight_dtype, const void* x, const void* ln_weight, const void* ln_bias,
+                             float eps, const void* weight, const void* bias, int post_act, const void* post_scale,
+                             const void* post_bias, void* y, void* stream) {
+  return run_linear(P, K, N, weight_dtype, x, weight, bias, kActLayerNorm, nullptr, nullptr, post_act, post_scale, post_bias, y, stream,
+                    ln_weight, ln_bias, eps);
 }
 
 }  // extern "C"

@@ -46,6 +46,7 @@ rope_qknorm_fwd_op = torch.ops.m2dscan.rope_qknorm_fwd
 rope_attention_fwd_op = torch.ops.m2dscan.rope_attention_fwd
 mlp_fwd_op = torch.ops.m2dscan.mlp_fwd
 linear_act_fwd_op = torch.ops.m2dscan.linear_act_fwd
+layernorm_linear_act_fwd_op = torch.ops.m2dscan.layernorm_linear_act_fwd
 
 # Keep the forward's anti-diagonal checkpoints for the backward (faster backward, more saved
 # memory) or rebuild them inside the backward (nothing saved beyond the inputs, like the
@@ -123,8 +124,13 @@ def _linear_act_fwd_fake(x, weight, bias, pre, pre_scale, pre_bias, post, post_s
     return x.new_empty((*x.shape[:-1], weight.shape[0]))
 
 
+@torch.library.register_fake("m2dscan::layernorm_linear_act_fwd")
+def _layernorm_linear_act_fwd_fake(x, ln_weight, ln_bias, eps, weight, bias, post, post_scale, post_bias):
+    return x.new_empty((*x.shape[:-1], weight.shape[0]))
+
+
 @torch.library.register_fake("m2dscan::mlp_fwd")
-def _mlp_fwd_fake(x, w1, b1, w2, b2):
+def _mlp_fwd_fake(x, w1, b1, w2, b2, ln_weight=None, ln_bias=None, eps=1e-5):
     return torch.empty_like(x)
 
 

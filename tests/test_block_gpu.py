@@ -1,5 +1,5 @@
 """GPU parity of the residual-block operators (m2d_layernorm_fwd, m2d_dwconv3x3_fwd, m2d_starrelu_fwd,
-m2d_scale_residual_fwd, m2d_scale_residual_layernorm_fwd, m2d_rope_qknorm_fwd, m2d_rope_attention_fwd, m2d_linear_fwd, m2d_mlp_fwd) through the C ABI, against the stock torch operators the reference uses (nn.LayerNorm, models/mamba2d.py:220;
+m2d_scale_residual_fwd, m2d_scale_residual_layernorm_fwd, m2d_rope_qknorm_fwd, m2d_rope_attention_fwd, m2d_linear_fwd, m2d_layernorm_linear_fwd, m2d_mlp_fwd) through the C ABI, against the stock torch operators the reference uses (nn.LayerNorm, models/mamba2d.py:220;
 depthwise nn.Conv2d, models/utils.py:101) evaluated in fp64 on the CPU.  Tolerances: fp32 2e-5,
 bf16 tensors 1e-2 (max error over max value; one bf16 rounding of the result is 4e-3)."""
 import pytest
@@ -268,6 +268,61 @@ def test_fused_mlp_matches_torch(cabi, shape, bias, wdtype):
     err = so.rel_err(got.float().cpu(), want)
     say(f"  rel err {err:.3e}")
     assert err < TOL[torch.bfloat16]
+
+
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16], ids=["w_f32", "w_bf16"])
+@pytest.mark.parametrize("shape", [(2 * 9 * 12, 64, 128), (1000, 128, 256), (333, 128, 512), (77, 64, 64), (5, 32, 16), (70000, 64, 128)],
+                         ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("post", [0, 1, 2], ids=lambda a: f"post{a}")
+def test_layernorm_in_front_of_a_linear_layer(cabi, shape, post, wdtype):
+    """m2d_layernorm_linear_fwd against the two kernels it replaces (their results agree up to the order of the sums
+    inside the norm, i.e. an occasional last bf16 bit of a normalised value) and against fp64."""
+    P, K, N = shape
+    say(f"\ncase layernorm+linear {shape} post={post} {wdtype}")
+    g = torch.Generator().manual_seed(P + K + N)
+    x = (torch.randn(P, K, generator=g) * 2 + 0.5).bfloat16().cuda()
+    lw = (torch.rand(K, generator=g) + 0.5).to(wdtype).cuda()
+    lb = (torch.randn(K, generator=g) * 0.3).to(wdtype).cuda()
+    w = (torch.randn(N, K, generator=g) / K ** 0.5).to(wdtype).cuda()
+    b = (torch.randn(N, generator=g) * 0.5).to(wdtype).cuda()
+    star = (torch.tensor([0.8944]).to(wdtype).cuda(), torch.tensor([-0.4472]).to(wdtype).cuda())
+    got = cabi.linear_fwd(x, w, b, post=post, post_params=star if post == 2 else None, ln=(lw, lb, 1e-5))
+    two = cabi.linear_fwd(cabi.layernorm_fwd(x, lw, lb, 1e-5), w, b, post=post, post_params=star if post == 2 else None)
+    n64 = torch.nn.functional.layer_norm(x.double().cpu(), (K,), lw.double().cpu(), lb.double().cpu(), 1e-5).bfloat16().double()
+    want = n64 @ w.bfloat16().double().cpu().T + b.double().cpu()
+    want = torch.nn.functional.gelu(want) if post == 1 else (star[0].double().cpu() * torch.relu(want) ** 2 + star[1].double().cpu()) if post == 2 else want
+    torch.cuda.synchronize()
+    assert got.shape == (P, N) and got.dtype == torch.bfloat16
+    assert so.rel_err(got.float().cpu(), want) < TOL[torch.bfloat16]
+    assert so.rel_err(got.float().cpu(), two.double().cpu()) < TOL[torch.bfloat16]
+
+
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16], ids=["w_f32", "w_bf16"])
+@pytest.mark.parametrize("shape", [(1000, 64), (333, 32), (70000, 64)], ids=lambda s: "x".join(map(str, s)))
+def test_layernorm_in_front_of_the_fused_mlp(cabi, shape, wdtype):
+    P, C = shape
+    say(f"\ncase layernorm+mlp {shape} {wdtype}")
+    g = torch.Generator().manual_seed(P + C + 1)
+    x = (torch.randn(P, C, generator=g) * 2 + 0.5).bfloat16().cuda()
+    lw = (torch.rand(C, generator=g) + 0.5).to(wdtype).cuda()
+    lb = (torch.randn(C, generator=g) * 0.3).to(wdtype).cuda()
+    w1 = (torch.randn(4 * C, C, generator=g) / C ** 0.5).to(wdtype).cuda()
+    w2 = (torch.randn(C, 4 * C, generator=g) / (4 * C) ** 0.5).to(wdtype).cuda()
+    b1 = (torch.randn(4 * C, generator=g) * 0.5).to(wdtype).cuda()
+    b2 = (torch.randn(C, generator=g) * 0.5).to(wdtype).cuda()
+    got = cabi.mlp_fwd(x, w1, b1, w2, b2, lw, lb, 1e-5)
+    two = cabi.mlp_fwd(cabi.layernorm_fwd(x, lw, lb, 1e-5), w1, b1, w2, b2)
+    torch.cuda.synchronize()
+    assert got.shape == x.shape and got.dtype == torch.bfloat16
+    assert so.rel_err(got.float().cpu(), two.double().cpu()) < TOL[torch.bfloat16]
+
+
+def test_layernorm_in_front_of_a_wide_layer_is_refused(cabi):
+    x = torch.zeros(8, 256, device="cuda", dtype=torch.bfloat16)
+    w = torch.ones(256, device="cuda")
+    with pytest.raises(cabi.M2DError) as e:
+        cabi.linear_fwd(x, torch.zeros(64, 256, device="cuda"), ln=(w, w, 1e-5))
+    assert e.value.status == 3      # M2D_ERR_UNSUPPORTED: more than 128 inputs
 
 
 def test_fused_mlp_limits_are_reported(cabi):
