@@ -1351,6 +1351,19 @@ hipEvent_t g_ev[2][2] = {{nullptr, nullptr}, {nullptr, nullptr}};
 
 inline size_t align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
 
+// Dynamic LDS of a workgroup: the forward's two staging buffers, the backward's exchange buffers, its
+// copy of A and two staging buffers.  A compute unit has 160 KB.
+constexpr size_t kLdsPerWorkgroup = 160 * 1024;
+template <typename T, int EC>
+constexpr size_t fwd_lds_bytes() { return 256 + 2 * (size_t)Stage<T, 3, kFwdWaves * 4 * EC, false, true>::kBytes; }
+template <typename T>
+constexpr size_t bwd_lds_bytes() {
+  return sizeof(float4) * kBwdWaves * 3 * 64 + sizeof(float) * kBwdWaves * 4 * 2 * kN + 256 +
+         2 * (size_t)Stage<T, 4, kBwdWaves * 4, true, false>::kBytes;
+}
+static_assert(fwd_lds_bytes<float, 1>() <= kLdsPerWorkgroup && fwd_lds_bytes<bf16_t, 1>() <= kLdsPerWorkgroup, "forward staging must fit the LDS");
+static_assert(bwd_lds_bytes<float>() <= kLdsPerWorkgroup && bwd_lds_bytes<bf16_t>() <= kLdsPerWorkgroup, "backward staging must fit the LDS");
+
 struct Geometry {
   int HB, hb_shift, CS, nbands, nblk;
   int S, T_total, rows_last;         // stream stride, total steps, rows of the last band
@@ -1436,8 +1449,11 @@ Geometry make_geometry(const m2d_desc* d) {
     g.nblk = g.nbands * g.nbb;
     g.nlaunch = kSliceLag * (g.nbands - 1) + (g.nbb + kSliceQ - 1) / kSliceQ;
   }
-  // forward: two channels per lane when that still yields enough waves to fill the device
-  const bool ec2 = (d->E % 2 == 0) && ((int64_t)B * ((d->E + kFwdWaves * g.CS * 2 - 1) / (kFwdWaves * g.CS * 2)) >= 256);
+  // forward: two channels per lane when that still yields enough waves to fill the device and the
+  // two staging buffers of such a workgroup fit the LDS (bf16 operands: 112 KB; fp32 ones do not)
+  const size_t lds_ec2 = d->dtype == M2D_BF16 ? fwd_lds_bytes<bf16_t, 2>() : fwd_lds_bytes<float, 2>();
+  const bool ec2 = (d->E % 2 == 0) && lds_ec2 <= kLdsPerWorkgroup &&
+                   ((int64_t)B * ((d->E + kFwdWaves * g.CS * 2 - 1) / (kFwdWaves * g.CS * 2)) >= 256);
   g.fwd_ec = ec2 ? 2 : 1;
   g.fwd_bpb = (d->E + kFwdWaves * g.CS * g.fwd_ec - 1) / (kFwdWaves * g.CS * g.fwd_ec);
   g.fwd_wpb = g.fwd_bpb * kFwdWaves;
@@ -1536,8 +1552,8 @@ int stage_bc(ScanParams& sp, const m2d_desc* d, const void* BT, const void* BL, 
 
 template <typename T, int EC, bool CK, bool WY, bool SX, int MODE>
 int launch_fwd_as(const ScanParams& sp, hipStream_t st) {
-  using SG = Stage<T, 3, kFwdWaves * 4 * EC, false, true>;
-  const size_t lds = 256 + 2 * (size_t)SG::kBytes;
+  constexpr size_t lds = fwd_lds_bytes<T, EC>();
+  if (lds > kLdsPerWorkgroup) return M2D_ERR_UNSUPPORTED;   // (make_geometry never picks such a layout)
   static std::atomic<uint64_t> seen{0};
   if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_fwd_kernel<T, EC, CK, WY, SX, MODE>), lds, seen)) return M2D_ERR_HIP;
   hipLaunchKernelGGL((m2d_fwd_kernel<T, EC, CK, WY, SX, MODE>), dim3((unsigned)sp.nwg), dim3(kFwdWaves * 64), lds, st, sp);
@@ -1606,8 +1622,7 @@ int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
 
 template <typename T, bool SX, int MODE>
 int launch_bwd(const ScanParams& sp, hipStream_t st) {
-  using SG = Stage<T, 4, kBwdWaves * 4, true, false>;
-  const size_t lds = sizeof(float4) * kBwdWaves * 3 * 64 + sizeof(float) * kBwdWaves * 4 * 2 * kN + 256 + 2 * (size_t)SG::kBytes;
+  constexpr size_t lds = bwd_lds_bytes<T>();
   static std::atomic<uint64_t> seen{0};
   if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_bwd_kernel<T, SX, MODE>), lds, seen)) return M2D_ERR_HIP;
   hipLaunchKernelGGL((m2d_bwd_kernel<T, SX, MODE>), dim3((unsigned)sp.nwg), dim3(kBwdWaves * 64), lds, st, sp);
