@@ -188,6 +188,33 @@ def _as_f32(t):
     return f
 
 
+# The kernels hold the 16 states of a cell in the registers of one lane (d_state of every
+# published Mamba2D configuration, models/mamba2d.py:23).  The recurrence is independent per state
+# and y is a sum over states (wf_cuda.cu:40-69, wavefront_cuda.py:156), so any other d_state is the
+# sum of scans over groups of 16 states, the last group padded with states whose B and C are zero
+# (they stay at zero and receive zero gradients); the skip term x*D goes with the first group.
+STATES_PER_CALL = 16
+
+
+def _scan_in_state_groups(x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip):
+    """wf_cuda_fn_pr for d_state != 16, composed of 16-state scans by differentiable tensor
+    operators (pad, slice, add), so the nine gradients follow by autograd."""
+    N = AT.shape[1]
+    if N < 1:
+        raise ValueError(f"d_state must be positive, got {N}")
+    pad = (-N) % STATES_PER_CALL
+    if pad:
+        AT, AL = F.pad(AT, (0, pad), value=-1.0), F.pad(AL, (0, pad), value=-1.0)
+        BT, BL, C = F.pad(BT, (0, pad)), F.pad(BL, (0, pad)), F.pad(C, (0, pad))
+    y = None
+    for n0 in range(0, N + pad, STATES_PER_CALL):
+        sl = slice(n0, n0 + STATES_PER_CALL)
+        part = wf_cuda_fn_pr.apply(x, deltaT, deltaL, AT[:, sl], AL[:, sl], BT[..., sl], BL[..., sl], C[..., sl],
+                                   D if n0 == 0 else torch.zeros_like(D), flip)
+        y = part if y is None else y + part
+    return y
+
+
 class wf_cuda_fn_pr(torch.autograd.Function):
     """Scan + output projection on precomputed parameters (reference ``wavefront_cuda.py:146-196``).
 
@@ -200,6 +227,8 @@ class wf_cuda_fn_pr(torch.autograd.Function):
     def apply(cls, x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip=False):
         # Whether autograd records the call is only known out here: forward() always runs with grad
         # mode off, and needs_input_grad is also set for parameters under torch.no_grad().
+        if AT.shape[1] != STATES_PER_CALL:
+            return _scan_in_state_groups(x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip)
         return super().apply(x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip, torch.is_grad_enabled())
 
     @staticmethod
@@ -227,8 +256,11 @@ class wf_cuda_fn_fr(torch.autograd.Function):
         with torch.no_grad():
             deltaT, deltaL, AT, AL, BT, BL, C = proj_params(
                 x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b)
-            y, _ = scan_fwd_op(_c(x), _c(deltaT), _c(deltaL), _c(AT), _c(AL), _c(BT), _c(BL), _c(C), _c(D),
-                               False, bool(flip))
+            if AT.shape[1] != STATES_PER_CALL:
+                y = _scan_in_state_groups(x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip)
+            else:
+                y, _ = scan_fwd_op(_c(x), _c(deltaT), _c(deltaL), _c(AT), _c(AL), _c(BT), _c(BL), _c(C), _c(D),
+                                   False, bool(flip))
         ctx.save_for_backward(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D)
         ctx.flip = bool(flip)
         return y
@@ -237,6 +269,11 @@ class wf_cuda_fn_fr(torch.autograd.Function):
     def backward(ctx, grad_output):
         x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D = ctx.saved_tensors
         dy = _c(grad_output.to(x.dtype))
+        if AT_log.shape[1] != STATES_PER_CALL:   # projections and the scans of the state groups again, under autograd
+            with torch.enable_grad():
+                leaves = [t.detach().requires_grad_(True) for t in ctx.saved_tensors]
+                y = _scan_in_state_groups(leaves[0], *proj_params(*leaves[:8]), leaves[8], ctx.flip)
+            return (*torch.autograd.grad(y, leaves, dy), None)
         with torch.enable_grad():
             leaves = [t.detach().requires_grad_(True) for t in
                       (x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b)]
@@ -253,7 +290,7 @@ class wf_cuda_fn_fr(torch.autograd.Function):
 
 def _proj_kernels_cover(x, AT_log, dt_projT_w) -> bool:
     """Shapes the projection kernels are built for; anything else takes the stock operators."""
-    return AT_log.shape[1] == 16 and dt_projT_w.shape[1] <= 32 and x.shape[-1] <= 4096
+    return AT_log.shape[1] == STATES_PER_CALL and dt_projT_w.shape[1] <= 32 and x.shape[-1] <= 4096
 
 
 class wf_cuda_fn_proj(torch.autograd.Function):

@@ -91,6 +91,48 @@ def test_entry_point_matches_oracle_fp32(wf, recomp, projections):
         assert so.rel_err(g.cpu(), gr) < 2e-4, name
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 2e-2)], ids=["f32", "bf16"])
+@pytest.mark.parametrize("N", [1, 8, 24, 32])
+def test_fn_pr_other_state_counts(wf, cscan, N, dtype, tol):
+    """d_state other than 16 (a constructor argument of the reference's block, models/mamba2d.py:23):
+    the operator splits the states into groups of 16, padding the last one."""
+    say(f"\ncase fn_pr N={N} {dtype}")
+    inp = so.make_inputs(3, 9, 17, 8, N, seed=21, dtype=dtype)
+    leaves = [inp[k].cuda().requires_grad_(True) for k in so.INPUT_NAMES]
+    y = wf.wf_cuda_fn_pr.apply(*leaves)
+    grads = torch.autograd.grad(y, leaves, inp["dy"].cuda())
+    ref_in = [inp[k].double() for k in so.INPUT_NAMES]
+    assert y.dtype == dtype and so.rel_err(y.float().cpu(), cscan.forward(*ref_in)) < tol
+    g_ref = cscan.backward(*ref_in, inp["dy"].double())
+    for k, g, leaf in zip(so.CScan.GRADS, grads, leaves):
+        assert g.dtype == leaf.dtype and g.shape == leaf.shape
+        assert so.rel_err(g.float().cpu(), g_ref[k]) < tol, k
+
+
+@pytest.mark.parametrize("recomp", ["partial", "full"])
+@pytest.mark.parametrize("N", [8, 20])
+def test_entry_point_other_state_counts_fp32(wf, recomp, N):
+    say(f"\ncase entry_point {recomp} N={N}")
+    B, H, W, E = 2, 16, 7, 32
+    R = math.ceil(E / 16)
+    p = make_block_params(E, N, R, 7, "cuda")
+    x = torch.randn(B, H, W, E, generator=torch.Generator().manual_seed(8)).cuda()
+    dy = torch.randn(B, H, W, E, generator=torch.Generator().manual_seed(9)).cuda()
+    leaves = [x.clone().requires_grad_(True)] + [p[k].clone().requires_grad_(True) for k in ORDER]
+    y = wf.wavefront_scan_cuda(*leaves, recomp=recomp, flip=(N == 20))
+    grads = torch.autograd.grad(y, leaves, dy)
+    ref_leaves = [t.detach().double().cpu().requires_grad_(True) for t in leaves]
+    xr, dyr = ref_leaves[0], dy.double().cpu()
+    if N == 20:   # bottom-right scan = flipped input, flipped output (models/mamba2d.py:163-173)
+        y_ref = torch.flip(so.wavefront_scan_ref(torch.flip(xr, (1, 2)), *ref_leaves[1:]), (1, 2))
+    else:
+        y_ref = so.wavefront_scan_ref(*ref_leaves)
+    g_ref = torch.autograd.grad(y_ref, ref_leaves, dyr)
+    assert so.rel_err(y.cpu(), y_ref.detach()) < 1e-4
+    for name, g, gr in zip(("x",) + ORDER, grads, g_ref):
+        assert g.shape == gr.shape and so.rel_err(g.cpu(), gr) < 2e-4, name
+
+
 def test_partial_and_full_agree_bf16(wf, projections):
     """The two recompute modes are the same function of the nine raw inputs."""
     say(f"\ncase partial_vs_full bf16 own_projections={projections}")
