@@ -178,7 +178,9 @@ std::vector<Tensor> proj_fwd(const Tensor& x, const Tensor& Wx, const Tensor& wT
   return o;
 }
 
-std::vector<Tensor> proj_bwd(const Tensor& x, const Tensor& low, const Tensor& dT, const Tensor& dL, const Tensor& Wx,
+// Returns a tuple, not a list: the operator writes into dx, and torch.compile can only functionalise a
+// mutating custom operator whose results are plain tensors.
+std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor> proj_bwd(const Tensor& x, const Tensor& low, const Tensor& dT, const Tensor& dL, const Tensor& Wx,
                              const Tensor& wT, const Tensor& wL, const Tensor& ddT, const Tensor& ddL, const Tensor& dBT,
                              const Tensor& dBL, const Tensor& dC, Tensor dx, bool round_weights, bool dpre) {
   TORCH_CHECK(dBT.dim() == 4 && wT.dim() == 2, "m2dscan: d_BT must be (B,H,W,N) and dt_projT_w (E, dt_rank)");
@@ -210,7 +212,7 @@ std::vector<Tensor> proj_bwd(const Tensor& x, const Tensor& low, const Tensor& d
                      dBT.data_ptr(), dBL.data_ptr(), dC.data_ptr(), dx.data_ptr(), g[0].data_ptr<float>(),
                      g[1].data_ptr<float>(), g[2].data_ptr<float>(), g[3].data_ptr<float>(), g[4].data_ptr<float>(),
                      ws.data_ptr(), static_cast<size_t>(ws.numel()), st));
-  return g;
+  return std::make_tuple(g[0], g[1], g[2], g[3], g[4]);
 }
 
 // ---- operators of the residual block (inference forward)
@@ -458,7 +460,7 @@ TORCH_LIBRARY(m2dscan, m) {
         "int d_state, bool round_weights, bool packed_bc=False) -> Tensor[]");
   m.def("proj_bwd(Tensor x, Tensor lowrank, Tensor deltaT, Tensor deltaL, Tensor x_proj_w, Tensor dt_projT_w, "
         "Tensor dt_projL_w, Tensor d_deltaT, Tensor d_deltaL, Tensor d_BT, Tensor d_BL, Tensor d_C, Tensor(a!) dx, "
-        "bool round_weights, bool dpre=False) -> Tensor[]");
+        "bool round_weights, bool dpre=False) -> (Tensor, Tensor, Tensor, Tensor, Tensor)");
   m.def("layernorm_fwd(Tensor x, Tensor weight, Tensor bias, float eps) -> Tensor");
   m.def("dwconv3x3_fwd(Tensor x, Tensor weight) -> Tensor");
   m.def("starrelu_fwd(Tensor x, Tensor scale, Tensor bias) -> Tensor");

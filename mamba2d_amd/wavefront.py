@@ -91,7 +91,7 @@ def _proj_fwd_fake(x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, 
 def _proj_bwd_fake(x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w, dt_projL_w, d_deltaT, d_deltaL, d_BT, d_BL, d_C, dx,
                    round_weights, dpre=False):
     b = dt_projT_w.new_empty((x.shape[-1],))
-    return [torch.empty_like(x_proj_w), torch.empty_like(dt_projT_w), b, torch.empty_like(dt_projL_w), torch.empty_like(b)]
+    return torch.empty_like(x_proj_w), torch.empty_like(dt_projT_w), b, torch.empty_like(dt_projL_w), torch.empty_like(b)
 
 
 @torch.library.register_fake("m2dscan::layernorm_fwd")
@@ -167,6 +167,8 @@ def _c(t):
     """Contiguous and 16-byte aligned (a contiguous view into a larger buffer may start anywhere)."""
     if not t.is_contiguous():
         return t.contiguous()
+    if torch.compiler.is_compiling():   # addresses are not known while tracing; the shim rejects a misaligned one
+        return t
     return t if t.data_ptr() % 16 == 0 else t.clone()
 
 
@@ -179,6 +181,8 @@ def _as_f32(t):
     spend eight small kernels per scan on casting weights that did not change."""
     if t.dtype == torch.float32:
         return _c(t)
+    if torch.compiler.is_compiling():   # a traced graph holds the cast itself
+        return t.detach().float().contiguous()
     key = id(t)
     hit = _F32_COPIES.get(key)
     if hit is not None and hit[0]() is t and hit[1] == t._version and hit[2] == t.data_ptr():
@@ -192,27 +196,72 @@ def _as_f32(t):
 # published Mamba2D configuration, models/mamba2d.py:23).  The recurrence is independent per state
 # and y is a sum over states (wf_cuda.cu:40-69, wavefront_cuda.py:156), so any other d_state is the
 # sum of scans over groups of 16 states, the last group padded with states whose B and C are zero
-# (they stay at zero and receive zero gradients); the skip term x*D goes with the first group.
+# (they stay at zero; their gradients are dropped); the skip term x*D goes with the first group.
 STATES_PER_CALL = 16
 
 
-def _scan_in_state_groups(x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip):
-    """wf_cuda_fn_pr for d_state != 16, composed of 16-state scans by differentiable tensor
-    operators (pad, slice, add), so the nine gradients follow by autograd."""
-    N = AT.shape[1]
-    if N < 1:
-        raise ValueError(f"d_state must be positive, got {N}")
-    pad = (-N) % STATES_PER_CALL
+def _state_groups(AT, AL, BT, BL, C):
+    """(AT, AL, BT, BL, C) cut along the state axis into contiguous groups of 16, the last one padded."""
+    pad = (-AT.shape[1]) % STATES_PER_CALL
     if pad:
         AT, AL = F.pad(AT, (0, pad), value=-1.0), F.pad(AL, (0, pad), value=-1.0)
         BT, BL, C = F.pad(BT, (0, pad)), F.pad(BL, (0, pad)), F.pad(C, (0, pad))
-    y = None
-    for n0 in range(0, N + pad, STATES_PER_CALL):
-        sl = slice(n0, n0 + STATES_PER_CALL)
-        part = wf_cuda_fn_pr.apply(x, deltaT, deltaL, AT[:, sl], AL[:, sl], BT[..., sl], BL[..., sl], C[..., sl],
-                                   D if n0 == 0 else torch.zeros_like(D), flip)
-        y = part if y is None else y + part
-    return y
+    return [tuple(t[..., n0:n0 + STATES_PER_CALL].contiguous() for t in (AT, AL, BT, BL, C))
+            for n0 in range(0, AT.shape[1], STATES_PER_CALL)]
+
+
+def _grouped_scan_fwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, keep, flip):
+    """scan_fwd for d_state != 16: y summed over the groups in fp32; one checkpoint buffer per group."""
+    if AT.shape[1] < 1:
+        raise ValueError(f"d_state must be positive, got {AT.shape[1]}")
+    y, cks, no_skip = None, [], torch.zeros_like(D)
+    for gi, grp in enumerate(_state_groups(AT, AL, BT, BL, C)):
+        part, ck = scan_fwd_op(x, deltaT, deltaL, *grp, D if gi == 0 else no_skip, keep, flip)
+        y = part.float() if y is None else y + part.float()
+        cks.append(ck)
+    return y.to(x.dtype), cks
+
+
+def _grouped_scan_bwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, cks, flip):
+    """scan_bwd for d_state != 16: gradients of x and the step sizes summed over the groups in fp32,
+    those of A, B, C put together along the state axis (padding dropped); d_D comes with the first group."""
+    N = AT.shape[1]
+    sums, per_state, d_D, no_skip = None, [], None, torch.zeros_like(D)
+    for gi, grp in enumerate(_state_groups(AT, AL, BT, BL, C)):
+        g = scan_bwd_op(x, deltaT, deltaL, *grp, D if gi == 0 else no_skip, dy, cks[gi], flip)
+        if gi == 0:
+            sums, d_D = [t.float() for t in g[:3]], g[8]
+        else:
+            sums = [a + t.float() for a, t in zip(sums, g[:3])]
+        per_state.append(g[3:8])
+    joined = [torch.cat([grp[k] for grp in per_state], dim=-1)[..., :N].contiguous() for k in range(5)]
+    return (*[t.to(x.dtype) for t in sums], *joined, d_D)
+
+
+class _ScanOnParams(torch.autograd.Function):
+    """The Function behind ``wf_cuda_fn_pr``: 16 states, and told by its caller whether autograd
+    records the call (``recording``)."""
+
+    @staticmethod
+    def forward(ctx, x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip=False, recording=True):
+        args = [_c(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D)]
+        keep = SAVE_CHECKPOINTS and recording and any(ctx.needs_input_grad)
+        ctx.flip = bool(flip)
+        if AT.shape[1] != STATES_PER_CALL:
+            y, cks = _grouped_scan_fwd(*args, keep, ctx.flip)
+            ctx.save_for_backward(*args, *cks)
+            return y
+        y, ck = scan_fwd_op(*args, keep, ctx.flip)
+        ctx.save_for_backward(*args, ck)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        args, cks = ctx.saved_tensors[:9], ctx.saved_tensors[9:]
+        dy = _c(grad_output.to(args[0].dtype))
+        if args[3].shape[1] != STATES_PER_CALL:
+            return (*_grouped_scan_bwd(*args, dy, cks, ctx.flip), None, None)
+        return (*scan_bwd_op(*args, dy, cks[0], ctx.flip), None, None)
 
 
 class wf_cuda_fn_pr(torch.autograd.Function):
@@ -221,30 +270,21 @@ class wf_cuda_fn_pr(torch.autograd.Function):
     ``apply(x, deltaT, deltaL, AT, AL, BT, BL, C, D[, flip]) -> y``; backward returns the nine
     gradients in input order.  ``flip=True`` (not in the reference) scans from the bottom-right
     corner, which equals flipping every spatial tensor before and y after
-    (``models/mamba2d.py:163-173``) without the copies."""
+    (``models/mamba2d.py:163-173``) without the copies.
+
+    ``apply`` hands the call to ``_ScanOnParams`` (the node that shows up as ``y.grad_fn``) together
+    with the grad mode of the caller: forward() always runs with grad mode off, and
+    needs_input_grad is also set for parameters under torch.no_grad(), so whether autograd records
+    the call is only known out here.  Written without ``super()``, and with forward and backward
+    that are complete without it (torch.compile may trace either), so that a compiled caller can
+    trace through the scan as it can through the reference's operator (``wavefront_cuda.py:25-57``)."""
+
+    forward = staticmethod(_ScanOnParams.forward)
+    backward = staticmethod(_ScanOnParams.backward)
 
     @classmethod
     def apply(cls, x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip=False):
-        # Whether autograd records the call is only known out here: forward() always runs with grad
-        # mode off, and needs_input_grad is also set for parameters under torch.no_grad().
-        if AT.shape[1] != STATES_PER_CALL:
-            return _scan_in_state_groups(x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip)
-        return super().apply(x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip, torch.is_grad_enabled())
-
-    @staticmethod
-    def forward(ctx, x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip=False, recording=True):
-        args = [_c(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D)]
-        keep = SAVE_CHECKPOINTS and recording and any(ctx.needs_input_grad)
-        y, ck = scan_fwd_op(*args, keep, bool(flip))
-        ctx.save_for_backward(*args, ck)
-        ctx.flip = bool(flip)
-        return y
-
-    @staticmethod
-    def backward(ctx, grad_output):
-        *args, ck = ctx.saved_tensors
-        dy = _c(grad_output.to(args[0].dtype))
-        return (*scan_bwd_op(*args, dy, ck, ctx.flip), None, None)
+        return _ScanOnParams.apply(x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip, torch.is_grad_enabled())
 
 
 class wf_cuda_fn_fr(torch.autograd.Function):
@@ -257,7 +297,7 @@ class wf_cuda_fn_fr(torch.autograd.Function):
             deltaT, deltaL, AT, AL, BT, BL, C = proj_params(
                 x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b)
             if AT.shape[1] != STATES_PER_CALL:
-                y = _scan_in_state_groups(x, deltaT, deltaL, AT, AL, BT, BL, C, D, flip)
+                y, _ = _grouped_scan_fwd(*[_c(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D)], False, bool(flip))
             else:
                 y, _ = scan_fwd_op(_c(x), _c(deltaT), _c(deltaL), _c(AT), _c(AL), _c(BT), _c(BL), _c(C), _c(D),
                                    False, bool(flip))
@@ -269,19 +309,19 @@ class wf_cuda_fn_fr(torch.autograd.Function):
     def backward(ctx, grad_output):
         x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D = ctx.saved_tensors
         dy = _c(grad_output.to(x.dtype))
-        if AT_log.shape[1] != STATES_PER_CALL:   # projections and the scans of the state groups again, under autograd
-            with torch.enable_grad():
-                leaves = [t.detach().requires_grad_(True) for t in ctx.saved_tensors]
-                y = _scan_in_state_groups(leaves[0], *proj_params(*leaves[:8]), leaves[8], ctx.flip)
-            return (*torch.autograd.grad(y, leaves, dy), None)
         with torch.enable_grad():
             leaves = [t.detach().requires_grad_(True) for t in
                       (x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b)]
             deltaT, deltaL, AT, AL, BT, BL, C = proj_params(*leaves)
         det = [_c(t.detach()) for t in (deltaT, deltaL, AT, AL, BT, BL, C)]
         none = x.new_empty((1,), dtype=torch.uint8)
-        d_x_scan, d_dT, d_dL, d_AT, d_AL, d_BT, d_BL, d_C, d_D = scan_bwd_op(
-            _c(x), det[0], det[1], det[2], det[3], det[4], det[5], det[6], _c(D), dy, none, ctx.flip)
+        if AT_log.shape[1] != STATES_PER_CALL:
+            n_groups = -(-AT_log.shape[1] // STATES_PER_CALL)
+            d_x_scan, d_dT, d_dL, d_AT, d_AL, d_BT, d_BL, d_C, d_D = _grouped_scan_bwd(
+                _c(x), *det, _c(D), dy, [none] * n_groups, ctx.flip)
+        else:
+            d_x_scan, d_dT, d_dL, d_AT, d_AL, d_BT, d_BL, d_C, d_D = scan_bwd_op(
+                _c(x), det[0], det[1], det[2], det[3], det[4], det[5], det[6], _c(D), dy, none, ctx.flip)
         grads = torch.autograd.grad([deltaT, deltaL, BT, BL, C, AT, AL], leaves,
                                     [d_dT, d_dL, d_BT, d_BL, d_C, d_AT, d_AL])
         d_x = d_x_scan + grads[0]   # d_x_scan already contains dy*D
@@ -300,19 +340,14 @@ class wf_cuda_fn_proj(torch.autograd.Function):
     are rounded to ``x.dtype`` (``wavefront_cuda.py:327-332``; here inside the kernels that pack
     them), then ``proj_params`` and ``wf_cuda_fn_pr`` (``:63-95``, ``:146-196``) or ``wf_cuda_fn_fr``
     (``:199-313``).  ``full=False`` keeps the projection outputs and the scan's checkpoints for the
-    backward; ``full=True`` keeps only x and the weights and rebuilds the rest in the backward."""
+    backward; ``full=True`` keeps only x and the weights and rebuilds the rest in the backward.
+    ``recording``: the caller's grad mode (see wf_cuda_fn_pr); the entry point passes it."""
 
     @staticmethod
     def _params(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D):
         """The parameters as fp32 tensors (no copy if they already are): the library itself forms
         A = -exp(A_log) and rounds everything to x.dtype as the reference's casts do."""
         return [_as_f32(t) for t in (AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D)]
-
-    @classmethod
-    def apply(cls, x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D, full=False, flip=False):
-        # see wf_cuda_fn_pr.apply
-        return super().apply(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D, full, flip,
-                             torch.is_grad_enabled())
 
     @staticmethod
     def forward(ctx, x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D,
@@ -368,7 +403,7 @@ def wavefront_scan_cuda(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_
     if FUSED_PROJECTIONS and _proj_kernels_cover(x, AT_log, dt_projT_w):
         # the casts of the weights to x.dtype happen inside (no copies of the parameters)
         return wf_cuda_fn_proj.apply(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D,
-                                     recomp == "full", flip)
+                                     recomp == "full", flip, torch.is_grad_enabled())
 
     x_proj_w = x_proj_w.to(x.dtype)
     dt_projT_w = dt_projT_w.to(x.dtype)

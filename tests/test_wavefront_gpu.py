@@ -133,6 +133,41 @@ def test_entry_point_other_state_counts_fp32(wf, recomp, N):
         assert g.shape == gr.shape and so.rel_err(g.cpu(), gr) < 2e-4, name
 
 
+@pytest.mark.parametrize("recomp", ["partial", "full"])
+@pytest.mark.parametrize("N", [16, 8])
+def test_entry_point_under_torch_compile(wf, projections, recomp, N):
+    """The reference registers its kernels as custom operators so that torch.compile traces through the
+    scan (wavefront_cuda.py:25-57).  Here: the entry point compiled with the aot_eager backend (dynamo
+    tracing, functionalisation, fake tensors of every operator; no code generation) gives the bits of
+    the eager call, forward and backward."""
+    say(f"\ncase torch.compile {recomp} N={N} own_projections={projections}")
+    import torch._dynamo
+    torch._dynamo.reset()
+    B, H, W, E = 2, 14, 20, 32
+    p = make_block_params(E, N, 2, 0, "cuda")
+    x = torch.randn(B, H, W, E, generator=torch.Generator().manual_seed(1)).cuda()
+    dy = torch.randn(B, H, W, E, generator=torch.Generator().manual_seed(2)).cuda()
+
+    def fn(*a):
+        return wf.wavefront_scan_cuda(*a, recomp=recomp) * 2.0
+
+    def run(f):
+        leaves = [x.clone().requires_grad_(True)] + [p[k].clone().requires_grad_(True) for k in ORDER]
+        y = f(*leaves)
+        return y, torch.autograd.grad(y, leaves, dy)
+
+    y0, g0 = run(fn)
+    # wf_cuda_fn_fr re-derives the projections under autograd inside its backward (requires_grad_ on
+    # detached copies, as the reference does at wavefront_cuda.py:262-296): dynamo breaks the graph there
+    # and runs that Function eagerly, so only the other paths are asked for one whole graph
+    through_fr = recomp == "full" and (N != 16 or not projections)
+    y1, g1 = run(torch.compile(fn, backend="aot_eager", fullgraph=not through_fr))
+    assert torch.equal(y0, y1)
+    for name, a, b in zip(("x",) + ORDER, g0, g1):
+        assert torch.equal(a, b), name
+    torch._dynamo.reset()
+
+
 def test_partial_and_full_agree_bf16(wf, projections):
     """The two recompute modes are the same function of the nine raw inputs."""
     say(f"\ncase partial_vs_full bf16 own_projections={projections}")
