@@ -37,6 +37,7 @@ WORKLOADS = {
     "cfg0": (2, 32, 14, 14, "f32"),
     "cfg3": None,   # M2D-T backbone inference, handled by backbone_inference()
     "entry": None,  # wavefront_scan_cuda (projections + scan) at the cfg1 shape, handled by entry_point()
+    "cfg2": None,   # the four M2D-T stage scans in sequence, handled by stage_sequence()
 }
 N = 16
 HBM_PEAK_GBS = 8000.0
@@ -136,6 +137,60 @@ def backbone_inference(args):
         "roofline": None, "cpu_baseline": None,
     }
     print(json.dumps(out))
+
+
+def stage_sequence(args):
+    """The four M2D-T stage scans one after the other, (E,H,W) = (64,56,56), (128,28,28), (320,14,14),
+    (512,7,7) at B=128, bf16 tensors with fp32 state.  One step = forward + backward of all four."""
+    import torch
+    from mamba2d_amd import cabi, wavefront
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device="cpu").manual_seed(0)
+    r = lambda *s: torch.randn(*s, generator=g)
+    sp = torch.nn.functional.softplus
+    stages, units, alg = [], 0, 0
+    for name in ("cfg1", "stage2", "stage3", "stage4"):
+        B, E, H, W, _ = WORKLOADS[name]
+        host = [r(B, H, W, E), sp(r(B, H, W, E)), sp(r(B, H, W, E)), -torch.exp(-4 * torch.rand(E, N, generator=g)),
+                -torch.exp(-4 * torch.rand(E, N, generator=g)), r(B, H, W, N), r(B, H, W, N), r(B, H, W, N), r(E)]
+        leaves = [t.to(torch.bfloat16).to(dev).requires_grad_(True) for t in host]
+        stages.append((leaves, [t.detach() for t in leaves], r(B, H, W, E).to(torch.bfloat16).to(dev)))
+        units += B * H * W * E * N
+        alg += sum(algorithmic_bytes(B, E, H, W, 2))
+
+    def fwd_only():
+        with torch.no_grad():
+            for _, frozen, _ in stages:
+                wavefront.wf_cuda_fn_pr.apply(*frozen)
+
+    def fwd_bwd():
+        for leaves, _, dy in stages:
+            torch.autograd.grad(wavefront.wf_cuda_fn_pr.apply(*leaves), leaves, dy)
+
+    def timed(fn):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / args.steps
+
+    fwd_ms, both_ms = timed(fwd_only), timed(fwd_bwd)
+    print(json.dumps({
+        "metric": "four M2D-T stage scans in sequence, fwd+bwd ms at B=128 N=16", "value": round(both_ms, 4), "unit": "ms",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(both_ms, 4),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 in/out, f32 state",
+        "data": "synthetic",
+        "config": {"workload": "cfg2: scans of (E,H,W) = (64,56,56), (128,28,28), (320,14,14), (512,7,7) in sequence, B=128 N=16"},
+        "fwd_ms": round(fwd_ms, 4), "fwd_bwd_ms": round(both_ms, 4),
+        "pct_hbm_roofline": {"fwd_bwd": round(100 * alg / (both_ms * 1e-3) / (HBM_PEAK_GBS * 1e9), 2)},
+        "valu_ceiling_frac": round(units * 48 / VALU_PEAK_SLOTS / (both_ms * 1e-3), 4),
+        "roofline": None, "cpu_baseline": None,
+    }))
 
 
 def entry_point(args):
@@ -251,6 +306,9 @@ def main():
         return
     if args.workload == "entry":
         entry_point(args)
+        return
+    if args.workload == "cfg2":
+        stage_sequence(args)
         return
     B, E, H, W, dts = WORKLOADS[args.workload]
     dtype = torch.bfloat16 if dts == "bf16" else torch.float32
