@@ -1449,11 +1449,16 @@ Geometry make_geometry(const m2d_desc* d) {
     g.nblk = g.nbands * g.nbb;
     g.nlaunch = kSliceLag * (g.nbands - 1) + (g.nbb + kSliceQ - 1) / kSliceQ;
   }
-  // forward: two channels per lane when that still yields enough waves to fill the device and the
-  // two staging buffers of such a workgroup fit the LDS (bf16 operands: 112 KB; fp32 ones do not)
+  // forward: two channels per lane where that saves rounds of workgroups (one workgroup per compute
+  // unit at a time, 256 units) and the two staging buffers of such a workgroup fit the LDS (bf16
+  // operands: 112 KB; fp32 ones do not).  A sweep with two channels per lane takes about 1.8 times
+  // as long as one with a single channel (measured: 1.6 at 28x28, 2.0 at 56x56), so it pays only
+  // when it at least halves the rounds: 128 channels x 128 images, not 32 channels x 256 images
+  // (where half of every workgroup would idle).
   const size_t lds_ec2 = d->dtype == M2D_BF16 ? fwd_lds_bytes<bf16_t, 2>() : fwd_lds_bytes<float, 2>();
-  const bool ec2 = (d->E % 2 == 0) && lds_ec2 <= kLdsPerWorkgroup &&
-                   ((int64_t)B * ((d->E + kFwdWaves * g.CS * 2 - 1) / (kFwdWaves * g.CS * 2)) >= 256);
+  const int64_t wg1 = (int64_t)B * ((d->E + kFwdWaves * g.CS - 1) / (kFwdWaves * g.CS));
+  const int64_t wg2 = (int64_t)B * ((d->E + kFwdWaves * g.CS * 2 - 1) / (kFwdWaves * g.CS * 2));
+  const bool ec2 = (d->E % 2 == 0) && lds_ec2 <= kLdsPerWorkgroup && 18 * ((wg2 + 255) / 256) < 10 * ((wg1 + 255) / 256);
   g.fwd_ec = ec2 ? 2 : 1;
   g.fwd_bpb = (d->E + kFwdWaves * g.CS * g.fwd_ec - 1) / (kFwdWaves * g.CS * g.fwd_ec);
   g.fwd_wpb = g.fwd_bpb * kFwdWaves;

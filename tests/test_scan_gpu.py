@@ -92,8 +92,10 @@ SHAPES = [
     (900, 2, 5, 2),   # 2-row images, several to a band
     (1, 512, 512, 2), # 37 bands of one large image (sliced sweep at the size of the latency benchmark's second point)
     (2, 300, 260, 4), # 22 bands, two images
-    (303, 10, 3, 12), # over 256 unstacked images, even channel count: two channels per lane where the staging fits the LDS (bf16)
+    (303, 10, 3, 12), # over 256 unstacked images, even channel count (once asked for two channels per lane in fp32, which does not fit the LDS)
     (260, 20, 5, 64), # the same with two padded bands and a full workgroup of channels
+    (128, 4, 3, 128), # 512 workgroups with one channel per lane, 256 with two: the bf16 forward takes two channels per lane
+    (256, 17, 4, 64), # the same from the batch side, two padded bands
 ]
 
 
