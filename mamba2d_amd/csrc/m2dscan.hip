@@ -51,6 +51,7 @@ constexpr int kHB = 16;           // rows per band = lanes per DPP row
 constexpr int kHBShift = 4;
 constexpr int kRB = 14;           // grid rows per band; lanes 0 and 15 of a row are boundary ghosts
 constexpr int kFwdWaves = 8;      // waves per forward workgroup
+constexpr int kFwdHalfWaves = 4;  // ... of a small batch (fewer workgroups of 8 than half the compute units)
 constexpr int kBwdWaves = 8;      // waves per backward workgroup
 constexpr int kZeroFloats = 64;     // page of zeros at the head of the set-up area
 constexpr int kModeSweep = 0, kModeSliced = 1, kModeStacked = 2;   // how the bands of the batch are scheduled
@@ -529,8 +530,10 @@ __device__ __forceinline__ void store_snapshot(float4* dst, float a, float b, fl
 // grid row, works on zero operands (its records come from the page of zeros), which keeps its
 // state finite and never reaches a cell of the grid: at column 0 the left gate is closed, and
 // what the lane below hands to a cell comes from the cell above it.  Only stores are predicated.
-template <typename T, int EC, bool CKPT, bool WRITE_Y, bool STAGE_X, int MODE>
-__global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParams pin) {
+// NW waves per workgroup: 8, or 4 where the batch is too small to give every compute unit a
+// workgroup of 8 (each wave then has a SIMD to itself).
+template <typename T, int EC, bool CKPT, bool WRITE_Y, bool STAGE_X, int MODE, int NW = kFwdWaves>
+__global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) {
   constexpr bool SLICED = MODE == kModeSliced, STACKED = MODE == kModeStacked;
   ScanParams p = pin;   // (stacked images: the height is shortened below for a last, shorter stack)
   if constexpr (!STACKED) {   // lets the compiler drop what only stacked images need
@@ -538,7 +541,7 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
     __builtin_assume(p.S >= kHB + kCK - 1);
   }
   constexpr int CS = 64 >> kHBShift;
-  constexpr int CW = kFwdWaves * CS * EC;
+  constexpr int CW = NW * CS * EC;
   constexpr bool PERM = true;
   constexpr bool AHEAD = EC == 1 && STAGE_X;   // operands of step t+1 are fetched from LDS during step t
   using SG = Stage<T, 3, CW, false, true>;
@@ -572,8 +575,8 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   const bool ch_ok = e_raw < p.E;                  // idle lanes still take part in staging and barriers
   const int e0 = ch_ok ? e_raw : p.E - EC;
   // every byte a lane may read is finite from the start (pads are never written again)
-  for (int i = threadIdx.x; i < (2 * SG::kBytes + 256) / 16; i += kFwdWaves * 64) smem[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-  StagePlan<T, 3, CW, false, true, kFwdWaves, true> plan;
+  for (int i = threadIdx.x; i < (2 * SG::kBytes + 256) / 16; i += NW * 64) smem[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+  StagePlan<T, 3, CW, false, true, NW, true> plan;
   plan.init(wave, lane);
 
   float a2t[EC][kN], a2l[EC][kN], dsk[EC];
@@ -735,7 +738,7 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   };
 
   Pos A = pos_of(p, m_lo * kCK - (kHB - 1));     // position of the stream index t0 - 15 (wave-uniform)
-  stage_block<T, 3, CW, false, true, STAGE_X, kFwdWaves, true>(p, plan, lds, b, A, e_wg0, wave, lane, X, DT, DL, DY);
+  stage_block<T, 3, CW, false, true, STAGE_X, NW, true>(p, plan, lds, b, A, e_wg0, wave, lane, X, DT, DL, DY);
   staging_fence();
   Ops opsA, opsB;
   if constexpr (AHEAD) fetch(lds, 0, opsA);
@@ -743,7 +746,7 @@ __global__ __launch_bounds__(kFwdWaves * 64) void m2d_fwd_kernel(const ScanParam
   for (int m = m_lo; m < m_hi; ++m) {
     const bool last = m + 1 == m_hi;
     if (!last)
-      stage_block<T, 3, CW, false, true, STAGE_X, kFwdWaves, true>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, pos_after(p, A, kCK), e_wg0, wave, lane, X, DT, DL, DY);
+      stage_block<T, 3, CW, false, true, STAGE_X, NW, true>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, pos_after(p, A, kCK), e_wg0, wave, lane, X, DT, DL, DY);
     bp = block_pos(p, A, r, ch_ok);
     K = lane_consts<false>(p, clamp_band(p, bp.bnd0), r, ch_ok);
     per_step_K = __any(bp.kw < kCK && special_boundary(p, bp.bnd0, r));
@@ -1354,8 +1357,8 @@ inline size_t align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
 // Dynamic LDS of a workgroup: the forward's two staging buffers, the backward's exchange buffers, its
 // copy of A and two staging buffers.  A compute unit has 160 KB.
 constexpr size_t kLdsPerWorkgroup = 160 * 1024;
-template <typename T, int EC>
-constexpr size_t fwd_lds_bytes() { return 256 + 2 * (size_t)Stage<T, 3, kFwdWaves * 4 * EC, false, true>::kBytes; }
+template <typename T, int EC, int NW = kFwdWaves>
+constexpr size_t fwd_lds_bytes() { return 256 + 2 * (size_t)Stage<T, 3, NW * 4 * EC, false, true>::kBytes; }
 template <typename T>
 constexpr size_t bwd_lds_bytes() {
   return sizeof(float4) * kBwdWaves * 3 * 64 + sizeof(float) * kBwdWaves * 4 * 2 * kN + 256 +
@@ -1367,7 +1370,7 @@ static_assert(bwd_lds_bytes<float>() <= kLdsPerWorkgroup && bwd_lds_bytes<bf16_t
 struct Geometry {
   int HB, hb_shift, CS, nbands, nblk;
   int S, T_total, rows_last;         // stream stride, total steps, rows of the last band
-  int fwd_ec, fwd_wpb, fwd_bpb;      // forward: channels per lane, waves and workgroups per image
+  int fwd_ec, fwd_nw, fwd_wpb, fwd_bpb;   // forward: channels per lane, waves per workgroup, waves and workgroups per image
   int bwd_wpb, bwd_bpb;              // backward: waves and workgroups (channel groups) per image
   bool stage_x;                      // x, delta, dy rows are whole 16-byte chunks: stage them through LDS
   bool sliced;                       // bands on workgroups of their own, swept by a sequence of launches
@@ -1460,8 +1463,12 @@ Geometry make_geometry(const m2d_desc* d) {
   const int64_t wg2 = (int64_t)B * ((d->E + kFwdWaves * g.CS * 2 - 1) / (kFwdWaves * g.CS * 2));
   const bool ec2 = (d->E % 2 == 0) && lds_ec2 <= kLdsPerWorkgroup && 18 * ((wg2 + 255) / 256) < 10 * ((wg1 + 255) / 256);
   g.fwd_ec = ec2 ? 2 : 1;
-  g.fwd_bpb = (d->E + kFwdWaves * g.CS * g.fwd_ec - 1) / (kFwdWaves * g.CS * g.fwd_ec);
-  g.fwd_wpb = g.fwd_bpb * kFwdWaves;
+  // forward of a small batch in one stream per image: workgroups of 4 waves (16 channels) where those
+  // are more than the workgroups of 8 and still no more than the compute units
+  const int64_t wg_half = (int64_t)B * ((d->E + kFwdHalfWaves * g.CS - 1) / (kFwdHalfWaves * g.CS));
+  g.fwd_nw = (!g.sliced && !g.stacked && !ec2 && wg_half > wg1 && wg_half <= 256) ? kFwdHalfWaves : kFwdWaves;
+  g.fwd_bpb = (d->E + g.fwd_nw * g.CS * g.fwd_ec - 1) / (g.fwd_nw * g.CS * g.fwd_ec);
+  g.fwd_wpb = g.fwd_bpb * g.fwd_nw;
   g.bwd_bpb = groups;
   g.bwd_wpb = g.bwd_bpb * kBwdWaves;
   g.stage_x = (d->E % (d->dtype == M2D_BF16 ? 8 : 4)) == 0;
@@ -1555,21 +1562,21 @@ int stage_bc(ScanParams& sp, const m2d_desc* d, const void* BT, const void* BL, 
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
-template <typename T, int EC, bool CK, bool WY, bool SX, int MODE>
+template <typename T, int EC, bool CK, bool WY, bool SX, int MODE, int NW>
 int launch_fwd_as(const ScanParams& sp, hipStream_t st) {
-  constexpr size_t lds = fwd_lds_bytes<T, EC>();
+  constexpr size_t lds = fwd_lds_bytes<T, EC, NW>();
   if (lds > kLdsPerWorkgroup) return M2D_ERR_UNSUPPORTED;   // (make_geometry never picks such a layout)
   static std::atomic<uint64_t> seen{0};
-  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_fwd_kernel<T, EC, CK, WY, SX, MODE>), lds, seen)) return M2D_ERR_HIP;
-  hipLaunchKernelGGL((m2d_fwd_kernel<T, EC, CK, WY, SX, MODE>), dim3((unsigned)sp.nwg), dim3(kFwdWaves * 64), lds, st, sp);
+  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_fwd_kernel<T, EC, CK, WY, SX, MODE, NW>), lds, seen)) return M2D_ERR_HIP;
+  hipLaunchKernelGGL((m2d_fwd_kernel<T, EC, CK, WY, SX, MODE, NW>), dim3((unsigned)sp.nwg), dim3(NW * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
-template <typename T, int EC, bool SX, int MODE>
+template <typename T, int EC, bool SX, int MODE, int NW = kFwdWaves>
 int launch_fwd_mode(const ScanParams& sp, bool ckpt, bool write_y, hipStream_t st) {
-  if (ckpt && write_y) return launch_fwd_as<T, EC, true, true, SX, MODE>(sp, st);
-  if (ckpt) return launch_fwd_as<T, EC, true, false, SX, MODE>(sp, st);
-  return launch_fwd_as<T, EC, false, true, SX, MODE>(sp, st);
+  if (ckpt && write_y) return launch_fwd_as<T, EC, true, true, SX, MODE, NW>(sp, st);
+  if (ckpt) return launch_fwd_as<T, EC, true, false, SX, MODE, NW>(sp, st);
+  return launch_fwd_as<T, EC, false, true, SX, MODE, NW>(sp, st);
 }
 
 template <typename T>
@@ -1587,6 +1594,9 @@ int launch_fwd(const ScanParams& sp0, const m2d_desc* d, const Geometry& g, bool
     }
     if (g.fwd_ec == 2)
       return g.stage_x ? launch_fwd_mode<T, 2, true, kModeSweep>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 2, false, kModeSweep>(sp, ckpt, write_y, st);
+    if (g.fwd_nw == kFwdHalfWaves)
+      return g.stage_x ? launch_fwd_mode<T, 1, true, kModeSweep, kFwdHalfWaves>(sp, ckpt, write_y, st)
+                       : launch_fwd_mode<T, 1, false, kModeSweep, kFwdHalfWaves>(sp, ckpt, write_y, st);
     return g.stage_x ? launch_fwd_mode<T, 1, true, kModeSweep>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 1, false, kModeSweep>(sp, ckpt, write_y, st);
   };
   if (!g.sliced) return once();

@@ -94,6 +94,9 @@ SHAPES = [
     (2, 300, 260, 4), # 22 bands, two images
     (303, 10, 3, 12), # over 256 unstacked images, even channel count (once asked for two channels per lane in fp32, which does not fit the LDS)
     (260, 20, 5, 64), # the same with two padded bands and a full workgroup of channels
+    (5, 30, 9, 32),   # small batch, three bands: forward workgroups of 4 waves (16 channels each)
+    (33, 57, 8, 48),  # the same with five bands in one padded stream, 99 workgroups of 4 waves
+    (4, 20, 11, 50),  # the same without x-staging, last workgroup partly filled
     (128, 4, 3, 128), # 512 workgroups with one channel per lane, 256 with two: the bf16 forward takes two channels per lane
     (256, 17, 4, 64), # the same from the batch side, two padded bands
 ]
