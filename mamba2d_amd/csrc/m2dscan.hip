@@ -1466,7 +1466,10 @@ Geometry make_geometry(const m2d_desc* d) {
   // forward of a small batch in one stream per image: workgroups of 4 waves (16 channels) where those
   // are more than the workgroups of 8 and still no more than the compute units
   const int64_t wg_half = (int64_t)B * ((d->E + kFwdHalfWaves * g.CS - 1) / (kFwdHalfWaves * g.CS));
-  g.fwd_nw = (!g.sliced && !g.stacked && !ec2 && wg_half > wg1 && wg_half <= 256) ? kFwdHalfWaves : kFwdWaves;
+  // (the sliced sweep has at most every kSliceLag-th launch window of a band under way at a time)
+  const int64_t together = g.sliced ? (((g.nbb + kSliceQ - 1) / kSliceQ + kSliceLag - 1) / kSliceLag < g.nbands
+                                           ? ((g.nbb + kSliceQ - 1) / kSliceQ + kSliceLag - 1) / kSliceLag : g.nbands) : 1;
+  g.fwd_nw = (!g.stacked && !ec2 && wg_half > wg1 && wg_half * together <= 256) ? kFwdHalfWaves : kFwdWaves;
   g.fwd_bpb = (d->E + g.fwd_nw * g.CS * g.fwd_ec - 1) / (g.fwd_nw * g.CS * g.fwd_ec);
   g.fwd_wpb = g.fwd_bpb * g.fwd_nw;
   g.bwd_bpb = groups;
@@ -1585,8 +1588,12 @@ int launch_fwd(const ScanParams& sp0, const m2d_desc* d, const Geometry& g, bool
   sp.bpb = g.fwd_bpb;
   sp.nwg = g.vB * g.fwd_bpb;
   auto once = [&]() {
-    if (g.sliced)   // (the sliced sweep is only chosen where one channel per lane is)
+    if (g.sliced) {   // (the sliced sweep is only chosen where one channel per lane is)
+      if (g.fwd_nw == kFwdHalfWaves)
+        return g.stage_x ? launch_fwd_mode<T, 1, true, kModeSliced, kFwdHalfWaves>(sp, ckpt, write_y, st)
+                         : launch_fwd_mode<T, 1, false, kModeSliced, kFwdHalfWaves>(sp, ckpt, write_y, st);
       return g.stage_x ? launch_fwd_mode<T, 1, true, kModeSliced>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 1, false, kModeSliced>(sp, ckpt, write_y, st);
+    }
     if (g.stacked) {
       if (g.fwd_ec == 2)
         return g.stage_x ? launch_fwd_mode<T, 2, true, kModeStacked>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 2, false, kModeStacked>(sp, ckpt, write_y, st);
