@@ -833,8 +833,10 @@ __device__ __forceinline__ constexpr int fold_state(int m, int qi) {
 // on zero operands.  For the adjoint this means that a row which has not reached its last column
 // yet keeps lambda = mu = 0 exactly, and that a row past column 0 carries finite values that are
 // multiplied by zero coefficients (delta, dy, x are zero there) wherever they meet a sum.
-template <typename T, bool STAGE_X, int MODE>
-__global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParams pin) {
+// NW waves per workgroup: 8, or 4 for small batches (see the forward kernel).  With 4 waves a thread
+// of the first three adds up both components of one lane's pair of channel sums.
+template <typename T, bool STAGE_X, int MODE, int NW = kBwdWaves>
+__global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) {
   constexpr bool SLICED = MODE == kModeSliced, STACKED = MODE == kModeStacked;
   ScanParams p = pin;   // (stacked images: the height is shortened below for a last, shorter stack)
   if constexpr (!STACKED) {   // lets the compiler drop what only stacked images need
@@ -843,7 +845,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   }
   constexpr int CS = 64 >> kHBShift;     // 4 channel slots
   constexpr int SLOT = 3 * 64;           // float2s per wave in one exchange buffer
-  constexpr int CW = kBwdWaves * CS;
+  constexpr int CW = NW * CS;
   constexpr bool PERM = true;
   using SG = Stage<T, 4, CW, true, false>;
   extern __shared__ float4 smem[];
@@ -851,8 +853,8 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   // alternately, so that one barrier per exchange is enough (a buffer is rewritten two exchanges
   // later, after a barrier that every wave reaches only once it has finished reading it).
   float2* slots = reinterpret_cast<float2*>(smem);                       // [2][wave][3][64]
-  float* a_lds = reinterpret_cast<float*>(smem + kBwdWaves * SLOT);      // [wave][CS][2][16], fold order
-  char* lds = reinterpret_cast<char*>(a_lds + kBwdWaves * CS * 2 * kN);  // 2 staging buffers
+  float* a_lds = reinterpret_cast<float*>(smem + NW * SLOT);      // [wave][CS][2][16], fold order
+  char* lds = reinterpret_cast<char*>(a_lds + NW * CS * 2 * kN);  // 2 staging buffers
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   int lb = logical_block(p.nwg);
@@ -888,7 +890,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   }
   const uint32_t a_base_off = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) float*)(a_lds + ch_loc * (2 * kN)));
   const float dsk = p.Df[e];
-  StagePlan<T, 4, CW, true, false, kBwdWaves, false> plan;
+  StagePlan<T, 4, CW, true, false, NW, false> plan;
   plan.init(wave, lane);
   settle_loads();
 
@@ -940,9 +942,10 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
   constexpr uint32_t kXK = SG::kXStepBytes;   // XD bytes per step
   // the sum that this thread adds up in the exchange (one float of one lane's float2, one tensor):
   // it belongs to lane row f_r, which is f_d positions ahead of this thread's own row
-  const int fid = wave * (2 * SLOT / kBwdWaves) + lane;
-  const bool f_on = lane < 2 * SLOT / kBwdWaves;
-  const int f_it = fid >> 1, f_comp = fid & 1;
+  constexpr bool PAIRS = NW * 64 < 2 * SLOT;   // fewer threads than sums: a thread takes a pair
+  const int fid = PAIRS ? wave * 64 + lane : wave * (2 * SLOT / NW) + lane;
+  const bool f_on = PAIRS ? fid < SLOT : lane < 2 * SLOT / NW;
+  const int f_it = PAIRS ? fid : fid >> 1, f_comp = PAIRS ? 0 : fid & 1;
   const int f_r = f_it & (kHB - 1), f_s = (f_it & 63) >> kHBShift, f_v = f_it >> 6;
   const int f_d = r - f_r;
   const uint32_t f_sub = (uint32_t)(f_v * kN + f_s * 4 + f_comp) * (uint32_t)sizeof(float);
@@ -991,7 +994,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
 
   Pos A = pos_of(p, (m_hi - 1) * kCK - (kHB - 1));   // position of the stream index t0 - 15 (wave-uniform)
   load_ckpt(m_hi - 1, A);
-  stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds, b, A, e_wg0, wave, lane, X, DT, DL, DY);
+  stage_block<T, 4, CW, true, false, STAGE_X, NW, false>(p, plan, lds, b, A, e_wg0, wave, lane, X, DT, DL, DY);
   staging_fence();
   int cur = 0;
   int xpar = 0;   // exchange buffer in use
@@ -1004,7 +1007,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
     for (int n = 0; n < kN; ++n) ck0[n] = cknext[n];
     const Pos Aprev = pos_before(A);
     if (m > m_lo)
-      stage_block<T, 4, CW, true, false, STAGE_X, kBwdWaves, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, Aprev, e_wg0, wave, lane, X, DT, DL, DY);
+      stage_block<T, 4, CW, true, false, STAGE_X, NW, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, Aprev, e_wg0, wave, lane, X, DT, DL, DY);
     bp = block_pos(p, A, r, ch_ok);
     fp = block_pos(p, A, f_r, f_on);
     band_consts(bp.bnd0);
@@ -1119,7 +1122,7 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
           const float dyl = dyv + gb1;
           float sT = 0.f, sL = 0.f, zT = 0.f, zL = 0.f;
           if (half == 1) { sT = part4[k][0]; sL = part4[k][1]; zT = part4[k][2]; zL = part4[k][3]; }
-          float* sw = reinterpret_cast<float*>(slots + (xpar * kBwdWaves + wave) * SLOT + lane);
+          float* sw = reinterpret_cast<float*>(slots + (xpar * NW + wave) * SLOT + lane);
           // A group of 4 states is folded over the 4 channel slots of the wave as soon as it is
           // done; afterwards the lane of slot q holds the channel sums of the states 4q..4q+3
           // (component mgl of its float2 after group mgl of this half).
@@ -1188,12 +1191,20 @@ __global__ __launch_bounds__(kBwdWaves * 64) void m2d_bwd_kernel(const ScanParam
           // groups) are added in wave order, one sum per thread, the same share for every wave
           __syncthreads();
           if ((fp.in_grid >> k) & 1u) {
-            const float* sl = reinterpret_cast<const float*>(slots + xpar * kBwdWaves * SLOT + f_it) + f_comp;
-            float s = sl[0];
-#pragma unroll
-            for (int w = 1; w < kBwdWaves; ++w) s += sl[2 * w * SLOT];
             const uint32_t off = f_off0 + (uint32_t)k * pstep + (k >= fp.kw ? pwrap_adj : 0u) + (uint32_t)(2 * half * sizeof(float));
-            *reinterpret_cast<float*>(PARTimg + off) = s;
+            if constexpr (PAIRS) {
+              const float2* sl = slots + xpar * NW * SLOT + f_it;
+              float2 s = sl[0];
+#pragma unroll
+              for (int w = 1; w < NW; ++w) { s.x += sl[w * SLOT].x; s.y += sl[w * SLOT].y; }
+              *reinterpret_cast<float2*>(PARTimg + off) = s;
+            } else {
+              const float* sl = reinterpret_cast<const float*>(slots + xpar * NW * SLOT + f_it) + f_comp;
+              float s = sl[0];
+#pragma unroll
+              for (int w = 1; w < NW; ++w) s += sl[2 * w * SLOT];
+              *reinterpret_cast<float*>(PARTimg + off) = s;
+            }
           }
           xpar ^= 1;
         }
@@ -1359,10 +1370,10 @@ inline size_t align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
 constexpr size_t kLdsPerWorkgroup = 160 * 1024;
 template <typename T, int EC, int NW = kFwdWaves>
 constexpr size_t fwd_lds_bytes() { return 256 + 2 * (size_t)Stage<T, 3, NW * 4 * EC, false, true>::kBytes; }
-template <typename T>
+template <typename T, int NW = kBwdWaves>
 constexpr size_t bwd_lds_bytes() {
-  return sizeof(float4) * kBwdWaves * 3 * 64 + sizeof(float) * kBwdWaves * 4 * 2 * kN + 256 +
-         2 * (size_t)Stage<T, 4, kBwdWaves * 4, true, false>::kBytes;
+  return sizeof(float4) * NW * 3 * 64 + sizeof(float) * NW * 4 * 2 * kN + 256 +
+         2 * (size_t)Stage<T, 4, NW * 4, true, false>::kBytes;
 }
 static_assert(fwd_lds_bytes<float, 1>() <= kLdsPerWorkgroup && fwd_lds_bytes<bf16_t, 1>() <= kLdsPerWorkgroup, "forward staging must fit the LDS");
 static_assert(bwd_lds_bytes<float>() <= kLdsPerWorkgroup && bwd_lds_bytes<bf16_t>() <= kLdsPerWorkgroup, "backward staging must fit the LDS");
@@ -1371,7 +1382,7 @@ struct Geometry {
   int HB, hb_shift, CS, nbands, nblk;
   int S, T_total, rows_last;         // stream stride, total steps, rows of the last band
   int fwd_ec, fwd_nw, fwd_wpb, fwd_bpb;   // forward: channels per lane, waves per workgroup, waves and workgroups per image
-  int bwd_wpb, bwd_bpb;              // backward: waves and workgroups (channel groups) per image
+  int bwd_nw, bwd_wpb, bwd_bpb;      // backward: waves per workgroup, waves and workgroups (channel groups) per image
   bool stage_x;                      // x, delta, dy rows are whole 16-byte chunks: stage them through LDS
   bool sliced;                       // bands on workgroups of their own, swept by a sequence of launches
   bool stacked;                      // images of one band stacked into tall images of independent bands
@@ -1472,8 +1483,9 @@ Geometry make_geometry(const m2d_desc* d) {
   g.fwd_nw = (!g.stacked && !ec2 && wg_half > wg1 && wg_half * together <= 256) ? kFwdHalfWaves : kFwdWaves;
   g.fwd_bpb = (d->E + g.fwd_nw * g.CS * g.fwd_ec - 1) / (g.fwd_nw * g.CS * g.fwd_ec);
   g.fwd_wpb = g.fwd_bpb * g.fwd_nw;
-  g.bwd_bpb = groups;
-  g.bwd_wpb = g.bwd_bpb * kBwdWaves;
+  g.bwd_nw = (!g.stacked && wg_half > (int64_t)B * groups && wg_half * together <= 256) ? kFwdHalfWaves : kBwdWaves;
+  g.bwd_bpb = (d->E + g.bwd_nw * g.CS - 1) / (g.bwd_nw * g.CS);
+  g.bwd_wpb = g.bwd_bpb * g.bwd_nw;
   g.stage_x = (d->E % (d->dtype == M2D_BF16 ? 8 : 4)) == 0;
   const size_t P = (size_t)d->B * d->H * d->W;
   g.prep_bytes = align_up(sizeof(float) * (kZeroFloats + (size_t)2 * d->E * kN + d->E));
@@ -1642,13 +1654,21 @@ int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   return rc;
 }
 
-template <typename T, bool SX, int MODE>
-int launch_bwd(const ScanParams& sp, hipStream_t st) {
-  constexpr size_t lds = bwd_lds_bytes<T>();
+template <typename T, bool SX, int MODE, int NW>
+int launch_bwd_as(const ScanParams& sp, hipStream_t st) {
+  constexpr size_t lds = bwd_lds_bytes<T, NW>();
   static std::atomic<uint64_t> seen{0};
-  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_bwd_kernel<T, SX, MODE>), lds, seen)) return M2D_ERR_HIP;
-  hipLaunchKernelGGL((m2d_bwd_kernel<T, SX, MODE>), dim3((unsigned)sp.nwg), dim3(kBwdWaves * 64), lds, st, sp);
+  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_bwd_kernel<T, SX, MODE, NW>), lds, seen)) return M2D_ERR_HIP;
+  hipLaunchKernelGGL((m2d_bwd_kernel<T, SX, MODE, NW>), dim3((unsigned)sp.nwg), dim3(NW * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+}
+
+template <typename T, bool SX, int MODE>
+int launch_bwd(const ScanParams& sp, hipStream_t st, int nw = kBwdWaves) {
+  if constexpr (MODE != kModeStacked) {
+    if (nw == kFwdHalfWaves) return launch_bwd_as<T, SX, MODE, kFwdHalfWaves>(sp, st);
+  }
+  return launch_bwd_as<T, SX, MODE, kBwdWaves>(sp, st);
 }
 
 template <typename T>
@@ -1681,7 +1701,7 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][0], st);
   if (!g.sliced) {
     if (g.stacked) rc = g.stage_x ? launch_bwd<T, true, kModeStacked>(sp, st) : launch_bwd<T, false, kModeStacked>(sp, st);
-    else rc = g.stage_x ? launch_bwd<T, true, kModeSweep>(sp, st) : launch_bwd<T, false, kModeSweep>(sp, st);
+    else rc = g.stage_x ? launch_bwd<T, true, kModeSweep>(sp, st, g.bwd_nw) : launch_bwd<T, false, kModeSweep>(sp, st, g.bwd_nw);
   } else {
     // as the forward, bottom-up: launch l advances the band k' from the bottom by Q blocks of its window
     const int nlb = (g.nbb + kSliceQ - 1) / kSliceQ;
@@ -1692,7 +1712,7 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
       if (k_lo > k_hi) continue;
       sp.sl_ell = l; sp.sl_band0 = g.nbands - 1 - k_hi;
       sp.nwg = (k_hi - k_lo + 1) * g.vB * g.bwd_bpb;
-      rc = g.stage_x ? launch_bwd<T, true, kModeSliced>(sp, st) : launch_bwd<T, false, kModeSliced>(sp, st);
+      rc = g.stage_x ? launch_bwd<T, true, kModeSliced>(sp, st, g.bwd_nw) : launch_bwd<T, false, kModeSliced>(sp, st, g.bwd_nw);
     }
   }
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][1], st);
