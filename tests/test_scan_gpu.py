@@ -97,6 +97,8 @@ SHAPES = [
     (5, 30, 9, 32),   # small batch, three bands: forward workgroups of 4 waves (16 channels each)
     (33, 57, 8, 48),  # the same with five bands in one padded stream, 99 workgroups of 4 waves
     (4, 20, 11, 50),  # the same without x-staging, last workgroup partly filled
+    (3, 30, 28, 32),  # workgroups of 4 waves, three bands back to back (stride = width)
+    (70, 44, 26, 32), # the same with four bands and 140 workgroups
     (1, 60, 40, 32),  # sliced sweep (five bands of one image) on forward workgroups of 4 waves
     (2, 100, 33, 48), # the same, eight bands of two images, three workgroups of 16 channels per band
     (128, 4, 3, 128), # 512 workgroups with one channel per lane, 256 with two: the bf16 forward takes two channels per lane
