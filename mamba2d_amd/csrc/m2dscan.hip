@@ -1491,10 +1491,13 @@ Geometry make_geometry(const m2d_desc* d) {
   // (the sliced sweep has at most every kSliceLag-th launch window of a band under way at a time)
   const int64_t together = g.sliced ? (((g.nbb + kSliceQ - 1) / kSliceQ + kSliceLag - 1) / kSliceLag < g.nbands
                                            ? ((g.nbb + kSliceQ - 1) / kSliceQ + kSliceLag - 1) / kSliceLag : g.nbands) : 1;
-  g.fwd_nw = (!g.stacked && !ec2 && wg_half > wg1 && wg_half * together <= 256) ? kFwdHalfWaves : kFwdWaves;
+  // (a sliced sweep may exceed the units by a few workgroups while most bands are under way: its first
+  // and last launches, with fewer bands, still gain)
+  const int64_t room = g.sliced ? 256 + 16 : 256;
+  g.fwd_nw = (!g.stacked && !ec2 && wg_half > wg1 && wg_half * together <= room) ? kFwdHalfWaves : kFwdWaves;
   g.fwd_bpb = (d->E + g.fwd_nw * g.CS * g.fwd_ec - 1) / (g.fwd_nw * g.CS * g.fwd_ec);
   g.fwd_wpb = g.fwd_bpb * g.fwd_nw;
-  g.bwd_nw = (!g.stacked && wg_half > (int64_t)B * groups && wg_half * together <= 256) ? kFwdHalfWaves : kBwdWaves;
+  g.bwd_nw = (!g.stacked && wg_half > (int64_t)B * groups && wg_half * together <= room) ? kFwdHalfWaves : kBwdWaves;
   g.bwd_bpb = (d->E + g.bwd_nw * g.CS - 1) / (g.bwd_nw * g.CS);
   g.bwd_wpb = g.bwd_bpb * g.bwd_nw;
   g.stage_x = (d->E % (d->dtype == M2D_BF16 ? 8 : 4)) == 0;
