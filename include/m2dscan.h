@@ -42,7 +42,8 @@ typedef enum m2d_status {
                                  for 32-bit offsets (H*W >= 2^24 cells or H*W*E >= 2^30 elements) */
   M2D_ERR_WORKSPACE = 4,      /* workspace or checkpoint buffer smaller than required */
   M2D_ERR_MISALIGNED = 5,     /* a tensor pointer is not 16-byte aligned / workspace not 256-byte aligned */
-  M2D_ERR_HIP = 6             /* a HIP runtime call or kernel launch failed */
+  M2D_ERR_HIP = 6,            /* a HIP runtime call or kernel launch failed */
+  M2D_ERR_TOO_LARGE = 7       /* m2d_scan_fwd_noalloc: the problem needs more scratch than the library's static buffer */
 } m2d_status;
 
 typedef enum m2d_dtype {
@@ -120,6 +121,23 @@ int m2d_scan_fwd(const m2d_desc* desc,
                  void* ckpt, size_t ckpt_bytes,
                  void* workspace, size_t workspace_bytes,
                  void* stream);
+
+/* m2d_scan_fwd without a checkpoint buffer and without a workspace argument, for callers that cannot
+ * allocate device memory (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * it).  It has no counterpart in the reference, whose Python side allocates every buffer with
+ * torch.empty.  The scratch that m2d_scan_fwd takes as `workspace` lives in a static device array
+ * of M2D_NOALLOC_SCRATCH_BYTES inside the library (each GPU the library runs on holds one copy until
+ * the process ends); the call allocates and frees nothing.  A problem whose
+ * m2d_scan_workspace_bytes(desc, M2D_PASS_FWD, 0) exceeds that size is rejected with
+ * M2D_ERR_TOO_LARGE before anything is launched.  All calls on one GPU share the array: two calls
+ * that overlap on one GPU (different streams or threads) race; calls on one stream are ordered. */
+#define M2D_NOALLOC_SCRATCH_BYTES (32u << 20)
+int m2d_scan_fwd_noalloc(const m2d_desc* desc,
+                         const void* x, const void* deltaT, const void* deltaL,
+                         const void* AT, const void* AL,
+                         const void* BT, const void* BL, const void* C, const void* D,
+                         void* y,
+                         void* stream);
 
 /* Fused backward: the nine gradients of the forward above for upstream gradient dy.
  * Replaces wavefront_cuda.py:169-196 (state recompute, wf_bwd of wf_cuda_bind.cpp:35,

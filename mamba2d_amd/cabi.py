@@ -22,7 +22,7 @@ M2D_FLAG_DPRE = 16
 M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
-           "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_bwd", "m2d_proj_workspace_bytes", "m2d_proj_fwd",
+           "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_fwd_noalloc", "m2d_scan_bwd", "m2d_proj_workspace_bytes", "m2d_proj_fwd",
            "m2d_proj_bwd", "m2d_layernorm_fwd", "m2d_dwconv3x3_fwd", "m2d_starrelu_fwd",
            "m2d_scale_residual_fwd", "m2d_scale_residual_layernorm_fwd", "m2d_rope_qknorm_fwd", "m2d_rope_attention_fwd", "m2d_mlp_fwd", "m2d_layernorm_linear_fwd", "m2d_linear_fwd", "m2d_profile_enable", "m2d_profile_last_ms")
 
@@ -56,6 +56,8 @@ def _load():
     lib.m2d_scan_ckpt_bytes.argtypes = [dp]
     lib.m2d_scan_fwd.restype = i32
     lib.m2d_scan_fwd.argtypes = [dp] + [vp] * 9 + [vp, vp, sz, vp, sz, vp]
+    lib.m2d_scan_fwd_noalloc.restype = i32
+    lib.m2d_scan_fwd_noalloc.argtypes = [dp] + [vp] * 9 + [vp, vp]
     lib.m2d_scan_bwd.restype = i32
     lib.m2d_scan_bwd.argtypes = [dp] + [vp] * 10 + [vp, sz] + [vp] * 9 + [vp, sz, vp]
     lib.m2d_proj_workspace_bytes.restype = sz
@@ -174,6 +176,21 @@ def scan_fwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, save_ckpt=False, flip=Fals
                            _ptr(y), _ptr(ck), ck.numel() if ck is not None else 0, _ptr(ws), ws.numel(),
                            _stream(x.device)))
     return (y, ck) if save_ckpt else y
+
+
+NOALLOC_SCRATCH_BYTES = 32 << 20
+M2D_ERR_TOO_LARGE = 7
+
+
+def scan_fwd_noalloc(x, deltaT, deltaL, AT, AL, BT, BL, C, D, y, flip=False):
+    """y through m2d_scan_fwd_noalloc: the caller brings the output too, the library's scratch is a
+    static device array, and nothing is allocated anywhere in the call."""
+    _same(x, deltaT, deltaL, AT, AL, BT, BL, C, D, y)
+    _shapes(x, deltaT, deltaL, AT, AL, BT, BL, C, D, y)
+    d = make_desc(x, AT.shape[1], flip)
+    check(lib.m2d_scan_fwd_noalloc(ctypes.byref(d), *[_ptr(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D)],
+                                   _ptr(y), _stream(x.device)))
+    return y
 
 
 def scan_bwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt=None, flip=False, dpre=False):

@@ -40,6 +40,11 @@
 
 #include "../../include/m2dscan.h"
 
+// Scratch of m2d_scan_fwd_noalloc: the workspace of a forward call, for callers that cannot
+// allocate.  Every device that loads the library holds its own copy at its own address; host code
+// only ever uses the address that hipGetSymbolAddress returns for the current device.
+static __device__ __align__(256) unsigned char scratch[M2D_NOALLOC_SCRATCH_BYTES];
+
 namespace {
 
 constexpr int kN = 16;            // states per channel
@@ -1760,6 +1765,7 @@ const char* m2d_status_str(int status) {
     case M2D_ERR_WORKSPACE: return "workspace or checkpoint buffer too small";
     case M2D_ERR_MISALIGNED: return "misaligned pointer (tensors 16 B, workspace/checkpoints 256 B)";
     case M2D_ERR_HIP: return "HIP runtime error";
+    case M2D_ERR_TOO_LARGE: return "problem needs more scratch than the static buffer of m2d_scan_fwd_noalloc holds (M2D_NOALLOC_SCRATCH_BYTES)";
     default: return "unknown status";
   }
 }
@@ -1838,6 +1844,26 @@ int m2d_scan_bwd(const m2d_desc* desc, const void* x, const void* deltaT, const 
   return desc->dtype == M2D_F32
              ? run_bwd<float>(desc, g, sp, AT, AL, BT, BL, C, D, ckpt, d_AT, d_AL, d_BT, d_BL, d_C, d_D, workspace, st)
              : run_bwd<bf16_t>(desc, g, sp, AT, AL, BT, BL, C, D, ckpt, d_AT, d_AL, d_BT, d_BL, d_C, d_D, workspace, st);
+}
+
+int m2d_scan_fwd_noalloc(const m2d_desc* desc, const void* x, const void* deltaT, const void* deltaL, const void* AT,
+                         const void* AL, const void* BT, const void* BL, const void* C, const void* D, void* y,
+                         void* stream) {
+  int rc = check_desc(desc);
+  if (rc) return rc;
+  if (workspace_bytes_of(make_geometry(desc), M2D_PASS_FWD, 0) > (size_t)M2D_NOALLOC_SCRATCH_BYTES) return M2D_ERR_TOO_LARGE;
+  // address of the current device's copy of the array, looked up once per device
+  static std::atomic<void*> addr[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return M2D_ERR_HIP;
+  void* ws = addr[dev].load(std::memory_order_acquire);
+  if (!ws) {
+    if (hipGetSymbolAddress(&ws, HIP_SYMBOL(scratch)) != hipSuccess || !ws) return M2D_ERR_HIP;
+    addr[dev].store(ws, std::memory_order_release);
+  }
+  // nothing in the workspace has to be zero on entry: the set-up kernel rewrites the page of zeros,
+  // boundary rows and carried state are written before they are read
+  return m2d_scan_fwd(desc, x, deltaT, deltaL, AT, AL, BT, BL, C, D, y, nullptr, 0, ws, (size_t)M2D_NOALLOC_SCRATCH_BYTES, stream);
 }
 
 }  // extern "C"

@@ -33,7 +33,7 @@ def test_header_symbols_are_exported(cabi):
 def test_version_and_status_strings(cabi):
     assert cabi.lib.m2d_version() >= 100
     assert cabi.status_str(0) == "ok"
-    for code in range(1, 7):
+    for code in range(1, 8):
         assert cabi.status_str(code) not in ("ok", "unknown status")
     assert cabi.status_str(99) == "unknown status"
 
