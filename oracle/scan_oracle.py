@@ -250,6 +250,66 @@ def wavefront_scan_ref(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_p
     return y
 
 
+class _RoundBothWays(torch.autograd.Function):
+    """Rounds a float64 tensor to bfloat16 values on the way forward and its gradient on the way back:
+    what a bf16 tensor between two stock operators does to the reference's data flow."""
+
+    @staticmethod
+    def forward(ctx, t):
+        return t.bfloat16().double()
+
+    @staticmethod
+    def backward(ctx, g):
+        return g.bfloat16().double()
+
+
+PARAM_ORDER = ("AT_log", "AL_log", "x_proj_w", "dt_projT_w", "dt_projT_b", "dt_projL_w", "dt_projL_b", "D")
+
+
+def entry_point_reference(x, params, dy, round_intermediates=False):
+    """The entry point (wavefront_cuda.py:315-347) in float64 for activations of x.dtype: the weights
+    are rounded to x.dtype first, as the reference's casts do (:327-332, and :88-94 for A), and every
+    product, the softplus and the scan are evaluated in float64.  With ``round_intermediates`` the
+    outputs of the three linear layers and of the softplus, and the gradients that flow back through
+    them, are rounded to bfloat16 as they are when the reference runs these stock operators on bf16
+    tensors (its own data flow, with exact arithmetic inside every operator).
+
+    Returns y, the nine gradients in the entry point's argument order, and for each of the five
+    projection weights the sum of the absolute values of the terms its gradient adds up
+    (``scales``): d_w = sum_p a_p b_p can cancel to far below sum_p |a_p b_p|, and an error bound that
+    is relative per term is relative to the latter.
+    """
+    dt = x.dtype
+    rw = lambda t: t.to(dt).double()
+    leaves = [x.double().requires_grad_(True)]
+    leaves += [(params[k].double() if k in ("AT_log", "AL_log") else rw(params[k])).requires_grad_(True) for k in PARAM_ORDER]
+    xx, ATl, ALl, xw, tw, tb, lw, lb, D = leaves
+    N, R = ATl.shape[1], tw.shape[1]
+    rb = _RoundBothWays.apply if round_intermediates else (lambda t: t)
+    AT = -torch.exp(ATl)
+    AL = -torch.exp(ALl)
+    if dt != torch.float64:   # A reaches the scan in x.dtype
+        AT = AT + (AT.detach().to(dt).double() - AT.detach())
+        AL = AL + (AL.detach().to(dt).double() - AL.detach())
+    z = rb(F.linear(xx, xw))
+    z.retain_grad()
+    rT, rL, BT, BL, C = torch.split(z, [R, R, N, N, N], dim=-1)
+    preT = rb(F.linear(rT, tw, tb))
+    preL = rb(F.linear(rL, lw, lb))
+    preT.retain_grad()
+    preL.retain_grad()
+    y = scan_forward_torch(xx, rb(F.softplus(preT)), rb(F.softplus(preL)), AT, AL, BT, BL, C, D)
+    y.backward(dy.double())
+    grads = [t.grad.detach() for t in leaves]
+    flat = lambda t: t.detach().reshape(-1, t.shape[-1]).abs()
+    scales = {
+        "x_proj_w": flat(z.grad).t() @ flat(xx),
+        "dt_projT_w": flat(preT.grad).t() @ flat(rT), "dt_projT_b": flat(preT.grad).sum(0),
+        "dt_projL_w": flat(preL.grad).t() @ flat(rL), "dt_projL_b": flat(preL.grad).sum(0),
+    }
+    return y.detach(), grads, scales
+
+
 # --------------------------------------------------------------------------------------
 # error metrics used by every parity test
 # --------------------------------------------------------------------------------------
