@@ -37,6 +37,7 @@
 
 #include <atomic>
 #include <stdint.h>
+#include <stdlib.h>
 
 #include "../../include/m2dscan.h"
 
@@ -255,48 +256,52 @@ template <bool PERM> __device__ __forceinline__ constexpr int sinv(int pos) {
 
 // ------------------------------------------------------------------------------ operand staging
 // The operands of a block of kCK steps of a band are copied to LDS one block ahead of their use
-// with direct global->LDS loads (no registers, asynchronous): lane i of a wave-wide load fills
-// the 16-byte chunk i of a 1 KB LDS window.  Regions of one buffer:
-//   BC : per (step k, lane row r) a record of 13 chunks: B_T, B_L, C of the cell (row r, column
-//        t0+k-r) as 3 x 16 fp32, plus one pad chunk so that the 16 rows fall in distinct banks;
-//   XD : per tensor (x, deltaT, deltaL[, dy]), step k and chunk of channels, the 16 lane rows side by
-//        side (chunk index = ((tensor*kCK + k)*kCpt + channel chunk)*16 + r, no padding: the rows of
-//        a wave-wide read fall in distinct banks); needs E to be a multiple of a chunk.  A wave-wide
-//        copy stays inside one tensor, so its base address is a scalar;
-//   TOP: per (k, channel) the 16 states of the last row of the band above at column t0+k;
-//   BOT: per (k, channel) the 16 muT of the first row of the band below at column t0+k-15.
-// With UNI, BC, TOP and BOT advance by the same number of bytes (kKStr) from one step to the
-// next, so a lane that reads "its record" finds it at one per-lane offset plus a constant per
-// step, whether it is a grid row (BC record) or a boundary ghost (TOP/BOT record).  Records of lanes and cells
-// outside the grid are filled from a page of zeros: such lanes compute on finite operands and
-// never need to be masked.
-template <typename T, int NT, int CW, bool WITH_BOT, bool UNI>
+// with direct global->LDS loads (no registers, asynchronous): lane i of a wave-wide copy fills
+// the 16-byte chunk i of a 1 KB LDS window.  Every copy is laid out so that the chunk a lane fills
+// belongs to the lane's own row (lane & 15): the position arithmetic of a block is done once per
+// lane and serves the lane's copies and its own loads and stores alike.  One buffer, in planes of
+// 256 bytes (16 chunks):
+//   per step k, kPlanes planes:
+//     planes 0..11   BC : plane 4*tensor + g holds, for the 16 lane rows r, the four values of state
+//                         group g of B_T, B_L, C (tensor 0, 1, 2) of the cell (row r, column t0+k-r);
+//     planes 12..    TOP: plane 12 + 4*h + g holds, for the channels 16h..16h+15 of the workgroup, state
+//                         group g of the last row of the band above at column t0+k;
+//     then (adjoint) BOT: the same for the muT of the first row of the band below at column t0+k-15;
+//   then XD: per tensor (x, deltaT, deltaL[, dy]), step k and chunk of channels, the 16 lane rows side by
+//        side (chunk index = ((tensor*kCK + k)*kCpt + channel chunk)*16 + r); needs E to be a multiple
+//        of a chunk.
+// A grid row reads the groups of its B_T, B_L, C at r*16 plus plane offsets; the upper ghost (lane 0)
+// reads the TOP planes of its channel as its B_T, the lower ghost (lane 15) the BOT planes as its C:
+// a per-lane base address under the same immediate offsets.  Chunks of rows and cells outside the grid
+// are filled from a page of zeros: such lanes compute on finite operands and never need to be masked.
+template <typename T, int NT, int CW, bool WITH_BOT>
 struct Stage {
   static constexpr int kElem = 16 / sizeof(T);           // elements per chunk
   static constexpr int kCpt = CW / kElem;                // chunks per tensor per cell
   static constexpr int kXStepBytes = kCpt * kHB * 16;    // XD bytes per tensor and step
   static constexpr int kXTauBytes = kCK * kXStepBytes;   // XD bytes per tensor
   static constexpr int kXTauInstr = kXTauBytes / 1024;   // wave-wide copies per tensor
-  static constexpr int kBRec = 13;                       // chunks per BC record (with pad)
-  static constexpr int kBStride = kBRec * 4;             // BC record stride in floats
-  static constexpr int kKChunks = kHB * kBRec > CW * 4 ? kHB * kBRec : CW * 4;   // chunks per step in BC / TOP / BOT
-  static constexpr int kKStr = kKChunks * 16;            // the same in bytes
-  static constexpr int kBChunks = kCK * kKChunks;
-  static constexpr int kXChunks = NT * kXTauBytes / 16;
+  static constexpr int kPlane = kHB * 16;                // bytes per plane
+  static constexpr int kG16 = CW / 16;                   // groups of 16 channels
+  static constexpr int kTopPlane = 12;
+  static constexpr int kBotPlane = kTopPlane + 4 * kG16;
+  // (adjoint: at least 24 planes, so that what a ghost reads 4 and 8 planes behind its boundary row is inside the step)
+  static constexpr int kPlanes = WITH_BOT ? (kTopPlane + 8 * kG16 > 24 ? kTopPlane + 8 * kG16 : 24) : kTopPlane + 4 * kG16;
+  static constexpr int kKStr = kPlanes * kPlane;         // bytes per step
+  static constexpr int kBLOff = 4 * kPlane, kCOff = 8 * kPlane;   // B_L and C planes behind the B_T planes
+  static constexpr int kXOff = kCK * kKStr;
+  static constexpr int kBytes = kXOff + NT * kXTauBytes; // one buffer
   static_assert(kXTauBytes % 1024 == 0, "a wave-wide copy must not straddle two tensors of XD");
-  static_assert((kCpt & (kCpt - 1)) == 0, "chunks per tensor row must be a power of two");
+  static_assert(kCpt == 2 || kCpt % 4 == 0, "a wave-wide copy of XD covers one step, or two halves of 32 lanes");
+  static_assert(CW % kElem == 0, "workgroup channel count must fill whole chunks");
+  static_assert(CW % 16 == 0, "boundary rows are copied 16 channels at a time");
   // byte offset inside a tensor's part of XD of channel `ch` (of the workgroup) for lane row r at step 0
   static __host__ __device__ constexpr uint32_t x_off(int r, int ch) {
     return (uint32_t)(((ch / kElem) * kHB + r) * 16 + (ch % kElem) * (int)sizeof(T));
   }
-  static constexpr int kTInstr = kCK * CW / 16;          // wave-wide copies that fill TOP (or BOT): 16 channels each
-  static constexpr int kXOff = kBChunks * 16;
-  static constexpr int kTOff = kXOff + kXChunks * 16;
-  static constexpr int kTKStr = UNI ? kKStr : CW * 64;   // bytes per step in TOP / BOT (UNI: the same as in BC)
-  static constexpr int kOOff = kTOff + kCK * kTKStr;
-  static constexpr int kBytes = kOOff + (WITH_BOT ? kCK * kTKStr : 0);   // one buffer
-  static_assert(CW % kElem == 0, "workgroup channel count must fill whole chunks");
-  static_assert(CW % 16 == 0, "boundary rows are copied 16 channels at a time");
+  // where the ghost of channel `ch` finds group 0 of the boundary row at step 0
+  static __host__ __device__ constexpr uint32_t top_off(int ch) { return (uint32_t)((kTopPlane + 4 * (ch / 16)) * kPlane + (ch % 16) * 16); }
+  static __host__ __device__ constexpr uint32_t bot_off(int ch) { return (uint32_t)((kBotPlane + 4 * (ch / 16)) * kPlane + (ch % 16) * 16); }
 };
 
 // One wave-wide direct load: lane i copies 16 bytes from its own global address to
@@ -313,36 +318,6 @@ __device__ __forceinline__ void lds_fill16(const void* src, char* lds_window) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(base) : "memory", "m0");
 }
 
-// The chunk -> (step, row, part of record) decomposition of the BC region depends only on the
-// thread.  It is worked out once (division by the odd record size) and kept as one packed word per
-// wave-wide copy: bits 0-3 row, 4-8 part, 9-10 step, bit 31 set if the chunk carries data.
-template <typename T, int NT, int CW, bool WITH_BOT, bool UNI, int NWAVES, bool KEEP>
-struct StagePlan {
-  using SG = Stage<T, NT, CW, WITH_BOT, UNI>;
-  static constexpr int kPer = NWAVES * 64;
-  static constexpr int kItB = (SG::kBChunks + kPer - 1) / kPer;
-  uint32_t bc[KEEP ? kItB : 1];
-  // `perk` chunks per step, of which the first kHB*reclen hold the records of the 16 lane rows
-  static __device__ __forceinline__ uint32_t word(int c, int nchunks, int perk, int reclen, int nparts) {
-    const int k = c / perk, rem = c - k * perk;
-    const int r = rem / reclen, part = rem - r * reclen;
-    return (c < nchunks && r < kHB && part < nparts) ? (0x80000000u | (k << 9) | (part << 4) | r) : 0u;
-  }
-  __device__ __forceinline__ void init(int wave, int lane) {
-    if constexpr (KEEP) {
-#pragma unroll
-      for (int i = 0; i < kItB; ++i) bc[i] = word(i * kPer + wave * 64 + lane, SG::kBChunks, SG::kKChunks, SG::kBRec, 12);
-    }
-  }
-  // Kernels short of registers work the word out again at every use instead of keeping it.
-  __device__ __forceinline__ uint32_t get_bc(int i, int wave, int lane) const {
-    uint32_t w;
-    if constexpr (KEEP) { w = bc[i]; } else { asm volatile("" : "+v"(lane)); w = word(i * kPer + wave * 64 + lane, SG::kBChunks, SG::kKChunks, SG::kBRec, 12); }
-    asm volatile("" : "+v"(w));   // unpack per use: the fields must not be hoisted into live registers
-    return w;
-  }
-};
-
 // Position of the stream index (index of A) + d, for 0 <= d < 19.  Strides below 19 (stacked
 // images) can wrap more than once.
 __device__ __forceinline__ Pos pos_after(const ScanParams& p, Pos A, int d) {
@@ -355,70 +330,6 @@ __device__ __forceinline__ Pos pos_after(const ScanParams& p, Pos A, int d) {
     if (q.col >= p.S) { q.col -= p.S; q.bnd += 1; }
   }
   return q;
-}
-
-// Stages the operands of a block of kCK steps; A is the position of the stream index
-// (first step of the block) - 15, from which every row's position in the block follows.
-template <typename T, int NT, int CW, bool WITH_BOT, bool UNI, bool STAGE_X, int NWAVES, bool KEEP>
-__device__ __forceinline__ void stage_block(const ScanParams& p, const StagePlan<T, NT, CW, WITH_BOT, UNI, NWAVES, KEEP>& plan, char* buf,
-                                            int b, Pos A, int e_wg0, int wave, int lane,
-                                            const T* x0, const T* x1, const T* x2, const T* x3) {
-  using SG = Stage<T, NT, CW, WITH_BOT, UNI>;
-  using PL = StagePlan<T, NT, CW, WITH_BOT, UNI, NWAVES, KEEP>;
-  // Source addresses are computed for every chunk and replaced by the page of zeros where the
-  // chunk is not a cell of the grid (selects, no divergent branches).  Cells of one image are
-  // addressed by 32-bit byte offsets from the image's base.
-  const int64_t img = (int64_t)b * p.Hs * p.W;
-  const char* zeros = reinterpret_cast<const char*>(p.zeros);
-  const char* bc_img = reinterpret_cast<const char*>(p.bt + img * p.bc_stride);
-#pragma unroll
-  for (int i = 0; i < PL::kItB; ++i) {
-    const uint32_t w = plan.get_bc(i, wave, lane);
-    const int r = w & 15, part = (w >> 4) & 31, k = (w >> 9) & 3;
-    const Pos q = pos_after(p, A, k - r + (kHB - 1));
-    const bool ok = (unsigned)q.bnd < (unsigned)p.nbands && q.col < p.W && r >= 1 && r <= band_rows(p, q.bnd);
-    const uint32_t off = (uint32_t)cell_of(p, q.bnd, r, q.col) * (uint32_t)(p.bc_stride * 4) + (uint32_t)(part * 16);
-    const char* src = ok ? bc_img + off : zeros;          // the packed record holds B_T, B_L, C back to back
-    if ((int)w < 0) lds_fill16<false>(src, buf + (i * PL::kPer + wave * 64) * 16);
-  }
-  if constexpr (STAGE_X) {
-    const int64_t img_bytes = img * p.E * (int64_t)sizeof(T);
-    for (int qi = wave; qi < NT * SG::kXTauInstr; qi += NWAVES) {
-      const int tau = qi / SG::kXTauInstr;                       // wave-uniform: one tensor per copy
-      const T* base = tau == 0 ? x0 : (tau == 1 ? x1 : (tau == 2 ? x2 : x3));
-      const char* t_img = reinterpret_cast<const char*>(base) + img_bytes;
-      const int c = (qi - tau * SG::kXTauInstr) * 64 + lane;      // chunk inside the tensor's part of XD
-      const int r = c & (kHB - 1), cc = (c >> kHBShift) & (SG::kCpt - 1), k = c / (kHB * SG::kCpt);
-      const Pos q = pos_after(p, A, k - r + (kHB - 1));
-      const int ch = e_wg0 + cc * SG::kElem;
-      const bool ok = (unsigned)q.bnd < (unsigned)p.nbands && q.col < p.W && r >= 1 && r <= band_rows(p, q.bnd) && ch < p.E;
-      const uint32_t off = (uint32_t)(cell_of(p, q.bnd, r, q.col) * p.E + ch) * (uint32_t)sizeof(T);
-      const char* src = ok ? t_img + off : zeros;
-      lds_fill16<false>(src, buf + SG::kXOff + qi * 1024);
-    }
-  }
-  // boundary rows were written earlier in this launch (or by the forward launch): read them
-  // past the L1.  One wave-wide copy moves the records of 16 channels at one step.
-  for (int qi = wave; qi < SG::kTInstr; qi += NWAVES) {
-    const int k = qi / (CW / 16), sub = qi - k * (CW / 16);
-    const int ch = e_wg0 + sub * 16 + (lane >> 2);
-    const Pos q = pos_after(p, A, k + (kHB - 1));    // the upper ghost is lane 0
-    const float* src = p.zeros;
-    if (!p.stacked && q.bnd >= 1 && q.bnd < p.nbands && q.col < p.W && ch < p.E)
-      src = p.top + ((((int64_t)(q.bnd - 1) * p.B + b) * p.W + q.col) * p.E + ch) * kN + (lane & 3) * 4;
-    lds_fill16<true>(src, buf + SG::kTOff + k * SG::kTKStr + sub * 1024);
-  }
-  if constexpr (WITH_BOT) {
-    for (int qi = wave; qi < SG::kTInstr; qi += NWAVES) {
-      const int k = qi / (CW / 16), sub = qi - k * (CW / 16);
-      const int ch = e_wg0 + sub * 16 + (lane >> 2);
-      const Pos q = pos_after(p, A, k);              // the lower ghost is lane 15
-      const float* src = p.zeros;
-      if (!p.stacked && q.bnd >= 0 && q.bnd + 1 < p.nbands && q.col < p.W && ch < p.E)
-        src = p.bot + (q.bnd + 1) * p.bot_stride + (((int64_t)b * p.W + q.col) * p.E + ch) * kN + (lane & 3) * 4;
-      lds_fill16<true>(src, buf + SG::kOOff + k * SG::kTKStr + sub * 1024);
-    }
-  }
 }
 
 // Every load the compiler knows about has returned (vmcnt 0, other counters untouched).  Placed
@@ -497,22 +408,25 @@ struct BlockPos {
   int kz;              // step of the block at which the row is at column 0 (>= kCK: never)
   uint32_t in_grid;    // bit k: the row is at a cell of the grid at step k
 };
-__device__ __forceinline__ BlockPos block_pos(const ScanParams& p, Pos A, int r, bool lane_ok) {
+// Lane row r is a row of the grid in the bands 0 .. row_bands(r) - 1 (none for a ghost lane; a row
+// beyond the height of the last band misses that one).  A lane constant.
+__device__ __forceinline__ int row_bands(const ScanParams& p, int r) {
+  return (r >= 1 && r <= kRB) ? p.nbands - 1 + (r <= p.rows_last ? 1 : 0) : 0;
+}
+// bits k < n of a block's steps
+__device__ __forceinline__ uint32_t steps_below(int n) { return (1u << (n < 0 ? 0 : (n > kCK ? kCK : n))) - 1u; }
+__device__ __forceinline__ BlockPos block_pos(const ScanParams& p, Pos A, int r, int rbands) {
   BlockPos q;
   const Pos at = pos_after(p, A, kHB - 1 - r);
   q.col0 = at.col; q.bnd0 = at.bnd;
   q.kw = p.S - q.col0;
   q.kz = q.col0 == 0 ? 0 : q.kw;
-  q.in_grid = 0;
-  const bool row = lane_ok && r >= 1 && r <= kRB;
-#pragma unroll
-  for (int k = 0; k < kCK; ++k) {
-    const bool wk = k >= q.kw;
-    const int bk = wk ? q.bnd0 + 1 : q.bnd0;
-    const int ck = wk ? q.col0 + k - p.S : q.col0 + k;
-    const bool in = row && (unsigned)bk < (unsigned)p.nbands && ck < p.W && r <= band_rows(p, bk);
-    q.in_grid |= in ? (1u << k) : 0u;
-  }
+  // in its band of the first step the row is on the grid while its column is below W (steps below kw and
+  // below W - col0), in the next band from step kw on while the new column, k - kw, is below W
+  const int w_left = p.W - q.col0;
+  const uint32_t m0 = steps_below(q.kw < w_left ? q.kw : w_left);
+  const uint32_t m1 = steps_below(q.kw + p.W) & ~steps_below(q.kw);
+  q.in_grid = ((unsigned)q.bnd0 < (unsigned)rbands ? m0 : 0u) | ((unsigned)(q.bnd0 + 1) < (unsigned)rbands ? m1 : 0u);
   return q;
 }
 __device__ __forceinline__ int clamp_band(const ScanParams& p, int bnd) { return bnd < 0 ? 0 : (bnd >= p.nbands ? p.nbands - 1 : bnd); }
@@ -520,6 +434,99 @@ __device__ __forceinline__ int clamp_band(const ScanParams& p, int bnd) { return
 // 0 has no row above) or into / out of the last band (fewer rows, no band below).
 __device__ __forceinline__ bool special_boundary(const ScanParams& p, int bnd_lo, int r) {
   return (!p.stacked && bnd_lo == 0 && r == 1) || (bnd_lo + 1 == p.nbands - 1 && (r > p.rows_last || r == kHB - 1));
+}
+
+// Stages the operands of a block of kCK steps.  A is the position of the stream index (first step
+// of the block) - 15; q and cell0 describe the lane's own row in that block (block_pos, and the cell
+// index of its position at the first step: what the lane's copies fetch is what the lane itself will
+// work on).  A wave copies the operands of one step of the block, wave % kCK (the waves that share a
+// step take its copies in turn), so a lane works out one cell per block.
+template <typename T, int NT, int CW, bool WITH_BOT, bool STAGE_X, int NWAVES>
+__device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int b, Pos A, const BlockPos& q, int cell0,
+                                            int e_wg0, int wave, int lane,
+                                            const T* x0, const T* x1, const T* x2, const T* x3) {
+  using SG = Stage<T, NT, CW, WITH_BOT>;
+  static_assert(NWAVES % kCK == 0, "every step of a block needs a wave");
+  constexpr int WPK = NWAVES / kCK;                       // waves per step
+  const int ks = wave & (kCK - 1), wsub = wave / kCK;     // (uniform) the wave's step, its turn among the waves of that step
+  // Source addresses are computed for every chunk and replaced by the page of zeros where the
+  // chunk is not a cell of the grid (selects, no divergent branches).  Cells of one image are
+  // addressed by 32-bit byte offsets from the image's base.
+  const int64_t img = (int64_t)b * p.Hs * p.W;
+  const char* zeros = reinterpret_cast<const char*>(p.zeros);
+  const char* bc_img = reinterpret_cast<const char*>(p.bt + img * p.bc_stride);
+  const int cstep = p.flip ? -1 : 1;                      // cells per column
+  const int wrapc = (kRB * p.W - p.S) * cstep;            // extra cells of a position reached through a band change
+  const int slot = lane >> kHBShift;
+  auto cell_at = [&](int k) { return cell0 + k * cstep + (k >= q.kw ? wrapc : 0); };
+  auto ok_at = [&](int k) { return ((q.in_grid >> k) & 1u) != 0; };
+  const int cell = cell_at(ks);
+  const bool ok = ok_at(ks);
+  char* kbuf = buf + ks * SG::kKStr;
+  // B_T, B_L, C: a copy moves the four state groups (lane >> 4) of one tensor for the 16 lane rows
+#pragma unroll
+  for (int tsr = 0; tsr < 3; ++tsr)
+    if (tsr % WPK == wsub) {
+      const uint32_t off = (uint32_t)cell * (uint32_t)(p.bc_stride * 4) + (uint32_t)(tsr * kN * 4 + slot * 16);
+      lds_fill16<false>(ok ? bc_img + off : zeros, kbuf + tsr * 4 * SG::kPlane);
+    }
+  if constexpr (STAGE_X) {
+    const int64_t img_bytes = img * p.E * (int64_t)sizeof(T);
+    if constexpr (SG::kCpt >= 4) {   // one step per copy: lanes = (channel chunk, row)
+      constexpr int per = SG::kCpt / 4;                    // copies per tensor and step
+#pragma unroll
+      for (int tau = 0; tau < NT; ++tau) {
+        const T* base = tau == 0 ? x0 : (tau == 1 ? x1 : (tau == 2 ? x2 : x3));
+        const char* t_img = reinterpret_cast<const char*>(base) + img_bytes;
+#pragma unroll
+        for (int i = 0; i < per; ++i)
+          if ((3 + tau * per + i) % WPK == wsub) {
+            const int ch = e_wg0 + (i * 4 + slot) * SG::kElem;
+            const uint32_t off = (uint32_t)(cell * p.E + ch) * (uint32_t)sizeof(T);
+            lds_fill16<false>((ok && ch < p.E) ? t_img + off : zeros,
+                              buf + SG::kXOff + tau * SG::kXTauBytes + ks * SG::kXStepBytes + i * 1024);
+          }
+      }
+    } else {                         // two steps per copy: lanes = (step, channel chunk, row); the wave of the even step copies
+      if ((ks & 1) == 0) {
+        const bool hi = lane >= 32;
+        const int cell2 = hi ? cell_at(ks + 1) : cell;
+        const bool ok2 = hi ? ok_at(ks + 1) : ok;
+        const int ch = e_wg0 + (slot & 1) * SG::kElem;
+        const uint32_t off = (uint32_t)(cell2 * p.E + ch) * (uint32_t)sizeof(T);
+#pragma unroll
+        for (int tau = 0; tau < NT; ++tau) {
+          const T* base = tau == 0 ? x0 : (tau == 1 ? x1 : (tau == 2 ? x2 : x3));
+          const char* t_img = reinterpret_cast<const char*>(base) + img_bytes;
+          lds_fill16<false>((ok2 && ch < p.E) ? t_img + off : zeros, buf + SG::kXOff + tau * SG::kXTauBytes + ks * SG::kXStepBytes);
+        }
+      }
+    }
+  }
+  // boundary rows were written earlier in this launch (or by the forward launch): read them
+  // past the L1.  One wave-wide copy moves the four state groups (lane >> 4) of 16 channels at one step.
+#pragma unroll
+  for (int g = 0; g < SG::kG16; ++g)
+    if ((3 + g) % WPK == wsub) {
+      const int ch = e_wg0 + g * 16 + (lane & (kHB - 1));
+      const Pos qa = pos_after(p, A, ks + (kHB - 1));    // the upper ghost is lane 0
+      const float* src = p.zeros;
+      if (!p.stacked && qa.bnd >= 1 && qa.bnd < p.nbands && qa.col < p.W && ch < p.E)
+        src = p.top + ((((int64_t)(qa.bnd - 1) * p.B + b) * p.W + qa.col) * p.E + ch) * kN + slot * 4;
+      lds_fill16<true>(src, kbuf + (SG::kTopPlane + 4 * g) * SG::kPlane);
+    }
+  if constexpr (WITH_BOT) {
+#pragma unroll
+    for (int g = 0; g < SG::kG16; ++g)
+      if ((3 + SG::kG16 + g) % WPK == wsub) {
+        const int ch = e_wg0 + g * 16 + (lane & (kHB - 1));
+        const Pos qa = pos_after(p, A, ks);              // the lower ghost is lane 15
+        const float* src = p.zeros;
+        if (!p.stacked && qa.bnd >= 0 && qa.bnd + 1 < p.nbands && qa.col < p.W && ch < p.E)
+          src = p.bot + (qa.bnd + 1) * p.bot_stride + (((int64_t)b * p.W + qa.col) * p.E + ch) * kN + slot * 4;
+        lds_fill16<true>(src, kbuf + (SG::kBotPlane + 4 * g) * SG::kPlane);
+      }
+  }
 }
 
 // ------------------------------------------------------------------------------------ forward
@@ -549,9 +556,9 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   constexpr int CW = NW * CS * EC;
   constexpr bool PERM = true;
   constexpr bool AHEAD = EC == 1 && STAGE_X;   // operands of step t+1 are fetched from LDS during step t
-  using SG = Stage<T, 3, CW, false, true>;
+  using SG = Stage<T, 3, CW, false>;
   extern __shared__ float4 smem[];
-  char* lds = reinterpret_cast<char*>(smem);       // two staging buffers and 256 bytes of slack
+  char* lds = reinterpret_cast<char*>(smem);       // two staging buffers
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   int lb = logical_block(p.nwg);
@@ -575,14 +582,13 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     p.rows_last = p.H - (p.nbands - 1) * kRB;
   }
   const int slot = lane >> kHBShift, r = lane & (kHB - 1);
+  const int rbands = row_bands(p, r);
   const int ch_loc = (wave * CS + slot) * EC;      // first channel of the lane inside the workgroup
   const int e_raw = e_wg0 + ch_loc;
   const bool ch_ok = e_raw < p.E;                  // idle lanes still take part in staging and barriers
   const int e0 = ch_ok ? e_raw : p.E - EC;
   // every byte a lane may read is finite from the start (pads are never written again)
-  for (int i = threadIdx.x; i < (2 * SG::kBytes + 256) / 16; i += NW * 64) smem[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-  StagePlan<T, 3, CW, false, true, NW, true> plan;
-  plan.init(wave, lane);
+  for (int i = threadIdx.x; i < 2 * SG::kBytes / 16; i += NW * 64) smem[i] = make_float4(0.f, 0.f, 0.f, 0.f);
 
   float a2t[EC][kN], a2l[EC][kN], dsk[EC];
 #pragma unroll
@@ -599,9 +605,9 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   const T* DL = static_cast<const T*>(p.dL);
   const T* DY = DL;   // not staged by the forward (NT = 3)
   const float ninf = -__builtin_huge_valf();
-  const int64_t cell0 = (int64_t)b * p.Hs * p.W;
+  const int64_t img_cell0 = (int64_t)b * p.Hs * p.W;
   // (B,H,W,E) tensors are addressed as image base (uniform) + 32-bit byte offset (per lane)
-  const int64_t img_bytes = cell0 * p.E * (int64_t)sizeof(T);
+  const int64_t img_bytes = img_cell0 * p.E * (int64_t)sizeof(T);
   char* Yimg = static_cast<char*>(p.y) + img_bytes;
   const char* Ximg = reinterpret_cast<const char*>(X) + img_bytes;
   const char* DTimg = reinterpret_cast<const char*>(DT) + img_bytes;
@@ -611,9 +617,12 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   const float g1 = r == 0 ? 1.f : 0.f;             // the ghost's T input coefficient
   const uint32_t wrap_adj = (uint32_t)(kRB * p.W - p.S) * estep;   // extra offset of a cell reached through a band change
 
-  // byte offsets of the lane's records inside a staging buffer (step 0)
-  const uint32_t rec_off = r == 0 ? SG::kTOff + ch_loc * kN * 4 : r * SG::kBStride * 4;
-  const uint32_t rec_cstep = r == 0 ? kN * 4 : 0;   // the ghost reads a record per channel, grid rows share theirs
+  // byte offsets of the lane's operand groups inside a staging buffer (step 0, group 0): a grid row
+  // reads B_T, B_L, C of its cell; the ghost reads the row above as its B_T (and row 0 of the B_L and C
+  // planes, zeros, as stand-ins for the other two, which it multiplies by 0)
+  const uint32_t row_off = r * 16;
+  const uint32_t rec_off = r == 0 ? SG::top_off(ch_loc) : row_off;
+  const uint32_t rec_cstep = r == 0 ? 16 : 0;   // the ghost reads a record per channel, grid rows share theirs
   const uint32_t xd_off = SG::kXOff + SG::x_off(r, ch_loc);
   constexpr uint32_t kXK = SG::kXStepBytes;   // XD bytes per step
 
@@ -638,24 +647,23 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     } else {   // straight from memory, for the lane's position at step k of the current block
 #pragma unroll
       for (int c = 0; c < EC; ++c) { o.xv[c] = 0.f; o.dtv[c] = 0.f; o.dlv[c] = 0.f; }
-      if ((bp.in_grid >> k) & 1u) {
+      if (ch_ok && ((bp.in_grid >> k) & 1u)) {
         const uint32_t off = cell_off0 + (uint32_t)k * estep + (k >= bp.kw ? wrap_adj : 0u);
         IO<T>::template ldv<EC>(reinterpret_cast<const T*>(Ximg + off), o.xv);
         IO<T>::template ldv<EC>(reinterpret_cast<const T*>(DTimg + off), o.dtv);
         IO<T>::template ldv<EC>(reinterpret_cast<const T*>(DLimg + off), o.dlv);
       }
     }
-    // a grid row reads B_T, B_L, C of its cell; the ghost reads the row above as its B_T (and
-    // the finite records next to it as stand-ins for the other two, which it multiplies by 0)
     const char* rec = bufc + rec_off + k * SG::kKStr;
+    const char* row = bufc + row_off + k * SG::kKStr;
 #pragma unroll
     for (int c = 0; c < EC; ++c)
 #pragma unroll
-      for (int q = 0; q < 4; ++q) o.bt[c][q] = reinterpret_cast<const float4*>(rec + c * rec_cstep)[q];
+      for (int q = 0; q < 4; ++q) o.bt[c][q] = *reinterpret_cast<const float4*>(rec + c * rec_cstep + q * SG::kPlane);
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      o.bl[q] = reinterpret_cast<const float4*>(rec + kN * 4)[q];
-      o.cc[q] = WRITE_Y ? reinterpret_cast<const float4*>(rec + 2 * kN * 4)[q] : make_float4(0, 0, 0, 0);
+      o.bl[q] = *reinterpret_cast<const float4*>(row + SG::kBLOff + q * SG::kPlane);
+      o.cc[q] = WRITE_Y ? *reinterpret_cast<const float4*>(row + SG::kCOff + q * SG::kPlane) : make_float4(0, 0, 0, 0);
     }
   };
 
@@ -684,7 +692,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     const float offL = col0 ? ninf : K.oL;
     const float cT = col0 ? K.cT0 : K.cT;
     const float cL = col0 ? K.cL0 : K.cL;
-    const bool inr = (bp.in_grid >> k) & 1u;
+    const bool inr = ch_ok && ((bp.in_grid >> k) & 1u);
     float yv[EC];
 #pragma unroll
     for (int c = 0; c < EC; ++c) {
@@ -743,19 +751,24 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   };
 
   Pos A = pos_of(p, m_lo * kCK - (kHB - 1));     // position of the stream index t0 - 15 (wave-uniform)
-  stage_block<T, 3, CW, false, true, STAGE_X, NW, true>(p, plan, lds, b, A, e_wg0, wave, lane, X, DT, DL, DY);
+  bp = block_pos(p, A, r, rbands);
+  int cell0 = cell_of(p, bp.bnd0, r, bp.col0);   // cell index of the lane's position at the first step of the block
+  stage_block<T, 3, CW, false, STAGE_X, NW>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
   staging_fence();
   Ops opsA, opsB;
   if constexpr (AHEAD) fetch(lds, 0, opsA);
   int cur = 0;
   for (int m = m_lo; m < m_hi; ++m) {
     const bool last = m + 1 == m_hi;
+    // the next block: where the lane's row will be is also what the lane's copies fetch
+    const Pos An = pos_after(p, A, kCK);
+    const BlockPos bpn = block_pos(p, An, r, rbands);
+    const int celln = cell_of(p, bpn.bnd0, r, bpn.col0);
     if (!last)
-      stage_block<T, 3, CW, false, true, STAGE_X, NW, true>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, pos_after(p, A, kCK), e_wg0, wave, lane, X, DT, DL, DY);
-    bp = block_pos(p, A, r, ch_ok);
+      stage_block<T, 3, CW, false, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, An, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
     K = lane_consts<false>(p, clamp_band(p, bp.bnd0), r, ch_ok);
     per_step_K = __any(bp.kw < kCK && special_boundary(p, bp.bnd0, r));
-    cell_off0 = (uint32_t)(cell_of(p, bp.bnd0, r, bp.col0) * p.E + e0) * (uint32_t)sizeof(T);
+    cell_off0 = (uint32_t)(cell0 * p.E + e0) * (uint32_t)sizeof(T);
     // Snapshot of the state before the block (after step t0-1) for the lanes whose previous
     // position was a cell of the grid; the others hold nothing the backward needs.  The stores are
     // issued inside the first step, each group of four states just before it is overwritten: the
@@ -772,7 +785,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     const char* bufn = lds + (cur ^ 1) * SG::kBytes;
     // (uniform) some lane writes y at each of the first three steps: the wave issues at least
     // three stores between the copies for the next block and the barrier that ends this one
-    const bool y_thrice = WRITE_Y && __any((bp.in_grid & 7u) == 7u);
+    const bool y_thrice = WRITE_Y && __any(ch_ok && (bp.in_grid & 7u) == 7u);
     auto next_block_landed = [&] {
       // the stores issued since (snapshot, y) need not have completed, only the copies before them
       if (snapped) {
@@ -812,8 +825,9 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
       __syncthreads();
     }
     cur ^= 1;
-    A.col += kCK;
-    if (A.col >= p.S) { A.col -= p.S; A.bnd += 1; }
+    A = An;
+    bp = bpn;
+    cell0 = celln;
   }
   if (SLICED && ch_ok && m_hi < (my_band + 1) * p.sl_nbb) {   // more of the band to come: hand the state to the next launch
 #pragma unroll
@@ -852,7 +866,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   constexpr int SLOT = 3 * 64;           // float2s per wave in one exchange buffer
   constexpr int CW = NW * CS;
   constexpr bool PERM = true;
-  using SG = Stage<T, 4, CW, true, false>;
+  using SG = Stage<T, 4, CW, true>;
   extern __shared__ float4 smem[];
   // Exchange buffers for the channel sums of one (step, half of the states): two of them, used
   // alternately, so that one barrier per exchange is enough (a buffer is rewritten two exchanges
@@ -884,6 +898,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   }
   const int e_wg0 = eg * CW;
   const int slot = lane >> kHBShift, r = lane & (kHB - 1);
+  const int rbands = row_bands(p, r);
   const int ch_loc = wave * CS + slot;
   const int e_raw = e_wg0 + ch_loc;
   const bool ch_ok = e_raw < p.E;           // padding lanes/waves still take part in the barriers
@@ -893,10 +908,10 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
     mine[spos<true>(r)] = p.A2T[e * kN + r];
     mine[kN + spos<true>(r)] = p.A2L[e * kN + r];
   }
+  // planes that no copy writes must hold finite values from the start
+  for (int i = threadIdx.x; i < 2 * SG::kBytes / 16; i += NW * 64) reinterpret_cast<float4*>(lds)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
   const uint32_t a_base_off = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) float*)(a_lds + ch_loc * (2 * kN)));
   const float dsk = p.Df[e];
-  StagePlan<T, 4, CW, true, false, NW, false> plan;
-  plan.init(wave, lane);
   settle_loads();
 
   const T* X = static_cast<const T*>(p.x);
@@ -904,9 +919,9 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   const T* DL = static_cast<const T*>(p.dL);
   const T* DY = static_cast<const T*>(p.dy);
   const float ninf = -__builtin_huge_valf();
-  const int64_t cell0 = (int64_t)b * p.Hs * p.W;
+  const int64_t img_cell0 = (int64_t)b * p.Hs * p.W;
   // (B,H,W,E) tensors: image base (uniform) + 32-bit byte offset (per lane)
-  const int64_t img_bytes = cell0 * p.E * (int64_t)sizeof(T);
+  const int64_t img_bytes = img_cell0 * p.E * (int64_t)sizeof(T);
   const char* Ximg = reinterpret_cast<const char*>(X) + img_bytes;
   const char* DTimg = reinterpret_cast<const char*>(DT) + img_bytes;
   const char* DLimg = reinterpret_cast<const char*>(DL) + img_bytes;
@@ -916,7 +931,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   char* DDLimg = static_cast<char*>(p.ddL) + img_bytes;
   char* BOTimg = reinterpret_cast<char*>(p.bot + (int64_t)b * p.W * p.E * kN);   // + band * bot_stride
   // per-workgroup channel sums: [channel group][cell][C, B_T, B_L][16]
-  char* PARTimg = reinterpret_cast<char*>(p.part + ((int64_t)eg * p.Ptot + cell0) * (3 * kN));
+  char* PARTimg = reinterpret_cast<char*>(p.part + ((int64_t)eg * p.Ptot + img_cell0) * (3 * kN));
 
   float accAT[kN], accAL[kN], accD = 0.f;
   float muT[kN], muL[kN];
@@ -940,19 +955,20 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   // its advance per step: a grid row reads (B_T, B_L, C) of its cell; the upper ghost (lane 0)
   // reads the row above as its B_T; the lower ghost (lane 15) reads the row of mu_T below as its C.
   // The neighbouring records that a ghost reads in the other two places are finite and meet zeros.
-  const uint32_t rec_off = r == 0 ? SG::kTOff + ch_loc * kN * 4
-                                  : (r == kHB - 1 ? SG::kOOff + ch_loc * kN * 4 - 2 * kN * 4 : r * SG::kBStride * 4);
-  const uint32_t rec_kstr = (r == 0 || r == kHB - 1) ? SG::kTKStr : SG::kKStr;
+  // The other two reads of a ghost land 4 and 8 planes from its boundary row: boundary rows of other
+  // channels, operands of other rows or planes nobody writes, finite all of them, and they meet zeros.
+  const uint32_t rec_off = r == 0 ? SG::top_off(ch_loc) : (r == kHB - 1 ? SG::bot_off(ch_loc) - SG::kCOff : r * 16);
   const uint32_t xd_off = SG::kXOff + SG::x_off(r, ch_loc);
   constexpr uint32_t kXK = SG::kXStepBytes;   // XD bytes per step
-  // the sum that this thread adds up in the exchange (one float of one lane's float2, one tensor):
-  // it belongs to lane row f_r, which is f_d positions ahead of this thread's own row
+  // The sum that this thread adds up in the exchange belongs to its own lane row r: one float of
+  // the float2 of the lane (slot f_s, row r) for tensor f_v (a whole float2 where a workgroup has
+  // fewer threads than sums).  The first 6 (3) waves do the adding.
   constexpr bool PAIRS = NW * 64 < 2 * SLOT;   // fewer threads than sums: a thread takes a pair
-  const int fid = PAIRS ? wave * 64 + lane : wave * (2 * SLOT / NW) + lane;
-  const bool f_on = PAIRS ? fid < SLOT : lane < 2 * SLOT / NW;
-  const int f_it = PAIRS ? fid : fid >> 1, f_comp = PAIRS ? 0 : fid & 1;
-  const int f_r = f_it & (kHB - 1), f_s = (f_it & 63) >> kHBShift, f_v = f_it >> 6;
-  const int f_d = r - f_r;
+  const int f_combo = wave * 4 + slot;
+  const bool f_on = f_combo < (PAIRS ? 12 : 24);
+  const int f_v = PAIRS ? f_combo >> 2 : f_combo >> 3, f_s = PAIRS ? f_combo & 3 : (f_combo >> 1) & 3;
+  const int f_comp = PAIRS ? 0 : f_combo & 1;
+  const int f_it = f_v * 64 + f_s * kHB + r;
   const uint32_t f_sub = (uint32_t)(f_v * kN + f_s * 4 + f_comp) * (uint32_t)sizeof(float);
   const float g1 = r == 0 ? 1.f : 0.f;
 
@@ -963,7 +979,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
 
   // per block: where the lane (and the lane row whose sums this thread adds up) is, and what
   // depends on it
-  BlockPos bp, fp;
+  BlockPos bp;
   LaneK K;
   float gb1 = 0.f;              // 1 on an active lower ghost: lambda = 1 * (row of mu_T below)
   uint32_t cell_off0 = 0;       // byte offset in a (H,W,E) image of the lane's cell at the first step of the block
@@ -977,8 +993,8 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
 
   // state snapshot at the start of the block whose position A is given (zero for lanes that were not under way)
   float cknext[kN];
-  auto load_ckpt = [&](int mm, Pos Am) {
-    if (mm == 0 || !snapshot_lane(p, pos_after(p, Am, kHB - 1 - r), r, ch_ok)) {
+  auto load_ckpt = [&](int mm, bool take) {   // take: the forward kept the lane's state before block mm
+    if (mm == 0 || !take) {
 #pragma unroll
       for (int n = 0; n < kN; ++n) cknext[n] = 0.f;
     } else {
@@ -998,8 +1014,11 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   };
 
   Pos A = pos_of(p, (m_hi - 1) * kCK - (kHB - 1));   // position of the stream index t0 - 15 (wave-uniform)
-  load_ckpt(m_hi - 1, A);
-  stage_block<T, 4, CW, true, false, STAGE_X, NW, false>(p, plan, lds, b, A, e_wg0, wave, lane, X, DT, DL, DY);
+  __syncthreads();   // the zeros are in place before the first copies land on them
+  bp = block_pos(p, A, r, rbands);
+  bool ck_take = snapshot_lane(p, Pos{bp.bnd0, bp.col0}, r, ch_ok);   // the lane restores a snapshot for the block to come
+  load_ckpt(m_hi - 1, ck_take);
+  stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds, b, A, bp, cell_of(p, bp.bnd0, r, bp.col0), e_wg0, wave, lane, X, DT, DL, DY);
   staging_fence();
   int cur = 0;
   int xpar = 0;   // exchange buffer in use
@@ -1011,14 +1030,21 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
 #pragma unroll
     for (int n = 0; n < kN; ++n) ck0[n] = cknext[n];
     const Pos Aprev = pos_before(A);
-    if (m > m_lo)
-      stage_block<T, 4, CW, true, false, STAGE_X, NW, false>(p, plan, lds + (cur ^ 1) * SG::kBytes, b, Aprev, e_wg0, wave, lane, X, DT, DL, DY);
-    bp = block_pos(p, A, r, ch_ok);
-    fp = block_pos(p, A, f_r, f_on);
+    {   // the block before: where the lane's row will be is also what the lane's copies fetch
+      const BlockPos bpn = block_pos(p, Aprev, r, rbands);
+      ck_take = snapshot_lane(p, Pos{bpn.bnd0, bpn.col0}, r, ch_ok);
+      if (m > m_lo)
+        stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, cell_of(p, bpn.bnd0, r, bpn.col0),
+                                                 e_wg0, wave, lane, X, DT, DL, DY);
+    }
+    bp = block_pos(p, A, r, rbands);
     band_consts(bp.bnd0);
     per_step_K = __any(bp.kw < kCK && special_boundary(p, bp.bnd0, r));
-    cell_off0 = (uint32_t)(cell_of(p, bp.bnd0, r, bp.col0) * p.E + e) * (uint32_t)sizeof(T);
-    f_off0 = (uint32_t)cell_of(p, fp.bnd0, f_r, fp.col0) * (uint32_t)(3 * kN * sizeof(float)) + f_sub;
+    {
+      const int cell0 = cell_of(p, bp.bnd0, r, bp.col0);
+      cell_off0 = (uint32_t)(cell0 * p.E + e) * (uint32_t)sizeof(T);
+      f_off0 = (uint32_t)cell0 * (uint32_t)(3 * kN * sizeof(float)) + f_sub;
+    }
 
     // The 16 states are swept in two halves of 8 (state groups 0,1 then 2,3), each half
     // recomputing and then back-propagating the whole block: only 5 x 8 recomputed states are
@@ -1050,7 +1076,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
           if constexpr (STAGE_X) {
             const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
             xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + SG::kXTauBytes / sizeof(T)); dlv = IO<T>::ld(xr + 2 * SG::kXTauBytes / sizeof(T));
-          } else if ((bp.in_grid >> k) & 1u) {
+          } else if (ch_ok && ((bp.in_grid >> k) & 1u)) {
             const uint32_t off = cell_off0 + (uint32_t)k * estep + (k >= bp.kw ? wrap_adj : 0u);
             xv = IO<T>::ld(reinterpret_cast<const T*>(Ximg + off));
             dtv = IO<T>::ld(reinterpret_cast<const T*>(DTimg + off));
@@ -1061,14 +1087,15 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
           uint32_t a_off = a_base_off;
           asm volatile("" : "+v"(a_off));
           const lds_float4* a_mine = (const lds_float4*)(uintptr_t)a_off;
-          const char* rec = bufc + (rec_off + k * rec_kstr);
+          const char* rec = bufc + (rec_off + k * SG::kKStr);
           const float sT = __builtin_fmaf(cT * dtv, xv, g1);
           const float sL = cL * dlv * xv;
 #pragma unroll
           for (int mgl = 0; mgl < 2; ++mgl) {
             const int mg = 2 * half + mgl;
             const v4f_t at4 = a_mine[mg], al4 = a_mine[kN / 4 + mg];
-            const float4 b4 = reinterpret_cast<const float4*>(rec)[mg], l4 = reinterpret_cast<const float4*>(rec + kN * 4)[mg];
+            const float4 b4 = *reinterpret_cast<const float4*>(rec + mg * SG::kPlane);
+            const float4 l4 = *reinterpret_cast<const float4*>(rec + SG::kBLOff + mg * SG::kPlane);
             const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
             const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w};
             float aT[4], aL[4];   // gates before chains, see the forward kernel
@@ -1098,7 +1125,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
         const int t = t0 + k;
         if (half == 1 && k == 0) staging_landed();   // before the last stores of the block, see the forward kernel
         // the states of the later steps are dead by now: their registers take the next snapshot
-        if (half == 1 && k == (kCK > 1 ? 1 : 0) && m > m_lo) load_ckpt(m - 1, Aprev);
+        if (half == 1 && k == (kCK > 1 ? 1 : 0) && m > m_lo) load_ckpt(m - 1, ck_take);
         if (t < p.T_total) {
           if (per_step_K) band_consts(k >= bp.kw ? bp.bnd0 + 1 : bp.bnd0);
           const bool col0 = bp.kz == k;
@@ -1106,7 +1133,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
           const float offL = col0 ? ninf : K.oL;
           const float cT = col0 ? K.cT0 : K.cT;
           const float cL = col0 ? K.cL0 : K.cL;
-          const bool inr = (bp.in_grid >> k) & 1u;
+          const bool inr = ch_ok && ((bp.in_grid >> k) & 1u);
           const uint32_t goff = cell_off0 + (uint32_t)k * estep + (k >= bp.kw ? wrap_adj : 0u);
           float xv = 0.f, dtv = 0.f, dlv = 0.f, dyv = 0.f;
           if constexpr (STAGE_X) {
@@ -1122,7 +1149,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
           uint32_t a_off = a_base_off;
           asm volatile("" : "+v"(a_off));
           const lds_float4* a_mine = (const lds_float4*)(uintptr_t)a_off;
-          const char* rec = bufc + (rec_off + k * rec_kstr);
+          const char* rec = bufc + (rec_off + k * SG::kKStr);
           const float qT = cT * dtv * xv, qL = cL * dlv * xv;   // zero on lanes that are not grid cells
           const float dyl = dyv + gb1;
           float sT = 0.f, sL = 0.f, zT = 0.f, zL = 0.f;
@@ -1135,8 +1162,9 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
           for (int mgl = 0; mgl < 2; ++mgl) {
             const int mg = 2 * half + mgl;
             const v4f_t at4 = a_mine[mg], al4 = a_mine[kN / 4 + mg];
-            const float4 b4 = reinterpret_cast<const float4*>(rec)[mg], l4 = reinterpret_cast<const float4*>(rec + kN * 4)[mg];
-            const float4 c4 = reinterpret_cast<const float4*>(rec + 2 * kN * 4)[mg];
+            const float4 b4 = *reinterpret_cast<const float4*>(rec + mg * SG::kPlane);
+            const float4 l4 = *reinterpret_cast<const float4*>(rec + SG::kBLOff + mg * SG::kPlane);
+            const float4 c4 = *reinterpret_cast<const float4*>(rec + SG::kCOff + mg * SG::kPlane);
             const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
             const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w}, cq[4] = {c4.x, c4.y, c4.z, c4.w};
             float vC[4], vBT[4], vBL[4];
@@ -1195,8 +1223,8 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
           // ---- across the waves of the workgroup: the per-wave slots (this half's two state
           // groups) are added in wave order, one sum per thread, the same share for every wave
           __syncthreads();
-          if ((fp.in_grid >> k) & 1u) {
-            const uint32_t off = f_off0 + (uint32_t)k * pstep + (k >= fp.kw ? pwrap_adj : 0u) + (uint32_t)(2 * half * sizeof(float));
+          if (f_on && ((bp.in_grid >> k) & 1u)) {
+            const uint32_t off = f_off0 + (uint32_t)k * pstep + (k >= bp.kw ? pwrap_adj : 0u) + (uint32_t)(2 * half * sizeof(float));
             if constexpr (PAIRS) {
               const float2* sl = slots + xpar * NW * SLOT + f_it;
               float2 s = sl[0];
@@ -1374,11 +1402,11 @@ inline size_t align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
 // copy of A and two staging buffers.  A compute unit has 160 KB.
 constexpr size_t kLdsPerWorkgroup = 160 * 1024;
 template <typename T, int EC, int NW = kFwdWaves>
-constexpr size_t fwd_lds_bytes() { return 256 + 2 * (size_t)Stage<T, 3, NW * 4 * EC, false, true>::kBytes; }
+constexpr size_t fwd_lds_bytes() { return 2 * (size_t)Stage<T, 3, NW * 4 * EC, false>::kBytes; }
 template <typename T, int NW = kBwdWaves>
 constexpr size_t bwd_lds_bytes() {
   return sizeof(float4) * NW * 3 * 64 + sizeof(float) * NW * 4 * 2 * kN + 256 +
-         2 * (size_t)Stage<T, 4, NW * 4, true, false>::kBytes;
+         2 * (size_t)Stage<T, 4, NW * 4, true>::kBytes;
 }
 static_assert(fwd_lds_bytes<float, 1>() <= kLdsPerWorkgroup && fwd_lds_bytes<bf16_t, 1>() <= kLdsPerWorkgroup, "forward staging must fit the LDS");
 static_assert(bwd_lds_bytes<float>() <= kLdsPerWorkgroup && bwd_lds_bytes<bf16_t>() <= kLdsPerWorkgroup, "backward staging must fit the LDS");
@@ -1481,11 +1509,12 @@ Geometry make_geometry(const m2d_desc* d) {
   }
   // forward: two channels per lane where that saves rounds of workgroups (one workgroup per compute
   // unit at a time, 256 units) and the two staging buffers of such a workgroup fit the LDS (bf16
-  // operands: 112 KB; fp32 ones do not).  A sweep with two channels per lane takes about 1.8 times
+  // operands only).  A sweep with two channels per lane takes about 1.8 times
   // as long as one with a single channel (measured: 1.6 at 28x28, 2.0 at 56x56), so it pays only
   // when it at least halves the rounds: 128 channels x 128 images, not 32 channels x 256 images
   // (where half of every workgroup would idle).
-  const size_t lds_ec2 = d->dtype == M2D_BF16 ? fwd_lds_bytes<bf16_t, 2>() : fwd_lds_bytes<float, 2>();
+  // (fp32 operands: such a kernel would need more registers than a lane has, and is not built)
+  const size_t lds_ec2 = d->dtype == M2D_BF16 ? fwd_lds_bytes<bf16_t, 2>() : kLdsPerWorkgroup + 1;
   const int64_t wg1 = (int64_t)B * ((d->E + kFwdWaves * g.CS - 1) / (kFwdWaves * g.CS));
   const int64_t wg2 = (int64_t)B * ((d->E + kFwdWaves * g.CS * 2 - 1) / (kFwdWaves * g.CS * 2));
   const bool ec2 = (d->E % 2 == 0) && lds_ec2 <= kLdsPerWorkgroup && 18 * ((wg2 + 255) / 256) < 10 * ((wg1 + 255) / 256);
@@ -1503,6 +1532,11 @@ Geometry make_geometry(const m2d_desc* d) {
   g.fwd_bpb = (d->E + g.fwd_nw * g.CS * g.fwd_ec - 1) / (g.fwd_nw * g.CS * g.fwd_ec);
   g.fwd_wpb = g.fwd_bpb * g.fwd_nw;
   g.bwd_nw = (!g.stacked && wg_half > (int64_t)B * groups && wg_half * together <= room) ? kFwdHalfWaves : kBwdWaves;
+  if (const char* ev = getenv("M2D_DEBUG_NW")) {   // experiment
+    const int v = atoi(ev);
+    if (!g.stacked && !ec2 && (v & 1)) { g.fwd_nw = kFwdHalfWaves; g.fwd_bpb = (d->E + g.fwd_nw * g.CS * g.fwd_ec - 1) / (g.fwd_nw * g.CS * g.fwd_ec); g.fwd_wpb = g.fwd_bpb * g.fwd_nw; }
+    if (!g.stacked && (v & 2)) g.bwd_nw = kFwdHalfWaves;
+  }
   g.bwd_bpb = (d->E + g.bwd_nw * g.CS - 1) / (g.bwd_nw * g.CS);
   g.bwd_wpb = g.bwd_bpb * g.bwd_nw;
   g.stage_x = (d->E % (d->dtype == M2D_BF16 ? 8 : 4)) == 0;
@@ -1626,10 +1660,12 @@ int launch_fwd(const ScanParams& sp0, const m2d_desc* d, const Geometry& g, bool
       return g.stage_x ? launch_fwd_mode<T, 1, true, kModeSliced>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 1, false, kModeSliced>(sp, ckpt, write_y, st);
     }
     if (g.stacked) {
+      if constexpr (sizeof(T) == 2)   // (fp32 operands of two channels per lane do not fit the LDS: never chosen, not built)
       if (g.fwd_ec == 2)
         return g.stage_x ? launch_fwd_mode<T, 2, true, kModeStacked>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 2, false, kModeStacked>(sp, ckpt, write_y, st);
       return g.stage_x ? launch_fwd_mode<T, 1, true, kModeStacked>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 1, false, kModeStacked>(sp, ckpt, write_y, st);
     }
+    if constexpr (sizeof(T) == 2)
     if (g.fwd_ec == 2)
       return g.stage_x ? launch_fwd_mode<T, 2, true, kModeSweep>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 2, false, kModeSweep>(sp, ckpt, write_y, st);
     if (g.fwd_nw == kFwdHalfWaves)
