@@ -267,6 +267,7 @@ template <bool PERM> __device__ __forceinline__ constexpr int sinv(int pos) {
 //     planes 12..    TOP: plane 12 + 4*h + g holds, for the channels 16h..16h+15 of the workgroup, state
 //                         group g of the last row of the band above at column t0+k;
 //     then (adjoint) BOT: the same for the muT of the first row of the band below at column t0+k-15;
+//     then           K  : chunk r holds the gate offsets and input coefficients of lane row r at this step;
 //   then XD: per tensor (x, deltaT, deltaL[, dy]), step k and chunk of channels, the 16 lane rows side by
 //        side (chunk index = ((tensor*kCK + k)*kCpt + channel chunk)*16 + r); needs E to be a multiple
 //        of a chunk.
@@ -287,7 +288,8 @@ struct Stage {
   static constexpr int kBotPlane = kTopPlane + 4 * kG16;
   // (adjoint: at least 24 planes, so that what a ghost reads 4 and 8 planes behind its boundary row is inside the step)
   static constexpr int kPlanes = WITH_BOT ? (kTopPlane + 8 * kG16 > 24 ? kTopPlane + 8 * kG16 : 24) : kTopPlane + 4 * kG16;
-  static constexpr int kKStr = kPlanes * kPlane;         // bytes per step
+  static constexpr int kConstPlane = kPlanes;            // plane of the rows' gate and input constants at this step
+  static constexpr int kKStr = (kPlanes + 1) * kPlane;   // bytes per step
   static constexpr int kBLOff = 4 * kPlane, kCOff = 8 * kPlane;   // B_L and C planes behind the B_T planes
   static constexpr int kXOff = kCK * kKStr;
   static constexpr int kBytes = kXOff + NT * kXTauBytes; // one buffer
@@ -446,6 +448,7 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int 
                                             int e_wg0, int wave, int lane,
                                             const T* x0, const T* x1, const T* x2, const T* x3) {
   using SG = Stage<T, NT, CW, WITH_BOT>;
+  constexpr bool BWD = WITH_BOT;
   static_assert(NWAVES % kCK == 0, "every step of a block needs a wave");
   constexpr int WPK = NWAVES / kCK;                       // waves per step
   const int ks = wave & (kCK - 1), wsub = wave / kCK;     // (uniform) the wave's step, its turn among the waves of that step
@@ -463,6 +466,17 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int 
   const int cell = cell_at(ks);
   const bool ok = ok_at(ks);
   char* kbuf = buf + ks * SG::kKStr;
+  // The constants of the 16 lane rows at this step: gate offsets (log2 of the coefficient that is
+  // folded into the gate) and input coefficients, with the cases of the grid's first row, of column 0
+  // and of the ghost lanes worked out here, once per row and step, instead of in every lane that
+  // sweeps the row.  Lanes read them back as one float4 (offT, offL, cT, cL).
+  if (wsub == 0) {
+    const int r = lane & (kHB - 1);
+    const LaneK K = lane_consts<BWD>(p, clamp_band(p, ks >= q.kw ? q.bnd0 + 1 : q.bnd0), r, true);
+    const bool col0 = q.kz == ks;
+    const float4 kk = make_float4(col0 ? K.oT0 : K.oT, col0 ? -__builtin_huge_valf() : K.oL, col0 ? K.cT0 : K.cT, col0 ? K.cL0 : K.cL);
+    if (slot == 0) *reinterpret_cast<float4*>(kbuf + SG::kConstPlane * SG::kPlane + r * 16) = kk;
+  }
   // B_T, B_L, C: a copy moves the four state groups (lane >> 4) of one tensor for the 16 lane rows
 #pragma unroll
   for (int tsr = 0; tsr < 3; ++tsr)
@@ -628,15 +642,14 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
 
   // per block: where the lane is and what depends on it
   BlockPos bp;
-  LaneK K;
   uint32_t cell_off0 = 0;       // byte offset in a (H,W,E) image of the lane's cell at the first step of the block
-  bool per_step_K = false;      // (uniform) a row crosses a band boundary that changes its constants inside the block
 
   // Operands of one step, read from the staging buffer one step ahead of their use so that the
   // LDS latency hides behind the arithmetic of the step before.
   struct Ops {
     float xv[EC], dtv[EC], dlv[EC];
     float4 bt[EC][4], bl[4], cc[4];
+    float4 kk;   // the row's constants at this step: gate offsets T, L and input coefficients T, L
   };
   auto fetch = [&](const char* bufc, int k, Ops& o) {
     if constexpr (STAGE_X) {
@@ -656,6 +669,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     }
     const char* rec = bufc + rec_off + k * SG::kKStr;
     const char* row = bufc + row_off + k * SG::kKStr;
+    o.kk = *reinterpret_cast<const float4*>(row + SG::kConstPlane * SG::kPlane);
 #pragma unroll
     for (int c = 0; c < EC; ++c)
 #pragma unroll
@@ -686,12 +700,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   bool ck_mine = false;       // the lane stores a snapshot in the first step of the current block
   float4* ckp = nullptr;      // where to
   auto step = [&](int k, const Ops& o) {
-    if (per_step_K) K = lane_consts<false>(p, clamp_band(p, k >= bp.kw ? bp.bnd0 + 1 : bp.bnd0), r, ch_ok);
-    const bool col0 = bp.kz == k;
-    const float offT = col0 ? K.oT0 : K.oT;
-    const float offL = col0 ? ninf : K.oL;
-    const float cT = col0 ? K.cT0 : K.cT;
-    const float cL = col0 ? K.cL0 : K.cL;
+    const float offT = o.kk.x, offL = o.kk.y, cT = o.kk.z, cL = o.kk.w;
     const bool inr = ch_ok && ((bp.in_grid >> k) & 1u);
     float yv[EC];
 #pragma unroll
@@ -766,8 +775,6 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     const int celln = cell_of(p, bpn.bnd0, r, bpn.col0);
     if (!last)
       stage_block<T, 3, CW, false, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, An, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
-    K = lane_consts<false>(p, clamp_band(p, bp.bnd0), r, ch_ok);
-    per_step_K = __any(bp.kw < kCK && special_boundary(p, bp.bnd0, r));
     cell_off0 = (uint32_t)(cell0 * p.E + e0) * (uint32_t)sizeof(T);
     // Snapshot of the state before the block (after step t0-1) for the lanes whose previous
     // position was a cell of the grid; the others hold nothing the backward needs.  The stores are
@@ -980,17 +987,11 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   // per block: where the lane (and the lane row whose sums this thread adds up) is, and what
   // depends on it
   BlockPos bp;
-  LaneK K;
-  float gb1 = 0.f;              // 1 on an active lower ghost: lambda = 1 * (row of mu_T below)
+  // 1 on the lower ghost: lambda = 1 * (row of mu_T below), which is staged as zeros where there is no band below
+  const float gb1 = r == kHB - 1 ? 1.f : 0.f;
+  const uint32_t row_const_off = SG::kConstPlane * SG::kPlane + r * 16;   // the row's constants at step 0 of a staging buffer
   uint32_t cell_off0 = 0;       // byte offset in a (H,W,E) image of the lane's cell at the first step of the block
   uint32_t f_off0 = 0;          // byte offset in the channel-sum image of this thread's sum at the first step
-  bool per_step_K = false;      // (uniform) a row crosses a band boundary that changes its constants inside the block
-  auto band_consts = [&](int bnd) {
-    const int bc = clamp_band(p, bnd);
-    K = lane_consts<true>(p, bc, r, ch_ok);
-    gb1 = (r == kHB - 1 && bc + 1 < p.nbands) ? 1.f : 0.f;
-  };
-
   // state snapshot at the start of the block whose position A is given (zero for lanes that were not under way)
   float cknext[kN];
   auto load_ckpt = [&](int mm, bool take) {   // take: the forward kept the lane's state before block mm
@@ -1038,8 +1039,6 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
                                                  e_wg0, wave, lane, X, DT, DL, DY);
     }
     bp = block_pos(p, A, r, rbands);
-    band_consts(bp.bnd0);
-    per_step_K = __any(bp.kw < kCK && special_boundary(p, bp.bnd0, r));
     {
       const int cell0 = cell_of(p, bp.bnd0, r, bp.col0);
       cell_off0 = (uint32_t)(cell0 * p.E + e) * (uint32_t)sizeof(T);
@@ -1066,12 +1065,8 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
       for (int k = 0; k < kCK; ++k) {
         const int t = t0 + k;
         if (t < p.T_total) {
-          if (per_step_K) band_consts(k >= bp.kw ? bp.bnd0 + 1 : bp.bnd0);
-          const bool col0 = bp.kz == k;
-          const float offT = col0 ? K.oT0 : K.oT;
-          const float offL = col0 ? ninf : K.oL;
-          const float cT = col0 ? K.cT0 : K.cT;
-          const float cL = col0 ? K.cL0 : K.cL;
+          const float4 kk = *reinterpret_cast<const float4*>(bufc + (row_const_off + k * SG::kKStr));
+          const float offT = kk.x, offL = kk.y, cT = kk.z, cL = kk.w;
           float xv = 0.f, dtv = 0.f, dlv = 0.f;
           if constexpr (STAGE_X) {
             const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
@@ -1127,12 +1122,8 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
         // the states of the later steps are dead by now: their registers take the next snapshot
         if (half == 1 && k == (kCK > 1 ? 1 : 0) && m > m_lo) load_ckpt(m - 1, ck_take);
         if (t < p.T_total) {
-          if (per_step_K) band_consts(k >= bp.kw ? bp.bnd0 + 1 : bp.bnd0);
-          const bool col0 = bp.kz == k;
-          const float offT = col0 ? K.oT0 : K.oT;
-          const float offL = col0 ? ninf : K.oL;
-          const float cT = col0 ? K.cT0 : K.cT;
-          const float cL = col0 ? K.cL0 : K.cL;
+          const float4 kk = *reinterpret_cast<const float4*>(bufc + (row_const_off + k * SG::kKStr));
+          const float offT = kk.x, offL = kk.y, cT = kk.z, cL = kk.w;
           const bool inr = ch_ok && ((bp.in_grid >> k) & 1u);
           const uint32_t goff = cell_off0 + (uint32_t)k * estep + (k >= bp.kw ? wrap_adj : 0u);
           float xv = 0.f, dtv = 0.f, dlv = 0.f, dyv = 0.f;
