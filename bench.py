@@ -41,11 +41,36 @@ WORKLOADS = {
 }
 N = 16
 HBM_PEAK_GBS = 8000.0
-VALU_PEAK_SLOTS = 38.3e12   # fp32 lane-operations per second of the whole device (measured)
 # HBM bytes per launch of the backward scan kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/scan_cfg1_kernel_trace_and_traffic.txt: 458190 KiB x 2.0 + 444036 KiB x 1.0); counters
-# cannot be read from inside this script, so the figure is carried here per workload.
+# (profiles/scan_cfg1_kernel_trace_and_traffic.txt); counters cannot be read from inside this script,
+# so the figure is carried here for the workload that has a counter run, and is null for the others.
 MEASURED_TRAFFIC = {"cfg1": 1.3931e9}
+# Issue slots per (cell, channel, state) of the scan kernels (a v_exp_f32 takes two on gfx950):
+# forward 2 exponent FMAs + 2 v_exp + 5 FMA-class (input term, two gate terms, y);
+# backward 10 for the recomputation, 24 for the adjoint (15 FMA-class, 4.5 for the gates of three steps in
+# four, 4.5 for the lane-swap sums over the channels of a wave).
+FWD_SLOTS, BWD_SLOTS = 11, 34
+
+
+def nominal_valu_slots_per_s():
+    """fp32 lane-operations per second the device can issue at its nominal clock: compute units x 64 lanes
+    x engine clock from the device properties.  Not measured here; under load the clock is lower."""
+    import torch
+    prop = torch.cuda.get_device_properties(0)
+    return prop.multi_processor_count * 64 * getattr(prop, "clock_rate", 2400000) * 1e3   # kHz; MI355X: 2.4 GHz
+
+
+def scan_roofline(name, B, E, H, W, s, bwd_kernel_ms, fwd_kernel_ms):
+    """The `roofline` object for the backward scan kernel (the dominant kernel) of a scan workload."""
+    fb, bb = algorithmic_bytes(B, E, H, W, s)
+    achieved = bb / (bwd_kernel_ms * 1e-3) / 1e9
+    return {
+        "kernel": "m2d_bwd_kernel", "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(name),
+        "kernel_ms": round(bwd_kernel_ms, 4), "algorithmic_bytes": bb,
+        "fwd_kernel_ms": round(fwd_kernel_ms, 4), "fwd_algorithmic_bytes": fb,
+        "fwd_kernel_frac": round(fb / (fwd_kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+    }
 
 
 def algorithmic_bytes(B, E, H, W, s):
@@ -63,8 +88,8 @@ def cpu_baseline(B, E, H, W, budget_s=20.0):
     from oracle import scan_oracle as so
 
     cs = so.CScan()
-    cores = len(os.sched_getaffinity(0))
-    threads = min(cores, 16)
+    cores = len(os.sched_getaffinity(0))   # host cores this process may run on
+    threads = min(cores, 16)               # OpenMP threads of the oracle (one image per thread)
     cs.set_threads(threads)
     per_image_units = H * W * E * N
     # ~60 ns per state update forward+backward on one core is a safe guess for sizing the sample
@@ -81,7 +106,8 @@ def cpu_baseline(B, E, H, W, budget_s=20.0):
         "value": round(((t1 - t0) + (t2 - t1)) * 1e3 * scale, 1),
         "fwd_ms": round((t1 - t0) * 1e3 * scale, 1),
         "unit": "ms",
-        "cores": threads,
+        "cores": cores,
+        "threads": threads,
         "kind": "port",
         "sample": f"fp32 C/OpenMP oracle, {bs} of {B} images forward+backward, scaled x{scale:g}",
     }
@@ -134,7 +160,15 @@ def backbone_inference(args):
         "images_per_s_bf16_weights": round(B / (ms_bf16 * 1e-3), 1),
         "images_per_s_autocast_fp32_weights": round(B / (ms_autocast * 1e-3), 1),
         "last_scan_kernel_ms": round(scan_ms, 4),
-        "roofline": None, "cpu_baseline": None,
+        # the library's largest kernel inside the model: the forward scan (the last one of a batch is the
+        # 28x28x128 scan of stage 2); the model's other time is spread over some 190 smaller launches
+        "roofline": {"kernel": "m2d_fwd_kernel (stage 2 scan, B=128 E=128 28x28)", "bound": "hbm",
+                     "achieved": round(algorithmic_bytes(128, 128, 28, 28, 2)[0] / (scan_ms * 1e-3) / 1e9, 1),
+                     "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(algorithmic_bytes(128, 128, 28, 28, 2)[0] / (scan_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                     "traffic": None, "kernel_ms": round(scan_ms, 4),
+                     "algorithmic_bytes": algorithmic_bytes(128, 128, 28, 28, 2)[0]},
+        "cpu_baseline": None,
     }
     print(json.dumps(out))
 
@@ -180,6 +214,20 @@ def stage_sequence(args):
         return e0.elapsed_time(e1) / args.steps
 
     fwd_ms, both_ms = timed(fwd_only), timed(fwd_bwd)
+    # kernel durations per stage from the library's own events (a second, untimed pass)
+    cabi.profile_enable(True)
+    per_stage = {}
+    for name, (leaves, _, dy) in zip(("cfg1", "stage2", "stage3", "stage4"), stages):
+        ks = []
+        for _ in range(5):
+            torch.autograd.grad(wavefront.wf_cuda_fn_pr.apply(*leaves), leaves, dy)
+            ks.append((cabi.profile_last_ms(cabi.M2D_PASS_FWD), cabi.profile_last_ms(cabi.M2D_PASS_BWD)))
+        B, E, H, W, _ = WORKLOADS[name]
+        f, b = sum(k[0] for k in ks) / len(ks), sum(k[1] for k in ks) / len(ks)
+        per_stage[name] = scan_roofline(name, B, E, H, W, 2, b, f)
+    dominant = max(per_stage, key=lambda k: per_stage[k]["kernel_ms"])
+    roof = dict(per_stage[dominant])
+    roof["kernel"] = f"m2d_bwd_kernel ({dominant} scan)"
     print(json.dumps({
         "metric": "four M2D-T stage scans in sequence, fwd+bwd ms at B=128 N=16", "value": round(both_ms, 4), "unit": "ms",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(both_ms, 4),
@@ -188,8 +236,10 @@ def stage_sequence(args):
         "config": {"workload": "cfg2: scans of (E,H,W) = (64,56,56), (128,28,28), (320,14,14), (512,7,7) in sequence, B=128 N=16"},
         "fwd_ms": round(fwd_ms, 4), "fwd_bwd_ms": round(both_ms, 4),
         "pct_hbm_roofline": {"fwd_bwd": round(100 * alg / (both_ms * 1e-3) / (HBM_PEAK_GBS * 1e9), 2)},
-        "valu_ceiling_frac": round(units * 48 / VALU_PEAK_SLOTS / (both_ms * 1e-3), 4),
-        "roofline": None, "cpu_baseline": None,
+        "valu_ceiling_frac_nominal": round(units * (FWD_SLOTS + BWD_SLOTS) / nominal_valu_slots_per_s() / (both_ms * 1e-3), 4),
+        "roofline": roof,
+        "per_stage_bwd_kernel": {k: {"kernel_ms": v["kernel_ms"], "frac": v["frac"], "fwd_kernel_ms": v["fwd_kernel_ms"]} for k, v in per_stage.items()},
+        "cpu_baseline": None,
     }))
 
 
@@ -255,6 +305,12 @@ def entry_point(args):
     # as the entry point calls it: the scan hands over the gradients before the softplus, the deltas are not read
     proj_bwd_ms = timed(lambda: cabi.proj_bwd(xd, outs[0], None, None, w32[0], w32[1], w32[3], *ups, dx,
                                               round_weights=True, dpre=True))
+    cabi.profile_enable(True)
+    ks = []
+    for _ in range(5):
+        fwd_bwd("partial")
+        ks.append((cabi.profile_last_ms(cabi.M2D_PASS_FWD), cabi.profile_last_ms(cabi.M2D_PASS_BWD)))
+    scan_fwd_ms, scan_bwd_ms = sum(k[0] for k in ks) / len(ks), sum(k[1] for k in ks) / len(ks)
     P, s = B * H * W, 2
     nw = (2 * R + 3 * N) * E + 2 * E * R + 2 * E
     proj_fwd_bytes = s * P * (E + 2 * R + 2 * E + 3 * N) + 4 * nw
@@ -273,7 +329,8 @@ def entry_point(args):
             "fwd_algorithmic_bytes": proj_fwd_bytes, "bwd_algorithmic_bytes": proj_bwd_bytes,
             "fwd_frac_of_hbm_peak": round(proj_fwd_bytes / (proj_fwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
             "bwd_frac_of_hbm_peak": round(proj_bwd_bytes / (proj_bwd_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
-        "roofline": None, "cpu_baseline": None,
+        "roofline": scan_roofline("entry", B, E, H, W, 2, scan_bwd_ms, scan_fwd_ms),
+        "cpu_baseline": None,
     }
     print(json.dumps(out))
 
@@ -377,7 +434,6 @@ def main():
     input_bytes = sum(t.numel() * t.element_size() for t in leaves) + dy.numel() * dy.element_size()
     s = 2 if dts == "bf16" else 4
     fb, bb = algorithmic_bytes(B, E, H, W, s)
-    achieved = bb / (bwd_kernel * 1e-3) / 1e9
     out = {
         "metric": "2D-scan fwd & fwd+bwd ms at B=128 D=64 56x56 N=16; % of HBM roofline",
         "value": round(step_ms, 4),
@@ -402,30 +458,17 @@ def main():
             "fwd": round(100 * fb / (fwd_ms * 1e-3) / (HBM_PEAK_GBS * 1e9), 2),
             "fwd_bwd": round(100 * (fb + bb) / (step_ms * 1e-3) / (HBM_PEAK_GBS * 1e9), 2),
         },
-        "roofline": {
-            "kernel": "m2d_bwd_kernel",
-            "bound": "hbm",
-            "achieved": round(achieved, 1),
-            "peak": HBM_PEAK_GBS,
-            "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": MEASURED_TRAFFIC.get(args.workload),
-            "kernel_ms": round(bwd_kernel, 4),
-            "algorithmic_bytes": bb,
-            "fwd_kernel_ms": round(fwd_kernel_ms, 4),
-            "fwd_kernel_frac": round(fb / (fwd_kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-        },
+        "roofline": scan_roofline(args.workload, B, E, H, W, s, bwd_kernel, fwd_kernel_ms),
     }
-    # Informational second ceiling: the scan is bounded by VALU issue, not by HBM.  Per (cell, channel,
-    # state) the forward needs 2 v_exp_f32 (2 issue slots each on gfx950) + 9 FMA-class operations = 13
-    # slots, the backward 11 for the recompute + 24 for the adjoint; the device issues 38.3e12 lane-slots/s
-    # (measured, profiles/microbench_gfx950.txt).
+    # Informational second ceiling: the scan is bounded by VALU issue, not by HBM.
     units = B * H * W * E * N
+    peak_slots = nominal_valu_slots_per_s()
     out["valu_ceiling"] = {
-        "peak_lane_slots_per_s": VALU_PEAK_SLOTS,
-        "fwd_slots_per_unit": 13, "bwd_slots_per_unit": 35, "units": units,
-        "fwd_kernel_frac": round(units * 13 / VALU_PEAK_SLOTS / (fwd_kernel_ms * 1e-3), 4),
-        "bwd_kernel_frac": round(units * 35 / VALU_PEAK_SLOTS / (bwd_kernel * 1e-3), 4),
+        "nominal_lane_slots_per_s": peak_slots,
+        "note": "compute units x 64 lanes x engine clock from the device properties; not measured by this script",
+        "fwd_slots_per_unit": FWD_SLOTS, "bwd_slots_per_unit": BWD_SLOTS, "units": units,
+        "fwd_kernel_frac": round(units * FWD_SLOTS / peak_slots / (fwd_kernel_ms * 1e-3), 4),
+        "bwd_kernel_frac": round(units * BWD_SLOTS / peak_slots / (bwd_kernel * 1e-3), 4),
     }
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(B, E, H, W)

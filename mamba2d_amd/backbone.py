@@ -61,7 +61,8 @@ def linear_act(lin, x, pre=ACT_NONE, post=ACT_NONE, star=None, norm=None):
     bound by the activations' bytes; wider layers are faster in the stock library); otherwise stock operators."""
     w, b = lin.weight, lin.bias
     N, K = w.shape
-    if (x.is_cuda and x.dtype == torch.bfloat16 and _inference(x, w) and w.dtype in (torch.float32, torch.bfloat16)
+    extra = [t for t in (b, *((star.scale, star.bias) if star is not None else ())) if t is not None]
+    if (x.is_cuda and x.dtype == torch.bfloat16 and _inference(x, w, *extra) and w.dtype in (torch.float32, torch.bfloat16)
             and K % 32 == 0 and K <= 256 and N % 16 == 0 and N <= 512 and x.numel() > 0
             and (star is None or star.scale.dtype == w.dtype)):
         ps = (star.scale, star.bias) if pre == ACT_STARRELU else (None, None)
@@ -138,7 +139,8 @@ class MLP(nn.Module):
         """fc2(GELU(fc1 x)), of norm(x) with ``norm`` (the block's norm2, which only the MLP reads)."""
         w1, w2 = self.fc1.weight, self.fc2.weight
         if (x.is_cuda and x.dtype == torch.bfloat16 and x.numel() > 0 and x.shape[-1] in (32, 64) and w1.shape[0] == 4 * w1.shape[1]
-                and _inference(x, w1, w2) and w1.dtype in (torch.float32, torch.bfloat16) and w2.dtype == w1.dtype):
+                and _inference(x, w1, w2, self.fc1.bias, self.fc2.bias) and w1.dtype in (torch.float32, torch.bfloat16)
+                and w2.dtype == w1.dtype):
             # both layers in one kernel: the hidden activations, four times x, never reach memory
             if norm is not None and _norm_joins(norm, x, w1):
                 return mlp_fwd_op(x.contiguous(), w1, self.fc1.bias, w2, self.fc2.bias, norm.weight, norm.bias, norm.eps)
@@ -148,7 +150,8 @@ class MLP(nn.Module):
     def takes_norm(self, x, norm):
         """norm(x) would not be written: the kernel of the first layer computes it."""
         w1 = self.fc1.weight
-        return (x.is_cuda and x.dtype == torch.bfloat16 and x.numel() > 0 and _inference(x, w1, self.fc2.weight)
+        return (x.is_cuda and x.dtype == torch.bfloat16 and x.numel() > 0
+                and _inference(x, w1, self.fc2.weight, self.fc1.bias, self.fc2.bias)
                 and w1.dtype in (torch.float32, torch.bfloat16) and self.fc2.weight.dtype == w1.dtype and _norm_joins(norm, x, w1)
                 and w1.shape[1] % 32 == 0 and w1.shape[1] <= 128 and w1.shape[0] % 16 == 0 and w1.shape[0] <= 512)
 
@@ -271,18 +274,21 @@ class RoPEAttention2D(nn.Module):
     def _rope_tables(self, H, W, device, dtype):
         key = (H, W, str(device), dtype)
         if key not in self._tables:
-            d = self.axis_dim
-            inv_freq = 1.0 / (self.rope_base ** (torch.arange(0, d // 2, device=device, dtype=torch.float32) / (d // 2)))
-            rows = torch.arange(H, device=device, dtype=torch.float32).repeat_interleave(W)
-            cols = torch.arange(W, device=device, dtype=torch.float32).repeat(H)
-            ang = torch.cat([rows[:, None] * inv_freq, cols[:, None] * inv_freq], dim=-1)   # (HW, d)
-            ang = ang.repeat_interleave(2, dim=-1)                                           # pairs share an angle
-            # layout per head: [row-rotated d | column-rotated d | untouched]
-            cos = torch.ones(H * W, self.head_dim, device=device)
-            sin = torch.zeros(H * W, self.head_dim, device=device)
-            cos[:, :2 * d] = torch.cat([ang[:, 0:d].cos(), ang[:, d:2 * d].cos()], dim=-1)
-            sin[:, :2 * d] = torch.cat([ang[:, 0:d].sin(), ang[:, d:2 * d].sin()], dim=-1)
-            self._tables[key] = (cos.to(dtype), sin.to(dtype))
+            # built outside inference mode (and without a graph): a table made under torch.inference_mode
+            # could not be saved for the backward pass of a later training call
+            with torch.inference_mode(False), torch.no_grad():
+                d = self.axis_dim
+                inv_freq = 1.0 / (self.rope_base ** (torch.arange(0, d // 2, device=device, dtype=torch.float32) / (d // 2)))
+                rows = torch.arange(H, device=device, dtype=torch.float32).repeat_interleave(W)
+                cols = torch.arange(W, device=device, dtype=torch.float32).repeat(H)
+                ang = torch.cat([rows[:, None] * inv_freq, cols[:, None] * inv_freq], dim=-1)   # (HW, d)
+                ang = ang.repeat_interleave(2, dim=-1)                                           # pairs share an angle
+                # layout per head: [row-rotated d | column-rotated d | untouched]
+                cos = torch.ones(H * W, self.head_dim, device=device)
+                sin = torch.zeros(H * W, self.head_dim, device=device)
+                cos[:, :2 * d] = torch.cat([ang[:, 0:d].cos(), ang[:, d:2 * d].cos()], dim=-1)
+                sin[:, :2 * d] = torch.cat([ang[:, 0:d].sin(), ang[:, d:2 * d].sin()], dim=-1)
+                self._tables[key] = (cos.to(dtype), sin.to(dtype))
         return self._tables[key]
 
     @staticmethod

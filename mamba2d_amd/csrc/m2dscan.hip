@@ -37,7 +37,6 @@
 
 #include <atomic>
 #include <stdint.h>
-#include <stdlib.h>
 
 #include "../../include/m2dscan.h"
 
@@ -432,12 +431,6 @@ __device__ __forceinline__ BlockPos block_pos(const ScanParams& p, Pos A, int r,
   return q;
 }
 __device__ __forceinline__ int clamp_band(const ScanParams& p, int bnd) { return bnd < 0 ? 0 : (bnd >= p.nbands ? p.nbands - 1 : bnd); }
-// A row changes its constants only when it moves between the first band and the second (grid row
-// 0 has no row above) or into / out of the last band (fewer rows, no band below).
-__device__ __forceinline__ bool special_boundary(const ScanParams& p, int bnd_lo, int r) {
-  return (!p.stacked && bnd_lo == 0 && r == 1) || (bnd_lo + 1 == p.nbands - 1 && (r > p.rows_last || r == kHB - 1));
-}
-
 // Stages the operands of a block of kCK steps.  A is the position of the stream index (first step
 // of the block) - 15; q and cell0 describe the lane's own row in that block (block_pos, and the cell
 // index of its position at the first step: what the lane's copies fetch is what the lane itself will
@@ -1017,9 +1010,10 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   Pos A = pos_of(p, (m_hi - 1) * kCK - (kHB - 1));   // position of the stream index t0 - 15 (wave-uniform)
   __syncthreads();   // the zeros are in place before the first copies land on them
   bp = block_pos(p, A, r, rbands);
+  int cell0 = cell_of(p, bp.bnd0, r, bp.col0);   // cell index of the lane's position at the first step of the block
   bool ck_take = snapshot_lane(p, Pos{bp.bnd0, bp.col0}, r, ch_ok);   // the lane restores a snapshot for the block to come
   load_ckpt(m_hi - 1, ck_take);
-  stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds, b, A, bp, cell_of(p, bp.bnd0, r, bp.col0), e_wg0, wave, lane, X, DT, DL, DY);
+  stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
   staging_fence();
   int cur = 0;
   int xpar = 0;   // exchange buffer in use
@@ -1030,20 +1024,15 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
     float ck0[kN];
 #pragma unroll
     for (int n = 0; n < kN; ++n) ck0[n] = cknext[n];
+    // the block before: where the lane's row will be is also what the lane's copies fetch
     const Pos Aprev = pos_before(A);
-    {   // the block before: where the lane's row will be is also what the lane's copies fetch
-      const BlockPos bpn = block_pos(p, Aprev, r, rbands);
-      ck_take = snapshot_lane(p, Pos{bpn.bnd0, bpn.col0}, r, ch_ok);
-      if (m > m_lo)
-        stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, cell_of(p, bpn.bnd0, r, bpn.col0),
-                                                 e_wg0, wave, lane, X, DT, DL, DY);
-    }
-    bp = block_pos(p, A, r, rbands);
-    {
-      const int cell0 = cell_of(p, bp.bnd0, r, bp.col0);
-      cell_off0 = (uint32_t)(cell0 * p.E + e) * (uint32_t)sizeof(T);
-      f_off0 = (uint32_t)cell0 * (uint32_t)(3 * kN * sizeof(float)) + f_sub;
-    }
+    const BlockPos bpn = block_pos(p, Aprev, r, rbands);
+    const int celln = cell_of(p, bpn.bnd0, r, bpn.col0);
+    ck_take = snapshot_lane(p, Pos{bpn.bnd0, bpn.col0}, r, ch_ok);
+    if (m > m_lo)
+      stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+    cell_off0 = (uint32_t)(cell0 * p.E + e) * (uint32_t)sizeof(T);
+    f_off0 = (uint32_t)cell0 * (uint32_t)(3 * kN * sizeof(float)) + f_sub;
 
     // The 16 states are swept in two halves of 8 (state groups 0,1 then 2,3), each half
     // recomputing and then back-propagating the whole block: only 5 x 8 recomputed states are
@@ -1236,6 +1225,8 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
     }
     __syncthreads();
     A = Aprev;
+    bp = bpn;
+    cell0 = celln;
     cur ^= 1;
   }
 
@@ -1430,8 +1421,24 @@ int check_desc(const m2d_desc* d) {
   return M2D_OK;
 }
 
+// Compute units of the current device, asked once per process (256 on MI355X, which is also what
+// a host without a GPU plans with: sizes queried there are the sizes of an MI355X).
+int device_cus() {
+  static const int n = [] {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess || prop.multiProcessorCount < 1) {
+      (void)hipGetLastError();   // no device: not an error of a later call
+      return 256;
+    }
+    return prop.multiProcessorCount;
+  }();
+  return n;
+}
+
 Geometry make_geometry(const m2d_desc* d) {
   Geometry g;
+  const int64_t ncu = device_cus();
   g.HB = kHB;
   g.hb_shift = kHBShift;
   g.CS = 64 / g.HB;
@@ -1449,7 +1456,7 @@ Geometry make_geometry(const m2d_desc* d) {
       if ((int64_t)ips * d->H * d->W * d->E >= ((int64_t)1 << 30)) break;   // a stack is addressed like one image
       const int vB = (d->B + ips - 1) / ips;
       const int nb = (ips * d->H + kRB - 1) / kRB;
-      const int64_t rounds = ((int64_t)vB * groups + 255) / 256;
+      const int64_t rounds = ((int64_t)vB * groups + ncu - 1) / ncu;
       const int64_t cost = rounds * ((nb - 1) * S + d->W + kRB + 8);
       if (best < 0 || cost < best) { best = cost; g.ips = ips; }
     }
@@ -1477,7 +1484,7 @@ Geometry make_geometry(const m2d_desc* d) {
   // Few images with many bands leave most of the device idle when each image is one sequential
   // stream.  Then every band gets workgroups of its own (a padded stream, one window of S steps
   // per band) and the sweep becomes a sequence of launches in which band k trails band k-1.
-  g.sliced = !g.stacked && g.nbands >= 4 && (int64_t)B * groups <= 64;
+  g.sliced = !g.stacked && g.nbands >= 4 && (int64_t)B * groups <= ncu / 4;
   if (g.sliced && g.nbands == 4) {
     // Four bands (more bands favour the sliced sweep again: 84x84 measured) and a batch that fills half the device with workgroups of 4 waves, but not with
     // every band under way on workgroups of its own: one stream per image on workgroups of 4 waves
@@ -1487,7 +1494,7 @@ Geometry make_geometry(const m2d_desc* d) {
     const int nlb = (s_sl / kCK + kSliceQ - 1) / kSliceQ;
     const int64_t under_way = (nlb + kSliceLag - 1) / kSliceLag < g.nbands ? (nlb + kSliceLag - 1) / kSliceLag : g.nbands;
     const int64_t half = (int64_t)B * ((d->E + kFwdHalfWaves * g.CS - 1) / (kFwdHalfWaves * g.CS));
-    if (half > (int64_t)B * groups && half <= 256 && half >= 128 && half * under_way > 256) g.sliced = false;
+    if (half > (int64_t)B * groups && half <= ncu && half >= ncu / 2 && half * under_way > ncu) g.sliced = false;
   }
   g.nbb = 0; g.nlaunch = 1;
   if (g.sliced) {
@@ -1508,7 +1515,7 @@ Geometry make_geometry(const m2d_desc* d) {
   const size_t lds_ec2 = d->dtype == M2D_BF16 ? fwd_lds_bytes<bf16_t, 2>() : kLdsPerWorkgroup + 1;
   const int64_t wg1 = (int64_t)B * ((d->E + kFwdWaves * g.CS - 1) / (kFwdWaves * g.CS));
   const int64_t wg2 = (int64_t)B * ((d->E + kFwdWaves * g.CS * 2 - 1) / (kFwdWaves * g.CS * 2));
-  const bool ec2 = (d->E % 2 == 0) && lds_ec2 <= kLdsPerWorkgroup && 18 * ((wg2 + 255) / 256) < 10 * ((wg1 + 255) / 256);
+  const bool ec2 = (d->E % 2 == 0) && lds_ec2 <= kLdsPerWorkgroup && 18 * ((wg2 + ncu - 1) / ncu) < 10 * ((wg1 + ncu - 1) / ncu);
   g.fwd_ec = ec2 ? 2 : 1;
   // forward of a small batch in one stream per image: workgroups of 4 waves (16 channels) where those
   // are more than the workgroups of 8 and still no more than the compute units
@@ -1518,16 +1525,11 @@ Geometry make_geometry(const m2d_desc* d) {
                                            ? ((g.nbb + kSliceQ - 1) / kSliceQ + kSliceLag - 1) / kSliceLag : g.nbands) : 1;
   // (a sliced sweep may exceed the units by a few workgroups while most bands are under way: its first
   // and last launches, with fewer bands, still gain)
-  const int64_t room = g.sliced ? 256 + 16 : 256;
+  const int64_t room = g.sliced ? ncu + ncu / 16 : ncu;
   g.fwd_nw = (!g.stacked && !ec2 && wg_half > wg1 && wg_half * together <= room) ? kFwdHalfWaves : kFwdWaves;
   g.fwd_bpb = (d->E + g.fwd_nw * g.CS * g.fwd_ec - 1) / (g.fwd_nw * g.CS * g.fwd_ec);
   g.fwd_wpb = g.fwd_bpb * g.fwd_nw;
   g.bwd_nw = (!g.stacked && wg_half > (int64_t)B * groups && wg_half * together <= room) ? kFwdHalfWaves : kBwdWaves;
-  if (const char* ev = getenv("M2D_DEBUG_NW")) {   // experiment
-    const int v = atoi(ev);
-    if (!g.stacked && !ec2 && (v & 1)) { g.fwd_nw = kFwdHalfWaves; g.fwd_bpb = (d->E + g.fwd_nw * g.CS * g.fwd_ec - 1) / (g.fwd_nw * g.CS * g.fwd_ec); g.fwd_wpb = g.fwd_bpb * g.fwd_nw; }
-    if (!g.stacked && (v & 2)) g.bwd_nw = kFwdHalfWaves;
-  }
   g.bwd_bpb = (d->E + g.bwd_nw * g.CS - 1) / (g.bwd_nw * g.CS);
   g.bwd_wpb = g.bwd_bpb * g.bwd_nw;
   g.stage_x = (d->E % (d->dtype == M2D_BF16 ? 8 : 4)) == 0;

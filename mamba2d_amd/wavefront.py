@@ -20,7 +20,6 @@ from __future__ import annotations
 
 import ctypes
 import os
-import weakref
 
 import torch
 import torch.nn.functional as F
@@ -58,14 +57,16 @@ SAVE_CHECKPOINTS = os.environ.get("M2D_SAVE_CHECKPOINTS", "1") != "0"
 FUSED_PROJECTIONS = os.environ.get("M2D_FUSED_PROJECTIONS", "1") != "0"
 
 
-def _ckpt_bytes(x, N, flip=False) -> int:
+def _ckpt_bytes(x, N, flip=False, packed_bc=False) -> int:
     d = cabi.make_desc(x, N, flip)
+    if packed_bc:   # the caller brings the packed B/C records: the buffer has no room for them
+        d.flags |= cabi.M2D_FLAG_PACKED_BC
     return int(cabi.lib.m2d_scan_ckpt_bytes(ctypes.byref(d)))
 
 
 @torch.library.register_fake("m2dscan::scan_fwd")
 def _scan_fwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, save_ckpt, flip, raw_params=False, packed_bc=False):
-    n = _ckpt_bytes(x, AT.shape[1]) if save_ckpt else 1
+    n = _ckpt_bytes(x, AT.shape[1], packed_bc=packed_bc) if save_ckpt else 1
     return torch.empty_like(x), x.new_empty((max(n, 1),), dtype=torch.uint8)
 
 
@@ -172,24 +173,13 @@ def _c(t):
     return t if t.data_ptr() % 16 == 0 else t.clone()
 
 
-_F32_COPIES = {}   # id(parameter) -> (weak reference, version, data pointer, fp32 copy)
-
-
 def _as_f32(t):
-    """The parameter as a contiguous, aligned fp32 tensor.  fp32 parameters pass through; for others
-    (a model held in bf16) the copy is kept until the parameter changes, so that a forward does not
-    spend eight small kernels per scan on casting weights that did not change."""
+    """The parameter as a contiguous, aligned fp32 tensor: fp32 parameters (the reference trains
+    bf16-mixed with fp32 parameters) pass through, others are cast on every call (no copy is kept: a
+    parameter can change through ``.data`` without any trace a cache could check)."""
     if t.dtype == torch.float32:
         return _c(t)
-    if torch.compiler.is_compiling():   # a traced graph holds the cast itself
-        return t.detach().float().contiguous()
-    key = id(t)
-    hit = _F32_COPIES.get(key)
-    if hit is not None and hit[0]() is t and hit[1] == t._version and hit[2] == t.data_ptr():
-        return hit[3]
-    f = _c(t.detach().float())
-    _F32_COPIES[key] = (weakref.ref(t, lambda _, k=key: _F32_COPIES.pop(k, None)), t._version, t.data_ptr(), f)
-    return f
+    return _c(t.detach().float())
 
 
 # The kernels hold the 16 states of a cell in the registers of one lane (d_state of every

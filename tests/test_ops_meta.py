@@ -44,3 +44,23 @@ def test_projection_ops_on_meta_tensors(wf, dtype):
     g = wf.proj_bwd_op(x, low, dT, dL, w[0], w[1], w[3], dT, dL, BT, BL, C, torch.empty_like(x), True)
     assert [tuple(t.shape) for t in g] == [tuple(t.shape) for t in w]
     assert all(t.dtype == torch.float32 for t in g)
+
+
+@pytest.mark.parametrize("packed", [False, True])
+@pytest.mark.parametrize("shape,dtype", [((2, 56, 56, 64), torch.bfloat16), ((1, 150, 90, 8), torch.float32), ((9, 7, 7, 32), torch.bfloat16)])
+def test_fake_checkpoint_size_matches_the_library(shape, dtype, packed):
+    """The fake of m2dscan::scan_fwd must size the checkpoint tensor as the real operator does, also when
+    the caller brings packed B/C records (then the buffer holds no copy of them): a backend that plans
+    memory from the fake's shapes would otherwise disagree with the kernel."""
+    import ctypes
+    from mamba2d_amd import cabi, wavefront  # noqa: F401  (registers the fakes)
+    B, H, W, E = shape
+    N = 16
+    m = lambda *s, dt=dtype: torch.empty(*s, dtype=dt, device="meta")
+    x = m(B, H, W, E)
+    bc = m(B, H, W, 3 * N, dt=torch.float32) if packed else m(B, H, W, N)
+    rest = (m(0), m(0)) if packed else (m(B, H, W, N), m(B, H, W, N))
+    y, ck = torch.ops.m2dscan.scan_fwd(x, m(B, H, W, E), m(B, H, W, E), m(E, N), m(E, N), bc, *rest, m(E), True, False, False, packed)
+    d = cabi.Desc(B, H, W, E, N, cabi.M2D_BF16 if dtype == torch.bfloat16 else cabi.M2D_F32,
+                  cabi.M2D_FLAG_PACKED_BC if packed else 0, 0)
+    assert ck.numel() == cabi.lib.m2d_scan_ckpt_bytes(ctypes.byref(d)) and y.shape == x.shape

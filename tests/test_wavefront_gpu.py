@@ -307,24 +307,24 @@ def test_entry_point_replays_from_a_graph(wf, shape, dtype):
             assert torch.equal(a, b), i
 
 
-def test_cached_parameter_casts_follow_the_parameters(wf):
-    """Parameters held in bf16 are cast to fp32 once and the copy is reused; an in-place update of a
-    parameter (an optimiser step, a checkpoint load) must show in the next call."""
-    say("\ncase cached parameter casts")
+def test_parameter_updates_through_data_show_in_the_next_call(wf):
+    """Parameters held in bf16 are cast to fp32 on every call: an update of a parameter, also one made
+    through ``.data`` (old-style optimisers, EMA swaps, weight clipping), which leaves no trace in the
+    tensor's version counter, must show in the next call."""
+    say("\ncase parameter updates through .data")
     B, H, W, E, N = 2, 6, 7, 32, 16
     R = math.ceil(E / 16)
-    p = {k: v.bfloat16() for k, v in make_block_params(E, N, R, 1, "cuda").items()}
+    p = {k: torch.nn.Parameter(v.bfloat16()) for k, v in make_block_params(E, N, R, 1, "cuda").items()}
     x = torch.randn(B, H, W, E, generator=torch.Generator().manual_seed(1)).cuda().bfloat16()
     args = [p[k] for k in ORDER]
     with torch.no_grad():
         y1 = wf.wavefront_scan_cuda(x, *args)
-        y2 = wf.wavefront_scan_cuda(x, *args)
-        assert torch.equal(y1, y2)
-        p["D"].mul_(2.0)                                   # y = scan + x * D
+        assert torch.equal(y1, wf.wavefront_scan_cuda(x, *args))
+        p["D"].data.mul_(2.0)                              # y = scan + x * D
         y3 = wf.wavefront_scan_cuda(x, *args)
         want = y1.float() + x.float() * (p["D"].float() / 2)
         assert so.rel_err(y3.float().cpu(), want.cpu()) < 2e-2 and not torch.equal(y1, y3)
-        fresh = [t.clone() for t in args]                  # same values in new tensors: no stale copy may be used
+        fresh = [t.detach().clone() for t in args]         # same values in new tensors
         assert torch.equal(wf.wavefront_scan_cuda(x, *fresh), y3)
 
 
