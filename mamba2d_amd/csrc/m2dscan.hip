@@ -60,8 +60,9 @@ constexpr int kFwdHalfWaves = 4;  // ... of a small batch (fewer workgroups of 8
 constexpr int kBwdWaves = 8;      // waves per backward workgroup
 constexpr int kZeroFloats = 64;     // page of zeros at the head of the set-up area
 constexpr int kModeSweep = 0, kModeSliced = 1, kModeStacked = 2;   // how the bands of the batch are scheduled
-constexpr int kSliceQ = 4;         // sliced sweep: blocks of steps per band and launch
-constexpr int kSliceLag = 2;       // sliced sweep: launches by which a band trails the band it depends on
+constexpr int kLinkLag = 7;        // linked sweep: blocks by which a band trails the band it depends on (see link_need_*)
+constexpr int kSpinLimit = 1 << 20;   // linked sweep: polls of a neighbour's progress before a workgroup gives up waiting
+constexpr uint32_t kLinkAbort = 0xffffffffu;   // progress value of a band that gave up: nobody waits for it
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -192,12 +193,13 @@ struct ScanParams {
   int T_total;                      // steps of the whole sweep
   int rows_last;                    // grid rows of the last band
   uint32_t magicS;                  // floor(2^32 / S)
-  // Sliced sweep (few images, many bands): every band has its own workgroups, a launch advances
-  // each active band by kSliceQ blocks, and a band trails the one it depends on by kSliceLag
-  // launches, so that what it reads was stored by an earlier launch.
-  int sliced, sl_ell, sl_band0;     // on/off, launch index, first active band of the launch
+  // Linked sweep (few images, many bands): every band has its own workgroups, all in one launch; a
+  // band publishes how many blocks of its window are done (boundary rows in memory) and the band
+  // that reads its boundary rows polls that count before it stages them.
+  int sliced;                       // on/off
   int sl_nbb;                       // blocks per band (S / kCK)
-  float* carry;                     // state handed from launch to launch: fwd [B][nbands][E][16][16], bwd [B][nbands][E][65][16]
+  uint32_t* prog;                   // [nbands][B][workgroups per image] blocks of the band's window whose boundary rows are in memory
+  uint32_t* link_err;               // set to 1 by a workgroup that gave up waiting (results are then invalid)
   int64_t bot_stride;               // floats between the mu_T rows of consecutive bands (0: one row buffer, bands in sequence)
   int pa_slots;                     // partial sums over positions per image (1, or one per band when sliced)
   // Stacked images (grids of one band whose height divides 14): `ips` images in a row of the batch
@@ -318,6 +320,59 @@ __device__ __forceinline__ void lds_fill16(const void* src, char* lds_window) {
   else
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(src), "s"(base) : "memory", "m0");
 }
+
+// ---- linked sweep: hand-off between the workgroups of neighbouring bands inside one launch.
+// Boundary rows and progress counts are written through to memory and read past the caches at
+// device scope (sc1), so that workgroups on different XCDs, whose L2 caches are not coherent with
+// each other, see them; plain vector loads and stores, no fences.  A workgroup only ever waits for
+// a workgroup with a lower index, which was dispatched before it, so the one with the lowest index
+// that is not finished is always running: every wait ends.  Should one not (a defect), the waiting
+// workgroup gives up after kSpinLimit polls, flags the error and tells its own dependants not to
+// wait either, so that the launch still ends.
+__device__ __forceinline__ uint32_t link_poll(const uint32_t* ptr) {
+  uint32_t v;
+  asm volatile("global_load_dword %0, %1, off sc1\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(ptr) : "memory");
+  return __builtin_amdgcn_readfirstlane(v);
+}
+__device__ __forceinline__ void link_publish(uint32_t* ptr, uint32_t v) {
+  asm volatile("global_store_dword %0, %1, off sc1" ::"v"(ptr), "v"(v) : "memory");
+}
+// 16 bytes of a boundary row, written through at device scope
+__device__ __forceinline__ void store_row_device_scope(float4* dst, float4 v) {
+  const v4f_t w = {v.x, v.y, v.z, v.w};
+  asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(w) : "memory");
+}
+struct Link {
+  uint32_t* mine = nullptr;         // this workgroup's progress count
+  const uint32_t* dep = nullptr;    // the count of the workgroup whose boundary rows this one reads (none: first band of the sweep)
+  uint32_t seen = 0;                // last value read from dep
+  bool gave_up = false;
+  uint32_t* err = nullptr;
+  // (uniform) returns once the neighbour has `need` blocks done
+  __device__ __forceinline__ void wait_for(uint32_t need) {
+    if (!dep || seen >= need) return;
+    for (int spin = 0; spin < kSpinLimit; ++spin) {
+      seen = link_poll(dep);
+      if (seen >= need) return;
+      __builtin_amdgcn_s_sleep(16);
+    }
+    seen = kLinkAbort;
+    gave_up = true;
+    if (threadIdx.x == 0) link_publish(err, 1u);
+  }
+  // after a barrier behind which `done` blocks of this band have their boundary rows in memory
+  __device__ __forceinline__ void publish(uint32_t done) {
+    if (threadIdx.x == 0) link_publish(mine, (gave_up || seen == kLinkAbort) ? kLinkAbort : done);
+  }
+};
+// Blocks of the neighbour's window that must be done before block j of a band's own window is staged.
+// Forward: the ghost of block j replays the columns 4j .. 4j+3 of the last row of the band above,
+// which lane 14 stored at the window's steps 4j+14 .. 4j+17, the last of them in block j+4.
+// Backward (blocks are swept from the last to the first, counts are blocks done from the end): the lower
+// ghost of block j reads the columns 4j-15 .. 4j-12 of the first row of the band below, which lane 1 stored
+// at steps 4j-14 .. 4j-11, the earliest of them in block j-4.
+__device__ __forceinline__ uint32_t link_need_fwd(int j, int nbb) { return (uint32_t)(j + 5 < nbb ? j + 5 : nbb); }
+__device__ __forceinline__ uint32_t link_need_bwd(int j, int nbb) { return (uint32_t)(j - 4 > 0 ? nbb - (j - 4) : nbb); }
 
 // Position of the stream index (index of A) + d, for 0 <= d < 19.  Strides below 19 (stacked
 // images) can wrap more than once.
@@ -568,17 +623,19 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   char* lds = reinterpret_cast<char*>(smem);       // two staging buffers
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  int lb = logical_block(p.nwg);
-  int m_lo = 0, m_hi = p.nblk;                     // blocks of steps this launch sweeps
-  int my_band = 0, band_q0 = 0;
-  if constexpr (SLICED) {
+  int lb = SLICED ? (int)blockIdx.x : logical_block(p.nwg);   // (linked bands keep the launch order: a band waits for a lower index)
+  int m_lo = 0, m_hi = p.nblk;                     // blocks of steps this workgroup sweeps
+  int my_band = 0;
+  Link link;
+  if constexpr (SLICED) {   // the window of one band
     const int per = p.B * p.bpb;
-    const int kk = lb / per;
-    lb -= kk * per;
-    my_band = p.sl_band0 + kk;
-    band_q0 = (p.sl_ell - kSliceLag * my_band) * kSliceQ;
-    m_lo = my_band * p.sl_nbb + band_q0;
-    m_hi = my_band * p.sl_nbb + (band_q0 + kSliceQ < p.sl_nbb ? band_q0 + kSliceQ : p.sl_nbb);
+    my_band = lb / per;
+    lb -= my_band * per;
+    m_lo = my_band * p.sl_nbb;
+    m_hi = m_lo + p.sl_nbb;
+    link.mine = p.prog + (int64_t)my_band * per + lb;
+    link.dep = my_band > 0 ? link.mine - per : nullptr;
+    link.err = p.link_err;
   }
   const int b = lb / p.bpb;
   const int e_wg0 = (lb % p.bpb) * CW;
@@ -679,17 +736,6 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   for (int c = 0; c < EC; ++c)
 #pragma unroll
     for (int n = 0; n < kN; ++n) h[c][n] = 0.f;
-  float* carry = SLICED ? p.carry + ((((int64_t)b * p.nbands + my_band) * p.E + e0) * kN) * kHB + r : nullptr;
-  if (SLICED && band_q0 > 0) {   // the band is under way: take over the state of the previous launch
-    if (ch_ok) {
-#pragma unroll
-      for (int c = 0; c < EC; ++c)
-#pragma unroll
-        for (int n = 0; n < kN; ++n) h[c][n] = carry[(c * kN + n) * kHB];
-    }
-    settle_loads();
-  }
-
   bool ck_mine = false;       // the lane stores a snapshot in the first step of the current block
   float4* ckp = nullptr;      // where to
   auto step = [&](int k, const Ops& o) {
@@ -744,8 +790,10 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
         for (int c = 0; c < EC; ++c)
 #pragma unroll
           for (int q = 0; q < 4; ++q)
-            tw[c * 4 + q] = make_float4(h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)],
-                                              h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
+          {
+            const float4 row = make_float4(h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)], h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
+            if constexpr (SLICED) store_row_device_scope(tw + c * 4 + q, row); else tw[c * 4 + q] = row;
+          }
       }
     }
     if (WRITE_Y && inr)
@@ -755,6 +803,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   Pos A = pos_of(p, m_lo * kCK - (kHB - 1));     // position of the stream index t0 - 15 (wave-uniform)
   bp = block_pos(p, A, r, rbands);
   int cell0 = cell_of(p, bp.bnd0, r, bp.col0);   // cell index of the lane's position at the first step of the block
+  if constexpr (SLICED) link.wait_for(link_need_fwd(0, p.sl_nbb));
   stage_block<T, 3, CW, false, STAGE_X, NW>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
   staging_fence();
   Ops opsA, opsB;
@@ -766,8 +815,10 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     const Pos An = pos_after(p, A, kCK);
     const BlockPos bpn = block_pos(p, An, r, rbands);
     const int celln = cell_of(p, bpn.bnd0, r, bpn.col0);
-    if (!last)
+    if (!last) {
+      if constexpr (SLICED) link.wait_for(link_need_fwd(m + 1 - m_lo, p.sl_nbb));
       stage_block<T, 3, CW, false, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, An, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+    }
     cell_off0 = (uint32_t)(cell0 * p.E + e0) * (uint32_t)sizeof(T);
     // Snapshot of the state before the block (after step t0-1) for the lanes whose previous
     // position was a cell of the grid; the others hold nothing the backward needs.  The stores are
@@ -808,6 +859,8 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
           // barrier, and no wave reads the current buffer any more.
           next_block_landed();
           __syncthreads();
+          // every wave has waited for what it issued before this block's copies: the blocks before this one are in memory
+          if constexpr (SLICED) link.publish((uint32_t)(m - m_lo));
           if (!last) fetch(bufn, 0, ahead);
         }
         step(k, now);   // also past the end of the sweep (last block): zero operands like any position off the grid, nothing stored
@@ -823,17 +876,17 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
         step(k, opsA);
       }
       __syncthreads();
+      if constexpr (SLICED) link.publish((uint32_t)(m - m_lo));
     }
     cur ^= 1;
     A = An;
     bp = bpn;
     cell0 = celln;
   }
-  if (SLICED && ch_ok && m_hi < (my_band + 1) * p.sl_nbb) {   // more of the band to come: hand the state to the next launch
-#pragma unroll
-    for (int c = 0; c < EC; ++c)
-#pragma unroll
-      for (int n = 0; n < kN; ++n) carry[(c * kN + n) * kHB] = h[c][n];
+  if constexpr (SLICED) {   // the whole window is done once every store of every wave has completed
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    link.publish((uint32_t)p.sl_nbb);
   }
 }
 
@@ -876,17 +929,20 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   char* lds = reinterpret_cast<char*>(a_lds + NW * CS * 2 * kN);  // 2 staging buffers
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  int lb = logical_block(p.nwg);
-  int m_lo = 0, m_hi = p.nblk;              // blocks of steps this launch sweeps (from m_hi - 1 down to m_lo)
-  int my_band = 0, band_q0 = 0;
-  if constexpr (SLICED) {
+  int lb = SLICED ? (int)blockIdx.x : logical_block(p.nwg);   // (linked bands keep the launch order: a band waits for a lower index)
+  int m_lo = 0, m_hi = p.nblk;              // blocks of steps this workgroup sweeps (from m_hi - 1 down to m_lo)
+  int my_band = 0;
+  Link link;
+  if constexpr (SLICED) {   // the window of one band; the bands are launched from the last to the first
     const int per = p.B * p.bpb;
     const int kk = lb / per;
     lb -= kk * per;
-    my_band = p.sl_band0 + kk;
-    band_q0 = (p.sl_ell - kSliceLag * (p.nbands - 1 - my_band)) * kSliceQ;   // blocks of the band already swept
-    m_hi = (my_band + 1) * p.sl_nbb - band_q0;
-    m_lo = m_hi - kSliceQ > my_band * p.sl_nbb ? m_hi - kSliceQ : my_band * p.sl_nbb;
+    my_band = p.nbands - 1 - kk;
+    m_lo = my_band * p.sl_nbb;
+    m_hi = m_lo + p.sl_nbb;
+    link.mine = p.prog + (int64_t)my_band * per + lb;
+    link.dep = my_band + 1 < p.nbands ? link.mine + per : nullptr;
+    link.err = p.link_err;
   }
   const int b = lb / p.bpb;
   const int eg = lb % p.bpb;
@@ -937,20 +993,6 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   float muT[kN], muL[kN];
 #pragma unroll
   for (int n = 0; n < kN; ++n) { accAT[n] = 0.f; accAL[n] = 0.f; muT[n] = 0.f; muL[n] = 0.f; }
-  // sliced sweep: adjoint state and position sums travel from launch to launch
-  float* carry = SLICED ? p.carry + ((((int64_t)b * p.nbands + my_band) * p.E + e) * (4 * kN + 1)) * kHB + r : nullptr;
-  if (SLICED && band_q0 > 0) {
-    if (ch_ok) {
-#pragma unroll
-      for (int n = 0; n < kN; ++n) {
-        muT[n] = carry[n * kHB]; muL[n] = carry[(kN + n) * kHB];
-        accAT[n] = carry[(2 * kN + n) * kHB]; accAL[n] = carry[(3 * kN + n) * kHB];
-      }
-      accD = carry[4 * kN * kHB];
-    }
-    settle_loads();
-  }
-
   // byte offsets of the lane's operand record inside a staging buffer at step 0 of a block, and
   // its advance per step: a grid row reads (B_T, B_L, C) of its cell; the upper ghost (lane 0)
   // reads the row above as its B_T; the lower ghost (lane 15) reads the row of mu_T below as its C.
@@ -1013,6 +1055,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   int cell0 = cell_of(p, bp.bnd0, r, bp.col0);   // cell index of the lane's position at the first step of the block
   bool ck_take = snapshot_lane(p, Pos{bp.bnd0, bp.col0}, r, ch_ok);   // the lane restores a snapshot for the block to come
   load_ckpt(m_hi - 1, ck_take);
+  if constexpr (SLICED) link.wait_for(link_need_bwd(p.sl_nbb - 1, p.sl_nbb));
   stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
   staging_fence();
   int cur = 0;
@@ -1029,8 +1072,10 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
     const BlockPos bpn = block_pos(p, Aprev, r, rbands);
     const int celln = cell_of(p, bpn.bnd0, r, bpn.col0);
     ck_take = snapshot_lane(p, Pos{bpn.bnd0, bpn.col0}, r, ch_ok);
-    if (m > m_lo)
+    if (m > m_lo) {
+      if constexpr (SLICED) link.wait_for(link_need_bwd(m - 1 - m_lo, p.sl_nbb));
       stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+    }
     cell_off0 = (uint32_t)(cell0 * p.E + e) * (uint32_t)sizeof(T);
     f_off0 = (uint32_t)cell0 * (uint32_t)(3 * kN * sizeof(float)) + f_sub;
 
@@ -1180,9 +1225,10 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
               char* bb = BOTimg + (wk ? bp.bnd0 + 1 : bp.bnd0) * p.bot_stride * (int64_t)sizeof(float) +
                          (uint32_t)(ck * p.E + e) * (uint32_t)(kN * sizeof(float));
 #pragma unroll
-              for (int q = 2 * half; q < 2 * half + 2; ++q)   // the two state groups of this half, as of this step
-                reinterpret_cast<float4*>(bb)[q] = make_float4(muT[sinv<PERM>(4 * q)], muT[sinv<PERM>(4 * q + 1)],
-                                                               muT[sinv<PERM>(4 * q + 2)], muT[sinv<PERM>(4 * q + 3)]);
+              for (int q = 2 * half; q < 2 * half + 2; ++q) {   // the two state groups of this half, as of this step
+                const float4 row = make_float4(muT[sinv<PERM>(4 * q)], muT[sinv<PERM>(4 * q + 1)], muT[sinv<PERM>(4 * q + 2)], muT[sinv<PERM>(4 * q + 3)]);
+                if constexpr (SLICED) store_row_device_scope(reinterpret_cast<float4*>(bb) + q, row); else reinterpret_cast<float4*>(bb)[q] = row;
+              }
             }
           }
           if (half == 0) {
@@ -1224,23 +1270,19 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
       }
     }
     __syncthreads();
+    // every wave has waited (before the last stores of this block) for all it had issued: the blocks swept before this one are in memory
+    if constexpr (SLICED) link.publish((uint32_t)(m_hi - 1 - m));
     A = Aprev;
     bp = bpn;
     cell0 = celln;
     cur ^= 1;
   }
-
-  if (SLICED && m_lo > my_band * p.sl_nbb) {   // more of the band to come: hand over to the next launch
-    if (ch_ok) {
-#pragma unroll
-      for (int n = 0; n < kN; ++n) {
-        carry[n * kHB] = muT[n]; carry[(kN + n) * kHB] = muL[n];
-        carry[(2 * kN + n) * kHB] = accAT[n]; carry[(3 * kN + n) * kHB] = accAL[n];
-      }
-      carry[4 * kN * kHB] = accD;
-    }
-    return;
+  if constexpr (SLICED) {   // the whole window is done once every store of every wave has completed
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    link.publish((uint32_t)p.sl_nbb);
   }
+
   // ---- sums over positions: reduce over the rows of the band (lanes of one channel slot)
   float red[2 * kN + 1];
 #pragma unroll
@@ -1271,9 +1313,12 @@ __device__ __forceinline__ float as_stored(float v, const bf16_t*) { return bf16
 // are rounded to T, which is what the reference's casts to x.dtype do (wavefront_cuda.py:72-73,
 // 90-91, 332).
 template <typename T, bool RAW>
-__global__ void m2d_prep_kernel(const void* ATv, const void* ALv, const void* Dv, float* zeros, float* A2T, float* A2L, float* Df, int E) {
+__global__ void m2d_prep_kernel(const void* ATv, const void* ALv, const void* Dv, float* zeros, float* A2T, float* A2L, float* Df, int E,
+                                uint32_t* link_words, int n_link_words) {
   const int idx = blockIdx.x * blockDim.x + threadIdx.x;
   if (idx < kZeroFloats) zeros[idx] = 0.f;
+  // linked sweep: error word and progress counts start at zero
+  for (int i = idx; i < n_link_words; i += gridDim.x * blockDim.x) link_words[i] = 0u;
   if constexpr (RAW) {
     const float *AT = static_cast<const float*>(ATv), *AL = static_cast<const float*>(ALv), *D = static_cast<const float*>(Dv);
     if (idx < E * kN) {
@@ -1399,11 +1444,11 @@ struct Geometry {
   int fwd_ec, fwd_nw, fwd_wpb, fwd_bpb;   // forward: channels per lane, waves per workgroup, waves and workgroups per image
   int bwd_nw, bwd_wpb, bwd_bpb;      // backward: waves per workgroup, waves and workgroups (channel groups) per image
   bool stage_x;                      // x, delta, dy rows are whole 16-byte chunks: stage them through LDS
-  bool sliced;                       // bands on workgroups of their own, swept by a sequence of launches
+  bool sliced;                       // linked sweep: bands on workgroups of their own, handing boundary rows to each other inside one launch
   bool stacked;                      // images of one band stacked into tall images of independent bands
   int ips, vB, vH;                   // images per stack; number and height of what the kernels sweep
-  int nbb, nlaunch;                  // sliced: blocks per band, launches per sweep
-  size_t carry_fwd_bytes, carry_bwd_bytes;
+  int nbb;                           // linked sweep: blocks per band
+  size_t link_bytes;                 // linked sweep: error word and the two arrays of progress counts (forward, backward)
   bool packed_bc;
   size_t prep_bytes, bc_bytes, ckpt_diag_bytes, top_bytes, bot_bytes, part_bytes, pa_bytes, pd_bytes;
 };
@@ -1483,7 +1528,7 @@ Geometry make_geometry(const m2d_desc* d) {
   g.nblk = (g.T_total + kCK - 1) / kCK;
   // Few images with many bands leave most of the device idle when each image is one sequential
   // stream.  Then every band gets workgroups of its own (a padded stream, one window of S steps
-  // per band) and the sweep becomes a sequence of launches in which band k trails band k-1.
+  // per band), all in one launch, and band k trails band k-1 by kLinkLag blocks of steps.
   g.sliced = !g.stacked && g.nbands >= 4 && (int64_t)B * groups <= ncu / 4;
   if (g.sliced && g.nbands == 4) {
     // Four bands (more bands favour the sliced sweep again: 84x84 measured) and a batch that fills half the device with workgroups of 4 waves, but not with
@@ -1491,19 +1536,18 @@ Geometry make_geometry(const m2d_desc* d) {
     // is then the faster schedule (56x56, 64 images of 32 channels: 0.99 -> 0.93 ms forward+backward).
     int s_sl = (d->W + kHB - 1 + kCK - 1) / kCK * kCK;
     if (s_sl < 28) s_sl = 28;
-    const int nlb = (s_sl / kCK + kSliceQ - 1) / kSliceQ;
-    const int64_t under_way = (nlb + kSliceLag - 1) / kSliceLag < g.nbands ? (nlb + kSliceLag - 1) / kSliceLag : g.nbands;
+    const int64_t lagged = (s_sl / kCK + kLinkLag) / (kLinkLag + 1);   // bands whose windows overlap in time (a block more for the polling)
+    const int64_t under_way = lagged < g.nbands ? lagged : g.nbands;
     const int64_t half = (int64_t)B * ((d->E + kFwdHalfWaves * g.CS - 1) / (kFwdHalfWaves * g.CS));
     if (half > (int64_t)B * groups && half <= ncu && half >= ncu / 2 && half * under_way > ncu) g.sliced = false;
   }
-  g.nbb = 0; g.nlaunch = 1;
+  g.nbb = 0;
   if (g.sliced) {
     g.S = (d->W + kHB - 1 + kCK - 1) / kCK * kCK;
     if (g.S < 28) g.S = 28;
     g.nbb = g.S / kCK;
     g.T_total = g.nbands * g.S;
     g.nblk = g.nbands * g.nbb;
-    g.nlaunch = kSliceLag * (g.nbands - 1) + (g.nbb + kSliceQ - 1) / kSliceQ;
   }
   // forward: two channels per lane where that saves rounds of workgroups (one workgroup per compute
   // unit at a time, 256 units) and the two staging buffers of such a workgroup fit the LDS (bf16
@@ -1520,11 +1564,10 @@ Geometry make_geometry(const m2d_desc* d) {
   // forward of a small batch in one stream per image: workgroups of 4 waves (16 channels) where those
   // are more than the workgroups of 8 and still no more than the compute units
   const int64_t wg_half = (int64_t)B * ((d->E + kFwdHalfWaves * g.CS - 1) / (kFwdHalfWaves * g.CS));
-  // (the sliced sweep has at most every kSliceLag-th launch window of a band under way at a time)
-  const int64_t together = g.sliced ? (((g.nbb + kSliceQ - 1) / kSliceQ + kSliceLag - 1) / kSliceLag < g.nbands
-                                           ? ((g.nbb + kSliceQ - 1) / kSliceQ + kSliceLag - 1) / kSliceLag : g.nbands) : 1;
-  // (a sliced sweep may exceed the units by a few workgroups while most bands are under way: its first
-  // and last launches, with fewer bands, still gain)
+  // (in the linked sweep the windows of about nbb / (kLinkLag + 1) bands overlap in time: the lag and a block for the polling)
+  const int64_t together = g.sliced ? ((g.nbb + kLinkLag) / (kLinkLag + 1) < g.nbands ? (g.nbb + kLinkLag) / (kLinkLag + 1) : g.nbands) : 1;
+  // (a linked sweep may exceed the units by a few workgroups while most bands are under way: its start
+  // and its end, with fewer bands, still gain)
   const int64_t room = g.sliced ? ncu + ncu / 16 : ncu;
   g.fwd_nw = (!g.stacked && !ec2 && wg_half > wg1 && wg_half * together <= room) ? kFwdHalfWaves : kFwdWaves;
   g.fwd_bpb = (d->E + g.fwd_nw * g.CS * g.fwd_ec - 1) / (g.fwd_nw * g.CS * g.fwd_ec);
@@ -1541,8 +1584,8 @@ Geometry make_geometry(const m2d_desc* d) {
   const bool rows = g.nbands > 1 && !g.stacked;   // boundary rows travel between bands
   g.top_bytes = rows ? align_up(sizeof(float) * (size_t)(g.nbands - 1) * B * d->W * d->E * kN) : 0;
   g.bot_bytes = rows ? align_up(sizeof(float) * (size_t)(g.sliced ? g.nbands : 1) * B * d->W * d->E * kN) : 0;
-  g.carry_fwd_bytes = g.sliced ? align_up(sizeof(float) * (size_t)B * g.nbands * d->E * kN * kHB) : 0;
-  g.carry_bwd_bytes = g.sliced ? align_up(sizeof(float) * (size_t)B * g.nbands * d->E * (4 * kN + 1) * kHB) : 0;
+  const size_t chains = (size_t)B * (g.fwd_bpb > g.bwd_bpb ? g.fwd_bpb : g.bwd_bpb);
+  g.link_bytes = g.sliced ? align_up(sizeof(uint32_t) * (64 + 2 * g.nbands * chains)) : 0;
   g.part_bytes = align_up(sizeof(float) * (size_t)g.bwd_bpb * 3 * P * kN);
   const size_t slots = g.sliced ? g.nbands : 1;
   g.pa_bytes = align_up(sizeof(float) * (size_t)B * slots * d->E * 2 * kN);
@@ -1554,11 +1597,11 @@ Geometry make_geometry(const m2d_desc* d) {
 size_t ckpt_bytes_of(const Geometry& g) { return g.ckpt_diag_bytes + g.top_bytes + g.bc_bytes; }
 
 size_t workspace_bytes_of(const Geometry& g, int pass, int have_ckpt) {
-  size_t n = g.prep_bytes + g.carry_fwd_bytes;   // (a backward without checkpoints runs a forward sweep first)
+  size_t n = g.prep_bytes + g.link_bytes;
   if (pass == M2D_PASS_FWD) {
     if (!have_ckpt) n += g.top_bytes + g.bc_bytes;
   } else {
-    n += g.part_bytes + g.pa_bytes + g.pd_bytes + g.bot_bytes + g.carry_bwd_bytes;
+    n += g.part_bytes + g.pa_bytes + g.pd_bytes + g.bot_bytes;
     if (!have_ckpt) n += ckpt_bytes_of(g);
   }
   return n;
@@ -1573,7 +1616,7 @@ void fill_common(ScanParams& sp, const m2d_desc* d, const Geometry& g) {
   sp.nbands = g.nbands; sp.nblk = g.nblk;
   sp.S = g.S; sp.T_total = g.T_total; sp.rows_last = g.rows_last;
   sp.magicS = (uint32_t)(((uint64_t)1 << 32) / (uint64_t)g.S);
-  sp.sliced = g.sliced ? 1 : 0; sp.sl_nbb = g.nbb; sp.sl_ell = 0; sp.sl_band0 = 0;
+  sp.sliced = g.sliced ? 1 : 0; sp.sl_nbb = g.nbb;
   sp.pa_slots = g.sliced ? g.nbands : 1;
   sp.bot_stride = g.sliced ? (int64_t)g.vB * d->W * d->E * kN : 0;
   sp.flip = (d->flags & M2D_FLAG_FLIP) ? 1 : 0;
@@ -1594,7 +1637,10 @@ inline bool allow_dynamic_lds(const void* kernel, size_t bytes, std::atomic<uint
 
 // Set-up area: [page of zeros][A_T*log2e][A_L*log2e][D], all fp32.
 template <typename T>
-int launch_prep(ScanParams& sp, const m2d_desc* d, const void* AT, const void* AL, const void* D, float* base, hipStream_t st) {
+int launch_prep(ScanParams& sp, const m2d_desc* d, const Geometry& g, const void* AT, const void* AL, const void* D, float* base,
+                uint32_t* link_words, hipStream_t st) {
+  const int n_link = (int)(g.link_bytes / sizeof(uint32_t));
+  sp.link_err = link_words;   // (the first 64 words: the error word; then forward counts, then backward counts)
   float* zeros = base;
   float* A2T = base + kZeroFloats;
   float* A2L = A2T + (size_t)d->E * kN;
@@ -1602,9 +1648,9 @@ int launch_prep(ScanParams& sp, const m2d_desc* d, const void* AT, const void* A
   sp.zeros = zeros; sp.A2T = A2T; sp.A2L = A2L; sp.Df = Df;
   const int n = d->E * kN > kZeroFloats ? d->E * kN : kZeroFloats;
   if (d->flags & M2D_FLAG_RAW_PARAMS)
-    hipLaunchKernelGGL((m2d_prep_kernel<T, true>), dim3((n + 255) / 256), dim3(256), 0, st, AT, AL, D, zeros, A2T, A2L, Df, d->E);
+    hipLaunchKernelGGL((m2d_prep_kernel<T, true>), dim3((n + 255) / 256), dim3(256), 0, st, AT, AL, D, zeros, A2T, A2L, Df, d->E, link_words, n_link);
   else
-    hipLaunchKernelGGL((m2d_prep_kernel<T, false>), dim3((n + 255) / 256), dim3(256), 0, st, AT, AL, D, zeros, A2T, A2L, Df, d->E);
+    hipLaunchKernelGGL((m2d_prep_kernel<T, false>), dim3((n + 255) / 256), dim3(256), 0, st, AT, AL, D, zeros, A2T, A2L, Df, d->E, link_words, n_link);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
@@ -1646,7 +1692,7 @@ int launch_fwd(const ScanParams& sp0, const m2d_desc* d, const Geometry& g, bool
   sp.bpb = g.fwd_bpb;
   sp.nwg = g.vB * g.fwd_bpb;
   auto once = [&]() {
-    if (g.sliced) {   // (the sliced sweep is only chosen where one channel per lane is)
+    if (g.sliced) {   // (the linked sweep is only chosen where one channel per lane is)
       if (g.fwd_nw == kFwdHalfWaves)
         return g.stage_x ? launch_fwd_mode<T, 1, true, kModeSliced, kFwdHalfWaves>(sp, ckpt, write_y, st)
                          : launch_fwd_mode<T, 1, false, kModeSliced, kFwdHalfWaves>(sp, ckpt, write_y, st);
@@ -1666,20 +1712,11 @@ int launch_fwd(const ScanParams& sp0, const m2d_desc* d, const Geometry& g, bool
                        : launch_fwd_mode<T, 1, false, kModeSweep, kFwdHalfWaves>(sp, ckpt, write_y, st);
     return g.stage_x ? launch_fwd_mode<T, 1, true, kModeSweep>(sp, ckpt, write_y, st) : launch_fwd_mode<T, 1, false, kModeSweep>(sp, ckpt, write_y, st);
   };
-  if (!g.sliced) return once();
-  // launch l advances band k by blocks [(l - lag*k)*Q, +Q) of its window, for the bands under way
-  const int nlb = (g.nbb + kSliceQ - 1) / kSliceQ;
-  for (int l = 0; l < g.nlaunch; ++l) {
-    int k_hi = l / kSliceLag, k_lo = (l - nlb + 1 + kSliceLag - 1) / kSliceLag;
-    if (l - nlb + 1 < 0) k_lo = 0;
-    if (k_hi > g.nbands - 1) k_hi = g.nbands - 1;
-    if (k_lo > k_hi) continue;
-    sp.sl_ell = l; sp.sl_band0 = k_lo;
-    sp.nwg = (k_hi - k_lo + 1) * g.vB * g.fwd_bpb;
-    const int rc = once();
-    if (rc) return rc;
+  if (g.sliced) {   // every band on workgroups of its own, band 0 first: a band waits for the one before it
+    sp.nwg = g.nbands * g.vB * g.fwd_bpb;
+    sp.prog = sp.link_err + 64;
   }
-  return M2D_OK;
+  return once();
 }
 
 template <typename T>
@@ -1688,11 +1725,11 @@ int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   char* w = static_cast<char*>(ws);
   float* prep = reinterpret_cast<float*>(w);
   w += g.prep_bytes;
-  sp.carry = reinterpret_cast<float*>(w); w += g.carry_fwd_bytes;
+  uint32_t* link_words = reinterpret_cast<uint32_t*>(w); w += g.link_bytes;
   char* keep = ckpt ? static_cast<char*>(ckpt) + g.ckpt_diag_bytes : w;   // [top][widened B,C]
   sp.ckpt = ckpt ? static_cast<float*>(ckpt) : nullptr;
   sp.top = reinterpret_cast<float*>(keep);
-  int rc = launch_prep<T>(sp, d, AT, AL, D, prep, st);
+  int rc = launch_prep<T>(sp, d, g, AT, AL, D, prep, link_words, st);
   if (rc) return rc;
   rc = stage_bc<T>(sp, d, BT, BL, C, reinterpret_cast<float*>(keep + g.top_bytes), false, st);
   if (rc) return rc;
@@ -1725,13 +1762,12 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
             void* dBL, void* dC, void* dD, void* ws, hipStream_t st) {
   char* w = static_cast<char*>(ws);
   float* prep = reinterpret_cast<float*>(w); w += g.prep_bytes;
-  float* carry_fwd = reinterpret_cast<float*>(w); w += g.carry_fwd_bytes;
-  float* carry_bwd = reinterpret_cast<float*>(w); w += g.carry_bwd_bytes;
+  uint32_t* link_words = reinterpret_cast<uint32_t*>(w); w += g.link_bytes;
   sp.part = reinterpret_cast<float*>(w); w += g.part_bytes;
   sp.pA = reinterpret_cast<float*>(w); w += g.pa_bytes;
   sp.pD = reinterpret_cast<float*>(w); w += g.pd_bytes;
   sp.bot = reinterpret_cast<float*>(w); w += g.bot_bytes;
-  int rc = launch_prep<T>(sp, d, AT, AL, D, prep, st);
+  int rc = launch_prep<T>(sp, d, g, AT, AL, D, prep, link_words, st);
   if (rc) return rc;
   char* ck = ckpt ? const_cast<char*>(static_cast<const char*>(ckpt)) : w;
   sp.ckpt = reinterpret_cast<float*>(ck);
@@ -1739,11 +1775,9 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   rc = stage_bc<T>(sp, d, BT, BL, C, reinterpret_cast<float*>(ck + g.ckpt_diag_bytes + g.top_bytes), ckpt != nullptr, st);
   if (rc) return rc;
   if (!ckpt) {   // rebuild the checkpoints with one forward sweep that writes no y
-    sp.carry = carry_fwd;
     rc = launch_fwd<T>(sp, d, g, true, false, st);
     if (rc) return rc;
   }
-  sp.carry = carry_bwd;
   sp.bpb = g.bwd_bpb;
   sp.nwg = g.vB * g.bwd_bpb;
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][0], st);
@@ -1751,17 +1785,10 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
     if (g.stacked) rc = g.stage_x ? launch_bwd<T, true, kModeStacked>(sp, st) : launch_bwd<T, false, kModeStacked>(sp, st);
     else rc = g.stage_x ? launch_bwd<T, true, kModeSweep>(sp, st, g.bwd_nw) : launch_bwd<T, false, kModeSweep>(sp, st, g.bwd_nw);
   } else {
-    // as the forward, bottom-up: launch l advances the band k' from the bottom by Q blocks of its window
-    const int nlb = (g.nbb + kSliceQ - 1) / kSliceQ;
-    for (int l = 0; l < g.nlaunch && !rc; ++l) {
-      int k_hi = l / kSliceLag, k_lo = (l - nlb + 1 + kSliceLag - 1) / kSliceLag;
-      if (l - nlb + 1 < 0) k_lo = 0;
-      if (k_hi > g.nbands - 1) k_hi = g.nbands - 1;
-      if (k_lo > k_hi) continue;
-      sp.sl_ell = l; sp.sl_band0 = g.nbands - 1 - k_hi;
-      sp.nwg = (k_hi - k_lo + 1) * g.vB * g.bwd_bpb;
-      rc = g.stage_x ? launch_bwd<T, true, kModeSliced>(sp, st, g.bwd_nw) : launch_bwd<T, false, kModeSliced>(sp, st, g.bwd_nw);
-    }
+    // every band on workgroups of its own, the last band first: a band waits for the one below it
+    sp.nwg = g.nbands * g.vB * g.bwd_bpb;
+    sp.prog = sp.link_err + 64 + (size_t)g.nbands * g.vB * (g.fwd_bpb > g.bwd_bpb ? g.fwd_bpb : g.bwd_bpb);
+    rc = g.stage_x ? launch_bwd<T, true, kModeSliced>(sp, st, g.bwd_nw) : launch_bwd<T, false, kModeSliced>(sp, st, g.bwd_nw);
   }
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][1], st);
   if (rc) return rc;
