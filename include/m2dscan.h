@@ -122,6 +122,15 @@ int m2d_scan_fwd(const m2d_desc* desc,
                  void* workspace, size_t workspace_bytes,
                  void* stream);
 
+/* Debugging aid for grids of many bands and few images, whose bands run on workgroups of their own
+ * inside one launch and wait for each other's boundary rows (a bounded wait: a workgroup that has
+ * polled about a million times gives up, so that the launch always ends; the results are then
+ * invalid).  Synchronises `stream` and reads, from the workspace of the last m2d_scan_fwd or
+ * m2d_scan_bwd call of this descriptor on it, whether any workgroup gave up: *gave_up = 0 or 1 (always
+ * 0 for problems that do not run that way).  No counterpart in the reference (its diagonals are
+ * ordered by kernel launches, wf_cuda.cu:203,259). */
+int m2d_scan_link_error(const m2d_desc* desc, const void* workspace, void* stream, int* gave_up);
+
 /* m2d_scan_fwd without a checkpoint buffer and without a workspace argument, for callers that cannot
  * allocate device memory (code under HIP graph capture, tight serving loops, harnesses that forbid
  * it).  It has no counterpart in the reference, whose Python side allocates every buffer with

@@ -22,7 +22,7 @@ M2D_FLAG_DPRE = 16
 M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
-           "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_fwd_noalloc", "m2d_scan_bwd", "m2d_proj_workspace_bytes", "m2d_proj_fwd",
+           "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_fwd_noalloc", "m2d_scan_link_error", "m2d_scan_bwd", "m2d_proj_workspace_bytes", "m2d_proj_fwd",
            "m2d_proj_bwd", "m2d_layernorm_fwd", "m2d_dwconv3x3_fwd", "m2d_starrelu_fwd",
            "m2d_scale_residual_fwd", "m2d_scale_residual_layernorm_fwd", "m2d_rope_qknorm_fwd", "m2d_rope_attention_fwd", "m2d_mlp_fwd", "m2d_layernorm_linear_fwd", "m2d_linear_fwd", "m2d_profile_enable", "m2d_profile_last_ms")
 
@@ -56,6 +56,8 @@ def _load():
     lib.m2d_scan_ckpt_bytes.argtypes = [dp]
     lib.m2d_scan_fwd.restype = i32
     lib.m2d_scan_fwd.argtypes = [dp] + [vp] * 9 + [vp, vp, sz, vp, sz, vp]
+    lib.m2d_scan_link_error.restype = i32
+    lib.m2d_scan_link_error.argtypes = [dp, vp, vp, ctypes.POINTER(ctypes.c_int)]
     lib.m2d_scan_fwd_noalloc.restype = i32
     lib.m2d_scan_fwd_noalloc.argtypes = [dp] + [vp] * 9 + [vp, vp]
     lib.m2d_scan_bwd.restype = i32
@@ -163,6 +165,17 @@ def _bytes(n, dev):
     return torch.empty(max(int(n), 1), dtype=torch.uint8, device=dev)
 
 
+CHECK_LINKS = False   # tests set this: every scan call then synchronises and raises if a workgroup gave up waiting
+
+
+def _check_links(d, ws, dev):
+    if CHECK_LINKS:
+        flag = ctypes.c_int(0)
+        check(lib.m2d_scan_link_error(ctypes.byref(d), _ptr(ws), _stream(dev), ctypes.byref(flag)))
+        if flag.value:
+            raise RuntimeError("m2dscan: a workgroup of the linked sweep gave up waiting for its neighbour")
+
+
 def scan_fwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, save_ckpt=False, flip=False):
     """y (and the checkpoint buffer when ``save_ckpt``) through m2d_scan_fwd."""
     _same(x, deltaT, deltaL, AT, AL, BT, BL, C, D)
@@ -175,6 +188,7 @@ def scan_fwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, save_ckpt=False, flip=Fals
     check(lib.m2d_scan_fwd(ctypes.byref(d), *[_ptr(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D)],
                            _ptr(y), _ptr(ck), ck.numel() if ck is not None else 0, _ptr(ws), ws.numel(),
                            _stream(x.device)))
+    _check_links(d, ws, x.device)
     return (y, ck) if save_ckpt else y
 
 
@@ -207,6 +221,7 @@ def scan_bwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt=None, flip=False,
     check(lib.m2d_scan_bwd(ctypes.byref(d), *[_ptr(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy)],
                            _ptr(ckpt), ckpt.numel() if ckpt is not None else 0, *[_ptr(t) for t in outs],
                            _ptr(ws), ws.numel(), _stream(x.device)))
+    _check_links(d, ws, x.device)
     return tuple(outs)
 
 

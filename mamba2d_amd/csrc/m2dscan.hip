@@ -61,7 +61,7 @@ constexpr int kBwdWaves = 8;      // waves per backward workgroup
 constexpr int kZeroFloats = 64;     // page of zeros at the head of the set-up area
 constexpr int kModeSweep = 0, kModeSliced = 1, kModeStacked = 2;   // how the bands of the batch are scheduled
 constexpr int kLinkLag = 7;        // linked sweep: blocks by which a band trails the band it depends on (see link_need_*)
-constexpr int kSpinLimit = 1 << 20;   // linked sweep: polls of a neighbour's progress before a workgroup gives up waiting
+constexpr int kSpinLimit = 1 << 21;   // linked sweep: polls of a neighbour's progress before a workgroup gives up waiting
 constexpr uint32_t kLinkAbort = 0xffffffffu;   // progress value of a band that gave up: nobody waits for it
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
@@ -354,7 +354,7 @@ struct Link {
     for (int spin = 0; spin < kSpinLimit; ++spin) {
       seen = link_poll(dep);
       if (seen >= need) return;
-      __builtin_amdgcn_s_sleep(16);
+      __builtin_amdgcn_s_sleep(4);
     }
     seen = kLinkAbort;
     gave_up = true;
@@ -1900,6 +1900,21 @@ int m2d_scan_bwd(const m2d_desc* desc, const void* x, const void* deltaT, const 
   return desc->dtype == M2D_F32
              ? run_bwd<float>(desc, g, sp, AT, AL, BT, BL, C, D, ckpt, d_AT, d_AL, d_BT, d_BL, d_C, d_D, workspace, st)
              : run_bwd<bf16_t>(desc, g, sp, AT, AL, BT, BL, C, D, ckpt, d_AT, d_AL, d_BT, d_BL, d_C, d_D, workspace, st);
+}
+
+int m2d_scan_link_error(const m2d_desc* desc, const void* workspace, void* stream, int* gave_up) {
+  int rc = check_desc(desc);
+  if (rc) return rc;
+  if (!workspace || !gave_up) return M2D_ERR_NULL_POINTER;
+  const Geometry g = make_geometry(desc);
+  *gave_up = 0;
+  if (!g.sliced) return M2D_OK;   // no workgroup of this problem waits for another
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  uint32_t word = 0;
+  if (hipStreamSynchronize(st) != hipSuccess) return M2D_ERR_HIP;
+  if (hipMemcpy(&word, static_cast<const char*>(workspace) + g.prep_bytes, sizeof(word), hipMemcpyDeviceToHost) != hipSuccess) return M2D_ERR_HIP;
+  *gave_up = word != 0;
+  return M2D_OK;
 }
 
 int m2d_scan_fwd_noalloc(const m2d_desc* desc, const void* x, const void* deltaT, const void* deltaL, const void* AT,

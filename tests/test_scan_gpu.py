@@ -23,6 +23,7 @@ TOL_ELEM = {torch.float32: 2e-3, torch.bfloat16: 5e-2}
 @pytest.fixture(scope="module")
 def cabi():
     from mamba2d_amd import cabi as m
+    m.CHECK_LINKS = True   # a workgroup of the linked sweep that gives up waiting fails the test by name
     return m
 
 
@@ -230,3 +231,26 @@ def test_batch_beyond_two_giga_elements(cabi):
             assert e < 2e-2, (k, e)
     del y, grads, big, a
     torch.cuda.empty_cache()
+
+
+def test_linked_sweep_repeats_bit_identically_on_reused_buffers(cabi):
+    """One image of 22 bands, eight times over with other problems of the same sizes in between, so that the
+    allocator hands the same workspace and boundary-row addresses to every call: a band must see its
+    neighbour's rows of THIS call (they cross between XCDs through memory), never what a cache kept."""
+    say("\ncase linked_sweep_repeats")
+    shapes = [(1, 300, 64, 16, 7), (1, 300, 64, 16, 8)]
+    runs = {}
+    for it in range(8):
+        for (B, H, W, E, seed) in shapes:
+            inp = {k: v.cuda() for k, v in so.make_inputs(B, H, W, E, 16, seed=seed, dtype=torch.float32).items()}
+            a = [inp[k] for k in so.INPUT_NAMES]
+            y, ck = cabi.scan_fwd(*a, save_ckpt=True)
+            g = cabi.scan_bwd(*a, inp["dy"], ckpt=ck)
+            torch.cuda.synchronize()
+            got = [y.clone()] + [t.clone() for t in g]
+            del y, ck, g
+            if seed in runs:
+                for u, v in zip(runs[seed], got):
+                    assert torch.equal(u, v), (it, seed)
+            else:
+                runs[seed] = got
