@@ -901,6 +901,16 @@ __device__ __forceinline__ constexpr int fold_state(int m, int qi) {
   return q * 4 + m;
 }
 
+// Exchange buffers of the backward kernel (channel sums across the waves of a workgroup), in units
+// of one (step, half of the states) buffer of [wave][3][64] float2.  Where the LDS has room for one
+// buffer per step of a block (kCK), the sums of a half are exchanged in one go after its kCK adjoint
+// steps: two barriers per half instead of one per step.  Otherwise two buffers are used alternately
+// with one barrier per step.
+template <typename T, int NW>
+constexpr int bwd_exchange_sets() {
+  return sizeof(float2) * kCK * NW * 3 * 64 + sizeof(float) * NW * 4 * 2 * kN + 256 +
+         2 * (size_t)Stage<T, 4, NW * 4, true>::kBytes <= 160 * 1024 ? kCK : 2;
+}
 // As in the forward, lanes are never masked: rows outside the grid and cells outside the row work
 // on zero operands.  For the adjoint this means that a row which has not reached its last column
 // yet keeps lambda = mu = 0 exactly, and that a row past column 0 carries finite values that are
@@ -921,11 +931,15 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   constexpr bool PERM = true;
   using SG = Stage<T, 4, CW, true>;
   extern __shared__ float4 smem[];
-  // Exchange buffers for the channel sums of one (step, half of the states): two of them, used
-  // alternately, so that one barrier per exchange is enough (a buffer is rewritten two exchanges
-  // later, after a barrier that every wave reaches only once it has finished reading it).
-  float2* slots = reinterpret_cast<float2*>(smem);                       // [2][wave][3][64]
-  float* a_lds = reinterpret_cast<float*>(smem + NW * SLOT);      // [wave][CS][2][16], fold order
+  // Exchange buffers for the channel sums of one (step, half of the states).  Either one per step of
+  // a block (BATCH): the waves fill them during the kCK adjoint steps of a half, meet at a barrier,
+  // add up, and meet again before the next half fills them.  Or two, used alternately, with one
+  // barrier per step (a buffer is rewritten two exchanges later, after a barrier that every wave
+  // reaches only once it has finished reading it).
+  constexpr int XSETS = bwd_exchange_sets<T, NW>();
+  constexpr bool BATCH = XSETS == kCK;
+  float2* slots = reinterpret_cast<float2*>(smem);                       // [XSETS][wave][3][64]
+  float* a_lds = reinterpret_cast<float*>(slots + XSETS * NW * SLOT);    // [wave][CS][2][16], fold order
   char* lds = reinterpret_cast<char*>(a_lds + NW * CS * 2 * kN);  // 2 staging buffers
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -1077,7 +1091,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
       stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
     }
     cell_off0 = (uint32_t)(cell0 * p.E + e) * (uint32_t)sizeof(T);
-    f_off0 = (uint32_t)cell0 * (uint32_t)(3 * kN * sizeof(float)) + f_sub;
+    f_off0 = (uint32_t)cell0 * (uint32_t)(3 * kN * sizeof(float)) + (BATCH ? (uint32_t)(slot * 4 * sizeof(float)) : f_sub);
 
     // The 16 states are swept in two halves of 8 (state groups 0,1 then 2,3), each half
     // recomputing and then back-propagating the whole block: only 5 x 8 recomputed states are
@@ -1149,6 +1163,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
         }
       }
       // ---- adjoint over the block, last step first
+      if (BATCH && half == 1) __syncthreads();   // the sums of the first half have been taken out of the exchange buffers
 #pragma unroll
       for (int k = kCK - 1; k >= 0; --k) {
         const int t = t0 + k;
@@ -1179,7 +1194,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
           const float dyl = dyv + gb1;
           float sT = 0.f, sL = 0.f, zT = 0.f, zL = 0.f;
           if (half == 1) { sT = part4[k][0]; sL = part4[k][1]; zT = part4[k][2]; zL = part4[k][3]; }
-          float* sw = reinterpret_cast<float*>(slots + (xpar * NW + wave) * SLOT + lane);
+          float* sw = reinterpret_cast<float*>(slots + ((BATCH ? k : xpar) * NW + wave) * SLOT + lane);
           // A group of 4 states is folded over the 4 channel slots of the wave as soon as it is
           // done; afterwards the lane of slot q holds the channel sums of the states 4q..4q+3
           // (component mgl of its float2 after group mgl of this half).
@@ -1248,24 +1263,46 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
           }
           // ---- across the waves of the workgroup: the per-wave slots (this half's two state
           // groups) are added in wave order, one sum per thread, the same share for every wave
-          __syncthreads();
-          if (f_on && ((bp.in_grid >> k) & 1u)) {
-            const uint32_t off = f_off0 + (uint32_t)k * pstep + (k >= bp.kw ? pwrap_adj : 0u) + (uint32_t)(2 * half * sizeof(float));
-            if constexpr (PAIRS) {
-              const float2* sl = slots + xpar * NW * SLOT + f_it;
-              float2 s = sl[0];
+          if constexpr (!BATCH) {
+            __syncthreads();
+            if (f_on && ((bp.in_grid >> k) & 1u)) {
+              const uint32_t off = f_off0 + (uint32_t)k * pstep + (k >= bp.kw ? pwrap_adj : 0u) + (uint32_t)(2 * half * sizeof(float));
+              if constexpr (PAIRS) {
+                const float2* sl = slots + xpar * NW * SLOT + f_it;
+                float2 s = sl[0];
 #pragma unroll
-              for (int w = 1; w < NW; ++w) { s.x += sl[w * SLOT].x; s.y += sl[w * SLOT].y; }
-              *reinterpret_cast<float2*>(PARTimg + off) = s;
-            } else {
-              const float* sl = reinterpret_cast<const float*>(slots + xpar * NW * SLOT + f_it) + f_comp;
-              float s = sl[0];
+                for (int w = 1; w < NW; ++w) { s.x += sl[w * SLOT].x; s.y += sl[w * SLOT].y; }
+                *reinterpret_cast<float2*>(PARTimg + off) = s;
+              } else {
+                const float* sl = reinterpret_cast<const float*>(slots + xpar * NW * SLOT + f_it) + f_comp;
+                float s = sl[0];
 #pragma unroll
-              for (int w = 1; w < NW; ++w) s += sl[2 * w * SLOT];
-              *reinterpret_cast<float*>(PARTimg + off) = s;
+                for (int w = 1; w < NW; ++w) s += sl[2 * w * SLOT];
+                *reinterpret_cast<float*>(PARTimg + off) = s;
+              }
+            }
+            xpar ^= 1;
+          }
+        }
+      }
+      if constexpr (BATCH) {
+        // ---- across the waves, all steps of this half at once: the kCK x 3 (step, tensor) sets of
+        // sums are dealt to the waves; a thread adds up the float2 of the lane (its slot, its row)
+        __syncthreads();
+#pragma unroll
+        for (int rd = 0; rd < (kCK * 3 + NW - 1) / NW; ++rd) {
+          const int j = rd * NW + wave;                    // (uniform)
+          if (j < kCK * 3) {
+            const int k = j / 3, v = j - 3 * k;
+            if ((bp.in_grid >> k) & 1u) {
+              const uint32_t off = f_off0 + (uint32_t)k * pstep + (k >= bp.kw ? pwrap_adj : 0u) + (uint32_t)((v * kN + 2 * half) * sizeof(float));
+              const float2* sl = slots + k * NW * SLOT + v * 64 + lane;
+              float2 sum = sl[0];
+#pragma unroll
+              for (int w = 1; w < NW; ++w) { sum.x += sl[w * SLOT].x; sum.y += sl[w * SLOT].y; }
+              *reinterpret_cast<float2*>(PARTimg + off) = sum;
             }
           }
-          xpar ^= 1;
         }
       }
     }
@@ -1432,7 +1469,7 @@ template <typename T, int EC, int NW = kFwdWaves>
 constexpr size_t fwd_lds_bytes() { return 2 * (size_t)Stage<T, 3, NW * 4 * EC, false>::kBytes; }
 template <typename T, int NW = kBwdWaves>
 constexpr size_t bwd_lds_bytes() {
-  return sizeof(float4) * NW * 3 * 64 + sizeof(float) * NW * 4 * 2 * kN + 256 +
+  return sizeof(float2) * bwd_exchange_sets<T, NW>() * NW * 3 * 64 + sizeof(float) * NW * 4 * 2 * kN + 256 +
          2 * (size_t)Stage<T, 4, NW * 4, true>::kBytes;
 }
 static_assert(fwd_lds_bytes<float, 1>() <= kLdsPerWorkgroup && fwd_lds_bytes<bf16_t, 1>() <= kLdsPerWorkgroup, "forward staging must fit the LDS");
