@@ -188,6 +188,8 @@ struct ScanParams {
   float* pD;                        // [B*pa_slots][E]
   int B, H, W, E;
   int nbands, nblk, bc_stride, flip;
+  int bc_direct;                    // forward without snapshots: B_T, B_L, C are staged from the caller's tensors (states in natural order)
+  const void* bcd[4];               // ... those tensors (B_T, B_L, C; the fourth entry pads)
   int dpre;                         // backward: d_deltaT, d_deltaL leave multiplied by the slope of the softplus that made the deltas
   int S;                            // stream stride: positions per band (>= W)
   int T_total;                      // steps of the whole sweep
@@ -491,7 +493,7 @@ __device__ __forceinline__ int clamp_band(const ScanParams& p, int bnd) { return
 // index of its position at the first step: what the lane's copies fetch is what the lane itself will
 // work on).  A wave copies the operands of one step of the block, wave % kCK (the waves that share a
 // step take its copies in turn), so a lane works out one cell per block.
-template <typename T, int NT, int CW, bool WITH_BOT, bool STAGE_X, int NWAVES>
+template <typename T, int NT, int CW, bool WITH_BOT, bool STAGE_X, int NWAVES, bool SKIP_BC = false>
 __device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int b, Pos A, const BlockPos& q, int cell0,
                                             int e_wg0, int wave, int lane,
                                             const T* x0, const T* x1, const T* x2, const T* x3) {
@@ -526,12 +528,14 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int 
     if (slot == 0) *reinterpret_cast<float4*>(kbuf + SG::kConstPlane * SG::kPlane + r * 16) = kk;
   }
   // B_T, B_L, C: a copy moves the four state groups (lane >> 4) of one tensor for the 16 lane rows
+  if constexpr (!SKIP_BC) {
 #pragma unroll
-  for (int tsr = 0; tsr < 3; ++tsr)
-    if (tsr % WPK == wsub) {
-      const uint32_t off = (uint32_t)cell * (uint32_t)(p.bc_stride * 4) + (uint32_t)(tsr * kN * 4 + slot * 16);
-      lds_fill16<false>(ok ? bc_img + off : zeros, kbuf + tsr * 4 * SG::kPlane);
-    }
+    for (int tsr = 0; tsr < 3; ++tsr)
+      if (tsr % WPK == wsub) {
+        const uint32_t off = (uint32_t)cell * (uint32_t)(p.bc_stride * 4) + (uint32_t)(tsr * kN * 4 + slot * 16);
+        lds_fill16<false>(ok ? bc_img + off : zeros, kbuf + tsr * 4 * SG::kPlane);
+      }
+  }
   if constexpr (STAGE_X) {
     const int64_t img_bytes = img * p.E * (int64_t)sizeof(T);
     if constexpr (SG::kCpt >= 4) {   // one step per copy: lanes = (channel chunk, row)
@@ -588,6 +592,65 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int 
           src = p.bot + (qa.bnd + 1) * p.bot_stride + (((int64_t)b * p.W + qa.col) * p.E + ch) * kN + slot * 4;
         lds_fill16<true>(src, kbuf + (SG::kBotPlane + 4 * g) * SG::kPlane);
       }
+  }
+}
+
+// B_T, B_L, C straight from the caller's tensors (forward without snapshots: no packed fp32 copy is
+// made).  The records keep the natural order of the states.  fp32 tensors are copied into the planes
+// of a staging buffer like every other operand, one block ahead (bc_direct_copy).  16-bit tensors
+// are copied as they are into a small buffer of their own two blocks ahead (bc_raw_copy: one
+// wave-wide copy moves the 16 rows of two (step, tensor) pairs, 32 bytes a row), and are widened from
+// there into the planes of the next block's staging buffer while the current block is worked on
+// (bc_widen): LDS to LDS, so that no wait for a vector load ever stands between a block's stores.
+constexpr int kRawBytes = kCK * 3 * kHB * kN * 2;   // 16-bit B_T, B_L, C of one block: 6 KB
+template <typename T, int CW, int NWAVES>
+__device__ __forceinline__ void bc_direct_copy(const ScanParams& p, const void* const* tensors, char* buf, int b, const BlockPos& q,
+                                               int cell0, int wave, int lane) {
+  using SG = Stage<T, 3, CW, false>;
+  static_assert(sizeof(T) == 4, "fp32 records need no widening");
+  constexpr int WPK = NWAVES / kCK;
+  const int ks = wave & (kCK - 1), wsub = wave / kCK;
+  const int cstep = p.flip ? -1 : 1;
+  const int cell = cell0 + ks * cstep + (ks >= q.kw ? (kRB * p.W - p.S) * cstep : 0);
+  const bool ok = ((q.in_grid >> ks) & 1u) != 0;
+  const int slot = lane >> kHBShift;
+  const int64_t img_bytes = (int64_t)b * p.Hs * p.W * (kN * (int64_t)sizeof(T));
+#pragma unroll
+  for (int tsr = 0; tsr < 3; ++tsr)
+    if (tsr % WPK == wsub) {
+      const char* t_img = static_cast<const char*>(tensors[tsr]) + img_bytes;
+      lds_fill16<false>(ok ? t_img + ((uint32_t)cell * 64u + (uint32_t)slot * 16u) : reinterpret_cast<const char*>(p.zeros),
+                        buf + ks * SG::kKStr + tsr * 4 * SG::kPlane);
+    }
+}
+// q, cell0: the lane's row in the block to copy (block_pos); `live` false: zeros (there is no such block)
+template <int NWAVES>
+__device__ __forceinline__ void bc_raw_copy(const ScanParams& p, const void* const* tensors, char* raw, int b, const BlockPos& q,
+                                            int cell0, int wave, int lane, bool live) {
+  const int cstep = p.flip ? -1 : 1;
+  const int wrapc = (kRB * p.W - p.S) * cstep;
+  const int sel = lane >> 5, hf = (lane >> kHBShift) & 1;
+  const int64_t img_bytes = (int64_t)b * p.Hs * p.W * (kN * 2);
+  for (int j = wave; j < kCK * 3 / 2; j += NWAVES) {   // (uniform) pairs (2j, 2j+1) of (step, tensor) = (c / 3, c % 3)
+    const int c0 = 2 * j, c1 = 2 * j + 1;
+    const int k = sel ? c1 / 3 : c0 / 3;
+    const char* t0 = static_cast<const char*>(tensors[c0 % 3]);
+    const char* t1 = static_cast<const char*>(tensors[c1 % 3]);
+    const int cell = cell0 + k * cstep + (k >= q.kw ? wrapc : 0);
+    const bool ok = live && ((q.in_grid >> k) & 1u) != 0;
+    const char* src = (sel ? t1 : t0) + img_bytes + ((uint32_t)cell * 32u + (uint32_t)hf * 16u);
+    lds_fill16<false>(ok ? src : reinterpret_cast<const char*>(p.zeros), raw + j * 1024);
+  }
+}
+template <typename T, int CW, int NWAVES>
+__device__ __forceinline__ void bc_widen(const char* raw, char* buf, int wave, int lane) {
+  using SG = Stage<T, 3, CW, false>;
+  const int r = lane & (kHB - 1), qd = lane >> kHBShift;   // row, group of four states
+  for (int c = wave; c < kCK * 3; c += NWAVES) {            // (uniform) (step, tensor) pairs
+    const int k = c / 3, tsr = c - 3 * k;
+    const uint2 v = *reinterpret_cast<const uint2*>(raw + c * 512 + (qd >> 1) * 256 + r * 16 + (qd & 1) * 8);
+    *reinterpret_cast<float4*>(buf + k * SG::kKStr + (tsr * 4 + qd) * SG::kPlane + r * 16) =
+        make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u));
   }
 }
 
@@ -661,6 +724,21 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     ld16f(p.A2L + (e0 + c) * kN, a2l[c]);
     dsk[c] = p.Df[e0 + c];
   }
+  // Records in natural state order (B_T, B_L, C straight from the caller's tensors): position j of a
+  // record holds state j, so the register that meets position j takes A of state j.
+  const bool direct = !CKPT && p.bc_direct != 0;   // (uniform)
+  if (direct) {
+#pragma unroll
+    for (int c = 0; c < EC; ++c) {
+      float t[kN], l[kN];
+#pragma unroll
+      for (int n = 0; n < kN; ++n) { t[n] = a2t[c][n]; l[n] = a2l[c][n]; }
+#pragma unroll
+      for (int j = 0; j < kN; ++j) { a2t[c][sinv<PERM>(j)] = t[j]; a2l[c][sinv<PERM>(j)] = l[j]; }
+    }
+  }
+  constexpr bool WIDEN = sizeof(T) == 2;            // 16-bit records pass through a buffer of their own
+  char* raw = lds + 2 * SG::kBytes;                 // [2][kRawBytes]
 
   settle_loads();
   __syncthreads();
@@ -804,7 +882,26 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   bp = block_pos(p, A, r, rbands);
   int cell0 = cell_of(p, bp.bnd0, r, bp.col0);   // cell index of the lane's position at the first step of the block
   if constexpr (SLICED) link.wait_for(link_need_fwd(0, p.sl_nbb));
-  stage_block<T, 3, CW, false, STAGE_X, NW>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+  BlockPos bpq = bp;     // 16-bit direct records: the block after the next (fetched two blocks ahead)
+  int cellq = cell0;
+  int rp = 0;            // ... and the half of `raw` it goes to
+  if (direct) {
+    if constexpr (WIDEN) {
+      bc_raw_copy<NW>(p, pin.bcd, raw, b, bp, cell0, wave, lane, true);
+      bpq = block_pos(p, pos_after(p, A, kCK), r, rbands);
+      cellq = cell_of(p, bpq.bnd0, r, bpq.col0);
+      bc_raw_copy<NW>(p, pin.bcd, raw + kRawBytes, b, bpq, cellq, wave, lane, m_lo + 1 < m_hi);
+    } else {
+      bc_direct_copy<T, CW, NW>(p, pin.bcd, lds, b, bp, cell0, wave, lane);
+    }
+    stage_block<T, 3, CW, false, STAGE_X, NW, true>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+    if constexpr (WIDEN) {
+      staging_fence();
+      bc_widen<T, CW, NW>(raw, lds, wave, lane);
+    }
+  } else {
+    stage_block<T, 3, CW, false, STAGE_X, NW>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+  }
   staging_fence();
   Ops opsA, opsB;
   if constexpr (AHEAD) fetch(lds, 0, opsA);
@@ -813,12 +910,29 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     const bool last = m + 1 == m_hi;
     // the next block: where the lane's row will be is also what the lane's copies fetch
     const Pos An = pos_after(p, A, kCK);
-    const BlockPos bpn = block_pos(p, An, r, rbands);
-    const int celln = cell_of(p, bpn.bnd0, r, bpn.col0);
+    BlockPos bpn;
+    int celln;
+    if (WIDEN && direct) {   // the next block was worked out a block ago; its records are in `raw` already
+      bpn = bpq;
+      celln = cellq;
+      bpq = block_pos(p, pos_after(p, An, kCK), r, rbands);
+      cellq = cell_of(p, bpq.bnd0, r, bpq.col0);
+      bc_raw_copy<NW>(p, pin.bcd, raw + rp * kRawBytes, b, bpq, cellq, wave, lane, m + 2 < m_hi);
+    } else {
+      bpn = block_pos(p, An, r, rbands);
+      celln = cell_of(p, bpn.bnd0, r, bpn.col0);
+    }
     if (!last) {
       if constexpr (SLICED) link.wait_for(link_need_fwd(m + 1 - m_lo, p.sl_nbb));
-      stage_block<T, 3, CW, false, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, An, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+      if (direct) {
+        if constexpr (!WIDEN) bc_direct_copy<T, CW, NW>(p, pin.bcd, lds + (cur ^ 1) * SG::kBytes, b, bpn, celln, wave, lane);
+        stage_block<T, 3, CW, false, STAGE_X, NW, true>(p, lds + (cur ^ 1) * SG::kBytes, b, An, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+        if constexpr (WIDEN) bc_widen<T, CW, NW>(raw + (rp ^ 1) * kRawBytes, lds + (cur ^ 1) * SG::kBytes, wave, lane);
+      } else {
+        stage_block<T, 3, CW, false, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, An, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+      }
     }
+    rp ^= 1;
     cell_off0 = (uint32_t)(cell0 * p.E + e0) * (uint32_t)sizeof(T);
     // Snapshot of the state before the block (after step t0-1) for the lanes whose previous
     // position was a cell of the grid; the others hold nothing the backward needs.  The stores are
@@ -1466,7 +1580,7 @@ inline size_t align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
 // copy of A and two staging buffers.  A compute unit has 160 KB.
 constexpr size_t kLdsPerWorkgroup = 160 * 1024;
 template <typename T, int EC, int NW = kFwdWaves>
-constexpr size_t fwd_lds_bytes() { return 2 * (size_t)Stage<T, 3, NW * 4 * EC, false>::kBytes; }
+constexpr size_t fwd_lds_bytes() { return 2 * (size_t)Stage<T, 3, NW * 4 * EC, false>::kBytes + (sizeof(T) == 2 ? 2 * kRawBytes : 0); }
 template <typename T, int NW = kBwdWaves>
 constexpr size_t bwd_lds_bytes() {
   return sizeof(float2) * bwd_exchange_sets<T, NW>() * NW * 3 * 64 + sizeof(float) * NW * 4 * 2 * kN + 256 +
@@ -1768,7 +1882,14 @@ int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   sp.top = reinterpret_cast<float*>(keep);
   int rc = launch_prep<T>(sp, d, g, AT, AL, D, prep, link_words, st);
   if (rc) return rc;
-  rc = stage_bc<T>(sp, d, BT, BL, C, reinterpret_cast<float*>(keep + g.top_bytes), false, st);
+  if (!ckpt && !g.packed_bc) {   // nothing will read a packed copy again: the kernel takes the tensors as they are
+    sp.bcd[0] = BT; sp.bcd[1] = BL; sp.bcd[2] = C; sp.bcd[3] = BT;
+    sp.bt = sp.bl = sp.cc = nullptr;
+    sp.bc_stride = 0;
+    sp.bc_direct = 1;
+  } else {
+    rc = stage_bc<T>(sp, d, BT, BL, C, reinterpret_cast<float*>(keep + g.top_bytes), false, st);
+  }
   if (rc) return rc;
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_FWD][0], st);
   rc = launch_fwd<T>(sp, d, g, ckpt != nullptr, true, st);

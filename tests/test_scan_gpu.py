@@ -48,6 +48,13 @@ def run_case(cabi, cscan, B, H, W, E, dtype, seed=0, flip=False, with_ckpt=True,
     a_dev = [dev[k] for k in names]
     if with_ckpt:
         y, ck = cabi.scan_fwd(*a_dev, save_ckpt=True, flip=flip)
+        # the forward that keeps no snapshots takes B_T, B_L, C straight from the tensors: a path of its own
+        y_inf = cabi.scan_fwd(*a_dev, flip=flip)
+        torch.cuda.synchronize()
+        e = so.rel_err(y_inf.float().cpu(), unflip(y_ref).copy())
+        say(f"  y (no snapshots) rel_err {e:.3e}")
+        assert e < TOL[dtype], ("y without snapshots", e)
+        assert so.elem_rel_err(y_inf.float().cpu(), unflip(y_ref).copy()) < TOL_ELEM[dtype]
     else:
         y, ck = cabi.scan_fwd(*a_dev, flip=flip), None
     torch.cuda.synchronize()
