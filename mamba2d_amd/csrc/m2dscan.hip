@@ -595,13 +595,15 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int 
   }
 }
 
-// B_T, B_L, C straight from the caller's tensors (forward without snapshots: no packed fp32 copy is
-// made).  The records keep the natural order of the states.  fp32 tensors are copied into the planes
-// of a staging buffer like every other operand, one block ahead (bc_direct_copy).  16-bit tensors
-// are copied as they are into a small buffer of their own two blocks ahead (bc_raw_copy: one
-// wave-wide copy moves the 16 rows of two (step, tensor) pairs, 32 bytes a row), and are widened from
-// there into the planes of the next block's staging buffer while the current block is worked on
-// (bc_widen): LDS to LDS, so that no wait for a vector load ever stands between a block's stores.
+// B_T, B_L, C straight from the caller's tensors, with no packed fp32 copy made first.
+// 16-bit tensors (both passes): copied as they are into a small buffer of their own two blocks ahead
+// (bc_raw_copy: one wave-wide copy moves the 16 rows of two (step, tensor) pairs, 32 bytes a row),
+// and widened from there into the planes of the next block's staging buffer, in fold order (spos),
+// while the current block is worked on (bc_widen): LDS to LDS, so that no wait for a vector load
+// ever stands between a block's stores.
+// fp32 tensors (forward without snapshots only): copied into the planes like every other operand,
+// one block ahead (bc_direct_copy); the records keep the natural order of the states, which the
+// forward kernel allows for in the order of its copy of A.
 constexpr int kRawBytes = kCK * 3 * kHB * kN * 2;   // 16-bit B_T, B_L, C of one block: 6 KB
 template <typename T, int CW, int NWAVES>
 __device__ __forceinline__ void bc_direct_copy(const ScanParams& p, const void* const* tensors, char* buf, int b, const BlockPos& q,
@@ -642,15 +644,20 @@ __device__ __forceinline__ void bc_raw_copy(const ScanParams& p, const void* con
     lds_fill16<false>(ok ? src : reinterpret_cast<const char*>(p.zeros), raw + j * 1024);
   }
 }
-template <typename T, int CW, int NWAVES>
+template <typename SG, int NWAVES>
 __device__ __forceinline__ void bc_widen(const char* raw, char* buf, int wave, int lane) {
-  using SG = Stage<T, 3, CW, false>;
-  const int r = lane & (kHB - 1), qd = lane >> kHBShift;   // row, group of four states
+  const int r = lane & (kHB - 1), qd = lane >> kHBShift;   // row, four consecutive states 4*qd + m
+  // state 4*qd + m belongs at position 4*m + perm(qd) of its record: word perm(qd) of plane m
+  const int word = qd == 1 ? 2 : (qd == 2 ? 1 : qd);
+  static_assert(spos<true>(4) == 2 && spos<true>(8) == 1 && spos<true>(13) == 7, "fold order");
   for (int c = wave; c < kCK * 3; c += NWAVES) {            // (uniform) (step, tensor) pairs
     const int k = c / 3, tsr = c - 3 * k;
     const uint2 v = *reinterpret_cast<const uint2*>(raw + c * 512 + (qd >> 1) * 256 + r * 16 + (qd & 1) * 8);
-    *reinterpret_cast<float4*>(buf + k * SG::kKStr + (tsr * 4 + qd) * SG::kPlane + r * 16) =
-        make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u));
+    float* dst = reinterpret_cast<float*>(buf + k * SG::kKStr + tsr * 4 * SG::kPlane + r * 16 + word * 4);
+    dst[0 * SG::kPlane / 4] = __uint_as_float(v.x << 16);
+    dst[1 * SG::kPlane / 4] = __uint_as_float(v.x & 0xffff0000u);
+    dst[2 * SG::kPlane / 4] = __uint_as_float(v.y << 16);
+    dst[3 * SG::kPlane / 4] = __uint_as_float(v.y & 0xffff0000u);
   }
 }
 
@@ -724,10 +731,11 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     ld16f(p.A2L + (e0 + c) * kN, a2l[c]);
     dsk[c] = p.Df[e0 + c];
   }
-  // Records in natural state order (B_T, B_L, C straight from the caller's tensors): position j of a
-  // record holds state j, so the register that meets position j takes A of state j.
-  const bool direct = !CKPT && p.bc_direct != 0;   // (uniform)
-  if (direct) {
+  // fp32 records in natural state order (B_T, B_L, C straight from the caller's tensors): position j
+  // of a record holds state j, so the register that meets position j takes A of state j.
+  constexpr bool WIDEN = sizeof(T) == 2;            // 16-bit records pass through a buffer of their own, in every forward
+  const bool direct = (WIDEN || !CKPT) && p.bc_direct != 0;   // (uniform)
+  if (!WIDEN && direct) {   // (never taken by a 16-bit kernel)
 #pragma unroll
     for (int c = 0; c < EC; ++c) {
       float t[kN], l[kN];
@@ -737,7 +745,6 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
       for (int j = 0; j < kN; ++j) { a2t[c][sinv<PERM>(j)] = t[j]; a2l[c][sinv<PERM>(j)] = l[j]; }
     }
   }
-  constexpr bool WIDEN = sizeof(T) == 2;            // 16-bit records pass through a buffer of their own
   char* raw = lds + 2 * SG::kBytes;                 // [2][kRawBytes]
 
   settle_loads();
@@ -897,7 +904,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     stage_block<T, 3, CW, false, STAGE_X, NW, true>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
     if constexpr (WIDEN) {
       staging_fence();
-      bc_widen<T, CW, NW>(raw, lds, wave, lane);
+      bc_widen<SG, NW>(raw, lds, wave, lane);
     }
   } else {
     stage_block<T, 3, CW, false, STAGE_X, NW>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
@@ -927,7 +934,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
       if (direct) {
         if constexpr (!WIDEN) bc_direct_copy<T, CW, NW>(p, pin.bcd, lds + (cur ^ 1) * SG::kBytes, b, bpn, celln, wave, lane);
         stage_block<T, 3, CW, false, STAGE_X, NW, true>(p, lds + (cur ^ 1) * SG::kBytes, b, An, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
-        if constexpr (WIDEN) bc_widen<T, CW, NW>(raw + (rp ^ 1) * kRawBytes, lds + (cur ^ 1) * SG::kBytes, wave, lane);
+        if constexpr (WIDEN) bc_widen<SG, NW>(raw + (rp ^ 1) * kRawBytes, lds + (cur ^ 1) * SG::kBytes, wave, lane);
       } else {
         stage_block<T, 3, CW, false, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, An, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
       }
@@ -1023,7 +1030,7 @@ __device__ __forceinline__ constexpr int fold_state(int m, int qi) {
 template <typename T, int NW>
 constexpr int bwd_exchange_sets() {
   return sizeof(float2) * kCK * NW * 3 * 64 + sizeof(float) * NW * 4 * 2 * kN + 256 +
-         2 * (size_t)Stage<T, 4, NW * 4, true>::kBytes <= 160 * 1024 ? kCK : 2;
+         2 * (size_t)Stage<T, 4, NW * 4, true>::kBytes + (sizeof(T) == 2 ? 2 * kRawBytes : 0) <= 160 * 1024 ? kCK : 2;
 }
 // As in the forward, lanes are never masked: rows outside the grid and cells outside the row work
 // on zero operands.  For the adjoint this means that a row which has not reached its last column
@@ -1055,6 +1062,9 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   float2* slots = reinterpret_cast<float2*>(smem);                       // [XSETS][wave][3][64]
   float* a_lds = reinterpret_cast<float*>(slots + XSETS * NW * SLOT);    // [wave][CS][2][16], fold order
   char* lds = reinterpret_cast<char*>(a_lds + NW * CS * 2 * kN);  // 2 staging buffers
+  constexpr bool WIDEN = sizeof(T) == 2;    // 16-bit B_T, B_L, C can come straight from the caller's tensors (bc_raw_copy, bc_widen)
+  char* raw = lds + 2 * SG::kBytes;         // [2][kRawBytes] for them
+  const bool direct = WIDEN && p.bc_direct != 0;   // (uniform)
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   int lb = SLICED ? (int)blockIdx.x : logical_block(p.nwg);   // (linked bands keep the launch order: a band waits for a lower index)
@@ -1184,7 +1194,21 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   bool ck_take = snapshot_lane(p, Pos{bp.bnd0, bp.col0}, r, ch_ok);   // the lane restores a snapshot for the block to come
   load_ckpt(m_hi - 1, ck_take);
   if constexpr (SLICED) link.wait_for(link_need_bwd(p.sl_nbb - 1, p.sl_nbb));
-  stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+  // the lane's row in the block two before (A2 = position of that block): what its raw copies fetch
+  auto raw_copy_for = [&](Pos A2, char* dst, bool live) {
+    const BlockPos q2 = block_pos(p, A2, r, rbands);
+    bc_raw_copy<NW>(p, pin.bcd, dst, b, q2, cell_of(p, q2.bnd0, r, q2.col0), wave, lane, live);
+  };
+  int rp = 0;   // half of `raw` that the next raw copy goes to
+  if (direct) {
+    bc_raw_copy<NW>(p, pin.bcd, raw, b, bp, cell0, wave, lane, true);
+    raw_copy_for(pos_before(A), raw + kRawBytes, m_hi - 2 >= m_lo);
+    stage_block<T, 4, CW, true, STAGE_X, NW, true>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+    staging_fence();
+    bc_widen<SG, NW>(raw, lds, wave, lane);
+  } else {
+    stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+  }
   staging_fence();
   int cur = 0;
   int xpar = 0;   // exchange buffer in use
@@ -1200,10 +1224,17 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
     const BlockPos bpn = block_pos(p, Aprev, r, rbands);
     const int celln = cell_of(p, bpn.bnd0, r, bpn.col0);
     ck_take = snapshot_lane(p, Pos{bpn.bnd0, bpn.col0}, r, ch_ok);
+    if (direct) raw_copy_for(pos_before(Aprev), raw + rp * kRawBytes, m - 2 >= m_lo);
     if (m > m_lo) {
       if constexpr (SLICED) link.wait_for(link_need_bwd(m - 1 - m_lo, p.sl_nbb));
-      stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+      if (direct) {
+        stage_block<T, 4, CW, true, STAGE_X, NW, true>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+        bc_widen<SG, NW>(raw + (rp ^ 1) * kRawBytes, lds + (cur ^ 1) * SG::kBytes, wave, lane);
+      } else {
+        stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+      }
     }
+    rp ^= 1;
     cell_off0 = (uint32_t)(cell0 * p.E + e) * (uint32_t)sizeof(T);
     f_off0 = (uint32_t)cell0 * (uint32_t)(3 * kN * sizeof(float)) + (BATCH ? (uint32_t)(slot * 4 * sizeof(float)) : f_sub);
 
@@ -1584,7 +1615,7 @@ constexpr size_t fwd_lds_bytes() { return 2 * (size_t)Stage<T, 3, NW * 4 * EC, f
 template <typename T, int NW = kBwdWaves>
 constexpr size_t bwd_lds_bytes() {
   return sizeof(float2) * bwd_exchange_sets<T, NW>() * NW * 3 * 64 + sizeof(float) * NW * 4 * 2 * kN + 256 +
-         2 * (size_t)Stage<T, 4, NW * 4, true>::kBytes;
+         2 * (size_t)Stage<T, 4, NW * 4, true>::kBytes + (sizeof(T) == 2 ? 2 * kRawBytes : 0);
 }
 static_assert(fwd_lds_bytes<float, 1>() <= kLdsPerWorkgroup && fwd_lds_bytes<bf16_t, 1>() <= kLdsPerWorkgroup, "forward staging must fit the LDS");
 static_assert(bwd_lds_bytes<float>() <= kLdsPerWorkgroup && bwd_lds_bytes<bf16_t>() <= kLdsPerWorkgroup, "backward staging must fit the LDS");
@@ -1730,7 +1761,8 @@ Geometry make_geometry(const m2d_desc* d) {
   const size_t P = (size_t)d->B * d->H * d->W;
   g.prep_bytes = align_up(sizeof(float) * (kZeroFloats + (size_t)2 * d->E * kN + d->E));
   g.packed_bc = (d->flags & M2D_FLAG_PACKED_BC) != 0;   // the caller brings the records: nothing to reserve
-  g.bc_bytes = g.packed_bc ? 0 : align_up(sizeof(float) * P * 48);
+  // (16-bit tensors are widened inside the scan kernels, nothing to reserve either)
+  g.bc_bytes = (g.packed_bc || d->dtype == M2D_BF16) ? 0 : align_up(sizeof(float) * P * 48);
   g.ckpt_diag_bytes = align_up(sizeof(float) * (size_t)B * g.nblk * d->E * kN * g.HB);
   const bool rows = g.nbands > 1 && !g.stacked;   // boundary rows travel between bands
   g.top_bytes = rows ? align_up(sizeof(float) * (size_t)(g.nbands - 1) * B * d->W * d->E * kN) : 0;
@@ -1882,7 +1914,7 @@ int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   sp.top = reinterpret_cast<float*>(keep);
   int rc = launch_prep<T>(sp, d, g, AT, AL, D, prep, link_words, st);
   if (rc) return rc;
-  if (!ckpt && !g.packed_bc) {   // nothing will read a packed copy again: the kernel takes the tensors as they are
+  if ((!ckpt || sizeof(T) == 2) && !g.packed_bc) {   // the kernel takes the tensors as they are (fp32: only where no backward will want the packed copy)
     sp.bcd[0] = BT; sp.bcd[1] = BL; sp.bcd[2] = C; sp.bcd[3] = BT;
     sp.bt = sp.bl = sp.cc = nullptr;
     sp.bc_stride = 0;
@@ -1930,7 +1962,14 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   char* ck = ckpt ? const_cast<char*>(static_cast<const char*>(ckpt)) : w;
   sp.ckpt = reinterpret_cast<float*>(ck);
   sp.top = reinterpret_cast<float*>(ck + g.ckpt_diag_bytes);
-  rc = stage_bc<T>(sp, d, BT, BL, C, reinterpret_cast<float*>(ck + g.ckpt_diag_bytes + g.top_bytes), ckpt != nullptr, st);
+  if (sizeof(T) == 2 && !g.packed_bc) {   // widened inside the kernels (also by the forward sweep below)
+    sp.bcd[0] = BT; sp.bcd[1] = BL; sp.bcd[2] = C; sp.bcd[3] = BT;
+    sp.bt = sp.bl = sp.cc = nullptr;
+    sp.bc_stride = 0;
+    sp.bc_direct = 1;
+  } else {
+    rc = stage_bc<T>(sp, d, BT, BL, C, reinterpret_cast<float*>(ck + g.ckpt_diag_bytes + g.top_bytes), ckpt != nullptr, st);
+  }
   if (rc) return rc;
   if (!ckpt) {   // rebuild the checkpoints with one forward sweep that writes no y
     rc = launch_fwd<T>(sp, d, g, true, false, st);
