@@ -87,6 +87,13 @@ typedef struct m2d_desc {
  * d_deltaL arguments as such and does not read deltaT and deltaL (they may be NULL).  This saves
  * m2d_proj_bwd reading the two step-size tensors and a pass of its own intermediate through memory. */
 #define M2D_FLAG_DPRE 16
+/* Scheduling hints for m2d_scan_fwd / m2d_scan_bwd (results agree to rounding either way; sizes
+ * queried and calls made for one problem must carry the same hints).  The library normally decides by
+ * itself: with few images it spreads the 16 states of a channel over the lanes of a wave (a wave per
+ * channel instead of per 4 channels), which shortens a sweep when the device is far from full.
+ * M2D_FLAG_SPLIT_STATES asks for that layout wherever it exists, M2D_FLAG_WHOLE_STATES forbids it. */
+#define M2D_FLAG_SPLIT_STATES 32
+#define M2D_FLAG_WHOLE_STATES 64
 
 #define M2D_PASS_FWD 0
 #define M2D_PASS_BWD 1

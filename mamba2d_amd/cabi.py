@@ -19,6 +19,8 @@ M2D_FLAG_ROUND_WEIGHTS = 2
 M2D_FLAG_RAW_PARAMS = 4
 M2D_FLAG_PACKED_BC = 8
 M2D_FLAG_DPRE = 16
+M2D_FLAG_SPLIT_STATES = 32
+M2D_FLAG_WHOLE_STATES = 64
 M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
@@ -117,6 +119,11 @@ def check(code: int) -> None:
         raise M2DError(code, status_str(code))
 
 
+# M2D_FLAG_SPLIT_STATES or M2D_FLAG_WHOLE_STATES to override the library's choice of lane layout in
+# scan_fwd / scan_bwd (0: the library decides); the tests run every case all three ways.
+SCHEDULE_HINT = 0
+
+
 def make_desc(x: torch.Tensor, N: int, flip: bool = False) -> Desc:
     B, H, W, E = x.shape
     if x.dtype == torch.float32:
@@ -125,7 +132,7 @@ def make_desc(x: torch.Tensor, N: int, flip: bool = False) -> Desc:
         dt = M2D_BF16
     else:
         raise TypeError(f"m2dscan supports float32 and bfloat16, got {x.dtype}")
-    return Desc(B, H, W, E, N, dt, M2D_FLAG_FLIP if flip else 0, 0)
+    return Desc(B, H, W, E, N, dt, (M2D_FLAG_FLIP if flip else 0) | SCHEDULE_HINT, 0)
 
 
 def _ptr(t):

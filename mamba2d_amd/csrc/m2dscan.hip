@@ -286,7 +286,7 @@ struct Stage {
   static constexpr int kXTauBytes = kCK * kXStepBytes;   // XD bytes per tensor
   static constexpr int kXTauInstr = kXTauBytes / 1024;   // wave-wide copies per tensor
   static constexpr int kPlane = kHB * 16;                // bytes per plane
-  static constexpr int kG16 = CW / 16;                   // groups of 16 channels
+  static constexpr int kG16 = (CW + 15) / 16;            // groups of 16 channels (a workgroup of fewer copies the rows of 16 all the same)
   static constexpr int kTopPlane = 12;
   static constexpr int kBotPlane = kTopPlane + 4 * kG16;
   // (adjoint: at least 24 planes, so that what a ghost reads 4 and 8 planes behind its boundary row is inside the step)
@@ -297,9 +297,9 @@ struct Stage {
   static constexpr int kXOff = kCK * kKStr;
   static constexpr int kBytes = kXOff + NT * kXTauBytes; // one buffer
   static_assert(kXTauBytes % 1024 == 0, "a wave-wide copy must not straddle two tensors of XD");
-  static_assert(kCpt == 2 || kCpt % 4 == 0, "a wave-wide copy of XD covers one step, or two halves of 32 lanes");
+  static_assert(kCpt <= 2 || kCpt % 4 == 0, "a wave-wide copy of XD covers one step, or two halves of 32 lanes (one chunk per cell: XD is not staged)");
   static_assert(CW % kElem == 0, "workgroup channel count must fill whole chunks");
-  static_assert(CW % 16 == 0, "boundary rows are copied 16 channels at a time");
+  static_assert(CW % 16 == 0 || CW < 16, "boundary rows are copied 16 channels at a time");
   // byte offset inside a tensor's part of XD of channel `ch` (of the workgroup) for lane row r at step 0
   static __host__ __device__ constexpr uint32_t x_off(int r, int ch) {
     return (uint32_t)(((ch / kElem) * kHB + r) * 16 + (ch % kElem) * (int)sizeof(T));
@@ -410,6 +410,19 @@ __device__ __forceinline__ void staging_landed_behind() {
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_waitcnt(0x0F70 | N);
   asm volatile("" ::: "memory");
+}
+// The same with a count that is only known at run time (uniform; counts above 7 wait as for 7).
+__device__ __forceinline__ void staging_landed_behind_n(int n) {
+  switch (n < 0 ? 0 : (n > 7 ? 7 : n)) {
+    case 0: staging_landed(); break;
+    case 1: staging_landed_behind<1>(); break;
+    case 2: staging_landed_behind<2>(); break;
+    case 3: staging_landed_behind<3>(); break;
+    case 4: staging_landed_behind<4>(); break;
+    case 5: staging_landed_behind<5>(); break;
+    case 6: staging_landed_behind<6>(); break;
+    default: staging_landed_behind<7>(); break;
+  }
 }
 // ... and those of the other waves too
 __device__ __forceinline__ void staging_fence() {
@@ -1011,6 +1024,244 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   }
 }
 
+// ------------------------------------------------------- forward, the states of a channel split over lanes
+// Few images leave most of the device idle with the kernel above (a wave per 4 channels of an
+// image), and a sweep then takes as long as one wave needs for its chain of instructions.  Here the
+// 16 states of ONE channel are split over the 4 lane groups of a wave (lane = (state group g, row r),
+// 4 states per lane): four times as many waves, each with about a third of the instructions per
+// step.  A workgroup has 8 waves = 8 channels.  Staging, schedules and memory formats are those of
+// m2d_fwd_kernel; y of a cell is the sum over the 4 lane groups (two lane-swap steps), stored by group 0.
+constexpr int kSplitWaves = 8;
+__device__ __forceinline__ float sum_over_groups(float v) {
+  v = fold16(v, v);
+  return fold32(v, v);
+}
+template <typename T, bool CKPT, bool WRITE_Y, bool STAGE_X, int MODE>
+__global__ __launch_bounds__(kSplitWaves * 64) void m2d_fwd_split_kernel(const ScanParams pin) {
+  static_assert(MODE != kModeStacked, "stacked images are many: they never need the split");
+  constexpr bool SLICED = MODE == kModeSliced;
+  const ScanParams& p = pin;
+  __builtin_assume(p.stacked == 0);
+  __builtin_assume(p.S >= kHB + kCK - 1);
+  constexpr int NW = kSplitWaves, CW = NW;
+  using SG = Stage<T, 3, CW, false>;
+  constexpr bool WIDEN = sizeof(T) == 2;
+  extern __shared__ float4 smem[];
+  char* lds = reinterpret_cast<char*>(smem);       // two staging buffers
+  char* raw = lds + 2 * SG::kBytes;                // [2][kRawBytes] (16-bit B_T, B_L, C on their way)
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  int lb = SLICED ? (int)blockIdx.x : logical_block(p.nwg);
+  int m_lo = 0, m_hi = p.nblk;
+  int my_band = 0;
+  Link link;
+  if constexpr (SLICED) {
+    const int per = p.B * p.bpb;
+    my_band = lb / per;
+    lb -= my_band * per;
+    m_lo = my_band * p.sl_nbb;
+    m_hi = m_lo + p.sl_nbb;
+    link.mine = p.prog + (int64_t)my_band * per + lb;
+    link.dep = my_band > 0 ? link.mine - per : nullptr;
+    link.err = p.link_err;
+  }
+  const int b = lb / p.bpb;
+  const int e_wg0 = (lb % p.bpb) * CW;
+  const int g = lane >> kHBShift, r = lane & (kHB - 1);   // state group, lane row
+  const int rbands = row_bands(p, r);
+  const int ch_loc = wave;                          // the wave's channel inside the workgroup
+  const bool ch_ok = e_wg0 + ch_loc < p.E;          // (uniform) idle waves still take part in staging and barriers
+  const int e0 = ch_ok ? e_wg0 + ch_loc : p.E - 1;
+  for (int i = threadIdx.x; i < 2 * SG::kBytes / 16; i += NW * 64) smem[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+
+  // Position 4g + w of a record is met by register w: state sinv(4g + w) in fold order, state 4g + w
+  // where the records come straight from fp32 tensors (natural order).
+  const bool direct = (WIDEN || !CKPT) && p.bc_direct != 0;   // (uniform)
+  float a2t[4], a2l[4];
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    const int q = w == 1 ? 2 : (w == 2 ? 1 : w);   // sinv<true>(4g + w) = q * 4 + g
+    const int n = (!WIDEN && direct) ? 4 * g + w : q * 4 + g;
+    a2t[w] = p.A2T[e0 * kN + n];
+    a2l[w] = p.A2L[e0 * kN + n];
+  }
+  static_assert(sinv<true>(1) == 8 && sinv<true>(6) == 5 && sinv<true>(15) == 15, "fold order");
+  const float dsk = p.Df[e0];
+  settle_loads();
+  __syncthreads();
+
+  const T* X = static_cast<const T*>(p.x);
+  const T* DT = static_cast<const T*>(p.dT);
+  const T* DL = static_cast<const T*>(p.dL);
+  const T* DY = DL;
+  const int64_t img_cell0 = (int64_t)b * p.Hs * p.W;
+  const int64_t img_bytes = img_cell0 * p.E * (int64_t)sizeof(T);
+  char* Yimg = static_cast<char*>(p.y) + img_bytes;
+  const char* Ximg = reinterpret_cast<const char*>(X) + img_bytes;
+  const char* DTimg = reinterpret_cast<const char*>(DT) + img_bytes;
+  const char* DLimg = reinterpret_cast<const char*>(DL) + img_bytes;
+  const uint32_t estep = (uint32_t)(p.flip ? -p.E : p.E) * (uint32_t)sizeof(T);
+  const uint32_t wrap_adj = (uint32_t)(kRB * p.W - p.S) * estep;
+  const float g1 = r == 0 ? 1.f : 0.f;             // the ghost's T input coefficient
+
+  // the lane's group of B_T (the ghost: of the row above), of B_L and C (the ghost: zeros of its own row)
+  const uint32_t row_off = r * 16 + g * SG::kPlane;
+  const uint32_t rec_off = r == 0 ? SG::top_off(ch_loc) + g * SG::kPlane : row_off;
+  const uint32_t const_off = SG::kConstPlane * SG::kPlane + r * 16;
+  const uint32_t xd_off = SG::kXOff + SG::x_off(r, ch_loc);
+  constexpr uint32_t kXK = SG::kXStepBytes;
+
+  BlockPos bp;
+  uint32_t cell_off0 = 0;
+  float h[4] = {0.f, 0.f, 0.f, 0.f};
+  bool ck_mine = false;
+  float4* ckp = nullptr;
+
+  auto step = [&](const char* bufc, int k) {
+    float xv = 0.f, dtv = 0.f, dlv = 0.f;
+    const bool inr = ch_ok && ((bp.in_grid >> k) & 1u);
+    const uint32_t goff = cell_off0 + (uint32_t)k * estep + (k >= bp.kw ? wrap_adj : 0u);
+    if constexpr (STAGE_X) {
+      const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
+      xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + SG::kXTauBytes / sizeof(T)); dlv = IO<T>::ld(xr + 2 * SG::kXTauBytes / sizeof(T));
+    } else if (inr) {
+      xv = IO<T>::ld(reinterpret_cast<const T*>(Ximg + goff));
+      dtv = IO<T>::ld(reinterpret_cast<const T*>(DTimg + goff));
+      dlv = IO<T>::ld(reinterpret_cast<const T*>(DLimg + goff));
+    }
+    const float4 kk = *reinterpret_cast<const float4*>(bufc + const_off + k * SG::kKStr);
+    const float4 b4 = *reinterpret_cast<const float4*>(bufc + rec_off + k * SG::kKStr);
+    const float4 l4 = *reinterpret_cast<const float4*>(bufc + row_off + SG::kBLOff + k * SG::kKStr);
+    const float4 c4 = WRITE_Y ? *reinterpret_cast<const float4*>(bufc + row_off + SG::kCOff + k * SG::kKStr) : make_float4(0, 0, 0, 0);
+    const float offT = kk.x, offL = kk.y, cT = kk.z, cL = kk.w;
+    const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w}, cq[4] = {c4.x, c4.y, c4.z, c4.w};
+    const float sT = __builtin_fmaf(cT * dtv, xv, g1);
+    const float sL = cL * dlv * xv;
+    // gates before chains (see m2d_fwd_kernel: no DPP multiply-add right behind the v_exp that makes its gate)
+    float aT[4], aL[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) aT[w] = fexp2(__builtin_fmaf(dtv, a2t[w], offT));
+    pin4(aT);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int w = 0; w < 4; ++w) aL[w] = fexp2(__builtin_fmaf(dlv, a2l[w], offL));
+    pin4(aL);
+    __builtin_amdgcn_sched_barrier(0);
+    if (CKPT && k == 0 && ck_mine) store_snapshot(ckp, h[0], h[1], h[2], h[3]);   // the lane's states as they are before this step
+    float acc = 0.f;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      float u = sL * lq[w];
+      u = __builtin_fmaf(sT, bq[w], u);
+      u = fma_row_below(aT[w], h[w], u);
+      const float hn = __builtin_fmaf(aL[w], h[w], u);
+      h[w] = hn;
+      if (WRITE_Y) acc = __builtin_fmaf(hn, cq[w], acc);
+    }
+    if (p.nbands > 1) {   // last row of a band: the next band's ghost will replay it
+      const bool wk = k >= bp.kw;
+      const int bk = wk ? bp.bnd0 + 1 : bp.bnd0;
+      if (inr && r == kRB && bk + 1 < p.nbands) {
+        const int ck = wk ? bp.col0 + k - p.S : bp.col0 + k;
+        float4* tw = reinterpret_cast<float4*>(p.top + ((((int64_t)bk * p.B + b) * p.W + ck) * p.E + e0) * kN) + g;
+        const float4 row = make_float4(h[0], h[1], h[2], h[3]);
+        if constexpr (SLICED) store_row_device_scope(tw, row); else *tw = row;
+      }
+    }
+    if constexpr (WRITE_Y) {
+      const float yv = __builtin_fmaf(xv, dsk, sum_over_groups(acc));
+      if (inr && g == 0) IO<T>::st(reinterpret_cast<T*>(Yimg + goff), yv);
+    }
+  };
+
+  Pos A = pos_of(p, m_lo * kCK - (kHB - 1));     // position of the stream index t0 - 15 (wave-uniform)
+  bp = block_pos(p, A, r, rbands);
+  int cell0 = cell_of(p, bp.bnd0, r, bp.col0);
+  if constexpr (SLICED) link.wait_for(link_need_fwd(0, p.sl_nbb));
+  BlockPos bpq = bp;     // 16-bit direct records: the block after the next (fetched two blocks ahead)
+  int cellq = cell0;
+  int rp = 0;
+  if (direct) {
+    if constexpr (WIDEN) {
+      bc_raw_copy<NW>(p, pin.bcd, raw, b, bp, cell0, wave, lane, true);
+      bpq = block_pos(p, pos_after(p, A, kCK), r, rbands);
+      cellq = cell_of(p, bpq.bnd0, r, bpq.col0);
+      bc_raw_copy<NW>(p, pin.bcd, raw + kRawBytes, b, bpq, cellq, wave, lane, m_lo + 1 < m_hi);
+    } else {
+      bc_direct_copy<T, CW, NW>(p, pin.bcd, lds, b, bp, cell0, wave, lane);
+    }
+    stage_block<T, 3, CW, false, STAGE_X, NW, true>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+    if constexpr (WIDEN) {
+      staging_fence();
+      bc_widen<SG, NW>(raw, lds, wave, lane);
+    }
+  } else {
+    stage_block<T, 3, CW, false, STAGE_X, NW>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+  }
+  staging_fence();
+  int cur = 0;
+  for (int m = m_lo; m < m_hi; ++m) {
+    const bool last = m + 1 == m_hi;
+    const Pos An = pos_after(p, A, kCK);
+    BlockPos bpn;
+    int celln;
+    if (WIDEN && direct) {
+      bpn = bpq;
+      celln = cellq;
+      bpq = block_pos(p, pos_after(p, An, kCK), r, rbands);
+      cellq = cell_of(p, bpq.bnd0, r, bpq.col0);
+      bc_raw_copy<NW>(p, pin.bcd, raw + rp * kRawBytes, b, bpq, cellq, wave, lane, m + 2 < m_hi);
+    } else {
+      bpn = block_pos(p, An, r, rbands);
+      celln = cell_of(p, bpn.bnd0, r, bpn.col0);
+    }
+    if (!last) {
+      if constexpr (SLICED) link.wait_for(link_need_fwd(m + 1 - m_lo, p.sl_nbb));
+      if (direct) {
+        if constexpr (!WIDEN) bc_direct_copy<T, CW, NW>(p, pin.bcd, lds + (cur ^ 1) * SG::kBytes, b, bpn, celln, wave, lane);
+        stage_block<T, 3, CW, false, STAGE_X, NW, true>(p, lds + (cur ^ 1) * SG::kBytes, b, An, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+        if constexpr (WIDEN) bc_widen<SG, NW>(raw + (rp ^ 1) * kRawBytes, lds + (cur ^ 1) * SG::kBytes, wave, lane);
+      } else {
+        stage_block<T, 3, CW, false, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, An, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+      }
+    }
+    rp ^= 1;
+    cell_off0 = (uint32_t)(cell0 * p.E + e0) * (uint32_t)sizeof(T);
+    ck_mine = false;
+    bool snapped = false;   // (uniform) the wave issues the store of a snapshot
+    if (CKPT && m > 0) {
+      Pos at; at.bnd = bp.bnd0; at.col = bp.col0;
+      ck_mine = snapshot_lane(p, at, r, ch_ok);
+      snapped = __any(ck_mine);
+      ckp = reinterpret_cast<float4*>(p.ckpt + ((((int64_t)b * p.nblk + m) * p.E + e0) * kN) * kHB) + g * kHB + r;
+    }
+    const char* bufc = lds + cur * SG::kBytes;
+    // (uniform) stores that the wave is sure to issue in the first three steps, after the copies for the
+    // next block: y where some lane is on the grid at all three, the boundary row where the band's last row
+    // is and another band follows.  They need not have completed when the block ends, only the copies.
+    const bool on3 = ch_ok && (bp.in_grid & 7u) == 7u;
+    const bool y_thrice = WRITE_Y && __any(on3);
+    const bool top_thrice = p.nbands > 1 && __any(on3 && r == kRB && bp.kw >= kCK && bp.bnd0 + 1 < p.nbands);
+    const int younger = (snapped ? 1 : 0) + (y_thrice ? 3 : 0) + (top_thrice ? 3 : 0);
+#pragma unroll
+    for (int k = 0; k < kCK; ++k) {
+      if (k == kCK - 1) staging_landed_behind_n(younger);
+      step(bufc, k);
+    }
+    __syncthreads();
+    if constexpr (SLICED) link.publish((uint32_t)(m - m_lo));
+    cur ^= 1;
+    A = An;
+    bp = bpn;
+    cell0 = celln;
+  }
+  if constexpr (SLICED) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    link.publish((uint32_t)p.sl_nbb);
+  }
+}
+
 // ----------------------------------------------------------------------------------- backward
 // Channel sums by lane-swap butterflies.  The wave holds 4 channel slots; for a group of 4 states
 // every lane lists its values v[0..3] and fold16(fold32(v0,v1), fold32(v2,v3)) leaves, in the
@@ -1486,6 +1737,328 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   }
 }
 
+// ------------------------------------------------------ backward, the states of a channel split over lanes
+// The counterpart of m2d_fwd_split_kernel: lane = (state group g, row r), 4 states per lane, a wave
+// per channel, 8 channels per workgroup.  With only 4 states a lane keeps the gates of all four
+// steps of a block from the recomputation to the adjoint, and sweeps a block in one pass.  Sums over
+// the states of a cell (for d_delta and d_x) are taken across the 4 lane groups by lane swaps; sums
+// over channels (d_C, d_BT, d_BL) across the 8 waves through LDS, as in m2d_bwd_kernel, a float4 of
+// four states per lane.  Memory formats are those of m2d_bwd_kernel.
+template <typename T, bool STAGE_X, int MODE>
+__global__ __launch_bounds__(kSplitWaves * 64) void m2d_bwd_split_kernel(const ScanParams pin) {
+  static_assert(MODE != kModeStacked, "stacked images are many: they never need the split");
+  constexpr bool SLICED = MODE == kModeSliced;
+  const ScanParams& p = pin;
+  __builtin_assume(p.stacked == 0);
+  __builtin_assume(p.S >= kHB + kCK - 1);
+  constexpr int NW = kSplitWaves, CW = NW;
+  constexpr int SLOT = 3 * 64;           // float4s per wave in one exchange buffer
+  using SG = Stage<T, 4, CW, true>;
+  constexpr bool WIDEN = sizeof(T) == 2;
+  extern __shared__ float4 smem[];
+  float4* slots = smem;                                            // [2][wave][3][64], used alternately: one barrier per step
+  char* lds = reinterpret_cast<char*>(slots + 2 * NW * SLOT);      // two staging buffers
+  char* raw = lds + 2 * SG::kBytes;                                // [2][kRawBytes]
+  const bool direct = WIDEN && p.bc_direct != 0;   // (uniform)
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  int lb = SLICED ? (int)blockIdx.x : logical_block(p.nwg);
+  int m_lo = 0, m_hi = p.nblk;
+  int my_band = 0;
+  Link link;
+  if constexpr (SLICED) {   // the window of one band; the bands are launched from the last to the first
+    const int per = p.B * p.bpb;
+    const int kk = lb / per;
+    lb -= kk * per;
+    my_band = p.nbands - 1 - kk;
+    m_lo = my_band * p.sl_nbb;
+    m_hi = m_lo + p.sl_nbb;
+    link.mine = p.prog + (int64_t)my_band * per + lb;
+    link.dep = my_band + 1 < p.nbands ? link.mine + per : nullptr;
+    link.err = p.link_err;
+  }
+  const int b = lb / p.bpb;
+  const int eg = lb % p.bpb;
+  const int e_wg0 = eg * CW;
+  const int g = lane >> kHBShift, r = lane & (kHB - 1);
+  const int rbands = row_bands(p, r);
+  const int ch_loc = wave;
+  const bool ch_ok = e_wg0 + ch_loc < p.E;   // (uniform)
+  const int e = ch_ok ? e_wg0 + ch_loc : p.E - 1;
+  for (int i = threadIdx.x; i < 2 * SG::kBytes / 16; i += NW * 64) reinterpret_cast<float4*>(lds)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+  // register w of the lane meets position 4g + w of a record: state perm(w) * 4 + g (fold order)
+  int state_of[4];
+  float a2t[4], a2l[4];
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    state_of[w] = (w == 1 ? 2 : (w == 2 ? 1 : w)) * 4 + g;
+    a2t[w] = p.A2T[e * kN + state_of[w]];
+    a2l[w] = p.A2L[e * kN + state_of[w]];
+  }
+  const float dsk = p.Df[e];
+  settle_loads();
+
+  const T* X = static_cast<const T*>(p.x);
+  const T* DT = static_cast<const T*>(p.dT);
+  const T* DL = static_cast<const T*>(p.dL);
+  const T* DY = static_cast<const T*>(p.dy);
+  const int64_t img_cell0 = (int64_t)b * p.Hs * p.W;
+  const int64_t img_bytes = img_cell0 * p.E * (int64_t)sizeof(T);
+  const char* Ximg = reinterpret_cast<const char*>(X) + img_bytes;
+  const char* DTimg = reinterpret_cast<const char*>(DT) + img_bytes;
+  const char* DLimg = reinterpret_cast<const char*>(DL) + img_bytes;
+  const char* DYimg = reinterpret_cast<const char*>(DY) + img_bytes;
+  // the three per-cell results are stored by three of the four lane groups: group 0 d_deltaT, 2 d_deltaL, 1 d_x
+  char* OUTimg = (g == 0 ? static_cast<char*>(p.ddT) : (g == 2 ? static_cast<char*>(p.ddL) : static_cast<char*>(p.dx))) + img_bytes;
+  char* BOTimg = reinterpret_cast<char*>(p.bot + (int64_t)b * p.W * p.E * kN);   // + band * bot_stride
+  char* PARTimg = reinterpret_cast<char*>(p.part + ((int64_t)eg * p.Ptot + img_cell0) * (3 * kN));
+
+  float accAT[4], accAL[4], accD = 0.f, muT[4], muL[4];
+#pragma unroll
+  for (int w = 0; w < 4; ++w) { accAT[w] = 0.f; accAL[w] = 0.f; muT[w] = 0.f; muL[w] = 0.f; }
+  // the lane's group of (B_T, B_L, C): a grid row reads those of its cell; the upper ghost (lane 0) the row
+  // above as its B_T; the lower ghost (lane 15) the row of mu_T below as its C (see m2d_bwd_kernel)
+  const uint32_t rec_off = (r == 0 ? SG::top_off(ch_loc) : (r == kHB - 1 ? SG::bot_off(ch_loc) - SG::kCOff : r * 16)) + g * SG::kPlane;
+  const uint32_t const_off = SG::kConstPlane * SG::kPlane + r * 16;
+  const uint32_t xd_off = SG::kXOff + SG::x_off(r, ch_loc);
+  constexpr uint32_t kXK = SG::kXStepBytes;
+  // channel sums: the first 6 waves add up; wave 2v + c takes components 2c, 2c+1 of every lane's float4 of
+  // tensor v.  They are kept per cell as [C, B_T, B_L][16] in the natural order of the states.
+  const bool f_on = wave < 6;
+  const int f_v = wave >> 1, f_c = wave & 1;
+  const uint32_t f_sub0 = (uint32_t)(f_v * kN + (f_c ? 1 : 0) * 4 + g) * (uint32_t)sizeof(float);   // component 2c: state perm(2c) * 4 + g, perm = (0, 2, 1, 3)
+  const uint32_t f_sub1 = (uint32_t)(f_v * kN + (f_c ? 3 : 2) * 4 + g) * (uint32_t)sizeof(float);   // component 2c + 1
+  const float g1 = r == 0 ? 1.f : 0.f;
+  const float gb1 = r == kHB - 1 ? 1.f : 0.f;
+  const uint32_t estep = (uint32_t)(p.flip ? -p.E : p.E) * (uint32_t)sizeof(T);
+  const uint32_t wrap_adj = (uint32_t)(kRB * p.W - p.S) * estep;
+  const uint32_t pstep = (uint32_t)(p.flip ? -1 : 1) * (uint32_t)(3 * kN * sizeof(float));
+  const uint32_t pwrap_adj = (uint32_t)(kRB * p.W - p.S) * pstep;
+
+  BlockPos bp;
+  uint32_t cell_off0 = 0, f_off0 = 0;
+  float cknext[4];
+  auto load_ckpt = [&](int mm, bool take) {   // take: the forward kept the lane's state before block mm
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (mm != 0 && take) v = (reinterpret_cast<const float4*>(p.ckpt + ((((int64_t)b * p.nblk + mm) * p.E + e) * kN) * kHB) + g * kHB)[r];
+    cknext[0] = v.x; cknext[1] = v.y; cknext[2] = v.z; cknext[3] = v.w;
+  };
+  auto pos_before = [&](Pos Q) {
+    Q.col -= kCK;
+    if (Q.col < 0) { Q.col += p.S; Q.bnd -= 1; }
+    return Q;
+  };
+
+  Pos A = pos_of(p, (m_hi - 1) * kCK - (kHB - 1));
+  __syncthreads();   // the zeros are in place before the first copies land on them
+  bp = block_pos(p, A, r, rbands);
+  int cell0 = cell_of(p, bp.bnd0, r, bp.col0);
+  bool ck_take = snapshot_lane(p, Pos{bp.bnd0, bp.col0}, r, ch_ok);
+  load_ckpt(m_hi - 1, ck_take);
+  if constexpr (SLICED) link.wait_for(link_need_bwd(p.sl_nbb - 1, p.sl_nbb));
+  auto raw_copy_for = [&](Pos A2, char* dst, bool live) {
+    const BlockPos q2 = block_pos(p, A2, r, rbands);
+    bc_raw_copy<NW>(p, pin.bcd, dst, b, q2, cell_of(p, q2.bnd0, r, q2.col0), wave, lane, live);
+  };
+  int rp = 0;
+  if (direct) {
+    bc_raw_copy<NW>(p, pin.bcd, raw, b, bp, cell0, wave, lane, true);
+    raw_copy_for(pos_before(A), raw + kRawBytes, m_hi - 2 >= m_lo);
+    stage_block<T, 4, CW, true, STAGE_X, NW, true>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+    staging_fence();
+    bc_widen<SG, NW>(raw, lds, wave, lane);
+  } else {
+    stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+  }
+  staging_fence();
+  int cur = 0;
+  int xpar = 0;
+
+  for (int m = m_hi - 1; m >= m_lo; --m) {
+    const int t0 = m * kCK;
+    const char* bufc = lds + cur * SG::kBytes;
+    float hb[kCK + 1][4], gT[kCK][4], gL[kCK][4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) hb[0][w] = cknext[w];
+    const Pos Aprev = pos_before(A);
+    const BlockPos bpn = block_pos(p, Aprev, r, rbands);
+    const int celln = cell_of(p, bpn.bnd0, r, bpn.col0);
+    ck_take = snapshot_lane(p, Pos{bpn.bnd0, bpn.col0}, r, ch_ok);
+    if (direct) raw_copy_for(pos_before(Aprev), raw + rp * kRawBytes, m - 2 >= m_lo);
+    if (m > m_lo) {
+      if constexpr (SLICED) link.wait_for(link_need_bwd(m - 1 - m_lo, p.sl_nbb));
+      if (direct) {
+        stage_block<T, 4, CW, true, STAGE_X, NW, true>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+        bc_widen<SG, NW>(raw + (rp ^ 1) * kRawBytes, lds + (cur ^ 1) * SG::kBytes, wave, lane);
+      } else {
+        stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+      }
+    }
+    rp ^= 1;
+    cell_off0 = (uint32_t)(cell0 * p.E + e) * (uint32_t)sizeof(T);
+    f_off0 = (uint32_t)cell0 * (uint32_t)(3 * kN * sizeof(float));
+
+    // ---- recompute the states of the block, keeping the gates
+#pragma unroll
+    for (int k = 0; k < kCK; ++k) {
+      if (t0 + k < p.T_total) {
+        const float4 kk = *reinterpret_cast<const float4*>(bufc + const_off + k * SG::kKStr);
+        const float offT = kk.x, offL = kk.y, cT = kk.z, cL = kk.w;
+        float xv = 0.f, dtv = 0.f, dlv = 0.f;
+        if constexpr (STAGE_X) {
+          const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
+          xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + SG::kXTauBytes / sizeof(T)); dlv = IO<T>::ld(xr + 2 * SG::kXTauBytes / sizeof(T));
+        } else if (ch_ok && ((bp.in_grid >> k) & 1u)) {
+          const uint32_t off = cell_off0 + (uint32_t)k * estep + (k >= bp.kw ? wrap_adj : 0u);
+          xv = IO<T>::ld(reinterpret_cast<const T*>(Ximg + off));
+          dtv = IO<T>::ld(reinterpret_cast<const T*>(DTimg + off));
+          dlv = IO<T>::ld(reinterpret_cast<const T*>(DLimg + off));
+        }
+        const char* rec = bufc + (rec_off + k * SG::kKStr);
+        const float4 b4 = *reinterpret_cast<const float4*>(rec);
+        const float4 l4 = *reinterpret_cast<const float4*>(rec + SG::kBLOff);
+        const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w};
+        const float sT = __builtin_fmaf(cT * dtv, xv, g1);
+        const float sL = cL * dlv * xv;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) gT[k][w] = fexp2(__builtin_fmaf(dtv, a2t[w], offT));
+        pin4(gT[k]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) gL[k][w] = fexp2(__builtin_fmaf(dlv, a2l[w], offL));
+        pin4(gL[k]);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          float u = sL * lq[w];
+          u = __builtin_fmaf(sT, bq[w], u);
+          u = fma_row_below(gT[k][w], hb[k][w], u);
+          hb[k + 1][w] = __builtin_fmaf(gL[k][w], hb[k][w], u);
+        }
+      } else {
+#pragma unroll
+        for (int w = 0; w < 4; ++w) { gT[k][w] = 0.f; gL[k][w] = 0.f; hb[k + 1][w] = 0.f; }
+      }
+    }
+    // ---- adjoint over the block, last step first
+#pragma unroll
+    for (int k = kCK - 1; k >= 0; --k) {
+      if (k == 0) staging_landed();   // before the last stores of the block
+      if (k == (kCK > 1 ? 1 : 0) && m > m_lo) load_ckpt(m - 1, ck_take);
+      if (t0 + k < p.T_total) {
+        const float4 kk = *reinterpret_cast<const float4*>(bufc + const_off + k * SG::kKStr);
+        const float cT = kk.z, cL = kk.w;
+        const bool inr = ch_ok && ((bp.in_grid >> k) & 1u);
+        const uint32_t goff = cell_off0 + (uint32_t)k * estep + (k >= bp.kw ? wrap_adj : 0u);
+        float xv = 0.f, dtv = 0.f, dlv = 0.f, dyv = 0.f;
+        if constexpr (STAGE_X) {
+          const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
+          xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + SG::kXTauBytes / sizeof(T)); dlv = IO<T>::ld(xr + 2 * SG::kXTauBytes / sizeof(T));
+          dyv = IO<T>::ld(xr + 3 * SG::kXTauBytes / sizeof(T));
+        } else if (inr) {
+          xv = IO<T>::ld(reinterpret_cast<const T*>(Ximg + goff));
+          dtv = IO<T>::ld(reinterpret_cast<const T*>(DTimg + goff));
+          dlv = IO<T>::ld(reinterpret_cast<const T*>(DLimg + goff));
+          dyv = IO<T>::ld(reinterpret_cast<const T*>(DYimg + goff));
+        }
+        const char* rec = bufc + (rec_off + k * SG::kKStr);
+        const float4 b4 = *reinterpret_cast<const float4*>(rec);
+        const float4 l4 = *reinterpret_cast<const float4*>(rec + SG::kBLOff);
+        const float4 c4 = *reinterpret_cast<const float4*>(rec + SG::kCOff);
+        const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w}, cq[4] = {c4.x, c4.y, c4.z, c4.w};
+        const float qT = cT * dtv * xv, qL = cL * dlv * xv;   // zero on lanes that are not grid cells
+        const float dyl = dyv + gb1;
+        float sT = 0.f, sL = 0.f, zT = 0.f, zL = 0.f;
+        float vC[4], vBT[4], vBL[4];
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          const float lam = __builtin_fmaf(dyl, cq[w], add_row_above(muL[w], muT[w]));
+          const float mT = gT[k][w] * lam, mL = gL[k][w] * lam;
+          muT[w] = mT;
+          muL[w] = mL;
+          const float ZT = mul_row_below(mT, hb[k][w]), ZL = mL * hb[k][w];
+          accAT[w] = __builtin_fmaf(ZT, dtv, accAT[w]);
+          accAL[w] = __builtin_fmaf(ZL, dlv, accAL[w]);
+          zT = __builtin_fmaf(ZT, a2t[w], zT);
+          zL = __builtin_fmaf(ZL, a2l[w], zL);
+          sT = __builtin_fmaf(lam, bq[w], sT);
+          sL = __builtin_fmaf(lam, lq[w], sL);
+          vBT[w] = qT * lam;
+          vBL[w] = qL * lam;
+          vC[w] = dyv * hb[k + 1][w];
+        }
+        float4* sw = slots + (xpar * NW + wave) * SLOT + lane;
+        sw[0] = make_float4(vC[0], vC[1], vC[2], vC[3]);
+        sw[64] = make_float4(vBT[0], vBT[1], vBT[2], vBT[3]);
+        sw[128] = make_float4(vBL[0], vBL[1], vBL[2], vBL[3]);
+        if (p.nbands > 1) {   // first row of a band: the lower ghost of the band above will replay its muT
+          const bool wk = k >= bp.kw;
+          if (inr && r == 1 && (wk ? bp.bnd0 + 1 : bp.bnd0) >= 1) {
+            const int ck = wk ? bp.col0 + k - p.S : bp.col0 + k;
+            float4* bb = reinterpret_cast<float4*>(BOTimg + (wk ? bp.bnd0 + 1 : bp.bnd0) * p.bot_stride * (int64_t)sizeof(float) +
+                                                   (uint32_t)(ck * p.E + e) * (uint32_t)(kN * sizeof(float))) + g;
+            const float4 row = make_float4(muT[0], muT[1], muT[2], muT[3]);
+            if constexpr (SLICED) store_row_device_scope(bb, row); else *bb = row;
+          }
+        }
+        // the lane's share (its 4 states) of d_deltaT, d_deltaL and d_x of the cell; summed over the 4
+        // groups, the totals arrive in the lanes of group 0, 2 and 1
+        const float pT = __builtin_fmaf(cT * xv, sT, kLn2 * zT);
+        const float pL = __builtin_fmaf(cL * xv, sL, kLn2 * zL);
+        const float pX = __builtin_fmaf(cT * dtv, sT, cL * dlv * sL);
+        float tot = fold16(fold32(pT, pL), fold32(pX, 0.f));
+        accD = __builtin_fmaf(dyv, xv, accD);
+        if (p.dpre && (g & 1) == 0) tot *= softplus_slope<T>(g == 0 ? dtv : dlv);   // gradients with respect to what the softplus was applied to
+        if (g == 1) tot = __builtin_fmaf(dyv, dsk, tot);
+        if (inr && g != 3) IO<T>::st(reinterpret_cast<T*>(OUTimg + goff), tot);
+        // ---- across the waves of the workgroup
+        __syncthreads();
+        if (f_on && ((bp.in_grid >> k) & 1u)) {
+          const uint32_t off = f_off0 + (uint32_t)k * pstep + (k >= bp.kw ? pwrap_adj : 0u);
+          const float2* sl = reinterpret_cast<const float2*>(slots + xpar * NW * SLOT + f_v * 64 + lane) + f_c;
+          float2 sum = sl[0];
+#pragma unroll
+          for (int w = 1; w < NW; ++w) { sum.x += sl[2 * w * SLOT].x; sum.y += sl[2 * w * SLOT].y; }
+          *reinterpret_cast<float*>(PARTimg + off + f_sub0) = sum.x;
+          *reinterpret_cast<float*>(PARTimg + off + f_sub1) = sum.y;
+        }
+        xpar ^= 1;
+      }
+    }
+    __syncthreads();
+    if constexpr (SLICED) link.publish((uint32_t)(m_hi - 1 - m));
+    A = Aprev;
+    bp = bpn;
+    cell0 = celln;
+    cur ^= 1;
+  }
+  if constexpr (SLICED) {
+    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __syncthreads();
+    link.publish((uint32_t)p.sl_nbb);
+  }
+
+  // ---- sums over positions: reduce over the rows of the band (the 16 lanes of a group)
+  float red[9];
+#pragma unroll
+  for (int w = 0; w < 4; ++w) { red[w] = accAT[w]; red[4 + w] = accAL[w]; }
+  red[8] = accD;
+#pragma unroll
+  for (int k = 0; k < 9; ++k) {
+    float v = red[k];
+#pragma unroll
+    for (int off = kHB >> 1; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    red[k] = v;
+  }
+  if (ch_ok && r == 0) {
+    const int64_t slot_e = ((int64_t)b * p.pa_slots + (SLICED ? my_band : 0)) * p.E + e;
+    float* pa = p.pA + slot_e * (2 * kN);
+#pragma unroll
+    for (int w = 0; w < 4; ++w) { pa[state_of[w]] = red[w]; pa[kN + state_of[w]] = red[4 + w]; }
+    if (g == 0) p.pD[slot_e] = red[8];
+  }
+}
+
 // -------------------------------------------------------------------------- small helper kernels
 // the value a tensor of type T would hold
 __device__ __forceinline__ float as_stored(float v, const float*) { return v; }
@@ -1625,6 +2198,7 @@ struct Geometry {
   int S, T_total, rows_last;         // stream stride, total steps, rows of the last band
   int fwd_ec, fwd_nw, fwd_wpb, fwd_bpb;   // forward: channels per lane, waves per workgroup, waves and workgroups per image
   int bwd_nw, bwd_wpb, bwd_bpb;      // backward: waves per workgroup, waves and workgroups (channel groups) per image
+  bool fwd_split, bwd_split;         // the states of a channel split over the lanes (a wave per channel: m2d_fwd_split_kernel, m2d_bwd_split_kernel)
   bool stage_x;                      // x, delta, dy rows are whole 16-byte chunks: stage them through LDS
   bool sliced;                       // linked sweep: bands on workgroups of their own, handing boundary rows to each other inside one launch
   bool stacked;                      // images of one band stacked into tall images of independent bands
@@ -1640,7 +2214,8 @@ int check_desc(const m2d_desc* d) {
   if (d->B < 1 || d->E < 1 || d->N < 1 || d->H < 2 || d->W < 2) return M2D_ERR_BAD_SHAPE;
   if (d->N != kN) return M2D_ERR_UNSUPPORTED;
   if (d->dtype != M2D_F32 && d->dtype != M2D_BF16) return M2D_ERR_UNSUPPORTED;
-  if (d->reserved != 0 || (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_RAW_PARAMS | M2D_FLAG_PACKED_BC | M2D_FLAG_DPRE))) return M2D_ERR_UNSUPPORTED;
+  if (d->reserved != 0 || (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_RAW_PARAMS | M2D_FLAG_PACKED_BC | M2D_FLAG_DPRE | M2D_FLAG_SPLIT_STATES | M2D_FLAG_WHOLE_STATES))) return M2D_ERR_UNSUPPORTED;
+  if ((d->flags & M2D_FLAG_SPLIT_STATES) && (d->flags & M2D_FLAG_WHOLE_STATES)) return M2D_ERR_UNSUPPORTED;
   if ((int64_t)d->B * d->H * d->W >= ((int64_t)1 << 40)) return M2D_ERR_BAD_SHAPE;
   // one image is addressed with 32-bit byte offsets from its base (fp32: 4 bytes per element;
   // the widest per-cell record, the channel sums, is 192 bytes)
@@ -1754,9 +2329,29 @@ Geometry make_geometry(const m2d_desc* d) {
   g.fwd_nw = (!g.stacked && !ec2 && wg_half > wg1 && wg_half * together <= room) ? kFwdHalfWaves : kFwdWaves;
   g.fwd_bpb = (d->E + g.fwd_nw * g.CS * g.fwd_ec - 1) / (g.fwd_nw * g.CS * g.fwd_ec);
   g.fwd_wpb = g.fwd_bpb * g.fwd_nw;
+  // Few waves under way (a wave per 4 channels, the bands of a linked sweep that overlap in time): fewer
+  // than three for every four SIMDs.  Then a wave per channel, each with a quarter of the states.
+  const int64_t waves_whole = (int64_t)B * ((d->E + g.CS - 1) / g.CS) * together;
+  const bool may_split = !g.stacked && !(d->flags & M2D_FLAG_WHOLE_STATES);
+  g.fwd_split = may_split && ((d->flags & M2D_FLAG_SPLIT_STATES) || waves_whole <= 3 * ncu);
+  if (g.fwd_split) {
+    g.fwd_ec = 1;
+    g.fwd_nw = kSplitWaves;
+    g.fwd_bpb = (d->E + kSplitWaves - 1) / kSplitWaves;
+    g.fwd_wpb = g.fwd_bpb * g.fwd_nw;
+  }
   g.bwd_nw = (!g.stacked && wg_half > (int64_t)B * groups && wg_half * together <= room) ? kFwdHalfWaves : kBwdWaves;
   g.bwd_bpb = (d->E + g.bwd_nw * g.CS - 1) / (g.bwd_nw * g.CS);
   g.bwd_wpb = g.bwd_bpb * g.bwd_nw;
+  // (the backward keeps one set of channel sums per workgroup of an image: with 8 channels per workgroup
+  // that memory is bounded here unless the caller insists)
+  const size_t split_part = sizeof(float) * (size_t)((d->E + kSplitWaves - 1) / kSplitWaves) * 3 * kN * (size_t)d->B * d->H * d->W;
+  g.bwd_split = may_split && ((d->flags & M2D_FLAG_SPLIT_STATES) || (waves_whole <= 3 * ncu && split_part <= ((size_t)2 << 30)));
+  if (g.bwd_split) {
+    g.bwd_nw = kSplitWaves;
+    g.bwd_bpb = (d->E + kSplitWaves - 1) / kSplitWaves;
+    g.bwd_wpb = g.bwd_bpb * g.bwd_nw;
+  }
   g.stage_x = (d->E % (d->dtype == M2D_BF16 ? 8 : 4)) == 0;
   const size_t P = (size_t)d->B * d->H * d->W;
   g.prep_bytes = align_up(sizeof(float) * (kZeroFloats + (size_t)2 * d->E * kN + d->E));
@@ -1862,6 +2457,32 @@ int launch_fwd_as(const ScanParams& sp, hipStream_t st) {
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
+template <typename T>
+constexpr size_t fwd_split_lds_bytes() { return 2 * (size_t)Stage<T, 3, kSplitWaves, false>::kBytes + (sizeof(T) == 2 ? 2 * kRawBytes : 0); }
+template <typename T, bool CK, bool WY, bool SX, int MODE>
+int launch_fwd_split_as(const ScanParams& sp, hipStream_t st) {
+  constexpr size_t lds = fwd_split_lds_bytes<T>();
+  static_assert(lds <= kLdsPerWorkgroup, "staging must fit the LDS");
+  static std::atomic<uint64_t> seen{0};
+  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_fwd_split_kernel<T, CK, WY, SX, MODE>), lds, seen)) return M2D_ERR_HIP;
+  hipLaunchKernelGGL((m2d_fwd_split_kernel<T, CK, WY, SX, MODE>), dim3((unsigned)sp.nwg), dim3(kSplitWaves * 64), lds, st, sp);
+  return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+}
+// (16-bit x and deltas of 8 channels are less than a 16-byte chunk per cell: read from memory, not staged)
+template <typename T, int MODE>
+int launch_fwd_split(const ScanParams& sp, bool stage_x, bool ckpt, bool write_y, hipStream_t st) {
+  if constexpr (sizeof(T) == 4) {
+    if (stage_x) {
+      if (ckpt && write_y) return launch_fwd_split_as<T, true, true, true, MODE>(sp, st);
+      if (ckpt) return launch_fwd_split_as<T, true, false, true, MODE>(sp, st);
+      return launch_fwd_split_as<T, false, true, true, MODE>(sp, st);
+    }
+  }
+  if (ckpt && write_y) return launch_fwd_split_as<T, true, true, false, MODE>(sp, st);
+  if (ckpt) return launch_fwd_split_as<T, true, false, false, MODE>(sp, st);
+  return launch_fwd_split_as<T, false, true, false, MODE>(sp, st);
+}
+
 template <typename T, int EC, bool SX, int MODE, int NW = kFwdWaves>
 int launch_fwd_mode(const ScanParams& sp, bool ckpt, bool write_y, hipStream_t st) {
   if (ckpt && write_y) return launch_fwd_as<T, EC, true, true, SX, MODE, NW>(sp, st);
@@ -1875,6 +2496,8 @@ int launch_fwd(const ScanParams& sp0, const m2d_desc* d, const Geometry& g, bool
   sp.bpb = g.fwd_bpb;
   sp.nwg = g.vB * g.fwd_bpb;
   auto once = [&]() {
+    if (g.fwd_split)
+      return g.sliced ? launch_fwd_split<T, kModeSliced>(sp, g.stage_x, ckpt, write_y, st) : launch_fwd_split<T, kModeSweep>(sp, g.stage_x, ckpt, write_y, st);
     if (g.sliced) {   // (the linked sweep is only chosen where one channel per lane is)
       if (g.fwd_nw == kFwdHalfWaves)
         return g.stage_x ? launch_fwd_mode<T, 1, true, kModeSliced, kFwdHalfWaves>(sp, ckpt, write_y, st)
@@ -1938,6 +2561,28 @@ int launch_bwd_as(const ScanParams& sp, hipStream_t st) {
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
+template <typename T>
+constexpr size_t bwd_split_lds_bytes() {
+  return sizeof(float4) * 2 * kSplitWaves * 3 * 64 + 2 * (size_t)Stage<T, 4, kSplitWaves, true>::kBytes + (sizeof(T) == 2 ? 2 * kRawBytes : 0);
+}
+template <typename T, bool SX, int MODE>
+int launch_bwd_split_as(const ScanParams& sp, hipStream_t st) {
+  constexpr size_t lds = bwd_split_lds_bytes<T>();
+  static_assert(lds <= kLdsPerWorkgroup, "exchange buffers and staging must fit the LDS");
+  static std::atomic<uint64_t> seen{0};
+  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_bwd_split_kernel<T, SX, MODE>), lds, seen)) return M2D_ERR_HIP;
+  hipLaunchKernelGGL((m2d_bwd_split_kernel<T, SX, MODE>), dim3((unsigned)sp.nwg), dim3(kSplitWaves * 64), lds, st, sp);
+  return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+}
+// (16-bit x, deltas and dy of 8 channels are less than a 16-byte chunk per cell: read from memory, not staged)
+template <typename T, int MODE>
+int launch_bwd_split(const ScanParams& sp, bool stage_x, hipStream_t st) {
+  if constexpr (sizeof(T) == 4) {
+    if (stage_x) return launch_bwd_split_as<T, true, MODE>(sp, st);
+  }
+  return launch_bwd_split_as<T, false, MODE>(sp, st);
+}
+
 template <typename T, bool SX, int MODE>
 int launch_bwd(const ScanParams& sp, hipStream_t st, int nw = kBwdWaves) {
   if constexpr (MODE != kModeStacked) {
@@ -1979,13 +2624,15 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   sp.nwg = g.vB * g.bwd_bpb;
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][0], st);
   if (!g.sliced) {
-    if (g.stacked) rc = g.stage_x ? launch_bwd<T, true, kModeStacked>(sp, st) : launch_bwd<T, false, kModeStacked>(sp, st);
+    if (g.bwd_split) rc = launch_bwd_split<T, kModeSweep>(sp, g.stage_x, st);
+    else if (g.stacked) rc = g.stage_x ? launch_bwd<T, true, kModeStacked>(sp, st) : launch_bwd<T, false, kModeStacked>(sp, st);
     else rc = g.stage_x ? launch_bwd<T, true, kModeSweep>(sp, st, g.bwd_nw) : launch_bwd<T, false, kModeSweep>(sp, st, g.bwd_nw);
   } else {
     // every band on workgroups of its own, the last band first: a band waits for the one below it
     sp.nwg = g.nbands * g.vB * g.bwd_bpb;
     sp.prog = sp.link_err + 64 + (size_t)g.nbands * g.vB * (g.fwd_bpb > g.bwd_bpb ? g.fwd_bpb : g.bwd_bpb);
-    rc = g.stage_x ? launch_bwd<T, true, kModeSliced>(sp, st, g.bwd_nw) : launch_bwd<T, false, kModeSliced>(sp, st, g.bwd_nw);
+    if (g.bwd_split) rc = launch_bwd_split<T, kModeSliced>(sp, g.stage_x, st);
+    else rc = g.stage_x ? launch_bwd<T, true, kModeSliced>(sp, st, g.bwd_nw) : launch_bwd<T, false, kModeSliced>(sp, st, g.bwd_nw);
   }
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][1], st);
   if (rc) return rc;

@@ -27,6 +27,17 @@ def cabi():
     return m
 
 
+@pytest.fixture(autouse=True, params=["auto", "split_states", "whole_states"])
+def lane_layout(request):
+    """Every case of this module runs three times: with the library's own choice of lane layout,
+    with the 16 states of a channel split over the lanes of a wave wherever that layout exists
+    (M2D_FLAG_SPLIT_STATES), and with that layout forbidden (M2D_FLAG_WHOLE_STATES)."""
+    from mamba2d_amd import cabi as m
+    m.SCHEDULE_HINT = {"auto": 0, "split_states": m.M2D_FLAG_SPLIT_STATES, "whole_states": m.M2D_FLAG_WHOLE_STATES}[request.param]
+    yield request.param
+    m.SCHEDULE_HINT = 0
+
+
 def say(*a):
     print(*a, flush=True)
     sys.stdout.flush()
