@@ -50,10 +50,11 @@ def test_descriptor_validation(cabi):
     assert cabi.lib.m2d_desc_check(None) == 1
     # spatial dims must exceed 1, like the reference's ValueError (wavefront_cuda.py:323-324)
     assert chk(D(cabi, H=1)) == 2 and chk(D(cabi, W=1)) == 2 and chk(D(cabi, B=0)) == 2
-    # flags 1 (flip), 4 (raw parameters), 8 (packed B/C) and 16 (gradients before the softplus) belong to the
-    # scan; 2 is a projection flag, 32 nobody's
+    # flags 1 (flip), 4 (raw parameters), 8 (packed B/C), 16 (gradients before the softplus) and the two lane
+    # layout hints 32 and 64 (one of them at most) belong to the scan; 2 is a projection flag, 128 nobody's
     assert chk(D(cabi, flags=4)) == 0 and chk(D(cabi, flags=29)) == 0 and chk(D(cabi, flags=2)) == 3
-    assert chk(D(cabi, N=8)) == 3 and chk(D(cabi, dtype=7)) == 3 and chk(D(cabi, flags=32)) == 3
+    assert chk(D(cabi, flags=32)) == 0 and chk(D(cabi, flags=64 | 1)) == 0 and chk(D(cabi, flags=96)) == 3
+    assert chk(D(cabi, N=8)) == 3 and chk(D(cabi, dtype=7)) == 3 and chk(D(cabi, flags=128)) == 3
     assert chk(D(cabi, reserved=1)) == 3
     # one image must fit 32-bit offsets: H*W < 2^24 cells, H*W*E < 2^30 elements
     assert chk(D(cabi, B=1, H=4096, W=4096, E=8)) == 3 and chk(D(cabi, B=1, H=2048, W=2048, E=256)) == 3
@@ -88,12 +89,18 @@ def test_buffer_sizes_scale_linearly_in_area(cabi):
     (B,H,W,E,N) fp32 state tensor for large grids."""
     sizes = {}
     for hw in (256, 512, 1024, 2048):
-        d = D(cabi, B=1, H=hw, W=hw, E=64)
+        # (one lane layout for all four sizes; the library's own choice is compared with it below)
+        d = D(cabi, B=1, H=hw, W=hw, E=64, flags=cabi.M2D_FLAG_WHOLE_STATES)
         ck = cabi.lib.m2d_scan_ckpt_bytes(ctypes.byref(d))
         wsb = cabi.lib.m2d_scan_workspace_bytes(ctypes.byref(d), 1, 1)
         sizes[hw] = (ck, wsb)
         full_state = hw * hw * 64 * 16 * 4
         assert ck < 0.6 * full_state
+        # splitting the states over the lanes keeps a set of channel sums per 8 channels instead of per 16 or 32:
+        # the library's own choice may cost up to that much more scratch, never more checkpoints
+        auto = D(cabi, B=1, H=hw, W=hw, E=64)
+        assert cabi.lib.m2d_scan_ckpt_bytes(ctypes.byref(auto)) <= ck * 1.01
+        assert cabi.lib.m2d_scan_workspace_bytes(ctypes.byref(auto), 1, 1) <= 2.5 * wsb
     for a, b in ((256, 512), (512, 1024), (1024, 2048)):
         for k in range(2):
             ratio = sizes[b][k] / sizes[a][k]
