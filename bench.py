@@ -44,7 +44,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the backward scan kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/scan_cfg1_kernel_trace_and_traffic.txt); counters cannot be read from inside this script,
 # so the figure is carried here for the workload that has a counter run, and is null for the others.
-MEASURED_TRAFFIC = {"cfg1": 1.3849e9}
+MEASURED_TRAFFIC = {"cfg1": 1.3965e9}
 # Issue slots per (cell, channel, state) of the scan kernels (a v_exp_f32 takes two on gfx950):
 # forward 2 exponent FMAs + 2 v_exp + 5 FMA-class (input term, two gate terms, y);
 # backward 10 for the recomputation, 24 for the adjoint (15 FMA-class, 4.5 for the gates of three steps in
@@ -62,10 +62,14 @@ def nominal_valu_slots_per_s():
 
 def scan_roofline(name, B, E, H, W, s, bwd_kernel_ms, fwd_kernel_ms):
     """The `roofline` object for the backward scan kernel (the dominant kernel) of a scan workload."""
+    from mamba2d_amd import cabi
     fb, bb = algorithmic_bytes(B, E, H, W, s)
     achieved = bb / (bwd_kernel_ms * 1e-3) / 1e9
+    dts = "bf16" if s == 2 else "f32"
+    plan_bwd = cabi.scan_plan(B, H, W, E, dts, cabi.M2D_PASS_BWD)
+    plan_fwd = cabi.scan_plan(B, H, W, E, dts, cabi.M2D_PASS_FWD)
     return {
-        "kernel": "m2d_bwd_kernel", "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+        "kernel": plan_bwd.split(":")[0], "schedule": plan_bwd, "fwd_schedule": plan_fwd, "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
         "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(name),
         "kernel_ms": round(bwd_kernel_ms, 4), "algorithmic_bytes": bb,
         "fwd_kernel_ms": round(fwd_kernel_ms, 4), "fwd_algorithmic_bytes": fb,
@@ -435,7 +439,8 @@ def main():
     s = 2 if dts == "bf16" else 4
     fb, bb = algorithmic_bytes(B, E, H, W, s)
     out = {
-        "metric": "2D-scan fwd & fwd+bwd ms at B=128 D=64 56x56 N=16; % of HBM roofline",
+        # (the headline metric is quoted on cfg1; the other scan workloads say their own shape)
+        "metric": f"2D-scan fwd & fwd+bwd ms at B={B} D={E} {H}x{W} N={N}; % of HBM roofline",
         "value": round(step_ms, 4),
         "unit": "ms",
         "n_gpus": 1,

@@ -138,6 +138,12 @@ int m2d_scan_fwd(const m2d_desc* desc,
  * ordered by kernel launches, wf_cuda.cu:203,259). */
 int m2d_scan_link_error(const m2d_desc* desc, const void* workspace, void* stream, int* gave_up);
 
+/* What the library will do with a problem: one line of text per pass (M2D_PASS_FWD / M2D_PASS_BWD), e.g.
+ * "m2d_bwd_split_kernel: linked sweep, 19 bands, 152 workgroups of 8 waves, 8 channels each, 4 states per lane".
+ * Writes at most `cap` bytes including the terminating 0; host only, touches no device.  Returns M2D_OK or the
+ * status m2d_desc_check gives.  No counterpart in the reference (which has one schedule). */
+int m2d_scan_plan(const m2d_desc* desc, int pass, char* text, size_t cap);
+
 /* m2d_scan_fwd without a checkpoint buffer and without a workspace argument, for callers that cannot
  * allocate device memory (code under HIP graph capture, tight serving loops, harnesses that forbid
  * it).  It has no counterpart in the reference, whose Python side allocates every buffer with

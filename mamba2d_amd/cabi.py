@@ -24,7 +24,7 @@ M2D_FLAG_WHOLE_STATES = 64
 M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
-           "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_fwd_noalloc", "m2d_scan_link_error", "m2d_scan_bwd", "m2d_proj_workspace_bytes", "m2d_proj_fwd",
+           "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_fwd_noalloc", "m2d_scan_link_error", "m2d_scan_plan", "m2d_scan_bwd", "m2d_proj_workspace_bytes", "m2d_proj_fwd",
            "m2d_proj_bwd", "m2d_layernorm_fwd", "m2d_dwconv3x3_fwd", "m2d_starrelu_fwd",
            "m2d_scale_residual_fwd", "m2d_scale_residual_layernorm_fwd", "m2d_rope_qknorm_fwd", "m2d_rope_attention_fwd", "m2d_mlp_fwd", "m2d_layernorm_linear_fwd", "m2d_linear_fwd", "m2d_profile_enable", "m2d_profile_last_ms")
 
@@ -60,6 +60,8 @@ def _load():
     lib.m2d_scan_fwd.argtypes = [dp] + [vp] * 9 + [vp, vp, sz, vp, sz, vp]
     lib.m2d_scan_link_error.restype = i32
     lib.m2d_scan_link_error.argtypes = [dp, vp, vp, ctypes.POINTER(ctypes.c_int)]
+    lib.m2d_scan_plan.restype = i32
+    lib.m2d_scan_plan.argtypes = [dp, i32, ctypes.c_char_p, sz]
     lib.m2d_scan_fwd_noalloc.restype = i32
     lib.m2d_scan_fwd_noalloc.argtypes = [dp] + [vp] * 9 + [vp, vp]
     lib.m2d_scan_bwd.restype = i32
@@ -181,6 +183,15 @@ def _check_links(d, ws, dev):
         check(lib.m2d_scan_link_error(ctypes.byref(d), _ptr(ws), _stream(dev), ctypes.byref(flag)))
         if flag.value:
             raise RuntimeError("m2dscan: a workgroup of the linked sweep gave up waiting for its neighbour")
+
+
+def scan_plan(B, H, W, E, dtype, pass_=M2D_PASS_FWD, N=16, flags=None):
+    """The library's one-line description of how it will run a pass of this problem (m2d_scan_plan)."""
+    dt = M2D_F32 if dtype in (torch.float32, "f32") else M2D_BF16
+    d = Desc(B, H, W, E, N, dt, SCHEDULE_HINT if flags is None else flags, 0)
+    buf = ctypes.create_string_buffer(256)
+    check(lib.m2d_scan_plan(ctypes.byref(d), pass_, buf, len(buf)))
+    return buf.value.decode()
 
 
 def scan_fwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, save_ckpt=False, flip=False):

@@ -36,6 +36,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <cstdio>
 #include <stdint.h>
 
 #include "../../include/m2dscan.h"
@@ -2744,6 +2745,30 @@ int m2d_scan_bwd(const m2d_desc* desc, const void* x, const void* deltaT, const 
   return desc->dtype == M2D_F32
              ? run_bwd<float>(desc, g, sp, AT, AL, BT, BL, C, D, ckpt, d_AT, d_AL, d_BT, d_BL, d_C, d_D, workspace, st)
              : run_bwd<bf16_t>(desc, g, sp, AT, AL, BT, BL, C, D, ckpt, d_AT, d_AL, d_BT, d_BL, d_C, d_D, workspace, st);
+}
+
+int m2d_scan_plan(const m2d_desc* desc, int pass, char* text, size_t cap) {
+  if (!desc || !text) return M2D_ERR_NULL_POINTER;
+  if (cap == 0 || (pass != M2D_PASS_FWD && pass != M2D_PASS_BWD)) return M2D_ERR_BAD_SHAPE;
+  const int rc = check_desc(desc);
+  if (rc != M2D_OK) { text[0] = 0; return rc; }
+  const Geometry g = make_geometry(desc);
+  const bool fwd = pass == M2D_PASS_FWD;
+  const bool split = fwd ? g.fwd_split : g.bwd_split;
+  const int nw = fwd ? g.fwd_nw : g.bwd_nw, bpb = fwd ? g.fwd_bpb : g.bwd_bpb;
+  const int per_lane = fwd ? g.fwd_ec : 1;
+  const long long wgs = (long long)(g.sliced ? g.nbands : 1) * g.vB * bpb;
+  char sched[96];
+  if (g.sliced) snprintf(sched, sizeof sched, "linked sweep, %d bands", g.nbands);
+  else if (g.stacked) snprintf(sched, sizeof sched, "stacked images, %d per stream, %d bands", g.ips, g.nbands);
+  else snprintf(sched, sizeof sched, "one stream per image, %d band%s back to back", g.nbands, g.nbands == 1 ? "" : "s");
+  if (split)
+    snprintf(text, cap, "%s: %s, %lld workgroups of %d waves, %d channels each, 4 states per lane",
+             fwd ? "m2d_fwd_split_kernel" : "m2d_bwd_split_kernel", sched, wgs, nw, nw);
+  else
+    snprintf(text, cap, "%s: %s, %lld workgroups of %d waves, %d channels each, 16 states per lane",
+             fwd ? "m2d_fwd_kernel" : "m2d_bwd_kernel", sched, wgs, nw, nw * g.CS * per_lane);
+  return M2D_OK;
 }
 
 int m2d_scan_link_error(const m2d_desc* desc, const void* workspace, void* stream, int* gave_up) {

@@ -109,6 +109,23 @@ def test_buffer_sizes_scale_linearly_in_area(cabi):
     assert cabi.lib.m2d_scan_ckpt_bytes(ctypes.byref(D(cabi, N=3))) == 0
 
 
+def test_plan_names_kernel_and_schedule(cabi):
+    """m2d_scan_plan (host only): which kernel and schedule a problem gets on a 256-unit device."""
+    import torch
+    big = cabi.scan_plan(128, 56, 56, 64, torch.bfloat16, cabi.M2D_PASS_BWD)
+    assert big.startswith("m2d_bwd_kernel: one stream per image, 4 bands back to back, 256 workgroups of 8 waves, 32 channels each")
+    one = cabi.scan_plan(1, 256, 256, 64, torch.float32, cabi.M2D_PASS_BWD)
+    assert one.startswith("m2d_bwd_split_kernel: linked sweep, 19 bands, 152 workgroups of 8 waves, 8 channels each, 4 states per lane")
+    whole = cabi.scan_plan(1, 256, 256, 64, torch.float32, cabi.M2D_PASS_FWD, flags=cabi.M2D_FLAG_WHOLE_STATES)
+    assert whole.startswith("m2d_fwd_kernel: linked sweep, 19 bands") and "16 states per lane" in whole
+    small = cabi.scan_plan(128, 7, 7, 512, torch.bfloat16, cabi.M2D_PASS_FWD)
+    assert small.startswith("m2d_fwd_kernel: stacked images")
+    # a short buffer truncates, a bad descriptor reports its status and an empty text
+    buf = ctypes.create_string_buffer(8)
+    assert cabi.lib.m2d_scan_plan(ctypes.byref(D(cabi)), 0, buf, 8) == 0 and len(buf.value) == 7
+    assert cabi.lib.m2d_scan_plan(ctypes.byref(D(cabi, H=1)), 0, buf, 8) == 2 and buf.value == b""
+
+
 def test_python_surface_matches_reference_names():
     """models/kernels/wavefront_cuda.py exposes these names; models/mamba2d.py:10 imports one."""
     from mamba2d_amd.kernels import wavefront_cuda as w
