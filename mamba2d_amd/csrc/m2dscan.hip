@@ -195,6 +195,7 @@ struct ScanParams {
   int S;                            // stream stride: positions per band (>= W)
   int T_total;                      // steps of the whole sweep
   int rows_last;                    // grid rows of the last band
+  int rb;                           // grid rows of every other band: 14 (kRB), or for stacked images the largest multiple of the image height below 15
   uint32_t magicS;                  // floor(2^32 / S)
   // Linked sweep (few images, many bands): every band has its own workgroups, all in one launch; a
   // band publishes how many blocks of its window are done (boundary rows in memory) and the band
@@ -236,10 +237,10 @@ __device__ __forceinline__ Pos pos_of(const ScanParams& p, int s) {
   Pos o; o.bnd = (int)q - 3; o.col = (int)rem;
   return o;
 }
-__device__ __forceinline__ int band_rows(const ScanParams& p, int bnd) { return bnd == p.nbands - 1 ? p.rows_last : kRB; }
+__device__ __forceinline__ int band_rows(const ScanParams& p, int bnd) { return bnd == p.nbands - 1 ? p.rows_last : p.rb; }
 // cell index inside its image of lane row r of band bnd at column col
 __device__ __forceinline__ int cell_of(const ScanParams& p, int bnd, int r, int col) {
-  const int cell = __mul24(bnd * kRB + r - 1, p.W) + col;   // rows and columns are far below 2^24
+  const int cell = __mul24(bnd * p.rb + r - 1, p.W) + col;   // rows and columns are far below 2^24
   return p.flip ? p.H * p.W - 1 - cell : cell;
 }
 
@@ -447,8 +448,8 @@ __device__ __forceinline__ LaneK lane_consts(const ScanParams& p, int bnd, int r
   // `bnd` is a band of the grid (callers clamp): a row that is before the first band or past the
   // last one works on zero operands with the constants of that band
   LaneK c;
-  c.real = ch_ok && r >= 1 && r <= kRB && r <= band_rows(p, bnd);
-  // grid row 0 of an image: no row above (stacked images: 14 is a multiple of the image height)
+  c.real = ch_ok && r >= 1 && r <= band_rows(p, bnd);
+  // grid row 0 of an image: no row above (stacked images: a band holds whole images)
   const bool first_row = p.stacked ? (r - 1) % p.Himg == 0 : (bnd == 0 && r == 1);
   const bool gbot = BWD && !p.stacked && r == kHB - 1 && bnd + 1 < p.nbands;
   c.oT = gbot ? 0.f : (!c.real || first_row ? ninf : -1.f);
@@ -467,7 +468,7 @@ __device__ __forceinline__ bool snapshot_lane(const ScanParams& p, Pos at, int r
   Pos pv;
   pv.bnd = at.col >= 1 ? at.bnd : at.bnd - 1;
   pv.col = at.col >= 1 ? at.col - 1 : p.S - 1;
-  const bool row_ok = r == 0 ? pv.bnd >= 1 : (r <= kRB && r <= band_rows(p, pv.bnd));
+  const bool row_ok = r == 0 ? pv.bnd >= 1 : r <= band_rows(p, pv.bnd);
   return ch_ok && (unsigned)pv.bnd < (unsigned)p.nbands && pv.col < p.W && row_ok;
 }
 
@@ -483,7 +484,7 @@ struct BlockPos {
 // Lane row r is a row of the grid in the bands 0 .. row_bands(r) - 1 (none for a ghost lane; a row
 // beyond the height of the last band misses that one).  A lane constant.
 __device__ __forceinline__ int row_bands(const ScanParams& p, int r) {
-  return (r >= 1 && r <= kRB) ? p.nbands - 1 + (r <= p.rows_last ? 1 : 0) : 0;
+  return (r >= 1 && r <= p.rb) ? p.nbands - 1 + (r <= p.rows_last ? 1 : 0) : 0;
 }
 // bits k < n of a block's steps
 __device__ __forceinline__ uint32_t steps_below(int n) { return (1u << (n < 0 ? 0 : (n > kCK ? kCK : n))) - 1u; }
@@ -523,7 +524,7 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int 
   const char* zeros = reinterpret_cast<const char*>(p.zeros);
   const char* bc_img = reinterpret_cast<const char*>(p.bt + img * p.bc_stride);
   const int cstep = p.flip ? -1 : 1;                      // cells per column
-  const int wrapc = (kRB * p.W - p.S) * cstep;            // extra cells of a position reached through a band change
+  const int wrapc = (p.rb * p.W - p.S) * cstep;            // extra cells of a position reached through a band change
   const int slot = lane >> kHBShift;
   auto cell_at = [&](int k) { return cell0 + k * cstep + (k >= q.kw ? wrapc : 0); };
   auto ok_at = [&](int k) { return ((q.in_grid >> k) & 1u) != 0; };
@@ -627,7 +628,7 @@ __device__ __forceinline__ void bc_direct_copy(const ScanParams& p, const void* 
   constexpr int WPK = NWAVES / kCK;
   const int ks = wave & (kCK - 1), wsub = wave / kCK;
   const int cstep = p.flip ? -1 : 1;
-  const int cell = cell0 + ks * cstep + (ks >= q.kw ? (kRB * p.W - p.S) * cstep : 0);
+  const int cell = cell0 + ks * cstep + (ks >= q.kw ? (p.rb * p.W - p.S) * cstep : 0);
   const bool ok = ((q.in_grid >> ks) & 1u) != 0;
   const int slot = lane >> kHBShift;
   const int64_t img_bytes = (int64_t)b * p.Hs * p.W * (kN * (int64_t)sizeof(T));
@@ -644,7 +645,7 @@ template <int NWAVES>
 __device__ __forceinline__ void bc_raw_copy(const ScanParams& p, const void* const* tensors, char* raw, int b, const BlockPos& q,
                                             int cell0, int wave, int lane, bool live) {
   const int cstep = p.flip ? -1 : 1;
-  const int wrapc = (kRB * p.W - p.S) * cstep;
+  const int wrapc = (p.rb * p.W - p.S) * cstep;
   const int sel = lane >> 5, hf = (lane >> kHBShift) & 1;
   const int64_t img_bytes = (int64_t)b * p.Hs * p.W * (kN * 2);
   for (int j = wave; j < kCK * 3 / 2; j += NWAVES) {   // (uniform) pairs (2j, 2j+1) of (step, tensor) = (c / 3, c % 3)
@@ -696,6 +697,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   ScanParams p = pin;   // (stacked images: the height is shortened below for a last, shorter stack)
   if constexpr (!STACKED) {   // lets the compiler drop what only stacked images need
     __builtin_assume(p.stacked == 0);
+    __builtin_assume(p.rb == kRB);
     __builtin_assume(p.S >= kHB + kCK - 1);
   }
   constexpr int CS = 64 >> kHBShift;
@@ -726,8 +728,8 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   if constexpr (STACKED) {   // the last stack of the batch may hold fewer images
     const int nimg = p.Breal - b * p.ips < p.ips ? p.Breal - b * p.ips : p.ips;
     p.H = nimg * p.Himg;
-    p.nbands = (p.H + kRB - 1) / kRB;
-    p.rows_last = p.H - (p.nbands - 1) * kRB;
+    p.nbands = (p.H + p.rb - 1) / p.rb;
+    p.rows_last = p.H - (p.nbands - 1) * p.rb;
   }
   const int slot = lane >> kHBShift, r = lane & (kHB - 1);
   const int rbands = row_bands(p, r);
@@ -778,7 +780,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   const uint32_t estep = (uint32_t)(p.flip ? -p.E : p.E) * (uint32_t)sizeof(T);   // one column further
 
   const float g1 = r == 0 ? 1.f : 0.f;             // the ghost's T input coefficient
-  const uint32_t wrap_adj = (uint32_t)(kRB * p.W - p.S) * estep;   // extra offset of a cell reached through a band change
+  const uint32_t wrap_adj = (uint32_t)(p.rb * p.W - p.S) * estep;   // extra offset of a cell reached through a band change
 
   // byte offsets of the lane's operand groups inside a staging buffer (step 0, group 0): a grid row
   // reads B_T, B_L, C of its cell; the ghost reads the row above as its B_T (and row 0 of the B_L and C
@@ -1043,6 +1045,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_fwd_split_kernel(const S
   constexpr bool SLICED = MODE == kModeSliced;
   const ScanParams& p = pin;
   __builtin_assume(p.stacked == 0);
+  __builtin_assume(p.rb == kRB);
   __builtin_assume(p.S >= kHB + kCK - 1);
   constexpr int NW = kSplitWaves, CW = NW;
   using SG = Stage<T, 3, CW, false>;
@@ -1102,7 +1105,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_fwd_split_kernel(const S
   const char* DTimg = reinterpret_cast<const char*>(DT) + img_bytes;
   const char* DLimg = reinterpret_cast<const char*>(DL) + img_bytes;
   const uint32_t estep = (uint32_t)(p.flip ? -p.E : p.E) * (uint32_t)sizeof(T);
-  const uint32_t wrap_adj = (uint32_t)(kRB * p.W - p.S) * estep;
+  const uint32_t wrap_adj = (uint32_t)(p.rb * p.W - p.S) * estep;
   const float g1 = r == 0 ? 1.f : 0.f;             // the ghost's T input coefficient
 
   // the lane's group of B_T (the ghost: of the row above), of B_L and C (the ghost: zeros of its own row)
@@ -1296,6 +1299,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   ScanParams p = pin;   // (stacked images: the height is shortened below for a last, shorter stack)
   if constexpr (!STACKED) {   // lets the compiler drop what only stacked images need
     __builtin_assume(p.stacked == 0);
+    __builtin_assume(p.rb == kRB);
     __builtin_assume(p.S >= kHB + kCK - 1);
   }
   constexpr int CS = 64 >> kHBShift;     // 4 channel slots
@@ -1339,8 +1343,8 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   if constexpr (STACKED) {   // the last stack of the batch may hold fewer images
     const int nimg = p.Breal - b * p.ips < p.ips ? p.Breal - b * p.ips : p.ips;
     p.H = nimg * p.Himg;
-    p.nbands = (p.H + kRB - 1) / kRB;
-    p.rows_last = p.H - (p.nbands - 1) * kRB;
+    p.nbands = (p.H + p.rb - 1) / p.rb;
+    p.rows_last = p.H - (p.nbands - 1) * p.rb;
   }
   const int e_wg0 = eg * CW;
   const int slot = lane >> kHBShift, r = lane & (kHB - 1);
@@ -1405,9 +1409,9 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   const float g1 = r == 0 ? 1.f : 0.f;
 
   const uint32_t estep = (uint32_t)(p.flip ? -p.E : p.E) * (uint32_t)sizeof(T);   // one column further
-  const uint32_t wrap_adj = (uint32_t)(kRB * p.W - p.S) * estep;   // extra offset of a cell reached through a band change
+  const uint32_t wrap_adj = (uint32_t)(p.rb * p.W - p.S) * estep;   // extra offset of a cell reached through a band change
   const uint32_t pstep = (uint32_t)(p.flip ? -1 : 1) * (uint32_t)(3 * kN * sizeof(float));
-  const uint32_t pwrap_adj = (uint32_t)(kRB * p.W - p.S) * pstep;
+  const uint32_t pwrap_adj = (uint32_t)(p.rb * p.W - p.S) * pstep;
 
   // per block: where the lane (and the lane row whose sums this thread adds up) is, and what
   // depends on it
@@ -1751,6 +1755,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_bwd_split_kernel(const S
   constexpr bool SLICED = MODE == kModeSliced;
   const ScanParams& p = pin;
   __builtin_assume(p.stacked == 0);
+  __builtin_assume(p.rb == kRB);
   __builtin_assume(p.S >= kHB + kCK - 1);
   constexpr int NW = kSplitWaves, CW = NW;
   constexpr int SLOT = 3 * 64;           // float4s per wave in one exchange buffer
@@ -1832,9 +1837,9 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_bwd_split_kernel(const S
   const float g1 = r == 0 ? 1.f : 0.f;
   const float gb1 = r == kHB - 1 ? 1.f : 0.f;
   const uint32_t estep = (uint32_t)(p.flip ? -p.E : p.E) * (uint32_t)sizeof(T);
-  const uint32_t wrap_adj = (uint32_t)(kRB * p.W - p.S) * estep;
+  const uint32_t wrap_adj = (uint32_t)(p.rb * p.W - p.S) * estep;
   const uint32_t pstep = (uint32_t)(p.flip ? -1 : 1) * (uint32_t)(3 * kN * sizeof(float));
-  const uint32_t pwrap_adj = (uint32_t)(kRB * p.W - p.S) * pstep;
+  const uint32_t pwrap_adj = (uint32_t)(p.rb * p.W - p.S) * pstep;
 
   BlockPos bp;
   uint32_t cell_off0 = 0, f_off0 = 0;
@@ -2197,6 +2202,7 @@ static_assert(bwd_lds_bytes<float>() <= kLdsPerWorkgroup && bwd_lds_bytes<bf16_t
 struct Geometry {
   int HB, hb_shift, CS, nbands, nblk;
   int S, T_total, rows_last;         // stream stride, total steps, rows of the last band
+  int rb;                            // grid rows per band
   int fwd_ec, fwd_nw, fwd_wpb, fwd_bpb;   // forward: channels per lane, waves per workgroup, waves and workgroups per image
   int bwd_nw, bwd_wpb, bwd_bpb;      // backward: waves per workgroup, waves and workgroups (channel groups) per image
   bool fwd_split, bwd_split;         // the states of a channel split over the lanes (a wave per channel: m2d_fwd_split_kernel, m2d_bwd_split_kernel)
@@ -2246,32 +2252,36 @@ Geometry make_geometry(const m2d_desc* d) {
   g.hb_shift = kHBShift;
   g.CS = 64 / g.HB;
   const int groups = (d->E + kBwdWaves * g.CS - 1) / (kBwdWaves * g.CS);   // workgroups per image
-  // Grids of a single band whose height divides 14 (14x14, 7x7): a sweep spends as many steps
-  // filling and draining the 16-lane pipeline as working.  `ips` consecutive images of the batch
-  // are then stacked into one tall image whose bands do not depend on each other and swept back to
-  // back with stride S = W.  ips is chosen for the fewest steps over all rounds of workgroups
-  // (one workgroup per CU at a time).
+  // Grids of a single band (14x14, 7x7, 10x10 ...): a sweep spends as many steps filling and
+  // draining the 16-lane pipeline as working.  `ips` consecutive images of the batch are then
+  // stacked into one tall image whose bands do not depend on each other and swept back to back with
+  // stride S = W; a band holds as many whole images as fit 14 rows (two of 7 rows, one of 10, four
+  // of 3), so no image straddles two bands.  ips is chosen for the fewest steps over all rounds of
+  // workgroups (one workgroup per CU at a time).
   g.stacked = false; g.ips = 1; g.vB = d->B; g.vH = d->H;
-  if (d->H <= kRB && kRB % d->H == 0 && d->B >= 2) {
+  g.rb = kRB;
+  const int rb_stacked = d->H <= kRB ? kRB / d->H * d->H : kRB;
+  if (d->H <= kRB && d->B >= 2) {
     const int S = d->W > 7 ? d->W : 7;
     int64_t best = -1;
     for (int ips = 1; ips <= 64 && ips <= d->B; ++ips) {
       if ((int64_t)ips * d->H * d->W * d->E >= ((int64_t)1 << 30)) break;   // a stack is addressed like one image
       const int vB = (d->B + ips - 1) / ips;
-      const int nb = (ips * d->H + kRB - 1) / kRB;
+      const int nb = (ips * d->H + rb_stacked - 1) / rb_stacked;
       const int64_t rounds = ((int64_t)vB * groups + ncu - 1) / ncu;
       const int64_t cost = rounds * ((nb - 1) * S + d->W + kRB + 8);
       if (best < 0 || cost < best) { best = cost; g.ips = ips; }
     }
     if (g.ips > 1) {
       g.stacked = true;
+      g.rb = rb_stacked;
       g.vB = (d->B + g.ips - 1) / g.ips;
       g.vH = g.ips * d->H;
     }
   }
   const int B = g.vB, H = g.vH;   // what the kernels sweep
-  g.nbands = (H + kRB - 1) / kRB;
-  g.rows_last = H - (g.nbands - 1) * kRB;
+  g.nbands = (H + g.rb - 1) / g.rb;
+  g.rows_last = H - (g.nbands - 1) * g.rb;
   // A band's ghost reads the row that the band before stored S - 14 steps earlier, one block
   // ahead of its use: S - 14 >= 12 steps cover the store, the block-end barrier and the staging.
   // Wide grids run the bands back to back (S = W); narrow ones are padded.  Stacked images have no
@@ -2393,7 +2403,7 @@ void fill_common(ScanParams& sp, const m2d_desc* d, const Geometry& g) {
   sp.stacked = g.stacked ? 1 : 0; sp.ips = g.ips; sp.Himg = d->H; sp.Breal = d->B; sp.Hs = g.vH;
   sp.Ptot = (int64_t)d->B * d->H * d->W;
   sp.nbands = g.nbands; sp.nblk = g.nblk;
-  sp.S = g.S; sp.T_total = g.T_total; sp.rows_last = g.rows_last;
+  sp.S = g.S; sp.T_total = g.T_total; sp.rows_last = g.rows_last; sp.rb = g.rb;
   sp.magicS = (uint32_t)(((uint64_t)1 << 32) / (uint64_t)g.S);
   sp.sliced = g.sliced ? 1 : 0; sp.sl_nbb = g.nbb;
   sp.pa_slots = g.sliced ? g.nbands : 1;

@@ -111,7 +111,13 @@ SHAPES = [
     (900, 2, 5, 2),   # 2-row images, several to a band
     (1, 512, 512, 2), # 37 bands of one large image (sliced sweep at the size of the latency benchmark's second point)
     (2, 300, 260, 4), # 22 bands, two images
-    (303, 10, 3, 12), # over 256 unstacked images, even channel count (once asked for two channels per lane in fp32, which does not fit the LDS)
+    (303, 10, 3, 12), # over 256 images of 10 rows: one image per band of a stack, 4 lane rows idle (once asked for two channels per lane in fp32, which does not fit the LDS)
+    (601, 5, 9, 8),   # 5-row images stacked, two to a band (bands of 10 rows), last stack shorter
+    (530, 12, 12, 16), # 12x12 (the last stage of a 384x384 input) stacked, one image per band of 12 rows
+    (700, 3, 17, 4),  # 3-row images stacked, four to a band of 12 rows
+    (300, 13, 6, 2),  # 13 rows: one image per band
+    (400, 8, 8, 32),  # 8x8 stacked, one image per band of 8 rows, full workgroup of channels
+    (37, 5, 9, 8),    # few 5-row images: one stream per image
     (260, 20, 5, 64), # the same with two padded bands and a full workgroup of channels
     (5, 30, 9, 32),   # small batch, three bands: forward workgroups of 4 waves (16 channels each)
     (33, 57, 8, 48),  # the same with five bands in one padded stream, 99 workgroups of 4 waves
