@@ -181,7 +181,7 @@ struct ScanParams {
   const float *A2T, *A2L, *Df;      // A*log2(e) and D in fp32, (E,16) / (E)
   const float* zeros;               // 256 bytes of zeros (source for out-of-grid staging chunks)
   void *y, *dx, *ddT, *ddL;
-  float* ckpt;                      // [B][nblk][E][4][16][4]        state snapshots, one per block of steps: [q][row][w] = state sinv(4q+w)
+  float* ckpt;                      // [B][nblk][E][4][16][4]        state snapshots, one per block of steps: [q][row][w] = state sinv(4q+w); bf16 for 16-bit tensors
   float* top;                       // [nbands-1][B][W][E][16]       last row of each band (forward states)
   float* bot;                       // [nbands or 1][B][W][E][16]    first-row muT of a band, for the band above (adjoint)
   float* part;                      // [G][P][3][16]                 per-workgroup channel sums of d_C, d_BT, d_BL
@@ -677,13 +677,46 @@ __device__ __forceinline__ void bc_widen(const char* raw, char* buf, int wave, i
 }
 
 // ------------------------------------------------------------------------------------ forward
-// Store of a snapshot quad with the non-temporal hint: the data is read back once, by the backward
-// pass, long after it has left the caches, and as an ordinary store it costs the forward kernel
-// 0.02 ms at B=128, E=64, 56x56.
+// A snapshot quad: the four states of one state group of a lane, as the forward keeps them for the
+// backward.  fp32 tensors keep them as they are.  16-bit tensors keep them rounded to bf16: the
+// reference rounds every state of its hidden-state tensor to the tensors' type (wf_cuda.cu:40-69 writes
+// hs in scalar_t), here only the one state in four steps that a block restarts from is; the forward's
+// snapshot stores were a quarter of the traffic of the whole training step.
+// Stored with the non-temporal hint: the data is read back once, by the backward pass, long after it
+// has left the caches, and as an ordinary store it costs the forward kernel 0.02 ms at B=128, E=64, 56x56.
 typedef float f4v __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ void store_snapshot(float4* dst, float a, float b, float c, float d) {
-  const f4v v = {a, b, c, d};
-  __builtin_nontemporal_store(v, reinterpret_cast<f4v*>(dst));
+typedef unsigned int u2v __attribute__((ext_vector_type(2)));
+template <typename T> struct Snap;
+template <> struct Snap<float> {
+  typedef f4v quad;
+  static __device__ __forceinline__ void store(quad* dst, float a, float b, float c, float d) {
+    const f4v v = {a, b, c, d};
+    __builtin_nontemporal_store(v, dst);
+  }
+  static __device__ __forceinline__ float4 load(const quad* src) { return widen(*src); }
+  static __device__ __forceinline__ quad zero() { return f4v{0.f, 0.f, 0.f, 0.f}; }
+  static __device__ __forceinline__ float4 widen(quad v) { return make_float4(v.x, v.y, v.z, v.w); }
+};
+template <> struct Snap<bf16_t> {
+  typedef u2v quad;
+  static __device__ __forceinline__ void store(quad* dst, float a, float b, float c, float d) {
+    // (a vector conversion is one v_cvt_pk_bf16_f32 per pair; two scalar casts and an OR are four instructions)
+    typedef float f2v __attribute__((ext_vector_type(2)));
+    typedef __bf16 b2v __attribute__((ext_vector_type(2)));
+    const u2v v = {__builtin_bit_cast(uint32_t, __builtin_convertvector((f2v){a, b}, b2v)),
+                   __builtin_bit_cast(uint32_t, __builtin_convertvector((f2v){c, d}, b2v))};
+    __builtin_nontemporal_store(v, dst);
+  }
+  static __device__ __forceinline__ float4 load(const quad* src) { return widen(*src); }
+  static __device__ __forceinline__ quad zero() { return u2v{0u, 0u}; }
+  static __device__ __forceinline__ float4 widen(quad v) {
+    return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u));
+  }
+};
+// first quad of the snapshot of channel e before block m of image b: [b][block][E][4 state groups][16 lane rows]
+template <typename T>
+__device__ __forceinline__ typename Snap<T>::quad* snapshot_at(const ScanParams& p, int b, int m, int e) {
+  return reinterpret_cast<typename Snap<T>::quad*>(p.ckpt) + (((int64_t)b * p.nblk + m) * p.E + e) * (kN / 4 * kHB);
 }
 // Lanes are never masked in the forward: a grid row that is between bands, or a lane that is no
 // grid row, works on zero operands (its records come from the page of zeros), which keeps its
@@ -838,7 +871,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
 #pragma unroll
     for (int n = 0; n < kN; ++n) h[c][n] = 0.f;
   bool ck_mine = false;       // the lane stores a snapshot in the first step of the current block
-  float4* ckp = nullptr;      // where to
+  typename Snap<T>::quad* ckp = nullptr;      // where to
   auto step = [&](int k, const Ops& o) {
     const float offT = o.kk.x, offL = o.kk.y, cT = o.kk.z, cL = o.kk.w;
     const bool inr = ch_ok && ((bp.in_grid >> k) & 1u);
@@ -866,7 +899,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
         pin4(aL);
         __builtin_amdgcn_sched_barrier(0);
         if (CKPT && k == 0 && ck_mine)   // the four states as they are before this step
-          store_snapshot(ckp + (c * 4 + q) * kHB, h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)],
+          Snap<T>::store(ckp + (c * 4 + q) * kHB, h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)],
                          h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
@@ -935,12 +968,17 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     const Pos An = pos_after(p, A, kCK);
     BlockPos bpn;
     int celln;
-    if (WIDEN && direct) {   // the next block was worked out a block ago; its records are in `raw` already
+    if (WIDEN && direct && EC == 1) {   // the next block was worked out a block ago; its records are in `raw` already
       bpn = bpq;
       celln = cellq;
       bpq = block_pos(p, pos_after(p, An, kCK), r, rbands);
       cellq = cell_of(p, bpq.bnd0, r, bpq.col0);
       bc_raw_copy<NW>(p, pin.bcd, raw + rp * kRawBytes, b, bpq, cellq, wave, lane, m + 2 < m_hi);
+    } else if (WIDEN && direct) {   // two channels per lane: no registers to carry a block's positions in; worked out twice
+      bpn = block_pos(p, An, r, rbands);
+      celln = cell_of(p, bpn.bnd0, r, bpn.col0);
+      const BlockPos q2 = block_pos(p, pos_after(p, An, kCK), r, rbands);
+      bc_raw_copy<NW>(p, pin.bcd, raw + rp * kRawBytes, b, q2, cell_of(p, q2.bnd0, r, q2.col0), wave, lane, m + 2 < m_hi);
     } else {
       bpn = block_pos(p, An, r, rbands);
       celln = cell_of(p, bpn.bnd0, r, bpn.col0);
@@ -967,7 +1005,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
       Pos at; at.bnd = bp.bnd0; at.col = bp.col0;
       ck_mine = snapshot_lane(p, at, r, ch_ok);
       snapped = __any(ck_mine);
-      ckp = reinterpret_cast<float4*>(p.ckpt + ((((int64_t)b * p.nblk + m) * p.E + e0) * kN) * kHB) + r;
+      ckp = snapshot_at<T>(p, b, m, e0) + r;
     }
     const char* bufc = lds + cur * SG::kBytes;
     const char* bufn = lds + (cur ^ 1) * SG::kBytes;
@@ -1119,7 +1157,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_fwd_split_kernel(const S
   uint32_t cell_off0 = 0;
   float h[4] = {0.f, 0.f, 0.f, 0.f};
   bool ck_mine = false;
-  float4* ckp = nullptr;
+  typename Snap<T>::quad* ckp = nullptr;
 
   auto step = [&](const char* bufc, int k) {
     float xv = 0.f, dtv = 0.f, dlv = 0.f;
@@ -1151,7 +1189,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_fwd_split_kernel(const S
     for (int w = 0; w < 4; ++w) aL[w] = fexp2(__builtin_fmaf(dlv, a2l[w], offL));
     pin4(aL);
     __builtin_amdgcn_sched_barrier(0);
-    if (CKPT && k == 0 && ck_mine) store_snapshot(ckp, h[0], h[1], h[2], h[3]);   // the lane's states as they are before this step
+    if (CKPT && k == 0 && ck_mine) Snap<T>::store(ckp, h[0], h[1], h[2], h[3]);   // the lane's states as they are before this step
     float acc = 0.f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
@@ -1237,7 +1275,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_fwd_split_kernel(const S
       Pos at; at.bnd = bp.bnd0; at.col = bp.col0;
       ck_mine = snapshot_lane(p, at, r, ch_ok);
       snapped = __any(ck_mine);
-      ckp = reinterpret_cast<float4*>(p.ckpt + ((((int64_t)b * p.nblk + m) * p.E + e0) * kN) * kHB) + g * kHB + r;
+      ckp = snapshot_at<T>(p, b, m, e0) + g * kHB + r;
     }
     const char* bufc = lds + cur * SG::kBytes;
     // (uniform) stores that the wave is sure to issue in the first three steps, after the copies for the
@@ -1422,19 +1460,16 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   uint32_t cell_off0 = 0;       // byte offset in a (H,W,E) image of the lane's cell at the first step of the block
   uint32_t f_off0 = 0;          // byte offset in the channel-sum image of this thread's sum at the first step
   // state snapshot at the start of the block whose position A is given (zero for lanes that were not under way)
-  float cknext[kN];
+  // (kept as it comes from memory until the block starts: nothing waits for the loads before then)
+  typename Snap<T>::quad cknext[4];
   auto load_ckpt = [&](int mm, bool take) {   // take: the forward kept the lane's state before block mm
     if (mm == 0 || !take) {
 #pragma unroll
-      for (int n = 0; n < kN; ++n) cknext[n] = 0.f;
+      for (int q = 0; q < 4; ++q) cknext[q] = Snap<T>::zero();
     } else {
-      const float4* ck = reinterpret_cast<const float4*>(p.ckpt + ((((int64_t)b * p.nblk + mm) * p.E + e) * kN) * kHB) + r;
+      const typename Snap<T>::quad* ck = snapshot_at<T>(p, b, mm, e) + r;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const float4 v = ck[q * kHB];
-        cknext[sinv<PERM>(4 * q)] = v.x; cknext[sinv<PERM>(4 * q + 1)] = v.y;
-        cknext[sinv<PERM>(4 * q + 2)] = v.z; cknext[sinv<PERM>(4 * q + 3)] = v.w;
-      }
+      for (int q = 0; q < 4; ++q) cknext[q] = ck[q * kHB];
     }
   };
   auto pos_before = [&](Pos Q) {   // kCK positions earlier
@@ -1474,7 +1509,11 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
     const char* bufc = lds + cur * SG::kBytes;
     float ck0[kN];
 #pragma unroll
-    for (int n = 0; n < kN; ++n) ck0[n] = cknext[n];
+    for (int q = 0; q < 4; ++q) {
+      const float4 v = Snap<T>::widen(cknext[q]);
+      ck0[sinv<PERM>(4 * q)] = v.x; ck0[sinv<PERM>(4 * q + 1)] = v.y;
+      ck0[sinv<PERM>(4 * q + 2)] = v.z; ck0[sinv<PERM>(4 * q + 3)] = v.w;
+    }
     // the block before: where the lane's row will be is also what the lane's copies fetch
     const Pos Aprev = pos_before(A);
     const BlockPos bpn = block_pos(p, Aprev, r, rbands);
@@ -1843,11 +1882,10 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_bwd_split_kernel(const S
 
   BlockPos bp;
   uint32_t cell_off0 = 0, f_off0 = 0;
-  float cknext[4];
+  typename Snap<T>::quad cknext = Snap<T>::zero();
   auto load_ckpt = [&](int mm, bool take) {   // take: the forward kept the lane's state before block mm
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (mm != 0 && take) v = (reinterpret_cast<const float4*>(p.ckpt + ((((int64_t)b * p.nblk + mm) * p.E + e) * kN) * kHB) + g * kHB)[r];
-    cknext[0] = v.x; cknext[1] = v.y; cknext[2] = v.z; cknext[3] = v.w;
+    cknext = Snap<T>::zero();
+    if (mm != 0 && take) cknext = *(snapshot_at<T>(p, b, mm, e) + g * kHB + r);
   };
   auto pos_before = [&](Pos Q) {
     Q.col -= kCK;
@@ -1884,8 +1922,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_bwd_split_kernel(const S
     const int t0 = m * kCK;
     const char* bufc = lds + cur * SG::kBytes;
     float hb[kCK + 1][4], gT[kCK][4], gL[kCK][4];
-#pragma unroll
-    for (int w = 0; w < 4; ++w) hb[0][w] = cknext[w];
+    { const float4 v = Snap<T>::widen(cknext); hb[0][0] = v.x; hb[0][1] = v.y; hb[0][2] = v.z; hb[0][3] = v.w; }
     const Pos Aprev = pos_before(A);
     const BlockPos bpn = block_pos(p, Aprev, r, rbands);
     const int celln = cell_of(p, bpn.bnd0, r, bpn.col0);
@@ -2369,7 +2406,7 @@ Geometry make_geometry(const m2d_desc* d) {
   g.packed_bc = (d->flags & M2D_FLAG_PACKED_BC) != 0;   // the caller brings the records: nothing to reserve
   // (16-bit tensors are widened inside the scan kernels, nothing to reserve either)
   g.bc_bytes = (g.packed_bc || d->dtype == M2D_BF16) ? 0 : align_up(sizeof(float) * P * 48);
-  g.ckpt_diag_bytes = align_up(sizeof(float) * (size_t)B * g.nblk * d->E * kN * g.HB);
+  g.ckpt_diag_bytes = align_up((d->dtype == M2D_BF16 ? 2 : sizeof(float)) * (size_t)B * g.nblk * d->E * kN * g.HB);   // (16-bit tensors: bf16 snapshots)
   const bool rows = g.nbands > 1 && !g.stacked;   // boundary rows travel between bands
   g.top_bytes = rows ? align_up(sizeof(float) * (size_t)(g.nbands - 1) * B * d->W * d->E * kN) : 0;
   g.bot_bytes = rows ? align_up(sizeof(float) * (size_t)(g.sliced ? g.nbands : 1) * B * d->W * d->E * kN) : 0;
