@@ -1507,13 +1507,6 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   for (int m = m_hi - 1; m >= m_lo; --m) {
     const int t0 = m * kCK;
     const char* bufc = lds + cur * SG::kBytes;
-    float ck0[kN];
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const float4 v = Snap<T>::widen(cknext[q]);
-      ck0[sinv<PERM>(4 * q)] = v.x; ck0[sinv<PERM>(4 * q + 1)] = v.y;
-      ck0[sinv<PERM>(4 * q + 2)] = v.z; ck0[sinv<PERM>(4 * q + 3)] = v.w;
-    }
     // the block before: where the lane's row will be is also what the lane's copies fetch
     const Pos Aprev = pos_before(A);
     const BlockPos bpn = block_pos(p, Aprev, r, rbands);
@@ -1541,13 +1534,16 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
     for (int half = 0; half < 2; ++half) {
       float hb[kCK + 1][8];
       float gT_last[8], gL_last[8];   // gates of the last step: the adjoint starts with them
+      // the states before the block: quad mg of the snapshot holds the states fold_state(mg, 0..3) in this order
+      // (widened here, half by half: until then the snapshot stays as it came from memory)
+      static_assert(sinv<PERM>(4 * 2 + 1) == fold_state(2, 1) && sinv<PERM>(4 * 3 + 2) == fold_state(3, 2), "snapshot quads are state groups");
 #pragma unroll
-      for (int mgl = 0; mgl < 2; ++mgl)
+      for (int mgl = 0; mgl < 2; ++mgl) {
+        const float4 v = Snap<T>::widen(cknext[2 * half + mgl]);
+        hb[0][4 * mgl + 0] = v.x; hb[0][4 * mgl + 1] = v.y; hb[0][4 * mgl + 2] = v.z; hb[0][4 * mgl + 3] = v.w;
 #pragma unroll
-        for (int qi = 0; qi < 4; ++qi) {
-          hb[0][4 * mgl + qi] = ck0[fold_state(2 * half + mgl, qi)];
-          gT_last[4 * mgl + qi] = 0.f; gL_last[4 * mgl + qi] = 0.f;
-        }
+        for (int qi = 0; qi < 4; ++qi) { gT_last[4 * mgl + qi] = 0.f; gL_last[4 * mgl + qi] = 0.f; }
+      }
       // ---- recompute the states of the block
 #pragma unroll
       for (int k = 0; k < kCK; ++k) {
