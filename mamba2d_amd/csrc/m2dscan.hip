@@ -2332,7 +2332,7 @@ Geometry make_geometry(const m2d_desc* d) {
   // per band), all in one launch, and band k trails band k-1 by kLinkLag blocks of steps.
   g.sliced = !g.stacked && g.nbands >= 4 && (int64_t)B * groups <= ncu / 4;
   if (g.sliced && g.nbands == 4) {
-    // Four bands (more bands favour the sliced sweep again: 84x84 measured) and a batch that fills half the device with workgroups of 4 waves, but not with
+    // Four bands (more bands favour the linked sweep again: 84x84 measured) and a batch that fills half the device with workgroups of 4 waves, but not with
     // every band under way on workgroups of its own: one stream per image on workgroups of 4 waves
     // is then the faster schedule (56x56, 64 images of 32 channels: 0.99 -> 0.93 ms forward+backward).
     int s_sl = (d->W + kHB - 1 + kCK - 1) / kCK * kCK;

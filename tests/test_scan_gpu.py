@@ -103,7 +103,7 @@ SHAPES = [
     (9, 7, 7, 6),     # 7x7 stage shape, channels not filling the second wave
     (5, 2, 2, 2),     # smallest legal grid
     (2, 28, 28, 8),   # two bands run back to back in one stream (W >= 26)
-    (1, 56, 56, 4),   # stage-1 spatial size: four bands, one image -> sequence of launches
+    (1, 56, 56, 4),   # stage-1 spatial size: four bands, one image: every band on workgroups of its own (linked sweep)
     (2, 33, 40, 2),   # three bands back to back, last one 5 rows
     (1, 10, 60, 2),   # wide single band
     (1, 60, 10, 3),   # tall and narrow: five padded bands, odd channel count
@@ -112,12 +112,12 @@ SHAPES = [
     (1, 64, 17, 10),  # channels not a multiple of the workgroup
     (1, 40, 4, 3),    # three bands narrower than the pipeline is deep
     (2, 31, 8, 2),    # three bands in one padded stream
-    (1, 150, 90, 8),  # 11 bands, one image: every band on workgroups of its own, swept by a sequence of launches
-    (70, 56, 30, 4),  # four bands back to back, more images than the sliced sweep takes
+    (1, 150, 90, 8),  # 11 bands, one image: every band on workgroups of its own inside one launch (linked sweep)
+    (70, 56, 30, 4),  # four bands back to back, more images than the linked sweep takes
     (301, 7, 7, 4),   # 7x7 images stacked two to a band, last stack of one image
     (600, 14, 14, 4), # 14x14 images stacked three to a sweep, bands back to back with stride 14
     (900, 2, 5, 2),   # 2-row images, several to a band
-    (1, 512, 512, 2), # 37 bands of one large image (sliced sweep at the size of the latency benchmark's second point)
+    (1, 512, 512, 2), # 37 bands of one large image (linked sweep at the size of the latency benchmark's second point)
     (2, 300, 260, 4), # 22 bands, two images
     (303, 10, 3, 12), # over 256 images of 10 rows: one image per band of a stack, 4 lane rows idle (once asked for two channels per lane in fp32, which does not fit the LDS)
     (601, 5, 9, 8),   # 5-row images stacked, two to a band (bands of 10 rows), last stack shorter
@@ -132,7 +132,7 @@ SHAPES = [
     (4, 20, 11, 50),  # the same without x-staging, last workgroup partly filled
     (3, 30, 28, 32),  # workgroups of 4 waves, three bands back to back (stride = width)
     (70, 44, 26, 32), # the same with four bands and 140 workgroups
-    (1, 60, 40, 32),  # sliced sweep (five bands of one image) on forward workgroups of 4 waves
+    (1, 60, 40, 32),  # linked sweep (five bands of one image)
     (2, 100, 33, 48), # the same, eight bands of two images, three workgroups of 16 channels per band
     (128, 4, 3, 128), # 512 workgroups with one channel per lane, 256 with two: the bf16 forward takes two channels per lane
     (256, 17, 4, 64), # the same from the batch side, two padded bands

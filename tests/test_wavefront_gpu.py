@@ -269,7 +269,7 @@ def test_no_checkpoints_are_kept_under_no_grad(wf, monkeypatch):
 def test_entry_point_replays_from_a_graph(wf, shape, dtype):
     """The library allocates nothing and never synchronises, so a caller can capture forward and backward
     in a HIP graph (here through torch).  Every replay, with eager work and synchronisations between the
-    replays, must give the bits of an eager run on the same inputs; the first shape is the sliced sweep
+    replays, must give the bits of an eager run on the same inputs; the first shape is the linked sweep
     of one image (a sequence of 40 launches per pass)."""
     say(f"\ncase graph {shape} {dtype}")
     B, H, W, E = shape

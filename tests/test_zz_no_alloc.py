@@ -47,7 +47,7 @@ def test_two_calls_in_a_row_second_smaller(cscan):
     # four bands back to back: uses the set-up area, the packed B/C records and the band boundary rows
     one_call(cabi, cscan, 4, 56, 56, 64, torch.bfloat16, seed=11)
     one_call(cabi, cscan, 2, 20, 9, 8, torch.float32, seed=12)
-    # sliced sweep (one image, five bands: state carried from launch to launch), then stacked images
+    # linked sweep (one image, five bands on workgroups of their own), then stacked images
     one_call(cabi, cscan, 1, 70, 50, 16, torch.float32, seed=13, flip=True)
     one_call(cabi, cscan, 9, 7, 7, 6, torch.bfloat16, seed=14)
 
