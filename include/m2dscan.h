@@ -113,8 +113,9 @@ int m2d_desc_check(const m2d_desc* desc);
  * Returns 0 for an invalid descriptor. */
 size_t m2d_scan_workspace_bytes(const m2d_desc* desc, int pass, int have_ckpt);
 
-/* Bytes of the checkpoint buffer (anti-diagonal state snapshots every few steps plus
- * band-boundary rows; linear in H*W, about 1/4 of the full state tensor in fp32). */
+/* Bytes of the checkpoint buffer (anti-diagonal state snapshots every 4 steps plus band-boundary
+ * rows; linear in H*W, about 1/4 of the reference's hs tensor: the snapshots have the width of the
+ * tensors' type, fp32 or bf16, as every state of hs has in the reference, wf_cuda.cu:5,59-67). */
 size_t m2d_scan_ckpt_bytes(const m2d_desc* desc);
 
 /* Fused forward:  y = sum_n h*C + x*D  with h from the recurrence of wf_cuda.cu:40-69.

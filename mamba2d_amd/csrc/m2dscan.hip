@@ -2415,7 +2415,7 @@ Geometry make_geometry(const m2d_desc* d) {
   return g;
 }
 
-// checkpoint buffer: [state snapshots][band boundary rows][widened B,C (bf16 input only)]
+// checkpoint buffer: [state snapshots][band boundary rows][packed B,C (fp32 tensors only)]
 size_t ckpt_bytes_of(const Geometry& g) { return g.ckpt_diag_bytes + g.top_bytes + g.bc_bytes; }
 
 size_t workspace_bytes_of(const Geometry& g, int pass, int have_ckpt) {
@@ -2576,7 +2576,7 @@ int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   float* prep = reinterpret_cast<float*>(w);
   w += g.prep_bytes;
   uint32_t* link_words = reinterpret_cast<uint32_t*>(w); w += g.link_bytes;
-  char* keep = ckpt ? static_cast<char*>(ckpt) + g.ckpt_diag_bytes : w;   // [top][widened B,C]
+  char* keep = ckpt ? static_cast<char*>(ckpt) + g.ckpt_diag_bytes : w;   // [top][packed B,C]
   sp.ckpt = ckpt ? static_cast<float*>(ckpt) : nullptr;
   sp.top = reinterpret_cast<float*>(keep);
   int rc = launch_prep<T>(sp, d, g, AT, AL, D, prep, link_words, st);
