@@ -2330,7 +2330,8 @@ Geometry make_geometry(const m2d_desc* d) {
   // Few images with many bands leave most of the device idle when each image is one sequential
   // stream.  Then every band gets workgroups of its own (a padded stream, one window of S steps
   // per band), all in one launch, and band k trails band k-1 by kLinkLag blocks of steps.
-  g.sliced = !g.stacked && g.nbands >= 4 && (int64_t)B * groups <= ncu / 4;
+  // (two or three bands: only where a band is much longer than the 28 steps by which a band trails its neighbour)
+  g.sliced = !g.stacked && (g.nbands >= 4 || (g.nbands >= 2 && d->W >= 64)) && (int64_t)B * groups <= ncu / 4;
   if (g.sliced && g.nbands == 4) {
     // Four bands (more bands favour the linked sweep again: 84x84 measured) and a batch that fills half the device with workgroups of 4 waves, but not with
     // every band under way on workgroups of its own: one stream per image on workgroups of 4 waves

@@ -126,6 +126,8 @@ SHAPES = [
     (300, 13, 6, 2),  # 13 rows: one image per band
     (400, 8, 8, 32),  # 8x8 stacked, one image per band of 8 rows, full workgroup of channels
     (37, 5, 9, 8),    # few 5-row images: one stream per image
+    (1, 28, 70, 8),   # two long bands of one image: linked sweep
+    (2, 40, 100, 4),  # three long bands of two images: linked sweep
     (260, 20, 5, 64), # the same with two padded bands and a full workgroup of channels
     (5, 30, 9, 32),   # small batch, three bands: forward workgroups of 4 waves (16 channels each)
     (33, 57, 8, 48),  # the same with five bands in one padded stream, 99 workgroups of 4 waves
