@@ -1743,8 +1743,10 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
       }
     }
     __syncthreads();
-    // every wave has waited (before the last stores of this block) for all it had issued: the blocks swept before this one are in memory
-    if constexpr (SLICED) link.publish((uint32_t)(m_hi - 1 - m));
+    // Every wave has waited, before the last adjoint step of this block, for all it had issued: the blocks swept
+    // before this one are in memory, and so are the rows this block stored in its steps 3, 2 and 1.  The band above
+    // needs, of the newest block it is told about, the steps 3 and 2 only (link_need_bwd), so this block counts.
+    if constexpr (SLICED) link.publish((uint32_t)(m_hi - m));
     A = Aprev;
     bp = bpn;
     cell0 = celln;
@@ -2065,7 +2067,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_bwd_split_kernel(const S
       }
     }
     __syncthreads();
-    if constexpr (SLICED) link.publish((uint32_t)(m_hi - 1 - m));
+    if constexpr (SLICED) link.publish((uint32_t)(m_hi - m));   // (this block counts: see m2d_bwd_kernel)
     A = Aprev;
     bp = bpn;
     cell0 = celln;
