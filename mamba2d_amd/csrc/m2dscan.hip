@@ -1012,9 +1012,20 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     // (uniform) some lane writes y at each of the first three steps: the wave issues at least
     // three stores between the copies for the next block and the barrier that ends this one
     const bool y_thrice = WRITE_Y && __any(ch_ok && (bp.in_grid & 7u) == 7u);
+    // (uniform, linked sweep) lane 14 stores the band's last row at each of the first three steps
+    const bool top_thrice = SLICED && __any(ch_ok && (bp.in_grid & 7u) == 7u && r == kRB && bp.kw >= kCK && bp.bnd0 + 1 < p.nbands);
     auto next_block_landed = [&] {
       // the stores issued since (snapshot, y) need not have completed, only the copies before them
-      if (snapped) {
+      if constexpr (SLICED) {
+        // Linked sweep: the band below needs, of the newest block it is told about, the last row of the steps 0 and 1
+        // only (link_need_fwd).  Only what is issued after the row of step 1 stays in flight (y of step 1, row and
+        // y of step 2), so that this block counts as done at its end.
+        if (top_thrice) {
+          if (y_thrice) staging_landed_behind<4 * EC + 2>(); else staging_landed_behind<4 * EC>();
+        } else {
+          if (y_thrice) staging_landed_behind<2>(); else staging_landed();
+        }
+      } else if (snapped) {
         if (y_thrice) staging_landed_behind<4 * EC + 3>(); else staging_landed_behind<4 * EC>();
       } else {
         if (y_thrice) staging_landed_behind<3>(); else staging_landed();
@@ -1034,8 +1045,8 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
           // barrier, and no wave reads the current buffer any more.
           next_block_landed();
           __syncthreads();
-          // every wave has waited for what it issued before this block's copies: the blocks before this one are in memory
-          if constexpr (SLICED) link.publish((uint32_t)(m - m_lo));
+          // every wave has waited for the rows it stored at the steps 0 and 1 of this block
+          if constexpr (SLICED) link.publish((uint32_t)(m - m_lo + 1));
           if (!last) fetch(bufn, 0, ahead);
         }
         step(k, now);   // also past the end of the sweep (last block): zero operands like any position off the grid, nothing stored
@@ -1051,7 +1062,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
         step(k, opsA);
       }
       __syncthreads();
-      if constexpr (SLICED) link.publish((uint32_t)(m - m_lo));
+      if constexpr (SLICED) link.publish((uint32_t)(m - m_lo + 1));
     }
     cur ^= 1;
     A = An;
@@ -1284,14 +1295,18 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_fwd_split_kernel(const S
     const bool on3 = ch_ok && (bp.in_grid & 7u) == 7u;
     const bool y_thrice = WRITE_Y && __any(on3);
     const bool top_thrice = p.nbands > 1 && __any(on3 && r == kRB && bp.kw >= kCK && bp.bnd0 + 1 < p.nbands);
-    const int younger = (snapped ? 1 : 0) + (y_thrice ? 3 : 0) + (top_thrice ? 3 : 0);
+    // Linked sweep: the band below needs, of the newest block it is told about, the boundary rows of the steps 0 and
+    // 1 only (link_need_fwd).  With just the stores issued after those of step 1 left in flight (y of step 1, row and
+    // y of step 2), this block counts as done at its end.
+    const int younger = SLICED ? (y_thrice ? 2 : 0) + (top_thrice ? 1 : 0)
+                               : (snapped ? 1 : 0) + (y_thrice ? 3 : 0) + (top_thrice ? 3 : 0);
 #pragma unroll
     for (int k = 0; k < kCK; ++k) {
       if (k == kCK - 1) staging_landed_behind_n(younger);
       step(bufc, k);
     }
     __syncthreads();
-    if constexpr (SLICED) link.publish((uint32_t)(m - m_lo));
+    if constexpr (SLICED) link.publish((uint32_t)(m - m_lo + 1));
     cur ^= 1;
     A = An;
     bp = bpn;
