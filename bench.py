@@ -347,6 +347,11 @@ def main():
     ap.add_argument("--workload", default="cfg1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-ckpt", action="store_true", help="rebuild checkpoints inside the backward")
+    ap.add_argument("--ckpt-interval", type=int, default=0, choices=(0, 4, 8, 16),
+                    help="steps between the state snapshots the forward keeps (0 or 4: the default; 8, 16: fewer "
+                         "snapshots, and the backward replays the forward in between)")
+    ap.add_argument("--dtype", default=None, choices=("f32", "bf16"),
+                    help="tensor type of a single-scan workload (default: the workload's own)")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (a known-size kernel to scale rocprofv3's "
                          "FETCH_SIZE / WRITE_SIZE readings by)")
@@ -361,6 +366,7 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     from mamba2d_amd import cabi, wavefront
+    wavefront.CKPT_INTERVAL = cabi.CKPT_INTERVAL = args.ckpt_interval
 
     if args.workload == "cfg3":
         backbone_inference(args)
@@ -372,6 +378,7 @@ def main():
         stage_sequence(args)
         return
     B, E, H, W, dts = WORKLOADS[args.workload]
+    dts = args.dtype or dts
     dtype = torch.bfloat16 if dts == "bf16" else torch.float32
     if args.no_ckpt:
         wavefront.SAVE_CHECKPOINTS = False
@@ -453,7 +460,8 @@ def main():
         "dtype": "bf16 in/out, f32 state" if dts == "bf16" else "f32",
         "data": "synthetic",
         "config": {"workload": f"{args.workload}: single scan fwd+bwd, B={B} E={E} {H}x{W} N={N}",
-                   "checkpoints": "saved by forward" if not args.no_ckpt else "rebuilt in backward"},
+                   "checkpoints": ("saved by forward" if not args.no_ckpt else "rebuilt in backward") +
+                                  (f", a snapshot every {args.ckpt_interval} steps" if args.ckpt_interval > 4 else "")},
         "fwd_ms": round(fwd_ms, 4),
         "fwd_bwd_ms": round(step_ms, 4),
         "wall_ms_per_step": round(t_wall, 4),

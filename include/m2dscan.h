@@ -59,7 +59,12 @@ typedef struct m2d_desc {
   int32_t B, H, W, E, N;
   int32_t dtype;              /* m2d_dtype */
   int32_t flags;
-  int32_t reserved;           /* must be 0 */
+  int32_t ckpt_interval;      /* steps between the state snapshots that m2d_scan_fwd keeps for m2d_scan_bwd:
+                                 0 (the default) or 4, 8, 16.  A longer interval shrinks the snapshot part of
+                                 the checkpoint buffer in proportion; the backward then replays the forward
+                                 over the steps in between (4 or 12 of every 8 or 16) before it sweeps them.
+                                 The forward and the backward of one problem must use the same value.
+                                 Ignored by the m2d_proj_* entry points. */
 } m2d_desc;
 
 #define M2D_FLAG_FLIP 1
@@ -113,9 +118,10 @@ int m2d_desc_check(const m2d_desc* desc);
  * Returns 0 for an invalid descriptor. */
 size_t m2d_scan_workspace_bytes(const m2d_desc* desc, int pass, int have_ckpt);
 
-/* Bytes of the checkpoint buffer (anti-diagonal state snapshots every 4 steps plus band-boundary
- * rows; linear in H*W, about 1/4 of the reference's hs tensor: the snapshots have the width of the
- * tensors' type, fp32 or bf16, as every state of hs has in the reference, wf_cuda.cu:5,59-67). */
+/* Bytes of the checkpoint buffer (anti-diagonal state snapshots every desc->ckpt_interval steps, 4 by
+ * default, plus band-boundary rows; linear in H*W, at the default about 1/4 of the reference's hs tensor:
+ * the snapshots have the width of the tensors' type, fp32 or bf16, as every state of hs has in the
+ * reference, wf_cuda.cu:5,59-67). */
 size_t m2d_scan_ckpt_bytes(const m2d_desc* desc);
 
 /* Fused forward:  y = sum_n h*C + x*D  with h from the recurrence of wf_cuda.cu:40-69.

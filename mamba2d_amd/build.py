@@ -10,6 +10,7 @@ from __future__ import annotations
 
 import glob
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -37,6 +38,12 @@ SOURCES = {
     "m2dblock.hip": [],
 }
 
+
+# Kernels that may keep a few values in scratch memory, and how many bytes per lane.  Only the backward kernel of
+# 8 waves in its replaying form (m2d_bwd_kernel<..., 8, true>: a checkpoint interval of 8 or 16 steps, not the
+# default): the same sweep as the default kernel, which fills all 256 registers, plus the addresses of the replay.
+# It reloads two to nine values a few times per block of steps; every other kernel must not spill at all.
+SPILL_ALLOWANCE = [(re.compile(r"m2d_bwd_kernelI\w*Li8ELb1EEEv"), 64)]
 
 def build_lib(verbose: bool = True) -> str:
     """Compiles the HIP sources into libm2dscan.so.  The device assembly of the same compile is
@@ -69,7 +76,8 @@ def build_lib(verbose: bool = True) -> str:
             if bad:
                 raise RuntimeError("hazard between inline-assembly DPP instructions and their producers:\n" +
                                    "\n".join(f"  {k}: {p}  ->  {c}" for k, p, c in bad[:8]))
-            spills = asmcheck.spills_in_file(path)
+            spills = [(k, n) for k, n in asmcheck.spills_in_file(path)
+                      if not any(pat.search(k) and n <= cap for pat, cap in SPILL_ALLOWANCE)]
             if spills:
                 raise RuntimeError("kernels that spill registers to scratch memory:\n" +
                                    "\n".join(f"  {k}: {n} bytes per lane" for k, n in spills[:8]))

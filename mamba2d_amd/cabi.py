@@ -30,7 +30,7 @@ EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspac
 
 
 class Desc(ctypes.Structure):
-    _fields_ = [(k, ctypes.c_int32) for k in ("B", "H", "W", "E", "N", "dtype", "flags", "reserved")]
+    _fields_ = [(k, ctypes.c_int32) for k in ("B", "H", "W", "E", "N", "dtype", "flags", "ckpt_interval")]
 
 
 class M2DError(RuntimeError):
@@ -124,6 +124,10 @@ def check(code: int) -> None:
 # M2D_FLAG_SPLIT_STATES or M2D_FLAG_WHOLE_STATES to override the library's choice of lane layout in
 # scan_fwd / scan_bwd (0: the library decides); the tests run every case all three ways.
 SCHEDULE_HINT = 0
+# Steps between the state snapshots that the forward keeps for the backward (m2d_desc.ckpt_interval): 0 or 4
+# (the default), 8 or 16.  Longer intervals shrink the checkpoint buffer and make the backward replay the
+# forward over the steps in between.  Set once, before the forward of a problem, and leave until its backward.
+CKPT_INTERVAL = 0
 
 
 def make_desc(x: torch.Tensor, N: int, flip: bool = False) -> Desc:
@@ -134,7 +138,7 @@ def make_desc(x: torch.Tensor, N: int, flip: bool = False) -> Desc:
         dt = M2D_BF16
     else:
         raise TypeError(f"m2dscan supports float32 and bfloat16, got {x.dtype}")
-    return Desc(B, H, W, E, N, dt, (M2D_FLAG_FLIP if flip else 0) | SCHEDULE_HINT, 0)
+    return Desc(B, H, W, E, N, dt, (M2D_FLAG_FLIP if flip else 0) | SCHEDULE_HINT, CKPT_INTERVAL)
 
 
 def _ptr(t):
@@ -185,11 +189,11 @@ def _check_links(d, ws, dev):
             raise RuntimeError("m2dscan: a workgroup of the linked sweep gave up waiting for its neighbour")
 
 
-def scan_plan(B, H, W, E, dtype, pass_=M2D_PASS_FWD, N=16, flags=None):
+def scan_plan(B, H, W, E, dtype, pass_=M2D_PASS_FWD, N=16, flags=None, ckpt_interval=None):
     """The library's one-line description of how it will run a pass of this problem (m2d_scan_plan)."""
     dt = M2D_F32 if dtype in (torch.float32, "f32") else M2D_BF16
-    d = Desc(B, H, W, E, N, dt, SCHEDULE_HINT if flags is None else flags, 0)
-    buf = ctypes.create_string_buffer(256)
+    d = Desc(B, H, W, E, N, dt, SCHEDULE_HINT if flags is None else flags, CKPT_INTERVAL if ckpt_interval is None else ckpt_interval)
+    buf = ctypes.create_string_buffer(320)
     check(lib.m2d_scan_plan(ctypes.byref(d), pass_, buf, len(buf)))
     return buf.value.decode()
 

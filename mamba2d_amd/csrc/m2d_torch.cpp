@@ -23,7 +23,7 @@ namespace {
 using at::Tensor;
 
 m2d_desc describe(const Tensor& x, const Tensor& AT, bool flip, bool raw_params = false, bool packed_bc = false,
-                  bool dpre = false) {
+                  bool dpre = false, int64_t ckpt_interval = 0) {
   TORCH_CHECK(x.dim() == 4, "m2dscan: x must be (B,H,W,E), got ", x.sizes());
   TORCH_CHECK(AT.dim() == 2, "m2dscan: AT must be (E,N), got ", AT.sizes());
   m2d_desc d{};
@@ -37,6 +37,9 @@ m2d_desc describe(const Tensor& x, const Tensor& AT, bool flip, bool raw_params 
   else TORCH_CHECK(false, "m2dscan: float32 and bfloat16 are supported, got ", x.scalar_type());
   d.flags = (flip ? M2D_FLAG_FLIP : 0) | (raw_params ? M2D_FLAG_RAW_PARAMS : 0) | (packed_bc ? M2D_FLAG_PACKED_BC : 0) |
             (dpre ? M2D_FLAG_DPRE : 0);
+  TORCH_CHECK(ckpt_interval == 0 || ckpt_interval == 4 || ckpt_interval == 8 || ckpt_interval == 16,
+              "m2dscan: ckpt_interval must be 0, 4, 8 or 16, got ", ckpt_interval);
+  d.ckpt_interval = static_cast<int32_t>(ckpt_interval);
   return d;
 }
 
@@ -86,8 +89,9 @@ Tensor bytes(size_t n, const Tensor& like) {
 
 std::tuple<Tensor, Tensor> scan_fwd(const Tensor& x, const Tensor& dT, const Tensor& dL, const Tensor& AT,
                                     const Tensor& AL, const Tensor& BT, const Tensor& BL, const Tensor& C,
-                                    const Tensor& D, bool save_ckpt, bool flip, bool raw_params, bool packed_bc) {
-  const m2d_desc d = describe(x, AT, flip, raw_params, packed_bc);
+                                    const Tensor& D, bool save_ckpt, bool flip, bool raw_params, bool packed_bc,
+                                    int64_t ckpt_interval) {
+  const m2d_desc d = describe(x, AT, flip, raw_params, packed_bc, false, ckpt_interval);
   expect_all(d, x, dT, dL, AT, AL, BT, BL, C, D);
   check(m2d_desc_check(&d));
   c10::DeviceGuard guard(x.device());
@@ -104,8 +108,9 @@ std::tuple<Tensor, Tensor> scan_fwd(const Tensor& x, const Tensor& dT, const Ten
 
 std::vector<Tensor> scan_bwd(const Tensor& x, const Tensor& dT, const Tensor& dL, const Tensor& AT, const Tensor& AL,
                              const Tensor& BT, const Tensor& BL, const Tensor& C, const Tensor& D, const Tensor& dy,
-                             const Tensor& ckpt, bool flip, bool raw_params, bool packed_bc, bool dpre) {
-  const m2d_desc d = describe(x, AT, flip, raw_params, packed_bc, dpre);
+                             const Tensor& ckpt, bool flip, bool raw_params, bool packed_bc, bool dpre,
+                             int64_t ckpt_interval) {
+  const m2d_desc d = describe(x, AT, flip, raw_params, packed_bc, dpre, ckpt_interval);
   expect_all(d, x, dT, dL, AT, AL, BT, BL, C, D);
   expect(dy, "dy", x, x.sizes());
   check(m2d_desc_check(&d));
@@ -453,9 +458,10 @@ int64_t abi_version() { return m2d_version(); }
 
 TORCH_LIBRARY(m2dscan, m) {
   m.def("scan_fwd(Tensor x, Tensor deltaT, Tensor deltaL, Tensor AT, Tensor AL, Tensor BT, Tensor BL, Tensor C, "
-        "Tensor D, bool save_ckpt, bool flip, bool raw_params=False, bool packed_bc=False) -> (Tensor, Tensor)");
+        "Tensor D, bool save_ckpt, bool flip, bool raw_params=False, bool packed_bc=False, int ckpt_interval=0) -> (Tensor, Tensor)");
   m.def("scan_bwd(Tensor x, Tensor deltaT, Tensor deltaL, Tensor AT, Tensor AL, Tensor BT, Tensor BL, Tensor C, "
-        "Tensor D, Tensor dy, Tensor ckpt, bool flip, bool raw_params=False, bool packed_bc=False, bool dpre=False) -> Tensor[]");
+        "Tensor D, Tensor dy, Tensor ckpt, bool flip, bool raw_params=False, bool packed_bc=False, bool dpre=False, "
+        "int ckpt_interval=0) -> Tensor[]");
   m.def("proj_fwd(Tensor x, Tensor x_proj_w, Tensor dt_projT_w, Tensor dt_projT_b, Tensor dt_projL_w, Tensor dt_projL_b, "
         "int d_state, bool round_weights, bool packed_bc=False) -> Tensor[]");
   m.def("proj_bwd(Tensor x, Tensor lowrank, Tensor deltaT, Tensor deltaL, Tensor x_proj_w, Tensor dt_projT_w, "

@@ -1124,7 +1124,7 @@ struct ProjGeometry {
 int check_proj(const m2d_desc* d, int R) {
   if (!d) return M2D_ERR_NULL_POINTER;
   if (d->B < 1 || d->H < 1 || d->W < 1 || d->E < 1 || d->N < 1 || R < 1) return M2D_ERR_BAD_SHAPE;
-  if (d->N != kN || (d->dtype != M2D_F32 && d->dtype != M2D_BF16) || d->reserved != 0) return M2D_ERR_UNSUPPORTED;
+  if (d->N != kN || (d->dtype != M2D_F32 && d->dtype != M2D_BF16)) return M2D_ERR_UNSUPPORTED;   // (ckpt_interval is the scan's)
   if (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_ROUND_WEIGHTS | M2D_FLAG_RAW_PARAMS | M2D_FLAG_PACKED_BC | M2D_FLAG_DPRE | M2D_FLAG_SPLIT_STATES | M2D_FLAG_WHOLE_STATES)) return M2D_ERR_UNSUPPORTED;
   if (R > kMaxR || d->E > 4096) return M2D_ERR_UNSUPPORTED;
   if ((int64_t)d->B * d->H * d->W >= ((int64_t)1 << 31) * kTP) return M2D_ERR_UNSUPPORTED;   // tiles counted in 32 bits

@@ -37,6 +37,7 @@
 
 #include <atomic>
 #include <cstdio>
+#include <cstring>
 #include <stdint.h>
 
 #include "../../include/m2dscan.h"
@@ -181,7 +182,7 @@ struct ScanParams {
   const float *A2T, *A2L, *Df;      // A*log2(e) and D in fp32, (E,16) / (E)
   const float* zeros;               // 256 bytes of zeros (source for out-of-grid staging chunks)
   void *y, *dx, *ddT, *ddL;
-  float* ckpt;                      // [B][nblk][E][4][16][4]        state snapshots, one per block of steps: [q][row][w] = state sinv(4q+w); bf16 for 16-bit tensors
+  float* ckpt;                      // [B][ck_nblk][E][4][16][4]     state snapshots, one per kept block of steps: [q][row][w] = state sinv(4q+w); bf16 for 16-bit tensors
   float* top;                       // [nbands-1][B][W][E][16]       last row of each band (forward states)
   float* bot;                       // [nbands or 1][B][W][E][16]    first-row muT of a band, for the band above (adjoint)
   float* part;                      // [G][P][3][16]                 per-workgroup channel sums of d_C, d_BT, d_BL
@@ -214,6 +215,13 @@ struct ScanParams {
   int64_t Ptot;                     // cells of the whole batch
   int bpb;                          // workgroups per image
   int nwg;                          // total workgroups
+  // Checkpoint interval: the forward keeps the snapshot of one block in 2^ck_shift (the first of every such group
+  // of a workgroup's window); the backward replays the forward over the other blocks of a group before it sweeps
+  // the group, and parks their snapshots in `ring`.
+  int ck_shift;
+  int ck_pb;                        // kept snapshots per band (linked sweep)
+  int ck_nblk;                      // kept snapshots per image
+  void* ring;                       // [workgroup][2^ck_shift - 1][channel of the workgroup][4][16] snapshot quads
 };
 
 // Workgroups are dealt round-robin to the 8 XCDs; renumber so that consecutive logical ids
@@ -689,34 +697,39 @@ typedef unsigned int u2v __attribute__((ext_vector_type(2)));
 template <typename T> struct Snap;
 template <> struct Snap<float> {
   typedef f4v quad;
-  static __device__ __forceinline__ void store(quad* dst, float a, float b, float c, float d) {
-    const f4v v = {a, b, c, d};
-    __builtin_nontemporal_store(v, dst);
-  }
+  static __device__ __forceinline__ quad pack(float a, float b, float c, float d) { return f4v{a, b, c, d}; }
+  static __device__ __forceinline__ void store(quad* dst, float a, float b, float c, float d) { __builtin_nontemporal_store(pack(a, b, c, d), dst); }
   static __device__ __forceinline__ float4 load(const quad* src) { return widen(*src); }
   static __device__ __forceinline__ quad zero() { return f4v{0.f, 0.f, 0.f, 0.f}; }
   static __device__ __forceinline__ float4 widen(quad v) { return make_float4(v.x, v.y, v.z, v.w); }
 };
 template <> struct Snap<bf16_t> {
   typedef u2v quad;
-  static __device__ __forceinline__ void store(quad* dst, float a, float b, float c, float d) {
+  static __device__ __forceinline__ quad pack(float a, float b, float c, float d) {
     // (a vector conversion is one v_cvt_pk_bf16_f32 per pair; two scalar casts and an OR are four instructions)
     typedef float f2v __attribute__((ext_vector_type(2)));
     typedef __bf16 b2v __attribute__((ext_vector_type(2)));
-    const u2v v = {__builtin_bit_cast(uint32_t, __builtin_convertvector((f2v){a, b}, b2v)),
-                   __builtin_bit_cast(uint32_t, __builtin_convertvector((f2v){c, d}, b2v))};
-    __builtin_nontemporal_store(v, dst);
+    return u2v{__builtin_bit_cast(uint32_t, __builtin_convertvector((f2v){a, b}, b2v)),
+               __builtin_bit_cast(uint32_t, __builtin_convertvector((f2v){c, d}, b2v))};
   }
+  static __device__ __forceinline__ void store(quad* dst, float a, float b, float c, float d) { __builtin_nontemporal_store(pack(a, b, c, d), dst); }
   static __device__ __forceinline__ float4 load(const quad* src) { return widen(*src); }
   static __device__ __forceinline__ quad zero() { return u2v{0u, 0u}; }
   static __device__ __forceinline__ float4 widen(quad v) {
     return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u));
   }
 };
-// first quad of the snapshot of channel e before block m of image b: [b][block][E][4 state groups][16 lane rows]
+// first quad of the kept snapshot number mi (snapshot_index) of channel e of image b: [b][kept block][E][4 state groups][16 lane rows]
 template <typename T>
-__device__ __forceinline__ typename Snap<T>::quad* snapshot_at(const ScanParams& p, int b, int m, int e) {
-  return reinterpret_cast<typename Snap<T>::quad*>(p.ckpt) + (((int64_t)b * p.nblk + m) * p.E + e) * (kN / 4 * kHB);
+__device__ __forceinline__ typename Snap<T>::quad* snapshot_at(const ScanParams& p, int b, int mi, int e) {
+  return reinterpret_cast<typename Snap<T>::quad*>(p.ckpt) + (((int64_t)b * p.ck_nblk + mi) * p.E + e) * (kN / 4 * kHB);
+}
+// Block m of a window that starts at block m_lo (the window of band `band` in the linked sweep, else the whole
+// stream): is its snapshot kept, and which of the image's kept snapshots is it.
+__device__ __forceinline__ bool snapshot_kept(const ScanParams& p, int m, int m_lo) { return ((m - m_lo) & ((1 << p.ck_shift) - 1)) == 0; }
+template <bool SLICED>
+__device__ __forceinline__ int snapshot_index(const ScanParams& p, int m, int m_lo, int band) {
+  return SLICED ? band * p.ck_pb + ((m - m_lo) >> p.ck_shift) : (m >> p.ck_shift);
 }
 // Lanes are never masked in the forward: a grid row that is between bands, or a lane that is no
 // grid row, works on zero operands (its records come from the page of zeros), which keeps its
@@ -1001,11 +1014,11 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     // waves of the whole grid run in step, and one burst of all snapshots would stall them.
     ck_mine = false;
     bool snapped = false;   // (uniform) the wave issues the 4*EC stores of a snapshot
-    if (CKPT && m > 0) {
+    if (CKPT && m > 0 && snapshot_kept(p, m, m_lo)) {
       Pos at; at.bnd = bp.bnd0; at.col = bp.col0;
       ck_mine = snapshot_lane(p, at, r, ch_ok);
       snapped = __any(ck_mine);
-      ckp = snapshot_at<T>(p, b, m, e0) + r;
+      ckp = snapshot_at<T>(p, b, snapshot_index<SLICED>(p, m, m_lo, my_band), e0) + r;
     }
     const char* bufc = lds + cur * SG::kBytes;
     const char* bufn = lds + (cur ^ 1) * SG::kBytes;
@@ -1282,11 +1295,11 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_fwd_split_kernel(const S
     cell_off0 = (uint32_t)(cell0 * p.E + e0) * (uint32_t)sizeof(T);
     ck_mine = false;
     bool snapped = false;   // (uniform) the wave issues the store of a snapshot
-    if (CKPT && m > 0) {
+    if (CKPT && m > 0 && snapshot_kept(p, m, m_lo)) {
       Pos at; at.bnd = bp.bnd0; at.col = bp.col0;
       ck_mine = snapshot_lane(p, at, r, ch_ok);
       snapped = __any(ck_mine);
-      ckp = snapshot_at<T>(p, b, m, e0) + g * kHB + r;
+      ckp = snapshot_at<T>(p, b, snapshot_index<SLICED>(p, m, m_lo, my_band), e0) + g * kHB + r;
     }
     const char* bufc = lds + cur * SG::kBytes;
     // (uniform) stores that the wave is sure to issue in the first three steps, after the copies for the
@@ -1346,7 +1359,12 @@ constexpr int bwd_exchange_sets() {
 // multiplied by zero coefficients (delta, dy, x are zero there) wherever they meet a sum.
 // NW waves per workgroup: 8, or 4 for small batches (see the forward kernel).  With 4 waves a thread
 // of the first three adds up both components of one lane's pair of channel sums.
-template <typename T, bool STAGE_X, int MODE, int NW = kBwdWaves>
+// REPLAY: the forward kept a snapshot for the first block only of every group of 2^ck_shift blocks (a longer
+// checkpoint interval).  Before the sweep enters a group, at its last block, the forward is replayed over the
+// group's other blocks from that snapshot, one block at a time through the idle staging buffer, and the state
+// before each block is parked in the workgroup's ring in memory, where the sweep then finds it like a snapshot.
+// A lane reads back only what it wrote itself.
+template <typename T, bool STAGE_X, int MODE, int NW = kBwdWaves, bool REPLAY = false>
 __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) {
   constexpr bool SLICED = MODE == kModeSliced, STACKED = MODE == kModeStacked;
   ScanParams p = pin;   // (stacked images: the height is shortened below for a last, shorter stack)
@@ -1477,12 +1495,32 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   // state snapshot at the start of the block whose position A is given (zero for lanes that were not under way)
   // (kept as it comes from memory until the block starts: nothing waits for the loads before then)
   typename Snap<T>::quad cknext[4];
+  // The replaying kernel of 8 waves (256 registers per lane) fetches the snapshot of a block when the block starts,
+  // not during the block before: the registers that would hold it meanwhile are what the kernel lacks, and waiting
+  // for the fetch costs less than spilling in the sweep (B=128, E=64, 56x56, interval 8: 1.05 against 1.10 ms).
+  // Workgroups of 4 waves have the registers (512x512, interval 8: 4.47 against 4.66 ms).
+  constexpr bool LATE_SNAPSHOT = REPLAY && NW == kBwdWaves;
+  constexpr int kRingSlot = CW * (kN / 4) * kHB;   // quads of one parked snapshot of the workgroup
+  // place of block mm in its group of 2^ck_shift blocks (0: the forward kept its snapshot)
+  auto member = [&](int mm) { return REPLAY ? (mm - m_lo) & ((1 << p.ck_shift) - 1) : 0; };
+  // Where the lane finds the state before block mm: a (uniform) base, in the checkpoints or in the workgroup's ring
+  // [member - 1][channel of the workgroup][state group][row], plus the same offset of the lane in both (channels
+  // past E point at the last channel's place: they park nothing and use nothing).
+  auto snapshot_of_lane = [&](int mm) {
+    const int mem = member(mm);
+    typename Snap<T>::quad* base =
+        (REPLAY && mem != 0) ? static_cast<typename Snap<T>::quad*>(p.ring) + ((int64_t)blockIdx.x * ((1 << p.ck_shift) - 1) + (mem - 1)) * kRingSlot - e_wg0 * (kN / 4 * kHB)
+                             : snapshot_at<T>(p, b, snapshot_index<SLICED>(p, mm, m_lo, my_band), 0);
+    return base + (e * (kN / 4 * kHB) + r);
+  };
+  // the sweep enters a group at block mm, and the block has no snapshot: the replay brings its state
+  auto opens_group = [&](int mm) { return REPLAY && member(mm) != 0 && (mm == m_hi - 1 || member(mm) == (1 << p.ck_shift) - 1); };
   auto load_ckpt = [&](int mm, bool take) {   // take: the forward kept the lane's state before block mm
     if (mm == 0 || !take) {
 #pragma unroll
       for (int q = 0; q < 4; ++q) cknext[q] = Snap<T>::zero();
     } else {
-      const typename Snap<T>::quad* ck = snapshot_at<T>(p, b, mm, e) + r;
+      const typename Snap<T>::quad* ck = snapshot_of_lane(mm);
 #pragma unroll
       for (int q = 0; q < 4; ++q) cknext[q] = ck[q * kHB];
     }
@@ -1498,7 +1536,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   bp = block_pos(p, A, r, rbands);
   int cell0 = cell_of(p, bp.bnd0, r, bp.col0);   // cell index of the lane's position at the first step of the block
   bool ck_take = snapshot_lane(p, Pos{bp.bnd0, bp.col0}, r, ch_ok);   // the lane restores a snapshot for the block to come
-  load_ckpt(m_hi - 1, ck_take);
+  if (!LATE_SNAPSHOT && !opens_group(m_hi - 1)) load_ckpt(m_hi - 1, ck_take);   // (else: after the replay that opens the first iteration)
   if constexpr (SLICED) link.wait_for(link_need_bwd(p.sl_nbb - 1, p.sl_nbb));
   // the lane's row in the block two before (A2 = position of that block): what its raw copies fetch
   auto raw_copy_for = [&](Pos A2, char* dst, bool live) {
@@ -1522,6 +1560,97 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   for (int m = m_hi - 1; m >= m_lo; --m) {
     const int t0 = m * kCK;
     const char* bufc = lds + cur * SG::kBytes;
+    if constexpr (REPLAY) {
+      // The sweep enters a group of blocks at a block without a snapshot: replay the forward from the group's first
+      // block up to this one.  The other staging buffer is idle (the operands of this block are in `bufc`, those of
+      // the block before are fetched further down), and so is the half of `raw` that the next raw copy goes to.
+      if (opens_group(m)) {
+        const int mem = member(m);
+        char* bufr = lds + (cur ^ 1) * SG::kBytes;
+        float hq[kN];   // hq[4 * mg + qi]: state fold_state(mg, qi), the order of the snapshot quads
+        for (int q = m - mem; q < m; ++q) {   // (uniform)
+          const Pos Aq = pos_of(p, q * kCK - (kHB - 1));
+          const BlockPos bq = block_pos(p, Aq, r, rbands);
+          const int cellq = cell_of(p, bq.bnd0, r, bq.col0);
+          if (direct) {
+            bc_raw_copy<NW>(p, pin.bcd, raw + rp * kRawBytes, b, bq, cellq, wave, lane, true);
+            stage_block<T, 4, CW, true, STAGE_X, NW, true>(p, bufr, b, Aq, bq, cellq, e_wg0, wave, lane, X, DT, DL, DY);
+            staging_fence();
+            bc_widen<SG, NW>(raw + rp * kRawBytes, bufr, wave, lane);
+          } else {
+            stage_block<T, 4, CW, true, STAGE_X, NW>(p, bufr, b, Aq, bq, cellq, e_wg0, wave, lane, X, DT, DL, DY);
+          }
+          staging_fence();
+          // the states before block q: the kept snapshot for the first block of the group, else what the replay of
+          // the block before left, and zero in both cases for a lane that was not under way (see snapshot_lane)
+          const bool take_q = q != 0 && snapshot_lane(p, Pos{bq.bnd0, bq.col0}, r, ch_ok);
+          if (q == m - mem) {
+            const typename Snap<T>::quad* ck = snapshot_of_lane(q);
+#pragma unroll
+            for (int mg = 0; mg < 4; ++mg) {
+              const float4 v = take_q ? Snap<T>::load(ck + mg * kHB) : make_float4(0.f, 0.f, 0.f, 0.f);
+              hq[4 * mg + 0] = v.x; hq[4 * mg + 1] = v.y; hq[4 * mg + 2] = v.z; hq[4 * mg + 3] = v.w;
+            }
+          } else {
+#pragma unroll
+            for (int n = 0; n < kN; ++n) hq[n] = take_q ? hq[n] : 0.f;
+          }
+          const uint32_t cell_offq = (uint32_t)(cellq * p.E + e) * (uint32_t)sizeof(T);
+#pragma unroll
+          for (int k = 0; k < kCK; ++k) {
+            const float4 kk = *reinterpret_cast<const float4*>(bufr + (row_const_off + k * SG::kKStr));
+            const float offT = kk.x, offL = kk.y, cT = kk.z, cL = kk.w;
+            float xv = 0.f, dtv = 0.f, dlv = 0.f;
+            if constexpr (STAGE_X) {
+              const T* xr = reinterpret_cast<const T*>(bufr + xd_off + k * kXK);
+              xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + SG::kXTauBytes / sizeof(T)); dlv = IO<T>::ld(xr + 2 * SG::kXTauBytes / sizeof(T));
+            } else if (ch_ok && ((bq.in_grid >> k) & 1u)) {
+              const uint32_t off = cell_offq + (uint32_t)k * estep + (k >= bq.kw ? wrap_adj : 0u);
+              xv = IO<T>::ld(reinterpret_cast<const T*>(Ximg + off));
+              dtv = IO<T>::ld(reinterpret_cast<const T*>(DTimg + off));
+              dlv = IO<T>::ld(reinterpret_cast<const T*>(DLimg + off));
+            }
+            uint32_t a_off = a_base_off;
+            asm volatile("" : "+v"(a_off));
+            const lds_float4* a_mine = (const lds_float4*)(uintptr_t)a_off;
+            const char* rec = bufr + (rec_off + k * SG::kKStr);
+            const float sT = __builtin_fmaf(cT * dtv, xv, g1);
+            const float sL = cL * dlv * xv;
+#pragma unroll
+            for (int mg = 0; mg < 4; ++mg) {
+              const v4f_t at4 = a_mine[mg], al4 = a_mine[kN / 4 + mg];
+              const float4 b4 = *reinterpret_cast<const float4*>(rec + mg * SG::kPlane);
+              const float4 l4 = *reinterpret_cast<const float4*>(rec + SG::kBLOff + mg * SG::kPlane);
+              const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
+              const float bq4[4] = {b4.x, b4.y, b4.z, b4.w}, lq4[4] = {l4.x, l4.y, l4.z, l4.w};
+              float aT[4], aL[4];   // gates before chains, see the forward kernel
+#pragma unroll
+              for (int qi = 0; qi < 4; ++qi) aT[qi] = fexp2(__builtin_fmaf(dtv, atq[qi], offT));
+              pin4(aT);
+              __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+              for (int qi = 0; qi < 4; ++qi) aL[qi] = fexp2(__builtin_fmaf(dlv, alq[qi], offL));
+              pin4(aL);
+              __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+              for (int qi = 0; qi < 4; ++qi) {
+                float u = sL * lq4[qi];
+                u = __builtin_fmaf(sT, bq4[qi], u);
+                u = fma_row_below(aT[qi], hq[4 * mg + qi], u);
+                hq[4 * mg + qi] = __builtin_fmaf(aL[qi], hq[4 * mg + qi], u);
+              }
+            }
+          }
+          typename Snap<T>::quad* park = snapshot_of_lane(q + 1);   // the states before block q + 1
+#pragma unroll
+          for (int mg = 0; mg < 4; ++mg)
+            if (ch_ok) park[mg * kHB] = Snap<T>::pack(hq[4 * mg], hq[4 * mg + 1], hq[4 * mg + 2], hq[4 * mg + 3]);   // (channels past E have no place of their own)
+          __syncthreads();   // every wave is done with the buffer before the next block's copies land in it
+        }
+        if constexpr (!LATE_SNAPSHOT) load_ckpt(m, ck_take);
+      }
+      if constexpr (LATE_SNAPSHOT) load_ckpt(m, ck_take);
+    }
     // the block before: where the lane's row will be is also what the lane's copies fetch
     const Pos Aprev = pos_before(A);
     const BlockPos bpn = block_pos(p, Aprev, r, rbands);
@@ -1620,7 +1749,8 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
         const int t = t0 + k;
         if (half == 1 && k == 0) staging_landed();   // before the last stores of the block, see the forward kernel
         // the states of the later steps are dead by now: their registers take the next snapshot
-        if (half == 1 && k == (kCK > 1 ? 1 : 0) && m > m_lo) load_ckpt(m - 1, ck_take);
+        // (a longer checkpoint interval: not where the block before is the last of its group, whose state the replay will bring)
+        if (!LATE_SNAPSHOT && half == 1 && k == (kCK > 1 ? 1 : 0) && m > m_lo && !opens_group(m - 1)) load_ckpt(m - 1, ck_take);
         if (t < p.T_total) {
           const float4 kk = *reinterpret_cast<const float4*>(bufc + (row_const_off + k * SG::kKStr));
           const float offT = kk.x, offL = kk.y, cT = kk.z, cL = kk.w;
@@ -1898,7 +2028,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_bwd_split_kernel(const S
   typename Snap<T>::quad cknext = Snap<T>::zero();
   auto load_ckpt = [&](int mm, bool take) {   // take: the forward kept the lane's state before block mm
     cknext = Snap<T>::zero();
-    if (mm != 0 && take) cknext = *(snapshot_at<T>(p, b, mm, e) + g * kHB + r);
+    if (mm != 0 && take) cknext = *(snapshot_at<T>(p, b, snapshot_index<SLICED>(p, mm, m_lo, my_band), e) + g * kHB + r);   // (this kernel: a snapshot for every block)
   };
   auto pos_before = [&](Pos Q) {
     Q.col -= kCK;
@@ -2262,6 +2392,8 @@ struct Geometry {
   int ips, vB, vH;                   // images per stack; number and height of what the kernels sweep
   int nbb;                           // linked sweep: blocks per band
   size_t link_bytes;                 // linked sweep: error word and the two arrays of progress counts (forward, backward)
+  int ck_shift, ck_pb, ck_nblk;      // checkpoint interval: log2 of the blocks per kept snapshot; kept snapshots per band (linked sweep) and per image
+  size_t ring_bytes;                 // backward with a longer interval: the replayed snapshots of every workgroup
   bool packed_bc;
   size_t prep_bytes, bc_bytes, ckpt_diag_bytes, top_bytes, bot_bytes, part_bytes, pa_bytes, pd_bytes;
 };
@@ -2271,7 +2403,7 @@ int check_desc(const m2d_desc* d) {
   if (d->B < 1 || d->E < 1 || d->N < 1 || d->H < 2 || d->W < 2) return M2D_ERR_BAD_SHAPE;
   if (d->N != kN) return M2D_ERR_UNSUPPORTED;
   if (d->dtype != M2D_F32 && d->dtype != M2D_BF16) return M2D_ERR_UNSUPPORTED;
-  if (d->reserved != 0 || (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_RAW_PARAMS | M2D_FLAG_PACKED_BC | M2D_FLAG_DPRE | M2D_FLAG_SPLIT_STATES | M2D_FLAG_WHOLE_STATES))) return M2D_ERR_UNSUPPORTED;
+  if ((d->ckpt_interval != 0 && d->ckpt_interval != 4 && d->ckpt_interval != 8 && d->ckpt_interval != 16) || (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_RAW_PARAMS | M2D_FLAG_PACKED_BC | M2D_FLAG_DPRE | M2D_FLAG_SPLIT_STATES | M2D_FLAG_WHOLE_STATES))) return M2D_ERR_UNSUPPORTED;
   if ((d->flags & M2D_FLAG_SPLIT_STATES) && (d->flags & M2D_FLAG_WHOLE_STATES)) return M2D_ERR_UNSUPPORTED;
   if ((int64_t)d->B * d->H * d->W >= ((int64_t)1 << 40)) return M2D_ERR_BAD_SHAPE;
   // one image is addressed with 32-bit byte offsets from its base (fp32: 4 bytes per element;
@@ -2311,7 +2443,10 @@ Geometry make_geometry(const m2d_desc* d) {
   g.stacked = false; g.ips = 1; g.vB = d->B; g.vH = d->H;
   g.rb = kRB;
   const int rb_stacked = d->H <= kRB ? kRB / d->H * d->H : kRB;
-  if (d->H <= kRB && d->B >= 2) {
+  // (a longer checkpoint interval is for grids whose snapshots weigh: images are not stacked then, nor are the states
+  // of a channel split over lanes, and every schedule left runs m2d_bwd_kernel, the one kernel that replays)
+  g.ck_shift = d->ckpt_interval == 16 ? 2 : (d->ckpt_interval == 8 ? 1 : 0);
+  if (d->H <= kRB && d->B >= 2 && g.ck_shift == 0) {
     const int S = d->W > 7 ? d->W : 7;
     int64_t best = -1;
     for (int ips = 1; ips <= 64 && ips <= d->B; ++ips) {
@@ -2394,7 +2529,7 @@ Geometry make_geometry(const m2d_desc* d) {
   // Few waves under way (a wave per 4 channels, the bands of a linked sweep that overlap in time): fewer
   // than three for every four SIMDs.  Then a wave per channel, each with a quarter of the states.
   const int64_t waves_whole = (int64_t)B * ((d->E + g.CS - 1) / g.CS) * together;
-  const bool may_split = !g.stacked && !(d->flags & M2D_FLAG_WHOLE_STATES);
+  const bool may_split = !g.stacked && !(d->flags & M2D_FLAG_WHOLE_STATES) && g.ck_shift == 0;
   g.fwd_split = may_split && ((d->flags & M2D_FLAG_SPLIT_STATES) || waves_whole <= 3 * ncu);
   if (g.fwd_split) {
     g.fwd_ec = 1;
@@ -2420,7 +2555,12 @@ Geometry make_geometry(const m2d_desc* d) {
   g.packed_bc = (d->flags & M2D_FLAG_PACKED_BC) != 0;   // the caller brings the records: nothing to reserve
   // (16-bit tensors are widened inside the scan kernels, nothing to reserve either)
   g.bc_bytes = (g.packed_bc || d->dtype == M2D_BF16) ? 0 : align_up(sizeof(float) * P * 48);
-  g.ckpt_diag_bytes = align_up((d->dtype == M2D_BF16 ? 2 : sizeof(float)) * (size_t)B * g.nblk * d->E * kN * g.HB);   // (16-bit tensors: bf16 snapshots)
+  const int every = 1 << g.ck_shift;
+  g.ck_pb = g.sliced ? (g.nbb + every - 1) / every : 0;
+  g.ck_nblk = g.sliced ? g.nbands * g.ck_pb : (g.nblk + every - 1) / every;
+  g.ckpt_diag_bytes = align_up((d->dtype == M2D_BF16 ? 2 : sizeof(float)) * (size_t)B * g.ck_nblk * d->E * kN * g.HB);   // (16-bit tensors: bf16 snapshots)
+  const size_t bwd_wgs = (size_t)(g.sliced ? g.nbands : 1) * B * g.bwd_bpb;
+  g.ring_bytes = g.ck_shift ? align_up((d->dtype == M2D_BF16 ? 2 : sizeof(float)) * bwd_wgs * (every - 1) * g.bwd_nw * g.CS * kN * g.HB) : 0;
   const bool rows = g.nbands > 1 && !g.stacked;   // boundary rows travel between bands
   g.top_bytes = rows ? align_up(sizeof(float) * (size_t)(g.nbands - 1) * B * d->W * d->E * kN) : 0;
   g.bot_bytes = rows ? align_up(sizeof(float) * (size_t)(g.sliced ? g.nbands : 1) * B * d->W * d->E * kN) : 0;
@@ -2441,7 +2581,7 @@ size_t workspace_bytes_of(const Geometry& g, int pass, int have_ckpt) {
   if (pass == M2D_PASS_FWD) {
     if (!have_ckpt) n += g.top_bytes + g.bc_bytes;
   } else {
-    n += g.part_bytes + g.pa_bytes + g.pd_bytes + g.bot_bytes;
+    n += g.part_bytes + g.pa_bytes + g.pd_bytes + g.bot_bytes + g.ring_bytes;
     if (!have_ckpt) n += ckpt_bytes_of(g);
   }
   return n;
@@ -2461,6 +2601,8 @@ void fill_common(ScanParams& sp, const m2d_desc* d, const Geometry& g) {
   sp.bot_stride = g.sliced ? (int64_t)g.vB * d->W * d->E * kN : 0;
   sp.flip = (d->flags & M2D_FLAG_FLIP) ? 1 : 0;
   sp.dpre = (d->flags & M2D_FLAG_DPRE) ? 1 : 0;
+  sp.ck_shift = g.ck_shift; sp.ck_pb = g.ck_pb; sp.ck_nblk = g.ck_nblk;
+  sp.ring = nullptr;
 }
 
 // A kernel that needs more than 64 KB of dynamic LDS has to be told so once per device (each
@@ -2614,12 +2756,12 @@ int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   return rc;
 }
 
-template <typename T, bool SX, int MODE, int NW>
+template <typename T, bool SX, int MODE, int NW, bool REPLAY = false>
 int launch_bwd_as(const ScanParams& sp, hipStream_t st) {
   constexpr size_t lds = bwd_lds_bytes<T, NW>();
   static std::atomic<uint64_t> seen{0};
-  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_bwd_kernel<T, SX, MODE, NW>), lds, seen)) return M2D_ERR_HIP;
-  hipLaunchKernelGGL((m2d_bwd_kernel<T, SX, MODE, NW>), dim3((unsigned)sp.nwg), dim3(NW * 64), lds, st, sp);
+  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_bwd_kernel<T, SX, MODE, NW, REPLAY>), lds, seen)) return M2D_ERR_HIP;
+  hipLaunchKernelGGL((m2d_bwd_kernel<T, SX, MODE, NW, REPLAY>), dim3((unsigned)sp.nwg), dim3(NW * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
@@ -2648,6 +2790,8 @@ int launch_bwd_split(const ScanParams& sp, bool stage_x, hipStream_t st) {
 template <typename T, bool SX, int MODE>
 int launch_bwd(const ScanParams& sp, hipStream_t st, int nw = kBwdWaves) {
   if constexpr (MODE != kModeStacked) {
+    if (sp.ck_shift > 0)   // a longer checkpoint interval: the kernel that replays the forward between snapshots
+      return nw == kFwdHalfWaves ? launch_bwd_as<T, SX, MODE, kFwdHalfWaves, true>(sp, st) : launch_bwd_as<T, SX, MODE, kBwdWaves, true>(sp, st);
     if (nw == kFwdHalfWaves) return launch_bwd_as<T, SX, MODE, kFwdHalfWaves>(sp, st);
   }
   return launch_bwd_as<T, SX, MODE, kBwdWaves>(sp, st);
@@ -2664,6 +2808,7 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   sp.pA = reinterpret_cast<float*>(w); w += g.pa_bytes;
   sp.pD = reinterpret_cast<float*>(w); w += g.pd_bytes;
   sp.bot = reinterpret_cast<float*>(w); w += g.bot_bytes;
+  sp.ring = w; w += g.ring_bytes;
   int rc = launch_prep<T>(sp, d, g, AT, AL, D, prep, link_words, st);
   if (rc) return rc;
   char* ck = ckpt ? const_cast<char*>(static_cast<const char*>(ckpt)) : w;
@@ -2829,6 +2974,10 @@ int m2d_scan_plan(const m2d_desc* desc, int pass, char* text, size_t cap) {
   else
     snprintf(text, cap, "%s: %s, %lld workgroups of %d waves, %d channels each, 16 states per lane",
              fwd ? "m2d_fwd_kernel" : "m2d_bwd_kernel", sched, wgs, nw, nw * g.CS * per_lane);
+  if (g.ck_shift) {
+    const size_t n = strlen(text);
+    if (n + 1 < cap) snprintf(text + n, cap - n, fwd ? ", a snapshot every %d steps" : ", a snapshot every %d steps and the forward replayed in between", kCK << g.ck_shift);
+  }
   return M2D_OK;
 }
 

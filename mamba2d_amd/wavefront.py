@@ -52,26 +52,33 @@ layernorm_linear_act_fwd_op = torch.ops.m2dscan.layernorm_linear_act_fwd
 # reference's partial recomputation).  Module-level switch, read at forward time.
 SAVE_CHECKPOINTS = os.environ.get("M2D_SAVE_CHECKPOINTS", "1") != "0"
 
+# Steps between the state snapshots that a forward keeps for its backward (m2d_desc.ckpt_interval): 0 or 4 (the
+# default), 8 or 16.  Longer intervals keep a half or a quarter of the snapshots, and the backward replays the
+# forward over the steps in between.  Read at forward time; a backward uses the value its forward ran with.
+CKPT_INTERVAL = int(os.environ.get("M2D_CKPT_INTERVAL", "0"))
+
 # The entry point computes the projections with the library's own kernels (wf_cuda_fn_proj) or
 # with stock torch operators followed by wf_cuda_fn_pr / wf_cuda_fn_fr.  Read at call time.
 FUSED_PROJECTIONS = os.environ.get("M2D_FUSED_PROJECTIONS", "1") != "0"
 
 
-def _ckpt_bytes(x, N, flip=False, packed_bc=False) -> int:
+def _ckpt_bytes(x, N, flip=False, packed_bc=False, ckpt_interval=0) -> int:
     d = cabi.make_desc(x, N, flip)
+    d.ckpt_interval = ckpt_interval
     if packed_bc:   # the caller brings the packed B/C records: the buffer has no room for them
         d.flags |= cabi.M2D_FLAG_PACKED_BC
     return int(cabi.lib.m2d_scan_ckpt_bytes(ctypes.byref(d)))
 
 
 @torch.library.register_fake("m2dscan::scan_fwd")
-def _scan_fwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, save_ckpt, flip, raw_params=False, packed_bc=False):
-    n = _ckpt_bytes(x, AT.shape[1], packed_bc=packed_bc) if save_ckpt else 1
+def _scan_fwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, save_ckpt, flip, raw_params=False, packed_bc=False, ckpt_interval=0):
+    n = _ckpt_bytes(x, AT.shape[1], packed_bc=packed_bc, ckpt_interval=ckpt_interval) if save_ckpt else 1
     return torch.empty_like(x), x.new_empty((max(n, 1),), dtype=torch.uint8)
 
 
 @torch.library.register_fake("m2dscan::scan_bwd")
-def _scan_bwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt, flip, raw_params=False, packed_bc=False, dpre=False):
+def _scan_bwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt, flip, raw_params=False, packed_bc=False, dpre=False,
+                   ckpt_interval=0):
     bc = [x.new_empty((*x.shape[:3], AT.shape[1])) for _ in range(3)]
     return [torch.empty_like(x), torch.empty_like(deltaT), torch.empty_like(deltaL), torch.empty_like(AT), torch.empty_like(AL),
             *bc, torch.empty_like(D)]
@@ -200,25 +207,25 @@ def _state_groups(AT, AL, BT, BL, C):
             for n0 in range(0, AT.shape[1], STATES_PER_CALL)]
 
 
-def _grouped_scan_fwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, keep, flip):
+def _grouped_scan_fwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, keep, flip, interval=0):
     """scan_fwd for d_state != 16: y summed over the groups in fp32; one checkpoint buffer per group."""
     if AT.shape[1] < 1:
         raise ValueError(f"d_state must be positive, got {AT.shape[1]}")
     y, cks, no_skip = None, [], torch.zeros_like(D)
     for gi, grp in enumerate(_state_groups(AT, AL, BT, BL, C)):
-        part, ck = scan_fwd_op(x, deltaT, deltaL, *grp, D if gi == 0 else no_skip, keep, flip)
+        part, ck = scan_fwd_op(x, deltaT, deltaL, *grp, D if gi == 0 else no_skip, keep, flip, ckpt_interval=interval)
         y = part.float() if y is None else y + part.float()
         cks.append(ck)
     return y.to(x.dtype), cks
 
 
-def _grouped_scan_bwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, cks, flip):
+def _grouped_scan_bwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, cks, flip, interval=0):
     """scan_bwd for d_state != 16: gradients of x and the step sizes summed over the groups in fp32,
     those of A, B, C put together along the state axis (padding dropped); d_D comes with the first group."""
     N = AT.shape[1]
     sums, per_state, d_D, no_skip = None, [], None, torch.zeros_like(D)
     for gi, grp in enumerate(_state_groups(AT, AL, BT, BL, C)):
-        g = scan_bwd_op(x, deltaT, deltaL, *grp, D if gi == 0 else no_skip, dy, cks[gi], flip)
+        g = scan_bwd_op(x, deltaT, deltaL, *grp, D if gi == 0 else no_skip, dy, cks[gi], flip, ckpt_interval=interval)
         if gi == 0:
             sums, d_D = [t.float() for t in g[:3]], g[8]
         else:
@@ -237,11 +244,12 @@ class _ScanOnParams(torch.autograd.Function):
         args = [_c(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D)]
         keep = SAVE_CHECKPOINTS and recording and any(ctx.needs_input_grad)
         ctx.flip = bool(flip)
+        ctx.interval = CKPT_INTERVAL
         if AT.shape[1] != STATES_PER_CALL:
-            y, cks = _grouped_scan_fwd(*args, keep, ctx.flip)
+            y, cks = _grouped_scan_fwd(*args, keep, ctx.flip, ctx.interval)
             ctx.save_for_backward(*args, *cks)
             return y
-        y, ck = scan_fwd_op(*args, keep, ctx.flip)
+        y, ck = scan_fwd_op(*args, keep, ctx.flip, ckpt_interval=ctx.interval)
         ctx.save_for_backward(*args, ck)
         return y
 
@@ -250,8 +258,8 @@ class _ScanOnParams(torch.autograd.Function):
         args, cks = ctx.saved_tensors[:9], ctx.saved_tensors[9:]
         dy = _c(grad_output.to(args[0].dtype))
         if args[3].shape[1] != STATES_PER_CALL:
-            return (*_grouped_scan_bwd(*args, dy, cks, ctx.flip), None, None)
-        return (*scan_bwd_op(*args, dy, cks[0], ctx.flip), None, None)
+            return (*_grouped_scan_bwd(*args, dy, cks, ctx.flip, ctx.interval), None, None)
+        return (*scan_bwd_op(*args, dy, cks[0], ctx.flip, ckpt_interval=ctx.interval), None, None)
 
 
 class wf_cuda_fn_pr(torch.autograd.Function):
@@ -308,10 +316,10 @@ class wf_cuda_fn_fr(torch.autograd.Function):
         if AT_log.shape[1] != STATES_PER_CALL:
             n_groups = -(-AT_log.shape[1] // STATES_PER_CALL)
             d_x_scan, d_dT, d_dL, d_AT, d_AL, d_BT, d_BL, d_C, d_D = _grouped_scan_bwd(
-                _c(x), *det, _c(D), dy, [none] * n_groups, ctx.flip)
+                _c(x), *det, _c(D), dy, [none] * n_groups, ctx.flip, CKPT_INTERVAL)
         else:
             d_x_scan, d_dT, d_dL, d_AT, d_AL, d_BT, d_BL, d_C, d_D = scan_bwd_op(
-                _c(x), det[0], det[1], det[2], det[3], det[4], det[5], det[6], _c(D), dy, none, ctx.flip)
+                _c(x), det[0], det[1], det[2], det[3], det[4], det[5], det[6], _c(D), dy, none, ctx.flip, ckpt_interval=CKPT_INTERVAL)
         grads = torch.autograd.grad([deltaT, deltaL, BT, BL, C, AT, AL], leaves,
                                     [d_dT, d_dL, d_BT, d_BL, d_C, d_AT, d_AL])
         d_x = d_x_scan + grads[0]   # d_x_scan already contains dy*D
@@ -348,7 +356,8 @@ class wf_cuda_fn_proj(torch.autograd.Function):
         # B_T, B_L, C go from the projection kernel to the scan as packed records (BT) and two empty tensors
         low, dT, dL, BT, BL, C = proj_fwd_op(x, *w32, AT_log.shape[1], True, True)
         keep = SAVE_CHECKPOINTS and not full and recording and any(ctx.needs_input_grad)
-        y, ck = scan_fwd_op(x, dT, dL, At, Al, BT, BL, C, D32, keep, bool(flip), True, True)
+        ctx.interval = CKPT_INTERVAL
+        y, ck = scan_fwd_op(x, dT, dL, At, Al, BT, BL, C, D32, keep, bool(flip), True, True, ctx.interval)
         if full:
             ctx.save_for_backward(x, *raw)
         else:
@@ -369,7 +378,7 @@ class wf_cuda_fn_proj(torch.autograd.Function):
         # with raw parameters the gradients of A_log and D come back in fp32; the gradients of the two
         # step sizes come back as gradients before the softplus, which is what the projections' backward wants
         d_x, d_dT, d_dL, d_At, d_Al, d_BT, d_BL, d_C, d_D = scan_bwd_op(x, dT, dL, At, Al, BT, BL, C, D32, dy, ck, ctx.flip,
-                                                                        True, True, True)
+                                                                        True, True, True, ctx.interval)
         # d_x holds the scan's own gradient (dy*D included); the projections add theirs in place
         g = proj_bwd_op(x, low, dT, dL, w32[0], w32[1], w32[3], d_dT, d_dL, d_BT, d_BL, d_C, d_x, True, True)
         grads = (d_At, d_Al, *g, d_D)

@@ -39,7 +39,7 @@ def test_version_and_status_strings(cabi):
 
 
 def D(cabi, **kw):
-    base = dict(B=2, H=14, W=14, E=32, N=16, dtype=0, flags=0, reserved=0)
+    base = dict(B=2, H=14, W=14, E=32, N=16, dtype=0, flags=0, ckpt_interval=0)
     base.update(kw)
     return cabi.Desc(**base)
 
@@ -55,7 +55,9 @@ def test_descriptor_validation(cabi):
     assert chk(D(cabi, flags=4)) == 0 and chk(D(cabi, flags=29)) == 0 and chk(D(cabi, flags=2)) == 3
     assert chk(D(cabi, flags=32)) == 0 and chk(D(cabi, flags=64 | 1)) == 0 and chk(D(cabi, flags=96)) == 3
     assert chk(D(cabi, N=8)) == 3 and chk(D(cabi, dtype=7)) == 3 and chk(D(cabi, flags=128)) == 3
-    assert chk(D(cabi, reserved=1)) == 3
+    # steps between snapshots: the default, 4, 8 or 16
+    assert all(chk(D(cabi, ckpt_interval=v)) == 0 for v in (0, 4, 8, 16))
+    assert all(chk(D(cabi, ckpt_interval=v)) == 3 for v in (1, 2, 12, 32, -4))
     # one image must fit 32-bit offsets: H*W < 2^24 cells, H*W*E < 2^30 elements
     assert chk(D(cabi, B=1, H=4096, W=4096, E=8)) == 3 and chk(D(cabi, B=1, H=2048, W=2048, E=256)) == 3
     assert chk(D(cabi, B=1, H=2048, W=2048, E=64)) == 0 and chk(D(cabi, B=4, H=4000, W=4000, E=32)) == 0
@@ -107,6 +109,30 @@ def test_buffer_sizes_scale_linearly_in_area(cabi):
             assert 3.5 < ratio < 4.5, (a, b, k, ratio)
     assert cabi.lib.m2d_scan_workspace_bytes(ctypes.byref(D(cabi, H=1)), 0, 0) == 0
     assert cabi.lib.m2d_scan_ckpt_bytes(ctypes.byref(D(cabi, N=3))) == 0
+
+
+def test_checkpoint_interval_shrinks_the_snapshots(cabi):
+    """m2d_desc.ckpt_interval = 8 / 16: a half / a quarter of the snapshots (band boundary rows and, for fp32, the
+    packed B|C stay), a small ring of replayed snapshots per workgroup in the backward's scratch, and the one
+    backward kernel that replays, whatever layout was asked for."""
+    import torch
+    for dtype, shape in ((1, (128, 56, 56, 64)), (0, (1, 2048, 2048, 64)), (1, (1, 2048, 2048, 64)), (0, (300, 7, 7, 32))):
+        B, H, W, E = shape
+        ck, ws = {}, {}
+        for iv in (0, 4, 8, 16):
+            d = D(cabi, B=B, H=H, W=W, E=E, dtype=dtype, ckpt_interval=iv, flags=cabi.M2D_FLAG_WHOLE_STATES)
+            ck[iv] = cabi.lib.m2d_scan_ckpt_bytes(ctypes.byref(d))
+            ws[iv] = cabi.lib.m2d_scan_workspace_bytes(ctypes.byref(d), 1, 1)
+        assert ck[4] == ck[0] and ws[4] == ws[0]
+        if H > 14:   # (7x7 images are stacked at the default interval and not at the others: other block counts)
+            assert ck[0] > ck[8] > ck[16]
+            # a half of the blocks dropped against three quarters (rounded up per window of a band)
+            assert abs((ck[0] - ck[8]) / (ck[0] - ck[16]) - 2 / 3) < 0.05
+            assert 0 < ws[8] - ws[0] < ws[16] - ws[0] <= 0.1 * ws[0] + (1 << 20)   # (three parked snapshots per workgroup)
+    plan = cabi.scan_plan(1, 256, 256, 64, torch.float32, cabi.M2D_PASS_BWD, flags=cabi.M2D_FLAG_SPLIT_STATES, ckpt_interval=16)
+    assert plan.startswith("m2d_bwd_kernel: linked sweep") and plan.endswith("a snapshot every 16 steps and the forward replayed in between")
+    assert cabi.scan_plan(300, 7, 7, 32, torch.float32, cabi.M2D_PASS_FWD, ckpt_interval=8).startswith("m2d_fwd_kernel: one stream per image")
+    assert cabi.scan_plan(300, 7, 7, 32, torch.float32, cabi.M2D_PASS_FWD, ckpt_interval=4).startswith("m2d_fwd_kernel: stacked images")
 
 
 def test_plan_names_kernel_and_schedule(cabi):

@@ -91,6 +91,44 @@ def test_entry_point_matches_oracle_fp32(wf, recomp, projections):
         assert so.rel_err(g.cpu(), gr) < 2e-4, name
 
 
+@pytest.mark.parametrize("interval", [8, 16])
+@pytest.mark.parametrize("recomp", ["partial", "full"])
+def test_entry_point_with_longer_checkpoint_interval(wf, recomp, interval, monkeypatch):
+    """wavefront.CKPT_INTERVAL reaches the library through the operators: fewer bytes saved for the backward,
+    the same gradients (the oracle's, to the entry point's fp32 bound); 24 states run as two groups."""
+    say(f"\ncase entry_point {recomp} ckpt_interval={interval}")
+    for N in (16, 24):
+        B, H, W, E = 2, 30, 12, 32
+        R = math.ceil(E / 16)
+        p = make_block_params(E, N, R, 0, "cuda")
+        x = torch.randn(B, H, W, E, generator=torch.Generator().manual_seed(1)).cuda()
+        dy = torch.randn(B, H, W, E, generator=torch.Generator().manual_seed(2)).cuda()
+        kept = {}
+        for iv in (0, interval):
+            monkeypatch.setattr(wf, "CKPT_INTERVAL", iv)
+            real, seen = wf.scan_fwd_op, []
+
+            def spy(*a, **kw):
+                out = real(*a, **kw)
+                seen.append(out[1].numel())
+                return out
+
+            monkeypatch.setattr(wf, "scan_fwd_op", spy)
+            leaves = [x.clone().requires_grad_(True)] + [p[k].clone().requires_grad_(True) for k in ORDER]
+            y = wf.wavefront_scan_cuda(*leaves, recomp=recomp)
+            grads = torch.autograd.grad(y, leaves, dy)
+            monkeypatch.setattr(wf, "scan_fwd_op", real)
+            kept[iv] = sum(seen)
+        if recomp == "partial":
+            assert kept[interval] < kept[0], kept
+        ref_leaves = [t.detach().double().cpu().requires_grad_(True) for t in leaves]
+        y_ref = so.wavefront_scan_ref(*ref_leaves)
+        g_ref = torch.autograd.grad(y_ref, ref_leaves, dy.double().cpu())
+        assert so.rel_err(y.cpu(), y_ref.detach()) < 1e-4
+        for name, g, gr in zip(("x",) + ORDER, grads, g_ref):
+            assert so.rel_err(g.cpu(), gr) < 2e-4, (N, name)
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 2e-2)], ids=["f32", "bf16"])
 @pytest.mark.parametrize("N", [1, 8, 24, 32])
 def test_fn_pr_other_state_counts(wf, cscan, N, dtype, tol):
@@ -245,9 +283,9 @@ def test_no_checkpoints_are_kept_under_no_grad(wf, monkeypatch):
     seen = []
     real = wf.scan_fwd_op
 
-    def spy(*a):
+    def spy(*a, **kw):
         seen.append(bool(a[9]))
-        return real(*a)
+        return real(*a, **kw)
 
     monkeypatch.setattr(wf, "scan_fwd_op", spy)
     inp = so.make_inputs(1, 6, 5, 8, 16, seed=2, dtype=torch.float32)
