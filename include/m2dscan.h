@@ -171,7 +171,9 @@ int m2d_scan_fwd_noalloc(const m2d_desc* desc,
 /* Fused backward: the nine gradients of the forward above for upstream gradient dy.
  * Replaces wavefront_cuda.py:169-196 (state recompute, wf_bwd of wf_cuda_bind.cpp:35,
  * fused_backward_math, output-projection backward).  ckpt may be NULL, in which case
- * the checkpoints are rebuilt inside the call (one extra forward sweep).
+ * the checkpoints are rebuilt inside the call (one extra forward sweep).  A ckpt buffer
+ * belongs to the inputs and the descriptor of the forward that filled it: besides the state
+ * snapshots it holds what that forward derived from AT, AL and D, which this call reuses.
  * d_AT, d_AL, d_D are written (not accumulated). */
 int m2d_scan_bwd(const m2d_desc* desc,
                  const void* x, const void* deltaT, const void* deltaL,

@@ -2573,8 +2573,10 @@ Geometry make_geometry(const m2d_desc* d) {
   return g;
 }
 
-// checkpoint buffer: [state snapshots][band boundary rows][packed B,C (fp32 tensors only)]
-size_t ckpt_bytes_of(const Geometry& g) { return g.ckpt_diag_bytes + g.top_bytes + g.bc_bytes; }
+// checkpoint buffer: [state snapshots][band boundary rows][packed B,C (fp32 tensors only)][set-up area]
+// (the set-up area -- page of zeros, A * log2 e, D -- is the forward's: a backward that gets the buffer needs no
+// set-up launch of its own, unless it has progress counts to clear)
+size_t ckpt_bytes_of(const Geometry& g) { return g.ckpt_diag_bytes + g.top_bytes + g.bc_bytes + g.prep_bytes; }
 
 size_t workspace_bytes_of(const Geometry& g, int pass, int have_ckpt) {
   size_t n = g.prep_bytes + g.link_bytes;
@@ -2620,7 +2622,7 @@ inline bool allow_dynamic_lds(const void* kernel, size_t bytes, std::atomic<uint
 // Set-up area: [page of zeros][A_T*log2e][A_L*log2e][D], all fp32.
 template <typename T>
 int launch_prep(ScanParams& sp, const m2d_desc* d, const Geometry& g, const void* AT, const void* AL, const void* D, float* base,
-                uint32_t* link_words, hipStream_t st) {
+                uint32_t* link_words, hipStream_t st, bool ready = false) {
   const int n_link = (int)(g.link_bytes / sizeof(uint32_t));
   sp.link_err = link_words;   // (the first 64 words: the error word; then forward counts, then backward counts)
   float* zeros = base;
@@ -2628,6 +2630,7 @@ int launch_prep(ScanParams& sp, const m2d_desc* d, const Geometry& g, const void
   float* A2L = A2T + (size_t)d->E * kN;
   float* Df = A2L + (size_t)d->E * kN;
   sp.zeros = zeros; sp.A2T = A2T; sp.A2L = A2L; sp.Df = Df;
+  if (ready && n_link == 0) return M2D_OK;   // the forward of this problem filled the area, and there is nothing to clear
   const int n = d->E * kN > kZeroFloats ? d->E * kN : kZeroFloats;
   if (d->flags & M2D_FLAG_RAW_PARAMS)
     hipLaunchKernelGGL((m2d_prep_kernel<T, true>), dim3((n + 255) / 256), dim3(256), 0, st, AT, AL, D, zeros, A2T, A2L, Df, d->E, link_words, n_link);
@@ -2739,6 +2742,7 @@ int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   char* keep = ckpt ? static_cast<char*>(ckpt) + g.ckpt_diag_bytes : w;   // [top][packed B,C]
   sp.ckpt = ckpt ? static_cast<float*>(ckpt) : nullptr;
   sp.top = reinterpret_cast<float*>(keep);
+  if (ckpt) prep = reinterpret_cast<float*>(keep + g.top_bytes + g.bc_bytes);   // kept for the backward
   int rc = launch_prep<T>(sp, d, g, AT, AL, D, prep, link_words, st);
   if (rc) return rc;
   if ((!ckpt || sizeof(T) == 2) && !g.packed_bc) {   // the kernel takes the tensors as they are (fp32: only where no backward will want the packed copy)
@@ -2809,9 +2813,10 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   sp.pD = reinterpret_cast<float*>(w); w += g.pd_bytes;
   sp.bot = reinterpret_cast<float*>(w); w += g.bot_bytes;
   sp.ring = w; w += g.ring_bytes;
-  int rc = launch_prep<T>(sp, d, g, AT, AL, D, prep, link_words, st);
-  if (rc) return rc;
   char* ck = ckpt ? const_cast<char*>(static_cast<const char*>(ckpt)) : w;
+  if (ckpt) prep = reinterpret_cast<float*>(ck + g.ckpt_diag_bytes + g.top_bytes + g.bc_bytes);   // as the forward left it
+  int rc = launch_prep<T>(sp, d, g, AT, AL, D, prep, link_words, st, ckpt != nullptr);
+  if (rc) return rc;
   sp.ckpt = reinterpret_cast<float*>(ck);
   sp.top = reinterpret_cast<float*>(ck + g.ckpt_diag_bytes);
   if (sizeof(T) == 2 && !g.packed_bc) {   // widened inside the kernels (also by the forward sweep below)
