@@ -883,8 +883,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   for (int c = 0; c < EC; ++c)
 #pragma unroll
     for (int n = 0; n < kN; ++n) h[c][n] = 0.f;
-  bool ck_mine = false;       // the lane stores a snapshot in the first step of the current block
-  typename Snap<T>::quad* ckp = nullptr;      // where to
+  typename Snap<T>::quad* ckp = nullptr;      // where the lane stores its snapshot in the first step of the current block
   auto step = [&](int k, const Ops& o) {
     const float offT = o.kk.x, offL = o.kk.y, cT = o.kk.z, cL = o.kk.w;
     const bool inr = ch_ok && ((bp.in_grid >> k) & 1u);
@@ -911,7 +910,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
         for (int w = 0; w < 4; ++w) aL[w] = fexp2(__builtin_fmaf(o.dlv[c], a2l[c][sinv<PERM>(4 * q + w)], offL));
         pin4(aL);
         __builtin_amdgcn_sched_barrier(0);
-        if (CKPT && k == 0 && ck_mine)   // the four states as they are before this step
+        if (CKPT && k == 0)   // the four states as they are before this step
           Snap<T>::store(ckp + (c * 4 + q) * kHB, h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)],
                          h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
 #pragma unroll
@@ -1008,17 +1007,18 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     }
     rp ^= 1;
     cell_off0 = (uint32_t)(cell0 * p.E + e0) * (uint32_t)sizeof(T);
-    // Snapshot of the state before the block (after step t0-1) for the lanes whose previous
-    // position was a cell of the grid; the others hold nothing the backward needs.  The stores are
-    // issued inside the first step, each group of four states just before it is overwritten: the
-    // waves of the whole grid run in step, and one burst of all snapshots would stall them.
-    ck_mine = false;
-    bool snapped = false;   // (uniform) the wave issues the 4*EC stores of a snapshot
-    if (CKPT && m > 0 && snapshot_kept(p, m, m_lo)) {
-      Pos at; at.bnd = bp.bnd0; at.col = bp.col0;
-      ck_mine = snapshot_lane(p, at, r, ch_ok);
-      snapped = __any(ck_mine);
-      ckp = snapshot_at<T>(p, b, snapshot_index<SLICED>(p, m, m_lo, my_band), e0) + r;
+    // Snapshot of the state before the block (after step t0-1).  The stores are issued inside the
+    // first step, each group of four states just before it is overwritten: the waves of the whole
+    // grid run in step, and one burst of all snapshots would stall them.  Every lane stores, with no
+    // branch inside the step (a predicate per lane splits the step into five scheduling regions:
+    // 0.292 against 0.281 ms at B=128, E=64, 56x56).  Only the lanes whose previous position was a
+    // cell of the grid hold something the backward needs (snapshot_lane), and only those it reads;
+    // the other lanes write to their own place all the same.  Channels past E, whose place is
+    // another channel's, and blocks whose snapshot is not kept (block 0; a longer checkpoint
+    // interval) write to the image's place for block 0, which nobody reads.
+    if constexpr (CKPT) {
+      const bool keep = m > 0 && snapshot_kept(p, m, m_lo);
+      ckp = snapshot_at<T>(p, b, (keep && ch_ok) ? snapshot_index<SLICED>(p, m, m_lo, my_band) : 0, e0) + r;
     }
     const char* bufc = lds + cur * SG::kBytes;
     const char* bufn = lds + (cur ^ 1) * SG::kBytes;
@@ -1038,7 +1038,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
         } else {
           if (y_thrice) staging_landed_behind<2>(); else staging_landed();
         }
-      } else if (snapped) {
+      } else if constexpr (CKPT) {
         if (y_thrice) staging_landed_behind<4 * EC + 3>(); else staging_landed_behind<4 * EC>();
       } else {
         if (y_thrice) staging_landed_behind<3>(); else staging_landed();
@@ -1180,7 +1180,6 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_fwd_split_kernel(const S
   BlockPos bp;
   uint32_t cell_off0 = 0;
   float h[4] = {0.f, 0.f, 0.f, 0.f};
-  bool ck_mine = false;
   typename Snap<T>::quad* ckp = nullptr;
 
   auto step = [&](const char* bufc, int k) {
@@ -1213,7 +1212,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_fwd_split_kernel(const S
     for (int w = 0; w < 4; ++w) aL[w] = fexp2(__builtin_fmaf(dlv, a2l[w], offL));
     pin4(aL);
     __builtin_amdgcn_sched_barrier(0);
-    if (CKPT && k == 0 && ck_mine) Snap<T>::store(ckp, h[0], h[1], h[2], h[3]);   // the lane's states as they are before this step
+    if (CKPT && k == 0) Snap<T>::store(ckp, h[0], h[1], h[2], h[3]);   // the lane's states as they are before this step
     float acc = 0.f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
@@ -1293,13 +1292,9 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_fwd_split_kernel(const S
     }
     rp ^= 1;
     cell_off0 = (uint32_t)(cell0 * p.E + e0) * (uint32_t)sizeof(T);
-    ck_mine = false;
-    bool snapped = false;   // (uniform) the wave issues the store of a snapshot
-    if (CKPT && m > 0 && snapshot_kept(p, m, m_lo)) {
-      Pos at; at.bnd = bp.bnd0; at.col = bp.col0;
-      ck_mine = snapshot_lane(p, at, r, ch_ok);
-      snapped = __any(ck_mine);
-      ckp = snapshot_at<T>(p, b, snapshot_index<SLICED>(p, m, m_lo, my_band), e0) + g * kHB + r;
+    if constexpr (CKPT) {   // every lane stores, without a branch inside the step: see m2d_fwd_kernel
+      const bool keep = m > 0 && snapshot_kept(p, m, m_lo);
+      ckp = snapshot_at<T>(p, b, (keep && ch_ok) ? snapshot_index<SLICED>(p, m, m_lo, my_band) : 0, e0) + g * kHB + r;
     }
     const char* bufc = lds + cur * SG::kBytes;
     // (uniform) stores that the wave is sure to issue in the first three steps, after the copies for the
@@ -1312,7 +1307,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_fwd_split_kernel(const S
     // 1 only (link_need_fwd).  With just the stores issued after those of step 1 left in flight (y of step 1, row and
     // y of step 2), this block counts as done at its end.
     const int younger = SLICED ? (y_thrice ? 2 : 0) + (top_thrice ? 1 : 0)
-                               : (snapped ? 1 : 0) + (y_thrice ? 3 : 0) + (top_thrice ? 3 : 0);
+                               : (CKPT ? 1 : 0) + (y_thrice ? 3 : 0) + (top_thrice ? 3 : 0);
 #pragma unroll
     for (int k = 0; k < kCK; ++k) {
       if (k == kCK - 1) staging_landed_behind_n(younger);
