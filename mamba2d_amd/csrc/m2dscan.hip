@@ -720,9 +720,11 @@ template <> struct Snap<bf16_t> {
   }
 };
 // first quad of the kept snapshot number mi (snapshot_index) of channel e of image b: [b][kept block][E][4 state groups][16 lane rows]
+// (nkept: kept snapshots per image, p.ck_nblk.  A kernel that only runs at the default interval passes p.nblk and
+// the block itself: it then needs none of the interval's parameters, which would cost it scalar registers.)
 template <typename T>
-__device__ __forceinline__ typename Snap<T>::quad* snapshot_at(const ScanParams& p, int b, int mi, int e) {
-  return reinterpret_cast<typename Snap<T>::quad*>(p.ckpt) + (((int64_t)b * p.ck_nblk + mi) * p.E + e) * (kN / 4 * kHB);
+__device__ __forceinline__ typename Snap<T>::quad* snapshot_at(const ScanParams& p, int b, int mi, int e, int nkept) {
+  return reinterpret_cast<typename Snap<T>::quad*>(p.ckpt) + (((int64_t)b * nkept + mi) * p.E + e) * (kN / 4 * kHB);
 }
 // Block m of a window that starts at block m_lo (the window of band `band` in the linked sweep, else the whole
 // stream): is its snapshot kept, and which of the image's kept snapshots is it.
@@ -1018,7 +1020,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     // interval) write to the image's place for block 0, which nobody reads.
     if constexpr (CKPT) {
       const bool keep = m > 0 && snapshot_kept(p, m, m_lo);
-      ckp = snapshot_at<T>(p, b, (keep && ch_ok) ? snapshot_index<SLICED>(p, m, m_lo, my_band) : 0, e0) + r;
+      ckp = snapshot_at<T>(p, b, (keep && ch_ok) ? snapshot_index<SLICED>(p, m, m_lo, my_band) : 0, e0, p.ck_nblk) + r;
     }
     const char* bufc = lds + cur * SG::kBytes;
     const char* bufn = lds + (cur ^ 1) * SG::kBytes;
@@ -1294,7 +1296,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_fwd_split_kernel(const S
     cell_off0 = (uint32_t)(cell0 * p.E + e0) * (uint32_t)sizeof(T);
     if constexpr (CKPT) {   // every lane stores, without a branch inside the step: see m2d_fwd_kernel
       const bool keep = m > 0 && snapshot_kept(p, m, m_lo);
-      ckp = snapshot_at<T>(p, b, (keep && ch_ok) ? snapshot_index<SLICED>(p, m, m_lo, my_band) : 0, e0) + g * kHB + r;
+      ckp = snapshot_at<T>(p, b, (keep && ch_ok) ? snapshot_index<SLICED>(p, m, m_lo, my_band) : 0, e0, p.ck_nblk) + g * kHB + r;
     }
     const char* bufc = lds + cur * SG::kBytes;
     // (uniform) stores that the wave is sure to issue in the first three steps, after the copies for the
@@ -1502,11 +1504,15 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   // [member - 1][channel of the workgroup][state group][row], plus the same offset of the lane in both (channels
   // past E point at the last channel's place: they park nothing and use nothing).
   auto snapshot_of_lane = [&](int mm) {
-    const int mem = member(mm);
-    typename Snap<T>::quad* base =
-        (REPLAY && mem != 0) ? static_cast<typename Snap<T>::quad*>(p.ring) + ((int64_t)blockIdx.x * ((1 << p.ck_shift) - 1) + (mem - 1)) * kRingSlot - e_wg0 * (kN / 4 * kHB)
-                             : snapshot_at<T>(p, b, snapshot_index<SLICED>(p, mm, m_lo, my_band), 0);
-    return base + (e * (kN / 4 * kHB) + r);
+    if constexpr (!REPLAY) {   // the default interval: a snapshot for every block, as before
+      return snapshot_at<T>(p, b, mm, e, p.nblk) + r;
+    } else {
+      const int mem = member(mm);
+      typename Snap<T>::quad* base =
+          mem != 0 ? static_cast<typename Snap<T>::quad*>(p.ring) + ((int64_t)blockIdx.x * ((1 << p.ck_shift) - 1) + (mem - 1)) * kRingSlot - e_wg0 * (kN / 4 * kHB)
+                   : snapshot_at<T>(p, b, snapshot_index<SLICED>(p, mm, m_lo, my_band), 0, p.ck_nblk);
+      return base + (e * (kN / 4 * kHB) + r);
+    }
   };
   // the sweep enters a group at block mm, and the block has no snapshot: the replay brings its state
   auto opens_group = [&](int mm) { return REPLAY && member(mm) != 0 && (mm == m_hi - 1 || member(mm) == (1 << p.ck_shift) - 1); };
@@ -2023,7 +2029,7 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_bwd_split_kernel(const S
   typename Snap<T>::quad cknext = Snap<T>::zero();
   auto load_ckpt = [&](int mm, bool take) {   // take: the forward kept the lane's state before block mm
     cknext = Snap<T>::zero();
-    if (mm != 0 && take) cknext = *(snapshot_at<T>(p, b, snapshot_index<SLICED>(p, mm, m_lo, my_band), e) + g * kHB + r);   // (this kernel: a snapshot for every block)
+    if (mm != 0 && take) cknext = *(snapshot_at<T>(p, b, mm, e, p.nblk) + g * kHB + r);   // (this kernel: a snapshot for every block)
   };
   auto pos_before = [&](Pos Q) {
     Q.col -= kCK;
