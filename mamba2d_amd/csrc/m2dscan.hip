@@ -685,6 +685,25 @@ __device__ __forceinline__ void bc_widen(const char* raw, char* buf, int wave, i
 }
 
 // ------------------------------------------------------------------------------------ forward
+// y on its way out (m2d_fwd_kernel).  A lane's y of one step is 2 or 4 bytes at a cell of its own row: stored
+// from the lane, a wave's y of one step goes to 16 different cache lines, 8 bytes each, and these stores cost
+// the kernel 3 % (inference) to 9 % (with the snapshot stores of a training forward) of its time.  Instead the
+// lanes drop y into LDS, a window of 4 steps at a time, and once per block every thread stores 8 or 16 bytes: the
+// channels of one wave at one cell, so that the 8 (4) threads of a cell write its 64 (32) bytes together.
+//   [wave][step of the window][lane row] chunks of the wave's channels (a wave's region is padded so that the
+//   same chunk of consecutive waves sits in different banks).  Where the cells are in the image, the threads read
+//   from a table that every lane fills once per block: byte offset of its row's cell at the block's first step,
+//   the step at which the row changes band, the steps at which it is on the grid (all lanes of a row write the
+//   same; the flush reads what slot 0 wrote).
+template <typename T, int EC, int NW>
+struct YTile {
+  static constexpr int kChunk = 4 * EC * (int)sizeof(T);            // bytes of a wave's channels at one cell: 8 or 16
+  static constexpr int kRegion = kCK * kHB * kChunk + kChunk;       // one wave's part of a window
+  static constexpr int kBytes = (NW * kRegion + 15) / 16 * 16;      // one window
+  static constexpr int kTableBytes = 4 * 64 * 8;                    // where the rows are: 4 blocks x 64 lanes x (offset, steps on the grid)
+  static_assert(kChunk == 8 || kChunk == 16, "a thread flushes one 8- or 16-byte chunk");
+  static_assert(kCK * kHB == 64 && kCK == 4, "a window is 64 cells: one per thread and wave-chunk");
+};
 // A snapshot quad: the four states of one state group of a lane, as the forward keeps them for the
 // backward.  fp32 tensors keep them as they are.  16-bit tensors keep them rounded to bf16: the
 // reference rounds every state of its hidden-state tensor to the tensors' type (wf_cuda.cu:40-69 writes
@@ -810,6 +829,15 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     }
   }
   char* raw = lds + 2 * SG::kBytes;                 // [2][kRawBytes]
+  // y leaves through LDS (see YTile) where a wave's channels at a cell are whole 8- or 16-byte chunks: the same
+  // condition as for staging x
+  constexpr bool YTILE = WRITE_Y && STAGE_X;
+  using YT = YTile<T, EC, NW>;
+  char* ywin = raw + (WIDEN ? 2 * kRawBytes : 0);   // [2 windows][YT::kBytes]
+  uint2* ytab = reinterpret_cast<uint2*>(ywin + 2 * YT::kBytes);   // [block & 3][lane]
+  if constexpr (YTILE) {   // the block before the first has no row on the grid
+    for (int i = threadIdx.x; i < 4 * 64; i += NW * 64) ytab[i] = make_uint2(0u, 0u);
+  }
 
   settle_loads();
   __syncthreads();
@@ -886,6 +914,8 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
 #pragma unroll
     for (int n = 0; n < kN; ++n) h[c][n] = 0.f;
   typename Snap<T>::quad* ckp = nullptr;      // where the lane stores its snapshot in the first step of the current block
+  int ypar = 0;                 // window that the current block fills
+  const uint32_t y_lane_off = (uint32_t)(wave * YT::kRegion + (r * CS + slot) * EC * (int)sizeof(T));
   auto step = [&](int k, const Ops& o) {
     const float offT = o.kk.x, offL = o.kk.y, cT = o.kk.z, cL = o.kk.w;
     const bool inr = ch_ok && ((bp.in_grid >> k) & 1u);
@@ -944,8 +974,34 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
           }
       }
     }
-    if (WRITE_Y && inr)
-      IO<T>::template stv<EC>(reinterpret_cast<T*>(Yimg + (cell_off0 + (uint32_t)k * estep + (k >= bp.kw ? wrap_adj : 0u))), yv);
+    if constexpr (YTILE) {   // no branch: a lane off the grid drops its y too, next to an offset that says so
+      // A window is flushed behind the barrier of its block.  With operands fetched a step ahead that barrier
+      // stands before the block's last step, which therefore opens the next window.
+      const int ks = AHEAD ? (k + 1) & (kCK - 1) : k;   // place of this step in its window
+      char* win = ywin + (AHEAD && k == kCK - 1 ? ypar ^ 1 : ypar) * YT::kBytes;
+      IO<T>::template stv<EC>(reinterpret_cast<T*>(win + y_lane_off + ks * (kHB * YT::kChunk)), yv);
+    } else {
+      if (WRITE_Y && inr)
+        IO<T>::template stv<EC>(reinterpret_cast<T*>(Yimg + (cell_off0 + (uint32_t)k * estep + (k >= bp.kw ? wrap_adj : 0u))), yv);
+    }
+  };
+  // One window of y from LDS to memory, after a barrier behind which every wave has written it: thread (cell c,
+  // wave j) takes the channels of wave j at cell c.  first_only: just the first step of the window (the last
+  // step of the sweep; the rest of the window is from two blocks ago).
+  auto flush_y = [&](int par, int m, bool first_only) {   // m: the block whose barrier this is
+    const char* win = ywin + par * YT::kBytes;
+    const int c = threadIdx.x / NW, j = threadIdx.x % NW;
+    const int ks = c >> kHBShift;                                  // the cell's step in the window ...
+    const int k = AHEAD ? (ks + kCK - 1) & (kCK - 1) : ks;         // ... and in its block,
+    const int blk = AHEAD && ks == 0 ? m - 1 : m;                  // which is the one before for the window's first step
+    const uint2 row = ytab[(blk & 3) * 64 + (c & (kHB - 1))];
+    const uint32_t off = row.x + (uint32_t)k * estep + (k >= (int)(row.y >> 8) ? wrap_adj : 0u);
+    if (((row.y >> k) & 1u) && e_wg0 + j * CS * EC < p.E && !(first_only && c >= kHB)) {
+      if constexpr (YT::kChunk == 8)
+        *reinterpret_cast<uint2*>(Yimg + off + j * YT::kChunk) = *reinterpret_cast<const uint2*>(win + j * YT::kRegion + c * YT::kChunk);
+      else
+        *reinterpret_cast<uint4*>(Yimg + off + j * YT::kChunk) = *reinterpret_cast<const uint4*>(win + j * YT::kRegion + c * YT::kChunk);
+    }
   };
 
   Pos A = pos_of(p, m_lo * kCK - (kHB - 1));     // position of the stream index t0 - 15 (wave-uniform)
@@ -1009,6 +1065,8 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     }
     rp ^= 1;
     cell_off0 = (uint32_t)(cell0 * p.E + e0) * (uint32_t)sizeof(T);
+    if constexpr (YTILE)
+      ytab[(m & 3) * 64 + lane] = make_uint2((uint32_t)(cell0 * p.E + e_wg0) * (uint32_t)sizeof(T), ((uint32_t)(bp.kw < kCK ? bp.kw : kCK) << 8) | (bp.in_grid & 15u));
     // Snapshot of the state before the block (after step t0-1).  The stores are issued inside the
     // first step, each group of four states just before it is overwritten: the waves of the whole
     // grid run in step, and one burst of all snapshots would stall them.  Every lane stores, with no
@@ -1026,7 +1084,8 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     const char* bufn = lds + (cur ^ 1) * SG::kBytes;
     // (uniform) some lane writes y at each of the first three steps: the wave issues at least
     // three stores between the copies for the next block and the barrier that ends this one
-    const bool y_thrice = WRITE_Y && __any(ch_ok && (bp.in_grid & 7u) == 7u);
+    // (y that leaves through LDS is stored once per block, before the copies for the next block: nothing to count)
+    const bool y_thrice = WRITE_Y && !YTILE && __any(ch_ok && (bp.in_grid & 7u) == 7u);
     // (uniform, linked sweep) lane 14 stores the band's last row at each of the first three steps
     const bool top_thrice = SLICED && __any(ch_ok && (bp.in_grid & 7u) == 7u && r == kRB && bp.kw >= kCK && bp.bnd0 + 1 < p.nbands);
     auto next_block_landed = [&] {
@@ -1062,6 +1121,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
           __syncthreads();
           // every wave has waited for the rows it stored at the steps 0 and 1 of this block
           if constexpr (SLICED) link.publish((uint32_t)(m - m_lo + 1));
+          if constexpr (YTILE) flush_y(ypar, m, false);   // the last step of the block before and the first three of this one
           if (!last) fetch(bufn, 0, ahead);
         }
         step(k, now);   // also past the end of the sweep (last block): zero operands like any position off the grid, nothing stored
@@ -1078,11 +1138,17 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
       }
       __syncthreads();
       if constexpr (SLICED) link.publish((uint32_t)(m - m_lo + 1));
+      if constexpr (YTILE) flush_y(ypar, m, false);   // the four steps of this block
     }
+    ypar ^= 1;
     cur ^= 1;
     A = An;
     bp = bpn;
     cell0 = celln;
+  }
+  if constexpr (YTILE && AHEAD) {   // the last step of the sweep
+    __syncthreads();
+    flush_y(ypar, m_hi, true);
   }
   if constexpr (SLICED) {   // the whole window is done once every store of every wave has completed
     __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -2371,7 +2437,9 @@ inline size_t align_up(size_t v, size_t a = 256) { return (v + a - 1) / a * a; }
 // copy of A and two staging buffers.  A compute unit has 160 KB.
 constexpr size_t kLdsPerWorkgroup = 160 * 1024;
 template <typename T, int EC, int NW = kFwdWaves>
-constexpr size_t fwd_lds_bytes() { return 2 * (size_t)Stage<T, 3, NW * 4 * EC, false>::kBytes + (sizeof(T) == 2 ? 2 * kRawBytes : 0); }
+constexpr size_t fwd_lds_bytes() {
+  return 2 * (size_t)Stage<T, 3, NW * 4 * EC, false>::kBytes + (sizeof(T) == 2 ? 2 * kRawBytes : 0) + 2 * (size_t)YTile<T, EC, NW>::kBytes + YTile<T, EC, NW>::kTableBytes;
+}
 template <typename T, int NW = kBwdWaves>
 constexpr size_t bwd_lds_bytes() {
   return sizeof(float2) * bwd_exchange_sets<T, NW>() * NW * 3 * 64 + sizeof(float) * NW * 4 * 2 * kN + 256 +
