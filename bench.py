@@ -44,7 +44,7 @@ HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the backward scan kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
 # (profiles/scan_cfg1_kernel_trace_and_traffic.txt); counters cannot be read from inside this script,
 # so the figure is carried here for the workload that has a counter run, and is null for the others.
-MEASURED_TRAFFIC = {"cfg1": 1.1205e9}
+MEASURED_TRAFFIC = {"cfg1": 1.1188e9}
 # Issue slots per (cell, channel, state) of the scan kernels (a v_exp_f32 takes two on gfx950):
 # forward 2 exponent FMAs + 2 v_exp + 5 FMA-class (input term, two gate terms, y);
 # backward 10 for the recomputation, 24 for the adjoint (15 FMA-class, 4.5 for the gates of three steps in
