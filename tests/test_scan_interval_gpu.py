@@ -60,7 +60,7 @@ def test_flipped_scan_and_rebuilt_checkpoints(cabi, cscan, shape, interval):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
-@pytest.mark.parametrize("shape", [(5, 40, 36, 32), (1, 90, 120, 16), (128, 28, 28, 64)], ids=lambda s: "x".join(map(str, s)))
+@pytest.mark.parametrize("shape", [(5, 40, 36, 32), (1, 90, 120, 16), (128, 28, 28, 64), (1, 1024, 1024, 64)], ids=lambda s: "x".join(map(str, s)))
 def test_same_results_as_the_default_interval(cabi, shape, dtype):
     inp = so.make_inputs(*shape, 16, seed=5, dtype=dtype)
     a = [inp[k].cuda() for k in so.INPUT_NAMES]

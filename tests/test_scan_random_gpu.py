@@ -39,3 +39,19 @@ def test_random_shape(cabi, cscan, case):
     B, H, W, E, dt, flip, ckpt, seed = case
     say(f"\ncase random B={B} H={H} W={W} E={E} {dt} flip={flip} ckpt={ckpt} seed={seed}")
     run_case(cabi, cscan, B, H, W, E, torch.float32 if dt == "f32" else torch.bfloat16, seed=seed, flip=flip, with_ckpt=ckpt)
+
+
+INTERVAL_CASES = draw_cases(777, 32)
+
+
+@pytest.mark.parametrize("case", INTERVAL_CASES, ids=lambda c: f"{c[0]}x{c[1]}x{c[2]}x{c[3]}-{c[4]}{'-flip' if c[5] else ''}{'-ckpt' if c[6] else ''}")
+def test_random_shape_with_longer_checkpoint_interval(cabi, cscan, case):
+    """The same sweep with a snapshot every 8 or 16 steps (the backward replays the forward in between)."""
+    B, H, W, E, dt, flip, ckpt, seed = case
+    interval = 8 if seed % 2 else 16
+    say(f"\ncase random interval={interval} B={B} H={H} W={W} E={E} {dt} flip={flip} ckpt={ckpt} seed={seed}")
+    cabi.CKPT_INTERVAL = interval
+    try:
+        run_case(cabi, cscan, B, H, W, E, torch.float32 if dt == "f32" else torch.bfloat16, seed=seed, flip=flip, with_ckpt=ckpt)
+    finally:
+        cabi.CKPT_INTERVAL = 0
