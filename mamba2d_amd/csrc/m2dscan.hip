@@ -576,7 +576,20 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int 
                               buf + SG::kXOff + tau * SG::kXTauBytes + ks * SG::kXStepBytes + i * 1024);
           }
       }
+    } else if constexpr (SG::kCpt == 1) {   // all four steps per copy: lanes = (step, row); tensor tau is copied by the wave of step tau
+      static_assert(kCK == 4 && NT <= kCK, "a wave-wide copy is the four steps of one tensor");
+      const int cell4 = cell_at(slot);
+      const bool ok4 = ok_at(slot) && e_wg0 < p.E;
+      const uint32_t off = (uint32_t)(cell4 * p.E + e_wg0) * (uint32_t)sizeof(T);
+#pragma unroll
+      for (int tau = 0; tau < NT; ++tau)
+        if (ks == tau && wsub == 0) {
+          const T* base = tau == 0 ? x0 : (tau == 1 ? x1 : (tau == 2 ? x2 : x3));
+          const char* t_img = reinterpret_cast<const char*>(base) + img_bytes;
+          lds_fill16<false>(ok4 ? t_img + off : zeros, buf + SG::kXOff + tau * SG::kXTauBytes);
+        }
     } else {                         // two steps per copy: lanes = (step, channel chunk, row); the wave of the even step copies
+      static_assert(SG::kCpt == 2, "two chunks of channels per cell");
       if ((ks & 1) == 0) {
         const bool hi = lane >= 32;
         const int cell2 = hi ? cell_at(ks + 1) : cell;
@@ -1165,19 +1178,20 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
 // step.  A workgroup has 8 waves = 8 channels.  Staging, schedules and memory formats are those of
 // m2d_fwd_kernel; y of a cell is the sum over the 4 lane groups (two lane-swap steps), stored by group 0.
 constexpr int kSplitWaves = 8;
+constexpr int kSplitHalfWaves = 4;   // where workgroups of 8 would leave compute units idle (fp32 tensors)
 __device__ __forceinline__ float sum_over_groups(float v) {
   v = fold16(v, v);
   return fold32(v, v);
 }
-template <typename T, bool CKPT, bool WRITE_Y, bool STAGE_X, int MODE>
-__global__ __launch_bounds__(kSplitWaves * 64) void m2d_fwd_split_kernel(const ScanParams pin) {
+template <typename T, bool CKPT, bool WRITE_Y, bool STAGE_X, int MODE, int NWS = kSplitWaves>
+__global__ __launch_bounds__(NWS * 64) void m2d_fwd_split_kernel(const ScanParams pin) {
   static_assert(MODE != kModeStacked, "stacked images are many: they never need the split");
   constexpr bool SLICED = MODE == kModeSliced;
   const ScanParams& p = pin;
   __builtin_assume(p.stacked == 0);
   __builtin_assume(p.rb == kRB);
   __builtin_assume(p.S >= kHB + kCK - 1);
-  constexpr int NW = kSplitWaves, CW = NW;
+  constexpr int NW = NWS, CW = NW;
   using SG = Stage<T, 3, CW, false>;
   constexpr bool WIDEN = sizeof(T) == 2;
   extern __shared__ float4 smem[];
@@ -1998,15 +2012,15 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
 // the states of a cell (for d_delta and d_x) are taken across the 4 lane groups by lane swaps; sums
 // over channels (d_C, d_BT, d_BL) across the 8 waves through LDS, as in m2d_bwd_kernel, a float4 of
 // four states per lane.  Memory formats are those of m2d_bwd_kernel.
-template <typename T, bool STAGE_X, int MODE>
-__global__ __launch_bounds__(kSplitWaves * 64) void m2d_bwd_split_kernel(const ScanParams pin) {
+template <typename T, bool STAGE_X, int MODE, int NWS = kSplitWaves>
+__global__ __launch_bounds__(NWS * 64) void m2d_bwd_split_kernel(const ScanParams pin) {
   static_assert(MODE != kModeStacked, "stacked images are many: they never need the split");
   constexpr bool SLICED = MODE == kModeSliced;
   const ScanParams& p = pin;
   __builtin_assume(p.stacked == 0);
   __builtin_assume(p.rb == kRB);
   __builtin_assume(p.S >= kHB + kCK - 1);
-  constexpr int NW = kSplitWaves, CW = NW;
+  constexpr int NW = NWS, CW = NW;
   constexpr int SLOT = 3 * 64;           // float4s per wave in one exchange buffer
   using SG = Stage<T, 4, CW, true>;
   constexpr bool WIDEN = sizeof(T) == 2;
@@ -2079,8 +2093,10 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_bwd_split_kernel(const S
   constexpr uint32_t kXK = SG::kXStepBytes;
   // channel sums: the first 6 waves add up; wave 2v + c takes components 2c, 2c+1 of every lane's float4 of
   // tensor v.  They are kept per cell as [C, B_T, B_L][16] in the natural order of the states.
-  const bool f_on = wave < 6;
-  const int f_v = wave >> 1, f_c = wave & 1;
+  // (workgroups of 4 waves: the first 3 add up, a whole float4 each)
+  constexpr bool QUADS = NW < 6;
+  const bool f_on = wave < (QUADS ? 3 : 6);
+  const int f_v = QUADS ? wave : wave >> 1, f_c = QUADS ? 0 : wave & 1;
   const uint32_t f_sub0 = (uint32_t)(f_v * kN + (f_c ? 1 : 0) * 4 + g) * (uint32_t)sizeof(float);   // component 2c: state perm(2c) * 4 + g, perm = (0, 2, 1, 3)
   const uint32_t f_sub1 = (uint32_t)(f_v * kN + (f_c ? 3 : 2) * 4 + g) * (uint32_t)sizeof(float);   // component 2c + 1
   const float g1 = r == 0 ? 1.f : 0.f;
@@ -2268,12 +2284,22 @@ __global__ __launch_bounds__(kSplitWaves * 64) void m2d_bwd_split_kernel(const S
         __syncthreads();
         if (f_on && ((bp.in_grid >> k) & 1u)) {
           const uint32_t off = f_off0 + (uint32_t)k * pstep + (k >= bp.kw ? pwrap_adj : 0u);
-          const float2* sl = reinterpret_cast<const float2*>(slots + xpar * NW * SLOT + f_v * 64 + lane) + f_c;
-          float2 sum = sl[0];
+          if constexpr (QUADS) {
+            const float4* sl = slots + xpar * NW * SLOT + f_v * 64 + lane;
+            float4 sum = sl[0];
 #pragma unroll
-          for (int w = 1; w < NW; ++w) { sum.x += sl[2 * w * SLOT].x; sum.y += sl[2 * w * SLOT].y; }
-          *reinterpret_cast<float*>(PARTimg + off + f_sub0) = sum.x;
-          *reinterpret_cast<float*>(PARTimg + off + f_sub1) = sum.y;
+            for (int w = 1; w < NW; ++w) { sum.x += sl[w * SLOT].x; sum.y += sl[w * SLOT].y; sum.z += sl[w * SLOT].z; sum.w += sl[w * SLOT].w; }
+            // component j holds state perm(j) * 4 + g, perm = (0, 2, 1, 3)
+            float* dst = reinterpret_cast<float*>(PARTimg + off + (uint32_t)(f_v * kN + g) * (uint32_t)sizeof(float));
+            dst[0] = sum.x; dst[8] = sum.y; dst[4] = sum.z; dst[12] = sum.w;
+          } else {
+            const float2* sl = reinterpret_cast<const float2*>(slots + xpar * NW * SLOT + f_v * 64 + lane) + f_c;
+            float2 sum = sl[0];
+#pragma unroll
+            for (int w = 1; w < NW; ++w) { sum.x += sl[2 * w * SLOT].x; sum.y += sl[2 * w * SLOT].y; }
+            *reinterpret_cast<float*>(PARTimg + off + f_sub0) = sum.x;
+            *reinterpret_cast<float*>(PARTimg + off + f_sub1) = sum.y;
+          }
         }
         xpar ^= 1;
       }
@@ -2600,10 +2626,14 @@ Geometry make_geometry(const m2d_desc* d) {
   const int64_t waves_whole = (int64_t)B * ((d->E + g.CS - 1) / g.CS) * together;
   const bool may_split = !g.stacked && !(d->flags & M2D_FLAG_WHOLE_STATES) && g.ck_shift == 0;
   g.fwd_split = may_split && ((d->flags & M2D_FLAG_SPLIT_STATES) || waves_whole <= 3 * ncu);
+  // Workgroups of 8 waves (8 channels) under way on at most half of the compute units: workgroups of 4 then run on
+  // twice as many, each wave with a SIMD to itself (a sweep of few images is as fast as one wave gets through its
+  // blocks).  fp32 tensors only.
+  const int split_nw = (d->dtype == M2D_F32 && 2 * (int64_t)B * ((d->E + kSplitWaves - 1) / kSplitWaves) * together <= ncu) ? kSplitHalfWaves : kSplitWaves;
   if (g.fwd_split) {
     g.fwd_ec = 1;
-    g.fwd_nw = kSplitWaves;
-    g.fwd_bpb = (d->E + kSplitWaves - 1) / kSplitWaves;
+    g.fwd_nw = split_nw;
+    g.fwd_bpb = (d->E + split_nw - 1) / split_nw;
     g.fwd_wpb = g.fwd_bpb * g.fwd_nw;
   }
   g.bwd_nw = (!g.stacked && wg_half > (int64_t)B * groups && wg_half * together <= room) ? kFwdHalfWaves : kBwdWaves;
@@ -2611,11 +2641,11 @@ Geometry make_geometry(const m2d_desc* d) {
   g.bwd_wpb = g.bwd_bpb * g.bwd_nw;
   // (the backward keeps one set of channel sums per workgroup of an image: with 8 channels per workgroup
   // that memory is bounded here unless the caller insists)
-  const size_t split_part = sizeof(float) * (size_t)((d->E + kSplitWaves - 1) / kSplitWaves) * 3 * kN * (size_t)d->B * d->H * d->W;
+  const size_t split_part = sizeof(float) * (size_t)((d->E + split_nw - 1) / split_nw) * 3 * kN * (size_t)d->B * d->H * d->W;
   g.bwd_split = may_split && ((d->flags & M2D_FLAG_SPLIT_STATES) || (waves_whole <= 3 * ncu && split_part <= ((size_t)2 << 30)));
   if (g.bwd_split) {
-    g.bwd_nw = kSplitWaves;
-    g.bwd_bpb = (d->E + kSplitWaves - 1) / kSplitWaves;
+    g.bwd_nw = split_nw;
+    g.bwd_bpb = (d->E + split_nw - 1) / split_nw;
     g.bwd_wpb = g.bwd_bpb * g.bwd_nw;
   }
   g.stage_x = (d->E % (d->dtype == M2D_BF16 ? 8 : 4)) == 0;
@@ -2733,21 +2763,31 @@ int launch_fwd_as(const ScanParams& sp, hipStream_t st) {
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
-template <typename T>
-constexpr size_t fwd_split_lds_bytes() { return 2 * (size_t)Stage<T, 3, kSplitWaves, false>::kBytes + (sizeof(T) == 2 ? 2 * kRawBytes : 0); }
-template <typename T, bool CK, bool WY, bool SX, int MODE>
+template <typename T, int NWS = kSplitWaves>
+constexpr size_t fwd_split_lds_bytes() { return 2 * (size_t)Stage<T, 3, NWS, false>::kBytes + (sizeof(T) == 2 ? 2 * kRawBytes : 0); }
+template <typename T, bool CK, bool WY, bool SX, int MODE, int NWS = kSplitWaves>
 int launch_fwd_split_as(const ScanParams& sp, hipStream_t st) {
-  constexpr size_t lds = fwd_split_lds_bytes<T>();
+  constexpr size_t lds = fwd_split_lds_bytes<T, NWS>();
   static_assert(lds <= kLdsPerWorkgroup, "staging must fit the LDS");
   static std::atomic<uint64_t> seen{0};
-  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_fwd_split_kernel<T, CK, WY, SX, MODE>), lds, seen)) return M2D_ERR_HIP;
-  hipLaunchKernelGGL((m2d_fwd_split_kernel<T, CK, WY, SX, MODE>), dim3((unsigned)sp.nwg), dim3(kSplitWaves * 64), lds, st, sp);
+  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_fwd_split_kernel<T, CK, WY, SX, MODE, NWS>), lds, seen)) return M2D_ERR_HIP;
+  hipLaunchKernelGGL((m2d_fwd_split_kernel<T, CK, WY, SX, MODE, NWS>), dim3((unsigned)sp.nwg), dim3(NWS * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 // (16-bit x and deltas of 8 channels are less than a 16-byte chunk per cell: read from memory, not staged)
 template <typename T, int MODE>
-int launch_fwd_split(const ScanParams& sp, bool stage_x, bool ckpt, bool write_y, hipStream_t st) {
+int launch_fwd_split(const ScanParams& sp, bool stage_x, bool ckpt, bool write_y, hipStream_t st, int nw = kSplitWaves) {
   if constexpr (sizeof(T) == 4) {
+    if (nw == kSplitHalfWaves) {   // (fp32 only: 4 channels of 16-bit tensors are no 16-byte chunk for the boundary rows' staging)
+      if (stage_x) {
+        if (ckpt && write_y) return launch_fwd_split_as<T, true, true, true, MODE, kSplitHalfWaves>(sp, st);
+        if (ckpt) return launch_fwd_split_as<T, true, false, true, MODE, kSplitHalfWaves>(sp, st);
+        return launch_fwd_split_as<T, false, true, true, MODE, kSplitHalfWaves>(sp, st);
+      }
+      if (ckpt && write_y) return launch_fwd_split_as<T, true, true, false, MODE, kSplitHalfWaves>(sp, st);
+      if (ckpt) return launch_fwd_split_as<T, true, false, false, MODE, kSplitHalfWaves>(sp, st);
+      return launch_fwd_split_as<T, false, true, false, MODE, kSplitHalfWaves>(sp, st);
+    }
     if (stage_x) {
       if (ckpt && write_y) return launch_fwd_split_as<T, true, true, true, MODE>(sp, st);
       if (ckpt) return launch_fwd_split_as<T, true, false, true, MODE>(sp, st);
@@ -2773,7 +2813,8 @@ int launch_fwd(const ScanParams& sp0, const m2d_desc* d, const Geometry& g, bool
   sp.nwg = g.vB * g.fwd_bpb;
   auto once = [&]() {
     if (g.fwd_split)
-      return g.sliced ? launch_fwd_split<T, kModeSliced>(sp, g.stage_x, ckpt, write_y, st) : launch_fwd_split<T, kModeSweep>(sp, g.stage_x, ckpt, write_y, st);
+      return g.sliced ? launch_fwd_split<T, kModeSliced>(sp, g.stage_x, ckpt, write_y, st, g.fwd_nw)
+                      : launch_fwd_split<T, kModeSweep>(sp, g.stage_x, ckpt, write_y, st, g.fwd_nw);
     if (g.sliced) {   // (the linked sweep is only chosen where one channel per lane is)
       if (g.fwd_nw == kFwdHalfWaves)
         return g.stage_x ? launch_fwd_mode<T, 1, true, kModeSliced, kFwdHalfWaves>(sp, ckpt, write_y, st)
@@ -2838,23 +2879,25 @@ int launch_bwd_as(const ScanParams& sp, hipStream_t st) {
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
-template <typename T>
+template <typename T, int NWS = kSplitWaves>
 constexpr size_t bwd_split_lds_bytes() {
-  return sizeof(float4) * 2 * kSplitWaves * 3 * 64 + 2 * (size_t)Stage<T, 4, kSplitWaves, true>::kBytes + (sizeof(T) == 2 ? 2 * kRawBytes : 0);
+  return sizeof(float4) * 2 * NWS * 3 * 64 + 2 * (size_t)Stage<T, 4, NWS, true>::kBytes + (sizeof(T) == 2 ? 2 * kRawBytes : 0);
 }
-template <typename T, bool SX, int MODE>
+template <typename T, bool SX, int MODE, int NWS = kSplitWaves>
 int launch_bwd_split_as(const ScanParams& sp, hipStream_t st) {
-  constexpr size_t lds = bwd_split_lds_bytes<T>();
+  constexpr size_t lds = bwd_split_lds_bytes<T, NWS>();
   static_assert(lds <= kLdsPerWorkgroup, "exchange buffers and staging must fit the LDS");
   static std::atomic<uint64_t> seen{0};
-  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_bwd_split_kernel<T, SX, MODE>), lds, seen)) return M2D_ERR_HIP;
-  hipLaunchKernelGGL((m2d_bwd_split_kernel<T, SX, MODE>), dim3((unsigned)sp.nwg), dim3(kSplitWaves * 64), lds, st, sp);
+  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_bwd_split_kernel<T, SX, MODE, NWS>), lds, seen)) return M2D_ERR_HIP;
+  hipLaunchKernelGGL((m2d_bwd_split_kernel<T, SX, MODE, NWS>), dim3((unsigned)sp.nwg), dim3(NWS * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 // (16-bit x, deltas and dy of 8 channels are less than a 16-byte chunk per cell: read from memory, not staged)
 template <typename T, int MODE>
-int launch_bwd_split(const ScanParams& sp, bool stage_x, hipStream_t st) {
+int launch_bwd_split(const ScanParams& sp, bool stage_x, hipStream_t st, int nw = kSplitWaves) {
   if constexpr (sizeof(T) == 4) {
+    if (nw == kSplitHalfWaves)
+      return stage_x ? launch_bwd_split_as<T, true, MODE, kSplitHalfWaves>(sp, st) : launch_bwd_split_as<T, false, MODE, kSplitHalfWaves>(sp, st);
     if (stage_x) return launch_bwd_split_as<T, true, MODE>(sp, st);
   }
   return launch_bwd_split_as<T, false, MODE>(sp, st);
@@ -2905,14 +2948,14 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   sp.nwg = g.vB * g.bwd_bpb;
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][0], st);
   if (!g.sliced) {
-    if (g.bwd_split) rc = launch_bwd_split<T, kModeSweep>(sp, g.stage_x, st);
+    if (g.bwd_split) rc = launch_bwd_split<T, kModeSweep>(sp, g.stage_x, st, g.bwd_nw);
     else if (g.stacked) rc = g.stage_x ? launch_bwd<T, true, kModeStacked>(sp, st) : launch_bwd<T, false, kModeStacked>(sp, st);
     else rc = g.stage_x ? launch_bwd<T, true, kModeSweep>(sp, st, g.bwd_nw) : launch_bwd<T, false, kModeSweep>(sp, st, g.bwd_nw);
   } else {
     // every band on workgroups of its own, the last band first: a band waits for the one below it
     sp.nwg = g.nbands * g.vB * g.bwd_bpb;
     sp.prog = sp.link_err + 64 + (size_t)g.nbands * g.vB * (g.fwd_bpb > g.bwd_bpb ? g.fwd_bpb : g.bwd_bpb);
-    if (g.bwd_split) rc = launch_bwd_split<T, kModeSliced>(sp, g.stage_x, st);
+    if (g.bwd_split) rc = launch_bwd_split<T, kModeSliced>(sp, g.stage_x, st, g.bwd_nw);
     else rc = g.stage_x ? launch_bwd<T, true, kModeSliced>(sp, st, g.bwd_nw) : launch_bwd<T, false, kModeSliced>(sp, st, g.bwd_nw);
   }
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][1], st);
