@@ -2774,11 +2774,11 @@ int launch_fwd_split_as(const ScanParams& sp, hipStream_t st) {
   hipLaunchKernelGGL((m2d_fwd_split_kernel<T, CK, WY, SX, MODE, NWS>), dim3((unsigned)sp.nwg), dim3(NWS * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
-// (16-bit x and deltas of 8 channels are less than a 16-byte chunk per cell: read from memory, not staged)
+// (x and deltas of a workgroup's channels are one or two 16-byte chunks per cell: 8 channels of 16-bit tensors, 8 or 4 of fp32)
 template <typename T, int MODE>
 int launch_fwd_split(const ScanParams& sp, bool stage_x, bool ckpt, bool write_y, hipStream_t st, int nw = kSplitWaves) {
   if constexpr (sizeof(T) == 4) {
-    if (nw == kSplitHalfWaves) {   // (fp32 only: 4 channels of 16-bit tensors are no 16-byte chunk for the boundary rows' staging)
+    if (nw == kSplitHalfWaves) {   // (fp32 only)
       if (stage_x) {
         if (ckpt && write_y) return launch_fwd_split_as<T, true, true, true, MODE, kSplitHalfWaves>(sp, st);
         if (ckpt) return launch_fwd_split_as<T, true, false, true, MODE, kSplitHalfWaves>(sp, st);
@@ -2788,11 +2788,11 @@ int launch_fwd_split(const ScanParams& sp, bool stage_x, bool ckpt, bool write_y
       if (ckpt) return launch_fwd_split_as<T, true, false, false, MODE, kSplitHalfWaves>(sp, st);
       return launch_fwd_split_as<T, false, true, false, MODE, kSplitHalfWaves>(sp, st);
     }
-    if (stage_x) {
-      if (ckpt && write_y) return launch_fwd_split_as<T, true, true, true, MODE>(sp, st);
-      if (ckpt) return launch_fwd_split_as<T, true, false, true, MODE>(sp, st);
-      return launch_fwd_split_as<T, false, true, true, MODE>(sp, st);
-    }
+  }
+  if (stage_x) {
+    if (ckpt && write_y) return launch_fwd_split_as<T, true, true, true, MODE>(sp, st);
+    if (ckpt) return launch_fwd_split_as<T, true, false, true, MODE>(sp, st);
+    return launch_fwd_split_as<T, false, true, true, MODE>(sp, st);
   }
   if (ckpt && write_y) return launch_fwd_split_as<T, true, true, false, MODE>(sp, st);
   if (ckpt) return launch_fwd_split_as<T, true, false, false, MODE>(sp, st);
@@ -2892,15 +2892,13 @@ int launch_bwd_split_as(const ScanParams& sp, hipStream_t st) {
   hipLaunchKernelGGL((m2d_bwd_split_kernel<T, SX, MODE, NWS>), dim3((unsigned)sp.nwg), dim3(NWS * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
-// (16-bit x, deltas and dy of 8 channels are less than a 16-byte chunk per cell: read from memory, not staged)
 template <typename T, int MODE>
 int launch_bwd_split(const ScanParams& sp, bool stage_x, hipStream_t st, int nw = kSplitWaves) {
   if constexpr (sizeof(T) == 4) {
     if (nw == kSplitHalfWaves)
       return stage_x ? launch_bwd_split_as<T, true, MODE, kSplitHalfWaves>(sp, st) : launch_bwd_split_as<T, false, MODE, kSplitHalfWaves>(sp, st);
-    if (stage_x) return launch_bwd_split_as<T, true, MODE>(sp, st);
   }
-  return launch_bwd_split_as<T, false, MODE>(sp, st);
+  return stage_x ? launch_bwd_split_as<T, true, MODE>(sp, st) : launch_bwd_split_as<T, false, MODE>(sp, st);
 }
 
 template <typename T, bool SX, int MODE>
