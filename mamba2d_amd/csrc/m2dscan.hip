@@ -291,7 +291,7 @@ template <bool PERM> __device__ __forceinline__ constexpr int sinv(int pos) {
 template <typename T, int NT, int CW, bool WITH_BOT>
 struct Stage {
   static constexpr int kElem = 16 / sizeof(T);           // elements per chunk
-  static constexpr int kCpt = CW / kElem;                // chunks per tensor per cell
+  static constexpr int kCpt = CW >= kElem ? CW / kElem : 1;   // chunks per tensor per cell (fewer channels than a chunk: the chunk they are in)
   static constexpr int kXStepBytes = kCpt * kHB * 16;    // XD bytes per tensor and step
   static constexpr int kXTauBytes = kCK * kXStepBytes;   // XD bytes per tensor
   static constexpr int kXTauInstr = kXTauBytes / 1024;   // wave-wide copies per tensor
@@ -308,7 +308,7 @@ struct Stage {
   static constexpr int kBytes = kXOff + NT * kXTauBytes; // one buffer
   static_assert(kXTauBytes % 1024 == 0, "a wave-wide copy must not straddle two tensors of XD");
   static_assert(kCpt <= 2 || kCpt % 4 == 0, "a wave-wide copy of XD covers one step, or two halves of 32 lanes (one chunk per cell: XD is not staged)");
-  static_assert(CW % kElem == 0, "workgroup channel count must fill whole chunks");
+  static_assert(CW % kElem == 0 || kElem % CW == 0, "a workgroup's channels fill whole chunks, or one part of a chunk");
   static_assert(CW % 16 == 0 || CW < 16, "boundary rows are copied 16 channels at a time");
   // byte offset inside a tensor's part of XD of channel `ch` (of the workgroup) for lane row r at step 0
   static __host__ __device__ constexpr uint32_t x_off(int r, int ch) {
@@ -579,8 +579,9 @@ __device__ __forceinline__ void stage_block(const ScanParams& p, char* buf, int 
     } else if constexpr (SG::kCpt == 1) {   // all four steps per copy: lanes = (step, row); tensor tau is copied by the wave of step tau
       static_assert(kCK == 4 && NT <= kCK, "a wave-wide copy is the four steps of one tensor");
       const int cell4 = cell_at(slot);
-      const bool ok4 = ok_at(slot) && e_wg0 < p.E;
-      const uint32_t off = (uint32_t)(cell4 * p.E + e_wg0) * (uint32_t)sizeof(T);
+      const int e_chunk = e_wg0 & ~(SG::kElem - 1);   // (a workgroup of fewer channels than a chunk copies the chunk they are in)
+      const bool ok4 = ok_at(slot) && e_chunk < p.E;
+      const uint32_t off = (uint32_t)(cell4 * p.E + e_chunk) * (uint32_t)sizeof(T);
 #pragma unroll
       for (int tau = 0; tau < NT; ++tau)
         if (ks == tau && wsub == 0) {
@@ -1178,7 +1179,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
 // step.  A workgroup has 8 waves = 8 channels.  Staging, schedules and memory formats are those of
 // m2d_fwd_kernel; y of a cell is the sum over the 4 lane groups (two lane-swap steps), stored by group 0.
 constexpr int kSplitWaves = 8;
-constexpr int kSplitHalfWaves = 4;   // where workgroups of 8 would leave compute units idle (fp32 tensors)
+constexpr int kSplitHalfWaves = 4;   // where workgroups of 8 would leave compute units idle
 __device__ __forceinline__ float sum_over_groups(float v) {
   v = fold16(v, v);
   return fold32(v, v);
@@ -1256,7 +1257,7 @@ __global__ __launch_bounds__(NWS * 64) void m2d_fwd_split_kernel(const ScanParam
   const uint32_t row_off = r * 16 + g * SG::kPlane;
   const uint32_t rec_off = r == 0 ? SG::top_off(ch_loc) + g * SG::kPlane : row_off;
   const uint32_t const_off = SG::kConstPlane * SG::kPlane + r * 16;
-  const uint32_t xd_off = SG::kXOff + SG::x_off(r, ch_loc);
+  const uint32_t xd_off = SG::kXOff + SG::x_off(r, ch_loc + (CW < SG::kElem ? e_wg0 & (SG::kElem - 1) : 0));   // (4 channels of a 16-bit tensor: their half of the chunk)
   constexpr uint32_t kXK = SG::kXStepBytes;
 
   BlockPos bp;
@@ -2089,7 +2090,7 @@ __global__ __launch_bounds__(NWS * 64) void m2d_bwd_split_kernel(const ScanParam
   // above as its B_T; the lower ghost (lane 15) the row of mu_T below as its C (see m2d_bwd_kernel)
   const uint32_t rec_off = (r == 0 ? SG::top_off(ch_loc) : (r == kHB - 1 ? SG::bot_off(ch_loc) - SG::kCOff : r * 16)) + g * SG::kPlane;
   const uint32_t const_off = SG::kConstPlane * SG::kPlane + r * 16;
-  const uint32_t xd_off = SG::kXOff + SG::x_off(r, ch_loc);
+  const uint32_t xd_off = SG::kXOff + SG::x_off(r, ch_loc + (CW < SG::kElem ? e_wg0 & (SG::kElem - 1) : 0));   // (4 channels of a 16-bit tensor: their half of the chunk)
   constexpr uint32_t kXK = SG::kXStepBytes;
   // channel sums: the first 6 waves add up; wave 2v + c takes components 2c, 2c+1 of every lane's float4 of
   // tensor v.  They are kept per cell as [C, B_T, B_L][16] in the natural order of the states.
@@ -2628,8 +2629,8 @@ Geometry make_geometry(const m2d_desc* d) {
   g.fwd_split = may_split && ((d->flags & M2D_FLAG_SPLIT_STATES) || waves_whole <= 3 * ncu);
   // Workgroups of 8 waves (8 channels) under way on at most half of the compute units: workgroups of 4 then run on
   // twice as many, each wave with a SIMD to itself (a sweep of few images is as fast as one wave gets through its
-  // blocks).  fp32 tensors only.
-  const int split_nw = (d->dtype == M2D_F32 && 2 * (int64_t)B * ((d->E + kSplitWaves - 1) / kSplitWaves) * together <= ncu) ? kSplitHalfWaves : kSplitWaves;
+  // blocks).
+  const int split_nw = 2 * (int64_t)B * ((d->E + kSplitWaves - 1) / kSplitWaves) * together <= ncu ? kSplitHalfWaves : kSplitWaves;
   if (g.fwd_split) {
     g.fwd_ec = 1;
     g.fwd_nw = split_nw;
@@ -2774,20 +2775,18 @@ int launch_fwd_split_as(const ScanParams& sp, hipStream_t st) {
   hipLaunchKernelGGL((m2d_fwd_split_kernel<T, CK, WY, SX, MODE, NWS>), dim3((unsigned)sp.nwg), dim3(NWS * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
-// (x and deltas of a workgroup's channels are one or two 16-byte chunks per cell: 8 channels of 16-bit tensors, 8 or 4 of fp32)
+// (x and deltas of a workgroup's channels are one or two 16-byte chunks per cell, or 4 channels of a 16-bit tensor half of one)
 template <typename T, int MODE>
 int launch_fwd_split(const ScanParams& sp, bool stage_x, bool ckpt, bool write_y, hipStream_t st, int nw = kSplitWaves) {
-  if constexpr (sizeof(T) == 4) {
-    if (nw == kSplitHalfWaves) {   // (fp32 only)
-      if (stage_x) {
-        if (ckpt && write_y) return launch_fwd_split_as<T, true, true, true, MODE, kSplitHalfWaves>(sp, st);
-        if (ckpt) return launch_fwd_split_as<T, true, false, true, MODE, kSplitHalfWaves>(sp, st);
-        return launch_fwd_split_as<T, false, true, true, MODE, kSplitHalfWaves>(sp, st);
-      }
-      if (ckpt && write_y) return launch_fwd_split_as<T, true, true, false, MODE, kSplitHalfWaves>(sp, st);
-      if (ckpt) return launch_fwd_split_as<T, true, false, false, MODE, kSplitHalfWaves>(sp, st);
-      return launch_fwd_split_as<T, false, true, false, MODE, kSplitHalfWaves>(sp, st);
+  if (nw == kSplitHalfWaves) {
+    if (stage_x) {
+      if (ckpt && write_y) return launch_fwd_split_as<T, true, true, true, MODE, kSplitHalfWaves>(sp, st);
+      if (ckpt) return launch_fwd_split_as<T, true, false, true, MODE, kSplitHalfWaves>(sp, st);
+      return launch_fwd_split_as<T, false, true, true, MODE, kSplitHalfWaves>(sp, st);
     }
+    if (ckpt && write_y) return launch_fwd_split_as<T, true, true, false, MODE, kSplitHalfWaves>(sp, st);
+    if (ckpt) return launch_fwd_split_as<T, true, false, false, MODE, kSplitHalfWaves>(sp, st);
+    return launch_fwd_split_as<T, false, true, false, MODE, kSplitHalfWaves>(sp, st);
   }
   if (stage_x) {
     if (ckpt && write_y) return launch_fwd_split_as<T, true, true, true, MODE>(sp, st);
@@ -2894,10 +2893,8 @@ int launch_bwd_split_as(const ScanParams& sp, hipStream_t st) {
 }
 template <typename T, int MODE>
 int launch_bwd_split(const ScanParams& sp, bool stage_x, hipStream_t st, int nw = kSplitWaves) {
-  if constexpr (sizeof(T) == 4) {
-    if (nw == kSplitHalfWaves)
-      return stage_x ? launch_bwd_split_as<T, true, MODE, kSplitHalfWaves>(sp, st) : launch_bwd_split_as<T, false, MODE, kSplitHalfWaves>(sp, st);
-  }
+  if (nw == kSplitHalfWaves)
+    return stage_x ? launch_bwd_split_as<T, true, MODE, kSplitHalfWaves>(sp, st) : launch_bwd_split_as<T, false, MODE, kSplitHalfWaves>(sp, st);
   return stage_x ? launch_bwd_split_as<T, true, MODE>(sp, st) : launch_bwd_split_as<T, false, MODE>(sp, st);
 }
 
