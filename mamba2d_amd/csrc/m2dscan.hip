@@ -510,6 +510,11 @@ __device__ __forceinline__ BlockPos block_pos(const ScanParams& p, Pos A, int r,
   q.in_grid = ((unsigned)q.bnd0 < (unsigned)rbands ? m0 : 0u) | ((unsigned)(q.bnd0 + 1) < (unsigned)rbands ? m1 : 0u);
   return q;
 }
+// The row by which a lane trails the head of the stream (block_pos): its own lane row -- except in a band of
+// stacked images that holds several of them, where a row trails by its place in its own image: the images do not
+// depend on each other, so the pipeline is only as deep as one image (two images of 7 rows: 7 steps instead of 14
+// to fill and to drain, 35 instead of 42 steps for a stream of 8 such images).
+__device__ __forceinline__ int skew_row(const ScanParams& p, int r) { return (p.stacked && r >= 1 && r <= p.rb) ? (r - 1) % p.Himg + 1 : r; }
 __device__ __forceinline__ int clamp_band(const ScanParams& p, int bnd) { return bnd < 0 ? 0 : (bnd >= p.nbands ? p.nbands - 1 : bnd); }
 // Stages the operands of a block of kCK steps.  A is the position of the stream index (first step
 // of the block) - 15; q and cell0 describe the lane's own row in that block (block_pos, and the cell
@@ -814,6 +819,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   }
   const int slot = lane >> kHBShift, r = lane & (kHB - 1);
   const int rbands = row_bands(p, r);
+  const int rk = STACKED ? skew_row(p, r) : r;     // the row by which the lane trails the head of the stream
   const int ch_loc = (wave * CS + slot) * EC;      // first channel of the lane inside the workgroup
   const int e_raw = e_wg0 + ch_loc;
   const bool ch_ok = e_raw < p.E;                  // idle lanes still take part in staging and barriers
@@ -1019,7 +1025,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   };
 
   Pos A = pos_of(p, m_lo * kCK - (kHB - 1));     // position of the stream index t0 - 15 (wave-uniform)
-  bp = block_pos(p, A, r, rbands);
+  bp = block_pos(p, A, rk, rbands);
   int cell0 = cell_of(p, bp.bnd0, r, bp.col0);   // cell index of the lane's position at the first step of the block
   if constexpr (SLICED) link.wait_for(link_need_fwd(0, p.sl_nbb));
   BlockPos bpq = bp;     // 16-bit direct records: the block after the next (fetched two blocks ahead)
@@ -1028,7 +1034,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   if (direct) {
     if constexpr (WIDEN) {
       bc_raw_copy<NW>(p, pin.bcd, raw, b, bp, cell0, wave, lane, true);
-      bpq = block_pos(p, pos_after(p, A, kCK), r, rbands);
+      bpq = block_pos(p, pos_after(p, A, kCK), rk, rbands);
       cellq = cell_of(p, bpq.bnd0, r, bpq.col0);
       bc_raw_copy<NW>(p, pin.bcd, raw + kRawBytes, b, bpq, cellq, wave, lane, m_lo + 1 < m_hi);
     } else {
@@ -1055,16 +1061,16 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     if (WIDEN && direct && EC == 1) {   // the next block was worked out a block ago; its records are in `raw` already
       bpn = bpq;
       celln = cellq;
-      bpq = block_pos(p, pos_after(p, An, kCK), r, rbands);
+      bpq = block_pos(p, pos_after(p, An, kCK), rk, rbands);
       cellq = cell_of(p, bpq.bnd0, r, bpq.col0);
       bc_raw_copy<NW>(p, pin.bcd, raw + rp * kRawBytes, b, bpq, cellq, wave, lane, m + 2 < m_hi);
     } else if (WIDEN && direct) {   // two channels per lane: no registers to carry a block's positions in; worked out twice
-      bpn = block_pos(p, An, r, rbands);
+      bpn = block_pos(p, An, rk, rbands);
       celln = cell_of(p, bpn.bnd0, r, bpn.col0);
-      const BlockPos q2 = block_pos(p, pos_after(p, An, kCK), r, rbands);
+      const BlockPos q2 = block_pos(p, pos_after(p, An, kCK), rk, rbands);
       bc_raw_copy<NW>(p, pin.bcd, raw + rp * kRawBytes, b, q2, cell_of(p, q2.bnd0, r, q2.col0), wave, lane, m + 2 < m_hi);
     } else {
-      bpn = block_pos(p, An, r, rbands);
+      bpn = block_pos(p, An, rk, rbands);
       celln = cell_of(p, bpn.bnd0, r, bpn.col0);
     }
     if (!last) {
@@ -1498,6 +1504,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   const int e_wg0 = eg * CW;
   const int slot = lane >> kHBShift, r = lane & (kHB - 1);
   const int rbands = row_bands(p, r);
+  const int rk = STACKED ? skew_row(p, r) : r;     // the row by which the lane trails the head of the stream
   const int ch_loc = wave * CS + slot;
   const int e_raw = e_wg0 + ch_loc;
   const bool ch_ok = e_raw < p.E;           // padding lanes/waves still take part in the barriers
@@ -1615,14 +1622,14 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
 
   Pos A = pos_of(p, (m_hi - 1) * kCK - (kHB - 1));   // position of the stream index t0 - 15 (wave-uniform)
   __syncthreads();   // the zeros are in place before the first copies land on them
-  bp = block_pos(p, A, r, rbands);
+  bp = block_pos(p, A, rk, rbands);
   int cell0 = cell_of(p, bp.bnd0, r, bp.col0);   // cell index of the lane's position at the first step of the block
   bool ck_take = snapshot_lane(p, Pos{bp.bnd0, bp.col0}, r, ch_ok);   // the lane restores a snapshot for the block to come
   if (!LATE_SNAPSHOT && !opens_group(m_hi - 1)) load_ckpt(m_hi - 1, ck_take);   // (else: after the replay that opens the first iteration)
   if constexpr (SLICED) link.wait_for(link_need_bwd(p.sl_nbb - 1, p.sl_nbb));
   // the lane's row in the block two before (A2 = position of that block): what its raw copies fetch
   auto raw_copy_for = [&](Pos A2, char* dst, bool live) {
-    const BlockPos q2 = block_pos(p, A2, r, rbands);
+    const BlockPos q2 = block_pos(p, A2, rk, rbands);
     bc_raw_copy<NW>(p, pin.bcd, dst, b, q2, cell_of(p, q2.bnd0, r, q2.col0), wave, lane, live);
   };
   int rp = 0;   // half of `raw` that the next raw copy goes to
@@ -1652,7 +1659,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
         float hq[kN];   // hq[4 * mg + qi]: state fold_state(mg, qi), the order of the snapshot quads
         for (int q = m - mem; q < m; ++q) {   // (uniform)
           const Pos Aq = pos_of(p, q * kCK - (kHB - 1));
-          const BlockPos bq = block_pos(p, Aq, r, rbands);
+          const BlockPos bq = block_pos(p, Aq, rk, rbands);
           const int cellq = cell_of(p, bq.bnd0, r, bq.col0);
           if (direct) {
             bc_raw_copy<NW>(p, pin.bcd, raw + rp * kRawBytes, b, bq, cellq, wave, lane, true);
@@ -1735,7 +1742,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
     }
     // the block before: where the lane's row will be is also what the lane's copies fetch
     const Pos Aprev = pos_before(A);
-    const BlockPos bpn = block_pos(p, Aprev, r, rbands);
+    const BlockPos bpn = block_pos(p, Aprev, rk, rbands);
     const int celln = cell_of(p, bpn.bnd0, r, bpn.col0);
     ck_take = snapshot_lane(p, Pos{bpn.bnd0, bpn.col0}, r, ch_ok);
     if (direct) raw_copy_for(pos_before(Aprev), raw + rp * kRawBytes, m - 2 >= m_lo);
@@ -2550,7 +2557,7 @@ Geometry make_geometry(const m2d_desc* d) {
       const int vB = (d->B + ips - 1) / ips;
       const int nb = (ips * d->H + rb_stacked - 1) / rb_stacked;
       const int64_t rounds = ((int64_t)vB * groups + ncu - 1) / ncu;
-      const int64_t cost = rounds * ((nb - 1) * S + d->W + kRB + 8);
+      const int64_t cost = rounds * ((nb - 1) * S + d->W + d->H + 8);
       if (best < 0 || cost < best) { best = cost; g.ips = ips; }
     }
     if (g.ips > 1) {
@@ -2569,7 +2576,7 @@ Geometry make_geometry(const m2d_desc* d) {
   // such dependence.
   if (g.stacked) {
     g.S = d->W > 7 ? d->W : 7;
-    g.T_total = (g.nbands - 1) * g.S + d->W + kRB;
+    g.T_total = (g.nbands - 1) * g.S + d->W + d->H;   // (the rows of an image trail its first row: skew_row)
   } else {
     g.S = (g.nbands > 1 && d->W >= 26) ? d->W : (d->W + kHB - 1 > 26 ? d->W + kHB - 1 : 26);
     g.T_total = (g.nbands - 1) * g.S + d->W + g.rows_last;
