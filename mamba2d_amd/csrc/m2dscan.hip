@@ -196,7 +196,7 @@ struct ScanParams {
   int S;                            // stream stride: positions per band (>= W)
   int T_total;                      // steps of the whole sweep
   int rows_last;                    // grid rows of the last band
-  int rb;                           // grid rows of every other band: 14 (kRB), or for stacked images the largest multiple of the image height below 15
+  int rb;                           // grid rows of every other band: 14 (kRB), or for stacked images the largest multiple of the image height up to 16
   uint32_t magicS;                  // floor(2^32 / S)
   // Linked sweep (few images, many bands): every band has its own workgroups, all in one launch; a
   // band publishes how many blocks of its window are done (boundary rows in memory) and the band
@@ -207,7 +207,7 @@ struct ScanParams {
   uint32_t* link_err;               // set to 1 by a workgroup that gave up waiting (results are then invalid)
   int64_t bot_stride;               // floats between the mu_T rows of consecutive bands (0: one row buffer, bands in sequence)
   int pa_slots;                     // partial sums over positions per image (1, or one per band when sliced)
-  // Stacked images (grids of one band whose height divides 14): `ips` images in a row of the batch
+  // Stacked images (grids of at most 16 rows, one band each): `ips` images in a row of the batch
   // are swept as one tall image whose bands do not depend on each other: B, H above are then the
   // number and height of the stacks, and a workgroup shortens H for a last, shorter stack.
   int stacked, ips, Himg, Breal;    // on/off, images per stack, rows per image, images in the batch
@@ -246,9 +246,12 @@ __device__ __forceinline__ Pos pos_of(const ScanParams& p, int s) {
   return o;
 }
 __device__ __forceinline__ int band_rows(const ScanParams& p, int bnd) { return bnd == p.nbands - 1 ? p.rows_last : p.rb; }
+// Row of its band that lane row r works on: lanes 1 .. 14 the rows 0 .. 13, lane 0 (-1) and lane 15 the ghosts of the
+// rows next to the band.  The bands of stacked images have no neighbours to replay: all 16 lanes are rows there.
+__device__ __forceinline__ int grid_row(const ScanParams& p, int r) { return p.stacked ? r : r - 1; }
 // cell index inside its image of lane row r of band bnd at column col
 __device__ __forceinline__ int cell_of(const ScanParams& p, int bnd, int r, int col) {
-  const int cell = __mul24(bnd * p.rb + r - 1, p.W) + col;   // rows and columns are far below 2^24
+  const int cell = __mul24(bnd * p.rb + grid_row(p, r), p.W) + col;   // rows and columns are far below 2^24
   return p.flip ? p.H * p.W - 1 - cell : cell;
 }
 
@@ -456,9 +459,10 @@ __device__ __forceinline__ LaneK lane_consts(const ScanParams& p, int bnd, int r
   // `bnd` is a band of the grid (callers clamp): a row that is before the first band or past the
   // last one works on zero operands with the constants of that band
   LaneK c;
-  c.real = ch_ok && r >= 1 && r <= band_rows(p, bnd);
+  const int gr = grid_row(p, r);
+  c.real = ch_ok && gr >= 0 && gr < band_rows(p, bnd);
   // grid row 0 of an image: no row above (stacked images: a band holds whole images)
-  const bool first_row = p.stacked ? (r - 1) % p.Himg == 0 : (bnd == 0 && r == 1);
+  const bool first_row = p.stacked ? gr % p.Himg == 0 : (bnd == 0 && gr == 0);
   const bool gbot = BWD && !p.stacked && r == kHB - 1 && bnd + 1 < p.nbands;
   c.oT = gbot ? 0.f : (!c.real || first_row ? ninf : -1.f);
   c.oL = !c.real ? ninf : (first_row ? 0.f : -1.f);
@@ -476,7 +480,8 @@ __device__ __forceinline__ bool snapshot_lane(const ScanParams& p, Pos at, int r
   Pos pv;
   pv.bnd = at.col >= 1 ? at.bnd : at.bnd - 1;
   pv.col = at.col >= 1 ? at.col - 1 : p.S - 1;
-  const bool row_ok = r == 0 ? pv.bnd >= 1 : r <= band_rows(p, pv.bnd);
+  const int gr = grid_row(p, r);
+  const bool row_ok = gr < 0 ? pv.bnd >= 1 : gr < band_rows(p, pv.bnd);
   return ch_ok && (unsigned)pv.bnd < (unsigned)p.nbands && pv.col < p.W && row_ok;
 }
 
@@ -492,7 +497,8 @@ struct BlockPos {
 // Lane row r is a row of the grid in the bands 0 .. row_bands(r) - 1 (none for a ghost lane; a row
 // beyond the height of the last band misses that one).  A lane constant.
 __device__ __forceinline__ int row_bands(const ScanParams& p, int r) {
-  return (r >= 1 && r <= p.rb) ? p.nbands - 1 + (r <= p.rows_last ? 1 : 0) : 0;
+  const int gr = grid_row(p, r);
+  return (gr >= 0 && gr < p.rb) ? p.nbands - 1 + (gr < p.rows_last ? 1 : 0) : 0;
 }
 // bits k < n of a block's steps
 __device__ __forceinline__ uint32_t steps_below(int n) { return (1u << (n < 0 ? 0 : (n > kCK ? kCK : n))) - 1u; }
@@ -514,7 +520,7 @@ __device__ __forceinline__ BlockPos block_pos(const ScanParams& p, Pos A, int r,
 // stacked images that holds several of them, where a row trails by its place in its own image: the images do not
 // depend on each other, so the pipeline is only as deep as one image (two images of 7 rows: 7 steps instead of 14
 // to fill and to drain, 35 instead of 42 steps for a stream of 8 such images).
-__device__ __forceinline__ int skew_row(const ScanParams& p, int r) { return (p.stacked && r >= 1 && r <= p.rb) ? (r - 1) % p.Himg + 1 : r; }
+__device__ __forceinline__ int skew_row(const ScanParams& p, int r) { return (p.stacked && r < p.rb) ? r % p.Himg : r; }   // (stacked: from 0, lane 0 is a row)
 __device__ __forceinline__ int clamp_band(const ScanParams& p, int bnd) { return bnd < 0 ? 0 : (bnd >= p.nbands ? p.nbands - 1 : bnd); }
 // Stages the operands of a block of kCK steps.  A is the position of the stream index (first step
 // of the block) - 15; q and cell0 describe the lane's own row in that block (block_pos, and the cell
@@ -875,15 +881,16 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   const char* DLimg = reinterpret_cast<const char*>(DL) + img_bytes;
   const uint32_t estep = (uint32_t)(p.flip ? -p.E : p.E) * (uint32_t)sizeof(T);   // one column further
 
-  const float g1 = r == 0 ? 1.f : 0.f;             // the ghost's T input coefficient
+  const float g1 = !STACKED && r == 0 ? 1.f : 0.f;   // the ghost's T input coefficient
   const uint32_t wrap_adj = (uint32_t)(p.rb * p.W - p.S) * estep;   // extra offset of a cell reached through a band change
 
   // byte offsets of the lane's operand groups inside a staging buffer (step 0, group 0): a grid row
   // reads B_T, B_L, C of its cell; the ghost reads the row above as its B_T (and row 0 of the B_L and C
   // planes, zeros, as stand-ins for the other two, which it multiplies by 0)
   const uint32_t row_off = r * 16;
-  const uint32_t rec_off = r == 0 ? SG::top_off(ch_loc) : row_off;
-  const uint32_t rec_cstep = r == 0 ? 16 : 0;   // the ghost reads a record per channel, grid rows share theirs
+  const bool ghost = !STACKED && r == 0;   // (stacked images: no row above a band to replay, lane 0 is a row like the others)
+  const uint32_t rec_off = ghost ? SG::top_off(ch_loc) : row_off;
+  const uint32_t rec_cstep = ghost ? 16 : 0;   // the ghost reads a record per channel, grid rows share theirs
   const uint32_t xd_off = SG::kXOff + SG::x_off(r, ch_loc);
   constexpr uint32_t kXK = SG::kXStepBytes;   // XD bytes per step
 
@@ -1549,7 +1556,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   // The neighbouring records that a ghost reads in the other two places are finite and meet zeros.
   // The other two reads of a ghost land 4 and 8 planes from its boundary row: boundary rows of other
   // channels, operands of other rows or planes nobody writes, finite all of them, and they meet zeros.
-  const uint32_t rec_off = r == 0 ? SG::top_off(ch_loc) : (r == kHB - 1 ? SG::bot_off(ch_loc) - SG::kCOff : r * 16);
+  const uint32_t rec_off = STACKED ? r * 16 : (r == 0 ? SG::top_off(ch_loc) : (r == kHB - 1 ? SG::bot_off(ch_loc) - SG::kCOff : r * 16));
   const uint32_t xd_off = SG::kXOff + SG::x_off(r, ch_loc);
   constexpr uint32_t kXK = SG::kXStepBytes;   // XD bytes per step
   // The sum that this thread adds up in the exchange belongs to its own lane row r: one float of
@@ -1562,7 +1569,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   const int f_comp = PAIRS ? 0 : f_combo & 1;
   const int f_it = f_v * 64 + f_s * kHB + r;
   const uint32_t f_sub = (uint32_t)(f_v * kN + f_s * 4 + f_comp) * (uint32_t)sizeof(float);
-  const float g1 = r == 0 ? 1.f : 0.f;
+  const float g1 = !STACKED && r == 0 ? 1.f : 0.f;   // (stacked images: all 16 lanes are rows, see grid_row)
 
   const uint32_t estep = (uint32_t)(p.flip ? -p.E : p.E) * (uint32_t)sizeof(T);   // one column further
   const uint32_t wrap_adj = (uint32_t)(p.rb * p.W - p.S) * estep;   // extra offset of a cell reached through a band change
@@ -1573,7 +1580,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   // depends on it
   BlockPos bp;
   // 1 on the lower ghost: lambda = 1 * (row of mu_T below), which is staged as zeros where there is no band below
-  const float gb1 = r == kHB - 1 ? 1.f : 0.f;
+  const float gb1 = !STACKED && r == kHB - 1 ? 1.f : 0.f;
   const uint32_t row_const_off = SG::kConstPlane * SG::kPlane + r * 16;   // the row's constants at step 0 of a staging buffer
   uint32_t cell_off0 = 0;       // byte offset in a (H,W,E) image of the lane's cell at the first step of the block
   uint32_t f_off0 = 0;          // byte offset in the channel-sum image of this thread's sum at the first step
@@ -2540,16 +2547,17 @@ Geometry make_geometry(const m2d_desc* d) {
   // Grids of a single band (14x14, 7x7, 10x10 ...): a sweep spends as many steps filling and
   // draining the 16-lane pipeline as working.  `ips` consecutive images of the batch are then
   // stacked into one tall image whose bands do not depend on each other and swept back to back with
-  // stride S = W; a band holds as many whole images as fit 14 rows (two of 7 rows, one of 10, four
-  // of 3), so no image straddles two bands.  ips is chosen for the fewest steps over all rounds of
+  // stride S = W; a band holds as many whole images as fit the 16 lanes (two of 7 or 8 rows, one of
+  // 10 or 16, five of 3: no row above or below a band is needed, so the two outer lanes are rows
+  // too), so no image straddles two bands.  ips is chosen for the fewest steps over all rounds of
   // workgroups (one workgroup per CU at a time).
   g.stacked = false; g.ips = 1; g.vB = d->B; g.vH = d->H;
   g.rb = kRB;
-  const int rb_stacked = d->H <= kRB ? kRB / d->H * d->H : kRB;
+  const int rb_stacked = d->H <= kHB ? kHB / d->H * d->H : kRB;   // (all 16 lanes are rows: the bands of a stack have no neighbours)
   // (a longer checkpoint interval is for grids whose snapshots weigh: images are not stacked then, nor are the states
   // of a channel split over lanes, and every schedule left runs m2d_bwd_kernel, the one kernel that replays)
   g.ck_shift = d->ckpt_interval == 16 ? 2 : (d->ckpt_interval == 8 ? 1 : 0);
-  if (d->H <= kRB && d->B >= 2 && g.ck_shift == 0) {
+  if (d->H <= kHB && d->B >= 2 && g.ck_shift == 0) {
     const int S = d->W > 7 ? d->W : 7;
     int64_t best = -1;
     for (int ips = 1; ips <= 64 && ips <= d->B; ++ips) {

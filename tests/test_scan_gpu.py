@@ -119,12 +119,17 @@ SHAPES = [
     (900, 2, 5, 2),   # 2-row images, several to a band
     (1, 512, 512, 2), # 37 bands of one large image (linked sweep at the size of the latency benchmark's second point)
     (2, 300, 260, 4), # 22 bands, two images
-    (303, 10, 3, 12), # over 256 images of 10 rows: one image per band of a stack, 4 lane rows idle (once asked for two channels per lane in fp32, which does not fit the LDS)
-    (601, 5, 9, 8),   # 5-row images stacked, two to a band (bands of 10 rows), last stack shorter
+    (303, 10, 3, 12), # over 256 images of 10 rows: one image per band of a stack, 6 lane rows idle (once asked for two channels per lane in fp32, which does not fit the LDS)
+    (601, 5, 9, 8),   # 5-row images stacked, three to a band (bands of 15 rows), last stack shorter
     (530, 12, 12, 16), # 12x12 (the last stage of a 384x384 input) stacked, one image per band of 12 rows
-    (700, 3, 17, 4),  # 3-row images stacked, four to a band of 12 rows
+    (700, 3, 17, 4),  # 3-row images stacked, five to a band of 15 rows
     (300, 13, 6, 2),  # 13 rows: one image per band
-    (400, 8, 8, 32),  # 8x8 stacked, one image per band of 8 rows, full workgroup of channels
+    (400, 8, 8, 32),  # 8x8 stacked, two images per band of 16 rows (the two outer lanes are rows in a stack), full workgroup of channels
+    (300, 16, 16, 32), # 16x16 stacked: a band is one image on all 16 lanes
+    (601, 15, 15, 6), # 15 rows: lane 0 is a row, lane 15 idle; last stack shorter
+    (1003, 4, 4, 8),  # four images of 4 rows on the 16 lanes, one band per stack
+    (3000, 2, 2, 4),  # eight images of 2 rows per band
+    (129, 8, 8, 512), # last stage of a 256x256 input at full width: 9 images per stream, the last band half filled
     (37, 5, 9, 8),    # few 5-row images: one stream per image
     (1, 28, 70, 8),   # two long bands of one image: linked sweep
     (2, 40, 100, 4),  # three long bands of two images: linked sweep
