@@ -148,7 +148,11 @@ def test_plan_names_kernel_and_schedule(cabi):
     whole = cabi.scan_plan(1, 256, 256, 64, torch.float32, cabi.M2D_PASS_FWD, flags=cabi.M2D_FLAG_WHOLE_STATES)
     assert whole.startswith("m2d_fwd_kernel: linked sweep, 19 bands") and "16 states per lane" in whole
     small = cabi.scan_plan(128, 7, 7, 512, torch.bfloat16, cabi.M2D_PASS_FWD)
-    assert small.startswith("m2d_fwd_kernel: stacked images")
+    assert small.startswith("m2d_fwd_kernel: stacked images, 8 per stream, 4 bands")   # two images of 7 rows per band
+    # the bands of a stack have no neighbours: all 16 lanes are rows (two 8-row images or one 16-row image per band)
+    assert cabi.scan_plan(128, 8, 8, 512, torch.bfloat16, cabi.M2D_PASS_BWD).startswith("m2d_bwd_kernel: stacked images, 8 per stream, 4 bands")
+    assert cabi.scan_plan(128, 16, 16, 320, torch.bfloat16, cabi.M2D_PASS_BWD).startswith("m2d_bwd_kernel: stacked images, 6 per stream, 6 bands")
+    assert cabi.scan_plan(2001, 3, 3, 8, torch.float32, cabi.M2D_PASS_FWD).startswith("m2d_fwd_kernel: stacked images, 8 per stream, 2 bands")   # five per band
     # a short buffer truncates, a bad descriptor reports its status and an empty text
     buf = ctypes.create_string_buffer(8)
     assert cabi.lib.m2d_scan_plan(ctypes.byref(D(cabi)), 0, buf, 8) == 0 and len(buf.value) == 7
