@@ -2769,26 +2769,38 @@ int stage_bc(ScanParams& sp, const m2d_desc* d, const void* BT, const void* BL, 
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
+// Development aid: -DM2D_QUICK builds only the kernels of many 16-bit images in one stream each, in workgroups of
+// 8 waves (a twentieth of the compile time); every other problem then answers M2D_ERR_UNSUPPORTED.
+#ifdef M2D_QUICK
+#define M2D_BUILT(T, SX, MODE, NW, OTHER) (sizeof(T) == 2 && (SX) && (MODE) == kModeSweep && (NW) == 8 && (OTHER))
+#else
+#define M2D_BUILT(T, SX, MODE, NW, OTHER) true
+#endif
+
 template <typename T, int EC, bool CK, bool WY, bool SX, int MODE, int NW>
 int launch_fwd_as(const ScanParams& sp, hipStream_t st) {
+  if constexpr (!M2D_BUILT(T, SX, MODE, NW, EC == 1)) return M2D_ERR_UNSUPPORTED; else {
   constexpr size_t lds = fwd_lds_bytes<T, EC, NW>();
   if (lds > kLdsPerWorkgroup) return M2D_ERR_UNSUPPORTED;   // (make_geometry never picks such a layout)
   static std::atomic<uint64_t> seen{0};
   if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_fwd_kernel<T, EC, CK, WY, SX, MODE, NW>), lds, seen)) return M2D_ERR_HIP;
   hipLaunchKernelGGL((m2d_fwd_kernel<T, EC, CK, WY, SX, MODE, NW>), dim3((unsigned)sp.nwg), dim3(NW * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+  }
 }
 
 template <typename T, int NWS = kSplitWaves>
 constexpr size_t fwd_split_lds_bytes() { return 2 * (size_t)Stage<T, 3, NWS, false>::kBytes + (sizeof(T) == 2 ? 2 * kRawBytes : 0); }
 template <typename T, bool CK, bool WY, bool SX, int MODE, int NWS = kSplitWaves>
 int launch_fwd_split_as(const ScanParams& sp, hipStream_t st) {
+  if constexpr (!M2D_BUILT(T, SX, MODE, NWS, false)) return M2D_ERR_UNSUPPORTED; else {
   constexpr size_t lds = fwd_split_lds_bytes<T, NWS>();
   static_assert(lds <= kLdsPerWorkgroup, "staging must fit the LDS");
   static std::atomic<uint64_t> seen{0};
   if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_fwd_split_kernel<T, CK, WY, SX, MODE, NWS>), lds, seen)) return M2D_ERR_HIP;
   hipLaunchKernelGGL((m2d_fwd_split_kernel<T, CK, WY, SX, MODE, NWS>), dim3((unsigned)sp.nwg), dim3(NWS * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+  }
 }
 // (x and deltas of a workgroup's channels are one or two 16-byte chunks per cell, or 4 channels of a 16-bit tensor half of one)
 template <typename T, int MODE>
@@ -2886,11 +2898,13 @@ int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
 
 template <typename T, bool SX, int MODE, int NW, bool REPLAY = false>
 int launch_bwd_as(const ScanParams& sp, hipStream_t st) {
+  if constexpr (!M2D_BUILT(T, SX, MODE, NW, !REPLAY)) return M2D_ERR_UNSUPPORTED; else {
   constexpr size_t lds = bwd_lds_bytes<T, NW>();
   static std::atomic<uint64_t> seen{0};
   if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_bwd_kernel<T, SX, MODE, NW, REPLAY>), lds, seen)) return M2D_ERR_HIP;
   hipLaunchKernelGGL((m2d_bwd_kernel<T, SX, MODE, NW, REPLAY>), dim3((unsigned)sp.nwg), dim3(NW * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+  }
 }
 
 template <typename T, int NWS = kSplitWaves>
@@ -2899,12 +2913,14 @@ constexpr size_t bwd_split_lds_bytes() {
 }
 template <typename T, bool SX, int MODE, int NWS = kSplitWaves>
 int launch_bwd_split_as(const ScanParams& sp, hipStream_t st) {
+  if constexpr (!M2D_BUILT(T, SX, MODE, NWS, false)) return M2D_ERR_UNSUPPORTED; else {
   constexpr size_t lds = bwd_split_lds_bytes<T, NWS>();
   static_assert(lds <= kLdsPerWorkgroup, "exchange buffers and staging must fit the LDS");
   static std::atomic<uint64_t> seen{0};
   if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_bwd_split_kernel<T, SX, MODE, NWS>), lds, seen)) return M2D_ERR_HIP;
   hipLaunchKernelGGL((m2d_bwd_split_kernel<T, SX, MODE, NWS>), dim3((unsigned)sp.nwg), dim3(NWS * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+  }
 }
 template <typename T, int MODE>
 int launch_bwd_split(const ScanParams& sp, bool stage_x, hipStream_t st, int nw = kSplitWaves) {

@@ -154,3 +154,21 @@ def test_two_stage_backbone_with_interleaved_directions(dtype, tol):
     e = so.rel_err(got, want)
     print(f"  rel_err {e:.3e}", flush=True)
     assert got.shape == want.shape == (2, 128, 12, 8) and e < tol
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, 3e-2)], ids=["f32", "bf16"])
+def test_m2d_t_full_depth_at_224(dtype, tol):
+    """The M2D-T backbone as the benchmark configuration runs it -- blocks [3, 3, 9, 3], channels [64, 128, 320,
+    512], scan mixers with the local path at stages 1-2 (odd blocks from the bottom-right corner), rotary attention
+    at stages 3-4 -- on one 3x224x224 image, every parameter randomised, against the float64 restatement of
+    models/mamba2d.py:340-386 fed the same state dict."""
+    from mamba2d_amd.backbone import M2D_T, Mamba2DBackbone
+    print(f"\ncase M2D-T [3,3,9,3] at 1x3x224x224 {dtype}", flush=True)
+    net = randomize(Mamba2DBackbone(**M2D_T), 41)
+    x = torch.randn(1, 3, 224, 224, generator=torch.Generator().manual_seed(42))
+    got = on_gpu(net, x, dtype)
+    want = bo.backbone(x.to(dtype).double(), ref_state(net, dtype), M2D_T["n_blocks"], M2D_T["inter_flip"])
+    e = so.rel_err(got, want)
+    print(f"  rel_err {e:.3e}", flush=True)
+    assert got.shape == want.shape == (1, 512, 7, 7) and e < tol
