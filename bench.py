@@ -351,7 +351,7 @@ def main():
     ap.add_argument("--workload", default="cfg1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-ckpt", action="store_true", help="rebuild checkpoints inside the backward")
-    ap.add_argument("--ckpt-interval", type=int, default=0, choices=(0, 4, 8, 16),
+    ap.add_argument("--ckpt-interval", type=int, default=0, choices=(0, 2, 4, 8, 16),
                     help="steps between the state snapshots the forward keeps (0 or 4: the default; 8, 16: fewer "
                          "snapshots, and the backward replays the forward in between)")
     ap.add_argument("--dtype", default=None, choices=("f32", "bf16"),
@@ -370,7 +370,7 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     from mamba2d_amd import cabi, wavefront
-    wavefront.CKPT_INTERVAL = cabi.CKPT_INTERVAL = args.ckpt_interval
+    cabi.CKPT_INTERVAL = args.ckpt_interval
 
     if args.workload == "cfg3":
         backbone_inference(args)

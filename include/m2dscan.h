@@ -60,11 +60,17 @@ typedef struct m2d_desc {
   int32_t dtype;              /* m2d_dtype */
   int32_t flags;
   int32_t ckpt_interval;      /* steps between the state snapshots that m2d_scan_fwd keeps for m2d_scan_bwd:
-                                 0 (the default) or 4, 8, 16.  A longer interval shrinks the snapshot part of
-                                 the checkpoint buffer in proportion; the backward then replays the forward
-                                 over the steps in between (4 or 12 of every 8 or 16) before it sweeps them.
-                                 The forward and the backward of one problem must use the same value.
-                                 Ignored by the m2d_proj_* entry points. */
+                                 0 (the library chooses), 2, 4, 8 or 16.
+                                 2: two snapshots per block of 4 steps; the backward then recomputes one step in two
+                                    and computes every gate once (its kernel is bound by instruction issue, not by
+                                    memory: it trades bytes for instructions).  Only where every image (or stack of
+                                    small images) is swept as one stream with all 16 states of a channel in one lane;
+                                    the other schedules (few large images) keep 4, also when 2 is asked for.
+                                 4: one snapshot per block; the backward recomputes the block.
+                                 8, 16: a half / a quarter of the snapshots of 4; the backward replays the forward
+                                    over the blocks in between (4 or 12 steps of every 8 or 16) before it sweeps them.
+                                 0 picks 2 where it exists, else 4.  The forward and the backward of one problem
+                                 must use the same value.  Ignored by the m2d_proj_* entry points. */
 } m2d_desc;
 
 #define M2D_FLAG_FLIP 1
@@ -118,8 +124,8 @@ int m2d_desc_check(const m2d_desc* desc);
  * Returns 0 for an invalid descriptor. */
 size_t m2d_scan_workspace_bytes(const m2d_desc* desc, int pass, int have_ckpt);
 
-/* Bytes of the checkpoint buffer (anti-diagonal state snapshots every desc->ckpt_interval steps, 4 by
- * default, plus band-boundary rows; linear in H*W, at the default about 1/4 of the reference's hs tensor:
+/* Bytes of the checkpoint buffer (anti-diagonal state snapshots every desc->ckpt_interval steps
+ * plus band-boundary rows; linear in H*W, at 4 steps about 1/4 of the reference's hs tensor, at 2 steps 1/2:
  * the snapshots have the width of the tensors' type, fp32 or bf16, as every state of hs has in the
  * reference, wf_cuda.cu:5,59-67). */
 size_t m2d_scan_ckpt_bytes(const m2d_desc* desc);

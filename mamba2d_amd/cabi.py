@@ -124,10 +124,26 @@ def check(code: int) -> None:
 # M2D_FLAG_SPLIT_STATES or M2D_FLAG_WHOLE_STATES to override the library's choice of lane layout in
 # scan_fwd / scan_bwd (0: the library decides); the tests run every case all three ways.
 SCHEDULE_HINT = 0
-# Steps between the state snapshots that the forward keeps for the backward (m2d_desc.ckpt_interval): 0 or 4
-# (the default), 8 or 16.  Longer intervals shrink the checkpoint buffer and make the backward replay the
+# Steps between the state snapshots that the forward keeps for the backward (m2d_desc.ckpt_interval).  0: the
+# library chooses (2 for batches of images swept one stream each, 4 for few large images); 2 or 4: that interval
+# where the schedule has it; 8 or 16: a half or a quarter of the snapshots of 4, and the backward replays the
 # forward over the steps in between.  Set once, before the forward of a problem, and leave until its backward.
-CKPT_INTERVAL = 0
+# The one switch of the package (mamba2d_amd.wavefront reads it here); environment: M2D_CKPT_INTERVAL.
+CKPT_INTERVALS = (0, 2, 4, 8, 16)
+
+
+def _interval_from_env() -> int:
+    text = os.environ.get("M2D_CKPT_INTERVAL", "0")
+    try:
+        v = int(text)
+    except ValueError:
+        v = None
+    if v not in CKPT_INTERVALS:
+        raise ValueError(f"m2dscan: M2D_CKPT_INTERVAL must be one of {CKPT_INTERVALS}, got {text!r}")
+    return v
+
+
+CKPT_INTERVAL = _interval_from_env()
 
 
 def make_desc(x: torch.Tensor, N: int, flip: bool = False) -> Desc:

@@ -39,6 +39,7 @@
 #include <cstdio>
 #include <cstring>
 #include <stdint.h>
+#include <type_traits>
 
 #include "../../include/m2dscan.h"
 
@@ -182,7 +183,7 @@ struct ScanParams {
   const float *A2T, *A2L, *Df;      // A*log2(e) and D in fp32, (E,16) / (E)
   const float* zeros;               // 256 bytes of zeros (source for out-of-grid staging chunks)
   void *y, *dx, *ddT, *ddL;
-  float* ckpt;                      // [B][ck_nblk][E][4][16][4]     state snapshots, one per kept block of steps: [q][row][w] = state sinv(4q+w); bf16 for 16-bit tensors
+  float* ckpt;                      // [B][ck_nblk][E][2][16][2][4]  state snapshots, one per kept block of steps: quad q of lane row r (see snap_quad) holds the states sinv(4q .. 4q+3); bf16 for 16-bit tensors
   float* top;                       // [nbands-1][B][W][E][16]       last row of each band (forward states)
   float* bot;                       // [nbands or 1][B][W][E][16]    first-row muT of a band, for the band above (adjoint)
   float* part;                      // [G][P][3][16]                 per-workgroup channel sums of d_C, d_BT, d_BL
@@ -219,6 +220,7 @@ struct ScanParams {
   // of a workgroup's window); the backward replays the forward over the other blocks of a group before it sweeps
   // the group, and parks their snapshots in `ring`.
   int ck_shift;
+  int ck_half;                      // a snapshot every 2 steps (before the steps 0 and 2 of every block, and one behind the last block): snapshot 2m + s is the state before step 4m + 2s
   int ck_pb;                        // kept snapshots per band (linked sweep)
   int ck_nblk;                      // kept snapshots per image
   void* ring;                       // [workgroup][2^ck_shift - 1][channel of the workgroup][4][16] snapshot quads
@@ -746,6 +748,9 @@ template <> struct Snap<float> {
   static __device__ __forceinline__ float4 load(const quad* src) { return widen(*src); }
   static __device__ __forceinline__ quad zero() { return f4v{0.f, 0.f, 0.f, 0.f}; }
   static __device__ __forceinline__ float4 widen(quad v) { return make_float4(v.x, v.y, v.z, v.w); }
+  // two neighbouring quads (a half of the states)
+  static __device__ __forceinline__ void load2(const quad* src, quad (&dst)[2]) { dst[0] = src[0]; dst[1] = src[1]; }
+  static __device__ __forceinline__ void store2(quad* dst, quad a, quad b) { __builtin_nontemporal_store(a, dst); __builtin_nontemporal_store(b, dst + 1); }
 };
 template <> struct Snap<bf16_t> {
   typedef u2v quad;
@@ -762,8 +767,20 @@ template <> struct Snap<bf16_t> {
   static __device__ __forceinline__ float4 widen(quad v) {
     return make_float4(__uint_as_float(v.x << 16), __uint_as_float(v.x & 0xffff0000u), __uint_as_float(v.y << 16), __uint_as_float(v.y & 0xffff0000u));
   }
+  // two neighbouring quads (a half of the states): one 16-byte piece
+  typedef unsigned int u4v __attribute__((ext_vector_type(4)));
+  static __device__ __forceinline__ void load2(const quad* src, quad (&dst)[2]) {
+    const u4v v = *reinterpret_cast<const u4v*>(src);
+    dst[0] = u2v{v.x, v.y}; dst[1] = u2v{v.z, v.w};
+  }
+  static __device__ __forceinline__ void store2(quad* dst, quad a, quad b) { __builtin_nontemporal_store(u4v{a.x, a.y, b.x, b.y}, reinterpret_cast<u4v*>(dst)); }
 };
-// first quad of the kept snapshot number mi (snapshot_index) of channel e of image b: [b][kept block][E][4 state groups][16 lane rows]
+// Inside the 64 quads of one channel's snapshot, the quads of lane row r: quad q (state group q) sits at
+// snap_lane(r) + snap_quad(q).  The two quads of a half of the states (0, 1 and 2, 3) are neighbours, so that a lane
+// moves them as one piece (16 bytes of bf16 states in one instruction): [half of the states][16 lane rows][2 quads].
+__device__ __forceinline__ constexpr int snap_quad(int q) { return (q >> 1) * (2 * kHB) + (q & 1); }
+__device__ __forceinline__ int snap_lane(int r) { return 2 * r; }
+// first quad of the kept snapshot number mi (snapshot_index) of channel e of image b: [b][kept block][E][2 halves of the states][16 lane rows][2 quads]
 // (nkept: kept snapshots per image, p.ck_nblk.  A kernel that only runs at the default interval passes p.nblk and
 // the block itself: it then needs none of the interval's parameters, which would cost it scalar registers.)
 template <typename T>
@@ -783,9 +800,11 @@ __device__ __forceinline__ int snapshot_index(const ScanParams& p, int m, int m_
 // what the lane below hands to a cell comes from the cell above it.  Only stores are predicated.
 // NW waves per workgroup: 8, or 4 where the batch is too small to give every compute unit a
 // workgroup of 8 (each wave then has a SIMD to itself).
-template <typename T, int EC, bool CKPT, bool WRITE_Y, bool STAGE_X, int MODE, int NW = kFwdWaves>
+// HALF: a snapshot every 2 steps instead of every 4 (m2d_bwd2_kernel restarts from them), and one more behind the sweep.
+template <typename T, int EC, bool CKPT, bool WRITE_Y, bool STAGE_X, int MODE, int NW = kFwdWaves, bool HALF = false>
 __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) {
   constexpr bool SLICED = MODE == kModeSliced, STACKED = MODE == kModeStacked;
+  static_assert(!HALF || (CKPT && !SLICED), "snapshots every 2 steps: kept by a forward of one stream per image or stack");
   ScanParams p = pin;   // (stacked images: the height is shortened below for a last, shorter stack)
   if constexpr (!STACKED) {   // lets the compiler drop what only stacked images need
     __builtin_assume(p.stacked == 0);
@@ -941,6 +960,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
 #pragma unroll
     for (int n = 0; n < kN; ++n) h[c][n] = 0.f;
   typename Snap<T>::quad* ckp = nullptr;      // where the lane stores its snapshot in the first step of the current block
+  typename Snap<T>::quad* ckp2 = nullptr;     // ... and (HALF) in its third step
   int ypar = 0;                 // window that the current block fills
   const uint32_t y_lane_off = (uint32_t)(wave * YT::kRegion + (r * CS + slot) * EC * (int)sizeof(T));
   auto step = [&](int k, const Ops& o) {
@@ -952,6 +972,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
       const float sT = __builtin_fmaf(cT * o.dtv[c], o.xv[c], g1);
       const float sL = cL * o.dlv[c] * o.xv[c];
       float acc = 0.f;
+      typename Snap<T>::quad pend = Snap<T>::zero();   // a quad that waits for its neighbour (16-bit snapshots: two bf16 quads leave as one 16-byte store)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const float4 b4 = o.bt[c][q], l4 = o.bl[q], c4 = o.cc[q];
@@ -969,9 +990,11 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
         for (int w = 0; w < 4; ++w) aL[w] = fexp2(__builtin_fmaf(o.dlv[c], a2l[c][sinv<PERM>(4 * q + w)], offL));
         pin4(aL);
         __builtin_amdgcn_sched_barrier(0);
-        if (CKPT && k == 0)   // the four states as they are before this step
-          Snap<T>::store(ckp + (c * 4 + q) * kHB, h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)],
-                         h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
+        if (CKPT && (k == 0 || (HALF && k == 2))) {   // the four states as they are before this step: stored with their neighbours' quad
+          const typename Snap<T>::quad pk = Snap<T>::pack(h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)], h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
+          if ((q & 1) == 0) pend = pk;
+          else Snap<T>::store2((k == 0 ? ckp : ckp2) + c * (kN / 4 * kHB) + snap_quad(q - 1), pend, pk);
+        }
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
           const int n = sinv<PERM>(4 * q + w);
@@ -1103,9 +1126,12 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     // the other lanes write to their own place all the same.  Channels past E, whose place is
     // another channel's, and blocks whose snapshot is not kept (block 0; a longer checkpoint
     // interval) write to the image's place for block 0, which nobody reads.
-    if constexpr (CKPT) {
+    if constexpr (CKPT && HALF) {   // snapshots 2m and 2m + 1 (snapshot 0, the state before the sweep, is the place nobody reads)
+      ckp = snapshot_at<T>(p, b, (m > 0 && ch_ok) ? 2 * m : 0, e0, p.ck_nblk) + snap_lane(r);
+      ckp2 = snapshot_at<T>(p, b, ch_ok ? 2 * m + 1 : 0, e0, p.ck_nblk) + snap_lane(r);
+    } else if constexpr (CKPT) {
       const bool keep = m > 0 && snapshot_kept(p, m, m_lo);
-      ckp = snapshot_at<T>(p, b, (keep && ch_ok) ? snapshot_index<SLICED>(p, m, m_lo, my_band) : 0, e0, p.ck_nblk) + r;
+      ckp = snapshot_at<T>(p, b, (keep && ch_ok) ? snapshot_index<SLICED>(p, m, m_lo, my_band) : 0, e0, p.ck_nblk) + snap_lane(r);
     }
     const char* bufc = lds + cur * SG::kBytes;
     const char* bufn = lds + (cur ^ 1) * SG::kBytes;
@@ -1127,7 +1153,10 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
           if (y_thrice) staging_landed_behind<2>(); else staging_landed();
         }
       } else if constexpr (CKPT) {
-        if (y_thrice) staging_landed_behind<4 * EC + 3>(); else staging_landed_behind<4 * EC>();
+        // snapshot stores of the steps before the last: per channel and snapshot two 16-byte pieces of bf16 quads or four fp32 quads
+        // (counting too few only waits longer, too many reads operands that have not landed; the wait's field counts to 15)
+        constexpr int kSnaps = (HALF ? 2 : 1) * EC * (sizeof(T) == 2 ? 2 : 4);
+        if (y_thrice) staging_landed_behind<(kSnaps + 3 < 15 ? kSnaps + 3 : 15)>(); else staging_landed_behind<(kSnaps < 15 ? kSnaps : 15)>();
       } else {
         if (y_thrice) staging_landed_behind<3>(); else staging_landed();
       }
@@ -1176,6 +1205,16 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   if constexpr (YTILE && AHEAD) {   // the last step of the sweep
     __syncthreads();
     flush_y(ypar, m_hi, true);
+  }
+  if constexpr (CKPT && HALF) {   // the state behind the last block: what the last step of the sweep left is among it
+    typename Snap<T>::quad* end = snapshot_at<T>(p, b, ch_ok ? 2 * p.nblk : 0, e0, p.ck_nblk) + snap_lane(r);
+#pragma unroll
+    for (int c = 0; c < EC; ++c)
+#pragma unroll
+      for (int q = 0; q < 4; q += 2)
+        Snap<T>::store2(end + c * (kN / 4 * kHB) + snap_quad(q),
+                        Snap<T>::pack(h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)], h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]),
+                        Snap<T>::pack(h[c][sinv<PERM>(4 * q + 4)], h[c][sinv<PERM>(4 * q + 5)], h[c][sinv<PERM>(4 * q + 6)], h[c][sinv<PERM>(4 * q + 7)]));
   }
   if constexpr (SLICED) {   // the whole window is done once every store of every wave has completed
     __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -1390,7 +1429,7 @@ __global__ __launch_bounds__(NWS * 64) void m2d_fwd_split_kernel(const ScanParam
     cell_off0 = (uint32_t)(cell0 * p.E + e0) * (uint32_t)sizeof(T);
     if constexpr (CKPT) {   // every lane stores, without a branch inside the step: see m2d_fwd_kernel
       const bool keep = m > 0 && snapshot_kept(p, m, m_lo);
-      ckp = snapshot_at<T>(p, b, (keep && ch_ok) ? snapshot_index<SLICED>(p, m, m_lo, my_band) : 0, e0, p.ck_nblk) + g * kHB + r;
+      ckp = snapshot_at<T>(p, b, (keep && ch_ok) ? snapshot_index<SLICED>(p, m, m_lo, my_band) : 0, e0, p.ck_nblk) + snap_lane(r) + snap_quad(g);
     }
     const char* bufc = lds + cur * SG::kBytes;
     // (uniform) stores that the wave is sure to issue in the first three steps, after the copies for the
@@ -1600,13 +1639,13 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   // past E point at the last channel's place: they park nothing and use nothing).
   auto snapshot_of_lane = [&](int mm) {
     if constexpr (!REPLAY) {   // the default interval: a snapshot for every block, as before
-      return snapshot_at<T>(p, b, mm, e, p.nblk) + r;
+      return snapshot_at<T>(p, b, mm, e, p.nblk) + snap_lane(r);
     } else {
       const int mem = member(mm);
       typename Snap<T>::quad* base =
           mem != 0 ? static_cast<typename Snap<T>::quad*>(p.ring) + ((int64_t)blockIdx.x * ((1 << p.ck_shift) - 1) + (mem - 1)) * kRingSlot - e_wg0 * (kN / 4 * kHB)
                    : snapshot_at<T>(p, b, snapshot_index<SLICED>(p, mm, m_lo, my_band), 0, p.ck_nblk);
-      return base + (e * (kN / 4 * kHB) + r);
+      return base + (e * (kN / 4 * kHB) + snap_lane(r));
     }
   };
   // the sweep enters a group at block mm, and the block has no snapshot: the replay brings its state
@@ -1618,7 +1657,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
     } else {
       const typename Snap<T>::quad* ck = snapshot_of_lane(mm);
 #pragma unroll
-      for (int q = 0; q < 4; ++q) cknext[q] = ck[q * kHB];
+      for (int q = 0; q < 4; q += 2) Snap<T>::load2(ck + snap_quad(q), *reinterpret_cast<typename Snap<T>::quad(*)[2]>(&cknext[q]));
     }
   };
   auto pos_before = [&](Pos Q) {   // kCK positions earlier
@@ -1684,7 +1723,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
             const typename Snap<T>::quad* ck = snapshot_of_lane(q);
 #pragma unroll
             for (int mg = 0; mg < 4; ++mg) {
-              const float4 v = take_q ? Snap<T>::load(ck + mg * kHB) : make_float4(0.f, 0.f, 0.f, 0.f);
+              const float4 v = take_q ? Snap<T>::load(ck + snap_quad(mg)) : make_float4(0.f, 0.f, 0.f, 0.f);
               hq[4 * mg + 0] = v.x; hq[4 * mg + 1] = v.y; hq[4 * mg + 2] = v.z; hq[4 * mg + 3] = v.w;
             }
           } else {
@@ -1740,7 +1779,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
           typename Snap<T>::quad* park = snapshot_of_lane(q + 1);   // the states before block q + 1
 #pragma unroll
           for (int mg = 0; mg < 4; ++mg)
-            if (ch_ok) park[mg * kHB] = Snap<T>::pack(hq[4 * mg], hq[4 * mg + 1], hq[4 * mg + 2], hq[4 * mg + 3]);   // (channels past E have no place of their own)
+            if (ch_ok) park[snap_quad(mg)] = Snap<T>::pack(hq[4 * mg], hq[4 * mg + 1], hq[4 * mg + 2], hq[4 * mg + 3]);   // (channels past E have no place of their own)
           __syncthreads();   // every wave is done with the buffer before the next block's copies land in it
         }
         if constexpr (!LATE_SNAPSHOT) load_ckpt(m, ck_take);
@@ -2020,6 +2059,437 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   }
 }
 
+// --------------------------------------------------- backward from snapshots every 2 steps
+// The same adjoint as m2d_bwd_kernel for a forward that kept the state before the steps 0 and 2 of every block
+// (and the state behind the last block): the kernel is out of instruction issue slots long before it is out of
+// memory bandwidth, so it reads twice the snapshots and recomputes one step in two instead of all four, and
+// computes the gates of every step once instead of 1.75 times.  A block is swept as two sub-blocks of 2 steps,
+// each in two halves of 8 states (the registers of a lane hold no more): restore the state before the sub-block,
+// recompute the state between its two steps keeping that step's gates, take the state behind the sub-block from
+// the snapshot after it, and run the adjoint over the two steps.  The snapshot quads of a half-pass are fetched
+// while the half-pass before is worked on.  Channel sums cross the waves through two exchange sets per half of
+// the states, used alternately by the half-passes: one barrier per half-pass, and the sums of one half are added
+// up while the other half is computed.
+// Schedules: one stream per image, or stacked images (not the linked sweep, whose problems are few large images
+// where the snapshots weigh most).
+template <typename T, int NW>
+constexpr int bwd2_exchange_sets() {   // sets of [wave][3][64] float2: 2 halves x 2 steps where they fit, else 2 used alternately per step
+  return sizeof(float2) * 4 * NW * 3 * 64 + sizeof(float) * NW * 4 * 2 * kN + 256 +
+         2 * (size_t)Stage<T, 4, NW * 4, true>::kBytes + (sizeof(T) == 2 ? 2 * kRawBytes : 0) <= 160 * 1024 ? 4 : 2;
+}
+template <typename T, bool STAGE_X, int MODE, int NW = kBwdWaves>
+__global__ __launch_bounds__(NW * 64) void m2d_bwd2_kernel(const ScanParams pin) {
+  static_assert(MODE != kModeSliced, "the linked sweep keeps a snapshot every 4 steps");
+  constexpr bool STACKED = MODE == kModeStacked;
+  ScanParams p = pin;   // (stacked images: the height is shortened below for a last, shorter stack)
+  if constexpr (!STACKED) {
+    __builtin_assume(p.stacked == 0);
+    __builtin_assume(p.rb == kRB);
+    __builtin_assume(p.S >= kHB + kCK - 1);
+  }
+  static_assert(kCK == 4, "two sub-blocks of 2 steps");
+  constexpr int CS = 64 >> kHBShift;     // 4 channel slots
+  constexpr int SLOT = 3 * 64;           // float2s per wave in one exchange set
+  constexpr int CW = NW * CS;
+  constexpr bool PERM = true;
+  using SG = Stage<T, 4, CW, true>;
+  extern __shared__ float4 smem[];
+  constexpr int XSETS = bwd2_exchange_sets<T, NW>();
+  constexpr bool BATCH = XSETS == 4;
+  float2* slots = reinterpret_cast<float2*>(smem);                       // BATCH: [half][step of the sub-block][wave][3][64], else [2][wave][3][64]
+  float* a_lds = reinterpret_cast<float*>(slots + XSETS * NW * SLOT);    // [wave][CS][2][16], fold order
+  char* lds = reinterpret_cast<char*>(a_lds + NW * CS * 2 * kN);         // 2 staging buffers
+  constexpr bool WIDEN = sizeof(T) == 2;
+  char* raw = lds + 2 * SG::kBytes;         // [2][kRawBytes]: 16-bit B_T, B_L, C on their way
+  const bool direct = WIDEN && p.bc_direct != 0;   // (uniform)
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int lb = logical_block(p.nwg);
+  const int m_hi = p.nblk;
+  const int b = lb / p.bpb;
+  const int eg = lb % p.bpb;
+  if constexpr (STACKED) {   // the last stack of the batch may hold fewer images
+    const int nimg = p.Breal - b * p.ips < p.ips ? p.Breal - b * p.ips : p.ips;
+    p.H = nimg * p.Himg;
+    p.nbands = (p.H + p.rb - 1) / p.rb;
+    p.rows_last = p.H - (p.nbands - 1) * p.rb;
+  }
+  const int e_wg0 = eg * CW;
+  const int slot = lane >> kHBShift, r = lane & (kHB - 1);
+  const int rbands = row_bands(p, r);
+  const int rk = STACKED ? skew_row(p, r) : r;
+  const int ch_loc = wave * CS + slot;
+  const int e_raw = e_wg0 + ch_loc;
+  const bool ch_ok = e_raw < p.E;
+  const int e = ch_ok ? e_raw : p.E - 1;
+  {  // A of the wave's channels into LDS in fold order (read back group by group)
+    float* mine = a_lds + ch_loc * (2 * kN);
+    mine[spos<true>(r)] = p.A2T[e * kN + r];
+    mine[kN + spos<true>(r)] = p.A2L[e * kN + r];
+  }
+  for (int i = threadIdx.x; i < 2 * SG::kBytes / 16; i += NW * 64) reinterpret_cast<float4*>(lds)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+  const uint32_t a_base_off = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) float*)(a_lds + ch_loc * (2 * kN)));
+  const float dsk = p.Df[e];
+  settle_loads();
+
+  const T* X = static_cast<const T*>(p.x);
+  const T* DT = static_cast<const T*>(p.dT);
+  const T* DL = static_cast<const T*>(p.dL);
+  const T* DY = static_cast<const T*>(p.dy);
+  const int64_t img_cell0 = (int64_t)b * p.Hs * p.W;
+  const int64_t img_bytes = img_cell0 * p.E * (int64_t)sizeof(T);
+  const char* Ximg = reinterpret_cast<const char*>(X) + img_bytes;
+  const char* DTimg = reinterpret_cast<const char*>(DT) + img_bytes;
+  const char* DLimg = reinterpret_cast<const char*>(DL) + img_bytes;
+  const char* DYimg = reinterpret_cast<const char*>(DY) + img_bytes;
+  char* DXimg = static_cast<char*>(p.dx) + img_bytes;
+  char* DDTimg = static_cast<char*>(p.ddT) + img_bytes;
+  char* DDLimg = static_cast<char*>(p.ddL) + img_bytes;
+  char* BOTimg = reinterpret_cast<char*>(p.bot + (int64_t)b * p.W * p.E * kN);
+  char* PARTimg = reinterpret_cast<char*>(p.part + ((int64_t)eg * p.Ptot + img_cell0) * (3 * kN));
+
+  float accAT[kN], accAL[kN], accD = 0.f;
+  float muT[kN], muL[kN];
+#pragma unroll
+  for (int n = 0; n < kN; ++n) { accAT[n] = 0.f; accAL[n] = 0.f; muT[n] = 0.f; muL[n] = 0.f; }
+  const uint32_t rec_off = STACKED ? r * 16 : (r == 0 ? SG::top_off(ch_loc) : (r == kHB - 1 ? SG::bot_off(ch_loc) - SG::kCOff : r * 16));
+  const uint32_t xd_off = SG::kXOff + SG::x_off(r, ch_loc);
+  constexpr uint32_t kXK = SG::kXStepBytes;
+  // the sum that this thread adds up in the exchange: see m2d_bwd_kernel
+  constexpr bool PAIRS = NW * 64 < 2 * SLOT;
+  const int f_combo = wave * 4 + slot;
+  const bool f_on = f_combo < (PAIRS ? 12 : 24);
+  const int f_v = PAIRS ? f_combo >> 2 : f_combo >> 3, f_s = PAIRS ? f_combo & 3 : (f_combo >> 1) & 3;
+  const int f_comp = PAIRS ? 0 : f_combo & 1;
+  const int f_it = f_v * 64 + f_s * kHB + r;
+  const uint32_t f_sub = (uint32_t)(f_v * kN + f_s * 4 + f_comp) * (uint32_t)sizeof(float);
+  const float g1 = !STACKED && r == 0 ? 1.f : 0.f;
+  const float gb1 = !STACKED && r == kHB - 1 ? 1.f : 0.f;
+  const uint32_t estep = (uint32_t)(p.flip ? -p.E : p.E) * (uint32_t)sizeof(T);
+  const uint32_t wrap_adj = (uint32_t)(p.rb * p.W - p.S) * estep;
+  const uint32_t pstep = (uint32_t)(p.flip ? -1 : 1) * (uint32_t)(3 * kN * sizeof(float));
+  const uint32_t pwrap_adj = (uint32_t)(p.rb * p.W - p.S) * pstep;
+  const uint32_t row_const_off = SG::kConstPlane * SG::kPlane + r * 16;
+
+  BlockPos bp;
+  uint32_t cell_off0 = 0, f_off0 = 0;
+  typedef typename Snap<T>::quad quad_t;
+  // The two quads (8 states) of snapshot `idx` that half `hf` of the states works on, as they come from memory
+  // (take: the forward left the lane's own state there, see snapshot_lane; snapshot 0 is the state before the sweep).
+  auto load_snap = [&](quad_t (&dst)[2], int idx, int hf, bool take) {
+    if (idx == 0 || !take) {
+      dst[0] = Snap<T>::zero(); dst[1] = Snap<T>::zero();
+    } else {
+      Snap<T>::load2(snapshot_at<T>(p, b, idx, e, p.ck_nblk) + snap_lane(r) + snap_quad(2 * hf), dst);
+    }
+  };
+  auto widen8 = [&](const quad_t (&src)[2], float (&dst)[8]) {
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+      const float4 v = Snap<T>::widen(src[q]);
+      dst[4 * q + 0] = v.x; dst[4 * q + 1] = v.y; dst[4 * q + 2] = v.z; dst[4 * q + 3] = v.w;
+    }
+  };
+  auto pos_at = [&](const BlockPos& q, int k) {   // the row's position at step k of the block (k <= kCK: one band change at most)
+    Pos o;
+    const bool w = k >= q.kw;
+    o.bnd = w ? q.bnd0 + 1 : q.bnd0;
+    o.col = w ? k - q.kw : q.col0 + k;
+    return o;
+  };
+  auto pos_before = [&](Pos Q) {
+    Q.col -= kCK;
+    if (Q.col < 0) { Q.col += p.S; Q.bnd -= 1; }
+    return Q;
+  };
+
+  Pos A = pos_of(p, (m_hi - 1) * kCK - (kHB - 1));
+  __syncthreads();   // the zeros are in place before the first copies land on them
+  bp = block_pos(p, A, rk, rbands);
+  int cell0 = cell_of(p, bp.bnd0, r, bp.col0);
+  // take[s]: whether the lane restores snapshot 2m + s of the block being swept (the states before its steps 0 and
+  // 2 and behind its step 3)
+  bool take0 = snapshot_lane(p, Pos{bp.bnd0, bp.col0}, r, ch_ok), take1 = snapshot_lane(p, pos_at(bp, 2), r, ch_ok);
+  const bool take2 = snapshot_lane(p, pos_at(bp, kCK), r, ch_ok);
+  // Snapshot quads on their way, per half of the states: qa[half] the state before the sub-block that the half's next
+  // half-pass sweeps (fetched two half-passes ahead: when the half's pass before starts), qn[half] the state behind
+  // that sub-block, which is the state before the sub-block that the half swept last (its qa, kept as it came).
+  quad_t qa[2][2], qn[2][2];
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf) {
+    load_snap(qa[hf], 2 * (m_hi - 1) + 1, hf, take1);
+    load_snap(qn[hf], 2 * (m_hi - 1) + 2, hf, take2);
+  }
+  auto raw_copy_for = [&](Pos A2, char* dst, bool live) {
+    const BlockPos q2 = block_pos(p, A2, rk, rbands);
+    bc_raw_copy<NW>(p, pin.bcd, dst, b, q2, cell_of(p, q2.bnd0, r, q2.col0), wave, lane, live);
+  };
+  int rp = 0;
+  if (direct) {
+    bc_raw_copy<NW>(p, pin.bcd, raw, b, bp, cell0, wave, lane, true);
+    raw_copy_for(pos_before(A), raw + kRawBytes, m_hi - 2 >= 0);
+    stage_block<T, 4, CW, true, STAGE_X, NW, true>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+    staging_fence();
+    bc_widen<SG, NW>(raw, lds, wave, lane);
+  } else {
+    stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+  }
+  staging_fence();
+  int cur = 0;
+  int xpar = 0;   // (one set per step: the exchange set in use)
+
+  for (int m = m_hi - 1; m >= 0; --m) {
+    const int t0 = m * kCK;
+    const char* bufc = lds + cur * SG::kBytes;
+    const Pos Aprev = pos_before(A);
+    const BlockPos bpn = block_pos(p, Aprev, rk, rbands);
+    const int celln = cell_of(p, bpn.bnd0, r, bpn.col0);
+    const bool take0n = snapshot_lane(p, Pos{bpn.bnd0, bpn.col0}, r, ch_ok), take1n = snapshot_lane(p, pos_at(bpn, 2), r, ch_ok);
+    if (direct) raw_copy_for(pos_before(Aprev), raw + rp * kRawBytes, m - 2 >= 0);
+    if (m > 0) {
+      if (direct) {
+        stage_block<T, 4, CW, true, STAGE_X, NW, true>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+        bc_widen<SG, NW>(raw + (rp ^ 1) * kRawBytes, lds + (cur ^ 1) * SG::kBytes, wave, lane);
+      } else {
+        stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+      }
+    }
+    rp ^= 1;
+    cell_off0 = (uint32_t)(cell0 * p.E + e) * (uint32_t)sizeof(T);
+    f_off0 = (uint32_t)cell0 * (uint32_t)(3 * kN * sizeof(float)) + (BATCH ? (uint32_t)(slot * 4 * sizeof(float)) : f_sub);
+
+#pragma unroll
+    for (int sub = 1; sub >= 0; --sub) {
+      const int k0 = 2 * sub;
+      float part2[2][4];   // the state sums of the first half wait here for the second
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        float ha[8], hb1[8], hn[8], gT[8], gL[8];
+        widen8(qa[half], ha);
+        widen8(qn[half], hn);
+        qn[half][0] = qa[half][0]; qn[half][1] = qa[half][1];
+        // the quads of this half's next pass (the first sub-block's passes fetch behind this block's copies for the
+        // second sub-block, the second's for the block to come, in time for that block's wait for everything in flight)
+        if (sub == 1) load_snap(qa[half], 2 * m, half, take0);
+        else if (m > 0) load_snap(qa[half], 2 * (m - 1) + 1, half, take1n);
+        // ---- recompute the state between the two steps
+        if (t0 + k0 < p.T_total) {
+          const int k = k0;
+          const float4 kk = *reinterpret_cast<const float4*>(bufc + (row_const_off + k * SG::kKStr));
+          const float offT = kk.x, offL = kk.y, cT = kk.z, cL = kk.w;
+          float xv = 0.f, dtv = 0.f, dlv = 0.f;
+          if constexpr (STAGE_X) {
+            const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
+            xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + SG::kXTauBytes / sizeof(T)); dlv = IO<T>::ld(xr + 2 * SG::kXTauBytes / sizeof(T));
+          } else if (ch_ok && ((bp.in_grid >> k) & 1u)) {
+            const uint32_t off = cell_off0 + (uint32_t)k * estep + (k >= bp.kw ? wrap_adj : 0u);
+            xv = IO<T>::ld(reinterpret_cast<const T*>(Ximg + off));
+            dtv = IO<T>::ld(reinterpret_cast<const T*>(DTimg + off));
+            dlv = IO<T>::ld(reinterpret_cast<const T*>(DLimg + off));
+          }
+          uint32_t a_off = a_base_off;
+          asm volatile("" : "+v"(a_off));
+          const lds_float4* a_mine = (const lds_float4*)(uintptr_t)a_off;
+          const char* rec = bufc + (rec_off + k * SG::kKStr);
+          const float sT = __builtin_fmaf(cT * dtv, xv, g1);
+          const float sL = cL * dlv * xv;
+#pragma unroll
+          for (int mgl = 0; mgl < 2; ++mgl) {
+            const int mg = 2 * half + mgl;
+            const v4f_t at4 = a_mine[mg], al4 = a_mine[kN / 4 + mg];
+            const float4 b4 = *reinterpret_cast<const float4*>(rec + mg * SG::kPlane);
+            const float4 l4 = *reinterpret_cast<const float4*>(rec + SG::kBLOff + mg * SG::kPlane);
+            const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
+            const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w};
+            float aT[4], aL[4];   // gates before chains, see the forward kernel
+#pragma unroll
+            for (int qi = 0; qi < 4; ++qi) aT[qi] = fexp2(__builtin_fmaf(dtv, atq[qi], offT));
+            pin4(aT);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int qi = 0; qi < 4; ++qi) aL[qi] = fexp2(__builtin_fmaf(dlv, alq[qi], offL));
+            pin4(aL);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int qi = 0; qi < 4; ++qi) {
+              const int s8 = 4 * mgl + qi;
+              float u = sL * lq[qi];
+              u = __builtin_fmaf(sT, bq[qi], u);
+              u = fma_row_below(aT[qi], ha[s8], u);
+              hb1[s8] = __builtin_fmaf(aL[qi], ha[s8], u);
+              gT[s8] = aT[qi]; gL[s8] = aL[qi];
+            }
+          }
+        }
+        // ---- adjoint over the sub-block, second step first
+#pragma unroll
+        for (int ks = 1; ks >= 0; --ks) {
+          const int k = k0 + ks;
+          const int t = t0 + k;
+          if (sub == 0 && half == 1 && ks == 0) staging_landed();   // before the last stores of the block, see the forward kernel
+          if (t < p.T_total) {
+            const float (&hbk)[8] = ks == 1 ? hb1 : ha;    // the state before this step
+            const float (&hnk)[8] = ks == 1 ? hn : hb1;    // ... and behind it
+            const float4 kk = *reinterpret_cast<const float4*>(bufc + (row_const_off + k * SG::kKStr));
+            const float offT = kk.x, offL = kk.y, cT = kk.z, cL = kk.w;
+            const bool inr = ch_ok && ((bp.in_grid >> k) & 1u);
+            const uint32_t goff = cell_off0 + (uint32_t)k * estep + (k >= bp.kw ? wrap_adj : 0u);
+            float xv = 0.f, dtv = 0.f, dlv = 0.f, dyv = 0.f;
+            if constexpr (STAGE_X) {
+              const T* xr = reinterpret_cast<const T*>(bufc + xd_off + k * kXK);
+              xv = IO<T>::ld(xr); dtv = IO<T>::ld(xr + SG::kXTauBytes / sizeof(T)); dlv = IO<T>::ld(xr + 2 * SG::kXTauBytes / sizeof(T));
+              dyv = IO<T>::ld(xr + 3 * SG::kXTauBytes / sizeof(T));
+            } else if (inr) {
+              xv = IO<T>::ld(reinterpret_cast<const T*>(Ximg + goff));
+              dtv = IO<T>::ld(reinterpret_cast<const T*>(DTimg + goff));
+              dlv = IO<T>::ld(reinterpret_cast<const T*>(DLimg + goff));
+              dyv = IO<T>::ld(reinterpret_cast<const T*>(DYimg + goff));
+            }
+            uint32_t a_off = a_base_off;
+            asm volatile("" : "+v"(a_off));
+            const lds_float4* a_mine = (const lds_float4*)(uintptr_t)a_off;
+            const char* rec = bufc + (rec_off + k * SG::kKStr);
+            const float qT = cT * dtv * xv, qL = cL * dlv * xv;   // zero on lanes that are not grid cells
+            const float dyl = dyv + gb1;
+            float sT = 0.f, sL = 0.f, zT = 0.f, zL = 0.f;
+            if (half == 1) { sT = part2[ks][0]; sL = part2[ks][1]; zT = part2[ks][2]; zL = part2[ks][3]; }
+            float* sw = reinterpret_cast<float*>(slots + ((BATCH ? 2 * half + ks : xpar) * NW + wave) * SLOT + lane);
+#pragma unroll
+            for (int mgl = 0; mgl < 2; ++mgl) {
+              const int mg = 2 * half + mgl;
+              const v4f_t at4 = a_mine[mg], al4 = a_mine[kN / 4 + mg];
+              const float4 b4 = *reinterpret_cast<const float4*>(rec + mg * SG::kPlane);
+              const float4 l4 = *reinterpret_cast<const float4*>(rec + SG::kBLOff + mg * SG::kPlane);
+              const float4 c4 = *reinterpret_cast<const float4*>(rec + SG::kCOff + mg * SG::kPlane);
+              const float atq[4] = {at4.x, at4.y, at4.z, at4.w}, alq[4] = {al4.x, al4.y, al4.z, al4.w};
+              const float bq[4] = {b4.x, b4.y, b4.z, b4.w}, lq[4] = {l4.x, l4.y, l4.z, l4.w}, cq[4] = {c4.x, c4.y, c4.z, c4.w};
+              float vC[4], vBT[4], vBL[4];
+#pragma unroll
+              for (int qi = 0; qi < 4; ++qi) {
+                const int n = fold_state(mg, qi), s8 = 4 * mgl + qi;
+                const float a2t = atq[qi], a2l = alq[qi];
+                const float aT = ks == 0 ? gT[s8] : fexp2(__builtin_fmaf(dtv, a2t, offT));
+                const float aL = ks == 0 ? gL[s8] : fexp2(__builtin_fmaf(dlv, a2l, offL));
+                const float lam = __builtin_fmaf(dyl, cq[qi], add_row_above(muL[n], muT[n]));
+                const float mT = aT * lam, mL = aL * lam;
+                muT[n] = mT;
+                muL[n] = mL;
+                const float ZT = mul_row_below(mT, hbk[s8]), ZL = mL * hbk[s8];
+                accAT[n] = __builtin_fmaf(ZT, dtv, accAT[n]);
+                accAL[n] = __builtin_fmaf(ZL, dlv, accAL[n]);
+                zT = __builtin_fmaf(ZT, a2t, zT);
+                zL = __builtin_fmaf(ZL, a2l, zL);
+                sT = __builtin_fmaf(lam, bq[qi], sT);
+                sL = __builtin_fmaf(lam, lq[qi], sL);
+                vBT[qi] = qT * lam;
+                vBL[qi] = qL * lam;
+                vC[qi] = dyv * hnk[s8];
+              }
+              sw[mgl] = fold16(fold32(vC[0], vC[1]), fold32(vC[2], vC[3]));
+              sw[64 * 2 + mgl] = fold16(fold32(vBT[0], vBT[1]), fold32(vBT[2], vBT[3]));
+              sw[128 * 2 + mgl] = fold16(fold32(vBL[0], vBL[1]), fold32(vBL[2], vBL[3]));
+            }
+            if (p.nbands > 1 && !p.stacked) {   // first row of a band: the lower ghost of the band above will replay its muT
+              const bool wk = k >= bp.kw;
+              if (inr && r == 1 && (wk ? bp.bnd0 + 1 : bp.bnd0) >= 1) {
+                const int ck = wk ? bp.col0 + k - p.S : bp.col0 + k;
+                char* bb = BOTimg + (wk ? bp.bnd0 + 1 : bp.bnd0) * p.bot_stride * (int64_t)sizeof(float) +
+                           (uint32_t)(ck * p.E + e) * (uint32_t)(kN * sizeof(float));
+#pragma unroll
+                for (int q = 2 * half; q < 2 * half + 2; ++q)
+                  reinterpret_cast<float4*>(bb)[q] = make_float4(muT[sinv<PERM>(4 * q)], muT[sinv<PERM>(4 * q + 1)], muT[sinv<PERM>(4 * q + 2)], muT[sinv<PERM>(4 * q + 3)]);
+              }
+            }
+            if (half == 0) {
+              part2[ks][0] = sT; part2[ks][1] = sL; part2[ks][2] = zT; part2[ks][3] = zL;
+            } else {
+              accD = __builtin_fmaf(dyv, xv, accD);
+              if (inr) {
+                float gdT = __builtin_fmaf(cT * xv, sT, kLn2 * zT), gdL = __builtin_fmaf(cL * xv, sL, kLn2 * zL);
+                if (p.dpre) {   // (uniform) gradients with respect to what the softplus was applied to
+                  gdT *= softplus_slope<T>(dtv);
+                  gdL *= softplus_slope<T>(dlv);
+                }
+                IO<T>::st(reinterpret_cast<T*>(DDTimg + goff), gdT);
+                IO<T>::st(reinterpret_cast<T*>(DDLimg + goff), gdL);
+                IO<T>::st(reinterpret_cast<T*>(DXimg + goff), __builtin_fmaf(cT * dtv, sT, __builtin_fmaf(cL * dlv, sL, dyv * dsk)));
+              }
+            }
+            if constexpr (!BATCH) {   // ---- across the waves, this step: as in m2d_bwd_kernel
+              __syncthreads();
+              if (f_on && ((bp.in_grid >> k) & 1u)) {
+                const uint32_t off = f_off0 + (uint32_t)k * pstep + (k >= bp.kw ? pwrap_adj : 0u) + (uint32_t)(2 * half * sizeof(float));
+                if constexpr (PAIRS) {
+                  const float2* sl = slots + xpar * NW * SLOT + f_it;
+                  float2 s = sl[0];
+#pragma unroll
+                  for (int w = 1; w < NW; ++w) { s.x += sl[w * SLOT].x; s.y += sl[w * SLOT].y; }
+                  *reinterpret_cast<float2*>(PARTimg + off) = s;
+                } else {
+                  const float* sl = reinterpret_cast<const float*>(slots + xpar * NW * SLOT + f_it) + f_comp;
+                  float s = sl[0];
+#pragma unroll
+                  for (int w = 1; w < NW; ++w) s += sl[2 * w * SLOT];
+                  *reinterpret_cast<float*>(PARTimg + off) = s;
+                }
+              }
+              xpar ^= 1;
+            }
+          }
+        }
+        if constexpr (BATCH) {
+          // ---- across the waves, both steps of this half-pass at once: the 2 x 3 (step, tensor) sets are dealt to the
+          // waves; a thread adds up the float2 of the lane (its slot, its row).  The other half's sets are being
+          // filled or added up by then; this half's are filled again two barriers from here.
+          __syncthreads();
+#pragma unroll
+          for (int rd = 0; rd < (2 * 3 + NW - 1) / NW; ++rd) {
+            const int jj = rd * NW + wave;                    // (uniform)
+            if (jj < 2 * 3) {
+              const int ks = jj / 3, v = jj - 3 * ks;
+              const int k = k0 + ks;
+              if (t0 + k < p.T_total && ((bp.in_grid >> k) & 1u)) {
+                const uint32_t off = f_off0 + (uint32_t)k * pstep + (k >= bp.kw ? pwrap_adj : 0u) + (uint32_t)((v * kN + 2 * half) * sizeof(float));
+                const float2* sl = slots + (2 * half + ks) * NW * SLOT + v * 64 + lane;
+                float2 sum = sl[0];
+#pragma unroll
+                for (int w = 1; w < NW; ++w) { sum.x += sl[w * SLOT].x; sum.y += sl[w * SLOT].y; }
+                *reinterpret_cast<float2*>(PARTimg + off) = sum;
+              }
+            }
+          }
+        }
+      }
+    }
+    if constexpr (!BATCH) __syncthreads();   // (BATCH: the barrier of the last half-pass ended the block)
+    A = Aprev;
+    bp = bpn;
+    cell0 = celln;
+    cur ^= 1;
+    take0 = take0n; take1 = take1n;
+  }
+
+  // ---- sums over positions: reduce over the rows of the band (lanes of one channel slot)
+  float red[2 * kN + 1];
+#pragma unroll
+  for (int n = 0; n < kN; ++n) { red[n] = accAT[n]; red[kN + n] = accAL[n]; }
+  red[2 * kN] = accD;
+#pragma unroll
+  for (int k = 0; k < 2 * kN + 1; ++k) {
+    float v = red[k];
+#pragma unroll
+    for (int off = kHB >> 1; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    red[k] = v;
+  }
+  if (ch_ok && r == 0) {
+    const int64_t slot_e = (int64_t)b * p.pa_slots * p.E + e;
+    float* pa = p.pA + slot_e * (2 * kN);
+#pragma unroll
+    for (int n = 0; n < 2 * kN; ++n) pa[n] = red[n];
+    p.pD[slot_e] = red[2 * kN];
+  }
+}
+
 // ------------------------------------------------------ backward, the states of a channel split over lanes
 // The counterpart of m2d_fwd_split_kernel: lane = (state group g, row r), 4 states per lane, a wave
 // per channel, 8 channels per workgroup.  With only 4 states a lane keeps the gates of all four
@@ -2126,7 +2596,11 @@ __global__ __launch_bounds__(NWS * 64) void m2d_bwd_split_kernel(const ScanParam
   typename Snap<T>::quad cknext = Snap<T>::zero();
   auto load_ckpt = [&](int mm, bool take) {   // take: the forward kept the lane's state before block mm
     cknext = Snap<T>::zero();
-    if (mm != 0 && take) cknext = *(snapshot_at<T>(p, b, mm, e, p.nblk) + g * kHB + r);   // (this kernel: a snapshot for every block)
+    if (mm != 0 && take) {
+      int ln = lane;
+      asm volatile("" : "+v"(ln));   // the lane's place is worked out here, not carried in a register across the block (the kernel has none to spare)
+      cknext = *(snapshot_at<T>(p, b, mm, e, p.nblk) + snap_lane(ln & (kHB - 1)) + snap_quad(ln >> kHBShift));
+    }   // (this kernel: a snapshot for every block)
   };
   auto pos_before = [&](Pos Q) {
     Q.col -= kCK;
@@ -2503,6 +2977,7 @@ struct Geometry {
   int nbb;                           // linked sweep: blocks per band
   size_t link_bytes;                 // linked sweep: error word and the two arrays of progress counts (forward, backward)
   int ck_shift, ck_pb, ck_nblk;      // checkpoint interval: log2 of the blocks per kept snapshot; kept snapshots per band (linked sweep) and per image
+  bool ck_half;                      // a snapshot every 2 steps: m2d_fwd_kernel<..., HALF> and m2d_bwd2_kernel
   size_t ring_bytes;                 // backward with a longer interval: the replayed snapshots of every workgroup
   bool packed_bc;
   size_t prep_bytes, bc_bytes, ckpt_diag_bytes, top_bytes, bot_bytes, part_bytes, pa_bytes, pd_bytes;
@@ -2513,7 +2988,7 @@ int check_desc(const m2d_desc* d) {
   if (d->B < 1 || d->E < 1 || d->N < 1 || d->H < 2 || d->W < 2) return M2D_ERR_BAD_SHAPE;
   if (d->N != kN) return M2D_ERR_UNSUPPORTED;
   if (d->dtype != M2D_F32 && d->dtype != M2D_BF16) return M2D_ERR_UNSUPPORTED;
-  if ((d->ckpt_interval != 0 && d->ckpt_interval != 4 && d->ckpt_interval != 8 && d->ckpt_interval != 16) || (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_RAW_PARAMS | M2D_FLAG_PACKED_BC | M2D_FLAG_DPRE | M2D_FLAG_SPLIT_STATES | M2D_FLAG_WHOLE_STATES))) return M2D_ERR_UNSUPPORTED;
+  if ((d->ckpt_interval != 0 && d->ckpt_interval != 2 && d->ckpt_interval != 4 && d->ckpt_interval != 8 && d->ckpt_interval != 16) || (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_RAW_PARAMS | M2D_FLAG_PACKED_BC | M2D_FLAG_DPRE | M2D_FLAG_SPLIT_STATES | M2D_FLAG_WHOLE_STATES))) return M2D_ERR_UNSUPPORTED;
   if ((d->flags & M2D_FLAG_SPLIT_STATES) && (d->flags & M2D_FLAG_WHOLE_STATES)) return M2D_ERR_UNSUPPORTED;
   if ((int64_t)d->B * d->H * d->W >= ((int64_t)1 << 40)) return M2D_ERR_BAD_SHAPE;
   // one image is addressed with 32-bit byte offsets from its base (fp32: 4 bytes per element;
@@ -2673,6 +3148,10 @@ Geometry make_geometry(const m2d_desc* d) {
   const int every = 1 << g.ck_shift;
   g.ck_pb = g.sliced ? (g.nbb + every - 1) / every : 0;
   g.ck_nblk = g.sliced ? g.nbands * g.ck_pb : (g.nblk + every - 1) / every;
+  // A snapshot every 2 steps, for the backward kernel that recomputes one step in two: where every image (or stack)
+  // is one stream and a lane holds all states of its channel.  Other schedules keep one every 4 steps.
+  g.ck_half = (d->ckpt_interval == 2 || d->ckpt_interval == 0) && !g.sliced && !g.fwd_split && !g.bwd_split;
+  if (g.ck_half) g.ck_nblk = 2 * g.nblk + 1;   // before the steps 0 and 2 of every block, and behind the last block
   g.ckpt_diag_bytes = align_up((d->dtype == M2D_BF16 ? 2 : sizeof(float)) * (size_t)B * g.ck_nblk * d->E * kN * g.HB);   // (16-bit tensors: bf16 snapshots)
   const size_t bwd_wgs = (size_t)(g.sliced ? g.nbands : 1) * B * g.bwd_bpb;
   g.ring_bytes = g.ck_shift ? align_up((d->dtype == M2D_BF16 ? 2 : sizeof(float)) * bwd_wgs * (every - 1) * g.bwd_nw * g.CS * kN * g.HB) : 0;
@@ -2718,7 +3197,7 @@ void fill_common(ScanParams& sp, const m2d_desc* d, const Geometry& g) {
   sp.bot_stride = g.sliced ? (int64_t)g.vB * d->W * d->E * kN : 0;
   sp.flip = (d->flags & M2D_FLAG_FLIP) ? 1 : 0;
   sp.dpre = (d->flags & M2D_FLAG_DPRE) ? 1 : 0;
-  sp.ck_shift = g.ck_shift; sp.ck_pb = g.ck_pb; sp.ck_nblk = g.ck_nblk;
+  sp.ck_shift = g.ck_shift; sp.ck_pb = g.ck_pb; sp.ck_nblk = g.ck_nblk; sp.ck_half = g.ck_half ? 1 : 0;
   sp.ring = nullptr;
 }
 
@@ -2777,14 +3256,14 @@ int stage_bc(ScanParams& sp, const m2d_desc* d, const void* BT, const void* BL, 
 #define M2D_BUILT(T, SX, MODE, NW, OTHER) true
 #endif
 
-template <typename T, int EC, bool CK, bool WY, bool SX, int MODE, int NW>
+template <typename T, int EC, bool CK, bool WY, bool SX, int MODE, int NW, bool HALF = false>
 int launch_fwd_as(const ScanParams& sp, hipStream_t st) {
   if constexpr (!M2D_BUILT(T, SX, MODE, NW, EC == 1)) return M2D_ERR_UNSUPPORTED; else {
   constexpr size_t lds = fwd_lds_bytes<T, EC, NW>();
   if (lds > kLdsPerWorkgroup) return M2D_ERR_UNSUPPORTED;   // (make_geometry never picks such a layout)
   static std::atomic<uint64_t> seen{0};
-  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_fwd_kernel<T, EC, CK, WY, SX, MODE, NW>), lds, seen)) return M2D_ERR_HIP;
-  hipLaunchKernelGGL((m2d_fwd_kernel<T, EC, CK, WY, SX, MODE, NW>), dim3((unsigned)sp.nwg), dim3(NW * 64), lds, st, sp);
+  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_fwd_kernel<T, EC, CK, WY, SX, MODE, NW, HALF>), lds, seen)) return M2D_ERR_HIP;
+  hipLaunchKernelGGL((m2d_fwd_kernel<T, EC, CK, WY, SX, MODE, NW, HALF>), dim3((unsigned)sp.nwg), dim3(NW * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
   }
 }
@@ -2827,6 +3306,9 @@ int launch_fwd_split(const ScanParams& sp, bool stage_x, bool ckpt, bool write_y
 
 template <typename T, int EC, bool SX, int MODE, int NW = kFwdWaves>
 int launch_fwd_mode(const ScanParams& sp, bool ckpt, bool write_y, hipStream_t st) {
+  if constexpr (MODE != kModeSliced) {
+    if (ckpt && sp.ck_half) return write_y ? launch_fwd_as<T, EC, true, true, SX, MODE, NW, true>(sp, st) : launch_fwd_as<T, EC, true, false, SX, MODE, NW, true>(sp, st);
+  }
   if (ckpt && write_y) return launch_fwd_as<T, EC, true, true, SX, MODE, NW>(sp, st);
   if (ckpt) return launch_fwd_as<T, EC, true, false, SX, MODE, NW>(sp, st);
   return launch_fwd_as<T, EC, false, true, SX, MODE, NW>(sp, st);
@@ -2907,6 +3389,23 @@ int launch_bwd_as(const ScanParams& sp, hipStream_t st) {
   }
 }
 
+template <typename T, int NW>
+constexpr size_t bwd2_lds_bytes() {
+  return sizeof(float2) * bwd2_exchange_sets<T, NW>() * NW * 3 * 64 + sizeof(float) * NW * 4 * 2 * kN + 256 +
+         2 * (size_t)Stage<T, 4, NW * 4, true>::kBytes + (sizeof(T) == 2 ? 2 * kRawBytes : 0);
+}
+template <typename T, bool SX, int MODE, int NW>
+int launch_bwd2_as(const ScanParams& sp, hipStream_t st) {
+  if constexpr (!M2D_BUILT(T, SX, MODE, NW, true)) return M2D_ERR_UNSUPPORTED; else {
+  constexpr size_t lds = bwd2_lds_bytes<T, NW>();
+  static_assert(lds <= kLdsPerWorkgroup, "exchange sets and staging must fit the LDS");
+  static std::atomic<uint64_t> seen{0};
+  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_bwd2_kernel<T, SX, MODE, NW>), lds, seen)) return M2D_ERR_HIP;
+  hipLaunchKernelGGL((m2d_bwd2_kernel<T, SX, MODE, NW>), dim3((unsigned)sp.nwg), dim3(NW * 64), lds, st, sp);
+  return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
+  }
+}
+
 template <typename T, int NWS = kSplitWaves>
 constexpr size_t bwd_split_lds_bytes() {
   return sizeof(float4) * 2 * NWS * 3 * 64 + 2 * (size_t)Stage<T, 4, NWS, true>::kBytes + (sizeof(T) == 2 ? 2 * kRawBytes : 0);
@@ -2931,6 +3430,12 @@ int launch_bwd_split(const ScanParams& sp, bool stage_x, hipStream_t st, int nw 
 
 template <typename T, bool SX, int MODE>
 int launch_bwd(const ScanParams& sp, hipStream_t st, int nw = kBwdWaves) {
+  if constexpr (MODE != kModeSliced) {
+    if (sp.ck_half) {   // snapshots every 2 steps
+      if constexpr (MODE != kModeStacked) { if (nw == kFwdHalfWaves) return launch_bwd2_as<T, SX, MODE, kFwdHalfWaves>(sp, st); }
+      return launch_bwd2_as<T, SX, MODE, kBwdWaves>(sp, st);
+    }
+  }
   if constexpr (MODE != kModeStacked) {
     if (sp.ck_shift > 0)   // a longer checkpoint interval: the kernel that replays the forward between snapshots
       return nw == kFwdHalfWaves ? launch_bwd_as<T, SX, MODE, kFwdHalfWaves, true>(sp, st) : launch_bwd_as<T, SX, MODE, kBwdWaves, true>(sp, st);
@@ -3115,8 +3620,9 @@ int m2d_scan_plan(const m2d_desc* desc, int pass, char* text, size_t cap) {
     snprintf(text, cap, "%s: %s, %lld workgroups of %d waves, %d channels each, 4 states per lane",
              fwd ? "m2d_fwd_split_kernel" : "m2d_bwd_split_kernel", sched, wgs, nw, nw);
   else
-    snprintf(text, cap, "%s: %s, %lld workgroups of %d waves, %d channels each, 16 states per lane",
-             fwd ? "m2d_fwd_kernel" : "m2d_bwd_kernel", sched, wgs, nw, nw * g.CS * per_lane);
+    snprintf(text, cap, "%s: %s, %lld workgroups of %d waves, %d channels each, 16 states per lane%s",
+             fwd ? "m2d_fwd_kernel" : (g.ck_half ? "m2d_bwd2_kernel" : "m2d_bwd_kernel"), sched, wgs, nw, nw * g.CS * per_lane,
+             g.ck_half ? (fwd ? ", a snapshot every 2 steps" : ", a snapshot every 2 steps and one step in two recomputed") : "");
   if (g.ck_shift) {
     const size_t n = strlen(text);
     if (n + 1 < cap) snprintf(text + n, cap - n, fwd ? ", a snapshot every %d steps" : ", a snapshot every %d steps and the forward replayed in between", kCK << g.ck_shift);

@@ -52,10 +52,26 @@ layernorm_linear_act_fwd_op = torch.ops.m2dscan.layernorm_linear_act_fwd
 # reference's partial recomputation).  Module-level switch, read at forward time.
 SAVE_CHECKPOINTS = os.environ.get("M2D_SAVE_CHECKPOINTS", "1") != "0"
 
-# Steps between the state snapshots that a forward keeps for its backward (m2d_desc.ckpt_interval): 0 or 4 (the
-# default), 8 or 16.  Longer intervals keep a half or a quarter of the snapshots, and the backward replays the
-# forward over the steps in between.  Read at forward time; a backward uses the value its forward ran with.
-CKPT_INTERVAL = int(os.environ.get("M2D_CKPT_INTERVAL", "0"))
+# Steps between the state snapshots that a forward keeps for its backward (m2d_desc.ckpt_interval).  0: the library
+# chooses (2 for batches of images that are swept one stream each, 4 for few large images); 2 or 4 ask for that
+# interval where the schedule has it; 8 or 16 keep a half or a quarter of the snapshots of 4, and the backward replays
+# the forward over the steps in between.  Read at forward time; a backward uses the value its forward ran with.
+# There is one switch: mamba2d_amd.cabi.CKPT_INTERVAL (environment: M2D_CKPT_INTERVAL); this module reads it there.
+CKPT_INTERVALS = cabi.CKPT_INTERVALS
+
+
+def _interval() -> int:
+    v = cabi.CKPT_INTERVAL
+    if v not in CKPT_INTERVALS:
+        raise ValueError(f"m2dscan: CKPT_INTERVAL must be one of {CKPT_INTERVALS}, got {v!r}")
+    return v
+
+
+def __getattr__(name):   # wavefront.CKPT_INTERVAL reads the one switch
+    if name == "CKPT_INTERVAL":
+        return cabi.CKPT_INTERVAL
+    raise AttributeError(name)
+
 
 # The entry point computes the projections with the library's own kernels (wf_cuda_fn_proj) or
 # with stock torch operators followed by wf_cuda_fn_pr / wf_cuda_fn_fr.  Read at call time.
@@ -244,7 +260,7 @@ class _ScanOnParams(torch.autograd.Function):
         args = [_c(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D)]
         keep = SAVE_CHECKPOINTS and recording and any(ctx.needs_input_grad)
         ctx.flip = bool(flip)
-        ctx.interval = CKPT_INTERVAL
+        ctx.interval = _interval()
         if AT.shape[1] != STATES_PER_CALL:
             y, cks = _grouped_scan_fwd(*args, keep, ctx.flip, ctx.interval)
             ctx.save_for_backward(*args, *cks)
@@ -301,6 +317,7 @@ class wf_cuda_fn_fr(torch.autograd.Function):
                                    False, bool(flip))
         ctx.save_for_backward(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, D)
         ctx.flip = bool(flip)
+        ctx.interval = _interval()   # (no snapshots are kept: only the rebuilding forward inside the backward uses it)
         return y
 
     @staticmethod
@@ -316,10 +333,10 @@ class wf_cuda_fn_fr(torch.autograd.Function):
         if AT_log.shape[1] != STATES_PER_CALL:
             n_groups = -(-AT_log.shape[1] // STATES_PER_CALL)
             d_x_scan, d_dT, d_dL, d_AT, d_AL, d_BT, d_BL, d_C, d_D = _grouped_scan_bwd(
-                _c(x), *det, _c(D), dy, [none] * n_groups, ctx.flip, CKPT_INTERVAL)
+                _c(x), *det, _c(D), dy, [none] * n_groups, ctx.flip, ctx.interval)
         else:
             d_x_scan, d_dT, d_dL, d_AT, d_AL, d_BT, d_BL, d_C, d_D = scan_bwd_op(
-                _c(x), det[0], det[1], det[2], det[3], det[4], det[5], det[6], _c(D), dy, none, ctx.flip, ckpt_interval=CKPT_INTERVAL)
+                _c(x), det[0], det[1], det[2], det[3], det[4], det[5], det[6], _c(D), dy, none, ctx.flip, ckpt_interval=ctx.interval)
         grads = torch.autograd.grad([deltaT, deltaL, BT, BL, C, AT, AL], leaves,
                                     [d_dT, d_dL, d_BT, d_BL, d_C, d_AT, d_AL])
         d_x = d_x_scan + grads[0]   # d_x_scan already contains dy*D
@@ -356,7 +373,7 @@ class wf_cuda_fn_proj(torch.autograd.Function):
         # B_T, B_L, C go from the projection kernel to the scan as packed records (BT) and two empty tensors
         low, dT, dL, BT, BL, C = proj_fwd_op(x, *w32, AT_log.shape[1], True, True)
         keep = SAVE_CHECKPOINTS and not full and recording and any(ctx.needs_input_grad)
-        ctx.interval = CKPT_INTERVAL
+        ctx.interval = _interval()
         y, ck = scan_fwd_op(x, dT, dL, At, Al, BT, BL, C, D32, keep, bool(flip), True, True, ctx.interval)
         if full:
             ctx.save_for_backward(x, *raw)

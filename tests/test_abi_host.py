@@ -55,9 +55,9 @@ def test_descriptor_validation(cabi):
     assert chk(D(cabi, flags=4)) == 0 and chk(D(cabi, flags=29)) == 0 and chk(D(cabi, flags=2)) == 3
     assert chk(D(cabi, flags=32)) == 0 and chk(D(cabi, flags=64 | 1)) == 0 and chk(D(cabi, flags=96)) == 3
     assert chk(D(cabi, N=8)) == 3 and chk(D(cabi, dtype=7)) == 3 and chk(D(cabi, flags=128)) == 3
-    # steps between snapshots: the default, 4, 8 or 16
-    assert all(chk(D(cabi, ckpt_interval=v)) == 0 for v in (0, 4, 8, 16))
-    assert all(chk(D(cabi, ckpt_interval=v)) == 3 for v in (1, 2, 12, 32, -4))
+    # steps between snapshots: the library's choice, 2, 4, 8 or 16
+    assert all(chk(D(cabi, ckpt_interval=v)) == 0 for v in (0, 2, 4, 8, 16))
+    assert all(chk(D(cabi, ckpt_interval=v)) == 3 for v in (1, 3, 12, 32, -4))
     # one image must fit 32-bit offsets: H*W < 2^24 cells, H*W*E < 2^30 elements
     assert chk(D(cabi, B=1, H=4096, W=4096, E=8)) == 3 and chk(D(cabi, B=1, H=2048, W=2048, E=256)) == 3
     assert chk(D(cabi, B=1, H=2048, W=2048, E=64)) == 0 and chk(D(cabi, B=4, H=4000, W=4000, E=32)) == 0
@@ -124,12 +124,17 @@ def test_checkpoint_interval_shrinks_the_snapshots(cabi):
             d = D(cabi, B=B, H=H, W=W, E=E, dtype=dtype, ckpt_interval=iv, flags=cabi.M2D_FLAG_WHOLE_STATES)
             ck[iv] = cabi.lib.m2d_scan_ckpt_bytes(ctypes.byref(d))
             ws[iv] = cabi.lib.m2d_scan_workspace_bytes(ctypes.byref(d), 1, 1)
-        assert ck[4] == ck[0] and ws[4] == ws[0]
-        if H > 14:   # (7x7 images are stacked at the default interval and not at the others: other block counts)
-            assert ck[0] > ck[8] > ck[16]
+        # left to itself the library keeps a snapshot every 2 steps for batches swept one stream per image or stack
+        # (twice the snapshots of 4 steps, and one behind the sweep), every 4 steps for the few large images of a linked sweep
+        if B > 1:
+            assert ck[0] > ck[4] and ws[4] == ws[0]
+        else:
+            assert ck[4] == ck[0] and ws[4] == ws[0]
+        if H > 14:   # (7x7 images are stacked at the shorter intervals and not at the others: other block counts)
+            assert ck[4] > ck[8] > ck[16]
             # a half of the blocks dropped against three quarters (rounded up per window of a band)
-            assert abs((ck[0] - ck[8]) / (ck[0] - ck[16]) - 2 / 3) < 0.05
-            assert 0 < ws[8] - ws[0] < ws[16] - ws[0] <= 0.1 * ws[0] + (1 << 20)   # (three parked snapshots per workgroup)
+            assert abs((ck[4] - ck[8]) / (ck[4] - ck[16]) - 2 / 3) < 0.05
+            assert 0 < ws[8] - ws[4] < ws[16] - ws[4] <= 0.1 * ws[4] + (1 << 20)   # (three parked snapshots per workgroup)
     plan = cabi.scan_plan(1, 256, 256, 64, torch.float32, cabi.M2D_PASS_BWD, flags=cabi.M2D_FLAG_SPLIT_STATES, ckpt_interval=16)
     assert plan.startswith("m2d_bwd_kernel: linked sweep") and plan.endswith("a snapshot every 16 steps and the forward replayed in between")
     assert cabi.scan_plan(300, 7, 7, 32, torch.float32, cabi.M2D_PASS_FWD, ckpt_interval=8).startswith("m2d_fwd_kernel: one stream per image")
@@ -140,7 +145,10 @@ def test_plan_names_kernel_and_schedule(cabi):
     """m2d_scan_plan (host only): which kernel and schedule a problem gets on a 256-unit device."""
     import torch
     big = cabi.scan_plan(128, 56, 56, 64, torch.bfloat16, cabi.M2D_PASS_BWD)
-    assert big.startswith("m2d_bwd_kernel: one stream per image, 4 bands back to back, 256 workgroups of 8 waves, 32 channels each")
+    assert big.startswith("m2d_bwd2_kernel: one stream per image, 4 bands back to back, 256 workgroups of 8 waves, 32 channels each")
+    assert big.endswith("a snapshot every 2 steps and one step in two recomputed")
+    big4 = cabi.scan_plan(128, 56, 56, 64, torch.bfloat16, cabi.M2D_PASS_BWD, ckpt_interval=4)
+    assert big4.startswith("m2d_bwd_kernel: one stream per image, 4 bands back to back, 256 workgroups of 8 waves, 32 channels each") and "snapshot" not in big4
     one = cabi.scan_plan(1, 256, 256, 64, torch.float32, cabi.M2D_PASS_BWD)
     assert one.startswith("m2d_bwd_split_kernel: linked sweep, 19 bands, 304 workgroups of 4 waves, 4 channels each, 4 states per lane")
     two = cabi.scan_plan(1, 512, 512, 64, torch.float32, cabi.M2D_PASS_BWD)   # (more bands under way: workgroups of 8)
@@ -150,8 +158,8 @@ def test_plan_names_kernel_and_schedule(cabi):
     small = cabi.scan_plan(128, 7, 7, 512, torch.bfloat16, cabi.M2D_PASS_FWD)
     assert small.startswith("m2d_fwd_kernel: stacked images, 8 per stream, 4 bands")   # two images of 7 rows per band
     # the bands of a stack have no neighbours: all 16 lanes are rows (two 8-row images or one 16-row image per band)
-    assert cabi.scan_plan(128, 8, 8, 512, torch.bfloat16, cabi.M2D_PASS_BWD).startswith("m2d_bwd_kernel: stacked images, 8 per stream, 4 bands")
-    assert cabi.scan_plan(128, 16, 16, 320, torch.bfloat16, cabi.M2D_PASS_BWD).startswith("m2d_bwd_kernel: stacked images, 6 per stream, 6 bands")
+    assert cabi.scan_plan(128, 8, 8, 512, torch.bfloat16, cabi.M2D_PASS_BWD).startswith("m2d_bwd2_kernel: stacked images, 8 per stream, 4 bands")
+    assert cabi.scan_plan(128, 16, 16, 320, torch.bfloat16, cabi.M2D_PASS_BWD).startswith("m2d_bwd2_kernel: stacked images, 6 per stream, 6 bands")
     assert cabi.scan_plan(2001, 3, 3, 8, torch.float32, cabi.M2D_PASS_FWD).startswith("m2d_fwd_kernel: stacked images, 8 per stream, 2 bands")   # five per band
     # a short buffer truncates, a bad descriptor reports its status and an empty text
     buf = ctypes.create_string_buffer(8)

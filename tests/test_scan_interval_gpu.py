@@ -1,8 +1,10 @@
-"""GPU parity of the scan with a longer checkpoint interval (m2d_desc.ckpt_interval = 8 or 16 steps).
+"""GPU parity of the scan at every checkpoint interval (m2d_desc.ckpt_interval).
 
-The forward then keeps the snapshot of one block of 4 steps in two or four, and the backward replays the
-forward over the blocks in between before it sweeps them.  Checked against the CPU oracle to the same bounds
-as the default interval, and against the library's own results at the default interval: y must be the same
+8 or 16 steps: the forward keeps the snapshot of one block of 4 steps in two or four, and the backward replays the
+forward over the blocks in between before it sweeps them.  2 steps (what the library picks by itself for batches of
+images swept one stream each): the forward keeps two snapshots per block, and m2d_bwd2_kernel recomputes one step
+in two; asked for explicitly, 4 steps keeps such a batch on m2d_bwd_kernel.  Checked against the CPU oracle to the
+same bounds whatever the interval, and against the library's own results at the other intervals: y must be the same
 bits (the forward's arithmetic does not depend on what it keeps), the gradients the same to rounding.
 """
 import ctypes
@@ -43,6 +45,49 @@ SHAPES = [
 ]
 
 
+# shapes that the library sweeps one stream per image or stack (with what the two-step interval adds: every schedule,
+# both workgroup sizes, channel counts that cannot be staged, a last stack that is shorter)
+SHAPES_PER_IMAGE = [s for s in SHAPES if s not in ((1, 70, 50, 2), (2, 130, 20, 2), (1, 150, 90, 8), (2, 100, 33, 48), (1, 512, 512, 2), (1, 64, 17, 10))] + [
+    (600, 14, 14, 4), (129, 8, 8, 512), (601, 5, 9, 8), (37, 5, 9, 8), (33, 57, 8, 48), (260, 20, 5, 64), (67, 56, 56, 64), (128, 28, 28, 128), (300, 16, 16, 32)]
+
+
+@pytest.mark.parametrize("interval", [2, 4], indirect=True)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("shape", SHAPES_PER_IMAGE, ids=lambda s: "x".join(map(str, s)))
+def test_parity_with_two_and_four_steps(cabi, cscan, shape, dtype, interval):
+    cabi.SCHEDULE_HINT = cabi.M2D_FLAG_WHOLE_STATES   # (small batches would split the states of a channel over lanes: a snapshot every 4 steps)
+    try:
+        plan = cabi.scan_plan(*shape, dtype, cabi.M2D_PASS_BWD)
+        say(f"\ninterval {interval} shape {shape} {dtype}: {plan}")
+        two = interval == 2 and "linked sweep" not in plan
+        assert plan.startswith("m2d_bwd2_kernel" if two else "m2d_bwd_kernel") and ("a snapshot every 2 steps" in plan) == two, plan
+        run_case(cabi, cscan, *shape, dtype)
+    finally:
+        cabi.SCHEDULE_HINT = 0
+
+
+@pytest.mark.parametrize("interval", [2, 4], indirect=True)
+@pytest.mark.parametrize("shape", [(2, 14, 14, 4), (3, 33, 40, 6), (301, 7, 7, 4), (70, 56, 30, 12)], ids=lambda s: "x".join(map(str, s)))
+def test_flipped_scan_and_rebuilt_checkpoints_two_and_four_steps(cabi, cscan, shape, interval):
+    run_case(cabi, cscan, *shape, torch.float32, flip=True)
+    run_case(cabi, cscan, *shape, torch.bfloat16, flip=True)
+    run_case(cabi, cscan, *shape, torch.bfloat16, with_ckpt=False)   # the backward runs the keeping forward itself
+    run_case(cabi, cscan, *shape, torch.float32, with_ckpt=False)
+
+
+def test_few_large_images_keep_four_steps(cabi):
+    """The two-step interval belongs to the schedules of many images; a linked sweep asked for it keeps a snapshot every
+    4 steps (sizes and plan say so), and the library never picks it there by itself."""
+    for iv in (0, 2):
+        plan = cabi.scan_plan(1, 256, 256, 64, torch.float32, cabi.M2D_PASS_BWD, ckpt_interval=iv)
+        assert "every 2 steps" not in plan and "linked sweep" in plan, plan
+    size = lambda iv: cabi.lib.m2d_scan_ckpt_bytes(ctypes.byref(cabi.Desc(1, 256, 256, 64, 16, cabi.M2D_F32, 0, iv)))
+    assert size(0) == size(2) == size(4)
+    many = lambda iv: cabi.lib.m2d_scan_ckpt_bytes(ctypes.byref(cabi.Desc(128, 56, 56, 64, 16, cabi.M2D_BF16, 0, iv)))
+    assert many(0) == many(2) > 1.7 * many(4)   # (twice the snapshots and one; the boundary rows stay)
+    assert "every 2 steps" in cabi.scan_plan(128, 56, 56, 64, torch.bfloat16, cabi.M2D_PASS_FWD)
+
+
 @pytest.mark.parametrize("interval", [8, 16], indirect=True)
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 @pytest.mark.parametrize("shape", SHAPES, ids=lambda s: "x".join(map(str, s)))
@@ -69,7 +114,7 @@ def test_same_results_as_the_default_interval(cabi, shape, dtype):
     res, sizes = {}, {}
     try:
         cabi.SCHEDULE_HINT = flags
-        for iv in (0, 8, 16):
+        for iv in (4, 2, 8, 16):
             cabi.CKPT_INTERVAL = iv
             y, ck = cabi.scan_fwd(*a, save_ckpt=True)
             g = cabi.scan_bwd(*a, dy, ckpt=ck)
@@ -81,12 +126,12 @@ def test_same_results_as_the_default_interval(cabi, shape, dtype):
         cabi.CKPT_INTERVAL = 0
         cabi.SCHEDULE_HINT = 0
     say(f"checkpoint bytes {sizes}")
-    assert sizes[0] > sizes[8] > sizes[16]
-    for iv in (8, 16):
-        assert torch.equal(res[iv][0], res[0][0]), "y depends on the interval"
-        for name, g, g0 in zip(so.CScan.GRADS, res[iv][1], res[0][1]):
+    assert sizes[2] >= sizes[4] > sizes[8] > sizes[16]   # (2: only where every image is one stream)
+    for iv in (2, 8, 16):
+        assert torch.equal(res[iv][0], res[4][0]), "y depends on the interval"
+        for name, g, g0 in zip(so.CScan.GRADS, res[iv][1], res[4][1]):
             # fp32: the replay repeats the forward's own arithmetic; bf16: a replayed state is rounded to bf16 once
             # more than a kept one, which moves gradients as the snapshots' own rounding does
             e = so.rel_err(g.float().cpu(), g0.float().cpu().double().numpy())
-            say(f"  interval {iv} {name}: {e:.2e} from the default interval's")
+            say(f"  interval {iv} {name}: {e:.2e} from the results at 4 steps")
             assert e < (1e-5 if dtype == torch.float32 else 1e-2), (iv, name, e)

@@ -94,7 +94,7 @@ def test_entry_point_matches_oracle_fp32(wf, recomp, projections):
 @pytest.mark.parametrize("interval", [8, 16])
 @pytest.mark.parametrize("recomp", ["partial", "full"])
 def test_entry_point_with_longer_checkpoint_interval(wf, recomp, interval, monkeypatch):
-    """wavefront.CKPT_INTERVAL reaches the library through the operators: fewer bytes saved for the backward,
+    """cabi.CKPT_INTERVAL (the one switch, which mamba2d_amd.wavefront reads) reaches the library through the operators: fewer bytes saved for the backward,
     the same gradients (the oracle's, to the entry point's fp32 bound); 24 states run as two groups."""
     say(f"\ncase entry_point {recomp} ckpt_interval={interval}")
     for N in (16, 24):
@@ -105,7 +105,7 @@ def test_entry_point_with_longer_checkpoint_interval(wf, recomp, interval, monke
         dy = torch.randn(B, H, W, E, generator=torch.Generator().manual_seed(2)).cuda()
         kept = {}
         for iv in (0, interval):
-            monkeypatch.setattr(wf, "CKPT_INTERVAL", iv)
+            monkeypatch.setattr(wf.cabi, "CKPT_INTERVAL", iv)
             real, seen = wf.scan_fwd_op, []
 
             def spy(*a, **kw):
