@@ -105,6 +105,15 @@ typedef struct m2d_desc {
  * M2D_FLAG_SPLIT_STATES asks for that layout wherever it exists, M2D_FLAG_WHOLE_STATES forbids it. */
 #define M2D_FLAG_SPLIT_STATES 32
 #define M2D_FLAG_WHOLE_STATES 64
+/* Test aid for the linked sweep (grids of many bands and few images, whose bands run on workgroups of their own
+ * inside one launch and wait for each other's boundary rows; see m2d_scan_link_error).  With this flag the
+ * workgroups of one band (forward: the second; backward: the last but one) wait for a neighbour that never
+ * reports, and every wait of the launch gives up after a few polls instead of about a million: the launch runs
+ * the path of a wait that gives up, and still ends normally.  What that path does: the workgroup sets the error
+ * word, tells its dependants not to wait, and overwrites its band's rows of y (forward) or of dx, d_deltaT,
+ * d_deltaL and its channels' shares of d_AT, d_AL, d_D (backward) with NaN, as does every band that depended
+ * on it; so a linked sweep that failed shows in the caller's tensors.  Ignored by other schedules. */
+#define M2D_FLAG_TEST_DEAD_LINK 128
 
 #define M2D_PASS_FWD 0
 #define M2D_PASS_BWD 1
@@ -144,8 +153,10 @@ int m2d_scan_fwd(const m2d_desc* desc,
 
 /* Debugging aid for grids of many bands and few images, whose bands run on workgroups of their own
  * inside one launch and wait for each other's boundary rows (a bounded wait: a workgroup that has
- * polled about a million times gives up, so that the launch always ends; the results are then
- * invalid).  Synchronises `stream` and reads, from the workspace of the last m2d_scan_fwd or
+ * polled about two million times -- seconds of wall time, which only another tenant of the device
+ * holding the compute units can cause -- gives up, so that the launch always ends; the results are then
+ * invalid, and the workgroup and every band after it overwrite their rows of the outputs with NaN).
+ * Synchronises `stream` and reads, from the workspace of the last m2d_scan_fwd or
  * m2d_scan_bwd call of this descriptor on it, whether any workgroup gave up: *gave_up = 0 or 1 (always
  * 0 for problems that do not run that way).  No counterpart in the reference (its diagonals are
  * ordered by kernel launches, wf_cuda.cu:203,259). */
@@ -164,8 +175,12 @@ int m2d_scan_plan(const m2d_desc* desc, int pass, char* text, size_t cap);
  * of M2D_NOALLOC_SCRATCH_BYTES inside the library (each GPU the library runs on holds one copy until
  * the process ends); the call allocates and frees nothing.  A problem whose
  * m2d_scan_workspace_bytes(desc, M2D_PASS_FWD, 0) exceeds that size is rejected with
- * M2D_ERR_TOO_LARGE before anything is launched.  All calls on one GPU share the array: two calls
- * that overlap on one GPU (different streams or threads) race; calls on one stream are ordered. */
+ * M2D_ERR_TOO_LARGE before anything is launched (this check comes first: a call with NULL tensors on
+ * a problem that is too large reports M2D_ERR_TOO_LARGE).  All calls on one GPU share the array: two calls
+ * that overlap on one GPU (different streams or threads) race; calls on one stream are ordered.  Besides
+ * boundary rows, the array holds the progress counts of a linked sweep: an overlapping call that clears
+ * them in mid-flight can make the other launch's waits give up (its rows of y then say NaN, see
+ * m2d_scan_link_error). */
 #define M2D_NOALLOC_SCRATCH_BYTES (32u << 20)
 int m2d_scan_fwd_noalloc(const m2d_desc* desc,
                          const void* x, const void* deltaT, const void* deltaL,

@@ -206,6 +206,7 @@ struct ScanParams {
   int sl_nbb;                       // blocks per band (S / kCK)
   uint32_t* prog;                   // [nbands][B][workgroups per image] blocks of the band's window whose boundary rows are in memory
   uint32_t* link_err;               // set to 1 by a workgroup that gave up waiting (results are then invalid)
+  int link_test;                    // test aid (M2D_FLAG_TEST_DEAD_LINK): 1 + the band whose neighbour never reports, and a wait gives up after a few polls
   int64_t bot_stride;               // floats between the mu_T rows of consecutive bands (0: one row buffer, bands in sequence)
   int pa_slots;                     // partial sums over positions per image (1, or one per band when sliced)
   // Stacked images (grids of at most 16 rows, one band each): `ips` images in a row of the batch
@@ -365,10 +366,22 @@ struct Link {
   uint32_t seen = 0;                // last value read from dep
   bool gave_up = false;
   uint32_t* err = nullptr;
+  int limit = kSpinLimit;           // polls before a wait gives up
+  // test aid: the workgroups of band `link_test - 1` wait for a count that nobody publishes (a word of the header,
+  // zero for the whole launch), and every wait of the launch gives up after a few polls: the give-up path runs, and
+  // every workgroup still ends
+  __device__ __forceinline__ void rig(const ScanParams& p, int band) {
+    if (p.link_test) {
+      limit = 16;
+      if (band == p.link_test - 1) dep = p.link_err + 1;
+    }
+  }
+  // this workgroup's results mean nothing: it gave up waiting, or a band it depends on did
+  __device__ __forceinline__ bool broken() const { return gave_up || seen == kLinkAbort; }
   // (uniform) returns once the neighbour has `need` blocks done
   __device__ __forceinline__ void wait_for(uint32_t need) {
     if (!dep || seen >= need) return;
-    for (int spin = 0; spin < kSpinLimit; ++spin) {
+    for (int spin = 0; spin < limit; ++spin) {
       seen = link_poll(dep);
       if (seen >= need) return;
       __builtin_amdgcn_s_sleep(4);
@@ -711,6 +724,24 @@ __device__ __forceinline__ void bc_widen(const char* raw, char* buf, int wave, i
   }
 }
 
+// A workgroup of the linked sweep whose results mean nothing (Link::broken) says so in the caller's tensors: it
+// overwrites its band's rows of up to three (B,H,W,E) tensors, for its own channels, with NaN, so that the failure
+// shows without anyone reading the error word.
+template <typename T>
+__device__ __forceinline__ void poison_band(const ScanParams& p, int band, int b, int e_wg0, int cw, void* t0, void* t1, void* t2) {
+  const int n = band_rows(p, band) * p.W * cw;
+  const float nan = __builtin_nanf("");
+  for (int i = threadIdx.x; i < n; i += blockDim.x) {
+    const int c = i % cw, at = i / cw;
+    if (e_wg0 + c >= p.E) continue;
+    const int cell = cell_of(p, band, at / p.W + 1, at % p.W);   // (lane row = row of the band + 1)
+    const int64_t el = ((int64_t)b * p.Hs * p.W + cell) * p.E + e_wg0 + c;
+    IO<T>::st(static_cast<T*>(t0) + el, nan);
+    if (t1) IO<T>::st(static_cast<T*>(t1) + el, nan);
+    if (t2) IO<T>::st(static_cast<T*>(t2) + el, nan);
+  }
+}
+
 // ------------------------------------------------------------------------------------ forward
 // y on its way out (m2d_fwd_kernel).  A lane's y of one step is 2 or 4 bytes at a cell of its own row: stored
 // from the lane, a wave's y of one step goes to 16 different cache lines, 8 bytes each, and these stores cost
@@ -833,6 +864,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     link.mine = p.prog + (int64_t)my_band * per + lb;
     link.dep = my_band > 0 ? link.mine - per : nullptr;
     link.err = p.link_err;
+    link.rig(p, my_band);
   }
   const int b = lb / p.bpb;
   const int e_wg0 = (lb % p.bpb) * CW;
@@ -1220,6 +1252,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
     link.publish((uint32_t)p.sl_nbb);
+    if (WRITE_Y && link.broken()) poison_band<T>(p, my_band, b, e_wg0, CW, p.y, nullptr, nullptr);
   }
 }
 
@@ -1265,6 +1298,7 @@ __global__ __launch_bounds__(NWS * 64) void m2d_fwd_split_kernel(const ScanParam
     link.mine = p.prog + (int64_t)my_band * per + lb;
     link.dep = my_band > 0 ? link.mine - per : nullptr;
     link.err = p.link_err;
+    link.rig(p, my_band);
   }
   const int b = lb / p.bpb;
   const int e_wg0 = (lb % p.bpb) * CW;
@@ -1459,6 +1493,7 @@ __global__ __launch_bounds__(NWS * 64) void m2d_fwd_split_kernel(const ScanParam
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
     link.publish((uint32_t)p.sl_nbb);
+    if (WRITE_Y && link.broken()) poison_band<T>(p, my_band, b, e_wg0, CW, p.y, nullptr, nullptr);
   }
 }
 
@@ -1538,6 +1573,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
     link.mine = p.prog + (int64_t)my_band * per + lb;
     link.dep = my_band + 1 < p.nbands ? link.mine + per : nullptr;
     link.err = p.link_err;
+    link.rig(p, my_band);
   }
   const int b = lb / p.bpb;
   const int eg = lb % p.bpb;
@@ -2032,17 +2068,21 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
     cell0 = celln;
     cur ^= 1;
   }
+  bool broken = false;
   if constexpr (SLICED) {   // the whole window is done once every store of every wave has completed
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
     link.publish((uint32_t)p.sl_nbb);
+    broken = link.broken() || link_poll(p.link_err) != 0u;   // (also a workgroup of the forward sweep that rebuilt the snapshots for this launch)
+    if (broken) poison_band<T>(p, my_band, b, e_wg0, CW, p.dx, p.ddT, p.ddL);
   }
 
   // ---- sums over positions: reduce over the rows of the band (lanes of one channel slot)
   float red[2 * kN + 1];
 #pragma unroll
   for (int n = 0; n < kN; ++n) { red[n] = accAT[n]; red[kN + n] = accAL[n]; }
-  red[2 * kN] = accD;
+  red[2 * kN] = broken ? __builtin_nanf("") : accD;
+  if (broken) { red[0] = __builtin_nanf(""); red[kN] = __builtin_nanf(""); }   // (d_AT, d_AL, d_D of the channel say so too)
 #pragma unroll
   for (int k = 0; k < 2 * kN + 1; ++k) {
     float v = red[k];
@@ -2530,6 +2570,7 @@ __global__ __launch_bounds__(NWS * 64) void m2d_bwd_split_kernel(const ScanParam
     link.mine = p.prog + (int64_t)my_band * per + lb;
     link.dep = my_band + 1 < p.nbands ? link.mine + per : nullptr;
     link.err = p.link_err;
+    link.rig(p, my_band);
   }
   const int b = lb / p.bpb;
   const int eg = lb % p.bpb;
@@ -2800,17 +2841,21 @@ __global__ __launch_bounds__(NWS * 64) void m2d_bwd_split_kernel(const ScanParam
     cell0 = celln;
     cur ^= 1;
   }
+  bool broken = false;
   if constexpr (SLICED) {
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
     link.publish((uint32_t)p.sl_nbb);
+    broken = link.broken() || link_poll(p.link_err) != 0u;   // (also a workgroup of the forward sweep that rebuilt the snapshots for this launch)
+    if (broken) poison_band<T>(p, my_band, b, e_wg0, CW, p.dx, p.ddT, p.ddL);
   }
 
   // ---- sums over positions: reduce over the rows of the band (the 16 lanes of a group)
   float red[9];
 #pragma unroll
   for (int w = 0; w < 4; ++w) { red[w] = accAT[w]; red[4 + w] = accAL[w]; }
-  red[8] = accD;
+  red[8] = broken ? __builtin_nanf("") : accD;
+  if (broken) { red[0] = __builtin_nanf(""); red[4] = __builtin_nanf(""); }   // (d_AT, d_AL, d_D of the channel say so too)
 #pragma unroll
   for (int k = 0; k < 9; ++k) {
     float v = red[k];
@@ -2988,7 +3033,7 @@ int check_desc(const m2d_desc* d) {
   if (d->B < 1 || d->E < 1 || d->N < 1 || d->H < 2 || d->W < 2) return M2D_ERR_BAD_SHAPE;
   if (d->N != kN) return M2D_ERR_UNSUPPORTED;
   if (d->dtype != M2D_F32 && d->dtype != M2D_BF16) return M2D_ERR_UNSUPPORTED;
-  if ((d->ckpt_interval != 0 && d->ckpt_interval != 2 && d->ckpt_interval != 4 && d->ckpt_interval != 8 && d->ckpt_interval != 16) || (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_RAW_PARAMS | M2D_FLAG_PACKED_BC | M2D_FLAG_DPRE | M2D_FLAG_SPLIT_STATES | M2D_FLAG_WHOLE_STATES))) return M2D_ERR_UNSUPPORTED;
+  if ((d->ckpt_interval != 0 && d->ckpt_interval != 2 && d->ckpt_interval != 4 && d->ckpt_interval != 8 && d->ckpt_interval != 16) || (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_RAW_PARAMS | M2D_FLAG_PACKED_BC | M2D_FLAG_DPRE | M2D_FLAG_SPLIT_STATES | M2D_FLAG_WHOLE_STATES | M2D_FLAG_TEST_DEAD_LINK))) return M2D_ERR_UNSUPPORTED;
   if ((d->flags & M2D_FLAG_SPLIT_STATES) && (d->flags & M2D_FLAG_WHOLE_STATES)) return M2D_ERR_UNSUPPORTED;
   if ((int64_t)d->B * d->H * d->W >= ((int64_t)1 << 40)) return M2D_ERR_BAD_SHAPE;
   // one image is addressed with 32-bit byte offsets from its base (fp32: 4 bytes per element;
@@ -3372,6 +3417,7 @@ int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
     rc = stage_bc<T>(sp, d, BT, BL, C, reinterpret_cast<float*>(keep + g.top_bytes), false, st);
   }
   if (rc) return rc;
+  if ((d->flags & M2D_FLAG_TEST_DEAD_LINK) && g.sliced && g.nbands >= 2) sp.link_test = 1 + 1;   // the second band's neighbour never reports
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_FWD][0], st);
   rc = launch_fwd<T>(sp, d, g, ckpt != nullptr, true, st);
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_FWD][1], st);
@@ -3477,6 +3523,7 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   }
   sp.bpb = g.bwd_bpb;
   sp.nwg = g.vB * g.bwd_bpb;
+  if ((d->flags & M2D_FLAG_TEST_DEAD_LINK) && g.sliced && g.nbands >= 2) sp.link_test = 1 + (g.nbands - 2);   // the last band but one waits for the last
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][0], st);
   if (!g.sliced) {
     if (g.bwd_split) rc = launch_bwd_split<T, kModeSweep>(sp, g.stage_x, st, g.bwd_nw);
