@@ -41,15 +41,20 @@ WORKLOADS = {
 }
 N = 16
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the backward scan kernel from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE
-# (profiles/scan_cfg1_kernel_trace_and_traffic.txt); counters cannot be read from inside this script,
-# so the figure is carried here for the workload that has a counter run, and is null for the others.
-MEASURED_TRAFFIC = {"cfg1": 1.1188e9}
-# Issue slots per (cell, channel, state) of the scan kernels (a v_exp_f32 takes two on gfx950):
-# forward 2 exponent FMAs + 2 v_exp + 5 FMA-class (input term, two gate terms, y);
-# backward 10 for the recomputation, 24 for the adjoint (15 FMA-class, 4.5 for the gates of three steps in
-# four, 4.5 for the lane-swap sums over the channels of a wave).
-FWD_SLOTS, BWD_SLOTS = 11, 34
+# HBM bytes per launch of the dominant kernel come from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs, which this
+# script cannot make from inside itself: `roofline.traffic` is null here, and the counter run of the same command is
+# summarised, with its figure, in the file that `roofline.traffic_profile` names.
+TRAFFIC_PROFILE = {"cfg1": "profiles/scan_cfg1_kernel_trace_and_traffic.txt"}
+# Vector-ALU operations per (cell, channel, state) of the scan kernels, as (multiply-add class, v_exp_f32):
+# forward: 2 exponent multiply-adds + 5 (input term, two gate terms, y), 2 gates;
+# backward with a snapshot every 4 steps (m2d_bwd_kernel): the block recomputed (2 + 4, 2 gates), the adjoint (17,
+#   the gates of three steps in four: 1.5 + 1.5), 4.5 for the lane-swap sums over the channels of a wave;
+# backward with a snapshot every 2 steps (m2d_bwd2_kernel): one step in two recomputed (1 + 2, 1 gate), the adjoint
+#   (17, the gates of one step in two: 1 + 1), 4.5 for the channel sums, 1 for unpacking the restored states.
+UNIT_OPS = {"fwd": (7, 2), "bwd4": (29, 3.5), "bwd2": (26.5, 2)}
+# nominal issue slots of the same (a v_exp_f32 takes two on gfx950)
+FWD_SLOTS = 11
+BWD_SLOTS = {"m2d_bwd_kernel": 36, "m2d_bwd2_kernel": 30.5}
 
 
 def nominal_valu_slots_per_s():
@@ -70,10 +75,46 @@ def scan_roofline(name, B, E, H, W, s, bwd_kernel_ms, fwd_kernel_ms):
     plan_fwd = cabi.scan_plan(B, H, W, E, dts, cabi.M2D_PASS_FWD)
     return {
         "kernel": plan_bwd.split(":")[0], "schedule": plan_bwd, "fwd_schedule": plan_fwd, "bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC.get(name),
+        "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None, "traffic_profile": TRAFFIC_PROFILE.get(name),
         "kernel_ms": round(bwd_kernel_ms, 4), "algorithmic_bytes": bb,
         "fwd_kernel_ms": round(fwd_kernel_ms, 4), "fwd_algorithmic_bytes": fb,
         "fwd_kernel_frac": round(fb / (fwd_kernel_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+    }
+
+
+def measured_valu_rates():
+    """Instruction rates of the device's vector ALUs from the library's probe kernel (m2d_valu_rate_probe), at the
+    two waves per SIMD that the scan kernels run: lane-operations per second of v_fma_f32 and v_exp_f32 with 16
+    independent chains per lane and with one dependent chain, and the forward scan's own mix in units per second."""
+    from mamba2d_amd import cabi
+    return {k: cabi.valu_rate_probe(k, 2) for k in ("fma", "exp", "fma_dependent", "exp_dependent", "scan_fwd_unit")}
+
+
+def valu_ceiling(units, fwd_kernel_ms, bwd_kernel_ms, bwd_kernel_name, rates=None):
+    """The `valu_ceiling` object: the scan is bound by instruction issue, not by HBM.  The measured ceiling of a
+    kernel is units x (multiply-adds / measured multiply-add rate + gates / measured v_exp_f32 rate): the time its
+    arithmetic alone would take at the rates the probe kernel reaches on this device in this process."""
+    rates = rates or measured_valu_rates()
+    peak_slots = nominal_valu_slots_per_s()
+    bwd_ops = UNIT_OPS["bwd2" if bwd_kernel_name.startswith("m2d_bwd2") else "bwd4"]
+    floor_ms = lambda ops: units * (ops[0] / rates["fma"] + ops[1] / rates["exp"]) * 1e3
+    bwd_slots = BWD_SLOTS.get(bwd_kernel_name.split(":")[0], 36)
+    return {
+        "measured_lane_slots_per_s": round(rates["fma"]),   # v_fma_f32, independent chains, 2 waves per SIMD, whole device
+        "measured_exp_per_s": round(rates["exp"]),
+        "measured_fma_dependent_per_s": round(rates["fma_dependent"]),
+        "measured_exp_dependent_per_s": round(rates["exp_dependent"]),
+        "measured_scan_fwd_units_per_s": round(rates["scan_fwd_unit"]),   # the forward's arithmetic alone, as a kernel of its own
+        "predicted_scan_fwd_units_per_s": round(1.0 / (UNIT_OPS["fwd"][0] / rates["fma"] + UNIT_OPS["fwd"][1] / rates["exp"])),
+        "units": units, "fwd_ops_per_unit": UNIT_OPS["fwd"], "bwd_ops_per_unit": bwd_ops,
+        "fwd_arithmetic_floor_ms": round(floor_ms(UNIT_OPS["fwd"]), 4), "bwd_arithmetic_floor_ms": round(floor_ms(bwd_ops), 4),
+        "fwd_kernel_frac_of_measured": round(floor_ms(UNIT_OPS["fwd"]) / fwd_kernel_ms, 4),
+        "bwd_kernel_frac_of_measured": round(floor_ms(bwd_ops) / bwd_kernel_ms, 4),
+        "nominal_lane_slots_per_s": peak_slots,
+        "note": "measured: m2d_valu_rate_probe in this process (16 independent chains per lane, 2 waves per SIMD); nominal: compute units x 64 lanes x engine clock from the device properties",
+        "fwd_slots_per_unit": FWD_SLOTS, "bwd_slots_per_unit": bwd_slots,
+        "fwd_kernel_frac": round(units * FWD_SLOTS / peak_slots / (fwd_kernel_ms * 1e-3), 4),
+        "bwd_kernel_frac": round(units * bwd_slots / peak_slots / (bwd_kernel_ms * 1e-3), 4),
     }
 
 
@@ -244,7 +285,7 @@ def stage_sequence(args):
         "config": {"workload": "cfg2: scans of (E,H,W) = (64,56,56), (128,28,28), (320,14,14), (512,7,7) in sequence, B=128 N=16"},
         "fwd_ms": round(fwd_ms, 4), "fwd_bwd_ms": round(both_ms, 4),
         "pct_hbm_roofline": {"fwd_bwd": round(100 * alg / (both_ms * 1e-3) / (HBM_PEAK_GBS * 1e9), 2)},
-        "valu_ceiling_frac_nominal": round(units * (FWD_SLOTS + BWD_SLOTS) / nominal_valu_slots_per_s() / (both_ms * 1e-3), 4),
+        "valu_ceiling_frac_nominal": round(units * (FWD_SLOTS + BWD_SLOTS["m2d_bwd2_kernel"]) / nominal_valu_slots_per_s() / (both_ms * 1e-3), 4),
         "roofline": roof,
         "per_stage_bwd_kernel": {k: {"kernel_ms": v["kernel_ms"], "frac": v["frac"], "fwd_kernel_ms": v["fwd_kernel_ms"]} for k, v in per_stage.items()},
         "cpu_baseline": None,
@@ -343,6 +384,116 @@ def entry_point(args):
     print(json.dumps(out))
 
 
+def _timed(fn, steps, warmup):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def _device_scan_inputs(B, E, H, W, dtype, seed):
+    """The synthetic inputs of a scan workload, drawn on the device (same distributions as the headline workload's)."""
+    import torch
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(seed)
+    r = lambda *s: torch.randn(*s, generator=g, device=dev)
+    sp = torch.nn.functional.softplus
+    host = [r(B, H, W, E), sp(r(B, H, W, E)), sp(r(B, H, W, E)), -torch.exp(-4 * torch.rand(E, N, generator=g, device=dev)),
+            -torch.exp(-4 * torch.rand(E, N, generator=g, device=dev)), r(B, H, W, N), r(B, H, W, N), r(B, H, W, N), r(E)]
+    leaves = [t.to(dtype).requires_grad_(True) for t in host]
+    return leaves, r(B, H, W, E).to(dtype)
+
+
+def _short_scan(name, steps, warmup):
+    """fwd and fwd+bwd of one scan workload in a few steps, with the kernel durations from the library's events."""
+    import torch
+    from mamba2d_amd import cabi, wavefront
+    B, E, H, W, dts = WORKLOADS[name]
+    dtype = torch.bfloat16 if dts == "bf16" else torch.float32
+    s = 2 if dts == "bf16" else 4
+    torch.cuda.empty_cache()
+    torch.cuda.reset_peak_memory_stats()
+    leaves, dy = _device_scan_inputs(B, E, H, W, dtype, seed=1)
+    frozen = [t.detach() for t in leaves]
+
+    def fwd_only():
+        with torch.no_grad():
+            wavefront.wf_cuda_fn_pr.apply(*frozen)
+
+    def fwd_bwd():
+        torch.autograd.grad(wavefront.wf_cuda_fn_pr.apply(*leaves), leaves, dy)
+
+    cabi.profile_enable(False)
+    fwd_ms, both_ms = _timed(fwd_only, steps, warmup), _timed(fwd_bwd, steps, warmup)
+    peak = torch.cuda.max_memory_allocated()
+    cabi.profile_enable(True)
+    ks = []
+    for _ in range(3):
+        fwd_bwd()
+        torch.cuda.synchronize()
+        ks.append((cabi.profile_last_ms(cabi.M2D_PASS_FWD), cabi.profile_last_ms(cabi.M2D_PASS_BWD)))
+    cabi.profile_enable(False)
+    fk, bk = sum(k[0] for k in ks) / len(ks), sum(k[1] for k in ks) / len(ks)
+    fb, bb = algorithmic_bytes(B, E, H, W, s)
+    roof = scan_roofline(name, B, E, H, W, s, bk, fk)
+    del leaves, frozen, dy
+    torch.cuda.empty_cache()
+    return {"workload": f"B={B} E={E} {H}x{W} {dts}", "fwd_ms": round(fwd_ms, 4), "fwd_bwd_ms": round(both_ms, 4), "steps": steps,
+            "peak_hbm_bytes": int(peak),
+            "pct_hbm_roofline_fwd_bwd": round(100 * (fb + bb) / (both_ms * 1e-3) / (HBM_PEAK_GBS * 1e9), 2),
+            "roofline": {k: roof[k] for k in ("kernel", "schedule", "bound", "achieved", "peak", "unit", "frac", "kernel_ms", "fwd_kernel_ms", "fwd_kernel_frac")}}
+
+
+def also_workloads(args, rates, cfg1_fwd_bwd_ms):
+    """Short measurements of the other configurations in the same process, after the timed region of the headline
+    workload: the four stage scans in sequence (cfg2), one image of 256x256 and of 2048x2048 (cfg4, with the
+    allocator's peak), and the entry point wavefront_scan_cuda with its projections at the headline shape."""
+    import math
+    import torch
+    from mamba2d_amd import wavefront as wf
+    out = {}
+    stages = {k: _short_scan(k, 10, 3) for k in ("stage2", "stage3", "stage4")}
+    # (the first stage is the headline workload itself; the stages run back to back on one stream, so the sum of their
+    # steps is what `--workload cfg2` times as one step)
+    out["cfg2"] = {"fwd_bwd_ms": round(cfg1_fwd_bwd_ms + sum(v["fwd_bwd_ms"] for v in stages.values()), 4), "stages": stages}
+    out["cfg4_256"] = _short_scan("hires256", 10, 3)
+    free, _ = torch.cuda.mem_get_info()
+    if free > 40 * 2**30:
+        out["cfg4_2048"] = _short_scan("hires2048", 3, 1)
+    # entry point: projections + scan, fp32 parameters initialised like an M2D block, bf16 activations
+    B, E, H, W = WORKLOADS["cfg1"][:4]
+    R = math.ceil(E / 16)
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(0)
+    dt = torch.exp(torch.rand(E, generator=g) * (math.log(0.1) - math.log(0.001)) + math.log(0.001)).clamp(min=1e-4)
+    inv_dt = dt + torch.log(-torch.expm1(-dt))
+    params = [torch.log(torch.arange(1, N + 1, dtype=torch.float32).repeat(E, 1)), torch.log(torch.arange(1, N + 1, dtype=torch.float32).repeat(E, 1)),
+              (torch.rand(2 * R + 3 * N, E, generator=g) * 2 - 1) / math.sqrt(E),
+              (torch.rand(E, R, generator=g) * 2 - 1) * R ** -0.5, inv_dt.clone(), (torch.rand(E, R, generator=g) * 2 - 1) * R ** -0.5, inv_dt.clone(), torch.ones(E)]
+    params = [p.to(dev).requires_grad_(True) for p in params]
+    gd = torch.Generator(device=dev).manual_seed(2)
+    x = torch.randn(B, H, W, E, generator=gd, device=dev).to(torch.bfloat16).requires_grad_(True)
+    dy = torch.randn(B, H, W, E, generator=gd, device=dev).to(torch.bfloat16)
+
+    def entry_fwd_bwd():
+        torch.autograd.grad(wf.wavefront_scan_cuda(x, *params), [x] + params, dy)
+
+    def entry_fwd():
+        with torch.no_grad():
+            wf.wavefront_scan_cuda(x, *params)
+
+    out["entry"] = {"workload": "wavefront_scan_cuda (projections + scan), B=128 E=64 56x56 N=16 dt_rank=4, bf16 activations, recomp=partial",
+                    "fwd_ms": round(_timed(entry_fwd, 10, 3), 4), "fwd_bwd_ms": round(_timed(entry_fwd_bwd, 10, 3), 4), "steps": 10}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -350,6 +501,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="cfg1", choices=sorted(WORKLOADS))
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-also", action="store_true", help="skip the short measurements of the other workloads that the default workload appends")
     ap.add_argument("--no-ckpt", action="store_true", help="rebuild checkpoints inside the backward")
     ap.add_argument("--ckpt-interval", type=int, default=0, choices=(0, 2, 4, 8, 16),
                     help="steps between the state snapshots the forward keeps (0 or 4: the default; 8, 16: fewer "
@@ -488,16 +640,12 @@ def main():
         },
         "roofline": scan_roofline(args.workload, B, E, H, W, s, bwd_kernel, fwd_kernel_ms),
     }
-    # Informational second ceiling: the scan is bounded by VALU issue, not by HBM.
-    units = B * H * W * E * N
-    peak_slots = nominal_valu_slots_per_s()
-    out["valu_ceiling"] = {
-        "nominal_lane_slots_per_s": peak_slots,
-        "note": "compute units x 64 lanes x engine clock from the device properties; not measured by this script",
-        "fwd_slots_per_unit": FWD_SLOTS, "bwd_slots_per_unit": BWD_SLOTS, "units": units,
-        "fwd_kernel_frac": round(units * FWD_SLOTS / peak_slots / (fwd_kernel_ms * 1e-3), 4),
-        "bwd_kernel_frac": round(units * BWD_SLOTS / peak_slots / (bwd_kernel * 1e-3), 4),
-    }
+    # Second ceiling: the scan is bounded by instruction issue, not by HBM.  Measured on this device by the library's
+    # probe kernel, outside the timed region.
+    rates = measured_valu_rates()
+    out["valu_ceiling"] = valu_ceiling(B * H * W * E * N, fwd_kernel_ms, bwd_kernel, out["roofline"]["schedule"], rates)
+    if args.workload == "cfg1" and not args.no_also:
+        out["also"] = also_workloads(args, rates, step_ms)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(B, E, H, W)
     else:

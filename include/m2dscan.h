@@ -350,6 +350,23 @@ int m2d_mlp_fwd(int64_t P, int C, int hidden, int weight_dtype, const void* x,
 int m2d_profile_enable(int on);
 int m2d_profile_last_ms(int pass, float* ms);
 
+/* Measurement aid; no counterpart in the reference.  What the vector ALUs of the current device issue per
+ * second, measured by a small kernel that fills the device with `waves_per_simd` waves per SIMD (1 to 8; the scan
+ * kernels run 2), each lane running 65536 operations of one kind on registers:
+ *   M2D_RATE_FMA, M2D_RATE_EXP                      v_fma_f32 / v_exp_f32, 16 independent chains per lane
+ *   M2D_RATE_FMA_DEPENDENT, M2D_RATE_EXP_DEPENDENT  one chain per lane: every operation waits for the one before
+ *   M2D_RATE_SCAN_FWD_UNIT                          the forward scan's arithmetic per (cell, channel, state): two gate
+ *                                                   exponents with their multiply-adds, five multiply-adds
+ * *per_second receives lane-operations per second over the whole device (units per second for the last kind).
+ * `scratch` is a device buffer of at least 1 KiB x compute units x waves_per_simd that the kernel writes its
+ * (meaningless) results to.  The call times six launches with a pair of events and synchronises on them. */
+#define M2D_RATE_FMA 0
+#define M2D_RATE_FMA_DEPENDENT 1
+#define M2D_RATE_EXP 2
+#define M2D_RATE_EXP_DEPENDENT 3
+#define M2D_RATE_SCAN_FWD_UNIT 4
+int m2d_valu_rate_probe(int kind, int waves_per_simd, void* scratch, size_t scratch_bytes, void* stream, double* per_second);
+
 #ifdef __cplusplus
 }
 #endif

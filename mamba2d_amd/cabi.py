@@ -27,7 +27,7 @@ M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
            "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_fwd_noalloc", "m2d_scan_link_error", "m2d_scan_plan", "m2d_scan_bwd", "m2d_proj_workspace_bytes", "m2d_proj_fwd",
            "m2d_proj_bwd", "m2d_layernorm_fwd", "m2d_dwconv3x3_fwd", "m2d_starrelu_fwd",
-           "m2d_scale_residual_fwd", "m2d_scale_residual_layernorm_fwd", "m2d_rope_qknorm_fwd", "m2d_rope_attention_fwd", "m2d_mlp_fwd", "m2d_layernorm_linear_fwd", "m2d_linear_fwd", "m2d_profile_enable", "m2d_profile_last_ms")
+           "m2d_scale_residual_fwd", "m2d_scale_residual_layernorm_fwd", "m2d_rope_qknorm_fwd", "m2d_rope_attention_fwd", "m2d_mlp_fwd", "m2d_layernorm_linear_fwd", "m2d_linear_fwd", "m2d_profile_enable", "m2d_profile_last_ms", "m2d_valu_rate_probe")
 
 
 class Desc(ctypes.Structure):
@@ -61,6 +61,8 @@ def _load():
     lib.m2d_scan_fwd.argtypes = [dp] + [vp] * 9 + [vp, vp, sz, vp, sz, vp]
     lib.m2d_scan_link_error.restype = i32
     lib.m2d_scan_link_error.argtypes = [dp, vp, vp, ctypes.POINTER(ctypes.c_int)]
+    lib.m2d_valu_rate_probe.restype = i32
+    lib.m2d_valu_rate_probe.argtypes = [i32, i32, vp, sz, vp, ctypes.POINTER(ctypes.c_double)]
     lib.m2d_scan_plan.restype = i32
     lib.m2d_scan_plan.argtypes = [dp, i32, ctypes.c_char_p, sz]
     lib.m2d_scan_fwd_noalloc.restype = i32
@@ -111,6 +113,19 @@ def profile_last_ms(which: int) -> float:
     ms = ctypes.c_float(0.0)
     check(lib.m2d_profile_last_ms(which, ctypes.byref(ms)))
     return float(ms.value)
+
+
+RATE_KINDS = {"fma": 0, "fma_dependent": 1, "exp": 2, "exp_dependent": 3, "scan_fwd_unit": 4}
+
+
+def valu_rate_probe(kind: str, waves_per_simd: int = 2, device=None) -> float:
+    """Lane-operations per second (units per second for "scan_fwd_unit") that the vector ALUs of the device issue,
+    measured by m2d_valu_rate_probe."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else device
+    scratch = torch.empty(1024 * torch.cuda.get_device_properties(dev).multi_processor_count * waves_per_simd, dtype=torch.uint8, device=dev)
+    rate = ctypes.c_double(0.0)
+    check(lib.m2d_valu_rate_probe(RATE_KINDS[kind], waves_per_simd, _ptr(scratch), scratch.numel(), _stream(dev), ctypes.byref(rate)))
+    return float(rate.value)
 
 
 def status_str(code: int) -> str:

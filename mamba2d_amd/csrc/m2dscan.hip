@@ -2986,6 +2986,63 @@ __global__ void m2d_finalize_kernel(const ScanParams p, T* dC, T* dBT, T* dBL, v
   }
 }
 
+
+// ------------------------------------------------------------------ instruction-rate probe
+// What the vector ALUs of this device issue per second, measured (m2d_valu_rate_probe): the scan kernels are
+// bound by instruction issue, and the ceiling they are priced against should not be a nominal clock times a lane
+// count.  Every lane runs kProbeIters x 16 operations of one kind on values that stay in registers:
+//   independent: 16 chains per lane (what a kernel with enough parallel work in a lane sees),
+//   dependent:   one chain per lane (every operation waits for the one before),
+// for v_fma_f32 and for v_exp_f32, and the forward scan's own mix per (cell, channel, state): two gate
+// exponents with their multiply-adds and the five multiply-adds of the state and output update.
+constexpr int kProbeIters = 4096;
+template <int KIND>
+__global__ __launch_bounds__(256) void m2d_rate_probe_kernel(float* out, float a, float b) {
+  float r[16];
+#pragma unroll
+  for (int i = 0; i < 16; ++i) r[i] = -(threadIdx.x * 0.001f + i) * 0.01f;
+  if constexpr (KIND == M2D_RATE_FMA) {
+    for (int it = 0; it < kProbeIters; ++it)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) r[i] = __builtin_fmaf(r[i], a, b);
+  } else if constexpr (KIND == M2D_RATE_FMA_DEPENDENT) {
+    for (int it = 0; it < kProbeIters; ++it)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) r[0] = __builtin_fmaf(r[0], a, b);
+  } else if constexpr (KIND == M2D_RATE_EXP) {
+    for (int it = 0; it < kProbeIters; ++it)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) r[i] = fexp2(r[i]);
+  } else if constexpr (KIND == M2D_RATE_EXP_DEPENDENT) {
+    for (int it = 0; it < kProbeIters; ++it)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) r[0] = fexp2(r[0]);
+  } else {   // M2D_RATE_SCAN_FWD_UNIT: r are 16 states; one iteration is one step of a cell and channel
+    float acc = 0.f, d = a, sT = b, sL = a * b;
+    for (int it = 0; it < kProbeIters; ++it) {
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const float gT = fexp2(__builtin_fmaf(d, -0.01f * (i + 1), -1.f));
+        const float gL = fexp2(__builtin_fmaf(sT, -0.02f * (i + 1), -1.f));
+        float u = sL * (0.5f + i);
+        u = __builtin_fmaf(sT, 0.25f * i, u);
+        u = __builtin_fmaf(gT, r[(i + 1) & 15], u);
+        r[i] = __builtin_fmaf(gL, r[i], u);
+        acc = __builtin_fmaf(r[i], d, acc);
+      }
+      // (the step's operands change from step to step, as a cell's do: nothing of a unit can leave the loop)
+      d = __builtin_fmaf(acc, 1e-30f, d);
+      sT = __builtin_fmaf(acc, 2e-30f, sT);
+      sL = __builtin_fmaf(acc, 3e-30f, sL);
+    }
+    r[0] += acc;
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) s += r[i];
+  out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
 // ------------------------------------------------------------------------------------ host side
 // Optional timing of the main kernel of each pass (off by default; see m2d_profile_enable).
 bool g_profile = false;
@@ -3689,6 +3746,40 @@ int m2d_scan_link_error(const m2d_desc* desc, const void* workspace, void* strea
   if (hipStreamSynchronize(st) != hipSuccess) return M2D_ERR_HIP;
   if (hipMemcpy(&word, static_cast<const char*>(workspace) + g.prep_bytes, sizeof(word), hipMemcpyDeviceToHost) != hipSuccess) return M2D_ERR_HIP;
   *gave_up = word != 0;
+  return M2D_OK;
+}
+
+int m2d_valu_rate_probe(int kind, int waves_per_simd, void* scratch, size_t scratch_bytes, void* stream, double* per_second) {
+  if (!scratch || !per_second) return M2D_ERR_NULL_POINTER;
+  if (kind < M2D_RATE_FMA || kind > M2D_RATE_SCAN_FWD_UNIT || waves_per_simd < 1 || waves_per_simd > 8) return M2D_ERR_UNSUPPORTED;
+  const int cus = device_cus();
+  const int blocks = cus * waves_per_simd;                 // 4 waves each: one per SIMD of a compute unit
+  if (scratch_bytes < (size_t)blocks * 256 * sizeof(float)) return M2D_ERR_WORKSPACE;
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  float* out = static_cast<float*>(scratch);
+  auto launch = [&] {
+    switch (kind) {
+      case M2D_RATE_FMA: hipLaunchKernelGGL(m2d_rate_probe_kernel<M2D_RATE_FMA>, dim3(blocks), dim3(256), 0, st, out, 1.0001f, 0.5f); break;
+      case M2D_RATE_FMA_DEPENDENT: hipLaunchKernelGGL(m2d_rate_probe_kernel<M2D_RATE_FMA_DEPENDENT>, dim3(blocks), dim3(256), 0, st, out, 1.0001f, 0.5f); break;
+      case M2D_RATE_EXP: hipLaunchKernelGGL(m2d_rate_probe_kernel<M2D_RATE_EXP>, dim3(blocks), dim3(256), 0, st, out, 1.0001f, 0.5f); break;
+      case M2D_RATE_EXP_DEPENDENT: hipLaunchKernelGGL(m2d_rate_probe_kernel<M2D_RATE_EXP_DEPENDENT>, dim3(blocks), dim3(256), 0, st, out, 1.0001f, 0.5f); break;
+      default: hipLaunchKernelGGL(m2d_rate_probe_kernel<M2D_RATE_SCAN_FWD_UNIT>, dim3(blocks), dim3(256), 0, st, out, 1.0001f, 0.5f); break;
+    }
+  };
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  if (hipEventCreate(&e0) != hipSuccess || hipEventCreate(&e1) != hipSuccess) { if (e0) (void)hipEventDestroy(e0); return M2D_ERR_HIP; }
+  constexpr int kReps = 5;
+  launch();   // (warm-up: code upload, clocks)
+  (void)hipEventRecord(e0, st);
+  for (int i = 0; i < kReps; ++i) launch();
+  (void)hipEventRecord(e1, st);
+  float ms = 0.f;
+  const bool ok = hipGetLastError() == hipSuccess && hipEventSynchronize(e1) == hipSuccess && hipEventElapsedTime(&ms, e0, e1) == hipSuccess && ms > 0.f;
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (!ok) return M2D_ERR_HIP;
+  // lane-operations (FMA, EXP kinds) or (cell, channel, state) units (the scan mix) per second, whole device
+  *per_second = (double)blocks * 256 * 16.0 * kProbeIters * kReps / (ms * 1e-3);
   return M2D_OK;
 }
 
