@@ -423,6 +423,19 @@ __device__ __forceinline__ Pos pos_after(const ScanParams& p, Pos A, int d) {
 // loop, where it would also wait for the asynchronous staging copies.
 __device__ __forceinline__ void settle_loads() { __builtin_amdgcn_s_waitcnt(0x0F70); }
 
+// Two waves share a SIMD where a workgroup has 8 (wave w and wave w + 4), and between two barriers both have the same
+// work.  Left alone the instruction arbiter favours the older wave throughout: it reaches the barrier early and
+// idles there while the younger one finishes alone, at the rate of a single wave (a quarter of the older waves'
+// time went into such waits in the backward kernel).  So the younger wave raises its priority for the first part of
+// every barrier interval and drops it for the rest, where age favours the older one again: both arrive together.
+// (s_setprio changes the wave's own priority among the waves of its SIMD, nothing else.)
+template <int NW>
+__device__ __forceinline__ void lead_if_younger(int wave, bool lead) {
+  if constexpr (NW == 8) {
+    if (wave >= NW / 2) { if (lead) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(0); }
+  }
+}
+
 // all direct-to-LDS loads of this wave have landed ...
 __device__ __forceinline__ void staging_landed() {
   asm volatile("" ::: "memory");
@@ -1207,11 +1220,13 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
           // barrier, and no wave reads the current buffer any more.
           next_block_landed();
           __syncthreads();
+          lead_if_younger<NW>(wave, true);   // (from here to the second step of the next block: half of the way to the next barrier)
           // every wave has waited for the rows it stored at the steps 0 and 1 of this block
           if constexpr (SLICED) link.publish((uint32_t)(m - m_lo + 1));
           if constexpr (YTILE) flush_y(ypar, m, false);   // the last step of the block before and the first three of this one
           if (!last) fetch(bufn, 0, ahead);
         }
+        if (k == 1) lead_if_younger<NW>(wave, false);
         step(k, now);   // also past the end of the sweep (last block): zero operands like any position off the grid, nothing stored
       }
     } else {
@@ -1221,6 +1236,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
         // block.  Waiting here, before the stores of the last step are issued, keeps the latency
         // of those stores off the critical path (the counter covers loads and stores alike).
         if (k == kCK - 1) next_block_landed();
+        if (k == 0 || k == kCK / 2) lead_if_younger<NW>(wave, k == 0);
         fetch(bufc, k, opsA);
         step(k, opsA);
       }
@@ -1849,6 +1865,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
     for (int half = 0; half < 2; ++half) {
       float hb[kCK + 1][8];
       float gT_last[8], gL_last[8];   // gates of the last step: the adjoint starts with them
+      if constexpr (BATCH) lead_if_younger<NW>(wave, true);   // (a barrier interval is a half: until the middle of its adjoint)
       // the states before the block: quad mg of the snapshot holds the states fold_state(mg, 0..3) in this order
       // (widened here, half by half: until then the snapshot stays as it came from memory)
       static_assert(sinv<PERM>(4 * 2 + 1) == fold_state(2, 1) && sinv<PERM>(4 * 3 + 2) == fold_state(3, 2), "snapshot quads are state groups");
@@ -1919,6 +1936,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
       for (int k = kCK - 1; k >= 0; --k) {
         const int t = t0 + k;
         if (half == 1 && k == 0) staging_landed();   // before the last stores of the block, see the forward kernel
+        if constexpr (BATCH) { if (k == 1) lead_if_younger<NW>(wave, false); }
         // the states of the later steps are dead by now: their registers take the next snapshot
         // (a longer checkpoint interval: not where the block before is the last of its group, whose state the replay will bring)
         if (!LATE_SNAPSHOT && half == 1 && k == (kCK > 1 ? 1 : 0) && m > m_lo && !opens_group(m - 1)) load_ckpt(m - 1, ck_take);
@@ -2305,6 +2323,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd2_kernel(const ScanParams pin)
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
         float ha[8], hb1[8], hn[8], gT[8], gL[8];
+        lead_if_younger<NW>(wave, true);    // (until the second step of the adjoint below)
         widen8(qa[half], ha);
         widen8(qn[half], hn);
         qn[half][0] = qa[half][0]; qn[half][1] = qa[half][1];
@@ -2366,6 +2385,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd2_kernel(const ScanParams pin)
         for (int ks = 1; ks >= 0; --ks) {
           const int k = k0 + ks;
           const int t = t0 + k;
+          if (ks == 0) lead_if_younger<NW>(wave, false);
           if (sub == 0 && half == 1 && ks == 0) staging_landed();   // before the last stores of the block, see the forward kernel
           if (t < p.T_total) {
             const float (&hbk)[8] = ks == 1 ? hb1 : ha;    // the state before this step
