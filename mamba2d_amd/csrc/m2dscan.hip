@@ -1496,6 +1496,7 @@ __global__ __launch_bounds__(NWS * 64) void m2d_fwd_split_kernel(const ScanParam
 #pragma unroll
     for (int k = 0; k < kCK; ++k) {
       if (k == kCK - 1) staging_landed_behind_n(younger);
+      if (k == 0 || k == kCK / 2) lead_if_younger<NW>(wave, k == 0);
       step(bufc, k);
     }
     __syncthreads();
