@@ -350,6 +350,24 @@ int m2d_mlp_fwd(int64_t P, int C, int hidden, int weight_dtype, const void* x,
 int m2d_profile_enable(int on);
 int m2d_profile_last_ms(int pass, float* ms);
 
+/* ---- The reference's native entry points at their own boundary -----------------------------------
+ * wf_fwd and wf_bwd as the reference's extension exports them (wf_cuda_bind.cpp:24-46), for callers of its
+ * custom operators mamba2d::wf_fwd / mamba2d::wf_bwd (wavefront_cuda.py:25-57): they materialise the state
+ * tensor hs (B,H,W,E,N), which the fused calls above never do, take any number of states N and the three
+ * element types the reference dispatches (wf_cuda.cu:182,240), and are not on the fast path.  dtype names the one
+ * element type of every tensor: M2D_F32, M2D_BF16 (fp32 arithmetic, every stored value rounded once) or M2D_F64.
+ *
+ * m2d_wf_fwd fills hs with the recurrence of wf_cuda.cu:40-69.
+ * m2d_wf_bwd is wf_cuda.cu:108-160: grad_output (B,H,W,E,N) holds dL/dhs on entry and dBX on return, dDAT and
+ * dDAL (B,H,W,E,N) are written, omega (2,B,H,E,N) is scratch; x is not read (as in the reference).
+ * All pointers are device pointers to contiguous arrays; one launch per call, nothing is allocated. */
+#define M2D_F64 2
+int m2d_wf_fwd(int B, int H, int W, int E, int N, int dtype, void* hs, const void* x, const void* deltaT,
+               const void* deltaL, const void* BT, const void* BL, const void* AT, const void* AL, void* stream);
+int m2d_wf_bwd(int B, int H, int W, int E, int N, int dtype, const void* hs, const void* x, const void* deltaT,
+               const void* deltaL, const void* AT, const void* AL, void* grad_output, void* dDAT, void* dDAL,
+               void* omega, void* stream);
+
 /* Measurement aid; no counterpart in the reference.  What the vector ALUs of the current device issue per
  * second, measured by a small kernel that fills the device with `waves_per_simd` waves per SIMD (1 to 8; the scan
  * kernels run 2), each lane running 65536 operations of one kind on registers:

@@ -36,6 +36,7 @@ SOURCES = {
     "m2dscan.hip": ["-mllvm", "-amdgpu-sched-strategy=iterative-ilp"],
     "m2dproj.hip": [],
     "m2dblock.hip": [],
+    "m2dcompat.hip": [],
 }
 
 

@@ -27,7 +27,7 @@ M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
            "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_fwd_noalloc", "m2d_scan_link_error", "m2d_scan_plan", "m2d_scan_bwd", "m2d_proj_workspace_bytes", "m2d_proj_fwd",
            "m2d_proj_bwd", "m2d_layernorm_fwd", "m2d_dwconv3x3_fwd", "m2d_starrelu_fwd",
-           "m2d_scale_residual_fwd", "m2d_scale_residual_layernorm_fwd", "m2d_rope_qknorm_fwd", "m2d_rope_attention_fwd", "m2d_mlp_fwd", "m2d_layernorm_linear_fwd", "m2d_linear_fwd", "m2d_profile_enable", "m2d_profile_last_ms", "m2d_valu_rate_probe")
+           "m2d_scale_residual_fwd", "m2d_scale_residual_layernorm_fwd", "m2d_rope_qknorm_fwd", "m2d_rope_attention_fwd", "m2d_mlp_fwd", "m2d_layernorm_linear_fwd", "m2d_linear_fwd", "m2d_profile_enable", "m2d_profile_last_ms", "m2d_valu_rate_probe", "m2d_wf_fwd", "m2d_wf_bwd")
 
 
 class Desc(ctypes.Structure):
@@ -63,6 +63,10 @@ def _load():
     lib.m2d_scan_link_error.argtypes = [dp, vp, vp, ctypes.POINTER(ctypes.c_int)]
     lib.m2d_valu_rate_probe.restype = i32
     lib.m2d_valu_rate_probe.argtypes = [i32, i32, vp, sz, vp, ctypes.POINTER(ctypes.c_double)]
+    lib.m2d_wf_fwd.restype = i32
+    lib.m2d_wf_fwd.argtypes = [i32] * 6 + [vp] * 9
+    lib.m2d_wf_bwd.restype = i32
+    lib.m2d_wf_bwd.argtypes = [i32] * 6 + [vp] * 11
     lib.m2d_scan_plan.restype = i32
     lib.m2d_scan_plan.argtypes = [dp, i32, ctypes.c_char_p, sz]
     lib.m2d_scan_fwd_noalloc.restype = i32

@@ -454,6 +454,51 @@ Tensor layernorm_linear_act_fwd(const Tensor& x, const Tensor& ln_weight, const 
 
 int64_t abi_version() { return m2d_version(); }
 
+// ---- the reference's own pair of in-place operators, mamba2d::wf_fwd and mamba2d::wf_bwd (wavefront_cuda.py:25-57),
+// for callers that use them directly: same names, argument order and mutated arguments; any number of states;
+// float64, float32 and bfloat16 (wf_cuda.cu:182,240).  They materialise hs and are not on the fast path.
+int wf_dtype(const Tensor& hs) {
+  if (hs.scalar_type() == at::kFloat) return M2D_F32;
+  if (hs.scalar_type() == at::kBFloat16) return M2D_BF16;
+  if (hs.scalar_type() == at::kDouble) return M2D_F64;
+  TORCH_CHECK(false, "mamba2d::wf_*: float64, float32 and bfloat16 are supported, got ", hs.scalar_type());
+}
+void wf_expect(const Tensor& t, const char* name, const Tensor& hs, at::IntArrayRef shape) {
+  TORCH_CHECK(t.device() == hs.device(), "mamba2d::wf_*: ", name, " is on ", t.device(), ", hs on ", hs.device());
+  TORCH_CHECK(t.scalar_type() == hs.scalar_type(), "mamba2d::wf_*: ", name, " has dtype ", t.scalar_type(), ", hs has ",
+              hs.scalar_type(), " (all tensors share one dtype, as the reference's accessors require)");
+  TORCH_CHECK(t.sizes() == shape, "mamba2d::wf_*: ", name, " has shape ", t.sizes(), ", expected ", shape);
+  TORCH_CHECK(t.is_contiguous(), "mamba2d::wf_*: ", name, " must be contiguous");
+}
+
+void wf_fwd(Tensor& hs, const Tensor& x, const Tensor& dT, const Tensor& dL, const Tensor& BT, const Tensor& BL,
+            const Tensor& AT, const Tensor& AL) {
+  TORCH_CHECK(hs.dim() == 5 && hs.is_contiguous(), "mamba2d::wf_fwd: hs must be a contiguous (B,H,W,E,N) tensor, got ", hs.sizes());
+  const int64_t B = hs.size(0), H = hs.size(1), W = hs.size(2), E = hs.size(3), N = hs.size(4);
+  wf_expect(x, "x", hs, {B, H, W, E}); wf_expect(dT, "deltaT", hs, {B, H, W, E}); wf_expect(dL, "deltaL", hs, {B, H, W, E});
+  wf_expect(BT, "BT", hs, {B, H, W, N}); wf_expect(BL, "BL", hs, {B, H, W, N});
+  wf_expect(AT, "AT", hs, {E, N}); wf_expect(AL, "AL", hs, {E, N});
+  c10::DeviceGuard guard(hs.device());
+  hipStream_t st = c10::hip::getCurrentHIPStream(hs.device().index()).stream();
+  check(m2d_wf_fwd((int)B, (int)H, (int)W, (int)E, (int)N, wf_dtype(hs), hs.data_ptr(), x.data_ptr(), dT.data_ptr(), dL.data_ptr(),
+                   BT.data_ptr(), BL.data_ptr(), AT.data_ptr(), AL.data_ptr(), st));
+}
+
+void wf_bwd(const Tensor& hs, const Tensor& x, const Tensor& dT, const Tensor& dL, const Tensor& AT, const Tensor& AL,
+            Tensor& grad_output, Tensor& dDAT, Tensor& dDAL, Tensor& omega) {
+  TORCH_CHECK(hs.dim() == 5 && hs.is_contiguous(), "mamba2d::wf_bwd: hs must be a contiguous (B,H,W,E,N) tensor, got ", hs.sizes());
+  const int64_t B = hs.size(0), H = hs.size(1), W = hs.size(2), E = hs.size(3), N = hs.size(4);
+  wf_expect(x, "x", hs, {B, H, W, E}); wf_expect(dT, "deltaT", hs, {B, H, W, E}); wf_expect(dL, "deltaL", hs, {B, H, W, E});
+  wf_expect(AT, "AT", hs, {E, N}); wf_expect(AL, "AL", hs, {E, N});
+  wf_expect(grad_output, "grad_output", hs, hs.sizes()); wf_expect(dDAT, "dDAT", hs, hs.sizes()); wf_expect(dDAL, "dDAL", hs, hs.sizes());
+  wf_expect(omega, "omega", hs, {2, B, H, E, N});
+  c10::DeviceGuard guard(hs.device());
+  hipStream_t st = c10::hip::getCurrentHIPStream(hs.device().index()).stream();
+  check(m2d_wf_bwd((int)B, (int)H, (int)W, (int)E, (int)N, wf_dtype(hs), hs.data_ptr(), x.data_ptr(), dT.data_ptr(), dL.data_ptr(),
+                   AT.data_ptr(), AL.data_ptr(), grad_output.data_ptr(), dDAT.data_ptr(), dDAL.data_ptr(), omega.data_ptr(), st));
+}
+
+
 }  // namespace
 
 TORCH_LIBRARY(m2dscan, m) {
@@ -501,4 +546,15 @@ TORCH_LIBRARY_IMPL(m2dscan, CUDA, m) {   // ROCm devices dispatch under the CUDA
   m.impl("mlp_fwd", &mlp_fwd);
   m.impl("layernorm_linear_act_fwd", &layernorm_linear_act_fwd);
   m.impl("linear_act_fwd", &linear_act_fwd);
+}
+
+TORCH_LIBRARY(mamba2d, m) {   // the reference's operator names (wavefront_cuda.py:25, :40), same mutated arguments
+  m.def("wf_fwd(Tensor(a!) hs, Tensor x, Tensor deltaT, Tensor deltaL, Tensor BT, Tensor BL, Tensor AT, Tensor AL) -> ()");
+  m.def("wf_bwd(Tensor hs, Tensor x, Tensor deltaT, Tensor deltaL, Tensor AT, Tensor AL, Tensor(a!) grad_output, "
+        "Tensor(b!) dDAT, Tensor(c!) dDAL, Tensor(d!) omega) -> ()");
+}
+
+TORCH_LIBRARY_IMPL(mamba2d, CUDA, m) {
+  m.impl("wf_fwd", &wf_fwd);
+  m.impl("wf_bwd", &wf_bwd);
 }

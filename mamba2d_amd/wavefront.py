@@ -34,6 +34,10 @@ torch.ops.load_library(_SHIM)
 
 scan_fwd_op = torch.ops.m2dscan.scan_fwd
 scan_bwd_op = torch.ops.m2dscan.scan_bwd
+# the reference's own pair of in-place operators, same names and mutated arguments (wavefront_cuda.py:25-57): hs is
+# materialised, any number of states, float64 / float32 / bfloat16.  Not on the fast path.
+wf_fwd_op = torch.ops.mamba2d.wf_fwd
+wf_bwd_op = torch.ops.mamba2d.wf_bwd
 proj_fwd_op = torch.ops.m2dscan.proj_fwd
 proj_bwd_op = torch.ops.m2dscan.proj_bwd
 layernorm_fwd_op = torch.ops.m2dscan.layernorm_fwd
@@ -98,6 +102,16 @@ def _scan_bwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt, flip, raw_
     bc = [x.new_empty((*x.shape[:3], AT.shape[1])) for _ in range(3)]
     return [torch.empty_like(x), torch.empty_like(deltaT), torch.empty_like(deltaL), torch.empty_like(AT), torch.empty_like(AL),
             *bc, torch.empty_like(D)]
+
+
+@torch.library.register_fake("mamba2d::wf_fwd")
+def _wf_fwd_fake(hs, x, deltaT, deltaL, BT, BL, AT, AL):
+    return None
+
+
+@torch.library.register_fake("mamba2d::wf_bwd")
+def _wf_bwd_fake(hs, x, deltaT, deltaL, AT, AL, grad_output, dDAT, dDAL, omega):
+    return None
 
 
 @torch.library.register_fake("m2dscan::proj_fwd")
@@ -170,6 +184,28 @@ def _rope_qknorm_fwd_fake(qkv, cos, sin, q_weight, q_bias, k_weight, k_bias, eps
     if token_major:
         return qkv.new_empty((B, L, nh, hd)).permute(0, 2, 1, 3), qkv.new_empty((B, L, nh, hd)).permute(0, 2, 1, 3)
     return qkv.new_empty((B, nh, L, hd)), qkv.new_empty((B, nh, L, hd))
+
+
+def fused_backward_math(dDAT, dDAL, dHS_total, deltaT, deltaL, AT, AL, BT, BL, x):
+    """The reference's tensor algebra behind ``wf_bwd`` (``wavefront_cuda.py:97-139``), for callers of the
+    operator pair ``wf_fwd_op`` / ``wf_bwd_op``: from ``dDAT``, ``dDAL`` and ``dBX`` (``dHS_total``), all
+    (B,H,W,E,N), the gradients ``(d_x_scan, d_deltaT, d_deltaL, d_AT, d_AL, d_BT, d_BL)``.  The fused backward
+    (``m2dscan::scan_bwd``) computes the same sums inside its kernel and never forms these tensors."""
+    H, W = dHS_total.shape[1:3]
+    zT = dDAT * torch.exp(deltaT.unsqueeze(-1) * AT)              # gradients with respect to the gate exponents
+    zL = dDAL * torch.exp(deltaL.unsqueeze(-1) * AL)
+    d_AT = torch.einsum("bhwen,bhwe->en", zT, deltaT)
+    d_AL = torch.einsum("bhwen,bhwe->en", zL, deltaL)
+    rows = torch.arange(H, device=x.device).view(1, H, 1, 1, 1)
+    cols = torch.arange(W, device=x.device).view(1, 1, W, 1, 1)
+    gT = dHS_total * (rows > 0)                                   # the T input reaches every row but the first,
+    gL = dHS_total * ((cols > 0) | (rows == 0))                   # the L input every column but the first, and the origin
+    d_deltaT = (zT * AT).sum(-1) + torch.einsum("bhwen,bhwn->bhwe", gT, BT) * x
+    d_deltaL = (zL * AL).sum(-1) + torch.einsum("bhwen,bhwn->bhwe", gL, BL) * x
+    d_BT = torch.einsum("bhwen,bhwe->bhwn", gT, deltaT * x)
+    d_BL = torch.einsum("bhwen,bhwe->bhwn", gL, deltaL * x)
+    d_x_scan = torch.einsum("bhwen,bhwn->bhwe", gT, BT) * deltaT + torch.einsum("bhwen,bhwn->bhwe", gL, BL) * deltaL
+    return d_x_scan, d_deltaT, d_deltaL, d_AT, d_AL, d_BT, d_BL
 
 
 def proj_params(x, AT_log, AL_log, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b):

@@ -64,3 +64,40 @@ def test_fake_checkpoint_size_matches_the_library(shape, dtype, packed):
     d = cabi.Desc(B, H, W, E, N, cabi.M2D_BF16 if dtype == torch.bfloat16 else cabi.M2D_F32,
                   cabi.M2D_FLAG_PACKED_BC if packed else 0, 0)
     assert ck.numel() == cabi.lib.m2d_scan_ckpt_bytes(ctypes.byref(d)) and y.shape == x.shape
+
+
+def test_reference_operator_pair_on_meta_tensors(wf):
+    """mamba2d::wf_fwd / mamba2d::wf_bwd carry the reference's names, argument order and mutated arguments
+    (wavefront_cuda.py:25-57) and trace on meta tensors (they return nothing, like the reference's fakes), and the
+    reference module's names resolve in the import-path twin."""
+    from mamba2d_amd.kernels import wavefront_cuda as twin
+    for name in ("wavefront_scan_cuda", "wf_cuda_fn_pr", "wf_cuda_fn_fr", "proj_params", "fused_backward_math", "wf_fwd_op", "wf_bwd_op"):
+        assert hasattr(twin, name), name
+    B, H, W, E, N = 2, 3, 4, 5, 6
+    m = lambda *s: torch.empty(*s, dtype=torch.float64, device="meta")
+    hs = m(B, H, W, E, N)
+    assert wf.wf_fwd_op(hs, m(B, H, W, E), m(B, H, W, E), m(B, H, W, E), m(B, H, W, N), m(B, H, W, N), m(E, N), m(E, N)) is None
+    assert wf.wf_bwd_op(hs, m(B, H, W, E), m(B, H, W, E), m(B, H, W, E), m(E, N), m(E, N), m(B, H, W, E, N), m(B, H, W, E, N),
+                        m(B, H, W, E, N), m(2, B, H, E, N)) is None
+    s_fwd, s_bwd = torch.ops.mamba2d.wf_fwd.default._schema, torch.ops.mamba2d.wf_bwd.default._schema
+    assert [a.name for a in s_fwd.arguments] == ["hs", "x", "deltaT", "deltaL", "BT", "BL", "AT", "AL"]
+    assert [a.name for a in s_bwd.arguments] == ["hs", "x", "deltaT", "deltaL", "AT", "AL", "grad_output", "dDAT", "dDAL", "omega"]
+    assert [a.name for a in s_fwd.arguments if a.is_write] == ["hs"]
+    assert [a.name for a in s_bwd.arguments if a.is_write] == ["grad_output", "dDAT", "dDAL", "omega"]
+
+
+def test_fused_backward_math_against_autograd():
+    """wavefront.fused_backward_math (the reference's algebra behind wf_bwd, wavefront_cuda.py:97-139) in float64 on
+    the CPU: fed the oracle's dDAT, dDAL, dBX it must return the oracle's gradients."""
+    from mamba2d_amd import wavefront as wf
+    from oracle import scan_oracle as so
+    B, H, W, E, N = 2, 4, 5, 3, 6
+    inp = {k: v.double() for k, v in so.make_inputs(B, H, W, E, N, seed=3, dtype=torch.float32).items()}
+    cs = so.CScan()
+    res = cs.backward(*[inp[k] for k in so.INPUT_NAMES], inp["dy"], want_intermediates=True)
+    t = lambda a: torch.from_numpy(a)
+    out = wf.fused_backward_math(t(res["dDAT"]), t(res["dDAL"]), t(res["dBX"]), inp["deltaT"], inp["deltaL"], inp["AT"], inp["AL"],
+                                 inp["BT"], inp["BL"], inp["x"])
+    want = [res["d_x"] - (inp["dy"] * inp["D"]).numpy(), res["d_deltaT"], res["d_deltaL"], res["d_AT"], res["d_AL"], res["d_BT"], res["d_BL"]]
+    for got, w in zip(out, want):
+        assert so.rel_err(got, w) < 1e-12
