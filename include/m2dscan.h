@@ -115,6 +115,14 @@ typedef struct m2d_desc {
  * on it; so a linked sweep that failed shows in the caller's tensors.  Ignored by other schedules. */
 #define M2D_FLAG_TEST_DEAD_LINK 128
 
+/* The sums over channels d_BT, d_BL, d_C travel from m2d_scan_bwd to m2d_proj_bwd_parts unfinished.  The scan's
+ * backward kernel adds them up over the channels of a workgroup and normally a small second kernel adds the
+ * workgroups of an image and rounds; where the only reader is the projections' backward, that reader can do the
+ * last step while it loads them.  With this flag m2d_scan_bwd writes, to its d_BT argument, the fp32 records
+ * [parts][B*H*W][d_C | d_BT | d_BL][16] with parts = m2d_scan_sum_parts(desc) (the caller sizes the buffer with
+ * it), and leaves d_BL and d_C alone (they may be NULL).  The records are only meaningful to this library. */
+#define M2D_FLAG_SUM_PARTS 256
+
 #define M2D_PASS_FWD 0
 #define M2D_PASS_BWD 1
 
@@ -245,6 +253,25 @@ int m2d_proj_bwd(const m2d_desc* desc, int dt_rank,
                  float* d_dt_projL_w, float* d_dt_projL_b,
                  void* workspace, size_t workspace_bytes,
                  void* stream);
+
+/* Number of per-workgroup partial sums that m2d_scan_bwd leaves with M2D_FLAG_SUM_PARTS for this descriptor
+ * (0 for an invalid one); host only. */
+int m2d_scan_sum_parts(const m2d_desc* desc);
+
+/* m2d_proj_bwd for gradients d_BT, d_BL, d_C that arrive as the partial sums of M2D_FLAG_SUM_PARTS: d_BT points to
+ * sum_parts records as described there, which are added up in their order as they are loaded and rounded to
+ * desc->dtype; d_BL and d_C are ignored.  sum_parts = 0 is m2d_proj_bwd.  Only where the products run on the matrix
+ * cores (bf16, E a multiple of 8); otherwise M2D_ERR_UNSUPPORTED. */
+int m2d_proj_bwd_parts(const m2d_desc* desc, int dt_rank, int sum_parts,
+                       const void* x, const void* lowrank, const void* deltaT, const void* deltaL,
+                       const float* x_proj_w, const float* dt_projT_w, const float* dt_projL_w,
+                       const void* d_deltaT, const void* d_deltaL,
+                       const void* d_BT, const void* d_BL, const void* d_C,
+                       void* dx,
+                       float* d_x_proj_w, float* d_dt_projT_w, float* d_dt_projT_b,
+                       float* d_dt_projL_w, float* d_dt_projL_b,
+                       void* workspace, size_t workspace_bytes,
+                       void* stream);
 
 /* ---- Two operators of the residual block around the scan (inference forward) -------------------
  * The reference's blocks normalise channel-last activations with nn.LayerNorm over 64 to 512

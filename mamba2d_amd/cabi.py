@@ -22,11 +22,12 @@ M2D_FLAG_DPRE = 16
 M2D_FLAG_SPLIT_STATES = 32
 M2D_FLAG_WHOLE_STATES = 64
 M2D_FLAG_TEST_DEAD_LINK = 128
+M2D_FLAG_SUM_PARTS = 256
 M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",
            "m2d_scan_ckpt_bytes", "m2d_scan_fwd", "m2d_scan_fwd_noalloc", "m2d_scan_link_error", "m2d_scan_plan", "m2d_scan_bwd", "m2d_proj_workspace_bytes", "m2d_proj_fwd",
-           "m2d_proj_bwd", "m2d_layernorm_fwd", "m2d_dwconv3x3_fwd", "m2d_starrelu_fwd",
+           "m2d_proj_bwd", "m2d_proj_bwd_parts", "m2d_scan_sum_parts", "m2d_layernorm_fwd", "m2d_dwconv3x3_fwd", "m2d_starrelu_fwd",
            "m2d_scale_residual_fwd", "m2d_scale_residual_layernorm_fwd", "m2d_rope_qknorm_fwd", "m2d_rope_attention_fwd", "m2d_mlp_fwd", "m2d_layernorm_linear_fwd", "m2d_linear_fwd", "m2d_profile_enable", "m2d_profile_last_ms", "m2d_valu_rate_probe", "m2d_wf_fwd", "m2d_wf_bwd")
 
 
@@ -79,6 +80,10 @@ def _load():
     lib.m2d_proj_fwd.argtypes = [dp, i32] + [vp] * 12 + [vp, sz, vp]
     lib.m2d_proj_bwd.restype = i32
     lib.m2d_proj_bwd.argtypes = [dp, i32] + [vp] * 18 + [vp, sz, vp]
+    lib.m2d_proj_bwd_parts.restype = i32
+    lib.m2d_proj_bwd_parts.argtypes = [dp, i32, i32] + [vp] * 18 + [vp, sz, vp]
+    lib.m2d_scan_sum_parts.restype = i32
+    lib.m2d_scan_sum_parts.argtypes = [dp]
     lib.m2d_layernorm_fwd.restype = i32
     lib.m2d_layernorm_fwd.argtypes = [ctypes.c_int64, i32, i32, i32, vp, vp, vp, ctypes.c_float, vp, vp]
     lib.m2d_dwconv3x3_fwd.restype = i32
@@ -265,9 +270,11 @@ def scan_fwd_noalloc(x, deltaT, deltaL, AT, AL, BT, BL, C, D, y, flip=False):
     return y
 
 
-def scan_bwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt=None, flip=False, dpre=False):
+def scan_bwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt=None, flip=False, dpre=False, sum_parts=False):
     """The nine gradients (order of the inputs) through m2d_scan_bwd.  ``dpre``: d_deltaT and d_deltaL
-    come multiplied by the slope of the softplus that made the deltas (M2D_FLAG_DPRE)."""
+    come multiplied by the slope of the softplus that made the deltas (M2D_FLAG_DPRE).  ``sum_parts``:
+    d_BT comes back as the float32 per-workgroup sums (parts,B,H,W,3N) for ``proj_bwd(sum_parts=parts)``,
+    d_BL and d_C as None (M2D_FLAG_SUM_PARTS)."""
     _same(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy)
     _shapes(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy)
     d = make_desc(x, AT.shape[1], flip)
@@ -275,6 +282,10 @@ def scan_bwd(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt=None, flip=False,
         d.flags |= M2D_FLAG_DPRE
     check(lib.m2d_desc_check(ctypes.byref(d)))
     outs = [torch.empty_like(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D)]
+    if sum_parts:
+        d.flags |= M2D_FLAG_SUM_PARTS
+        parts = lib.m2d_scan_sum_parts(ctypes.byref(d))
+        outs[5:8] = [x.new_empty((parts, *x.shape[:3], 3 * AT.shape[1]), dtype=torch.float32), None, None]
     ws = _bytes(lib.m2d_scan_workspace_bytes(ctypes.byref(d), M2D_PASS_BWD, int(ckpt is not None)), x.device)
     check(lib.m2d_scan_bwd(ctypes.byref(d), *[_ptr(t) for t in (x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy)],
                            _ptr(ckpt), ckpt.numel() if ckpt is not None else 0, *[_ptr(t) for t in outs],
@@ -314,22 +325,29 @@ def proj_fwd(x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, N=16, 
 
 
 def proj_bwd(x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w, dt_projL_w, d_deltaT, d_deltaL, d_BT, d_BL, d_C, dx,
-             round_weights=False, dpre=False):
+             round_weights=False, dpre=False, sum_parts=0):
     """Adds the gradient through the projections to ``dx`` in place and returns the five weight
     gradients (x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b; float32) through m2d_proj_bwd.
     ``dpre``: d_deltaT and d_deltaL are gradients before the softplus (M2D_FLAG_DPRE); deltaT and deltaL
-    may then be None."""
-    N = d_BT.shape[-1]
+    may then be None.  ``sum_parts`` > 0: d_BT is the (sum_parts,B,H,W,3N) float32 tensor of
+    ``scan_bwd(sum_parts=True)``, d_BL and d_C are None (m2d_proj_bwd_parts)."""
+    N = d_BT.shape[-1] // 3 if sum_parts else d_BT.shape[-1]
     zb = torch.zeros(x.shape[-1], device=x.device)
     R = _proj_check(x, x_proj_w, dt_projT_w, zb, dt_projL_w, zb, N)
     B, H, W, E = x.shape
     given = [t for t in (deltaT, deltaL) if t is not None]
     if not dpre and len(given) < 2:
         raise ValueError("m2dscan: deltaT and deltaL are needed unless dpre is set")
-    _same(x, lowrank, *given, d_deltaT, d_deltaL, d_BT, d_BL, d_C, dx)
+    if sum_parts:
+        _same(x, lowrank, *given, d_deltaT, d_deltaL, dx)
+        if d_BT.dtype != torch.float32 or d_BT.device != x.device or not d_BT.is_contiguous():
+            raise ValueError("m2dscan: with sum_parts d_BT must be a contiguous float32 tensor on x's device")
+        bc = {"d_BT": (d_BT, (sum_parts, B, H, W, 3 * N))}
+    else:
+        _same(x, lowrank, *given, d_deltaT, d_deltaL, d_BT, d_BL, d_C, dx)
+        bc = {"d_BT": (d_BT, (B, H, W, N)), "d_BL": (d_BL, (B, H, W, N)), "d_C": (d_C, (B, H, W, N))}
     want = {"lowrank": (lowrank, (B, H, W, 2 * R)),
-            "d_deltaT": (d_deltaT, (B, H, W, E)), "d_deltaL": (d_deltaL, (B, H, W, E)), "d_BT": (d_BT, (B, H, W, N)),
-            "d_BL": (d_BL, (B, H, W, N)), "d_C": (d_C, (B, H, W, N)), "dx": (dx, (B, H, W, E))}
+            "d_deltaT": (d_deltaT, (B, H, W, E)), "d_deltaL": (d_deltaL, (B, H, W, E)), **bc, "dx": (dx, (B, H, W, E))}
     for k, t in zip(("deltaT", "deltaL"), (deltaT, deltaL)):
         if t is not None:
             want[k] = (t, (B, H, W, E))
@@ -340,7 +358,7 @@ def proj_bwd(x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w, dt_projL_w, d_del
     d.flags = (M2D_FLAG_ROUND_WEIGHTS if round_weights else 0) | (M2D_FLAG_DPRE if dpre else 0)
     outs = [torch.empty_like(t) for t in (x_proj_w, dt_projT_w, zb, dt_projL_w, zb)]
     ws = _bytes(lib.m2d_proj_workspace_bytes(ctypes.byref(d), R, M2D_PASS_BWD), x.device)
-    check(lib.m2d_proj_bwd(ctypes.byref(d), R, *[_ptr(t) for t in (x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w,
+    check(lib.m2d_proj_bwd_parts(ctypes.byref(d), R, int(sum_parts), *[_ptr(t) for t in (x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w,
                                                                   dt_projL_w, d_deltaT, d_deltaL, d_BT, d_BL, d_C, dx)],
                            *[_ptr(t) for t in outs], _ptr(ws), ws.numel(), _stream(x.device)))
     return tuple(outs)

@@ -109,8 +109,9 @@ std::tuple<Tensor, Tensor> scan_fwd(const Tensor& x, const Tensor& dT, const Ten
 std::vector<Tensor> scan_bwd(const Tensor& x, const Tensor& dT, const Tensor& dL, const Tensor& AT, const Tensor& AL,
                              const Tensor& BT, const Tensor& BL, const Tensor& C, const Tensor& D, const Tensor& dy,
                              const Tensor& ckpt, bool flip, bool raw_params, bool packed_bc, bool dpre,
-                             int64_t ckpt_interval) {
-  const m2d_desc d = describe(x, AT, flip, raw_params, packed_bc, dpre, ckpt_interval);
+                             int64_t ckpt_interval, bool sum_parts) {
+  m2d_desc d = describe(x, AT, flip, raw_params, packed_bc, dpre, ckpt_interval);
+  if (sum_parts) d.flags |= M2D_FLAG_SUM_PARTS;   // d_BT comes back as the fp32 per-workgroup sums for proj_bwd(sum_parts = its first size)
   expect_all(d, x, dT, dL, AT, AL, BT, BL, C, D);
   expect(dy, "dy", x, x.sizes());
   check(m2d_desc_check(&d));
@@ -124,6 +125,11 @@ std::vector<Tensor> scan_bwd(const Tensor& x, const Tensor& dT, const Tensor& dL
   std::vector<Tensor> g = {at::empty_like(x),  at::empty_like(dT), at::empty_like(dL), at::empty_like(AT), at::empty_like(AL),
                            at::empty(bc_shape, x.options()), at::empty(bc_shape, x.options()), at::empty(bc_shape, x.options()),
                            at::empty_like(D)};
+  if (sum_parts) {
+    g[5] = at::empty({m2d_scan_sum_parts(&d), d.B, d.H, d.W, 3 * d.N}, x.options().dtype(at::kFloat));
+    g[6] = at::empty({0}, x.options());
+    g[7] = at::empty({0}, x.options());
+  }
   Tensor ws = bytes(m2d_scan_workspace_bytes(&d, M2D_PASS_BWD, have), x);
   hipStream_t st = c10::hip::getCurrentHIPStream(x.device().index()).stream();
   check(m2d_scan_bwd(&d, x.data_ptr(), dT.data_ptr(), dL.data_ptr(), AT.data_ptr(), AL.data_ptr(), BT.data_ptr(),
@@ -187,9 +193,10 @@ std::vector<Tensor> proj_fwd(const Tensor& x, const Tensor& Wx, const Tensor& wT
 // mutating custom operator whose results are plain tensors.
 std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor> proj_bwd(const Tensor& x, const Tensor& low, const Tensor& dT, const Tensor& dL, const Tensor& Wx,
                              const Tensor& wT, const Tensor& wL, const Tensor& ddT, const Tensor& ddL, const Tensor& dBT,
-                             const Tensor& dBL, const Tensor& dC, Tensor dx, bool round_weights, bool dpre) {
-  TORCH_CHECK(dBT.dim() == 4 && wT.dim() == 2, "m2dscan: d_BT must be (B,H,W,N) and dt_projT_w (E, dt_rank)");
-  const int64_t N = dBT.size(3);
+                             const Tensor& dBL, const Tensor& dC, Tensor dx, bool round_weights, bool dpre, int64_t sum_parts) {
+  TORCH_CHECK(sum_parts >= 0 && dBT.dim() == (sum_parts ? 5 : 4) && wT.dim() == 2,
+              "m2dscan: d_BT must be (B,H,W,N), or (sum_parts,B,H,W,3N) as scan_bwd(sum_parts=True) returns it, and dt_projT_w (E, dt_rank)");
+  const int64_t N = sum_parts ? dBT.size(4) / 3 : dBT.size(3);
   m2d_desc d = describe_proj(x, N, round_weights);
   if (dpre) d.flags |= M2D_FLAG_DPRE;   // d_deltaT, d_deltaL are gradients before the softplus; deltaT, deltaL are not read
   const int64_t B = d.B, H = d.H, W = d.W, E = d.E, R = wT.size(1);
@@ -201,9 +208,15 @@ std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor> proj_bwd(const Tensor& x, con
   expect(dL, "deltaL", x, {B, H, W, E});
   expect(ddT, "d_deltaT", x, {B, H, W, E});
   expect(ddL, "d_deltaL", x, {B, H, W, E});
-  expect(dBT, "d_BT", x, {B, H, W, N});
-  expect(dBL, "d_BL", x, {B, H, W, N});
-  expect(dC, "d_C", x, {B, H, W, N});
+  if (sum_parts) {
+    TORCH_CHECK(dBT.device() == x.device() && dBT.scalar_type() == at::kFloat && dBT.is_contiguous() &&
+                dBT.sizes() == at::IntArrayRef({sum_parts, B, H, W, 3 * N}),
+                "m2dscan: d_BT must be the contiguous float32 (sum_parts,B,H,W,3N) tensor of scan_bwd(sum_parts=True)");
+  } else {
+    expect(dBT, "d_BT", x, {B, H, W, N});
+    expect(dBL, "d_BL", x, {B, H, W, N});
+    expect(dC, "d_C", x, {B, H, W, N});
+  }
   expect(dx, "dx", x, {B, H, W, E});
   c10::DeviceGuard guard(x.device());
   std::vector<Tensor> g = {at::empty_like(Wx), at::empty_like(wT), at::empty({E}, wT.options()), at::empty_like(wL),
@@ -212,7 +225,7 @@ std::tuple<Tensor, Tensor, Tensor, Tensor, Tensor> proj_bwd(const Tensor& x, con
   TORCH_CHECK(need > 0, "m2dscan: projection shapes outside what the kernels are built for (N = 16, dt_rank <= 32, E <= 4096)");
   Tensor ws = bytes(need, x);
   hipStream_t st = c10::hip::getCurrentHIPStream(x.device().index()).stream();
-  check(m2d_proj_bwd(&d, static_cast<int>(R), x.data_ptr(), low.data_ptr(), dT.data_ptr(), dL.data_ptr(),
+  check(m2d_proj_bwd_parts(&d, static_cast<int>(R), static_cast<int>(sum_parts), x.data_ptr(), low.data_ptr(), dT.data_ptr(), dL.data_ptr(),
                      Wx.data_ptr<float>(), wT.data_ptr<float>(), wL.data_ptr<float>(), ddT.data_ptr(), ddL.data_ptr(),
                      dBT.data_ptr(), dBL.data_ptr(), dC.data_ptr(), dx.data_ptr(), g[0].data_ptr<float>(),
                      g[1].data_ptr<float>(), g[2].data_ptr<float>(), g[3].data_ptr<float>(), g[4].data_ptr<float>(),
@@ -506,12 +519,12 @@ TORCH_LIBRARY(m2dscan, m) {
         "Tensor D, bool save_ckpt, bool flip, bool raw_params=False, bool packed_bc=False, int ckpt_interval=0) -> (Tensor, Tensor)");
   m.def("scan_bwd(Tensor x, Tensor deltaT, Tensor deltaL, Tensor AT, Tensor AL, Tensor BT, Tensor BL, Tensor C, "
         "Tensor D, Tensor dy, Tensor ckpt, bool flip, bool raw_params=False, bool packed_bc=False, bool dpre=False, "
-        "int ckpt_interval=0) -> Tensor[]");
+        "int ckpt_interval=0, bool sum_parts=False) -> Tensor[]");
   m.def("proj_fwd(Tensor x, Tensor x_proj_w, Tensor dt_projT_w, Tensor dt_projT_b, Tensor dt_projL_w, Tensor dt_projL_b, "
         "int d_state, bool round_weights, bool packed_bc=False) -> Tensor[]");
   m.def("proj_bwd(Tensor x, Tensor lowrank, Tensor deltaT, Tensor deltaL, Tensor x_proj_w, Tensor dt_projT_w, "
         "Tensor dt_projL_w, Tensor d_deltaT, Tensor d_deltaL, Tensor d_BT, Tensor d_BL, Tensor d_C, Tensor(a!) dx, "
-        "bool round_weights, bool dpre=False) -> (Tensor, Tensor, Tensor, Tensor, Tensor)");
+        "bool round_weights, bool dpre=False, int sum_parts=0) -> (Tensor, Tensor, Tensor, Tensor, Tensor)");
   m.def("layernorm_fwd(Tensor x, Tensor weight, Tensor bias, float eps) -> Tensor");
   m.def("dwconv3x3_fwd(Tensor x, Tensor weight) -> Tensor");
   m.def("starrelu_fwd(Tensor x, Tensor scale, Tensor bias) -> Tensor");

@@ -87,6 +87,7 @@ struct ProjArgs {
   const void *x, *r, *dT, *dL;           // x (P,E); r (P,2R) = low-rank inputs of the two dt projections; delta (P,E)
   const void *ddT, *ddL, *dBT, *dBL, *dC;
   int dpre_given;                        // ddT, ddL hold the gradients before the softplus already (dT, dL are not read)
+  int sum_parts;                         // > 0: dBT points to that many fp32 records [P][dC | dBT | dBL][16] to add up (the scan's per-workgroup sums)
   void *r_out, *dT_out, *dL_out, *BT_out, *BL_out, *C_out, *dx;
   float* bc_packed;                      // (P,48) fp32 records for the scan kernels instead of BT_out, BL_out, C_out (or null)
   // packed weights, fp32, zero where padded
@@ -658,10 +659,27 @@ __global__ __launch_bounds__(kThreads, M2D_PROJ_OCC) void m2d_proj_bwd_data_mfma
   // dB_T, dB_L, dC: lane l holds 4 values of position l >> 2
   const int cb = l >> 2, n0 = 4 * (l & 3);
   uint2 bc[3];
+  if (a.sum_parts > 0) {   // (uniform) the scan's per-workgroup channel sums, added up here in their order and rounded once
+    const float* rec = static_cast<const float*>(a.dBT) + (p0 + cb) * (3 * kN) + n0;
 #pragma unroll
-  for (int w = 0; w < 3; ++w) {
-    const bf16_t* src = static_cast<const bf16_t*>(w == 0 ? a.dBT : (w == 1 ? a.dBL : a.dC)) + p0 * kN;
-    bc[w] = cb < rows ? *reinterpret_cast<const uint2*>(src + (uint32_t)(cb * kN + n0)) : make_uint2(0, 0);
+    for (int w = 0; w < 3; ++w) {
+      const int v = w == 0 ? 1 : (w == 1 ? 2 : 0);   // the records hold dC, dBT, dBL in this order
+      float4 sum = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (cb < rows) {
+        sum = *reinterpret_cast<const float4*>(rec + v * kN);
+        for (int g = 1; g < a.sum_parts; ++g) {
+          const float4 o = *reinterpret_cast<const float4*>(rec + (int64_t)g * a.P * (3 * kN) + v * kN);
+          sum.x += o.x; sum.y += o.y; sum.z += o.z; sum.w += o.w;
+        }
+      }
+      bc[w] = make_uint2(pack2(sum.x, sum.y), pack2(sum.z, sum.w));
+    }
+  } else {
+#pragma unroll
+    for (int w = 0; w < 3; ++w) {
+      const bf16_t* src = static_cast<const bf16_t*>(w == 0 ? a.dBT : (w == 1 ? a.dBL : a.dC)) + p0 * kN;
+      bc[w] = cb < rows ? *reinterpret_cast<const uint2*>(src + (uint32_t)(cb * kN + n0)) : make_uint2(0, 0);
+    }
   }
 
   // dz[., rank] = dpre w, channels as the inner dimension
@@ -1295,10 +1313,21 @@ int m2d_proj_bwd(const m2d_desc* desc, int dt_rank, const void* x, const void* l
                  const void* d_deltaT, const void* d_deltaL, const void* d_BT, const void* d_BL, const void* d_C,
                  void* dx, float* d_x_proj_w, float* d_dt_projT_w, float* d_dt_projT_b, float* d_dt_projL_w,
                  float* d_dt_projL_b, void* workspace, size_t workspace_bytes, void* stream) {
+  return m2d_proj_bwd_parts(desc, dt_rank, 0, x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w, dt_projL_w, d_deltaT, d_deltaL, d_BT, d_BL,
+                            d_C, dx, d_x_proj_w, d_dt_projT_w, d_dt_projT_b, d_dt_projL_w, d_dt_projL_b, workspace, workspace_bytes, stream);
+}
+
+int m2d_proj_bwd_parts(const m2d_desc* desc, int dt_rank, int sum_parts, const void* x, const void* lowrank, const void* deltaT,
+                       const void* deltaL, const float* x_proj_w, const float* dt_projT_w, const float* dt_projL_w,
+                       const void* d_deltaT, const void* d_deltaL, const void* d_BT, const void* d_BL, const void* d_C,
+                       void* dx, float* d_x_proj_w, float* d_dt_projT_w, float* d_dt_projT_b, float* d_dt_projL_w,
+                       float* d_dt_projL_b, void* workspace, size_t workspace_bytes, void* stream) {
   int rc = check_proj(desc, dt_rank);
   if (rc) return rc;
+  if (sum_parts < 0) return M2D_ERR_BAD_SHAPE;
+  if (sum_parts > 0 && !proj_geometry(desc, dt_rank).mfma) return M2D_ERR_UNSUPPORTED;
   const bool given = (desc->flags & M2D_FLAG_DPRE) != 0;   // d_deltaT, d_deltaL are dpre: deltaT, deltaL are not read
-  const void* req[] = {x, lowrank, x_proj_w, dt_projT_w, dt_projL_w, d_deltaT, d_deltaL, d_BT, d_BL, d_C,
+  const void* req[] = {x, lowrank, x_proj_w, dt_projT_w, dt_projL_w, d_deltaT, d_deltaL, d_BT, sum_parts ? d_BT : d_BL, sum_parts ? d_BT : d_C,
                        dx, d_x_proj_w, d_dt_projT_w, d_dt_projT_b, d_dt_projL_w, d_dt_projL_b, workspace};
   for (const void* q : req) if (!q) return M2D_ERR_NULL_POINTER;
   if (!given && (!deltaT || !deltaL)) return M2D_ERR_NULL_POINTER;
@@ -1328,7 +1357,7 @@ int m2d_proj_bwd(const m2d_desc* desc, int dt_rank, const void* x, const void* l
   if (!launched()) return M2D_ERR_HIP;
   ProjArgs a = {};
   fill(a, g);
-  a.x = x; a.r = lowrank; a.dT = deltaT; a.dL = deltaL; a.dpre_given = given ? 1 : 0;
+  a.x = x; a.r = lowrank; a.dT = deltaT; a.dL = deltaL; a.dpre_given = given ? 1 : 0; a.sum_parts = sum_parts;
   a.ddT = d_deltaT; a.ddL = d_deltaL; a.dBT = d_BT; a.dBL = d_BL; a.dC = d_C; a.dx = dx;
   a.Wp = k.Wp; a.wTp = k.wTp; a.wLp = k.wLp;
   a.wTtb = k.wTtb; a.wLtb = k.wLtb; a.WxTb = k.WxTb;

@@ -2954,9 +2954,9 @@ __global__ void m2d_pack_bc_kernel(const T* BT, const T* BL, const T* C, float* 
 // RAW: d_AT, d_AL, d_D are fp32 and refer to the parameters as the module holds them:
 // A = -exp(A_log), so d_A_log = d_A * A (A is at hand as A2 / log2 e).
 template <typename T, bool RAW>
-__global__ void m2d_finalize_kernel(const ScanParams p, T* dC, T* dBT, T* dBL, void* dATv, void* dALv, void* dDv) {
+__global__ void m2d_finalize_kernel(const ScanParams p, T* dC, T* dBT, T* dBL, void* dATv, void* dALv, void* dDv, int parts_stay) {
   const int64_t P = p.Ptot;
-  const int64_t nquad = 3 * P * (kN / 4);
+  const int64_t nquad = parts_stay ? 0 : 3 * P * (kN / 4);   // (parts_stay: the reader of d_C, d_BT, d_BL adds up the per-workgroup sums itself)
   const int64_t gid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (gid < nquad) {
     // per-workgroup sums are laid out [channel group][cell][C, B_T, B_L][16]: consecutive threads
@@ -3111,7 +3111,7 @@ int check_desc(const m2d_desc* d) {
   if (d->B < 1 || d->E < 1 || d->N < 1 || d->H < 2 || d->W < 2) return M2D_ERR_BAD_SHAPE;
   if (d->N != kN) return M2D_ERR_UNSUPPORTED;
   if (d->dtype != M2D_F32 && d->dtype != M2D_BF16) return M2D_ERR_UNSUPPORTED;
-  if ((d->ckpt_interval != 0 && d->ckpt_interval != 2 && d->ckpt_interval != 4 && d->ckpt_interval != 8 && d->ckpt_interval != 16) || (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_RAW_PARAMS | M2D_FLAG_PACKED_BC | M2D_FLAG_DPRE | M2D_FLAG_SPLIT_STATES | M2D_FLAG_WHOLE_STATES | M2D_FLAG_TEST_DEAD_LINK))) return M2D_ERR_UNSUPPORTED;
+  if ((d->ckpt_interval != 0 && d->ckpt_interval != 2 && d->ckpt_interval != 4 && d->ckpt_interval != 8 && d->ckpt_interval != 16) || (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_RAW_PARAMS | M2D_FLAG_PACKED_BC | M2D_FLAG_DPRE | M2D_FLAG_SPLIT_STATES | M2D_FLAG_WHOLE_STATES | M2D_FLAG_TEST_DEAD_LINK | M2D_FLAG_SUM_PARTS))) return M2D_ERR_UNSUPPORTED;
   if ((d->flags & M2D_FLAG_SPLIT_STATES) && (d->flags & M2D_FLAG_WHOLE_STATES)) return M2D_ERR_UNSUPPORTED;
   if ((int64_t)d->B * d->H * d->W >= ((int64_t)1 << 40)) return M2D_ERR_BAD_SHAPE;
   // one image is addressed with 32-bit byte offsets from its base (fp32: 4 bytes per element;
@@ -3576,6 +3576,7 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   float* prep = reinterpret_cast<float*>(w); w += g.prep_bytes;
   uint32_t* link_words = reinterpret_cast<uint32_t*>(w); w += g.link_bytes;
   sp.part = reinterpret_cast<float*>(w); w += g.part_bytes;
+  if (d->flags & M2D_FLAG_SUM_PARTS) sp.part = static_cast<float*>(dBT);   // the per-workgroup channel sums go to the caller, as they are
   sp.pA = reinterpret_cast<float*>(w); w += g.pa_bytes;
   sp.pD = reinterpret_cast<float*>(w); w += g.pd_bytes;
   sp.bot = reinterpret_cast<float*>(w); w += g.bot_bytes;
@@ -3617,14 +3618,15 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][1], st);
   if (rc) return rc;
   const int64_t P = (int64_t)d->B * d->H * d->W;
-  const int64_t quad_blocks = (3 * P * (kN / 4) + 255) / 256;
+  const int parts_stay = (d->flags & M2D_FLAG_SUM_PARTS) ? 1 : 0;
+  const int64_t quad_blocks = parts_stay ? 0 : (3 * P * (kN / 4) + 255) / 256;
   const int64_t tail_blocks = (((int64_t)d->E * 2 * kN + d->E) * 16 + 255) / 256;   // 16 lanes per position sum
   if (d->flags & M2D_FLAG_RAW_PARAMS)
     hipLaunchKernelGGL((m2d_finalize_kernel<T, true>), dim3((unsigned)(quad_blocks + tail_blocks)), dim3(256), 0, st, sp,
-                       static_cast<T*>(dC), static_cast<T*>(dBT), static_cast<T*>(dBL), dAT, dAL, dD);
+                       static_cast<T*>(dC), static_cast<T*>(dBT), static_cast<T*>(dBL), dAT, dAL, dD, parts_stay);
   else
     hipLaunchKernelGGL((m2d_finalize_kernel<T, false>), dim3((unsigned)(quad_blocks + tail_blocks)), dim3(256), 0, st, sp,
-                       static_cast<T*>(dC), static_cast<T*>(dBT), static_cast<T*>(dBL), dAT, dAL, dD);
+                       static_cast<T*>(dC), static_cast<T*>(dBT), static_cast<T*>(dBL), dAT, dAL, dD, parts_stay);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
@@ -3708,8 +3710,9 @@ int m2d_scan_bwd(const m2d_desc* desc, const void* x, const void* deltaT, const 
   int rc = check_desc(desc);
   if (rc) return rc;
   const bool packed = (desc->flags & M2D_FLAG_PACKED_BC) != 0;   // B_T carries the records, B_L and C are not read
+  const bool parts = (desc->flags & M2D_FLAG_SUM_PARTS) != 0;   // d_BT receives the per-workgroup sums, d_BL and d_C are not written
   const void* req[] = {x, deltaT, deltaL, AT, AL, BT, packed ? BT : BL, packed ? BT : C, D, dy, dx, d_deltaT, d_deltaL,
-                       d_AT, d_AL, d_BT, d_BL, d_C, d_D, workspace};
+                       d_AT, d_AL, d_BT, parts ? d_BT : d_BL, parts ? d_BT : d_C, d_D, workspace};
   for (const void* q : req) if (!q) return M2D_ERR_NULL_POINTER;
   for (const void* q : req) if (misaligned(q, 16)) return M2D_ERR_MISALIGNED;
   if (misaligned(workspace, 256) || (ckpt && misaligned(ckpt, 256))) return M2D_ERR_MISALIGNED;
@@ -3724,6 +3727,11 @@ int m2d_scan_bwd(const m2d_desc* desc, const void* x, const void* deltaT, const 
   return desc->dtype == M2D_F32
              ? run_bwd<float>(desc, g, sp, AT, AL, BT, BL, C, D, ckpt, d_AT, d_AL, d_BT, d_BL, d_C, d_D, workspace, st)
              : run_bwd<bf16_t>(desc, g, sp, AT, AL, BT, BL, C, D, ckpt, d_AT, d_AL, d_BT, d_BL, d_C, d_D, workspace, st);
+}
+
+int m2d_scan_sum_parts(const m2d_desc* desc) {
+  if (check_desc(desc) != M2D_OK) return 0;
+  return make_geometry(desc).bwd_bpb;
 }
 
 int m2d_scan_plan(const m2d_desc* desc, int pass, char* text, size_t cap) {

@@ -98,8 +98,15 @@ def _scan_fwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, save_ckpt, flip, raw
 
 @torch.library.register_fake("m2dscan::scan_bwd")
 def _scan_bwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt, flip, raw_params=False, packed_bc=False, dpre=False,
-                   ckpt_interval=0):
+                   ckpt_interval=0, sum_parts=False):
     bc = [x.new_empty((*x.shape[:3], AT.shape[1])) for _ in range(3)]
+    if sum_parts:   # the per-workgroup sums of d_C, d_BT, d_BL in fp32, as many as the library's plan has channel groups
+        d = cabi.Desc(*x.shape, AT.shape[1], cabi.M2D_BF16 if x.dtype == torch.bfloat16 else cabi.M2D_F32,
+                      (cabi.M2D_FLAG_FLIP if flip else 0) | (cabi.M2D_FLAG_RAW_PARAMS if raw_params else 0)
+                      | (cabi.M2D_FLAG_PACKED_BC if packed_bc else 0) | (cabi.M2D_FLAG_DPRE if dpre else 0) | cabi.M2D_FLAG_SUM_PARTS,
+                      ckpt_interval)
+        parts = int(cabi.lib.m2d_scan_sum_parts(ctypes.byref(d)))
+        bc = [x.new_empty((parts, *x.shape[:3], 3 * AT.shape[1]), dtype=torch.float32), x.new_empty((0,)), x.new_empty((0,))]
     return [torch.empty_like(x), torch.empty_like(deltaT), torch.empty_like(deltaL), torch.empty_like(AT), torch.empty_like(AL),
             *bc, torch.empty_like(D)]
 
@@ -127,7 +134,7 @@ def _proj_fwd_fake(x, x_proj_w, dt_projT_w, dt_projT_b, dt_projL_w, dt_projL_b, 
 
 @torch.library.register_fake("m2dscan::proj_bwd")
 def _proj_bwd_fake(x, lowrank, deltaT, deltaL, x_proj_w, dt_projT_w, dt_projL_w, d_deltaT, d_deltaL, d_BT, d_BL, d_C, dx,
-                   round_weights, dpre=False):
+                   round_weights, dpre=False, sum_parts=0):
     b = dt_projT_w.new_empty((x.shape[-1],))
     return torch.empty_like(x_proj_w), torch.empty_like(dt_projT_w), b, torch.empty_like(dt_projL_w), torch.empty_like(b)
 
@@ -430,10 +437,14 @@ class wf_cuda_fn_proj(torch.autograd.Function):
             low, dT, dL, BT, BL, C, ck = ctx.saved_tensors[9:]
         # with raw parameters the gradients of A_log and D come back in fp32; the gradients of the two
         # step sizes come back as gradients before the softplus, which is what the projections' backward wants
+        # the sums over channels d_BT, d_BL, d_C have one reader here, the projections' backward: where its products run on the
+        # matrix cores it takes the scan's per-workgroup sums as they are and adds them up while it loads them
+        parts = x.dtype == torch.bfloat16 and x.shape[-1] % 8 == 0
         d_x, d_dT, d_dL, d_At, d_Al, d_BT, d_BL, d_C, d_D = scan_bwd_op(x, dT, dL, At, Al, BT, BL, C, D32, dy, ck, ctx.flip,
-                                                                        True, True, True, ctx.interval)
+                                                                        True, True, True, ctx.interval, parts)
         # d_x holds the scan's own gradient (dy*D included); the projections add theirs in place
-        g = proj_bwd_op(x, low, dT, dL, w32[0], w32[1], w32[3], d_dT, d_dL, d_BT, d_BL, d_C, d_x, True, True)
+        g = proj_bwd_op(x, low, dT, dL, w32[0], w32[1], w32[3], d_dT, d_dL, d_BT, d_BL, d_C, d_x, True, True,
+                        d_BT.shape[0] if parts else 0)
         grads = (d_At, d_Al, *g, d_D)
         return (d_x, *[t.to(r.dtype) for t, r in zip(grads, raw)], None, None, None)
 
