@@ -93,6 +93,25 @@ def spilling_kernels(text: str):
     return out
 
 
+_LABEL = re.compile(r"^(_Z\w+):")
+_SCRATCH_OP = re.compile(r"^\s+scratch_(load|store)")
+
+
+def scratch_accesses(text: str):
+    """Number of scratch loads and stores in the body of every kernel: {kernel: count}.  A kernel whose descriptor asks
+    for scratch memory and which has none of them only parks scalar registers in lanes of a vector register; the
+    compiler reserves a few bytes for that register and never touches them."""
+    out, kernel = {}, None
+    for line in text.splitlines():
+        m = _LABEL.match(line)
+        if m:
+            kernel = m.group(1)
+            out.setdefault(kernel, 0)
+        elif kernel and _SCRATCH_OP.match(line):
+            out[kernel] += 1
+    return out
+
+
 def spills_in_file(path: str):
     with open(path) as f:
         return spilling_kernels(f.read())

@@ -46,6 +46,12 @@ SOURCES = {
 # It reloads two to nine values a few times per block of steps; every other kernel must not spill at all.
 SPILL_ALLOWANCE = [(re.compile(r"m2d_bwd_kernelI\w*Li8ELb1EEEv"), 64)]
 
+# A kernel that runs out of scalar registers parks some in lanes of a vector register; the compiler then reserves a
+# few bytes of scratch for that register without ever storing it.  Allowed up to this many bytes per lane, and only
+# where the kernel has no scratch load or store at all.
+UNTOUCHED_SCRATCH = 64
+
+
 def build_lib(verbose: bool = True) -> str:
     """Compiles the HIP sources into libm2dscan.so.  The device assembly of the same compile is
     kept (-save-temps) and checked for the hazards that inline assembly hides from the compiler
@@ -77,8 +83,11 @@ def build_lib(verbose: bool = True) -> str:
             if bad:
                 raise RuntimeError("hazard between inline-assembly DPP instructions and their producers:\n" +
                                    "\n".join(f"  {k}: {p}  ->  {c}" for k, p, c in bad[:8]))
+            with open(path) as f:
+                accesses = asmcheck.scratch_accesses(f.read())
             spills = [(k, n) for k, n in asmcheck.spills_in_file(path)
-                      if not any(pat.search(k) and n <= cap for pat, cap in SPILL_ALLOWANCE)]
+                      if not any(pat.search(k) and n <= cap for pat, cap in SPILL_ALLOWANCE)
+                      and not (n <= UNTOUCHED_SCRATCH and accesses.get(k, 1) == 0)]
             if spills:
                 raise RuntimeError("kernels that spill registers to scratch memory:\n" +
                                    "\n".join(f"  {k}: {n} bytes per lane" for k, n in spills[:8]))

@@ -65,6 +65,10 @@ constexpr int kZeroFloats = 64;     // page of zeros at the head of the set-up a
 constexpr int kModeSweep = 0, kModeSliced = 1, kModeStacked = 2;   // how the bands of the batch are scheduled
 constexpr int kLinkLag = 7;        // linked sweep: blocks by which a band trails the band it depends on (see link_need_*)
 constexpr int kSpinLimit = 1 << 21;   // linked sweep: polls of a neighbour's progress before a workgroup gives up waiting
+// Words from one progress count of the linked sweep to the next: a count has 256 bytes to itself.  Side by side in one
+// cache line, the counts of a band's workgroups were written by 16 workgroups while 64 waves polled the line, and
+// every hand-off waited for that line (256x256, E=64: forward 0.46 -> 0.34 ms with the counts apart).
+constexpr int kLinkStride = 64;
 constexpr uint32_t kLinkAbort = 0xffffffffu;   // progress value of a band that gave up: nobody waits for it
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
@@ -360,13 +364,15 @@ __device__ __forceinline__ void store_row_device_scope(float4* dst, float4 v) {
   const v4f_t w = {v.x, v.y, v.z, v.w};
   asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(dst), "v"(w) : "memory");
 }
-struct Link {
+template <int PUB>   // the thread that publishes: one of a wave that waits, so that it knows of a wait given up
+struct LinkT {
   uint32_t* mine = nullptr;         // this workgroup's progress count
   const uint32_t* dep = nullptr;    // the count of the workgroup whose boundary rows this one reads (none: first band of the sweep)
   uint32_t seen = 0;                // last value read from dep
   bool gave_up = false;
   uint32_t* err = nullptr;
   int limit = kSpinLimit;           // polls before a wait gives up
+  static constexpr int pub = PUB;
   // test aid: the workgroups of band `link_test - 1` wait for a count that nobody publishes (a word of the header,
   // zero for the whole launch), and every wait of the launch gives up after a few polls: the give-up path runs, and
   // every workgroup still ends
@@ -388,13 +394,14 @@ struct Link {
     }
     seen = kLinkAbort;
     gave_up = true;
-    if (threadIdx.x == 0) link_publish(err, 1u);
+    if ((int)threadIdx.x == pub) link_publish(err, 1u);
   }
   // after a barrier behind which `done` blocks of this band have their boundary rows in memory
   __device__ __forceinline__ void publish(uint32_t done) {
-    if (threadIdx.x == 0) link_publish(mine, (gave_up || seen == kLinkAbort) ? kLinkAbort : done);
+    if ((int)threadIdx.x == pub) link_publish(mine, (gave_up || seen == kLinkAbort) ? kLinkAbort : done);
   }
 };
+using Link = LinkT<0>;
 // Blocks of the neighbour's window that must be done before block j of a band's own window is staged.
 // Forward: the ghost of block j replays the columns 4j .. 4j+3 of the last row of the band above,
 // which lane 14 stored at the window's steps 4j+14 .. 4j+17, the last of them in block j+4.
@@ -874,8 +881,8 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     lb -= my_band * per;
     m_lo = my_band * p.sl_nbb;
     m_hi = m_lo + p.sl_nbb;
-    link.mine = p.prog + (int64_t)my_band * per + lb;
-    link.dep = my_band > 0 ? link.mine - per : nullptr;
+    link.mine = p.prog + ((int64_t)my_band * per + lb) * kLinkStride;
+    link.dep = my_band > 0 ? link.mine - per * kLinkStride : nullptr;
     link.err = p.link_err;
     link.rig(p, my_band);
   }
@@ -1281,12 +1288,26 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
 // m2d_fwd_kernel; y of a cell is the sum over the 4 lane groups (two lane-swap steps), stored by group 0.
 constexpr int kSplitWaves = 8;
 constexpr int kSplitHalfWaves = 4;   // where workgroups of 8 would leave compute units idle
+// Linked sweep in workgroups of 4 waves: a step of a wave that has a SIMD to itself takes as long as its chain of
+// instructions, and of those under a third are the step's arithmetic; the rest stages the next block (positions,
+// addresses, copies, the wait for the neighbouring band).  So such a workgroup gets 4 more waves that do nothing but
+// stage (and, in the backward, add up the channel sums of every step), one to a SIMD beside a wave that does nothing
+// but sweep: the two chains run side by side.
+constexpr int kAll = 0, kSweeper = 1, kStager = 2;   // what a wave of such a workgroup does
+#ifndef M2D_SPLIT_HELPERS
+#define M2D_SPLIT_HELPERS 4
+#endif
+#ifndef M2D_SPLIT_HELPERS8
+#define M2D_SPLIT_HELPERS8 0
+#endif
+template <int MODE, int NWS>
+constexpr int split_helpers() { return MODE != kModeSliced ? 0 : (NWS == kSplitHalfWaves ? M2D_SPLIT_HELPERS : M2D_SPLIT_HELPERS8); }
 __device__ __forceinline__ float sum_over_groups(float v) {
   v = fold16(v, v);
   return fold32(v, v);
 }
 template <typename T, bool CKPT, bool WRITE_Y, bool STAGE_X, int MODE, int NWS = kSplitWaves>
-__global__ __launch_bounds__(NWS * 64) void m2d_fwd_split_kernel(const ScanParams pin) {
+__global__ __launch_bounds__((NWS + split_helpers<MODE, NWS>()) * 64) void m2d_fwd_split_kernel(const ScanParams pin) {
   static_assert(MODE != kModeStacked, "stacked images are many: they never need the split");
   constexpr bool SLICED = MODE == kModeSliced;
   const ScanParams& p = pin;
@@ -1294,6 +1315,8 @@ __global__ __launch_bounds__(NWS * 64) void m2d_fwd_split_kernel(const ScanParam
   __builtin_assume(p.rb == kRB);
   __builtin_assume(p.S >= kHB + kCK - 1);
   constexpr int NW = NWS, CW = NW;
+  constexpr int NH = split_helpers<MODE, NWS>();   // waves that only stage (then the first NW waves only sweep)
+  constexpr int NSTG = NH ? NH : NW;               // waves that share the copies of a block
   using SG = Stage<T, 3, CW, false>;
   constexpr bool WIDEN = sizeof(T) == 2;
   extern __shared__ float4 smem[];
@@ -1304,26 +1327,29 @@ __global__ __launch_bounds__(NWS * 64) void m2d_fwd_split_kernel(const ScanParam
   int lb = SLICED ? (int)blockIdx.x : logical_block(p.nwg);
   int m_lo = 0, m_hi = p.nblk;
   int my_band = 0;
-  Link link;
+  LinkT<NH ? NW * 64 : 0> link;
   if constexpr (SLICED) {
     const int per = p.B * p.bpb;
     my_band = lb / per;
     lb -= my_band * per;
     m_lo = my_band * p.sl_nbb;
     m_hi = m_lo + p.sl_nbb;
-    link.mine = p.prog + (int64_t)my_band * per + lb;
-    link.dep = my_band > 0 ? link.mine - per : nullptr;
+    link.mine = p.prog + ((int64_t)my_band * per + lb) * kLinkStride;
+    link.dep = my_band > 0 ? link.mine - per * kLinkStride : nullptr;
     link.err = p.link_err;
     link.rig(p, my_band);
   }
+  const bool helper = NH && wave >= NW;             // (uniform) stages, never sweeps
+  const bool stages = !NH || helper;
+  const int swave = NH ? wave - NW : wave;          // the wave's turn among those that stage
   const int b = lb / p.bpb;
   const int e_wg0 = (lb % p.bpb) * CW;
   const int g = lane >> kHBShift, r = lane & (kHB - 1);   // state group, lane row
   const int rbands = row_bands(p, r);
-  const int ch_loc = wave;                          // the wave's channel inside the workgroup
-  const bool ch_ok = e_wg0 + ch_loc < p.E;          // (uniform) idle waves still take part in staging and barriers
+  const int ch_loc = helper ? 0 : wave;             // the wave's channel inside the workgroup
+  const bool ch_ok = !helper && e_wg0 + ch_loc < p.E;   // (uniform) idle waves still take part in staging and barriers
   const int e0 = ch_ok ? e_wg0 + ch_loc : p.E - 1;
-  for (int i = threadIdx.x; i < 2 * SG::kBytes / 16; i += NW * 64) smem[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int i = threadIdx.x; i < 2 * SG::kBytes / 16; i += (NW + NH) * 64) smem[i] = make_float4(0.f, 0.f, 0.f, 0.f);
 
   // Position 4g + w of a record is met by register w: state sinv(4g + w) in fold order, state 4g + w
   // where the records come straight from fp32 tensors (natural order).
@@ -1427,29 +1453,35 @@ __global__ __launch_bounds__(NWS * 64) void m2d_fwd_split_kernel(const ScanParam
   Pos A = pos_of(p, m_lo * kCK - (kHB - 1));     // position of the stream index t0 - 15 (wave-uniform)
   bp = block_pos(p, A, r, rbands);
   int cell0 = cell_of(p, bp.bnd0, r, bp.col0);
-  if constexpr (SLICED) link.wait_for(link_need_fwd(0, p.sl_nbb));
+  if constexpr (SLICED) { if (stages) link.wait_for(link_need_fwd(0, p.sl_nbb)); }
   BlockPos bpq = bp;     // 16-bit direct records: the block after the next (fetched two blocks ahead)
   int cellq = cell0;
   int rp = 0;
   if (direct) {
     if constexpr (WIDEN) {
-      bc_raw_copy<NW>(p, pin.bcd, raw, b, bp, cell0, wave, lane, true);
+      if (stages) bc_raw_copy<NSTG>(p, pin.bcd, raw, b, bp, cell0, swave, lane, true);
       bpq = block_pos(p, pos_after(p, A, kCK), r, rbands);
       cellq = cell_of(p, bpq.bnd0, r, bpq.col0);
-      bc_raw_copy<NW>(p, pin.bcd, raw + kRawBytes, b, bpq, cellq, wave, lane, m_lo + 1 < m_hi);
+      if (stages) bc_raw_copy<NSTG>(p, pin.bcd, raw + kRawBytes, b, bpq, cellq, swave, lane, m_lo + 1 < m_hi);
     } else {
-      bc_direct_copy<T, CW, NW>(p, pin.bcd, lds, b, bp, cell0, wave, lane);
+      if (stages) bc_direct_copy<T, CW, NSTG>(p, pin.bcd, lds, b, bp, cell0, swave, lane);
     }
-    stage_block<T, 3, CW, false, STAGE_X, NW, true>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+    if (stages) stage_block<T, 3, CW, false, STAGE_X, NSTG, true>(p, lds, b, A, bp, cell0, e_wg0, swave, lane, X, DT, DL, DY);
     if constexpr (WIDEN) {
       staging_fence();
-      bc_widen<SG, NW>(raw, lds, wave, lane);
+      if (stages) bc_widen<SG, NSTG>(raw, lds, swave, lane);
     }
   } else {
-    stage_block<T, 3, CW, false, STAGE_X, NW>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+    if (stages) stage_block<T, 3, CW, false, STAGE_X, NSTG>(p, lds, b, A, bp, cell0, e_wg0, swave, lane, X, DT, DL, DY);
   }
   staging_fence();
   int cur = 0;
+  // The sweep over the blocks of the window, as a wave of the given role runs it: kAll stages and sweeps; with waves
+  // that only stage, those run it as kStager and the others as kSweeper, each with its own part of the work and all
+  // with the same barriers.
+  auto sweep = [&](auto role) {
+  constexpr int ROLE = decltype(role)::value;
+  constexpr bool STAGES = ROLE != kSweeper, SWEEPS = ROLE != kStager;
   for (int m = m_lo; m < m_hi; ++m) {
     const bool last = m + 1 == m_hi;
     const Pos An = pos_after(p, A, kCK);
@@ -1460,22 +1492,23 @@ __global__ __launch_bounds__(NWS * 64) void m2d_fwd_split_kernel(const ScanParam
       celln = cellq;
       bpq = block_pos(p, pos_after(p, An, kCK), r, rbands);
       cellq = cell_of(p, bpq.bnd0, r, bpq.col0);
-      bc_raw_copy<NW>(p, pin.bcd, raw + rp * kRawBytes, b, bpq, cellq, wave, lane, m + 2 < m_hi);
+      if constexpr (STAGES) bc_raw_copy<NSTG>(p, pin.bcd, raw + rp * kRawBytes, b, bpq, cellq, swave, lane, m + 2 < m_hi);
     } else {
       bpn = block_pos(p, An, r, rbands);
       celln = cell_of(p, bpn.bnd0, r, bpn.col0);
     }
-    if (!last) {
+    if (STAGES && !last) {
       if constexpr (SLICED) link.wait_for(link_need_fwd(m + 1 - m_lo, p.sl_nbb));
       if (direct) {
-        if constexpr (!WIDEN) bc_direct_copy<T, CW, NW>(p, pin.bcd, lds + (cur ^ 1) * SG::kBytes, b, bpn, celln, wave, lane);
-        stage_block<T, 3, CW, false, STAGE_X, NW, true>(p, lds + (cur ^ 1) * SG::kBytes, b, An, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
-        if constexpr (WIDEN) bc_widen<SG, NW>(raw + (rp ^ 1) * kRawBytes, lds + (cur ^ 1) * SG::kBytes, wave, lane);
+        if constexpr (!WIDEN) bc_direct_copy<T, CW, NSTG>(p, pin.bcd, lds + (cur ^ 1) * SG::kBytes, b, bpn, celln, swave, lane);
+        stage_block<T, 3, CW, false, STAGE_X, NSTG, true>(p, lds + (cur ^ 1) * SG::kBytes, b, An, bpn, celln, e_wg0, swave, lane, X, DT, DL, DY);
+        if constexpr (WIDEN) bc_widen<SG, NSTG>(raw + (rp ^ 1) * kRawBytes, lds + (cur ^ 1) * SG::kBytes, swave, lane);
       } else {
-        stage_block<T, 3, CW, false, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, An, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+        stage_block<T, 3, CW, false, STAGE_X, NSTG>(p, lds + (cur ^ 1) * SG::kBytes, b, An, bpn, celln, e_wg0, swave, lane, X, DT, DL, DY);
       }
     }
     rp ^= 1;
+    if constexpr (SWEEPS) {
     cell_off0 = (uint32_t)(cell0 * p.E + e0) * (uint32_t)sizeof(T);
     if constexpr (CKPT) {   // every lane stores, without a branch inside the step: see m2d_fwd_kernel
       const bool keep = m > 0 && snapshot_kept(p, m, m_lo);
@@ -1499,18 +1532,31 @@ __global__ __launch_bounds__(NWS * 64) void m2d_fwd_split_kernel(const ScanParam
       if (k == 0 || k == kCK / 2) lead_if_younger<NW>(wave, k == 0);
       step(bufc, k);
     }
+    } else {
+      staging_landed();   // the next block's operands are in place
+    }
     __syncthreads();
-    if constexpr (SLICED) link.publish((uint32_t)(m - m_lo + 1));
+    if constexpr (SLICED && STAGES) link.publish((uint32_t)(m - m_lo + 1));
     cur ^= 1;
     A = An;
     bp = bpn;
     cell0 = celln;
   }
+  };
+  if constexpr (NH == 0) sweep(std::integral_constant<int, kAll>{});
+  else if (helper) sweep(std::integral_constant<int, kStager>{});
+  else sweep(std::integral_constant<int, kSweeper>{});
   if constexpr (SLICED) {
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
     link.publish((uint32_t)p.sl_nbb);
-    if (WRITE_Y && link.broken()) poison_band<T>(p, my_band, b, e_wg0, CW, p.y, nullptr, nullptr);
+    bool broken = link.broken();
+    if constexpr (NH > 0) {   // only the waves that wait know: they tell the others (the staging buffers are free now)
+      if ((int)threadIdx.x == link.pub) *reinterpret_cast<volatile uint32_t*>(lds) = broken ? 1u : 0u;
+      __syncthreads();
+      broken = *reinterpret_cast<volatile uint32_t*>(lds) != 0u;
+    }
+    if (WRITE_Y && broken) poison_band<T>(p, my_band, b, e_wg0, CW, p.y, nullptr, nullptr);
   }
 }
 
@@ -1587,8 +1633,8 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
     my_band = p.nbands - 1 - kk;
     m_lo = my_band * p.sl_nbb;
     m_hi = m_lo + p.sl_nbb;
-    link.mine = p.prog + (int64_t)my_band * per + lb;
-    link.dep = my_band + 1 < p.nbands ? link.mine + per : nullptr;
+    link.mine = p.prog + ((int64_t)my_band * per + lb) * kLinkStride;
+    link.dep = my_band + 1 < p.nbands ? link.mine + per * kLinkStride : nullptr;
     link.err = p.link_err;
     link.rig(p, my_band);
   }
@@ -2559,7 +2605,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd2_kernel(const ScanParams pin)
 // over channels (d_C, d_BT, d_BL) across the 8 waves through LDS, as in m2d_bwd_kernel, a float4 of
 // four states per lane.  Memory formats are those of m2d_bwd_kernel.
 template <typename T, bool STAGE_X, int MODE, int NWS = kSplitWaves>
-__global__ __launch_bounds__(NWS * 64) void m2d_bwd_split_kernel(const ScanParams pin) {
+__global__ __launch_bounds__((NWS + split_helpers<MODE, NWS>()) * 64) void m2d_bwd_split_kernel(const ScanParams pin) {
   static_assert(MODE != kModeStacked, "stacked images are many: they never need the split");
   constexpr bool SLICED = MODE == kModeSliced;
   const ScanParams& p = pin;
@@ -2567,6 +2613,9 @@ __global__ __launch_bounds__(NWS * 64) void m2d_bwd_split_kernel(const ScanParam
   __builtin_assume(p.rb == kRB);
   __builtin_assume(p.S >= kHB + kCK - 1);
   constexpr int NW = NWS, CW = NW;
+  constexpr int NH = split_helpers<MODE, NWS>();   // waves that only stage and add up the channel sums (then the first NW waves only sweep)
+  constexpr int NSTG = NH ? NH : NW;               // waves that share the copies of a block
+  static_assert(NH == 0 || NH >= 3, "three waves add up the channel sums");
   constexpr int SLOT = 3 * 64;           // float4s per wave in one exchange buffer
   using SG = Stage<T, 4, CW, true>;
   constexpr bool WIDEN = sizeof(T) == 2;
@@ -2580,7 +2629,7 @@ __global__ __launch_bounds__(NWS * 64) void m2d_bwd_split_kernel(const ScanParam
   int lb = SLICED ? (int)blockIdx.x : logical_block(p.nwg);
   int m_lo = 0, m_hi = p.nblk;
   int my_band = 0;
-  Link link;
+  LinkT<NH ? NW * 64 : 0> link;
   if constexpr (SLICED) {   // the window of one band; the bands are launched from the last to the first
     const int per = p.B * p.bpb;
     const int kk = lb / per;
@@ -2588,20 +2637,23 @@ __global__ __launch_bounds__(NWS * 64) void m2d_bwd_split_kernel(const ScanParam
     my_band = p.nbands - 1 - kk;
     m_lo = my_band * p.sl_nbb;
     m_hi = m_lo + p.sl_nbb;
-    link.mine = p.prog + (int64_t)my_band * per + lb;
-    link.dep = my_band + 1 < p.nbands ? link.mine + per : nullptr;
+    link.mine = p.prog + ((int64_t)my_band * per + lb) * kLinkStride;
+    link.dep = my_band + 1 < p.nbands ? link.mine + per * kLinkStride : nullptr;
     link.err = p.link_err;
     link.rig(p, my_band);
   }
+  const bool helper = NH && wave >= NW;      // (uniform) stages and adds up, never sweeps
+  const bool stages = !NH || helper;
+  const int swave = NH ? wave - NW : wave;   // the wave's turn among those that stage
   const int b = lb / p.bpb;
   const int eg = lb % p.bpb;
   const int e_wg0 = eg * CW;
   const int g = lane >> kHBShift, r = lane & (kHB - 1);
   const int rbands = row_bands(p, r);
-  const int ch_loc = wave;
-  const bool ch_ok = e_wg0 + ch_loc < p.E;   // (uniform)
+  const int ch_loc = helper ? 0 : wave;
+  const bool ch_ok = !helper && e_wg0 + ch_loc < p.E;   // (uniform)
   const int e = ch_ok ? e_wg0 + ch_loc : p.E - 1;
-  for (int i = threadIdx.x; i < 2 * SG::kBytes / 16; i += NW * 64) reinterpret_cast<float4*>(lds)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int i = threadIdx.x; i < 2 * SG::kBytes / 16; i += (NW + NH) * 64) reinterpret_cast<float4*>(lds)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
   // register w of the lane meets position 4g + w of a record: state perm(w) * 4 + g (fold order)
   int state_of[4];
   float a2t[4], a2l[4];
@@ -2641,9 +2693,10 @@ __global__ __launch_bounds__(NWS * 64) void m2d_bwd_split_kernel(const ScanParam
   // channel sums: the first 6 waves add up; wave 2v + c takes components 2c, 2c+1 of every lane's float4 of
   // tensor v.  They are kept per cell as [C, B_T, B_L][16] in the natural order of the states.
   // (workgroups of 4 waves: the first 3 add up, a whole float4 each)
-  constexpr bool QUADS = NW < 6;
-  const bool f_on = wave < (QUADS ? 3 : 6);
-  const int f_v = QUADS ? wave : wave >> 1, f_c = QUADS ? 0 : wave & 1;
+  // (with waves that only stage: the first 3 of those, a whole float4 each)
+  constexpr bool QUADS = NH > 0 || NW < 6;
+  const bool f_on = NH ? (helper && swave < 3) : wave < (QUADS ? 3 : 6);
+  const int f_v = QUADS ? swave : wave >> 1, f_c = QUADS ? 0 : wave & 1;
   const uint32_t f_sub0 = (uint32_t)(f_v * kN + (f_c ? 1 : 0) * 4 + g) * (uint32_t)sizeof(float);   // component 2c: state perm(2c) * 4 + g, perm = (0, 2, 1, 3)
   const uint32_t f_sub1 = (uint32_t)(f_v * kN + (f_c ? 3 : 2) * 4 + g) * (uint32_t)sizeof(float);   // component 2c + 1
   const float g1 = r == 0 ? 1.f : 0.f;
@@ -2676,49 +2729,56 @@ __global__ __launch_bounds__(NWS * 64) void m2d_bwd_split_kernel(const ScanParam
   int cell0 = cell_of(p, bp.bnd0, r, bp.col0);
   bool ck_take = snapshot_lane(p, Pos{bp.bnd0, bp.col0}, r, ch_ok);
   load_ckpt(m_hi - 1, ck_take);
-  if constexpr (SLICED) link.wait_for(link_need_bwd(p.sl_nbb - 1, p.sl_nbb));
+  if constexpr (SLICED) { if (stages) link.wait_for(link_need_bwd(p.sl_nbb - 1, p.sl_nbb)); }
   auto raw_copy_for = [&](Pos A2, char* dst, bool live) {
+    if (!stages) return;   // (uniform)
     const BlockPos q2 = block_pos(p, A2, r, rbands);
-    bc_raw_copy<NW>(p, pin.bcd, dst, b, q2, cell_of(p, q2.bnd0, r, q2.col0), wave, lane, live);
+    bc_raw_copy<NSTG>(p, pin.bcd, dst, b, q2, cell_of(p, q2.bnd0, r, q2.col0), swave, lane, live);
   };
   int rp = 0;
   if (direct) {
-    bc_raw_copy<NW>(p, pin.bcd, raw, b, bp, cell0, wave, lane, true);
+    if (stages) bc_raw_copy<NSTG>(p, pin.bcd, raw, b, bp, cell0, swave, lane, true);
     raw_copy_for(pos_before(A), raw + kRawBytes, m_hi - 2 >= m_lo);
-    stage_block<T, 4, CW, true, STAGE_X, NW, true>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+    if (stages) stage_block<T, 4, CW, true, STAGE_X, NSTG, true>(p, lds, b, A, bp, cell0, e_wg0, swave, lane, X, DT, DL, DY);
     staging_fence();
-    bc_widen<SG, NW>(raw, lds, wave, lane);
+    if (stages) bc_widen<SG, NSTG>(raw, lds, swave, lane);
   } else {
-    stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+    if (stages) stage_block<T, 4, CW, true, STAGE_X, NSTG>(p, lds, b, A, bp, cell0, e_wg0, swave, lane, X, DT, DL, DY);
   }
   staging_fence();
   int cur = 0;
   int xpar = 0;
 
+  // The sweep over the blocks of the window, as a wave of the given role runs it (see m2d_fwd_split_kernel); the
+  // waves that stage also add up the channel sums of every step.
+  auto sweep = [&](auto role) {
+  constexpr int ROLE = decltype(role)::value;
+  constexpr bool STAGES = ROLE != kSweeper, SWEEPS = ROLE != kStager;
   for (int m = m_hi - 1; m >= m_lo; --m) {
     const int t0 = m * kCK;
     const char* bufc = lds + cur * SG::kBytes;
     float hb[kCK + 1][4], gT[kCK][4], gL[kCK][4];
-    { const float4 v = Snap<T>::widen(cknext); hb[0][0] = v.x; hb[0][1] = v.y; hb[0][2] = v.z; hb[0][3] = v.w; }
+    if constexpr (SWEEPS) { const float4 v = Snap<T>::widen(cknext); hb[0][0] = v.x; hb[0][1] = v.y; hb[0][2] = v.z; hb[0][3] = v.w; }
     const Pos Aprev = pos_before(A);
     const BlockPos bpn = block_pos(p, Aprev, r, rbands);
     const int celln = cell_of(p, bpn.bnd0, r, bpn.col0);
-    ck_take = snapshot_lane(p, Pos{bpn.bnd0, bpn.col0}, r, ch_ok);
-    if (direct) raw_copy_for(pos_before(Aprev), raw + rp * kRawBytes, m - 2 >= m_lo);
-    if (m > m_lo) {
+    if constexpr (SWEEPS) ck_take = snapshot_lane(p, Pos{bpn.bnd0, bpn.col0}, r, ch_ok);
+    if constexpr (STAGES) { if (direct) raw_copy_for(pos_before(Aprev), raw + rp * kRawBytes, m - 2 >= m_lo); }
+    if (STAGES && m > m_lo) {
       if constexpr (SLICED) link.wait_for(link_need_bwd(m - 1 - m_lo, p.sl_nbb));
       if (direct) {
-        stage_block<T, 4, CW, true, STAGE_X, NW, true>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
-        bc_widen<SG, NW>(raw + (rp ^ 1) * kRawBytes, lds + (cur ^ 1) * SG::kBytes, wave, lane);
+        stage_block<T, 4, CW, true, STAGE_X, NSTG, true>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, swave, lane, X, DT, DL, DY);
+        bc_widen<SG, NSTG>(raw + (rp ^ 1) * kRawBytes, lds + (cur ^ 1) * SG::kBytes, swave, lane);
       } else {
-        stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+        stage_block<T, 4, CW, true, STAGE_X, NSTG>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, swave, lane, X, DT, DL, DY);
       }
     }
     rp ^= 1;
-    cell_off0 = (uint32_t)(cell0 * p.E + e) * (uint32_t)sizeof(T);
-    f_off0 = (uint32_t)cell0 * (uint32_t)(3 * kN * sizeof(float));
+    if constexpr (SWEEPS) cell_off0 = (uint32_t)(cell0 * p.E + e) * (uint32_t)sizeof(T);
+    if constexpr (STAGES) f_off0 = (uint32_t)cell0 * (uint32_t)(3 * kN * sizeof(float));
 
     // ---- recompute the states of the block, keeping the gates
+    if constexpr (SWEEPS)
 #pragma unroll
     for (int k = 0; k < kCK; ++k) {
       if (t0 + k < p.T_total) {
@@ -2764,8 +2824,9 @@ __global__ __launch_bounds__(NWS * 64) void m2d_bwd_split_kernel(const ScanParam
 #pragma unroll
     for (int k = kCK - 1; k >= 0; --k) {
       if (k == 0) staging_landed();   // before the last stores of the block
-      if (k == (kCK > 1 ? 1 : 0) && m > m_lo) load_ckpt(m - 1, ck_take);
+      if constexpr (SWEEPS) { if (k == (kCK > 1 ? 1 : 0) && m > m_lo) load_ckpt(m - 1, ck_take); }
       if (t0 + k < p.T_total) {
+       if constexpr (SWEEPS) {
         const float4 kk = *reinterpret_cast<const float4*>(bufc + const_off + k * SG::kKStr);
         const float cT = kk.z, cL = kk.w;
         const bool inr = ch_ok && ((bp.in_grid >> k) & 1u);
@@ -2831,15 +2892,16 @@ __global__ __launch_bounds__(NWS * 64) void m2d_bwd_split_kernel(const ScanParam
         if (p.dpre && (g & 1) == 0) tot *= softplus_slope<T>(g == 0 ? dtv : dlv);   // gradients with respect to what the softplus was applied to
         if (g == 1) tot = __builtin_fmaf(dyv, dsk, tot);
         if (inr && g != 3) IO<T>::st(reinterpret_cast<T*>(OUTimg + goff), tot);
+       }
         // ---- across the waves of the workgroup
         __syncthreads();
-        if (f_on && ((bp.in_grid >> k) & 1u)) {
+        if (STAGES && f_on && ((bp.in_grid >> k) & 1u)) {
           const uint32_t off = f_off0 + (uint32_t)k * pstep + (k >= bp.kw ? pwrap_adj : 0u);
           if constexpr (QUADS) {
             const float4* sl = slots + xpar * NW * SLOT + f_v * 64 + lane;
             float4 sum = sl[0];
 #pragma unroll
-            for (int w = 1; w < NW; ++w) { sum.x += sl[w * SLOT].x; sum.y += sl[w * SLOT].y; sum.z += sl[w * SLOT].z; sum.w += sl[w * SLOT].w; }
+            for (int w = 1; w < NW; ++w) { const float4 o = sl[w * SLOT]; sum.x += o.x; sum.y += o.y; sum.z += o.z; sum.w += o.w; }
             // component j holds state perm(j) * 4 + g, perm = (0, 2, 1, 3)
             float* dst = reinterpret_cast<float*>(PARTimg + off + (uint32_t)(f_v * kN + g) * (uint32_t)sizeof(float));
             dst[0] = sum.x; dst[8] = sum.y; dst[4] = sum.z; dst[12] = sum.w;
@@ -2856,18 +2918,27 @@ __global__ __launch_bounds__(NWS * 64) void m2d_bwd_split_kernel(const ScanParam
       }
     }
     __syncthreads();
-    if constexpr (SLICED) link.publish((uint32_t)(m_hi - m));   // (this block counts: see m2d_bwd_kernel)
+    if constexpr (SLICED && STAGES) link.publish((uint32_t)(m_hi - m));   // (this block counts: see m2d_bwd_kernel)
     A = Aprev;
     bp = bpn;
     cell0 = celln;
     cur ^= 1;
   }
+  };
+  if constexpr (NH == 0) sweep(std::integral_constant<int, kAll>{});
+  else if (helper) sweep(std::integral_constant<int, kStager>{});
+  else sweep(std::integral_constant<int, kSweeper>{});
   bool broken = false;
   if constexpr (SLICED) {
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
     link.publish((uint32_t)p.sl_nbb);
     broken = link.broken() || link_poll(p.link_err) != 0u;   // (also a workgroup of the forward sweep that rebuilt the snapshots for this launch)
+    if constexpr (NH > 0) {   // only the waves that wait know of a wait given up: they tell the others (the staging buffers are free now)
+      if ((int)threadIdx.x == link.pub) *reinterpret_cast<volatile uint32_t*>(lds) = link.broken() ? 1u : 0u;
+      __syncthreads();
+      broken = broken || *reinterpret_cast<volatile uint32_t*>(lds) != 0u;
+    }
     if (broken) poison_band<T>(p, my_band, b, e_wg0, CW, p.dx, p.ddT, p.ddL);
   }
 
@@ -3243,7 +3314,13 @@ Geometry make_geometry(const m2d_desc* d) {
   // Workgroups of 8 waves (8 channels) under way on at most half of the compute units: workgroups of 4 then run on
   // twice as many, each wave with a SIMD to itself (a sweep of few images is as fast as one wave gets through its
   // blocks).
-  const int split_nw = 2 * (int64_t)B * ((d->E + kSplitWaves - 1) / kSplitWaves) * together <= ncu ? kSplitHalfWaves : kSplitWaves;
+  // In the linked sweep a workgroup of 4 has 4 more waves that stage for it (split_helpers), which is worth more than
+  // a compute unit for every workgroup under way: up to 7 workgroups for every 5 units (measured, E=64 fp32: 512x512
+  // 3.14 -> 2.54 ms forward+backward kernels and 640x640 3.90 -> 3.62 with workgroups of 4; 768x768 4.76 -> 5.08).
+  const int64_t wg4 = (int64_t)B * ((d->E + kSplitHalfWaves - 1) / kSplitHalfWaves) * together;
+  const bool helped = g.sliced && split_helpers<kModeSliced, kSplitHalfWaves>() > 0;
+  const int split_nw = (helped ? 5 * wg4 <= 7 * ncu : 2 * (int64_t)B * ((d->E + kSplitWaves - 1) / kSplitWaves) * together <= ncu)
+                           ? kSplitHalfWaves : kSplitWaves;
   if (g.fwd_split) {
     g.fwd_ec = 1;
     g.fwd_nw = split_nw;
@@ -3282,7 +3359,7 @@ Geometry make_geometry(const m2d_desc* d) {
   g.top_bytes = rows ? align_up(sizeof(float) * (size_t)(g.nbands - 1) * B * d->W * d->E * kN) : 0;
   g.bot_bytes = rows ? align_up(sizeof(float) * (size_t)(g.sliced ? g.nbands : 1) * B * d->W * d->E * kN) : 0;
   const size_t chains = (size_t)B * (g.fwd_bpb > g.bwd_bpb ? g.fwd_bpb : g.bwd_bpb);
-  g.link_bytes = g.sliced ? align_up(sizeof(uint32_t) * (64 + 2 * g.nbands * chains)) : 0;
+  g.link_bytes = g.sliced ? align_up(sizeof(uint32_t) * (64 + 2 * g.nbands * chains * kLinkStride)) : 0;
   g.part_bytes = align_up(sizeof(float) * (size_t)g.bwd_bpb * 3 * P * kN);
   const size_t slots = g.sliced ? g.nbands : 1;
   g.pa_bytes = align_up(sizeof(float) * (size_t)B * slots * d->E * 2 * kN);
@@ -3371,9 +3448,12 @@ int stage_bc(ScanParams& sp, const m2d_desc* d, const void* BT, const void* BL, 
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
 }
 
-// Development aid: -DM2D_QUICK builds only the kernels of many 16-bit images in one stream each, in workgroups of
-// 8 waves (a twentieth of the compile time); every other problem then answers M2D_ERR_UNSUPPORTED.
-#ifdef M2D_QUICK
+// Development aid: -DM2D_QUICK=1 builds only the kernels of many 16-bit images in one stream each, in workgroups of
+// 8 waves (a twentieth of the compile time), -DM2D_QUICK=2 (3) only the linked sweep of fp32 (16-bit) images in workgroups of 4 waves;
+// every other problem then answers M2D_ERR_UNSUPPORTED.
+#if defined(M2D_QUICK) && M2D_QUICK >= 2
+#define M2D_BUILT(T, SX, MODE, NW, OTHER) (sizeof(T) == (M2D_QUICK == 3 ? 2 : 4) && (MODE) == kModeSliced && (NW) == (M2D_QUICK == 4 ? 8 : 4) && (M2D_QUICK != 4 || !(OTHER)))
+#elif defined(M2D_QUICK)
 #define M2D_BUILT(T, SX, MODE, NW, OTHER) (sizeof(T) == 2 && (SX) && (MODE) == kModeSweep && (NW) == 8 && (OTHER))
 #else
 #define M2D_BUILT(T, SX, MODE, NW, OTHER) true
@@ -3400,7 +3480,7 @@ int launch_fwd_split_as(const ScanParams& sp, hipStream_t st) {
   static_assert(lds <= kLdsPerWorkgroup, "staging must fit the LDS");
   static std::atomic<uint64_t> seen{0};
   if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_fwd_split_kernel<T, CK, WY, SX, MODE, NWS>), lds, seen)) return M2D_ERR_HIP;
-  hipLaunchKernelGGL((m2d_fwd_split_kernel<T, CK, WY, SX, MODE, NWS>), dim3((unsigned)sp.nwg), dim3(NWS * 64), lds, st, sp);
+  hipLaunchKernelGGL((m2d_fwd_split_kernel<T, CK, WY, SX, MODE, NWS>), dim3((unsigned)sp.nwg), dim3((NWS + split_helpers<MODE, NWS>()) * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
   }
 }
@@ -3541,7 +3621,7 @@ int launch_bwd_split_as(const ScanParams& sp, hipStream_t st) {
   static_assert(lds <= kLdsPerWorkgroup, "exchange buffers and staging must fit the LDS");
   static std::atomic<uint64_t> seen{0};
   if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_bwd_split_kernel<T, SX, MODE, NWS>), lds, seen)) return M2D_ERR_HIP;
-  hipLaunchKernelGGL((m2d_bwd_split_kernel<T, SX, MODE, NWS>), dim3((unsigned)sp.nwg), dim3(NWS * 64), lds, st, sp);
+  hipLaunchKernelGGL((m2d_bwd_split_kernel<T, SX, MODE, NWS>), dim3((unsigned)sp.nwg), dim3((NWS + split_helpers<MODE, NWS>()) * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
   }
 }
@@ -3611,7 +3691,7 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   } else {
     // every band on workgroups of its own, the last band first: a band waits for the one below it
     sp.nwg = g.nbands * g.vB * g.bwd_bpb;
-    sp.prog = sp.link_err + 64 + (size_t)g.nbands * g.vB * (g.fwd_bpb > g.bwd_bpb ? g.fwd_bpb : g.bwd_bpb);
+    sp.prog = sp.link_err + 64 + (size_t)g.nbands * g.vB * (g.fwd_bpb > g.bwd_bpb ? g.fwd_bpb : g.bwd_bpb) * kLinkStride;
     if (g.bwd_split) rc = launch_bwd_split<T, kModeSliced>(sp, g.stage_x, st, g.bwd_nw);
     else rc = g.stage_x ? launch_bwd<T, true, kModeSliced>(sp, st, g.bwd_nw) : launch_bwd<T, false, kModeSliced>(sp, st, g.bwd_nw);
   }
@@ -3749,9 +3829,13 @@ int m2d_scan_plan(const m2d_desc* desc, int pass, char* text, size_t cap) {
   if (g.sliced) snprintf(sched, sizeof sched, "linked sweep, %d bands", g.nbands);
   else if (g.stacked) snprintf(sched, sizeof sched, "stacked images, %d per stream, %d bands", g.ips, g.nbands);
   else snprintf(sched, sizeof sched, "one stream per image, %d band%s back to back", g.nbands, g.nbands == 1 ? "" : "s");
-  if (split)
-    snprintf(text, cap, "%s: %s, %lld workgroups of %d waves, %d channels each, 4 states per lane",
-             fwd ? "m2d_fwd_split_kernel" : "m2d_bwd_split_kernel", sched, wgs, nw, nw);
+  if (split) {
+    const int helpers = !g.sliced ? 0 : (nw == kSplitHalfWaves ? split_helpers<kModeSliced, kSplitHalfWaves>() : split_helpers<kModeSliced, kSplitWaves>());
+    char extra[48] = "";
+    if (helpers) snprintf(extra, sizeof extra, " and %d that stage", helpers);
+    snprintf(text, cap, "%s: %s, %lld workgroups of %d waves%s, %d channels each, 4 states per lane",
+             fwd ? "m2d_fwd_split_kernel" : "m2d_bwd_split_kernel", sched, wgs, nw, extra, nw);
+  }
   else
     snprintf(text, cap, "%s: %s, %lld workgroups of %d waves, %d channels each, 16 states per lane%s",
              fwd ? "m2d_fwd_kernel" : (g.ck_half ? "m2d_bwd2_kernel" : "m2d_bwd_kernel"), sched, wgs, nw, nw * g.CS * per_lane,
