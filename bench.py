@@ -504,8 +504,9 @@ def main():
     ap.add_argument("--no-also", action="store_true", help="skip the short measurements of the other workloads that the default workload appends")
     ap.add_argument("--no-ckpt", action="store_true", help="rebuild checkpoints inside the backward")
     ap.add_argument("--ckpt-interval", type=int, default=0, choices=(0, 2, 4, 8, 16),
-                    help="steps between the state snapshots the forward keeps (0 or 4: the default; 8, 16: fewer "
-                         "snapshots, and the backward replays the forward in between)")
+                    help="steps between the state snapshots the forward keeps (0: the library's choice, 2 where every "
+                         "image or stack has a stream to itself and 4 elsewhere; 8, 16: fewer snapshots, and the backward "
+                         "replays the forward in between)")
     ap.add_argument("--dtype", default=None, choices=("f32", "bf16"),
                     help="tensor type of a single-scan workload (default: the workload's own)")
     ap.add_argument("--calib-copy", action="store_true",

@@ -1294,14 +1294,11 @@ constexpr int kSplitHalfWaves = 4;   // where workgroups of 8 would leave comput
 // stage (and, in the backward, add up the channel sums of every step), one to a SIMD beside a wave that does nothing
 // but sweep: the two chains run side by side.
 constexpr int kAll = 0, kSweeper = 1, kStager = 2;   // what a wave of such a workgroup does
-#ifndef M2D_SPLIT_HELPERS
-#define M2D_SPLIT_HELPERS 4
-#endif
-#ifndef M2D_SPLIT_HELPERS8
-#define M2D_SPLIT_HELPERS8 0
-#endif
+// (Workgroups of 8 sweeping waves stay as they are: with 8 more the backward no longer fits the registers of a lane
+// at 4 waves to a SIMD and ran a quarter slower, 768x768 and 1024x1024; with 4 more the compiler fails.)
+constexpr int kSplitHelpers = 4;
 template <int MODE, int NWS>
-constexpr int split_helpers() { return MODE != kModeSliced ? 0 : (NWS == kSplitHalfWaves ? M2D_SPLIT_HELPERS : M2D_SPLIT_HELPERS8); }
+constexpr int split_helpers() { return (MODE == kModeSliced && NWS == kSplitHalfWaves) ? kSplitHelpers : 0; }
 __device__ __forceinline__ float sum_over_groups(float v) {
   v = fold16(v, v);
   return fold32(v, v);
@@ -3452,7 +3449,7 @@ int stage_bc(ScanParams& sp, const m2d_desc* d, const void* BT, const void* BL, 
 // 8 waves (a twentieth of the compile time), -DM2D_QUICK=2 (3) only the linked sweep of fp32 (16-bit) images in workgroups of 4 waves;
 // every other problem then answers M2D_ERR_UNSUPPORTED.
 #if defined(M2D_QUICK) && M2D_QUICK >= 2
-#define M2D_BUILT(T, SX, MODE, NW, OTHER) (sizeof(T) == (M2D_QUICK == 3 ? 2 : 4) && (MODE) == kModeSliced && (NW) == (M2D_QUICK == 4 ? 8 : 4) && (M2D_QUICK != 4 || !(OTHER)))
+#define M2D_BUILT(T, SX, MODE, NW, OTHER) (sizeof(T) == (M2D_QUICK == 3 ? 2 : 4) && (MODE) == kModeSliced && (NW) == 4)
 #elif defined(M2D_QUICK)
 #define M2D_BUILT(T, SX, MODE, NW, OTHER) (sizeof(T) == 2 && (SX) && (MODE) == kModeSweep && (NW) == 8 && (OTHER))
 #else
