@@ -852,8 +852,17 @@ __device__ __forceinline__ int snapshot_index(const ScanParams& p, int m, int m_
 // NW waves per workgroup: 8, or 4 where the batch is too small to give every compute unit a
 // workgroup of 8 (each wave then has a SIMD to itself).
 // HALF: a snapshot every 2 steps instead of every 4 (m2d_bwd2_kernel restarts from them), and one more behind the sweep.
+// Workgroups of 4 waves (few workgroups: each wave has a SIMD to itself) get 4 more waves that only stage: positions,
+// copies, the wait for the neighbouring band of a linked sweep, the flush of y, the cross-wave channel sums of the
+// backward; the first 4 only sweep.  A lone wave gets through a step as fast as its chain of instructions allows, and a
+// quarter of that chain was staging (B=64, E=64, 56x56 bf16 with the copies left out: forward 0.220 -> 0.166 ms, backward
+// 0.550 -> 0.458 ms).  Both kinds run the same loop, compiled once per role, with the same barriers.
+constexpr int kAll = 0, kSweeper = 1, kStager = 2;   // what a wave does: both, only sweep, only stage
+constexpr int kWholeHelpers = 4;
+template <int MODE, int NW, int EC = 1>
+constexpr int whole_helpers() { return (MODE != kModeStacked && NW == kFwdHalfWaves && EC == 1) ? kWholeHelpers : 0; }
 template <typename T, int EC, bool CKPT, bool WRITE_Y, bool STAGE_X, int MODE, int NW = kFwdWaves, bool HALF = false>
-__global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) {
+__global__ __launch_bounds__((NW + whole_helpers<MODE, NW, EC>()) * 64) void m2d_fwd_kernel(const ScanParams pin) {
   constexpr bool SLICED = MODE == kModeSliced, STACKED = MODE == kModeStacked;
   static_assert(!HALF || (CKPT && !SLICED), "snapshots every 2 steps: kept by a forward of one stream per image or stack");
   ScanParams p = pin;   // (stacked images: the height is shortened below for a last, shorter stack)
@@ -866,6 +875,8 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   constexpr int CW = NW * CS * EC;
   constexpr bool PERM = true;
   constexpr bool AHEAD = EC == 1 && STAGE_X;   // operands of step t+1 are fetched from LDS during step t
+  constexpr int NH = whole_helpers<MODE, NW, EC>();   // waves that only stage (then the first NW waves only sweep)
+  constexpr int NSTG = NH ? NH : NW;                  // waves that share the copies of a block
   using SG = Stage<T, 3, CW, false>;
   extern __shared__ float4 smem[];
   char* lds = reinterpret_cast<char*>(smem);       // two staging buffers
@@ -874,7 +885,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   int lb = SLICED ? (int)blockIdx.x : logical_block(p.nwg);   // (linked bands keep the launch order: a band waits for a lower index)
   int m_lo = 0, m_hi = p.nblk;                     // blocks of steps this workgroup sweeps
   int my_band = 0;
-  Link link;
+  LinkT<NH ? NW * 64 : 0> link;
   if constexpr (SLICED) {   // the window of one band
     const int per = p.B * p.bpb;
     my_band = lb / per;
@@ -894,15 +905,19 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     p.nbands = (p.H + p.rb - 1) / p.rb;
     p.rows_last = p.H - (p.nbands - 1) * p.rb;
   }
+  const bool helper = NH && wave >= NW;            // (uniform) stages, never sweeps
+  const bool stages = !NH || helper;
+  const int swave = NH ? wave - NW : wave;         // the wave's turn among those that stage
+  const int stid = NH ? (int)threadIdx.x - NW * 64 : (int)threadIdx.x;   // ... and the thread's among their threads
   const int slot = lane >> kHBShift, r = lane & (kHB - 1);
   const int rbands = row_bands(p, r);
   const int rk = STACKED ? skew_row(p, r) : r;     // the row by which the lane trails the head of the stream
-  const int ch_loc = (wave * CS + slot) * EC;      // first channel of the lane inside the workgroup
+  const int ch_loc = ((helper ? swave : wave) * CS + slot) * EC;   // first channel of the lane inside the workgroup
   const int e_raw = e_wg0 + ch_loc;
-  const bool ch_ok = e_raw < p.E;                  // idle lanes still take part in staging and barriers
-  const int e0 = ch_ok ? e_raw : p.E - EC;
+  const bool ch_ok = !helper && e_raw < p.E;       // idle lanes still take part in staging and barriers
+  const int e0 = e_raw < p.E ? e_raw : p.E - EC;
   // every byte a lane may read is finite from the start (pads are never written again)
-  for (int i = threadIdx.x; i < 2 * SG::kBytes / 16; i += NW * 64) smem[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int i = threadIdx.x; i < 2 * SG::kBytes / 16; i += (NW + NH) * 64) smem[i] = make_float4(0.f, 0.f, 0.f, 0.f);
 
   float a2t[EC][kN], a2l[EC][kN], dsk[EC];
 #pragma unroll
@@ -933,7 +948,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   char* ywin = raw + (WIDEN ? 2 * kRawBytes : 0);   // [2 windows][YT::kBytes]
   uint2* ytab = reinterpret_cast<uint2*>(ywin + 2 * YT::kBytes);   // [block & 3][lane]
   if constexpr (YTILE) {   // the block before the first has no row on the grid
-    for (int i = threadIdx.x; i < 4 * 64; i += NW * 64) ytab[i] = make_uint2(0u, 0u);
+    for (int i = threadIdx.x; i < 4 * 64; i += (NW + NH) * 64) ytab[i] = make_uint2(0u, 0u);
   }
 
   settle_loads();
@@ -1092,7 +1107,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   // step of the sweep; the rest of the window is from two blocks ago).
   auto flush_y = [&](int par, int m, bool first_only) {   // m: the block whose barrier this is
     const char* win = ywin + par * YT::kBytes;
-    const int c = threadIdx.x / NW, j = threadIdx.x % NW;
+    const int c = stid / NW, j = stid % NW;
     const int ks = c >> kHBShift;                                  // the cell's step in the window ...
     const int k = AHEAD ? (ks + kCK - 1) & (kCK - 1) : ks;         // ... and in its block,
     const int blk = AHEAD && ks == 0 ? m - 1 : m;                  // which is the one before for the window's first step
@@ -1109,31 +1124,35 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
   Pos A = pos_of(p, m_lo * kCK - (kHB - 1));     // position of the stream index t0 - 15 (wave-uniform)
   bp = block_pos(p, A, rk, rbands);
   int cell0 = cell_of(p, bp.bnd0, r, bp.col0);   // cell index of the lane's position at the first step of the block
-  if constexpr (SLICED) link.wait_for(link_need_fwd(0, p.sl_nbb));
+  if constexpr (SLICED) { if (stages) link.wait_for(link_need_fwd(0, p.sl_nbb)); }
   BlockPos bpq = bp;     // 16-bit direct records: the block after the next (fetched two blocks ahead)
   int cellq = cell0;
   int rp = 0;            // ... and the half of `raw` it goes to
   if (direct) {
     if constexpr (WIDEN) {
-      bc_raw_copy<NW>(p, pin.bcd, raw, b, bp, cell0, wave, lane, true);
+      if (stages) bc_raw_copy<NSTG>(p, pin.bcd, raw, b, bp, cell0, swave, lane, true);
       bpq = block_pos(p, pos_after(p, A, kCK), rk, rbands);
       cellq = cell_of(p, bpq.bnd0, r, bpq.col0);
-      bc_raw_copy<NW>(p, pin.bcd, raw + kRawBytes, b, bpq, cellq, wave, lane, m_lo + 1 < m_hi);
+      if (stages) bc_raw_copy<NSTG>(p, pin.bcd, raw + kRawBytes, b, bpq, cellq, swave, lane, m_lo + 1 < m_hi);
     } else {
-      bc_direct_copy<T, CW, NW>(p, pin.bcd, lds, b, bp, cell0, wave, lane);
+      if (stages) bc_direct_copy<T, CW, NSTG>(p, pin.bcd, lds, b, bp, cell0, swave, lane);
     }
-    stage_block<T, 3, CW, false, STAGE_X, NW, true>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+    if (stages) stage_block<T, 3, CW, false, STAGE_X, NSTG, true>(p, lds, b, A, bp, cell0, e_wg0, swave, lane, X, DT, DL, DY);
     if constexpr (WIDEN) {
       staging_fence();
-      bc_widen<SG, NW>(raw, lds, wave, lane);
+      if (stages) bc_widen<SG, NSTG>(raw, lds, swave, lane);
     }
   } else {
-    stage_block<T, 3, CW, false, STAGE_X, NW>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+    if (stages) stage_block<T, 3, CW, false, STAGE_X, NSTG>(p, lds, b, A, bp, cell0, e_wg0, swave, lane, X, DT, DL, DY);
   }
   staging_fence();
   Ops opsA, opsB;
-  if constexpr (AHEAD) fetch(lds, 0, opsA);
+  if constexpr (AHEAD) { if (!helper) fetch(lds, 0, opsA); }
   int cur = 0;
+  // The sweep over the blocks of the window, as a wave of the given role runs it.
+  auto sweep = [&](auto role) {
+  constexpr int ROLE = decltype(role)::value;
+  constexpr bool STAGES = ROLE != kSweeper, SWEEPS = ROLE != kStager;
   for (int m = m_lo; m < m_hi; ++m) {
     const bool last = m + 1 == m_hi;
     // the next block: where the lane's row will be is also what the lane's copies fetch
@@ -1145,27 +1164,35 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
       celln = cellq;
       bpq = block_pos(p, pos_after(p, An, kCK), rk, rbands);
       cellq = cell_of(p, bpq.bnd0, r, bpq.col0);
-      bc_raw_copy<NW>(p, pin.bcd, raw + rp * kRawBytes, b, bpq, cellq, wave, lane, m + 2 < m_hi);
+      if constexpr (STAGES) bc_raw_copy<NSTG>(p, pin.bcd, raw + rp * kRawBytes, b, bpq, cellq, swave, lane, m + 2 < m_hi);
     } else if (WIDEN && direct) {   // two channels per lane: no registers to carry a block's positions in; worked out twice
       bpn = block_pos(p, An, rk, rbands);
       celln = cell_of(p, bpn.bnd0, r, bpn.col0);
-      const BlockPos q2 = block_pos(p, pos_after(p, An, kCK), rk, rbands);
-      bc_raw_copy<NW>(p, pin.bcd, raw + rp * kRawBytes, b, q2, cell_of(p, q2.bnd0, r, q2.col0), wave, lane, m + 2 < m_hi);
+      if constexpr (STAGES) {
+        const BlockPos q2 = block_pos(p, pos_after(p, An, kCK), rk, rbands);
+        bc_raw_copy<NSTG>(p, pin.bcd, raw + rp * kRawBytes, b, q2, cell_of(p, q2.bnd0, r, q2.col0), swave, lane, m + 2 < m_hi);
+      }
     } else {
       bpn = block_pos(p, An, rk, rbands);
       celln = cell_of(p, bpn.bnd0, r, bpn.col0);
     }
-    if (!last) {
+    if (STAGES && !last) {
       if constexpr (SLICED) link.wait_for(link_need_fwd(m + 1 - m_lo, p.sl_nbb));
       if (direct) {
-        if constexpr (!WIDEN) bc_direct_copy<T, CW, NW>(p, pin.bcd, lds + (cur ^ 1) * SG::kBytes, b, bpn, celln, wave, lane);
-        stage_block<T, 3, CW, false, STAGE_X, NW, true>(p, lds + (cur ^ 1) * SG::kBytes, b, An, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
-        if constexpr (WIDEN) bc_widen<SG, NW>(raw + (rp ^ 1) * kRawBytes, lds + (cur ^ 1) * SG::kBytes, wave, lane);
+        if constexpr (!WIDEN) bc_direct_copy<T, CW, NSTG>(p, pin.bcd, lds + (cur ^ 1) * SG::kBytes, b, bpn, celln, swave, lane);
+        stage_block<T, 3, CW, false, STAGE_X, NSTG, true>(p, lds + (cur ^ 1) * SG::kBytes, b, An, bpn, celln, e_wg0, swave, lane, X, DT, DL, DY);
+        if constexpr (WIDEN) bc_widen<SG, NSTG>(raw + (rp ^ 1) * kRawBytes, lds + (cur ^ 1) * SG::kBytes, swave, lane);
       } else {
-        stage_block<T, 3, CW, false, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, An, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+        stage_block<T, 3, CW, false, STAGE_X, NSTG>(p, lds + (cur ^ 1) * SG::kBytes, b, An, bpn, celln, e_wg0, swave, lane, X, DT, DL, DY);
       }
     }
     rp ^= 1;
+    if constexpr (!SWEEPS) {   // a wave that only stages: its copies have landed, then what follows the block's barrier
+      staging_landed();
+      __syncthreads();
+      if constexpr (SLICED) link.publish((uint32_t)(m - m_lo + 1));
+      if constexpr (YTILE) flush_y(ypar, m, false);
+    } else {
     cell_off0 = (uint32_t)(cell0 * p.E + e0) * (uint32_t)sizeof(T);
     if constexpr (YTILE)
       ytab[(m & 3) * 64 + lane] = make_uint2((uint32_t)(cell0 * p.E + e_wg0) * (uint32_t)sizeof(T), ((uint32_t)(bp.kw < kCK ? bp.kw : kCK) << 8) | (bp.in_grid & 15u));
@@ -1195,6 +1222,8 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     const bool top_thrice = SLICED && __any(ch_ok && (bp.in_grid & 7u) == 7u && r == kRB && bp.kw >= kCK && bp.bnd0 + 1 < p.nbands);
     auto next_block_landed = [&] {
       // the stores issued since (snapshot, y) need not have completed, only the copies before them
+      // (a wave that only sweeps has issued no copies, but waits all the same: with it, every store older than a block
+      // has completed, which the boundary rows that a later band of this workgroup reads back rely on)
       if constexpr (SLICED) {
         // Linked sweep: the band below needs, of the newest block it is told about, the last row of the steps 0 and 1
         // only (link_need_fwd).  Only what is issued after the row of step 1 stays in flight (y of step 1, row and
@@ -1229,8 +1258,8 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
           __syncthreads();
           lead_if_younger<NW>(wave, true);   // (from here to the second step of the next block: half of the way to the next barrier)
           // every wave has waited for the rows it stored at the steps 0 and 1 of this block
-          if constexpr (SLICED) link.publish((uint32_t)(m - m_lo + 1));
-          if constexpr (YTILE) flush_y(ypar, m, false);   // the last step of the block before and the first three of this one
+          if constexpr (SLICED && STAGES) link.publish((uint32_t)(m - m_lo + 1));
+          if constexpr (YTILE && STAGES) flush_y(ypar, m, false);   // the last step of the block before and the first three of this one
           if (!last) fetch(bufn, 0, ahead);
         }
         if (k == 1) lead_if_younger<NW>(wave, false);
@@ -1248,8 +1277,9 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
         step(k, opsA);
       }
       __syncthreads();
-      if constexpr (SLICED) link.publish((uint32_t)(m - m_lo + 1));
-      if constexpr (YTILE) flush_y(ypar, m, false);   // the four steps of this block
+      if constexpr (SLICED && STAGES) link.publish((uint32_t)(m - m_lo + 1));
+      if constexpr (YTILE && STAGES) flush_y(ypar, m, false);   // the four steps of this block
+    }
     }
     ypar ^= 1;
     cur ^= 1;
@@ -1257,11 +1287,15 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     bp = bpn;
     cell0 = celln;
   }
+  };
+  if constexpr (NH == 0) sweep(std::integral_constant<int, kAll>{});
+  else if (helper) sweep(std::integral_constant<int, kStager>{});
+  else sweep(std::integral_constant<int, kSweeper>{});
   if constexpr (YTILE && AHEAD) {   // the last step of the sweep
     __syncthreads();
-    flush_y(ypar, m_hi, true);
+    if (stages) flush_y(ypar, m_hi, true);
   }
-  if constexpr (CKPT && HALF) {   // the state behind the last block: what the last step of the sweep left is among it
+  if constexpr (CKPT && HALF) if (!helper) {   // the state behind the last block: what the last step of the sweep left is among it
     typename Snap<T>::quad* end = snapshot_at<T>(p, b, ch_ok ? 2 * p.nblk : 0, e0, p.ck_nblk) + snap_lane(r);
 #pragma unroll
     for (int c = 0; c < EC; ++c)
@@ -1275,7 +1309,13 @@ __global__ __launch_bounds__(NW * 64) void m2d_fwd_kernel(const ScanParams pin) 
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
     link.publish((uint32_t)p.sl_nbb);
-    if (WRITE_Y && link.broken()) poison_band<T>(p, my_band, b, e_wg0, CW, p.y, nullptr, nullptr);
+    bool broken = link.broken();
+    if constexpr (NH > 0) {   // only the waves that wait know: they tell the others (the staging buffers are free now)
+      if ((int)threadIdx.x == link.pub) *reinterpret_cast<volatile uint32_t*>(lds) = broken ? 1u : 0u;
+      __syncthreads();
+      broken = *reinterpret_cast<volatile uint32_t*>(lds) != 0u;
+    }
+    if (WRITE_Y && broken) poison_band<T>(p, my_band, b, e_wg0, CW, p.y, nullptr, nullptr);
   }
 }
 
@@ -1293,7 +1333,6 @@ constexpr int kSplitHalfWaves = 4;   // where workgroups of 8 would leave comput
 // addresses, copies, the wait for the neighbouring band).  So such a workgroup gets 4 more waves that do nothing but
 // stage (and, in the backward, add up the channel sums of every step), one to a SIMD beside a wave that does nothing
 // but sweep: the two chains run side by side.
-constexpr int kAll = 0, kSweeper = 1, kStager = 2;   // what a wave of such a workgroup does
 // (Workgroups of 8 sweeping waves stay as they are: with 8 more the backward no longer fits the registers of a lane
 // at 4 waves to a SIMD and ran a quarter slower, 768x768 and 1024x1024; with 4 more the compiler fails.)
 constexpr int kSplitHelpers = 4;
@@ -1590,7 +1629,7 @@ constexpr int bwd_exchange_sets() {
 // before each block is parked in the workgroup's ring in memory, where the sweep then finds it like a snapshot.
 // A lane reads back only what it wrote itself.
 template <typename T, bool STAGE_X, int MODE, int NW = kBwdWaves, bool REPLAY = false>
-__global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) {
+__global__ __launch_bounds__((NW + (REPLAY ? 0 : whole_helpers<MODE, NW>())) * 64) void m2d_bwd_kernel(const ScanParams pin) {
   constexpr bool SLICED = MODE == kModeSliced, STACKED = MODE == kModeStacked;
   ScanParams p = pin;   // (stacked images: the height is shortened below for a last, shorter stack)
   if constexpr (!STACKED) {   // lets the compiler drop what only stacked images need
@@ -1602,6 +1641,8 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   constexpr int SLOT = 3 * 64;           // float2s per wave in one exchange buffer
   constexpr int CW = NW * CS;
   constexpr bool PERM = true;
+  constexpr int NH = REPLAY ? 0 : whole_helpers<MODE, NW>();   // waves that only stage and add up the channel sums (then the first NW waves only sweep)
+  constexpr int NSTG = NH ? NH : NW;                           // waves that share the copies of a block and the sums of a half
   using SG = Stage<T, 4, CW, true>;
   extern __shared__ float4 smem[];
   // Exchange buffers for the channel sums of one (step, half of the states).  Either one per step of
@@ -1611,6 +1652,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   // reaches only once it has finished reading it).
   constexpr int XSETS = bwd_exchange_sets<T, NW>();
   constexpr bool BATCH = XSETS == kCK;
+  static_assert(NH == 0 || BATCH, "the waves that stage add up the sums of a half in one go");
   float2* slots = reinterpret_cast<float2*>(smem);                       // [XSETS][wave][3][64]
   float* a_lds = reinterpret_cast<float*>(slots + XSETS * NW * SLOT);    // [wave][CS][2][16], fold order
   char* lds = reinterpret_cast<char*>(a_lds + NW * CS * 2 * kN);  // 2 staging buffers
@@ -1622,7 +1664,7 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   int lb = SLICED ? (int)blockIdx.x : logical_block(p.nwg);   // (linked bands keep the launch order: a band waits for a lower index)
   int m_lo = 0, m_hi = p.nblk;              // blocks of steps this workgroup sweeps (from m_hi - 1 down to m_lo)
   int my_band = 0;
-  Link link;
+  LinkT<NH ? NW * 64 : 0> link;
   if constexpr (SLICED) {   // the window of one band; the bands are launched from the last to the first
     const int per = p.B * p.bpb;
     const int kk = lb / per;
@@ -1644,20 +1686,23 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
     p.rows_last = p.H - (p.nbands - 1) * p.rb;
   }
   const int e_wg0 = eg * CW;
+  const bool helper = NH && wave >= NW;      // (uniform) stages and adds up, never sweeps
+  const bool stages = !NH || helper;
+  const int swave = NH ? wave - NW : wave;   // the wave's turn among those that stage
   const int slot = lane >> kHBShift, r = lane & (kHB - 1);
   const int rbands = row_bands(p, r);
   const int rk = STACKED ? skew_row(p, r) : r;     // the row by which the lane trails the head of the stream
-  const int ch_loc = wave * CS + slot;
+  const int ch_loc = (helper ? swave : wave) * CS + slot;
   const int e_raw = e_wg0 + ch_loc;
-  const bool ch_ok = e_raw < p.E;           // padding lanes/waves still take part in the barriers
-  const int e = ch_ok ? e_raw : p.E - 1;
-  {  // A of the wave's channels into LDS in fold order (read back group by group)
+  const bool ch_ok = !helper && e_raw < p.E;   // padding lanes/waves still take part in the barriers
+  const int e = e_raw < p.E ? e_raw : p.E - 1;
+  if (!helper) {  // A of the wave's channels into LDS in fold order (read back group by group)
     float* mine = a_lds + ch_loc * (2 * kN);
     mine[spos<true>(r)] = p.A2T[e * kN + r];
     mine[kN + spos<true>(r)] = p.A2L[e * kN + r];
   }
   // planes that no copy writes must hold finite values from the start
-  for (int i = threadIdx.x; i < 2 * SG::kBytes / 16; i += NW * 64) reinterpret_cast<float4*>(lds)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int i = threadIdx.x; i < 2 * SG::kBytes / 16; i += (NW + NH) * 64) reinterpret_cast<float4*>(lds)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
   const uint32_t a_base_off = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) float*)(a_lds + ch_loc * (2 * kN)));
   const float dsk = p.Df[e];
   settle_loads();
@@ -1768,26 +1813,30 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
   int cell0 = cell_of(p, bp.bnd0, r, bp.col0);   // cell index of the lane's position at the first step of the block
   bool ck_take = snapshot_lane(p, Pos{bp.bnd0, bp.col0}, r, ch_ok);   // the lane restores a snapshot for the block to come
   if (!LATE_SNAPSHOT && !opens_group(m_hi - 1)) load_ckpt(m_hi - 1, ck_take);   // (else: after the replay that opens the first iteration)
-  if constexpr (SLICED) link.wait_for(link_need_bwd(p.sl_nbb - 1, p.sl_nbb));
+  if constexpr (SLICED) { if (stages) link.wait_for(link_need_bwd(p.sl_nbb - 1, p.sl_nbb)); }
   // the lane's row in the block two before (A2 = position of that block): what its raw copies fetch
   auto raw_copy_for = [&](Pos A2, char* dst, bool live) {
     const BlockPos q2 = block_pos(p, A2, rk, rbands);
-    bc_raw_copy<NW>(p, pin.bcd, dst, b, q2, cell_of(p, q2.bnd0, r, q2.col0), wave, lane, live);
+    bc_raw_copy<NSTG>(p, pin.bcd, dst, b, q2, cell_of(p, q2.bnd0, r, q2.col0), swave, lane, live);
   };
   int rp = 0;   // half of `raw` that the next raw copy goes to
   if (direct) {
-    bc_raw_copy<NW>(p, pin.bcd, raw, b, bp, cell0, wave, lane, true);
-    raw_copy_for(pos_before(A), raw + kRawBytes, m_hi - 2 >= m_lo);
-    stage_block<T, 4, CW, true, STAGE_X, NW, true>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+    if (stages) bc_raw_copy<NSTG>(p, pin.bcd, raw, b, bp, cell0, swave, lane, true);
+    if (stages) raw_copy_for(pos_before(A), raw + kRawBytes, m_hi - 2 >= m_lo);
+    if (stages) stage_block<T, 4, CW, true, STAGE_X, NSTG, true>(p, lds, b, A, bp, cell0, e_wg0, swave, lane, X, DT, DL, DY);
     staging_fence();
-    bc_widen<SG, NW>(raw, lds, wave, lane);
+    if (stages) bc_widen<SG, NSTG>(raw, lds, swave, lane);
   } else {
-    stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+    if (stages) stage_block<T, 4, CW, true, STAGE_X, NSTG>(p, lds, b, A, bp, cell0, e_wg0, swave, lane, X, DT, DL, DY);
   }
   staging_fence();
   int cur = 0;
   int xpar = 0;   // exchange buffer in use
 
+  // The sweep over the blocks of the window, as a wave of the given role runs it (see m2d_fwd_kernel).
+  auto sweep = [&](auto role) {
+  constexpr int ROLE = decltype(role)::value;
+  constexpr bool STAGES = ROLE != kSweeper, SWEEPS = ROLE != kStager;
   for (int m = m_hi - 1; m >= m_lo; --m) {
     const int t0 = m * kCK;
     const char* bufc = lds + cur * SG::kBytes;
@@ -1886,20 +1935,20 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
     const Pos Aprev = pos_before(A);
     const BlockPos bpn = block_pos(p, Aprev, rk, rbands);
     const int celln = cell_of(p, bpn.bnd0, r, bpn.col0);
-    ck_take = snapshot_lane(p, Pos{bpn.bnd0, bpn.col0}, r, ch_ok);
-    if (direct) raw_copy_for(pos_before(Aprev), raw + rp * kRawBytes, m - 2 >= m_lo);
-    if (m > m_lo) {
+    if constexpr (SWEEPS) ck_take = snapshot_lane(p, Pos{bpn.bnd0, bpn.col0}, r, ch_ok);
+    if constexpr (STAGES) { if (direct) raw_copy_for(pos_before(Aprev), raw + rp * kRawBytes, m - 2 >= m_lo); }
+    if (STAGES && m > m_lo) {
       if constexpr (SLICED) link.wait_for(link_need_bwd(m - 1 - m_lo, p.sl_nbb));
       if (direct) {
-        stage_block<T, 4, CW, true, STAGE_X, NW, true>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
-        bc_widen<SG, NW>(raw + (rp ^ 1) * kRawBytes, lds + (cur ^ 1) * SG::kBytes, wave, lane);
+        stage_block<T, 4, CW, true, STAGE_X, NSTG, true>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, swave, lane, X, DT, DL, DY);
+        bc_widen<SG, NSTG>(raw + (rp ^ 1) * kRawBytes, lds + (cur ^ 1) * SG::kBytes, swave, lane);
       } else {
-        stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+        stage_block<T, 4, CW, true, STAGE_X, NSTG>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, swave, lane, X, DT, DL, DY);
       }
     }
     rp ^= 1;
-    cell_off0 = (uint32_t)(cell0 * p.E + e) * (uint32_t)sizeof(T);
-    f_off0 = (uint32_t)cell0 * (uint32_t)(3 * kN * sizeof(float)) + (BATCH ? (uint32_t)(slot * 4 * sizeof(float)) : f_sub);
+    if constexpr (SWEEPS) cell_off0 = (uint32_t)(cell0 * p.E + e) * (uint32_t)sizeof(T);
+    if constexpr (STAGES) f_off0 = (uint32_t)cell0 * (uint32_t)(3 * kN * sizeof(float)) + (BATCH ? (uint32_t)(slot * 4 * sizeof(float)) : f_sub);
 
     // The 16 states are swept in two halves of 8 (state groups 0,1 then 2,3), each half
     // recomputing and then back-propagating the whole block: only 5 x 8 recomputed states are
@@ -1907,6 +1956,9 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
     float part4[kCK][4];
 #pragma unroll
     for (int half = 0; half < 2; ++half) {
+     if constexpr (!SWEEPS) {   // a wave that only stages: the barriers of a half, and its copies landed before the last one of the block
+      if (BATCH && half == 1) { __syncthreads(); staging_landed(); }
+     } else {
       float hb[kCK + 1][8];
       float gT_last[8], gL_last[8];   // gates of the last step: the adjoint starts with them
       if constexpr (BATCH) lead_if_younger<NW>(wave, true);   // (a barrier interval is a half: until the middle of its adjoint)
@@ -2099,13 +2151,15 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
           }
         }
       }
+     }
       if constexpr (BATCH) {
         // ---- across the waves, all steps of this half at once: the kCK x 3 (step, tensor) sets of
         // sums are dealt to the waves; a thread adds up the float2 of the lane (its slot, its row)
         __syncthreads();
+        if constexpr (STAGES)
 #pragma unroll
-        for (int rd = 0; rd < (kCK * 3 + NW - 1) / NW; ++rd) {
-          const int j = rd * NW + wave;                    // (uniform)
+        for (int rd = 0; rd < (kCK * 3 + NSTG - 1) / NSTG; ++rd) {
+          const int j = rd * NSTG + swave;                 // (uniform)
           if (j < kCK * 3) {
             const int k = j / 3, v = j - 3 * k;
             if ((bp.in_grid >> k) & 1u) {
@@ -2124,18 +2178,27 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd_kernel(const ScanParams pin) 
     // Every wave has waited, before the last adjoint step of this block, for all it had issued: the blocks swept
     // before this one are in memory, and so are the rows this block stored in its steps 3, 2 and 1.  The band above
     // needs, of the newest block it is told about, the steps 3 and 2 only (link_need_bwd), so this block counts.
-    if constexpr (SLICED) link.publish((uint32_t)(m_hi - m));
+    if constexpr (SLICED && STAGES) link.publish((uint32_t)(m_hi - m));
     A = Aprev;
     bp = bpn;
     cell0 = celln;
     cur ^= 1;
   }
+  };
+  if constexpr (NH == 0) sweep(std::integral_constant<int, kAll>{});
+  else if (helper) sweep(std::integral_constant<int, kStager>{});
+  else sweep(std::integral_constant<int, kSweeper>{});
   bool broken = false;
   if constexpr (SLICED) {   // the whole window is done once every store of every wave has completed
     __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
     link.publish((uint32_t)p.sl_nbb);
     broken = link.broken() || link_poll(p.link_err) != 0u;   // (also a workgroup of the forward sweep that rebuilt the snapshots for this launch)
+    if constexpr (NH > 0) {   // only the waves that wait know of a wait given up: they tell the others (the staging buffers are free now)
+      if ((int)threadIdx.x == link.pub) *reinterpret_cast<volatile uint32_t*>(lds) = link.broken() ? 1u : 0u;
+      __syncthreads();
+      broken = broken || *reinterpret_cast<volatile uint32_t*>(lds) != 0u;
+    }
     if (broken) poison_band<T>(p, my_band, b, e_wg0, CW, p.dx, p.ddT, p.ddL);
   }
 
@@ -2180,7 +2243,7 @@ constexpr int bwd2_exchange_sets() {   // sets of [wave][3][64] float2: 2 halves
          2 * (size_t)Stage<T, 4, NW * 4, true>::kBytes + (sizeof(T) == 2 ? 2 * kRawBytes : 0) <= 160 * 1024 ? 4 : 2;
 }
 template <typename T, bool STAGE_X, int MODE, int NW = kBwdWaves>
-__global__ __launch_bounds__(NW * 64) void m2d_bwd2_kernel(const ScanParams pin) {
+__global__ __launch_bounds__((NW + whole_helpers<MODE, NW>()) * 64) void m2d_bwd2_kernel(const ScanParams pin) {
   static_assert(MODE != kModeSliced, "the linked sweep keeps a snapshot every 4 steps");
   constexpr bool STACKED = MODE == kModeStacked;
   ScanParams p = pin;   // (stacked images: the height is shortened below for a last, shorter stack)
@@ -2194,10 +2257,13 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd2_kernel(const ScanParams pin)
   constexpr int SLOT = 3 * 64;           // float2s per wave in one exchange set
   constexpr int CW = NW * CS;
   constexpr bool PERM = true;
+  constexpr int NH = whole_helpers<MODE, NW>();   // waves that only stage and add up the channel sums (then the first NW waves only sweep)
+  constexpr int NSTG = NH ? NH : NW;              // waves that share the copies of a block and the sums of a half-pass
   using SG = Stage<T, 4, CW, true>;
   extern __shared__ float4 smem[];
   constexpr int XSETS = bwd2_exchange_sets<T, NW>();
   constexpr bool BATCH = XSETS == 4;
+  static_assert(NH == 0 || BATCH, "the waves that stage add up the sums of a half-pass in one go");
   float2* slots = reinterpret_cast<float2*>(smem);                       // BATCH: [half][step of the sub-block][wave][3][64], else [2][wave][3][64]
   float* a_lds = reinterpret_cast<float*>(slots + XSETS * NW * SLOT);    // [wave][CS][2][16], fold order
   char* lds = reinterpret_cast<char*>(a_lds + NW * CS * 2 * kN);         // 2 staging buffers
@@ -2217,19 +2283,22 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd2_kernel(const ScanParams pin)
     p.rows_last = p.H - (p.nbands - 1) * p.rb;
   }
   const int e_wg0 = eg * CW;
+  const bool helper = NH && wave >= NW;      // (uniform) stages and adds up, never sweeps
+  const bool stages = !NH || helper;
+  const int swave = NH ? wave - NW : wave;   // the wave's turn among those that stage
   const int slot = lane >> kHBShift, r = lane & (kHB - 1);
   const int rbands = row_bands(p, r);
   const int rk = STACKED ? skew_row(p, r) : r;
-  const int ch_loc = wave * CS + slot;
+  const int ch_loc = (helper ? swave : wave) * CS + slot;
   const int e_raw = e_wg0 + ch_loc;
-  const bool ch_ok = e_raw < p.E;
-  const int e = ch_ok ? e_raw : p.E - 1;
-  {  // A of the wave's channels into LDS in fold order (read back group by group)
+  const bool ch_ok = !helper && e_raw < p.E;
+  const int e = e_raw < p.E ? e_raw : p.E - 1;
+  if (!helper) {  // A of the wave's channels into LDS in fold order (read back group by group)
     float* mine = a_lds + ch_loc * (2 * kN);
     mine[spos<true>(r)] = p.A2T[e * kN + r];
     mine[kN + spos<true>(r)] = p.A2L[e * kN + r];
   }
-  for (int i = threadIdx.x; i < 2 * SG::kBytes / 16; i += NW * 64) reinterpret_cast<float4*>(lds)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+  for (int i = threadIdx.x; i < 2 * SG::kBytes / 16; i += (NW + NH) * 64) reinterpret_cast<float4*>(lds)[i] = make_float4(0.f, 0.f, 0.f, 0.f);
   const uint32_t a_base_off = (uint32_t)(uintptr_t)((__attribute__((address_space(3))) float*)(a_lds + ch_loc * (2 * kN)));
   const float dsk = p.Df[e];
   settle_loads();
@@ -2324,41 +2393,46 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd2_kernel(const ScanParams pin)
   }
   auto raw_copy_for = [&](Pos A2, char* dst, bool live) {
     const BlockPos q2 = block_pos(p, A2, rk, rbands);
-    bc_raw_copy<NW>(p, pin.bcd, dst, b, q2, cell_of(p, q2.bnd0, r, q2.col0), wave, lane, live);
+    bc_raw_copy<NSTG>(p, pin.bcd, dst, b, q2, cell_of(p, q2.bnd0, r, q2.col0), swave, lane, live);
   };
   int rp = 0;
   if (direct) {
-    bc_raw_copy<NW>(p, pin.bcd, raw, b, bp, cell0, wave, lane, true);
-    raw_copy_for(pos_before(A), raw + kRawBytes, m_hi - 2 >= 0);
-    stage_block<T, 4, CW, true, STAGE_X, NW, true>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+    if (stages) bc_raw_copy<NSTG>(p, pin.bcd, raw, b, bp, cell0, swave, lane, true);
+    if (stages) raw_copy_for(pos_before(A), raw + kRawBytes, m_hi - 2 >= 0);
+    if (stages) stage_block<T, 4, CW, true, STAGE_X, NSTG, true>(p, lds, b, A, bp, cell0, e_wg0, swave, lane, X, DT, DL, DY);
     staging_fence();
-    bc_widen<SG, NW>(raw, lds, wave, lane);
+    if (stages) bc_widen<SG, NSTG>(raw, lds, swave, lane);
   } else {
-    stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds, b, A, bp, cell0, e_wg0, wave, lane, X, DT, DL, DY);
+    if (stages) stage_block<T, 4, CW, true, STAGE_X, NSTG>(p, lds, b, A, bp, cell0, e_wg0, swave, lane, X, DT, DL, DY);
   }
   staging_fence();
   int cur = 0;
   int xpar = 0;   // (one set per step: the exchange set in use)
 
+  // The sweep over the blocks, as a wave of the given role runs it (see m2d_fwd_kernel).
+  auto sweep = [&](auto role) {
+  constexpr int ROLE = decltype(role)::value;
+  constexpr bool STAGES = ROLE != kSweeper, SWEEPS = ROLE != kStager;
   for (int m = m_hi - 1; m >= 0; --m) {
     const int t0 = m * kCK;
     const char* bufc = lds + cur * SG::kBytes;
     const Pos Aprev = pos_before(A);
     const BlockPos bpn = block_pos(p, Aprev, rk, rbands);
     const int celln = cell_of(p, bpn.bnd0, r, bpn.col0);
-    const bool take0n = snapshot_lane(p, Pos{bpn.bnd0, bpn.col0}, r, ch_ok), take1n = snapshot_lane(p, pos_at(bpn, 2), r, ch_ok);
-    if (direct) raw_copy_for(pos_before(Aprev), raw + rp * kRawBytes, m - 2 >= 0);
-    if (m > 0) {
+    bool take0n = false, take1n = false;
+    if constexpr (SWEEPS) { take0n = snapshot_lane(p, Pos{bpn.bnd0, bpn.col0}, r, ch_ok); take1n = snapshot_lane(p, pos_at(bpn, 2), r, ch_ok); }
+    if constexpr (STAGES) { if (direct) raw_copy_for(pos_before(Aprev), raw + rp * kRawBytes, m - 2 >= 0); }
+    if (STAGES && m > 0) {
       if (direct) {
-        stage_block<T, 4, CW, true, STAGE_X, NW, true>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
-        bc_widen<SG, NW>(raw + (rp ^ 1) * kRawBytes, lds + (cur ^ 1) * SG::kBytes, wave, lane);
+        stage_block<T, 4, CW, true, STAGE_X, NSTG, true>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, swave, lane, X, DT, DL, DY);
+        bc_widen<SG, NSTG>(raw + (rp ^ 1) * kRawBytes, lds + (cur ^ 1) * SG::kBytes, swave, lane);
       } else {
-        stage_block<T, 4, CW, true, STAGE_X, NW>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, wave, lane, X, DT, DL, DY);
+        stage_block<T, 4, CW, true, STAGE_X, NSTG>(p, lds + (cur ^ 1) * SG::kBytes, b, Aprev, bpn, celln, e_wg0, swave, lane, X, DT, DL, DY);
       }
     }
     rp ^= 1;
-    cell_off0 = (uint32_t)(cell0 * p.E + e) * (uint32_t)sizeof(T);
-    f_off0 = (uint32_t)cell0 * (uint32_t)(3 * kN * sizeof(float)) + (BATCH ? (uint32_t)(slot * 4 * sizeof(float)) : f_sub);
+    if constexpr (SWEEPS) cell_off0 = (uint32_t)(cell0 * p.E + e) * (uint32_t)sizeof(T);
+    if constexpr (STAGES) f_off0 = (uint32_t)cell0 * (uint32_t)(3 * kN * sizeof(float)) + (BATCH ? (uint32_t)(slot * 4 * sizeof(float)) : f_sub);
 
 #pragma unroll
     for (int sub = 1; sub >= 0; --sub) {
@@ -2366,6 +2440,9 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd2_kernel(const ScanParams pin)
       float part2[2][4];   // the state sums of the first half wait here for the second
 #pragma unroll
       for (int half = 0; half < 2; ++half) {
+       if constexpr (!SWEEPS) {   // a wave that only stages: its copies have landed before the barrier that ends the block
+        if (sub == 0 && half == 1) staging_landed();
+       } else {
         float ha[8], hb1[8], hn[8], gT[8], gL[8];
         lead_if_younger<NW>(wave, true);    // (until the second step of the adjoint below)
         widen8(qa[half], ha);
@@ -2541,14 +2618,16 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd2_kernel(const ScanParams pin)
             }
           }
         }
+       }
         if constexpr (BATCH) {
           // ---- across the waves, both steps of this half-pass at once: the 2 x 3 (step, tensor) sets are dealt to the
           // waves; a thread adds up the float2 of the lane (its slot, its row).  The other half's sets are being
           // filled or added up by then; this half's are filled again two barriers from here.
           __syncthreads();
+          if constexpr (STAGES)
 #pragma unroll
-          for (int rd = 0; rd < (2 * 3 + NW - 1) / NW; ++rd) {
-            const int jj = rd * NW + wave;                    // (uniform)
+          for (int rd = 0; rd < (2 * 3 + NSTG - 1) / NSTG; ++rd) {
+            const int jj = rd * NSTG + swave;                 // (uniform)
             if (jj < 2 * 3) {
               const int ks = jj / 3, v = jj - 3 * ks;
               const int k = k0 + ks;
@@ -2572,6 +2651,10 @@ __global__ __launch_bounds__(NW * 64) void m2d_bwd2_kernel(const ScanParams pin)
     cur ^= 1;
     take0 = take0n; take1 = take1n;
   }
+  };
+  if constexpr (NH == 0) sweep(std::integral_constant<int, kAll>{});
+  else if (helper) sweep(std::integral_constant<int, kStager>{});
+  else sweep(std::integral_constant<int, kSweeper>{});
 
   // ---- sums over positions: reduce over the rows of the band (lanes of one channel slot)
   float red[2 * kN + 1];
@@ -3307,7 +3390,11 @@ Geometry make_geometry(const m2d_desc* d) {
   // than three for every four SIMDs.  Then a wave per channel, each with a quarter of the states.
   const int64_t waves_whole = (int64_t)B * ((d->E + g.CS - 1) / g.CS) * together;
   const bool may_split = !g.stacked && !(d->flags & M2D_FLAG_WHOLE_STATES) && g.ck_shift == 0;
-  g.fwd_split = may_split && ((d->flags & M2D_FLAG_SPLIT_STATES) || waves_whole <= 3 * ncu);
+  // One stream per image: only while the workgroups of 8 channels all run at once.  The backward has a compute unit to
+  // itself, so one workgroup more than units is a second round of them, and the whole-state kernels in workgroups of 4
+  // waves are then ahead (B=33..48 at 56x56x64 bf16: forward+backward kernels 0.85 -> 0.76 ms; B=32: 0.48 against 0.76).
+  const bool few_enough = waves_whole <= 3 * ncu && (g.sliced || (int64_t)B * ((d->E + kSplitWaves - 1) / kSplitWaves) <= ncu);
+  g.fwd_split = may_split && ((d->flags & M2D_FLAG_SPLIT_STATES) || few_enough);
   // Workgroups of 8 waves (8 channels) under way on at most half of the compute units: workgroups of 4 then run on
   // twice as many, each wave with a SIMD to itself (a sweep of few images is as fast as one wave gets through its
   // blocks).
@@ -3330,7 +3417,7 @@ Geometry make_geometry(const m2d_desc* d) {
   // (the backward keeps one set of channel sums per workgroup of an image: with 8 channels per workgroup
   // that memory is bounded here unless the caller insists)
   const size_t split_part = sizeof(float) * (size_t)((d->E + split_nw - 1) / split_nw) * 3 * kN * (size_t)d->B * d->H * d->W;
-  g.bwd_split = may_split && ((d->flags & M2D_FLAG_SPLIT_STATES) || (waves_whole <= 3 * ncu && split_part <= ((size_t)2 << 30)));
+  g.bwd_split = may_split && ((d->flags & M2D_FLAG_SPLIT_STATES) || (few_enough && split_part <= ((size_t)2 << 30)));
   if (g.bwd_split) {
     g.bwd_nw = split_nw;
     g.bwd_bpb = (d->E + split_nw - 1) / split_nw;
@@ -3448,10 +3535,10 @@ int stage_bc(ScanParams& sp, const m2d_desc* d, const void* BT, const void* BL, 
 // Development aid: -DM2D_QUICK=1 builds only the kernels of many 16-bit images in one stream each, in workgroups of
 // 8 waves (a twentieth of the compile time), -DM2D_QUICK=2 (3) only the linked sweep of fp32 (16-bit) images in workgroups of 4 waves;
 // every other problem then answers M2D_ERR_UNSUPPORTED.
-#if defined(M2D_QUICK) && M2D_QUICK >= 2
+#if defined(M2D_QUICK) && M2D_QUICK >= 2 && M2D_QUICK <= 3
 #define M2D_BUILT(T, SX, MODE, NW, OTHER) (sizeof(T) == (M2D_QUICK == 3 ? 2 : 4) && (MODE) == kModeSliced && (NW) == 4)
 #elif defined(M2D_QUICK)
-#define M2D_BUILT(T, SX, MODE, NW, OTHER) (sizeof(T) == 2 && (SX) && (MODE) == kModeSweep && (NW) == 8 && (OTHER))
+#define M2D_BUILT(T, SX, MODE, NW, OTHER) (sizeof(T) == 2 && (SX) && (MODE) == kModeSweep && (NW) == (M2D_QUICK == 1 ? 8 : 4) && (OTHER))
 #else
 #define M2D_BUILT(T, SX, MODE, NW, OTHER) true
 #endif
@@ -3463,7 +3550,7 @@ int launch_fwd_as(const ScanParams& sp, hipStream_t st) {
   if (lds > kLdsPerWorkgroup) return M2D_ERR_UNSUPPORTED;   // (make_geometry never picks such a layout)
   static std::atomic<uint64_t> seen{0};
   if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_fwd_kernel<T, EC, CK, WY, SX, MODE, NW, HALF>), lds, seen)) return M2D_ERR_HIP;
-  hipLaunchKernelGGL((m2d_fwd_kernel<T, EC, CK, WY, SX, MODE, NW, HALF>), dim3((unsigned)sp.nwg), dim3(NW * 64), lds, st, sp);
+  hipLaunchKernelGGL((m2d_fwd_kernel<T, EC, CK, WY, SX, MODE, NW, HALF>), dim3((unsigned)sp.nwg), dim3((NW + whole_helpers<MODE, NW, EC>()) * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
   }
 }
@@ -3585,7 +3672,7 @@ int launch_bwd_as(const ScanParams& sp, hipStream_t st) {
   constexpr size_t lds = bwd_lds_bytes<T, NW>();
   static std::atomic<uint64_t> seen{0};
   if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_bwd_kernel<T, SX, MODE, NW, REPLAY>), lds, seen)) return M2D_ERR_HIP;
-  hipLaunchKernelGGL((m2d_bwd_kernel<T, SX, MODE, NW, REPLAY>), dim3((unsigned)sp.nwg), dim3(NW * 64), lds, st, sp);
+  hipLaunchKernelGGL((m2d_bwd_kernel<T, SX, MODE, NW, REPLAY>), dim3((unsigned)sp.nwg), dim3((NW + (REPLAY ? 0 : whole_helpers<MODE, NW>())) * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
   }
 }
@@ -3602,7 +3689,7 @@ int launch_bwd2_as(const ScanParams& sp, hipStream_t st) {
   static_assert(lds <= kLdsPerWorkgroup, "exchange sets and staging must fit the LDS");
   static std::atomic<uint64_t> seen{0};
   if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_bwd2_kernel<T, SX, MODE, NW>), lds, seen)) return M2D_ERR_HIP;
-  hipLaunchKernelGGL((m2d_bwd2_kernel<T, SX, MODE, NW>), dim3((unsigned)sp.nwg), dim3(NW * 64), lds, st, sp);
+  hipLaunchKernelGGL((m2d_bwd2_kernel<T, SX, MODE, NW>), dim3((unsigned)sp.nwg), dim3((NW + whole_helpers<MODE, NW>()) * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
   }
 }
@@ -3833,10 +3920,15 @@ int m2d_scan_plan(const m2d_desc* desc, int pass, char* text, size_t cap) {
     snprintf(text, cap, "%s: %s, %lld workgroups of %d waves%s, %d channels each, 4 states per lane",
              fwd ? "m2d_fwd_split_kernel" : "m2d_bwd_split_kernel", sched, wgs, nw, extra, nw);
   }
-  else
-    snprintf(text, cap, "%s: %s, %lld workgroups of %d waves, %d channels each, 16 states per lane%s",
-             fwd ? "m2d_fwd_kernel" : (g.ck_half ? "m2d_bwd2_kernel" : "m2d_bwd_kernel"), sched, wgs, nw, nw * g.CS * per_lane,
+  else {
+    // (workgroups of 4 waves have waves that only stage, except in the backward that replays the forward between snapshots)
+    const bool helped = !g.stacked && nw == kFwdHalfWaves && per_lane == 1 && (fwd || g.ck_shift == 0);
+    char extra[48] = "";
+    if (helped) snprintf(extra, sizeof extra, " and %d that stage", kWholeHelpers);
+    snprintf(text, cap, "%s: %s, %lld workgroups of %d waves%s, %d channels each, 16 states per lane%s",
+             fwd ? "m2d_fwd_kernel" : (g.ck_half ? "m2d_bwd2_kernel" : "m2d_bwd_kernel"), sched, wgs, nw, extra, nw * g.CS * per_lane,
              g.ck_half ? (fwd ? ", a snapshot every 2 steps" : ", a snapshot every 2 steps and one step in two recomputed") : "");
+  }
   if (g.ck_shift) {
     const size_t n = strlen(text);
     if (n + 1 < cap) snprintf(text + n, cap - n, fwd ? ", a snapshot every %d steps" : ", a snapshot every %d steps and the forward replayed in between", kCK << g.ck_shift);
