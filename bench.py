@@ -35,6 +35,7 @@ WORKLOADS = {
     "hires1024": (1, 64, 1024, 1024, "f32"),
     "hires2048": (1, 64, 2048, 2048, "f32"),
     "cfg0": (2, 32, 14, 14, "f32"),
+    "train64": (64, 64, 56, 56, "bf16"),   # the reference's training batch per GPU (configs/M2D-T-ImageNet.yaml) at the stage-1 shape
     "cfg3": None,   # M2D-T backbone inference, handled by backbone_inference()
     "entry": None,  # wavefront_scan_cuda (projections + scan) at the cfg1 shape, handled by entry_point()
     "cfg2": None,   # the four M2D-T stage scans in sequence, handled by stage_sequence()
@@ -454,7 +455,8 @@ def _short_scan(name, steps, warmup):
 def also_workloads(args, rates, cfg1_fwd_bwd_ms):
     """Short measurements of the other configurations in the same process, after the timed region of the headline
     workload: the four stage scans in sequence (cfg2), one image of 256x256 and of 2048x2048 (cfg4, with the
-    allocator's peak), and the entry point wavefront_scan_cuda with its projections at the headline shape."""
+    allocator's peak), the stage-1 scan at the reference's training batch of 64, and the entry point
+    wavefront_scan_cuda with its projections at the headline shape."""
     import math
     import torch
     from mamba2d_amd import wavefront as wf
@@ -464,6 +466,7 @@ def also_workloads(args, rates, cfg1_fwd_bwd_ms):
     # steps is what `--workload cfg2` times as one step)
     out["cfg2"] = {"fwd_bwd_ms": round(cfg1_fwd_bwd_ms + sum(v["fwd_bwd_ms"] for v in stages.values()), 4), "stages": stages}
     out["cfg4_256"] = _short_scan("hires256", 10, 3)
+    out["train64"] = _short_scan("train64", 10, 3)   # (not a configuration of the baseline: the batch the reference trains with)
     free, _ = torch.cuda.mem_get_info()
     if free > 40 * 2**30:
         out["cfg4_2048"] = _short_scan("hires2048", 3, 1)
