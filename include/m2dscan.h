@@ -123,6 +123,13 @@ typedef struct m2d_desc {
  * it), and leaves d_BL and d_C alone (they may be NULL).  The records are only meaningful to this library. */
 #define M2D_FLAG_SUM_PARTS 256
 
+/* bf16 tensors keep their state snapshots rounded to bf16 (the reference keeps every state of its hidden-state tensor
+ * in the tensors' type); with this flag m2d_scan_fwd keeps them in fp32 and m2d_scan_bwd reads them so: twice the
+ * checkpoint bytes of an interval of 4 steps, which the flag implies (ckpt_interval 0 or 4; others are refused), and
+ * the whole-state kernels in workgroups of 4 sweeping waves, which is slower wherever another plan would have been
+ * chosen.  Both passes of a problem must agree on it.  No effect on fp32 tensors. */
+#define M2D_FLAG_FP32_SNAPSHOTS 512
+
 #define M2D_PASS_FWD 0
 #define M2D_PASS_BWD 1
 

@@ -44,7 +44,7 @@ SOURCES = {
 # 8 waves in its replaying form (m2d_bwd_kernel<..., 8, true>: a checkpoint interval of 8 or 16 steps, not the
 # default): the same sweep as the default kernel, which fills all 256 registers, plus the addresses of the replay.
 # It reloads two to nine values a few times per block of steps; every other kernel must not spill at all.
-SPILL_ALLOWANCE = [(re.compile(r"m2d_bwd_kernelI\w*Li8ELb1EEEv"), 64)]
+SPILL_ALLOWANCE = [(re.compile(r"m2d_bwd_kernelI\w*Li8ELb1E\w*EEv"), 64)]   # (<..., 8 waves, REPLAY = true, snapshot type>)
 
 # A kernel that runs out of scalar registers parks some in lanes of a vector register; the compiler then reserves a
 # few bytes of scratch for that register without ever storing it.  Allowed up to this many bytes per lane, and only

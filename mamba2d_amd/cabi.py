@@ -23,6 +23,7 @@ M2D_FLAG_SPLIT_STATES = 32
 M2D_FLAG_WHOLE_STATES = 64
 M2D_FLAG_TEST_DEAD_LINK = 128
 M2D_FLAG_SUM_PARTS = 256
+M2D_FLAG_FP32_SNAPSHOTS = 512
 M2D_PASS_FWD, M2D_PASS_BWD = 0, 1
 
 EXPORTS = ("m2d_version", "m2d_status_str", "m2d_desc_check", "m2d_scan_workspace_bytes",

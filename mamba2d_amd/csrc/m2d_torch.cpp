@@ -37,9 +37,11 @@ m2d_desc describe(const Tensor& x, const Tensor& AT, bool flip, bool raw_params 
   else TORCH_CHECK(false, "m2dscan: float32 and bfloat16 are supported, got ", x.scalar_type());
   d.flags = (flip ? M2D_FLAG_FLIP : 0) | (raw_params ? M2D_FLAG_RAW_PARAMS : 0) | (packed_bc ? M2D_FLAG_PACKED_BC : 0) |
             (dpre ? M2D_FLAG_DPRE : 0);
-  TORCH_CHECK(ckpt_interval == 0 || ckpt_interval == 2 || ckpt_interval == 4 || ckpt_interval == 8 || ckpt_interval == 16,
-              "m2dscan: ckpt_interval must be 0, 2, 4, 8 or 16, got ", ckpt_interval);
-  d.ckpt_interval = static_cast<int32_t>(ckpt_interval);
+  // (-4: a snapshot every 4 steps, kept in fp32 also for bf16 tensors, M2D_FLAG_FP32_SNAPSHOTS)
+  TORCH_CHECK(ckpt_interval == 0 || ckpt_interval == 2 || ckpt_interval == 4 || ckpt_interval == 8 || ckpt_interval == 16 || ckpt_interval == -4,
+              "m2dscan: ckpt_interval must be 0, 2, 4, 8 or 16 (or -4: every 4 steps, in fp32), got ", ckpt_interval);
+  if (ckpt_interval == -4) d.flags |= M2D_FLAG_FP32_SNAPSHOTS;
+  d.ckpt_interval = static_cast<int32_t>(ckpt_interval == -4 ? 4 : ckpt_interval);
   return d;
 }
 

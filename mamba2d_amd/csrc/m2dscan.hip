@@ -861,7 +861,8 @@ constexpr int kAll = 0, kSweeper = 1, kStager = 2;   // what a wave does: both, 
 constexpr int kWholeHelpers = 4;
 template <int MODE, int NW, int EC = 1>
 constexpr int whole_helpers() { return (MODE != kModeStacked && NW == kFwdHalfWaves && EC == 1) ? kWholeHelpers : 0; }
-template <typename T, int EC, bool CKPT, bool WRITE_Y, bool STAGE_X, int MODE, int NW = kFwdWaves, bool HALF = false>
+// ST: the type the snapshots are kept in (T; float for bf16 tensors where the caller asks for fp32 snapshots).
+template <typename T, int EC, bool CKPT, bool WRITE_Y, bool STAGE_X, int MODE, int NW = kFwdWaves, bool HALF = false, typename ST = T>
 __global__ __launch_bounds__((NW + whole_helpers<MODE, NW, EC>()) * 64) void m2d_fwd_kernel(const ScanParams pin) {
   constexpr bool SLICED = MODE == kModeSliced, STACKED = MODE == kModeStacked;
   static_assert(!HALF || (CKPT && !SLICED), "snapshots every 2 steps: kept by a forward of one stream per image or stack");
@@ -1026,8 +1027,8 @@ __global__ __launch_bounds__((NW + whole_helpers<MODE, NW, EC>()) * 64) void m2d
   for (int c = 0; c < EC; ++c)
 #pragma unroll
     for (int n = 0; n < kN; ++n) h[c][n] = 0.f;
-  typename Snap<T>::quad* ckp = nullptr;      // where the lane stores its snapshot in the first step of the current block
-  typename Snap<T>::quad* ckp2 = nullptr;     // ... and (HALF) in its third step
+  typename Snap<ST>::quad* ckp = nullptr;      // where the lane stores its snapshot in the first step of the current block
+  typename Snap<ST>::quad* ckp2 = nullptr;     // ... and (HALF) in its third step
   int ypar = 0;                 // window that the current block fills
   const uint32_t y_lane_off = (uint32_t)(wave * YT::kRegion + (r * CS + slot) * EC * (int)sizeof(T));
   auto step = [&](int k, const Ops& o) {
@@ -1039,7 +1040,7 @@ __global__ __launch_bounds__((NW + whole_helpers<MODE, NW, EC>()) * 64) void m2d
       const float sT = __builtin_fmaf(cT * o.dtv[c], o.xv[c], g1);
       const float sL = cL * o.dlv[c] * o.xv[c];
       float acc = 0.f;
-      typename Snap<T>::quad pend = Snap<T>::zero();   // a quad that waits for its neighbour (16-bit snapshots: two bf16 quads leave as one 16-byte store)
+      typename Snap<ST>::quad pend = Snap<ST>::zero();   // a quad that waits for its neighbour (16-bit snapshots: two bf16 quads leave as one 16-byte store)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const float4 b4 = o.bt[c][q], l4 = o.bl[q], c4 = o.cc[q];
@@ -1058,9 +1059,9 @@ __global__ __launch_bounds__((NW + whole_helpers<MODE, NW, EC>()) * 64) void m2d
         pin4(aL);
         __builtin_amdgcn_sched_barrier(0);
         if (CKPT && (k == 0 || (HALF && k == 2))) {   // the four states as they are before this step: stored with their neighbours' quad
-          const typename Snap<T>::quad pk = Snap<T>::pack(h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)], h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
+          const typename Snap<ST>::quad pk = Snap<ST>::pack(h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)], h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]);
           if ((q & 1) == 0) pend = pk;
-          else Snap<T>::store2((k == 0 ? ckp : ckp2) + c * (kN / 4 * kHB) + snap_quad(q - 1), pend, pk);
+          else Snap<ST>::store2((k == 0 ? ckp : ckp2) + c * (kN / 4 * kHB) + snap_quad(q - 1), pend, pk);
         }
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
@@ -1206,11 +1207,11 @@ __global__ __launch_bounds__((NW + whole_helpers<MODE, NW, EC>()) * 64) void m2d
     // another channel's, and blocks whose snapshot is not kept (block 0; a longer checkpoint
     // interval) write to the image's place for block 0, which nobody reads.
     if constexpr (CKPT && HALF) {   // snapshots 2m and 2m + 1 (snapshot 0, the state before the sweep, is the place nobody reads)
-      ckp = snapshot_at<T>(p, b, (m > 0 && ch_ok) ? 2 * m : 0, e0, p.ck_nblk) + snap_lane(r);
-      ckp2 = snapshot_at<T>(p, b, ch_ok ? 2 * m + 1 : 0, e0, p.ck_nblk) + snap_lane(r);
+      ckp = snapshot_at<ST>(p, b, (m > 0 && ch_ok) ? 2 * m : 0, e0, p.ck_nblk) + snap_lane(r);
+      ckp2 = snapshot_at<ST>(p, b, ch_ok ? 2 * m + 1 : 0, e0, p.ck_nblk) + snap_lane(r);
     } else if constexpr (CKPT) {
       const bool keep = m > 0 && snapshot_kept(p, m, m_lo);
-      ckp = snapshot_at<T>(p, b, (keep && ch_ok) ? snapshot_index<SLICED>(p, m, m_lo, my_band) : 0, e0, p.ck_nblk) + snap_lane(r);
+      ckp = snapshot_at<ST>(p, b, (keep && ch_ok) ? snapshot_index<SLICED>(p, m, m_lo, my_band) : 0, e0, p.ck_nblk) + snap_lane(r);
     }
     const char* bufc = lds + cur * SG::kBytes;
     const char* bufn = lds + (cur ^ 1) * SG::kBytes;
@@ -1236,7 +1237,7 @@ __global__ __launch_bounds__((NW + whole_helpers<MODE, NW, EC>()) * 64) void m2d
       } else if constexpr (CKPT) {
         // snapshot stores of the steps before the last: per channel and snapshot two 16-byte pieces of bf16 quads or four fp32 quads
         // (counting too few only waits longer, too many reads operands that have not landed; the wait's field counts to 15)
-        constexpr int kSnaps = (HALF ? 2 : 1) * EC * (sizeof(T) == 2 ? 2 : 4);
+        constexpr int kSnaps = (HALF ? 2 : 1) * EC * (sizeof(ST) == 2 ? 2 : 4);
         if (y_thrice) staging_landed_behind<(kSnaps + 3 < 15 ? kSnaps + 3 : 15)>(); else staging_landed_behind<(kSnaps < 15 ? kSnaps : 15)>();
       } else {
         if (y_thrice) staging_landed_behind<3>(); else staging_landed();
@@ -1296,14 +1297,14 @@ __global__ __launch_bounds__((NW + whole_helpers<MODE, NW, EC>()) * 64) void m2d
     if (stages) flush_y(ypar, m_hi, true);
   }
   if constexpr (CKPT && HALF) if (!helper) {   // the state behind the last block: what the last step of the sweep left is among it
-    typename Snap<T>::quad* end = snapshot_at<T>(p, b, ch_ok ? 2 * p.nblk : 0, e0, p.ck_nblk) + snap_lane(r);
+    typename Snap<ST>::quad* end = snapshot_at<ST>(p, b, ch_ok ? 2 * p.nblk : 0, e0, p.ck_nblk) + snap_lane(r);
 #pragma unroll
     for (int c = 0; c < EC; ++c)
 #pragma unroll
       for (int q = 0; q < 4; q += 2)
-        Snap<T>::store2(end + c * (kN / 4 * kHB) + snap_quad(q),
-                        Snap<T>::pack(h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)], h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]),
-                        Snap<T>::pack(h[c][sinv<PERM>(4 * q + 4)], h[c][sinv<PERM>(4 * q + 5)], h[c][sinv<PERM>(4 * q + 6)], h[c][sinv<PERM>(4 * q + 7)]));
+        Snap<ST>::store2(end + c * (kN / 4 * kHB) + snap_quad(q),
+                        Snap<ST>::pack(h[c][sinv<PERM>(4 * q)], h[c][sinv<PERM>(4 * q + 1)], h[c][sinv<PERM>(4 * q + 2)], h[c][sinv<PERM>(4 * q + 3)]),
+                        Snap<ST>::pack(h[c][sinv<PERM>(4 * q + 4)], h[c][sinv<PERM>(4 * q + 5)], h[c][sinv<PERM>(4 * q + 6)], h[c][sinv<PERM>(4 * q + 7)]));
   }
   if constexpr (SLICED) {   // the whole window is done once every store of every wave has completed
     __builtin_amdgcn_s_waitcnt(0x0F70);
@@ -1628,7 +1629,7 @@ constexpr int bwd_exchange_sets() {
 // group's other blocks from that snapshot, one block at a time through the idle staging buffer, and the state
 // before each block is parked in the workgroup's ring in memory, where the sweep then finds it like a snapshot.
 // A lane reads back only what it wrote itself.
-template <typename T, bool STAGE_X, int MODE, int NW = kBwdWaves, bool REPLAY = false>
+template <typename T, bool STAGE_X, int MODE, int NW = kBwdWaves, bool REPLAY = false, typename ST = T>
 __global__ __launch_bounds__((NW + (REPLAY ? 0 : whole_helpers<MODE, NW>())) * 64) void m2d_bwd_kernel(const ScanParams pin) {
   constexpr bool SLICED = MODE == kModeSliced, STACKED = MODE == kModeStacked;
   ScanParams p = pin;   // (stacked images: the height is shortened below for a last, shorter stack)
@@ -1766,7 +1767,7 @@ __global__ __launch_bounds__((NW + (REPLAY ? 0 : whole_helpers<MODE, NW>())) * 6
   uint32_t f_off0 = 0;          // byte offset in the channel-sum image of this thread's sum at the first step
   // state snapshot at the start of the block whose position A is given (zero for lanes that were not under way)
   // (kept as it comes from memory until the block starts: nothing waits for the loads before then)
-  typename Snap<T>::quad cknext[4];
+  typename Snap<ST>::quad cknext[4];
   // The replaying kernel of 8 waves (256 registers per lane) fetches the snapshot of a block when the block starts,
   // not during the block before: the registers that would hold it meanwhile are what the kernel lacks, and waiting
   // for the fetch costs less than spilling in the sweep (B=128, E=64, 56x56, interval 8: 1.05 against 1.10 ms).
@@ -1780,12 +1781,12 @@ __global__ __launch_bounds__((NW + (REPLAY ? 0 : whole_helpers<MODE, NW>())) * 6
   // past E point at the last channel's place: they park nothing and use nothing).
   auto snapshot_of_lane = [&](int mm) {
     if constexpr (!REPLAY) {   // the default interval: a snapshot for every block, as before
-      return snapshot_at<T>(p, b, mm, e, p.nblk) + snap_lane(r);
+      return snapshot_at<ST>(p, b, mm, e, p.nblk) + snap_lane(r);
     } else {
       const int mem = member(mm);
-      typename Snap<T>::quad* base =
-          mem != 0 ? static_cast<typename Snap<T>::quad*>(p.ring) + ((int64_t)blockIdx.x * ((1 << p.ck_shift) - 1) + (mem - 1)) * kRingSlot - e_wg0 * (kN / 4 * kHB)
-                   : snapshot_at<T>(p, b, snapshot_index<SLICED>(p, mm, m_lo, my_band), 0, p.ck_nblk);
+      typename Snap<ST>::quad* base =
+          mem != 0 ? static_cast<typename Snap<ST>::quad*>(p.ring) + ((int64_t)blockIdx.x * ((1 << p.ck_shift) - 1) + (mem - 1)) * kRingSlot - e_wg0 * (kN / 4 * kHB)
+                   : snapshot_at<ST>(p, b, snapshot_index<SLICED>(p, mm, m_lo, my_band), 0, p.ck_nblk);
       return base + (e * (kN / 4 * kHB) + snap_lane(r));
     }
   };
@@ -1794,11 +1795,11 @@ __global__ __launch_bounds__((NW + (REPLAY ? 0 : whole_helpers<MODE, NW>())) * 6
   auto load_ckpt = [&](int mm, bool take) {   // take: the forward kept the lane's state before block mm
     if (mm == 0 || !take) {
 #pragma unroll
-      for (int q = 0; q < 4; ++q) cknext[q] = Snap<T>::zero();
+      for (int q = 0; q < 4; ++q) cknext[q] = Snap<ST>::zero();
     } else {
-      const typename Snap<T>::quad* ck = snapshot_of_lane(mm);
+      const typename Snap<ST>::quad* ck = snapshot_of_lane(mm);
 #pragma unroll
-      for (int q = 0; q < 4; q += 2) Snap<T>::load2(ck + snap_quad(q), *reinterpret_cast<typename Snap<T>::quad(*)[2]>(&cknext[q]));
+      for (int q = 0; q < 4; q += 2) Snap<ST>::load2(ck + snap_quad(q), *reinterpret_cast<typename Snap<ST>::quad(*)[2]>(&cknext[q]));
     }
   };
   auto pos_before = [&](Pos Q) {   // kCK positions earlier
@@ -1865,10 +1866,10 @@ __global__ __launch_bounds__((NW + (REPLAY ? 0 : whole_helpers<MODE, NW>())) * 6
           // the block before left, and zero in both cases for a lane that was not under way (see snapshot_lane)
           const bool take_q = q != 0 && snapshot_lane(p, Pos{bq.bnd0, bq.col0}, r, ch_ok);
           if (q == m - mem) {
-            const typename Snap<T>::quad* ck = snapshot_of_lane(q);
+            const typename Snap<ST>::quad* ck = snapshot_of_lane(q);
 #pragma unroll
             for (int mg = 0; mg < 4; ++mg) {
-              const float4 v = take_q ? Snap<T>::load(ck + snap_quad(mg)) : make_float4(0.f, 0.f, 0.f, 0.f);
+              const float4 v = take_q ? Snap<ST>::load(ck + snap_quad(mg)) : make_float4(0.f, 0.f, 0.f, 0.f);
               hq[4 * mg + 0] = v.x; hq[4 * mg + 1] = v.y; hq[4 * mg + 2] = v.z; hq[4 * mg + 3] = v.w;
             }
           } else {
@@ -1921,10 +1922,10 @@ __global__ __launch_bounds__((NW + (REPLAY ? 0 : whole_helpers<MODE, NW>())) * 6
               }
             }
           }
-          typename Snap<T>::quad* park = snapshot_of_lane(q + 1);   // the states before block q + 1
+          typename Snap<ST>::quad* park = snapshot_of_lane(q + 1);   // the states before block q + 1
 #pragma unroll
           for (int mg = 0; mg < 4; ++mg)
-            if (ch_ok) park[snap_quad(mg)] = Snap<T>::pack(hq[4 * mg], hq[4 * mg + 1], hq[4 * mg + 2], hq[4 * mg + 3]);   // (channels past E have no place of their own)
+            if (ch_ok) park[snap_quad(mg)] = Snap<ST>::pack(hq[4 * mg], hq[4 * mg + 1], hq[4 * mg + 2], hq[4 * mg + 3]);   // (channels past E have no place of their own)
           __syncthreads();   // every wave is done with the buffer before the next block's copies land in it
         }
         if constexpr (!LATE_SNAPSHOT) load_ckpt(m, ck_take);
@@ -1967,7 +1968,7 @@ __global__ __launch_bounds__((NW + (REPLAY ? 0 : whole_helpers<MODE, NW>())) * 6
       static_assert(sinv<PERM>(4 * 2 + 1) == fold_state(2, 1) && sinv<PERM>(4 * 3 + 2) == fold_state(3, 2), "snapshot quads are state groups");
 #pragma unroll
       for (int mgl = 0; mgl < 2; ++mgl) {
-        const float4 v = Snap<T>::widen(cknext[2 * half + mgl]);
+        const float4 v = Snap<ST>::widen(cknext[2 * half + mgl]);
         hb[0][4 * mgl + 0] = v.x; hb[0][4 * mgl + 1] = v.y; hb[0][4 * mgl + 2] = v.z; hb[0][4 * mgl + 3] = v.w;
 #pragma unroll
         for (int qi = 0; qi < 4; ++qi) { gT_last[4 * mgl + qi] = 0.f; gL_last[4 * mgl + qi] = 0.f; }
@@ -3252,6 +3253,7 @@ struct Geometry {
   size_t link_bytes;                 // linked sweep: error word and the two arrays of progress counts (forward, backward)
   int ck_shift, ck_pb, ck_nblk;      // checkpoint interval: log2 of the blocks per kept snapshot; kept snapshots per band (linked sweep) and per image
   bool ck_half;                      // a snapshot every 2 steps: m2d_fwd_kernel<..., HALF> and m2d_bwd2_kernel
+  bool snap32;                       // bf16 tensors with fp32 snapshots (M2D_FLAG_FP32_SNAPSHOTS)
   size_t ring_bytes;                 // backward with a longer interval: the replayed snapshots of every workgroup
   bool packed_bc;
   size_t prep_bytes, bc_bytes, ckpt_diag_bytes, top_bytes, bot_bytes, part_bytes, pa_bytes, pd_bytes;
@@ -3262,7 +3264,8 @@ int check_desc(const m2d_desc* d) {
   if (d->B < 1 || d->E < 1 || d->N < 1 || d->H < 2 || d->W < 2) return M2D_ERR_BAD_SHAPE;
   if (d->N != kN) return M2D_ERR_UNSUPPORTED;
   if (d->dtype != M2D_F32 && d->dtype != M2D_BF16) return M2D_ERR_UNSUPPORTED;
-  if ((d->ckpt_interval != 0 && d->ckpt_interval != 2 && d->ckpt_interval != 4 && d->ckpt_interval != 8 && d->ckpt_interval != 16) || (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_RAW_PARAMS | M2D_FLAG_PACKED_BC | M2D_FLAG_DPRE | M2D_FLAG_SPLIT_STATES | M2D_FLAG_WHOLE_STATES | M2D_FLAG_TEST_DEAD_LINK | M2D_FLAG_SUM_PARTS))) return M2D_ERR_UNSUPPORTED;
+  if ((d->ckpt_interval != 0 && d->ckpt_interval != 2 && d->ckpt_interval != 4 && d->ckpt_interval != 8 && d->ckpt_interval != 16) || (d->flags & ~(M2D_FLAG_FLIP | M2D_FLAG_RAW_PARAMS | M2D_FLAG_PACKED_BC | M2D_FLAG_DPRE | M2D_FLAG_SPLIT_STATES | M2D_FLAG_WHOLE_STATES | M2D_FLAG_TEST_DEAD_LINK | M2D_FLAG_SUM_PARTS | M2D_FLAG_FP32_SNAPSHOTS))) return M2D_ERR_UNSUPPORTED;
+  if ((d->flags & M2D_FLAG_FP32_SNAPSHOTS) && d->dtype == M2D_BF16 && (d->ckpt_interval == 2 || d->ckpt_interval == 8 || d->ckpt_interval == 16)) return M2D_ERR_UNSUPPORTED;   // (fp32 snapshots: every 4 steps)
   if ((d->flags & M2D_FLAG_SPLIT_STATES) && (d->flags & M2D_FLAG_WHOLE_STATES)) return M2D_ERR_UNSUPPORTED;
   if ((int64_t)d->B * d->H * d->W >= ((int64_t)1 << 40)) return M2D_ERR_BAD_SHAPE;
   // one image is addressed with 32-bit byte offsets from its base (fp32: 4 bytes per element;
@@ -3306,7 +3309,10 @@ Geometry make_geometry(const m2d_desc* d) {
   // (a longer checkpoint interval is for grids whose snapshots weigh: images are not stacked then, nor are the states
   // of a channel split over lanes, and every schedule left runs m2d_bwd_kernel, the one kernel that replays)
   g.ck_shift = d->ckpt_interval == 16 ? 2 : (d->ckpt_interval == 8 ? 1 : 0);
-  if (d->H <= kHB && d->B >= 2 && g.ck_shift == 0) {
+  // bf16 tensors with fp32 snapshots: a snapshot every 4 steps, the whole-state kernels in workgroups of 4 sweeping
+  // waves (the only ones with registers to spare for quads twice as wide), one stream per image or the linked sweep
+  g.snap32 = (d->flags & M2D_FLAG_FP32_SNAPSHOTS) && d->dtype == M2D_BF16;
+  if (d->H <= kHB && d->B >= 2 && g.ck_shift == 0 && !g.snap32) {
     const int S = d->W > 7 ? d->W : 7;
     int64_t best = -1;
     for (int ips = 1; ips <= 64 && ips <= d->B; ++ips) {
@@ -3423,6 +3429,13 @@ Geometry make_geometry(const m2d_desc* d) {
     g.bwd_bpb = (d->E + split_nw - 1) / split_nw;
     g.bwd_wpb = g.bwd_bpb * g.bwd_nw;
   }
+  if (g.snap32) {
+    g.fwd_split = g.bwd_split = false;
+    g.fwd_ec = 1;
+    g.fwd_nw = g.bwd_nw = kFwdHalfWaves;
+    g.fwd_bpb = g.bwd_bpb = (d->E + kFwdHalfWaves * g.CS - 1) / (kFwdHalfWaves * g.CS);
+    g.fwd_wpb = g.bwd_wpb = g.fwd_bpb * kFwdHalfWaves;
+  }
   g.stage_x = (d->E % (d->dtype == M2D_BF16 ? 8 : 4)) == 0;
   const size_t P = (size_t)d->B * d->H * d->W;
   g.prep_bytes = align_up(sizeof(float) * (kZeroFloats + (size_t)2 * d->E * kN + d->E));
@@ -3434,9 +3447,9 @@ Geometry make_geometry(const m2d_desc* d) {
   g.ck_nblk = g.sliced ? g.nbands * g.ck_pb : (g.nblk + every - 1) / every;
   // A snapshot every 2 steps, for the backward kernel that recomputes one step in two: where every image (or stack)
   // is one stream and a lane holds all states of its channel.  Other schedules keep one every 4 steps.
-  g.ck_half = (d->ckpt_interval == 2 || d->ckpt_interval == 0) && !g.sliced && !g.fwd_split && !g.bwd_split;
+  g.ck_half = (d->ckpt_interval == 2 || d->ckpt_interval == 0) && !g.sliced && !g.fwd_split && !g.bwd_split && !g.snap32;
   if (g.ck_half) g.ck_nblk = 2 * g.nblk + 1;   // before the steps 0 and 2 of every block, and behind the last block
-  g.ckpt_diag_bytes = align_up((d->dtype == M2D_BF16 ? 2 : sizeof(float)) * (size_t)B * g.ck_nblk * d->E * kN * g.HB);   // (16-bit tensors: bf16 snapshots)
+  g.ckpt_diag_bytes = align_up((d->dtype == M2D_BF16 && !g.snap32 ? 2 : sizeof(float)) * (size_t)B * g.ck_nblk * d->E * kN * g.HB);   // (16-bit tensors: bf16 snapshots unless fp32 ones are asked for)
   const size_t bwd_wgs = (size_t)(g.sliced ? g.nbands : 1) * B * g.bwd_bpb;
   g.ring_bytes = g.ck_shift ? align_up((d->dtype == M2D_BF16 ? 2 : sizeof(float)) * bwd_wgs * (every - 1) * g.bwd_nw * g.CS * kN * g.HB) : 0;
   const bool rows = g.nbands > 1 && !g.stacked;   // boundary rows travel between bands
@@ -3543,14 +3556,14 @@ int stage_bc(ScanParams& sp, const m2d_desc* d, const void* BT, const void* BL, 
 #define M2D_BUILT(T, SX, MODE, NW, OTHER) true
 #endif
 
-template <typename T, int EC, bool CK, bool WY, bool SX, int MODE, int NW, bool HALF = false>
+template <typename T, int EC, bool CK, bool WY, bool SX, int MODE, int NW, bool HALF = false, typename ST = T>
 int launch_fwd_as(const ScanParams& sp, hipStream_t st) {
   if constexpr (!M2D_BUILT(T, SX, MODE, NW, EC == 1)) return M2D_ERR_UNSUPPORTED; else {
   constexpr size_t lds = fwd_lds_bytes<T, EC, NW>();
   if (lds > kLdsPerWorkgroup) return M2D_ERR_UNSUPPORTED;   // (make_geometry never picks such a layout)
   static std::atomic<uint64_t> seen{0};
-  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_fwd_kernel<T, EC, CK, WY, SX, MODE, NW, HALF>), lds, seen)) return M2D_ERR_HIP;
-  hipLaunchKernelGGL((m2d_fwd_kernel<T, EC, CK, WY, SX, MODE, NW, HALF>), dim3((unsigned)sp.nwg), dim3((NW + whole_helpers<MODE, NW, EC>()) * 64), lds, st, sp);
+  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_fwd_kernel<T, EC, CK, WY, SX, MODE, NW, HALF, ST>), lds, seen)) return M2D_ERR_HIP;
+  hipLaunchKernelGGL((m2d_fwd_kernel<T, EC, CK, WY, SX, MODE, NW, HALF, ST>), dim3((unsigned)sp.nwg), dim3((NW + whole_helpers<MODE, NW, EC>()) * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
   }
 }
@@ -3607,6 +3620,16 @@ int launch_fwd(const ScanParams& sp0, const m2d_desc* d, const Geometry& g, bool
   sp.bpb = g.fwd_bpb;
   sp.nwg = g.vB * g.fwd_bpb;
   auto once = [&]() {
+    if constexpr (sizeof(T) == 2) {
+      if (g.snap32 && ckpt) {   // bf16 tensors, fp32 snapshots: the forward that keeps them (for the caller, or rebuilt inside the backward)
+        if (g.sliced) {
+          if (g.stage_x) return write_y ? launch_fwd_as<T, 1, true, true, true, kModeSliced, kFwdHalfWaves, false, float>(sp, st) : launch_fwd_as<T, 1, true, false, true, kModeSliced, kFwdHalfWaves, false, float>(sp, st);
+          return write_y ? launch_fwd_as<T, 1, true, true, false, kModeSliced, kFwdHalfWaves, false, float>(sp, st) : launch_fwd_as<T, 1, true, false, false, kModeSliced, kFwdHalfWaves, false, float>(sp, st);
+        }
+        if (g.stage_x) return write_y ? launch_fwd_as<T, 1, true, true, true, kModeSweep, kFwdHalfWaves, false, float>(sp, st) : launch_fwd_as<T, 1, true, false, true, kModeSweep, kFwdHalfWaves, false, float>(sp, st);
+        return write_y ? launch_fwd_as<T, 1, true, true, false, kModeSweep, kFwdHalfWaves, false, float>(sp, st) : launch_fwd_as<T, 1, true, false, false, kModeSweep, kFwdHalfWaves, false, float>(sp, st);
+      }
+    }
     if (g.fwd_split)
       return g.sliced ? launch_fwd_split<T, kModeSliced>(sp, g.stage_x, ckpt, write_y, st, g.fwd_nw)
                       : launch_fwd_split<T, kModeSweep>(sp, g.stage_x, ckpt, write_y, st, g.fwd_nw);
@@ -3666,13 +3689,13 @@ int run_fwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   return rc;
 }
 
-template <typename T, bool SX, int MODE, int NW, bool REPLAY = false>
+template <typename T, bool SX, int MODE, int NW, bool REPLAY = false, typename ST = T>
 int launch_bwd_as(const ScanParams& sp, hipStream_t st) {
   if constexpr (!M2D_BUILT(T, SX, MODE, NW, !REPLAY)) return M2D_ERR_UNSUPPORTED; else {
   constexpr size_t lds = bwd_lds_bytes<T, NW>();
   static std::atomic<uint64_t> seen{0};
-  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_bwd_kernel<T, SX, MODE, NW, REPLAY>), lds, seen)) return M2D_ERR_HIP;
-  hipLaunchKernelGGL((m2d_bwd_kernel<T, SX, MODE, NW, REPLAY>), dim3((unsigned)sp.nwg), dim3((NW + (REPLAY ? 0 : whole_helpers<MODE, NW>())) * 64), lds, st, sp);
+  if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_bwd_kernel<T, SX, MODE, NW, REPLAY, ST>), lds, seen)) return M2D_ERR_HIP;
+  hipLaunchKernelGGL((m2d_bwd_kernel<T, SX, MODE, NW, REPLAY, ST>), dim3((unsigned)sp.nwg), dim3((NW + (REPLAY ? 0 : whole_helpers<MODE, NW>())) * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
   }
 }
@@ -3717,7 +3740,10 @@ int launch_bwd_split(const ScanParams& sp, bool stage_x, hipStream_t st, int nw 
 }
 
 template <typename T, bool SX, int MODE>
-int launch_bwd(const ScanParams& sp, hipStream_t st, int nw = kBwdWaves) {
+int launch_bwd(const ScanParams& sp, hipStream_t st, int nw = kBwdWaves, bool snap32 = false) {
+  if constexpr (sizeof(T) == 2 && MODE != kModeStacked) {
+    if (snap32) return launch_bwd_as<T, SX, MODE, kFwdHalfWaves, false, float>(sp, st);   // bf16 tensors, fp32 snapshots
+  }
   if constexpr (MODE != kModeSliced) {
     if (sp.ck_half) {   // snapshots every 2 steps
       if constexpr (MODE != kModeStacked) { if (nw == kFwdHalfWaves) return launch_bwd2_as<T, SX, MODE, kFwdHalfWaves>(sp, st); }
@@ -3771,13 +3797,13 @@ int run_bwd(const m2d_desc* d, const Geometry& g, ScanParams sp, const void* AT,
   if (!g.sliced) {
     if (g.bwd_split) rc = launch_bwd_split<T, kModeSweep>(sp, g.stage_x, st, g.bwd_nw);
     else if (g.stacked) rc = g.stage_x ? launch_bwd<T, true, kModeStacked>(sp, st) : launch_bwd<T, false, kModeStacked>(sp, st);
-    else rc = g.stage_x ? launch_bwd<T, true, kModeSweep>(sp, st, g.bwd_nw) : launch_bwd<T, false, kModeSweep>(sp, st, g.bwd_nw);
+    else rc = g.stage_x ? launch_bwd<T, true, kModeSweep>(sp, st, g.bwd_nw, g.snap32) : launch_bwd<T, false, kModeSweep>(sp, st, g.bwd_nw, g.snap32);
   } else {
     // every band on workgroups of its own, the last band first: a band waits for the one below it
     sp.nwg = g.nbands * g.vB * g.bwd_bpb;
     sp.prog = sp.link_err + 64 + (size_t)g.nbands * g.vB * (g.fwd_bpb > g.bwd_bpb ? g.fwd_bpb : g.bwd_bpb) * kLinkStride;
     if (g.bwd_split) rc = launch_bwd_split<T, kModeSliced>(sp, g.stage_x, st, g.bwd_nw);
-    else rc = g.stage_x ? launch_bwd<T, true, kModeSliced>(sp, st, g.bwd_nw) : launch_bwd<T, false, kModeSliced>(sp, st, g.bwd_nw);
+    else rc = g.stage_x ? launch_bwd<T, true, kModeSliced>(sp, st, g.bwd_nw, g.snap32) : launch_bwd<T, false, kModeSliced>(sp, st, g.bwd_nw, g.snap32);
   }
   if (g_profile) (void)hipEventRecord(g_ev[M2D_PASS_BWD][1], st);
   if (rc) return rc;

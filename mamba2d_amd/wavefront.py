@@ -64,10 +64,22 @@ SAVE_CHECKPOINTS = os.environ.get("M2D_SAVE_CHECKPOINTS", "1") != "0"
 CKPT_INTERVALS = cabi.CKPT_INTERVALS
 
 
+# bf16 tensors keep their snapshots rounded to bf16, as the reference keeps its whole hidden-state tensor
+# (wf_cuda.cu:5,59-67).  True: kept in fp32 (M2D_FLAG_FP32_SNAPSHOTS: an interval of 4 steps, twice the bytes, slower
+# kernels; gradient elements then meet the bound of the forward).  Read at forward time like the interval, and handed
+# to the operators as the interval -4 ("every 4 steps, in fp32"), so that a backward uses what its forward ran with.
+FP32_SNAPSHOTS = os.environ.get("M2D_FP32_SNAPSHOTS", "0") == "1"
+FP32_SNAPSHOT_INTERVAL = -4
+
+
 def _interval() -> int:
     v = cabi.CKPT_INTERVAL
     if v not in CKPT_INTERVALS:
         raise ValueError(f"m2dscan: CKPT_INTERVAL must be one of {CKPT_INTERVALS}, got {v!r}")
+    if FP32_SNAPSHOTS:
+        if v not in (0, 4):
+            raise ValueError(f"m2dscan: FP32_SNAPSHOTS keeps a snapshot every 4 steps, CKPT_INTERVAL is {v}")
+        return FP32_SNAPSHOT_INTERVAL
     return v
 
 
@@ -84,7 +96,9 @@ FUSED_PROJECTIONS = os.environ.get("M2D_FUSED_PROJECTIONS", "1") != "0"
 
 def _ckpt_bytes(x, N, flip=False, packed_bc=False, ckpt_interval=0) -> int:
     d = cabi.make_desc(x, N, flip)
-    d.ckpt_interval = ckpt_interval
+    d.ckpt_interval = 4 if ckpt_interval == FP32_SNAPSHOT_INTERVAL else ckpt_interval
+    if ckpt_interval == FP32_SNAPSHOT_INTERVAL:
+        d.flags |= cabi.M2D_FLAG_FP32_SNAPSHOTS
     if packed_bc:   # the caller brings the packed B/C records: the buffer has no room for them
         d.flags |= cabi.M2D_FLAG_PACKED_BC
     return int(cabi.lib.m2d_scan_ckpt_bytes(ctypes.byref(d)))
@@ -103,8 +117,9 @@ def _scan_bwd_fake(x, deltaT, deltaL, AT, AL, BT, BL, C, D, dy, ckpt, flip, raw_
     if sum_parts:   # the per-workgroup sums of d_C, d_BT, d_BL in fp32, as many as the library's plan has channel groups
         d = cabi.Desc(*x.shape, AT.shape[1], cabi.M2D_BF16 if x.dtype == torch.bfloat16 else cabi.M2D_F32,
                       (cabi.M2D_FLAG_FLIP if flip else 0) | (cabi.M2D_FLAG_RAW_PARAMS if raw_params else 0)
-                      | (cabi.M2D_FLAG_PACKED_BC if packed_bc else 0) | (cabi.M2D_FLAG_DPRE if dpre else 0) | cabi.M2D_FLAG_SUM_PARTS,
-                      ckpt_interval)
+                      | (cabi.M2D_FLAG_PACKED_BC if packed_bc else 0) | (cabi.M2D_FLAG_DPRE if dpre else 0) | cabi.M2D_FLAG_SUM_PARTS
+                      | (cabi.M2D_FLAG_FP32_SNAPSHOTS if ckpt_interval == FP32_SNAPSHOT_INTERVAL else 0),
+                      4 if ckpt_interval == FP32_SNAPSHOT_INTERVAL else ckpt_interval)
         parts = int(cabi.lib.m2d_scan_sum_parts(ctypes.byref(d)))
         bc = [x.new_empty((parts, *x.shape[:3], 3 * AT.shape[1]), dtype=torch.float32), x.new_empty((0,)), x.new_empty((0,))]
     return [torch.empty_like(x), torch.empty_like(deltaT), torch.empty_like(deltaL), torch.empty_like(AT), torch.empty_like(AL),

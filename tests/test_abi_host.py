@@ -51,11 +51,13 @@ def test_descriptor_validation(cabi):
     # spatial dims must exceed 1, like the reference's ValueError (wavefront_cuda.py:323-324)
     assert chk(D(cabi, H=1)) == 2 and chk(D(cabi, W=1)) == 2 and chk(D(cabi, B=0)) == 2
     # flags 1 (flip), 4 (raw parameters), 8 (packed B/C), 16 (gradients before the softplus) and the two lane
-    # layout hints 32 and 64 (one of them at most) belong to the scan, and so do the test aid 128 and the
-    # unfinished channel sums 256; 2 is a projection flag, 512 nobody's
+    # layout hints 32 and 64 (one of them at most) belong to the scan, and so do the test aid 128, the
+    # unfinished channel sums 256 and the fp32 snapshots of bf16 tensors 512 (at the default interval or 4); 2 is a projection
+    # flag, 1024 nobody's
     assert chk(D(cabi, flags=4)) == 0 and chk(D(cabi, flags=29)) == 0 and chk(D(cabi, flags=2)) == 3
     assert chk(D(cabi, flags=32)) == 0 and chk(D(cabi, flags=64 | 1)) == 0 and chk(D(cabi, flags=96)) == 3
-    assert chk(D(cabi, N=8)) == 3 and chk(D(cabi, dtype=7)) == 3 and chk(D(cabi, flags=128)) == 0 and chk(D(cabi, flags=256)) == 0 and chk(D(cabi, flags=512)) == 3
+    assert chk(D(cabi, N=8)) == 3 and chk(D(cabi, dtype=7)) == 3 and chk(D(cabi, flags=128)) == 0 and chk(D(cabi, flags=256)) == 0 and chk(D(cabi, flags=512)) == 0 and chk(D(cabi, flags=1024)) == 3
+    assert chk(D(cabi, dtype=1, flags=512, ckpt_interval=4)) == 0 and chk(D(cabi, dtype=1, flags=512, ckpt_interval=2)) == 3 and chk(D(cabi, dtype=0, flags=512, ckpt_interval=8)) == 0
     # steps between snapshots: the library's choice, 2, 4, 8 or 16
     assert all(chk(D(cabi, ckpt_interval=v)) == 0 for v in (0, 2, 4, 8, 16))
     assert all(chk(D(cabi, ckpt_interval=v)) == 3 for v in (1, 3, 12, 32, -4))
