@@ -1334,17 +1334,19 @@ constexpr int kSplitHalfWaves = 4;   // where workgroups of 8 would leave comput
 // addresses, copies, the wait for the neighbouring band).  So such a workgroup gets 4 more waves that do nothing but
 // stage (and, in the backward, add up the channel sums of every step), one to a SIMD beside a wave that does nothing
 // but sweep: the two chains run side by side.
-// (Workgroups of 8 sweeping waves stay as they are: with 8 more the backward no longer fits the registers of a lane
-// at 4 waves to a SIMD and ran a quarter slower, 768x768 and 1024x1024; with 4 more the compiler fails.)
+// Workgroups of 8 sweeping waves have the same 4 (3 waves to a SIMD, 168 registers a lane: 1024x1024x64 fp32 forward
+// 2.29 -> 2.10 ms, backward 4.97 -> 4.39), except where rows are not whole 16-byte chunks (SX false: the compiler's
+// register allocator fails on those kernels at 768 threads).  With 8 more the backward no longer fits the registers
+// of a lane at 4 waves to a SIMD and ran a quarter slower.
 constexpr int kSplitHelpers = 4;
-template <int MODE, int NWS>
-constexpr int split_helpers() { return (MODE == kModeSliced && NWS == kSplitHalfWaves) ? kSplitHelpers : 0; }
+template <int MODE, int NWS, bool SX = true>
+constexpr int split_helpers() { return (MODE == kModeSliced && (NWS == kSplitHalfWaves || SX)) ? kSplitHelpers : 0; }
 __device__ __forceinline__ float sum_over_groups(float v) {
   v = fold16(v, v);
   return fold32(v, v);
 }
 template <typename T, bool CKPT, bool WRITE_Y, bool STAGE_X, int MODE, int NWS = kSplitWaves>
-__global__ __launch_bounds__((NWS + split_helpers<MODE, NWS>()) * 64) void m2d_fwd_split_kernel(const ScanParams pin) {
+__global__ __launch_bounds__((NWS + split_helpers<MODE, NWS, STAGE_X>()) * 64) void m2d_fwd_split_kernel(const ScanParams pin) {
   static_assert(MODE != kModeStacked, "stacked images are many: they never need the split");
   constexpr bool SLICED = MODE == kModeSliced;
   const ScanParams& p = pin;
@@ -1352,7 +1354,7 @@ __global__ __launch_bounds__((NWS + split_helpers<MODE, NWS>()) * 64) void m2d_f
   __builtin_assume(p.rb == kRB);
   __builtin_assume(p.S >= kHB + kCK - 1);
   constexpr int NW = NWS, CW = NW;
-  constexpr int NH = split_helpers<MODE, NWS>();   // waves that only stage (then the first NW waves only sweep)
+  constexpr int NH = split_helpers<MODE, NWS, STAGE_X>();   // waves that only stage (then the first NW waves only sweep)
   constexpr int NSTG = NH ? NH : NW;               // waves that share the copies of a block
   using SG = Stage<T, 3, CW, false>;
   constexpr bool WIDEN = sizeof(T) == 2;
@@ -2686,7 +2688,7 @@ __global__ __launch_bounds__((NW + whole_helpers<MODE, NW>()) * 64) void m2d_bwd
 // over channels (d_C, d_BT, d_BL) across the 8 waves through LDS, as in m2d_bwd_kernel, a float4 of
 // four states per lane.  Memory formats are those of m2d_bwd_kernel.
 template <typename T, bool STAGE_X, int MODE, int NWS = kSplitWaves>
-__global__ __launch_bounds__((NWS + split_helpers<MODE, NWS>()) * 64) void m2d_bwd_split_kernel(const ScanParams pin) {
+__global__ __launch_bounds__((NWS + split_helpers<MODE, NWS, STAGE_X>()) * 64) void m2d_bwd_split_kernel(const ScanParams pin) {
   static_assert(MODE != kModeStacked, "stacked images are many: they never need the split");
   constexpr bool SLICED = MODE == kModeSliced;
   const ScanParams& p = pin;
@@ -2694,7 +2696,7 @@ __global__ __launch_bounds__((NWS + split_helpers<MODE, NWS>()) * 64) void m2d_b
   __builtin_assume(p.rb == kRB);
   __builtin_assume(p.S >= kHB + kCK - 1);
   constexpr int NW = NWS, CW = NW;
-  constexpr int NH = split_helpers<MODE, NWS>();   // waves that only stage and add up the channel sums (then the first NW waves only sweep)
+  constexpr int NH = split_helpers<MODE, NWS, STAGE_X>();   // waves that only stage and add up the channel sums (then the first NW waves only sweep)
   constexpr int NSTG = NH ? NH : NW;               // waves that share the copies of a block
   static_assert(NH == 0 || NH >= 3, "three waves add up the channel sums");
   constexpr int SLOT = 3 * 64;           // float4s per wave in one exchange buffer
@@ -3404,9 +3406,10 @@ Geometry make_geometry(const m2d_desc* d) {
   // Workgroups of 8 waves (8 channels) under way on at most half of the compute units: workgroups of 4 then run on
   // twice as many, each wave with a SIMD to itself (a sweep of few images is as fast as one wave gets through its
   // blocks).
-  // In the linked sweep a workgroup of 4 has 4 more waves that stage for it (split_helpers), which is worth more than
-  // a compute unit for every workgroup under way: up to 7 workgroups for every 5 units (measured, E=64 fp32: 512x512
-  // 3.14 -> 2.54 ms forward+backward kernels and 640x640 3.90 -> 3.62 with workgroups of 4; 768x768 4.76 -> 5.08).
+  // In the linked sweep both sizes of workgroup have 4 more waves that stage for them (split_helpers); workgroups of
+  // 4 stay ahead up to 7 of them under way for every 5 units (measured, E=64 fp32, forward+backward kernels with
+  // workgroups of 4 against 8: 384x384 1.65 against 1.86 ms, 512x512 2.56 against 2.61, 640x640 3.63 against 3.29,
+  // 768x768 5.08 against 4.10).
   const int64_t wg4 = (int64_t)B * ((d->E + kSplitHalfWaves - 1) / kSplitHalfWaves) * together;
   const bool helped = g.sliced && split_helpers<kModeSliced, kSplitHalfWaves>() > 0;
   const int split_nw = (helped ? 5 * wg4 <= 7 * ncu : 2 * (int64_t)B * ((d->E + kSplitWaves - 1) / kSplitWaves) * together <= ncu)
@@ -3577,7 +3580,7 @@ int launch_fwd_split_as(const ScanParams& sp, hipStream_t st) {
   static_assert(lds <= kLdsPerWorkgroup, "staging must fit the LDS");
   static std::atomic<uint64_t> seen{0};
   if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_fwd_split_kernel<T, CK, WY, SX, MODE, NWS>), lds, seen)) return M2D_ERR_HIP;
-  hipLaunchKernelGGL((m2d_fwd_split_kernel<T, CK, WY, SX, MODE, NWS>), dim3((unsigned)sp.nwg), dim3((NWS + split_helpers<MODE, NWS>()) * 64), lds, st, sp);
+  hipLaunchKernelGGL((m2d_fwd_split_kernel<T, CK, WY, SX, MODE, NWS>), dim3((unsigned)sp.nwg), dim3((NWS + split_helpers<MODE, NWS, SX>()) * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
   }
 }
@@ -3728,7 +3731,7 @@ int launch_bwd_split_as(const ScanParams& sp, hipStream_t st) {
   static_assert(lds <= kLdsPerWorkgroup, "exchange buffers and staging must fit the LDS");
   static std::atomic<uint64_t> seen{0};
   if (!allow_dynamic_lds(reinterpret_cast<const void*>(&m2d_bwd_split_kernel<T, SX, MODE, NWS>), lds, seen)) return M2D_ERR_HIP;
-  hipLaunchKernelGGL((m2d_bwd_split_kernel<T, SX, MODE, NWS>), dim3((unsigned)sp.nwg), dim3((NWS + split_helpers<MODE, NWS>()) * 64), lds, st, sp);
+  hipLaunchKernelGGL((m2d_bwd_split_kernel<T, SX, MODE, NWS>), dim3((unsigned)sp.nwg), dim3((NWS + split_helpers<MODE, NWS, SX>()) * 64), lds, st, sp);
   return hipGetLastError() == hipSuccess ? M2D_OK : M2D_ERR_HIP;
   }
 }
@@ -3940,7 +3943,7 @@ int m2d_scan_plan(const m2d_desc* desc, int pass, char* text, size_t cap) {
   else if (g.stacked) snprintf(sched, sizeof sched, "stacked images, %d per stream, %d bands", g.ips, g.nbands);
   else snprintf(sched, sizeof sched, "one stream per image, %d band%s back to back", g.nbands, g.nbands == 1 ? "" : "s");
   if (split) {
-    const int helpers = !g.sliced ? 0 : (nw == kSplitHalfWaves ? split_helpers<kModeSliced, kSplitHalfWaves>() : split_helpers<kModeSliced, kSplitWaves>());
+    const int helpers = !g.sliced ? 0 : (nw == kSplitHalfWaves ? split_helpers<kModeSliced, kSplitHalfWaves>() : g.stage_x ? split_helpers<kModeSliced, kSplitWaves, true>() : split_helpers<kModeSliced, kSplitWaves, false>());
     char extra[48] = "";
     if (helpers) snprintf(extra, sizeof extra, " and %d that stage", helpers);
     snprintf(text, cap, "%s: %s, %lld workgroups of %d waves%s, %d channels each, 4 states per lane",

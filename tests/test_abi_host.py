@@ -155,7 +155,9 @@ def test_plan_names_kernel_and_schedule(cabi):
     one = cabi.scan_plan(1, 256, 256, 64, torch.float32, cabi.M2D_PASS_BWD)
     assert one.startswith("m2d_bwd_split_kernel: linked sweep, 19 bands, 304 workgroups of 4 waves and 4 that stage, 4 channels each, 4 states per lane")
     two = cabi.scan_plan(1, 768, 768, 64, torch.float32, cabi.M2D_PASS_BWD)   # (more bands under way: workgroups of 8)
-    assert two.startswith("m2d_bwd_split_kernel: linked sweep, 55 bands, 440 workgroups of 8 waves, 8 channels each, 4 states per lane")
+    assert two.startswith("m2d_bwd_split_kernel: linked sweep, 55 bands, 440 workgroups of 8 waves and 4 that stage, 8 channels each, 4 states per lane")
+    ragged = cabi.scan_plan(1, 768, 768, 62, torch.float32, cabi.M2D_PASS_BWD)   # (rows that are no whole 16-byte chunks: no staging waves beside 8)
+    assert ragged.startswith("m2d_bwd_split_kernel: linked sweep, 55 bands, 440 workgroups of 8 waves, 8 channels each, 4 states per lane")
     whole = cabi.scan_plan(1, 256, 256, 64, torch.float32, cabi.M2D_PASS_FWD, flags=cabi.M2D_FLAG_WHOLE_STATES)
     assert whole.startswith("m2d_fwd_kernel: linked sweep, 19 bands") and "16 states per lane" in whole
     small = cabi.scan_plan(128, 7, 7, 512, torch.bfloat16, cabi.M2D_PASS_FWD)

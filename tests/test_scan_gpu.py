@@ -143,6 +143,8 @@ SHAPES = [
     (2, 100, 33, 48), # the same, eight bands of two images, three workgroups of 16 channels per band
     (128, 4, 3, 128), # 512 workgroups with one channel per lane, 256 with two: the bf16 forward takes two channels per lane
     (256, 17, 4, 64), # the same from the batch side, two padded bands
+    (1, 160, 340, 128), # linked sweep with so many bands under way that workgroups take 8 channels: 8 waves and 4 that stage
+    (1, 160, 340, 122), # the same with rows that are no whole 16-byte chunks: 8 waves that also stage
 ]
 
 
