@@ -1329,18 +1329,19 @@ __global__ __launch_bounds__((NW + whole_helpers<MODE, NW, EC>()) * 64) void m2d
 // m2d_fwd_kernel; y of a cell is the sum over the 4 lane groups (two lane-swap steps), stored by group 0.
 constexpr int kSplitWaves = 8;
 constexpr int kSplitHalfWaves = 4;   // where workgroups of 8 would leave compute units idle
-// Linked sweep in workgroups of 4 waves: a step of a wave that has a SIMD to itself takes as long as its chain of
+// Workgroups of 4 waves: a step of a wave that has a SIMD to itself takes as long as its chain of
 // instructions, and of those under a third are the step's arithmetic; the rest stages the next block (positions,
 // addresses, copies, the wait for the neighbouring band).  So such a workgroup gets 4 more waves that do nothing but
 // stage (and, in the backward, add up the channel sums of every step), one to a SIMD beside a wave that does nothing
 // but sweep: the two chains run side by side.
 // Workgroups of 8 sweeping waves have the same 4 (3 waves to a SIMD, 168 registers a lane: 1024x1024x64 fp32 forward
-// 2.29 -> 2.10 ms, backward 4.97 -> 4.39), except where rows are not whole 16-byte chunks (SX false: the compiler's
+// 2.29 -> 2.10 ms, backward 4.97 -> 4.39; 32 images of 56x56x64 bf16, one stream each, 0.146 -> 0.134 and 0.338 ->
+// 0.284), except where rows are not whole 16-byte chunks (SX false: the compiler's
 // register allocator fails on those kernels at 768 threads).  With 8 more the backward no longer fits the registers
 // of a lane at 4 waves to a SIMD and ran a quarter slower.
 constexpr int kSplitHelpers = 4;
 template <int MODE, int NWS, bool SX = true>
-constexpr int split_helpers() { return (MODE == kModeSliced && (NWS == kSplitHalfWaves || SX)) ? kSplitHelpers : 0; }
+constexpr int split_helpers() { return (NWS == kSplitHalfWaves || SX) ? kSplitHelpers : 0; }
 __device__ __forceinline__ float sum_over_groups(float v) {
   v = fold16(v, v);
   return fold32(v, v);
@@ -3406,14 +3407,13 @@ Geometry make_geometry(const m2d_desc* d) {
   // Workgroups of 8 waves (8 channels) under way on at most half of the compute units: workgroups of 4 then run on
   // twice as many, each wave with a SIMD to itself (a sweep of few images is as fast as one wave gets through its
   // blocks).
-  // In the linked sweep both sizes of workgroup have 4 more waves that stage for them (split_helpers); workgroups of
+  // Both sizes of workgroup have 4 more waves that stage for them (split_helpers).  In the linked sweep workgroups of
   // 4 stay ahead up to 7 of them under way for every 5 units (measured, E=64 fp32, forward+backward kernels with
   // workgroups of 4 against 8: 384x384 1.65 against 1.86 ms, 512x512 2.56 against 2.61, 640x640 3.63 against 3.29,
   // 768x768 5.08 against 4.10).
   const int64_t wg4 = (int64_t)B * ((d->E + kSplitHalfWaves - 1) / kSplitHalfWaves) * together;
-  const bool helped = g.sliced && split_helpers<kModeSliced, kSplitHalfWaves>() > 0;
-  const int split_nw = (helped ? 5 * wg4 <= 7 * ncu : 2 * (int64_t)B * ((d->E + kSplitWaves - 1) / kSplitWaves) * together <= ncu)
-                           ? kSplitHalfWaves : kSplitWaves;
+  // (one stream per image: workgroups of 4 only while each has a compute unit)
+  const int split_nw = (g.sliced ? 5 * wg4 <= 7 * ncu : wg4 <= ncu) ? kSplitHalfWaves : kSplitWaves;
   if (g.fwd_split) {
     g.fwd_ec = 1;
     g.fwd_nw = split_nw;
@@ -3943,7 +3943,7 @@ int m2d_scan_plan(const m2d_desc* desc, int pass, char* text, size_t cap) {
   else if (g.stacked) snprintf(sched, sizeof sched, "stacked images, %d per stream, %d bands", g.ips, g.nbands);
   else snprintf(sched, sizeof sched, "one stream per image, %d band%s back to back", g.nbands, g.nbands == 1 ? "" : "s");
   if (split) {
-    const int helpers = !g.sliced ? 0 : (nw == kSplitHalfWaves ? split_helpers<kModeSliced, kSplitHalfWaves>() : g.stage_x ? split_helpers<kModeSliced, kSplitWaves, true>() : split_helpers<kModeSliced, kSplitWaves, false>());
+    const int helpers = (nw == kSplitHalfWaves ? split_helpers<kModeSliced, kSplitHalfWaves>() : g.stage_x ? split_helpers<kModeSliced, kSplitWaves, true>() : split_helpers<kModeSliced, kSplitWaves, false>());
     char extra[48] = "";
     if (helpers) snprintf(extra, sizeof extra, " and %d that stage", helpers);
     snprintf(text, cap, "%s: %s, %lld workgroups of %d waves%s, %d channels each, 4 states per lane",
