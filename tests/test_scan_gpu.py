@@ -295,3 +295,38 @@ def test_linked_sweep_repeats_bit_identically_on_reused_buffers(cabi):
                     assert torch.equal(u, v), (it, seed)
             else:
                 runs[seed] = got
+
+
+def test_linked_sweeps_on_two_streams_at_once(cabi):
+    """Two linked sweeps under way on the device at the same time, one per stream, each with workspaces of its own: the
+    workgroups of one launch wait only for lower workgroups of the same launch, which the device has started before
+    them, so neither launch can hold the other up for good.  Each must give the bits of its run alone."""
+    say("\ncase linked_sweeps_two_streams")
+    probs = []
+    for (B, H, W, E, dtype, seed) in [(1, 300, 120, 32, torch.float32, 3), (2, 150, 200, 24, torch.bfloat16, 4)]:
+        inp = {k: v.cuda() for k, v in so.make_inputs(B, H, W, E, 16, seed=seed, dtype=dtype).items()}
+        probs.append(([inp[k] for k in so.INPUT_NAMES], inp["dy"]))
+        assert "linked sweep" in cabi.scan_plan(B, H, W, E, dtype, cabi.M2D_PASS_BWD)
+
+    def run(a, dy):
+        y, ck = cabi.scan_fwd(*a, save_ckpt=True)
+        return [y] + list(cabi.scan_bwd(*a, dy, ckpt=ck))
+
+    alone = [[t.clone() for t in run(*p)] for p in probs]
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]   # default priority
+    check, cabi.CHECK_LINKS = cabi.CHECK_LINKS, False      # (the check synchronises after every call)
+    try:
+        for it in range(6):
+            outs = []
+            for s, p in zip(streams, probs):
+                s.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(s):
+                    outs.append(run(*p))
+            torch.cuda.synchronize()
+            for want, got in zip(alone, outs):
+                for u, v in zip(want, got):
+                    assert torch.equal(u, v), it
+            del outs
+    finally:
+        cabi.CHECK_LINKS = check
