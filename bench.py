@@ -454,21 +454,22 @@ def _short_scan(name, steps, warmup):
 
 def also_workloads(args, rates, cfg1_fwd_bwd_ms):
     """Short measurements of the other configurations in the same process, after the timed region of the headline
-    workload: the four stage scans in sequence (cfg2), one image of 256x256 and of 2048x2048 (cfg4, with the
+    workload: the four stage scans in sequence (cfg2), one image of 256x256, 1024x1024 and 2048x2048 (cfg4, with the
     allocator's peak), the stage-1 scan at the reference's training batch of 64, and the entry point
     wavefront_scan_cuda with its projections at the headline shape."""
     import math
     import torch
     from mamba2d_amd import wavefront as wf
     out = {}
-    stages = {k: _short_scan(k, 10, 3) for k in ("stage2", "stage3", "stage4")}
+    stages = {k: _short_scan(k, 30, 5) for k in ("stage2", "stage3", "stage4")}
     # (the first stage is the headline workload itself; the stages run back to back on one stream, so the sum of their
     # steps is what `--workload cfg2` times as one step)
     out["cfg2"] = {"fwd_bwd_ms": round(cfg1_fwd_bwd_ms + sum(v["fwd_bwd_ms"] for v in stages.values()), 4), "stages": stages}
-    out["cfg4_256"] = _short_scan("hires256", 10, 3)
-    out["train64"] = _short_scan("train64", 10, 3)   # (not a configuration of the baseline: the batch the reference trains with)
+    out["cfg4_256"] = _short_scan("hires256", 30, 5)
+    out["train64"] = _short_scan("train64", 30, 5)   # (not a configuration of the baseline: the batch the reference trains with)
     free, _ = torch.cuda.mem_get_info()
     if free > 40 * 2**30:
+        out["cfg4_1024"] = _short_scan("hires1024", 10, 3)
         out["cfg4_2048"] = _short_scan("hires2048", 3, 1)
     # entry point: projections + scan, fp32 parameters initialised like an M2D block, bf16 activations
     B, E, H, W = WORKLOADS["cfg1"][:4]
@@ -493,7 +494,7 @@ def also_workloads(args, rates, cfg1_fwd_bwd_ms):
             wf.wavefront_scan_cuda(x, *params)
 
     out["entry"] = {"workload": "wavefront_scan_cuda (projections + scan), B=128 E=64 56x56 N=16 dt_rank=4, bf16 activations, recomp=partial",
-                    "fwd_ms": round(_timed(entry_fwd, 10, 3), 4), "fwd_bwd_ms": round(_timed(entry_fwd_bwd, 10, 3), 4), "steps": 10}
+                    "fwd_ms": round(_timed(entry_fwd, 30, 5), 4), "fwd_bwd_ms": round(_timed(entry_fwd_bwd, 30, 5), 4), "steps": 30}
     return out
 
 
